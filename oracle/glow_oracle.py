@@ -1,0 +1,356 @@
+"""numpy-facing loader for ``libglow_oracle.so`` (the CPU restatement).
+
+TEST INFRASTRUCTURE: the checker and the timed CPU baseline, never a product
+code path. Every function forwards to the C function of the same name in
+``glow_oracle.c``, which cites the reference lines it restates.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libglow_oracle.so")
+
+ASYMMETRIC, SYMMETRIC, SYMMETRIC_WITH_UNSIGNED, SYMMETRIC_POW2 = 0, 1, 2, 3
+U8_F32, U8_F16, U4_F16, U4_F32 = 0, 1, 2, 3
+ACT_NONE, ACT_RELU, ACT_CLIP, ACT_TANH, ACT_SIGMOID, ACT_LEAKY_RELU = range(6)
+
+
+def build(force=False):
+    """Compile the restatement (and oracle/_ref when the reference is there)."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.check_call(["make", "-C", _HERE, "all"],
+                              stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+class ConvGeom(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in (
+        "N", "IH", "IW", "IC", "OH", "OW", "OC", "KH", "KW", "strideH",
+        "strideW", "padT", "padL", "dilH", "dilW", "group")]
+
+
+def conv_geom(N, IH, IW, IC, OC, kernel, stride, pads, group=1, dilation=(1, 1)):
+    """pads = (top, left, bottom, right). Output size as Glow computes it
+    (calculateConvPoolOutputDims, include/glow/Graph/Nodes.h)."""
+    KH, KW = kernel
+    sh, sw = stride
+    pt, pl, pb, pr = pads
+    dh, dw = dilation
+    OH = (IH + pt + pb - (KH - 1) * dh - 1) // sh + 1
+    OW = (IW + pl + pr - (KW - 1) * dw - 1) // sw + 1
+    return ConvGeom(N, IH, IW, IC, OH, OW, OC, KH, KW, sh, sw, pt, pl, dh, dw,
+                    group)
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        _lib = C.CDLL(_LIB_PATH)
+        _lib.go_scale_i32.restype = C.c_int32
+        _lib.go_scale_i32.argtypes = [C.c_int32] * 5
+        _lib.go_clip_i8.restype = C.c_int8
+        _lib.go_clip_i8.argtypes = [C.c_int32]
+        _lib.go_f32_to_f16.restype = C.c_uint16
+        _lib.go_f32_to_f16.argtypes = [C.c_float]
+        _lib.go_f16_to_f32.restype = C.c_float
+        _lib.go_f16_to_f32.argtypes = [C.c_uint16]
+        _lib.go_quantize_value_i8.restype = C.c_int8
+        _lib.go_quantize_value_i8.argtypes = [C.c_float, C.c_float, C.c_int32]
+        _lib.go_quantize_value_i32.restype = C.c_int32
+        _lib.go_quantize_value_i32.argtypes = [C.c_float, C.c_float, C.c_int32]
+        _lib.go_fused_row_bytes.restype = C.c_size_t
+        _lib.go_fused_row_bytes.argtypes = [C.c_size_t, C.c_int]
+        _lib.go_activation_i32.restype = C.c_int32
+    return _lib
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p) if a is not None else None
+
+
+def _c(a, dt):
+    return np.ascontiguousarray(a, dtype=dt)
+
+
+def _i32v(a):
+    return _c(a, np.int32)
+
+
+# ---- scalars ---------------------------------------------------------------
+
+def scale_i32(x, pre, post, scale, offset):
+    return lib().go_scale_i32(int(x), int(pre), int(post), int(scale), int(offset))
+
+
+def clip_i8(v):
+    return lib().go_clip_i8(int(v))
+
+
+def activation_i32(x, offset, act, args=()):
+    a = _i32v(list(args) + [0, 0, 0])
+    return lib().go_activation_i32(C.c_int32(int(x)), C.c_int32(int(offset)),
+                                   C.c_int32(int(act)), _p(a))
+
+
+def f32_to_f16_bits(x):
+    return lib().go_f32_to_f16(float(x))
+
+
+def f16_bits_to_f32(h):
+    return lib().go_f16_to_f32(int(h))
+
+
+def quantize_scale_offset_32to8(scale, offset=0):
+    """-> (pre, post, scale, offset)"""
+    out = (C.c_int32 * 4)()
+    lib().go_quantize_scale_offset_32to8(C.c_float(scale), C.c_int32(offset), out)
+    return tuple(out)
+
+
+def choose_qparams(mn, mx, schema=ASYMMETRIC, qty=8):
+    s = C.c_float()
+    o = C.c_int32()
+    lib().go_choose_qparams(C.c_float(mn), C.c_float(mx), C.c_int(schema),
+                            C.c_int(qty), C.byref(s), C.byref(o))
+    return s.value, o.value
+
+
+def specialize_bias_weights_qparams(bias_scale, bias_offset, input_scale,
+                                    weights_scale, bias_is_i32=True,
+                                    bias_zero=False):
+    bs = C.c_float(bias_scale)
+    bo = C.c_int32(bias_offset)
+    ws = C.c_float(weights_scale)
+    lib().go_specialize_bias_weights_qparams(
+        C.byref(bs), C.byref(bo), C.c_float(input_scale), C.byref(ws),
+        C.c_int(bias_is_i32), C.c_int(bias_zero))
+    return bs.value, bo.value, ws.value
+
+
+def quantize_value_i8(x, scale, offset):
+    return lib().go_quantize_value_i8(x, scale, offset)
+
+
+def quantize_value_i32(x, scale, offset):
+    return lib().go_quantize_value_i32(x, scale, offset)
+
+
+def rowwise_quantize_i8(w, schema=SYMMETRIC):
+    w = _c(w, np.float32)
+    rows, cols = w.shape
+    q = np.empty((rows, cols), np.int8)
+    s = np.empty(rows, np.float32)
+    o = np.empty(rows, np.int32)
+    lib().go_rowwise_quantize_i8(_p(w), C.c_size_t(rows), C.c_size_t(cols),
+                                 C.c_int(schema), _p(q), _p(s), _p(o))
+    return q, s, o
+
+
+def fused_row_bytes(cols, kind):
+    return lib().go_fused_row_bytes(cols, kind)
+
+
+def fused_rowwise_quantize(x, kind):
+    x = _c(x, np.float32)
+    rows, cols = x.shape
+    out = np.zeros((rows, fused_row_bytes(cols, kind)), np.uint8)
+    lib().go_fused_rowwise_quantize(_p(x), C.c_size_t(rows), C.c_size_t(cols),
+                                    C.c_int(kind), _p(out))
+    return out
+
+
+# ---- elementwise -----------------------------------------------------------
+
+def quantize_i8(x, scale, offset):
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, np.int8)
+    lib().go_quantize_i8(_p(out), _p(x), C.c_size_t(x.size), C.c_float(scale),
+                         C.c_int32(offset))
+    return out
+
+
+def dequantize_i8(q, scale, offset):
+    q = _c(q, np.int8)
+    out = np.empty(q.shape, np.float32)
+    lib().go_dequantize_i8(_p(out), _p(q), C.c_size_t(q.size), C.c_float(scale),
+                           C.c_int32(offset))
+    return out
+
+
+def rescale_i8(q, out_offset, in_offset, pre, post, scale):
+    q = _c(q, np.int8)
+    out = np.empty(q.shape, np.int8)
+    lib().go_rescale_i8(_p(out), _p(q), C.c_size_t(q.size),
+                        C.c_int32(out_offset), C.c_int32(in_offset),
+                        C.c_int32(pre), C.c_int32(post), C.c_int32(scale))
+    return out
+
+
+# ---- FC / matmul -------------------------------------------------------------
+
+def _bias(bias):
+    bias = np.ascontiguousarray(bias)
+    if bias.dtype == np.int8:
+        return bias, 1
+    return _c(bias, np.int32), 0
+
+
+def fc_i8(x, w_kn, bias, out_offset, in_offset, w_offset, bias_offset, biasP,
+          outP):
+    """biasP/outP = (pre, post, scale)."""
+    x = _c(x, np.int8)
+    w_kn = _c(w_kn, np.int8)
+    M, K = x.shape
+    N = w_kn.shape[1]
+    bias, b8 = _bias(bias)
+    out = np.empty((M, N), np.int8)
+    lib().go_fc_i8(_p(out), _p(x), _p(w_kn), _p(bias), C.c_int(b8),
+                   C.c_size_t(M), C.c_size_t(K), C.c_size_t(N),
+                   C.c_int32(out_offset), C.c_int32(in_offset),
+                   C.c_int32(w_offset), C.c_int32(bias_offset),
+                   *[C.c_int32(int(v)) for v in biasP],
+                   *[C.c_int32(int(v)) for v in outP])
+    return out
+
+
+def rwq_fc_i8(x, w_nk, bias, w_offsets, bias_pre, bias_post, bias_scale,
+              out_pre, out_post, out_scale, out_offset, in_offset, bias_offset):
+    x = _c(x, np.int8)
+    w_nk = _c(w_nk, np.int8)
+    M, K = x.shape
+    N = w_nk.shape[0]
+    bias, b8 = _bias(bias)
+    vs = [_i32v(v) for v in (w_offsets, bias_pre, bias_post, bias_scale,
+                             out_pre, out_post, out_scale)]
+    out = np.empty((M, N), np.int8)
+    lib().go_rwq_fc_i8(_p(out), _p(x), _p(w_nk), _p(bias), C.c_int(b8),
+                       *[_p(v) for v in vs], C.c_size_t(M), C.c_size_t(K),
+                       C.c_size_t(N), C.c_int32(out_offset),
+                       C.c_int32(in_offset), C.c_int32(bias_offset))
+    return out
+
+
+def matmul_i8(lhs, rhs, out_offset, lhs_offset, rhs_offset, outP):
+    lhs = _c(lhs, np.int8)
+    rhs = _c(rhs, np.int8)
+    M, K = lhs.shape
+    N = rhs.shape[1]
+    out = np.empty((M, N), np.int8)
+    lib().go_matmul_i8(_p(out), _p(lhs), _p(rhs), C.c_size_t(M), C.c_size_t(K),
+                       C.c_size_t(N), C.c_int32(out_offset),
+                       C.c_int32(lhs_offset), C.c_int32(rhs_offset),
+                       *[C.c_int32(int(v)) for v in outP])
+    return out
+
+
+# ---- convolution -------------------------------------------------------------
+
+def _act_args(args):
+    return _i32v(list(args) + [0, 0, 0])
+
+
+def conv2d_i8(x, filt, bias, geom, out_offset, in_offset, filter_offset,
+              bias_offset, biasP, outP, act=ACT_NONE, act_args=()):
+    x = _c(x, np.int8)
+    filt = _c(filt, np.int8)
+    bias, b8 = _bias(bias)
+    out = np.empty((geom.N, geom.OH, geom.OW, geom.OC), np.int8)
+    aa = _act_args(act_args)
+    lib().go_conv2d_i8(_p(out), _p(x), _p(filt), _p(bias), C.c_int(b8),
+                       C.byref(geom), C.c_int32(out_offset),
+                       C.c_int32(in_offset), C.c_int32(filter_offset),
+                       C.c_int32(bias_offset),
+                       *[C.c_int32(int(v)) for v in biasP],
+                       *[C.c_int32(int(v)) for v in outP], C.c_int32(act),
+                       _p(aa))
+    return out
+
+
+def cwq_conv2d_i8(x, filt, bias, geom, out_offset, in_offset, filter_offsets,
+                  bias_offsets, bias_pre, bias_post, bias_scale, out_pre,
+                  out_post, out_scale, act=ACT_NONE, act_args=()):
+    x = _c(x, np.int8)
+    filt = _c(filt, np.int8)
+    bias, b8 = _bias(bias)
+    vs = [_i32v(v) for v in (filter_offsets, bias_offsets, bias_pre, bias_post,
+                             bias_scale, out_pre, out_post, out_scale)]
+    out = np.empty((geom.N, geom.OH, geom.OW, geom.OC), np.int8)
+    aa = _act_args(act_args)
+    lib().go_cwq_conv2d_i8(_p(out), _p(x), _p(filt), _p(bias), C.c_int(b8),
+                           C.byref(geom), C.c_int32(out_offset),
+                           C.c_int32(in_offset), *[_p(v) for v in vs],
+                           C.c_int32(act), _p(aa))
+    return out
+
+
+# ---- fused-rowwise SLWS ------------------------------------------------------
+
+def _idx(indices):
+    indices = np.ascontiguousarray(indices)
+    if indices.dtype == np.int64:
+        return indices, 1
+    return _c(indices, np.int32), 0
+
+
+def frwq_slws_f32(data, weights, indices, lengths, out_cols=None):
+    data = _c(data, np.uint8)
+    weights = _c(weights, np.float32)
+    indices, i64 = _idx(indices)
+    lengths = _i32v(lengths)
+    in_line = data.shape[1]
+    out_line = in_line - 8 if out_cols is None else out_cols
+    out = np.empty((lengths.size, out_line), np.float32)
+    lib().go_frwq_slws_f32(_p(out), _p(data), _p(weights), _p(indices),
+                           C.c_int(i64), _p(lengths), C.c_size_t(lengths.size),
+                           C.c_size_t(in_line), C.c_size_t(out_line))
+    return out
+
+
+def frwq_slws_generic(data, kind, weights, indices, lengths, out_f16=False,
+                      fp16_accum=False):
+    """weights: None (plain SLS), float32 array, or float16 array."""
+    data = _c(data, np.uint8)
+    indices, i64 = _idx(indices)
+    lengths = _i32v(lengths)
+    in_line = data.shape[1]
+    so = 8 if kind in (U8_F32, U4_F32) else 4
+    out_line = (in_line - so) * (2 if kind in (U4_F16, U4_F32) else 1)
+    w16 = 0
+    if weights is not None:
+        weights = np.ascontiguousarray(weights)
+        if weights.dtype == np.float16:
+            w16 = 1
+        else:
+            weights = _c(weights, np.float32)
+    out = np.empty((lengths.size, out_line),
+                   np.float16 if out_f16 else np.float32)
+    lib().go_frwq_slws_generic(_p(out), C.c_int(out_f16), _p(data),
+                               C.c_int(kind), _p(weights), C.c_int(w16),
+                               _p(indices), C.c_int(i64), _p(lengths),
+                               C.c_size_t(lengths.size), C.c_size_t(in_line),
+                               C.c_size_t(out_line), C.c_int(fp16_accum))
+    return out
+
+
+def embedding_bag_byte_rowwise_offsets_f32(data, weights, indices, offsets,
+                                           has_end_offset):
+    data = _c(data, np.uint8)
+    weights = _c(weights, np.float32)
+    indices = _i32v(indices)
+    offsets = _i32v(offsets)
+    in_line = data.shape[1]
+    out_line = in_line - 8
+    segs = offsets.size
+    out = np.empty((segs - (1 if has_end_offset else 0), out_line), np.float32)
+    lib().go_embedding_bag_byte_rowwise_offsets_f32(
+        _p(out), _p(data), _p(weights), _p(indices), _p(offsets),
+        C.c_size_t(segs), C.c_size_t(indices.size), C.c_size_t(in_line),
+        C.c_size_t(out_line), C.c_int(has_end_offset))
+    return out

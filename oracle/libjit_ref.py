@@ -1,0 +1,226 @@
+"""ctypes access to oracle/_ref/libjit_ref*.so: the reference's own libjit
+kernel sources compiled unmodified by oracle/Makefile (only where the
+reference tree is mounted).
+
+TEST INFRASTRUCTURE: used to validate the restatement in glow_oracle.c and to
+write the golden vectors under tests/golden. Signatures follow
+lib/LLVMIRCodeGen/libjit/libjit_matmul.cpp:395-450, libjit_conv.cpp:496-562,
+libjit.cpp:2416-2481, 2998-3056 (dim_t is uint64_t, libjit_dim_t.h:37).
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def path(fastmath=False):
+    name = "libjit_ref_fastmath.so" if fastmath else "libjit_ref.so"
+    return os.path.join(_HERE, "_ref", name)
+
+
+def available(fastmath=False):
+    return os.path.exists(path(fastmath))
+
+
+_libs = {}
+
+
+def lib(fastmath=False):
+    if fastmath not in _libs:
+        l = C.CDLL(path(fastmath))
+        l.libjit_element_quantize_kernel_i8.restype = C.c_int8
+        l.libjit_element_quantize_kernel_i8.argtypes = [
+            C.c_uint64, C.c_void_p, C.c_float, C.c_int32]
+        l.libjit_element_dequantize_kernel_i8.restype = C.c_float
+        l.libjit_element_dequantize_kernel_i8.argtypes = [
+            C.c_uint64, C.c_void_p, C.c_float, C.c_int32]
+        l.libjit_element_rescale_kernel_i8.restype = C.c_int8
+        l.libjit_element_rescale_kernel_i8.argtypes = [
+            C.c_uint64, C.c_void_p] + [C.c_int32] * 5
+        _libs[fastmath] = l
+    return _libs[fastmath]
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p) if a is not None else None
+
+
+def _c(a, dt):
+    return np.ascontiguousarray(a, dtype=dt)
+
+
+def _dims(*d):
+    return np.asarray(d, dtype=np.uint64)
+
+
+def _i32v(a):
+    return _c(a, np.int32)
+
+
+def quantize_i8(x, scale, offset, fastmath=False):
+    x = _c(x, np.float32).ravel()
+    f = lib(fastmath).libjit_element_quantize_kernel_i8
+    px = x.ctypes.data
+    return np.array([f(i, px, scale, offset) for i in range(x.size)], np.int8)
+
+
+def dequantize_i8(q, scale, offset, fastmath=False):
+    q = _c(q, np.int8).ravel()
+    f = lib(fastmath).libjit_element_dequantize_kernel_i8
+    pq = q.ctypes.data
+    return np.array([f(i, pq, scale, offset) for i in range(q.size)], np.float32)
+
+
+def rescale_i8(q, out_offset, in_offset, pre, post, scale, fastmath=False):
+    q = _c(q, np.int8).ravel()
+    f = lib(fastmath).libjit_element_rescale_kernel_i8
+    pq = q.ctypes.data
+    return np.array([f(i, pq, out_offset, in_offset, pre, post, scale)
+                     for i in range(q.size)], np.int8)
+
+
+def fc_i8(x, w_kn, bias, out_offset, in_offset, w_offset, bias_offset, biasP,
+          outP, fastmath=False):
+    x = _c(x, np.int8)
+    w_kn = _c(w_kn, np.int8)
+    bias = np.ascontiguousarray(bias)
+    M, K = x.shape
+    N = w_kn.shape[1]
+    out = np.empty((M, N), np.int8)
+    fn = (lib(fastmath).libjit_fc_i8_i8 if bias.dtype == np.int8
+          else lib(fastmath).libjit_fc_i8_i32)
+    od, idm, wd, bd = _dims(M, N), _dims(M, K), _dims(K, N), _dims(N)
+    fn(_p(out), _p(x), _p(w_kn), _p(bias), _p(od), _p(idm), _p(wd), _p(bd),
+       C.c_int32(out_offset), C.c_int32(in_offset), C.c_int32(w_offset),
+       C.c_int32(bias_offset), *[C.c_int32(int(v)) for v in biasP],
+       *[C.c_int32(int(v)) for v in outP])
+    return out
+
+
+def rwq_fc_i8(x, w_nk, bias, w_offsets, bias_pre, bias_post, bias_scale,
+              out_pre, out_post, out_scale, out_offset, in_offset, bias_offset,
+              fastmath=False):
+    x = _c(x, np.int8)
+    w_nk = _c(w_nk, np.int8)
+    bias = np.ascontiguousarray(bias)
+    M, K = x.shape
+    N = w_nk.shape[0]
+    out = np.empty((M, N), np.int8)
+    fn = (lib(fastmath).libjit_rowwise_quantized_fc_i8_i8
+          if bias.dtype == np.int8
+          else lib(fastmath).libjit_rowwise_quantized_fc_i8_i32)
+    vs = [_i32v(v) for v in (w_offsets, bias_pre, bias_post, bias_scale,
+                             out_pre, out_post, out_scale)]
+    od, idm, wd, bd = _dims(M, N), _dims(M, K), _dims(N, K), _dims(N)
+    fn(_p(out), _p(x), _p(w_nk), _p(bias), *[_p(v) for v in vs], _p(od),
+       _p(idm), _p(wd), _p(bd), C.c_uint64(N), C.c_int32(out_offset),
+       C.c_int32(in_offset), C.c_int32(bias_offset))
+    return out
+
+
+def matmul_i8(lhs, rhs, out_offset, lhs_offset, rhs_offset, outP,
+              fastmath=False):
+    lhs = _c(lhs, np.int8)
+    rhs = _c(rhs, np.int8)
+    M, K = lhs.shape
+    N = rhs.shape[1]
+    out = np.empty((M, N), np.int8)
+    od, ld, rd = _dims(M, N), _dims(M, K), _dims(K, N)
+    lib(fastmath).libjit_matmul_i8(
+        _p(out), _p(lhs), _p(rhs), _p(od), _p(ld), _p(rd),
+        C.c_int32(out_offset), C.c_int32(lhs_offset), C.c_int32(rhs_offset),
+        *[C.c_int32(int(v)) for v in outP])
+    return out
+
+
+def _conv_dims(g, filt):
+    od = _dims(g.N, g.OH, g.OW, g.OC)
+    idm = _dims(g.N, g.IH, g.IW, g.IC)
+    fd = _dims(*filt.shape)
+    bd = _dims(g.OC)
+    ks = _dims(g.KH, g.KW)
+    st = _dims(g.strideH, g.strideW)
+    # bottom / right pads are not read by the kernels; output dims carry them
+    pd = _dims(g.padT, g.padL, g.padT, g.padL)
+    dl = _dims(g.dilH, g.dilW)
+    return od, idm, fd, bd, ks, st, pd, dl
+
+
+def conv2d_i8(x, filt, bias, g, out_offset, in_offset, filter_offset,
+              bias_offset, biasP, outP, act=0, act_args=(), depth_unroll=None,
+              fastmath=False):
+    x = _c(x, np.int8)
+    filt = _c(filt, np.int8)
+    bias = np.ascontiguousarray(bias)
+    out = np.empty((g.N, g.OH, g.OW, g.OC), np.int8)
+    od, idm, fd, bd, ks, st, pd, dl = _conv_dims(g, filt)
+    if depth_unroll is None:  # LLVMIRGen.cpp:2527-2538
+        depth_unroll = 8 if (g.OC // g.group) % 8 == 0 else 1
+    aa = _i32v(list(act_args) + [0, 0, 0])
+    fn = (lib(fastmath).libjit_conv2d_i8_i8 if bias.dtype == np.int8
+          else lib(fastmath).libjit_conv2d_i8_i32)
+    fn(_p(out), _p(x), _p(filt), _p(bias), _p(od), _p(idm), _p(fd), _p(bd),
+       _p(ks), _p(st), _p(pd), C.c_uint64(g.group), C.c_int32(out_offset),
+       C.c_int32(in_offset), C.c_int32(filter_offset), C.c_int32(bias_offset),
+       *[C.c_int32(int(v)) for v in biasP], *[C.c_int32(int(v)) for v in outP],
+       C.c_uint(depth_unroll), _p(dl), C.c_int32(act), _p(aa))
+    return out
+
+
+def cwq_conv2d_i8(x, filt, bias, g, out_offset, in_offset, filter_offsets,
+                  bias_offsets, bias_pre, bias_post, bias_scale, out_pre,
+                  out_post, out_scale, act=0, act_args=(), fastmath=False):
+    x = _c(x, np.int8)
+    filt = _c(filt, np.int8)
+    bias = np.ascontiguousarray(bias)
+    out = np.empty((g.N, g.OH, g.OW, g.OC), np.int8)
+    od, idm, fd, bd, ks, st, pd, dl = _conv_dims(g, filt)
+    vs = [_i32v(v) for v in (filter_offsets, bias_offsets, bias_pre, bias_post,
+                             bias_scale, out_pre, out_post, out_scale)]
+    aa = _i32v(list(act_args) + [0, 0, 0])
+    fn = (lib(fastmath).libjit_channelwise_quantized_conv2d_i8_i8
+          if bias.dtype == np.int8
+          else lib(fastmath).libjit_channelwise_quantized_conv2d_i8_i32)
+    fn(_p(out), _p(x), _p(filt), _p(bias), _p(od), _p(idm), _p(fd), _p(bd),
+       _p(ks), _p(st), _p(pd), C.c_uint64(g.group), _p(dl),
+       C.c_int32(out_offset), C.c_int32(in_offset), *[_p(v) for v in vs],
+       C.c_int32(act), _p(aa))
+    return out
+
+
+def frwq_slws_f32(data, weights, indices, lengths, out_cols=None,
+                  fastmath=False):
+    data = _c(data, np.uint8)
+    weights = _c(weights, np.float32)
+    indices = np.ascontiguousarray(indices)
+    lengths = _i32v(lengths)
+    in_line = data.shape[1]
+    out_line = in_line - 8 if out_cols is None else out_cols
+    out = np.empty((lengths.size, out_line), np.float32)
+    if indices.dtype == np.int64:
+        fn = lib(fastmath).libjit_fused_rowwise_quantized_sparse_lengths_weighted_sum_f_u
+    else:
+        indices = _c(indices, np.int32)
+        fn = lib(fastmath).libjit_fused_rowwise_quantized_sparse_lengths_weighted_sum_f_i32
+    fn(_p(out), _p(data), _p(weights), _p(indices), _p(lengths),
+       C.c_uint64(lengths.size), C.c_uint64(in_line), C.c_uint64(out_line))
+    return out
+
+
+def embedding_bag_byte_rowwise_offsets_f32(data, weights, indices, offsets,
+                                           has_end_offset, fastmath=False):
+    data = _c(data, np.uint8)
+    weights = _c(weights, np.float32)
+    indices = _i32v(indices)
+    offsets = _i32v(offsets)
+    in_line = data.shape[1]
+    out_line = in_line - 8
+    segs = offsets.size
+    out = np.empty((segs - (1 if has_end_offset else 0), out_line), np.float32)
+    lib(fastmath).libjit_embedding_bag_byte_rowwise_offsets_f(
+        _p(out), _p(data), _p(weights), _p(indices), _p(offsets),
+        C.c_uint64(segs), C.c_uint64(indices.size), C.c_uint64(in_line),
+        C.c_uint64(out_line), C.c_bool(has_end_offset))
+    return out

@@ -1,0 +1,119 @@
+"""Writes the golden vectors under tests/golden/*.npz.
+
+Run in the authoring container (where the reference tree is mounted and
+oracle/Makefile has built oracle/_ref from the reference's unmodified libjit
+sources):   python tests/golden/make_golden.py
+
+Each file holds the seeded inputs, the derived integer parameters and the
+outputs the REFERENCE's compiled kernels produced for them. The fixtures are
+data only; they let the oracle and the HIP kernels be checked where the
+reference is absent (the GPU box)."""
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
+
+from oracle import glow_oracle as go  # noqa: E402
+from oracle import libjit_ref as ref  # noqa: E402
+from tests import cases  # noqa: E402
+
+
+def geom_vec(g):
+    return np.array([getattr(g, n) for n, _ in g._fields_], np.int32)
+
+
+def save(name, **kw):
+    path = os.path.join(HERE, name + ".npz")
+    np.savez_compressed(path, **kw)
+    print(name, os.path.getsize(path), "bytes")
+
+
+def main():
+    assert ref.available(), "build oracle/_ref first (make -C oracle)"
+
+    # elementwise
+    rng = np.random.default_rng(100)
+    x = np.concatenate([rng.normal(0, 3, 2000),
+                        (np.arange(-200, 200) + 0.5) * 0.25]).astype(np.float32)
+    q = np.arange(-128, 128).astype(np.int8)
+    el = dict(x=x, q=q)
+    for i, (s, o) in enumerate([(0.25, 4), (0.05, -7), (0.0173, 33)]):
+        el[f"quant{i}_params"] = np.array([s, o], np.float64)
+        el[f"quant{i}_out"] = ref.quantize_i8(x, s, o)
+        el[f"dequant{i}_out"] = ref.dequantize_i8(q, s, o)
+    for i, (r, io, oo) in enumerate([(0.0123, -5, 7), (0.5, 0, -128), (1.7, 20, -3),
+                                     (2.0, 1, 1)]):
+        pre, post, sc, _ = go.quantize_scale_offset_32to8(r, 0)
+        el[f"rescale{i}_params"] = np.array([oo, io, pre, post, sc], np.int32)
+        el[f"rescale{i}_out"] = ref.rescale_i8(q, oo, io, pre, post, sc)
+    save("elementwise", **el)
+
+    # RowwiseQuantizedFullyConnected
+    fc = {}
+    for tag, (M, K, N), kw in [
+            ("sym", (9, 70, 20), dict()),
+            ("asym", (16, 128, 48), dict(symmetric=False)),
+            ("bias8", (5, 33, 7), dict(symmetric=False, bias_i8=True,
+                                       bias_scale=0.01, bias_offset=3))]:
+        c = cases.rwq_fc_case(200, M, K, N, **kw)
+        for k, v in c.items():
+            fc[f"{tag}_{k}"] = np.asarray(v)
+        fc[f"{tag}_out"] = ref.rwq_fc_i8(*cases.rwq_fc_args(c))
+    save("rwq_fc", **fc)
+
+    # plain FullyConnected + MatMul
+    pf = {}
+    for tag, shape, b8 in [("i32", (6, 50, 12), False), ("i8", (3, 21, 5), True)]:
+        c = cases.fc_case(300, *shape, bias_i8=b8)
+        for k, v in c.items():
+            pf[f"{tag}_{k}"] = np.asarray(v)
+        pf[f"{tag}_out"] = ref.fc_i8(*cases.fc_args(c))
+        pf[f"{tag}_matmul_out"] = ref.matmul_i8(
+            c["x"], c["w"], c["out_offset"], c["in_offset"], c["w_offset"], c["outP"])
+    save("fc", **pf)
+
+    # ChannelwiseQuantizedConvolution
+    cv = {}
+    for tag, kw in [
+            ("relu3x3", dict(N=2, H=8, W=8, IC=16, OC=16)),
+            ("stride2", dict(N=1, H=9, W=9, IC=8, OC=4, stride=(2, 2), pads=(0, 1, 2, 1))),
+            ("group_dil", dict(N=1, H=8, W=6, IC=8, OC=8, group=2, dilation=(2, 1),
+                               kernel=(2, 3), act=go.ACT_NONE, symmetric=False,
+                               in_offset=-9, out_offset=5)),
+            ("clip5x5", dict(N=1, H=5, W=5, IC=3, OC=5, kernel=(5, 5),
+                             pads=(2, 2, 2, 2), act=go.ACT_CLIP)),
+            ("leaky_b8", dict(N=1, H=6, W=7, IC=4, OC=8, act=go.ACT_LEAKY_RELU,
+                              out_offset=10, bias_i8=True))]:
+        c = cases.cwq_conv_case(400, **kw)
+        for k, v in c.items():
+            if k == "geom":
+                cv[f"{tag}_geom"] = geom_vec(v)
+            else:
+                cv[f"{tag}_{k}"] = np.asarray(v, dtype=np.int32 if k == "act_args" else None)
+        cv[f"{tag}_out"] = ref.cwq_conv2d_i8(*cases.cwq_conv_args(c))
+    save("cwq_conv", **cv)
+
+    # FusedRowwiseQuantizedSparseLengthsWeightedSum (8-bit, fp32)
+    sl = {}
+    rng = np.random.default_rng(500)
+    for tag, (rows, cols, bags, mean), idt in [
+            ("d128", (400, 128, 24, 40), np.int64),
+            ("d37", (100, 37, 12, 6), np.int32)]:
+        table = cases.random_fused_table(rng, rows, cols)
+        lengths, idx, w = cases.slws_batch(501, rows, bags, mean, 1.05, idt)
+        lengths[3] = 0  # an empty bag
+        total = int(lengths.sum())
+        idx, w = idx[:total], w[:total]
+        sl[f"{tag}_table"] = table
+        sl[f"{tag}_lengths"] = lengths
+        sl[f"{tag}_indices"] = idx
+        sl[f"{tag}_weights"] = w
+        sl[f"{tag}_out"] = ref.frwq_slws_f32(table, w, idx, lengths)
+    save("frwq_slws", **sl)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,65 @@
+"""Reads the committed golden vectors (tests/golden/*.npz, written by
+tests/golden/make_golden.py from the reference's compiled libjit) back into
+the argument tuples the oracle wrappers and the HIP wrappers share."""
+import os
+
+import numpy as np
+
+from oracle import glow_oracle as go
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _load(name):
+    with np.load(os.path.join(GOLDEN, name + ".npz")) as z:
+        return {k: z[k] for k in z.files}
+
+
+def _tags(d, suffix="_out"):
+    return sorted({k[:-len(suffix)] for k in d if k.endswith(suffix)
+                   and "matmul" not in k})
+
+
+def elementwise():
+    return _load("elementwise")
+
+
+def rwq_fc_cases():
+    d = _load("rwq_fc")
+    for t in _tags(d):
+        g = lambda k: d[f"{t}_{k}"]
+        args = (g("x"), g("w"), g("bias"), g("w_offsets"), g("bias_pre"),
+                g("bias_post"), g("bias_scale"), g("out_pre"), g("out_post"),
+                g("out_scale"), int(g("out_offset")), int(g("in_offset")),
+                int(g("bias_offset")))
+        yield t, args, g("out")
+
+
+def fc_cases():
+    d = _load("fc")
+    for t in _tags(d):
+        g = lambda k: d[f"{t}_{k}"]
+        args = (g("x"), g("w"), g("bias"), int(g("out_offset")),
+                int(g("in_offset")), int(g("w_offset")), int(g("bias_offset")),
+                tuple(int(v) for v in g("biasP")), tuple(int(v) for v in g("outP")))
+        yield t, args, g("out"), g("matmul_out")
+
+
+def cwq_conv_cases():
+    d = _load("cwq_conv")
+    for t in _tags(d):
+        g = lambda k: d[f"{t}_{k}"]
+        geom = go.ConvGeom(*[int(v) for v in g("geom")])
+        args = (g("x"), g("filt"), g("bias"), geom, int(g("out_offset")),
+                int(g("in_offset")), g("f_offsets"), g("b_offsets"),
+                g("bias_pre"), g("bias_post"), g("bias_scale"), g("out_pre"),
+                g("out_post"), g("out_scale"), int(g("act")),
+                tuple(int(v) for v in g("act_args")))
+        yield t, args, g("out")
+
+
+def slws_cases():
+    d = _load("frwq_slws")
+    for t in _tags(d):
+        g = lambda k: d[f"{t}_{k}"]
+        yield t, (g("table"), g("weights"), g("indices"), g("lengths")), g("out")

@@ -1,0 +1,61 @@
+"""The CPU oracle reproduces every committed golden vector (outputs of the
+reference's compiled libjit kernels) bit for bit. CPU only; runs where the
+reference tree is absent."""
+import numpy as np
+
+from oracle import glow_oracle as go
+from tests import golden_io as gio
+
+
+def test_elementwise_golden():
+    d = gio.elementwise()
+    i = 0
+    while f"quant{i}_params" in d:
+        s, o = d[f"quant{i}_params"]
+        np.testing.assert_array_equal(go.quantize_i8(d["x"], float(s), int(o)),
+                                      d[f"quant{i}_out"])
+        np.testing.assert_array_equal(go.dequantize_i8(d["q"], float(s), int(o)),
+                                      d[f"dequant{i}_out"])
+        i += 1
+    assert i == 3
+    i = 0
+    while f"rescale{i}_params" in d:
+        oo, io, pre, post, sc = (int(v) for v in d[f"rescale{i}_params"])
+        np.testing.assert_array_equal(
+            go.rescale_i8(d["q"], oo, io, pre, post, sc), d[f"rescale{i}_out"])
+        i += 1
+    assert i == 4
+
+
+def test_rwq_fc_golden():
+    n = 0
+    for _, args, want in gio.rwq_fc_cases():
+        np.testing.assert_array_equal(go.rwq_fc_i8(*args), want)
+        n += 1
+    assert n == 3
+
+
+def test_fc_golden():
+    n = 0
+    for _, args, want, mm in gio.fc_cases():
+        np.testing.assert_array_equal(go.fc_i8(*args), want)
+        x, w, _, oo, io, wo, _, _, outP = args
+        np.testing.assert_array_equal(go.matmul_i8(x, w, oo, io, wo, outP), mm)
+        n += 1
+    assert n == 2
+
+
+def test_cwq_conv_golden():
+    n = 0
+    for _, args, want in gio.cwq_conv_cases():
+        np.testing.assert_array_equal(go.cwq_conv2d_i8(*args), want)
+        n += 1
+    assert n == 5
+
+
+def test_slws_golden():
+    n = 0
+    for _, (table, w, idx, lens), want in gio.slws_cases():
+        np.testing.assert_array_equal(go.frwq_slws_f32(table, w, idx, lens), want)
+        n += 1
+    assert n == 2

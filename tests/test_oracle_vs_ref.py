@@ -1,0 +1,153 @@
+"""Validates the restatement in oracle/glow_oracle.c against the reference's
+own libjit sources compiled unmodified into oracle/_ref (plain and with the
+reference's default fast-math flags). Skipped where oracle/_ref was not built
+(the reference tree is only mounted in the authoring container). CPU only."""
+import numpy as np
+import pytest
+
+from oracle import glow_oracle as go
+from oracle import libjit_ref as ref
+from tests import cases
+
+pytestmark = pytest.mark.skipif(not ref.available(),
+                                reason="oracle/_ref not built (no reference tree)")
+
+FM = [False, True]
+
+
+@pytest.mark.parametrize("fastmath", FM)
+def test_rescale_exhaustive_int8(fastmath):
+    q = np.arange(-128, 128).astype(np.int8)
+    rng = np.random.default_rng(0)
+    ratios = [0.0003, 0.004, 0.05, 0.3, 0.5, 0.9, 1.0, 1.7, 2.0, 3.3, 8.0]
+    for r in ratios:
+        pre, post, sc, _ = go.quantize_scale_offset_32to8(r, 0)
+        for _ in range(3):
+            io, oo = int(rng.integers(-128, 128)), int(rng.integers(-128, 128))
+            np.testing.assert_array_equal(
+                go.rescale_i8(q, oo, io, pre, post, sc),
+                ref.rescale_i8(q, oo, io, pre, post, sc, fastmath))
+
+
+def test_quantize_dequantize_vs_ref():
+    rng = np.random.default_rng(1)
+    x = np.concatenate([rng.normal(0, 3, 3000),
+                        (np.arange(-300, 300) + 0.5) * 0.25,  # exact ties
+                        [0.0, -0.0, 1e-30, 31.875, -32.0, 1e4, -1e4]]).astype(np.float32)
+    for scale, off in [(0.25, 4), (0.05, -7), (0.1, 0), (1.0, -128), (0.0173, 33)]:
+        np.testing.assert_array_equal(go.quantize_i8(x, scale, off),
+                                      ref.quantize_i8(x, scale, off))
+        # fast-math may turn x/scale into x*(1/scale): at most 1 LSB, and only
+        # next to rounding ties
+        d = (go.quantize_i8(x, scale, off).astype(int) -
+             ref.quantize_i8(x, scale, off, True).astype(int))
+        assert np.max(np.abs(d)) <= 1
+    q = np.arange(-128, 128).astype(np.int8)
+    for scale, off in [(0.25, 4), (0.0371, -100), (3.0, 127)]:
+        for fm in FM:
+            np.testing.assert_array_equal(go.dequantize_i8(q, scale, off),
+                                          ref.dequantize_i8(q, scale, off, fm))
+
+
+@pytest.mark.parametrize("fastmath", FM)
+@pytest.mark.parametrize("shape", [(1, 1, 1), (3, 17, 5), (16, 64, 32), (33, 100, 7)])
+def test_rwq_fc_vs_ref(shape, fastmath):
+    M, K, N = shape
+    for seed, sym, b8 in [(1, True, False), (2, False, False), (3, False, True)]:
+        c = cases.rwq_fc_case(seed, M, K, N, symmetric=sym, bias_i8=b8,
+                              bias_scale=(0.01 if b8 else 5e-5),
+                              bias_offset=(3 if b8 else 0))
+        np.testing.assert_array_equal(
+            go.rwq_fc_i8(*cases.rwq_fc_args(c)),
+            ref.rwq_fc_i8(*cases.rwq_fc_args(c), fastmath=fastmath))
+
+
+def test_rwq_fc_config1_full_shape_vs_ref():
+    c = cases.rwq_fc_case(2024, 128, 1024, 1024)
+    got = go.rwq_fc_i8(*cases.rwq_fc_args(c))
+    np.testing.assert_array_equal(got, ref.rwq_fc_i8(*cases.rwq_fc_args(c)))
+    # the case is meaningful: outputs are neither all saturated nor all zero
+    assert 0.05 < np.mean(np.abs(got.astype(int)) < 127) and got.std() > 5
+
+
+@pytest.mark.parametrize("fastmath", FM)
+def test_fc_and_matmul_vs_ref(fastmath):
+    for seed, (M, K, N), b8 in [(1, (4, 9, 6), False), (2, (17, 40, 23), True),
+                                (3, (1, 128, 10), False)]:
+        c = cases.fc_case(seed, M, K, N, bias_i8=b8)
+        np.testing.assert_array_equal(go.fc_i8(*cases.fc_args(c)),
+                                      ref.fc_i8(*cases.fc_args(c), fastmath=fastmath))
+        np.testing.assert_array_equal(
+            go.matmul_i8(c["x"], c["w"], c["out_offset"], c["in_offset"],
+                         c["w_offset"], c["outP"]),
+            ref.matmul_i8(c["x"], c["w"], c["out_offset"], c["in_offset"],
+                          c["w_offset"], c["outP"], fastmath=fastmath))
+
+
+CONV_CASES = [
+    dict(N=2, H=7, W=6, IC=8, OC=16),
+    dict(N=1, H=9, W=9, IC=6, OC=4, kernel=(3, 3), stride=(2, 2), pads=(0, 1, 2, 1)),
+    dict(N=2, H=8, W=5, IC=8, OC=8, group=2, dilation=(2, 1), kernel=(2, 3)),
+    dict(N=1, H=5, W=5, IC=3, OC=5, kernel=(5, 5), pads=(2, 2, 2, 2), act=go.ACT_CLIP),
+    dict(N=1, H=6, W=6, IC=4, OC=4, kernel=(1, 1), pads=(0, 0, 0, 0), act=go.ACT_NONE,
+         symmetric=False, in_offset=-9, out_offset=5),
+    dict(N=1, H=6, W=7, IC=4, OC=8, act=go.ACT_LEAKY_RELU, out_offset=10, bias_i8=True),
+]
+
+
+@pytest.mark.parametrize("fastmath", FM)
+@pytest.mark.parametrize("kw", CONV_CASES)
+def test_cwq_conv_vs_ref(kw, fastmath):
+    c = cases.cwq_conv_case(7, **kw)
+    got = go.cwq_conv2d_i8(*cases.cwq_conv_args(c))
+    np.testing.assert_array_equal(
+        got, ref.cwq_conv2d_i8(*cases.cwq_conv_args(c), fastmath=fastmath))
+    # uniform-parameter convolution, with and without the depth-8 unrolling
+    oc = c["geom"].OC
+    args = (c["x"], c["filt"], c["bias"], c["geom"], c["out_offset"],
+            c["in_offset"], int(c["f_offsets"][0]), int(c["b_offsets"][0]),
+            (c["bias_pre"][0], c["bias_post"][0], c["bias_scale"][0]),
+            (c["out_pre"][0], c["out_post"][0], c["out_scale"][0]),
+            c["act"], c["act_args"])
+    u = go.conv2d_i8(*args)
+    np.testing.assert_array_equal(u, ref.conv2d_i8(*args, fastmath=fastmath))
+    np.testing.assert_array_equal(
+        u, ref.conv2d_i8(*args, depth_unroll=1, fastmath=fastmath))
+    assert oc == u.shape[-1]
+
+
+def test_cwq_conv_resnet_layer_shape_vs_ref():
+    # the ResNet-50 3x3x64->64 layer at batch 2 (batch 32 is the same loop nest)
+    c = cases.cwq_conv_case(11, 2, 56, 56, 64, 64)
+    got = go.cwq_conv2d_i8(*cases.cwq_conv_args(c))
+    np.testing.assert_array_equal(got, ref.cwq_conv2d_i8(*cases.cwq_conv_args(c)))
+    assert got.std() > 5 and np.mean(got == c["out_offset"]) > 0.1  # ReLU bites
+
+
+@pytest.mark.parametrize("idt", [np.int64, np.int32])
+def test_slws_vs_ref(idt):
+    rng = np.random.default_rng(3)
+    for rows, cols, bags, mean in [(50, 8, 20, 3), (1000, 128, 64, 40), (300, 37, 10, 12)]:
+        table = cases.random_fused_table(rng, rows, cols)
+        lengths, idx, w = cases.slws_batch(5, rows, bags, mean, 1.05, idt)
+        a = go.frwq_slws_f32(table, w, idx, lengths)
+        np.testing.assert_array_equal(a, ref.frwq_slws_f32(table, w, idx, lengths))
+        # the reference's default flags (fast-math, FMA where the host has it)
+        # stay within the 1e-5 relative tolerance of the restatement
+        b = ref.frwq_slws_f32(table, w, idx, lengths, fastmath=True)
+        np.testing.assert_allclose(b, a, rtol=1e-5, atol=1e-5 * np.abs(a).max())
+        # the Interpreter formula (q*scale+offset)*w is bit-identical here
+        np.testing.assert_array_equal(
+            a, go.frwq_slws_generic(table, go.U8_F32, w, idx, lengths))
+
+
+def test_embedding_bag_vs_ref():
+    rng = np.random.default_rng(4)
+    table = cases.random_fused_table(rng, 200, 16)
+    lengths, idx, w = cases.slws_batch(6, 200, 12, 5, 1.1, np.int32)
+    offs = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    for end in (True, False):
+        o = offs if end else offs[:-1]
+        np.testing.assert_array_equal(
+            go.embedding_bag_byte_rowwise_offsets_f32(table, w, idx, o, end),
+            ref.embedding_bag_byte_rowwise_offsets_f32(table, w, idx, o, end))
