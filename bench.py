@@ -1,0 +1,295 @@
+"""Benchmark of the MI355X quantized-inference hot path on ONE GPU.
+
+Headline workload (one step = one pass of the hot path over one batch):
+FusedRowwiseQuantizedSparseLengthsWeightedSum over a uint8 fused-rowwise table
+of 4M rows x 128 dims (fp32 scale and offset per row, 136-byte rows, 544 MB),
+4096 bags with Poisson(40) lengths, Zipf(1.05) int64 indices, fp32 weights
+U[0,1), fp32 output [4096 x 128]. Throughput is counted the way the
+reference's SLS benchmark counts bytes (tests/benchmark/CommonSLSEB.h:120-176:
+every lookup moves its row, scale and offset, index and weight; plus lengths
+and output; no credit for cache hits).
+
+Prints ONE JSON line. Besides the headline it reports, under "extra", the
+int8 matrix-core kernels (RowwiseQuantizedFullyConnected at the single-FC
+configuration and at a large shape, ChannelwiseQuantizedConvolution at the
+ResNet-50 3x3x64 layer shape) and the elementwise kernels, each with its own
+roofline fraction, and times the CPU oracle on this host's cores.
+
+  python bench.py --gpus 1 --steps 200 --warmup 20
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E, published
+INT8_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA, published (5.0 POP/s)
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--batches", type=int, default=8,
+                    help="distinct index batches cycled through by the steps")
+    ap.add_argument("--rows", type=int, default=4_000_000)
+    ap.add_argument("--cpu-seconds", type=float, default=12.0,
+                    help="wall-clock budget of the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true",
+                    help="headline workload only")
+    ap.add_argument("--only", default="",
+                    help="run a single extra kernel (profiling aid): "
+                         "slws|fc_large|fc_c1|conv_c3|quantize|dequantize|rescale")
+    return ap.parse_args()
+
+
+def timed_launches(capi, fn, steps, warmup, stream=None):
+    """Average seconds per launch: HIP events around `steps` launches on the
+    stream they are issued on, device idle before and after."""
+    for i in range(warmup):
+        fn(i)
+    capi.sync()
+    e0, e1 = capi.Event(), capi.Event()
+    e0.record(stream)
+    for i in range(steps):
+        fn(warmup + i)
+    e1.record(stream)
+    e1.sync()
+    capi.sync()
+    return e0.elapsed_ms(e1) * 1e-3 / steps
+
+
+def slws_bytes(total_lookups, bags, cols, row_bytes):
+    """Algorithmic bytes of one launch (reference CommonSLSEB.h:120-176)."""
+    return total_lookups * (row_bytes + 8 + 4) + bags * 4 + bags * cols * 4
+
+
+def bench_slws(capi, cases, args, table, d_table):
+    rows, cols, bags = args.rows, 128, 4096
+    row_bytes = cols + 8
+    batches = []
+    for b in range(args.batches):
+        lengths, idx, w = cases.slws_batch(1000 + b, rows, bags, 40, 1.05, np.int64)
+        batches.append(dict(
+            lengths=lengths, idx=idx, w=w, total=int(lengths.sum()),
+            d_len=capi.to_device(lengths), d_idx=capi.to_device(idx),
+            d_w=capi.to_device(w)))
+    d_out = capi.DeviceBuffer.empty((bags, cols), np.float32)
+
+    def step(i):
+        b = batches[i % len(batches)]
+        capi.launch_frwq_slws(d_out, False, d_table, rows, capi.FUSED_U8_F32,
+                              b["d_w"], False, b["d_idx"], True, b["total"],
+                              b["d_len"], bags, row_bytes, cols)
+
+    sec = timed_launches(capi, step, args.steps, args.warmup)
+    mean_total = float(np.mean([batches[(args.warmup + i) % len(batches)]["total"]
+                                for i in range(args.steps)]))
+    nbytes = slws_bytes(mean_total, bags, cols, row_bytes)
+    return dict(sec=sec, bytes=nbytes, batches=batches, mean_lookups=mean_total,
+                d_out=d_out)
+
+
+def cpu_baseline_slws(table, batches, budget_s, gpu_out, gpu_batch):
+    """The CPU leg: the oracle (the restated libjit loop, one thread) over
+    whole batches of the same workload until the time budget is used. As the
+    checker it also confirms the GPU output of the last timed step."""
+    from oracle import glow_oracle as go
+    want = go.frwq_slws_f32(table, gpu_batch["w"], gpu_batch["idx"],
+                            gpu_batch["lengths"])
+    parity = bool(np.array_equal(gpu_out, want))
+    done_bytes, n = 0.0, 0
+    t0 = time.perf_counter()
+    while True:
+        b = batches[n % len(batches)]
+        go.frwq_slws_f32(table, b["w"], b["idx"], b["lengths"])
+        done_bytes += slws_bytes(b["total"], 4096, 128, 136)
+        n += 1
+        el = time.perf_counter() - t0
+        if el >= budget_s or n >= 4000:
+            break
+    return dict(value=done_bytes / el / 1e9, unit="GB/s", cores=1, kind="port",
+                sample=f"{n} full batches of 4096 bags (single thread, "
+                       f"{el:.1f} s) of the same table and index batches"), parity
+
+
+def bench_fc(capi, cases, M, K, N, steps, warmup, seed=5):
+    c = cases.rwq_fc_case(seed, M, K, N) if M * K <= (1 << 24) else None
+    rng = np.random.default_rng(seed)
+    if c is None:
+        # large shape: same distributions, parameters from a small case
+        small = cases.rwq_fc_case(seed, 8, 64, N)
+        c = dict(small)
+        c["x"] = np.clip(np.rint(rng.normal(0, 40, (M, K))), -128, 127).astype(np.int8)
+        c["w"] = rng.integers(-127, 128, (N, K)).astype(np.int8)
+    d = {k: capi.to_device(np.ascontiguousarray(v)) for k, v in c.items()
+         if isinstance(v, np.ndarray)}
+    d_out = capi.DeviceBuffer.empty((M, N), np.int8)
+
+    def step(_):
+        capi.launch_rwq_fc_i8(d_out, d["x"], d["w"], d["bias"], False,
+                              d["w_offsets"], d["bias_pre"], d["bias_post"],
+                              d["bias_scale"], d["out_pre"], d["out_post"],
+                              d["out_scale"], M, K, N, c["out_offset"],
+                              c["in_offset"], c["bias_offset"], True)
+
+    sec = timed_launches(capi, step, steps, warmup)
+    ops = 2.0 * M * N * K
+    return dict(workload=f"rwq_fc M{M} K{K} N{N}", ms=sec * 1e3,
+                tops=ops / sec / 1e12,
+                roofline=dict(bound="mfma", achieved=ops / sec / 1e12,
+                              peak=INT8_PEAK_TOPS, unit="TOP/s",
+                              frac=ops / sec / 1e12 / INT8_PEAK_TOPS,
+                              traffic=None),
+                gbps=(M * K + N * K + M * N + 8 * 4 * N) / sec / 1e9)
+
+
+def bench_conv(capi, cases, steps, warmup):
+    c = cases.cwq_conv_case(7, 32, 56, 56, 64, 64, in_offset=-128)
+    g = capi._geom(c["geom"])
+    d = {k: capi.to_device(np.ascontiguousarray(v)) for k, v in c.items()
+         if isinstance(v, np.ndarray)}
+    d_out = capi.DeviceBuffer.empty((g.N, g.OH, g.OW, g.OC), np.int8)
+
+    def step(_):
+        capi.launch_cwq_conv2d_i8(d_out, d["x"], d["filt"], d["bias"], False, g,
+                                  c["out_offset"], c["in_offset"],
+                                  d["f_offsets"], d["b_offsets"], d["bias_pre"],
+                                  d["bias_post"], d["bias_scale"], d["out_pre"],
+                                  d["out_post"], d["out_scale"], c["act"],
+                                  c["act_args"], True)
+
+    sec = timed_launches(capi, step, steps, warmup)
+    ops = 2.0 * g.N * g.OH * g.OW * g.OC * g.KH * g.KW * g.IC
+    nbytes = c["x"].size + d_out.nbytes + c["filt"].size + 9 * 4 * g.OC
+    return dict(workload="cwq_conv2d 32x56x56x64 3x3x64->64 s1 p1 relu",
+                ms=sec * 1e3, tops=ops / sec / 1e12, gbps=nbytes / sec / 1e9,
+                roofline=dict(bound="mfma", achieved=ops / sec / 1e12,
+                              peak=INT8_PEAK_TOPS, unit="TOP/s",
+                              frac=ops / sec / 1e12 / INT8_PEAK_TOPS,
+                              traffic=None))
+
+
+def bench_elementwise(capi, which, steps, warmup):
+    n = 64 * 56 * 56 * 64 * 4  # four ResNet stem activations: 51.4M elements
+    rng = np.random.default_rng(3)
+    if which == "quantize":
+        src = capi.to_device(rng.normal(0, 1, n).astype(np.float32))
+        dst = capi.DeviceBuffer.empty((n,), np.int8)
+        fn = lambda _: capi.launch_quantize_i8(dst, src, n, 0.02, -3)
+        nbytes = n * 5
+    elif which == "dequantize":
+        src = capi.to_device(rng.integers(-128, 128, n).astype(np.int8))
+        dst = capi.DeviceBuffer.empty((n,), np.float32)
+        fn = lambda _: capi.launch_dequantize_i8(dst, src, n, 0.02, -3)
+        nbytes = n * 5
+    else:
+        src = capi.to_device(rng.integers(-128, 128, n).astype(np.int8))
+        dst = capi.DeviceBuffer.empty((n,), np.int8)
+        fn = lambda _: capi.launch_rescale_i8(dst, src, n, 3, -5, 2, 15, 300)
+        nbytes = n * 2
+    sec = timed_launches(capi, fn, steps, warmup)
+    return dict(workload=f"{which}_i8 n={n}", ms=sec * 1e3,
+                gbps=nbytes / sec / 1e9,
+                roofline=dict(bound="hbm", achieved=nbytes / sec / 1e9,
+                              peak=HBM_PEAK_GBPS, unit="GB/s",
+                              frac=nbytes / sec / 1e9 / HBM_PEAK_GBPS,
+                              traffic=None))
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one MI355X; multi-GPU runs are not part of "
+              "this build (the path shards by bags with no exchange). "
+              "Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    from glow_amd import capi
+    from glow_amd import workloads as cases
+
+    capi.init(0)
+    info = capi.device_info()
+    extra = {}
+    only = args.only
+
+    if only in ("fc_large", "fc_c1", "conv_c3", "quantize", "dequantize", "rescale"):
+        if only == "fc_large":
+            r = bench_fc(capi, cases, 8192, 4096, 4096, args.steps, args.warmup)
+        elif only == "fc_c1":
+            r = bench_fc(capi, cases, 128, 1024, 1024, args.steps, args.warmup)
+        elif only == "conv_c3":
+            r = bench_conv(capi, cases, args.steps, args.warmup)
+        else:
+            r = bench_elementwise(capi, only, args.steps, args.warmup)
+        print(json.dumps(r))
+        return
+
+    rng = np.random.default_rng(42)
+    table = cases.random_fused_table(rng, args.rows, 128)
+    d_table = capi.to_device(table)
+    s = bench_slws(capi, cases, args, table, d_table)
+    gbps = s["bytes"] / s["sec"] / 1e9
+
+    # CPU leg: baseline timing, and the check of the last timed step's output
+    last = s["batches"][(args.warmup + args.steps - 1) % len(s["batches"])]
+    cpu, parity = None, None
+    if not only:
+        cpu, parity = cpu_baseline_slws(table, s["batches"], args.cpu_seconds,
+                                        s["d_out"].numpy(), last)
+
+    if not args.no_extra and not only:
+        st, wu = max(20, args.steps // 4), max(3, args.warmup // 4)
+        extra["rwq_fc_c1"] = bench_fc(capi, cases, 128, 1024, 1024, args.steps, args.warmup)
+        extra["rwq_fc_large"] = bench_fc(capi, cases, 8192, 4096, 4096, st, wu)
+        extra["cwq_conv_c3"] = bench_conv(capi, cases, args.steps, args.warmup)
+        for w in ("quantize", "dequantize", "rescale"):
+            extra[w] = bench_elementwise(capi, w, st, wu)
+
+    out = {
+        "metric": "FusedRowwiseQuantizedSLWS algorithmic GB/s (1 GPU)",
+        "value": gbps,
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": s["sec"] * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u8->f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "FusedRowwiseQuantizedSparseLengthsWeightedSum, uint8 "
+                        f"fused-rowwise table {args.rows} x 128 (136-byte rows), "
+                        "4096 bags Poisson(40), Zipf(1.05) int64 indices, fp32 "
+                        "weights, fp32 out",
+            "index_batches_cycled": args.batches,
+            "mean_lookups_per_step": s["mean_lookups"],
+            "bytes_per_step": s["bytes"],
+            "device": info.name.decode(), "arch": info.arch.decode(),
+            "compute_units": info.compute_units,
+        },
+        "parity_with_oracle": parity,
+        "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
+                     "traffic": None,
+                     "kernel": "slws_kernel<64,2,false,false,false>"},
+        "cpu_baseline": cpu,
+        "extra": extra,
+    }
+    print(json.dumps(out))
+    if parity is False:
+        sys.exit(1)
+
+
+if __name__ == "__main__":
+    main()

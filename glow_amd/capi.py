@@ -1,0 +1,585 @@
+"""ctypes binding of libglow_mi355x.so (the C ABI in include/glow_mi355x.h)
+plus thin numpy conveniences used by the tests, the smoke check and the
+benchmark. There is no CPU fallback: if the library is missing or a call
+fails, an exception is raised."""
+import ctypes as C
+import os
+
+import numpy as np
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "libglow_mi355x.so")
+
+FUSED_U8_F32, FUSED_U8_F16, FUSED_U4_F16, FUSED_U4_F32 = 0, 1, 2, 3
+ACT_NONE, ACT_RELU, ACT_CLIP, ACT_TANH, ACT_SIGMOID, ACT_LEAKY_RELU = range(6)
+SCHEMA_ASYMMETRIC, SCHEMA_SYMMETRIC, SCHEMA_SYMMETRIC_WITH_UNSIGNED, \
+    SCHEMA_SYMMETRIC_POWER2 = range(4)
+QTY_INT8, QTY_INT16, QTY_INT32, QTY_UINT8 = 8, 16, 32, 108
+REGION_CONSTANTS, REGION_MUTABLE, REGION_ACTIVATIONS = 0, 1, 2
+
+# Every symbol include/glow_mi355x.h declares (checked by the CPU test suite).
+EXPORTS = [
+    "mi355x_last_error", "mi355x_num_devices", "mi355x_init",
+    "mi355x_device_info", "mi355x_malloc", "mi355x_free", "mi355x_host_alloc",
+    "mi355x_host_free", "mi355x_memcpy_h2d", "mi355x_memcpy_d2h",
+    "mi355x_memcpy_d2d", "mi355x_fill_u8", "mi355x_stream_create",
+    "mi355x_stream_destroy", "mi355x_stream_sync", "mi355x_device_sync",
+    "mi355x_event_create", "mi355x_event_destroy", "mi355x_event_record",
+    "mi355x_event_sync", "mi355x_event_elapsed_ms", "mi355x_arena_create",
+    "mi355x_arena_destroy", "mi355x_arena_ptr", "mi355x_arena_upload",
+    "mi355x_arena_download", "mi355x_arena_bytes",
+    "mi355x_quantize_scale_offset_32to8", "mi355x_choose_quantization_params",
+    "mi355x_fused_row_bytes", "mi355x_fused_rowwise_quantize_host",
+    "mi355x_rowwise_quantize_i8_host", "mi355x_quantize_i8",
+    "mi355x_dequantize_i8", "mi355x_rescale_i8", "mi355x_rwq_fc_i8",
+    "mi355x_fc_i8", "mi355x_matmul_i8", "mi355x_transpose2d_i8",
+    "mi355x_cwq_conv2d_i8", "mi355x_conv2d_i8", "mi355x_frwq_slws",
+    "mi355x_embedding_bag_rowwise_offsets",
+]
+
+
+class MI355XError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__(f"mi355x status {code}: {msg}")
+        self.code = code
+
+
+class Info(C.Structure):
+    _fields_ = [("name", C.c_char * 128), ("arch", C.c_char * 64),
+                ("compute_units", C.c_int32), ("clock_khz", C.c_int32),
+                ("total_memory", C.c_uint64), ("free_memory", C.c_uint64),
+                ("device", C.c_int32), ("lds_bytes_per_block", C.c_int32)]
+
+
+class ConvGeom(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in (
+        "N", "IH", "IW", "IC", "OH", "OW", "OC", "KH", "KW", "strideH",
+        "strideW", "padT", "padL", "dilH", "dilW", "group")]
+
+
+_lib = None
+
+
+def lib():
+    """The loaded library. Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise MI355XError(
+                -4, f"{LIB_PATH} is not built (run __graft_entry__.build())")
+        l = C.CDLL(LIB_PATH)
+        l.mi355x_last_error.restype = C.c_char_p
+        l.mi355x_fused_row_bytes.restype = C.c_size_t
+        l.mi355x_fused_row_bytes.argtypes = [C.c_size_t, C.c_int]
+        l.mi355x_arena_bytes.restype = C.c_uint64
+        l.mi355x_arena_bytes.argtypes = [C.c_void_p]
+        l.mi355x_quantize_scale_offset_32to8.restype = None
+        _lib = l
+    return _lib
+
+
+def check(rc):
+    if rc != 0:
+        raise MI355XError(rc, lib().mi355x_last_error().decode())
+
+
+def _vp(x):
+    """void* from a DeviceBuffer, an int address, a numpy array or None."""
+    if x is None:
+        return C.c_void_p(0)
+    if isinstance(x, DeviceBuffer):
+        return C.c_void_p(x.ptr)
+    if isinstance(x, np.ndarray):
+        return C.c_void_p(x.ctypes.data)
+    return C.c_void_p(int(x))
+
+
+def _sz(v):
+    return C.c_size_t(int(v))
+
+
+def _i32(v):
+    return C.c_int32(int(v))
+
+
+# ---- device / memory ---------------------------------------------------------
+
+_initialised = False
+
+
+def init(device=0):
+    global _initialised
+    check(lib().mi355x_init(C.c_int(device)))
+    _initialised = True
+
+
+def num_devices():
+    n = C.c_int(0)
+    rc = lib().mi355x_num_devices(C.byref(n))
+    return n.value if rc == 0 else 0
+
+
+def device_info():
+    info = Info()
+    check(lib().mi355x_device_info(C.byref(info)))
+    return info
+
+
+def sync():
+    check(lib().mi355x_device_sync())
+
+
+class DeviceBuffer:
+    """A device allocation that frees itself; `ptr` is the device address."""
+
+    def __init__(self, nbytes):
+        self.nbytes = int(nbytes)
+        p = C.c_void_p(0)
+        check(lib().mi355x_malloc(C.byref(p), _sz(max(self.nbytes, 1))))
+        self.ptr = p.value
+
+    @classmethod
+    def from_numpy(cls, a, stream=None):
+        a = np.ascontiguousarray(a)
+        b = cls(a.nbytes)
+        b.dtype, b.shape = a.dtype, a.shape
+        if a.nbytes:
+            check(lib().mi355x_memcpy_h2d(_vp(b.ptr), _vp(a), _sz(a.nbytes),
+                                          _vp(stream)))
+            check(lib().mi355x_stream_sync(_vp(stream)))
+        return b
+
+    @classmethod
+    def empty(cls, shape, dtype):
+        shape = tuple(int(s) for s in np.atleast_1d(shape))
+        b = cls(int(np.prod(shape)) * np.dtype(dtype).itemsize)
+        b.dtype, b.shape = np.dtype(dtype), shape
+        return b
+
+    def upload(self, a, stream=None):
+        a = np.ascontiguousarray(a)
+        assert a.nbytes <= self.nbytes
+        check(lib().mi355x_memcpy_h2d(_vp(self.ptr), _vp(a), _sz(a.nbytes),
+                                      _vp(stream)))
+        check(lib().mi355x_stream_sync(_vp(stream)))
+
+    def numpy(self, stream=None):
+        out = np.empty(self.shape, self.dtype)
+        if out.nbytes:
+            check(lib().mi355x_memcpy_d2h(_vp(out), _vp(self.ptr),
+                                          _sz(out.nbytes), _vp(stream)))
+        check(lib().mi355x_stream_sync(_vp(stream)))
+        return out
+
+    def fill(self, value, stream=None):
+        check(lib().mi355x_fill_u8(_vp(self.ptr), C.c_int(value),
+                                   _sz(self.nbytes), _vp(stream)))
+
+    def free(self):
+        if self.ptr:
+            lib().mi355x_free(_vp(self.ptr))
+            self.ptr = 0
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def to_device(a):
+    return DeviceBuffer.from_numpy(a)
+
+
+class Stream:
+    def __init__(self):
+        p = C.c_void_p(0)
+        check(lib().mi355x_stream_create(C.byref(p)))
+        self.ptr = p.value
+
+    def sync(self):
+        check(lib().mi355x_stream_sync(_vp(self.ptr)))
+
+    def __del__(self):
+        try:
+            if self.ptr:
+                lib().mi355x_stream_destroy(_vp(self.ptr))
+        except Exception:
+            pass
+
+
+class Event:
+    def __init__(self):
+        p = C.c_void_p(0)
+        check(lib().mi355x_event_create(C.byref(p)))
+        self.ptr = p.value
+
+    def record(self, stream=None):
+        check(lib().mi355x_event_record(_vp(self.ptr), _vp(stream)))
+
+    def sync(self):
+        check(lib().mi355x_event_sync(_vp(self.ptr)))
+
+    def elapsed_ms(self, later):
+        ms = C.c_float(0)
+        check(lib().mi355x_event_elapsed_ms(_vp(self.ptr), _vp(later.ptr),
+                                            C.byref(ms)))
+        return ms.value
+
+    def __del__(self):
+        try:
+            if self.ptr:
+                lib().mi355x_event_destroy(_vp(self.ptr))
+        except Exception:
+            pass
+
+
+class Arena:
+    """constants | mutable | activations in one HBM allocation."""
+
+    def __init__(self, const_bytes, mutable_bytes, activation_bytes):
+        p = C.c_void_p(0)
+        check(lib().mi355x_arena_create(_sz(const_bytes), _sz(mutable_bytes),
+                                        _sz(activation_bytes), C.byref(p)))
+        self.handle = p.value
+
+    def ptr(self, region, offset):
+        p = C.c_void_p(0)
+        check(lib().mi355x_arena_ptr(_vp(self.handle), C.c_int(region),
+                                     _sz(offset), C.byref(p)))
+        return p.value
+
+    def upload(self, region, offset, a, stream=None):
+        a = np.ascontiguousarray(a)
+        check(lib().mi355x_arena_upload(_vp(self.handle), C.c_int(region),
+                                        _sz(offset), _vp(a), _sz(a.nbytes),
+                                        _vp(stream)))
+        check(lib().mi355x_stream_sync(_vp(stream)))
+
+    def download(self, region, offset, shape, dtype, stream=None):
+        out = np.empty(shape, dtype)
+        check(lib().mi355x_arena_download(_vp(self.handle), C.c_int(region),
+                                          _sz(offset), _vp(out),
+                                          _sz(out.nbytes), _vp(stream)))
+        check(lib().mi355x_stream_sync(_vp(stream)))
+        return out
+
+    @property
+    def nbytes(self):
+        return lib().mi355x_arena_bytes(_vp(self.handle))
+
+    def destroy(self):
+        if self.handle:
+            check(lib().mi355x_arena_destroy(_vp(self.handle)))
+            self.handle = 0
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+# ---- host-side parameter derivation ------------------------------------------
+
+def quantize_scale_offset_32to8(scale, offset=0):
+    out = (C.c_int32 * 4)()
+    lib().mi355x_quantize_scale_offset_32to8(C.c_float(scale), _i32(offset), out)
+    return tuple(out)
+
+
+def choose_quantization_params(mn, mx, schema=SCHEMA_ASYMMETRIC, qty=QTY_INT8):
+    s = C.c_float()
+    o = C.c_int32()
+    check(lib().mi355x_choose_quantization_params(
+        C.c_float(mn), C.c_float(mx), C.c_int(schema), C.c_int(qty),
+        C.byref(s), C.byref(o)))
+    return s.value, o.value
+
+
+def fused_row_bytes(cols, kind):
+    return lib().mi355x_fused_row_bytes(cols, kind)
+
+
+def fused_rowwise_quantize_host(x, kind):
+    x = np.ascontiguousarray(x, np.float32)
+    rows, cols = x.shape
+    out = np.zeros((rows, fused_row_bytes(cols, kind)), np.uint8)
+    check(lib().mi355x_fused_rowwise_quantize_host(
+        _vp(x), _sz(rows), _sz(cols), C.c_int(kind), _vp(out)))
+    return out
+
+
+def rowwise_quantize_i8_host(w, schema=SCHEMA_SYMMETRIC):
+    w = np.ascontiguousarray(w, np.float32)
+    rows, cols = w.shape
+    q = np.empty((rows, cols), np.int8)
+    s = np.empty(rows, np.float32)
+    o = np.empty(rows, np.int32)
+    check(lib().mi355x_rowwise_quantize_i8_host(
+        _vp(w), _sz(rows), _sz(cols), C.c_int(schema), _vp(q), _vp(s), _vp(o)))
+    return q, s, o
+
+
+# ---- raw launches on device buffers (used by the benchmark) --------------------
+
+def launch_quantize_i8(dst, src, n, scale, offset, stream=None):
+    check(lib().mi355x_quantize_i8(_vp(dst), _vp(src), _sz(n), C.c_float(scale),
+                                   _i32(offset), _vp(stream)))
+
+
+def launch_dequantize_i8(dst, src, n, scale, offset, stream=None):
+    check(lib().mi355x_dequantize_i8(_vp(dst), _vp(src), _sz(n),
+                                     C.c_float(scale), _i32(offset),
+                                     _vp(stream)))
+
+
+def launch_rescale_i8(dst, src, n, out_offset, in_offset, pre, post, scale,
+                      stream=None):
+    check(lib().mi355x_rescale_i8(_vp(dst), _vp(src), _sz(n), _i32(out_offset),
+                                  _i32(in_offset), _i32(pre), _i32(post),
+                                  _i32(scale), _vp(stream)))
+
+
+def launch_rwq_fc_i8(out, x, w, bias, bias_is_i8, w_offsets, bias_pre,
+                     bias_post, bias_scale, out_pre, out_post, out_scale, M, K,
+                     N, out_offset, in_offset, bias_offset,
+                     w_offsets_all_zero=False, stream=None):
+    check(lib().mi355x_rwq_fc_i8(
+        _vp(out), _vp(x), _vp(w), _vp(bias), C.c_int(bias_is_i8),
+        _vp(w_offsets), _vp(bias_pre), _vp(bias_post), _vp(bias_scale),
+        _vp(out_pre), _vp(out_post), _vp(out_scale), _sz(M), _sz(K), _sz(N),
+        _i32(out_offset), _i32(in_offset), _i32(bias_offset),
+        C.c_int(bool(w_offsets_all_zero)), _vp(stream)))
+
+
+def launch_cwq_conv2d_i8(out, x, filt, bias, bias_is_i8, geom, out_offset,
+                         in_offset, f_offsets, b_offsets, bias_pre, bias_post,
+                         bias_scale, out_pre, out_post, out_scale, act,
+                         act_args, f_offsets_all_zero=False, stream=None):
+    aa = (C.c_int32 * 3)(*(list(act_args) + [0, 0, 0])[:3])
+    check(lib().mi355x_cwq_conv2d_i8(
+        _vp(out), _vp(x), _vp(filt), _vp(bias), C.c_int(bias_is_i8),
+        C.byref(geom), _i32(out_offset), _i32(in_offset), _vp(f_offsets),
+        _vp(b_offsets), _vp(bias_pre), _vp(bias_post), _vp(bias_scale),
+        _vp(out_pre), _vp(out_post), _vp(out_scale), _i32(act), aa,
+        C.c_int(bool(f_offsets_all_zero)), _vp(stream)))
+
+
+def launch_frwq_slws(dest, out_is_f16, data, data_rows, kind, weights,
+                     weights_are_f16, indices, idx_is_64, num_indices, lengths,
+                     segments, in_line, out_line, fp16_accum=False,
+                     stream=None):
+    check(lib().mi355x_frwq_slws(
+        _vp(dest), C.c_int(bool(out_is_f16)), _vp(data), _sz(data_rows),
+        C.c_int(kind), _vp(weights), C.c_int(bool(weights_are_f16)),
+        _vp(indices), C.c_int(bool(idx_is_64)), _sz(num_indices), _vp(lengths),
+        _sz(segments), _sz(in_line), _sz(out_line), C.c_int(bool(fp16_accum)),
+        _vp(stream)))
+
+
+# ---- numpy in / numpy out conveniences (tests, smoke) --------------------------
+
+def _geom(g):
+    """Accepts this module's ConvGeom or any ctypes struct with the same
+    fields (the oracle's)."""
+    if isinstance(g, ConvGeom):
+        return g
+    return ConvGeom(*[getattr(g, n) for n, _ in ConvGeom._fields_])
+
+
+def quantize_i8(x, scale, offset):
+    x = np.ascontiguousarray(x, np.float32)
+    d_in = to_device(x)
+    d_out = DeviceBuffer.empty(x.shape, np.int8)
+    launch_quantize_i8(d_out, d_in, x.size, scale, offset)
+    return d_out.numpy()
+
+
+def dequantize_i8(q, scale, offset):
+    q = np.ascontiguousarray(q, np.int8)
+    d_in = to_device(q)
+    d_out = DeviceBuffer.empty(q.shape, np.float32)
+    launch_dequantize_i8(d_out, d_in, q.size, scale, offset)
+    return d_out.numpy()
+
+
+def rescale_i8(q, out_offset, in_offset, pre, post, scale):
+    q = np.ascontiguousarray(q, np.int8)
+    d_in = to_device(q)
+    d_out = DeviceBuffer.empty(q.shape, np.int8)
+    launch_rescale_i8(d_out, d_in, q.size, out_offset, in_offset, pre, post,
+                      scale)
+    return d_out.numpy()
+
+
+def _dev_i32(v):
+    return to_device(np.ascontiguousarray(v, np.int32))
+
+
+def _bias_dev(bias):
+    bias = np.ascontiguousarray(bias)
+    if bias.dtype == np.int8:
+        return to_device(bias), 1
+    return to_device(bias.astype(np.int32)), 0
+
+
+def rwq_fc_i8(x, w_nk, bias, w_offsets, bias_pre, bias_post, bias_scale,
+              out_pre, out_post, out_scale, out_offset, in_offset, bias_offset,
+              w_offsets_all_zero=None):
+    x = np.ascontiguousarray(x, np.int8)
+    w_nk = np.ascontiguousarray(w_nk, np.int8)
+    M, K = x.shape
+    N = w_nk.shape[0]
+    if w_offsets_all_zero is None:
+        w_offsets_all_zero = not np.any(w_offsets)
+    d_x, d_w = to_device(x), to_device(w_nk)
+    d_b, b8 = _bias_dev(bias)
+    vs = [_dev_i32(v) for v in (w_offsets, bias_pre, bias_post, bias_scale,
+                                out_pre, out_post, out_scale)]
+    d_out = DeviceBuffer.empty((M, N), np.int8)
+    launch_rwq_fc_i8(d_out, d_x, d_w, d_b, b8, *vs, M, K, N, out_offset,
+                     in_offset, bias_offset, w_offsets_all_zero)
+    return d_out.numpy()
+
+
+def fc_i8(x, w_kn, bias, out_offset, in_offset, w_offset, bias_offset, biasP,
+          outP):
+    x = np.ascontiguousarray(x, np.int8)
+    w_kn = np.ascontiguousarray(w_kn, np.int8)
+    M, K = x.shape
+    N = w_kn.shape[1]
+    d_x, d_w = to_device(x), to_device(w_kn)
+    d_ws = DeviceBuffer.empty((N, K), np.int8)
+    d_b, b8 = _bias_dev(bias)
+    d_out = DeviceBuffer.empty((M, N), np.int8)
+    check(lib().mi355x_fc_i8(
+        _vp(d_out), _vp(d_x), _vp(d_w), _vp(d_ws), C.c_int(1), _vp(d_b),
+        C.c_int(b8), _sz(M), _sz(K), _sz(N), _i32(out_offset), _i32(in_offset),
+        _i32(w_offset), _i32(bias_offset), *[_i32(v) for v in biasP],
+        *[_i32(v) for v in outP], _vp(None)))
+    return d_out.numpy()
+
+
+def matmul_i8(lhs, rhs_kn, out_offset, lhs_offset, rhs_offset, outP):
+    lhs = np.ascontiguousarray(lhs, np.int8)
+    rhs_kn = np.ascontiguousarray(rhs_kn, np.int8)
+    M, K = lhs.shape
+    N = rhs_kn.shape[1]
+    d_l, d_r = to_device(lhs), to_device(rhs_kn)
+    d_ws = DeviceBuffer.empty((N, K), np.int8)
+    d_out = DeviceBuffer.empty((M, N), np.int8)
+    check(lib().mi355x_matmul_i8(
+        _vp(d_out), _vp(d_l), _vp(d_r), _vp(d_ws), C.c_int(1), _sz(M), _sz(K),
+        _sz(N), _i32(out_offset), _i32(lhs_offset), _i32(rhs_offset),
+        *[_i32(v) for v in outP], _vp(None)))
+    return d_out.numpy()
+
+
+def transpose2d_i8(a):
+    a = np.ascontiguousarray(a, np.int8)
+    d_a = to_device(a)
+    d_o = DeviceBuffer.empty((a.shape[1], a.shape[0]), np.int8)
+    check(lib().mi355x_transpose2d_i8(_vp(d_o), _vp(d_a), _sz(a.shape[0]),
+                                      _sz(a.shape[1]), _vp(None)))
+    return d_o.numpy()
+
+
+def cwq_conv2d_i8(x, filt, bias, geom, out_offset, in_offset, f_offsets,
+                  b_offsets, bias_pre, bias_post, bias_scale, out_pre, out_post,
+                  out_scale, act=ACT_NONE, act_args=(), f_offsets_all_zero=None):
+    g = _geom(geom)
+    x = np.ascontiguousarray(x, np.int8)
+    filt = np.ascontiguousarray(filt, np.int8)
+    if f_offsets_all_zero is None:
+        f_offsets_all_zero = not np.any(f_offsets)
+    d_x, d_f = to_device(x), to_device(filt)
+    d_b, b8 = _bias_dev(bias)
+    vs = [_dev_i32(v) for v in (f_offsets, b_offsets, bias_pre, bias_post,
+                                bias_scale, out_pre, out_post, out_scale)]
+    d_out = DeviceBuffer.empty((g.N, g.OH, g.OW, g.OC), np.int8)
+    launch_cwq_conv2d_i8(d_out, d_x, d_f, d_b, b8, g, out_offset, in_offset,
+                         *vs, act, act_args, f_offsets_all_zero)
+    return d_out.numpy()
+
+
+def conv2d_i8(x, filt, bias, geom, out_offset, in_offset, filter_offset,
+              bias_offset, biasP, outP, act=ACT_NONE, act_args=()):
+    g = _geom(geom)
+    x = np.ascontiguousarray(x, np.int8)
+    filt = np.ascontiguousarray(filt, np.int8)
+    d_x, d_f = to_device(x), to_device(filt)
+    d_b, b8 = _bias_dev(bias)
+    d_out = DeviceBuffer.empty((g.N, g.OH, g.OW, g.OC), np.int8)
+    aa = (C.c_int32 * 3)(*(list(act_args) + [0, 0, 0])[:3])
+    check(lib().mi355x_conv2d_i8(
+        _vp(d_out), _vp(d_x), _vp(d_f), _vp(d_b), C.c_int(b8), C.byref(g),
+        _i32(out_offset), _i32(in_offset), _i32(filter_offset),
+        _i32(bias_offset), *[_i32(v) for v in biasP], *[_i32(v) for v in outP],
+        _i32(act), aa, _vp(None)))
+    return d_out.numpy()
+
+
+def _fused_cols(in_line, kind):
+    so = 8 if kind in (FUSED_U8_F32, FUSED_U4_F32) else 4
+    return (in_line - so) * (2 if kind in (FUSED_U4_F16, FUSED_U4_F32) else 1)
+
+
+def frwq_slws(data, kind, weights, indices, lengths, out_f16=False,
+              fp16_accum=False, d_data=None):
+    """weights: None (plain SLS), float32 or float16 array. `d_data` lets a
+    caller reuse a table already resident on the device."""
+    data_shape = data.shape
+    in_line = data_shape[1]
+    out_line = _fused_cols(in_line, kind)
+    if d_data is None:
+        d_data = to_device(np.ascontiguousarray(data, np.uint8))
+    indices = np.ascontiguousarray(indices)
+    if indices.dtype != np.int64:
+        indices = indices.astype(np.int32)
+    lengths = np.ascontiguousarray(lengths, np.int32)
+    d_w, w16 = None, 0
+    if weights is not None:
+        weights = np.ascontiguousarray(weights)
+        if weights.dtype == np.float16:
+            w16 = 1
+        else:
+            weights = weights.astype(np.float32)
+        d_w = to_device(weights)
+    d_idx, d_len = to_device(indices), to_device(lengths)
+    d_out = DeviceBuffer.empty((lengths.size, out_line),
+                               np.float16 if out_f16 else np.float32)
+    d_out.fill(0xFF)  # poison: every row must be written by the kernel
+    launch_frwq_slws(d_out, out_f16, d_data, data_shape[0], kind, d_w, w16,
+                     d_idx, indices.dtype == np.int64, indices.size, d_len,
+                     lengths.size, in_line, out_line, fp16_accum)
+    return d_out.numpy()
+
+
+def embedding_bag_rowwise_offsets(data, kind, weights, indices, offsets,
+                                  has_end_offset, out_f16=False,
+                                  fp16_accum=False):
+    data = np.ascontiguousarray(data, np.uint8)
+    in_line = data.shape[1]
+    out_line = _fused_cols(in_line, kind)
+    indices = np.ascontiguousarray(indices, np.int32)
+    offsets = np.ascontiguousarray(offsets, np.int32)
+    d_w, w16 = None, 0
+    if weights is not None:
+        weights = np.ascontiguousarray(weights)
+        if weights.dtype == np.float16:
+            w16 = 1
+        else:
+            weights = weights.astype(np.float32)
+        d_w = to_device(weights)
+    d_data, d_idx, d_off = to_device(data), to_device(indices), to_device(offsets)
+    rows = offsets.size - (1 if has_end_offset else 0)
+    d_out = DeviceBuffer.empty((rows, out_line),
+                               np.float16 if out_f16 else np.float32)
+    d_out.fill(0xFF)
+    check(lib().mi355x_embedding_bag_rowwise_offsets(
+        _vp(d_out), C.c_int(bool(out_f16)), _vp(d_data), _sz(data.shape[0]),
+        C.c_int(kind), _vp(d_w), C.c_int(w16), _vp(d_idx), _sz(indices.size),
+        _vp(d_off), _sz(offsets.size), C.c_int(bool(has_end_offset)),
+        _sz(in_line), _sz(out_line), C.c_int(bool(fp16_accum)), _vp(None)))
+    return d_out.numpy()

@@ -1,0 +1,217 @@
+// Quantized and ChannelwiseQuantized 2-D convolution for int8 NHWC tensors as
+// an implicit GEMM on the int8 matrix cores (reference
+// lib/LLVMIRCodeGen/libjit/libjit_conv.cpp:49-239, 496-562).
+//
+// GEMM view per group: rows = output pixels (n, oh, ow), columns = output
+// channels of the group, K = (fx, fy, c) in the filter's own memory order
+// [OC][KH][KW][IC/group]. A-tile rows are gathered from the NHWC input on the
+// fly, 16 channel bytes at a time. The CPU loop skips taps that fall into the
+// padding; a tap whose bytes all equal the input offset contributes
+// (in - inOffset) = 0 just the same, so out-of-image taps are filled with the
+// input offset and the dense contraction of gemm_i8.h applies unchanged.
+#include "gemm_i8.h"
+
+namespace mi355x {
+
+struct ConvRows {
+  const int8_t *in;
+  int N, IH, IW, IC, OH, OW;
+  int KW, ICg;
+  int strideH, strideW, padT, padL, dilH, dilW;
+  int M;                 // N*OH*OW
+  int fill;              // input offset replicated into four bytes
+  int c_base;            // first input channel of the group
+
+  struct Row {
+    const int8_t *img;   // input image n, channel c_base
+    int ih0, iw0;
+    bool ok;
+  };
+  __device__ __forceinline__ void set_group(int g) { c_base = g * ICg; }
+  __device__ __forceinline__ Row row(int m) const {
+    Row r;
+    r.ok = m < M;
+    const int mm = r.ok ? m : 0;
+    const int n = mm / (OH * OW);
+    const int rem = mm - n * (OH * OW);
+    const int oh = rem / OW, ow = rem - oh * OW;
+    r.img = in + (long long)n * IH * IW * IC + c_base;
+    r.ih0 = oh * strideH - padT;
+    r.iw0 = ow * strideW - padL;
+    return r;
+  }
+  // 16 bytes A[m][k..k+15]; ALIGNED needs ICg % 16 == 0 so a chunk never
+  // straddles a tap, and 16-byte aligned pixels.
+  template <bool ALIGNED>
+  __device__ __forceinline__ int4 load(const Row &r, int k, int K) const {
+    if (!r.ok || k >= K) return make_int4(0, 0, 0, 0);
+    if constexpr (ALIGNED) {
+      const int tap = k / ICg, c = k - tap * ICg;
+      const int fx = tap / KW, fy = tap - fx * KW;
+      const int ih = r.ih0 + fx * dilH, iw = r.iw0 + fy * dilW;
+      if (ih < 0 || iw < 0 || ih >= IH || iw >= IW)
+        return make_int4(fill, fill, fill, fill);
+      return *reinterpret_cast<const int4 *>(
+          r.img + ((long long)ih * IW + iw) * IC + c);
+    } else {
+      uint32_t w[4] = {0, 0, 0, 0};
+      const int n = min(16, K - k);
+      for (int b = 0; b < n; b++) {
+        const int kk = k + b;
+        const int tap = kk / ICg, c = kk - tap * ICg;
+        const int fx = tap / KW, fy = tap - fx * KW;
+        const int ih = r.ih0 + fx * dilH, iw = r.iw0 + fy * dilW;
+        uint32_t v = (uint32_t)fill & 0xff;
+        if (ih >= 0 && iw >= 0 && ih < IH && iw < IW)
+          v = (uint8_t)r.img[((long long)ih * IW + iw) * IC + c];
+        w[b >> 2] |= v << (8 * (b & 3));
+      }
+      return make_int4((int)w[0], (int)w[1], (int)w[2], (int)w[3]);
+    }
+  }
+};
+
+static int conv_common(int8_t *out, const int8_t *in, const int8_t *filter,
+                       const mi355x_conv_geom *g, Epilogue ep, bool need_sa,
+                       void *stream) {
+  MI355X_REQUIRE(g, "geom is NULL");
+  MI355X_REQUIRE(g->N >= 0 && g->IH > 0 && g->IW > 0 && g->IC > 0 &&
+                     g->OH >= 0 && g->OW >= 0 && g->OC > 0 && g->KH > 0 &&
+                     g->KW > 0 && g->strideH > 0 && g->strideW > 0 &&
+                     g->dilH > 0 && g->dilW > 0 && g->group > 0 &&
+                     g->padT >= 0 && g->padL >= 0,
+                 "invalid convolution geometry");
+  MI355X_REQUIRE(g->IC % g->group == 0 && g->OC % g->group == 0,
+                 "channels not divisible by group");
+  const long long M = (long long)g->N * g->OH * g->OW;
+  if (M == 0) return MI355X_OK;
+  MI355X_REQUIRE(out && in && filter, "NULL tensor");
+  const int ICg = g->IC / g->group, OCg = g->OC / g->group;
+  const long long K = (long long)g->KH * g->KW * ICg;
+  MI355X_REQUIRE(M < (1LL << 30) && K < (1LL << 30), "convolution too large");
+  // the last tap of the last output pixel must start inside pad + image
+  MI355X_REQUIRE((long long)(g->OH - 1) * g->strideH - g->padT < g->IH &&
+                     (long long)(g->OW - 1) * g->strideW - g->padL < g->IW,
+                 "output size inconsistent with input size, stride and pads");
+  MI355X_REQUIRE(ep.a_off >= -128 && ep.a_off <= 127,
+                 "input offset %d outside the int8 range", ep.a_off);
+  MI355X_REQUIRE(ep.act == MI355X_ACT_NONE || ep.act == MI355X_ACT_RELU ||
+                     ep.act == MI355X_ACT_CLIP ||
+                     ep.act == MI355X_ACT_LEAKY_RELU,
+                 "fused activation %d is not supported for quantized types",
+                 ep.act);
+  if (ep.act == MI355X_ACT_LEAKY_RELU)
+    MI355X_REQUIRE(shift_ok(ep.a0) && shift_ok(ep.a1),
+                   "leaky-relu pre/post shift outside [0, 31]");
+
+  ConvRows A;
+  A.in = in;
+  A.N = g->N; A.IH = g->IH; A.IW = g->IW; A.IC = g->IC;
+  A.OH = g->OH; A.OW = g->OW;
+  A.KW = g->KW; A.ICg = ICg;
+  A.strideH = g->strideH; A.strideW = g->strideW;
+  A.padT = g->padT; A.padL = g->padL;
+  A.dilH = g->dilH; A.dilW = g->dilW;
+  A.M = (int)M;
+  A.fill = (int)(0x01010101u * (uint32_t)(uint8_t)(int8_t)ep.a_off);
+  A.c_base = 0;
+  DenseRows B{filter, K, OCg};
+  ep.out = out;
+  ep.ldc = g->OC;
+  const bool al_a = (ICg % 16 == 0) && (g->IC % 16 == 0) &&
+                    ((((uintptr_t)in) & 15) == 0);
+  const bool al_b = (K % 16 == 0) && ((((uintptr_t)filter) & 15) == 0);
+  const bool need_sb = ep.a_off != 0;
+  return gemm_dispatch(A, B, ep, (int)M, OCg, (int)K, g->group,
+                       (long long)OCg * K, need_sa, need_sb, al_a && al_b,
+                       al_a && al_b, as_stream(stream));
+}
+
+static void set_act(Epilogue &ep, int32_t act_type, const int32_t *act_args) {
+  ep.act = act_type;
+  ep.a0 = ep.a1 = ep.a2 = 0;
+  if (act_args) {
+    if (act_type == MI355X_ACT_CLIP) {
+      ep.a0 = act_args[0];
+      ep.a1 = act_args[1];
+    } else if (act_type == MI355X_ACT_LEAKY_RELU) {
+      ep.a0 = act_args[0];
+      ep.a1 = act_args[1];
+      ep.a2 = act_args[2];
+    }
+  }
+}
+
+} // namespace mi355x
+
+using namespace mi355x;
+
+extern "C" {
+
+int mi355x_cwq_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
+                         const void *bias, int bias_is_i8,
+                         const mi355x_conv_geom *geom, int32_t out_offset,
+                         int32_t in_offset, const int32_t *filter_offsets,
+                         const int32_t *bias_offsets, const int32_t *bias_pre,
+                         const int32_t *bias_post, const int32_t *bias_scale,
+                         const int32_t *out_pre, const int32_t *out_post,
+                         const int32_t *out_scale, int32_t act_type,
+                         const int32_t *act_args, int filter_offsets_all_zero,
+                         void *stream) {
+  MI355X_REQUIRE(bias && filter_offsets && bias_offsets && bias_pre &&
+                     bias_post && bias_scale && out_pre && out_post && out_scale,
+                 "NULL per-channel parameter vector");
+  MI355X_REQUIRE(act_args || (act_type != MI355X_ACT_CLIP &&
+                              act_type != MI355X_ACT_LEAKY_RELU),
+                 "act_args is NULL");
+  Epilogue ep{};
+  ep.bias = bias;
+  ep.bias_is_i8 = bias_is_i8;
+  ep.b_off = ColParam{bias_offsets, 0};
+  ep.bias_pre = ColParam{bias_pre, 0};
+  ep.bias_post = ColParam{bias_post, 0};
+  ep.bias_scale = ColParam{bias_scale, 0};
+  ep.w_off = ColParam{filter_offsets, 0};
+  ep.out_pre = ColParam{out_pre, 0};
+  ep.out_post = ColParam{out_post, 0};
+  ep.out_scale = ColParam{out_scale, 0};
+  ep.a_off = in_offset;
+  ep.out_off = out_offset;
+  set_act(ep, act_type, act_args);
+  return conv_common(out, in, filter, geom, ep, !filter_offsets_all_zero,
+                     stream);
+}
+
+int mi355x_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
+                     const void *bias, int bias_is_i8,
+                     const mi355x_conv_geom *geom, int32_t out_offset,
+                     int32_t in_offset, int32_t filter_offset,
+                     int32_t bias_offset, int32_t bias_pre, int32_t bias_post,
+                     int32_t bias_scale, int32_t out_pre, int32_t out_post,
+                     int32_t out_scale, int32_t act_type,
+                     const int32_t *act_args, void *stream) {
+  MI355X_REQUIRE(bias, "bias is NULL");
+  MI355X_REQUIRE(shift_ok(bias_pre) && shift_ok(bias_post) &&
+                     shift_ok(out_pre) && shift_ok(out_post),
+                 "pre/post shift outside [0, 31]");
+  MI355X_REQUIRE(act_args || (act_type != MI355X_ACT_CLIP &&
+                              act_type != MI355X_ACT_LEAKY_RELU),
+                 "act_args is NULL");
+  Epilogue ep{};
+  ep.bias = bias;
+  ep.bias_is_i8 = bias_is_i8;
+  ep.b_off = ColParam{nullptr, bias_offset};
+  ep.bias_pre = ColParam{nullptr, bias_pre};
+  ep.bias_post = ColParam{nullptr, bias_post};
+  ep.bias_scale = ColParam{nullptr, bias_scale};
+  ep.w_off = ColParam{nullptr, filter_offset};
+  ep.out_pre = ColParam{nullptr, out_pre};
+  ep.out_post = ColParam{nullptr, out_post};
+  ep.out_scale = ColParam{nullptr, out_scale};
+  ep.a_off = in_offset;
+  ep.out_off = out_offset;
+  set_act(ep, act_type, act_args);
+  return conv_common(out, in, filter, geom, ep, filter_offset != 0, stream);
+}
+
+} // extern "C"

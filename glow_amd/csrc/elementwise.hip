@@ -1,0 +1,164 @@
+// Quantize / Dequantize / RescaleQuantized for int8 tensors: the HBM-bound
+// elementwise instructions of the quantized path (reference
+// lib/LLVMIRCodeGen/libjit/libjit.cpp:2998-3038). Each lane moves 16 elements
+// per trip with 16-byte accesses on the int8 side and 4 x 16 bytes on the
+// fp32 side; tensors whose base is not 16-byte aligned, and the last n % 16
+// elements, go through the scalar tail.
+#include "common.h"
+#include "requant.h"
+
+namespace mi355x {
+
+constexpr int kEwThreads = 256;
+constexpr int kEwPerLane = 16;
+
+// clip((int32)nearbyintf(x / scale + offset)): IEEE division and
+// round-half-even, each operation rounded on its own.
+__device__ __forceinline__ int32_t quantize_one(float x, float scale,
+                                                float offset) {
+  float r = rintf(__fadd_rn(__fdiv_rn(x, scale), offset));
+  return clip_i8((int32_t)r);
+}
+
+__device__ __forceinline__ uint32_t pack4(int32_t a, int32_t b, int32_t c,
+                                          int32_t d) {
+  return (uint32_t)(a & 0xff) | ((uint32_t)(b & 0xff) << 8) |
+         ((uint32_t)(c & 0xff) << 16) | ((uint32_t)(d & 0xff) << 24);
+}
+
+__device__ __forceinline__ int32_t sext8(uint32_t w, int i) {
+  return (int32_t)(int8_t)(w >> (8 * i));
+}
+
+__global__ __launch_bounds__(kEwThreads) void quantize_i8_kernel(
+    int8_t *__restrict__ dst, const float *__restrict__ src, size_t n,
+    size_t vec_chunks, float scale, float offset) {
+  const size_t t = (size_t)blockIdx.x * kEwThreads + threadIdx.x;
+  if (t < vec_chunks) {
+    const float4 *s = reinterpret_cast<const float4 *>(src) + t * 4;
+    float4 a = s[0], b = s[1], c = s[2], d = s[3];
+    uint4 o;
+    o.x = pack4(quantize_one(a.x, scale, offset), quantize_one(a.y, scale, offset),
+                quantize_one(a.z, scale, offset), quantize_one(a.w, scale, offset));
+    o.y = pack4(quantize_one(b.x, scale, offset), quantize_one(b.y, scale, offset),
+                quantize_one(b.z, scale, offset), quantize_one(b.w, scale, offset));
+    o.z = pack4(quantize_one(c.x, scale, offset), quantize_one(c.y, scale, offset),
+                quantize_one(c.z, scale, offset), quantize_one(c.w, scale, offset));
+    o.w = pack4(quantize_one(d.x, scale, offset), quantize_one(d.y, scale, offset),
+                quantize_one(d.z, scale, offset), quantize_one(d.w, scale, offset));
+    reinterpret_cast<uint4 *>(dst)[t] = o;
+  }
+  // scalar tail: elements [vec_chunks*16, n), one per lane from the front
+  const size_t tail0 = vec_chunks * kEwPerLane;
+  const size_t stride = (size_t)gridDim.x * kEwThreads;
+  for (size_t i = tail0 + t; i < n; i += stride)
+    dst[i] = (int8_t)quantize_one(src[i], scale, offset);
+}
+
+__global__ __launch_bounds__(kEwThreads) void dequantize_i8_kernel(
+    float *__restrict__ dst, const int8_t *__restrict__ src, size_t n,
+    size_t vec_chunks, float scale, int32_t offset) {
+  const size_t t = (size_t)blockIdx.x * kEwThreads + threadIdx.x;
+  if (t < vec_chunks) {
+    uint4 q = reinterpret_cast<const uint4 *>(src)[t];
+    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+    float4 *d = reinterpret_cast<float4 *>(dst) + t * 4;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      float4 f;
+      f.x = __fmul_rn(scale, (float)(sext8(w[j], 0) - offset));
+      f.y = __fmul_rn(scale, (float)(sext8(w[j], 1) - offset));
+      f.z = __fmul_rn(scale, (float)(sext8(w[j], 2) - offset));
+      f.w = __fmul_rn(scale, (float)(sext8(w[j], 3) - offset));
+      d[j] = f;
+    }
+  }
+  const size_t tail0 = vec_chunks * kEwPerLane;
+  const size_t stride = (size_t)gridDim.x * kEwThreads;
+  for (size_t i = tail0 + t; i < n; i += stride)
+    dst[i] = __fmul_rn(scale, (float)((int32_t)src[i] - offset));
+}
+
+__global__ __launch_bounds__(kEwThreads) void rescale_i8_kernel(
+    int8_t *__restrict__ dst, const int8_t *__restrict__ src, size_t n,
+    size_t vec_chunks, int32_t out_offset, int32_t in_offset, int32_t pre,
+    int32_t post, int32_t scale) {
+  const size_t t = (size_t)blockIdx.x * kEwThreads + threadIdx.x;
+  if (t < vec_chunks) {
+    uint4 q = reinterpret_cast<const uint4 *>(src)[t];
+    uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      int32_t r[4];
+#pragma unroll
+      for (int b = 0; b < 4; b++)
+        r[b] = clip_i8(scale_i32(sext8(w[j], b) - in_offset, pre, post, scale,
+                                 out_offset));
+      w[j] = pack4(r[0], r[1], r[2], r[3]);
+    }
+    reinterpret_cast<uint4 *>(dst)[t] = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+  const size_t tail0 = vec_chunks * kEwPerLane;
+  const size_t stride = (size_t)gridDim.x * kEwThreads;
+  for (size_t i = tail0 + t; i < n; i += stride)
+    dst[i] = (int8_t)clip_i8(scale_i32((int32_t)src[i] - in_offset, pre, post,
+                                       scale, out_offset));
+}
+
+static bool aligned16(const void *a, const void *b) {
+  return (((uintptr_t)a | (uintptr_t)b) & 15) == 0;
+}
+
+// Grid covering `vec_chunks` 16-element chunks, and at least one block so the
+// tail loop runs.
+static unsigned ew_blocks(size_t vec_chunks) {
+  size_t b = (vec_chunks + kEwThreads - 1) / kEwThreads;
+  return (unsigned)(b ? b : 1);
+}
+
+} // namespace mi355x
+
+using namespace mi355x;
+
+extern "C" {
+
+int mi355x_quantize_i8(int8_t *dst, const float *src, size_t n, float scale,
+                       int32_t offset, void *stream) {
+  if (n == 0) return MI355X_OK;
+  MI355X_REQUIRE(dst && src, "NULL tensor");
+  MI355X_REQUIRE(n / kEwPerLane / kEwThreads < 0x7fffffffu, "tensor too large");
+  const size_t chunks = aligned16(dst, src) ? n / kEwPerLane : 0;
+  hipLaunchKernelGGL(quantize_i8_kernel, dim3(ew_blocks(chunks)),
+                     dim3(kEwThreads), 0, as_stream(stream), dst, src, n,
+                     chunks, scale, (float)offset);
+  return check_launch("quantize_i8");
+}
+
+int mi355x_dequantize_i8(float *dst, const int8_t *src, size_t n, float scale,
+                         int32_t offset, void *stream) {
+  if (n == 0) return MI355X_OK;
+  MI355X_REQUIRE(dst && src, "NULL tensor");
+  MI355X_REQUIRE(n / kEwPerLane / kEwThreads < 0x7fffffffu, "tensor too large");
+  const size_t chunks = aligned16(dst, src) ? n / kEwPerLane : 0;
+  hipLaunchKernelGGL(dequantize_i8_kernel, dim3(ew_blocks(chunks)),
+                     dim3(kEwThreads), 0, as_stream(stream), dst, src, n,
+                     chunks, scale, offset);
+  return check_launch("dequantize_i8");
+}
+
+int mi355x_rescale_i8(int8_t *dst, const int8_t *src, size_t n,
+                      int32_t out_offset, int32_t in_offset, int32_t pre,
+                      int32_t post, int32_t scale, void *stream) {
+  if (n == 0) return MI355X_OK;
+  MI355X_REQUIRE(dst && src, "NULL tensor");
+  MI355X_REQUIRE(shift_ok(pre) && shift_ok(post),
+                 "pre/post shift outside [0, 31]: %d %d", pre, post);
+  MI355X_REQUIRE(n / kEwPerLane / kEwThreads < 0x7fffffffu, "tensor too large");
+  const size_t chunks = aligned16(dst, src) ? n / kEwPerLane : 0;
+  hipLaunchKernelGGL(rescale_i8_kernel, dim3(ew_blocks(chunks)),
+                     dim3(kEwThreads), 0, as_stream(stream), dst, src, n,
+                     chunks, out_offset, in_offset, pre, post, scale);
+  return check_launch("rescale_i8");
+}
+
+} // extern "C"

@@ -1,0 +1,47 @@
+// Device-side integer requantisation shared by every quantized kernel.
+// Semantics follow Glow's CPU backend bit for bit (reference
+// lib/LLVMIRCodeGen/libjit/libjit_defs.h:147-233): 32-bit wrap-around
+// arithmetic, arithmetic right shifts, round-to-nearest on the post-shift,
+// activation applied after the requantisation and before the int8 clip.
+#ifndef GLOW_MI355X_REQUANT_H
+#define GLOW_MI355X_REQUANT_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mi355x {
+
+// libjit_scale<int32_t>: ((((in >> pre) * scale) + rtn) >> post) + offset.
+__device__ __forceinline__ int32_t scale_i32(int32_t in, int32_t pre,
+                                             int32_t post, int32_t scale,
+                                             int32_t offset) {
+  uint32_t rtn = (post > 0) ? (1u << (post - 1)) : 0u;
+  uint32_t m = (uint32_t)(in >> pre) * (uint32_t)scale + rtn;
+  return (int32_t)((uint32_t)((int32_t)m >> post) + (uint32_t)offset);
+}
+
+__device__ __forceinline__ int32_t clip_i8(int32_t v) {
+  return min(max(v, -128), 127);
+}
+
+// libjit_activation_i32; act follows glow::FusedActivation.
+__device__ __forceinline__ int32_t activation_i32(int32_t v, int32_t offset,
+                                                  int32_t act, int32_t a0,
+                                                  int32_t a1, int32_t a2) {
+  switch (act) {
+  case 1: // RELU
+    return max(v, offset);
+  case 2: // CLIP
+    return min(max(v, a0), a1);
+  case 5: // LEAKY_RELU
+    return v >= offset
+               ? v
+               : scale_i32((int32_t)((uint32_t)v - (uint32_t)offset), a0, a1,
+                           a2, offset);
+  default: // NONE (fused tanh / sigmoid are rejected on the host)
+    return v;
+  }
+}
+
+} // namespace mi355x
+#endif

@@ -1,0 +1,442 @@
+// FusedRowwiseQuantizedSparseLengthsWeightedSum / Sum and the offsets-based
+// EmbeddingBag twin, for 8-bit and 4-bit fused rows with fp32 or fp16
+// scale/offset (reference lib/LLVMIRCodeGen/libjit/libjit.cpp:1253-1276,
+// 2454-2481; lib/Backends/Interpreter/InterpreterNodes.cpp:5764-5889).
+//
+// One bag per group of LPB lanes (a whole 64-lane wavefront for rows of 64+
+// data bytes, so the row index is wave-uniform and every row read is one
+// coalesced request). A lane owns BPL consecutive data bytes of the row and
+// keeps their running sums in registers. For each batch of up to 64 lookups
+// lane j first fetches index j, weight j and the (scale, offset) pair of row j;
+// then all row reads of the batch are issued back to back before the first one
+// is consumed, so a bag costs three dependent memory round trips however long
+// it is. The sums are formed in bag order with separately rounded multiply
+// and add, which reproduces the CPU loop bit for bit.
+//
+// The start of a bag in the index list is the exclusive prefix sum of the
+// lengths. A block sums the lengths in front of it itself (from the start of
+// its chunk of kChunkBags bags, plus one pre-summed value per earlier chunk),
+// which keeps the common small-batch case at a single launch.
+#include "common.h"
+
+#include <hip/hip_fp16.h>
+
+#include <mutex>
+
+namespace mi355x {
+
+constexpr int kSlwsThreads = 256;
+constexpr int kBatch = 64;         // lookups fetched per round
+constexpr int kChunkBags = 8192;   // bags per pre-summed chunk
+constexpr int kMaxChunks = 16384;  // workspace entries (int64 each)
+
+struct SlwsArgs {
+  void *dest;
+  const uint8_t *data;
+  const void *weights;     // fp32 / fp16 / NULL
+  const void *indices;     // int64 / int32
+  const int32_t *lengths;  // lengths mode
+  const int32_t *offsets;  // offsets mode (NULL in lengths mode)
+  const int64_t *chunk_sums; // lengths mode with more than one chunk
+  int64_t data_rows;
+  int64_t num_indices;
+  int64_t segments;        // number of output rows
+  int32_t offsets_have_end;
+  int32_t in_line;         // bytes per fused row
+  int32_t data_bytes;      // quantized bytes per row (before scale/offset)
+  int32_t out_cols;
+  int32_t out16, w16, idx64;
+};
+
+template <int LPB> __device__ __forceinline__ int bcast_i(int v, int j) {
+  if constexpr (LPB == 64) {
+    return __builtin_amdgcn_readlane(v, j);
+  } else {
+    return __shfl(v, j, LPB);
+  }
+}
+template <int LPB> __device__ __forceinline__ float bcast_f(float v, int j) {
+  return __int_as_float(bcast_i<LPB>(__float_as_int(v), j));
+}
+
+__device__ __forceinline__ uint32_t load_u32_any(const uint8_t *p) {
+  if ((((uintptr_t)p) & 3) == 0) return *reinterpret_cast<const uint32_t *>(p);
+  return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) |
+         ((uint32_t)p[3] << 24);
+}
+
+__device__ __forceinline__ float f16round(float v) {
+  return __half2float(__float2half_rn(v));
+}
+
+// acc += w * (scale * q + offset), each operation rounded on its own; with
+// fp16 accumulation the product and the sum are rounded to binary16 the way
+// glow::float16's operator+= does (reference include/glow/Support/Float16.h).
+template <bool ACC16>
+__device__ __forceinline__ float accumulate(float acc, float w, float s,
+                                            float o, uint32_t q) {
+  float d = __fadd_rn(__fmul_rn(s, (float)q), o);
+  float t = __fmul_rn(d, w);
+  if constexpr (ACC16) {
+    return f16round(__fadd_rn(acc, f16round(t)));
+  } else {
+    return __fadd_rn(acc, t);
+  }
+}
+
+template <int LPB, int BPL, bool IS4, bool SO16, bool ACC16>
+__global__ __launch_bounds__(kSlwsThreads) void slws_kernel(SlwsArgs a) {
+  constexpr int kGroups = kSlwsThreads / LPB;      // bags per block
+  constexpr int kColsPerByte = IS4 ? 2 : 1;
+  constexpr int kColsPerLane = BPL * kColsPerByte;
+  __shared__ long long s_part[kSlwsThreads / 64];
+  __shared__ int s_own[kGroups];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int sub = tid % LPB;                        // lane within the bag group
+  const int grp = tid / LPB;
+  const long long first_bag = (long long)blockIdx.x * kGroups;
+  const long long bag = first_bag + grp;
+
+  long long start = 0;
+  int len = 0;
+  if (a.offsets) {
+    if (bag < a.segments) {
+      start = a.offsets[bag];
+      long long end = (!a.offsets_have_end && bag == a.segments - 1)
+                          ? a.num_indices
+                          : (long long)a.offsets[bag + 1];
+      len = end > start ? (int)(end - start) : 0;
+    }
+  } else {
+    // exclusive prefix sum of the clamped lengths in front of this block
+    const long long chunk = first_bag / kChunkBags;
+    const long long lo = chunk * kChunkBags;
+    long long below = 0;
+    const int32_t *lbase = a.lengths + lo;
+    const int n_before = (int)(first_bag - lo); // < kChunkBags, multiple of 4
+    if ((((uintptr_t)lbase) & 15) == 0) {
+      // all loads issued before the first add: one memory round trip
+      constexpr int kVecTrips = kChunkBags / 4 / kSlwsThreads;
+      const int4 *l4 = reinterpret_cast<const int4 *>(lbase);
+      const int nvec = n_before / 4;
+      int4 x[kVecTrips];
+#pragma unroll
+      for (int u = 0; u < kVecTrips; u++) {
+        const int v = tid + u * kSlwsThreads;
+        x[u] = v < nvec ? l4[v] : make_int4(0, 0, 0, 0);
+      }
+#pragma unroll
+      for (int u = 0; u < kVecTrips; u++)
+        below += (long long)max(x[u].x, 0) + max(x[u].y, 0) + (long long)max(x[u].z, 0) + max(x[u].w, 0);
+    } else {
+      for (int i = tid; i < n_before; i += kSlwsThreads) below += max(lbase[i], 0);
+    }
+    if (a.chunk_sums) {
+      for (long long c = tid; c < chunk; c += kSlwsThreads) below += a.chunk_sums[c];
+    }
+    if (tid < kGroups) {
+      long long b = first_bag + tid;
+      int v = b < a.segments ? a.lengths[b] : 0;
+      s_own[tid] = v > 0 ? v : 0;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) below += __shfl_down(below, off, 64);
+    if (lane == 0) s_part[tid >> 6] = below;
+    __syncthreads();
+    start = 0;
+#pragma unroll
+    for (int w = 0; w < kSlwsThreads / 64; w++) start += s_part[w];
+    for (int g = 0; g < grp; g++) start += s_own[g];
+    len = s_own[grp];
+  }
+  if (bag >= a.segments) len = 0;
+
+  const int n_passes = (a.data_bytes + LPB * BPL - 1) / (LPB * BPL);
+  for (int pass = 0; pass < n_passes; pass++) {
+    const int byte0 = (pass * LPB + sub) * BPL;       // first data byte of lane
+    const bool lane_live = byte0 < a.data_bytes;
+    float acc[kColsPerLane];
+#pragma unroll
+    for (int c = 0; c < kColsPerLane; c++) acc[c] = 0.0f;
+
+    for (int base = 0; base < len; base += kBatch) {
+      const int cnt = min(kBatch, len - base);
+      // round 1: lookup `sub + k*LPB` of the batch is fetched by lane `sub`
+      constexpr int kPerLane = kBatch / LPB;
+      int row_lo[kPerLane];
+      float wgt[kPerLane], scl[kPerLane], ofs[kPerLane];
+#pragma unroll
+      for (int k = 0; k < kPerLane; k++) {
+        const int j = sub + k * LPB;
+        long long pos = start + base + j;
+        long long row = -1;
+        float w = 0.0f;
+        if (j < cnt && pos < a.num_indices) {
+          row = a.idx64 ? reinterpret_cast<const long long *>(a.indices)[pos]
+                        : (long long)reinterpret_cast<const int *>(a.indices)[pos];
+          if (!a.weights) {
+            w = 1.0f;
+          } else if (a.w16) {
+            w = __half2float(reinterpret_cast<const __half *>(a.weights)[pos]);
+          } else {
+            w = reinterpret_cast<const float *>(a.weights)[pos];
+          }
+        }
+        float s = 0.0f, o = 0.0f;
+        if (row >= 0 && row < a.data_rows) {
+          const uint8_t *so = a.data + row * a.in_line + a.data_bytes;
+          if constexpr (SO16) {
+            uint32_t v = load_u32_any(so);
+            s = __half2float(__ushort_as_half((unsigned short)(v & 0xffff)));
+            o = __half2float(__ushort_as_half((unsigned short)(v >> 16)));
+          } else {
+            s = __uint_as_float(load_u32_any(so));
+            o = __uint_as_float(load_u32_any(so + 4));
+          }
+        } else {
+          row = 0; // skipped lookup: reads row 0, contributes w * 0
+          w = 0.0f;
+        }
+        row_lo[k] = (int)row; // data_rows * in_line is checked to fit 2^31 rows
+        wgt[k] = w;
+        scl[k] = s;
+        ofs[k] = o;
+      }
+      // round 2: all row reads of the batch in flight before the first use
+      uint32_t q[kBatch];
+#pragma unroll
+      for (int j = 0; j < kBatch; j++) {
+        q[j] = 0;
+        if (j < cnt) {
+          const int row = bcast_i<LPB>(row_lo[j / LPB], j % LPB);
+          if (lane_live) {
+            const uint8_t *p = a.data + (long long)row * a.in_line + byte0;
+            if constexpr (BPL == 2) {
+              q[j] = *reinterpret_cast<const unsigned short *>(p);
+            } else {
+              q[j] = *p;
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < kBatch; j++) {
+        if (j < cnt) {
+          const float w = bcast_f<LPB>(wgt[j / LPB], j % LPB);
+          const float s = bcast_f<LPB>(scl[j / LPB], j % LPB);
+          const float o = bcast_f<LPB>(ofs[j / LPB], j % LPB);
+#pragma unroll
+          for (int b = 0; b < BPL; b++) {
+            const uint32_t byte = (q[j] >> (8 * b)) & 0xff;
+            if constexpr (IS4) {
+              acc[2 * b] = accumulate<ACC16>(acc[2 * b], w, s, o, byte & 15);
+              acc[2 * b + 1] = accumulate<ACC16>(acc[2 * b + 1], w, s, o, byte >> 4);
+            } else {
+              acc[b] = accumulate<ACC16>(acc[b], w, s, o, byte);
+            }
+          }
+        }
+      }
+    }
+
+    if (bag < a.segments && lane_live) {
+      const int col0 = byte0 * kColsPerByte;
+      const long long o0 = bag * (long long)a.out_cols + col0;
+      if (a.out16) {
+        __half *d = reinterpret_cast<__half *>(a.dest) + o0;
+#pragma unroll
+        for (int c = 0; c < kColsPerLane; c++)
+          if (col0 + c < a.out_cols) d[c] = __float2half_rn(acc[c]);
+      } else {
+        float *d = reinterpret_cast<float *>(a.dest) + o0;
+        if (kColsPerLane == 2 && col0 + 1 < a.out_cols &&
+            ((((uintptr_t)d) & 7) == 0)) {
+          *reinterpret_cast<float2 *>(d) = make_float2(acc[0], acc[1]);
+        } else {
+#pragma unroll
+          for (int c = 0; c < kColsPerLane; c++)
+            if (col0 + c < a.out_cols) d[c] = acc[c];
+        }
+      }
+    }
+  }
+}
+
+// Sum of the clamped lengths of each chunk of kChunkBags bags.
+__global__ __launch_bounds__(256) void slws_chunk_sums_kernel(
+    const int32_t *lengths, long long segments, int64_t *chunk_sums) {
+  __shared__ long long s_part[4];
+  const long long lo = (long long)blockIdx.x * kChunkBags;
+  const long long hi = min(lo + (long long)kChunkBags, segments);
+  long long sum = 0;
+  for (long long i = lo + threadIdx.x; i < hi; i += 256) {
+    int v = lengths[i];
+    sum += v > 0 ? v : 0;
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) sum += __shfl_down(sum, off, 64);
+  if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = sum;
+  __syncthreads();
+  if (threadIdx.x == 0)
+    chunk_sums[blockIdx.x] = s_part[0] + s_part[1] + s_part[2] + s_part[3];
+}
+
+// Per-device workspace for the chunk sums, allocated on first use and kept.
+static std::mutex g_ws_mutex;
+static int64_t *g_ws[64] = {nullptr};
+
+static int chunk_workspace(int64_t **ws) {
+  int dev = 0;
+  MI355X_HIP(hipGetDevice(&dev));
+  MI355X_REQUIRE(dev >= 0 && dev < 64, "device index %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  if (!g_ws[dev]) {
+    MI355X_HIP(hipMalloc((void **)&g_ws[dev], kMaxChunks * sizeof(int64_t)));
+  }
+  *ws = g_ws[dev];
+  return MI355X_OK;
+}
+
+template <int LPB, int BPL>
+static void launch_kind(int kind, bool acc16, dim3 grid, hipStream_t st,
+                        const SlwsArgs &a) {
+#define MI355X_SLWS_LAUNCH(IS4, SO16, ACC16)                                   \
+  hipLaunchKernelGGL((slws_kernel<LPB, BPL, IS4, SO16, ACC16>), grid,          \
+                     dim3(kSlwsThreads), 0, st, a)
+  switch (kind) {
+  case MI355X_FUSED_U8_F32:
+    MI355X_SLWS_LAUNCH(false, false, false);
+    break;
+  case MI355X_FUSED_U8_F16:
+    if (acc16) MI355X_SLWS_LAUNCH(false, true, true);
+    else MI355X_SLWS_LAUNCH(false, true, false);
+    break;
+  case MI355X_FUSED_U4_F16:
+    if (acc16) MI355X_SLWS_LAUNCH(true, true, true);
+    else MI355X_SLWS_LAUNCH(true, true, false);
+    break;
+  default:
+    MI355X_SLWS_LAUNCH(true, false, false);
+    break;
+  }
+#undef MI355X_SLWS_LAUNCH
+}
+
+static int slws_dispatch(void *dest, int out_is_f16, const uint8_t *data,
+                         size_t data_rows, int kind, const void *weights,
+                         int weights_are_f16, const void *indices,
+                         int idx_is_64, size_t num_indices,
+                         const int32_t *lengths, const int32_t *offsets,
+                         int has_end_offset, size_t out_rows,
+                         size_t in_line_size, size_t out_line_size,
+                         int fp16_accum, void *stream) {
+  if (out_rows == 0) return MI355X_OK;
+  MI355X_REQUIRE(kind >= 0 && kind <= 3, "unknown fused kind %d", kind);
+  MI355X_REQUIRE(dest && (lengths || offsets), "NULL tensor");
+  const bool is4 = kind == MI355X_FUSED_U4_F16 || kind == MI355X_FUSED_U4_F32;
+  const bool so16 = kind == MI355X_FUSED_U8_F16 || kind == MI355X_FUSED_U4_F16;
+  const size_t so_bytes = so16 ? 4 : 8;
+  MI355X_REQUIRE(in_line_size > so_bytes, "in_line_size %zu too small",
+                 in_line_size);
+  const size_t data_bytes = in_line_size - so_bytes;
+  const size_t cols = is4 ? data_bytes * 2 : data_bytes;
+  MI355X_REQUIRE(out_line_size == cols,
+                 "out_line_size %zu does not match %zu columns of the fused row",
+                 out_line_size, cols);
+  MI355X_REQUIRE(in_line_size < (1u << 20) && data_rows < (1ull << 31) &&
+                     out_rows < (1ull << 40),
+                 "table or batch too large");
+  MI355X_REQUIRE(num_indices == 0 || (indices && data),
+                 "NULL indices or data with num_indices > 0");
+  hipStream_t st = as_stream(stream);
+
+  SlwsArgs a;
+  a.dest = dest;
+  a.data = data;
+  a.weights = weights;
+  a.indices = indices;
+  a.lengths = lengths;
+  a.offsets = offsets;
+  a.chunk_sums = nullptr;
+  a.data_rows = (int64_t)data_rows;
+  a.num_indices = (int64_t)num_indices;
+  a.segments = (int64_t)out_rows;
+  a.offsets_have_end = has_end_offset;
+  a.in_line = (int32_t)in_line_size;
+  a.data_bytes = (int32_t)data_bytes;
+  a.out_cols = (int32_t)cols;
+  a.out16 = out_is_f16;
+  a.w16 = weights_are_f16;
+  a.idx64 = idx_is_64;
+
+  if (!offsets) {
+    const size_t chunks = (out_rows + kChunkBags - 1) / kChunkBags;
+    if (chunks > 1) {
+      MI355X_REQUIRE(chunks <= (size_t)kMaxChunks, "more than %d bags",
+                     kMaxChunks * kChunkBags);
+      int64_t *ws = nullptr;
+      int rc = chunk_workspace(&ws);
+      if (rc != MI355X_OK) return rc;
+      hipLaunchKernelGGL(slws_chunk_sums_kernel, dim3((unsigned)chunks),
+                         dim3(256), 0, st, lengths, (long long)out_rows, ws);
+      rc = check_launch("slws_chunk_sums");
+      if (rc != MI355X_OK) return rc;
+      a.chunk_sums = ws;
+    }
+  }
+
+  const bool acc16 = out_is_f16 && fp16_accum && so16;
+  const bool even = (in_line_size % 2 == 0) && (((uintptr_t)data) % 2 == 0);
+  int lpb = 64;
+  if (even && data_bytes <= 32) lpb = 16;
+  else if (even && data_bytes <= 64) lpb = 32;
+  const size_t groups = kSlwsThreads / lpb;
+  const size_t blocks = (out_rows + groups - 1) / groups;
+  MI355X_REQUIRE(blocks < 0x7fffffffu, "too many bags");
+  dim3 grid((unsigned)blocks);
+  if (!even) launch_kind<64, 1>(kind, acc16, grid, st, a);
+  else if (lpb == 16) launch_kind<16, 2>(kind, acc16, grid, st, a);
+  else if (lpb == 32) launch_kind<32, 2>(kind, acc16, grid, st, a);
+  else launch_kind<64, 2>(kind, acc16, grid, st, a);
+  return check_launch("frwq_slws");
+}
+
+} // namespace mi355x
+
+using namespace mi355x;
+
+extern "C" {
+
+int mi355x_frwq_slws(void *dest, int out_is_f16, const uint8_t *data,
+                     size_t data_rows, int kind, const void *weights,
+                     int weights_are_f16, const void *indices, int idx_is_64,
+                     size_t num_indices, const int32_t *lengths,
+                     size_t segments, size_t in_line_size,
+                     size_t out_line_size, int fp16_accum, void *stream) {
+  MI355X_REQUIRE(segments == 0 || lengths, "lengths is NULL");
+  return slws_dispatch(dest, out_is_f16, data, data_rows, kind, weights,
+                       weights_are_f16, indices, idx_is_64, num_indices,
+                       lengths, nullptr, 0, segments, in_line_size,
+                       out_line_size, fp16_accum, stream);
+}
+
+int mi355x_embedding_bag_rowwise_offsets(
+    void *dest, int out_is_f16, const uint8_t *data, size_t data_rows,
+    int kind, const void *weights, int weights_are_f16, const int32_t *indices,
+    size_t num_indices, const int32_t *offsets, size_t segments,
+    int has_end_offset, size_t in_line_size, size_t out_line_size,
+    int fp16_accum, void *stream) {
+  MI355X_REQUIRE(segments == 0 || offsets, "offsets is NULL");
+  if (has_end_offset) {
+    MI355X_REQUIRE(segments >= 1, "has_end_offset needs at least one offset");
+    segments -= 1;
+  }
+  return slws_dispatch(dest, out_is_f16, data, data_rows, kind, weights,
+                       weights_are_f16, indices, 0, num_indices, nullptr,
+                       offsets, has_end_offset, segments, in_line_size,
+                       out_line_size, fp16_accum, stream);
+}
+
+} // extern "C"

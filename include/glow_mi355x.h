@@ -1,0 +1,288 @@
+/*
+ * glow_mi355x.h - C ABI of the MI355X (gfx950) kernel library for Glow's
+ * quantized-inference hot path.
+ *
+ * This is the layer a glow::Backend / CompiledFunction / DeviceManager for
+ * MI355X calls where Glow's CPU backend calls into libjit: one entry point
+ * per lowered quantized instruction, taking DEVICE pointers, plain sizes and
+ * the same integer parameters the CPU code generator derives
+ * (lib/LLVMIRCodeGen/LLVMIRGen.cpp). Each entry point cites the libjit
+ * function it replaces; "reference" paths are relative to the pytorch/glow
+ * tree.
+ *
+ * Conventions
+ *   - every function returns MI355X_OK (0) or a negative mi355x_status; the
+ *     message of the last failure on the calling thread is
+ *     mi355x_last_error().
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ *     Launches are asynchronous; nothing here synchronises unless it says so.
+ *   - all tensors are dense, row-major, in device memory unless a parameter
+ *     is documented as a host pointer.
+ *   - shift amounts (pre, post) must lie in [0, 31].
+ */
+#ifndef GLOW_MI355X_H
+#define GLOW_MI355X_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Status codes; the names follow glow::ErrorValue::ErrorCode
+ * (reference include/glow/Support/Error.h:292-337) where one applies. */
+typedef enum {
+  MI355X_OK = 0,
+  MI355X_ERR_INVALID_ARGUMENT = -1,
+  MI355X_ERR_RUNTIME = -2,              /* RUNTIME_ERROR: a HIP call failed   */
+  MI355X_ERR_OUT_OF_DEVICE_MEMORY = -3, /* RUNTIME_OUT_OF_DEVICE_MEMORY        */
+  MI355X_ERR_NOT_SUPPORTED = -4,        /* DEVICE_FEATURE_NOT_SUPPORTED        */
+  MI355X_ERR_NET_NOT_FOUND = -5,        /* RUNTIME_NET_NOT_FOUND               */
+  MI355X_ERR_DEVICE_NOT_FOUND = -6,     /* RUNTIME_DEVICE_NOT_FOUND            */
+  MI355X_ERR_NET_BUSY = -7              /* RUNTIME_NET_BUSY                    */
+} mi355x_status;
+
+const char *mi355x_last_error(void);
+
+/* ---- device, memory, streams, events ------------------------------------ */
+/* Replaces what CPUDeviceManager gets from the host OS: device discovery and
+ * memory accounting (reference lib/Backends/CPU/CPUDeviceManager.cpp:36-63,
+ * DeviceManager.h:189-204). */
+
+typedef struct {
+  char name[128];
+  char arch[64];            /* e.g. "gfx950:sramecc+:xnack-" */
+  int32_t compute_units;
+  int32_t clock_khz;
+  uint64_t total_memory;
+  uint64_t free_memory;
+  int32_t device;
+  int32_t lds_bytes_per_block;
+} mi355x_info;
+
+int mi355x_num_devices(int *count);
+/* Selects `device` for the calling thread and checks that it is a gfx950. */
+int mi355x_init(int device);
+int mi355x_device_info(mi355x_info *info);
+
+int mi355x_malloc(void **dptr, size_t bytes);
+int mi355x_free(void *dptr);
+/* Pinned host memory for I/O buffers (DeviceManager::allocateDeviceIOBuffer,
+ * reference include/glow/Backends/DeviceManager.h:122-127). */
+int mi355x_host_alloc(void **hptr, size_t bytes);
+int mi355x_host_free(void *hptr);
+int mi355x_memcpy_h2d(void *dst, const void *src, size_t bytes, void *stream);
+int mi355x_memcpy_d2h(void *dst, const void *src, size_t bytes, void *stream);
+int mi355x_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream);
+/* Fills with a kernel (safe inside a captured graph). */
+int mi355x_fill_u8(void *dst, int value, size_t bytes, void *stream);
+
+int mi355x_stream_create(void **stream);
+int mi355x_stream_destroy(void *stream);
+int mi355x_stream_sync(void *stream);
+int mi355x_device_sync(void);
+int mi355x_event_create(void **event);
+int mi355x_event_destroy(void *event);
+int mi355x_event_record(void *event, void *stream);
+int mi355x_event_sync(void *event);
+int mi355x_event_elapsed_ms(void *start, void *stop, float *ms);
+
+/* ---- static memory plan ---------------------------------------------------- */
+/* One HBM allocation per compiled function laid out as
+ * constants | mutable (placeholders) | activations with the byte offsets
+ * Glow's RuntimeBundle assigns (reference lib/Backend/BackendUtils.cpp:702-730,
+ * RuntimeSymbolInfo BackendUtils.h:41-62); replaces the per-run host
+ * allocations of LLVMCompiledFunction::execute
+ * (lib/LLVMIRCodeGen/LLVMCompiledFunction.cpp:81-96). */
+typedef struct mi355x_arena mi355x_arena;
+enum { MI355X_REGION_CONSTANTS = 0, MI355X_REGION_MUTABLE = 1,
+       MI355X_REGION_ACTIVATIONS = 2 };
+int mi355x_arena_create(size_t const_bytes, size_t mutable_bytes,
+                        size_t activation_bytes, mi355x_arena **arena);
+int mi355x_arena_destroy(mi355x_arena *arena);
+/* Device address of region base + offset (NULL and an error when outside). */
+int mi355x_arena_ptr(mi355x_arena *arena, int region, size_t offset,
+                     void **dptr);
+int mi355x_arena_upload(mi355x_arena *arena, int region, size_t offset,
+                        const void *host, size_t bytes, void *stream);
+int mi355x_arena_download(mi355x_arena *arena, int region, size_t offset,
+                          void *host, size_t bytes, void *stream);
+uint64_t mi355x_arena_bytes(const mi355x_arena *arena);
+
+/* ---- host-side parameter derivation (no GPU involved) ----------------------- */
+
+/* quantization::quantizeScaleOffset32To8 (reference
+ * lib/Quantization/Base/Base.cpp:234-359). out = {pre, post, scale, offset}. */
+void mi355x_quantize_scale_offset_32to8(float scale, int32_t offset,
+                                        int32_t out[4]);
+
+/* quantization::Schema (reference include/glow/Quantization/Base/Base.h:217) */
+enum { MI355X_SCHEMA_ASYMMETRIC = 0, MI355X_SCHEMA_SYMMETRIC = 1,
+       MI355X_SCHEMA_SYMMETRIC_WITH_UNSIGNED = 2,
+       MI355X_SCHEMA_SYMMETRIC_POWER2 = 3 };
+/* Quantized element kinds for the range lookup (Base.cpp:361-403). */
+enum { MI355X_QTY_INT8 = 8, MI355X_QTY_INT16 = 16, MI355X_QTY_INT32 = 32,
+       MI355X_QTY_UINT8 = 108 };
+/* quantization::chooseQuantizationParams with Calibration::None (reference
+ * lib/Quantization/Base/Base.cpp:433-565). */
+int mi355x_choose_quantization_params(float min, float max, int schema,
+                                      int qty, float *scale, int32_t *offset);
+
+/* Fused-rowwise element kinds (reference include/glow/Base/Type.h:424-433):
+ * row = [data | scale | offset], scale/offset fp32 or fp16; 4-bit rows hold
+ * two columns per byte, even column in the low nibble. */
+enum { MI355X_FUSED_U8_F32 = 0, MI355X_FUSED_U8_F16 = 1,
+       MI355X_FUSED_U4_F16 = 2, MI355X_FUSED_U4_F32 = 3 };
+size_t mi355x_fused_row_bytes(size_t cols, int kind);
+/* quantization::tensorFusedRowwiseQuantization<T> on HOST buffers (reference
+ * include/glow/Quantization/Base/Base.h:598-678). */
+int mi355x_fused_rowwise_quantize_host(const float *in, size_t rows,
+                                       size_t cols, int kind, uint8_t *out);
+/* quantization::tensorRowwiseQuantization<float,int32_t,int8_t> on HOST
+ * buffers (reference Base.h:522-557): per-row parameters + int8 weights. */
+int mi355x_rowwise_quantize_i8_host(const float *in, size_t rows, size_t cols,
+                                    int schema, int8_t *out, float *scales,
+                                    int32_t *offsets);
+
+/* ---- elementwise ------------------------------------------------------------ */
+
+/* libjit_element_quantize_kernel_i8 (reference
+ * lib/LLVMIRCodeGen/libjit/libjit.cpp:2998-3002) over n elements. */
+int mi355x_quantize_i8(int8_t *dst, const float *src, size_t n, float scale,
+                       int32_t offset, void *stream);
+/* libjit_element_dequantize_kernel_i8 (libjit.cpp:3016-3019). */
+int mi355x_dequantize_i8(float *dst, const int8_t *src, size_t n, float scale,
+                         int32_t offset, void *stream);
+/* libjit_element_rescale_kernel_i8 (libjit.cpp:3031-3038). */
+int mi355x_rescale_i8(int8_t *dst, const int8_t *src, size_t n,
+                      int32_t out_offset, int32_t in_offset, int32_t pre,
+                      int32_t post, int32_t scale, void *stream);
+
+/* ---- FullyConnected / MatMul -------------------------------------------------- */
+
+/* libjit_rowwise_quantized_fc_i8_i32 / _i8_i8 (reference
+ * lib/LLVMIRCodeGen/libjit/libjit_matmul.cpp:284-316, 425-450).
+ * in [M x K], weights [N x K] (not transposed), bias int32[N] or int8[N]
+ * (bias_is_i8), seven int32[N] per-row parameter vectors, out int8 [M x N].
+ * weights_offsets_all_zero != 0 promises that every weights_offsets[j] is 0
+ * (symmetric weights), which skips the activation row sums. */
+int mi355x_rwq_fc_i8(int8_t *out, const int8_t *in, const int8_t *weights,
+                     const void *bias, int bias_is_i8,
+                     const int32_t *weights_offsets, const int32_t *bias_pre,
+                     const int32_t *bias_post, const int32_t *bias_scale,
+                     const int32_t *out_pre, const int32_t *out_post,
+                     const int32_t *out_scale, size_t M, size_t K, size_t N,
+                     int32_t out_offset, int32_t in_offset,
+                     int32_t bias_offset, int weights_offsets_all_zero,
+                     void *stream);
+
+/* libjit_fc_i8_i32 / _i8_i8 (libjit_matmul.cpp:254-280, 395-422).
+ * weights_kn is [K x N] as Glow stores FullyConnected weights; the kernel
+ * consumes the [N x K] transpose, which is written to `weights_nk_workspace`
+ * (K*N bytes, device) when repack != 0 and read from there otherwise (weights
+ * are constants: repack once at load time). */
+int mi355x_fc_i8(int8_t *out, const int8_t *in, const int8_t *weights_kn,
+                 int8_t *weights_nk_workspace, int repack, const void *bias,
+                 int bias_is_i8, size_t M, size_t K, size_t N,
+                 int32_t out_offset, int32_t in_offset, int32_t weights_offset,
+                 int32_t bias_offset, int32_t bias_pre, int32_t bias_post,
+                 int32_t bias_scale, int32_t out_pre, int32_t out_post,
+                 int32_t out_scale, void *stream);
+
+/* libjit_matmul_i8 (libjit_matmul.cpp:353-371). lhs [M x K], rhs_kn [K x N];
+ * workspace and repack as for mi355x_fc_i8. */
+int mi355x_matmul_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs_kn,
+                     int8_t *rhs_nk_workspace, int repack, size_t M, size_t K,
+                     size_t N, int32_t out_offset, int32_t lhs_offset,
+                     int32_t rhs_offset, int32_t out_pre, int32_t out_post,
+                     int32_t out_scale, void *stream);
+
+/* libjit_transpose_i8 for a 2-D tensor: dst [cols x rows] = src [rows x cols]^T */
+int mi355x_transpose2d_i8(int8_t *dst, const int8_t *src, size_t rows,
+                          size_t cols, void *stream);
+
+/* ---- Convolution -------------------------------------------------------------- */
+
+/* NHWC input [N,IH,IW,IC], filter [OC,KH,KW,IC/group], output [N,OH,OW,OC];
+ * pads are {top, left}; the output size carries bottom/right. */
+typedef struct {
+  int32_t N, IH, IW, IC;
+  int32_t OH, OW, OC;
+  int32_t KH, KW;
+  int32_t strideH, strideW;
+  int32_t padT, padL;
+  int32_t dilH, dilW;
+  int32_t group;
+} mi355x_conv_geom;
+
+/* glow::FusedActivation (reference include/glow/Graph/Nodes.h:276-283);
+ * act_args are the quantized arguments emitConstQuantActivationArgs builds
+ * (LLVMIRGen.cpp:618-662): CLIP {min, max}; LEAKY_RELU {pre, post, scale}. */
+enum { MI355X_ACT_NONE = 0, MI355X_ACT_RELU = 1, MI355X_ACT_CLIP = 2,
+       MI355X_ACT_TANH = 3, MI355X_ACT_SIGMOID = 4, MI355X_ACT_LEAKY_RELU = 5 };
+
+/* libjit_channelwise_quantized_conv2d_i8_i32 / _i8_i8 (reference
+ * lib/LLVMIRCodeGen/libjit/libjit_conv.cpp:151-239, 530-562). Eight int32[OC]
+ * per-channel vectors on the device; act_args is a HOST array of 3 ints. */
+int mi355x_cwq_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
+                         const void *bias, int bias_is_i8,
+                         const mi355x_conv_geom *geom, int32_t out_offset,
+                         int32_t in_offset, const int32_t *filter_offsets,
+                         const int32_t *bias_offsets, const int32_t *bias_pre,
+                         const int32_t *bias_post, const int32_t *bias_scale,
+                         const int32_t *out_pre, const int32_t *out_post,
+                         const int32_t *out_scale, int32_t act_type,
+                         const int32_t *act_args,
+                         int filter_offsets_all_zero, void *stream);
+
+/* libjit_conv2d_i8_i32 / _i8_i8 (libjit_conv.cpp:49-147, 496-528). */
+int mi355x_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
+                     const void *bias, int bias_is_i8,
+                     const mi355x_conv_geom *geom, int32_t out_offset,
+                     int32_t in_offset, int32_t filter_offset,
+                     int32_t bias_offset, int32_t bias_pre, int32_t bias_post,
+                     int32_t bias_scale, int32_t out_pre, int32_t out_post,
+                     int32_t out_scale, int32_t act_type,
+                     const int32_t *act_args, void *stream);
+
+/* ---- fused-rowwise SparseLengths(Weighted)Sum ----------------------------------- */
+
+/* libjit_fused_rowwise_quantized_sparse_lengths_weighted_sum_f_u / _f_i32
+ * (reference lib/LLVMIRCodeGen/libjit/libjit.cpp:1253-1276, 2416-2428) for
+ * MI355X_FUSED_U8_F32 with fp32 weights and output, and the Interpreter's
+ * fwdFusedRowwiseQuantizedSparseLengthsWeightedSumImpl (reference
+ * lib/Backends/Interpreter/InterpreterNodes.cpp:5764-5889) for the other
+ * kinds, fp16 weights/output and fp16 accumulation.
+ *   dest     [segments x out_line_size] fp32, or fp16 when out_is_f16
+ *   data     [data_rows x in_line_size] fused rows
+ *   weights  fp32 (or fp16 when weights_are_f16); NULL = all ones
+ *            (FusedRowwiseQuantizedSparseLengthsSum, Lower.cpp:1590-1606)
+ *   indices  int64 when idx_is_64 else int32, num_indices entries of which
+ *            the first sum(lengths) are used
+ *   lengths  int32[segments]
+ * Every output row is written (empty bags give zeros). Unlike the reference,
+ * an index outside [0, data_rows) or a position beyond num_indices is skipped
+ * instead of read. */
+int mi355x_frwq_slws(void *dest, int out_is_f16, const uint8_t *data,
+                     size_t data_rows, int kind, const void *weights,
+                     int weights_are_f16, const void *indices, int idx_is_64,
+                     size_t num_indices, const int32_t *lengths,
+                     size_t segments, size_t in_line_size,
+                     size_t out_line_size, int fp16_accum, void *stream);
+
+/* libjit_embedding_bag_byte_rowwise_offsets_f (libjit.cpp:2454-2481) and the
+ * Interpreter's 4-bit / fp16 twin: bags are given by int32 start offsets
+ * (`segments` entries, the last one being the end offset when
+ * has_end_offset). Output has segments - has_end_offset rows. */
+int mi355x_embedding_bag_rowwise_offsets(
+    void *dest, int out_is_f16, const uint8_t *data, size_t data_rows,
+    int kind, const void *weights, int weights_are_f16, const int32_t *indices,
+    size_t num_indices, const int32_t *offsets, size_t segments,
+    int has_end_offset, size_t in_line_size, size_t out_line_size,
+    int fp16_accum, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GLOW_MI355X_H */
