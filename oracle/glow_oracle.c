@@ -336,13 +336,20 @@ void go_fused_rowwise_quantize(const float *in, size_t rows, size_t cols,
 /* ------------------------------------------------------------------------ */
 
 /* libjit.cpp:2998-3002: clip((int32)nearbyintf(in/scale + offset)).
- * The float -> int32 conversion is only defined for |v| < 2^31; callers stay
- * inside that domain. */
+ * The reference's float -> int32 conversion is undefined for |v| >= 2^31 (on
+ * x86 it happens to yield INT32_MIN for either sign). Beyond that range this
+ * restatement saturates before the clip, which is what Glow's host-side
+ * quantization::quantize does through int64 (Base.h:323-329); inside the
+ * range the two agree. */
 void go_quantize_i8(int8_t *dst, const float *src, size_t n, float scale,
                     int32_t offset) {
   for (size_t i = 0; i < n; i++) {
     float r = nearbyintf(src[i] / scale + (float)offset);
-    dst[i] = go_clip_i8((int32_t)r);
+    int32_t v;
+    if (r >= 2147483648.0f) v = INT32_MAX;
+    else if (r <= -2147483648.0f) v = INT32_MIN;
+    else v = (int32_t)r;
+    dst[i] = go_clip_i8(v);
   }
 }
 
