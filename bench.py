@@ -41,6 +41,8 @@ def parse():
     ap.add_argument("--batches", type=int, default=8,
                     help="distinct index batches cycled through by the steps")
     ap.add_argument("--rows", type=int, default=4_000_000)
+    ap.add_argument("--bags", type=int, default=4096,
+                    help="bags per step (4096 is the headline configuration)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0,
                     help="wall-clock budget of the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true",
@@ -51,20 +53,32 @@ def parse():
     return ap.parse_args()
 
 
-def timed_launches(capi, fn, steps, warmup, stream=None):
-    """Average seconds per launch: HIP events around `steps` launches on the
-    stream they are issued on, device idle before and after."""
+def timed_launches(capi, fn, steps, warmup):
+    """Average seconds per launch. `fn(i, stream)` issues launch i. After
+    `warmup` eager launches, the `steps` timed launches are recorded into one
+    launch graph and replayed, so the figure is the device-side rate and not
+    the host's enqueue rate (a Python -> ctypes -> HIP launch costs 4-6 us,
+    more than some of these kernels take). HIP events bracket the replay on
+    the stream it runs on, with the device idle before and after."""
+    stream = capi.Stream()
     for i in range(warmup):
-        fn(i)
+        fn(i, stream)
+    stream.sync()
+    with capi.Graph(stream) as graph:
+        for i in range(steps):
+            fn(warmup + i, stream)
+    graph.launch()          # untimed first replay (uploads the graph)
+    stream.sync()
     capi.sync()
     e0, e1 = capi.Event(), capi.Event()
     e0.record(stream)
-    for i in range(steps):
-        fn(warmup + i)
+    graph.launch()
     e1.record(stream)
     e1.sync()
     capi.sync()
-    return e0.elapsed_ms(e1) * 1e-3 / steps
+    sec = e0.elapsed_ms(e1) * 1e-3 / steps
+    graph.destroy()
+    return sec
 
 
 def slws_bytes(total_lookups, bags, cols, row_bytes):
@@ -73,7 +87,7 @@ def slws_bytes(total_lookups, bags, cols, row_bytes):
 
 
 def bench_slws(capi, cases, args, table, d_table):
-    rows, cols, bags = args.rows, 128, 4096
+    rows, cols, bags = args.rows, 128, args.bags
     row_bytes = cols + 8
     batches = []
     for b in range(args.batches):
@@ -84,11 +98,11 @@ def bench_slws(capi, cases, args, table, d_table):
             d_w=capi.to_device(w)))
     d_out = capi.DeviceBuffer.empty((bags, cols), np.float32)
 
-    def step(i):
+    def step(i, stream):
         b = batches[i % len(batches)]
         capi.launch_frwq_slws(d_out, False, d_table, rows, capi.FUSED_U8_F32,
                               b["d_w"], False, b["d_idx"], True, b["total"],
-                              b["d_len"], bags, row_bytes, cols)
+                              b["d_len"], bags, row_bytes, cols, stream=stream)
 
     sec = timed_launches(capi, step, args.steps, args.warmup)
     mean_total = float(np.mean([batches[(args.warmup + i) % len(batches)]["total"]
@@ -111,13 +125,13 @@ def cpu_baseline_slws(table, batches, budget_s, gpu_out, gpu_batch):
     while True:
         b = batches[n % len(batches)]
         go.frwq_slws_f32(table, b["w"], b["idx"], b["lengths"])
-        done_bytes += slws_bytes(b["total"], 4096, 128, 136)
+        done_bytes += slws_bytes(b["total"], b["lengths"].size, 128, 136)
         n += 1
         el = time.perf_counter() - t0
         if el >= budget_s or n >= 4000:
             break
     return dict(value=done_bytes / el / 1e9, unit="GB/s", cores=1, kind="port",
-                sample=f"{n} full batches of 4096 bags (single thread, "
+                sample=f"{n} full batches of {batches[0]['lengths'].size} bags (single thread, "
                        f"{el:.1f} s) of the same table and index batches"), parity
 
 
@@ -134,12 +148,13 @@ def bench_fc(capi, cases, M, K, N, steps, warmup, seed=5):
          if isinstance(v, np.ndarray)}
     d_out = capi.DeviceBuffer.empty((M, N), np.int8)
 
-    def step(_):
+    def step(_, stream):
         capi.launch_rwq_fc_i8(d_out, d["x"], d["w"], d["bias"], False,
                               d["w_offsets"], d["bias_pre"], d["bias_post"],
                               d["bias_scale"], d["out_pre"], d["out_post"],
                               d["out_scale"], M, K, N, c["out_offset"],
-                              c["in_offset"], c["bias_offset"], True)
+                              c["in_offset"], c["bias_offset"], True,
+                              stream=stream)
 
     sec = timed_launches(capi, step, steps, warmup)
     ops = 2.0 * M * N * K
@@ -159,13 +174,13 @@ def bench_conv(capi, cases, steps, warmup):
          if isinstance(v, np.ndarray)}
     d_out = capi.DeviceBuffer.empty((g.N, g.OH, g.OW, g.OC), np.int8)
 
-    def step(_):
+    def step(_, stream):
         capi.launch_cwq_conv2d_i8(d_out, d["x"], d["filt"], d["bias"], False, g,
                                   c["out_offset"], c["in_offset"],
                                   d["f_offsets"], d["b_offsets"], d["bias_pre"],
                                   d["bias_post"], d["bias_scale"], d["out_pre"],
                                   d["out_post"], d["out_scale"], c["act"],
-                                  c["act_args"], True)
+                                  c["act_args"], True, stream=stream)
 
     sec = timed_launches(capi, step, steps, warmup)
     ops = 2.0 * g.N * g.OH * g.OW * g.OC * g.KH * g.KW * g.IC
@@ -184,17 +199,17 @@ def bench_elementwise(capi, which, steps, warmup):
     if which == "quantize":
         src = capi.to_device(rng.normal(0, 1, n).astype(np.float32))
         dst = capi.DeviceBuffer.empty((n,), np.int8)
-        fn = lambda _: capi.launch_quantize_i8(dst, src, n, 0.02, -3)
+        fn = lambda _, st: capi.launch_quantize_i8(dst, src, n, 0.02, -3, st)
         nbytes = n * 5
     elif which == "dequantize":
         src = capi.to_device(rng.integers(-128, 128, n).astype(np.int8))
         dst = capi.DeviceBuffer.empty((n,), np.float32)
-        fn = lambda _: capi.launch_dequantize_i8(dst, src, n, 0.02, -3)
+        fn = lambda _, st: capi.launch_dequantize_i8(dst, src, n, 0.02, -3, st)
         nbytes = n * 5
     else:
         src = capi.to_device(rng.integers(-128, 128, n).astype(np.int8))
         dst = capi.DeviceBuffer.empty((n,), np.int8)
-        fn = lambda _: capi.launch_rescale_i8(dst, src, n, 3, -5, 2, 15, 300)
+        fn = lambda _, st: capi.launch_rescale_i8(dst, src, n, 3, -5, 2, 15, 300, st)
         nbytes = n * 2
     sec = timed_launches(capi, fn, steps, warmup)
     return dict(workload=f"{which}_i8 n={n}", ms=sec * 1e3,
@@ -270,7 +285,7 @@ def main():
         "config": {
             "workload": "FusedRowwiseQuantizedSparseLengthsWeightedSum, uint8 "
                         f"fused-rowwise table {args.rows} x 128 (136-byte rows), "
-                        "4096 bags Poisson(40), Zipf(1.05) int64 indices, fp32 "
+                        f"{args.bags} bags Poisson(40), Zipf(1.05) int64 indices, fp32 "
                         "weights, fp32 out",
             "index_batches_cycled": args.batches,
             "mean_lookups_per_step": s["mean_lookups"],

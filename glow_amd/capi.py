@@ -28,6 +28,8 @@ EXPORTS = [
     "mi355x_event_sync", "mi355x_event_elapsed_ms", "mi355x_arena_create",
     "mi355x_arena_destroy", "mi355x_arena_ptr", "mi355x_arena_upload",
     "mi355x_arena_download", "mi355x_arena_bytes",
+    "mi355x_graph_begin_capture", "mi355x_graph_end_capture",
+    "mi355x_graph_launch", "mi355x_graph_destroy",
     "mi355x_quantize_scale_offset_32to8", "mi355x_choose_quantization_params",
     "mi355x_fused_row_bytes", "mi355x_fused_rowwise_quantize_host",
     "mi355x_rowwise_quantize_i8_host", "mi355x_quantize_i8",
@@ -84,10 +86,11 @@ def check(rc):
 
 
 def _vp(x):
-    """void* from a DeviceBuffer, an int address, a numpy array or None."""
+    """void* from a DeviceBuffer / Stream / Event, an int address, a numpy
+    array or None."""
     if x is None:
         return C.c_void_p(0)
-    if isinstance(x, DeviceBuffer):
+    if isinstance(x, (DeviceBuffer, Stream, Event)):
         return C.c_void_p(x.ptr)
     if isinstance(x, np.ndarray):
         return C.c_void_p(x.ctypes.data)
@@ -230,6 +233,42 @@ class Event:
         try:
             if self.ptr:
                 lib().mi355x_event_destroy(_vp(self.ptr))
+        except Exception:
+            pass
+
+
+class Graph:
+    """Records the launches issued on `stream` inside the `with` block and
+    replays them with launch()."""
+
+    def __init__(self, stream):
+        self.stream = stream
+        self.handle = 0
+
+    def __enter__(self):
+        check(lib().mi355x_graph_begin_capture(_vp(self.stream.ptr)))
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        p = C.c_void_p(0)
+        rc = lib().mi355x_graph_end_capture(_vp(self.stream.ptr), C.byref(p))
+        if exc_type is None:
+            check(rc)
+        self.handle = p.value or 0
+        return False
+
+    def launch(self, stream=None):
+        s = stream if stream is not None else self.stream
+        check(lib().mi355x_graph_launch(_vp(self.handle), _vp(s.ptr)))
+
+    def destroy(self):
+        if self.handle:
+            check(lib().mi355x_graph_destroy(_vp(self.handle)))
+            self.handle = 0
+
+    def __del__(self):
+        try:
+            self.destroy()
         except Exception:
             pass
 

@@ -5,6 +5,12 @@
 // fp32 side; tensors whose base is not 16-byte aligned, and the last n % 16
 // elements, go through the scalar tail.
 #include "common.h"
+
+// Every multiply and add below must round on its own (the CPU code this
+// reproduces has no fused multiply-add). The pragma covers contraction in the
+// front end; the build must also pass -ffp-contract=off (the Makefile does),
+// because HIP's default "fast" mode fuses in the back end regardless.
+#pragma clang fp contract(off)
 #include "requant.h"
 
 namespace mi355x {

@@ -226,6 +226,59 @@ int mi355x_event_elapsed_ms(void *start, void *stop, float *ms) {
   return MI355X_OK;
 }
 
+struct mi355x_graph {
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+};
+
+int mi355x_graph_begin_capture(void *stream) {
+  MI355X_REQUIRE(stream, "graph capture needs a created stream, not the default one");
+  MI355X_HIP(hipStreamBeginCapture(as_stream(stream),
+                                   hipStreamCaptureModeThreadLocal));
+  return MI355X_OK;
+}
+
+int mi355x_graph_end_capture(void *stream, mi355x_graph **graph) {
+  MI355X_REQUIRE(stream && graph, "NULL argument");
+  *graph = nullptr;
+  hipGraph_t g = nullptr;
+  MI355X_HIP(hipStreamEndCapture(as_stream(stream), &g));
+  hipGraphExec_t e = nullptr;
+  hipError_t err = hipGraphInstantiate(&e, g, nullptr, nullptr, 0);
+  if (err != hipSuccess) {
+    (void)hipGraphDestroy(g);
+    return fail(MI355X_ERR_RUNTIME, "hipGraphInstantiate: %s",
+                hipGetErrorString(err));
+  }
+  mi355x_graph *out = new (std::nothrow) mi355x_graph();
+  if (!out) {
+    (void)hipGraphExecDestroy(e);
+    (void)hipGraphDestroy(g);
+    return fail(MI355X_ERR_RUNTIME, "host allocation failed");
+  }
+  out->graph = g;
+  out->exec = e;
+  *graph = out;
+  return MI355X_OK;
+}
+
+int mi355x_graph_launch(mi355x_graph *graph, void *stream) {
+  MI355X_REQUIRE(graph && graph->exec, "graph is NULL");
+  MI355X_HIP(hipGraphLaunch(graph->exec, as_stream(stream)));
+  return MI355X_OK;
+}
+
+int mi355x_graph_destroy(mi355x_graph *graph) {
+  if (!graph) return MI355X_OK;
+  hipError_t e1 = graph->exec ? hipGraphExecDestroy(graph->exec) : hipSuccess;
+  hipError_t e2 = graph->graph ? hipGraphDestroy(graph->graph) : hipSuccess;
+  delete graph;
+  if (e1 != hipSuccess || e2 != hipSuccess)
+    return fail(MI355X_ERR_RUNTIME, "graph destroy: %s",
+                hipGetErrorString(e1 != hipSuccess ? e1 : e2));
+  return MI355X_OK;
+}
+
 static size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 int mi355x_arena_create(size_t const_bytes, size_t mutable_bytes,

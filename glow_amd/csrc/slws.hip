@@ -4,20 +4,32 @@
 // 2454-2481; lib/Backends/Interpreter/InterpreterNodes.cpp:5764-5889).
 //
 // One bag per group of LPB lanes (a whole 64-lane wavefront for rows of 64+
-// data bytes, so the row index is wave-uniform and every row read is one
-// coalesced request). A lane owns BPL consecutive data bytes of the row and
-// keeps their running sums in registers. For each batch of up to 64 lookups
-// lane j first fetches index j, weight j and the (scale, offset) pair of row j;
-// then all row reads of the batch are issued back to back before the first one
-// is consumed, so a bag costs three dependent memory round trips however long
-// it is. The sums are formed in bag order with separately rounded multiply
-// and add, which reproduces the CPU loop bit for bit.
+// data bytes, so every row read is one coalesced request). A lane owns BPL
+// consecutive data bytes of the row and keeps their running sums in
+// registers. For each batch of up to 64 lookups lane j first fetches index j,
+// weight j and the (scale, offset) pair of row j; then all row reads of the
+// batch are issued back to back before the first one is consumed, so a bag
+// costs three dependent memory round trips however long it is. The sums are
+// formed in bag order with separately rounded multiply and add, which
+// reproduces the CPU loop bit for bit.
+//
+// In the wavefront-per-bag kernel the per-lookup values (row byte offset,
+// weight, scale, offset) are handed from lane j to the whole wave through a
+// wave-private LDS slot read back at a uniform address (a broadcast), which
+// keeps the vector ALU for the five operations per element the arithmetic
+// needs (convert, multiply, add, multiply, add).
 //
 // The start of a bag in the index list is the exclusive prefix sum of the
 // lengths. A block sums the lengths in front of it itself (from the start of
 // its chunk of kChunkBags bags, plus one pre-summed value per earlier chunk),
 // which keeps the common small-batch case at a single launch.
 #include "common.h"
+
+// Every multiply and add below must round on its own (the CPU code this
+// reproduces has no fused multiply-add). The pragma covers contraction in the
+// front end; the build must also pass -ffp-contract=off (the Makefile does),
+// because HIP's default "fast" mode fuses in the back end regardless.
+#pragma clang fp contract(off)
 
 #include <hip/hip_fp16.h>
 
@@ -27,8 +39,8 @@ namespace mi355x {
 
 constexpr int kSlwsThreads = 256;
 constexpr int kBatch = 64;         // lookups fetched per round
-constexpr int kChunkBags = 8192;   // bags per pre-summed chunk
-constexpr int kMaxChunks = 16384;  // workspace entries (int64 each)
+constexpr int kChunkBags = 4096;   // bags per pre-summed chunk
+constexpr int kMaxChunks = 32768;  // workspace entries (int64 each)
 
 struct SlwsArgs {
   void *dest;
@@ -47,6 +59,9 @@ struct SlwsArgs {
   int32_t out_cols;
   int32_t out16, w16, idx64;
 };
+
+typedef uint8_t __attribute__((address_space(1))) global_u8;
+typedef unsigned short __attribute__((address_space(1))) global_u16;
 
 template <int LPB> __device__ __forceinline__ int bcast_i(int v, int j) {
   if constexpr (LPB == 64) {
@@ -84,23 +99,38 @@ __device__ __forceinline__ float accumulate(float acc, float w, float s,
   }
 }
 
-template <int LPB, int BPL, bool IS4, bool SO16, bool ACC16>
-__global__ __launch_bounds__(kSlwsThreads) void slws_kernel(SlwsArgs a) {
-  constexpr int kGroups = kSlwsThreads / LPB;      // bags per block
-  constexpr int kColsPerByte = IS4 ? 2 : 1;
-  constexpr int kColsPerLane = BPL * kColsPerByte;
-  __shared__ long long s_part[kSlwsThreads / 64];
-  __shared__ int s_own[kGroups];
+// Sum of v over the 64 lanes of the wave, returned wave-uniform. Lanes are
+// combined inside each row of 16 with DPP moves (no LDS round trip), the four
+// row totals are read out as scalars.
+__device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
+  int x = (int)v;
+  x += __builtin_amdgcn_update_dpp(0, x, 0xB1, 0xf, 0xf, true);  // quad_perm [1,0,3,2]
+  x += __builtin_amdgcn_update_dpp(0, x, 0x4E, 0xf, 0xf, true);  // quad_perm [2,3,0,1]
+  x += __builtin_amdgcn_update_dpp(0, x, 0x141, 0xf, 0xf, true); // row_half_mirror
+  x += __builtin_amdgcn_update_dpp(0, x, 0x140, 0xf, 0xf, true); // row_mirror
+  return (uint32_t)__builtin_amdgcn_readlane(x, 0) +
+         (uint32_t)__builtin_amdgcn_readlane(x, 16) +
+         (uint32_t)__builtin_amdgcn_readlane(x, 32) +
+         (uint32_t)__builtin_amdgcn_readlane(x, 48);
+}
 
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int sub = tid % LPB;                        // lane within the bag group
-  const int grp = tid / LPB;
-  const long long first_bag = (long long)blockIdx.x * kGroups;
-  const long long bag = first_bag + grp;
+__device__ __forceinline__ uint32_t clamp_len(int v) {
+  return v > 0 ? (uint32_t)v : 0u;
+}
 
-  long long start = 0;
-  int len = 0;
+// Position of the first lookup of `bag` in the index list and its length.
+// Lengths mode: exclusive prefix sum of the clamped lengths in front of the
+// block (summed by the block itself, all loads in one memory round trip) plus
+// the lengths of the block's earlier bags. Sums inside a chunk are 32-bit:
+// positions are checked against num_indices before any use, so absurd lengths
+// cannot cause an out-of-range read. Offsets mode: read off the offsets vector.
+template <int kGroups>
+__device__ __forceinline__ void bag_span(const SlwsArgs &a, int tid, int grp,
+                                         long long bag, long long first_bag,
+                                         long long *s_part, int *s_own,
+                                         long long &start, int &len) {
+  start = 0;
+  len = 0;
   if (a.offsets) {
     if (bag < a.segments) {
       start = a.offsets[bag];
@@ -110,48 +140,71 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_kernel(SlwsArgs a) {
       len = end > start ? (int)(end - start) : 0;
     }
   } else {
-    // exclusive prefix sum of the clamped lengths in front of this block
     const long long chunk = first_bag / kChunkBags;
     const long long lo = chunk * kChunkBags;
-    long long below = 0;
     const int32_t *lbase = a.lengths + lo;
     const int n_before = (int)(first_bag - lo); // < kChunkBags, multiple of 4
+    uint32_t part = 0;
     if ((((uintptr_t)lbase) & 15) == 0) {
-      // all loads issued before the first add: one memory round trip
       constexpr int kVecTrips = kChunkBags / 4 / kSlwsThreads;
       const int4 *l4 = reinterpret_cast<const int4 *>(lbase);
       const int nvec = n_before / 4;
-      int4 x[kVecTrips];
+      if (nvec > 0) {
+        // every trip loads (indices past the end re-read the last vector and
+        // are masked out), so all loads are in flight together
+        int4 x[kVecTrips];
 #pragma unroll
-      for (int u = 0; u < kVecTrips; u++) {
-        const int v = tid + u * kSlwsThreads;
-        x[u] = v < nvec ? l4[v] : make_int4(0, 0, 0, 0);
+        for (int u = 0; u < kVecTrips; u++)
+          x[u] = l4[min(tid + u * kSlwsThreads, nvec - 1)];
+#pragma unroll
+        for (int u = 0; u < kVecTrips; u++) {
+          const uint32_t t = clamp_len(x[u].x) + clamp_len(x[u].y) +
+                             clamp_len(x[u].z) + clamp_len(x[u].w);
+          part += (tid + u * kSlwsThreads < nvec) ? t : 0u;
+        }
       }
-#pragma unroll
-      for (int u = 0; u < kVecTrips; u++)
-        below += (long long)max(x[u].x, 0) + max(x[u].y, 0) + (long long)max(x[u].z, 0) + max(x[u].w, 0);
     } else {
-      for (int i = tid; i < n_before; i += kSlwsThreads) below += max(lbase[i], 0);
+      for (int i = tid; i < n_before; i += kSlwsThreads) part += clamp_len(lbase[i]);
     }
+    long long below = 0;
     if (a.chunk_sums) {
       for (long long c = tid; c < chunk; c += kSlwsThreads) below += a.chunk_sums[c];
+      below = (long long)wave_sum_u32((uint32_t)below) +
+              ((long long)wave_sum_u32((uint32_t)(below >> 32)) << 32);
     }
     if (tid < kGroups) {
-      long long b = first_bag + tid;
-      int v = b < a.segments ? a.lengths[b] : 0;
-      s_own[tid] = v > 0 ? v : 0;
+      const long long b = first_bag + tid;
+      s_own[tid] = (int)min(clamp_len(b < a.segments ? a.lengths[b] : 0),
+                            0x7fffffffu);
     }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) below += __shfl_down(below, off, 64);
-    if (lane == 0) s_part[tid >> 6] = below;
+    below += wave_sum_u32(part);
+    if ((tid & 63) == 0) s_part[tid >> 6] = below;
     __syncthreads();
-    start = 0;
 #pragma unroll
     for (int w = 0; w < kSlwsThreads / 64; w++) start += s_part[w];
     for (int g = 0; g < grp; g++) start += s_own[g];
     len = s_own[grp];
   }
   if (bag >= a.segments) len = 0;
+}
+
+template <int LPB, int BPL, bool IS4, bool SO16, bool ACC16>
+__global__ __launch_bounds__(kSlwsThreads) void slws_kernel(SlwsArgs a) {
+  constexpr int kGroups = kSlwsThreads / LPB;      // bags per block
+  constexpr int kColsPerByte = IS4 ? 2 : 1;
+  constexpr int kColsPerLane = BPL * kColsPerByte;
+  __shared__ long long s_part[kSlwsThreads / 64];
+  __shared__ int s_own[kGroups];
+
+  const int tid = threadIdx.x;
+  const int sub = tid % LPB;                        // lane within the bag group
+  const int grp = tid / LPB;
+  const long long first_bag = (long long)blockIdx.x * kGroups;
+  const long long bag = first_bag + grp;
+
+  long long start = 0;
+  int len = 0;
+  bag_span<kGroups>(a, tid, grp, bag, first_bag, s_part, s_own, start, len);
 
   const int n_passes = (a.data_bytes + LPB * BPL - 1) / (LPB * BPL);
   for (int pass = 0; pass < n_passes; pass++) {
@@ -253,7 +306,179 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_kernel(SlwsArgs a) {
         float *d = reinterpret_cast<float *>(a.dest) + o0;
         if (kColsPerLane == 2 && col0 + 1 < a.out_cols &&
             ((((uintptr_t)d) & 7) == 0)) {
-          *reinterpret_cast<float2 *>(d) = make_float2(acc[0], acc[1]);
+          *reinterpret_cast<float2 *>(d) =
+              make_float2(acc[0], acc[kColsPerLane - 1]);
+        } else {
+#pragma unroll
+          for (int c = 0; c < kColsPerLane; c++)
+            if (col0 + c < a.out_cols) d[c] = acc[c];
+        }
+      }
+    }
+  }
+}
+
+// Orders this wave's LDS writes before its later LDS reads of other lanes'
+// slots. LDS operations of one wave execute in order; the fences keep the
+// compiler from moving them across.
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// One bag per wavefront. OFF32: every row's byte offset fits 32 bits, so row
+// addresses are formed as a uniform base plus a 32-bit per-lane offset.
+template <int BPL, bool IS4, bool SO16, bool ACC16, bool OFF32>
+__global__ __launch_bounds__(kSlwsThreads) void slws_wave_kernel(SlwsArgs a) {
+  constexpr int kGroups = kSlwsThreads / 64;
+  constexpr int kColsPerByte = IS4 ? 2 : 1;
+  constexpr int kColsPerLane = BPL * kColsPerByte;
+  constexpr int kGroup = 4;   // lookups handled under one uniform branch
+  __shared__ long long s_part[kGroups];
+  __shared__ int s_own[kGroups];
+  // per wave, per lookup of the batch: {row offset or row, weight, scale, offset}
+  __shared__ int4 s_look[kGroups][kBatch];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const long long first_bag = (long long)blockIdx.x * kGroups;
+  const long long bag = first_bag + wave;
+
+  long long start_v = 0;
+  int len_v = 0;
+  bag_span<kGroups>(a, tid, wave, bag, first_bag, s_part, s_own, start_v, len_v);
+  // wave-uniform from here on: keep them in scalar registers
+  const int len = __builtin_amdgcn_readfirstlane(len_v);
+  const long long start =
+      ((long long)__builtin_amdgcn_readfirstlane((int)(start_v >> 32)) << 32) |
+      (unsigned int)__builtin_amdgcn_readfirstlane((int)start_v);
+  int4 *look = s_look[wave];
+
+  const int n_passes = (a.data_bytes + 64 * BPL - 1) / (64 * BPL);
+  for (int pass = 0; pass < n_passes; pass++) {
+    const int byte0 = (pass * 64 + lane) * BPL;
+    const bool lane_live = byte0 < a.data_bytes;
+    // lanes past the end of the row read its first bytes and store nothing
+    const uint32_t lane_off = lane_live ? (uint32_t)byte0 : 0u;
+    float acc[kColsPerLane];
+#pragma unroll
+    for (int c = 0; c < kColsPerLane; c++) acc[c] = 0.0f;
+
+    for (int base = 0; base < len; base += kBatch) {
+      const int cnt = min(kBatch, len - base);
+      // round 1: lane j fetches lookup j of the batch
+      int my_key;
+      {
+        const long long pos = start + base + lane;
+        long long row = -1;
+        float w = 0.0f;
+        if (lane < cnt && pos < a.num_indices) {
+          row = a.idx64 ? reinterpret_cast<const long long *>(a.indices)[pos]
+                        : (long long)reinterpret_cast<const int *>(a.indices)[pos];
+          if (!a.weights) {
+            w = 1.0f;
+          } else if (a.w16) {
+            w = __half2float(reinterpret_cast<const __half *>(a.weights)[pos]);
+          } else {
+            w = reinterpret_cast<const float *>(a.weights)[pos];
+          }
+        }
+        float s = 0.0f, o = 0.0f;
+        if (row >= 0 && row < a.data_rows) {
+          const uint8_t *so = a.data + row * a.in_line + a.data_bytes;
+          if constexpr (SO16) {
+            uint32_t v = load_u32_any(so);
+            s = __half2float(__ushort_as_half((unsigned short)(v & 0xffff)));
+            o = __half2float(__ushort_as_half((unsigned short)(v >> 16)));
+          } else {
+            s = __uint_as_float(load_u32_any(so));
+            o = __uint_as_float(load_u32_any(so + 4));
+          }
+        } else {
+          row = 0; // skipped lookup: reads row 0, contributes w * 0
+          w = 0.0f;
+        }
+        my_key = OFF32 ? (int)(uint32_t)(row * a.in_line) : (int)row;
+        look[lane] = make_int4(my_key, __float_as_int(w), __float_as_int(s),
+                               __float_as_int(o));
+      }
+      wave_lds_sync();
+      // round 2: all row reads of the batch in flight before the first use.
+      // Lookups are taken four at a time under one uniform branch; slots
+      // beyond cnt hold {row 0, w 0, scale 0, offset 0} and add exactly +0.
+      uint32_t q[kBatch];
+#pragma unroll
+      for (int g = 0; g < kBatch / kGroup; g++) {
+        if (g * kGroup < cnt) {
+          // An opaque copy of the 32-bit lane offset keeps its widening next
+          // to the loads, which lets them use the scalar-base + 32-bit
+          // vector-offset addressing form (global address space).
+          uint32_t off = lane_off;
+          asm volatile("" : "+v"(off));
+#pragma unroll
+          for (int u = 0; u < kGroup; u++) {
+            const int j = g * kGroup + u;
+            const int key = __builtin_amdgcn_readlane(my_key, j);
+            // uniform row base (kept in scalar registers) + per-lane offset
+            const uint8_t *rowp;
+            if constexpr (OFF32) {
+              rowp = a.data + (uint32_t)key;
+            } else {
+              rowp = a.data + (long long)key * a.in_line;
+            }
+            asm volatile("" : "+s"(rowp));
+            const global_u8 *p = (const global_u8 *)rowp + off;
+            if constexpr (BPL == 2) {
+              q[j] = *(const global_u16 *)p;
+            } else {
+              q[j] = *p;
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int g = 0; g < kBatch / kGroup; g++) {
+        if (g * kGroup < cnt) {
+          int4 r[kGroup];
+#pragma unroll
+          for (int u = 0; u < kGroup; u++) r[u] = look[g * kGroup + u];
+#pragma unroll
+          for (int u = 0; u < kGroup; u++) {
+            const int j = g * kGroup + u;
+            const float w = __int_as_float(r[u].y), s = __int_as_float(r[u].z),
+                        o = __int_as_float(r[u].w);
+#pragma unroll
+            for (int b = 0; b < BPL; b++) {
+              const uint32_t byte = (q[j] >> (8 * b)) & 0xff;
+              if constexpr (IS4) {
+                acc[2 * b] = accumulate<ACC16>(acc[2 * b], w, s, o, byte & 15);
+                acc[2 * b + 1] = accumulate<ACC16>(acc[2 * b + 1], w, s, o, byte >> 4);
+              } else {
+                acc[b] = accumulate<ACC16>(acc[b], w, s, o, byte);
+              }
+            }
+          }
+        }
+      }
+      wave_lds_sync(); // slots are rewritten by the next batch
+    }
+
+    if (bag < a.segments && lane_live) {
+      const int col0 = byte0 * kColsPerByte;
+      const long long o0 = bag * (long long)a.out_cols + col0;
+      if (a.out16) {
+        __half *d = reinterpret_cast<__half *>(a.dest) + o0;
+#pragma unroll
+        for (int c = 0; c < kColsPerLane; c++)
+          if (col0 + c < a.out_cols) d[c] = __float2half_rn(acc[c]);
+      } else {
+        float *d = reinterpret_cast<float *>(a.dest) + o0;
+        if (kColsPerLane == 2 && col0 + 1 < a.out_cols &&
+            ((((uintptr_t)d) & 7) == 0)) {
+          *reinterpret_cast<float2 *>(d) =
+              make_float2(acc[0], acc[kColsPerLane - 1]);
         } else {
 #pragma unroll
           for (int c = 0; c < kColsPerLane; c++)
@@ -322,6 +547,31 @@ static void launch_kind(int kind, bool acc16, dim3 grid, hipStream_t st,
     break;
   }
 #undef MI355X_SLWS_LAUNCH
+}
+
+template <int BPL, bool OFF32>
+static void launch_wave_kind(int kind, bool acc16, dim3 grid, hipStream_t st,
+                             const SlwsArgs &a) {
+#define MI355X_SLWS_WAVE(IS4, SO16, ACC16)                                     \
+  hipLaunchKernelGGL((slws_wave_kernel<BPL, IS4, SO16, ACC16, OFF32>), grid,   \
+                     dim3(kSlwsThreads), 0, st, a)
+  switch (kind) {
+  case MI355X_FUSED_U8_F32:
+    MI355X_SLWS_WAVE(false, false, false);
+    break;
+  case MI355X_FUSED_U8_F16:
+    if (acc16) MI355X_SLWS_WAVE(false, true, true);
+    else MI355X_SLWS_WAVE(false, true, false);
+    break;
+  case MI355X_FUSED_U4_F16:
+    if (acc16) MI355X_SLWS_WAVE(true, true, true);
+    else MI355X_SLWS_WAVE(true, true, false);
+    break;
+  default:
+    MI355X_SLWS_WAVE(true, false, false);
+    break;
+  }
+#undef MI355X_SLWS_WAVE
 }
 
 static int slws_dispatch(void *dest, int out_is_f16, const uint8_t *data,
@@ -396,10 +646,13 @@ static int slws_dispatch(void *dest, int out_is_f16, const uint8_t *data,
   const size_t blocks = (out_rows + groups - 1) / groups;
   MI355X_REQUIRE(blocks < 0x7fffffffu, "too many bags");
   dim3 grid((unsigned)blocks);
-  if (!even) launch_kind<64, 1>(kind, acc16, grid, st, a);
-  else if (lpb == 16) launch_kind<16, 2>(kind, acc16, grid, st, a);
+  const bool off32 = (unsigned long long)data_rows * in_line_size <= 0xffffffffull;
+  if (lpb == 16) launch_kind<16, 2>(kind, acc16, grid, st, a);
   else if (lpb == 32) launch_kind<32, 2>(kind, acc16, grid, st, a);
-  else launch_kind<64, 2>(kind, acc16, grid, st, a);
+  else if (!even && off32) launch_wave_kind<1, true>(kind, acc16, grid, st, a);
+  else if (!even) launch_wave_kind<1, false>(kind, acc16, grid, st, a);
+  else if (off32) launch_wave_kind<2, true>(kind, acc16, grid, st, a);
+  else launch_wave_kind<2, false>(kind, acc16, grid, st, a);
   return check_launch("frwq_slws");
 }
 

@@ -88,6 +88,22 @@ int mi355x_event_record(void *event, void *stream);
 int mi355x_event_sync(void *event);
 int mi355x_event_elapsed_ms(void *start, void *stop, float *ms);
 
+/* ---- launch graphs ---------------------------------------------------------- */
+/* A compiled function is a fixed sequence of kernel launches on fixed
+ * addresses (Glow plans all memory statically), so the sequence can be
+ * recorded once and replayed per inference without paying the host-side
+ * launch cost of every kernel; replaces the per-instruction dispatch loop of
+ * LLVMCompiledFunction::execute / jitmain (reference
+ * lib/LLVMIRCodeGen/LLVMCompiledFunction.cpp:73-150). Capture needs a stream
+ * made by mi355x_stream_create (not the default stream). Entry points that
+ * allocate on first use (mi355x_frwq_slws with more than 4096 bags) must have
+ * run once on the device before they are captured. */
+typedef struct mi355x_graph mi355x_graph;
+int mi355x_graph_begin_capture(void *stream);
+int mi355x_graph_end_capture(void *stream, mi355x_graph **graph);
+int mi355x_graph_launch(mi355x_graph *graph, void *stream);
+int mi355x_graph_destroy(mi355x_graph *graph);
+
 /* ---- static memory plan ---------------------------------------------------- */
 /* One HBM allocation per compiled function laid out as
  * constants | mutable (placeholders) | activations with the byte offsets
