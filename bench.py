@@ -147,6 +147,9 @@ def bench_fc(capi, cases, M, K, N, steps, warmup, seed=5):
     d = {k: capi.to_device(np.ascontiguousarray(v)) for k, v in c.items()
          if isinstance(v, np.ndarray)}
     d_out = capi.DeviceBuffer.empty((M, N), np.int8)
+    # weights are constants: their row sums are formed once, outside the steps
+    d_sums = capi.DeviceBuffer.empty((N,), np.int32)
+    capi.launch_rowsum_i8(d_sums, d["w"], N, K)
 
     def step(_, stream):
         capi.launch_rwq_fc_i8(d_out, d["x"], d["w"], d["bias"], False,
@@ -154,7 +157,7 @@ def bench_fc(capi, cases, M, K, N, steps, warmup, seed=5):
                               d["bias_scale"], d["out_pre"], d["out_post"],
                               d["out_scale"], M, K, N, c["out_offset"],
                               c["in_offset"], c["bias_offset"], True,
-                              stream=stream)
+                              w_row_sums=d_sums, stream=stream)
 
     sec = timed_launches(capi, step, steps, warmup)
     ops = 2.0 * M * N * K
@@ -173,6 +176,8 @@ def bench_conv(capi, cases, steps, warmup):
     d = {k: capi.to_device(np.ascontiguousarray(v)) for k, v in c.items()
          if isinstance(v, np.ndarray)}
     d_out = capi.DeviceBuffer.empty((g.N, g.OH, g.OW, g.OC), np.int8)
+    d_sums = capi.DeviceBuffer.empty((g.OC,), np.int32)
+    capi.launch_rowsum_i8(d_sums, d["filt"], g.OC, c["filt"].size // g.OC)
 
     def step(_, stream):
         capi.launch_cwq_conv2d_i8(d_out, d["x"], d["filt"], d["bias"], False, g,
@@ -180,7 +185,8 @@ def bench_conv(capi, cases, steps, warmup):
                                   d["f_offsets"], d["b_offsets"], d["bias_pre"],
                                   d["bias_post"], d["bias_scale"], d["out_pre"],
                                   d["out_post"], d["out_scale"], c["act"],
-                                  c["act_args"], True, stream=stream)
+                                  c["act_args"], True, f_row_sums=d_sums,
+                                  stream=stream)
 
     sec = timed_launches(capi, step, steps, warmup)
     ops = 2.0 * g.N * g.OH * g.OW * g.OC * g.KH * g.KW * g.IC

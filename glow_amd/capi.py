@@ -33,7 +33,8 @@ EXPORTS = [
     "mi355x_quantize_scale_offset_32to8", "mi355x_choose_quantization_params",
     "mi355x_fused_row_bytes", "mi355x_fused_rowwise_quantize_host",
     "mi355x_rowwise_quantize_i8_host", "mi355x_quantize_i8",
-    "mi355x_dequantize_i8", "mi355x_rescale_i8", "mi355x_rwq_fc_i8",
+    "mi355x_dequantize_i8", "mi355x_rescale_i8", "mi355x_rowsum_i8",
+    "mi355x_rwq_fc_i8",
     "mi355x_fc_i8", "mi355x_matmul_i8", "mi355x_transpose2d_i8",
     "mi355x_cwq_conv2d_i8", "mi355x_conv2d_i8", "mi355x_frwq_slws",
     "mi355x_embedding_bag_rowwise_offsets",
@@ -380,29 +381,35 @@ def launch_rescale_i8(dst, src, n, out_offset, in_offset, pre, post, scale,
                                   _i32(scale), _vp(stream)))
 
 
+def launch_rowsum_i8(sums, rows, n_rows, K, stream=None):
+    check(lib().mi355x_rowsum_i8(_vp(sums), _vp(rows), _sz(n_rows), _sz(K),
+                                 _vp(stream)))
+
+
 def launch_rwq_fc_i8(out, x, w, bias, bias_is_i8, w_offsets, bias_pre,
                      bias_post, bias_scale, out_pre, out_post, out_scale, M, K,
                      N, out_offset, in_offset, bias_offset,
-                     w_offsets_all_zero=False, stream=None):
+                     w_offsets_all_zero=False, w_row_sums=None, stream=None):
     check(lib().mi355x_rwq_fc_i8(
         _vp(out), _vp(x), _vp(w), _vp(bias), C.c_int(bias_is_i8),
         _vp(w_offsets), _vp(bias_pre), _vp(bias_post), _vp(bias_scale),
         _vp(out_pre), _vp(out_post), _vp(out_scale), _sz(M), _sz(K), _sz(N),
         _i32(out_offset), _i32(in_offset), _i32(bias_offset),
-        C.c_int(bool(w_offsets_all_zero)), _vp(stream)))
+        C.c_int(bool(w_offsets_all_zero)), _vp(w_row_sums), _vp(stream)))
 
 
 def launch_cwq_conv2d_i8(out, x, filt, bias, bias_is_i8, geom, out_offset,
                          in_offset, f_offsets, b_offsets, bias_pre, bias_post,
                          bias_scale, out_pre, out_post, out_scale, act,
-                         act_args, f_offsets_all_zero=False, stream=None):
+                         act_args, f_offsets_all_zero=False, f_row_sums=None,
+                         stream=None):
     aa = (C.c_int32 * 3)(*(list(act_args) + [0, 0, 0])[:3])
     check(lib().mi355x_cwq_conv2d_i8(
         _vp(out), _vp(x), _vp(filt), _vp(bias), C.c_int(bias_is_i8),
         C.byref(geom), _i32(out_offset), _i32(in_offset), _vp(f_offsets),
         _vp(b_offsets), _vp(bias_pre), _vp(bias_post), _vp(bias_scale),
         _vp(out_pre), _vp(out_post), _vp(out_scale), _i32(act), aa,
-        C.c_int(bool(f_offsets_all_zero)), _vp(stream)))
+        C.c_int(bool(f_offsets_all_zero)), _vp(f_row_sums), _vp(stream)))
 
 
 def launch_frwq_slws(dest, out_is_f16, data, data_rows, kind, weights,
@@ -463,9 +470,28 @@ def _bias_dev(bias):
     return to_device(bias.astype(np.int32)), 0
 
 
+def rowsum_i8(rows):
+    rows = np.ascontiguousarray(rows, np.int8)
+    n, K = rows.shape[0], int(np.prod(rows.shape[1:]))
+    d_rows = to_device(rows)
+    d_sums = DeviceBuffer.empty((n,), np.int32)
+    launch_rowsum_i8(d_sums, d_rows, n, K)
+    return d_sums.numpy()
+
+
+def _row_sums_dev(d_rows, n, K, wanted):
+    """Device vector of weight row sums when `wanted`, else None (the kernel
+    then forms them itself)."""
+    if not wanted:
+        return None
+    d_sums = DeviceBuffer.empty((n,), np.int32)
+    launch_rowsum_i8(d_sums, d_rows, n, K)
+    return d_sums
+
+
 def rwq_fc_i8(x, w_nk, bias, w_offsets, bias_pre, bias_post, bias_scale,
               out_pre, out_post, out_scale, out_offset, in_offset, bias_offset,
-              w_offsets_all_zero=None):
+              w_offsets_all_zero=None, precomputed_sums=True):
     x = np.ascontiguousarray(x, np.int8)
     w_nk = np.ascontiguousarray(w_nk, np.int8)
     M, K = x.shape
@@ -477,13 +503,14 @@ def rwq_fc_i8(x, w_nk, bias, w_offsets, bias_pre, bias_post, bias_scale,
     vs = [_dev_i32(v) for v in (w_offsets, bias_pre, bias_post, bias_scale,
                                 out_pre, out_post, out_scale)]
     d_out = DeviceBuffer.empty((M, N), np.int8)
+    d_sums = _row_sums_dev(d_w, N, K, precomputed_sums)
     launch_rwq_fc_i8(d_out, d_x, d_w, d_b, b8, *vs, M, K, N, out_offset,
-                     in_offset, bias_offset, w_offsets_all_zero)
+                     in_offset, bias_offset, w_offsets_all_zero, d_sums)
     return d_out.numpy()
 
 
 def fc_i8(x, w_kn, bias, out_offset, in_offset, w_offset, bias_offset, biasP,
-          outP):
+          outP, precomputed_sums=False):
     x = np.ascontiguousarray(x, np.int8)
     w_kn = np.ascontiguousarray(w_kn, np.int8)
     M, K = x.shape
@@ -492,11 +519,17 @@ def fc_i8(x, w_kn, bias, out_offset, in_offset, w_offset, bias_offset, biasP,
     d_ws = DeviceBuffer.empty((N, K), np.int8)
     d_b, b8 = _bias_dev(bias)
     d_out = DeviceBuffer.empty((M, N), np.int8)
+    repack, d_sums = 1, None
+    if precomputed_sums:  # what a backend does once at load time
+        check(lib().mi355x_transpose2d_i8(_vp(d_ws), _vp(d_w), _sz(K), _sz(N),
+                                          _vp(None)))
+        d_sums = _row_sums_dev(d_ws, N, K, True)
+        repack = 0
     check(lib().mi355x_fc_i8(
-        _vp(d_out), _vp(d_x), _vp(d_w), _vp(d_ws), C.c_int(1), _vp(d_b),
+        _vp(d_out), _vp(d_x), _vp(d_w), _vp(d_ws), C.c_int(repack), _vp(d_b),
         C.c_int(b8), _sz(M), _sz(K), _sz(N), _i32(out_offset), _i32(in_offset),
         _i32(w_offset), _i32(bias_offset), *[_i32(v) for v in biasP],
-        *[_i32(v) for v in outP], _vp(None)))
+        *[_i32(v) for v in outP], _vp(d_sums), _vp(None)))
     return d_out.numpy()
 
 
@@ -526,7 +559,8 @@ def transpose2d_i8(a):
 
 def cwq_conv2d_i8(x, filt, bias, geom, out_offset, in_offset, f_offsets,
                   b_offsets, bias_pre, bias_post, bias_scale, out_pre, out_post,
-                  out_scale, act=ACT_NONE, act_args=(), f_offsets_all_zero=None):
+                  out_scale, act=ACT_NONE, act_args=(), f_offsets_all_zero=None,
+                  precomputed_sums=True):
     g = _geom(geom)
     x = np.ascontiguousarray(x, np.int8)
     filt = np.ascontiguousarray(filt, np.int8)
@@ -537,13 +571,15 @@ def cwq_conv2d_i8(x, filt, bias, geom, out_offset, in_offset, f_offsets,
     vs = [_dev_i32(v) for v in (f_offsets, b_offsets, bias_pre, bias_post,
                                 bias_scale, out_pre, out_post, out_scale)]
     d_out = DeviceBuffer.empty((g.N, g.OH, g.OW, g.OC), np.int8)
+    d_sums = _row_sums_dev(d_f, g.OC, filt.size // g.OC, precomputed_sums)
     launch_cwq_conv2d_i8(d_out, d_x, d_f, d_b, b8, g, out_offset, in_offset,
-                         *vs, act, act_args, f_offsets_all_zero)
+                         *vs, act, act_args, f_offsets_all_zero, d_sums)
     return d_out.numpy()
 
 
 def conv2d_i8(x, filt, bias, geom, out_offset, in_offset, filter_offset,
-              bias_offset, biasP, outP, act=ACT_NONE, act_args=()):
+              bias_offset, biasP, outP, act=ACT_NONE, act_args=(),
+              precomputed_sums=False):
     g = _geom(geom)
     x = np.ascontiguousarray(x, np.int8)
     filt = np.ascontiguousarray(filt, np.int8)
@@ -551,11 +587,12 @@ def conv2d_i8(x, filt, bias, geom, out_offset, in_offset, filter_offset,
     d_b, b8 = _bias_dev(bias)
     d_out = DeviceBuffer.empty((g.N, g.OH, g.OW, g.OC), np.int8)
     aa = (C.c_int32 * 3)(*(list(act_args) + [0, 0, 0])[:3])
+    d_sums = _row_sums_dev(d_f, g.OC, filt.size // g.OC, precomputed_sums)
     check(lib().mi355x_conv2d_i8(
         _vp(d_out), _vp(d_x), _vp(d_f), _vp(d_b), C.c_int(b8), C.byref(g),
         _i32(out_offset), _i32(in_offset), _i32(filter_offset),
         _i32(bias_offset), *[_i32(v) for v in biasP], *[_i32(v) for v in outP],
-        _i32(act), aa, _vp(None)))
+        _i32(act), aa, _vp(d_sums), _vp(None)))
     return d_out.numpy()
 
 

@@ -40,6 +40,16 @@ struct ConvRows {
     r.iw0 = ow * strideW - padL;
     return r;
   }
+  // address of the 16 bytes A[m][k..k+15] of an existing row (ICg % 16 == 0):
+  // inside the image, or a chunk of input-offset bytes for a padding tap
+  __device__ __forceinline__ const int8_t *chunk_ptr(const Row &r, int k) const {
+    const int tap = k / ICg, c = k - tap * ICg;
+    const int fx = tap / KW, fy = tap - fx * KW;
+    const int ih = r.ih0 + fx * dilH, iw = r.iw0 + fy * dilW;
+    if (ih < 0 || iw < 0 || ih >= IH || iw >= IW)
+      return reinterpret_cast<const int8_t *>(g_fill_table.b) + ((fill & 0xff) << 4);
+    return r.img + ((long long)ih * IW + iw) * IC + c;
+  }
   // 16 bytes A[m][k..k+15]; ALIGNED needs ICg % 16 == 0 so a chunk never
   // straddles a tap, and 16-byte aligned pixels.
   template <bool ALIGNED>
@@ -121,10 +131,10 @@ static int conv_common(int8_t *out, const int8_t *in, const int8_t *filter,
   const bool al_a = (ICg % 16 == 0) && (g->IC % 16 == 0) &&
                     ((((uintptr_t)in) & 15) == 0);
   const bool al_b = (K % 16 == 0) && ((((uintptr_t)filter) & 15) == 0);
-  const bool need_sb = ep.a_off != 0;
+  const bool need_sb = ep.a_off != 0 && !ep.sum_b;
   return gemm_dispatch(A, B, ep, (int)M, OCg, (int)K, g->group,
                        (long long)OCg * K, need_sa, need_sb, al_a && al_b,
-                       al_a && al_b, as_stream(stream));
+                       as_stream(stream));
 }
 
 static void set_act(Epilogue &ep, int32_t act_type, const int32_t *act_args) {
@@ -157,7 +167,7 @@ int mi355x_cwq_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
                          const int32_t *out_pre, const int32_t *out_post,
                          const int32_t *out_scale, int32_t act_type,
                          const int32_t *act_args, int filter_offsets_all_zero,
-                         void *stream) {
+                         const int32_t *filter_row_sums, void *stream) {
   MI355X_REQUIRE(bias && filter_offsets && bias_offsets && bias_pre &&
                      bias_post && bias_scale && out_pre && out_post && out_scale,
                  "NULL per-channel parameter vector");
@@ -178,6 +188,7 @@ int mi355x_cwq_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
   ep.a_off = in_offset;
   ep.out_off = out_offset;
   set_act(ep, act_type, act_args);
+  ep.sum_b = filter_row_sums;
   return conv_common(out, in, filter, geom, ep, !filter_offsets_all_zero,
                      stream);
 }
@@ -189,7 +200,8 @@ int mi355x_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
                      int32_t bias_offset, int32_t bias_pre, int32_t bias_post,
                      int32_t bias_scale, int32_t out_pre, int32_t out_post,
                      int32_t out_scale, int32_t act_type,
-                     const int32_t *act_args, void *stream) {
+                     const int32_t *act_args, const int32_t *filter_row_sums,
+                     void *stream) {
   MI355X_REQUIRE(bias, "bias is NULL");
   MI355X_REQUIRE(shift_ok(bias_pre) && shift_ok(bias_post) &&
                      shift_ok(out_pre) && shift_ok(out_post),
@@ -211,6 +223,7 @@ int mi355x_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
   ep.a_off = in_offset;
   ep.out_off = out_offset;
   set_act(ep, act_type, act_args);
+  ep.sum_b = filter_row_sums;
   return conv_common(out, in, filter, geom, ep, filter_offset != 0, stream);
 }
 

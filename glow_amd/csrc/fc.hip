@@ -26,6 +26,31 @@ __global__ __launch_bounds__(256) void transpose2d_i8_kernel(
   }
 }
 
+// sums[r] = sum_k rows[r][k]; one wavefront per row, 16 bytes per lane and trip.
+__global__ __launch_bounds__(256) void rowsum_i8_kernel(
+    int32_t *__restrict__ sums, const int8_t *__restrict__ rows, long long n_rows,
+    int K, int vec_ok) {
+  const long long r = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= n_rows) return;
+  const int lane = threadIdx.x & 63;
+  const int8_t *p = rows + r * K;
+  int acc = 0;
+  int k = 0;
+  if (vec_ok) {
+    for (; k + 1024 <= K; k += 1024) {
+      const int4 v = *reinterpret_cast<const int4 *>(p + k + lane * 16);
+      acc = __builtin_amdgcn_sdot4(v.x, 0x01010101, acc, false);
+      acc = __builtin_amdgcn_sdot4(v.y, 0x01010101, acc, false);
+      acc = __builtin_amdgcn_sdot4(v.z, 0x01010101, acc, false);
+      acc = __builtin_amdgcn_sdot4(v.w, 0x01010101, acc, false);
+    }
+  }
+  for (int i = k + lane; i < K; i += 64) acc += p[i];
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) acc += __shfl_down(acc, off, 64);
+  if (lane == 0) sums[r] = acc;
+}
+
 static bool aligned_rows(const void *p, size_t ld) {
   return ((((uintptr_t)p) & 15) == 0) && (ld % 16 == 0);
 }
@@ -47,10 +72,10 @@ static int fc_common(int8_t *out, const int8_t *in, const int8_t *w_nk,
   Epilogue ep = ep_in;
   ep.out = out;
   ep.ldc = (long long)N;
-  const bool al_a = aligned_rows(in, K), al_b = aligned_rows(w_nk, K);
-  const bool need_sb = ep.a_off != 0;
+  const bool aligned = aligned_rows(in, K) && aligned_rows(w_nk, K);
+  const bool need_sb = ep.a_off != 0 && !ep.sum_b;
   return gemm_dispatch(A, B, ep, (int)M, (int)N, (int)K, 1, 0, need_sa, need_sb,
-                       al_a, al_b, as_stream(stream));
+                       aligned, as_stream(stream));
 }
 
 } // namespace mi355x
@@ -72,6 +97,18 @@ int mi355x_transpose2d_i8(int8_t *dst, const int8_t *src, size_t rows,
   return check_launch("transpose2d_i8");
 }
 
+int mi355x_rowsum_i8(int32_t *sums, const int8_t *rows, size_t n_rows, size_t K,
+                     void *stream) {
+  if (n_rows == 0) return MI355X_OK;
+  MI355X_REQUIRE(sums && (rows || K == 0), "NULL tensor");
+  MI355X_REQUIRE(K < (1u << 30) && (n_rows + 3) / 4 < 0x7fffffffu,
+                 "matrix too large");
+  hipLaunchKernelGGL(rowsum_i8_kernel, dim3((unsigned)((n_rows + 3) / 4)),
+                     dim3(256), 0, as_stream(stream), sums, rows,
+                     (long long)n_rows, (int)K, (int)aligned_rows(rows, K));
+  return check_launch("rowsum_i8");
+}
+
 int mi355x_rwq_fc_i8(int8_t *out, const int8_t *in, const int8_t *weights,
                      const void *bias, int bias_is_i8,
                      const int32_t *weights_offsets, const int32_t *bias_pre,
@@ -80,7 +117,7 @@ int mi355x_rwq_fc_i8(int8_t *out, const int8_t *in, const int8_t *weights,
                      const int32_t *out_scale, size_t M, size_t K, size_t N,
                      int32_t out_offset, int32_t in_offset,
                      int32_t bias_offset, int weights_offsets_all_zero,
-                     void *stream) {
+                     const int32_t *weights_row_sums, void *stream) {
   if (M == 0 || N == 0) return MI355X_OK;
   MI355X_REQUIRE(out && in && weights && bias, "NULL tensor");
   MI355X_REQUIRE(weights_offsets && bias_pre && bias_post && bias_scale &&
@@ -102,6 +139,7 @@ int mi355x_rwq_fc_i8(int8_t *out, const int8_t *in, const int8_t *weights,
   ep.a_off = in_offset;
   ep.out_off = out_offset;
   ep.act = MI355X_ACT_NONE;
+  ep.sum_b = weights_row_sums;
   return fc_common(out, in, weights, ep, M, K, N, !weights_offsets_all_zero,
                    stream);
 }
@@ -112,7 +150,8 @@ int mi355x_fc_i8(int8_t *out, const int8_t *in, const int8_t *weights_kn,
                  int32_t out_offset, int32_t in_offset, int32_t weights_offset,
                  int32_t bias_offset, int32_t bias_pre, int32_t bias_post,
                  int32_t bias_scale, int32_t out_pre, int32_t out_post,
-                 int32_t out_scale, void *stream) {
+                 int32_t out_scale, const int32_t *weights_row_sums,
+                 void *stream) {
   if (M == 0 || N == 0) return MI355X_OK;
   MI355X_REQUIRE(out && in && weights_nk_workspace && bias, "NULL tensor");
   MI355X_REQUIRE(shift_ok(bias_pre) && shift_ok(bias_post) &&
@@ -139,6 +178,7 @@ int mi355x_fc_i8(int8_t *out, const int8_t *in, const int8_t *weights_kn,
   ep.a_off = in_offset;
   ep.out_off = out_offset;
   ep.act = MI355X_ACT_NONE;
+  ep.sum_b = weights_row_sums;
   return fc_common(out, in, weights_nk_workspace, ep, M, K, N,
                    weights_offset != 0, stream);
 }

@@ -14,11 +14,19 @@
 // with the row sums taken from the operand fragments (v_dot4) while they pass
 // through registers. Everything is exact modulo 2^32, like the CPU loop.
 //
-// Block tile BM x BN, K step 64 bytes, waves own WM x WN sub-tiles. Global ->
-// registers -> LDS with two LDS stages (one barrier per K step); LDS rows are
-// padded to 80 bytes so the 16-byte fragment reads of 16 consecutive rows
-// fall on distinct banks. The int8 results are staged through LDS and leave
-// as 16-byte row segments.
+// Block tile BM x BN, K step 64 bytes, waves own WM x WN sub-tiles. Two main
+// loops share one epilogue:
+//   gemm_i8_dma_kernel  K % 64 == 0 and 16-byte aligned operands. Tiles go
+//       global -> LDS directly (global_load_lds_dwordx4, no staging registers)
+//       through a ring of STAGES LDS buffers, so loads run STAGES-1 K steps
+//       ahead of the matrix cores; one barrier per K step. LDS rows are 64
+//       bytes, unpadded; the 16-byte chunk kc of row r sits at position
+//       kc ^ ((r >> 2) & 3), which makes the fragment reads of 16 consecutive
+//       rows fall on distinct banks.
+//   gemm_i8_kernel      everything else (K tails, unaligned rows, 3-channel
+//       convolutions): global -> registers -> LDS with two stages and rows
+//       padded to 80 bytes.
+// The int8 results are staged through LDS and leave as 16-byte row segments.
 #ifndef GLOW_MI355X_GEMM_I8_H
 #define GLOW_MI355X_GEMM_I8_H
 
@@ -47,6 +55,7 @@ struct Epilogue {
   int bias_is_i8;
   ColParam b_off, bias_pre, bias_post, bias_scale;
   ColParam w_off, out_pre, out_post, out_scale;
+  const int32_t *sum_b; // precomputed sum_k B[n][k] per output column, or NULL
   int32_t a_off;        // offset of the A operand (activations)
   int32_t out_off;
   int32_t act, a0, a1, a2;
@@ -64,6 +73,10 @@ struct DenseRows {
   __device__ __forceinline__ void set_group(int) {}
   __device__ __forceinline__ Row row(int r) const {
     return Row{p + (long long)r * ld, r < rows};
+  }
+  // address of the 16 bytes [k, k+16) of a row that exists
+  __device__ __forceinline__ const int8_t *chunk_ptr(const Row &r, int k) const {
+    return r.base + k;
   }
   template <bool ALIGNED>
   __device__ __forceinline__ int4 load(const Row &r, int k, int K) const {
@@ -100,6 +113,128 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
   tn = in_panel / rows_here;
 }
 
+// Shared epilogue. Accumulator layout of v_mfma_i32_32x32x32_i8: lane l holds
+// column l % 32 and, in register r, row 8*(r/4) + 4*(l/32) + r%4 of the tile.
+// Must be entered after a block barrier (LDS is reused).
+template <int BM, int BN, int WM, int WN, bool NEED_SA, bool NEED_SB,
+          bool LEAKY>
+__device__ __forceinline__ void gemm_epilogue_impl(
+    v16i (&acc)[WM / 32][WN / 32], int (&sa)[WM / 32], int (&sb)[WN / 32],
+    int8_t *lds, const Epilogue &ep, int M, int N, int K, int m0, int n0,
+    int n_base) {
+  constexpr int WAVES_N = BN / WN;
+  constexpr int THREADS = (BM / WM) * (BN / WN) * 64;
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int OUT_STRIDE = BN + 16;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int l32 = lane & 31, lhi = lane >> 5;
+
+  // LDS is free now: [row sums of A per wave | int8 output tile]
+  int32_t *s_sumA = reinterpret_cast<int32_t *>(lds);            // BM ints
+  int8_t *s_out = lds + BM * 4;
+  if constexpr (NEED_SA) {
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+      sa[i] += __shfl_xor(sa[i], 32, 64);
+      // waves of one block row hold identical sums; all may write
+      if (lhi == 0) s_sumA[wm * WM + i * 32 + l32] = sa[i];
+    }
+  }
+  if constexpr (NEED_SB) {
+#pragma unroll
+    for (int j = 0; j < TN; j++) sb[j] += __shfl_xor(sb[j], 32, 64);
+  }
+  __syncthreads();
+
+  // Activation and the final int8 clip as one clamp to [lo, hi]:
+  // clip(min(max(y, a0), a1)) == min(max(y, clip(a0)), clip(a1)), RELU being
+  // the clamp [out_off, +inf) and NONE the clamp (-inf, +inf).
+  int32_t lo = -128, hi = 127;
+  if (ep.act == 1) lo = clip_i8(ep.out_off);
+  if (ep.act == 2) {
+    lo = clip_i8(ep.a0);
+    hi = clip_i8(ep.a1);
+  }
+
+#pragma unroll
+  for (int j = 0; j < TN; j++) {
+    const int nl = n0 + wn * WN + j * 32 + l32;   // column within the group
+    const bool n_ok = nl < N;
+    const int n = n_base + (n_ok ? nl : 0);       // global output column
+    const int32_t woff = ep.w_off.at(n);
+    const int32_t opre = ep.out_pre.at(n), opost = ep.out_post.at(n);
+    const int32_t oscale = ep.out_scale.at(n);
+    uint32_t colc = (uint32_t)K * (uint32_t)ep.a_off * (uint32_t)woff;
+    if constexpr (NEED_SB) {
+      colc -= (uint32_t)ep.a_off * (uint32_t)sb[j];
+    } else if (ep.sum_b) {
+      colc -= (uint32_t)ep.a_off * (uint32_t)ep.sum_b[n];
+    }
+    if (ep.bias) {
+      const int32_t b = ep.bias_is_i8
+                            ? (int32_t) reinterpret_cast<const int8_t *>(ep.bias)[n]
+                            : reinterpret_cast<const int32_t *>(ep.bias)[n];
+      colc += (uint32_t)scale_i32((int32_t)((uint32_t)b - (uint32_t)ep.b_off.at(n)),
+                                  ep.bias_pre.at(n), ep.bias_post.at(n),
+                                  ep.bias_scale.at(n), 0);
+    }
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int ml = wm * WM + i * 32 + (r >> 2) * 8 + lhi * 4 + (r & 3);
+        uint32_t v = (uint32_t)acc[i][j][r] + colc;
+        if constexpr (NEED_SA) v -= (uint32_t)woff * (uint32_t)s_sumA[ml];
+        int32_t y = scale_i32((int32_t)v, opre, opost, oscale, ep.out_off);
+        if constexpr (LEAKY) {
+          if (y < ep.out_off)
+            y = scale_i32((int32_t)((uint32_t)y - (uint32_t)ep.out_off), ep.a0,
+                          ep.a1, ep.a2, ep.out_off);
+        }
+        s_out[ml * OUT_STRIDE + wn * WN + j * 32 + l32] =
+            (int8_t)min(max(y, lo), hi);
+      }
+    }
+  }
+  __syncthreads();
+
+  // coalesced copy-out: 16-byte row segments where the output allows it
+  const int cols_here = min(BN, N - n0);
+  const int rows_here = min(BM, M - m0);
+  int8_t *obase = ep.out + (long long)m0 * ep.ldc + n_base + n0;
+  const bool vec_ok = (cols_here % 16 == 0) && (ep.ldc % 16 == 0) &&
+                      ((((uintptr_t)obase) & 15) == 0);
+  if (vec_ok) {
+    const int segs = cols_here / 16;
+    for (int c = tid; c < rows_here * segs; c += THREADS) {
+      const int r = c / segs, s = c - r * segs;
+      *reinterpret_cast<int4 *>(obase + (long long)r * ep.ldc + s * 16) =
+          *reinterpret_cast<const int4 *>(s_out + r * OUT_STRIDE + s * 16);
+    }
+  } else {
+    for (int c = tid; c < rows_here * cols_here; c += THREADS) {
+      const int r = c / cols_here, s = c - r * cols_here;
+      obase[(long long)r * ep.ldc + s] = s_out[r * OUT_STRIDE + s];
+    }
+  }
+}
+
+template <int BM, int BN, int WM, int WN, bool NEED_SA, bool NEED_SB>
+__device__ __forceinline__ void gemm_epilogue(
+    v16i (&acc)[WM / 32][WN / 32], int (&sa)[WM / 32], int (&sb)[WN / 32],
+    int8_t *lds, const Epilogue &ep, int M, int N, int K, int m0, int n0,
+    int n_base) {
+  if (ep.act == 5) // LEAKY_RELU: rare, kept out of the common instruction stream
+    gemm_epilogue_impl<BM, BN, WM, WN, NEED_SA, NEED_SB, true>(
+        acc, sa, sb, lds, ep, M, N, K, m0, n0, n_base);
+  else
+    gemm_epilogue_impl<BM, BN, WM, WN, NEED_SA, NEED_SB, false>(
+        acc, sa, sb, lds, ep, M, N, K, m0, n0, n_base);
+}
+
 template <int BM, int BN, int WM, int WN, bool NEED_SA, bool NEED_SB,
           bool AL_A, bool AL_B, class ARows>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_i8_kernel(
@@ -113,7 +248,6 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_i8_kernel(
   constexpr int B_CH = BN * CH_ROW / THREADS;
   static_assert(BM * CH_ROW % THREADS == 0 && BN * CH_ROW % THREADS == 0, "");
   constexpr int STAGE = (BM + BN) * kLdsStride;
-  constexpr int OUT_STRIDE = BN + 16;
 
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
 
@@ -232,109 +366,234 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_i8_kernel(
     __syncthreads();
   }
 
-  // ---- epilogue --------------------------------------------------------------
-  // LDS is free now: [row sums of A per wave | int8 output tile]
-  int32_t *s_sumA = reinterpret_cast<int32_t *>(lds);            // BM ints
-  int8_t *s_out = lds + BM * 4;
-  if constexpr (NEED_SA) {
-#pragma unroll
-    for (int i = 0; i < TM; i++) {
-      sa[i] += __shfl_xor(sa[i], 32, 64);
-      // waves of one block row hold identical sums; all may write
-      if (lhi == 0) s_sumA[wm * WM + i * 32 + l32] = sa[i];
-    }
-  }
-  if constexpr (NEED_SB) {
-#pragma unroll
-    for (int j = 0; j < TN; j++) sb[j] += __shfl_xor(sb[j], 32, 64);
-  }
-  __syncthreads();
+  gemm_epilogue<BM, BN, WM, WN, NEED_SA, NEED_SB>(acc, sa, sb, lds, ep, M, N, K,
+                                                  m0, n0, n_base);
+}
 
+// ---- direct-to-LDS main loop ---------------------------------------------------
+
+// 16 bytes per lane from global memory straight into LDS at
+// lds_addr + 16 * lane (M0 carries the wave-uniform LDS address). Issued
+// through inline assembly so that the compiler's own wait-count insertion
+// does not serialise later LDS reads against loads still in flight; the
+// kernel below waits explicitly with dma_wait<N>().
+__device__ __forceinline__ void dma16(const void *gptr, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+               :
+               : "s"(lds_addr), "v"(gptr)
+               : "memory");
+}
+
+// Waits until at most N of this wave's vector-memory operations are pending.
+template <int N> __device__ __forceinline__ void dma_wait() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+// Bytes whose value equals their row index: row v of this table is a 16-byte
+// chunk filled with the byte v. Out-of-image convolution taps are loaded from
+// it (a direct-to-LDS load cannot synthesise a constant).
+struct FillTable {
+  uint8_t b[256 * 16];
+  constexpr FillTable() : b{} {
+    for (int i = 0; i < 256 * 16; i++) b[i] = (uint8_t)(i / 16);
+  }
+};
+__device__ __attribute__((aligned(16))) const FillTable g_fill_table{};
+
+__device__ __forceinline__ uint32_t lds_address(const void *p) {
+  return (uint32_t)(uintptr_t)(
+      (const __attribute__((address_space(3))) void *)p);
+}
+
+template <int BM, int BN, int WM, int WN, int STAGES, bool NEED_SA,
+          bool NEED_SB, class ARows>
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_i8_dma_kernel(
+    ARows A, DenseRows B, Epilogue ep, int M, int N, int K, int tiles_m,
+    int tiles_n, long long b_group_stride, int n_per_group) {
+  constexpr int WAVES_N = BN / WN;
+  constexpr int WAVES = (BM / WM) * (BN / WN);
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int STAGE = (BM + BN) * kBK;             // bytes per ring slot
+  // one load instruction moves a group of 16 rows x 64 bytes
+  constexpr int A_LOADS = BM / 16 / WAVES, B_LOADS = BN / 16 / WAVES;
+  constexpr int LOADS = A_LOADS + B_LOADS;
+  static_assert(BM / 16 % WAVES == 0 && BN / 16 % WAVES == 0, "tile vs waves");
+  static_assert(STAGES >= 2 && (STAGES - 1) * LOADS < 64, "ring depth");
+
+  extern __shared__ __attribute__((aligned(16))) int8_t lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int l32 = lane & 31, lhi = lane >> 5;
+
+  const int grp = blockIdx.y;
+  A.set_group(grp);
+  B.p += (long long)grp * b_group_stride;
+  const int n_base = grp * n_per_group;
+
+  int tm, tn;
+  tile_of_block(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  // Load plan. Lane i of a group load owns row (i >> 2) of the group and the
+  // LDS chunk position (i & 3); the chunk stored there is kc = pos ^ swizzle.
+  const int row_in_grp = lane >> 2;
+  const int kc_lane = ((lane & 3) ^ ((lane >> 4) & 3)) * 16;
+  typename ARows::Row arow[A_LOADS];
+  const int8_t *bptr[B_LOADS];
+  uint32_t a_dst[A_LOADS], b_dst[B_LOADS];
+  const uint32_t lds0 = lds_address(lds);
 #pragma unroll
-  for (int j = 0; j < TN; j++) {
-    const int nl = n0 + wn * WN + j * 32 + l32;   // column within the group
-    const bool n_ok = nl < N;
-    const int n = n_base + (n_ok ? nl : 0);       // global output column
-    const int32_t woff = ep.w_off.at(n);
-    const int32_t opre = ep.out_pre.at(n), opost = ep.out_post.at(n);
-    const int32_t oscale = ep.out_scale.at(n);
-    uint32_t colc = (uint32_t)K * (uint32_t)ep.a_off * (uint32_t)woff;
-    if constexpr (NEED_SB) colc -= (uint32_t)ep.a_off * (uint32_t)sb[j];
-    if (ep.bias) {
-      const int32_t b = ep.bias_is_i8
-                            ? (int32_t) reinterpret_cast<const int8_t *>(ep.bias)[n]
-                            : reinterpret_cast<const int32_t *>(ep.bias)[n];
-      colc += (uint32_t)scale_i32((int32_t)((uint32_t)b - (uint32_t)ep.b_off.at(n)),
-                                  ep.bias_pre.at(n), ep.bias_post.at(n),
-                                  ep.bias_scale.at(n), 0);
+  for (int i = 0; i < A_LOADS; i++) {
+    const int g = i * WAVES + wave;
+    arow[i] = A.row(min(m0 + g * 16 + row_in_grp, M - 1));
+    a_dst[i] = g * 1024;
+  }
+#pragma unroll
+  for (int i = 0; i < B_LOADS; i++) {
+    const int g = i * WAVES + wave;
+    bptr[i] = B.p + (long long)min(n0 + g * 16 + row_in_grp, N - 1) * B.ld + kc_lane;
+    b_dst[i] = BM * kBK + g * 1024;
+  }
+
+  const int KT = K / kBK;
+  // prologue: STAGES-1 tiles in flight (tiles past the end are re-reads of
+  // the last one into slots nobody consumes, which keeps the counts uniform)
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; s++) {
+    const uint32_t slot = lds0 + (uint32_t)s * STAGE;
+    const int k0 = min(s, KT - 1) * kBK;
+#pragma unroll
+    for (int i = 0; i < A_LOADS; i++)
+      dma16(A.chunk_ptr(arow[i], k0 + kc_lane), slot + a_dst[i]);
+#pragma unroll
+    for (int i = 0; i < B_LOADS; i++) dma16(bptr[i] + k0, slot + b_dst[i]);
+  }
+
+  v16i acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+  int sa[TM], sb[TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++) sa[i] = 0;
+#pragma unroll
+  for (int j = 0; j < TN; j++) sb[j] = 0;
+
+  // fragment addresses: row (l & 31) of a 32-row sub-tile, chunk ks*2 + (l>>5)
+  const int swz = (lane >> 2) & 3;
+  int frag_off[kBK / 32];
+#pragma unroll
+  for (int ks = 0; ks < kBK / 32; ks++)
+    frag_off[ks] = l32 * kBK + (((ks * 2 + lhi) ^ swz) << 4);
+  const int a_base = wm * WM * kBK;
+  const int b_base = BM * kBK + wn * WN * kBK;
+
+  static_assert(kBK == 64 && STAGES >= 3, "two 32-byte k slices per stage");
+  v4i af[2][TM], bf[2][TN];
+  // fragment f of a k slice: the TM A fragments, then the TN B fragments
+  auto read_frag = [&](const int8_t *stage, int ks, int buf, int f) {
+    if (f < TM)
+      af[buf][f] = *reinterpret_cast<const v4i *>(stage + a_base + f * 32 * kBK + frag_off[ks]);
+    else
+      bf[buf][f - TM] = *reinterpret_cast<const v4i *>(stage + b_base + (f - TM) * 32 * kBK + frag_off[ks]);
+  };
+  auto issue_load = [&](int nk, int i) {
+    const uint32_t slot = lds0 + (uint32_t)(nk % STAGES) * STAGE;
+    const int k0 = min(nk, KT - 1) * kBK;
+    if (i < A_LOADS)
+      dma16(A.chunk_ptr(arow[i], k0 + kc_lane), slot + a_dst[i]);
+    else
+      dma16(bptr[i - A_LOADS] + k0, slot + b_dst[i - A_LOADS]);
+  };
+  // The MFMAs of one k slice with the memory operations of the next slice
+  // spread between them: a wave issues in order, so a burst of loads that
+  // fills the memory queues would hold back the MFMAs queued behind it.
+  auto multiply = [&](int buf, auto &&between) {
+    if constexpr (NEED_SA) {
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+          sa[i] = __builtin_amdgcn_sdot4(af[buf][i][q], 0x01010101, sa[i], false);
+    }
+    if constexpr (NEED_SB) {
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+          sb[j] = __builtin_amdgcn_sdot4(bf[buf][j][q], 0x01010101, sb[j], false);
     }
 #pragma unroll
-    for (int i = 0; i < TM; i++) {
+    for (int i = 0; i < TM; i++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const int ml = wm * WM + i * 32 + (r >> 2) * 8 + lhi * 4 + (r & 3);
-        uint32_t v = (uint32_t)acc[i][j][r] + colc;
-        if constexpr (NEED_SA) v -= (uint32_t)woff * (uint32_t)s_sumA[ml];
-        int32_t y = scale_i32((int32_t)v, opre, opost, oscale, ep.out_off);
-        y = activation_i32(y, ep.out_off, ep.act, ep.a0, ep.a1, ep.a2);
-        s_out[ml * OUT_STRIDE + wn * WN + j * 32 + l32] = (int8_t)clip_i8(y);
+      for (int j = 0; j < TN; j++) {
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[buf][i], bf[buf][j],
+                                                          acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        between(i * TN + j);
+        __builtin_amdgcn_sched_barrier(0);
       }
-    }
-  }
-  __syncthreads();
+  };
+  constexpr int MFMAS = TM * TN;
+  constexpr int FRAGS = TM + TN;
+  // operation x of n is slotted in after MFMA t when x is in
+  // [t*n/MFMAS, (t+1)*n/MFMAS): spread evenly over the slice
 
-  // coalesced copy-out: 16-byte row segments where the output allows it
-  const int cols_here = min(BN, N - n0);
-  const int rows_here = min(BM, M - m0);
-  int8_t *obase = ep.out + (long long)m0 * ep.ldc + n_base + n0;
-  const bool vec_ok = (cols_here % 16 == 0) && (ep.ldc % 16 == 0) &&
-                      ((((uintptr_t)obase) & 15) == 0);
-  if (vec_ok) {
-    const int segs = cols_here / 16;
-    for (int c = tid; c < rows_here * segs; c += THREADS) {
-      const int r = c / segs, s = c - r * segs;
-      *reinterpret_cast<int4 *>(obase + (long long)r * ep.ldc + s * 16) =
-          *reinterpret_cast<const int4 *>(s_out + r * OUT_STRIDE + s * 16);
-    }
-  } else {
-    for (int c = tid; c < rows_here * cols_here; c += THREADS) {
-      const int r = c / cols_here, s = c - r * cols_here;
-      obase[(long long)r * ep.ldc + s] = s_out[r * OUT_STRIDE + s];
-    }
+  dma_wait<(STAGES - 2) * LOADS>(); // tile 0 has landed
+  __syncthreads();
+#pragma unroll
+  for (int f = 0; f < FRAGS; f++) read_frag(lds, 0, 0, f);
+  for (int kt = 0; kt < KT; kt++) {
+    const int8_t *cur = lds + (kt % STAGES) * STAGE;
+    const int8_t *nxt = lds + ((kt + 1) % STAGES) * STAGE;
+    // slice 0 runs while the fragments of slice 1 arrive
+    multiply(0, [&](int t) {
+#pragma unroll
+      for (int f = t * FRAGS / MFMAS; f < (t + 1) * FRAGS / MFMAS; f++)
+        read_frag(cur, 1, 1, f);
+    });
+    // tile kt+1 has landed once at most STAGES-3 newer tiles are pending; past
+    // the barrier every wave is done reading tile kt-1, whose slot is refilled
+    dma_wait<(STAGES - 3) * LOADS>();
+    __syncthreads();
+    // slice 1 runs while slice 0 of the next tile is read and tile
+    // kt+STAGES-1 is requested
+    multiply(1, [&](int t) {
+#pragma unroll
+      for (int f = t * FRAGS / MFMAS; f < (t + 1) * FRAGS / MFMAS; f++)
+        read_frag(nxt, 0, 0, f);
+#pragma unroll
+      for (int i = t * LOADS / MFMAS; i < (t + 1) * LOADS / MFMAS; i++)
+        issue_load(kt + STAGES - 1, i);
+    });
   }
+  dma_wait<0>(); // drain the re-reads before LDS is reused
+  __syncthreads();
+  gemm_epilogue<BM, BN, WM, WN, NEED_SA, NEED_SB>(acc, sa, sb, lds, ep, M, N, K,
+                                                  m0, n0, n_base);
+}
+
+template <int BM, int BN> constexpr size_t gemm_epilogue_lds_bytes() {
+  return (size_t)BM * 4 + (size_t)BM * (BN + 16);
 }
 
 template <int BM, int BN> constexpr size_t gemm_lds_bytes() {
   constexpr size_t stages = 2 * (size_t)(BM + BN) * kLdsStride;
-  constexpr size_t epi = (size_t)BM * 4 + (size_t)BM * (BN + 16);
+  constexpr size_t epi = gemm_epilogue_lds_bytes<BM, BN>();
   return stages > epi ? stages : epi;
 }
 
-// Launches one tile configuration. `groups` > 1 is the grouped convolution.
-template <int BM, int BN, int WM, int WN, bool SA, bool SB, bool AL_A,
-          bool AL_B, class ARows>
-static int gemm_launch(const ARows &A, const DenseRows &B, const Epilogue &ep,
-                       int M, int N, int K, int groups,
-                       long long b_group_stride, hipStream_t st) {
-  constexpr int THREADS = (BM / WM) * (BN / WN) * 64;
-  constexpr size_t lds = gemm_lds_bytes<BM, BN>();
-  auto kern = gemm_i8_kernel<BM, BN, WM, WN, SA, SB, AL_A, AL_B, ARows>;
-  if (lds > 48 * 1024) {
-    static bool attr_set = false; // per instantiation
-    if (!attr_set) {
-      MI355X_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     (int)lds));
-      attr_set = true;
-    }
-  }
-  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-  const long long total = (long long)tiles_m * tiles_n;
-  MI355X_REQUIRE(total < 0x7fffffffLL && groups < 65536, "problem too large");
-  hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)groups),
-                     dim3(THREADS), lds, st, A, B, ep, M, N, K, tiles_m,
-                     tiles_n, b_group_stride, N);
-  return check_launch("gemm_i8");
+template <int BM, int BN, int STAGES> constexpr size_t gemm_dma_lds_bytes() {
+  constexpr size_t ring = (size_t)STAGES * (BM + BN) * kBK;
+  constexpr size_t epi = gemm_epilogue_lds_bytes<BM, BN>();
+  return ring > epi ? ring : epi;
 }
 
 // LDS a block may use on the current device (cached per process).
@@ -352,49 +611,128 @@ static size_t lds_limit() {
   return limit;
 }
 
-// Picks the tile configuration from the problem size: the 256x256 tile for
-// large problems (a wave owns 128x128, which halves LDS traffic per MFMA), and
-// smaller tiles when the grid would otherwise not fill 256 CUs.
-template <bool SA, bool SB, bool AL_A, bool AL_B, class ARows>
-static int gemm_dispatch_tiles(const ARows &A, const DenseRows &B,
-                               const Epilogue &ep, int M, int N, int K,
-                               int groups, long long b_group_stride,
-                               hipStream_t st) {
-  auto tiles = [&](int bm, int bn) {
-    return (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn) * groups;
-  };
-  if (tiles(256, 256) >= 256 && N >= 192 &&
-      gemm_lds_bytes<256, 256>() <= lds_limit())
-    return gemm_launch<256, 256, 128, 128, SA, SB, AL_A, AL_B>(
-        A, B, ep, M, N, K, groups, b_group_stride, st);
-  if (tiles(128, 128) >= 256 && N >= 96)
-    return gemm_launch<128, 128, 64, 64, SA, SB, AL_A, AL_B>(
-        A, B, ep, M, N, K, groups, b_group_stride, st);
-  if (tiles(128, 64) >= 256 || M >= 1024)
-    return gemm_launch<128, 64, 32, 64, SA, SB, AL_A, AL_B>(
-        A, B, ep, M, N, K, groups, b_group_stride, st);
-  return gemm_launch<64, 64, 32, 32, SA, SB, AL_A, AL_B>(
-      A, B, ep, M, N, K, groups, b_group_stride, st);
+template <class Kern>
+static int set_lds_attr(Kern kern, size_t lds, bool &done) {
+  if (lds > 48 * 1024 && !done) {
+    MI355X_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   (int)lds));
+    done = true;
+  }
+  return MI355X_OK;
 }
 
+struct GemmShape {
+  int M, N, K, groups;
+  long long b_group_stride;
+};
+
+// Launches one tile configuration of the register-staged kernel. `groups` > 1
+// is the grouped convolution.
+template <int BM, int BN, int WM, int WN, bool AL_A, bool AL_B, class ARows>
+static int gemm_launch(const ARows &A, const DenseRows &B, const Epilogue &ep,
+                       const GemmShape &g, hipStream_t st) {
+  constexpr int THREADS = (BM / WM) * (BN / WN) * 64;
+  constexpr size_t lds = gemm_lds_bytes<BM, BN>();
+  auto kern = gemm_i8_kernel<BM, BN, WM, WN, true, true, AL_A, AL_B, ARows>;
+  static bool attr_set = false; // per instantiation
+  int rc = set_lds_attr(kern, lds, attr_set);
+  if (rc != MI355X_OK) return rc;
+  const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
+  const long long total = (long long)tiles_m * tiles_n;
+  MI355X_REQUIRE(total < 0x7fffffffLL && g.groups < 65536, "problem too large");
+  hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)g.groups),
+                     dim3(THREADS), lds, st, A, B, ep, g.M, g.N, g.K, tiles_m,
+                     tiles_n, g.b_group_stride, g.N);
+  return check_launch("gemm_i8");
+}
+
+// Same for the direct-to-LDS kernel.
+template <int BM, int BN, int WM, int WN, int STAGES, bool SA, bool SB,
+          class ARows>
+static int gemm_dma_launch(const ARows &A, const DenseRows &B,
+                           const Epilogue &ep, const GemmShape &g,
+                           hipStream_t st) {
+  constexpr int THREADS = (BM / WM) * (BN / WN) * 64;
+  constexpr size_t lds = gemm_dma_lds_bytes<BM, BN, STAGES>();
+  auto kern = gemm_i8_dma_kernel<BM, BN, WM, WN, STAGES, SA, SB, ARows>;
+  static bool attr_set = false; // per instantiation
+  int rc = set_lds_attr(kern, lds, attr_set);
+  if (rc != MI355X_OK) return rc;
+  const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
+  const long long total = (long long)tiles_m * tiles_n;
+  MI355X_REQUIRE(total < 0x7fffffffLL && g.groups < 65536, "problem too large");
+  hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)g.groups),
+                     dim3(THREADS), lds, st, A, B, ep, g.M, g.N, g.K, tiles_m,
+                     tiles_n, g.b_group_stride, g.N);
+  return check_launch("gemm_i8_dma");
+}
+
+// Tile choice from the problem size: 256x256 for large problems (a wave owns
+// 128x128, which halves LDS traffic per MFMA), smaller tiles when the grid
+// would otherwise not fill 256 CUs.
+enum class Tile { T256, T128, T128x64, T64 };
+static Tile pick_tile(const GemmShape &g, size_t lds_256) {
+  auto tiles = [&](int bm, int bn) {
+    return (long long)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * g.groups;
+  };
+  if (tiles(256, 256) >= 256 && g.N >= 192 && lds_256 <= lds_limit())
+    return Tile::T256;
+  if (tiles(128, 128) >= 256 && g.N >= 96) return Tile::T128;
+  if (tiles(128, 64) >= 256 || g.M >= 1024) return Tile::T128x64;
+  return Tile::T64;
+}
+
+template <bool SA, bool SB, class ARows>
+static int gemm_dma_tiles(const ARows &A, const DenseRows &B, const Epilogue &ep,
+                          const GemmShape &g, hipStream_t st) {
+  switch (pick_tile(g, gemm_dma_lds_bytes<256, 256, 4>())) {
+  case Tile::T256:
+    return gemm_dma_launch<256, 256, 128, 128, 4, SA, SB>(A, B, ep, g, st);
+  case Tile::T128:
+    return gemm_dma_launch<128, 128, 64, 64, 3, SA, SB>(A, B, ep, g, st);
+  case Tile::T128x64:
+    return gemm_dma_launch<128, 64, 32, 64, 3, SA, SB>(A, B, ep, g, st);
+  default:
+    return gemm_dma_launch<64, 64, 32, 32, 4, SA, SB>(A, B, ep, g, st);
+  }
+}
+
+template <bool AL_A, bool AL_B, class ARows>
+static int gemm_staged_tiles(const ARows &A, const DenseRows &B,
+                             const Epilogue &ep, const GemmShape &g,
+                             hipStream_t st) {
+  switch (pick_tile(g, gemm_lds_bytes<256, 256>())) {
+  case Tile::T256:
+    return gemm_launch<256, 256, 128, 128, AL_A, AL_B>(A, B, ep, g, st);
+  case Tile::T128:
+    return gemm_launch<128, 128, 64, 64, AL_A, AL_B>(A, B, ep, g, st);
+  case Tile::T128x64:
+    return gemm_launch<128, 64, 32, 64, AL_A, AL_B>(A, B, ep, g, st);
+  default:
+    return gemm_launch<64, 64, 32, 32, AL_A, AL_B>(A, B, ep, g, st);
+  }
+}
+
+// need_sa / need_sb: whether the row sums of A / B have to be formed inside
+// the kernel (a non-zero B offset; a non-zero A offset without precomputed
+// ep.sum_b). aligned: both operands allow 16-byte chunk
+// loads (16-byte aligned rows; for convolutions also IC/group % 16 == 0).
 template <class ARows>
 static int gemm_dispatch(const ARows &A, const DenseRows &B, const Epilogue &ep,
                          int M, int N, int K, int groups,
                          long long b_group_stride, bool need_sa, bool need_sb,
-                         bool al_a, bool al_b, hipStream_t st) {
-#define MI355X_GEMM_CASE(SA, SB, AA, AB)                                       \
-  if (need_sa == SA && need_sb == SB && al_a == AA && al_b == AB)              \
-    return gemm_dispatch_tiles<SA, SB, AA, AB>(A, B, ep, M, N, K, groups,      \
-                                               b_group_stride, st);
-  // aligned operands: all four row-sum combinations
-  MI355X_GEMM_CASE(false, false, true, true)
-  MI355X_GEMM_CASE(false, true, true, true)
-  MI355X_GEMM_CASE(true, false, true, true)
-  MI355X_GEMM_CASE(true, true, true, true)
-#undef MI355X_GEMM_CASE
-  // any unaligned operand: the byte-wise loaders with both row sums
-  return gemm_dispatch_tiles<true, true, false, false>(A, B, ep, M, N, K, groups,
-                                                       b_group_stride, st);
+                         bool aligned, hipStream_t st) {
+  const GemmShape g{M, N, K, groups, b_group_stride};
+  if (aligned && K >= kBK && K % kBK == 0) {
+    if (need_sa && need_sb) return gemm_dma_tiles<true, true>(A, B, ep, g, st);
+    if (need_sa) return gemm_dma_tiles<true, false>(A, B, ep, g, st);
+    if (need_sb) return gemm_dma_tiles<false, true>(A, B, ep, g, st);
+    return gemm_dma_tiles<false, false>(A, B, ep, g, st);
+  }
+  // K tails and unaligned operands: register-staged loop, both row sums kept
+  if (aligned) return gemm_staged_tiles<true, true>(A, B, ep, g, st);
+  return gemm_staged_tiles<false, false>(A, B, ep, g, st);
 }
 
 } // namespace mi355x

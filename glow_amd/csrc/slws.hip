@@ -124,68 +124,91 @@ __device__ __forceinline__ uint32_t clamp_len(int v) {
 // the lengths of the block's earlier bags. Sums inside a chunk are 32-bit:
 // positions are checked against num_indices before any use, so absurd lengths
 // cannot cause an out-of-range read. Offsets mode: read off the offsets vector.
+// Offsets mode: span of `bag` read off the offsets vector.
+__device__ __forceinline__ void bag_span_offsets(const SlwsArgs &a,
+                                                 long long bag,
+                                                 long long &start, int &len) {
+  start = 0;
+  len = 0;
+  if (bag < a.segments) {
+    start = a.offsets[bag];
+    const long long end = (!a.offsets_have_end && bag == a.segments - 1)
+                              ? a.num_indices
+                              : (long long)a.offsets[bag + 1];
+    len = end > start ? (int)min(end - start, 0x7fffffffLL) : 0;
+  }
+}
+
+// Lengths mode, first half: every wave leaves the sum of the clamped lengths
+// it has seen in front of the block in s_part[wave], and the block's own
+// clamped lengths go to s_own[]. Ends with a block barrier.
+template <int kGroups>
+__device__ __forceinline__ void block_prefix(const SlwsArgs &a, int tid,
+                                             long long first_bag,
+                                             long long *s_part, int *s_own) {
+  const long long chunk = first_bag / kChunkBags;
+  const long long lo = chunk * kChunkBags;
+  const int32_t *lbase = a.lengths + lo;
+  const int n_before = (int)(first_bag - lo); // < kChunkBags, multiple of 4
+  uint32_t part = 0;
+  if ((((uintptr_t)lbase) & 15) == 0) {
+    constexpr int kVecTrips = kChunkBags / 4 / kSlwsThreads;
+    const int4 *l4 = reinterpret_cast<const int4 *>(lbase);
+    const int nvec = n_before / 4;
+    if (nvec > 0) {
+      // every trip loads (indices past the end re-read the last vector and
+      // are masked out), so all loads are in flight together
+      int4 x[kVecTrips];
+#pragma unroll
+      for (int u = 0; u < kVecTrips; u++)
+        x[u] = l4[min(tid + u * kSlwsThreads, nvec - 1)];
+#pragma unroll
+      for (int u = 0; u < kVecTrips; u++) {
+        const uint32_t t = clamp_len(x[u].x) + clamp_len(x[u].y) +
+                           clamp_len(x[u].z) + clamp_len(x[u].w);
+        part += (tid + u * kSlwsThreads < nvec) ? t : 0u;
+      }
+    }
+  } else {
+    for (int i = tid; i < n_before; i += kSlwsThreads) part += clamp_len(lbase[i]);
+  }
+  long long below = 0;
+  if (a.chunk_sums) {
+    for (long long c = tid; c < chunk; c += kSlwsThreads) below += a.chunk_sums[c];
+    below = (long long)wave_sum_u32((uint32_t)below) +
+            ((long long)wave_sum_u32((uint32_t)(below >> 32)) << 32);
+  }
+  if (tid < kGroups) {
+    const long long b = first_bag + tid;
+    s_own[tid] = (int)min(clamp_len(b < a.segments ? a.lengths[b] : 0),
+                          0x7fffffffu);
+  }
+  below += wave_sum_u32(part);
+  if ((tid & 63) == 0) s_part[tid >> 6] = below;
+  __syncthreads();
+}
+
+// Position of the first lookup of `bag` in the index list and its length.
+// Lengths mode: exclusive prefix sum of the clamped lengths in front of the
+// block (summed by the block itself, all loads in one memory round trip) plus
+// the lengths of the block's earlier bags. Sums inside a chunk are 32-bit:
+// positions are checked against num_indices before any use, so absurd lengths
+// cannot cause an out-of-range read.
 template <int kGroups>
 __device__ __forceinline__ void bag_span(const SlwsArgs &a, int tid, int grp,
                                          long long bag, long long first_bag,
                                          long long *s_part, int *s_own,
                                          long long &start, int &len) {
-  start = 0;
-  len = 0;
   if (a.offsets) {
-    if (bag < a.segments) {
-      start = a.offsets[bag];
-      long long end = (!a.offsets_have_end && bag == a.segments - 1)
-                          ? a.num_indices
-                          : (long long)a.offsets[bag + 1];
-      len = end > start ? (int)(end - start) : 0;
-    }
-  } else {
-    const long long chunk = first_bag / kChunkBags;
-    const long long lo = chunk * kChunkBags;
-    const int32_t *lbase = a.lengths + lo;
-    const int n_before = (int)(first_bag - lo); // < kChunkBags, multiple of 4
-    uint32_t part = 0;
-    if ((((uintptr_t)lbase) & 15) == 0) {
-      constexpr int kVecTrips = kChunkBags / 4 / kSlwsThreads;
-      const int4 *l4 = reinterpret_cast<const int4 *>(lbase);
-      const int nvec = n_before / 4;
-      if (nvec > 0) {
-        // every trip loads (indices past the end re-read the last vector and
-        // are masked out), so all loads are in flight together
-        int4 x[kVecTrips];
-#pragma unroll
-        for (int u = 0; u < kVecTrips; u++)
-          x[u] = l4[min(tid + u * kSlwsThreads, nvec - 1)];
-#pragma unroll
-        for (int u = 0; u < kVecTrips; u++) {
-          const uint32_t t = clamp_len(x[u].x) + clamp_len(x[u].y) +
-                             clamp_len(x[u].z) + clamp_len(x[u].w);
-          part += (tid + u * kSlwsThreads < nvec) ? t : 0u;
-        }
-      }
-    } else {
-      for (int i = tid; i < n_before; i += kSlwsThreads) part += clamp_len(lbase[i]);
-    }
-    long long below = 0;
-    if (a.chunk_sums) {
-      for (long long c = tid; c < chunk; c += kSlwsThreads) below += a.chunk_sums[c];
-      below = (long long)wave_sum_u32((uint32_t)below) +
-              ((long long)wave_sum_u32((uint32_t)(below >> 32)) << 32);
-    }
-    if (tid < kGroups) {
-      const long long b = first_bag + tid;
-      s_own[tid] = (int)min(clamp_len(b < a.segments ? a.lengths[b] : 0),
-                            0x7fffffffu);
-    }
-    below += wave_sum_u32(part);
-    if ((tid & 63) == 0) s_part[tid >> 6] = below;
-    __syncthreads();
-#pragma unroll
-    for (int w = 0; w < kSlwsThreads / 64; w++) start += s_part[w];
-    for (int g = 0; g < grp; g++) start += s_own[g];
-    len = s_own[grp];
+    bag_span_offsets(a, bag, start, len);
+    return;
   }
-  if (bag >= a.segments) len = 0;
+  block_prefix<kGroups>(a, tid, first_bag, s_part, s_own);
+  start = 0;
+#pragma unroll
+  for (int w = 0; w < kSlwsThreads / 64; w++) start += s_part[w];
+  for (int g = 0; g < grp; g++) start += s_own[g];
+  len = bag < a.segments ? s_own[grp] : 0;
 }
 
 template <int LPB, int BPL, bool IS4, bool SO16, bool ACC16>
@@ -336,7 +359,7 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_wave_kernel(SlwsArgs a) {
   constexpr int kColsPerLane = BPL * kColsPerByte;
   constexpr int kGroup = 4;   // lookups handled under one uniform branch
   __shared__ long long s_part[kGroups];
-  __shared__ int s_own[kGroups];
+  __shared__ __attribute__((aligned(16))) int s_own[kGroups];
   // per wave, per lookup of the batch: {row offset or row, weight, scale, offset}
   __shared__ int4 s_look[kGroups][kBatch];
 
@@ -346,14 +369,33 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_wave_kernel(SlwsArgs a) {
   const long long first_bag = (long long)blockIdx.x * kGroups;
   const long long bag = first_bag + wave;
 
-  long long start_v = 0;
-  int len_v = 0;
-  bag_span<kGroups>(a, tid, wave, bag, first_bag, s_part, s_own, start_v, len_v);
-  // wave-uniform from here on: keep them in scalar registers
-  const int len = __builtin_amdgcn_readfirstlane(len_v);
-  const long long start =
-      ((long long)__builtin_amdgcn_readfirstlane((int)(start_v >> 32)) << 32) |
-      (unsigned int)__builtin_amdgcn_readfirstlane((int)start_v);
+  // start and len are wave-uniform: keep them in scalar registers
+  long long start;
+  int len;
+  if (a.offsets) {
+    long long start_v;
+    int len_v;
+    bag_span_offsets(a, bag, start_v, len_v);
+    len = __builtin_amdgcn_readfirstlane(len_v);
+    start = ((long long)__builtin_amdgcn_readfirstlane((int)(start_v >> 32)) << 32) |
+            (unsigned int)__builtin_amdgcn_readfirstlane((int)start_v);
+  } else {
+    static_assert(kGroups == 4, "the own-length selects below assume 4 waves");
+    block_prefix<kGroups>(a, tid, first_bag, s_part, s_own);
+    const long long block_start = s_part[0] + s_part[1] + s_part[2] + s_part[3];
+    const int4 own = *reinterpret_cast<const int4 *>(s_own);
+    const int w = __builtin_amdgcn_readfirstlane(wave);
+    const int o0 = __builtin_amdgcn_readfirstlane(own.x);
+    const int o1 = __builtin_amdgcn_readfirstlane(own.y);
+    const int o2 = __builtin_amdgcn_readfirstlane(own.z);
+    const int o3 = __builtin_amdgcn_readfirstlane(own.w);
+    const long long bs =
+        ((long long)__builtin_amdgcn_readfirstlane((int)(block_start >> 32)) << 32) |
+        (unsigned int)__builtin_amdgcn_readfirstlane((int)block_start);
+    start = bs + (w > 0 ? o0 : 0) + (w > 1 ? o1 : 0) + (w > 2 ? o2 : 0);
+    len = w == 0 ? o0 : (w == 1 ? o1 : (w == 2 ? o2 : o3));
+    if (bag >= a.segments) len = 0;
+  }
   int4 *look = s_look[wave];
 
   const int n_passes = (a.data_bytes + 64 * BPL - 1) / (64 * BPL);

@@ -177,6 +177,18 @@ int mi355x_rescale_i8(int8_t *dst, const int8_t *src, size_t n,
 
 /* ---- FullyConnected / MatMul -------------------------------------------------- */
 
+/* sums[r] = sum over k of rows[r][k] for an int8 matrix [n_rows x K] with K
+ * contiguous. The matrix-core kernels below contract raw bytes and apply the
+ * operand offsets afterwards, which needs sum_k W[n][k] per output column
+ * whenever the input offset is non-zero. Weights and filters are constants, so
+ * a backend computes these sums once when a network is loaded and passes them
+ * as `weights_row_sums` / `filter_row_sums`; with NULL there the kernels form
+ * the sums on the fly at a visible cost in matrix-core utilisation. No
+ * counterpart in the reference (its scalar loops subtract the offsets
+ * element by element). */
+int mi355x_rowsum_i8(int32_t *sums, const int8_t *rows, size_t n_rows, size_t K,
+                     void *stream);
+
 /* libjit_rowwise_quantized_fc_i8_i32 / _i8_i8 (reference
  * lib/LLVMIRCodeGen/libjit/libjit_matmul.cpp:284-316, 425-450).
  * in [M x K], weights [N x K] (not transposed), bias int32[N] or int8[N]
@@ -191,20 +203,22 @@ int mi355x_rwq_fc_i8(int8_t *out, const int8_t *in, const int8_t *weights,
                      const int32_t *out_scale, size_t M, size_t K, size_t N,
                      int32_t out_offset, int32_t in_offset,
                      int32_t bias_offset, int weights_offsets_all_zero,
-                     void *stream);
+                     const int32_t *weights_row_sums, void *stream);
 
 /* libjit_fc_i8_i32 / _i8_i8 (libjit_matmul.cpp:254-280, 395-422).
  * weights_kn is [K x N] as Glow stores FullyConnected weights; the kernel
  * consumes the [N x K] transpose, which is written to `weights_nk_workspace`
  * (K*N bytes, device) when repack != 0 and read from there otherwise (weights
- * are constants: repack once at load time). */
+ * are constants: repack once at load time). weights_row_sums, if given, are
+ * the row sums of that [N x K] transpose. */
 int mi355x_fc_i8(int8_t *out, const int8_t *in, const int8_t *weights_kn,
                  int8_t *weights_nk_workspace, int repack, const void *bias,
                  int bias_is_i8, size_t M, size_t K, size_t N,
                  int32_t out_offset, int32_t in_offset, int32_t weights_offset,
                  int32_t bias_offset, int32_t bias_pre, int32_t bias_post,
                  int32_t bias_scale, int32_t out_pre, int32_t out_post,
-                 int32_t out_scale, void *stream);
+                 int32_t out_scale, const int32_t *weights_row_sums,
+                 void *stream);
 
 /* libjit_matmul_i8 (libjit_matmul.cpp:353-371). lhs [M x K], rhs_kn [K x N];
  * workspace and repack as for mi355x_fc_i8. */
@@ -240,7 +254,9 @@ enum { MI355X_ACT_NONE = 0, MI355X_ACT_RELU = 1, MI355X_ACT_CLIP = 2,
 
 /* libjit_channelwise_quantized_conv2d_i8_i32 / _i8_i8 (reference
  * lib/LLVMIRCodeGen/libjit/libjit_conv.cpp:151-239, 530-562). Eight int32[OC]
- * per-channel vectors on the device; act_args is a HOST array of 3 ints. */
+ * per-channel vectors on the device; act_args is a HOST array of 3 ints.
+ * filter_row_sums (optional) = mi355x_rowsum_i8 of the filter viewed as
+ * [OC x KH*KW*IC/group]. */
 int mi355x_cwq_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
                          const void *bias, int bias_is_i8,
                          const mi355x_conv_geom *geom, int32_t out_offset,
@@ -250,7 +266,8 @@ int mi355x_cwq_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
                          const int32_t *out_pre, const int32_t *out_post,
                          const int32_t *out_scale, int32_t act_type,
                          const int32_t *act_args,
-                         int filter_offsets_all_zero, void *stream);
+                         int filter_offsets_all_zero,
+                         const int32_t *filter_row_sums, void *stream);
 
 /* libjit_conv2d_i8_i32 / _i8_i8 (libjit_conv.cpp:49-147, 496-528). */
 int mi355x_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
@@ -260,7 +277,8 @@ int mi355x_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
                      int32_t bias_offset, int32_t bias_pre, int32_t bias_post,
                      int32_t bias_scale, int32_t out_pre, int32_t out_post,
                      int32_t out_scale, int32_t act_type,
-                     const int32_t *act_args, void *stream);
+                     const int32_t *act_args, const int32_t *filter_row_sums,
+                     void *stream);
 
 /* ---- fused-rowwise SparseLengths(Weighted)Sum ----------------------------------- */
 

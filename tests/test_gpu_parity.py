@@ -111,6 +111,9 @@ def test_rwq_fc_vs_oracle(shape):
                               bias_offset=(3 if b8 else 0))
         want = go.rwq_fc_i8(*cases.rwq_fc_args(c))
         np.testing.assert_array_equal(capi.rwq_fc_i8(*cases.rwq_fc_args(c)), want)
+        # without precomputed weight row sums the kernel forms them itself
+        np.testing.assert_array_equal(
+            capi.rwq_fc_i8(*cases.rwq_fc_args(c), precomputed_sums=False), want)
     # zero input offset and symmetric weights: the path without row sums
     c = cases.rwq_fc_case(9, M, K, N, in_offset=0)
     np.testing.assert_array_equal(capi.rwq_fc_i8(*cases.rwq_fc_args(c)),
@@ -165,13 +168,23 @@ def test_fc_vs_oracle(shape):
     for b8 in (False, True):
         say("fc", shape, "bias8" if b8 else "bias32")
         c = cases.fc_case(shape[0], *shape, bias_i8=b8)
-        np.testing.assert_array_equal(capi.fc_i8(*cases.fc_args(c)),
-                                      go.fc_i8(*cases.fc_args(c)))
+        want = go.fc_i8(*cases.fc_args(c))
+        np.testing.assert_array_equal(capi.fc_i8(*cases.fc_args(c)), want)
+        np.testing.assert_array_equal(
+            capi.fc_i8(*cases.fc_args(c), precomputed_sums=True), want)
     np.testing.assert_array_equal(
         capi.matmul_i8(c["x"], c["w"], c["out_offset"], c["in_offset"],
                        c["w_offset"], c["outP"]),
         go.matmul_i8(c["x"], c["w"], c["out_offset"], c["in_offset"],
                      c["w_offset"], c["outP"]))
+
+
+def test_rowsum():
+    rng = np.random.default_rng(16)
+    for shape in [(1, 1), (5, 100), (64, 1024), (300, 2048 + 37), (7, 3, 3, 64)]:
+        a = rng.integers(-128, 128, shape).astype(np.int8)
+        want = a.reshape(shape[0], -1).astype(np.int32).sum(1)
+        np.testing.assert_array_equal(capi.rowsum_i8(a), want)
 
 
 def test_transpose2d():
@@ -224,6 +237,8 @@ def test_cwq_conv_vs_oracle(kw):
     c = cases.cwq_conv_case(31, **kw)
     want = go.cwq_conv2d_i8(*cases.cwq_conv_args(c))
     np.testing.assert_array_equal(capi.cwq_conv2d_i8(*cases.cwq_conv_args(c)), want)
+    np.testing.assert_array_equal(
+        capi.cwq_conv2d_i8(*cases.cwq_conv_args(c), precomputed_sums=False), want)
     assert want.std() > 1
     # uniform-parameter convolution through its own entry point
     args = (c["x"], c["filt"], c["bias"], c["geom"], c["out_offset"],
