@@ -29,6 +29,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+# HBM bytes per launch of the default workloads (FETCH_SIZE + WRITE_SIZE of two
+# counter runs, scaled by what the counters read for a plain copy of known
+# size). They hold for the default sizes only; other sizes report null.
+MEASURED_TRAFFIC = {"slws": 24.03e6, "fc_large": 236.3e6, "conv_c3": 13.32e6}
+
 HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E, published
 INT8_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA, published (5.0 POP/s)
 
@@ -49,7 +54,8 @@ def parse():
                     help="headline workload only")
     ap.add_argument("--only", default="",
                     help="run a single extra kernel (profiling aid): "
-                         "slws|fc_large|fc_c1|conv_c3|quantize|dequantize|rescale")
+                         "slws|fc_large|fc_c1|conv_c3|quantize|dequantize|"
+                         "rescale|copy")
     return ap.parse_args()
 
 
@@ -112,6 +118,71 @@ def bench_slws(capi, cases, args, table, d_table):
                 d_out=d_out)
 
 
+def bench_slws_with_h2d(capi, s, args, d_table):
+    """Same launches, but every step first copies its indices, weights and
+    lengths from pinned host memory: what a DeviceManager does per request."""
+    import ctypes as C
+    rows, cols, bags = args.rows, 128, args.bags
+    pinned = []
+    for b in s["batches"]:
+        ent = {}
+        for key, arr in (("idx", b["idx"]), ("w", b["w"]), ("lengths", b["lengths"])):
+            hp = C.c_void_p(0)
+            capi.check(capi.lib().mi355x_host_alloc(C.byref(hp), C.c_size_t(max(arr.nbytes, 1))))
+            C.memmove(hp.value, arr.ctypes.data, arr.nbytes)
+            ent[key] = (hp, arr.nbytes)
+        pinned.append(ent)
+
+    def step(i, stream):
+        b = s["batches"][i % len(s["batches"])]
+        h = pinned[i % len(pinned)]
+        for key, dst in (("idx", b["d_idx"]), ("w", b["d_w"]), ("lengths", b["d_len"])):
+            hp, n = h[key]
+            capi.check(capi.lib().mi355x_memcpy_h2d(C.c_void_p(dst.ptr), hp, C.c_size_t(n),
+                                                    C.c_void_p(stream.ptr)))
+        capi.launch_frwq_slws(s["d_out"], False, d_table, rows, capi.FUSED_U8_F32,
+                              b["d_w"], False, b["d_idx"], True, b["total"],
+                              b["d_len"], bags, cols + 8, cols, stream=stream)
+
+    sec = timed_launches(capi, step, args.steps, args.warmup)
+    for h in pinned:
+        for hp, _ in h.values():
+            capi.lib().mi355x_host_free(hp)
+    return dict(workload="SLWS headline step + H2D of indices, weights, lengths "
+                         "from pinned host memory", ms=sec * 1e3,
+                gbps=s["bytes"] / sec / 1e9,
+                h2d_bytes_per_step=s["mean_lookups"] * 12 + bags * 4)
+
+
+def cpu_all_cores_slws(table, batches, budget_s):
+    """The oracle on every host core this process may use, one whole batch per
+    thread at a time (the reference's CPU backend exposes one device per
+    hardware thread, lib/Backends/CPU/CPUBackend.cpp:114-116)."""
+    import threading
+    from oracle import glow_oracle as go
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
+    cores = max(1, min(cores, 16))
+    done = [0.0] * cores
+    t0 = time.perf_counter()
+
+    def work(t):
+        n = t
+        while time.perf_counter() - t0 < budget_s:
+            b = batches[n % len(batches)]
+            go.frwq_slws_f32(table, b["w"], b["idx"], b["lengths"])
+            done[t] += slws_bytes(b["total"], b["lengths"].size, 128, 136)
+            n += cores
+
+    th = [threading.Thread(target=work, args=(t,)) for t in range(cores)]
+    for t in th:
+        t.start()
+    for t in th:
+        t.join()
+    el = time.perf_counter() - t0
+    return dict(value=sum(done) / el / 1e9, unit="GB/s", cores=cores, kind="port",
+                sample=f"whole batches for {el:.1f} s, one batch per thread at a time")
+
+
 def cpu_baseline_slws(table, batches, budget_s, gpu_out, gpu_batch):
     """The CPU leg: the oracle (the restated libjit loop, one thread) over
     whole batches of the same workload until the time budget is used. As the
@@ -166,7 +237,8 @@ def bench_fc(capi, cases, M, K, N, steps, warmup, seed=5):
                 roofline=dict(bound="mfma", achieved=ops / sec / 1e12,
                               peak=INT8_PEAK_TOPS, unit="TOP/s",
                               frac=ops / sec / 1e12 / INT8_PEAK_TOPS,
-                              traffic=None),
+                              traffic=(MEASURED_TRAFFIC["fc_large"]
+                                       if (M, K, N) == (8192, 4096, 4096) else None)),
                 gbps=(M * K + N * K + M * N + 8 * 4 * N) / sec / 1e9)
 
 
@@ -196,7 +268,7 @@ def bench_conv(capi, cases, steps, warmup):
                 roofline=dict(bound="mfma", achieved=ops / sec / 1e12,
                               peak=INT8_PEAK_TOPS, unit="TOP/s",
                               frac=ops / sec / 1e12 / INT8_PEAK_TOPS,
-                              traffic=None))
+                              traffic=MEASURED_TRAFFIC["conv_c3"]))
 
 
 def bench_elementwise(capi, which, steps, warmup):
@@ -212,13 +284,20 @@ def bench_elementwise(capi, which, steps, warmup):
         dst = capi.DeviceBuffer.empty((n,), np.float32)
         fn = lambda _, st: capi.launch_dequantize_i8(dst, src, n, 0.02, -3, st)
         nbytes = n * 5
+    elif which == "copy":
+        # plain copy of known size: what the HBM byte counters are scaled by
+        n = 256 << 20
+        src = capi.to_device(rng.integers(-128, 128, n).astype(np.int8))
+        dst = capi.DeviceBuffer.empty((n,), np.int8)
+        fn = lambda _, st: capi.launch_copy_u8(dst, src, n, st)
+        nbytes = n * 2
     else:
         src = capi.to_device(rng.integers(-128, 128, n).astype(np.int8))
         dst = capi.DeviceBuffer.empty((n,), np.int8)
         fn = lambda _, st: capi.launch_rescale_i8(dst, src, n, 3, -5, 2, 15, 300, st)
         nbytes = n * 2
     sec = timed_launches(capi, fn, steps, warmup)
-    return dict(workload=f"{which}_i8 n={n}", ms=sec * 1e3,
+    return dict(workload=f"{which}_u8 n={n}" if which == "copy" else f"{which}_i8 n={n}", ms=sec * 1e3,
                 gbps=nbytes / sec / 1e9,
                 roofline=dict(bound="hbm", achieved=nbytes / sec / 1e9,
                               peak=HBM_PEAK_GBPS, unit="GB/s",
@@ -242,7 +321,8 @@ def main():
     extra = {}
     only = args.only
 
-    if only in ("fc_large", "fc_c1", "conv_c3", "quantize", "dequantize", "rescale"):
+    if only in ("fc_large", "fc_c1", "conv_c3", "quantize", "dequantize", "rescale",
+                "copy"):
         if only == "fc_large":
             r = bench_fc(capi, cases, 8192, 4096, 4096, args.steps, args.warmup)
         elif only == "fc_c1":
@@ -263,12 +343,16 @@ def main():
     # CPU leg: baseline timing, and the check of the last timed step's output
     last = s["batches"][(args.warmup + args.steps - 1) % len(s["batches"])]
     cpu, parity = None, None
-    if not only:
+    if not only and args.cpu_seconds > 0:
         cpu, parity = cpu_baseline_slws(table, s["batches"], args.cpu_seconds,
                                         s["d_out"].numpy(), last)
 
     if not args.no_extra and not only:
         st, wu = max(20, args.steps // 4), max(3, args.warmup // 4)
+        extra["slws_with_h2d"] = bench_slws_with_h2d(capi, s, args, d_table)
+        if args.cpu_seconds > 0:
+            extra["cpu_all_cores"] = cpu_all_cores_slws(table, s["batches"],
+                                                        args.cpu_seconds / 2)
         extra["rwq_fc_c1"] = bench_fc(capi, cases, 128, 1024, 1024, args.steps, args.warmup)
         extra["rwq_fc_large"] = bench_fc(capi, cases, 8192, 4096, 4096, st, wu)
         extra["cwq_conv_c3"] = bench_conv(capi, cases, args.steps, args.warmup)
@@ -302,8 +386,10 @@ def main():
         "parity_with_oracle": parity,
         "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
-                     "traffic": None,
-                     "kernel": "slws_kernel<64,2,false,false,false>"},
+                     "traffic": (MEASURED_TRAFFIC["slws"]
+                                 if (args.rows, args.bags, args.batches) ==
+                                 (4_000_000, 4096, 8) else None),
+                     "kernel": "slws_wave_kernel<2,false,false,false,true>"},
         "cpu_baseline": cpu,
         "extra": extra,
     }

@@ -22,7 +22,7 @@ EXPORTS = [
     "mi355x_last_error", "mi355x_num_devices", "mi355x_init",
     "mi355x_device_info", "mi355x_malloc", "mi355x_free", "mi355x_host_alloc",
     "mi355x_host_free", "mi355x_memcpy_h2d", "mi355x_memcpy_d2h",
-    "mi355x_memcpy_d2d", "mi355x_fill_u8", "mi355x_stream_create",
+    "mi355x_memcpy_d2d", "mi355x_fill_u8", "mi355x_copy_u8", "mi355x_stream_create",
     "mi355x_stream_destroy", "mi355x_stream_sync", "mi355x_device_sync",
     "mi355x_event_create", "mi355x_event_destroy", "mi355x_event_record",
     "mi355x_event_sync", "mi355x_event_elapsed_ms", "mi355x_arena_create",
@@ -379,6 +379,10 @@ def launch_rescale_i8(dst, src, n, out_offset, in_offset, pre, post, scale,
     check(lib().mi355x_rescale_i8(_vp(dst), _vp(src), _sz(n), _i32(out_offset),
                                   _i32(in_offset), _i32(pre), _i32(post),
                                   _i32(scale), _vp(stream)))
+
+
+def launch_copy_u8(dst, src, nbytes, stream=None):
+    check(lib().mi355x_copy_u8(_vp(dst), _vp(src), _sz(nbytes), _vp(stream)))
 
 
 def launch_rowsum_i8(sums, rows, n_rows, K, stream=None):

@@ -36,6 +36,23 @@ __global__ void fill_u8_kernel(uint8_t *dst, uint8_t v, size_t n) {
   for (; i < n; i += stride) dst[i] = v;
 }
 
+// 16 bytes per lane and trip; head and tail bytes one at a time.
+__global__ __launch_bounds__(256) void copy_u8_kernel(uint8_t *__restrict__ dst,
+                                                      const uint8_t *__restrict__ src,
+                                                      size_t n, int vec_ok) {
+  const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  size_t done = 0;
+  if (vec_ok) {
+    const size_t nv = n / 16;
+    const int4 *s4 = reinterpret_cast<const int4 *>(src);
+    int4 *d4 = reinterpret_cast<int4 *>(dst);
+    for (size_t i = tid; i < nv; i += stride) d4[i] = s4[i];
+    done = nv * 16;
+  }
+  for (size_t i = done + tid; i < n; i += stride) dst[i] = src[i];
+}
+
 } // namespace mi355x
 
 using namespace mi355x;
@@ -169,6 +186,19 @@ int mi355x_fill_u8(void *dst, int value, size_t bytes, void *stream) {
   hipLaunchKernelGGL(fill_u8_kernel, dim3((unsigned)blocks), dim3(256), 0,
                      as_stream(stream), (uint8_t *)dst, (uint8_t)value, bytes);
   return check_launch("fill_u8");
+}
+
+int mi355x_copy_u8(void *dst, const void *src, size_t bytes, void *stream) {
+  if (bytes == 0) return MI355X_OK;
+  MI355X_REQUIRE(dst && src, "NULL pointer in device copy");
+  size_t blocks = (bytes / 16 + 255) / 256;
+  if (blocks < 1) blocks = 1;
+  if (blocks > 256 * 32) blocks = 256 * 32;
+  const int vec_ok = ((((uintptr_t)dst) | ((uintptr_t)src)) & 15) == 0;
+  hipLaunchKernelGGL(copy_u8_kernel, dim3((unsigned)blocks), dim3(256), 0,
+                     as_stream(stream), (uint8_t *)dst, (const uint8_t *)src,
+                     bytes, vec_ok);
+  return check_launch("copy_u8");
 }
 
 int mi355x_stream_create(void **stream) {

@@ -228,6 +228,12 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_kernel(SlwsArgs a) {
   long long start = 0;
   int len = 0;
   bag_span<kGroups>(a, tid, grp, bag, first_bag, s_part, s_own, start, len);
+  // a bag cannot use more lookups than the index list holds: bounds the loop
+  // below whatever the lengths say
+  {
+    const long long room = a.num_indices - start;
+    len = room <= 0 ? 0 : (int)min((long long)len, room);
+  }
 
   const int n_passes = (a.data_bytes + LPB * BPL - 1) / (LPB * BPL);
   for (int pass = 0; pass < n_passes; pass++) {
@@ -395,6 +401,12 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_wave_kernel(SlwsArgs a) {
     start = bs + (w > 0 ? o0 : 0) + (w > 1 ? o1 : 0) + (w > 2 ? o2 : 0);
     len = w == 0 ? o0 : (w == 1 ? o1 : (w == 2 ? o2 : o3));
     if (bag >= a.segments) len = 0;
+  }
+  // a bag cannot use more lookups than the index list holds: bounds the loop
+  // below whatever the lengths say
+  {
+    const long long room = a.num_indices - start;
+    len = room <= 0 ? 0 : (int)min((long long)len, room);
   }
   int4 *look = s_look[wave];
 

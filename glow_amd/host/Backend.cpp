@@ -1,0 +1,689 @@
+// Compile side of the MI355X backend: verifies each lowered instruction,
+// derives the integer kernel parameters the way Glow's CPU code generator does
+// (reference lib/LLVMIRCodeGen/LLVMIRGen.cpp:618-662, 1670-1690, 2161-2320,
+// 2501-2599, 2695-2798, 3638-3659) and emits a list of C-ABI launches.
+#include "Backend.h"
+
+#include "glow_mi355x.h"
+
+#include <cmath>
+#include <sstream>
+
+namespace glow_mi355x {
+
+namespace {
+
+struct S32To8 { int32_t pre, post, scale; };
+S32To8 s32to8(float ratio) {
+  int32_t o[4];
+  mi355x_quantize_scale_offset_32to8(ratio, 0, o);
+  return {o[0], o[1], o[2]};
+}
+
+// quantization::quantize<int32_t> (reference Base.h:323-329)
+int32_t quantizeI32(float x, float scale, int32_t offset) {
+  float r = x / scale + (float)offset;
+  double v = std::nearbyintf(r);
+  if (v > 2147483647.0) v = 2147483647.0;
+  if (v < -2147483648.0) v = -2147483648.0;
+  return (int32_t)v;
+}
+
+// Byte offsets of compiler-made buffers inside the generated region.
+class Generated {
+public:
+  // initialised int32 vector
+  size_t addI32(const std::vector<int32_t> &v) {
+    const size_t off = image_.size();
+    image_.resize(alignUp(off + v.size() * 4, kTensorAlignment), 0);
+    std::memcpy(image_.data() + off, v.data(), v.size() * 4);
+    return off;
+  }
+  // uninitialised scratch placed after every initialised buffer
+  size_t addScratch(size_t bytes) {
+    const size_t off = scratch_;
+    scratch_ = alignUp(scratch_ + bytes, 256);
+    return off; // relative to scratchBase(), fixed up by the caller at the end
+  }
+  std::vector<uint8_t> image_;
+  size_t scratch_ = 0;
+};
+
+struct Operand {
+  const Value *v;
+  // region + offset -> device pointer at launch time
+  uint8_t *ptr(const DeviceBindings &b) const {
+    switch (v->category) {
+    case SymbolCategory::Constant: return b.constants + v->offset;
+    case SymbolCategory::Placeholder: return b.mutableMem + v->offset;
+    default: return b.activations + v->offset;
+    }
+  }
+  const Type &ty() const { return v->type; }
+};
+
+std::string kv(const char *k, long long v) { return strFormat(" %s=%lld", k, v); }
+
+std::string vecStr(const char *k, const std::vector<int32_t> &v) {
+  std::string s = strFormat(" %s=[", k);
+  for (size_t i = 0; i < v.size(); i++) s += (i ? "," : "") + std::to_string(v[i]);
+  return s + "]";
+}
+
+} // namespace
+
+#define CHECK_OP(cond, ...)                                                    \
+  do {                                                                         \
+    if (!(cond))                                                               \
+      return MI355X_MAKE_ERR(ErrorCode::COMPILE_UNSUPPORTED_NODE_AFTER_OPTIMIZE, \
+                             "%s '%s': %s", kindName(I.kind), I.name.c_str(),  \
+                             strFormat(__VA_ARGS__).c_str());                  \
+  } while (0)
+
+namespace {
+
+class Compiler {
+public:
+  // `function` is the index of the function whose activations may be used;
+  // a negative one accepts any activation (single-instruction probes).
+  Compiler(const Module &M, const std::vector<Instruction> &insts, int function,
+           const BackendOptions &o)
+      : M_(M), insts_(insts), function_(function), opts_(o) {}
+
+  Error run(MI355XFunction &out) {
+    for (const auto &I : insts_) {
+      MI355X_RETURN_IF_ERR(checkOperands(I));
+      switch (I.kind) {
+      case Kind::Quantize: MI355X_RETURN_IF_ERR(quantize(I, out)); break;
+      case Kind::Dequantize: MI355X_RETURN_IF_ERR(dequantize(I, out)); break;
+      case Kind::RescaleQuantized: MI355X_RETURN_IF_ERR(rescale(I, out)); break;
+      case Kind::FullyConnected: MI355X_RETURN_IF_ERR(fc(I, out)); break;
+      case Kind::RowwiseQuantizedFullyConnected: MI355X_RETURN_IF_ERR(rwqfc(I, out)); break;
+      case Kind::MatMul: MI355X_RETURN_IF_ERR(matmul(I, out)); break;
+      case Kind::Convolution: MI355X_RETURN_IF_ERR(conv(I, out, false)); break;
+      case Kind::ChannelwiseQuantizedConvolution: MI355X_RETURN_IF_ERR(conv(I, out, true)); break;
+      case Kind::FusedRowwiseQuantizedSparseLengthsWeightedSum:
+        MI355X_RETURN_IF_ERR(slws(I, out, true)); break;
+      case Kind::FusedRowwiseQuantizedSparseLengthsSum:
+        MI355X_RETURN_IF_ERR(slws(I, out, false)); break;
+      default:
+        return MI355X_MAKE_ERR(ErrorCode::COMPILE_UNSUPPORTED_NODE_AFTER_OPTIMIZE,
+                               "instruction kind %d is not supported", (int)I.kind);
+      }
+    }
+    // scratch buffers follow the initialised image
+    scratchBase_ = alignUp(gen_.image_.size(), 256);
+    *scratchBasePtr_ = scratchBase_;
+    out.generated = std::move(gen_.image_);
+    genTotal_ = scratchBase_ + gen_.scratch_;
+    return Error::success();
+  }
+
+  size_t generatedTotal() const { return genTotal_; }
+  const std::map<int, std::pair<bool, bool>> &io() const { return io_; }
+
+private:
+  static constexpr int kArity[(int)Kind::NumKinds] = {2, 2, 2, 4, 6, 3, 4, 8, 5, 4};
+
+  Error checkOperands(const Instruction &I) {
+    CHECK_OP((int)I.kind >= 0 && (int)I.kind < (int)Kind::NumKinds, "unknown kind");
+    CHECK_OP((int)I.operands.size() == kArity[(int)I.kind], "expects %d operands, has %zu",
+             kArity[(int)I.kind], I.operands.size());
+    for (size_t i = 0; i < I.operands.size(); i++) {
+      const int id = I.operands[i];
+      CHECK_OP(M_.validId(id), "operand %zu is not a value of the module", i);
+      const Value &v = M_.value(id);
+      CHECK_OP(v.category != SymbolCategory::Activation || function_ < 0 ||
+                   v.function == function_,
+               "operand %zu is an activation of another function", i);
+      CHECK_OP(!(i == 0 && v.category == SymbolCategory::Constant),
+               "destination is a constant");
+      auto &f = io_[id];
+      if (i == 0) f.second = true; else f.first = true;
+    }
+    return Error::success();
+  }
+
+  Operand op(const Instruction &I, int i) const { return Operand{&M_.value(I.operands[(size_t)i])}; }
+
+  template <typename T> const T *constData(const Operand &o) const {
+    return reinterpret_cast<const T *>(M_.constantsImage().data() + o.v->offset);
+  }
+
+  // pointer into the scratch part of the generated region; the base is only
+  // known once every instruction has been seen
+  std::function<uint8_t *(const DeviceBindings &)> scratchPtr(size_t rel) {
+    auto base = scratchBasePtr_;
+    return [base, rel](const DeviceBindings &b) { return b.generated + *base + rel; };
+  }
+
+  Error quantize(const Instruction &I, MI355XFunction &out) {
+    Operand d = op(I, 0), s = op(I, 1);
+    CHECK_OP(d.ty().kind == ElemKind::Int8QTy && s.ty().kind == ElemKind::FloatTy,
+             "needs float -> i8, has %s -> %s", s.ty().str().c_str(), d.ty().str().c_str());
+    CHECK_OP(d.ty().size() == s.ty().size(), "size mismatch");
+    const size_t n = (size_t)d.ty().size();
+    const float sc = d.ty().scale;
+    const int32_t off = d.ty().offset;
+    out.launches.push_back({"mi355x_quantize_i8", I.name,
+                            strFormat(" n=%zu scale=%.9g offset=%d", n, (double)sc, off),
+                            [=](const DeviceBindings &b) {
+                              return mi355x_quantize_i8((int8_t *)d.ptr(b), (const float *)s.ptr(b),
+                                                        n, sc, off, b.stream);
+                            }});
+    return Error::success();
+  }
+
+  Error dequantize(const Instruction &I, MI355XFunction &out) {
+    Operand d = op(I, 0), s = op(I, 1);
+    CHECK_OP(d.ty().kind == ElemKind::FloatTy && s.ty().kind == ElemKind::Int8QTy,
+             "needs i8 -> float, has %s -> %s", s.ty().str().c_str(), d.ty().str().c_str());
+    CHECK_OP(d.ty().size() == s.ty().size(), "size mismatch");
+    const size_t n = (size_t)d.ty().size();
+    const float sc = s.ty().scale;
+    const int32_t off = s.ty().offset;
+    out.launches.push_back({"mi355x_dequantize_i8", I.name,
+                            strFormat(" n=%zu scale=%.9g offset=%d", n, (double)sc, off),
+                            [=](const DeviceBindings &b) {
+                              return mi355x_dequantize_i8((float *)d.ptr(b), (const int8_t *)s.ptr(b),
+                                                          n, sc, off, b.stream);
+                            }});
+    return Error::success();
+  }
+
+  Error rescale(const Instruction &I, MI355XFunction &out) {
+    Operand d = op(I, 0), s = op(I, 1);
+    CHECK_OP(d.ty().kind == ElemKind::Int8QTy && s.ty().kind == ElemKind::Int8QTy,
+             "needs i8 -> i8");
+    CHECK_OP(d.ty().size() == s.ty().size(), "size mismatch");
+    const size_t n = (size_t)d.ty().size();
+    const S32To8 p = s32to8(s.ty().scale / d.ty().scale);
+    const int32_t oo = d.ty().offset, io = s.ty().offset;
+    out.launches.push_back(
+        {"mi355x_rescale_i8", I.name,
+         strFormat(" n=%zu", n) + kv("out_offset", oo) + kv("in_offset", io) +
+             kv("pre", p.pre) + kv("post", p.post) + kv("scale", p.scale),
+         [=](const DeviceBindings &b) {
+           return mi355x_rescale_i8((int8_t *)d.ptr(b), (const int8_t *)s.ptr(b), n, oo, io,
+                                    p.pre, p.post, p.scale, b.stream);
+         }});
+    return Error::success();
+  }
+
+  static bool biasKindOk(ElemKind k) { return k == ElemKind::Int32QTy || k == ElemKind::Int8QTy; }
+
+  Error fc(const Instruction &I, MI355XFunction &out) {
+    Operand d = op(I, 0), s = op(I, 1), w = op(I, 2), bi = op(I, 3);
+    CHECK_OP(d.ty().kind == ElemKind::Int8QTy && s.ty().kind == ElemKind::Int8QTy &&
+                 w.ty().kind == ElemKind::Int8QTy && biasKindOk(bi.ty().kind),
+             "needs i8 input, weights and output and an i32 or i8 bias");
+    CHECK_OP(s.ty().dims.size() == 2 && w.ty().dims.size() == 2 && d.ty().dims.size() == 2 &&
+                 bi.ty().dims.size() == 1,
+             "needs 2-D input, weights and output and a 1-D bias");
+    const size_t M = (size_t)s.ty().dims[0], K = (size_t)s.ty().dims[1], N = (size_t)w.ty().dims[1];
+    CHECK_OP((size_t)w.ty().dims[0] == K && (size_t)d.ty().dims[0] == M &&
+                 (size_t)d.ty().dims[1] == N && (size_t)bi.ty().dims[0] == N,
+             "shape mismatch: %s x %s + %s -> %s", s.ty().str().c_str(), w.ty().str().c_str(),
+             bi.ty().str().c_str(), d.ty().str().c_str());
+    const float mm = s.ty().scale * w.ty().scale;
+    const S32To8 bp = s32to8(bi.ty().scale / mm), opp = s32to8(mm / d.ty().scale);
+    const int bias8 = bi.ty().kind == ElemKind::Int8QTy;
+    const int32_t oo = d.ty().offset, io = s.ty().offset, wo = w.ty().offset, bo = bi.ty().offset;
+    auto work = scratchPtr(gen_.addScratch(K * N));
+    const bool wConst = w.v->category == SymbolCategory::Constant;
+    const bool sums = wConst && opts_.precomputeWeightRowSums && io != 0;
+    auto sumPtr = scratchPtr(sums ? gen_.addScratch(N * 4) : 0);
+    if (wConst) {
+      out.setup.push_back({"mi355x_transpose2d_i8", I.name, strFormat(" rows=%zu cols=%zu", K, N),
+                           [=](const DeviceBindings &b) {
+                             return mi355x_transpose2d_i8((int8_t *)work(b), (const int8_t *)w.ptr(b),
+                                                          K, N, b.stream);
+                           }});
+      if (sums)
+        out.setup.push_back({"mi355x_rowsum_i8", I.name, strFormat(" rows=%zu K=%zu", N, K),
+                             [=](const DeviceBindings &b) {
+                               return mi355x_rowsum_i8((int32_t *)sumPtr(b), (const int8_t *)work(b),
+                                                       N, K, b.stream);
+                             }});
+    }
+    const int repack = wConst ? 0 : 1;
+    out.launches.push_back(
+        {"mi355x_fc_i8", I.name,
+         strFormat(" M=%zu K=%zu N=%zu", M, K, N) + kv("out_offset", oo) + kv("in_offset", io) +
+             kv("weights_offset", wo) + kv("bias_offset", bo) + kv("bias_pre", bp.pre) +
+             kv("bias_post", bp.post) + kv("bias_scale", bp.scale) + kv("out_pre", opp.pre) +
+             kv("out_post", opp.post) + kv("out_scale", opp.scale) + kv("bias_is_i8", bias8) +
+             kv("repack", repack) + kv("row_sums", sums),
+         [=](const DeviceBindings &b) {
+           return mi355x_fc_i8((int8_t *)d.ptr(b), (const int8_t *)s.ptr(b), (const int8_t *)w.ptr(b),
+                               (int8_t *)work(b), repack, bi.ptr(b), bias8, M, K, N, oo, io, wo, bo,
+                               bp.pre, bp.post, bp.scale, opp.pre, opp.post, opp.scale,
+                               sums ? (const int32_t *)sumPtr(b) : nullptr, b.stream);
+         }});
+    return Error::success();
+  }
+
+  Error matmul(const Instruction &I, MI355XFunction &out) {
+    Operand d = op(I, 0), l = op(I, 1), r = op(I, 2);
+    CHECK_OP(d.ty().kind == ElemKind::Int8QTy && l.ty().kind == ElemKind::Int8QTy &&
+                 r.ty().kind == ElemKind::Int8QTy,
+             "needs i8 operands");
+    CHECK_OP(l.ty().dims.size() == 2 && r.ty().dims.size() == 2 && d.ty().dims.size() == 2,
+             "needs 2-D operands");
+    const size_t M = (size_t)l.ty().dims[0], K = (size_t)l.ty().dims[1], N = (size_t)r.ty().dims[1];
+    CHECK_OP((size_t)r.ty().dims[0] == K && (size_t)d.ty().dims[0] == M && (size_t)d.ty().dims[1] == N,
+             "shape mismatch");
+    const S32To8 p = s32to8(l.ty().scale * r.ty().scale / d.ty().scale);
+    const int32_t oo = d.ty().offset, lo = l.ty().offset, ro = r.ty().offset;
+    auto work = scratchPtr(gen_.addScratch(K * N));
+    const bool rConst = r.v->category == SymbolCategory::Constant;
+    if (rConst)
+      out.setup.push_back({"mi355x_transpose2d_i8", I.name, strFormat(" rows=%zu cols=%zu", K, N),
+                           [=](const DeviceBindings &b) {
+                             return mi355x_transpose2d_i8((int8_t *)work(b), (const int8_t *)r.ptr(b),
+                                                          K, N, b.stream);
+                           }});
+    const int repack = rConst ? 0 : 1;
+    out.launches.push_back(
+        {"mi355x_matmul_i8", I.name,
+         strFormat(" M=%zu K=%zu N=%zu", M, K, N) + kv("out_offset", oo) + kv("lhs_offset", lo) +
+             kv("rhs_offset", ro) + kv("out_pre", p.pre) + kv("out_post", p.post) +
+             kv("out_scale", p.scale) + kv("repack", repack),
+         [=](const DeviceBindings &b) {
+           return mi355x_matmul_i8((int8_t *)d.ptr(b), (const int8_t *)l.ptr(b), (const int8_t *)r.ptr(b),
+                                   (int8_t *)work(b), repack, M, K, N, oo, lo, ro, p.pre, p.post,
+                                   p.scale, b.stream);
+         }});
+    return Error::success();
+  }
+
+  Error rwqfc(const Instruction &I, MI355XFunction &out) {
+    Operand d = op(I, 0), s = op(I, 1), w = op(I, 2), bi = op(I, 3), sc = op(I, 4), of = op(I, 5);
+    CHECK_OP(d.ty().kind == ElemKind::Int8QTy && s.ty().kind == ElemKind::Int8QTy &&
+                 w.ty().kind == ElemKind::Int8QTy && biasKindOk(bi.ty().kind),
+             "needs i8 input, weights and output and an i32 or i8 bias");
+    CHECK_OP(sc.ty().kind == ElemKind::FloatTy && of.ty().kind == ElemKind::Int32ITy,
+             "needs float scales and int32 offsets");
+    CHECK_OP(sc.v->category == SymbolCategory::Constant && of.v->category == SymbolCategory::Constant &&
+                 w.v->category == SymbolCategory::Constant,
+             "weights, scales and offsets must be constants");
+    CHECK_OP(s.ty().dims.size() == 2 && w.ty().dims.size() == 2 && d.ty().dims.size() == 2,
+             "needs 2-D input, weights and output");
+    const size_t M = (size_t)s.ty().dims[0], K = (size_t)s.ty().dims[1], N = (size_t)w.ty().dims[0];
+    CHECK_OP((size_t)w.ty().dims[1] == K && (size_t)d.ty().dims[0] == M &&
+                 (size_t)d.ty().dims[1] == N && (size_t)bi.ty().size() == N &&
+                 (size_t)sc.ty().size() == N && (size_t)of.ty().size() == N,
+             "shape mismatch: %s x %s^T + %s -> %s", s.ty().str().c_str(), w.ty().str().c_str(),
+             bi.ty().str().c_str(), d.ty().str().c_str());
+    const float *scales = constData<float>(sc);
+    const int32_t *offsets = constData<int32_t>(of);
+    std::vector<int32_t> bpre(N), bpost(N), bscale(N), opre(N), opost(N), oscale(N);
+    bool allZero = true;
+    for (size_t j = 0; j < N; j++) {
+      const float mm = s.ty().scale * scales[j];
+      const S32To8 bp = s32to8(bi.ty().scale / mm), opp = s32to8(mm / d.ty().scale);
+      bpre[j] = bp.pre; bpost[j] = bp.post; bscale[j] = bp.scale;
+      opre[j] = opp.pre; opost[j] = opp.post; oscale[j] = opp.scale;
+      allZero = allZero && offsets[j] == 0;
+    }
+    const size_t o0 = gen_.addI32(bpre), o1 = gen_.addI32(bpost), o2 = gen_.addI32(bscale),
+                 o3 = gen_.addI32(opre), o4 = gen_.addI32(opost), o5 = gen_.addI32(oscale);
+    const int bias8 = bi.ty().kind == ElemKind::Int8QTy;
+    const int32_t oo = d.ty().offset, io = s.ty().offset, bo = bi.ty().offset;
+    const bool sums = opts_.precomputeWeightRowSums && io != 0;
+    auto sumPtr = scratchPtr(sums ? gen_.addScratch(N * 4) : 0);
+    if (sums)
+      out.setup.push_back({"mi355x_rowsum_i8", I.name, strFormat(" rows=%zu K=%zu", N, K),
+                           [=](const DeviceBindings &b) {
+                             return mi355x_rowsum_i8((int32_t *)sumPtr(b), (const int8_t *)w.ptr(b), N,
+                                                     K, b.stream);
+                           }});
+    out.launches.push_back(
+        {"mi355x_rwq_fc_i8", I.name,
+         strFormat(" M=%zu K=%zu N=%zu", M, K, N) + kv("out_offset", oo) + kv("in_offset", io) +
+             kv("bias_offset", bo) + kv("bias_is_i8", bias8) + kv("weights_offsets_all_zero", allZero) +
+             kv("row_sums", sums) + vecStr("bias_pre", bpre) + vecStr("bias_post", bpost) +
+             vecStr("bias_scale", bscale) + vecStr("out_pre", opre) + vecStr("out_post", opost) +
+             vecStr("out_scale", oscale),
+         [=](const DeviceBindings &b) {
+           auto g = [&](size_t o) { return (const int32_t *)(b.generated + o); };
+           return mi355x_rwq_fc_i8((int8_t *)d.ptr(b), (const int8_t *)s.ptr(b), (const int8_t *)w.ptr(b),
+                                   bi.ptr(b), bias8, (const int32_t *)of.ptr(b), g(o0), g(o1), g(o2),
+                                   g(o3), g(o4), g(o5), M, K, N, oo, io, bo, allZero ? 1 : 0,
+                                   sums ? (const int32_t *)sumPtr(b) : nullptr, b.stream);
+         }});
+    return Error::success();
+  }
+
+  Error conv(const Instruction &I, MI355XFunction &out, bool channelwise) {
+    Operand d = op(I, 0), s = op(I, 1), f = op(I, 2), bi = op(I, 3);
+    CHECK_OP((int)I.iattrs.size() == ConvAttrs::kCount, "expects %d integer attributes",
+             ConvAttrs::kCount);
+    CHECK_OP(d.ty().kind == ElemKind::Int8QTy && s.ty().kind == ElemKind::Int8QTy &&
+                 f.ty().kind == ElemKind::Int8QTy && biasKindOk(bi.ty().kind),
+             "needs i8 input, filter and output and an i32 or i8 bias");
+    CHECK_OP(s.ty().dims.size() == 4 && f.ty().dims.size() == 4 && d.ty().dims.size() == 4,
+             "needs NHWC input and output and an [OC,KH,KW,IC/group] filter");
+    const auto &a = I.iattrs;
+    mi355x_conv_geom g;
+    g.N = (int32_t)s.ty().dims[0]; g.IH = (int32_t)s.ty().dims[1];
+    g.IW = (int32_t)s.ty().dims[2]; g.IC = (int32_t)s.ty().dims[3];
+    g.OH = (int32_t)d.ty().dims[1]; g.OW = (int32_t)d.ty().dims[2]; g.OC = (int32_t)d.ty().dims[3];
+    g.KH = (int32_t)a[0]; g.KW = (int32_t)a[1]; g.strideH = (int32_t)a[2]; g.strideW = (int32_t)a[3];
+    g.padT = (int32_t)a[4]; g.padL = (int32_t)a[5];
+    const int64_t padB = a[6], padR = a[7];
+    g.group = (int32_t)a[8]; g.dilH = (int32_t)a[9]; g.dilW = (int32_t)a[10];
+    const int32_t act = (int32_t)a[11];
+    CHECK_OP(g.KH > 0 && g.KW > 0 && g.strideH > 0 && g.strideW > 0 && g.group > 0 && g.dilH > 0 &&
+                 g.dilW > 0 && g.padT >= 0 && g.padL >= 0 && padB >= 0 && padR >= 0,
+             "invalid kernel, stride, pad, group or dilation");
+    CHECK_OP(g.IC % g.group == 0 && g.OC % g.group == 0, "channels not divisible by group");
+    CHECK_OP(f.ty().dims[0] == g.OC && f.ty().dims[1] == g.KH && f.ty().dims[2] == g.KW &&
+                 f.ty().dims[3] == g.IC / g.group,
+             "filter %s does not match", f.ty().str().c_str());
+    CHECK_OP(d.ty().dims[0] == g.N && bi.ty().size() == g.OC, "batch or bias size mismatch");
+    // calculateConvPoolOutputDims (reference include/glow/Graph/Nodes.h / Utils)
+    const int64_t oh = (g.IH + g.padT + padB - (g.KH - 1) * g.dilH - 1) / g.strideH + 1;
+    const int64_t ow = (g.IW + g.padL + padR - (g.KW - 1) * g.dilW - 1) / g.strideW + 1;
+    CHECK_OP(oh == g.OH && ow == g.OW, "output %s does not match the computed %lld x %lld",
+             d.ty().str().c_str(), (long long)oh, (long long)ow);
+    CHECK_OP(act == NONE || act == RELU || act == CLIP || act == LEAKY_RELU,
+             "fused activation %d is not supported for quantized types", act);
+    // emitConstQuantActivationArgs (LLVMIRGen.cpp:618-662)
+    std::vector<int32_t> actArgs(3, 0);
+    if (act == CLIP) {
+      CHECK_OP(I.fattrs.size() == 2, "fused Clip needs {min, max}");
+      actArgs[0] = quantizeI32(I.fattrs[0], d.ty().scale, d.ty().offset);
+      actArgs[1] = quantizeI32(I.fattrs[1], d.ty().scale, d.ty().offset);
+    } else if (act == LEAKY_RELU) {
+      CHECK_OP(I.fattrs.size() == 1, "fused LeakyRelu needs {alpha}");
+      const S32To8 p = s32to8(I.fattrs[0]);
+      actArgs = {p.pre, p.post, p.scale};
+    } else {
+      CHECK_OP(I.fattrs.empty(), "activation takes no arguments");
+    }
+    CHECK_OP(f.v->category == SymbolCategory::Constant, "filter must be a constant");
+    const size_t OC = (size_t)g.OC, Kf = (size_t)g.KH * g.KW * (g.IC / g.group);
+    const int bias8 = bi.ty().kind == ElemKind::Int8QTy;
+    const int32_t oo = d.ty().offset, io = s.ty().offset;
+    const bool sums = opts_.precomputeWeightRowSums && io != 0;
+    auto sumPtr = scratchPtr(sums ? gen_.addScratch(OC * 4) : 0);
+    if (sums)
+      out.setup.push_back({"mi355x_rowsum_i8", I.name, strFormat(" rows=%zu K=%zu", OC, Kf),
+                           [=](const DeviceBindings &b) {
+                             return mi355x_rowsum_i8((int32_t *)sumPtr(b), (const int8_t *)f.ptr(b), OC,
+                                                     Kf, b.stream);
+                           }});
+    std::string geomStr = strFormat(" N=%d IH=%d IW=%d IC=%d OH=%d OW=%d OC=%d KH=%d KW=%d sH=%d sW=%d "
+                                    "padT=%d padL=%d dH=%d dW=%d group=%d",
+                                    g.N, g.IH, g.IW, g.IC, g.OH, g.OW, g.OC, g.KH, g.KW, g.strideH,
+                                    g.strideW, g.padT, g.padL, g.dilH, g.dilW, g.group);
+    if (!channelwise) {
+      const float mm = s.ty().scale * f.ty().scale;
+      const S32To8 bp = s32to8(bi.ty().scale / mm), opp = s32to8(mm / d.ty().scale);
+      const int32_t fo = f.ty().offset, bo = bi.ty().offset;
+      out.launches.push_back(
+          {"mi355x_conv2d_i8", I.name,
+           geomStr + kv("out_offset", oo) + kv("in_offset", io) + kv("filter_offset", fo) +
+               kv("bias_offset", bo) + kv("bias_pre", bp.pre) + kv("bias_post", bp.post) +
+               kv("bias_scale", bp.scale) + kv("out_pre", opp.pre) + kv("out_post", opp.post) +
+               kv("out_scale", opp.scale) + kv("act", act) + vecStr("act_args", actArgs) +
+               kv("bias_is_i8", bias8) + kv("row_sums", sums),
+           [=](const DeviceBindings &b) {
+             return mi355x_conv2d_i8((int8_t *)d.ptr(b), (const int8_t *)s.ptr(b), (const int8_t *)f.ptr(b),
+                                     bi.ptr(b), bias8, &g, oo, io, fo, bo, bp.pre, bp.post, bp.scale,
+                                     opp.pre, opp.post, opp.scale, act, actArgs.data(),
+                                     sums ? (const int32_t *)sumPtr(b) : nullptr, b.stream);
+           }});
+      return Error::success();
+    }
+    Operand fs = op(I, 4), fo = op(I, 5), bs = op(I, 6), bo = op(I, 7);
+    CHECK_OP(fs.ty().kind == ElemKind::FloatTy && bs.ty().kind == ElemKind::FloatTy &&
+                 fo.ty().kind == ElemKind::Int32ITy && bo.ty().kind == ElemKind::Int32ITy,
+             "needs float scales and int32 offsets");
+    CHECK_OP(fs.v->category == SymbolCategory::Constant && fo.v->category == SymbolCategory::Constant &&
+                 bs.v->category == SymbolCategory::Constant && bo.v->category == SymbolCategory::Constant,
+             "filter/bias scales and offsets must be constants");
+    CHECK_OP((size_t)fs.ty().size() == OC && (size_t)fo.ty().size() == OC &&
+                 (size_t)bs.ty().size() == OC && (size_t)bo.ty().size() == OC,
+             "per-channel vectors must have one entry per output channel");
+    const float *fsc = constData<float>(fs), *bsc = constData<float>(bs);
+    const int32_t *fof = constData<int32_t>(fo);
+    std::vector<int32_t> bpre(OC), bpost(OC), bscale(OC), opre(OC), opost(OC), oscale(OC);
+    bool allZero = true;
+    for (size_t c = 0; c < OC; c++) {
+      const float mm = s.ty().scale * fsc[c];
+      const S32To8 bp = s32to8(bsc[c] / mm), opp = s32to8(mm / d.ty().scale);
+      bpre[c] = bp.pre; bpost[c] = bp.post; bscale[c] = bp.scale;
+      opre[c] = opp.pre; opost[c] = opp.post; oscale[c] = opp.scale;
+      allZero = allZero && fof[c] == 0;
+    }
+    const size_t o0 = gen_.addI32(bpre), o1 = gen_.addI32(bpost), o2 = gen_.addI32(bscale),
+                 o3 = gen_.addI32(opre), o4 = gen_.addI32(opost), o5 = gen_.addI32(oscale);
+    out.launches.push_back(
+        {"mi355x_cwq_conv2d_i8", I.name,
+         geomStr + kv("out_offset", oo) + kv("in_offset", io) + kv("act", act) +
+             vecStr("act_args", actArgs) + kv("bias_is_i8", bias8) +
+             kv("filter_offsets_all_zero", allZero) + kv("row_sums", sums) + vecStr("bias_pre", bpre) +
+             vecStr("bias_post", bpost) + vecStr("bias_scale", bscale) + vecStr("out_pre", opre) +
+             vecStr("out_post", opost) + vecStr("out_scale", oscale),
+         [=](const DeviceBindings &b) {
+           auto gp = [&](size_t o) { return (const int32_t *)(b.generated + o); };
+           return mi355x_cwq_conv2d_i8((int8_t *)d.ptr(b), (const int8_t *)s.ptr(b),
+                                       (const int8_t *)f.ptr(b), bi.ptr(b), bias8, &g, oo, io,
+                                       (const int32_t *)fo.ptr(b), (const int32_t *)bo.ptr(b), gp(o0),
+                                       gp(o1), gp(o2), gp(o3), gp(o4), gp(o5), act, actArgs.data(),
+                                       allZero ? 1 : 0, sums ? (const int32_t *)sumPtr(b) : nullptr,
+                                       b.stream);
+         }});
+    return Error::success();
+  }
+
+  Error slws(const Instruction &I, MI355XFunction &out, bool weighted) {
+    Operand d = op(I, 0), data = op(I, 1);
+    Operand w = weighted ? op(I, 2) : Operand{nullptr};
+    Operand idx = op(I, weighted ? 3 : 2), len = op(I, weighted ? 4 : 3);
+    CHECK_OP(isFused(data.ty().kind) && data.ty().dims.size() == 2,
+             "data must be a 2-D fused-rowwise tensor, has %s", data.ty().str().c_str());
+    int kind = MI355X_FUSED_U8_F32;
+    bool fp16Scale = false, fourBit = false;
+    switch (data.ty().kind) {
+    case ElemKind::UInt8FusedQTy: kind = MI355X_FUSED_U8_F32; break;
+    case ElemKind::UInt8FusedFP16QTy: kind = MI355X_FUSED_U8_F16; fp16Scale = true; break;
+    case ElemKind::UInt4FusedFP16QTy: kind = MI355X_FUSED_U4_F16; fp16Scale = fourBit = true; break;
+    default: kind = MI355X_FUSED_U4_F32; fourBit = true; break;
+    }
+    const ElemKind dk = d.ty().kind;
+    CHECK_OP(dk == ElemKind::FloatTy || dk == ElemKind::Float16Ty, "result must be float or float16");
+    // type legality of the reference (lib/Backends/Interpreter/Interpreter.cpp:526-567)
+    if (fp16Scale)
+      CHECK_OP(dk == ElemKind::Float16Ty, "fp16-scale data needs a float16 result");
+    ElemKind wk = dk; // the lowered plain sum uses a splat of the result kind
+    if (weighted) {
+      wk = w.ty().kind;
+      CHECK_OP(wk == ElemKind::FloatTy || wk == ElemKind::Float16Ty, "weights must be float or float16");
+      if (!fp16Scale)
+        CHECK_OP(wk == dk, "fp32-scale data needs weights and result of the same kind");
+    }
+    CHECK_OP(idx.ty().kind == ElemKind::Int64ITy || idx.ty().kind == ElemKind::Int32ITy,
+             "indices must be int64 or int32");
+    CHECK_OP(len.ty().kind == ElemKind::Int32ITy, "lengths must be int32");
+    CHECK_OP(d.ty().dims.size() == 2 && d.ty().dims[0] == len.ty().size(),
+             "result must be [lengths x columns]");
+    if (weighted) CHECK_OP(w.ty().size() == idx.ty().size(), "weights and indices differ in size");
+    const size_t rows = (size_t)data.ty().dims[0], inLine = (size_t)data.ty().dims[1];
+    const size_t outLine = (size_t)d.ty().dims[1];
+    const size_t so = fp16Scale ? 4 : 8;
+    CHECK_OP(inLine > so && (inLine - so) * (fourBit ? 2 : 1) == outLine,
+             "row of %zu bytes does not hold %zu columns", inLine, outLine);
+    const bool acc16 = !I.iattrs.empty() && I.iattrs[0] != 0 && fp16Scale;
+    const size_t nIdx = (size_t)idx.ty().size(), segs = (size_t)len.ty().size();
+    const int out16 = dk == ElemKind::Float16Ty, w16 = wk == ElemKind::Float16Ty;
+    const int idx64 = idx.ty().kind == ElemKind::Int64ITy;
+    out.launches.push_back(
+        {"mi355x_frwq_slws", I.name,
+         strFormat(" rows=%zu in_line=%zu out_line=%zu segments=%zu num_indices=%zu", rows, inLine,
+                   outLine, segs, nIdx) +
+             kv("kind", kind) + kv("out_is_f16", out16) + kv("weighted", weighted) +
+             kv("weights_are_f16", w16) + kv("idx_is_64", idx64) + kv("fp16_accum", acc16),
+         [=](const DeviceBindings &b) {
+           return mi355x_frwq_slws(d.ptr(b), out16, data.ptr(b), rows, kind,
+                                   weighted ? (const void *)w.ptr(b) : nullptr, w16, idx.ptr(b), idx64,
+                                   nIdx, (const int32_t *)len.ptr(b), segs, inLine, outLine,
+                                   acc16 ? 1 : 0, b.stream);
+         }});
+    return Error::success();
+  }
+
+  const Module &M_;
+  const std::vector<Instruction> &insts_;
+  int function_;
+  BackendOptions opts_;
+  Generated gen_;
+  size_t scratchBase_ = 0, genTotal_ = 0;
+  std::shared_ptr<size_t> scratchBasePtr_ = std::make_shared<size_t>(0);
+  std::map<int, std::pair<bool, bool>> io_; // value id -> (read, written)
+};
+
+constexpr int Compiler::kArity[];
+
+} // namespace
+
+Expected<std::unique_ptr<MI355XFunction>> MI355XBackend::compile(const Function &F,
+                                                                 const BackendOptions &opts) const {
+  const Module &M = *F.module();
+  Compiler C(M, F.instructions(), F.index(), opts);
+  auto fn = std::unique_ptr<MI355XFunction>(new MI355XFunction(RuntimeBundle(), F.name()));
+  Error e = C.run(*fn);
+  if (e) return e;
+  RuntimeBundle rb;
+  rb.constantWeightVarsMemSize = M.constantsSize();
+  rb.mutableWeightVarsMemSize = M.mutableSize();
+  rb.activationsMemSize = F.activationsSize();
+  rb.generatedConstantsMemSize = C.generatedTotal();
+  for (int id = 0; id < M.numValues(); id++) {
+    const Value &v = M.value(id);
+    if (v.category == SymbolCategory::Activation && v.function != F.index()) continue;
+    RuntimeSymbolInfo si;
+    si.size = v.type.sizeInBytes();
+    si.offset = v.offset;
+    si.type = v.type;
+    si.symbolCategory = v.category;
+    auto it = C.io().find(id);
+    if (it != C.io().end() && v.category == SymbolCategory::Placeholder) {
+      si.input = it->second.first;
+      si.output = it->second.second;
+    }
+    rb.symbolTable[v.name] = si;
+  }
+  fn->setRuntimeBundle(std::move(rb));
+  return fn;
+}
+
+bool MI355XBackend::isOpSupported(const Module &M, const Instruction &I, std::string *why) const {
+  std::vector<Instruction> one{I};
+  Compiler C(M, one, -1, BackendOptions());
+  MI355XFunction scratch(RuntimeBundle(), "probe");
+  Error e = C.run(scratch);
+  if (e && why) *why = e.message();
+  return !e;
+}
+
+bool MI355XBackend::shouldLower(Kind k) const {
+  switch (k) {
+  case Kind::FullyConnected:
+  case Kind::Convolution:
+  case Kind::RowwiseQuantizedFullyConnected:
+  case Kind::ChannelwiseQuantizedConvolution:
+    return false;
+  default:
+    return true;
+  }
+}
+
+bool MI355XBackend::supportsFusedActivation(Kind parent, FusedActivation act) const {
+  if (parent != Kind::Convolution && parent != Kind::ChannelwiseQuantizedConvolution) return false;
+  return act == RELU || act == CLIP || act == LEAKY_RELU;
+}
+
+unsigned MI355XBackend::numDevices() {
+  int n = 0;
+  if (mi355x_num_devices(&n) != MI355X_OK) return 0;
+  return n < 0 ? 0u : (unsigned)n;
+}
+
+MI355XFunction::~MI355XFunction() { dropGraph(); }
+
+void MI355XFunction::dropGraph() {
+  if (graph_) {
+    mi355x_graph_destroy(graph_);
+    graph_ = nullptr;
+  }
+}
+
+static bool sameBindings(const DeviceBindings &a, const DeviceBindings &b) {
+  return a.constants == b.constants && a.generated == b.generated &&
+         a.mutableMem == b.mutableMem && a.activations == b.activations;
+}
+
+Error MI355XFunction::captureGraph(const DeviceBindings &b) {
+  dropGraph();
+  if (launches.empty()) return Error::success();
+  if (!b.stream)
+    return MI355X_MAKE_ERR(ErrorCode::RUNTIME_ERROR, "graph capture needs a created stream");
+  if (mi355x_graph_begin_capture(b.stream) != MI355X_OK)
+    return MI355X_MAKE_ERR(ErrorCode::RUNTIME_ERROR, "%s", mi355x_last_error());
+  int rc = MI355X_OK;
+  std::string failed;
+  for (const auto &l : launches) {
+    rc = l.run(b);
+    if (rc != MI355X_OK) {
+      failed = l.kernel + " (" + l.inst + "): " + mi355x_last_error();
+      break;
+    }
+  }
+  mi355x_graph *g = nullptr;
+  const int rc2 = mi355x_graph_end_capture(b.stream, &g);
+  if (rc != MI355X_OK) {
+    if (g) mi355x_graph_destroy(g);
+    return MI355X_MAKE_ERR(ErrorCode::RUNTIME_ERROR, "%s", failed.c_str());
+  }
+  if (rc2 != MI355X_OK)
+    return MI355X_MAKE_ERR(ErrorCode::RUNTIME_ERROR, "%s", mi355x_last_error());
+  graph_ = g;
+  graphBindings_ = b;
+  return Error::success();
+}
+
+Error MI355XFunction::execute(ExecutionContext *ctx) {
+  DeviceBindings *b = ctx ? ctx->getDeviceBindings() : nullptr;
+  if (!b)
+    return MI355X_MAKE_ERR(ErrorCode::RUNTIME_ERROR,
+                           "function %s executed without device bindings", name_.c_str());
+  if (graph_ && sameBindings(*b, graphBindings_)) {
+    if (mi355x_graph_launch(graph_, b->stream) != MI355X_OK)
+      return MI355X_MAKE_ERR(ErrorCode::RUNTIME_ERROR, "%s", mi355x_last_error());
+    return Error::success();
+  }
+  for (const auto &l : launches) {
+    const int rc = l.run(*b);
+    if (rc != MI355X_OK)
+      return MI355X_MAKE_ERR(rc == MI355X_ERR_NOT_SUPPORTED ? ErrorCode::DEVICE_FEATURE_NOT_SUPPORTED
+                                                            : ErrorCode::RUNTIME_ERROR,
+                             "%s (%s): %s", l.kernel.c_str(), l.inst.c_str(), mi355x_last_error());
+  }
+  return Error::success();
+}
+
+std::string MI355XFunction::describe() const {
+  std::ostringstream os;
+  os << "function " << name_ << " constants=" << bundle_.constantWeightVarsMemSize
+     << " generated=" << bundle_.generatedConstantsMemSize
+     << " mutable=" << bundle_.mutableWeightVarsMemSize
+     << " activations=" << bundle_.activationsMemSize << "\n";
+  for (const auto &l : setup) os << "setup " << l.kernel << " inst=" << l.inst << l.params << "\n";
+  for (const auto &l : launches) os << "launch " << l.kernel << " inst=" << l.inst << l.params << "\n";
+  return os.str();
+}
+
+} // namespace glow_mi355x

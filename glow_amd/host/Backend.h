@@ -1,0 +1,144 @@
+// MI355XBackend and MI355XFunction: the compile side of the drop-in boundary.
+// Mirrors glow::Backend (reference include/glow/Backend/Backend.h:67-325) and
+// glow::CompiledFunction (include/glow/Backend/CompiledFunction.h:29-98) for
+// the quantized hot path; kernels are reached only through the C ABI of
+// glow_mi355x.h.
+#ifndef GLOW_MI355X_HOST_BACKEND_H
+#define GLOW_MI355X_HOST_BACKEND_H
+
+#include "Program.h"
+
+#include <functional>
+#include <map>
+#include <memory>
+#include <string>
+#include <vector>
+
+struct mi355x_graph;
+
+namespace glow_mi355x {
+
+// Where a run's buffers live on the device (ExecutionContext::DeviceBindings,
+// reference include/glow/ExecutionContext/ExecutionContext.h:31-43).
+struct DeviceBindings {
+  uint8_t *constants = nullptr;   // module constants
+  uint8_t *generated = nullptr;   // constants the compiler derived for one function
+  uint8_t *mutableMem = nullptr;  // placeholders
+  uint8_t *activations = nullptr; // one function's activations
+  void *stream = nullptr;
+};
+
+// PlaceholderBindings: placeholder name -> host tensor (not owned).
+class PlaceholderBindings {
+public:
+  void insert(const std::string &name, Tensor *t) { map_[name] = t; }
+  Tensor *get(const std::string &name) const {
+    auto it = map_.find(name);
+    return it == map_.end() ? nullptr : it->second;
+  }
+  const std::map<std::string, Tensor *> &pairs() const { return map_; }
+
+private:
+  std::map<std::string, Tensor *> map_;
+};
+
+class ExecutionContext {
+public:
+  PlaceholderBindings *getPlaceholderBindings() { return &bindings_; }
+  void setDeviceBindings(std::unique_ptr<DeviceBindings> b) { device_ = std::move(b); }
+  DeviceBindings *getDeviceBindings() { return device_.get(); }
+
+private:
+  PlaceholderBindings bindings_;
+  std::unique_ptr<DeviceBindings> device_;
+};
+
+// RuntimeSymbolInfo (BackendUtils.h:41-62)
+struct RuntimeSymbolInfo {
+  size_t size = 0, offset = 0;
+  Type type;
+  bool input = false, output = false;
+  SymbolCategory symbolCategory = SymbolCategory::Activation;
+};
+
+// RuntimeBundle (BackendUtils.h:66-150): sizes of the regions and the table.
+struct RuntimeBundle {
+  std::map<std::string, RuntimeSymbolInfo> symbolTable;
+  size_t constantWeightVarsMemSize = 0;
+  size_t mutableWeightVarsMemSize = 0;
+  size_t activationsMemSize = 0;
+  size_t generatedConstantsMemSize = 0; // no counterpart: kernel parameter vectors
+  size_t getConstantWeightSize() const {
+    return constantWeightVarsMemSize + generatedConstantsMemSize;
+  }
+};
+
+// One kernel launch of a compiled function.
+struct KernelLaunch {
+  std::string kernel;  // C-ABI entry point
+  std::string inst;    // instruction name
+  std::string params;  // the derived integer parameters, for inspection
+  std::function<int(const DeviceBindings &)> run; // returns an mi355x_status
+};
+
+class MI355XFunction {
+public:
+  MI355XFunction(RuntimeBundle bundle, std::string name)
+      : bundle_(std::move(bundle)), name_(std::move(name)) {}
+  ~MI355XFunction();
+
+  // CompiledFunction::execute: the context must carry DeviceBindings (the
+  // device manager sets them). Launches are asynchronous on the bound stream.
+  Error execute(ExecutionContext *ctx);
+  std::string getCompileBackendName() const { return "MI355X"; }
+  const RuntimeBundle &getRuntimeBundle() const { return bundle_; }
+  void setRuntimeBundle(RuntimeBundle b) { bundle_ = std::move(b); }
+  const std::string &name() const { return name_; }
+
+  // Launch lists: `setup` runs once after the constants are resident (weight
+  // repacking, row sums); `launches` is the function body.
+  std::vector<KernelLaunch> setup, launches;
+  // Host image of the generated constants (uploaded by the device manager).
+  std::vector<uint8_t> generated;
+  // Text listing of the launches with their parameters.
+  std::string describe() const;
+
+  // Records the body into a launch graph bound to these buffers; later
+  // execute() calls with the same bindings replay it.
+  Error captureGraph(const DeviceBindings &b);
+  void dropGraph();
+
+private:
+  RuntimeBundle bundle_;
+  std::string name_;
+  mi355x_graph *graph_ = nullptr;
+  DeviceBindings graphBindings_;
+};
+
+struct BackendOptions {
+  bool precomputeWeightRowSums = true; // form sum_k W[n][k] once at load time
+};
+
+class MI355XBackend {
+public:
+  std::string getBackendName() const { return getName(); }
+  static std::string getName() { return "MI355X"; }
+  static unsigned numDevices(); // devices the runtime reports (0 without a GPU)
+
+  // Backend::compile (Backend.h:108-109)
+  Expected<std::unique_ptr<MI355XFunction>> compile(const Function &F,
+                                                    const BackendOptions &opts = {}) const;
+  // Backend::isOpSupported (Backend.h:145): by instruction kind and operand types.
+  bool isOpSupported(const Module &M, const Instruction &I, std::string *why = nullptr) const;
+  // Backend::shouldLower (Backend.h:197): FullyConnected, Convolution stay
+  // un-lowered like on the CPU backend (CPUBackend.cpp:71-84).
+  bool shouldLower(Kind k) const;
+  // Backend::supportsFusedActivation (Backend.h:228-230, CPUBackend.cpp:86-112)
+  bool supportsFusedActivation(Kind parent, FusedActivation act) const;
+  // Backend::canDoIndexTypeDemotion: SLS indices stay int64 like on the CPU
+  // backend (CPUBackend.cpp:147-159); int32 indices are accepted as given.
+  bool canDoIndexTypeDemotion(Kind k) const { (void)k; return false; }
+};
+
+} // namespace glow_mi355x
+#endif

@@ -1,0 +1,378 @@
+#include "DeviceManager.h"
+
+#include "glow_mi355x.h"
+
+#include <future>
+
+namespace glow_mi355x {
+
+namespace {
+Error fromStatus(int rc, const char *what) {
+  if (rc == MI355X_OK) return Error::success();
+  ErrorCode c = ErrorCode::RUNTIME_ERROR;
+  if (rc == MI355X_ERR_OUT_OF_DEVICE_MEMORY) c = ErrorCode::RUNTIME_OUT_OF_DEVICE_MEMORY;
+  else if (rc == MI355X_ERR_NOT_SUPPORTED) c = ErrorCode::DEVICE_FEATURE_NOT_SUPPORTED;
+  else if (rc == MI355X_ERR_DEVICE_NOT_FOUND) c = ErrorCode::RUNTIME_DEVICE_NOT_FOUND;
+  return MI355X_MAKE_ERR(c, "%s: %s", what, mi355x_last_error());
+}
+} // namespace
+
+MI355XDeviceManager::~MI355XDeviceManager() { (void)stop(true); }
+
+void MI355XDeviceManager::enqueue(std::function<void()> work) {
+  {
+    std::lock_guard<std::mutex> lk(mu_);
+    queue_.push_back(std::move(work));
+  }
+  cv_.notify_one();
+}
+
+void MI355XDeviceManager::workerLoop() {
+  for (;;) {
+    std::function<void()> work;
+    {
+      std::unique_lock<std::mutex> lk(mu_);
+      cv_.wait(lk, [this] { return stopping_ || !queue_.empty(); });
+      if (queue_.empty()) return; // stopping and drained
+      work = std::move(queue_.front());
+      queue_.pop_front();
+    }
+    work();
+  }
+}
+
+Error MI355XDeviceManager::init() {
+  {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (running_) return Error::success();
+    running_ = true;
+    stopping_ = false;
+  }
+  worker_ = std::thread([this] { workerLoop(); });
+  // the device is bound to the worker thread, so bind it there
+  std::promise<Error> done;
+  auto fut = done.get_future();
+  enqueue([this, &done] {
+    int n = 0;
+    if (mi355x_num_devices(&n) != MI355X_OK || config_.deviceID < 0 || config_.deviceID >= n) {
+      done.set_value(MI355X_MAKE_ERR(ErrorCode::RUNTIME_DEVICE_NOT_FOUND,
+                                     "no MI355X device %d (%d visible)", config_.deviceID, n));
+      return;
+    }
+    int rc = mi355x_init(config_.deviceID);
+    if (rc != MI355X_OK) {
+      done.set_value(MI355X_MAKE_ERR(ErrorCode::RUNTIME_DEVICE_NOT_FOUND, "%s", mi355x_last_error()));
+      return;
+    }
+    mi355x_info info;
+    rc = mi355x_device_info(&info);
+    if (rc == MI355X_OK) rc = mi355x_stream_create(&stream_);
+    if (rc != MI355X_OK) {
+      done.set_value(fromStatus(rc, "device set-up"));
+      return;
+    }
+    info_.name = info.name;
+    info_.arch = info.arch;
+    info_.totalMemory = info.total_memory;
+    info_.computeUnits = info.compute_units;
+    maxMemoryBytes_ = config_.deviceMemory ? config_.deviceMemory : info.free_memory;
+    done.set_value(Error::success());
+  });
+  Error e = fut.get();
+  if (e) (void)stop(true);
+  return e;
+}
+
+Error MI355XDeviceManager::stop(bool block) {
+  (void)block;
+  {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (!running_) return Error::success();
+  }
+  std::promise<void> done;
+  auto fut = done.get_future();
+  enqueue([this, &done] {
+    for (auto &kv : functions_) release(kv.second);
+    functions_.clear();
+    for (auto &kv : modules_)
+      if (kv.second.arena) mi355x_arena_destroy(kv.second.arena);
+    modules_.clear();
+    usedMemoryBytes_ = 0;
+    if (stream_) {
+      mi355x_stream_sync(stream_);
+      mi355x_stream_destroy(stream_);
+      stream_ = nullptr;
+    }
+    done.set_value();
+  });
+  fut.get();
+  {
+    std::lock_guard<std::mutex> lk(mu_);
+    stopping_ = true;
+  }
+  cv_.notify_all();
+  if (worker_.joinable()) worker_.join();
+  {
+    std::lock_guard<std::mutex> lk(mu_);
+    running_ = false;
+  }
+  return Error::success();
+}
+
+void MI355XDeviceManager::addNetwork(const Module *module, FunctionMapTy functions,
+                                     ReadyCBTy readyCB) {
+  {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (!running_ || stopping_) {
+      readyCB(module, MI355X_MAKE_ERR(ErrorCode::RUNTIME_REQUEST_REFUSED,
+                                      "device manager is not running"));
+      return;
+    }
+  }
+  enqueue([this, module, functions, readyCB]() mutable {
+    addNetworkImpl(module, std::move(functions), std::move(readyCB));
+  });
+}
+
+void MI355XDeviceManager::evictNetwork(std::string functionName, EvictFunctionCBTy evictCB) {
+  {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (!running_ || stopping_) {
+      evictCB(functionName, MI355X_MAKE_ERR(ErrorCode::RUNTIME_REQUEST_REFUSED,
+                                            "device manager is not running"));
+      return;
+    }
+  }
+  enqueue([this, functionName, evictCB]() mutable {
+    evictNetworkImpl(std::move(functionName), std::move(evictCB));
+  });
+}
+
+RunIdentifierTy MI355XDeviceManager::runFunction(std::string functionName,
+                                                 std::unique_ptr<ExecutionContext> ctx,
+                                                 ResultCBTy resultCB) {
+  const RunIdentifierTy id = nextRun_++;
+  {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (!running_ || stopping_) {
+      resultCB(id, MI355X_MAKE_ERR(ErrorCode::RUNTIME_REQUEST_REFUSED,
+                                   "device manager is not running"),
+               std::move(ctx));
+      return id;
+    }
+  }
+  // std::function needs copyable captures: hand the context over by raw pointer
+  ExecutionContext *raw = ctx.release();
+  enqueue([this, id, functionName, raw, resultCB]() mutable {
+    runFunctionImpl(id, std::move(functionName), std::unique_ptr<ExecutionContext>(raw),
+                    std::move(resultCB));
+  });
+  return id;
+}
+
+void MI355XDeviceManager::release(FunctionResident &fr) {
+  if (fr.fn) fr.fn->dropGraph();
+  if (fr.arena) mi355x_arena_destroy(fr.arena);
+  fr.arena = nullptr;
+  usedMemoryBytes_ -= fr.bytes;
+  auto it = modules_.find(fr.module);
+  if (it != modules_.end() && --it->second.users == 0) {
+    if (it->second.arena) mi355x_arena_destroy(it->second.arena);
+    usedMemoryBytes_ -= it->second.bytes;
+    modules_.erase(it);
+  }
+}
+
+Error MI355XDeviceManager::makeResident(const Module *module, const std::string &name,
+                                        MI355XFunction *fn) {
+  const RuntimeBundle &rb = fn->getRuntimeBundle();
+  ModuleResident &mr = modules_[module];
+  if (!mr.arena && mr.users == 0) {
+    int rc = mi355x_arena_create(module->constantsSize(), module->mutableSize(), 0, &mr.arena);
+    if (rc != MI355X_OK) {
+      modules_.erase(module);
+      return fromStatus(rc, "module arena");
+    }
+    mr.bytes = mi355x_arena_bytes(mr.arena);
+    usedMemoryBytes_ += mr.bytes;
+    if (module->constantsSize()) {
+      rc = mi355x_arena_upload(mr.arena, MI355X_REGION_CONSTANTS, 0,
+                               module->constantsImage().data(), module->constantsSize(), stream_);
+      if (rc == MI355X_OK) rc = mi355x_stream_sync(stream_);
+      if (rc != MI355X_OK) {
+        mi355x_arena_destroy(mr.arena);
+        usedMemoryBytes_ -= mr.bytes;
+        modules_.erase(module);
+        return fromStatus(rc, "constants upload");
+      }
+    }
+  }
+  mr.users++;
+  FunctionResident fr;
+  fr.fn = fn;
+  fr.module = module;
+  auto failWith = [&](Error e) {
+    release(fr);
+    return e;
+  };
+  int rc = mi355x_arena_create(rb.generatedConstantsMemSize, 0, rb.activationsMemSize, &fr.arena);
+  if (rc != MI355X_OK) return failWith(fromStatus(rc, "function arena"));
+  fr.bytes = mi355x_arena_bytes(fr.arena);
+  usedMemoryBytes_ += fr.bytes;
+  void *p = nullptr;
+  mi355x_arena_ptr(mr.arena, MI355X_REGION_CONSTANTS, 0, &p);
+  fr.bindings.constants = (uint8_t *)p;
+  mi355x_arena_ptr(mr.arena, MI355X_REGION_MUTABLE, 0, &p);
+  fr.bindings.mutableMem = (uint8_t *)p;
+  mi355x_arena_ptr(fr.arena, MI355X_REGION_CONSTANTS, 0, &p);
+  fr.bindings.generated = (uint8_t *)p;
+  mi355x_arena_ptr(fr.arena, MI355X_REGION_ACTIVATIONS, 0, &p);
+  fr.bindings.activations = (uint8_t *)p;
+  fr.bindings.stream = stream_;
+  if (!fn->generated.empty()) {
+    rc = mi355x_arena_upload(fr.arena, MI355X_REGION_CONSTANTS, 0, fn->generated.data(),
+                             fn->generated.size(), stream_);
+    if (rc != MI355X_OK) return failWith(fromStatus(rc, "generated constants upload"));
+  }
+  for (const auto &l : fn->setup) {
+    rc = l.run(fr.bindings);
+    if (rc != MI355X_OK) return failWith(fromStatus(rc, l.kernel.c_str()));
+  }
+  rc = mi355x_stream_sync(stream_);
+  if (rc != MI355X_OK) return failWith(fromStatus(rc, "set-up launches"));
+  if (config_.useLaunchGraphs) {
+    // one eager pass first: entry points that allocate on first use must have
+    // run before they are recorded
+    for (const auto &l : fn->launches) {
+      rc = l.run(fr.bindings);
+      if (rc != MI355X_OK) return failWith(fromStatus(rc, l.kernel.c_str()));
+    }
+    rc = mi355x_stream_sync(stream_);
+    if (rc != MI355X_OK) return failWith(fromStatus(rc, "first pass"));
+    Error e = fn->captureGraph(fr.bindings);
+    if (e) return failWith(std::move(e));
+  }
+  functions_.emplace(name, fr);
+  return Error::success();
+}
+
+void MI355XDeviceManager::addNetworkImpl(const Module *module, FunctionMapTy functions,
+                                         ReadyCBTy readyCB) {
+  uint64_t need = 0;
+  for (const auto &f : functions) {
+    if (functions_.count(f.first)) {
+      readyCB(module, MI355X_MAKE_ERR(ErrorCode::RUNTIME_ERROR,
+                                      "Failed to add network: already have a function called %s",
+                                      f.first.c_str()));
+      return;
+    }
+    if (!f.second || f.second->getCompileBackendName() != "MI355X") {
+      readyCB(module, MI355X_MAKE_ERR(ErrorCode::RUNTIME_ERROR,
+                                      "Failed to add network: function %s is not an MI355XFunction",
+                                      f.first.c_str()));
+      return;
+    }
+    const RuntimeBundle &rb = f.second->getRuntimeBundle();
+    need += rb.generatedConstantsMemSize + rb.activationsMemSize;
+  }
+  if (!modules_.count(module)) need += module->constantsSize() + module->mutableSize();
+  if (usedMemoryBytes_ + need > maxMemoryBytes_) {
+    readyCB(module, MI355X_MAKE_ERR(ErrorCode::RUNTIME_OUT_OF_DEVICE_MEMORY,
+                                    "Failed to add network: not enough memory (%llu needed, "
+                                    "%llu available)",
+                                    (unsigned long long)need,
+                                    (unsigned long long)(maxMemoryBytes_ - usedMemoryBytes_)));
+    return;
+  }
+  std::vector<std::string> added;
+  for (const auto &f : functions) {
+    Error e = makeResident(module, f.first, f.second);
+    if (e) {
+      for (const auto &n : added) {
+        release(functions_[n]);
+        functions_.erase(n);
+      }
+      readyCB(module, std::move(e));
+      return;
+    }
+    added.push_back(f.first);
+  }
+  readyCB(module, Error::success());
+}
+
+void MI355XDeviceManager::evictNetworkImpl(std::string functionName, EvictFunctionCBTy evictCB) {
+  auto it = functions_.find(functionName);
+  if (it == functions_.end()) {
+    evictCB(functionName, MI355X_MAKE_ERR(ErrorCode::RUNTIME_NET_NOT_FOUND,
+                                          "Could not find function with name %s to evict",
+                                          functionName.c_str()));
+    return;
+  }
+  mi355x_stream_sync(stream_);
+  release(it->second);
+  functions_.erase(it);
+  evictCB(functionName, Error::success());
+}
+
+void MI355XDeviceManager::runFunctionImpl(RunIdentifierTy id, std::string functionName,
+                                          std::unique_ptr<ExecutionContext> ctx,
+                                          ResultCBTy resultCB) {
+  auto it = functions_.find(functionName);
+  if (it == functions_.end()) {
+    resultCB(id, MI355X_MAKE_ERR(ErrorCode::RUNTIME_NET_NOT_FOUND, "Function %s not found",
+                                 functionName.c_str()),
+             std::move(ctx));
+    return;
+  }
+  if (!ctx) {
+    resultCB(id, MI355X_MAKE_ERR(ErrorCode::RUNTIME_ERROR, "no execution context"), nullptr);
+    return;
+  }
+  FunctionResident &fr = it->second;
+  const RuntimeBundle &rb = fr.fn->getRuntimeBundle();
+  PlaceholderBindings *pb = ctx->getPlaceholderBindings();
+  Error err;
+  // inputs: host tensor -> placeholder slot (a tensor smaller than the slot
+  // fills its front, like the reference's partial tensors)
+  for (const auto &kv : pb->pairs()) {
+    auto st = rb.symbolTable.find(kv.first);
+    if (st == rb.symbolTable.end() || st->second.symbolCategory != SymbolCategory::Placeholder)
+      continue;
+    if (!st->second.input || !kv.second) continue;
+    if (kv.second->sizeInBytes() > st->second.size) {
+      err = MI355X_MAKE_ERR(ErrorCode::RUNTIME_ERROR, "tensor bound to %s has %zu bytes, slot %zu",
+                            kv.first.c_str(), kv.second->sizeInBytes(), st->second.size);
+      break;
+    }
+    int rc = mi355x_memcpy_h2d(fr.bindings.mutableMem + st->second.offset, kv.second->data(),
+                               kv.second->sizeInBytes(), stream_);
+    if (rc != MI355X_OK) {
+      err = fromStatus(rc, "input copy");
+      break;
+    }
+  }
+  if (!err) {
+    ctx->setDeviceBindings(std::unique_ptr<DeviceBindings>(new DeviceBindings(fr.bindings)));
+    err = fr.fn->execute(ctx.get());
+  }
+  if (!err) {
+    for (const auto &kv : pb->pairs()) {
+      auto st = rb.symbolTable.find(kv.first);
+      if (st == rb.symbolTable.end() || st->second.symbolCategory != SymbolCategory::Placeholder)
+        continue;
+      if (!st->second.output || !kv.second) continue;
+      const size_t n = std::min(kv.second->sizeInBytes(), st->second.size);
+      int rc = mi355x_memcpy_d2h(kv.second->data(), fr.bindings.mutableMem + st->second.offset, n,
+                                 stream_);
+      if (rc != MI355X_OK) {
+        err = fromStatus(rc, "output copy");
+        break;
+      }
+    }
+  }
+  const int rc = mi355x_stream_sync(stream_);
+  if (!err && rc != MI355X_OK) err = fromStatus(rc, "run");
+  resultCB(id, std::move(err), std::move(ctx));
+}
+
+} // namespace glow_mi355x

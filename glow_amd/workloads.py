@@ -86,7 +86,8 @@ def rwq_fc_case(seed, M, K, N, in_scale=0.05, out_scale=0.1, out_offset=0,
                 bias_pre=bpre, bias_post=bpost, bias_scale=bscale,
                 out_pre=opre, out_post=opost, out_scale=oscale,
                 out_offset=int(out_offset), in_offset=int(in_offset),
-                bias_offset=int(bias_offset))
+                bias_offset=int(bias_offset), in_scale_f=float(in_scale),
+                out_scale_f=float(out_scale), bias_scale_f=float(bias_scale))
 
 
 def rwq_fc_args(c):
@@ -112,7 +113,9 @@ def fc_case(seed, M, K, N, bias_i8=False, host=None):
                 in_offset=int(rng.integers(-10, 11)),
                 w_offset=int(rng.integers(-5, 6)),
                 bias_offset=int(rng.integers(-3, 4)) if bias_i8 else 0,
-                biasP=biasP, outP=outP)
+                biasP=biasP, outP=outP, in_scale_f=float(in_scale),
+                w_scale_f=float(w_scale), out_scale_f=float(out_scale),
+                bias_scale_f=float(b_scale))
 
 
 def fc_args(c):
@@ -151,17 +154,21 @@ def cwq_conv_case(seed, N, H, W, IC, OC, kernel=(3, 3), stride=(1, 1),
     bpre, bpost, bscale = s32to8_vec(b_scales / mm, host)
     opre, opost, oscale = s32to8_vec(mm / np.float32(out_scale), host)
     g = host.conv_geom(N, H, W, IC, OC, kernel, stride, pads, group, dilation)
-    act_args = ()
+    act_args, act_fargs = (), ()
     if act == ACT_CLIP:
-        act_args = (host.quantize_value_i32(0.0, out_scale, out_offset),
-                    host.quantize_value_i32(6.0 * out_scale * 20, out_scale, out_offset))
+        act_fargs = (0.0, float(np.float32(6.0 * out_scale * 20)))
+        act_args = (host.quantize_value_i32(act_fargs[0], out_scale, out_offset),
+                    host.quantize_value_i32(act_fargs[1], out_scale, out_offset))
     elif act == ACT_LEAKY_RELU:
+        act_fargs = (0.1,)
         act_args = host.s32to8(0.1, 0)[:3]
     return dict(x=x, filt=filt, bias=bias, geom=g, out_offset=int(out_offset),
                 in_offset=int(in_offset), f_offsets=f_offsets,
                 b_offsets=b_offsets, bias_pre=bpre, bias_post=bpost,
                 bias_scale=bscale, out_pre=opre, out_post=opost,
-                out_scale=oscale, act=act, act_args=act_args)
+                out_scale=oscale, act=act, act_args=act_args,
+                act_fargs=act_fargs, f_scales=f_scales, b_scales=np.asarray(b_scales, np.float32),
+                in_scale_f=float(in_scale), out_scale_f=float(out_scale))
 
 
 def cwq_conv_args(c):

@@ -77,6 +77,10 @@ int mi355x_memcpy_d2h(void *dst, const void *src, size_t bytes, void *stream);
 int mi355x_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream);
 /* Fills with a kernel (safe inside a captured graph). */
 int mi355x_fill_u8(void *dst, int value, size_t bytes, void *stream);
+/* Device-to-device copy done by a kernel: a graph node with a known HBM
+ * footprint (bytes read + bytes written), which is also what the hardware
+ * byte counters are calibrated against. */
+int mi355x_copy_u8(void *dst, const void *src, size_t bytes, void *stream);
 
 int mi355x_stream_create(void **stream);
 int mi355x_stream_destroy(void *stream);

@@ -1,0 +1,123 @@
+/*
+ * glow_mi355x_host.h - flat C view of the MI355X backend's host layer
+ * (glow_amd/host: MI355XBackend, MI355XFunction, MI355XDeviceManager), for
+ * harnesses and tests that are not C++. The C++ classes mirror glow::Backend,
+ * glow::CompiledFunction and glow::runtime::DeviceManager (reference
+ * include/glow/Backend/Backend.h:67-325, include/glow/Backend/CompiledFunction.h:29-98,
+ * include/glow/Backends/DeviceManager.h:47-241); this header only wraps them:
+ * build a module of constants, placeholders and lowered instructions, compile
+ * it, make it resident on the device, run it.
+ *
+ * Every int-returning function gives a non-negative result on success and
+ * -(error code) on failure, where the error code is one of
+ * MI355X_HOST_ERR_* (the names follow glow::ErrorValue::ErrorCode, reference
+ * include/glow/Support/Error.h:292-337); mi355x_host_last_error() holds the
+ * message for the calling thread.
+ */
+#ifndef GLOW_MI355X_HOST_H
+#define GLOW_MI355X_HOST_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  MI355X_HOST_SUCCESS = 0,
+  MI355X_HOST_ERR_UNKNOWN = 1,
+  MI355X_HOST_ERR_RUNTIME_ERROR = 2,
+  MI355X_HOST_ERR_RUNTIME_OUT_OF_DEVICE_MEMORY = 3,
+  MI355X_HOST_ERR_RUNTIME_NET_NOT_FOUND = 4,
+  MI355X_HOST_ERR_RUNTIME_REQUEST_REFUSED = 5,
+  MI355X_HOST_ERR_RUNTIME_DEVICE_NOT_FOUND = 6,
+  MI355X_HOST_ERR_RUNTIME_DEVICE_NONRECOVERABLE = 7,
+  MI355X_HOST_ERR_RUNTIME_NET_BUSY = 8,
+  MI355X_HOST_ERR_DEVICE_FEATURE_NOT_SUPPORTED = 9,
+  MI355X_HOST_ERR_COMPILE_UNSUPPORTED_NODE_AFTER_OPTIMIZE = 10,
+  MI355X_HOST_ERR_COMPILE_CONTEXT_MALFORMED = 11
+};
+const char *mi355x_host_last_error(void);
+const char *mi355x_host_error_name(int code);
+
+/* glow::ElemKind subset (reference include/glow/Base/Type.h:401-433) */
+enum {
+  MI355X_HOST_FLOAT = 0, MI355X_HOST_FLOAT16 = 1, MI355X_HOST_INT8Q = 2,
+  MI355X_HOST_INT32Q = 3, MI355X_HOST_INT32I = 4, MI355X_HOST_INT64I = 5,
+  MI355X_HOST_UINT8_FUSED = 6, MI355X_HOST_UINT8_FUSED_FP16 = 7,
+  MI355X_HOST_UINT4_FUSED_FP16 = 8, MI355X_HOST_UINT4_FUSED = 9,
+  MI355X_HOST_BOOL = 10
+};
+
+/* Instruction kinds: Glow's IR instruction names (operand order of
+ * tools/ClassGen/InstrGen.cpp, destination first). */
+enum {
+  MI355X_HOST_QUANTIZE = 0,            /* Dest, Src */
+  MI355X_HOST_DEQUANTIZE = 1,          /* Dest, Src */
+  MI355X_HOST_RESCALE_QUANTIZED = 2,   /* Dest, Src */
+  MI355X_HOST_FULLY_CONNECTED = 3,     /* Dest, Src, Weights[K,N], Bias */
+  MI355X_HOST_ROWWISE_QUANTIZED_FC = 4,/* Dest, Src, Weights[N,K], Bias, Scales, Offsets */
+  MI355X_HOST_MATMUL = 5,              /* Dest, LHS, RHS */
+  MI355X_HOST_CONVOLUTION = 6,         /* Dest, Src, Filter, Bias; 12 iattrs */
+  MI355X_HOST_CHANNELWISE_QUANTIZED_CONV = 7, /* + FilterScales, FilterOffsets, BiasScales, BiasOffsets */
+  MI355X_HOST_FRWQ_SLWS = 8,           /* Dest, Data, Weights, Indices, Lengths; iattrs {useFP16Accumulation} */
+  MI355X_HOST_FRWQ_SLS = 9             /* Dest, Data, Indices, Lengths; iattrs {useFP16Accumulation} */
+};
+/* Convolution iattrs: kernelH, kernelW, strideH, strideW, padT, padL, padB,
+ * padR, group, dilationH, dilationW, fusedActivation (glow::FusedActivation);
+ * fattrs: the float activation arguments (Clip {min,max}, LeakyRelu {alpha}). */
+
+typedef struct mi355x_host_module mi355x_host_module;
+typedef struct mi355x_host_dm mi355x_host_dm;
+
+mi355x_host_module *mi355x_host_module_create(const char *name);
+void mi355x_host_module_destroy(mi355x_host_module *m);
+/* Module::createConstant / createPlaceholder; return the value id. */
+int mi355x_host_add_constant(mi355x_host_module *m, const char *name, int elem_kind,
+                             const int64_t *dims, int ndims, float scale, int32_t offset,
+                             const void *payload);
+int mi355x_host_add_placeholder(mi355x_host_module *m, const char *name, int elem_kind,
+                                const int64_t *dims, int ndims, float scale, int32_t offset);
+/* Module::createFunction; returns the function index. */
+int mi355x_host_create_function(mi355x_host_module *m, const char *name);
+/* AllocActivationInst of one function; returns the value id. */
+int mi355x_host_add_activation(mi355x_host_module *m, int function, const char *name,
+                               int elem_kind, const int64_t *dims, int ndims, float scale,
+                               int32_t offset);
+int mi355x_host_add_instruction(mi355x_host_module *m, int function, int kind, const char *name,
+                                const int *operands, int n_operands, const int64_t *iattrs,
+                                int n_iattrs, const float *fattrs, int n_fattrs);
+/* Backend::isOpSupported for one would-be instruction: 1, or 0 with the
+ * reason in mi355x_host_last_error(). */
+int mi355x_host_is_op_supported(mi355x_host_module *m, int kind, const int *operands,
+                                int n_operands, const int64_t *iattrs, int n_iattrs,
+                                const float *fattrs, int n_fattrs);
+/* Backend::compile of one function; the compiled function stays with the module. */
+int mi355x_host_compile(mi355x_host_module *m, int function, int precompute_weight_row_sums);
+/* Listing of the compiled function's launches and derived parameters; returns
+ * the length needed (text is truncated to cap-1 bytes). */
+int mi355x_host_describe(mi355x_host_module *m, int function, char *buf, size_t cap);
+/* RuntimeBundle sizes: out = {constants, generated, mutable, activations}. */
+int mi355x_host_bundle_sizes(mi355x_host_module *m, int function, uint64_t out[4]);
+
+/* DeviceManager. memory_bytes 0 = what the device reports free. */
+mi355x_host_dm *mi355x_host_dm_create(int device, uint64_t memory_bytes, int use_launch_graphs);
+void mi355x_host_dm_destroy(mi355x_host_dm *dm);
+int mi355x_host_dm_init(mi355x_host_dm *dm);
+int mi355x_host_dm_stop(mi355x_host_dm *dm);
+/* addNetwork with every compiled function of the module; waits for the callback. */
+int mi355x_host_dm_add_network(mi355x_host_dm *dm, mi355x_host_module *m);
+int mi355x_host_dm_evict_network(mi355x_host_dm *dm, const char *function_name);
+/* runFunction; binds n host buffers to placeholders by name (inputs are read,
+ * outputs written, `bytes[i]` may be smaller than the placeholder), waits for
+ * the result callback. */
+int mi355x_host_dm_run(mi355x_host_dm *dm, const char *function_name, const char *const *names,
+                       void *const *buffers, const size_t *bytes, int n);
+uint64_t mi355x_host_dm_maximum_memory(mi355x_host_dm *dm);
+uint64_t mi355x_host_dm_available_memory(mi355x_host_dm *dm);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GLOW_MI355X_HOST_H */

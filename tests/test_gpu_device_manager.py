@@ -1,0 +1,235 @@
+"""MI355XDeviceManager on the GPU, in the shape of the reference's
+DeviceManagerTest (tests/unittests/DeviceManagerTest.cpp:132-673): add a
+network, run it, run it again, several functions and modules, eviction, memory
+accounting and the error codes; every result is compared with the oracle."""
+import numpy as np
+import pytest
+
+from glow_amd import host as H
+from tests import cases, host_cases
+from oracle import glow_oracle as go
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture
+def dm():
+    d = H.DeviceManager().init()
+    yield d
+    d.stop()
+
+
+def _rwq_expected(c, x=None):
+    args = list(cases.rwq_fc_args(c))
+    if x is not None:
+        args[0] = x
+    return go.rwq_fc_i8(*args)
+
+
+def test_basic(dm):
+    c = cases.rwq_fc_case(11, 32, 256, 192)
+    m, f = host_cases.rwq_fc_module(c)
+    m.compile(f)
+    dm.add_network(m)
+    out = np.zeros((32, 192), np.int8)
+    dm.run("main", {"input": c["x"], "output": out})
+    assert np.array_equal(out, _rwq_expected(c))
+
+
+@pytest.mark.parametrize("graphs", [True, False])
+def test_multi_run(graphs):
+    d = H.DeviceManager(use_launch_graphs=graphs).init()
+    try:
+        c = cases.rwq_fc_case(12, 16, 128, 64, symmetric=False)
+        m, f = host_cases.rwq_fc_module(c)
+        m.compile(f)
+        d.add_network(m)
+        rng = np.random.default_rng(0)
+        for _ in range(4):
+            x = rng.integers(-128, 128, c["x"].shape).astype(np.int8)
+            out = np.zeros((16, 64), np.int8)
+            d.run("main", {"input": x, "output": out})
+            assert np.array_equal(out, _rwq_expected(c, x))
+    finally:
+        d.stop()
+
+
+def test_pipeline_quantize_fc_dequantize(dm):
+    """Quantize -> RWQ-FC -> Rescale -> Dequantize through activations."""
+    c = cases.rwq_fc_case(13, 8, 64, 48)
+    M, K, N = 8, 64, 48
+    m = H.Module("pipe")
+    xin = m.placeholder("input", (M, K), H.FLOAT, np.float32)
+    yout = m.placeholder("output", (M, N), H.FLOAT, np.float32)
+    w = m.constant("weights", c["w"], H.INT8Q)
+    b = m.constant("bias", c["bias"], H.INT32Q, c["bias_scale_f"], c["bias_offset"])
+    sc = m.constant("scales", c["w_scales"])
+    of = m.constant("offsets", c["w_offsets"], H.INT32I)
+    f = m.function("main")
+    q = m.activation(f, "q", (M, K), H.INT8Q, c["in_scale_f"], c["in_offset"])
+    y = m.activation(f, "y", (M, N), H.INT8Q, c["out_scale_f"], c["out_offset"])
+    z = m.activation(f, "z", (M, N), H.INT8Q, 0.23, 5)
+    m.instruction(f, H.QUANTIZE, "quant", [q, xin])
+    m.instruction(f, H.ROWWISE_QUANTIZED_FC, "fc", [y, q, w, b, sc, of])
+    m.instruction(f, H.RESCALE_QUANTIZED, "rescale", [z, y])
+    m.instruction(f, H.DEQUANTIZE, "dequant", [yout, z])
+    m.compile(f)
+    dm.add_network(m)
+    rng = np.random.default_rng(1)
+    x = rng.normal(0, 2.0, (M, K)).astype(np.float32)
+    out = np.zeros((M, N), np.float32)
+    dm.run("main", {"input": x, "output": out})
+    xq = go.quantize_i8(x, c["in_scale_f"], c["in_offset"])
+    yq = _rwq_expected(c, xq)
+    pre, post, scale, _ = go.quantize_scale_offset_32to8(
+        float(np.float32(c["out_scale_f"]) / np.float32(0.23)), 0)
+    zq = go.rescale_i8(yq, 5, c["out_offset"], pre, post, scale)
+    want = go.dequantize_i8(zq, 0.23, 5)
+    assert np.array_equal(out, want)
+
+
+def test_multi_function_and_eviction(dm):
+    c1 = cases.rwq_fc_case(14, 8, 64, 32)
+    c2 = cases.cwq_conv_case(15, 2, 10, 10, 16, 32, in_offset=-3)
+    m1, f1 = host_cases.rwq_fc_module(c1, name="fc_net")
+    m2, f2 = host_cases.cwq_conv_module(c2, name="conv_net")
+    m1.compile(f1)
+    m2.compile(f2)
+    before = dm.available_memory
+    dm.add_network(m1)
+    dm.add_network(m2)
+    assert dm.available_memory < before
+    o1 = np.zeros((8, 32), np.int8)
+    g = c2["geom"]
+    o2 = np.zeros((g.N, g.OH, g.OW, g.OC), np.int8)
+    dm.run("fc_net", {"input": c1["x"], "output": o1})
+    dm.run("conv_net", {"input": c2["x"], "output": o2})
+    assert np.array_equal(o1, _rwq_expected(c1))
+    assert np.array_equal(o2, go.cwq_conv2d_i8(*cases.cwq_conv_args(c2)))
+    dm.evict_network("fc_net")
+    with pytest.raises(H.HostError) as e:
+        dm.run("fc_net", {"input": c1["x"], "output": o1})
+    assert e.value.code_name == "RUNTIME_NET_NOT_FOUND"
+    with pytest.raises(H.HostError) as e:
+        dm.evict_network("fc_net")
+    assert e.value.code_name == "RUNTIME_NET_NOT_FOUND"
+    # the other network is untouched, and the name can be used again
+    o2[:] = 0
+    dm.run("conv_net", {"input": c2["x"], "output": o2})
+    assert np.array_equal(o2, go.cwq_conv2d_i8(*cases.cwq_conv_args(c2)))
+    dm.add_network(m1)
+    o1[:] = 0
+    dm.run("fc_net", {"input": c1["x"], "output": o1})
+    assert np.array_equal(o1, _rwq_expected(c1))
+    dm.evict_network("fc_net")
+    dm.evict_network("conv_net")
+    assert dm.available_memory == before
+
+
+def test_two_functions_of_one_module_share_its_constants(dm):
+    c = cases.rwq_fc_case(16, 8, 64, 32)
+    m, f = host_cases.rwq_fc_module(c, name="a")
+    # second function of the same module: rescale of the same input
+    g = m.function("b")
+    vals = {n: i for i, n in enumerate(["input", "output", "weights", "bias", "scales", "offsets"])}
+    r = m.placeholder("rescaled", (8, 64), H.INT8Q, np.int8, 0.11, -1)
+    m.instruction(g, H.RESCALE_QUANTIZED, "r", [r, vals["input"]])
+    m.compile(f)
+    m.compile(g)
+    dm.add_network(m)
+    out = np.zeros((8, 32), np.int8)
+    dm.run("a", {"input": c["x"], "output": out})
+    assert np.array_equal(out, _rwq_expected(c))
+    res = np.zeros((8, 64), np.int8)
+    dm.run("b", {"input": c["x"], "rescaled": res})
+    pre, post, scale, _ = go.quantize_scale_offset_32to8(
+        float(np.float32(c["in_scale_f"]) / np.float32(0.11)), 0)
+    assert np.array_equal(res, go.rescale_i8(c["x"], -1, c["in_offset"], pre, post, scale))
+
+
+def test_duplicate_name_and_out_of_memory():
+    c = cases.rwq_fc_case(17, 8, 64, 32)
+    m, f = host_cases.rwq_fc_module(c)
+    m.compile(f)
+    small = H.DeviceManager(memory_bytes=1024).init()
+    try:
+        assert small.maximum_memory == 1024
+        with pytest.raises(H.HostError) as e:
+            small.add_network(m)
+        assert e.value.code_name == "RUNTIME_OUT_OF_DEVICE_MEMORY"
+        assert small.available_memory == 1024
+    finally:
+        small.stop()
+    d = H.DeviceManager().init()
+    try:
+        d.add_network(m)
+        with pytest.raises(H.HostError) as e:
+            d.add_network(m)
+        assert "already have a function called main" in str(e.value)
+    finally:
+        d.stop()
+
+
+def test_partial_input_tensor(dm):
+    """A bound tensor smaller than its placeholder fills the front of it
+    (DeviceManagerTest PartialTensorCopy)."""
+    m = H.Module()
+    a = m.placeholder("a", (4, 16), H.INT8Q, np.int8, 0.5, 0)
+    b = m.placeholder("b", (4, 16), H.FLOAT, np.float32)
+    f = m.function("main")
+    m.instruction(f, H.DEQUANTIZE, "d", [b, a])
+    m.compile(f)
+    dm.add_network(m)
+    full = np.arange(64, dtype=np.int8).reshape(4, 16)
+    out = np.zeros((4, 16), np.float32)
+    dm.run("main", {"a": full, "b": out})
+    assert np.array_equal(out, full.astype(np.float32) * 0.5)
+    half = (np.arange(32, dtype=np.int8) - 7).reshape(2, 16)
+    out2 = np.zeros((2, 16), np.float32)
+    dm.run("main", {"a": half, "b": out2})
+    assert np.array_equal(out2, half.astype(np.float32) * 0.5)
+    too_big = np.zeros((5, 16), np.int8)
+    with pytest.raises(H.HostError):
+        dm.run("main", {"a": too_big, "b": out})
+
+
+def test_slws_network(dm):
+    rng = np.random.default_rng(18)
+    rows, cols, bags = 5000, 128, 300
+    table = cases.random_fused_table(rng, rows, cols)
+    lengths, idx, w = cases.slws_batch(19, rows, bags, 12, 1.05, np.int64)
+    n = idx.size + 50      # statically sized index/weight tensors, only sum(lengths) used
+    m = H.Module("slws")
+    data = m.constant("data", table, H.UINT8_FUSED)
+    wv = m.placeholder("weights", (n,), H.FLOAT, np.float32)
+    iv = m.placeholder("indices", (n,), H.INT64I, np.int64)
+    lv = m.placeholder("lengths", (bags,), H.INT32I, np.int32)
+    out = m.placeholder("output", (bags, cols), H.FLOAT, np.float32)
+    f = m.function("main")
+    m.instruction(f, H.FRWQ_SLWS, "slws", [out, data, wv, iv, lv], [0])
+    m.compile(f)
+    dm.add_network(m)
+    res = np.zeros((bags, cols), np.float32)
+    dm.run("main", {"weights": w, "indices": idx, "lengths": lengths, "output": res})
+    assert np.array_equal(res, go.frwq_slws_f32(table, w, idx, lengths))
+
+
+def test_fc_and_conv_networks(dm):
+    c = cases.fc_case(20, 24, 96, 80)
+    m, f = host_cases.fc_module(c)
+    m.compile(f)
+    dm.add_network(m)
+    out = np.zeros((24, 80), np.int8)
+    dm.run("main", {"input": c["x"], "output": out})
+    assert np.array_equal(out, go.fc_i8(*cases.fc_args(c)))
+    dm.evict_network("main")
+    for act in (cases._w.ACT_CLIP, cases._w.ACT_LEAKY_RELU):
+        cc = cases.cwq_conv_case(21, 2, 12, 12, 32, 32, act=act, in_offset=4, symmetric=False)
+        mc, fc = host_cases.cwq_conv_module(cc)
+        mc.compile(fc)
+        dm.add_network(mc)
+        g = cc["geom"]
+        o = np.zeros((g.N, g.OH, g.OW, g.OC), np.int8)
+        dm.run("main", {"input": cc["x"], "output": o})
+        assert np.array_equal(o, go.cwq_conv2d_i8(*cases.cwq_conv_args(cc)))
+        dm.evict_network("main")

@@ -1,0 +1,190 @@
+"""CPU tests of the backend's host layer: the flat C view exports what its
+header declares; MI355XBackend::compile derives the same integer kernel
+parameters from float scales as the oracle's restatement of the reference code
+generator (LLVMIRGen.cpp:2161-2320, 2695-2798); unsupported instructions and a
+missing device come back as the reference's error codes."""
+import os
+import re
+
+import numpy as np
+import pytest
+
+from glow_amd import host as H
+from tests import cases, host_cases
+from oracle import glow_oracle as go
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_exports_match_header():
+    text = open(os.path.join(ROOT, "include", "glow_mi355x_host.h")).read()
+    declared = sorted(set(re.findall(r"\b(mi355x_host_[a-z0-9_]+)\s*\(", text)))
+    assert declared == sorted(H.EXPORTS)
+    L = H.lib()
+    for name in declared:
+        assert hasattr(L, name), name
+
+
+def test_host_library_does_not_link_the_oracle():
+    import subprocess
+    out = subprocess.run(["ldd", os.path.join(ROOT, "glow_amd", "libglow_mi355x_host.so")],
+                         capture_output=True, text=True).stdout
+    assert "oracle" not in out and "libjit" not in out
+    assert "libglow_mi355x.so" in out
+
+
+def _launch(m, f, kernel):
+    rows = [r for r in H.parse_listing(m.describe(f)) if r["kernel"] == kernel and r["phase"] == "launch"]
+    assert len(rows) == 1
+    return rows[0]
+
+
+@pytest.mark.parametrize("seed,symmetric,bias_i8", [(1, True, False), (2, False, False), (3, True, True)])
+def test_rwqfc_parameters(seed, symmetric, bias_i8):
+    c = cases.rwq_fc_case(seed, 8, 64, 48, symmetric=symmetric, bias_i8=bias_i8,
+                          bias_scale=0.01 if bias_i8 else 5e-5,
+                          bias_offset=-2 if bias_i8 else 0)
+    m, f = host_cases.rwq_fc_module(c, bias_i8=bias_i8)
+    m.compile(f)
+    r = _launch(m, f, "mi355x_rwq_fc_i8")
+    for k in ("bias_pre", "bias_post", "bias_scale", "out_pre", "out_post", "out_scale"):
+        assert r[k] == c[k].tolist(), k
+    assert (r["M"], r["K"], r["N"]) == (8, 64, 48)
+    assert r["out_offset"] == c["out_offset"] and r["in_offset"] == c["in_offset"]
+    assert r["bias_offset"] == c["bias_offset"] and r["bias_is_i8"] == int(bias_i8)
+    assert r["weights_offsets_all_zero"] == int(symmetric)
+    # row sums are only worth forming when the input offset is non-zero
+    setup = [x for x in H.parse_listing(m.describe(f)) if x["phase"] == "setup"]
+    assert (len(setup) == 1) == (c["in_offset"] != 0)
+
+
+def test_fc_parameters():
+    c = cases.fc_case(4, 8, 32, 24)
+    m, f = host_cases.fc_module(c)
+    m.compile(f)
+    r = _launch(m, f, "mi355x_fc_i8")
+    assert (r["bias_pre"], r["bias_post"], r["bias_scale"]) == tuple(c["biasP"])
+    assert (r["out_pre"], r["out_post"], r["out_scale"]) == tuple(c["outP"])
+    assert r["weights_offset"] == c["w_offset"] and r["repack"] == 0
+    kernels = [x["kernel"] for x in H.parse_listing(m.describe(f)) if x["phase"] == "setup"]
+    assert kernels[0] == "mi355x_transpose2d_i8"     # [K x N] -> [N x K] once, at load
+
+
+@pytest.mark.parametrize("act", [cases._w.ACT_NONE, cases._w.ACT_RELU, cases._w.ACT_CLIP,
+                                 cases._w.ACT_LEAKY_RELU])
+def test_cwq_conv_parameters(act):
+    c = cases.cwq_conv_case(5, 2, 9, 9, 16, 32, act=act, in_offset=-7, symmetric=False)
+    m, f = host_cases.cwq_conv_module(c)
+    m.compile(f)
+    r = _launch(m, f, "mi355x_cwq_conv2d_i8")
+    for k in ("bias_pre", "bias_post", "bias_scale", "out_pre", "out_post", "out_scale"):
+        assert r[k] == c[k].tolist(), k
+    want = list(c["act_args"]) + [0] * (3 - len(c["act_args"]))
+    assert r["act_args"] == want and r["act"] == act
+    g = c["geom"]
+    assert (r["OH"], r["OW"], r["OC"], r["KH"], r["KW"]) == (g.OH, g.OW, g.OC, g.KH, g.KW)
+    assert r["filter_offsets_all_zero"] == 0
+
+
+def test_rescale_parameters():
+    m = H.Module()
+    a = m.placeholder("a", (5, 7), H.INT8Q, np.int8, 0.37, -4)
+    b = m.placeholder("b", (5, 7), H.INT8Q, np.int8, 0.05, 9)
+    f = m.function("main")
+    m.instruction(f, H.RESCALE_QUANTIZED, "r", [b, a])
+    m.compile(f)
+    r = _launch(m, f, "mi355x_rescale_i8")
+    pre, post, scale, _ = go.quantize_scale_offset_32to8(float(np.float32(0.37) / np.float32(0.05)), 0)
+    assert (r["pre"], r["post"], r["scale"]) == (pre, post, scale)
+    assert (r["in_offset"], r["out_offset"], r["n"]) == (-4, 9, 35)
+
+
+def test_memory_plan_is_aligned_and_disjoint():
+    c = cases.rwq_fc_case(1, 8, 64, 48)
+    m, f = host_cases.rwq_fc_module(c)
+    m.compile(f)
+    s = m.bundle_sizes(f)
+    # weights 48*64, bias 48*4, scales 48*4, offsets 48*4, each rounded to 64
+    assert s["constants"] == 3072 + 192 * 3
+    assert s["mutable"] == 8 * 64 + 8 * 48 + (64 - (8 * 48) % 64) % 64
+    assert s["generated"] >= 6 * 192 and s["generated"] % 64 == 0
+    assert s["activations"] == 0
+
+
+def _slws_module(data_kind, dest_kind, w_kind):
+    m = H.Module()
+    row = {H.UINT8_FUSED: 16 + 8, H.UINT8_FUSED_FP16: 16 + 4,
+           H.UINT4_FUSED_FP16: 8 + 4, H.UINT4_FUSED: 8 + 8}[data_kind]
+    data = m.placeholder("data", (10, row), data_kind, np.uint8)
+    dest = m.placeholder("dest", (3, 16), dest_kind, np.float32)
+    w = m.placeholder("w", (12,), w_kind, np.float32)
+    idx = m.placeholder("idx", (12,), H.INT64I, np.int64)
+    ln = m.placeholder("len", (3,), H.INT32I, np.int32)
+    return m, [dest, data, w, idx, ln]
+
+
+def test_slws_type_legality_follows_the_reference():
+    # fp32-scale data: (float weights, float result) or (f16, f16) only;
+    # fp16-scale data: float16 result, float or float16 weights.
+    ok = [(H.UINT8_FUSED, H.FLOAT, H.FLOAT), (H.UINT8_FUSED, H.FLOAT16, H.FLOAT16),
+          (H.UINT4_FUSED_FP16, H.FLOAT16, H.FLOAT), (H.UINT4_FUSED_FP16, H.FLOAT16, H.FLOAT16),
+          (H.UINT8_FUSED_FP16, H.FLOAT16, H.FLOAT16), (H.UINT4_FUSED, H.FLOAT, H.FLOAT)]
+    bad = [(H.UINT8_FUSED, H.FLOAT, H.FLOAT16), (H.UINT8_FUSED, H.FLOAT16, H.FLOAT),
+           (H.UINT4_FUSED_FP16, H.FLOAT, H.FLOAT), (H.UINT8_FUSED_FP16, H.FLOAT, H.FLOAT16)]
+    for d, r, w in ok:
+        m, ops = _slws_module(d, r, w)
+        assert m.is_op_supported(H.FRWQ_SLWS, ops, [0])[0], (d, r, w)
+    for d, r, w in bad:
+        m, ops = _slws_module(d, r, w)
+        assert not m.is_op_supported(H.FRWQ_SLWS, ops, [0])[0], (d, r, w)
+
+
+def test_unsupported_instructions_are_compile_errors():
+    m = H.Module()
+    a = m.placeholder("a", (4, 4), H.FLOAT, np.float32)
+    b = m.placeholder("b", (4, 4), H.FLOAT, np.float32)
+    f = m.function("main")
+    m.instruction(f, H.QUANTIZE, "q", [b, a])          # float -> float
+    with pytest.raises(H.HostError) as e:
+        m.compile(f)
+    assert e.value.code_name == "COMPILE_UNSUPPORTED_NODE_AFTER_OPTIMIZE"
+    f2 = m.function("other")
+    m.instruction(f2, 77, "mystery", [b, a])
+    with pytest.raises(H.HostError) as e:
+        m.compile(f2)
+    assert e.value.code_name == "COMPILE_UNSUPPORTED_NODE_AFTER_OPTIMIZE"
+    # fused Sigmoid/Tanh are rejected for quantized convolutions like on the CPU backend
+    c = cases.cwq_conv_case(5, 1, 5, 5, 16, 16, act=cases._w.ACT_RELU)
+    c["act"] = cases._w.ACT_SIGMOID
+    m2, f3 = host_cases.cwq_conv_module(c)
+    with pytest.raises(H.HostError):
+        m2.compile(f3)
+
+
+def test_shape_mismatch_is_reported_with_the_instruction_name():
+    c = cases.rwq_fc_case(1, 8, 64, 48)
+    c["bias"] = c["bias"][:-1]
+    m, f = host_cases.rwq_fc_module(c)
+    with pytest.raises(H.HostError) as e:
+        m.compile(f)
+    assert "rwqfc" in str(e.value) and "shape mismatch" in str(e.value)
+
+
+def test_device_manager_without_a_device():
+    from glow_amd import capi
+    if capi.num_devices() > 0:
+        pytest.skip("a GPU is present")
+    dm = H.DeviceManager()
+    with pytest.raises(H.HostError) as e:
+        dm.init()
+    assert e.value.code_name == "RUNTIME_DEVICE_NOT_FOUND"
+    # requests to a manager that is not running are refused, not queued
+    c = cases.rwq_fc_case(1, 8, 64, 48)
+    m, f = host_cases.rwq_fc_module(c)
+    m.compile(f)
+    with pytest.raises(H.HostError) as e:
+        dm.add_network(m)
+    assert e.value.code_name == "RUNTIME_REQUEST_REFUSED"
+    with pytest.raises(H.HostError) as e:
+        dm.run("main", {})
+    assert e.value.code_name == "RUNTIME_REQUEST_REFUSED"
