@@ -22,7 +22,8 @@ EXPORTS = [
     "mi355x_last_error", "mi355x_num_devices", "mi355x_init",
     "mi355x_device_info", "mi355x_malloc", "mi355x_free", "mi355x_host_alloc",
     "mi355x_host_free", "mi355x_memcpy_h2d", "mi355x_memcpy_d2h",
-    "mi355x_memcpy_d2d", "mi355x_fill_u8", "mi355x_copy_u8", "mi355x_stream_create",
+    "mi355x_memcpy_d2d", "mi355x_fill_u8", "mi355x_copy_u8", "mi355x_add_i8", "mi355x_add_relu_i8",
+    "mi355x_relu_i8", "mi355x_max_pool_i8", "mi355x_avg_pool_i8", "mi355x_softmax_f32", "mi355x_stream_create",
     "mi355x_stream_destroy", "mi355x_stream_sync", "mi355x_device_sync",
     "mi355x_event_create", "mi355x_event_destroy", "mi355x_event_record",
     "mi355x_event_sync", "mi355x_event_elapsed_ms", "mi355x_arena_create",
@@ -663,3 +664,90 @@ def embedding_bag_rowwise_offsets(data, kind, weights, indices, offsets,
         _vp(d_off), _sz(offsets.size), C.c_int(bool(has_end_offset)),
         _sz(in_line), _sz(out_line), C.c_int(bool(fp16_accum)), _vp(None)))
     return d_out.numpy()
+
+
+# ---- int8 glue operators ------------------------------------------------------
+
+def _i32s(vals):
+    return [_i32(int(v)) for v in vals]
+
+
+def launch_add_i8(dst, lhs, rhs, n, dest_offset, lhs_offset, rhs_offset, lhsP, rhsP,
+                  stream=None):
+    check(lib().mi355x_add_i8(_vp(dst), _vp(lhs), _vp(rhs), _sz(n), _i32(dest_offset),
+                              _i32(lhs_offset), _i32(rhs_offset), *_i32s(lhsP),
+                              *_i32s(rhsP), _vp(stream)))
+
+
+def launch_add_relu_i8(dst, lhs, rhs, n, sum_offset, lhs_offset, rhs_offset, lhsP, rhsP,
+                       dest_offset, destP, stream=None):
+    check(lib().mi355x_add_relu_i8(_vp(dst), _vp(lhs), _vp(rhs), _sz(n), _i32(sum_offset),
+                                   _i32(lhs_offset), _i32(rhs_offset), *_i32s(lhsP),
+                                   *_i32s(rhsP), _i32(dest_offset), *_i32s(destP),
+                                   _vp(stream)))
+
+
+def add_i8(lhs, rhs, dest_offset, lhs_offset, rhs_offset, lhsP, rhsP):
+    lhs = np.ascontiguousarray(lhs, np.int8)
+    rhs = np.ascontiguousarray(rhs, np.int8)
+    dl, dr = to_device(lhs), to_device(rhs)
+    out = DeviceBuffer.empty(lhs.shape, np.int8)
+    launch_add_i8(out, dl, dr, lhs.size, dest_offset, lhs_offset, rhs_offset, lhsP, rhsP)
+    return out.numpy()
+
+
+def add_relu_i8(lhs, rhs, sum_offset, lhs_offset, rhs_offset, lhsP, rhsP, dest_offset, destP):
+    lhs = np.ascontiguousarray(lhs, np.int8)
+    rhs = np.ascontiguousarray(rhs, np.int8)
+    dl, dr = to_device(lhs), to_device(rhs)
+    out = DeviceBuffer.empty(lhs.shape, np.int8)
+    launch_add_relu_i8(out, dl, dr, lhs.size, sum_offset, lhs_offset, rhs_offset, lhsP, rhsP,
+                       dest_offset, destP)
+    return out.numpy()
+
+
+def relu_i8(src, src_offset, dest_offset, destP):
+    src = np.ascontiguousarray(src, np.int8)
+    ds = to_device(src)
+    out = DeviceBuffer.empty(src.shape, np.int8)
+    check(lib().mi355x_relu_i8(_vp(out), _vp(ds), _sz(src.size), _i32(src_offset),
+                               _i32(dest_offset), *_i32s(destP), _vp(None)))
+    return out.numpy()
+
+
+def _pool_sizes(x, kernel, stride, pads):
+    N, IH, IW, Cn = x.shape
+    OH = (IH + pads[0] + pads[2] - kernel[0]) // stride[0] + 1
+    OW = (IW + pads[1] + pads[3] - kernel[1]) // stride[1] + 1
+    sz = [_sz(int(v)) for v in (N, IH, IW, Cn, OH, OW, kernel[0], kernel[1], stride[0],
+                                stride[1], pads[0], pads[1])]
+    return (N, OH, OW, Cn), sz
+
+
+def max_pool_i8(x, kernel, stride, pads, out_offset):
+    """pads = (top, left, bottom, right)."""
+    x = np.ascontiguousarray(x, np.int8)
+    shape, sz = _pool_sizes(x, kernel, stride, pads)
+    dx = to_device(x)
+    out = DeviceBuffer.empty(shape, np.int8)
+    check(lib().mi355x_max_pool_i8(_vp(out), _vp(dx), *sz, _i32(out_offset), _vp(None)))
+    return out.numpy()
+
+
+def avg_pool_i8(x, kernel, stride, pads, count_include_pads, out_offset, in_offset, outP):
+    x = np.ascontiguousarray(x, np.int8)
+    shape, sz = _pool_sizes(x, kernel, stride, pads)
+    dx = to_device(x)
+    out = DeviceBuffer.empty(shape, np.int8)
+    check(lib().mi355x_avg_pool_i8(_vp(out), _vp(dx), *sz, C.c_int(int(count_include_pads)),
+                                   _i32(out_offset), _i32(in_offset), *_i32s(outP), _vp(None)))
+    return out.numpy()
+
+
+def softmax_f32(x):
+    x = np.ascontiguousarray(x, np.float32)
+    dx = to_device(x)
+    out = DeviceBuffer.empty(x.shape, np.float32)
+    check(lib().mi355x_softmax_f32(_vp(out), _vp(dx), _sz(x.shape[0]), _sz(x.shape[1]),
+                                   _vp(None)))
+    return out.numpy()

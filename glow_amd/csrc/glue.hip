@@ -1,0 +1,393 @@
+// The int8 glue operators between the matrix-core kernels of a quantized
+// network: ElementAdd (optionally followed by Relu in the same pass), Relu,
+// MaxPool, AvgPool on NHWC int8 tensors, and the fp32 SoftMax at the end
+// (reference lib/LLVMIRCodeGen/libjit/libjit.cpp:1593-1603, 1851-1858,
+// 812-884, 2592-2597, 2812-2880, 3058-3082). All are HBM-bound: 16-byte
+// accesses along the channel dimension, integer arithmetic bit-identical to
+// the CPU code.
+#include "common.h"
+
+#pragma clang fp contract(off)
+#include "requant.h"
+
+namespace mi355x {
+
+constexpr int kGlueThreads = 256;
+
+__device__ __forceinline__ uint32_t pack4b(int32_t a, int32_t b, int32_t c, int32_t d) {
+  return (uint32_t)(a & 0xff) | ((uint32_t)(b & 0xff) << 8) |
+         ((uint32_t)(c & 0xff) << 16) | ((uint32_t)(d & 0xff) << 24);
+}
+__device__ __forceinline__ int32_t sx8(uint32_t w, int i) {
+  return (int32_t)(int8_t)(w >> (8 * i));
+}
+
+struct AddParams {
+  int32_t dest_off, lhs_off, rhs_off;
+  int32_t lhs_pre, lhs_post, lhs_scale, rhs_pre, rhs_post, rhs_scale;
+  // optional Relu stage applied to the (already clipped) sum
+  int32_t relu_dest_off, relu_pre, relu_post, relu_scale;
+};
+
+template <bool RELU>
+__device__ __forceinline__ int32_t add_one(int32_t l, int32_t r, const AddParams &p) {
+  const int32_t a = scale_i32(l - p.lhs_off, p.lhs_pre, p.lhs_post, p.lhs_scale, 0);
+  const int32_t b = scale_i32(r - p.rhs_off, p.rhs_pre, p.rhs_post, p.rhs_scale, 0);
+  int32_t v = clip_i8((int32_t)((uint32_t)a + (uint32_t)b + (uint32_t)p.dest_off));
+  if (RELU) {
+    // libjit_element_relu_i8 with srcOffset = the sum's offset
+    const int32_t so = (int32_t)(int8_t)p.dest_off;
+    v = max(v, so);
+    v = clip_i8(scale_i32(v - so, p.relu_pre, p.relu_post, p.relu_scale, p.relu_dest_off));
+  }
+  return v;
+}
+
+template <bool RELU>
+__global__ __launch_bounds__(kGlueThreads) void add_i8_kernel(
+    int8_t *__restrict__ dst, const int8_t *__restrict__ lhs,
+    const int8_t *__restrict__ rhs, size_t n, size_t vec_chunks, AddParams p) {
+  const size_t t = (size_t)blockIdx.x * kGlueThreads + threadIdx.x;
+  if (t < vec_chunks) {
+    const uint4 a = reinterpret_cast<const uint4 *>(lhs)[t];
+    const uint4 b = reinterpret_cast<const uint4 *>(rhs)[t];
+    const uint32_t wa[4] = {a.x, a.y, a.z, a.w}, wb[4] = {b.x, b.y, b.z, b.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      o[j] = pack4b(add_one<RELU>(sx8(wa[j], 0), sx8(wb[j], 0), p),
+                    add_one<RELU>(sx8(wa[j], 1), sx8(wb[j], 1), p),
+                    add_one<RELU>(sx8(wa[j], 2), sx8(wb[j], 2), p),
+                    add_one<RELU>(sx8(wa[j], 3), sx8(wb[j], 3), p));
+    reinterpret_cast<uint4 *>(dst)[t] = make_uint4(o[0], o[1], o[2], o[3]);
+  }
+  const size_t stride = (size_t)gridDim.x * kGlueThreads;
+  for (size_t i = vec_chunks * 16 + t; i < n; i += stride)
+    dst[i] = (int8_t)add_one<RELU>(lhs[i], rhs[i], p);
+}
+
+__device__ __forceinline__ int32_t relu_one(int32_t v, int32_t so, int32_t doff,
+                                            int32_t pre, int32_t post, int32_t scale) {
+  v = max(v, so);
+  return clip_i8(scale_i32(v - so, pre, post, scale, doff));
+}
+
+__global__ __launch_bounds__(kGlueThreads) void relu_i8_kernel(
+    int8_t *__restrict__ dst, const int8_t *__restrict__ src, size_t n,
+    size_t vec_chunks, int32_t so, int32_t doff, int32_t pre, int32_t post,
+    int32_t scale) {
+  const size_t t = (size_t)blockIdx.x * kGlueThreads + threadIdx.x;
+  if (t < vec_chunks) {
+    const uint4 a = reinterpret_cast<const uint4 *>(src)[t];
+    const uint32_t wa[4] = {a.x, a.y, a.z, a.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      o[j] = pack4b(relu_one(sx8(wa[j], 0), so, doff, pre, post, scale),
+                    relu_one(sx8(wa[j], 1), so, doff, pre, post, scale),
+                    relu_one(sx8(wa[j], 2), so, doff, pre, post, scale),
+                    relu_one(sx8(wa[j], 3), so, doff, pre, post, scale));
+    reinterpret_cast<uint4 *>(dst)[t] = make_uint4(o[0], o[1], o[2], o[3]);
+  }
+  const size_t stride = (size_t)gridDim.x * kGlueThreads;
+  for (size_t i = vec_chunks * 16 + t; i < n; i += stride)
+    dst[i] = (int8_t)relu_one(src[i], so, doff, pre, post, scale);
+}
+
+struct PoolGeom {
+  int N, IH, IW, C, OH, OW, KH, KW, SH, SW, padT, padL;
+};
+
+// window of valid taps of one output position (libjit_defs.h:257-275)
+__device__ __forceinline__ void pool_window(int in_min, int in_size, int k, int &lo, int &len) {
+  lo = max(0, -in_min);
+  const int hi = min(k, in_size - in_min);
+  len = max(0, hi - lo);
+}
+
+// One thread per output pixel and group of VEC channels (VEC bytes per load).
+template <int VEC>
+__global__ __launch_bounds__(kGlueThreads) void max_pool_i8_kernel(
+    int8_t *__restrict__ out, const int8_t *__restrict__ in, PoolGeom g,
+    int32_t out_offset, long long total) {
+  const long long t = (long long)blockIdx.x * kGlueThreads + threadIdx.x;
+  if (t >= total) return;
+  const int cg = g.C / VEC;
+  const int c0 = (int)(t % cg) * VEC;
+  long long pix = t / cg;
+  const int ow = (int)(pix % g.OW);
+  pix /= g.OW;
+  const int oh = (int)(pix % g.OH);
+  const int n = (int)(pix / g.OH);
+  int h0, hl, w0, wl;
+  const int ih_min = oh * g.SH - g.padT, iw_min = ow * g.SW - g.padL;
+  pool_window(ih_min, g.IH, g.KH, h0, hl);
+  pool_window(iw_min, g.IW, g.KW, w0, wl);
+  int32_t m[VEC];
+#pragma unroll
+  for (int i = 0; i < VEC; i++) m[i] = -128;
+  for (int fh = 0; fh < hl; fh++)
+    for (int fw = 0; fw < wl; fw++) {
+      const int8_t *p = in + (((long long)n * g.IH + (ih_min + h0 + fh)) * g.IW +
+                              (iw_min + w0 + fw)) * g.C + c0;
+      if constexpr (VEC == 16) {
+        const uint4 v = *reinterpret_cast<const uint4 *>(p);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 16; i++) m[i] = max(m[i], sx8(w[i >> 2], i & 3));
+      } else {
+        m[0] = max(m[0], (int32_t)p[0]);
+      }
+    }
+  const bool empty = hl == 0 || wl == 0;
+  int8_t *q = out + (((long long)n * g.OH + oh) * g.OW + ow) * g.C + c0;
+  if constexpr (VEC == 16) {
+    uint32_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      o[j] = empty ? pack4b(out_offset, out_offset, out_offset, out_offset)
+                   : pack4b(m[4 * j], m[4 * j + 1], m[4 * j + 2], m[4 * j + 3]);
+    *reinterpret_cast<uint4 *>(q) = make_uint4(o[0], o[1], o[2], o[3]);
+  } else {
+    q[0] = (int8_t)(empty ? out_offset : m[0]);
+  }
+}
+
+// libjit_div_round_i32 (libjit_defs.h:239-244)
+__device__ __forceinline__ int32_t div_round_i32(int32_t v, int32_t d) {
+  const int32_t rnd = d >> 1;
+  return v > 0 ? (v + rnd) / d : (v - rnd) / d;
+}
+
+template <int VEC>
+__global__ __launch_bounds__(kGlueThreads) void avg_pool_i8_kernel(
+    int8_t *__restrict__ out, const int8_t *__restrict__ in, PoolGeom g,
+    int count_include_pads, int32_t out_offset, int32_t in_offset, int32_t pre,
+    int32_t post, int32_t scale, long long total) {
+  const long long t = (long long)blockIdx.x * kGlueThreads + threadIdx.x;
+  if (t >= total) return;
+  const int cg = g.C / VEC;
+  const int c0 = (int)(t % cg) * VEC;
+  long long pix = t / cg;
+  const int ow = (int)(pix % g.OW);
+  pix /= g.OW;
+  const int oh = (int)(pix % g.OH);
+  const int n = (int)(pix / g.OH);
+  int h0, hl, w0, wl;
+  const int ih_min = oh * g.SH - g.padT, iw_min = ow * g.SW - g.padL;
+  pool_window(ih_min, g.IH, g.KH, h0, hl);
+  pool_window(iw_min, g.IW, g.KW, w0, wl);
+  int32_t s[VEC];
+#pragma unroll
+  for (int i = 0; i < VEC; i++) s[i] = 0;
+  for (int fh = 0; fh < hl; fh++)
+    for (int fw = 0; fw < wl; fw++) {
+      const int8_t *p = in + (((long long)n * g.IH + (ih_min + h0 + fh)) * g.IW +
+                              (iw_min + w0 + fw)) * g.C + c0;
+      if constexpr (VEC == 4) {
+        const uint32_t w = *reinterpret_cast<const uint32_t *>(p);
+#pragma unroll
+        for (int i = 0; i < 4; i++) s[i] += sx8(w, i) - in_offset;
+      } else {
+        s[0] += (int32_t)p[0] - in_offset;
+      }
+    }
+  const int32_t area = hl * wl;
+  int32_t r[VEC];
+#pragma unroll
+  for (int i = 0; i < VEC; i++) {
+    if (count_include_pads) {
+      r[i] = clip_i8(scale_i32(s[i], pre, post, scale, out_offset));
+    } else if (area == 0) {
+      r[i] = (int32_t)(int8_t)out_offset;
+    } else {
+      const int32_t v = scale_i32(s[i], pre, post, scale, 0);
+      r[i] = clip_i8((int32_t)((uint32_t)div_round_i32(v, area) + (uint32_t)out_offset));
+    }
+  }
+  int8_t *q = out + (((long long)n * g.OH + oh) * g.OW + ow) * g.C + c0;
+  if constexpr (VEC == 4)
+    *reinterpret_cast<uint32_t *>(q) = pack4b(r[0], r[1], r[2], r[3]);
+  else
+    q[0] = (int8_t)r[0];
+}
+
+__device__ __forceinline__ float block_reduce(float v, float *s, bool is_max) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float o = __shfl_xor(v, off, 64);
+    v = is_max ? fmaxf(v, o) : __fadd_rn(v, o);
+  }
+  __syncthreads();
+  if (lane == 0) s[wave] = v;
+  __syncthreads();
+  float r = s[0];
+  for (int w = 1; w < kGlueThreads / 64; w++) r = is_max ? fmaxf(r, s[w]) : __fadd_rn(r, s[w]);
+  return r;
+}
+
+// One block per row: max, exp and sum, divide (libjit_softmax_f). The sum is
+// formed in a different order than the CPU's sequential loop, so results agree
+// to fp32 rounding, not bit for bit.
+__global__ __launch_bounds__(kGlueThreads) void softmax_f32_kernel(
+    float *__restrict__ out, const float *__restrict__ in, int cols) {
+  __shared__ float s[kGlueThreads / 64];
+  const float *x = in + (long long)blockIdx.x * cols;
+  float *y = out + (long long)blockIdx.x * cols;
+  float m = -INFINITY;
+  for (int i = threadIdx.x; i < cols; i += kGlueThreads) m = fmaxf(m, x[i]);
+  m = block_reduce(m, s, true);
+  float sum = 0.0f;
+  for (int i = threadIdx.x; i < cols; i += kGlueThreads) {
+    const float e = expf(__fsub_rn(x[i], m));
+    y[i] = e;
+    sum = __fadd_rn(sum, e);
+  }
+  sum = block_reduce(sum, s, false);
+  for (int i = threadIdx.x; i < cols; i += kGlueThreads) y[i] = __fdiv_rn(y[i], sum);
+}
+
+static bool al16(const void *a, const void *b, const void *c) {
+  return (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c) & 15) == 0;
+}
+static unsigned glue_blocks(size_t work) {
+  size_t b = (work + kGlueThreads - 1) / kGlueThreads;
+  return (unsigned)(b ? b : 1);
+}
+static bool shifts_ok(int32_t a, int32_t b) { return a >= 0 && a <= 31 && b >= 0 && b <= 31; }
+
+static int pool_geom(PoolGeom &g, size_t N, size_t IH, size_t IW, size_t C, size_t OH,
+                     size_t OW, size_t kH, size_t kW, size_t sH, size_t sW, size_t padT,
+                     size_t padL) {
+  MI355X_REQUIRE(IH > 0 && IW > 0 && C > 0 && kH > 0 && kW > 0 && sH > 0 && sW > 0,
+                 "invalid pooling geometry");
+  const size_t lim = 1u << 30;
+  MI355X_REQUIRE(N < lim && IH < lim && IW < lim && C < lim && OH < lim && OW < lim &&
+                     kH < lim && kW < lim && sH < lim && sW < lim && padT < lim && padL < lim,
+                 "pooling dimensions too large");
+  // every window must start at or before the last input row / column
+  MI355X_REQUIRE(OH == 0 || (OH - 1) * sH < IH + padT, "output height inconsistent with input");
+  MI355X_REQUIRE(OW == 0 || (OW - 1) * sW < IW + padL, "output width inconsistent with input");
+  g = PoolGeom{(int)N, (int)IH, (int)IW, (int)C, (int)OH, (int)OW, (int)kH, (int)kW,
+               (int)sH, (int)sW, (int)padT, (int)padL};
+  return MI355X_OK;
+}
+
+} // namespace mi355x
+
+using namespace mi355x;
+
+extern "C" {
+
+int mi355x_add_i8(int8_t *dst, const int8_t *lhs, const int8_t *rhs, size_t n,
+                  int32_t dest_offset, int32_t lhs_offset, int32_t rhs_offset,
+                  int32_t lhs_pre, int32_t lhs_post, int32_t lhs_scale, int32_t rhs_pre,
+                  int32_t rhs_post, int32_t rhs_scale, void *stream) {
+  if (n == 0) return MI355X_OK;
+  MI355X_REQUIRE(dst && lhs && rhs, "NULL tensor");
+  MI355X_REQUIRE(shifts_ok(lhs_pre, lhs_post) && shifts_ok(rhs_pre, rhs_post),
+                 "pre/post shift outside [0, 31]");
+  MI355X_REQUIRE(n / 16 / kGlueThreads < 0x7fffffffu, "tensor too large");
+  AddParams p{dest_offset, lhs_offset, rhs_offset, lhs_pre, lhs_post, lhs_scale,
+              rhs_pre, rhs_post, rhs_scale, 0, 0, 0, 0};
+  const size_t chunks = al16(dst, lhs, rhs) ? n / 16 : 0;
+  hipLaunchKernelGGL(add_i8_kernel<false>, dim3(glue_blocks(chunks)), dim3(kGlueThreads), 0,
+                     as_stream(stream), dst, lhs, rhs, n, chunks, p);
+  return check_launch("add_i8");
+}
+
+int mi355x_add_relu_i8(int8_t *dst, const int8_t *lhs, const int8_t *rhs, size_t n,
+                       int32_t sum_offset, int32_t lhs_offset, int32_t rhs_offset,
+                       int32_t lhs_pre, int32_t lhs_post, int32_t lhs_scale, int32_t rhs_pre,
+                       int32_t rhs_post, int32_t rhs_scale, int32_t dest_offset,
+                       int32_t dest_pre, int32_t dest_post, int32_t dest_scale, void *stream) {
+  if (n == 0) return MI355X_OK;
+  MI355X_REQUIRE(dst && lhs && rhs, "NULL tensor");
+  MI355X_REQUIRE(shifts_ok(lhs_pre, lhs_post) && shifts_ok(rhs_pre, rhs_post) &&
+                     shifts_ok(dest_pre, dest_post),
+                 "pre/post shift outside [0, 31]");
+  MI355X_REQUIRE(sum_offset >= -128 && sum_offset <= 127 && dest_offset >= -128 &&
+                     dest_offset <= 127,
+                 "offsets outside the int8 range");
+  MI355X_REQUIRE(n / 16 / kGlueThreads < 0x7fffffffu, "tensor too large");
+  AddParams p{sum_offset, lhs_offset, rhs_offset, lhs_pre, lhs_post, lhs_scale,
+              rhs_pre, rhs_post, rhs_scale, dest_offset, dest_pre, dest_post, dest_scale};
+  const size_t chunks = al16(dst, lhs, rhs) ? n / 16 : 0;
+  hipLaunchKernelGGL(add_i8_kernel<true>, dim3(glue_blocks(chunks)), dim3(kGlueThreads), 0,
+                     as_stream(stream), dst, lhs, rhs, n, chunks, p);
+  return check_launch("add_relu_i8");
+}
+
+int mi355x_relu_i8(int8_t *dst, const int8_t *src, size_t n, int32_t src_offset,
+                   int32_t dest_offset, int32_t dest_pre, int32_t dest_post,
+                   int32_t dest_scale, void *stream) {
+  if (n == 0) return MI355X_OK;
+  MI355X_REQUIRE(dst && src, "NULL tensor");
+  MI355X_REQUIRE(shifts_ok(dest_pre, dest_post), "pre/post shift outside [0, 31]");
+  MI355X_REQUIRE(src_offset >= -128 && src_offset <= 127 && dest_offset >= -128 &&
+                     dest_offset <= 127,
+                 "offsets outside the int8 range");
+  MI355X_REQUIRE(n / 16 / kGlueThreads < 0x7fffffffu, "tensor too large");
+  const size_t chunks = al16(dst, src, src) ? n / 16 : 0;
+  hipLaunchKernelGGL(relu_i8_kernel, dim3(glue_blocks(chunks)), dim3(kGlueThreads), 0,
+                     as_stream(stream), dst, src, n, chunks, src_offset, dest_offset, dest_pre,
+                     dest_post, dest_scale);
+  return check_launch("relu_i8");
+}
+
+int mi355x_max_pool_i8(int8_t *out, const int8_t *in, size_t N, size_t IH, size_t IW, size_t C,
+                       size_t OH, size_t OW, size_t kH, size_t kW, size_t sH, size_t sW,
+                       size_t padT, size_t padL, int32_t out_offset, void *stream) {
+  if (N == 0 || OH == 0 || OW == 0) return MI355X_OK;
+  MI355X_REQUIRE(out && in, "NULL tensor");
+  PoolGeom g;
+  int rc = pool_geom(g, N, IH, IW, C, OH, OW, kH, kW, sH, sW, padT, padL);
+  if (rc != MI355X_OK) return rc;
+  const bool vec = (C % 16 == 0) && al16(out, in, in);
+  const long long total = (long long)N * OH * OW * (vec ? C / 16 : C);
+  MI355X_REQUIRE(total / kGlueThreads < 0x7fffffffLL, "tensor too large");
+  if (vec)
+    hipLaunchKernelGGL(max_pool_i8_kernel<16>, dim3(glue_blocks((size_t)total)),
+                       dim3(kGlueThreads), 0, as_stream(stream), out, in, g, out_offset, total);
+  else
+    hipLaunchKernelGGL(max_pool_i8_kernel<1>, dim3(glue_blocks((size_t)total)),
+                       dim3(kGlueThreads), 0, as_stream(stream), out, in, g, out_offset, total);
+  return check_launch("max_pool_i8");
+}
+
+int mi355x_avg_pool_i8(int8_t *out, const int8_t *in, size_t N, size_t IH, size_t IW, size_t C,
+                       size_t OH, size_t OW, size_t kH, size_t kW, size_t sH, size_t sW,
+                       size_t padT, size_t padL, int count_include_pads, int32_t out_offset,
+                       int32_t in_offset, int32_t out_pre, int32_t out_post, int32_t out_scale,
+                       void *stream) {
+  if (N == 0 || OH == 0 || OW == 0) return MI355X_OK;
+  MI355X_REQUIRE(out && in, "NULL tensor");
+  MI355X_REQUIRE(shifts_ok(out_pre, out_post), "pre/post shift outside [0, 31]");
+  PoolGeom g;
+  int rc = pool_geom(g, N, IH, IW, C, OH, OW, kH, kW, sH, sW, padT, padL);
+  if (rc != MI355X_OK) return rc;
+  const bool vec = (C % 4 == 0) && ((((uintptr_t)out | (uintptr_t)in) & 3) == 0);
+  const long long total = (long long)N * OH * OW * (vec ? C / 4 : C);
+  MI355X_REQUIRE(total / kGlueThreads < 0x7fffffffLL, "tensor too large");
+  if (vec)
+    hipLaunchKernelGGL(avg_pool_i8_kernel<4>, dim3(glue_blocks((size_t)total)),
+                       dim3(kGlueThreads), 0, as_stream(stream), out, in, g, count_include_pads,
+                       out_offset, in_offset, out_pre, out_post, out_scale, total);
+  else
+    hipLaunchKernelGGL(avg_pool_i8_kernel<1>, dim3(glue_blocks((size_t)total)),
+                       dim3(kGlueThreads), 0, as_stream(stream), out, in, g, count_include_pads,
+                       out_offset, in_offset, out_pre, out_post, out_scale, total);
+  return check_launch("avg_pool_i8");
+}
+
+int mi355x_softmax_f32(float *out, const float *in, size_t rows, size_t cols, void *stream) {
+  if (rows == 0 || cols == 0) return MI355X_OK;
+  MI355X_REQUIRE(out && in, "NULL tensor");
+  MI355X_REQUIRE(rows < 0x7fffffffu && cols < 0x7fffffffu, "tensor too large");
+  hipLaunchKernelGGL(softmax_f32_kernel, dim3((unsigned)rows), dim3(kGlueThreads), 0,
+                     as_stream(stream), out, in, (int)cols);
+  return check_launch("softmax_f32");
+}
+
+} // extern "C"

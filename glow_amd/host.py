@@ -13,7 +13,8 @@ _LIB = None
 (FLOAT, FLOAT16, INT8Q, INT32Q, INT32I, INT64I, UINT8_FUSED, UINT8_FUSED_FP16,
  UINT4_FUSED_FP16, UINT4_FUSED, BOOL) = range(11)
 (QUANTIZE, DEQUANTIZE, RESCALE_QUANTIZED, FULLY_CONNECTED, ROWWISE_QUANTIZED_FC,
- MATMUL, CONVOLUTION, CHANNELWISE_QUANTIZED_CONV, FRWQ_SLWS, FRWQ_SLS) = range(10)
+ MATMUL, CONVOLUTION, CHANNELWISE_QUANTIZED_CONV, FRWQ_SLWS, FRWQ_SLS, ELEMENT_ADD,
+ RELU, MAX_POOL, AVG_POOL, SOFTMAX) = range(15)
 ACT_NONE, ACT_RELU, ACT_CLIP, ACT_TANH, ACT_SIGMOID, ACT_LEAKY_RELU = range(6)
 
 ERROR_NAMES = ["SUCCESS", "UNKNOWN", "RUNTIME_ERROR", "RUNTIME_OUT_OF_DEVICE_MEMORY",
@@ -30,7 +31,7 @@ EXPORTS = [
     "mi355x_host_describe", "mi355x_host_bundle_sizes", "mi355x_host_dm_create",
     "mi355x_host_dm_destroy", "mi355x_host_dm_init", "mi355x_host_dm_stop",
     "mi355x_host_dm_add_network", "mi355x_host_dm_evict_network", "mi355x_host_dm_run",
-    "mi355x_host_dm_maximum_memory", "mi355x_host_dm_available_memory",
+    "mi355x_host_dm_time_function", "mi355x_host_dm_maximum_memory", "mi355x_host_dm_available_memory",
 ]
 
 
@@ -135,8 +136,9 @@ class Module:
             self._h, kind, *self._inst_args(operands, iattrs, fattrs)))
         return bool(rc), (lib().mi355x_host_last_error().decode() if not rc else "")
 
-    def compile(self, fn, precompute_weight_row_sums=True):
-        _check(lib().mi355x_host_compile(self._h, fn, int(precompute_weight_row_sums)))
+    def compile(self, fn, precompute_weight_row_sums=True, fuse_add_relu=True):
+        opts = (1 if precompute_weight_row_sums else 0) | (2 if fuse_add_relu else 0)
+        _check(lib().mi355x_host_compile(self._h, fn, opts))
 
     def describe(self, fn):
         n = _check(lib().mi355x_host_describe(self._h, fn, None, C.c_size_t(0)))
@@ -220,6 +222,13 @@ class DeviceManager:
         cb = (C.c_void_p * len(names))(*[a.ctypes.data for a in arrs])
         cs = (C.c_size_t * len(names))(*[a.nbytes for a in arrs])
         _check(lib().mi355x_host_dm_run(self._h, name.encode(), cn, cb, cs, len(names)))
+
+    def time_function(self, name, iterations):
+        """Average device milliseconds per replay, no host copies."""
+        ms = C.c_float(0)
+        _check(lib().mi355x_host_dm_time_function(self._h, name.encode(), int(iterations),
+                                                  C.byref(ms)))
+        return ms.value
 
     @property
     def maximum_memory(self):

@@ -91,9 +91,26 @@ public:
       : M_(M), insts_(insts), function_(function), opts_(o) {}
 
   Error run(MI355XFunction &out) {
-    for (const auto &I : insts_) {
-      MI355X_RETURN_IF_ERR(checkOperands(I));
+    for (const auto &I : insts_) MI355X_RETURN_IF_ERR(checkOperands(I));
+    for (size_t at = 0; at < insts_.size(); at++) {
+      const Instruction &I = insts_[at];
       switch (I.kind) {
+      case Kind::ElementAdd: {
+        // an add whose only reader is the Relu right behind it becomes one pass
+        const Instruction *relu = nullptr;
+        if (opts_.fuseAddRelu && at + 1 < insts_.size() && insts_[at + 1].kind == Kind::Relu &&
+            insts_[at + 1].operands[1] == I.operands[0] &&
+            M_.value(I.operands[0]).category == SymbolCategory::Activation &&
+            readers(I.operands[0]) == 1)
+          relu = &insts_[at + 1];
+        MI355X_RETURN_IF_ERR(add(I, relu, out));
+        if (relu) at++;
+        break;
+      }
+      case Kind::Relu: MI355X_RETURN_IF_ERR(relu(I, out)); break;
+      case Kind::MaxPool: MI355X_RETURN_IF_ERR(pool(I, out, false)); break;
+      case Kind::AvgPool: MI355X_RETURN_IF_ERR(pool(I, out, true)); break;
+      case Kind::SoftMax: MI355X_RETURN_IF_ERR(softmax(I, out)); break;
       case Kind::Quantize: MI355X_RETURN_IF_ERR(quantize(I, out)); break;
       case Kind::Dequantize: MI355X_RETURN_IF_ERR(dequantize(I, out)); break;
       case Kind::RescaleQuantized: MI355X_RETURN_IF_ERR(rescale(I, out)); break;
@@ -123,7 +140,7 @@ public:
   const std::map<int, std::pair<bool, bool>> &io() const { return io_; }
 
 private:
-  static constexpr int kArity[(int)Kind::NumKinds] = {2, 2, 2, 4, 6, 3, 4, 8, 5, 4};
+  static constexpr int kArity[(int)Kind::NumKinds] = {2, 2, 2, 4, 6, 3, 4, 8, 5, 4, 3, 2, 2, 2, 2};
 
   Error checkOperands(const Instruction &I) {
     CHECK_OP((int)I.kind >= 0 && (int)I.kind < (int)Kind::NumKinds, "unknown kind");
@@ -145,6 +162,139 @@ private:
   }
 
   Operand op(const Instruction &I, int i) const { return Operand{&M_.value(I.operands[(size_t)i])}; }
+
+  int readers(int id) const {
+    int n = 0;
+    for (const auto &I : insts_)
+      for (size_t i = 1; i < I.operands.size(); i++) n += I.operands[i] == id;
+    return n;
+  }
+
+  Error add(const Instruction &I, const Instruction *reluI, MI355XFunction &out) {
+    Operand d = op(I, 0), l = op(I, 1), r = op(I, 2);
+    CHECK_OP(d.ty().kind == ElemKind::Int8QTy && l.ty().kind == ElemKind::Int8QTy &&
+                 r.ty().kind == ElemKind::Int8QTy,
+             "needs i8 operands");
+    CHECK_OP(d.ty().size() == l.ty().size() && d.ty().size() == r.ty().size(), "size mismatch");
+    const size_t n = (size_t)d.ty().size();
+    const S32To8 lp = s32to8(l.ty().scale / d.ty().scale), rp = s32to8(r.ty().scale / d.ty().scale);
+    const int32_t doff = d.ty().offset, lo = l.ty().offset, ro = r.ty().offset;
+    std::string params = strFormat(" n=%zu", n) + kv("dest_offset", doff) + kv("lhs_offset", lo) +
+                         kv("rhs_offset", ro) + kv("lhs_pre", lp.pre) + kv("lhs_post", lp.post) +
+                         kv("lhs_scale", lp.scale) + kv("rhs_pre", rp.pre) + kv("rhs_post", rp.post) +
+                         kv("rhs_scale", rp.scale);
+    if (!reluI) {
+      out.launches.push_back({"mi355x_add_i8", I.name, params, [=](const DeviceBindings &b) {
+                                return mi355x_add_i8((int8_t *)d.ptr(b), (const int8_t *)l.ptr(b),
+                                                     (const int8_t *)r.ptr(b), n, doff, lo, ro, lp.pre,
+                                                     lp.post, lp.scale, rp.pre, rp.post, rp.scale,
+                                                     b.stream);
+                              }});
+      return Error::success();
+    }
+    const Instruction &R = *reluI;
+    Operand rd = op(R, 0);
+    {
+      const Instruction &I = R; // for the message
+      CHECK_OP(rd.ty().kind == ElemKind::Int8QTy && rd.ty().size() == d.ty().size(),
+               "needs an i8 result of the same size");
+    }
+    const S32To8 dp = s32to8(d.ty().scale / rd.ty().scale);
+    const int32_t rdo = rd.ty().offset;
+    params += kv("relu_dest_offset", rdo) + kv("relu_pre", dp.pre) + kv("relu_post", dp.post) +
+              kv("relu_scale", dp.scale);
+    out.launches.push_back({"mi355x_add_relu_i8", I.name + "+" + R.name, params,
+                            [=](const DeviceBindings &b) {
+                              return mi355x_add_relu_i8((int8_t *)rd.ptr(b), (const int8_t *)l.ptr(b),
+                                                        (const int8_t *)r.ptr(b), n, doff, lo, ro,
+                                                        lp.pre, lp.post, lp.scale, rp.pre, rp.post,
+                                                        rp.scale, rdo, dp.pre, dp.post, dp.scale,
+                                                        b.stream);
+                            }});
+    return Error::success();
+  }
+
+  Error relu(const Instruction &I, MI355XFunction &out) {
+    Operand d = op(I, 0), s = op(I, 1);
+    CHECK_OP(d.ty().kind == ElemKind::Int8QTy && s.ty().kind == ElemKind::Int8QTy, "needs i8 -> i8");
+    CHECK_OP(d.ty().size() == s.ty().size(), "size mismatch");
+    const size_t n = (size_t)d.ty().size();
+    const S32To8 p = s32to8(s.ty().scale / d.ty().scale);
+    const int32_t so = s.ty().offset, doff = d.ty().offset;
+    out.launches.push_back(
+        {"mi355x_relu_i8", I.name,
+         strFormat(" n=%zu", n) + kv("src_offset", so) + kv("dest_offset", doff) + kv("pre", p.pre) +
+             kv("post", p.post) + kv("scale", p.scale),
+         [=](const DeviceBindings &b) {
+           return mi355x_relu_i8((int8_t *)d.ptr(b), (const int8_t *)s.ptr(b), n, so, doff, p.pre,
+                                 p.post, p.scale, b.stream);
+         }});
+    return Error::success();
+  }
+
+  Error pool(const Instruction &I, MI355XFunction &out, bool avg) {
+    Operand d = op(I, 0), s = op(I, 1);
+    CHECK_OP((int)I.iattrs.size() == (avg ? 9 : 8), "expects %d integer attributes", avg ? 9 : 8);
+    CHECK_OP(d.ty().kind == ElemKind::Int8QTy && s.ty().kind == ElemKind::Int8QTy, "needs i8 -> i8");
+    CHECK_OP(d.ty().dims.size() == 4 && s.ty().dims.size() == 4, "needs NHWC tensors");
+    const auto &a = I.iattrs;
+    for (int i = 0; i < 8; i++) CHECK_OP(a[(size_t)i] >= 0, "negative attribute");
+    CHECK_OP(a[0] > 0 && a[1] > 0 && a[2] > 0 && a[3] > 0, "kernel and stride must be positive");
+    const size_t N = (size_t)s.ty().dims[0], IH = (size_t)s.ty().dims[1], IW = (size_t)s.ty().dims[2],
+                 C = (size_t)s.ty().dims[3];
+    const int64_t oh = ((int64_t)IH + a[4] + a[6] - a[0]) / a[2] + 1;
+    const int64_t ow = ((int64_t)IW + a[5] + a[7] - a[1]) / a[3] + 1;
+    CHECK_OP(d.ty().dims[0] == (int64_t)N && d.ty().dims[3] == (int64_t)C && d.ty().dims[1] == oh &&
+                 d.ty().dims[2] == ow,
+             "output %s does not match the computed %lld x %lld", d.ty().str().c_str(), (long long)oh,
+             (long long)ow);
+    const size_t OH = (size_t)oh, OW = (size_t)ow, kH = (size_t)a[0], kW = (size_t)a[1],
+                 sH = (size_t)a[2], sW = (size_t)a[3], pT = (size_t)a[4], pL = (size_t)a[5];
+    const int32_t doff = d.ty().offset;
+    std::string geom = strFormat(" N=%zu IH=%zu IW=%zu C=%zu OH=%zu OW=%zu KH=%zu KW=%zu sH=%zu sW=%zu "
+                                 "padT=%zu padL=%zu",
+                                 N, IH, IW, C, OH, OW, kH, kW, sH, sW, pT, pL);
+    if (!avg) {
+      // the reference passes the values through: both sides share their parameters
+      CHECK_OP(d.ty().scale == s.ty().scale && d.ty().offset == s.ty().offset,
+               "input and output must share scale and offset");
+      out.launches.push_back({"mi355x_max_pool_i8", I.name, geom + kv("out_offset", doff),
+                              [=](const DeviceBindings &b) {
+                                return mi355x_max_pool_i8((int8_t *)d.ptr(b), (const int8_t *)s.ptr(b),
+                                                          N, IH, IW, C, OH, OW, kH, kW, sH, sW, pT, pL,
+                                                          doff, b.stream);
+                              }});
+      return Error::success();
+    }
+    const int cip = a[8] != 0;
+    float sc = s.ty().scale / d.ty().scale;
+    if (cip) sc = sc / (float)(a[0] * a[1]);
+    const S32To8 p = s32to8(sc);
+    const int32_t so = s.ty().offset;
+    out.launches.push_back(
+        {"mi355x_avg_pool_i8", I.name,
+         geom + kv("count_include_pads", cip) + kv("out_offset", doff) + kv("in_offset", so) +
+             kv("pre", p.pre) + kv("post", p.post) + kv("scale", p.scale),
+         [=](const DeviceBindings &b) {
+           return mi355x_avg_pool_i8((int8_t *)d.ptr(b), (const int8_t *)s.ptr(b), N, IH, IW, C, OH, OW,
+                                     kH, kW, sH, sW, pT, pL, cip, doff, so, p.pre, p.post, p.scale,
+                                     b.stream);
+         }});
+    return Error::success();
+  }
+
+  Error softmax(const Instruction &I, MI355XFunction &out) {
+    Operand d = op(I, 0), s = op(I, 1);
+    CHECK_OP(d.ty().kind == ElemKind::FloatTy && s.ty().kind == ElemKind::FloatTy, "needs float tensors");
+    CHECK_OP(s.ty().dims.size() == 2 && d.ty().dims == s.ty().dims, "needs equal 2-D shapes");
+    const size_t rows = (size_t)s.ty().dims[0], cols = (size_t)s.ty().dims[1];
+    out.launches.push_back({"mi355x_softmax_f32", I.name, strFormat(" rows=%zu cols=%zu", rows, cols),
+                            [=](const DeviceBindings &b) {
+                              return mi355x_softmax_f32((float *)d.ptr(b), (const float *)s.ptr(b), rows,
+                                                        cols, b.stream);
+                            }});
+    return Error::success();
+  }
 
   template <typename T> const T *constData(const Operand &o) const {
     return reinterpret_cast<const T *>(M_.constantsImage().data() + o.v->offset);
@@ -595,6 +745,8 @@ bool MI355XBackend::shouldLower(Kind k) const {
   case Kind::Convolution:
   case Kind::RowwiseQuantizedFullyConnected:
   case Kind::ChannelwiseQuantizedConvolution:
+  case Kind::Relu:
+  case Kind::SoftMax:
     return false;
   default:
     return true;

@@ -117,6 +117,7 @@ private:
 
 struct BackendOptions {
   bool precomputeWeightRowSums = true; // form sum_k W[n][k] once at load time
+  bool fuseAddRelu = true;             // ElementAdd + Relu of its result in one pass
 };
 
 class MI355XBackend {

@@ -170,6 +170,52 @@ RunIdentifierTy MI355XDeviceManager::runFunction(std::string functionName,
   return id;
 }
 
+Expected<float> MI355XDeviceManager::timeFunction(const std::string &functionName, int iterations) {
+  {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (!running_ || stopping_)
+      return MI355X_MAKE_ERR(ErrorCode::RUNTIME_REQUEST_REFUSED, "device manager is not running");
+  }
+  if (iterations < 1)
+    return MI355X_MAKE_ERR(ErrorCode::RUNTIME_ERROR, "iterations must be positive");
+  std::promise<std::pair<Error, float>> done;
+  auto fut = done.get_future();
+  enqueue([this, &done, functionName, iterations] {
+    auto it = functions_.find(functionName);
+    if (it == functions_.end()) {
+      done.set_value({MI355X_MAKE_ERR(ErrorCode::RUNTIME_NET_NOT_FOUND, "Function %s not found",
+                                      functionName.c_str()),
+                      0.0f});
+      return;
+    }
+    FunctionResident &fr = it->second;
+    ExecutionContext ctx;
+    ctx.setDeviceBindings(std::unique_ptr<DeviceBindings>(new DeviceBindings(fr.bindings)));
+    void *e0 = nullptr, *e1 = nullptr;
+    Error err;
+    float ms = 0.0f;
+    int rc = mi355x_event_create(&e0);
+    if (rc == MI355X_OK) rc = mi355x_event_create(&e1);
+    if (rc == MI355X_OK) rc = mi355x_stream_sync(stream_);
+    if (rc == MI355X_OK) rc = mi355x_event_record(e0, stream_);
+    if (rc != MI355X_OK) err = fromStatus(rc, "timing set-up");
+    for (int i = 0; i < iterations && !err; i++) err = fr.fn->execute(&ctx);
+    if (!err) {
+      rc = mi355x_event_record(e1, stream_);
+      if (rc == MI355X_OK) rc = mi355x_event_sync(e1);
+      if (rc == MI355X_OK) rc = mi355x_event_elapsed_ms(e0, e1, &ms);
+      if (rc != MI355X_OK) err = fromStatus(rc, "timing");
+    }
+    mi355x_stream_sync(stream_);
+    if (e0) mi355x_event_destroy(e0);
+    if (e1) mi355x_event_destroy(e1);
+    done.set_value({std::move(err), ms / (float)iterations});
+  });
+  auto r = fut.get();
+  if (r.first) return r.first;
+  return r.second;
+}
+
 void MI355XDeviceManager::release(FunctionResident &fr) {
   if (fr.fn) fr.fn->dropGraph();
   if (fr.arena) mi355x_arena_destroy(fr.arena);

@@ -57,6 +57,12 @@ public:
   RunIdentifierTy runFunction(std::string functionName, std::unique_ptr<ExecutionContext> ctx,
                               ResultCBTy resultCB);
 
+  // Benchmark aid without a counterpart in the reference: replays a resident
+  // function `iterations` times on the data its placeholders already hold (no
+  // host copies) and reports the average device time per replay, measured
+  // with events on the manager's stream. Blocks until done.
+  Expected<float> timeFunction(const std::string &functionName, int iterations);
+
   uint64_t getMaximumMemory() const { return maxMemoryBytes_; }
   uint64_t getAvailableMemory() const { return maxMemoryBytes_ - usedMemoryBytes_; }
   bool isMemoryAvailable(uint64_t estimate) const {

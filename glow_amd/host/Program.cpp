@@ -87,6 +87,11 @@ const char *kindName(Kind k) {
     return "FusedRowwiseQuantizedSparseLengthsWeightedSum";
   case Kind::FusedRowwiseQuantizedSparseLengthsSum:
     return "FusedRowwiseQuantizedSparseLengthsSum";
+  case Kind::ElementAdd: return "ElementAdd";
+  case Kind::Relu: return "Relu";
+  case Kind::MaxPool: return "MaxPool";
+  case Kind::AvgPool: return "AvgPool";
+  case Kind::SoftMax: return "SoftMax";
   default: return "?";
   }
 }

@@ -45,6 +45,11 @@ enum class Kind : int32_t {
   ChannelwiseQuantizedConvolution, // (Dest, Src, Filter, Bias, FilterScales, FilterOffsets, BiasScales, BiasOffsets) + conv attributes
   FusedRowwiseQuantizedSparseLengthsWeightedSum, // (Dest, Data, Weights, Indices, Lengths); iattrs {useFP16Accumulation}
   FusedRowwiseQuantizedSparseLengthsSum,         // (Dest, Data, Indices, Lengths); iattrs {useFP16Accumulation}
+  ElementAdd,                   // (Dest, LHS, RHS)
+  Relu,                         // (Dest, Src)
+  MaxPool,                      // (Dest, Src); iattrs {kernelH, kernelW, strideH, strideW, padT, padL, padB, padR}
+  AvgPool,                      // (Dest, Src); MaxPool's iattrs + {countIncludePads}
+  SoftMax,                      // (Dest, Src), float [rows x cols]
   NumKinds
 };
 const char *kindName(Kind k);

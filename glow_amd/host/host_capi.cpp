@@ -103,11 +103,12 @@ int mi355x_host_is_op_supported(mi355x_host_module *m, int kind, const int *oper
   return ok ? 1 : 0;
 }
 
-int mi355x_host_compile(mi355x_host_module *m, int function, int sums) {
+int mi355x_host_compile(mi355x_host_module *m, int function, int options) {
   Function *f = fn(m, function);
   if (!f) return failMsg(ErrorCode::COMPILE_CONTEXT_MALFORMED, "no such function");
   BackendOptions o;
-  o.precomputeWeightRowSums = sums != 0;
+  o.precomputeWeightRowSums = (options & MI355X_HOST_OPT_WEIGHT_ROW_SUMS) != 0;
+  o.fuseAddRelu = (options & MI355X_HOST_OPT_FUSE_ADD_RELU) != 0;
   auto r = MI355XBackend().compile(*f, o);
   if (!r) return fail(r.error());
   m->compiled[function] = std::move(r.get());
@@ -196,6 +197,15 @@ int mi355x_host_dm_run(mi355x_host_dm *dm, const char *name, const char *const *
                      });
   Error e = fut.get();
   return e ? fail(e) : 0;
+}
+
+int mi355x_host_dm_time_function(mi355x_host_dm *dm, const char *name, int iterations,
+                                 float *ms_per_iteration) {
+  if (!dm || !name || !ms_per_iteration) return failMsg(ErrorCode::RUNTIME_ERROR, "NULL argument");
+  auto r = dm->dm.timeFunction(name, iterations);
+  if (!r) return fail(r.error());
+  *ms_per_iteration = r.get();
+  return 0;
 }
 
 uint64_t mi355x_host_dm_maximum_memory(mi355x_host_dm *dm) { return dm ? dm->dm.getMaximumMemory() : 0; }

@@ -179,6 +179,54 @@ int mi355x_rescale_i8(int8_t *dst, const int8_t *src, size_t n,
                       int32_t out_offset, int32_t in_offset, int32_t pre,
                       int32_t post, int32_t scale, void *stream);
 
+/* ---- int8 glue operators ------------------------------------------------------ */
+
+/* libjit_element_add_kernel_i8 (reference lib/LLVMIRCodeGen/libjit/libjit.cpp:
+ * 1593-1603, 1675-1676) over n elements: clip(scale(lhs - lhs_offset; lhsP) +
+ * scale(rhs - rhs_offset; rhsP) + dest_offset), parameters as derived in
+ * LLVMIRGen.cpp:1716-1771 (lhsScale/destScale, rhsScale/destScale). */
+int mi355x_add_i8(int8_t *dst, const int8_t *lhs, const int8_t *rhs, size_t n,
+                  int32_t dest_offset, int32_t lhs_offset, int32_t rhs_offset,
+                  int32_t lhs_pre, int32_t lhs_post, int32_t lhs_scale,
+                  int32_t rhs_pre, int32_t rhs_post, int32_t rhs_scale,
+                  void *stream);
+/* ElementAdd followed by Relu in one pass over memory (the CPU backend stacks
+ * both data-parallel instructions into one loop, LLVMIRGen.cpp:1465-1499 for
+ * Relu's parameters): the sum is clipped to int8 at `sum_offset` exactly as the
+ * separate add would store it, then libjit_element_relu_i8 is applied with that
+ * value as its source. */
+int mi355x_add_relu_i8(int8_t *dst, const int8_t *lhs, const int8_t *rhs,
+                       size_t n, int32_t sum_offset, int32_t lhs_offset,
+                       int32_t rhs_offset, int32_t lhs_pre, int32_t lhs_post,
+                       int32_t lhs_scale, int32_t rhs_pre, int32_t rhs_post,
+                       int32_t rhs_scale, int32_t dest_offset, int32_t dest_pre,
+                       int32_t dest_post, int32_t dest_scale, void *stream);
+/* libjit_element_relu_i8 (libjit.cpp:1851-1858): clip(scale(max(src,
+ * src_offset) - src_offset; destP, dest_offset)). */
+int mi355x_relu_i8(int8_t *dst, const int8_t *src, size_t n, int32_t src_offset,
+                   int32_t dest_offset, int32_t dest_pre, int32_t dest_post,
+                   int32_t dest_scale, void *stream);
+/* libjit_max_pool_i8 (libjit.cpp:812-884, 2592-2597): NHWC int8, pads {top,
+ * left}; a window with no valid tap yields out_offset. */
+int mi355x_max_pool_i8(int8_t *out, const int8_t *in, size_t N, size_t IH,
+                       size_t IW, size_t C, size_t OH, size_t OW, size_t kH,
+                       size_t kW, size_t sH, size_t sW, size_t padT,
+                       size_t padL, int32_t out_offset, void *stream);
+/* libjit_avg_pool_i8 (libjit.cpp:2812-2880); the scale parameters are those of
+ * LLVMIRGen.cpp:3003-3048 (srcScale/destScale, divided by the kernel area when
+ * count_include_pads). */
+int mi355x_avg_pool_i8(int8_t *out, const int8_t *in, size_t N, size_t IH,
+                       size_t IW, size_t C, size_t OH, size_t OW, size_t kH,
+                       size_t kW, size_t sH, size_t sW, size_t padT,
+                       size_t padL, int count_include_pads, int32_t out_offset,
+                       int32_t in_offset, int32_t out_pre, int32_t out_post,
+                       int32_t out_scale, void *stream);
+/* libjit_softmax_f (libjit.cpp:3058-3082) on fp32 [rows x cols]. The row sum is
+ * reduced in parallel, so results match the CPU to fp32 rounding (1e-5
+ * relative), not bit for bit. */
+int mi355x_softmax_f32(float *out, const float *in, size_t rows, size_t cols,
+                       void *stream);
+
 /* ---- FullyConnected / MatMul -------------------------------------------------- */
 
 /* sums[r] = sum over k of rows[r][k] for an int8 matrix [n_rows x K] with K

@@ -62,7 +62,12 @@ enum {
   MI355X_HOST_CONVOLUTION = 6,         /* Dest, Src, Filter, Bias; 12 iattrs */
   MI355X_HOST_CHANNELWISE_QUANTIZED_CONV = 7, /* + FilterScales, FilterOffsets, BiasScales, BiasOffsets */
   MI355X_HOST_FRWQ_SLWS = 8,           /* Dest, Data, Weights, Indices, Lengths; iattrs {useFP16Accumulation} */
-  MI355X_HOST_FRWQ_SLS = 9             /* Dest, Data, Indices, Lengths; iattrs {useFP16Accumulation} */
+  MI355X_HOST_FRWQ_SLS = 9,            /* Dest, Data, Indices, Lengths; iattrs {useFP16Accumulation} */
+  MI355X_HOST_ELEMENT_ADD = 10,        /* Dest, LHS, RHS */
+  MI355X_HOST_RELU = 11,               /* Dest, Src */
+  MI355X_HOST_MAX_POOL = 12,           /* Dest, Src; iattrs kernelH, kernelW, strideH, strideW, padT, padL, padB, padR */
+  MI355X_HOST_AVG_POOL = 13,           /* Dest, Src; MaxPool's iattrs + countIncludePads */
+  MI355X_HOST_SOFTMAX = 14             /* Dest, Src (float, [rows x cols]) */
 };
 /* Convolution iattrs: kernelH, kernelW, strideH, strideW, padT, padL, padB,
  * padR, group, dilationH, dilationW, fusedActivation (glow::FusedActivation);
@@ -93,8 +98,14 @@ int mi355x_host_add_instruction(mi355x_host_module *m, int function, int kind, c
 int mi355x_host_is_op_supported(mi355x_host_module *m, int kind, const int *operands,
                                 int n_operands, const int64_t *iattrs, int n_iattrs,
                                 const float *fattrs, int n_fattrs);
-/* Backend::compile of one function; the compiled function stays with the module. */
-int mi355x_host_compile(mi355x_host_module *m, int function, int precompute_weight_row_sums);
+/* Backend::compile of one function; the compiled function stays with the
+ * module. `options` is a set of MI355X_HOST_OPT_* bits (BackendOptions). */
+enum {
+  MI355X_HOST_OPT_WEIGHT_ROW_SUMS = 1, /* form sum_k W[n][k] once at load time */
+  MI355X_HOST_OPT_FUSE_ADD_RELU = 2,   /* ElementAdd + Relu of its result in one pass */
+  MI355X_HOST_OPT_DEFAULT = 3
+};
+int mi355x_host_compile(mi355x_host_module *m, int function, int options);
 /* Listing of the compiled function's launches and derived parameters; returns
  * the length needed (text is truncated to cap-1 bytes). */
 int mi355x_host_describe(mi355x_host_module *m, int function, char *buf, size_t cap);
@@ -114,6 +125,11 @@ int mi355x_host_dm_evict_network(mi355x_host_dm *dm, const char *function_name);
  * the result callback. */
 int mi355x_host_dm_run(mi355x_host_dm *dm, const char *function_name, const char *const *names,
                        void *const *buffers, const size_t *bytes, int n);
+/* Benchmark aid (no counterpart in the reference): replays a resident function
+ * `iterations` times on the data already in its placeholders, without host
+ * copies, and reports the average device milliseconds per replay. */
+int mi355x_host_dm_time_function(mi355x_host_dm *dm, const char *function_name, int iterations,
+                                 float *ms_per_iteration);
 uint64_t mi355x_host_dm_maximum_memory(mi355x_host_dm *dm);
 uint64_t mi355x_host_dm_available_memory(mi355x_host_dm *dm);
 

@@ -670,3 +670,124 @@ void go_embedding_bag_byte_rowwise_offsets_f32(
     }
   }
 }
+
+/* ---- int8 glue operators ----------------------------------------------- */
+
+/* libjit.cpp:1593-1603 with body lhs + rhs (:1675-1676) */
+void go_add_i8(int8_t *dest, const int8_t *lhs, const int8_t *rhs, size_t n,
+               int32_t destOffset, int32_t lhsOffset, int32_t rhsOffset,
+               int32_t lhsPre, int32_t lhsPost, int32_t lhsScale,
+               int32_t rhsPre, int32_t rhsPost, int32_t rhsScale) {
+  for (size_t i = 0; i < n; i++) {
+    const int32_t l = go_scale_i32(lhs[i] - lhsOffset, lhsPre, lhsPost, lhsScale, 0);
+    const int32_t r = go_scale_i32(rhs[i] - rhsOffset, rhsPre, rhsPost, rhsScale, 0);
+    dest[i] = go_clip_i8((int32_t)((uint32_t)l + (uint32_t)r + (uint32_t)destOffset));
+  }
+}
+
+/* libjit.cpp:1851-1858 */
+void go_relu_i8(int8_t *dest, const int8_t *src, size_t n, int8_t srcOffset,
+                int8_t destOffset, int32_t destPre, int32_t destPost,
+                int32_t destScale) {
+  for (size_t i = 0; i < n; i++) {
+    const int32_t v = src[i] > srcOffset ? src[i] : srcOffset;
+    dest[i] = go_clip_i8(go_scale_i32(v - srcOffset, destPre, destPost, destScale, destOffset));
+  }
+}
+
+/* window limits of libjit_defs.h:257-275 */
+static void window(ptrdiff_t inMin, size_t inSize, size_t k, ptrdiff_t *lo, ptrdiff_t *len) {
+  const ptrdiff_t fmin = inMin < 0 ? -inMin : 0;
+  ptrdiff_t fmax = (ptrdiff_t)inSize - inMin;
+  if ((ptrdiff_t)k < fmax) fmax = (ptrdiff_t)k;
+  *lo = fmin;
+  *len = fmax - fmin > 0 ? fmax - fmin : 0;
+}
+
+/* libjit.cpp:812-884 */
+void go_max_pool_i8(int8_t *out, const int8_t *in, size_t N, size_t IH,
+                    size_t IW, size_t C, size_t OH, size_t OW, size_t kH,
+                    size_t kW, size_t sH, size_t sW, size_t padT, size_t padL,
+                    int32_t outOffset) {
+  for (size_t n = 0; n < N; n++)
+    for (size_t oh = 0; oh < OH; oh++) {
+      ptrdiff_t h0, hl;
+      const ptrdiff_t ihMin = (ptrdiff_t)(oh * sH) - (ptrdiff_t)padT;
+      window(ihMin, IH, kH, &h0, &hl);
+      for (size_t ow = 0; ow < OW; ow++) {
+        ptrdiff_t w0, wl;
+        const ptrdiff_t iwMin = (ptrdiff_t)(ow * sW) - (ptrdiff_t)padL;
+        window(iwMin, IW, kW, &w0, &wl);
+        for (size_t c = 0; c < C; c++) {
+          int8_t m = INT8_MIN;
+          for (ptrdiff_t fh = 0; fh < hl; fh++)
+            for (ptrdiff_t fw = 0; fw < wl; fw++) {
+              const int8_t v = in[((n * IH + (size_t)(ihMin + h0 + fh)) * IW +
+                                   (size_t)(iwMin + w0 + fw)) * C + c];
+              if (v > m) m = v;
+            }
+          *out++ = (hl > 0 && wl > 0) ? m : (int8_t)outOffset;
+        }
+      }
+    }
+}
+
+/* libjit_defs.h:239-244 */
+static int32_t div_round_i32(int32_t input, int32_t divider) {
+  const int32_t rnd = divider >> 1;
+  return input > 0 ? (input + rnd) / divider : (input - rnd) / divider;
+}
+
+/* libjit.cpp:2812-2880 */
+void go_avg_pool_i8(int8_t *out, const int8_t *in, size_t N, size_t IH,
+                    size_t IW, size_t C, size_t OH, size_t OW, size_t kH,
+                    size_t kW, size_t sH, size_t sW, size_t padT, size_t padL,
+                    int countIncludePads, int32_t outOffset, int32_t inOffset,
+                    int32_t outPre, int32_t outPost, int32_t outScale) {
+  for (size_t n = 0; n < N; n++)
+    for (size_t oh = 0; oh < OH; oh++) {
+      ptrdiff_t h0, hl;
+      const ptrdiff_t ihMin = (ptrdiff_t)(oh * sH) - (ptrdiff_t)padT;
+      window(ihMin, IH, kH, &h0, &hl);
+      for (size_t ow = 0; ow < OW; ow++) {
+        ptrdiff_t w0, wl;
+        const ptrdiff_t iwMin = (ptrdiff_t)(ow * sW) - (ptrdiff_t)padL;
+        window(iwMin, IW, kW, &w0, &wl);
+        for (size_t c = 0; c < C; c++) {
+          int32_t sum = 0;
+          for (ptrdiff_t fh = 0; fh < hl; fh++)
+            for (ptrdiff_t fw = 0; fw < wl; fw++)
+              sum += in[((n * IH + (size_t)(ihMin + h0 + fh)) * IW +
+                         (size_t)(iwMin + w0 + fw)) * C + c] - inOffset;
+          if (countIncludePads) {
+            *out++ = go_clip_i8(go_scale_i32(sum, outPre, outPost, outScale, outOffset));
+          } else {
+            const int32_t area = (int32_t)(hl * wl);
+            if (area == 0) {
+              *out++ = (int8_t)outOffset;
+            } else {
+              sum = go_scale_i32(sum, outPre, outPost, outScale, 0);
+              *out++ = go_clip_i8(div_round_i32(sum, area) + outOffset);
+            }
+          }
+        }
+      }
+    }
+}
+
+/* libjit.cpp:3058-3082 */
+void go_softmax_f32(float *out, const float *in, size_t rows, size_t cols) {
+  for (size_t n = 0; n < rows; n++) {
+    const float *x = in + n * cols;
+    float *y = out + n * cols;
+    float mx = x[0];
+    for (size_t i = 1; i < cols; i++) mx = x[i] > mx ? x[i] : mx;
+    float sum = 0;
+    for (size_t i = 0; i < cols; i++) {
+      const float e = expf(x[i] - mx);
+      sum += e;
+      y[i] = e;
+    }
+    for (size_t i = 0; i < cols; i++) y[i] = y[i] / sum;
+  }
+}

@@ -196,6 +196,31 @@ void go_embedding_bag_byte_rowwise_offsets_f32(
     size_t numIndices, size_t inLineSize, size_t outLineSize,
     int hasEndOffset);
 
+/* ---- int8 glue operators (ResNet-style graphs) --------------------------- */
+
+/* libjit_element_add_kernel_i8 (libjit.cpp:1593-1603, 1675-1676) over n. */
+void go_add_i8(int8_t *dest, const int8_t *lhs, const int8_t *rhs, size_t n,
+               int32_t destOffset, int32_t lhsOffset, int32_t rhsOffset,
+               int32_t lhsPre, int32_t lhsPost, int32_t lhsScale,
+               int32_t rhsPre, int32_t rhsPost, int32_t rhsScale);
+/* libjit_element_relu_i8 (libjit.cpp:1851-1858) over n. */
+void go_relu_i8(int8_t *dest, const int8_t *src, size_t n, int8_t srcOffset,
+                int8_t destOffset, int32_t destPre, int32_t destPost,
+                int32_t destScale);
+/* libjit_max_pool_i8 (libjit.cpp:812-884, 2592-2597); NHWC, pads {top, left}. */
+void go_max_pool_i8(int8_t *out, const int8_t *in, size_t N, size_t IH,
+                    size_t IW, size_t C, size_t OH, size_t OW, size_t kH,
+                    size_t kW, size_t sH, size_t sW, size_t padT, size_t padL,
+                    int32_t outOffset);
+/* libjit_avg_pool_i8 (libjit.cpp:2812-2880). */
+void go_avg_pool_i8(int8_t *out, const int8_t *in, size_t N, size_t IH,
+                    size_t IW, size_t C, size_t OH, size_t OW, size_t kH,
+                    size_t kW, size_t sH, size_t sW, size_t padT, size_t padL,
+                    int countIncludePads, int32_t outOffset, int32_t inOffset,
+                    int32_t outPre, int32_t outPost, int32_t outScale);
+/* libjit_softmax_f (libjit.cpp:3058-3082) on [rows x cols]. */
+void go_softmax_f32(float *out, const float *in, size_t rows, size_t cols);
+
 #ifdef __cplusplus
 }
 #endif

@@ -354,3 +354,63 @@ def embedding_bag_byte_rowwise_offsets_f32(data, weights, indices, offsets,
         C.c_size_t(segs), C.c_size_t(indices.size), C.c_size_t(in_line),
         C.c_size_t(out_line), C.c_int(has_end_offset))
     return out
+
+
+# ---- int8 glue operators -----------------------------------------------------
+
+def add_i8(lhs, rhs, dest_offset, lhs_offset, rhs_offset, lhsP, rhsP):
+    """lhsP / rhsP = (pre, post, scale)."""
+    lhs = _c(lhs, np.int8)
+    rhs = _c(rhs, np.int8)
+    out = np.empty(lhs.shape, np.int8)
+    lib().go_add_i8(_p(out), _p(lhs), _p(rhs), C.c_size_t(lhs.size),
+                    C.c_int32(dest_offset), C.c_int32(lhs_offset), C.c_int32(rhs_offset),
+                    *[C.c_int32(int(v)) for v in lhsP], *[C.c_int32(int(v)) for v in rhsP])
+    return out
+
+
+def relu_i8(src, src_offset, dest_offset, destP):
+    src = _c(src, np.int8)
+    out = np.empty(src.shape, np.int8)
+    lib().go_relu_i8(_p(out), _p(src), C.c_size_t(src.size), C.c_int8(src_offset),
+                     C.c_int8(dest_offset), *[C.c_int32(int(v)) for v in destP])
+    return out
+
+
+def pool_out_dims(IH, IW, kernel, stride, pads):
+    """pads = (top, left, bottom, right)."""
+    OH = (IH + pads[0] + pads[2] - kernel[0]) // stride[0] + 1
+    OW = (IW + pads[1] + pads[3] - kernel[1]) // stride[1] + 1
+    return OH, OW
+
+
+def _pool_args(x, kernel, stride, pads):
+    N, IH, IW, Cn = x.shape
+    OH, OW = pool_out_dims(IH, IW, kernel, stride, pads)
+    out = np.empty((N, OH, OW, Cn), np.int8)
+    sz = [C.c_size_t(int(v)) for v in (N, IH, IW, Cn, OH, OW, kernel[0], kernel[1],
+                                       stride[0], stride[1], pads[0], pads[1])]
+    return out, sz
+
+
+def max_pool_i8(x, kernel, stride, pads, out_offset):
+    x = _c(x, np.int8)
+    out, sz = _pool_args(x, kernel, stride, pads)
+    lib().go_max_pool_i8(_p(out), _p(x), *sz, C.c_int32(out_offset))
+    return out
+
+
+def avg_pool_i8(x, kernel, stride, pads, count_include_pads, out_offset, in_offset, outP):
+    x = _c(x, np.int8)
+    out, sz = _pool_args(x, kernel, stride, pads)
+    lib().go_avg_pool_i8(_p(out), _p(x), *sz, C.c_int(int(count_include_pads)),
+                         C.c_int32(out_offset), C.c_int32(in_offset),
+                         *[C.c_int32(int(v)) for v in outP])
+    return out
+
+
+def softmax_f32(x):
+    x = _c(x, np.float32)
+    out = np.empty_like(x)
+    lib().go_softmax_f32(_p(out), _p(x), C.c_size_t(x.shape[0]), C.c_size_t(x.shape[1]))
+    return out

@@ -224,3 +224,61 @@ def embedding_bag_byte_rowwise_offsets_f32(data, weights, indices, offsets,
         C.c_uint64(segs), C.c_uint64(indices.size), C.c_uint64(in_line),
         C.c_uint64(out_line), C.c_bool(has_end_offset))
     return out
+
+
+# ---- int8 glue operators (libjit.cpp:1593-1603, 1851-1858, 2592-2597, 2812-2880, 3058-3082) ----
+
+def add_i8(lhs, rhs, dest_offset, lhs_offset, rhs_offset, lhsP, rhsP, fastmath=False):
+    lhs = _c(lhs, np.int8).ravel()
+    rhs = _c(rhs, np.int8).ravel()
+    f = lib(fastmath).libjit_element_add_kernel_i8
+    f.restype = C.c_int8
+    f.argtypes = [C.c_uint64, C.c_void_p, C.c_void_p] + [C.c_int32] * 9
+    pl, pr = lhs.ctypes.data, rhs.ctypes.data
+    return np.array([f(i, pl, pr, dest_offset, lhs_offset, rhs_offset,
+                       *[int(v) for v in lhsP], *[int(v) for v in rhsP])
+                     for i in range(lhs.size)], np.int8)
+
+
+def relu_i8(src, src_offset, dest_offset, destP, fastmath=False):
+    src = _c(src, np.int8).ravel()
+    f = lib(fastmath).libjit_element_relu_i8
+    f.restype = C.c_int8
+    f.argtypes = [C.c_uint64, C.c_void_p, C.c_int8, C.c_int8] + [C.c_int32] * 3
+    ps = src.ctypes.data
+    return np.array([f(i, ps, src_offset, dest_offset, *[int(v) for v in destP])
+                     for i in range(src.size)], np.int8)
+
+
+def _pool_dims(x, kernel, stride, pads):
+    N, IH, IW, Cn = x.shape
+    OH = (IH + pads[0] + pads[2] - kernel[0]) // stride[0] + 1
+    OW = (IW + pads[1] + pads[3] - kernel[1]) // stride[1] + 1
+    return (np.empty((N, OH, OW, Cn), np.int8), _dims(N, IH, IW, Cn), _dims(N, OH, OW, Cn),
+            _dims(*kernel), _dims(*stride), _dims(*pads))
+
+
+def max_pool_i8(x, kernel, stride, pads, out_offset, fastmath=False):
+    x = _c(x, np.int8)
+    out, idm, od, ks, st, pd = _pool_dims(x, kernel, stride, pads)
+    lib(fastmath).libjit_max_pool_i8(_p(x), _p(out), _p(idm), _p(od), _p(ks), _p(st), _p(pd),
+                                     C.c_int32(out_offset))
+    return out
+
+
+def avg_pool_i8(x, kernel, stride, pads, count_include_pads, out_offset, in_offset, outP,
+                fastmath=False):
+    x = _c(x, np.int8)
+    out, idm, od, ks, st, pd = _pool_dims(x, kernel, stride, pads)
+    lib(fastmath).libjit_avg_pool_i8(_p(x), _p(out), _p(idm), _p(od), _p(ks), _p(st), _p(pd),
+                                     C.c_bool(bool(count_include_pads)), C.c_int32(out_offset),
+                                     C.c_int32(in_offset), *[C.c_int32(int(v)) for v in outP])
+    return out
+
+
+def softmax_f32(x, fastmath=False):
+    x = _c(x, np.float32)
+    out = np.empty_like(x)
+    d = _dims(*x.shape)
+    lib(fastmath).libjit_softmax_f(_p(x), _p(out), _p(d), _p(d))
+    return out

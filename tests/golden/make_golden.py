@@ -31,8 +31,51 @@ def save(name, **kw):
     print(name, os.path.getsize(path), "bytes")
 
 
+def glue():
+    """int8 glue operators: add, relu, max pool, avg pool; fp32 softmax."""
+    rng = np.random.default_rng(600)
+    gl = {}
+    a = rng.integers(-128, 128, (3, 7, 5, 6)).astype(np.int8)
+    b = rng.integers(-128, 128, a.shape).astype(np.int8)
+    gl["a"], gl["b"] = a, b
+    for i, (ls, rs, ds, lo, ro, do) in enumerate([(0.05, 0.07, 0.11, 3, -4, 5),
+                                                  (0.3, 0.002, 0.1, -128, 0, -128),
+                                                  (1.0, 1.0, 1.0, 0, 0, 0)]):
+        lp = go.quantize_scale_offset_32to8(float(np.float32(ls) / np.float32(ds)), lo)[:3]
+        rp = go.quantize_scale_offset_32to8(float(np.float32(rs) / np.float32(ds)), ro)[:3]
+        gl[f"add{i}_params"] = np.array([do, lo, ro, *lp, *rp], np.int32)
+        gl[f"add{i}_out"] = ref.add_i8(a, b, do, lo, ro, lp, rp).reshape(a.shape)
+    for i, (ss, ds, so, do) in enumerate([(0.1, 0.1, -20, -128), (0.05, 0.2, 7, 7),
+                                          (0.4, 0.013, -128, -100)]):
+        dp = go.quantize_scale_offset_32to8(float(np.float32(ss) / np.float32(ds)), 0)[:3]
+        gl[f"relu{i}_params"] = np.array([so, do, *dp], np.int32)
+        gl[f"relu{i}_out"] = ref.relu_i8(a, so, do, dp).reshape(a.shape)
+    x = rng.integers(-128, 128, (2, 9, 11, 20)).astype(np.int8)
+    gl["x"] = x
+    pools = [((3, 3), (2, 2), (1, 1, 1, 1)), ((2, 3), (1, 2), (0, 1, 0, 1)),
+             ((9, 11), (1, 1), (0, 0, 0, 0)), ((3, 3), (3, 3), (2, 2, 2, 2))]
+    for i, (k, st, pd) in enumerate(pools):
+        gl[f"pool{i}_geom"] = np.array([*k, *st, *pd], np.int32)
+        gl[f"maxpool{i}_out"] = ref.max_pool_i8(x, k, st, pd, -7)
+        for cip in (0, 1):
+            sc = np.float32(0.06) / np.float32(0.05)
+            if cip:
+                sc = sc / np.float32(k[0] * k[1])
+            op = go.quantize_scale_offset_32to8(float(sc), 0)[:3]
+            gl[f"avgpool{i}_{cip}_params"] = np.array([cip, 4, -9, *op], np.int32)
+            gl[f"avgpool{i}_{cip}_out"] = ref.avg_pool_i8(x, k, st, pd, cip, 4, -9, op)
+    logits = rng.normal(0, 3, (5, 1000)).astype(np.float32)
+    logits[1] *= 10
+    gl["logits"] = logits
+    gl["softmax_out"] = ref.softmax_f32(logits)
+    save("glue", **gl)
+
+
 def main():
     assert ref.available(), "build oracle/_ref first (make -C oracle)"
+    if sys.argv[1:] == ["glue"]:
+        glue()
+        return
 
     # elementwise
     rng = np.random.default_rng(100)
@@ -113,6 +156,7 @@ def main():
         sl[f"{tag}_weights"] = w
         sl[f"{tag}_out"] = ref.frwq_slws_f32(table, w, idx, lengths)
     save("frwq_slws", **sl)
+    glue()
 
 
 if __name__ == "__main__":

@@ -63,3 +63,31 @@ def slws_cases():
     for t in _tags(d):
         g = lambda k: d[f"{t}_{k}"]
         yield t, (g("table"), g("weights"), g("indices"), g("lengths")), g("out")
+
+
+def glue():
+    """Golden int8 glue operators. Yields (name, callable(impl) -> got, want)
+    where `impl` is a module with add_i8 / relu_i8 / max_pool_i8 / avg_pool_i8 /
+    softmax_f32 in the oracle wrappers' signature."""
+    d = _load("glue")
+    a, b, x = d["a"], d["b"], d["x"]
+    out = []
+    for i in range(3):
+        p = [int(v) for v in d[f"add{i}_params"]]
+        out.append((f"add{i}", lambda m, p=p: m.add_i8(a, b, p[0], p[1], p[2], p[3:6], p[6:9]),
+                    d[f"add{i}_out"]))
+        p = [int(v) for v in d[f"relu{i}_params"]]
+        out.append((f"relu{i}", lambda m, p=p: m.relu_i8(a, p[0], p[1], p[2:5]),
+                    d[f"relu{i}_out"]))
+    for i in range(4):
+        g = [int(v) for v in d[f"pool{i}_geom"]]
+        k, st, pd = g[0:2], g[2:4], g[4:8]
+        out.append((f"maxpool{i}", lambda m, k=k, st=st, pd=pd: m.max_pool_i8(x, k, st, pd, -7),
+                    d[f"maxpool{i}_out"]))
+        for cip in (0, 1):
+            p = [int(v) for v in d[f"avgpool{i}_{cip}_params"]]
+            out.append((f"avgpool{i}_{cip}",
+                        lambda m, k=k, st=st, pd=pd, p=p: m.avg_pool_i8(x, k, st, pd, p[0], p[1],
+                                                                       p[2], p[3:6]),
+                        d[f"avgpool{i}_{cip}_out"]))
+    return out, d["logits"], d["softmax_out"]

@@ -59,3 +59,11 @@ def test_slws_golden():
         np.testing.assert_array_equal(go.frwq_slws_f32(table, w, idx, lens), want)
         n += 1
     assert n == 2
+
+
+def test_glue_golden():
+    ops, logits, softmax = gio.glue()
+    for name, call, want in ops:
+        np.testing.assert_array_equal(call(go), want, err_msg=name)
+    # libm's expf may differ by an ulp between hosts; the sums are sequential
+    np.testing.assert_allclose(go.softmax_f32(logits), softmax, rtol=2e-6, atol=1e-30)

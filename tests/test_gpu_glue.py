@@ -1,0 +1,113 @@
+"""int8 glue operators on the GPU through the C ABI: bit-exact against the
+oracle and the golden vectors of the reference's compiled libjit; fp32 softmax
+within 1e-5 relative."""
+import numpy as np
+import pytest
+
+from glow_amd import capi
+from oracle import glow_oracle as go
+from tests import golden_io as gio
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _init():
+    capi.init(0)
+
+
+def _p(ratio):
+    return go.quantize_scale_offset_32to8(float(np.float32(ratio)), 0)[:3]
+
+
+def test_glue_golden():
+    ops, logits, softmax = gio.glue()
+    for name, call, want in ops:
+        np.testing.assert_array_equal(call(capi), want, err_msg=name)
+    np.testing.assert_allclose(capi.softmax_f32(logits), softmax, rtol=1e-5, atol=1e-30)
+
+
+@pytest.mark.parametrize("shape", [(1,), (15,), (16,), (4099,), (3, 7, 11, 13), (64, 56, 56, 64)])
+def test_add_and_relu(shape):
+    rng = np.random.default_rng(sum(shape))
+    a = rng.integers(-128, 128, shape).astype(np.int8)
+    b = rng.integers(-128, 128, shape).astype(np.int8)
+    for ls, rs, ds, lo, ro, do in [(0.05, 0.07, 0.11, 3, -4, 5), (0.3, 0.002, 0.1, -128, 0, -128),
+                                   (0.9, 1.1, 0.25, 100, -100, 0)]:
+        lp, rp = _p(np.float32(ls) / np.float32(ds)), _p(np.float32(rs) / np.float32(ds))
+        want = go.add_i8(a, b, do, lo, ro, lp, rp)
+        np.testing.assert_array_equal(capi.add_i8(a, b, do, lo, ro, lp, rp), want)
+        dp = _p(np.float32(ds) / np.float32(0.2))
+        want_r = go.relu_i8(want, do, -7, dp)
+        np.testing.assert_array_equal(capi.relu_i8(want, do, -7, dp), want_r)
+        # the fused pass gives what the two separate instructions give
+        np.testing.assert_array_equal(
+            capi.add_relu_i8(a, b, do, lo, ro, lp, rp, -7, dp), want_r)
+
+
+def test_elementwise_unaligned_views():
+    """Tensors that start at an odd device address take the scalar path."""
+    rng = np.random.default_rng(5)
+    n = 1000
+    a = rng.integers(-128, 128, n + 1).astype(np.int8)
+    b = rng.integers(-128, 128, n + 1).astype(np.int8)
+    da, db = capi.to_device(a), capi.to_device(b)
+    out = capi.DeviceBuffer.empty((n + 1,), np.int8)
+    out.fill(0)
+    lp, rp = _p(0.5), _p(0.7)
+    capi.launch_add_i8(out.ptr + 1, da.ptr + 1, db.ptr + 1, n, 1, 2, 3, lp, rp)
+    got = out.numpy()
+    assert got[0] == 0
+    np.testing.assert_array_equal(got[1:], go.add_i8(a[1:], b[1:], 1, 2, 3, lp, rp))
+
+
+POOLS = [
+    ((2, 9, 11, 20), (3, 3), (2, 2), (1, 1, 1, 1)),
+    ((2, 9, 11, 32), (3, 3), (2, 2), (1, 1, 1, 1)),      # 16-byte channel groups
+    ((1, 8, 8, 16), (2, 2), (2, 2), (0, 0, 0, 0)),
+    ((3, 7, 7, 64), (7, 7), (1, 1), (0, 0, 0, 0)),       # global pooling
+    ((1, 6, 5, 3), (3, 2), (1, 2), (2, 1, 2, 1)),
+    ((1, 5, 5, 4), (3, 3), (3, 3), (2, 2, 2, 2)),        # windows that start in the padding
+    ((2, 112, 112, 64), (3, 3), (2, 2), (1, 1, 1, 1)),   # the ResNet stem pool
+]
+
+
+@pytest.mark.parametrize("shape,k,st,pd", POOLS)
+def test_max_pool(shape, k, st, pd):
+    rng = np.random.default_rng(shape[1] * 31 + shape[3])
+    x = rng.integers(-128, 128, shape).astype(np.int8)
+    np.testing.assert_array_equal(capi.max_pool_i8(x, k, st, pd, -5),
+                                  go.max_pool_i8(x, k, st, pd, -5))
+
+
+@pytest.mark.parametrize("shape,k,st,pd", POOLS)
+@pytest.mark.parametrize("cip", [0, 1])
+def test_avg_pool(shape, k, st, pd, cip):
+    rng = np.random.default_rng(shape[1] * 37 + shape[3] + cip)
+    x = rng.integers(-128, 128, shape).astype(np.int8)
+    sc = np.float32(0.06) / np.float32(0.05)
+    if cip:
+        sc = sc / np.float32(k[0] * k[1])
+    op = _p(sc)
+    np.testing.assert_array_equal(capi.avg_pool_i8(x, k, st, pd, cip, 4, -9, op),
+                                  go.avg_pool_i8(x, k, st, pd, cip, 4, -9, op))
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 1), (3, 7), (64, 1000), (5, 5000)])
+def test_softmax(rows, cols):
+    rng = np.random.default_rng(rows + cols)
+    x = rng.normal(0, 5, (rows, cols)).astype(np.float32)
+    got = capi.softmax_f32(x)
+    np.testing.assert_allclose(got, go.softmax_f32(x), rtol=1e-5, atol=1e-30)
+    np.testing.assert_allclose(got.sum(axis=1), 1.0, rtol=1e-5)
+
+
+def test_argument_errors():
+    with pytest.raises(capi.MI355XError):
+        capi.add_i8(np.zeros(4, np.int8), np.zeros(4, np.int8), 0, 0, 0, (0, 40, 1), (0, 0, 1))
+    x = np.zeros((1, 4, 4, 4), np.int8)
+    d = capi.to_device(x)
+    with pytest.raises(capi.MI355XError):   # output larger than the input allows
+        capi.check(capi.lib().mi355x_max_pool_i8(
+            capi._vp(d), capi._vp(d), *[capi._sz(v) for v in (1, 4, 4, 4, 9, 9, 2, 2, 1, 1, 0, 0)],
+            capi._i32(0), capi._vp(None)))

@@ -188,3 +188,58 @@ def test_device_manager_without_a_device():
     with pytest.raises(H.HostError) as e:
         dm.run("main", {})
     assert e.value.code_name == "RUNTIME_REQUEST_REFUSED"
+
+
+def _resblock_tail(fuse):
+    """conv output + residual -> ElementAdd -> Relu, the tail of a ResNet block."""
+    m = H.Module()
+    a = m.placeholder("a", (2, 4, 4, 16), H.INT8Q, np.int8, 0.05, 3)
+    b = m.placeholder("b", (2, 4, 4, 16), H.INT8Q, np.int8, 0.07, -4)
+    out = m.placeholder("out", (2, 4, 4, 16), H.INT8Q, np.int8, 0.2, -128)
+    f = m.function("main")
+    s = m.activation(f, "sum", (2, 4, 4, 16), H.INT8Q, 0.11, 5)
+    m.instruction(f, H.ELEMENT_ADD, "add", [s, a, b])
+    m.instruction(f, H.RELU, "relu", [out, s])
+    m.compile(f, fuse_add_relu=fuse)
+    return H.parse_listing(m.describe(f))
+
+
+def test_add_relu_parameters_and_fusion():
+    lp = go.quantize_scale_offset_32to8(float(np.float32(0.05) / np.float32(0.11)), 0)[:3]
+    rp = go.quantize_scale_offset_32to8(float(np.float32(0.07) / np.float32(0.11)), 0)[:3]
+    dp = go.quantize_scale_offset_32to8(float(np.float32(0.11) / np.float32(0.2)), 0)[:3]
+    sep = _resblock_tail(False)
+    assert [r["kernel"] for r in sep] == ["mi355x_add_i8", "mi355x_relu_i8"]
+    assert (sep[0]["lhs_pre"], sep[0]["lhs_post"], sep[0]["lhs_scale"]) == lp
+    assert (sep[0]["rhs_pre"], sep[0]["rhs_post"], sep[0]["rhs_scale"]) == rp
+    assert (sep[0]["dest_offset"], sep[0]["lhs_offset"], sep[0]["rhs_offset"]) == (5, 3, -4)
+    assert (sep[1]["pre"], sep[1]["post"], sep[1]["scale"]) == dp
+    assert (sep[1]["src_offset"], sep[1]["dest_offset"]) == (5, -128)
+    fused = _resblock_tail(True)
+    assert [r["kernel"] for r in fused] == ["mi355x_add_relu_i8"]
+    assert (fused[0]["relu_pre"], fused[0]["relu_post"], fused[0]["relu_scale"]) == dp
+    assert fused[0]["relu_dest_offset"] == -128 and fused[0]["dest_offset"] == 5
+
+
+def test_pool_parameters_and_checks():
+    m = H.Module()
+    x = m.placeholder("x", (2, 9, 9, 16), H.INT8Q, np.int8, 0.06, -9)
+    mp = m.placeholder("mp", (2, 5, 5, 16), H.INT8Q, np.int8, 0.06, -9)
+    ap = m.placeholder("ap", (2, 5, 5, 16), H.INT8Q, np.int8, 0.05, 4)
+    f = m.function("main")
+    attrs = [3, 3, 2, 2, 1, 1, 1, 1]
+    m.instruction(f, H.MAX_POOL, "maxpool", [mp, x], attrs)
+    m.instruction(f, H.AVG_POOL, "avgpool", [ap, x], attrs + [1])
+    m.compile(f)
+    rows = H.parse_listing(m.describe(f))
+    assert rows[0]["kernel"] == "mi355x_max_pool_i8" and rows[0]["out_offset"] == -9
+    sc = np.float32(0.06) / np.float32(0.05) / np.float32(9)
+    assert (rows[1]["pre"], rows[1]["post"], rows[1]["scale"]) == \
+        go.quantize_scale_offset_32to8(float(sc), 0)[:3]
+    assert (rows[1]["in_offset"], rows[1]["out_offset"], rows[1]["count_include_pads"]) == (-9, 4, 1)
+    # max pool passes values through: differing parameters are rejected
+    bad = m.placeholder("bad", (2, 5, 5, 16), H.INT8Q, np.int8, 0.07, -9)
+    assert not m.is_op_supported(H.MAX_POOL, [bad, x], attrs)[0]
+    wrong = m.placeholder("wrong", (2, 4, 4, 16), H.INT8Q, np.int8, 0.06, -9)
+    ok, why = m.is_op_supported(H.MAX_POOL, [wrong, x], attrs)
+    assert not ok and "computed 5 x 5" in why

@@ -151,3 +151,30 @@ def test_embedding_bag_vs_ref():
         np.testing.assert_array_equal(
             go.embedding_bag_byte_rowwise_offsets_f32(table, w, idx, o, end),
             ref.embedding_bag_byte_rowwise_offsets_f32(table, w, idx, o, end))
+
+
+def test_glue_ops_vs_ref():
+    rng = np.random.default_rng(77)
+    a = rng.integers(-128, 128, (2, 5, 6, 9)).astype(np.int8)
+    b = rng.integers(-128, 128, a.shape).astype(np.int8)
+    for _ in range(6):
+        ls, rs, ds = rng.uniform(0.001, 0.5, 3).astype(np.float32)
+        lo, ro, do = (int(v) for v in rng.integers(-128, 128, 3))
+        lp = go.quantize_scale_offset_32to8(float(ls / ds), 0)[:3]
+        rp = go.quantize_scale_offset_32to8(float(rs / ds), 0)[:3]
+        np.testing.assert_array_equal(go.add_i8(a, b, do, lo, ro, lp, rp).ravel(),
+                                      ref.add_i8(a, b, do, lo, ro, lp, rp))
+        np.testing.assert_array_equal(go.relu_i8(a, lo, do, lp).ravel(),
+                                      ref.relu_i8(a, lo, do, lp))
+    x = rng.integers(-128, 128, (2, 10, 7, 12)).astype(np.int8)
+    for k, st, pd in [((3, 3), (2, 2), (1, 1, 1, 1)), ((2, 2), (2, 2), (0, 0, 0, 0)),
+                      ((10, 7), (1, 1), (0, 0, 0, 0)), ((4, 3), (3, 2), (3, 2, 3, 2)),
+                      ((1, 1), (1, 1), (0, 0, 0, 0))]:
+        np.testing.assert_array_equal(go.max_pool_i8(x, k, st, pd, 11),
+                                      ref.max_pool_i8(x, k, st, pd, 11))
+        for cip in (0, 1):
+            op = go.quantize_scale_offset_32to8(float(rng.uniform(0.01, 2.0)), 0)[:3]
+            np.testing.assert_array_equal(go.avg_pool_i8(x, k, st, pd, cip, -3, 8, op),
+                                          ref.avg_pool_i8(x, k, st, pd, cip, -3, 8, op))
+    z = rng.normal(0, 4, (7, 333)).astype(np.float32)
+    np.testing.assert_array_equal(go.softmax_f32(z), ref.softmax_f32(z))

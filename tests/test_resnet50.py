@@ -1,0 +1,75 @@
+"""The int8 ResNet-50 harness: the description builds and compiles on the CPU;
+on the GPU the whole network, run through MI355XDeviceManager, gives the same
+int8 logits as the oracle executing the same quantized graph instruction by
+instruction (bit-exact), and the same fp32 probabilities within 1e-5."""
+import numpy as np
+import pytest
+
+from glow_amd import host as H
+from glow_amd.harness import net as netlib
+from glow_amd.harness import resnet50
+from tests import oracle_exec
+
+SMALL = ((16, 2, 1), (32, 1, 2))     # two stages are enough to cover every block shape
+
+
+def _small(batch=2, size=32, classes=10):
+    return resnet50.make(batch=batch, size=size, profile_images=4, seed=3, layers=SMALL,
+                         classes=classes)
+
+
+def test_structure_of_the_full_network():
+    steps = resnet50.build_fp32(0)
+    convs = [s for s in steps if s[0] == "conv"]
+    assert len(convs) == 53                      # 1 stem + 16 blocks x 3 + 4 shortcuts
+    assert sum(1 for s in steps if s[0] == "add") == 16
+    assert steps[-1][3][0].shape == (1000, 2048)
+
+
+def test_small_network_compiles_and_fuses():
+    net = _small()
+    m, f = netlib.to_module(net)
+    m.compile(f)
+    rows = H.parse_listing(m.describe(f))
+    kernels = [r["kernel"] for r in rows if r["phase"] == "launch"]
+    assert kernels.count("mi355x_cwq_conv2d_i8") == 1 + 3 * 3 + 1   # stem, 3 blocks, 1 shortcut
+    assert kernels.count("mi355x_add_relu_i8") == 3 and "mi355x_add_i8" not in kernels
+    assert kernels[-1] == "mi355x_softmax_f32" and kernels[0] == "mi355x_quantize_i8"
+    # post-ReLU tensors use the unsigned range: offset -128
+    assert net.tensors["stem"].offset == -128
+    assert net.ops_count() > 0
+
+
+def test_oracle_executes_the_small_network():
+    net = _small(batch=1)
+    x = resnet50.synthetic_images(9, 1, 32)
+    v = oracle_exec.run(net, {"input": x})
+    assert v["prob"].shape == (1, 10)
+    np.testing.assert_allclose(v["prob"].sum(), 1.0, rtol=1e-5)
+    assert len(np.unique(v["logits_q"])) > 1
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fuse", [True, False])
+def test_device_matches_oracle(fuse):
+    net = resnet50.make(batch=2, size=64, profile_images=4, seed=5,
+                        layers=((64, 2, 1), (128, 2, 2), (256, 1, 2)), classes=100)
+    m, f = netlib.to_module(net)
+    m.compile(f, fuse_add_relu=fuse)
+    dm = H.DeviceManager().init()
+    try:
+        dm.add_network(m)
+        x = resnet50.synthetic_images(11, 2, 64)
+        logits = np.zeros((2, 100), np.int8)
+        prob = np.zeros((2, 100), np.float32)
+        dm.run("main", {"input": x, "logits_q": logits, "prob": prob})
+        want = oracle_exec.run(net, {"input": x})
+        np.testing.assert_array_equal(logits, want["logits_q"])
+        np.testing.assert_allclose(prob, want["prob"], rtol=1e-5, atol=1e-30)
+        # a second batch through the same resident network
+        x2 = resnet50.synthetic_images(12, 2, 64)
+        dm.run("main", {"input": x2, "logits_q": logits, "prob": prob})
+        np.testing.assert_array_equal(logits, oracle_exec.run(net, {"input": x2})["logits_q"])
+        assert dm.time_function("main", 3) > 0
+    finally:
+        dm.stop()
