@@ -50,12 +50,14 @@ def parse():
                     help="bags per step (4096 is the headline configuration)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0,
                     help="wall-clock budget of the CPU baseline leg")
+    ap.add_argument("--resnet-batch", type=int, default=64)
+    ap.add_argument("--resnet-profile-images", type=int, default=100)
     ap.add_argument("--no-extra", action="store_true",
                     help="headline workload only")
     ap.add_argument("--only", default="",
                     help="run a single extra kernel (profiling aid): "
                          "slws|fc_large|fc_c1|conv_c3|quantize|dequantize|"
-                         "rescale|copy")
+                         "rescale|copy|resnet50")
     return ap.parse_args()
 
 
@@ -305,6 +307,47 @@ def bench_elementwise(capi, which, steps, warmup):
                               traffic=None))
 
 
+def bench_resnet50(args):
+    """Int8 ResNet-50 at batch 64, 224x224 through MI355XDeviceManager:
+    images/s of the resident network replayed on device-resident input
+    (device time), and of whole requests including the fp32 input upload and
+    the result download."""
+    from glow_amd import host as H
+    from glow_amd.harness import net as netlib
+    from glow_amd.harness import resnet50
+    batch, size = args.resnet_batch, 224
+    t0 = time.perf_counter()
+    net = resnet50.make(batch=batch, size=size, profile_images=args.resnet_profile_images)
+    t_build = time.perf_counter() - t0
+    m, f = netlib.to_module(net)
+    m.compile(f)
+    dm = H.DeviceManager().init()
+    try:
+        dm.add_network(m)
+        x = resnet50.synthetic_images(77, batch, size)
+        prob = np.zeros((batch, 1000), np.float32)
+        logits = np.zeros((batch, 1000), np.int8)
+        dm.run("main", {"input": x, "prob": prob, "logits_q": logits})
+        reps = max(3, args.steps // 10)
+        ms = dm.time_function("main", reps)
+        t1 = time.perf_counter()
+        for _ in range(3):
+            dm.run("main", {"input": x, "prob": prob, "logits_q": logits})
+        e2e = (time.perf_counter() - t1) / 3
+    finally:
+        dm.stop()
+    ops = net.ops_count()
+    return dict(workload=f"int8 ResNet-50, batch {batch}, {size}x{size}x3, channelwise-quantized "
+                         f"convolutions, rowwise-quantized FC, fp32 softmax; "
+                         f"{args.resnet_profile_images} profiling images",
+                images_per_s=batch / (ms * 1e-3), ms_per_batch=ms,
+                images_per_s_with_host_copies=batch / e2e,
+                tops=ops / (ms * 1e-3) / 1e12, gop_per_image=ops / batch / 1e9,
+                launches_per_batch=len([r for r in H.parse_listing(m.describe(f))
+                                        if r["phase"] == "launch"]),
+                prob_row_sum=float(prob[0].sum()), host_build_seconds=t_build)
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -315,6 +358,10 @@ def main():
 
     from glow_amd import capi
     from glow_amd import workloads as cases
+
+    if args.only == "resnet50":
+        print(json.dumps(bench_resnet50(args)))
+        return
 
     capi.init(0)
     info = capi.device_info()
@@ -358,6 +405,7 @@ def main():
         extra["cwq_conv_c3"] = bench_conv(capi, cases, args.steps, args.warmup)
         for w in ("quantize", "dequantize", "rescale"):
             extra[w] = bench_elementwise(capi, w, st, wu)
+        extra["resnet50_int8"] = bench_resnet50(args)
 
     out = {
         "metric": "FusedRowwiseQuantizedSLWS algorithmic GB/s (1 GPU)",

@@ -22,7 +22,8 @@ EXPORTS = [
     "mi355x_last_error", "mi355x_num_devices", "mi355x_init",
     "mi355x_device_info", "mi355x_malloc", "mi355x_free", "mi355x_host_alloc",
     "mi355x_host_free", "mi355x_memcpy_h2d", "mi355x_memcpy_d2h",
-    "mi355x_memcpy_d2d", "mi355x_fill_u8", "mi355x_copy_u8", "mi355x_add_i8", "mi355x_add_relu_i8",
+    "mi355x_memcpy_d2d", "mi355x_fill_u8", "mi355x_copy_u8", "mi355x_gemm_tile_override",
+    "mi355x_cwq_conv2d_add_i8", "mi355x_add_i8", "mi355x_add_relu_i8",
     "mi355x_relu_i8", "mi355x_max_pool_i8", "mi355x_avg_pool_i8", "mi355x_softmax_f32", "mi355x_stream_create",
     "mi355x_stream_destroy", "mi355x_stream_sync", "mi355x_device_sync",
     "mi355x_event_create", "mi355x_event_destroy", "mi355x_event_record",
@@ -417,6 +418,36 @@ def launch_cwq_conv2d_i8(out, x, filt, bias, bias_is_i8, geom, out_offset,
         C.c_int(bool(f_offsets_all_zero)), _vp(f_row_sums), _vp(stream)))
 
 
+class FusedAdd(C.Structure):
+    """mi355x_fused_add: the ElementAdd (+ Relu) behind a convolution."""
+    _fields_ = [(n, C.c_int32) for n in (
+        "sum_offset", "residual_offset", "conv_pre", "conv_post", "conv_scale",
+        "residual_pre", "residual_post", "residual_scale", "relu", "dest_offset",
+        "dest_pre", "dest_post", "dest_scale")]
+
+
+def fused_add(sum_offset, residual_offset, convP, resP, relu=False, dest_offset=0,
+              destP=(0, 0, 1)):
+    return FusedAdd(sum_offset, residual_offset, *[int(v) for v in convP],
+                    *[int(v) for v in resP], int(bool(relu)), dest_offset,
+                    *[int(v) for v in destP])
+
+
+def launch_cwq_conv2d_add_i8(out, x, filt, bias, bias_is_i8, geom, conv_offset,
+                             in_offset, f_offsets, b_offsets, bias_pre, bias_post,
+                             bias_scale, out_pre, out_post, out_scale, act,
+                             act_args, f_offsets_all_zero, f_row_sums, residual,
+                             add, stream=None):
+    aa = (C.c_int32 * 3)(*(list(act_args) + [0, 0, 0])[:3])
+    check(lib().mi355x_cwq_conv2d_add_i8(
+        _vp(out), _vp(x), _vp(filt), _vp(bias), C.c_int(bias_is_i8),
+        C.byref(geom), _i32(conv_offset), _i32(in_offset), _vp(f_offsets),
+        _vp(b_offsets), _vp(bias_pre), _vp(bias_post), _vp(bias_scale),
+        _vp(out_pre), _vp(out_post), _vp(out_scale), _i32(act), aa,
+        C.c_int(bool(f_offsets_all_zero)), _vp(f_row_sums), _vp(residual),
+        C.byref(add), _vp(stream)))
+
+
 def launch_frwq_slws(dest, out_is_f16, data, data_rows, kind, weights,
                      weights_are_f16, indices, idx_is_64, num_indices, lengths,
                      segments, in_line, out_line, fp16_accum=False,
@@ -579,6 +610,26 @@ def cwq_conv2d_i8(x, filt, bias, geom, out_offset, in_offset, f_offsets,
     d_sums = _row_sums_dev(d_f, g.OC, filt.size // g.OC, precomputed_sums)
     launch_cwq_conv2d_i8(d_out, d_x, d_f, d_b, b8, g, out_offset, in_offset,
                          *vs, act, act_args, f_offsets_all_zero, d_sums)
+    return d_out.numpy()
+
+
+def cwq_conv2d_add_i8(x, filt, bias, geom, out_offset, in_offset, f_offsets,
+                      b_offsets, bias_pre, bias_post, bias_scale, out_pre, out_post,
+                      out_scale, act, act_args, residual, add):
+    """The convolution of cwq_conv2d_i8 followed by ElementAdd with `residual`
+    (and Relu when add.relu) in one kernel."""
+    g = _geom(geom)
+    x = np.ascontiguousarray(x, np.int8)
+    filt = np.ascontiguousarray(filt, np.int8)
+    residual = np.ascontiguousarray(residual, np.int8)
+    d_x, d_f, d_r = to_device(x), to_device(filt), to_device(residual)
+    d_b, b8 = _bias_dev(bias)
+    vs = [_dev_i32(v) for v in (f_offsets, b_offsets, bias_pre, bias_post,
+                                bias_scale, out_pre, out_post, out_scale)]
+    d_out = DeviceBuffer.empty((g.N, g.OH, g.OW, g.OC), np.int8)
+    d_sums = _row_sums_dev(d_f, g.OC, filt.size // g.OC, True)
+    launch_cwq_conv2d_add_i8(d_out, d_x, d_f, d_b, b8, g, out_offset, in_offset,
+                             *vs, act, act_args, not np.any(f_offsets), d_sums, d_r, add)
     return d_out.numpy()
 
 

@@ -113,6 +113,15 @@ static int conv_common(int8_t *out, const int8_t *in, const int8_t *filter,
   if (ep.act == MI355X_ACT_LEAKY_RELU)
     MI355X_REQUIRE(shift_ok(ep.a0) && shift_ok(ep.a1),
                    "leaky-relu pre/post shift outside [0, 31]");
+  if (ep.add.res) {
+    MI355X_REQUIRE(shift_ok(ep.add.own_pre) && shift_ok(ep.add.own_post) &&
+                       shift_ok(ep.add.res_pre) && shift_ok(ep.add.res_post) &&
+                       (!ep.add.relu || (shift_ok(ep.add.dest_pre) &&
+                                         shift_ok(ep.add.dest_post))),
+                   "fused add: pre/post shift outside [0, 31]");
+    MI355X_REQUIRE(!ep.add.relu || (ep.add.sum_off >= -128 && ep.add.sum_off <= 127),
+                   "fused add: sum offset outside the int8 range");
+  }
 
   ConvRows A;
   A.in = in;
@@ -189,6 +198,57 @@ int mi355x_cwq_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
   ep.out_off = out_offset;
   set_act(ep, act_type, act_args);
   ep.sum_b = filter_row_sums;
+  return conv_common(out, in, filter, geom, ep, !filter_offsets_all_zero,
+                     stream);
+}
+
+int mi355x_cwq_conv2d_add_i8(
+    int8_t *out, const int8_t *in, const int8_t *filter, const void *bias,
+    int bias_is_i8, const mi355x_conv_geom *geom, int32_t conv_offset,
+    int32_t in_offset, const int32_t *filter_offsets,
+    const int32_t *bias_offsets, const int32_t *bias_pre,
+    const int32_t *bias_post, const int32_t *bias_scale, const int32_t *out_pre,
+    const int32_t *out_post, const int32_t *out_scale, int32_t act_type,
+    const int32_t *act_args, int filter_offsets_all_zero,
+    const int32_t *filter_row_sums, const int8_t *residual,
+    const mi355x_fused_add *add, void *stream) {
+  MI355X_REQUIRE(bias && filter_offsets && bias_offsets && bias_pre &&
+                     bias_post && bias_scale && out_pre && out_post && out_scale,
+                 "NULL per-channel parameter vector");
+  MI355X_REQUIRE(act_args || (act_type != MI355X_ACT_CLIP &&
+                              act_type != MI355X_ACT_LEAKY_RELU),
+                 "act_args is NULL");
+  MI355X_REQUIRE(residual && add, "NULL residual or add parameters");
+  Epilogue ep{};
+  ep.bias = bias;
+  ep.bias_is_i8 = bias_is_i8;
+  ep.b_off = ColParam{bias_offsets, 0};
+  ep.bias_pre = ColParam{bias_pre, 0};
+  ep.bias_post = ColParam{bias_post, 0};
+  ep.bias_scale = ColParam{bias_scale, 0};
+  ep.w_off = ColParam{filter_offsets, 0};
+  ep.out_pre = ColParam{out_pre, 0};
+  ep.out_post = ColParam{out_post, 0};
+  ep.out_scale = ColParam{out_scale, 0};
+  ep.a_off = in_offset;
+  ep.out_off = conv_offset;
+  set_act(ep, act_type, act_args);
+  ep.sum_b = filter_row_sums;
+  ep.add.res = residual;
+  ep.add.sum_off = add->sum_offset;
+  ep.add.own_off = conv_offset;
+  ep.add.res_off = add->residual_offset;
+  ep.add.own_pre = add->conv_pre;
+  ep.add.own_post = add->conv_post;
+  ep.add.own_scale = add->conv_scale;
+  ep.add.res_pre = add->residual_pre;
+  ep.add.res_post = add->residual_post;
+  ep.add.res_scale = add->residual_scale;
+  ep.add.relu = add->relu;
+  ep.add.dest_off = add->dest_offset;
+  ep.add.dest_pre = add->dest_pre;
+  ep.add.dest_post = add->dest_post;
+  ep.add.dest_scale = add->dest_scale;
   return conv_common(out, in, filter, geom, ep, !filter_offsets_all_zero,
                      stream);
 }

@@ -8,6 +8,8 @@
 
 namespace mi355x {
 
+int g_tile_override = -1;
+
 // dst [cols x rows] = src [rows x cols]^T through a 64x64 LDS tile.
 __global__ __launch_bounds__(256) void transpose2d_i8_kernel(
     int8_t *__restrict__ dst, const int8_t *__restrict__ src, int rows,
@@ -83,6 +85,12 @@ static int fc_common(int8_t *out, const int8_t *in, const int8_t *w_nk,
 using namespace mi355x;
 
 extern "C" {
+
+int mi355x_gemm_tile_override(int tile) {
+  MI355X_REQUIRE(tile >= -1 && tile <= 3, "tile %d outside [-1, 3]", tile);
+  g_tile_override = tile;
+  return MI355X_OK;
+}
 
 int mi355x_transpose2d_i8(int8_t *dst, const int8_t *src, size_t rows,
                           size_t cols, void *stream) {

@@ -48,6 +48,43 @@ struct ColParam {
   __device__ __forceinline__ int32_t at(int n) const { return v ? v[n] : s; }
 };
 
+// A residual tensor added to the (already clipped) int8 result while the
+// output tile is written, optionally followed by Relu: what ElementAdd and Relu
+// instructions behind a convolution compute, without the round trip through
+// memory. Same arithmetic as the standalone kernels.
+struct FusedAdd {
+  const int8_t *res;    // [M x ldc] like the output, or NULL
+  int32_t sum_off, own_off, res_off;
+  int32_t own_pre, own_post, own_scale;   // rescale of this kernel's result
+  int32_t res_pre, res_post, res_scale;   // rescale of the residual
+  int32_t relu;                           // apply the Relu stage below
+  int32_t dest_off, dest_pre, dest_post, dest_scale;
+};
+
+__device__ __forceinline__ int32_t fused_add_one(int32_t own, int32_t res,
+                                                 const FusedAdd &f) {
+  const int32_t a = scale_i32(own - f.own_off, f.own_pre, f.own_post, f.own_scale, 0);
+  const int32_t b = scale_i32(res - f.res_off, f.res_pre, f.res_post, f.res_scale, 0);
+  int32_t v = clip_i8((int32_t)((uint32_t)a + (uint32_t)b + (uint32_t)f.sum_off));
+  if (f.relu) {
+    const int32_t so = (int32_t)(int8_t)f.sum_off;
+    v = max(v, so);
+    v = clip_i8(scale_i32(v - so, f.dest_pre, f.dest_post, f.dest_scale, f.dest_off));
+  }
+  return v;
+}
+
+__device__ __forceinline__ uint32_t fused_add_word(uint32_t own, uint32_t res,
+                                                   const FusedAdd &f) {
+  uint32_t o = 0;
+#pragma unroll
+  for (int b = 0; b < 4; b++)
+    o |= (uint32_t)(fused_add_one((int32_t)(int8_t)(own >> (8 * b)),
+                                  (int32_t)(int8_t)(res >> (8 * b)), f) & 0xff)
+         << (8 * b);
+  return o;
+}
+
 struct Epilogue {
   int8_t *out;
   long long ldc;        // elements between output rows
@@ -59,6 +96,7 @@ struct Epilogue {
   int32_t a_off;        // offset of the A operand (activations)
   int32_t out_off;
   int32_t act, a0, a1, a2;
+  FusedAdd add;         // add.res == NULL: none
 };
 
 // Row-major [rows x K] operand (activations, or weights with K contiguous).
@@ -207,17 +245,29 @@ __device__ __forceinline__ void gemm_epilogue_impl(
   int8_t *obase = ep.out + (long long)m0 * ep.ldc + n_base + n0;
   const bool vec_ok = (cols_here % 16 == 0) && (ep.ldc % 16 == 0) &&
                       ((((uintptr_t)obase) & 15) == 0);
-  if (vec_ok) {
+  const int8_t *rbase =
+      ep.add.res ? ep.add.res + (long long)m0 * ep.ldc + n_base + n0 : nullptr;
+  if (vec_ok && (!rbase || ((((uintptr_t)rbase) & 15) == 0))) {
     const int segs = cols_here / 16;
     for (int c = tid; c < rows_here * segs; c += THREADS) {
       const int r = c / segs, s = c - r * segs;
-      *reinterpret_cast<int4 *>(obase + (long long)r * ep.ldc + s * 16) =
-          *reinterpret_cast<const int4 *>(s_out + r * OUT_STRIDE + s * 16);
+      int4 v = *reinterpret_cast<const int4 *>(s_out + r * OUT_STRIDE + s * 16);
+      if (rbase) {
+        const int4 q =
+            *reinterpret_cast<const int4 *>(rbase + (long long)r * ep.ldc + s * 16);
+        v.x = (int)fused_add_word((uint32_t)v.x, (uint32_t)q.x, ep.add);
+        v.y = (int)fused_add_word((uint32_t)v.y, (uint32_t)q.y, ep.add);
+        v.z = (int)fused_add_word((uint32_t)v.z, (uint32_t)q.z, ep.add);
+        v.w = (int)fused_add_word((uint32_t)v.w, (uint32_t)q.w, ep.add);
+      }
+      *reinterpret_cast<int4 *>(obase + (long long)r * ep.ldc + s * 16) = v;
     }
   } else {
     for (int c = tid; c < rows_here * cols_here; c += THREADS) {
       const int r = c / cols_here, s = c - r * cols_here;
-      obase[(long long)r * ep.ldc + s] = s_out[r * OUT_STRIDE + s];
+      int32_t v = s_out[r * OUT_STRIDE + s];
+      if (rbase) v = fused_add_one(v, rbase[(long long)r * ep.ldc + s], ep.add);
+      obase[(long long)r * ep.ldc + s] = (int8_t)v;
     }
   }
 }
@@ -672,15 +722,26 @@ static int gemm_dma_launch(const ARows &A, const DenseRows &B,
 // 128x128, which halves LDS traffic per MFMA), smaller tiles when the grid
 // would otherwise not fill 256 CUs.
 enum class Tile { T256, T128, T128x64, T64 };
+// Tuning aid: a value in [0, 3] forces that tile for every following launch.
+extern int g_tile_override;
 static Tile pick_tile(const GemmShape &g, size_t lds_256) {
   auto tiles = [&](int bm, int bn) {
     return (long long)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * g.groups;
   };
-  if (tiles(256, 256) >= 256 && g.N >= 192 && lds_256 <= lds_limit())
+  if (g_tile_override >= 0 && g_tile_override <= 3 &&
+      (g_tile_override != 0 || lds_256 <= lds_limit()))
+    return (Tile)g_tile_override;
+  // Measured on the convolution shapes of ResNet-50 and on large FCs: the
+  // 256x256 tile (one wave per SIMD) only pays off when the K loop is long
+  // enough to amortise its prologue and epilogue; short K loops want many
+  // small resident workgroups; few-row problems want 64x64 to fill the chip.
+  if (tiles(256, 256) >= 256 && g.N >= 256 && g.K >= 1024 &&
+      lds_256 <= lds_limit())
     return Tile::T256;
-  if (tiles(128, 128) >= 256 && g.N >= 96) return Tile::T128;
-  if (tiles(128, 64) >= 256 || g.M >= 1024) return Tile::T128x64;
-  return Tile::T64;
+  if (tiles(128, 128) >= 256 && g.N >= 128 && g.K >= 512) return Tile::T128;
+  if (tiles(128, 64) >= 256) return Tile::T128x64;
+  if (tiles(64, 64) >= 256 || g.M < 1024) return Tile::T64;
+  return Tile::T128x64;
 }
 
 template <bool SA, bool SB, class ARows>

@@ -118,7 +118,28 @@ public:
       case Kind::RowwiseQuantizedFullyConnected: MI355X_RETURN_IF_ERR(rwqfc(I, out)); break;
       case Kind::MatMul: MI355X_RETURN_IF_ERR(matmul(I, out)); break;
       case Kind::Convolution: MI355X_RETURN_IF_ERR(conv(I, out, false)); break;
-      case Kind::ChannelwiseQuantizedConvolution: MI355X_RETURN_IF_ERR(conv(I, out, true)); break;
+      case Kind::ChannelwiseQuantizedConvolution: {
+        // conv -> ElementAdd(conv, residual) [-> Relu] with no other reader of
+        // the intermediate tensors: one kernel
+        const Instruction *addI = nullptr, *reluI = nullptr;
+        if (opts_.fuseConvAdd && at + 1 < insts_.size() && insts_[at + 1].kind == Kind::ElementAdd) {
+          const Instruction &A = insts_[at + 1];
+          const int cd = I.operands[0];
+          const bool lhs = A.operands[1] == cd, rhs = A.operands[2] == cd;
+          if ((lhs != rhs) && M_.value(cd).category == SymbolCategory::Activation &&
+              readers(cd) == 1 && M_.value(cd).type.dims == M_.value(A.operands[0]).type.dims) {
+            addI = &A;
+            if (opts_.fuseAddRelu && at + 2 < insts_.size() && insts_[at + 2].kind == Kind::Relu &&
+                insts_[at + 2].operands[1] == A.operands[0] &&
+                M_.value(A.operands[0]).category == SymbolCategory::Activation &&
+                readers(A.operands[0]) == 1)
+              reluI = &insts_[at + 2];
+          }
+        }
+        MI355X_RETURN_IF_ERR(conv(I, out, true, addI, reluI));
+        at += (addI ? 1 : 0) + (reluI ? 1 : 0);
+        break;
+      }
       case Kind::FusedRowwiseQuantizedSparseLengthsWeightedSum:
         MI355X_RETURN_IF_ERR(slws(I, out, true)); break;
       case Kind::FusedRowwiseQuantizedSparseLengthsSum:
@@ -505,7 +526,8 @@ private:
     return Error::success();
   }
 
-  Error conv(const Instruction &I, MI355XFunction &out, bool channelwise) {
+  Error conv(const Instruction &I, MI355XFunction &out, bool channelwise,
+             const Instruction *addI = nullptr, const Instruction *reluI = nullptr) {
     Operand d = op(I, 0), s = op(I, 1), f = op(I, 2), bi = op(I, 3);
     CHECK_OP((int)I.iattrs.size() == ConvAttrs::kCount, "expects %d integer attributes",
              ConvAttrs::kCount);
@@ -610,6 +632,61 @@ private:
     }
     const size_t o0 = gen_.addI32(bpre), o1 = gen_.addI32(bpost), o2 = gen_.addI32(bscale),
                  o3 = gen_.addI32(opre), o4 = gen_.addI32(opost), o5 = gen_.addI32(oscale);
+    if (addI) {
+      const Instruction &A = *addI;
+      const bool convIsLhs = A.operands[1] == I.operands[0];
+      Operand sum = op(A, 0), res = op(A, convIsLhs ? 2 : 1);
+      {
+        const Instruction &I = A; // for the message
+        CHECK_OP(sum.ty().kind == ElemKind::Int8QTy && res.ty().kind == ElemKind::Int8QTy &&
+                     res.ty().size() == sum.ty().size(),
+                 "needs i8 operands of one size");
+      }
+      mi355x_fused_add fa;
+      const S32To8 cp = s32to8(d.ty().scale / sum.ty().scale), rp = s32to8(res.ty().scale / sum.ty().scale);
+      fa.sum_offset = sum.ty().offset;
+      fa.residual_offset = res.ty().offset;
+      fa.conv_pre = cp.pre; fa.conv_post = cp.post; fa.conv_scale = cp.scale;
+      fa.residual_pre = rp.pre; fa.residual_post = rp.post; fa.residual_scale = rp.scale;
+      fa.relu = reluI ? 1 : 0;
+      fa.dest_offset = 0; fa.dest_pre = 0; fa.dest_post = 0; fa.dest_scale = 1;
+      Operand fin = sum;
+      std::string name = I.name + "+" + A.name;
+      if (reluI) {
+        fin = op(*reluI, 0);
+        {
+          const Instruction &I = *reluI;
+          CHECK_OP(fin.ty().kind == ElemKind::Int8QTy && fin.ty().size() == sum.ty().size(),
+                   "needs an i8 result of the same size");
+        }
+        const S32To8 dp = s32to8(sum.ty().scale / fin.ty().scale);
+        fa.dest_offset = fin.ty().offset;
+        fa.dest_pre = dp.pre; fa.dest_post = dp.post; fa.dest_scale = dp.scale;
+        name += "+" + reluI->name;
+      }
+      out.launches.push_back(
+          {"mi355x_cwq_conv2d_add_i8", name,
+           geomStr + kv("out_offset", oo) + kv("in_offset", io) + kv("act", act) +
+               vecStr("act_args", actArgs) + kv("bias_is_i8", bias8) +
+               kv("filter_offsets_all_zero", allZero) + kv("row_sums", sums) +
+               kv("sum_offset", fa.sum_offset) + kv("residual_offset", fa.residual_offset) +
+               kv("conv_pre", fa.conv_pre) + kv("conv_post", fa.conv_post) +
+               kv("conv_scale", fa.conv_scale) + kv("residual_pre", fa.residual_pre) +
+               kv("residual_post", fa.residual_post) + kv("residual_scale", fa.residual_scale) +
+               kv("relu", fa.relu) + kv("relu_dest_offset", fa.dest_offset) +
+               kv("relu_pre", fa.dest_pre) + kv("relu_post", fa.dest_post) +
+               kv("relu_scale", fa.dest_scale),
+           [=](const DeviceBindings &b) {
+             auto gp = [&](size_t o) { return (const int32_t *)(b.generated + o); };
+             return mi355x_cwq_conv2d_add_i8(
+                 (int8_t *)fin.ptr(b), (const int8_t *)s.ptr(b), (const int8_t *)f.ptr(b), bi.ptr(b),
+                 bias8, &g, oo, io, (const int32_t *)fo.ptr(b), (const int32_t *)bo.ptr(b), gp(o0),
+                 gp(o1), gp(o2), gp(o3), gp(o4), gp(o5), act, actArgs.data(), allZero ? 1 : 0,
+                 sums ? (const int32_t *)sumPtr(b) : nullptr, (const int8_t *)res.ptr(b), &fa,
+                 b.stream);
+           }});
+      return Error::success();
+    }
     out.launches.push_back(
         {"mi355x_cwq_conv2d_i8", I.name,
          geomStr + kv("out_offset", oo) + kv("in_offset", io) + kv("act", act) +

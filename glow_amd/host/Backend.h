@@ -118,6 +118,7 @@ private:
 struct BackendOptions {
   bool precomputeWeightRowSums = true; // form sum_k W[n][k] once at load time
   bool fuseAddRelu = true;             // ElementAdd + Relu of its result in one pass
+  bool fuseConvAdd = true;             // convolution + ElementAdd (+ Relu) in one kernel
 };
 
 class MI355XBackend {

@@ -280,6 +280,12 @@ int mi355x_matmul_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs_kn,
                      int32_t rhs_offset, int32_t out_pre, int32_t out_post,
                      int32_t out_scale, void *stream);
 
+/* Tuning aid (no counterpart in the reference): forces the workgroup tile of
+ * every following matrix-core launch of this process: 0 = 256x256, 1 = 128x128,
+ * 2 = 128x64, 3 = 64x64; -1 = chosen from the problem shape (the default).
+ * Results do not depend on the tile. */
+int mi355x_gemm_tile_override(int tile);
+
 /* libjit_transpose_i8 for a 2-D tensor: dst [cols x rows] = src [rows x cols]^T */
 int mi355x_transpose2d_i8(int8_t *dst, const int8_t *src, size_t rows,
                           size_t cols, void *stream);
@@ -320,6 +326,32 @@ int mi355x_cwq_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
                          const int32_t *act_args,
                          int filter_offsets_all_zero,
                          const int32_t *filter_row_sums, void *stream);
+
+/* ChannelwiseQuantizedConvolution whose result feeds an ElementAdd with a
+ * residual tensor of the output's shape, optionally followed by Relu: the
+ * three instructions in one kernel. The convolution result is clipped to int8
+ * at `conv_offset` exactly as mi355x_cwq_conv2d_i8 would store it; then
+ * libjit_element_add_kernel_i8 (libjit.cpp:1593-1603) with that value and
+ * residual[i], and, when add->relu, libjit_element_relu_i8 (libjit.cpp:1851-1858)
+ * are applied while the tile is written. `out` receives the final tensor. */
+typedef struct {
+  int32_t sum_offset;                              /* ElementAdd's destination offset */
+  int32_t residual_offset;
+  int32_t conv_pre, conv_post, conv_scale;         /* convScale / sumScale */
+  int32_t residual_pre, residual_post, residual_scale; /* residualScale / sumScale */
+  int32_t relu;                                    /* 0: store the sum */
+  int32_t dest_offset, dest_pre, dest_post, dest_scale; /* Relu: sumScale / destScale */
+} mi355x_fused_add;
+int mi355x_cwq_conv2d_add_i8(
+    int8_t *out, const int8_t *in, const int8_t *filter, const void *bias,
+    int bias_is_i8, const mi355x_conv_geom *geom, int32_t conv_offset,
+    int32_t in_offset, const int32_t *filter_offsets,
+    const int32_t *bias_offsets, const int32_t *bias_pre,
+    const int32_t *bias_post, const int32_t *bias_scale, const int32_t *out_pre,
+    const int32_t *out_post, const int32_t *out_scale, int32_t act_type,
+    const int32_t *act_args, int filter_offsets_all_zero,
+    const int32_t *filter_row_sums, const int8_t *residual,
+    const mi355x_fused_add *add, void *stream);
 
 /* libjit_conv2d_i8_i32 / _i8_i8 (libjit_conv.cpp:49-147, 496-528). */
 int mi355x_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,

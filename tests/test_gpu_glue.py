@@ -111,3 +111,26 @@ def test_argument_errors():
         capi.check(capi.lib().mi355x_max_pool_i8(
             capi._vp(d), capi._vp(d), *[capi._sz(v) for v in (1, 4, 4, 4, 9, 9, 2, 2, 1, 1, 0, 0)],
             capi._i32(0), capi._vp(None)))
+
+
+@pytest.mark.parametrize("relu", [False, True])
+@pytest.mark.parametrize("shape", [(2, 14, 14, 64, 256, 1), (1, 9, 9, 16, 40, 3), (3, 7, 7, 32, 64, 3)])
+def test_conv_with_fused_residual_add(shape, relu):
+    """Convolution + ElementAdd (+ Relu) in one kernel equals the separate
+    instructions executed by the oracle."""
+    from tests import cases
+    N, Hh, W, IC, OC, k = shape
+    pad = 1 if k == 3 else 0
+    c = cases.cwq_conv_case(91, N, Hh, W, IC, OC, kernel=(k, k), pads=(pad,) * 4,
+                            act=cases._w.ACT_NONE, in_offset=-5, out_offset=6)
+    conv = go.cwq_conv2d_i8(*cases.cwq_conv_args(c))
+    rng = np.random.default_rng(92)
+    res = rng.integers(-128, 128, conv.shape).astype(np.int8)
+    cs, rs, ss, ds = np.float32(c["out_scale_f"]), np.float32(0.09), np.float32(0.13), np.float32(0.2)
+    cp, rp, dp = _p(cs / ss), _p(rs / ss), _p(ss / ds)
+    want = go.add_i8(conv, res, 11, c["out_offset"], -20, cp, rp)
+    if relu:
+        want = go.relu_i8(want, 11, -128, dp)
+    add = capi.fused_add(11, -20, cp, rp, relu, -128, dp)
+    got = capi.cwq_conv2d_add_i8(*cases.cwq_conv_args(c), res, add)
+    np.testing.assert_array_equal(got, want)

@@ -32,8 +32,15 @@ def test_small_network_compiles_and_fuses():
     m.compile(f)
     rows = H.parse_listing(m.describe(f))
     kernels = [r["kernel"] for r in rows if r["phase"] == "launch"]
-    assert kernels.count("mi355x_cwq_conv2d_i8") == 1 + 3 * 3 + 1   # stem, 3 blocks, 1 shortcut
-    assert kernels.count("mi355x_add_relu_i8") == 3 and "mi355x_add_i8" not in kernels
+    # stem, 3 blocks x 3, 1 shortcut; the last convolution of each block takes
+    # the residual add and the Relu with it
+    assert kernels.count("mi355x_cwq_conv2d_i8") == 1 + 3 * 2 + 1
+    assert kernels.count("mi355x_cwq_conv2d_add_i8") == 3
+    assert "mi355x_add_relu_i8" not in kernels and "mi355x_add_i8" not in kernels
+    m2, f2 = netlib.to_module(net)
+    m2.compile(f2, fuse_conv_add=False)
+    k2 = [r["kernel"] for r in H.parse_listing(m2.describe(f2)) if r["phase"] == "launch"]
+    assert k2.count("mi355x_add_relu_i8") == 3 and k2.count("mi355x_cwq_conv2d_i8") == 11
     assert kernels[-1] == "mi355x_softmax_f32" and kernels[0] == "mi355x_quantize_i8"
     # post-ReLU tensors use the unsigned range: offset -128
     assert net.tensors["stem"].offset == -128
@@ -50,12 +57,12 @@ def test_oracle_executes_the_small_network():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("fuse", [True, False])
+@pytest.mark.parametrize("fuse", [(True, True), (True, False), (False, False)])
 def test_device_matches_oracle(fuse):
     net = resnet50.make(batch=2, size=64, profile_images=4, seed=5,
                         layers=((64, 2, 1), (128, 2, 2), (256, 1, 2)), classes=100)
     m, f = netlib.to_module(net)
-    m.compile(f, fuse_add_relu=fuse)
+    m.compile(f, fuse_conv_add=fuse[0], fuse_add_relu=fuse[1])
     dm = H.DeviceManager().init()
     try:
         dm.add_network(m)
