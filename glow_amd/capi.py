@@ -24,7 +24,9 @@ EXPORTS = [
     "mi355x_host_free", "mi355x_memcpy_h2d", "mi355x_memcpy_d2h",
     "mi355x_memcpy_d2d", "mi355x_fill_u8", "mi355x_copy_u8", "mi355x_gemm_tile_override",
     "mi355x_cwq_conv2d_add_i8", "mi355x_add_i8", "mi355x_add_relu_i8",
-    "mi355x_relu_i8", "mi355x_max_pool_i8", "mi355x_avg_pool_i8", "mi355x_softmax_f32", "mi355x_stream_create",
+    "mi355x_relu_i8", "mi355x_convert_f16_to_f32", "mi355x_insert_rows",
+    "mi355x_batch_transpose_i8", "mi355x_gather", "mi355x_batch_matmul_i8", "mi355x_sigmoid_f32",
+    "mi355x_max_pool_i8", "mi355x_avg_pool_i8", "mi355x_softmax_f32", "mi355x_stream_create",
     "mi355x_stream_destroy", "mi355x_stream_sync", "mi355x_device_sync",
     "mi355x_event_create", "mi355x_event_destroy", "mi355x_event_record",
     "mi355x_event_sync", "mi355x_event_elapsed_ms", "mi355x_arena_create",
@@ -801,4 +803,79 @@ def softmax_f32(x):
     out = DeviceBuffer.empty(x.shape, np.float32)
     check(lib().mi355x_softmax_f32(_vp(out), _vp(dx), _sz(x.shape[0]), _sz(x.shape[1]),
                                    _vp(None)))
+    return out.numpy()
+
+
+# ---- data movement and the small operators of ranking models -------------------
+# (device buffers are bound to names so they outlive the launch)
+
+def convert_f16_to_f32(x):
+    x = np.ascontiguousarray(x, np.float16)
+    dx = to_device(x)
+    out = DeviceBuffer.empty(x.shape, np.float32)
+    check(lib().mi355x_convert_f16_to_f32(_vp(out), _vp(dx), _sz(x.size), _vp(None)))
+    return out.numpy()
+
+
+def concat_rows(parts):
+    """Concat of 2-D arrays of one dtype along dimension 1 through InsertTensor."""
+    parts = [np.ascontiguousarray(p) for p in parts]
+    rows, item = parts[0].shape[0], parts[0].dtype.itemsize
+    width = sum(p.shape[1] for p in parts)
+    out = DeviceBuffer.empty((rows, width), parts[0].dtype)
+    held, off = [], 0
+    for p in parts:
+        dp = to_device(p)
+        held.append(dp)
+        check(lib().mi355x_insert_rows(_vp(out), _vp(dp), _sz(rows), _sz(p.shape[1] * item),
+                                       _sz(width * item), _sz(off * item), _vp(None)))
+        off += p.shape[1]
+    return out.numpy()
+
+
+def batch_transpose_i8(x):
+    x = np.ascontiguousarray(x, np.int8)
+    b, r, c = x.shape
+    dx = to_device(x)
+    out = DeviceBuffer.empty((b, c, r), np.int8)
+    check(lib().mi355x_batch_transpose_i8(_vp(out), _vp(dx), _sz(b), _sz(r), _sz(c), _vp(None)))
+    return out.numpy()
+
+
+def gather(data, indices, batch_dims=0):
+    """Gather along the first non-batch dimension (batch_dims 0 or 1)."""
+    data = np.ascontiguousarray(data)
+    indices = np.ascontiguousarray(indices)
+    assert indices.dtype in (np.int32, np.int64) and indices.ndim == 1
+    samples = data.shape[0] if batch_dims else 1
+    inner = data.shape[batch_dims + 1:]
+    slice_bytes = int(np.prod(inner, dtype=np.int64)) * data.dtype.itemsize
+    sample_bytes = data.shape[batch_dims] * slice_bytes
+    shape = (data.shape[:batch_dims]) + (indices.size,) + inner
+    dd, di = to_device(data), to_device(indices)
+    out = DeviceBuffer.empty(shape, data.dtype)
+    check(lib().mi355x_gather(_vp(out), _vp(dd), _vp(di), C.c_int(indices.dtype == np.int64),
+                              _sz(indices.size), _sz(slice_bytes), _sz(samples),
+                              _sz(sample_bytes), _vp(None)))
+    return out.numpy()
+
+
+def batch_matmul_i8(lhs, rhs, out_offset, lhs_offset, rhs_offset, outP):
+    lhs = np.ascontiguousarray(lhs, np.int8)
+    rhs = np.ascontiguousarray(rhs, np.int8)
+    b, m, k = lhs.shape
+    n = rhs.shape[2]
+    dl, dr = to_device(lhs), to_device(rhs)
+    out = DeviceBuffer.empty((b, m, n), np.int8)
+    check(lib().mi355x_batch_matmul_i8(_vp(out), _vp(dl), _vp(dr), _sz(b), _sz(m), _sz(k),
+                                       _sz(n), _i32(out_offset), _i32(lhs_offset),
+                                       _i32(rhs_offset), *_i32s(outP), _vp(None)))
+    return out.numpy()
+
+
+def sigmoid_f32(x):
+    x = np.ascontiguousarray(x, np.float32)
+    dx = to_device(x)
+    out = DeviceBuffer.empty(x.shape, np.float32)
+    check(lib().mi355x_sigmoid_f32(_vp(out), _vp(dx), _sz(x.size), _vp(None)))
     return out.numpy()

@@ -7,6 +7,8 @@
 // the CPU code.
 #include "common.h"
 
+#include <hip/hip_fp16.h>
+
 #pragma clang fp contract(off)
 #include "requant.h"
 
@@ -248,6 +250,102 @@ __global__ __launch_bounds__(kGlueThreads) void softmax_f32_kernel(
   for (int i = threadIdx.x; i < cols; i += kGlueThreads) y[i] = __fdiv_rn(y[i], sum);
 }
 
+// ---- data movement and the small operators of ranking models ----------------
+
+__global__ __launch_bounds__(kGlueThreads) void convert_f16_f32_kernel(
+    float *__restrict__ dst, const __half *__restrict__ src, size_t n) {
+  const size_t stride = (size_t)gridDim.x * kGlueThreads;
+  for (size_t i = (size_t)blockIdx.x * kGlueThreads + threadIdx.x; i < n; i += stride)
+    dst[i] = __half2float(src[i]);
+}
+
+// dst[r][off + b] = src[r][b]: rows of row_bytes bytes into rows of a wider tensor
+__global__ __launch_bounds__(kGlueThreads) void insert_rows_kernel(
+    uint8_t *__restrict__ dst, const uint8_t *__restrict__ src, long long rows,
+    long long row_bytes, long long dst_stride, long long dst_off, int unit) {
+  const long long per_row = row_bytes / unit;
+  const long long total = rows * per_row;
+  const long long stride = (long long)gridDim.x * kGlueThreads;
+  for (long long i = (long long)blockIdx.x * kGlueThreads + threadIdx.x; i < total; i += stride) {
+    const long long r = i / per_row, c = (i - r * per_row) * unit;
+    const uint8_t *s = src + r * row_bytes + c;
+    uint8_t *d = dst + r * dst_stride + dst_off + c;
+    if (unit == 16) *reinterpret_cast<uint4 *>(d) = *reinterpret_cast<const uint4 *>(s);
+    else if (unit == 4) *reinterpret_cast<uint32_t *>(d) = *reinterpret_cast<const uint32_t *>(s);
+    else *d = *s;
+  }
+}
+
+// dst [B][cols][rows] = src [B][rows][cols]
+__global__ __launch_bounds__(kGlueThreads) void batch_transpose_i8_kernel(
+    int8_t *__restrict__ dst, const int8_t *__restrict__ src, long long batch, int rows,
+    int cols) {
+  const long long per = (long long)rows * cols;
+  const long long total = batch * per;
+  const long long stride = (long long)gridDim.x * kGlueThreads;
+  for (long long i = (long long)blockIdx.x * kGlueThreads + threadIdx.x; i < total; i += stride) {
+    const long long b = i / per;
+    const int e = (int)(i - b * per);        // index in the destination sample
+    const int c = e / rows, r = e - c * rows;
+    dst[i] = src[b * per + (long long)r * cols + c];
+  }
+}
+
+// libjit_gather: dest[sample][i] = data[sample][indices[i]] for slices of
+// slice_bytes bytes; an index outside the sample yields zero bytes.
+template <typename IDX>
+__global__ __launch_bounds__(kGlueThreads) void gather_kernel(
+    uint8_t *__restrict__ dst, const uint8_t *__restrict__ data, const IDX *__restrict__ idx,
+    long long num_indices, long long slice_bytes, long long samples, long long sample_bytes) {
+  const long long total = samples * num_indices * slice_bytes;
+  const long long stride = (long long)gridDim.x * kGlueThreads;
+  const long long slices = sample_bytes / slice_bytes;
+  for (long long i = (long long)blockIdx.x * kGlueThreads + threadIdx.x; i < total; i += stride) {
+    const long long b = i % slice_bytes;
+    const long long t = i / slice_bytes;
+    const long long k = t % num_indices, smp = t / num_indices;
+    const long long sl = (long long)idx[k];
+    dst[i] = (sl >= 0 && sl < slices) ? data[smp * sample_bytes + sl * slice_bytes + b] : 0;
+  }
+}
+
+// One workgroup per sample: out[b] = clip(scale(sum_k (L-lo)(R-ro); outP) + oo),
+// libjit_matmul_i8 on each [M x K] x [K x N] pair of a batch of small matrices.
+__global__ __launch_bounds__(kGlueThreads) void batch_matmul_i8_kernel(
+    int8_t *__restrict__ out, const int8_t *__restrict__ lhs, const int8_t *__restrict__ rhs,
+    int M, int K, int N, int32_t oo, int32_t lo, int32_t ro, int32_t pre, int32_t post,
+    int32_t scale) {
+  extern __shared__ int8_t sm[];
+  int8_t *sl = sm, *sr = sm + (size_t)M * K;
+  const long long b = blockIdx.x;
+  const int8_t *L = lhs + b * (long long)M * K, *R = rhs + b * (long long)K * N;
+  for (int i = threadIdx.x; i < M * K; i += kGlueThreads) sl[i] = L[i];
+  for (int i = threadIdx.x; i < K * N; i += kGlueThreads) sr[i] = R[i];
+  __syncthreads();
+  int8_t *O = out + b * (long long)M * N;
+  for (int e = threadIdx.x; e < M * N; e += kGlueThreads) {
+    const int i = e / N, j = e - i * N;
+    uint32_t acc = 0;
+    for (int k = 0; k < K; k++)
+      acc += (uint32_t)(((int32_t)sl[i * K + k] - lo) * ((int32_t)sr[k * N + j] - ro));
+    O[e] = (int8_t)clip_i8(scale_i32((int32_t)acc, pre, post, scale, oo));
+  }
+}
+
+// libjit_sigmoid_kernel_f: 1 / (expf(-x) + 1)
+__global__ __launch_bounds__(kGlueThreads) void sigmoid_f32_kernel(
+    float *__restrict__ dst, const float *__restrict__ src, size_t n) {
+  const size_t stride = (size_t)gridDim.x * kGlueThreads;
+  for (size_t i = (size_t)blockIdx.x * kGlueThreads + threadIdx.x; i < n; i += stride)
+    dst[i] = __fdiv_rn(1.0f, __fadd_rn(expf(-src[i]), 1.0f));
+}
+
+static unsigned capped_blocks(size_t work) {
+  size_t b = (work + kGlueThreads - 1) / kGlueThreads;
+  if (b > 256 * 64) b = 256 * 64;
+  return (unsigned)(b ? b : 1);
+}
+
 static bool al16(const void *a, const void *b, const void *c) {
   return (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c) & 15) == 0;
 }
@@ -379,6 +477,92 @@ int mi355x_avg_pool_i8(int8_t *out, const int8_t *in, size_t N, size_t IH, size_
                        dim3(kGlueThreads), 0, as_stream(stream), out, in, g, count_include_pads,
                        out_offset, in_offset, out_pre, out_post, out_scale, total);
   return check_launch("avg_pool_i8");
+}
+
+int mi355x_convert_f16_to_f32(float *dst, const void *src, size_t n, void *stream) {
+  if (n == 0) return MI355X_OK;
+  MI355X_REQUIRE(dst && src, "NULL tensor");
+  hipLaunchKernelGGL(convert_f16_f32_kernel, dim3(capped_blocks(n)), dim3(kGlueThreads), 0,
+                     as_stream(stream), dst, (const __half *)src, n);
+  return check_launch("convert_f16_to_f32");
+}
+
+int mi355x_insert_rows(void *dst, const void *src, size_t rows, size_t row_bytes,
+                       size_t dst_row_stride, size_t dst_offset, void *stream) {
+  if (rows == 0 || row_bytes == 0) return MI355X_OK;
+  MI355X_REQUIRE(dst && src, "NULL tensor");
+  MI355X_REQUIRE(dst_offset + row_bytes <= dst_row_stride,
+                 "slice of %zu bytes at offset %zu does not fit rows of %zu bytes", row_bytes,
+                 dst_offset, dst_row_stride);
+  MI355X_REQUIRE(rows < (1ull << 40) && dst_row_stride < (1ull << 40), "tensor too large");
+  const uintptr_t all = (uintptr_t)dst | (uintptr_t)src | row_bytes | dst_row_stride | dst_offset;
+  const int unit = (all % 16 == 0) ? 16 : (all % 4 == 0) ? 4 : 1;
+  hipLaunchKernelGGL(insert_rows_kernel, dim3(capped_blocks(rows * (row_bytes / unit))),
+                     dim3(kGlueThreads), 0, as_stream(stream), (uint8_t *)dst,
+                     (const uint8_t *)src, (long long)rows, (long long)row_bytes,
+                     (long long)dst_row_stride, (long long)dst_offset, unit);
+  return check_launch("insert_rows");
+}
+
+int mi355x_batch_transpose_i8(int8_t *dst, const int8_t *src, size_t batch, size_t rows,
+                              size_t cols, void *stream) {
+  if (batch == 0 || rows == 0 || cols == 0) return MI355X_OK;
+  MI355X_REQUIRE(dst && src, "NULL tensor");
+  MI355X_REQUIRE(rows < (1u << 15) && cols < (1u << 15) && batch < (1ull << 32),
+                 "matrices too large");
+  hipLaunchKernelGGL(batch_transpose_i8_kernel, dim3(capped_blocks(batch * rows * cols)),
+                     dim3(kGlueThreads), 0, as_stream(stream), dst, src, (long long)batch,
+                     (int)rows, (int)cols);
+  return check_launch("batch_transpose_i8");
+}
+
+int mi355x_gather(void *dst, const void *data, const void *indices, int idx_is_64,
+                  size_t num_indices, size_t slice_bytes, size_t num_samples,
+                  size_t sample_bytes, void *stream) {
+  if (num_indices == 0 || slice_bytes == 0 || num_samples == 0) return MI355X_OK;
+  MI355X_REQUIRE(dst && data && indices, "NULL tensor");
+  MI355X_REQUIRE(sample_bytes % slice_bytes == 0, "sample is not a whole number of slices");
+  MI355X_REQUIRE(num_indices < (1ull << 32) && slice_bytes < (1ull << 32) &&
+                     num_samples < (1ull << 32) && sample_bytes < (1ull << 40),
+                 "tensor too large");
+  const size_t total = num_samples * num_indices * slice_bytes;
+  if (idx_is_64)
+    hipLaunchKernelGGL(gather_kernel<long long>, dim3(capped_blocks(total)), dim3(kGlueThreads), 0,
+                       as_stream(stream), (uint8_t *)dst, (const uint8_t *)data,
+                       (const long long *)indices, (long long)num_indices, (long long)slice_bytes,
+                       (long long)num_samples, (long long)sample_bytes);
+  else
+    hipLaunchKernelGGL(gather_kernel<int>, dim3(capped_blocks(total)), dim3(kGlueThreads), 0,
+                       as_stream(stream), (uint8_t *)dst, (const uint8_t *)data,
+                       (const int *)indices, (long long)num_indices, (long long)slice_bytes,
+                       (long long)num_samples, (long long)sample_bytes);
+  return check_launch("gather");
+}
+
+int mi355x_batch_matmul_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs, size_t batch,
+                           size_t M, size_t K, size_t N, int32_t out_offset, int32_t lhs_offset,
+                           int32_t rhs_offset, int32_t out_pre, int32_t out_post,
+                           int32_t out_scale, void *stream) {
+  if (batch == 0 || M == 0 || N == 0) return MI355X_OK;
+  MI355X_REQUIRE(out && lhs && rhs, "NULL tensor");
+  MI355X_REQUIRE(shifts_ok(out_pre, out_post), "pre/post shift outside [0, 31]");
+  MI355X_REQUIRE(batch < 0x7fffffffu, "batch too large");
+  const size_t lds = (M + N) * K;
+  MI355X_REQUIRE(lds <= 64 * 1024 && M * N < (1u << 24),
+                 "matrices of %zu x %zu x %zu do not fit the small-matrix kernel (use "
+                 "mi355x_matmul_i8 per sample)", M, K, N);
+  hipLaunchKernelGGL(batch_matmul_i8_kernel, dim3((unsigned)batch), dim3(kGlueThreads), lds,
+                     as_stream(stream), out, lhs, rhs, (int)M, (int)K, (int)N, out_offset,
+                     lhs_offset, rhs_offset, out_pre, out_post, out_scale);
+  return check_launch("batch_matmul_i8");
+}
+
+int mi355x_sigmoid_f32(float *dst, const float *src, size_t n, void *stream) {
+  if (n == 0) return MI355X_OK;
+  MI355X_REQUIRE(dst && src, "NULL tensor");
+  hipLaunchKernelGGL(sigmoid_f32_kernel, dim3(capped_blocks(n)), dim3(kGlueThreads), 0,
+                     as_stream(stream), dst, src, n);
+  return check_launch("sigmoid_f32");
 }
 
 int mi355x_softmax_f32(float *out, const float *in, size_t rows, size_t cols, void *stream) {

@@ -48,6 +48,17 @@ class Net:
     def activation(self, name, shape, kind, scale=1.0, offset=0):
         return self._add(Tensor(name, kind, shape, "activation", scale, offset))
 
+    def view(self, name, source, shape):
+        """The bytes of `source` under another shape (same kind and parameters)."""
+        s = self.tensors[source]
+        t = Tensor(name, s.kind, shape, "view", s.scale, s.offset)
+        t.source = source
+        return self._add(t)
+
+    def root(self, name):
+        t = self.tensors[name]
+        return self.root(t.source) if t.role == "view" else name
+
     def op(self, kind, name, operands, iattrs=(), fattrs=()):
         for o in operands:
             assert o in self.tensors, o
@@ -82,6 +93,10 @@ def to_module(net, function="main"):
     for t in net.tensors.values():
         if t.role == "activation":
             ids[t.name] = m.activation(f, t.name, t.shape, t.kind, t.scale, t.offset)
+        elif t.role == "view":      # sources precede their views in insertion order
+            if t.source not in ids:
+                raise ValueError(f"view {t.name} precedes its source {t.source}")
+            ids[t.name] = m.view(t.name, ids[t.source], t.shape, t.kind, t.scale, t.offset)
     for o in net.ops:
         m.instruction(f, o.kind, o.name, [ids[n] for n in o.operands], o.iattrs, o.fattrs)
     return m, f

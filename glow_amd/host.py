@@ -14,7 +14,8 @@ _LIB = None
  UINT4_FUSED_FP16, UINT4_FUSED, BOOL) = range(11)
 (QUANTIZE, DEQUANTIZE, RESCALE_QUANTIZED, FULLY_CONNECTED, ROWWISE_QUANTIZED_FC,
  MATMUL, CONVOLUTION, CHANNELWISE_QUANTIZED_CONV, FRWQ_SLWS, FRWQ_SLS, ELEMENT_ADD,
- RELU, MAX_POOL, AVG_POOL, SOFTMAX) = range(15)
+ RELU, MAX_POOL, AVG_POOL, SOFTMAX, CONVERT_TO, INSERT_TENSOR, TRANSPOSE, GATHER,
+ BATCH_MATMUL, SIGMOID) = range(21)
 ACT_NONE, ACT_RELU, ACT_CLIP, ACT_TANH, ACT_SIGMOID, ACT_LEAKY_RELU = range(6)
 
 ERROR_NAMES = ["SUCCESS", "UNKNOWN", "RUNTIME_ERROR", "RUNTIME_OUT_OF_DEVICE_MEMORY",
@@ -26,7 +27,7 @@ ERROR_NAMES = ["SUCCESS", "UNKNOWN", "RUNTIME_ERROR", "RUNTIME_OUT_OF_DEVICE_MEM
 EXPORTS = [
     "mi355x_host_last_error", "mi355x_host_error_name", "mi355x_host_module_create",
     "mi355x_host_module_destroy", "mi355x_host_add_constant", "mi355x_host_add_placeholder",
-    "mi355x_host_create_function", "mi355x_host_add_activation",
+    "mi355x_host_create_function", "mi355x_host_add_activation", "mi355x_host_add_view",
     "mi355x_host_add_instruction", "mi355x_host_is_op_supported", "mi355x_host_compile",
     "mi355x_host_describe", "mi355x_host_bundle_sizes", "mi355x_host_dm_create",
     "mi355x_host_dm_destroy", "mi355x_host_dm_init", "mi355x_host_dm_stop",
@@ -119,6 +120,11 @@ class Module:
         d, nd = _dims(shape)
         return _check(lib().mi355x_host_add_activation(
             self._h, fn, name.encode(), kind, d, nd, C.c_float(scale), C.c_int32(offset)))
+
+    def view(self, name, source, shape, kind, scale=1.0, offset=0):
+        d, nd = _dims(shape)
+        return _check(lib().mi355x_host_add_view(
+            self._h, name.encode(), source, kind, d, nd, C.c_float(scale), C.c_int32(offset)))
 
     @staticmethod
     def _inst_args(operands, iattrs, fattrs):

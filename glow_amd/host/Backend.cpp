@@ -111,6 +111,12 @@ public:
       case Kind::MaxPool: MI355X_RETURN_IF_ERR(pool(I, out, false)); break;
       case Kind::AvgPool: MI355X_RETURN_IF_ERR(pool(I, out, true)); break;
       case Kind::SoftMax: MI355X_RETURN_IF_ERR(softmax(I, out)); break;
+      case Kind::ConvertTo:
+      case Kind::InsertTensor:
+      case Kind::Transpose:
+      case Kind::Gather:
+      case Kind::BatchMatMul:
+      case Kind::Sigmoid: MI355X_RETURN_IF_ERR(movement(I, out)); break;
       case Kind::Quantize: MI355X_RETURN_IF_ERR(quantize(I, out)); break;
       case Kind::Dequantize: MI355X_RETURN_IF_ERR(dequantize(I, out)); break;
       case Kind::RescaleQuantized: MI355X_RETURN_IF_ERR(rescale(I, out)); break;
@@ -161,7 +167,8 @@ public:
   const std::map<int, std::pair<bool, bool>> &io() const { return io_; }
 
 private:
-  static constexpr int kArity[(int)Kind::NumKinds] = {2, 2, 2, 4, 6, 3, 4, 8, 5, 4, 3, 2, 2, 2, 2};
+  static constexpr int kArity[(int)Kind::NumKinds] = {2, 2, 2, 4, 6, 3, 4, 8, 5, 4, 3, 2, 2, 2, 2,
+                                                       2, 2, 2, 3, 3, 2};
 
   Error checkOperands(const Instruction &I) {
     CHECK_OP((int)I.kind >= 0 && (int)I.kind < (int)Kind::NumKinds, "unknown kind");
@@ -184,10 +191,13 @@ private:
 
   Operand op(const Instruction &I, int i) const { return Operand{&M_.value(I.operands[(size_t)i])}; }
 
+  // number of operands that read the memory of `id` (through it or a view)
   int readers(int id) const {
+    const int root = M_.value(id).root;
     int n = 0;
     for (const auto &I : insts_)
-      for (size_t i = 1; i < I.operands.size(); i++) n += I.operands[i] == id;
+      for (size_t i = 1; i < I.operands.size(); i++)
+        n += M_.validId(I.operands[i]) && M_.value(I.operands[i]).root == root;
     return n;
   }
 
@@ -302,6 +312,124 @@ private:
                                      b.stream);
          }});
     return Error::success();
+  }
+
+  // data movement and the small operators of ranking models
+  Error movement(const Instruction &I, MI355XFunction &out) {
+    Operand d = op(I, 0), s = op(I, 1);
+    switch (I.kind) {
+    case Kind::ConvertTo: {
+      CHECK_OP(d.ty().kind == ElemKind::FloatTy && s.ty().kind == ElemKind::Float16Ty,
+               "only float16 -> float is supported");
+      CHECK_OP(d.ty().size() == s.ty().size(), "size mismatch");
+      const size_t n = (size_t)d.ty().size();
+      out.launches.push_back({"mi355x_convert_f16_to_f32", I.name, strFormat(" n=%zu", n),
+                              [=](const DeviceBindings &b) {
+                                return mi355x_convert_f16_to_f32((float *)d.ptr(b), s.ptr(b), n, b.stream);
+                              }});
+      return Error::success();
+    }
+    case Kind::Sigmoid: {
+      CHECK_OP(d.ty().kind == ElemKind::FloatTy && s.ty().kind == ElemKind::FloatTy, "needs float tensors");
+      CHECK_OP(d.ty().size() == s.ty().size(), "size mismatch");
+      const size_t n = (size_t)d.ty().size();
+      out.launches.push_back({"mi355x_sigmoid_f32", I.name, strFormat(" n=%zu", n),
+                              [=](const DeviceBindings &b) {
+                                return mi355x_sigmoid_f32((float *)d.ptr(b), (const float *)s.ptr(b), n, b.stream);
+                              }});
+      return Error::success();
+    }
+    case Kind::InsertTensor: {
+      CHECK_OP(d.ty().kind == s.ty().kind && d.ty().dims.size() == 2 && s.ty().dims.size() == 2,
+               "needs 2-D tensors of one element kind");
+      CHECK_OP(!isQuantized(d.ty().kind) || (d.ty().scale == s.ty().scale && d.ty().offset == s.ty().offset),
+               "slice and tensor must share scale and offset");
+      CHECK_OP(I.iattrs.size() == 1 && I.iattrs[0] >= 0, "expects the inner offset");
+      const size_t es = elemSize(d.ty().kind);
+      const size_t rows = (size_t)s.ty().dims[0], w = (size_t)s.ty().dims[1], W = (size_t)d.ty().dims[1];
+      const size_t off = (size_t)I.iattrs[0];
+      CHECK_OP(d.ty().dims[0] == s.ty().dims[0] && off + w <= W, "slice does not fit");
+      out.launches.push_back({"mi355x_insert_rows", I.name,
+                              strFormat(" rows=%zu row_bytes=%zu stride=%zu offset=%zu", rows, w * es, W * es, off * es),
+                              [=](const DeviceBindings &b) {
+                                return mi355x_insert_rows(d.ptr(b), s.ptr(b), rows, w * es, W * es, off * es, b.stream);
+                              }});
+      return Error::success();
+    }
+    case Kind::Transpose: {
+      CHECK_OP(d.ty().kind == ElemKind::Int8QTy && s.ty().kind == ElemKind::Int8QTy, "needs i8 tensors");
+      CHECK_OP(d.ty().scale == s.ty().scale && d.ty().offset == s.ty().offset,
+               "input and output must share scale and offset");
+      const auto &sd = s.ty().dims;
+      const auto &dd = d.ty().dims;
+      size_t batch = 1, rows = 0, cols = 0;
+      if (I.iattrs == std::vector<int64_t>{1, 0} && sd.size() == 2) {
+        rows = (size_t)sd[0]; cols = (size_t)sd[1];
+        CHECK_OP(dd.size() == 2 && dd[0] == sd[1] && dd[1] == sd[0], "shape mismatch");
+      } else if (I.iattrs == std::vector<int64_t>{0, 2, 1} && sd.size() == 3) {
+        batch = (size_t)sd[0]; rows = (size_t)sd[1]; cols = (size_t)sd[2];
+        CHECK_OP(dd.size() == 3 && dd[0] == sd[0] && dd[1] == sd[2] && dd[2] == sd[1], "shape mismatch");
+      } else {
+        CHECK_OP(false, "only the shuffles {1,0} and {0,2,1} are supported");
+      }
+      out.launches.push_back({"mi355x_batch_transpose_i8", I.name,
+                              strFormat(" batch=%zu rows=%zu cols=%zu", batch, rows, cols),
+                              [=](const DeviceBindings &b) {
+                                return mi355x_batch_transpose_i8((int8_t *)d.ptr(b), (const int8_t *)s.ptr(b),
+                                                                 batch, rows, cols, b.stream);
+                              }});
+      return Error::success();
+    }
+    case Kind::Gather: {
+      Operand idx = op(I, 2);
+      CHECK_OP(d.ty().kind == s.ty().kind, "data and result must have one element kind");
+      CHECK_OP(idx.ty().kind == ElemKind::Int64ITy || idx.ty().kind == ElemKind::Int32ITy,
+               "indices must be int64 or int32");
+      CHECK_OP(idx.ty().dims.size() == 1, "indices must be 1-D");
+      CHECK_OP(I.iattrs.size() == 1 && (I.iattrs[0] == 0 || I.iattrs[0] == 1), "batchDims must be 0 or 1");
+      const size_t bd = (size_t)I.iattrs[0];
+      const auto &sd = s.ty().dims;
+      CHECK_OP(sd.size() > bd, "data has too few dimensions");
+      size_t slice = elemSize(s.ty().kind);
+      for (size_t i = bd + 1; i < sd.size(); i++) slice *= (size_t)sd[i];
+      const size_t samples = bd ? (size_t)sd[0] : 1, sample = (size_t)sd[bd] * slice;
+      const size_t nIdx = (size_t)idx.ty().size();
+      CHECK_OP((size_t)d.ty().sizeInBytes() == samples * nIdx * slice, "result size mismatch");
+      const int i64 = idx.ty().kind == ElemKind::Int64ITy;
+      out.launches.push_back({"mi355x_gather", I.name,
+                              strFormat(" num_indices=%zu slice_bytes=%zu samples=%zu sample_bytes=%zu", nIdx, slice, samples, sample),
+                              [=](const DeviceBindings &b) {
+                                return mi355x_gather(d.ptr(b), s.ptr(b), idx.ptr(b), i64, nIdx, slice, samples, sample, b.stream);
+                              }});
+      return Error::success();
+    }
+    default: { // BatchMatMul
+      Operand r = op(I, 2);
+      CHECK_OP(d.ty().kind == ElemKind::Int8QTy && s.ty().kind == ElemKind::Int8QTy &&
+                   r.ty().kind == ElemKind::Int8QTy,
+               "needs i8 operands");
+      CHECK_OP(d.ty().dims.size() == 3 && s.ty().dims.size() == 3 && r.ty().dims.size() == 3,
+               "needs 3-D operands");
+      const size_t B = (size_t)s.ty().dims[0], M = (size_t)s.ty().dims[1], K = (size_t)s.ty().dims[2],
+                   N = (size_t)r.ty().dims[2];
+      CHECK_OP((size_t)r.ty().dims[0] == B && (size_t)r.ty().dims[1] == K && (size_t)d.ty().dims[0] == B &&
+                   (size_t)d.ty().dims[1] == M && (size_t)d.ty().dims[2] == N,
+               "shape mismatch");
+      CHECK_OP((M + N) * K <= 64 * 1024, "matrices too large for the small-matrix kernel");
+      const S32To8 p = s32to8(s.ty().scale * r.ty().scale / d.ty().scale);
+      const int32_t oo = d.ty().offset, lo = s.ty().offset, ro = r.ty().offset;
+      out.launches.push_back({"mi355x_batch_matmul_i8", I.name,
+                              strFormat(" B=%zu M=%zu K=%zu N=%zu", B, M, K, N) + kv("out_offset", oo) +
+                                  kv("lhs_offset", lo) + kv("rhs_offset", ro) + kv("out_pre", p.pre) +
+                                  kv("out_post", p.post) + kv("out_scale", p.scale),
+                              [=](const DeviceBindings &b) {
+                                return mi355x_batch_matmul_i8((int8_t *)d.ptr(b), (const int8_t *)s.ptr(b),
+                                                              (const int8_t *)r.ptr(b), B, M, K, N, oo, lo, ro,
+                                                              p.pre, p.post, p.scale, b.stream);
+                              }});
+      return Error::success();
+    }
+    }
   }
 
   Error softmax(const Instruction &I, MI355XFunction &out) {

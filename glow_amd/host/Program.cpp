@@ -92,12 +92,33 @@ const char *kindName(Kind k) {
   case Kind::MaxPool: return "MaxPool";
   case Kind::AvgPool: return "AvgPool";
   case Kind::SoftMax: return "SoftMax";
+  case Kind::ConvertTo: return "ConvertTo";
+  case Kind::InsertTensor: return "InsertTensor";
+  case Kind::Transpose: return "Transpose";
+  case Kind::Gather: return "Gather";
+  case Kind::BatchMatMul: return "BatchMatMul";
+  case Kind::Sigmoid: return "Sigmoid";
   default: return "?";
   }
 }
 
+int Module::createView(const std::string &name, int src, const Type &t) {
+  if (!validId(src)) return -1;
+  const Value &s = values_[(size_t)src];
+  if (t.sizeInBytes() > s.type.sizeInBytes()) return -1;
+  Value v;
+  v.name = name;
+  v.type = t;
+  v.category = s.category;
+  v.offset = s.offset;
+  v.function = s.function;
+  v.root = s.root;
+  return addValue(std::move(v));
+}
+
 int Module::addValue(Value v) {
   v.id = (int)values_.size();
+  if (v.root < 0) v.root = v.id;
   values_.push_back(std::move(v));
   return values_.back().id;
 }

@@ -31,6 +31,7 @@ struct Value {
   SymbolCategory category = SymbolCategory::Activation;
   size_t offset = 0; // byte offset inside the region of its category
   int function = -1; // owning function for activations
+  int root = -1;     // the value whose memory this one is a view of (itself if none)
 };
 
 // Instruction kinds: the names are Glow's IR instruction names without "Inst".
@@ -50,6 +51,12 @@ enum class Kind : int32_t {
   MaxPool,                      // (Dest, Src); iattrs {kernelH, kernelW, strideH, strideW, padT, padL, padB, padR}
   AvgPool,                      // (Dest, Src); MaxPool's iattrs + {countIncludePads}
   SoftMax,                      // (Dest, Src), float [rows x cols]
+  ConvertTo,                    // (Dest float, Src float16)
+  InsertTensor,                 // (Dest [R,W], Src [R,w]); iattrs {offset in the inner dimension}
+  Transpose,                    // (Dest, Src) int8; iattrs = shuffle, {1,0} or {0,2,1}
+  Gather,                       // (Dest, Data, Indices); iattrs {batchDims (0 or 1)}
+  BatchMatMul,                  // (Dest [B,M,N], LHS [B,M,K], RHS [B,K,N]) int8
+  Sigmoid,                      // (Dest, Src) float
   NumKinds
 };
 const char *kindName(Kind k);
@@ -155,6 +162,9 @@ public:
   // Module::createPlaceholder
   int createPlaceholder(const std::string &name, const Type &t);
   Function *createFunction(const std::string &name);
+  // TensorViewInst: another type over the bytes of `src` (a reshape); the view
+  // must not be larger than its source. Returns -1 when it is.
+  int createView(const std::string &name, int src, const Type &t);
 
   const Value &value(int id) const { return values_.at((size_t)id); }
   bool validId(int id) const { return id >= 0 && (size_t)id < values_.size(); }

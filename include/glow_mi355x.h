@@ -227,6 +227,36 @@ int mi355x_avg_pool_i8(int8_t *out, const int8_t *in, size_t N, size_t IH,
 int mi355x_softmax_f32(float *out, const float *in, size_t rows, size_t cols,
                        void *stream);
 
+/* ---- data movement and the small operators of ranking models ------------------ */
+
+/* ConvertTo Float16 -> Float (exact). */
+int mi355x_convert_f16_to_f32(float *dst, const void *src, size_t n, void *stream);
+/* InsertTensor of a 2-D slice along the inner dimension, as Concat lowers to
+ * (reference libjit_insert_tensor, libjit.cpp:156-260): for each of `rows`
+ * rows, row_bytes bytes of src go to dst + r*dst_row_stride + dst_offset. */
+int mi355x_insert_rows(void *dst, const void *src, size_t rows, size_t row_bytes,
+                       size_t dst_row_stride, size_t dst_offset, void *stream);
+/* Transpose of the two inner dimensions of [batch x rows x cols] int8. */
+int mi355x_batch_transpose_i8(int8_t *dst, const int8_t *src, size_t batch, size_t rows,
+                              size_t cols, void *stream);
+/* libjit_gather (libjit.cpp:418-440, gather64/gather32 entry points :2083-2130):
+ * dest[sample][i] = slice indices[i] of data[sample]; slices of slice_bytes
+ * bytes, samples of sample_bytes bytes. Unlike the reference an index outside
+ * the sample yields zeros instead of an out-of-bounds read. */
+int mi355x_gather(void *dst, const void *data, const void *indices, int idx_is_64,
+                  size_t num_indices, size_t slice_bytes, size_t num_samples,
+                  size_t sample_bytes, void *stream);
+/* BatchMatMul of small int8 matrices, i.e. libjit_matmul_i8
+ * (libjit_matmul.cpp:353-371) on every [M x K] x [K x N] pair of the batch (what
+ * the node lowers to). (M + N) * K must not exceed 64 KiB. */
+int mi355x_batch_matmul_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs, size_t batch,
+                           size_t M, size_t K, size_t N, int32_t out_offset, int32_t lhs_offset,
+                           int32_t rhs_offset, int32_t out_pre, int32_t out_post,
+                           int32_t out_scale, void *stream);
+/* libjit_sigmoid_kernel_f (libjit.cpp:1913-1916): 1 / (expf(-x) + 1); agrees
+ * with the CPU to fp32 rounding of expf (1e-5 relative). */
+int mi355x_sigmoid_f32(float *dst, const float *src, size_t n, void *stream);
+
 /* ---- FullyConnected / MatMul -------------------------------------------------- */
 
 /* sums[r] = sum over k of rows[r][k] for an int8 matrix [n_rows x K] with K

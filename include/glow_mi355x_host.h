@@ -67,7 +67,13 @@ enum {
   MI355X_HOST_RELU = 11,               /* Dest, Src */
   MI355X_HOST_MAX_POOL = 12,           /* Dest, Src; iattrs kernelH, kernelW, strideH, strideW, padT, padL, padB, padR */
   MI355X_HOST_AVG_POOL = 13,           /* Dest, Src; MaxPool's iattrs + countIncludePads */
-  MI355X_HOST_SOFTMAX = 14             /* Dest, Src (float, [rows x cols]) */
+  MI355X_HOST_SOFTMAX = 14,            /* Dest, Src (float, [rows x cols]) */
+  MI355X_HOST_CONVERT_TO = 15,         /* Dest float, Src float16 */
+  MI355X_HOST_INSERT_TENSOR = 16,      /* Dest [R,W], Src [R,w]; iattrs {inner offset} */
+  MI355X_HOST_TRANSPOSE = 17,          /* Dest, Src int8; iattrs shuffle {1,0} or {0,2,1} */
+  MI355X_HOST_GATHER = 18,             /* Dest, Data, Indices; iattrs {batchDims} */
+  MI355X_HOST_BATCH_MATMUL = 19,       /* Dest [B,M,N], LHS [B,M,K], RHS [B,K,N] int8 */
+  MI355X_HOST_SIGMOID = 20             /* Dest, Src float */
 };
 /* Convolution iattrs: kernelH, kernelW, strideH, strideW, padT, padL, padB,
  * padR, group, dilationH, dilationW, fusedActivation (glow::FusedActivation);
@@ -90,6 +96,9 @@ int mi355x_host_create_function(mi355x_host_module *m, const char *name);
 int mi355x_host_add_activation(mi355x_host_module *m, int function, const char *name,
                                int elem_kind, const int64_t *dims, int ndims, float scale,
                                int32_t offset);
+/* TensorViewInst: a value of another type over the bytes of `source` (reshape). */
+int mi355x_host_add_view(mi355x_host_module *m, const char *name, int source, int elem_kind,
+                         const int64_t *dims, int ndims, float scale, int32_t offset);
 int mi355x_host_add_instruction(mi355x_host_module *m, int function, int kind, const char *name,
                                 const int *operands, int n_operands, const int64_t *iattrs,
                                 int n_iattrs, const float *fattrs, int n_fattrs);

@@ -791,3 +791,24 @@ void go_softmax_f32(float *out, const float *in, size_t rows, size_t cols) {
     for (size_t i = 0; i < cols; i++) y[i] = y[i] / sum;
   }
 }
+
+/* libjit.cpp:1913-1916 */
+void go_sigmoid_f32(float *out, const float *in, size_t n) {
+  for (size_t i = 0; i < n; i++) {
+    const float e = expf(-in[i]);
+    out[i] = 1 / (e + 1);
+  }
+}
+
+/* libjit.cpp:418-440 */
+void go_gather(uint8_t *dest, const uint8_t *data, const int64_t *indices,
+               size_t numIndices, size_t sliceBytes, size_t numSamples,
+               size_t sampleBytes) {
+  size_t outIdx = 0;
+  for (size_t s = 0; s < numSamples; s++)
+    for (size_t i = 0; i < numIndices; i++) {
+      memcpy(dest + outIdx * sliceBytes,
+             data + s * sampleBytes + (size_t)indices[i] * sliceBytes, sliceBytes);
+      outIdx++;
+    }
+}

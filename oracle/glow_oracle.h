@@ -220,6 +220,12 @@ void go_avg_pool_i8(int8_t *out, const int8_t *in, size_t N, size_t IH,
                     int32_t outPre, int32_t outPost, int32_t outScale);
 /* libjit_softmax_f (libjit.cpp:3058-3082) on [rows x cols]. */
 void go_softmax_f32(float *out, const float *in, size_t rows, size_t cols);
+/* libjit_sigmoid_kernel_f (libjit.cpp:1913-1916, the build without fast-math). */
+void go_sigmoid_f32(float *out, const float *in, size_t n);
+/* libjit_gather (libjit.cpp:418-440) on byte slices. */
+void go_gather(uint8_t *dest, const uint8_t *data, const int64_t *indices,
+               size_t numIndices, size_t sliceBytes, size_t numSamples,
+               size_t sampleBytes);
 
 #ifdef __cplusplus
 }

@@ -414,3 +414,31 @@ def softmax_f32(x):
     out = np.empty_like(x)
     lib().go_softmax_f32(_p(out), _p(x), C.c_size_t(x.shape[0]), C.c_size_t(x.shape[1]))
     return out
+
+
+# ---- data movement and the small operators of ranking models -----------------
+
+def sigmoid_f32(x):
+    x = _c(x, np.float32)
+    out = np.empty_like(x)
+    lib().go_sigmoid_f32(_p(out), _p(x), C.c_size_t(x.size))
+    return out
+
+
+def gather(data, indices, batch_dims=0):
+    data = np.ascontiguousarray(data)
+    idx = _c(indices, np.int64)
+    samples = data.shape[0] if batch_dims else 1
+    inner = data.shape[batch_dims + 1:]
+    slice_bytes = int(np.prod(inner, dtype=np.int64)) * data.dtype.itemsize
+    sample_bytes = data.shape[batch_dims] * slice_bytes
+    out = np.empty(data.shape[:batch_dims] + (idx.size,) + inner, data.dtype)
+    lib().go_gather(_p(out), _p(data), _p(idx), C.c_size_t(idx.size), C.c_size_t(slice_bytes),
+                    C.c_size_t(samples), C.c_size_t(sample_bytes))
+    return out
+
+
+def batch_matmul_i8(lhs, rhs, out_offset, lhs_offset, rhs_offset, outP):
+    """BatchMatMul as it is lowered: libjit_matmul_i8 on every pair of the batch."""
+    return np.stack([matmul_i8(lhs[b], rhs[b], out_offset, lhs_offset, rhs_offset, outP)
+                     for b in range(lhs.shape[0])])

@@ -282,3 +282,22 @@ def softmax_f32(x, fastmath=False):
     d = _dims(*x.shape)
     lib(fastmath).libjit_softmax_f(_p(x), _p(out), _p(d), _p(d))
     return out
+
+
+def sigmoid_f32(x, fastmath=False):
+    x = _c(x, np.float32).ravel()
+    f = lib(fastmath).libjit_sigmoid_kernel_f
+    f.restype = C.c_float
+    f.argtypes = [C.c_uint64, C.c_void_p, C.c_void_p, C.c_void_p]
+    px = x.ctypes.data
+    return np.array([f(i, px, None, None) for i in range(x.size)], np.float32)
+
+
+def gather64_i8(data, indices, num_samples, sample_size, slice_size):
+    data = _c(data, np.int8)
+    idx = _c(indices, np.int64)
+    out = np.empty(num_samples * idx.size * slice_size, np.int8)
+    lib().libjit_gather64_i8(_p(out), _p(data), _p(idx), C.c_uint64(idx.size),
+                             C.c_uint64(slice_size), C.c_uint64(num_samples),
+                             C.c_uint64(sample_size))
+    return out

@@ -18,10 +18,44 @@ def _f(x):
     return np.float32(x)
 
 
+class _Values:
+    """Tensor values by name; a view shares the storage of its source."""
+
+    def __init__(self, net):
+        self.net = net
+        self.flat = {}
+
+    def _storage(self, name):
+        root = self.net.root(name)
+        if root not in self.flat:
+            t = self.net.tensors[root]
+            self.flat[root] = np.zeros(int(np.prod(t.shape, dtype=np.int64)), t.dtype)
+        return self.flat[root]
+
+    def get(self, name):
+        t = self.net.tensors[name]
+        n = int(np.prod(t.shape, dtype=np.int64))
+        return self._storage(name)[:n].reshape(t.shape)
+
+    def set(self, name, value):
+        t = self.net.tensors[name]
+        value = np.asarray(value)
+        flat = self._storage(name)
+        flat[:value.size] = value.astype(t.dtype, copy=False).ravel()
+
+    def __getitem__(self, name):
+        return self.get(name)
+
+
 def run(net, inputs):
-    """inputs: placeholder name -> array. Returns every tensor's value by name."""
-    v = {t.name: t.data for t in net.tensors.values() if t.role == "constant"}
-    v.update(inputs)
+    """inputs: placeholder name -> array (may be shorter than the placeholder).
+    Returns the tensor values, indexable by name."""
+    v = _Values(net)
+    for t in net.tensors.values():
+        if t.role == "constant":
+            v.set(t.name, t.data)
+    for k, x in inputs.items():
+        v.set(k, x)
     T = net.tensors
     for o in net.ops:
         t = [T[n] for n in o.operands]
@@ -73,7 +107,30 @@ def run(net, inputs):
             r = go.cwq_conv2d_i8(a[1], a[2], a[3], g, d.offset, t[1].offset, a[5], a[7],
                                  bp[:, 0], bp[:, 1], bp[:, 2], op[:, 0], op[:, 1], op[:, 2],
                                  act, args)
+        elif o.kind in (H.FRWQ_SLS, H.FRWQ_SLWS):
+            weighted = o.kind == H.FRWQ_SLWS
+            data, w = a[1], (a[2] if weighted else None)
+            idx, ln = (a[3], a[4]) if weighted else (a[2], a[3])
+            kind = {H.UINT8_FUSED: go.U8_F32, H.UINT8_FUSED_FP16: go.U8_F16,
+                    H.UINT4_FUSED_FP16: go.U4_F16, H.UINT4_FUSED: go.U4_F32}[t[1].kind]
+            r = go.frwq_slws_generic(data, kind, w, idx, ln, out_f16=d.kind == H.FLOAT16,
+                                     fp16_accum=bool(o.iattrs and o.iattrs[0]))
+        elif o.kind == H.CONVERT_TO:
+            r = a[1].astype(np.float32)
+        elif o.kind == H.SIGMOID:
+            r = go.sigmoid_f32(a[1])
+        elif o.kind == H.INSERT_TENSOR:
+            off = o.iattrs[0]
+            a[0][:, off:off + a[1].shape[1]] = a[1]
+            continue
+        elif o.kind == H.TRANSPOSE:
+            r = np.ascontiguousarray(np.transpose(a[1], o.iattrs))
+        elif o.kind == H.GATHER:
+            r = go.gather(a[1], a[2], o.iattrs[0])
+        elif o.kind == H.BATCH_MATMUL:
+            r = go.batch_matmul_i8(a[1], a[2], d.offset, t[1].offset, t[2].offset,
+                                   _s(_f(t[1].scale) * _f(t[2].scale) / _f(d.scale)))
         else:
             raise NotImplementedError(f"instruction kind {o.kind}")
-        v[d.name] = np.asarray(r).reshape(d.shape)
+        v.set(d.name, r)
     return v

@@ -1,0 +1,56 @@
+"""The DLRM-style harness: builds and compiles on the CPU; on the GPU the whole
+network through MI355XDeviceManager matches the oracle executing the same
+quantized graph: bit-exact int8 logits (the fp16 pooled embeddings feeding them
+included), sigmoid within 1e-5."""
+import numpy as np
+import pytest
+
+from glow_amd import host as H
+from glow_amd.harness import dlrm
+from glow_amd.harness import net as netlib
+from tests import oracle_exec
+
+SMALL = dict(tables=3, rows=2000, dim=16, batch=64, mean_len=5, bottom=(32, 16), top=(32, 1))
+
+
+def test_builds_and_compiles():
+    net, max_idx = dlrm.make(seed=2, **SMALL)
+    m, f = netlib.to_module(net)
+    m.compile(f)
+    k = [r["kernel"] for r in H.parse_listing(m.describe(f)) if r["phase"] == "launch"]
+    assert k.count("mi355x_frwq_slws") == 3 and k.count("mi355x_rwq_fc_i8") == 4
+    assert k.count("mi355x_batch_matmul_i8") == 1 and k.count("mi355x_gather") == 1
+    assert k[-1] == "mi355x_sigmoid_f32"
+    # 4 vectors of 16 -> 6 pairs + 16 dense outputs feed the top MLP
+    assert net.tensors["top_in"].shape == (64, 22)
+
+
+def test_oracle_executes_the_small_network():
+    net, max_idx = dlrm.make(seed=2, **SMALL)
+    inp = dlrm.Inputs(7, 3, 2000, 64, 5, 1.1, 13)
+    v = oracle_exec.run(net, dlrm.bindings(net, inp, max_idx))
+    p = v["prob"]
+    assert p.shape == (64, 1) and np.all((p >= 0) & (p <= 1))
+    assert len(np.unique(v["logit_q"])) > 1 and len(np.unique(v["pairs"])) > 1
+
+
+@pytest.mark.gpu
+def test_device_matches_oracle():
+    cfg = dict(tables=4, rows=5000, dim=64, batch=256, mean_len=8, bottom=(64, 64), top=(128, 1))
+    net, max_idx = dlrm.make(seed=3, **cfg)
+    m, f = netlib.to_module(net)
+    m.compile(f)
+    dm = H.DeviceManager().init()
+    try:
+        dm.add_network(m)
+        for seed in (11, 12):
+            inp = dlrm.Inputs(seed, 4, 5000, 256, 8, 1.1, 13)
+            b = dlrm.bindings(net, inp, max_idx)
+            logit = np.zeros((256, 1), np.int8)
+            prob = np.zeros((256, 1), np.float32)
+            dm.run("main", dict(b, logit_q=logit, prob=prob))
+            want = oracle_exec.run(net, b)
+            np.testing.assert_array_equal(logit, want["logit_q"])
+            np.testing.assert_allclose(prob, want["prob"], rtol=1e-5, atol=1e-30)
+    finally:
+        dm.stop()

@@ -1,0 +1,70 @@
+"""Data movement and the small operators of ranking models on the GPU through
+the C ABI, against the oracle (bit-exact; fp32 sigmoid within 1e-5)."""
+import numpy as np
+import pytest
+
+from glow_amd import capi
+from oracle import glow_oracle as go
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _init():
+    capi.init(0)
+
+
+def test_convert_f16_to_f32():
+    rng = np.random.default_rng(1)
+    x = np.concatenate([rng.normal(0, 100, 4097), [0, -0.0, 65504, -65504, 6e-8, np.inf]]).astype(np.float16)
+    np.testing.assert_array_equal(capi.convert_f16_to_f32(x), x.astype(np.float32))
+
+
+@pytest.mark.parametrize("dtype,widths", [(np.int8, (64, 351)), (np.int8, (16, 32, 48)),
+                                          (np.float32, (13, 64)), (np.int8, (3, 5, 7))])
+def test_concat_through_insert(dtype, widths):
+    rng = np.random.default_rng(2)
+    parts = [rng.integers(-100, 100, (37, w)).astype(dtype) for w in widths]
+    np.testing.assert_array_equal(capi.concat_rows(parts), np.concatenate(parts, axis=1))
+
+
+def test_insert_rejects_overflowing_slice():
+    d = capi.DeviceBuffer.empty((4, 8), np.int8)
+    with pytest.raises(capi.MI355XError):
+        capi.check(capi.lib().mi355x_insert_rows(capi._vp(d), capi._vp(d), capi._sz(4), capi._sz(6),
+                                                 capi._sz(8), capi._sz(4), capi._vp(None)))
+
+
+def test_batch_transpose():
+    rng = np.random.default_rng(3)
+    x = rng.integers(-128, 128, (50, 27, 64)).astype(np.int8)
+    np.testing.assert_array_equal(capi.batch_transpose_i8(x), x.transpose(0, 2, 1))
+
+
+@pytest.mark.parametrize("idt", [np.int32, np.int64])
+def test_gather(idt):
+    rng = np.random.default_rng(4)
+    data = rng.integers(-128, 128, (33, 729)).astype(np.int8)
+    iu = np.triu_indices(27, 1)
+    idx = (iu[0] * 27 + iu[1]).astype(idt)
+    np.testing.assert_array_equal(capi.gather(data, idx, 1), go.gather(data, idx, 1))
+    table = rng.normal(0, 1, (100, 6, 4)).astype(np.float32)
+    rows = rng.integers(0, 100, 17).astype(idt)
+    np.testing.assert_array_equal(capi.gather(table, rows, 0), go.gather(table, rows, 0))
+
+
+@pytest.mark.parametrize("b,m,k,n", [(64, 27, 64, 27), (3, 5, 7, 9), (1, 1, 1, 1), (10, 32, 16, 8)])
+def test_batch_matmul(b, m, k, n):
+    rng = np.random.default_rng(b + m)
+    lhs = rng.integers(-128, 128, (b, m, k)).astype(np.int8)
+    rhs = rng.integers(-128, 128, (b, k, n)).astype(np.int8)
+    for oo, lo, ro, ratio in [(3, -4, 5, 0.004), (-128, 0, 0, 0.0007), (0, 127, -128, 0.02)]:
+        p = go.quantize_scale_offset_32to8(ratio, 0)[:3]
+        np.testing.assert_array_equal(capi.batch_matmul_i8(lhs, rhs, oo, lo, ro, p),
+                                      go.batch_matmul_i8(lhs, rhs, oo, lo, ro, p))
+
+
+def test_sigmoid():
+    rng = np.random.default_rng(5)
+    x = np.concatenate([rng.normal(0, 5, 10000), [0.0, 30.0, -30.0, 88.0, -88.0]]).astype(np.float32)
+    np.testing.assert_allclose(capi.sigmoid_f32(x), go.sigmoid_f32(x), rtol=1e-5, atol=1e-37)

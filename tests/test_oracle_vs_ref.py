@@ -178,3 +178,15 @@ def test_glue_ops_vs_ref():
                                           ref.avg_pool_i8(x, k, st, pd, cip, -3, 8, op))
     z = rng.normal(0, 4, (7, 333)).astype(np.float32)
     np.testing.assert_array_equal(go.softmax_f32(z), ref.softmax_f32(z))
+
+
+def test_ranking_glue_vs_ref():
+    rng = np.random.default_rng(78)
+    x = np.concatenate([rng.normal(0, 4, 500), [0.0, -0.0, 50.0, -50.0, 88.0, -88.0]]).astype(np.float32)
+    np.testing.assert_array_equal(go.sigmoid_f32(x), ref.sigmoid_f32(x))
+    data = rng.integers(-128, 128, (6, 20, 3)).astype(np.int8)
+    idx = rng.integers(0, 20, 9)
+    np.testing.assert_array_equal(go.gather(data, idx, 1).ravel(),
+                                  ref.gather64_i8(data, idx, 6, 60, 3))
+    np.testing.assert_array_equal(go.gather(data, idx, 1), np.take(data, idx, axis=1))
+    np.testing.assert_array_equal(go.gather(data, idx[:4] % 6, 0), data[idx[:4] % 6])
