@@ -52,12 +52,13 @@ def parse():
                     help="wall-clock budget of the CPU baseline leg")
     ap.add_argument("--resnet-batch", type=int, default=64)
     ap.add_argument("--resnet-profile-images", type=int, default=100)
+    ap.add_argument("--dlrm-rows", type=int, default=1_000_000)
     ap.add_argument("--no-extra", action="store_true",
                     help="headline workload only")
     ap.add_argument("--only", default="",
                     help="run a single extra kernel (profiling aid): "
                          "slws|fc_large|fc_c1|conv_c3|quantize|dequantize|"
-                         "rescale|copy|resnet50")
+                         "rescale|copy|resnet50|dlrm")
     return ap.parse_args()
 
 
@@ -307,6 +308,41 @@ def bench_elementwise(capi, which, steps, warmup):
                               traffic=None))
 
 
+def cpu_baseline_mfma_kernels(budget_s):
+    """The oracle (the restated libjit loops, one thread) on the single-FC
+    configuration and on a bounded slice of the ResNet 3x3 convolution: the
+    reference's CPU path for the two matrix-core workloads."""
+    from oracle import glow_oracle as go
+    from tests import cases as ocases
+    out = {}
+    c = ocases.rwq_fc_case(5, 128, 1024, 1024)
+    args_ = ocases.rwq_fc_args(c)
+    n, t0 = 0, time.perf_counter()
+    while True:
+        go.rwq_fc_i8(*args_)
+        n += 1
+        el = time.perf_counter() - t0
+        if el >= budget_s / 2 or n >= 200:
+            break
+    out["rwq_fc_c1"] = dict(value=2.0 * 128 * 1024 * 1024 * n / el / 1e9, unit="GOP/s", cores=1,
+                            kind="port", sample=f"{n} full passes of M128 K1024 N1024 in {el:.1f} s")
+    # two images of the 32-image batch (same layer shape), repeated
+    cc = ocases.cwq_conv_case(7, 2, 56, 56, 64, 64, in_offset=-128)
+    cargs = ocases.cwq_conv_args(cc)
+    n, t0 = 0, time.perf_counter()
+    while True:
+        go.cwq_conv2d_i8(*cargs)
+        n += 1
+        el = time.perf_counter() - t0
+        if el >= budget_s / 2 or n >= 200:
+            break
+    out["cwq_conv_c3"] = dict(value=2.0 * 2 * 56 * 56 * 64 * 576 * n / el / 1e9, unit="GOP/s",
+                              cores=1, kind="port",
+                              sample=f"{n} passes over 2 of the 32 images (56x56x64, 3x3x64->64) "
+                                     f"in {el:.1f} s")
+    return out
+
+
 def bench_resnet50(args):
     """Int8 ResNet-50 at batch 64, 224x224 through MI355XDeviceManager:
     images/s of the resident network replayed on device-resident input
@@ -348,6 +384,46 @@ def bench_resnet50(args):
                 prob_row_sum=float(prob[0].sum()), host_build_seconds=t_build)
 
 
+def bench_dlrm(args):
+    """DLRM-style ranking net, batch 4096: 26 tables of 1M x 64 (4-bit fused,
+    fp16 scale/offset), Poisson(20) bags of Zipf(1.1) int64 indices, int8 MLPs
+    13-512-256-64 and 415-512-256-1, dot interaction, sigmoid."""
+    from glow_amd import host as H
+    from glow_amd.harness import dlrm
+    from glow_amd.harness import net as netlib
+    batch, tables = 4096, 26
+    t0 = time.perf_counter()
+    net, max_idx = dlrm.make(tables=tables, rows=args.dlrm_rows, batch=batch)
+    t_build = time.perf_counter() - t0
+    m, f = netlib.to_module(net)
+    m.compile(f)
+    dm = H.DeviceManager().init()
+    try:
+        dm.add_network(m)
+        inp = dlrm.Inputs(99, tables, args.dlrm_rows, batch, 20, 1.1, 13)
+        b = dlrm.bindings(net, inp, max_idx)
+        prob = np.zeros((batch, 1), np.float32)
+        dm.run("main", dict(b, prob=prob))
+        reps = max(5, args.steps // 4)
+        ms = dm.time_function("main", reps)
+        t1 = time.perf_counter()
+        for _ in range(3):
+            dm.run("main", dict(b, prob=prob))
+        e2e = (time.perf_counter() - t1) / 3
+    finally:
+        dm.stop()
+    lookups = int(sum(int(l.sum()) for l in inp.lengths))
+    sls_bytes = lookups * (36 + 8) + tables * batch * (4 + 64 * 2)
+    return dict(workload=f"DLRM-style net, batch {batch}, {tables} tables x {args.dlrm_rows} rows x 64 "
+                         "(4-bit fused, fp16 scale/offset), Poisson(20) bags, Zipf(1.1) int64 indices",
+                samples_per_s=batch / (ms * 1e-3), ms_per_batch=ms,
+                samples_per_s_with_host_copies=batch / e2e,
+                lookups_per_batch=lookups, sls_algorithmic_mb_per_batch=sls_bytes / 1e6,
+                launches_per_batch=len([r for r in H.parse_listing(m.describe(f))
+                                        if r["phase"] == "launch"]),
+                prob_mean=float(prob.mean()), host_build_seconds=t_build)
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -361,6 +437,9 @@ def main():
 
     if args.only == "resnet50":
         print(json.dumps(bench_resnet50(args)))
+        return
+    if args.only == "dlrm":
+        print(json.dumps(bench_dlrm(args)))
         return
 
     capi.init(0)
@@ -400,12 +479,14 @@ def main():
         if args.cpu_seconds > 0:
             extra["cpu_all_cores"] = cpu_all_cores_slws(table, s["batches"],
                                                         args.cpu_seconds / 2)
+            extra["cpu_mfma_kernels"] = cpu_baseline_mfma_kernels(args.cpu_seconds / 2)
         extra["rwq_fc_c1"] = bench_fc(capi, cases, 128, 1024, 1024, args.steps, args.warmup)
         extra["rwq_fc_large"] = bench_fc(capi, cases, 8192, 4096, 4096, st, wu)
         extra["cwq_conv_c3"] = bench_conv(capi, cases, args.steps, args.warmup)
         for w in ("quantize", "dequantize", "rescale"):
             extra[w] = bench_elementwise(capi, w, st, wu)
         extra["resnet50_int8"] = bench_resnet50(args)
+        extra["dlrm_int8"] = bench_dlrm(args)
 
     out = {
         "metric": "FusedRowwiseQuantizedSLWS algorithmic GB/s (1 GPU)",

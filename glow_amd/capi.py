@@ -28,7 +28,7 @@ EXPORTS = [
     "mi355x_batch_transpose_i8", "mi355x_gather", "mi355x_batch_matmul_i8", "mi355x_sigmoid_f32",
     "mi355x_max_pool_i8", "mi355x_avg_pool_i8", "mi355x_softmax_f32", "mi355x_stream_create",
     "mi355x_stream_destroy", "mi355x_stream_sync", "mi355x_device_sync",
-    "mi355x_event_create", "mi355x_event_destroy", "mi355x_event_record",
+    "mi355x_event_create", "mi355x_event_destroy", "mi355x_event_record", "mi355x_stream_wait_event",
     "mi355x_event_sync", "mi355x_event_elapsed_ms", "mi355x_arena_create",
     "mi355x_arena_destroy", "mi355x_arena_ptr", "mi355x_arena_upload",
     "mi355x_arena_download", "mi355x_arena_bytes",

@@ -244,6 +244,12 @@ int mi355x_event_record(void *event, void *stream) {
   return MI355X_OK;
 }
 
+int mi355x_stream_wait_event(void *stream, void *event) {
+  MI355X_REQUIRE(event, "event is NULL");
+  MI355X_HIP(hipStreamWaitEvent(as_stream(stream), (hipEvent_t)event, 0));
+  return MI355X_OK;
+}
+
 int mi355x_event_sync(void *event) {
   MI355X_REQUIRE(event, "event is NULL");
   MI355X_HIP(hipEventSynchronize((hipEvent_t)event));

@@ -6,6 +6,7 @@
 
 #include "glow_mi355x.h"
 
+#include <algorithm>
 #include <cmath>
 #include <sstream>
 
@@ -94,6 +95,7 @@ public:
     for (const auto &I : insts_) MI355X_RETURN_IF_ERR(checkOperands(I));
     for (size_t at = 0; at < insts_.size(); at++) {
       const Instruction &I = insts_[at];
+      const size_t firstLaunch = out.launches.size(), firstInst = at;
       switch (I.kind) {
       case Kind::ElementAdd: {
         // an add whose only reader is the Relu right behind it becomes one pass
@@ -154,7 +156,11 @@ public:
         return MI355X_MAKE_ERR(ErrorCode::COMPILE_UNSUPPORTED_NODE_AFTER_OPTIMIZE,
                                "instruction kind %d is not supported", (int)I.kind);
       }
+      // what the launches of instructions [firstInst, at] read and write
+      for (size_t l = firstLaunch; l < out.launches.size(); l++)
+        for (size_t k = firstInst; k <= at; k++) noteAccesses(insts_[k], out.launches[l]);
     }
+    assignLevels(out);
     // scratch buffers follow the initialised image
     scratchBase_ = alignUp(gen_.image_.size(), 256);
     *scratchBasePtr_ = scratchBase_;
@@ -190,6 +196,53 @@ private:
   }
 
   Operand op(const Instruction &I, int i) const { return Operand{&M_.value(I.operands[(size_t)i])}; }
+
+  void noteAccesses(const Instruction &J, KernelLaunch &L) const {
+    // pooled lookups over more than 4096 bags go through a per-device scratch
+    // buffer inside the kernel library: such launches must not overlap
+    if ((J.kind == Kind::FusedRowwiseQuantizedSparseLengthsWeightedSum ||
+         J.kind == Kind::FusedRowwiseQuantizedSparseLengthsSum) &&
+        M_.value(J.operands.back()).type.size() > 4096) {
+      Access shared;
+      shared.root = -2;
+      L.writes.push_back(shared);
+    }
+    for (size_t i = 0; i < J.operands.size(); i++) {
+      const Value &v = M_.value(J.operands[i]);
+      Access a;
+      a.root = v.root;
+      if (J.kind == Kind::InsertTensor && i == 0 && v.type.dims.size() == 2) {
+        // only the columns [offset, offset + width) of each row are written
+        const Value &src = M_.value(J.operands[1]);
+        const long long es = (long long)elemSize(v.type.kind);
+        a.lo = J.iattrs.empty() ? 0 : J.iattrs[0] * es;
+        a.hi = a.lo + (src.type.dims.size() == 2 ? src.type.dims[1] * es : 0);
+        if (v.id != v.root) a.hi = -1; // a view's rows need not line up with its source's
+      }
+      (i == 0 ? L.writes : L.reads).push_back(a);
+    }
+  }
+
+  static bool conflict(const KernelLaunch &early, const KernelLaunch &late) {
+    for (const auto &w : early.writes) {
+      for (const auto &r : late.reads) if (w.overlaps(r)) return true;   // read after write
+      for (const auto &x : late.writes) if (w.overlaps(x)) return true;  // write after write
+    }
+    for (const auto &r : early.reads)
+      for (const auto &w : late.writes) if (r.overlaps(w)) return true;  // write after read
+    return false;
+  }
+
+  // level = longest chain of conflicting launches in front of a launch
+  static void assignLevels(MI355XFunction &out) {
+    auto &L = out.launches;
+    for (size_t i = 0; i < L.size(); i++) {
+      int lvl = 0;
+      for (size_t j = 0; j < i; j++)
+        if (L[j].level >= lvl && conflict(L[j], L[i])) lvl = L[j].level + 1;
+      L[i].level = lvl;
+    }
+  }
 
   // number of operands that read the memory of `id` (through it or a view)
   int readers(int id) const {
@@ -983,24 +1036,64 @@ static bool sameBindings(const DeviceBindings &a, const DeviceBindings &b) {
          a.mutableMem == b.mutableMem && a.activations == b.activations;
 }
 
-Error MI355XFunction::captureGraph(const DeviceBindings &b) {
+Error MI355XFunction::captureGraph(const DeviceBindings &b, const std::vector<void *> &sideStreams) {
   dropGraph();
   if (launches.empty()) return Error::success();
   if (!b.stream)
     return MI355X_MAKE_ERR(ErrorCode::RUNTIME_ERROR, "graph capture needs a created stream");
-  if (mi355x_graph_begin_capture(b.stream) != MI355X_OK)
+  // launches grouped by dependence level, in program order inside a level
+  int levels = 0;
+  for (const auto &l : launches) levels = std::max(levels, l.level + 1);
+  std::vector<std::vector<const KernelLaunch *>> byLevel((size_t)levels);
+  for (const auto &l : launches) byLevel[(size_t)l.level].push_back(&l);
+  const size_t nSide = sideStreams.size();
+  // one fork event, and one join event per side stream
+  void *fork = nullptr;
+  std::vector<void *> joins(nSide, nullptr);
+  auto cleanup = [&] {
+    if (fork) mi355x_event_destroy(fork);
+    for (void *e : joins) if (e) mi355x_event_destroy(e);
+  };
+  if (nSide) {
+    int rc = mi355x_event_create(&fork);
+    for (size_t i = 0; i < nSide && rc == MI355X_OK; i++) rc = mi355x_event_create(&joins[i]);
+    if (rc != MI355X_OK) {
+      cleanup();
+      return MI355X_MAKE_ERR(ErrorCode::RUNTIME_ERROR, "%s", mi355x_last_error());
+    }
+  }
+  if (mi355x_graph_begin_capture(b.stream) != MI355X_OK) {
+    cleanup();
     return MI355X_MAKE_ERR(ErrorCode::RUNTIME_ERROR, "%s", mi355x_last_error());
+  }
   int rc = MI355X_OK;
   std::string failed;
-  for (const auto &l : launches) {
-    rc = l.run(b);
+  for (const auto &group : byLevel) {
+    const size_t branches = std::min(group.size(), nSide + 1);
+    if (branches > 1) {
+      rc = mi355x_event_record(fork, b.stream);
+      for (size_t s = 0; s + 1 < branches && rc == MI355X_OK; s++)
+        rc = mi355x_stream_wait_event(sideStreams[s], fork);
+    }
+    for (size_t i = 0; i < group.size() && rc == MI355X_OK; i++) {
+      DeviceBindings bb = b;
+      const size_t lane = i % branches;       // 0 = the capturing stream itself
+      if (lane) bb.stream = sideStreams[lane - 1];
+      rc = group[i]->run(bb);
+      if (rc != MI355X_OK) failed = group[i]->kernel + " (" + group[i]->inst + "): " + mi355x_last_error();
+    }
+    for (size_t s = 0; s + 1 < branches && rc == MI355X_OK; s++) {
+      rc = mi355x_event_record(joins[s], sideStreams[s]);
+      if (rc == MI355X_OK) rc = mi355x_stream_wait_event(b.stream, joins[s]);
+    }
     if (rc != MI355X_OK) {
-      failed = l.kernel + " (" + l.inst + "): " + mi355x_last_error();
+      if (failed.empty()) failed = mi355x_last_error();
       break;
     }
   }
   mi355x_graph *g = nullptr;
   const int rc2 = mi355x_graph_end_capture(b.stream, &g);
+  cleanup();
   if (rc != MI355X_OK) {
     if (g) mi355x_graph_destroy(g);
     return MI355X_MAKE_ERR(ErrorCode::RUNTIME_ERROR, "%s", failed.c_str());
@@ -1039,7 +1132,8 @@ std::string MI355XFunction::describe() const {
      << " mutable=" << bundle_.mutableWeightVarsMemSize
      << " activations=" << bundle_.activationsMemSize << "\n";
   for (const auto &l : setup) os << "setup " << l.kernel << " inst=" << l.inst << l.params << "\n";
-  for (const auto &l : launches) os << "launch " << l.kernel << " inst=" << l.inst << l.params << "\n";
+  for (const auto &l : launches)
+    os << "launch " << l.kernel << " inst=" << l.inst << " level=" << l.level << l.params << "\n";
   return os.str();
 }
 

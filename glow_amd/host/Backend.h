@@ -73,12 +73,31 @@ struct RuntimeBundle {
   }
 };
 
+// Memory a launch touches: the value (by its root, so views alias) and, for
+// slices inserted into rows of a wider tensor, the byte range inside a row.
+struct Access {
+  int root = -1;
+  long long lo = 0, hi = -1; // hi < 0: the whole value
+  bool overlaps(const Access &o) const {
+    if (root != o.root) return false;
+    if (hi < 0 || o.hi < 0) return true;
+    return lo < o.hi && o.lo < hi;
+  }
+};
+
 // One kernel launch of a compiled function.
 struct KernelLaunch {
+  KernelLaunch(std::string k, std::string i, std::string p,
+               std::function<int(const struct DeviceBindings &)> r)
+      : kernel(std::move(k)), inst(std::move(i)), params(std::move(p)), run(std::move(r)) {}
   std::string kernel;  // C-ABI entry point
   std::string inst;    // instruction name
   std::string params;  // the derived integer parameters, for inspection
   std::function<int(const DeviceBindings &)> run; // returns an mi355x_status
+  // Dependence information: launches of one level touch disjoint memory (or
+  // only read common memory) and may run side by side.
+  std::vector<Access> reads, writes;
+  int level = 0;
 };
 
 class MI355XFunction {
@@ -104,8 +123,9 @@ public:
   std::string describe() const;
 
   // Records the body into a launch graph bound to these buffers; later
-  // execute() calls with the same bindings replay it.
-  Error captureGraph(const DeviceBindings &b);
+  // execute() calls with the same bindings replay it. With side streams the
+  // launches of one dependence level are recorded as parallel branches.
+  Error captureGraph(const DeviceBindings &b, const std::vector<void *> &sideStreams = {});
   void dropGraph();
 
 private:

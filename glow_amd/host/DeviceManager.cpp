@@ -67,6 +67,11 @@ Error MI355XDeviceManager::init() {
     mi355x_info info;
     rc = mi355x_device_info(&info);
     if (rc == MI355X_OK) rc = mi355x_stream_create(&stream_);
+    for (int i = 1; i < config_.graphBranches && rc == MI355X_OK; i++) {
+      void *s = nullptr;
+      rc = mi355x_stream_create(&s);
+      if (rc == MI355X_OK) sideStreams_.push_back(s);
+    }
     if (rc != MI355X_OK) {
       done.set_value(fromStatus(rc, "device set-up"));
       return;
@@ -103,6 +108,8 @@ Error MI355XDeviceManager::stop(bool block) {
       mi355x_stream_destroy(stream_);
       stream_ = nullptr;
     }
+    for (void *s : sideStreams_) mi355x_stream_destroy(s);
+    sideStreams_.clear();
     done.set_value();
   });
   fut.get();
@@ -295,7 +302,7 @@ Error MI355XDeviceManager::makeResident(const Module *module, const std::string 
     }
     rc = mi355x_stream_sync(stream_);
     if (rc != MI355X_OK) return failWith(fromStatus(rc, "first pass"));
-    Error e = fn->captureGraph(fr.bindings);
+    Error e = fn->captureGraph(fr.bindings, sideStreams_);
     if (e) return failWith(std::move(e));
   }
   functions_.emplace(name, fr);

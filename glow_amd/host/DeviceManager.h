@@ -32,6 +32,7 @@ struct DeviceConfig {
   int deviceID = 0;
   uint64_t deviceMemory = 0;  // 0 = what the device reports as free at init
   bool useLaunchGraphs = true; // record each function once, replay per run
+  int graphBranches = 4;       // independent launches recorded side by side (1 = a chain)
 };
 
 struct DeviceInfo {
@@ -101,6 +102,7 @@ private:
   std::map<std::string, FunctionResident> functions_;
   std::map<const Module *, ModuleResident> modules_;
   void *stream_ = nullptr;
+  std::vector<void *> sideStreams_; // branches of captured graphs
 
   std::thread worker_;
   std::mutex mu_;

@@ -89,6 +89,9 @@ int mi355x_device_sync(void);
 int mi355x_event_create(void **event);
 int mi355x_event_destroy(void *event);
 int mi355x_event_record(void *event, void *stream);
+/* Work queued on `stream` after this call waits for `event`. Inside a graph
+ * capture this makes `stream` a branch of the captured graph. */
+int mi355x_stream_wait_event(void *stream, void *event);
 int mi355x_event_sync(void *event);
 int mi355x_event_elapsed_ms(void *start, void *stop, float *ms);
 

@@ -122,7 +122,11 @@ int mi355x_host_describe(mi355x_host_module *m, int function, char *buf, size_t 
 /* RuntimeBundle sizes: out = {constants, generated, mutable, activations}. */
 int mi355x_host_bundle_sizes(mi355x_host_module *m, int function, uint64_t out[4]);
 
-/* DeviceManager. memory_bytes 0 = what the device reports free. */
+/* DeviceManager. memory_bytes 0 = what the device reports free.
+ * use_launch_graphs: 0 = launch kernel by kernel; 1 = record each function as a
+ * launch graph whose independent launches form parallel branches (default
+ * width); n > 1 = the same with up to n branches (n = 2 ... ; a chain needs
+ * the C++ DeviceConfig). */
 mi355x_host_dm *mi355x_host_dm_create(int device, uint64_t memory_bytes, int use_launch_graphs);
 void mi355x_host_dm_destroy(mi355x_host_dm *dm);
 int mi355x_host_dm_init(mi355x_host_dm *dm);
