@@ -8,7 +8,7 @@
 
 namespace mi355x {
 
-int g_tile_override = -1;
+thread_local int g_tile_override = -1;
 
 // dst [cols x rows] = src [rows x cols]^T through a 64x64 LDS tile.
 __global__ __launch_bounds__(256) void transpose2d_i8_kernel(
@@ -87,7 +87,7 @@ using namespace mi355x;
 extern "C" {
 
 int mi355x_gemm_tile_override(int tile) {
-  MI355X_REQUIRE(tile >= -1 && tile <= 3, "tile %d outside [-1, 3]", tile);
+  MI355X_REQUIRE(tile >= -1 && tile <= 5, "tile %d outside [-1, 5]", tile);
   g_tile_override = tile;
   return MI355X_OK;
 }

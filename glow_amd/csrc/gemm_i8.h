@@ -458,7 +458,8 @@ __device__ __forceinline__ uint32_t lds_address(const void *p) {
 
 template <int BM, int BN, int WM, int WN, int STAGES, bool NEED_SA,
           bool NEED_SB, class ARows>
-__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_i8_dma_kernel(
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
+                             (BM * BN == 256 * 128) ? 2 : 1) void gemm_i8_dma_kernel(
     ARows A, DenseRows B, Epilogue ep, int M, int N, int K, int tiles_m,
     int tiles_n, long long b_group_stride, int n_per_group) {
   constexpr int WAVES_N = BN / WN;
@@ -721,14 +722,15 @@ static int gemm_dma_launch(const ARows &A, const DenseRows &B,
 // Tile choice from the problem size: 256x256 for large problems (a wave owns
 // 128x128, which halves LDS traffic per MFMA), smaller tiles when the grid
 // would otherwise not fill 256 CUs.
-enum class Tile { T256, T128, T128x64, T64 };
-// Tuning aid: a value in [0, 3] forces that tile for every following launch.
-extern int g_tile_override;
+enum class Tile { T256, T128, T128x64, T64, T256x128, T128x256 };
+// Tuning aid: a value in [0, 5] forces that tile for the following launches of
+// the calling thread.
+extern thread_local int g_tile_override;
 static Tile pick_tile(const GemmShape &g, size_t lds_256) {
   auto tiles = [&](int bm, int bn) {
     return (long long)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * g.groups;
   };
-  if (g_tile_override >= 0 && g_tile_override <= 3 &&
+  if (g_tile_override >= 0 && g_tile_override <= 5 &&
       (g_tile_override != 0 || lds_256 <= lds_limit()))
     return (Tile)g_tile_override;
   // Measured on the convolution shapes of ResNet-50 and on large FCs: the
@@ -738,6 +740,9 @@ static Tile pick_tile(const GemmShape &g, size_t lds_256) {
   if (tiles(256, 256) >= 256 && g.N >= 256 && g.K >= 1024 &&
       lds_256 <= lds_limit())
     return Tile::T256;
+  // short K loops with wide outputs: 256x128 tiles, two workgroups per CU, so
+  // one workgroup's epilogue overlaps the other's loads
+  if (tiles(256, 128) >= 256 && g.N >= 256 && g.K <= 512) return Tile::T256x128;
   if (tiles(128, 128) >= 256 && g.N >= 128 && g.K >= 512) return Tile::T128;
   if (tiles(128, 64) >= 256) return Tile::T128x64;
   if (tiles(64, 64) >= 256 || g.M < 1024) return Tile::T64;
@@ -754,6 +759,10 @@ static int gemm_dma_tiles(const ARows &A, const DenseRows &B, const Epilogue &ep
     return gemm_dma_launch<128, 128, 64, 64, 3, SA, SB>(A, B, ep, g, st);
   case Tile::T128x64:
     return gemm_dma_launch<128, 64, 32, 64, 3, SA, SB>(A, B, ep, g, st);
+  case Tile::T256x128:
+    return gemm_dma_launch<256, 128, 128, 64, 3, SA, SB>(A, B, ep, g, st);
+  case Tile::T128x256:
+    return gemm_dma_launch<128, 256, 64, 128, 3, SA, SB>(A, B, ep, g, st);
   default:
     return gemm_dma_launch<64, 64, 32, 32, 4, SA, SB>(A, B, ep, g, st);
   }
@@ -770,6 +779,9 @@ static int gemm_staged_tiles(const ARows &A, const DenseRows &B,
     return gemm_launch<128, 128, 64, 64, AL_A, AL_B>(A, B, ep, g, st);
   case Tile::T128x64:
     return gemm_launch<128, 64, 32, 64, AL_A, AL_B>(A, B, ep, g, st);
+  case Tile::T256x128:
+  case Tile::T128x256:
+    return gemm_launch<128, 128, 64, 64, AL_A, AL_B>(A, B, ep, g, st);
   default:
     return gemm_launch<64, 64, 32, 32, AL_A, AL_B>(A, B, ep, g, st);
   }

@@ -157,8 +157,13 @@ public:
                                "instruction kind %d is not supported", (int)I.kind);
       }
       // what the launches of instructions [firstInst, at] read and write
-      for (size_t l = firstLaunch; l < out.launches.size(); l++)
+      for (size_t l = firstLaunch; l < out.launches.size(); l++) {
         for (size_t k = firstInst; k <= at; k++) noteAccesses(insts_[k], out.launches[l]);
+        const std::string &kn = out.launches[l].kernel;
+        out.launches[l].tunable = kn == "mi355x_fc_i8" || kn == "mi355x_rwq_fc_i8" ||
+                                  kn == "mi355x_matmul_i8" || kn == "mi355x_conv2d_i8" ||
+                                  kn == "mi355x_cwq_conv2d_i8" || kn == "mi355x_cwq_conv2d_add_i8";
+      }
     }
     assignLevels(out);
     // scratch buffers follow the initialised image
@@ -1022,6 +1027,14 @@ unsigned MI355XBackend::numDevices() {
   return n < 0 ? 0u : (unsigned)n;
 }
 
+int KernelLaunch::launch(const DeviceBindings &b) const {
+  if (!tunable || tile < 0) return run(b);
+  mi355x_gemm_tile_override(tile);
+  const int rc = run(b);
+  mi355x_gemm_tile_override(-1);
+  return rc;
+}
+
 MI355XFunction::~MI355XFunction() { dropGraph(); }
 
 void MI355XFunction::dropGraph() {
@@ -1079,7 +1092,7 @@ Error MI355XFunction::captureGraph(const DeviceBindings &b, const std::vector<vo
       DeviceBindings bb = b;
       const size_t lane = i % branches;       // 0 = the capturing stream itself
       if (lane) bb.stream = sideStreams[lane - 1];
-      rc = group[i]->run(bb);
+      rc = group[i]->launch(bb);
       if (rc != MI355X_OK) failed = group[i]->kernel + " (" + group[i]->inst + "): " + mi355x_last_error();
     }
     for (size_t s = 0; s + 1 < branches && rc == MI355X_OK; s++) {
@@ -1116,7 +1129,7 @@ Error MI355XFunction::execute(ExecutionContext *ctx) {
     return Error::success();
   }
   for (const auto &l : launches) {
-    const int rc = l.run(*b);
+    const int rc = l.launch(*b);
     if (rc != MI355X_OK)
       return MI355X_MAKE_ERR(rc == MI355X_ERR_NOT_SUPPORTED ? ErrorCode::DEVICE_FEATURE_NOT_SUPPORTED
                                                             : ErrorCode::RUNTIME_ERROR,
@@ -1133,7 +1146,8 @@ std::string MI355XFunction::describe() const {
      << " activations=" << bundle_.activationsMemSize << "\n";
   for (const auto &l : setup) os << "setup " << l.kernel << " inst=" << l.inst << l.params << "\n";
   for (const auto &l : launches)
-    os << "launch " << l.kernel << " inst=" << l.inst << " level=" << l.level << l.params << "\n";
+    os << "launch " << l.kernel << " inst=" << l.inst << " level=" << l.level << " tile=" << l.tile
+       << l.params << "\n";
   return os.str();
 }
 

@@ -98,7 +98,14 @@ struct KernelLaunch {
   // only read common memory) and may run side by side.
   std::vector<Access> reads, writes;
   int level = 0;
+  // Matrix-core launches can run with several workgroup tiles; `tile` is the
+  // one to use (-1: the library's choice from the shape).
+  bool tunable = false;
+  int tile = -1;
+  // Issues the launch (with its tile, if it has one).
+  int launch(const DeviceBindings &b) const;
 };
+constexpr int kNumTiles = 6;
 
 class MI355XFunction {
 public:

@@ -297,16 +297,56 @@ Error MI355XDeviceManager::makeResident(const Module *module, const std::string 
     // one eager pass first: entry points that allocate on first use must have
     // run before they are recorded
     for (const auto &l : fn->launches) {
-      rc = l.run(fr.bindings);
+      rc = l.launch(fr.bindings);
       if (rc != MI355X_OK) return failWith(fromStatus(rc, l.kernel.c_str()));
     }
     rc = mi355x_stream_sync(stream_);
     if (rc != MI355X_OK) return failWith(fromStatus(rc, "first pass"));
+    if (config_.autotuneTiles) {
+      Error te = tuneTiles(fn, fr.bindings);
+      if (te) return failWith(std::move(te));
+    }
     Error e = fn->captureGraph(fr.bindings, sideStreams_);
     if (e) return failWith(std::move(e));
   }
   functions_.emplace(name, fr);
   return Error::success();
+}
+
+// For every matrix-core launch: run each tile a few times on the resident data
+// and keep the fastest (results do not depend on the tile).
+Error MI355XDeviceManager::tuneTiles(MI355XFunction *fn, const DeviceBindings &b) {
+  void *e0 = nullptr, *e1 = nullptr;
+  int rc = mi355x_event_create(&e0);
+  if (rc == MI355X_OK) rc = mi355x_event_create(&e1);
+  Error err;
+  constexpr int kRuns = 4;
+  for (auto &l : fn->launches) {
+    if (!l.tunable || rc != MI355X_OK) continue;
+    float best = 0.0f;
+    int bestTile = -1;
+    for (int t = -1; t < kNumTiles && rc == MI355X_OK; t++) {
+      l.tile = t;
+      rc = l.launch(b); // warm-up, also rejects tiles the shape cannot use
+      if (rc != MI355X_OK) { rc = MI355X_OK; continue; }
+      rc = mi355x_event_record(e0, stream_);
+      for (int i = 0; i < kRuns && rc == MI355X_OK; i++) rc = l.launch(b);
+      if (rc == MI355X_OK) rc = mi355x_event_record(e1, stream_);
+      if (rc == MI355X_OK) rc = mi355x_event_sync(e1);
+      float ms = 0.0f;
+      if (rc == MI355X_OK) rc = mi355x_event_elapsed_ms(e0, e1, &ms);
+      if (rc == MI355X_OK && (bestTile == -1 && t == -1 ? true : ms < best)) {
+        best = ms;
+        bestTile = t;
+      }
+    }
+    l.tile = bestTile;
+  }
+  if (rc != MI355X_OK) err = fromStatus(rc, "tile tuning");
+  if (e0) mi355x_event_destroy(e0);
+  if (e1) mi355x_event_destroy(e1);
+  mi355x_stream_sync(stream_);
+  return err;
 }
 
 void MI355XDeviceManager::addNetworkImpl(const Module *module, FunctionMapTy functions,

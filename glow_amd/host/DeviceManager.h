@@ -33,6 +33,7 @@ struct DeviceConfig {
   uint64_t deviceMemory = 0;  // 0 = what the device reports as free at init
   bool useLaunchGraphs = true; // record each function once, replay per run
   int graphBranches = 4;       // independent launches recorded side by side (1 = a chain)
+  bool autotuneTiles = true;   // time the tile candidates of each matrix-core launch at load
 };
 
 struct DeviceInfo {
@@ -91,6 +92,7 @@ private:
   void runFunctionImpl(RunIdentifierTy id, std::string functionName,
                        std::unique_ptr<ExecutionContext> ctx, ResultCBTy resultCB);
   Error makeResident(const Module *module, const std::string &name, MI355XFunction *fn);
+  Error tuneTiles(MI355XFunction *fn, const DeviceBindings &b);
   void release(FunctionResident &fr);
   void enqueue(std::function<void()> work);
   void workerLoop();
