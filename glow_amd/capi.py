@@ -25,7 +25,7 @@ EXPORTS = [
     "mi355x_memcpy_d2d", "mi355x_fill_u8", "mi355x_copy_u8", "mi355x_gemm_tile_override",
     "mi355x_cwq_conv2d_add_i8", "mi355x_add_i8", "mi355x_add_relu_i8",
     "mi355x_relu_i8", "mi355x_convert_f16_to_f32", "mi355x_insert_rows",
-    "mi355x_batch_transpose_i8", "mi355x_gather", "mi355x_batch_matmul_i8", "mi355x_sigmoid_f32",
+    "mi355x_batch_transpose_i8", "mi355x_space_to_depth2_i8", "mi355x_gather", "mi355x_batch_matmul_i8", "mi355x_sigmoid_f32",
     "mi355x_max_pool_i8", "mi355x_avg_pool_i8", "mi355x_softmax_f32", "mi355x_stream_create",
     "mi355x_stream_destroy", "mi355x_stream_sync", "mi355x_device_sync",
     "mi355x_event_create", "mi355x_event_destroy", "mi355x_event_record", "mi355x_stream_wait_event",
@@ -878,4 +878,15 @@ def sigmoid_f32(x):
     dx = to_device(x)
     out = DeviceBuffer.empty(x.shape, np.float32)
     check(lib().mi355x_sigmoid_f32(_vp(out), _vp(dx), _sz(x.size), _vp(None)))
+    return out.numpy()
+
+
+def space_to_depth2_i8(x, pad_t, pad_l, bh, bw, cout, fill):
+    x = np.ascontiguousarray(x, np.int8)
+    n, ih, iw, c = x.shape
+    dx = to_device(x)
+    out = DeviceBuffer.empty((n, bh, bw, cout), np.int8)
+    check(lib().mi355x_space_to_depth2_i8(_vp(out), _vp(dx), _sz(n), _sz(ih), _sz(iw), _sz(c),
+                                          _sz(pad_t), _sz(pad_l), _sz(bh), _sz(bw), _sz(cout),
+                                          _i32(fill), _vp(None)))
     return out.numpy()

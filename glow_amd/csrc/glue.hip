@@ -332,6 +332,28 @@ __global__ __launch_bounds__(kGlueThreads) void batch_matmul_i8_kernel(
   }
 }
 
+// dst[n][bh][bw][(dh*2+dw)*C + c] = src[n][2bh+dh-padT][2bw+dw-padL][c]; positions
+// outside the image and channels from 4C up hold `fill`. One thread per
+// destination pixel.
+__global__ __launch_bounds__(kGlueThreads) void space_to_depth2_i8_kernel(
+    int8_t *__restrict__ dst, const int8_t *__restrict__ src, int N, int IH, int IW, int C,
+    int padT, int padL, int BH, int BW, int Cout, int fill, long long total) {
+  const long long t = (long long)blockIdx.x * kGlueThreads + threadIdx.x;
+  if (t >= total) return;
+  const int bw = (int)(t % BW);
+  long long r = t / BW;
+  const int bh = (int)(r % BH);
+  const int n = (int)(r / BH);
+  int8_t *d = dst + t * Cout;
+  for (int q = 0; q < 4; q++) {
+    const int ih = 2 * bh + (q >> 1) - padT, iw = 2 * bw + (q & 1) - padL;
+    const bool in = ih >= 0 && ih < IH && iw >= 0 && iw < IW;
+    const int8_t *p = src + (((long long)n * IH + (in ? ih : 0)) * IW + (in ? iw : 0)) * C;
+    for (int c = 0; c < C; c++) d[q * C + c] = in ? p[c] : (int8_t)fill;
+  }
+  for (int c = 4 * C; c < Cout; c++) d[c] = (int8_t)fill;
+}
+
 // libjit_sigmoid_kernel_f: 1 / (expf(-x) + 1)
 __global__ __launch_bounds__(kGlueThreads) void sigmoid_f32_kernel(
     float *__restrict__ dst, const float *__restrict__ src, size_t n) {
@@ -555,6 +577,24 @@ int mi355x_batch_matmul_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs, si
                      as_stream(stream), out, lhs, rhs, (int)M, (int)K, (int)N, out_offset,
                      lhs_offset, rhs_offset, out_pre, out_post, out_scale);
   return check_launch("batch_matmul_i8");
+}
+
+int mi355x_space_to_depth2_i8(int8_t *dst, const int8_t *src, size_t N, size_t IH, size_t IW,
+                              size_t C, size_t padT, size_t padL, size_t BH, size_t BW,
+                              size_t Cout, int32_t fill, void *stream) {
+  if (N == 0 || BH == 0 || BW == 0) return MI355X_OK;
+  MI355X_REQUIRE(dst && src, "NULL tensor");
+  MI355X_REQUIRE(C > 0 && Cout >= 4 * C && Cout < 4096, "needs 4*C <= Cout < 4096");
+  const size_t lim = 1u << 30;
+  MI355X_REQUIRE(N < lim && IH < lim && IW < lim && BH < lim && BW < lim && padT < lim && padL < lim,
+                 "dimensions too large");
+  MI355X_REQUIRE(fill >= -128 && fill <= 127, "fill outside the int8 range");
+  const long long total = (long long)N * BH * BW;
+  MI355X_REQUIRE(total / kGlueThreads < 0x7fffffffLL, "tensor too large");
+  hipLaunchKernelGGL(space_to_depth2_i8_kernel, dim3(glue_blocks((size_t)total)),
+                     dim3(kGlueThreads), 0, as_stream(stream), dst, src, (int)N, (int)IH, (int)IW,
+                     (int)C, (int)padT, (int)padL, (int)BH, (int)BW, (int)Cout, fill, total);
+  return check_launch("space_to_depth2_i8");
 }
 
 int mi355x_sigmoid_f32(float *dst, const float *src, size_t n, void *stream) {

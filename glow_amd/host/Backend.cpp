@@ -40,6 +40,12 @@ public:
     std::memcpy(image_.data() + off, v.data(), v.size() * 4);
     return off;
   }
+  size_t addBytes(const std::vector<int8_t> &v) {
+    const size_t off = image_.size();
+    image_.resize(alignUp(off + v.size(), kTensorAlignment), 0);
+    std::memcpy(image_.data() + off, v.data(), v.size());
+    return off;
+  }
   // uninitialised scratch placed after every initialised buffer
   size_t addScratch(size_t bytes) {
     const size_t off = scratch_;
@@ -818,6 +824,77 @@ private:
     }
     const size_t o0 = gen_.addI32(bpre), o1 = gen_.addI32(bpost), o2 = gen_.addI32(bscale),
                  o3 = gen_.addI32(opre), o4 = gen_.addI32(opost), o5 = gen_.addI32(oscale);
+    // A stride-2 convolution over at most 4 channels (the first layer of an
+    // image network) cannot feed the matrix cores 16 bytes at a time. Space-to-
+    // depth by 2 turns it into a stride-1 convolution over 16 channels on a
+    // half-size image: same sums, since padded taps meet (input == inOffset)
+    // and padded filter entries equal the filter offset, both contributing 0.
+    bool fitsI8 = true;
+    for (size_t c = 0; c < OC; c++) fitsI8 = fitsI8 && fof[c] >= -128 && fof[c] <= 127;
+    if (opts_.spaceToDepthStem && !addI && g.strideH == 2 && g.strideW == 2 && g.dilH == 1 &&
+        g.dilW == 1 && g.group == 1 && g.IC * 4 <= 16 && fitsI8) {
+      const int KH2 = (g.KH + 1) / 2, KW2 = (g.KW + 1) / 2, C2 = 16;
+      const size_t BH = (size_t)g.OH + KH2 - 1, BW = (size_t)g.OW + KW2 - 1;
+      const int8_t *F = constData<int8_t>(f);
+      std::vector<int8_t> F2((size_t)OC * KH2 * KW2 * C2);
+      for (size_t oc = 0; oc < OC; oc++)
+        for (int bh = 0; bh < KH2; bh++)
+          for (int bw = 0; bw < KW2; bw++)
+            for (int ch = 0; ch < C2; ch++) {
+              const int q = ch / g.IC, c = ch % g.IC;
+              const int kh = 2 * bh + (q >> 1), kw = 2 * bw + (q & 1);
+              int8_t v = (int8_t)fof[oc];
+              if (ch < 4 * g.IC && kh < g.KH && kw < g.KW)
+                v = F[((oc * g.KH + kh) * g.KW + kw) * g.IC + c];
+              F2[((oc * KH2 + bh) * KW2 + bw) * C2 + ch] = v;
+            }
+      const size_t f2 = gen_.addBytes(F2);
+      const size_t K2 = (size_t)KH2 * KW2 * C2;
+      auto sPtr = scratchPtr(gen_.addScratch((size_t)g.N * BH * BW * C2));
+      auto sum2 = scratchPtr(sums ? gen_.addScratch(OC * 4) : 0);
+      if (sums)
+        out.setup.push_back({"mi355x_rowsum_i8", I.name, strFormat(" rows=%zu K=%zu", OC, K2),
+                             [=](const DeviceBindings &b) {
+                               return mi355x_rowsum_i8((int32_t *)sum2(b), (const int8_t *)(b.generated + f2),
+                                                       OC, K2, b.stream);
+                             }});
+      mi355x_conv_geom g2 = g;
+      g2.IH = (int32_t)BH; g2.IW = (int32_t)BW; g2.IC = C2;
+      g2.KH = KH2; g2.KW = KW2; g2.strideH = g2.strideW = 1; g2.padT = g2.padL = 0;
+      Access priv;                       // the private image orders the two launches
+      priv.root = -100 - (int)out.launches.size();
+      const size_t N = (size_t)g.N, IH = (size_t)g.IH, IW = (size_t)g.IW, IC = (size_t)g.IC,
+                   pT = (size_t)g.padT, pL = (size_t)g.padL;
+      out.launches.push_back(
+          {"mi355x_space_to_depth2_i8", I.name + ".s2d",
+           strFormat(" N=%zu IH=%zu IW=%zu C=%zu padT=%zu padL=%zu BH=%zu BW=%zu Cout=%d", N, IH, IW, IC,
+                     pT, pL, BH, BW, C2) + kv("fill", io),
+           [=](const DeviceBindings &b) {
+             return mi355x_space_to_depth2_i8((int8_t *)sPtr(b), (const int8_t *)s.ptr(b), N, IH, IW, IC,
+                                              pT, pL, BH, BW, (size_t)C2, io, b.stream);
+           }});
+      out.launches.back().writes.push_back(priv);
+      out.launches.push_back(
+          {"mi355x_cwq_conv2d_i8", I.name,
+           strFormat(" N=%d IH=%d IW=%d IC=%d OH=%d OW=%d OC=%d KH=%d KW=%d sH=1 sW=1 padT=0 padL=0 dH=1 "
+                     "dW=1 group=1 space_to_depth=1", g2.N, g2.IH, g2.IW, g2.IC, g2.OH, g2.OW, g2.OC,
+                     g2.KH, g2.KW) +
+               kv("out_offset", oo) + kv("in_offset", io) + kv("act", act) + vecStr("act_args", actArgs) +
+               kv("bias_is_i8", bias8) + kv("filter_offsets_all_zero", allZero) + kv("row_sums", sums) +
+               vecStr("bias_pre", bpre) + vecStr("bias_post", bpost) + vecStr("bias_scale", bscale) +
+               vecStr("out_pre", opre) + vecStr("out_post", opost) + vecStr("out_scale", oscale),
+           [=](const DeviceBindings &b) {
+             auto gp = [&](size_t o) { return (const int32_t *)(b.generated + o); };
+             return mi355x_cwq_conv2d_i8((int8_t *)d.ptr(b), (const int8_t *)sPtr(b),
+                                         (const int8_t *)(b.generated + f2), bi.ptr(b), bias8, &g2, oo, io,
+                                         (const int32_t *)fo.ptr(b), (const int32_t *)bo.ptr(b), gp(o0),
+                                         gp(o1), gp(o2), gp(o3), gp(o4), gp(o5), act, actArgs.data(),
+                                         allZero ? 1 : 0, sums ? (const int32_t *)sum2(b) : nullptr,
+                                         b.stream);
+           }});
+      out.launches.back().reads.push_back(priv);
+      return Error::success();
+    }
     if (addI) {
       const Instruction &A = *addI;
       const bool convIsLhs = A.operands[1] == I.operands[0];

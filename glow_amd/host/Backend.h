@@ -146,6 +146,7 @@ struct BackendOptions {
   bool precomputeWeightRowSums = true; // form sum_k W[n][k] once at load time
   bool fuseAddRelu = true;             // ElementAdd + Relu of its result in one pass
   bool fuseConvAdd = true;             // convolution + ElementAdd (+ Relu) in one kernel
+  bool spaceToDepthStem = true;        // stride-2 convolutions over <= 4 channels via space-to-depth
 };
 
 class MI355XBackend {

@@ -256,6 +256,14 @@ int mi355x_batch_matmul_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs, si
                            size_t M, size_t K, size_t N, int32_t out_offset, int32_t lhs_offset,
                            int32_t rhs_offset, int32_t out_pre, int32_t out_post,
                            int32_t out_scale, void *stream);
+/* Space-to-depth by 2 of a padded NHWC int8 image, the layout change that turns
+ * a stride-2 convolution over few channels into a stride-1 convolution over
+ * 4x the channels (SpaceToDepth with block size 2, plus padding):
+ * dst[n][bh][bw][(dh*2+dw)*C + c] = src[n][2bh+dh-padT][2bw+dw-padL][c], `fill`
+ * outside the image and in channels [4C, Cout). dst is [N, BH, BW, Cout]. */
+int mi355x_space_to_depth2_i8(int8_t *dst, const int8_t *src, size_t N, size_t IH, size_t IW,
+                              size_t C, size_t padT, size_t padL, size_t BH, size_t BW,
+                              size_t Cout, int32_t fill, void *stream);
 /* libjit_sigmoid_kernel_f (libjit.cpp:1913-1916): 1 / (expf(-x) + 1); agrees
  * with the CPU to fp32 rounding of expf (1e-5 relative). */
 int mi355x_sigmoid_f32(float *dst, const float *src, size_t n, void *stream);

@@ -134,3 +134,20 @@ def test_conv_with_fused_residual_add(shape, relu):
     add = capi.fused_add(11, -20, cp, rp, relu, -128, dp)
     got = capi.cwq_conv2d_add_i8(*cases.cwq_conv_args(c), res, add)
     np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("shape,pads", [((2, 16, 16, 3), (3, 3)), ((1, 9, 7, 4), (0, 1)), ((3, 8, 8, 1), (1, 0))])
+def test_space_to_depth(shape, pads):
+    rng = np.random.default_rng(shape[1])
+    x = rng.integers(-128, 128, shape).astype(np.int8)
+    n, ih, iw, c = shape
+    bh, bw, cout, fill = (ih + pads[0] + 4) // 2, (iw + pads[1] + 4) // 2, 16, -9
+    xp = np.full((n, 2 * bh, 2 * bw, c), fill, np.int8)
+    hh, ww = min(ih, 2 * bh - pads[0]), min(iw, 2 * bw - pads[1])
+    xp[:, pads[0]:pads[0] + hh, pads[1]:pads[1] + ww] = x[:, :hh, :ww]
+    want = np.full((n, bh, bw, cout), fill, np.int8)
+    for dh in range(2):
+        for dw in range(2):
+            q = dh * 2 + dw
+            want[..., q * c:(q + 1) * c] = xp[:, dh::2, dw::2]
+    np.testing.assert_array_equal(capi.space_to_depth2_i8(x, pads[0], pads[1], bh, bw, cout, fill), want)

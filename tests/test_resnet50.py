@@ -38,10 +38,15 @@ def test_small_network_compiles_and_fuses():
     assert kernels.count("mi355x_cwq_conv2d_add_i8") == 3
     assert "mi355x_add_relu_i8" not in kernels and "mi355x_add_i8" not in kernels
     m2, f2 = netlib.to_module(net)
-    m2.compile(f2, fuse_conv_add=False)
+    m2.compile(f2, fuse_conv_add=False, space_to_depth_stem=False)
     k2 = [r["kernel"] for r in H.parse_listing(m2.describe(f2)) if r["phase"] == "launch"]
     assert k2.count("mi355x_add_relu_i8") == 3 and k2.count("mi355x_cwq_conv2d_i8") == 11
     assert kernels[-1] == "mi355x_softmax_f32" and kernels[0] == "mi355x_quantize_i8"
+    # the 7x7 stride-2 stem over 3 channels runs as a 4x4 stride-1 convolution
+    # over a space-to-depth image of 16 channels
+    assert kernels[1] == "mi355x_space_to_depth2_i8"
+    stem = [r for r in rows if r.get("space_to_depth") == 1][0]
+    assert (stem["KH"], stem["KW"], stem["IC"], stem["IH"]) == (4, 4, 16, 16 + 3)
     # post-ReLU tensors use the unsigned range: offset -128
     assert net.tensors["stem"].offset == -128
     assert net.ops_count() > 0
@@ -57,12 +62,12 @@ def test_oracle_executes_the_small_network():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("fuse", [(True, True), (True, False), (False, False)])
+@pytest.mark.parametrize("fuse", [(True, True, True), (True, False, False), (False, False, True)])
 def test_device_matches_oracle(fuse):
     net = resnet50.make(batch=2, size=64, profile_images=4, seed=5,
                         layers=((64, 2, 1), (128, 2, 2), (256, 1, 2)), classes=100)
     m, f = netlib.to_module(net)
-    m.compile(f, fuse_conv_add=fuse[0], fuse_add_relu=fuse[1])
+    m.compile(f, fuse_conv_add=fuse[0], fuse_add_relu=fuse[1], space_to_depth_stem=fuse[2])
     dm = H.DeviceManager().init()
     try:
         dm.add_network(m)
