@@ -424,6 +424,9 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_wave_kernel(SlwsArgs a) {
       const int cnt = min(kBatch, len - base);
       // round 1: lane j fetches lookup j of the batch
       int my_key;
+      uint32_t so_lo = 0, so_hi = 0;
+      float my_w;
+      bool my_valid;
       {
         const long long pos = start + base + lane;
         long long row = -1;
@@ -439,26 +442,22 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_wave_kernel(SlwsArgs a) {
             w = reinterpret_cast<const float *>(a.weights)[pos];
           }
         }
-        float s = 0.0f, o = 0.0f;
-        if (row >= 0 && row < a.data_rows) {
-          const uint8_t *so = a.data + row * a.in_line + a.data_bytes;
-          if constexpr (SO16) {
-            uint32_t v = load_u32_any(so);
-            s = __half2float(__ushort_as_half((unsigned short)(v & 0xffff)));
-            o = __half2float(__ushort_as_half((unsigned short)(v >> 16)));
-          } else {
-            s = __uint_as_float(load_u32_any(so));
-            o = __uint_as_float(load_u32_any(so + 4));
-          }
-        } else {
-          row = 0; // skipped lookup: reads row 0, contributes w * 0
+        // a skipped lookup reads row 0 and contributes w * 0
+        my_valid = row >= 0 && row < a.data_rows;
+        if (!my_valid) {
+          row = 0;
           w = 0.0f;
         }
+        my_w = w;
         my_key = OFF32 ? (int)(uint32_t)(row * a.in_line) : (int)row;
-        look[lane] = make_int4(my_key, __float_as_int(w), __float_as_int(s),
-                               __float_as_int(o));
+        // The row's scale and offset are requested here and consumed only
+        // after the row reads below have been issued, so that the two
+        // dependent round trips (index -> scale/offset, index -> row bytes)
+        // overlap instead of following each other.
+        const uint8_t *so = a.data + row * a.in_line + a.data_bytes;
+        so_lo = load_u32_any(so);
+        if constexpr (!SO16) so_hi = load_u32_any(so + 4);
       }
-      wave_lds_sync();
       // round 2: all row reads of the batch in flight before the first use.
       // Lookups are taken four at a time under one uniform branch; slots
       // beyond cnt hold {row 0, w 0, scale 0, offset 0} and add exactly +0.
@@ -492,6 +491,20 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_wave_kernel(SlwsArgs a) {
           }
         }
       }
+      {
+        float s, o;
+        if constexpr (SO16) {
+          s = __half2float(__ushort_as_half((unsigned short)(so_lo & 0xffff)));
+          o = __half2float(__ushort_as_half((unsigned short)(so_lo >> 16)));
+        } else {
+          s = __uint_as_float(so_lo);
+          o = __uint_as_float(so_hi);
+        }
+        if (!my_valid) s = o = 0.0f;
+        look[lane] = make_int4(my_key, __float_as_int(my_w), __float_as_int(s),
+                               __float_as_int(o));
+      }
+      wave_lds_sync();
 #pragma unroll
       for (int g = 0; g < kBatch / kGroup; g++) {
         if (g * kGroup < cnt) {
