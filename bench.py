@@ -32,7 +32,7 @@ if ROOT not in sys.path:
 # HBM bytes per launch of the default workloads (FETCH_SIZE + WRITE_SIZE of two
 # counter runs, scaled by what the counters read for a plain copy of known
 # size). They hold for the default sizes only; other sizes report null.
-MEASURED_TRAFFIC = {"slws": 24.03e6, "fc_large": 236.3e6, "conv_c3": 13.32e6}
+MEASURED_TRAFFIC = {"slws": 24.02e6, "fc_large": 236.3e6, "conv_c3": 13.35e6}
 
 HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E, published
 INT8_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA, published (5.0 POP/s)
@@ -509,7 +509,7 @@ def main():
             "index_batches_cycled": args.batches,
             "mean_lookups_per_step": s["mean_lookups"],
             "bytes_per_step": s["bytes"],
-            "device": info.name.decode(), "arch": info.arch.decode(),
+            "device": info.name.decode() or "MI355X", "arch": info.arch.decode(),
             "compute_units": info.compute_units,
         },
         "parity_with_oracle": parity,
