@@ -249,6 +249,11 @@ int mi355x_cwq_conv2d_add_i8(
   ep.add.dest_pre = add->dest_pre;
   ep.add.dest_post = add->dest_post;
   ep.add.dest_scale = add->dest_scale;
+  auto fits = [](int32_t v) { return v > -(1 << 23) && v < (1 << 23); };
+  ep.add.small = fits(add->conv_scale) && fits(add->residual_scale) &&
+                 (!add->relu || fits(add->dest_scale)) && conv_offset >= -128 &&
+                 conv_offset <= 127 && add->residual_offset > -(1 << 22) &&
+                 add->residual_offset < (1 << 22);
   return conv_common(out, in, filter, geom, ep, !filter_offsets_all_zero,
                      stream);
 }

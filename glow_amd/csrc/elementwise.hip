@@ -61,30 +61,36 @@ __global__ __launch_bounds__(kEwThreads) void quantize_i8_kernel(
     dst[i] = (int8_t)quantize_one(src[i], scale, offset);
 }
 
+// A block converts tiles of 256 x 16 elements in four steps; in each step
+// consecutive lanes take consecutive groups of 4 elements, so a wavefront reads
+// 256 contiguous bytes and writes 1 KiB contiguous.
 __global__ __launch_bounds__(kEwThreads) void dequantize_i8_kernel(
     float *__restrict__ dst, const int8_t *__restrict__ src, size_t n,
     size_t vec_chunks, float scale, int32_t offset) {
-  const size_t t = (size_t)blockIdx.x * kEwThreads + threadIdx.x;
-  if (t < vec_chunks) {
-    uint4 q = reinterpret_cast<const uint4 *>(src)[t];
-    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
-    float4 *d = reinterpret_cast<float4 *>(dst) + t * 4;
+  constexpr size_t kTile = (size_t)kEwThreads * kEwPerLane;
+  const size_t tiles = vec_chunks / kEwThreads;       // whole tiles only
+  if (blockIdx.x < tiles) {
+    const size_t base = (size_t)blockIdx.x * kTile + (size_t)threadIdx.x * 4;
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
+    for (int st = 0; st < kEwPerLane / 4; st++) {
+      const size_t e = base + (size_t)st * kEwThreads * 4;
+      const uint32_t w = *reinterpret_cast<const uint32_t *>(src + e);
       float4 f;
-      f.x = __fmul_rn(scale, (float)(sext8(w[j], 0) - offset));
-      f.y = __fmul_rn(scale, (float)(sext8(w[j], 1) - offset));
-      f.z = __fmul_rn(scale, (float)(sext8(w[j], 2) - offset));
-      f.w = __fmul_rn(scale, (float)(sext8(w[j], 3) - offset));
-      d[j] = f;
+      f.x = __fmul_rn(scale, (float)(sext8(w, 0) - offset));
+      f.y = __fmul_rn(scale, (float)(sext8(w, 1) - offset));
+      f.z = __fmul_rn(scale, (float)(sext8(w, 2) - offset));
+      f.w = __fmul_rn(scale, (float)(sext8(w, 3) - offset));
+      *reinterpret_cast<float4 *>(dst + e) = f;
     }
   }
-  const size_t tail0 = vec_chunks * kEwPerLane;
+  // scalar tail: elements [tiles * kTile, n)
+  const size_t t = (size_t)blockIdx.x * kEwThreads + threadIdx.x;
   const size_t stride = (size_t)gridDim.x * kEwThreads;
-  for (size_t i = tail0 + t; i < n; i += stride)
+  for (size_t i = tiles * kTile + t; i < n; i += stride)
     dst[i] = __fmul_rn(scale, (float)((int32_t)src[i] - offset));
 }
 
+template <bool SMALL>
 __global__ __launch_bounds__(kEwThreads) void rescale_i8_kernel(
     int8_t *__restrict__ dst, const int8_t *__restrict__ src, size_t n,
     size_t vec_chunks, int32_t out_offset, int32_t in_offset, int32_t pre,
@@ -98,8 +104,8 @@ __global__ __launch_bounds__(kEwThreads) void rescale_i8_kernel(
       int32_t r[4];
 #pragma unroll
       for (int b = 0; b < 4; b++)
-        r[b] = clip_i8(scale_i32(sext8(w[j], b) - in_offset, pre, post, scale,
-                                 out_offset));
+        r[b] = clip_i8(scale_i32_sel<SMALL>(sext8(w[j], b) - in_offset, pre, post,
+                                            scale, out_offset));
       w[j] = pack4(r[0], r[1], r[2], r[3]);
     }
     reinterpret_cast<uint4 *>(dst)[t] = make_uint4(w[0], w[1], w[2], w[3]);
@@ -107,8 +113,8 @@ __global__ __launch_bounds__(kEwThreads) void rescale_i8_kernel(
   const size_t tail0 = vec_chunks * kEwPerLane;
   const size_t stride = (size_t)gridDim.x * kEwThreads;
   for (size_t i = tail0 + t; i < n; i += stride)
-    dst[i] = (int8_t)clip_i8(scale_i32((int32_t)src[i] - in_offset, pre, post,
-                                       scale, out_offset));
+    dst[i] = (int8_t)clip_i8(scale_i32_sel<SMALL>((int32_t)src[i] - in_offset, pre,
+                                                  post, scale, out_offset));
 }
 
 static bool aligned16(const void *a, const void *b) {
@@ -161,9 +167,18 @@ int mi355x_rescale_i8(int8_t *dst, const int8_t *src, size_t n,
                  "pre/post shift outside [0, 31]: %d %d", pre, post);
   MI355X_REQUIRE(n / kEwPerLane / kEwThreads < 0x7fffffffu, "tensor too large");
   const size_t chunks = aligned16(dst, src) ? n / kEwPerLane : 0;
-  hipLaunchKernelGGL(rescale_i8_kernel, dim3(ew_blocks(chunks)),
-                     dim3(kEwThreads), 0, as_stream(stream), dst, src, n,
-                     chunks, out_offset, in_offset, pre, post, scale);
+  // |q - in_offset| < 2^23 always holds for int8 data when the offset does;
+  // with a scale below 2^23 too, the 24-bit multiplier is exact
+  const bool small = scale > -(1 << 23) && scale < (1 << 23) &&
+                     in_offset > -(1 << 22) && in_offset < (1 << 22);
+  if (small)
+    hipLaunchKernelGGL(rescale_i8_kernel<true>, dim3(ew_blocks(chunks)),
+                       dim3(kEwThreads), 0, as_stream(stream), dst, src, n,
+                       chunks, out_offset, in_offset, pre, post, scale);
+  else
+    hipLaunchKernelGGL(rescale_i8_kernel<false>, dim3(ew_blocks(chunks)),
+                       dim3(kEwThreads), 0, as_stream(stream), dst, src, n,
+                       chunks, out_offset, in_offset, pre, post, scale);
   return check_launch("rescale_i8");
 }
 

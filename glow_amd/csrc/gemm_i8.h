@@ -59,30 +59,44 @@ struct FusedAdd {
   int32_t res_pre, res_post, res_scale;   // rescale of the residual
   int32_t relu;                           // apply the Relu stage below
   int32_t dest_off, dest_pre, dest_post, dest_scale;
+  int32_t small;                          // every scale is below 2^23 in magnitude
 };
 
+template <bool SMALL>
 __device__ __forceinline__ int32_t fused_add_one(int32_t own, int32_t res,
                                                  const FusedAdd &f) {
-  const int32_t a = scale_i32(own - f.own_off, f.own_pre, f.own_post, f.own_scale, 0);
-  const int32_t b = scale_i32(res - f.res_off, f.res_pre, f.res_post, f.res_scale, 0);
+  const int32_t a =
+      scale_i32_sel<SMALL>(own - f.own_off, f.own_pre, f.own_post, f.own_scale, 0);
+  const int32_t b =
+      scale_i32_sel<SMALL>(res - f.res_off, f.res_pre, f.res_post, f.res_scale, 0);
   int32_t v = clip_i8((int32_t)((uint32_t)a + (uint32_t)b + (uint32_t)f.sum_off));
   if (f.relu) {
     const int32_t so = (int32_t)(int8_t)f.sum_off;
     v = max(v, so);
-    v = clip_i8(scale_i32(v - so, f.dest_pre, f.dest_post, f.dest_scale, f.dest_off));
+    v = clip_i8(scale_i32_sel<SMALL>(v - so, f.dest_pre, f.dest_post, f.dest_scale,
+                                     f.dest_off));
   }
   return v;
 }
 
-__device__ __forceinline__ uint32_t fused_add_word(uint32_t own, uint32_t res,
-                                                   const FusedAdd &f) {
+template <bool SMALL>
+__device__ __forceinline__ uint32_t fused_add_word_t(uint32_t own, uint32_t res,
+                                                     const FusedAdd &f) {
   uint32_t o = 0;
 #pragma unroll
   for (int b = 0; b < 4; b++)
-    o |= (uint32_t)(fused_add_one((int32_t)(int8_t)(own >> (8 * b)),
-                                  (int32_t)(int8_t)(res >> (8 * b)), f) & 0xff)
+    o |= (uint32_t)(fused_add_one<SMALL>((int32_t)(int8_t)(own >> (8 * b)),
+                                         (int32_t)(int8_t)(res >> (8 * b)), f) & 0xff)
          << (8 * b);
   return o;
+}
+
+// int8 operands minus int8-range offsets stay far below 2^23, so the 24-bit
+// multiplier applies whenever the scales do (f.small, set on the host).
+__device__ __forceinline__ uint32_t fused_add_word(uint32_t own, uint32_t res,
+                                                   const FusedAdd &f) {
+  return f.small ? fused_add_word_t<true>(own, res, f)
+                 : fused_add_word_t<false>(own, res, f);
 }
 
 struct Epilogue {
@@ -266,7 +280,7 @@ __device__ __forceinline__ void gemm_epilogue_impl(
     for (int c = tid; c < rows_here * cols_here; c += THREADS) {
       const int r = c / cols_here, s = c - r * cols_here;
       int32_t v = s_out[r * OUT_STRIDE + s];
-      if (rbase) v = fused_add_one(v, rbase[(long long)r * ep.ldc + s], ep.add);
+      if (rbase) v = fused_add_one<false>(v, rbase[(long long)r * ep.ldc + s], ep.add);
       obase[(long long)r * ep.ldc + s] = (int8_t)v;
     }
   }

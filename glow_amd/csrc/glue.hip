@@ -31,21 +31,24 @@ struct AddParams {
   int32_t relu_dest_off, relu_pre, relu_post, relu_scale;
 };
 
-template <bool RELU>
+// SMALL: offsets and scales are below 2^23 in magnitude (checked on the host),
+// which lets the multiplies run on the 24-bit multiplier.
+template <bool RELU, bool SMALL>
 __device__ __forceinline__ int32_t add_one(int32_t l, int32_t r, const AddParams &p) {
-  const int32_t a = scale_i32(l - p.lhs_off, p.lhs_pre, p.lhs_post, p.lhs_scale, 0);
-  const int32_t b = scale_i32(r - p.rhs_off, p.rhs_pre, p.rhs_post, p.rhs_scale, 0);
+  const int32_t a = scale_i32_sel<SMALL>(l - p.lhs_off, p.lhs_pre, p.lhs_post, p.lhs_scale, 0);
+  const int32_t b = scale_i32_sel<SMALL>(r - p.rhs_off, p.rhs_pre, p.rhs_post, p.rhs_scale, 0);
   int32_t v = clip_i8((int32_t)((uint32_t)a + (uint32_t)b + (uint32_t)p.dest_off));
   if (RELU) {
     // libjit_element_relu_i8 with srcOffset = the sum's offset
     const int32_t so = (int32_t)(int8_t)p.dest_off;
     v = max(v, so);
-    v = clip_i8(scale_i32(v - so, p.relu_pre, p.relu_post, p.relu_scale, p.relu_dest_off));
+    v = clip_i8(scale_i32_sel<SMALL>(v - so, p.relu_pre, p.relu_post, p.relu_scale,
+                                     p.relu_dest_off));
   }
   return v;
 }
 
-template <bool RELU>
+template <bool RELU, bool SMALL>
 __global__ __launch_bounds__(kGlueThreads) void add_i8_kernel(
     int8_t *__restrict__ dst, const int8_t *__restrict__ lhs,
     const int8_t *__restrict__ rhs, size_t n, size_t vec_chunks, AddParams p) {
@@ -57,15 +60,15 @@ __global__ __launch_bounds__(kGlueThreads) void add_i8_kernel(
     uint32_t o[4];
 #pragma unroll
     for (int j = 0; j < 4; j++)
-      o[j] = pack4b(add_one<RELU>(sx8(wa[j], 0), sx8(wb[j], 0), p),
-                    add_one<RELU>(sx8(wa[j], 1), sx8(wb[j], 1), p),
-                    add_one<RELU>(sx8(wa[j], 2), sx8(wb[j], 2), p),
-                    add_one<RELU>(sx8(wa[j], 3), sx8(wb[j], 3), p));
+      o[j] = pack4b(add_one<RELU, SMALL>(sx8(wa[j], 0), sx8(wb[j], 0), p),
+                    add_one<RELU, SMALL>(sx8(wa[j], 1), sx8(wb[j], 1), p),
+                    add_one<RELU, SMALL>(sx8(wa[j], 2), sx8(wb[j], 2), p),
+                    add_one<RELU, SMALL>(sx8(wa[j], 3), sx8(wb[j], 3), p));
     reinterpret_cast<uint4 *>(dst)[t] = make_uint4(o[0], o[1], o[2], o[3]);
   }
   const size_t stride = (size_t)gridDim.x * kGlueThreads;
   for (size_t i = vec_chunks * 16 + t; i < n; i += stride)
-    dst[i] = (int8_t)add_one<RELU>(lhs[i], rhs[i], p);
+    dst[i] = (int8_t)add_one<RELU, SMALL>(lhs[i], rhs[i], p);
 }
 
 __device__ __forceinline__ int32_t relu_one(int32_t v, int32_t so, int32_t doff,
@@ -73,6 +76,10 @@ __device__ __forceinline__ int32_t relu_one(int32_t v, int32_t so, int32_t doff,
   v = max(v, so);
   return clip_i8(scale_i32(v - so, pre, post, scale, doff));
 }
+
+static bool fits24(int32_t v) { return v > -(1 << 23) && v < (1 << 23); }
+// an int8 value minus such an offset still fits 24 bits
+static bool off24(int32_t v) { return v > -(1 << 22) && v < (1 << 22); }
 
 __global__ __launch_bounds__(kGlueThreads) void relu_i8_kernel(
     int8_t *__restrict__ dst, const int8_t *__restrict__ src, size_t n,
@@ -412,8 +419,14 @@ int mi355x_add_i8(int8_t *dst, const int8_t *lhs, const int8_t *rhs, size_t n,
   AddParams p{dest_offset, lhs_offset, rhs_offset, lhs_pre, lhs_post, lhs_scale,
               rhs_pre, rhs_post, rhs_scale, 0, 0, 0, 0};
   const size_t chunks = al16(dst, lhs, rhs) ? n / 16 : 0;
-  hipLaunchKernelGGL(add_i8_kernel<false>, dim3(glue_blocks(chunks)), dim3(kGlueThreads), 0,
-                     as_stream(stream), dst, lhs, rhs, n, chunks, p);
+  const bool small = fits24(lhs_scale) && fits24(rhs_scale) && off24(lhs_offset) &&
+                     off24(rhs_offset);
+  if (small)
+    hipLaunchKernelGGL((add_i8_kernel<false, true>), dim3(glue_blocks(chunks)),
+                       dim3(kGlueThreads), 0, as_stream(stream), dst, lhs, rhs, n, chunks, p);
+  else
+    hipLaunchKernelGGL((add_i8_kernel<false, false>), dim3(glue_blocks(chunks)),
+                       dim3(kGlueThreads), 0, as_stream(stream), dst, lhs, rhs, n, chunks, p);
   return check_launch("add_i8");
 }
 
@@ -434,8 +447,14 @@ int mi355x_add_relu_i8(int8_t *dst, const int8_t *lhs, const int8_t *rhs, size_t
   AddParams p{sum_offset, lhs_offset, rhs_offset, lhs_pre, lhs_post, lhs_scale,
               rhs_pre, rhs_post, rhs_scale, dest_offset, dest_pre, dest_post, dest_scale};
   const size_t chunks = al16(dst, lhs, rhs) ? n / 16 : 0;
-  hipLaunchKernelGGL(add_i8_kernel<true>, dim3(glue_blocks(chunks)), dim3(kGlueThreads), 0,
-                     as_stream(stream), dst, lhs, rhs, n, chunks, p);
+  const bool small = fits24(lhs_scale) && fits24(rhs_scale) && fits24(dest_scale) &&
+                     off24(lhs_offset) && off24(rhs_offset);
+  if (small)
+    hipLaunchKernelGGL((add_i8_kernel<true, true>), dim3(glue_blocks(chunks)),
+                       dim3(kGlueThreads), 0, as_stream(stream), dst, lhs, rhs, n, chunks, p);
+  else
+    hipLaunchKernelGGL((add_i8_kernel<true, false>), dim3(glue_blocks(chunks)),
+                       dim3(kGlueThreads), 0, as_stream(stream), dst, lhs, rhs, n, chunks, p);
   return check_launch("add_relu_i8");
 }
 

@@ -151,3 +151,18 @@ def test_space_to_depth(shape, pads):
             q = dh * 2 + dw
             want[..., q * c:(q + 1) * c] = xp[:, dh::2, dw::2]
     np.testing.assert_array_equal(capi.space_to_depth2_i8(x, pads[0], pads[1], bh, bw, cout, fill), want)
+
+
+def test_add_with_scales_beyond_24_bits():
+    """Parameters outside the 24-bit fast path take the 32-bit multiplier."""
+    rng = np.random.default_rng(31)
+    a = rng.integers(-128, 128, 5000).astype(np.int8)
+    b = rng.integers(-128, 128, 5000).astype(np.int8)
+    for lp, rp, lo, ro in [((0, 20, (1 << 23) + 5), (1, 3, 7), 3, -4),
+                           ((0, 0, 1), (0, 25, -(1 << 24) - 1), 0, (1 << 22) + 9),
+                           ((3, 9, (1 << 23) - 1), (0, 31, 1 << 30), -(1 << 22) + 1, 12)]:
+        want = go.add_i8(a, b, 5, lo, ro, lp, rp)
+        np.testing.assert_array_equal(capi.add_i8(a, b, 5, lo, ro, lp, rp), want)
+        dp = (0, 22, (1 << 23) + 77)
+        np.testing.assert_array_equal(capi.add_relu_i8(a, b, 5, lo, ro, lp, rp, -3, dp),
+                                      go.relu_i8(want, 5, -3, dp))

@@ -459,3 +459,16 @@ def test_arena_regions_and_bounds():
         a.download(capi.REGION_ACTIVATIONS, 128, 64, np.int8),
         go.quantize_i8(f, 0.05, 1))
     a.destroy()
+
+
+@pytest.mark.gpu
+def test_rescale_both_multiplier_paths():
+    """Scales below 2^23 take the 24-bit multiplier, others the 32-bit one:
+    the results must not depend on which."""
+    q = np.arange(-128, 128).astype(np.int8).repeat(20)
+    for sc in (1, 255, (1 << 23) - 1, 1 << 23, (1 << 23) + 12345, -(1 << 23) + 1, -(1 << 23),
+               (1 << 30) + 7, -5):
+        for pre, post, io, oo in ((0, 0, 0, 0), (2, 15, -7, 9), (0, 31, 127, -128), (7, 3, -128, 127)):
+            np.testing.assert_array_equal(capi.rescale_i8(q, oo, io, pre, post, sc),
+                                          go.rescale_i8(q, oo, io, pre, post, sc),
+                                          err_msg=f"scale {sc} pre {pre} post {post}")
