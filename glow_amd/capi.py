@@ -23,7 +23,7 @@ EXPORTS = [
     "mi355x_device_info", "mi355x_malloc", "mi355x_free", "mi355x_host_alloc",
     "mi355x_host_free", "mi355x_memcpy_h2d", "mi355x_memcpy_d2h",
     "mi355x_memcpy_d2d", "mi355x_fill_u8", "mi355x_copy_u8", "mi355x_gemm_tile_override",
-    "mi355x_cwq_conv2d_add_i8", "mi355x_add_i8", "mi355x_add_relu_i8",
+    "mi355x_cwq_conv2d_add_i8", "mi355x_frwq_sls_multi", "mi355x_add_i8", "mi355x_add_relu_i8",
     "mi355x_relu_i8", "mi355x_convert_f16_to_f32", "mi355x_insert_rows",
     "mi355x_batch_transpose_i8", "mi355x_space_to_depth2_i8", "mi355x_gather", "mi355x_batch_matmul_i8", "mi355x_sigmoid_f32",
     "mi355x_max_pool_i8", "mi355x_avg_pool_i8", "mi355x_softmax_f32", "mi355x_stream_create",
@@ -890,3 +890,55 @@ def space_to_depth2_i8(x, pad_t, pad_l, bh, bw, cout, fill):
                                           _sz(pad_t), _sz(pad_l), _sz(bh), _sz(bw), _sz(cout),
                                           _i32(fill), _vp(None)))
     return out.numpy()
+
+
+class SlsTable(C.Structure):
+    """mi355x_sls_table: one table of a multi-table pooled lookup."""
+    _fields_ = [("data", C.c_void_p), ("indices", C.c_void_p), ("lengths", C.c_void_p),
+                ("dest", C.c_void_p), ("data_rows", C.c_uint64), ("num_indices", C.c_uint64)]
+
+
+SLS_OUT_F32, SLS_OUT_F16, SLS_OUT_I8, SLS_OUT_I8_VIA_F16 = range(4)
+
+
+def frwq_sls_multi(tables, kind, indices, lengths, out_kind=SLS_OUT_F32, out_scale=1.0,
+                   out_offset=0, fp16_accum=False):
+    """tables, indices, lengths: equally long lists (one entry per table; tables
+    of one shape, indices of one dtype). Dense output kinds return a list of
+    [bags x cols] arrays; the int8 kinds return the concatenation
+    [bags x tables*cols] that the fused InsertTensors build."""
+    n = len(tables)
+    tabs = [np.ascontiguousarray(t, np.uint8) for t in tables]
+    idx = [np.ascontiguousarray(i) for i in indices]
+    lens = [np.ascontiguousarray(l, np.int32) for l in lengths]
+    in_line = tabs[0].shape[1]
+    cols = _fused_cols(in_line, kind)
+    bags = lens[0].size
+    d_t = [to_device(t) for t in tabs]
+    d_i = [to_device(i if i.size else np.zeros(1, i.dtype)) for i in idx]
+    d_l = [to_device(l) for l in lens]
+    q8 = out_kind >= SLS_OUT_I8
+    if q8:
+        out = DeviceBuffer.empty((bags, n * cols), np.int8)
+        dests = [out.ptr + t * cols for t in range(n)]
+        stride = n * cols
+    else:
+        dt = np.float16 if out_kind == SLS_OUT_F16 else np.float32
+        outs = [DeviceBuffer.empty((bags, cols), dt) for _ in range(n)]
+        dests = [o.ptr for o in outs]
+        stride = 0
+    arr = (SlsTable * n)()
+    for t in range(n):
+        arr[t] = SlsTable(d_t[t].ptr, d_i[t].ptr, d_l[t].ptr, dests[t], tabs[t].shape[0],
+                          idx[t].size)
+    d_arr = DeviceBuffer(C.sizeof(arr))
+    check(lib().mi355x_memcpy_h2d(_vp(d_arr), C.byref(arr), _sz(C.sizeof(arr)), _vp(None)))
+    sync()
+    check(lib().mi355x_frwq_sls_multi(
+        _vp(d_arr), _sz(n), _sz(max(t.shape[0] for t in tabs)), C.c_int(kind),
+        C.c_int(idx[0].dtype == np.int64), _sz(bags), _sz(in_line), _sz(cols),
+        C.c_int(out_kind), C.c_float(out_scale), _i32(out_offset), _sz(stride),
+        C.c_int(bool(fp16_accum)), _vp(None)))
+    if q8:
+        return out.numpy()
+    return [o.numpy() for o in outs]

@@ -58,7 +58,64 @@ struct SlwsArgs {
   int32_t data_bytes;      // quantized bytes per row (before scale/offset)
   int32_t out_cols;
   int32_t out16, w16, idx64;
+  // multi-table launches: blockIdx.y selects the table whose pointers replace
+  // the ones above
+  const mi355x_sls_table *tables;
+  // output transform: 0 = fp32 / fp16 rows as above; 1 = round to fp16 when
+  // out16 (what the operator stores), then Quantize to int8 with (q_scale,
+  // q_offset), rows q_stride bytes apart (ConvertTo + Quantize + InsertTensor
+  // behind the lookup)
+  int32_t out_q8;
+  float q_scale, q_offset;
+  int64_t q_stride;
 };
+
+__device__ __forceinline__ void select_table(SlwsArgs &a) {
+  if (a.tables) {
+    const mi355x_sls_table t = a.tables[blockIdx.y];
+    a.data = t.data;
+    a.indices = t.indices;
+    a.lengths = t.lengths;
+    a.dest = t.dest;
+    a.data_rows = (int64_t)t.data_rows;
+    a.num_indices = (int64_t)t.num_indices;
+  }
+}
+
+// Stores the columns [col0, col0 + N) of output row `bag`.
+template <int N>
+__device__ __forceinline__ void store_columns(const SlwsArgs &a, long long bag, int col0,
+                                              const float (&acc)[N]) {
+  if (a.out_q8) {
+    int8_t *d = reinterpret_cast<int8_t *>(a.dest) + bag * a.q_stride + col0;
+#pragma unroll
+    for (int c = 0; c < N; c++) {
+      if (col0 + c < a.out_cols) {
+        const float v = a.out16 ? __half2float(__float2half_rn(acc[c])) : acc[c];
+        // the Quantize kernel's expression (the conversion saturates)
+        const float r = rintf(__fadd_rn(__fdiv_rn(v, a.q_scale), a.q_offset));
+        d[c] = (int8_t)min(max((int32_t)r, -128), 127);
+      }
+    }
+    return;
+  }
+  const long long o0 = bag * (long long)a.out_cols + col0;
+  if (a.out16) {
+    __half *d = reinterpret_cast<__half *>(a.dest) + o0;
+#pragma unroll
+    for (int c = 0; c < N; c++)
+      if (col0 + c < a.out_cols) d[c] = __float2half_rn(acc[c]);
+  } else {
+    float *d = reinterpret_cast<float *>(a.dest) + o0;
+    if (N == 2 && col0 + 1 < a.out_cols && ((((uintptr_t)d) & 7) == 0)) {
+      *reinterpret_cast<float2 *>(d) = make_float2(acc[0], acc[N - 1]);
+    } else {
+#pragma unroll
+      for (int c = 0; c < N; c++)
+        if (col0 + c < a.out_cols) d[c] = acc[c];
+    }
+  }
+}
 
 typedef uint8_t __attribute__((address_space(1))) global_u8;
 typedef unsigned short __attribute__((address_space(1))) global_u16;
@@ -213,6 +270,7 @@ __device__ __forceinline__ void bag_span(const SlwsArgs &a, int tid, int grp,
 
 template <int LPB, int BPL, bool IS4, bool SO16, bool ACC16>
 __global__ __launch_bounds__(kSlwsThreads) void slws_kernel(SlwsArgs a) {
+  select_table(a);
   constexpr int kGroups = kSlwsThreads / LPB;      // bags per block
   constexpr int kColsPerByte = IS4 ? 2 : 1;
   constexpr int kColsPerLane = BPL * kColsPerByte;
@@ -323,27 +381,8 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_kernel(SlwsArgs a) {
       }
     }
 
-    if (bag < a.segments && lane_live) {
-      const int col0 = byte0 * kColsPerByte;
-      const long long o0 = bag * (long long)a.out_cols + col0;
-      if (a.out16) {
-        __half *d = reinterpret_cast<__half *>(a.dest) + o0;
-#pragma unroll
-        for (int c = 0; c < kColsPerLane; c++)
-          if (col0 + c < a.out_cols) d[c] = __float2half_rn(acc[c]);
-      } else {
-        float *d = reinterpret_cast<float *>(a.dest) + o0;
-        if (kColsPerLane == 2 && col0 + 1 < a.out_cols &&
-            ((((uintptr_t)d) & 7) == 0)) {
-          *reinterpret_cast<float2 *>(d) =
-              make_float2(acc[0], acc[kColsPerLane - 1]);
-        } else {
-#pragma unroll
-          for (int c = 0; c < kColsPerLane; c++)
-            if (col0 + c < a.out_cols) d[c] = acc[c];
-        }
-      }
-    }
+    if (bag < a.segments && lane_live)
+      store_columns<kColsPerLane>(a, bag, byte0 * kColsPerByte, acc);
   }
 }
 
@@ -360,6 +399,7 @@ __device__ __forceinline__ void wave_lds_sync() {
 // addresses are formed as a uniform base plus a 32-bit per-lane offset.
 template <int BPL, bool IS4, bool SO16, bool ACC16, bool OFF32>
 __global__ __launch_bounds__(kSlwsThreads) void slws_wave_kernel(SlwsArgs a) {
+  select_table(a);
   constexpr int kGroups = kSlwsThreads / 64;
   constexpr int kColsPerByte = IS4 ? 2 : 1;
   constexpr int kColsPerLane = BPL * kColsPerByte;
@@ -532,27 +572,8 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_wave_kernel(SlwsArgs a) {
       wave_lds_sync(); // slots are rewritten by the next batch
     }
 
-    if (bag < a.segments && lane_live) {
-      const int col0 = byte0 * kColsPerByte;
-      const long long o0 = bag * (long long)a.out_cols + col0;
-      if (a.out16) {
-        __half *d = reinterpret_cast<__half *>(a.dest) + o0;
-#pragma unroll
-        for (int c = 0; c < kColsPerLane; c++)
-          if (col0 + c < a.out_cols) d[c] = __float2half_rn(acc[c]);
-      } else {
-        float *d = reinterpret_cast<float *>(a.dest) + o0;
-        if (kColsPerLane == 2 && col0 + 1 < a.out_cols &&
-            ((((uintptr_t)d) & 7) == 0)) {
-          *reinterpret_cast<float2 *>(d) =
-              make_float2(acc[0], acc[kColsPerLane - 1]);
-        } else {
-#pragma unroll
-          for (int c = 0; c < kColsPerLane; c++)
-            if (col0 + c < a.out_cols) d[c] = acc[c];
-        }
-      }
-    }
+    if (bag < a.segments && lane_live)
+      store_columns<kColsPerLane>(a, bag, byte0 * kColsPerByte, acc);
   }
 }
 
@@ -641,6 +662,16 @@ static void launch_wave_kind(int kind, bool acc16, dim3 grid, hipStream_t st,
 #undef MI355X_SLWS_WAVE
 }
 
+// Several tables in one launch and/or the int8 output transform.
+struct SlwsExtra {
+  const mi355x_sls_table *tables = nullptr; // device array
+  size_t n_tables = 1;
+  int out_q8 = 0;
+  float q_scale = 1.0f;
+  int32_t q_offset = 0;
+  size_t q_stride = 0;
+};
+
 static int slws_dispatch(void *dest, int out_is_f16, const uint8_t *data,
                          size_t data_rows, int kind, const void *weights,
                          int weights_are_f16, const void *indices,
@@ -648,10 +679,12 @@ static int slws_dispatch(void *dest, int out_is_f16, const uint8_t *data,
                          const int32_t *lengths, const int32_t *offsets,
                          int has_end_offset, size_t out_rows,
                          size_t in_line_size, size_t out_line_size,
-                         int fp16_accum, void *stream) {
-  if (out_rows == 0) return MI355X_OK;
+                         int fp16_accum, void *stream,
+                         const SlwsExtra &x = SlwsExtra()) {
+  if (out_rows == 0 || x.n_tables == 0) return MI355X_OK;
   MI355X_REQUIRE(kind >= 0 && kind <= 3, "unknown fused kind %d", kind);
-  MI355X_REQUIRE(dest && (lengths || offsets), "NULL tensor");
+  MI355X_REQUIRE(x.tables || (dest && (lengths || offsets)), "NULL tensor");
+  MI355X_REQUIRE(x.n_tables <= 65535, "more than 65535 tables");
   const bool is4 = kind == MI355X_FUSED_U4_F16 || kind == MI355X_FUSED_U4_F32;
   const bool so16 = kind == MI355X_FUSED_U8_F16 || kind == MI355X_FUSED_U4_F16;
   const size_t so_bytes = so16 ? 4 : 8;
@@ -665,8 +698,11 @@ static int slws_dispatch(void *dest, int out_is_f16, const uint8_t *data,
   MI355X_REQUIRE(in_line_size < (1u << 20) && data_rows < (1ull << 31) &&
                      out_rows < (1ull << 40),
                  "table or batch too large");
-  MI355X_REQUIRE(num_indices == 0 || (indices && data),
+  MI355X_REQUIRE(x.tables || num_indices == 0 || (indices && data),
                  "NULL indices or data with num_indices > 0");
+  MI355X_REQUIRE(!x.tables || out_rows <= (size_t)kChunkBags,
+                 "a multi-table launch takes at most %d bags per table", kChunkBags);
+  MI355X_REQUIRE(!x.out_q8 || x.q_stride >= cols, "output rows overlap");
   hipStream_t st = as_stream(stream);
 
   SlwsArgs a;
@@ -687,6 +723,11 @@ static int slws_dispatch(void *dest, int out_is_f16, const uint8_t *data,
   a.out16 = out_is_f16;
   a.w16 = weights_are_f16;
   a.idx64 = idx_is_64;
+  a.tables = x.tables;
+  a.out_q8 = x.out_q8;
+  a.q_scale = x.q_scale;
+  a.q_offset = (float)x.q_offset;
+  a.q_stride = (int64_t)x.q_stride;
 
   if (!offsets) {
     const size_t chunks = (out_rows + kChunkBags - 1) / kChunkBags;
@@ -712,7 +753,7 @@ static int slws_dispatch(void *dest, int out_is_f16, const uint8_t *data,
   const size_t groups = kSlwsThreads / lpb;
   const size_t blocks = (out_rows + groups - 1) / groups;
   MI355X_REQUIRE(blocks < 0x7fffffffu, "too many bags");
-  dim3 grid((unsigned)blocks);
+  dim3 grid((unsigned)blocks, (unsigned)x.n_tables);
   const bool off32 = (unsigned long long)data_rows * in_line_size <= 0xffffffffull;
   if (lpb == 16) launch_kind<16, 2>(kind, acc16, grid, st, a);
   else if (lpb == 32) launch_kind<32, 2>(kind, acc16, grid, st, a);
@@ -728,6 +769,28 @@ static int slws_dispatch(void *dest, int out_is_f16, const uint8_t *data,
 using namespace mi355x;
 
 extern "C" {
+
+int mi355x_frwq_sls_multi(const mi355x_sls_table *tables, size_t n_tables,
+                          size_t max_data_rows, int kind, int idx_is_64,
+                          size_t segments, size_t in_line_size,
+                          size_t out_line_size, int out_kind, float out_scale,
+                          int32_t out_offset, size_t dest_row_stride,
+                          int fp16_accum, void *stream) {
+  if (n_tables == 0 || segments == 0) return MI355X_OK;
+  MI355X_REQUIRE(tables, "tables is NULL");
+  MI355X_REQUIRE(out_kind >= 0 && out_kind <= 3, "unknown output kind %d", out_kind);
+  SlwsExtra x;
+  x.tables = tables;
+  x.n_tables = n_tables;
+  x.out_q8 = out_kind >= 2;
+  x.q_scale = out_scale;
+  x.q_offset = out_offset;
+  x.q_stride = dest_row_stride;
+  const int out16 = out_kind == MI355X_SLS_OUT_F16 || out_kind == MI355X_SLS_OUT_I8_VIA_F16;
+  return slws_dispatch(nullptr, out16, nullptr, max_data_rows, kind, nullptr, 0, nullptr,
+                       idx_is_64, 0, nullptr, nullptr, 0, segments, in_line_size,
+                       out_line_size, fp16_accum, stream, x);
+}
 
 int mi355x_frwq_slws(void *dest, int out_is_f16, const uint8_t *data,
                      size_t data_rows, int kind, const void *weights,

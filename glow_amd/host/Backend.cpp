@@ -156,8 +156,12 @@ public:
       }
       case Kind::FusedRowwiseQuantizedSparseLengthsWeightedSum:
         MI355X_RETURN_IF_ERR(slws(I, out, true)); break;
-      case Kind::FusedRowwiseQuantizedSparseLengthsSum:
-        MI355X_RETURN_IF_ERR(slws(I, out, false)); break;
+      case Kind::FusedRowwiseQuantizedSparseLengthsSum: {
+        const size_t used = opts_.fuseSlsChains ? multiSls(at, out) : 0;
+        if (used) at += used - 1;
+        else MI355X_RETURN_IF_ERR(slws(I, out, false));
+        break;
+      }
       default:
         return MI355X_MAKE_ERR(ErrorCode::COMPILE_UNSUPPORTED_NODE_AFTER_OPTIMIZE,
                                "instruction kind %d is not supported", (int)I.kind);
@@ -967,6 +971,146 @@ private:
                                        b.stream);
          }});
     return Error::success();
+  }
+
+  // One pooled lookup followed by [ConvertTo,] Quantize and InsertTensor, each
+  // intermediate read only by the next instruction.
+  struct SlsChain {
+    Operand data, idx, len, dest; // dest: the tensor the int8 rows are inserted into
+    size_t colOffset = 0;         // where, in elements
+    size_t length = 0;            // instructions in the chain
+    int kind = 0, idx64 = 0, viaF16 = 0, acc16 = 0;
+    size_t rows = 0, inLine = 0, cols = 0, segs = 0, nIdx = 0;
+    float qScale = 1.0f;
+    int32_t qOffset = 0;
+  };
+
+  bool matchSlsChain(size_t at, SlsChain &c) const {
+    if (at + 2 >= insts_.size()) return false;
+    const Instruction &S = insts_[at];
+    if (S.kind != Kind::FusedRowwiseQuantizedSparseLengthsSum) return false;
+    auto onlyReadBy = [&](int id, const Instruction &J) {
+      return M_.value(id).category == SymbolCategory::Activation && readers(id) == 1 &&
+             J.operands[1] == id;
+    };
+    size_t p = at + 1;
+    int cur = S.operands[0];
+    const Value &sd = M_.value(cur);
+    if (sd.type.dims.size() != 2) return false;
+    if (sd.type.kind == ElemKind::Float16Ty) {
+      const Instruction &Cv = insts_[p];
+      if (Cv.kind != Kind::ConvertTo || !onlyReadBy(cur, Cv)) return false;
+      if (M_.value(Cv.operands[0]).type.kind != ElemKind::FloatTy) return false;
+      cur = Cv.operands[0];
+      p++;
+      c.viaF16 = 1;
+    } else if (sd.type.kind != ElemKind::FloatTy) {
+      return false;
+    }
+    if (p + 1 >= insts_.size()) return false;
+    const Instruction &Q = insts_[p], &Ins = insts_[p + 1];
+    if (Q.kind != Kind::Quantize || !onlyReadBy(cur, Q)) return false;
+    const Value &qv = M_.value(Q.operands[0]);
+    if (qv.type.kind != ElemKind::Int8QTy) return false;
+    if (Ins.kind != Kind::InsertTensor || !onlyReadBy(qv.id, Ins) || Ins.iattrs.size() != 1) return false;
+    const Value &dv = M_.value(Ins.operands[0]);
+    if (dv.type.kind != ElemKind::Int8QTy || dv.type.dims.size() != 2 || dv.id != dv.root) return false;
+    if (dv.type.scale != qv.type.scale || dv.type.offset != qv.type.offset) return false;
+    const Value &data = M_.value(S.operands[1]), &idx = M_.value(S.operands[2]),
+                &len = M_.value(S.operands[3]);
+    if (!isFused(data.type.kind) || data.type.dims.size() != 2) return false;
+    bool fp16Scale = false, fourBit = false;
+    switch (data.type.kind) {
+    case ElemKind::UInt8FusedQTy: c.kind = MI355X_FUSED_U8_F32; break;
+    case ElemKind::UInt8FusedFP16QTy: c.kind = MI355X_FUSED_U8_F16; fp16Scale = true; break;
+    case ElemKind::UInt4FusedFP16QTy: c.kind = MI355X_FUSED_U4_F16; fp16Scale = fourBit = true; break;
+    default: c.kind = MI355X_FUSED_U4_F32; fourBit = true; break;
+    }
+    if (fp16Scale && !c.viaF16) return false; // not a legal lookup: let slws() report it
+    if (idx.type.kind != ElemKind::Int64ITy && idx.type.kind != ElemKind::Int32ITy) return false;
+    if (len.type.kind != ElemKind::Int32ITy) return false;
+    c.rows = (size_t)data.type.dims[0];
+    c.inLine = (size_t)data.type.dims[1];
+    c.cols = (size_t)sd.type.dims[1];
+    c.segs = (size_t)len.type.size();
+    c.nIdx = (size_t)idx.type.size();
+    const size_t so = fp16Scale ? 4 : 8;
+    if (c.inLine <= so || (c.inLine - so) * (fourBit ? 2 : 1) != c.cols) return false;
+    if ((size_t)sd.type.dims[0] != c.segs || c.segs > 4096 || c.segs == 0) return false;
+    if ((size_t)dv.type.dims[0] != c.segs) return false;
+    if (qv.type.size() != sd.type.size()) return false;
+    c.colOffset = (size_t)Ins.iattrs[0];
+    if (Ins.iattrs[0] < 0 || c.colOffset + c.cols > (size_t)dv.type.dims[1]) return false;
+    c.idx64 = idx.type.kind == ElemKind::Int64ITy;
+    c.acc16 = !S.iattrs.empty() && S.iattrs[0] != 0 && fp16Scale;
+    c.qScale = qv.type.scale;
+    c.qOffset = qv.type.offset;
+    c.data = Operand{&data};
+    c.idx = Operand{&idx};
+    c.len = Operand{&len};
+    c.dest = Operand{&dv};
+    c.length = p + 2 - at;
+    return true;
+  }
+
+  // Consecutive lookup chains of one shape feeding one tensor become a single
+  // multi-table launch. Returns the number of instructions consumed (0: none).
+  size_t multiSls(size_t at, MI355XFunction &out) {
+    std::vector<SlsChain> group;
+    size_t pos = at;
+    for (;;) {
+      SlsChain c;
+      if (!matchSlsChain(pos, c)) break;
+      if (!group.empty()) {
+        const SlsChain &g = group[0];
+        if (c.kind != g.kind || c.idx64 != g.idx64 || c.viaF16 != g.viaF16 || c.acc16 != g.acc16 ||
+            c.inLine != g.inLine || c.cols != g.cols || c.segs != g.segs || c.qScale != g.qScale ||
+            c.qOffset != g.qOffset || c.dest.v != g.dest.v)
+          break;
+      }
+      group.push_back(c);
+      pos += c.length;
+      if (group.size() == 1024) break;
+    }
+    if (group.empty()) return 0;
+    const size_t n = group.size();
+    const SlsChain g = group[0];
+    size_t maxRows = 0;
+    for (const auto &c : group) maxRows = std::max(maxRows, c.rows);
+    auto tabPtr = scratchPtr(gen_.addScratch(n * sizeof(mi355x_sls_table)));
+    const size_t stride = (size_t)g.dest.ty().dims[1];
+    const std::string name = insts_[at].name + (n > 1 ? "..." + insts_[pos - 1].name : "");
+    // the table array holds device addresses: written once the buffers are bound
+    out.setup.push_back({"mi355x_memcpy_h2d", name, strFormat(" tables=%zu", n),
+                         [=](const DeviceBindings &b) {
+                           std::vector<mi355x_sls_table> t(n);
+                           for (size_t i = 0; i < n; i++) {
+                             t[i].data = group[i].data.ptr(b);
+                             t[i].indices = group[i].idx.ptr(b);
+                             t[i].lengths = (const int32_t *)group[i].len.ptr(b);
+                             t[i].dest = group[i].dest.ptr(b) + group[i].colOffset;
+                             t[i].data_rows = group[i].rows;
+                             t[i].num_indices = group[i].nIdx;
+                           }
+                           int rc = mi355x_memcpy_h2d(tabPtr(b), t.data(), n * sizeof(mi355x_sls_table),
+                                                      b.stream);
+                           if (rc == MI355X_OK) rc = mi355x_stream_sync(b.stream);
+                           return rc;
+                         }});
+    const int outKind = g.viaF16 ? MI355X_SLS_OUT_I8_VIA_F16 : MI355X_SLS_OUT_I8;
+    out.launches.push_back(
+        {"mi355x_frwq_sls_multi", name,
+         strFormat(" tables=%zu max_rows=%zu in_line=%zu out_line=%zu segments=%zu stride=%zu", n, maxRows,
+                   g.inLine, g.cols, g.segs, stride) +
+             kv("kind", g.kind) + kv("idx_is_64", g.idx64) + kv("out_kind", outKind) +
+             strFormat(" out_scale=%.9g", (double)g.qScale) + kv("out_offset", g.qOffset) +
+             kv("fp16_accum", g.acc16),
+         [=](const DeviceBindings &b) {
+           return mi355x_frwq_sls_multi((const mi355x_sls_table *)tabPtr(b), n, maxRows, g.kind, g.idx64,
+                                        g.segs, g.inLine, g.cols, outKind, g.qScale, g.qOffset, stride,
+                                        g.acc16, b.stream);
+         }});
+    return pos - at;
   }
 
   Error slws(const Instruction &I, MI355XFunction &out, bool weighted) {

@@ -147,6 +147,7 @@ struct BackendOptions {
   bool fuseAddRelu = true;             // ElementAdd + Relu of its result in one pass
   bool fuseConvAdd = true;             // convolution + ElementAdd (+ Relu) in one kernel
   bool spaceToDepthStem = true;        // stride-2 convolutions over <= 4 channels via space-to-depth
+  bool fuseSlsChains = true;           // pooled lookups + ConvertTo/Quantize/InsertTensor, many tables per launch
 };
 
 class MI355XBackend {

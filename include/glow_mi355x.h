@@ -432,6 +432,40 @@ int mi355x_frwq_slws(void *dest, int out_is_f16, const uint8_t *data,
                      size_t segments, size_t in_line_size,
                      size_t out_line_size, int fp16_accum, void *stream);
 
+/* FusedRowwiseQuantizedSparseLengthsSum over several tables of one shape in ONE
+ * launch (a ranking model pools dozens of tables per request, each too small
+ * to fill the chip on its own), optionally with the instructions that follow
+ * each lookup folded into its store. No counterpart in the reference, whose
+ * CPU backend runs the tables one after another.
+ *   tables    DEVICE array of n_tables entries (all pointers device pointers;
+ *             data 16-byte aligned)
+ *   segments  bags per table (at most 4096); every table has in_line_size-byte
+ *             rows of `kind`, at most max_data_rows of them
+ *   out_kind  MI355X_SLS_OUT_F32 / _F16: dense [segments x out_line_size] rows at
+ *             tables[t].dest, as mi355x_frwq_slws writes them;
+ *             MI355X_SLS_OUT_I8 / _I8_VIA_F16: Quantize(out_scale, out_offset) of
+ *             the fp32 result (_I8) or of the result rounded to fp16 and
+ *             converted back (_I8_VIA_F16: lookup with a Float16 result, ConvertTo
+ *             Float, Quantize), int8 rows dest_row_stride bytes apart starting at
+ *             tables[t].dest (InsertTensor into a wider tensor).
+ * Indices are int64 (idx_is_64) or int32 for all tables; no weights. */
+typedef struct {
+  const uint8_t *data;
+  const void *indices;
+  const int32_t *lengths;
+  void *dest;
+  uint64_t data_rows;
+  uint64_t num_indices;
+} mi355x_sls_table;
+enum { MI355X_SLS_OUT_F32 = 0, MI355X_SLS_OUT_F16 = 1, MI355X_SLS_OUT_I8 = 2,
+       MI355X_SLS_OUT_I8_VIA_F16 = 3 };
+int mi355x_frwq_sls_multi(const mi355x_sls_table *tables, size_t n_tables,
+                          size_t max_data_rows, int kind, int idx_is_64,
+                          size_t segments, size_t in_line_size,
+                          size_t out_line_size, int out_kind, float out_scale,
+                          int32_t out_offset, size_t dest_row_stride,
+                          int fp16_accum, void *stream);
+
 /* libjit_embedding_bag_byte_rowwise_offsets_f (libjit.cpp:2454-2481) and the
  * Interpreter's 4-bit / fp16 twin: bags are given by int32 start offsets
  * (`segments` entries, the last one being the end offset when

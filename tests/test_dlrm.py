@@ -17,8 +17,18 @@ def test_builds_and_compiles():
     net, max_idx = dlrm.make(seed=2, **SMALL)
     m, f = netlib.to_module(net)
     m.compile(f)
+    rows = [r for r in H.parse_listing(m.describe(f)) if r["phase"] == "launch"]
+    k = [r["kernel"] for r in rows]
+    # the three lookups with their ConvertTo / Quantize / InsertTensor are one launch
+    assert k.count("mi355x_frwq_sls_multi") == 1 and "mi355x_frwq_slws" not in k
+    multi = rows[k.index("mi355x_frwq_sls_multi")]
+    assert (multi["tables"], multi["out_kind"], multi["stride"]) == (3, 3, 4 * 16)
+    assert k.count("mi355x_convert_f16_to_f32") == 0 and k.count("mi355x_insert_rows") == 3
+    m, f = netlib.to_module(net)
+    m.compile(f, fuse_sls_chains=False)
     k = [r["kernel"] for r in H.parse_listing(m.describe(f)) if r["phase"] == "launch"]
     assert k.count("mi355x_frwq_slws") == 3 and k.count("mi355x_rwq_fc_i8") == 4
+    assert k.count("mi355x_convert_f16_to_f32") == 3 and k.count("mi355x_insert_rows") == 6
     assert k.count("mi355x_batch_matmul_i8") == 1 and k.count("mi355x_gather") == 1
     assert k[-1] == "mi355x_sigmoid_f32"
     # 4 vectors of 16 -> 6 pairs + 16 dense outputs feed the top MLP
@@ -35,11 +45,12 @@ def test_oracle_executes_the_small_network():
 
 
 @pytest.mark.gpu
-def test_device_matches_oracle():
+@pytest.mark.parametrize("fuse", [True, False])
+def test_device_matches_oracle(fuse):
     cfg = dict(tables=4, rows=5000, dim=64, batch=256, mean_len=8, bottom=(64, 64), top=(128, 1))
     net, max_idx = dlrm.make(seed=3, **cfg)
     m, f = netlib.to_module(net)
-    m.compile(f)
+    m.compile(f, fuse_sls_chains=fuse)
     dm = H.DeviceManager().init()
     try:
         dm.add_network(m)

@@ -68,3 +68,34 @@ def test_sigmoid():
     rng = np.random.default_rng(5)
     x = np.concatenate([rng.normal(0, 5, 10000), [0.0, 30.0, -30.0, 88.0, -88.0]]).astype(np.float32)
     np.testing.assert_allclose(capi.sigmoid_f32(x), go.sigmoid_f32(x), rtol=1e-5, atol=1e-37)
+
+
+@pytest.mark.parametrize("kind,cols,idt", [(2, 64, np.int64), (0, 128, np.int32), (1, 40, np.int64),
+                                           (3, 16, np.int32)])
+def test_multi_table_sls(kind, cols, idt):
+    """Several tables in one launch give what one launch per table gives; with
+    the int8 output kinds, what ConvertTo + Quantize + InsertTensor behind each
+    lookup give."""
+    from tests import cases
+    rng = np.random.default_rng(40 + kind)
+    n, bags = 5, 300
+    tables = [cases.random_fused_table(rng, 700 + 10 * t, cols, kind) for t in range(n)]
+    lens, idx = [], []
+    for t in range(n):
+        ln, ix, _ = cases.slws_batch(50 + t, tables[t].shape[0], bags, 7, 1.1, idt, weighted=False)
+        if t == 2:
+            ln[:] = 0                       # a table whose bags are all empty
+            ix = ix[:0]
+        lens.append(ln)
+        idx.append(ix)
+    f16 = kind in (1, 2)
+    want = [go.frwq_slws_generic(tables[t], kind, None, idx[t], lens[t], out_f16=f16) for t in range(n)]
+    got = capi.frwq_sls_multi(tables, kind, idx, lens,
+                              capi.SLS_OUT_F16 if f16 else capi.SLS_OUT_F32)
+    for t in range(n):
+        np.testing.assert_array_equal(got[t], want[t], err_msg=f"table {t}")
+    scale, off = 0.37, -11
+    wq = np.concatenate([go.quantize_i8(w.astype(np.float32), scale, off) for w in want], axis=1)
+    gq = capi.frwq_sls_multi(tables, kind, idx, lens,
+                             capi.SLS_OUT_I8_VIA_F16 if f16 else capi.SLS_OUT_I8, scale, off)
+    np.testing.assert_array_equal(gq, wq)
