@@ -1270,61 +1270,94 @@ static bool sameBindings(const DeviceBindings &a, const DeviceBindings &b) {
          a.mutableMem == b.mutableMem && a.activations == b.activations;
 }
 
+static bool launchesConflict(const KernelLaunch &early, const KernelLaunch &late) {
+  for (const auto &w : early.writes) {
+    for (const auto &r : late.reads) if (w.overlaps(r)) return true;
+    for (const auto &x : late.writes) if (w.overlaps(x)) return true;
+  }
+  for (const auto &r : early.reads)
+    for (const auto &w : late.writes) if (r.overlaps(w)) return true;
+  return false;
+}
+
+// The launches form a dependence DAG (read/write sets). Each launch is put on
+// the stream ("lane") of its latest predecessor when it can continue that
+// chain, on an unused lane otherwise; dependences across lanes become event
+// waits. Captured this way the graph runs independent chains side by side.
 Error MI355XFunction::captureGraph(const DeviceBindings &b, const std::vector<void *> &sideStreams) {
   dropGraph();
   if (launches.empty()) return Error::success();
   if (!b.stream)
     return MI355X_MAKE_ERR(ErrorCode::RUNTIME_ERROR, "graph capture needs a created stream");
-  // launches grouped by dependence level, in program order inside a level
-  int levels = 0;
-  for (const auto &l : launches) levels = std::max(levels, l.level + 1);
-  std::vector<std::vector<const KernelLaunch *>> byLevel((size_t)levels);
-  for (const auto &l : launches) byLevel[(size_t)l.level].push_back(&l);
-  const size_t nSide = sideStreams.size();
-  // one fork event, and one join event per side stream
+  const size_t n = launches.size(), nLanes = sideStreams.size() + 1;
+  std::vector<std::vector<size_t>> preds(n);
+  for (size_t i = 0; i < n; i++)
+    for (size_t j = 0; j < i; j++)
+      if (launchesConflict(launches[j], launches[i])) preds[i].push_back(j);
+  std::vector<int> lane(n, 0);
+  std::vector<long long> last(nLanes, -1);    // last launch put on each lane
+  for (size_t i = 0; i < n; i++) {
+    int pick = -1;
+    for (auto it = preds[i].rbegin(); it != preds[i].rend() && pick < 0; ++it)
+      if (last[(size_t)lane[*it]] == (long long)*it) pick = lane[*it]; // continue a chain
+    if (pick < 0)
+      for (size_t l = 0; l < nLanes && pick < 0; l++)
+        if (last[l] < 0) pick = (int)l;                                  // an unused lane
+    if (pick < 0) pick = preds[i].empty() ? 0 : lane[preds[i].back()];
+    lane[i] = pick;
+    last[(size_t)pick] = (long long)i;
+  }
+  // which launches need an event recorded behind them
+  std::vector<char> needsEvent(n, 0);
+  for (size_t i = 0; i < n; i++)
+    for (size_t p : preds[i])
+      if (lane[p] != lane[i]) needsEvent[p] = 1;
+  for (size_t l = 1; l < nLanes; l++)
+    if (last[l] >= 0) needsEvent[(size_t)last[l]] = 1;                   // joined at the end
+  std::vector<void *> events(n, nullptr);
   void *fork = nullptr;
-  std::vector<void *> joins(nSide, nullptr);
+  auto streamOf = [&](int l) { return l == 0 ? b.stream : sideStreams[(size_t)l - 1]; };
   auto cleanup = [&] {
     if (fork) mi355x_event_destroy(fork);
-    for (void *e : joins) if (e) mi355x_event_destroy(e);
+    for (void *e : events) if (e) mi355x_event_destroy(e);
   };
-  if (nSide) {
-    int rc = mi355x_event_create(&fork);
-    for (size_t i = 0; i < nSide && rc == MI355X_OK; i++) rc = mi355x_event_create(&joins[i]);
-    if (rc != MI355X_OK) {
-      cleanup();
-      return MI355X_MAKE_ERR(ErrorCode::RUNTIME_ERROR, "%s", mi355x_last_error());
-    }
+  int rc = mi355x_event_create(&fork);
+  for (size_t i = 0; i < n && rc == MI355X_OK; i++)
+    if (needsEvent[i]) rc = mi355x_event_create(&events[i]);
+  if (rc != MI355X_OK) {
+    cleanup();
+    return MI355X_MAKE_ERR(ErrorCode::RUNTIME_ERROR, "%s", mi355x_last_error());
   }
   if (mi355x_graph_begin_capture(b.stream) != MI355X_OK) {
     cleanup();
     return MI355X_MAKE_ERR(ErrorCode::RUNTIME_ERROR, "%s", mi355x_last_error());
   }
-  int rc = MI355X_OK;
   std::string failed;
-  for (const auto &group : byLevel) {
-    const size_t branches = std::min(group.size(), nSide + 1);
-    if (branches > 1) {
-      rc = mi355x_event_record(fork, b.stream);
-      for (size_t s = 0; s + 1 < branches && rc == MI355X_OK; s++)
-        rc = mi355x_stream_wait_event(sideStreams[s], fork);
+  std::vector<char> forked(nLanes, 0);
+  forked[0] = 1;
+  rc = mi355x_event_record(fork, b.stream);
+  for (size_t i = 0; i < n && rc == MI355X_OK; i++) {
+    void *st = streamOf(lane[i]);
+    if (!forked[(size_t)lane[i]]) {         // a side lane joins the capture
+      rc = mi355x_stream_wait_event(st, fork);
+      forked[(size_t)lane[i]] = 1;
     }
-    for (size_t i = 0; i < group.size() && rc == MI355X_OK; i++) {
-      DeviceBindings bb = b;
-      const size_t lane = i % branches;       // 0 = the capturing stream itself
-      if (lane) bb.stream = sideStreams[lane - 1];
-      rc = group[i]->launch(bb);
-      if (rc != MI355X_OK) failed = group[i]->kernel + " (" + group[i]->inst + "): " + mi355x_last_error();
-    }
-    for (size_t s = 0; s + 1 < branches && rc == MI355X_OK; s++) {
-      rc = mi355x_event_record(joins[s], sideStreams[s]);
-      if (rc == MI355X_OK) rc = mi355x_stream_wait_event(b.stream, joins[s]);
-    }
+    for (size_t p : preds[i])
+      if (lane[p] != lane[i] && rc == MI355X_OK) rc = mi355x_stream_wait_event(st, events[p]);
+    if (rc != MI355X_OK) break;
+    DeviceBindings bb = b;
+    bb.stream = st;
+    rc = launches[i].launch(bb);
     if (rc != MI355X_OK) {
-      if (failed.empty()) failed = mi355x_last_error();
+      failed = launches[i].kernel + " (" + launches[i].inst + "): " + mi355x_last_error();
       break;
     }
+    if (needsEvent[i]) rc = mi355x_event_record(events[i], st);
   }
+  // every side lane flows back into the capturing stream
+  for (size_t l = 1; l < nLanes && rc == MI355X_OK; l++)
+    if (last[l] >= 0 && forked[l]) rc = mi355x_stream_wait_event(b.stream, events[(size_t)last[l]]);
+  if (rc != MI355X_OK && failed.empty()) failed = mi355x_last_error();
   mi355x_graph *g = nullptr;
   const int rc2 = mi355x_graph_end_capture(b.stream, &g);
   cleanup();
