@@ -472,3 +472,25 @@ def test_rescale_both_multiplier_paths():
             np.testing.assert_array_equal(capi.rescale_i8(q, oo, io, pre, post, sc),
                                           go.rescale_i8(q, oo, io, pre, post, sc),
                                           err_msg=f"scale {sc} pre {pre} post {post}")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tile", list(range(6)))
+def test_every_gemm_tile_gives_the_same_result(tile):
+    """Results do not depend on the workgroup tile."""
+    c = cases.rwq_fc_case(60 + tile, 700, 192, 330, symmetric=False)
+    cc = cases.cwq_conv_case(70 + tile, 3, 20, 20, 32, 96, in_offset=-4, symmetric=False)
+    cg = cases.cwq_conv_case(80 + tile, 2, 12, 12, 64, 64, group=2, in_offset=3)
+    want_fc = go.rwq_fc_i8(*cases.rwq_fc_args(c))
+    want_cv = go.cwq_conv2d_i8(*cases.cwq_conv_args(cc))
+    want_cg = go.cwq_conv2d_i8(*cases.cwq_conv_args(cg))
+    capi.check(capi.lib().mi355x_gemm_tile_override(tile))
+    try:
+        got_fc = capi.rwq_fc_i8(*cases.rwq_fc_args(c))
+        got_cv = capi.cwq_conv2d_i8(*cases.cwq_conv_args(cc))
+        got_cg = capi.cwq_conv2d_i8(*cases.cwq_conv_args(cg))
+    finally:
+        capi.check(capi.lib().mi355x_gemm_tile_override(-1))
+    np.testing.assert_array_equal(got_fc, want_fc)
+    np.testing.assert_array_equal(got_cv, want_cv)
+    np.testing.assert_array_equal(got_cg, want_cg)
