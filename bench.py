@@ -360,9 +360,11 @@ def bench_resnet50(args):
     dm = H.DeviceManager().init()
     try:
         dm.add_network(m)
-        x = resnet50.synthetic_images(77, batch, size)
-        prob = np.zeros((batch, 1000), np.float32)
-        logits = np.zeros((batch, 1000), np.int8)
+        # request buffers in pinned host memory (allocateDeviceIOBuffer)
+        from glow_amd import capi
+        x = capi.pinned_copy(resnet50.synthetic_images(77, batch, size))
+        prob = capi.pinned_empty((batch, 1000), np.float32)
+        logits = capi.pinned_empty((batch, 1000), np.int8)
         dm.run("main", {"input": x, "prob": prob, "logits_q": logits})
         reps = max(3, args.steps // 10)
         ms = dm.time_function("main", reps)
@@ -401,8 +403,9 @@ def bench_dlrm(args):
     try:
         dm.add_network(m)
         inp = dlrm.Inputs(99, tables, args.dlrm_rows, batch, 20, 1.1, 13)
-        b = dlrm.bindings(net, inp, max_idx)
-        prob = np.zeros((batch, 1), np.float32)
+        from glow_amd import capi
+        b = {k: capi.pinned_copy(v) for k, v in dlrm.bindings(net, inp, max_idx).items()}
+        prob = capi.pinned_empty((batch, 1), np.float32)
         dm.run("main", dict(b, prob=prob))
         reps = max(5, args.steps // 4)
         ms = dm.time_function("main", reps)

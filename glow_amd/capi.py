@@ -199,6 +199,48 @@ def to_device(a):
     return DeviceBuffer.from_numpy(a)
 
 
+class _Pinned:
+    """Owner of one pinned host allocation (DeviceManager::allocateDeviceIOBuffer)."""
+
+    def __init__(self, nbytes):
+        p = C.c_void_p(0)
+        check(lib().mi355x_host_alloc(C.byref(p), _sz(max(int(nbytes), 1))))
+        self.ptr = p.value
+
+    def __del__(self):
+        try:
+            if self.ptr:
+                lib().mi355x_host_free(C.c_void_p(self.ptr))
+                self.ptr = 0
+        except Exception:
+            pass
+
+
+def pinned_empty(shape, dtype):
+    """A numpy array in pinned host memory: copies to and from the device run at
+    full PCIe rate and asynchronously. The memory lives as long as the array."""
+    dtype = np.dtype(dtype)
+    shape = tuple(int(s) for s in np.atleast_1d(shape))
+    n = int(np.prod(shape, dtype=np.int64)) * dtype.itemsize
+    owner = _Pinned(n)
+    buf = (C.c_char * max(n, 1)).from_address(owner.ptr)
+    arr = np.frombuffer(buf, dtype=dtype, count=n // dtype.itemsize).reshape(shape)
+    _PINNED_OWNERS[id(buf)] = owner
+    # the ctypes buffer is the array's base; tie the allocation's life to it
+    import weakref
+    weakref.finalize(buf, _PINNED_OWNERS.pop, id(buf), None)
+    return arr
+
+
+_PINNED_OWNERS = {}
+
+
+def pinned_copy(a):
+    out = pinned_empty(a.shape, a.dtype)
+    out[...] = a
+    return out
+
+
 class Stream:
     def __init__(self):
         p = C.c_void_p(0)

@@ -494,3 +494,16 @@ def test_every_gemm_tile_gives_the_same_result(tile):
     np.testing.assert_array_equal(got_fc, want_fc)
     np.testing.assert_array_equal(got_cv, want_cv)
     np.testing.assert_array_equal(got_cg, want_cg)
+
+
+@pytest.mark.gpu
+def test_pinned_host_arrays_round_trip():
+    a = capi.pinned_copy(np.arange(100000, dtype=np.float32).reshape(100, 1000))
+    d = capi.to_device(a)
+    b = capi.pinned_empty(a.shape, a.dtype)
+    capi.check(capi.lib().mi355x_memcpy_d2h(capi._vp(b), capi._vp(d), capi._sz(a.nbytes), capi._vp(None)))
+    capi.sync()
+    np.testing.assert_array_equal(a, b)
+    del a, b
+    import gc
+    gc.collect()
