@@ -23,7 +23,8 @@ EXPORTS = [
     "mi355x_device_info", "mi355x_malloc", "mi355x_free", "mi355x_host_alloc",
     "mi355x_host_free", "mi355x_memcpy_h2d", "mi355x_memcpy_d2h",
     "mi355x_memcpy_d2d", "mi355x_fill_u8", "mi355x_copy_u8", "mi355x_gemm_tile_override",
-    "mi355x_cwq_conv2d_add_i8", "mi355x_frwq_sls_multi", "mi355x_add_i8", "mi355x_add_relu_i8",
+    "mi355x_cwq_conv2d_add_i8", "mi355x_frwq_sls_multi",
+    "mi355x_specialize_bias_weights_qparams", "mi355x_rwq_slws", "mi355x_add_i8", "mi355x_add_relu_i8",
     "mi355x_relu_i8", "mi355x_convert_f16_to_f32", "mi355x_insert_rows",
     "mi355x_batch_transpose_i8", "mi355x_space_to_depth2_i8", "mi355x_gather", "mi355x_batch_matmul_i8", "mi355x_sigmoid_f32",
     "mi355x_max_pool_i8", "mi355x_avg_pool_i8", "mi355x_softmax_f32", "mi355x_stream_create",
@@ -381,6 +382,16 @@ def choose_quantization_params(mn, mx, schema=SCHEMA_ASYMMETRIC, qty=QTY_INT8):
         C.c_float(mn), C.c_float(mx), C.c_int(schema), C.c_int(qty),
         C.byref(s), C.byref(o)))
     return s.value, o.value
+
+
+def specialize_bias_weights_qparams(bias_scale, bias_offset, input_scale, weights_scale,
+                                    bias_is_i32=True, bias_is_zero=False):
+    """-> (bias_scale, bias_offset, weights_scale)."""
+    bs, bo, ws = C.c_float(bias_scale), C.c_int32(bias_offset), C.c_float(weights_scale)
+    check(lib().mi355x_specialize_bias_weights_qparams(
+        C.byref(bs), C.byref(bo), C.c_float(input_scale), C.byref(ws),
+        C.c_int(int(bias_is_i32)), C.c_int(int(bias_is_zero))))
+    return bs.value, bo.value, ws.value
 
 
 def fused_row_bytes(cols, kind):
@@ -984,3 +995,23 @@ def frwq_sls_multi(tables, kind, indices, lengths, out_kind=SLS_OUT_F32, out_sca
     if q8:
         return out.numpy()
     return [o.numpy() for o in outs]
+
+
+def rwq_slws(data, scales, offsets, weights, indices, lengths):
+    """RowwiseQuantizedSparseLengthsWeightedSum: uint8 rows, separate fp32
+    scales and offsets per row."""
+    data = np.ascontiguousarray(data, np.uint8)
+    scales = np.ascontiguousarray(scales, np.float32)
+    offsets = np.ascontiguousarray(offsets, np.float32)
+    indices = np.ascontiguousarray(indices)
+    lengths = np.ascontiguousarray(lengths, np.int32)
+    d_d, d_s, d_o = to_device(data), to_device(scales), to_device(offsets)
+    d_i = to_device(indices if indices.size else np.zeros(1, indices.dtype))
+    d_l = to_device(lengths)
+    d_w = None if weights is None else to_device(np.ascontiguousarray(weights, np.float32))
+    out = DeviceBuffer.empty((lengths.size, data.shape[1]), np.float32)
+    check(lib().mi355x_rwq_slws(_vp(out), _vp(d_d), _sz(data.shape[0]), _vp(d_s), _vp(d_o),
+                                _vp(d_w), _vp(d_i), C.c_int(indices.dtype == np.int64),
+                                _sz(indices.size), _vp(d_l), _sz(lengths.size),
+                                _sz(data.shape[1]), _vp(None)))
+    return out.numpy()

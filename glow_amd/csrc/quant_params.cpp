@@ -207,6 +207,25 @@ int mi355x_fused_rowwise_quantize_host(const float *in, size_t rows,
   return MI355X_OK;
 }
 
+int mi355x_specialize_bias_weights_qparams(float *bias_scale, int32_t *bias_offset,
+                                           float input_scale, float *weights_scale,
+                                           int bias_is_i32, int bias_is_zero) {
+  MI355X_REQUIRE(bias_scale && bias_offset && weights_scale, "NULL argument");
+  // an int32 bias always gets offset 0: its range makes that free
+  if (bias_is_i32) *bias_offset = 0;
+  const float product = input_scale * *weights_scale;
+  if (product >= *bias_scale || bias_is_zero) {
+    // the bias can take the accumulator's own scale without saturating
+    *bias_scale = product;
+  } else if (bias_is_i32) {
+    // otherwise the weights scale gives way, and the product is formed again
+    // so that it equals the bias scale exactly
+    *weights_scale = *bias_scale / input_scale;
+    *bias_scale = input_scale * *weights_scale;
+  }
+  return MI355X_OK;
+}
+
 int mi355x_rowwise_quantize_i8_host(const float *in, size_t rows, size_t cols,
                                     int schema, int8_t *out, float *scales,
                                     int32_t *offsets) {

@@ -58,6 +58,9 @@ struct SlwsArgs {
   int32_t data_bytes;      // quantized bytes per row (before scale/offset)
   int32_t out_cols;
   int32_t out16, w16, idx64;
+  // rowwise (not fused) tables: scale and offset of row r are sep_scales[r],
+  // sep_offsets[r] (fp32) and rows hold data bytes only
+  const float *sep_scales, *sep_offsets;
   // multi-table launches: blockIdx.y selects the table whose pointers replace
   // the ones above
   const mi355x_sls_table *tables;
@@ -331,6 +334,9 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_kernel(SlwsArgs a) {
             uint32_t v = load_u32_any(so);
             s = __half2float(__ushort_as_half((unsigned short)(v & 0xffff)));
             o = __half2float(__ushort_as_half((unsigned short)(v >> 16)));
+          } else if (a.sep_scales) {
+            s = a.sep_scales[row];
+            o = a.sep_offsets[row];
           } else {
             s = __uint_as_float(load_u32_any(so));
             o = __uint_as_float(load_u32_any(so + 4));
@@ -494,9 +500,14 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_wave_kernel(SlwsArgs a) {
         // after the row reads below have been issued, so that the two
         // dependent round trips (index -> scale/offset, index -> row bytes)
         // overlap instead of following each other.
-        const uint8_t *so = a.data + row * a.in_line + a.data_bytes;
-        so_lo = load_u32_any(so);
-        if constexpr (!SO16) so_hi = load_u32_any(so + 4);
+        if (!SO16 && a.sep_scales) {
+          so_lo = __float_as_uint(a.sep_scales[row]);
+          so_hi = __float_as_uint(a.sep_offsets[row]);
+        } else {
+          const uint8_t *so = a.data + row * a.in_line + a.data_bytes;
+          so_lo = load_u32_any(so);
+          if constexpr (!SO16) so_hi = load_u32_any(so + 4);
+        }
       }
       // round 2: all row reads of the batch in flight before the first use.
       // Lookups are taken four at a time under one uniform branch; slots
@@ -664,6 +675,7 @@ static void launch_wave_kind(int kind, bool acc16, dim3 grid, hipStream_t st,
 
 // Several tables in one launch and/or the int8 output transform.
 struct SlwsExtra {
+  const float *sep_scales = nullptr, *sep_offsets = nullptr; // rowwise tables
   const mi355x_sls_table *tables = nullptr; // device array
   size_t n_tables = 1;
   int out_q8 = 0;
@@ -687,7 +699,7 @@ static int slws_dispatch(void *dest, int out_is_f16, const uint8_t *data,
   MI355X_REQUIRE(x.n_tables <= 65535, "more than 65535 tables");
   const bool is4 = kind == MI355X_FUSED_U4_F16 || kind == MI355X_FUSED_U4_F32;
   const bool so16 = kind == MI355X_FUSED_U8_F16 || kind == MI355X_FUSED_U4_F16;
-  const size_t so_bytes = so16 ? 4 : 8;
+  const size_t so_bytes = x.sep_scales ? 0 : (so16 ? 4 : 8);
   MI355X_REQUIRE(in_line_size > so_bytes, "in_line_size %zu too small",
                  in_line_size);
   const size_t data_bytes = in_line_size - so_bytes;
@@ -723,6 +735,8 @@ static int slws_dispatch(void *dest, int out_is_f16, const uint8_t *data,
   a.out16 = out_is_f16;
   a.w16 = weights_are_f16;
   a.idx64 = idx_is_64;
+  a.sep_scales = x.sep_scales;
+  a.sep_offsets = x.sep_offsets;
   a.tables = x.tables;
   a.out_q8 = x.out_q8;
   a.q_scale = x.q_scale;
@@ -790,6 +804,21 @@ int mi355x_frwq_sls_multi(const mi355x_sls_table *tables, size_t n_tables,
   return slws_dispatch(nullptr, out16, nullptr, max_data_rows, kind, nullptr, 0, nullptr,
                        idx_is_64, 0, nullptr, nullptr, 0, segments, in_line_size,
                        out_line_size, fp16_accum, stream, x);
+}
+
+int mi355x_rwq_slws(float *dest, const uint8_t *data, size_t data_rows,
+                    const float *scales, const float *offsets, const float *weights,
+                    const void *indices, int idx_is_64, size_t num_indices,
+                    const int32_t *lengths, size_t segments, size_t line_size,
+                    void *stream) {
+  MI355X_REQUIRE(segments == 0 || lengths, "lengths is NULL");
+  MI355X_REQUIRE(segments == 0 || (scales && offsets), "NULL scales or offsets");
+  SlwsExtra x;
+  x.sep_scales = scales;
+  x.sep_offsets = offsets;
+  return slws_dispatch(dest, 0, data, data_rows, MI355X_FUSED_U8_F32, weights, 0, indices,
+                       idx_is_64, num_indices, lengths, nullptr, 0, segments, line_size,
+                       line_size, 0, stream, x);
 }
 
 int mi355x_frwq_slws(void *dest, int out_is_f16, const uint8_t *data,

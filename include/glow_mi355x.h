@@ -152,6 +152,15 @@ enum { MI355X_QTY_INT8 = 8, MI355X_QTY_INT16 = 16, MI355X_QTY_INT32 = 32,
 int mi355x_choose_quantization_params(float min, float max, int schema,
                                       int qty, float *scale, int32_t *offset);
 
+/* quantization::specializeBiasWeightsQuantizationParams (reference
+ * lib/Quantization/Base/Base.cpp:594-629): makes the bias scale equal
+ * inputScale * weightsScale (adjusting the weights scale for an int32 bias whose
+ * own scale is larger), offset 0 for an int32 bias. In/out: bias_scale,
+ * bias_offset, weights_scale. */
+int mi355x_specialize_bias_weights_qparams(float *bias_scale, int32_t *bias_offset,
+                                           float input_scale, float *weights_scale,
+                                           int bias_is_i32, int bias_is_zero);
+
 /* Fused-rowwise element kinds (reference include/glow/Base/Type.h:424-433):
  * row = [data | scale | offset], scale/offset fp32 or fp16; 4-bit rows hold
  * two columns per byte, even column in the low nibble. */
@@ -431,6 +440,16 @@ int mi355x_frwq_slws(void *dest, int out_is_f16, const uint8_t *data,
                      size_t num_indices, const int32_t *lengths,
                      size_t segments, size_t in_line_size,
                      size_t out_line_size, int fp16_accum, void *stream);
+
+/* libjit_rowwise_quantized_sparse_lengths_weighted_sum_f_u / _f_i32 (reference
+ * libjit.cpp:1232-1251, 2400-2414): the table holds uint8 rows of line_size
+ * bytes, the fp32 scale and offset of row r are scales[r] and offsets[r].
+ * weights NULL = all ones. */
+int mi355x_rwq_slws(float *dest, const uint8_t *data, size_t data_rows,
+                    const float *scales, const float *offsets, const float *weights,
+                    const void *indices, int idx_is_64, size_t num_indices,
+                    const int32_t *lengths, size_t segments, size_t line_size,
+                    void *stream);
 
 /* FusedRowwiseQuantizedSparseLengthsSum over several tables of one shape in ONE
  * launch (a ranking model pools dozens of tables per request, each too small

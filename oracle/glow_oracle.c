@@ -812,3 +812,25 @@ void go_gather(uint8_t *dest, const uint8_t *data, const int64_t *indices,
       outIdx++;
     }
 }
+
+/* libjit.cpp:1232-1251 */
+void go_rwq_slws_f32(float *dest, const uint8_t *data, const float *scales,
+                     const float *offsets, const float *weights,
+                     const void *indices, int indicesAre64, const int32_t *lengths,
+                     size_t segments, size_t lineSize) {
+  memset(dest, 0, segments * lineSize * sizeof(float));
+  size_t cur = 0;
+  for (size_t i = 0; i < segments; i++) {
+    for (int32_t j = 0; j < lengths[i]; j++) {
+      const float weight = weights[cur];
+      const size_t line = indicesAre64 ? (size_t)((const int64_t *)indices)[cur]
+                                       : (size_t)((const int32_t *)indices)[cur];
+      const float scale = scales[line], offset = offsets[line];
+      for (size_t k = 0; k < lineSize; k++) {
+        const float f = scale * (float)data[line * lineSize + k] + offset;
+        dest[i * lineSize + k] += weight * f;
+      }
+      cur++;
+    }
+  }
+}

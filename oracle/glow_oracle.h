@@ -188,6 +188,13 @@ void go_frwq_slws_generic(void *dest, int outIsF16, const uint8_t *data,
                           size_t inLineSize, size_t outLineSize,
                           int fp16Accum);
 
+/* libjit.cpp:1232-1251 (RowwiseQuantizedSparseLengthsWeightedSum: separate
+ * per-row scales and offsets). */
+void go_rwq_slws_f32(float *dest, const uint8_t *data, const float *scales,
+                     const float *offsets, const float *weights,
+                     const void *indices, int indicesAre64, const int32_t *lengths,
+                     size_t segments, size_t lineSize);
+
 /* libjit.cpp:2454-2481 (EmbeddingBagByteRowwiseOffsets, int32 indices and
  * offsets). */
 void go_embedding_bag_byte_rowwise_offsets_f32(

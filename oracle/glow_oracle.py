@@ -442,3 +442,15 @@ def batch_matmul_i8(lhs, rhs, out_offset, lhs_offset, rhs_offset, outP):
     """BatchMatMul as it is lowered: libjit_matmul_i8 on every pair of the batch."""
     return np.stack([matmul_i8(lhs[b], rhs[b], out_offset, lhs_offset, rhs_offset, outP)
                      for b in range(lhs.shape[0])])
+
+
+def rwq_slws_f32(data, scales, offsets, weights, indices, lengths):
+    data = _c(data, np.uint8)
+    scales, offsets, weights = _c(scales, np.float32), _c(offsets, np.float32), _c(weights, np.float32)
+    indices, i64 = _idx(indices)
+    lengths = _i32v(lengths)
+    out = np.empty((lengths.size, data.shape[1]), np.float32)
+    lib().go_rwq_slws_f32(_p(out), _p(data), _p(scales), _p(offsets), _p(weights), _p(indices),
+                          C.c_int(i64), _p(lengths), C.c_size_t(lengths.size),
+                          C.c_size_t(data.shape[1]))
+    return out

@@ -301,3 +301,18 @@ def gather64_i8(data, indices, num_samples, sample_size, slice_size):
                              C.c_uint64(slice_size), C.c_uint64(num_samples),
                              C.c_uint64(sample_size))
     return out
+
+
+def rwq_slws_f32(data, scales, offsets, weights, indices, lengths, fastmath=False):
+    """libjit.cpp:2400-2414"""
+    data = _c(data, np.uint8)
+    scales, offsets, weights = _c(scales, np.float32), _c(offsets, np.float32), _c(weights, np.float32)
+    indices = np.ascontiguousarray(indices)
+    lengths = _i32v(lengths)
+    out = np.empty((lengths.size, data.shape[1]), np.float32)
+    fn = (lib(fastmath).libjit_rowwise_quantized_sparse_lengths_weighted_sum_f_u
+          if indices.dtype == np.int64
+          else lib(fastmath).libjit_rowwise_quantized_sparse_lengths_weighted_sum_f_i32)
+    fn(_p(out), _p(data), _p(scales), _p(offsets), _p(weights), _p(indices), _p(lengths),
+       C.c_uint64(lengths.size), C.c_uint64(data.shape[1]))
+    return out

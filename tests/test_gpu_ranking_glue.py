@@ -99,3 +99,22 @@ def test_multi_table_sls(kind, cols, idt):
     gq = capi.frwq_sls_multi(tables, kind, idx, lens,
                              capi.SLS_OUT_I8_VIA_F16 if f16 else capi.SLS_OUT_I8, scale, off)
     np.testing.assert_array_equal(gq, wq)
+
+
+@pytest.mark.parametrize("cols,idt", [(128, np.int64), (37, np.int32), (64, np.int64), (16, np.int32)])
+def test_rowwise_quantized_slws(cols, idt):
+    """Separate per-row scales and offsets instead of fused rows (bit-exact)."""
+    rng = np.random.default_rng(cols)
+    rows, bags = 3000, 500
+    data = rng.integers(0, 256, (rows, cols), dtype=np.uint8)
+    scales = rng.uniform(0.001, 0.1, rows).astype(np.float32)
+    offsets = rng.normal(0, 1, rows).astype(np.float32)
+    lengths = rng.poisson(9, bags).astype(np.int32)
+    lengths[7] = 0
+    idx = rng.integers(0, rows, int(lengths.sum())).astype(idt)
+    w = rng.random(idx.size).astype(np.float32)
+    np.testing.assert_array_equal(capi.rwq_slws(data, scales, offsets, w, idx, lengths),
+                                  go.rwq_slws_f32(data, scales, offsets, w, idx, lengths))
+    ones = np.ones(idx.size, np.float32)
+    np.testing.assert_array_equal(capi.rwq_slws(data, scales, offsets, None, idx, lengths),
+                                  go.rwq_slws_f32(data, scales, offsets, ones, idx, lengths))

@@ -113,3 +113,16 @@ def test_rowwise_quantize_equals_oracle():
         for got, want in zip(capi.rowwise_quantize_i8_host(w, schema),
                              go.rowwise_quantize_i8(w, schema)):
             np.testing.assert_array_equal(got, want)
+
+
+def test_specialize_bias_weights_qparams_equals_oracle():
+    rng = np.random.default_rng(12)
+    for _ in range(200):
+        bs = float(np.float32(10 ** rng.uniform(-8, 0)))
+        ws = float(np.float32(10 ** rng.uniform(-4, 0)))
+        ins = float(np.float32(10 ** rng.uniform(-3, 0)))
+        bo = int(rng.integers(-5, 6))
+        for i32 in (True, False):
+            for zero in (False, True):
+                assert capi.specialize_bias_weights_qparams(bs, bo, ins, ws, i32, zero) == \
+                    go.specialize_bias_weights_qparams(bs, bo, ins, ws, i32, zero)

@@ -190,3 +190,18 @@ def test_ranking_glue_vs_ref():
                                   ref.gather64_i8(data, idx, 6, 60, 3))
     np.testing.assert_array_equal(go.gather(data, idx, 1), np.take(data, idx, axis=1))
     np.testing.assert_array_equal(go.gather(data, idx[:4] % 6, 0), data[idx[:4] % 6])
+
+
+@pytest.mark.parametrize("idt", [np.int64, np.int32])
+def test_rwq_slws_vs_ref(idt):
+    rng = np.random.default_rng(79)
+    rows, cols, bags = 300, 37, 40
+    data = rng.integers(0, 256, (rows, cols), dtype=np.uint8)
+    scales = rng.uniform(0.001, 0.1, rows).astype(np.float32)
+    offsets = rng.normal(0, 1, rows).astype(np.float32)
+    lengths = rng.poisson(6, bags).astype(np.int32)
+    lengths[5] = 0
+    idx = rng.integers(0, rows, int(lengths.sum())).astype(idt)
+    w = rng.random(idx.size).astype(np.float32)
+    np.testing.assert_array_equal(go.rwq_slws_f32(data, scales, offsets, w, idx, lengths),
+                                  ref.rwq_slws_f32(data, scales, offsets, w, idx, lengths))
