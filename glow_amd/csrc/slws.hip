@@ -191,11 +191,15 @@ __device__ __forceinline__ void bag_span_offsets(const SlwsArgs &a,
   start = 0;
   len = 0;
   if (bag < a.segments) {
-    start = a.offsets[bag];
-    const long long end = (!a.offsets_have_end && bag == a.segments - 1)
-                              ? a.num_indices
-                              : (long long)a.offsets[bag + 1];
-    len = end > start ? (int)min(end - start, 0x7fffffffLL) : 0;
+    // both ends are clamped into the index list, so that offsets that make no
+    // sense (negative, decreasing, past the end) give short or empty bags and
+    // never a position outside the list
+    start = min(max((long long)a.offsets[bag], 0LL), (long long)a.num_indices);
+    long long end = (!a.offsets_have_end && bag == a.segments - 1)
+                        ? a.num_indices
+                        : (long long)a.offsets[bag + 1];
+    end = min(max(end, start), (long long)a.num_indices);
+    len = (int)min(end - start, 0x7fffffffLL);
   }
 }
 

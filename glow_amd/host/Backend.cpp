@@ -119,6 +119,8 @@ public:
       case Kind::MaxPool: MI355X_RETURN_IF_ERR(pool(I, out, false)); break;
       case Kind::AvgPool: MI355X_RETURN_IF_ERR(pool(I, out, true)); break;
       case Kind::SoftMax: MI355X_RETURN_IF_ERR(softmax(I, out)); break;
+      case Kind::RowwiseQuantizedSparseLengthsWeightedSum:
+      case Kind::EmbeddingBagByteRowwiseOffsets: MI355X_RETURN_IF_ERR(otherLookups(I, out)); break;
       case Kind::ConvertTo:
       case Kind::InsertTensor:
       case Kind::Transpose:
@@ -189,7 +191,7 @@ public:
 
 private:
   static constexpr int kArity[(int)Kind::NumKinds] = {2, 2, 2, 4, 6, 3, 4, 8, 5, 4, 3, 2, 2, 2, 2,
-                                                       2, 2, 2, 3, 3, 2};
+                                                       2, 2, 2, 3, 3, 2, 7, 5};
 
   Error checkOperands(const Instruction &I) {
     CHECK_OP((int)I.kind >= 0 && (int)I.kind < (int)Kind::NumKinds, "unknown kind");
@@ -970,6 +972,60 @@ private:
                                        allZero ? 1 : 0, sums ? (const int32_t *)sumPtr(b) : nullptr,
                                        b.stream);
          }});
+    return Error::success();
+  }
+
+  // The two other pooled-lookup forms of the CPU backend (fp32 throughout).
+  Error otherLookups(const Instruction &I, MI355XFunction &out) {
+    Operand d = op(I, 0), data = op(I, 1);
+    CHECK_OP(d.ty().kind == ElemKind::FloatTy && d.ty().dims.size() == 2, "result must be 2-D float");
+    CHECK_OP(data.ty().dims.size() == 2, "data must be 2-D");
+    const size_t rows = (size_t)data.ty().dims[0], line = (size_t)data.ty().dims[1];
+    if (I.kind == Kind::RowwiseQuantizedSparseLengthsWeightedSum) {
+      Operand sc = op(I, 2), of = op(I, 3), w = op(I, 4), idx = op(I, 5), len = op(I, 6);
+      CHECK_OP(elemSize(data.ty().kind) == 1 && !isFused(data.ty().kind), "data must be plain 8-bit rows");
+      CHECK_OP(sc.ty().kind == ElemKind::FloatTy && of.ty().kind == ElemKind::FloatTy &&
+                   w.ty().kind == ElemKind::FloatTy,
+               "scales, offsets and weights must be float");
+      CHECK_OP((size_t)sc.ty().size() == rows && (size_t)of.ty().size() == rows,
+               "one scale and offset per row");
+      CHECK_OP(idx.ty().kind == ElemKind::Int64ITy || idx.ty().kind == ElemKind::Int32ITy,
+               "indices must be int64 or int32");
+      CHECK_OP(len.ty().kind == ElemKind::Int32ITy && w.ty().size() == idx.ty().size(),
+               "lengths must be int32; one weight per index");
+      CHECK_OP(d.ty().dims[0] == len.ty().size() && (size_t)d.ty().dims[1] == line, "result shape mismatch");
+      const size_t nIdx = (size_t)idx.ty().size(), segs = (size_t)len.ty().size();
+      const int i64 = idx.ty().kind == ElemKind::Int64ITy;
+      out.launches.push_back({"mi355x_rwq_slws", I.name,
+                              strFormat(" rows=%zu line=%zu segments=%zu num_indices=%zu", rows, line, segs, nIdx) +
+                                  kv("idx_is_64", i64),
+                              [=](const DeviceBindings &b) {
+                                return mi355x_rwq_slws((float *)d.ptr(b), data.ptr(b), rows, (const float *)sc.ptr(b),
+                                                       (const float *)of.ptr(b), (const float *)w.ptr(b), idx.ptr(b),
+                                                       i64, nIdx, (const int32_t *)len.ptr(b), segs, line, b.stream);
+                              }});
+      return Error::success();
+    }
+    Operand w = op(I, 2), idx = op(I, 3), offs = op(I, 4);
+    CHECK_OP(data.ty().kind == ElemKind::UInt8FusedQTy, "data must be ui8fused");
+    CHECK_OP(w.ty().kind == ElemKind::FloatTy && idx.ty().kind == ElemKind::Int32ITy &&
+                 offs.ty().kind == ElemKind::Int32ITy,
+             "needs float weights and int32 indices and offsets");
+    CHECK_OP(I.iattrs.size() == 1, "expects {hasEndOffset}");
+    const int hasEnd = I.iattrs[0] != 0;
+    const size_t segs = (size_t)offs.ty().size(), nIdx = (size_t)idx.ty().size();
+    CHECK_OP(line > 8 && (size_t)d.ty().dims[1] == line - 8 && (size_t)d.ty().dims[0] + hasEnd == segs &&
+                 w.ty().size() == idx.ty().size(),
+             "shape mismatch");
+    out.launches.push_back({"mi355x_embedding_bag_rowwise_offsets", I.name,
+                            strFormat(" rows=%zu in_line=%zu segments=%zu num_indices=%zu", rows, line, segs, nIdx) +
+                                kv("has_end_offset", hasEnd),
+                            [=](const DeviceBindings &b) {
+                              return mi355x_embedding_bag_rowwise_offsets(
+                                  d.ptr(b), 0, data.ptr(b), rows, MI355X_FUSED_U8_F32, w.ptr(b), 0,
+                                  (const int32_t *)idx.ptr(b), nIdx, (const int32_t *)offs.ptr(b), segs, hasEnd,
+                                  line, line - 8, 0, b.stream);
+                            }});
     return Error::success();
   }
 

@@ -248,6 +248,13 @@ Error MI355XDeviceManager::makeResident(const Module *module, const std::string 
     }
     mr.bytes = mi355x_arena_bytes(mr.arena);
     usedMemoryBytes_ += mr.bytes;
+    // placeholders start as zeros: the first (untimed) pass over a new network
+    // runs before any request has filled them
+    if (module->mutableSize()) {
+      void *mp = nullptr;
+      mi355x_arena_ptr(mr.arena, MI355X_REGION_MUTABLE, 0, &mp);
+      mi355x_fill_u8(mp, 0, module->mutableSize(), stream_);
+    }
     if (module->constantsSize()) {
       rc = mi355x_arena_upload(mr.arena, MI355X_REGION_CONSTANTS, 0,
                                module->constantsImage().data(), module->constantsSize(), stream_);
@@ -272,6 +279,11 @@ Error MI355XDeviceManager::makeResident(const Module *module, const std::string 
   if (rc != MI355X_OK) return failWith(fromStatus(rc, "function arena"));
   fr.bytes = mi355x_arena_bytes(fr.arena);
   usedMemoryBytes_ += fr.bytes;
+  if (rb.activationsMemSize) {
+    void *ap = nullptr;
+    mi355x_arena_ptr(fr.arena, MI355X_REGION_ACTIVATIONS, 0, &ap);
+    mi355x_fill_u8(ap, 0, rb.activationsMemSize, stream_);
+  }
   void *p = nullptr;
   mi355x_arena_ptr(mr.arena, MI355X_REGION_CONSTANTS, 0, &p);
   fr.bindings.constants = (uint8_t *)p;

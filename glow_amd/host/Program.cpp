@@ -98,6 +98,8 @@ const char *kindName(Kind k) {
   case Kind::Gather: return "Gather";
   case Kind::BatchMatMul: return "BatchMatMul";
   case Kind::Sigmoid: return "Sigmoid";
+  case Kind::RowwiseQuantizedSparseLengthsWeightedSum: return "RowwiseQuantizedSparseLengthsWeightedSum";
+  case Kind::EmbeddingBagByteRowwiseOffsets: return "EmbeddingBagByteRowwiseOffsets";
   default: return "?";
   }
 }

@@ -57,6 +57,8 @@ enum class Kind : int32_t {
   Gather,                       // (Dest, Data, Indices); iattrs {batchDims (0 or 1)}
   BatchMatMul,                  // (Dest [B,M,N], LHS [B,M,K], RHS [B,K,N]) int8
   Sigmoid,                      // (Dest, Src) float
+  RowwiseQuantizedSparseLengthsWeightedSum, // (Dest, Data u8 [rows,cols], Scales, Offsets, Weights, Indices, Lengths)
+  EmbeddingBagByteRowwiseOffsets, // (Dest, Data, Weights, Indices, Offsets); iattrs {hasEndOffset}
   NumKinds
 };
 const char *kindName(Kind k);

@@ -73,7 +73,9 @@ enum {
   MI355X_HOST_TRANSPOSE = 17,          /* Dest, Src int8; iattrs shuffle {1,0} or {0,2,1} */
   MI355X_HOST_GATHER = 18,             /* Dest, Data, Indices; iattrs {batchDims} */
   MI355X_HOST_BATCH_MATMUL = 19,       /* Dest [B,M,N], LHS [B,M,K], RHS [B,K,N] int8 */
-  MI355X_HOST_SIGMOID = 20             /* Dest, Src float */
+  MI355X_HOST_SIGMOID = 20,            /* Dest, Src float */
+  MI355X_HOST_RWQ_SLWS = 21,           /* Dest, Data u8, Scales, Offsets, Weights, Indices, Lengths */
+  MI355X_HOST_EMBEDDING_BAG_BYTE_ROWWISE_OFFSETS = 22 /* Dest, Data, Weights, Indices, Offsets; iattrs {hasEndOffset} */
 };
 /* Convolution iattrs: kernelH, kernelW, strideH, strideW, padT, padL, padB,
  * padR, group, dilationH, dilationW, fusedActivation (glow::FusedActivation);

@@ -233,3 +233,42 @@ def test_fc_and_conv_networks(dm):
         dm.run("main", {"input": cc["x"], "output": o})
         assert np.array_equal(o, go.cwq_conv2d_i8(*cases.cwq_conv_args(cc)))
         dm.evict_network("main")
+
+
+def test_other_lookup_forms(dm):
+    """RowwiseQuantizedSparseLengthsWeightedSum and EmbeddingBagByteRowwiseOffsets
+    as instructions of one function."""
+    rng = np.random.default_rng(23)
+    rows, cols, bags = 800, 32, 60
+    data = rng.integers(0, 256, (rows, cols), dtype=np.uint8)
+    scales = rng.uniform(0.001, 0.1, rows).astype(np.float32)
+    offs = rng.normal(0, 1, rows).astype(np.float32)
+    fused = cases.random_fused_table(rng, rows, cols)
+    lengths = rng.poisson(5, bags).astype(np.int32)
+    n = int(lengths.sum())
+    idx = rng.integers(0, rows, n).astype(np.int32)
+    w = rng.random(n).astype(np.float32)
+    starts = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)     # with the end offset
+    m = H.Module("lookups")
+    c_data = m.constant("data", data, H.INT8Q)
+    c_sc = m.constant("scales", scales)
+    c_of = m.constant("offsets", offs)
+    c_fused = m.constant("fused", fused, H.UINT8_FUSED)
+    p_w = m.placeholder("weights", (n,), H.FLOAT, np.float32)
+    p_i = m.placeholder("indices", (n,), H.INT32I, np.int32)
+    p_l = m.placeholder("lengths", (bags,), H.INT32I, np.int32)
+    p_s = m.placeholder("starts", (bags + 1,), H.INT32I, np.int32)
+    o1 = m.placeholder("out_rwq", (bags, cols), H.FLOAT, np.float32)
+    o2 = m.placeholder("out_bag", (bags, cols), H.FLOAT, np.float32)
+    f = m.function("main")
+    m.instruction(f, H.RWQ_SLWS, "rwq", [o1, c_data, c_sc, c_of, p_w, p_i, p_l])
+    m.instruction(f, H.EMBEDDING_BAG_BYTE_ROWWISE_OFFSETS, "bag", [o2, c_fused, p_w, p_i, p_s], [1])
+    m.compile(f)
+    dm.add_network(m)
+    r1 = np.zeros((bags, cols), np.float32)
+    r2 = np.zeros((bags, cols), np.float32)
+    dm.run("main", {"weights": w, "indices": idx, "lengths": lengths, "starts": starts,
+                    "out_rwq": r1, "out_bag": r2})
+    np.testing.assert_array_equal(r1, go.rwq_slws_f32(data, scales, offs, w, idx, lengths))
+    np.testing.assert_array_equal(
+        r2, go.embedding_bag_byte_rowwise_offsets_f32(fused, w, idx, starts, True))

@@ -507,3 +507,26 @@ def test_pinned_host_arrays_round_trip():
     del a, b
     import gc
     gc.collect()
+
+
+@pytest.mark.gpu
+def test_embedding_bag_with_senseless_offsets_stays_in_bounds():
+    """Negative, decreasing and oversized start offsets give short or empty
+    bags; valid bags next to them are unaffected."""
+    rng = np.random.default_rng(77)
+    rows, cols = 500, 64
+    table = cases.random_fused_table(rng, rows, cols)
+    idx = rng.integers(0, rows, 200).astype(np.int32)
+    w = rng.random(200).astype(np.float32)
+    offs = np.array([0, 10, -50, 30, 25, 40, 100000, 60, 200], np.int32)
+    got = capi.embedding_bag_rowwise_offsets(table, capi.FUSED_U8_F32, w, idx, offs, True)
+    # bag 0 = [0,10) and bag 7 = [60,200) are well formed
+    good = go.embedding_bag_byte_rowwise_offsets_f32(table, w, idx, np.array([0, 10], np.int32), True)
+    np.testing.assert_array_equal(got[0], good[0])
+    good7 = go.embedding_bag_byte_rowwise_offsets_f32(table, w, idx, np.array([60, 200], np.int32), True)
+    np.testing.assert_array_equal(got[7], good7[0])
+    assert np.all(np.isfinite(got))
+    # [40, 100000) is cut at the end of the index list; [100000, 60) is empty
+    cut = go.embedding_bag_byte_rowwise_offsets_f32(table, w, idx, np.array([40, 200], np.int32), True)
+    np.testing.assert_array_equal(got[5], cut[0])
+    assert not got[6].any()
