@@ -137,6 +137,13 @@ struct DenseRows {
     if constexpr (ALIGNED) {
       return *reinterpret_cast<const int4 *>(r.base + k);
     } else {
+      // a whole chunk inside the row: one 16-byte load from a byte-aligned
+      // address (global memory takes unaligned vector loads)
+      if (k + 16 <= K) {
+        struct __attribute__((packed, aligned(1))) Chunk { int x, y, z, w; };
+        const Chunk c = *reinterpret_cast<const Chunk *>(r.base + k);
+        return make_int4(c.x, c.y, c.z, c.w);
+      }
       uint32_t w[4] = {0, 0, 0, 0};
       const int n = min(16, K - k);
       for (int b = 0; b < n; b++)
