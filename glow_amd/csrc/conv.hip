@@ -40,15 +40,23 @@ struct ConvRows {
     r.iw0 = ow * strideW - padL;
     return r;
   }
-  // address of the 16 bytes A[m][k..k+15] of an existing row (ICg % 16 == 0):
-  // inside the image, or a chunk of input-offset bytes for a padding tap
-  __device__ __forceinline__ const int8_t *chunk_ptr(const Row &r, int k) const {
+  // the filter tap and channel that the 16 bytes A[m][k..k+15] of any row
+  // come from (ICg % 16 == 0, so a chunk never straddles a tap)
+  struct Loc {
+    int dh, dw, c;
+  };
+  __device__ __forceinline__ Loc locate(int k) const {
     const int tap = k / ICg, c = k - tap * ICg;
     const int fx = tap / KW, fy = tap - fx * KW;
-    const int ih = r.ih0 + fx * dilH, iw = r.iw0 + fy * dilW;
+    return Loc{fx * dilH, fy * dilW, c};
+  }
+  // address of those bytes for an existing row: inside the image, or a chunk
+  // of input-offset bytes for a padding tap
+  __device__ __forceinline__ const int8_t *chunk_ptr(const Row &r, const Loc &l) const {
+    const int ih = r.ih0 + l.dh, iw = r.iw0 + l.dw;
     if (ih < 0 || iw < 0 || ih >= IH || iw >= IW)
       return reinterpret_cast<const int8_t *>(g_fill_table.b) + ((fill & 0xff) << 4);
-    return r.img + ((long long)ih * IW + iw) * IC + c;
+    return r.img + ((long long)ih * IW + iw) * IC + l.c;
   }
   // 16 bytes A[m][k..k+15]; ALIGNED needs ICg % 16 == 0 so a chunk never
   // straddles a tap, and 16-byte aligned pixels.

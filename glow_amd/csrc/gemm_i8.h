@@ -126,9 +126,14 @@ struct DenseRows {
   __device__ __forceinline__ Row row(int r) const {
     return Row{p + (long long)r * ld, r < rows};
   }
-  // address of the 16 bytes [k, k+16) of a row that exists
-  __device__ __forceinline__ const int8_t *chunk_ptr(const Row &r, int k) const {
-    return r.base + k;
+  // where the 16 bytes [k, k+16) sit inside any row
+  struct Loc {
+    int k;
+  };
+  __device__ __forceinline__ Loc locate(int k) const { return Loc{k}; }
+  // address of those bytes in a row that exists
+  __device__ __forceinline__ const int8_t *chunk_ptr(const Row &r, const Loc &l) const {
+    return r.base + l.k;
   }
   template <bool ALIGNED>
   __device__ __forceinline__ int4 load(const Row &r, int k, int K) const {
@@ -491,7 +496,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
   constexpr int A_LOADS = BM / 16 / WAVES, B_LOADS = BN / 16 / WAVES;
   constexpr int LOADS = A_LOADS + B_LOADS;
   static_assert(BM / 16 % WAVES == 0 && BN / 16 % WAVES == 0, "tile vs waves");
-  static_assert(STAGES >= 2 && (STAGES - 1) * LOADS < 64, "ring depth");
+  static_assert(STAGES >= 3 && (STAGES - 1) * LOADS < 64, "ring depth");
 
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
 
@@ -532,18 +537,33 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
   }
 
   const int KT = K / kBK;
-  // prologue: STAGES-1 tiles in flight (tiles past the end are re-reads of
-  // the last one into slots nobody consumes, which keeps the counts uniform)
+  // A tile's loads are issued in two halves, H0 then H1, so that the memory
+  // pipeline sees a steady trickle instead of one burst per K step.
+  constexpr int H0 = LOADS / 2;
+  // `loc` is A.locate() of this lane's chunk of tile nk (one locate serves
+  // every row of the tile and both halves of its loads)
+  auto locate_tile = [&](int nk) { return A.locate(min(nk, KT - 1) * kBK + kc_lane); };
+  auto issue_load = [&](int nk, int i, const typename ARows::Loc &loc) {
+    const uint32_t slot = lds0 + (uint32_t)(nk % STAGES) * STAGE;
+    const int k0 = min(nk, KT - 1) * kBK;
+    if (i < A_LOADS)
+      dma16(A.chunk_ptr(arow[i], loc), slot + a_dst[i]);
+    else
+      dma16(bptr[i - A_LOADS] + k0, slot + b_dst[i - A_LOADS]);
+  };
+  // prologue: tiles 0..STAGES-2 and the first half of tile STAGES-1 in flight
+  // (tiles past the end are re-reads of the last one into slots nobody
+  // consumes, which keeps the counts uniform)
 #pragma unroll
   for (int s = 0; s < STAGES - 1; s++) {
-    const uint32_t slot = lds0 + (uint32_t)s * STAGE;
-    const int k0 = min(s, KT - 1) * kBK;
+    const typename ARows::Loc loc = locate_tile(s);
 #pragma unroll
-    for (int i = 0; i < A_LOADS; i++)
-      dma16(A.chunk_ptr(arow[i], k0 + kc_lane), slot + a_dst[i]);
-#pragma unroll
-    for (int i = 0; i < B_LOADS; i++) dma16(bptr[i] + k0, slot + b_dst[i]);
+    for (int i = 0; i < LOADS; i++) issue_load(s, i, loc);
   }
+  // the tile whose second half is still to be requested
+  typename ARows::Loc half_loc = locate_tile(STAGES - 1);
+#pragma unroll
+  for (int i = 0; i < H0; i++) issue_load(STAGES - 1, i, half_loc);
 
   v16i acc[TM][TN];
 #pragma unroll
@@ -576,14 +596,6 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
     else
       bf[buf][f - TM] = *reinterpret_cast<const v4i *>(stage + b_base + (f - TM) * 32 * kBK + frag_off[ks]);
   };
-  auto issue_load = [&](int nk, int i) {
-    const uint32_t slot = lds0 + (uint32_t)(nk % STAGES) * STAGE;
-    const int k0 = min(nk, KT - 1) * kBK;
-    if (i < A_LOADS)
-      dma16(A.chunk_ptr(arow[i], k0 + kc_lane), slot + a_dst[i]);
-    else
-      dma16(bptr[i - A_LOADS] + k0, slot + b_dst[i - A_LOADS]);
-  };
   // The MFMAs of one k slice with the memory operations of the next slice
   // spread between them: a wave issues in order, so a burst of loads that
   // fills the memory queues would hold back the MFMAs queued behind it.
@@ -615,35 +627,50 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
   };
   constexpr int MFMAS = TM * TN;
   constexpr int FRAGS = TM + TN;
-  // operation x of n is slotted in after MFMA t when x is in
-  // [t*n/MFMAS, (t+1)*n/MFMAS): spread evenly over the slice
+  // Fragment read f is slotted in after MFMA t when f is in
+  // [t*FRAGS/MFMAS, (t+1)*FRAGS/MFMAS): spread evenly, each in the last slot
+  // of its interval. Load x of n goes to the middle of its interval, which are
+  // the slots the reads leave empty when there are fewer operations than
+  // MFMAs (a read and a load behind the same MFMA take longer to issue than
+  // the MFMA runs, which stalls the next one).
+  auto frags_in_slot = [&](int t, const int8_t *stage, int ks, int buf) {
+#pragma unroll
+    for (int f = t * FRAGS / MFMAS; f < (t + 1) * FRAGS / MFMAS; f++)
+      read_frag(stage, ks, buf, f);
+  };
+  auto loads_in_slot = [&](int t, int nk, int first, int n,
+                           const typename ARows::Loc &loc) {
+#pragma unroll
+    for (int x = 0; x < n; x++)
+      if (min(MFMAS - 1, (2 * x + 1) * MFMAS / (2 * n)) == t)
+        issue_load(nk, first + x, loc);
+  };
 
-  dma_wait<(STAGES - 2) * LOADS>(); // tile 0 has landed
+  // tile 0 has landed once only the newer requests are pending
+  dma_wait<(STAGES - 2) * LOADS + H0>();
   __syncthreads();
 #pragma unroll
   for (int f = 0; f < FRAGS; f++) read_frag(lds, 0, 0, f);
   for (int kt = 0; kt < KT; kt++) {
     const int8_t *cur = lds + (kt % STAGES) * STAGE;
     const int8_t *nxt = lds + ((kt + 1) % STAGES) * STAGE;
-    // slice 0 runs while the fragments of slice 1 arrive
+    // slice 0 runs while the fragments of slice 1 arrive and the second half
+    // of tile kt+STAGES-1 is requested (its slot held tile kt-1, which every
+    // wave had read before the previous barrier)
     multiply(0, [&](int t) {
-#pragma unroll
-      for (int f = t * FRAGS / MFMAS; f < (t + 1) * FRAGS / MFMAS; f++)
-        read_frag(cur, 1, 1, f);
+      frags_in_slot(t, cur, 1, 1);
+      loads_in_slot(t, kt + STAGES - 1, H0, LOADS - H0, half_loc);
     });
-    // tile kt+1 has landed once at most STAGES-3 newer tiles are pending; past
-    // the barrier every wave is done reading tile kt-1, whose slot is refilled
-    dma_wait<(STAGES - 3) * LOADS>();
+    // tile kt+1 has landed once only tiles kt+2..kt+STAGES-1 are pending; past
+    // the barrier every wave holds tile kt in registers, so its slot is free
+    dma_wait<(STAGES - 2) * LOADS>();
     __syncthreads();
-    // slice 1 runs while slice 0 of the next tile is read and tile
-    // kt+STAGES-1 is requested
+    // slice 1 runs while slice 0 of the next tile is read and the first half
+    // of tile kt+STAGES is requested into the slot of tile kt
+    half_loc = locate_tile(kt + STAGES);
     multiply(1, [&](int t) {
-#pragma unroll
-      for (int f = t * FRAGS / MFMAS; f < (t + 1) * FRAGS / MFMAS; f++)
-        read_frag(nxt, 0, 0, f);
-#pragma unroll
-      for (int i = t * LOADS / MFMAS; i < (t + 1) * LOADS / MFMAS; i++)
-        issue_load(kt + STAGES - 1, i);
+      frags_in_slot(t, nxt, 0, 0);
+      loads_in_slot(t, kt + STAGES, 0, H0, half_loc);
     });
   }
   dma_wait<0>(); // drain the re-reads before LDS is reused
