@@ -193,7 +193,11 @@ def cpu_baseline_slws(table, batches, budget_s, gpu_out, gpu_batch):
     from oracle import glow_oracle as go
     want = go.frwq_slws_f32(table, gpu_batch["w"], gpu_batch["idx"],
                             gpu_batch["lengths"])
-    parity = bool(np.array_equal(gpu_out, want))
+    # default (fused multiply-add) arithmetic: equal to the sequential CPU loop
+    # to rounding; the bar is 1e-5 of the magnitude a bag adds up
+    from glow_amd import workloads
+    parity = workloads.slws_error_ratio(gpu_out, want, table, gpu_batch["w"],
+                                        gpu_batch["idx"], gpu_batch["lengths"])
     done_bytes, n = 0.0, 0
     t0 = time.perf_counter()
     while True:
@@ -515,18 +519,19 @@ def main():
             "device": info.name.decode() or "MI355X", "arch": info.arch.decode(),
             "compute_units": info.compute_units,
         },
-        "parity_with_oracle": parity,
+        "parity_with_oracle": (None if parity is None else bool(parity <= 1e-5)),
+        "max_error_over_bag_magnitude": parity,
         "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
                      "traffic": (MEASURED_TRAFFIC["slws"]
                                  if (args.rows, args.bags, args.batches) ==
                                  (4_000_000, 4096, 8) else None),
-                     "kernel": "slws_wave_kernel<2,false,false,false,true>"},
+                     "kernel": "slws_rows_kernel<false,false,32,true>"},
         "cpu_baseline": cpu,
         "extra": extra,
     }
     print(json.dumps(out))
-    if parity is False:
+    if parity is not None and not parity <= 1e-5:
         sys.exit(1)
 
 

@@ -24,7 +24,7 @@ EXPORTS = [
     "mi355x_host_free", "mi355x_memcpy_h2d", "mi355x_memcpy_d2h",
     "mi355x_memcpy_d2d", "mi355x_fill_u8", "mi355x_copy_u8", "mi355x_gemm_tile_override",
     "mi355x_cwq_conv2d_add_i8", "mi355x_frwq_sls_multi",
-    "mi355x_specialize_bias_weights_qparams", "mi355x_rwq_slws", "mi355x_add_i8", "mi355x_add_relu_i8",
+    "mi355x_specialize_bias_weights_qparams", "mi355x_rwq_slws", "mi355x_slws_set_fused_math", "mi355x_add_i8", "mi355x_add_relu_i8",
     "mi355x_relu_i8", "mi355x_convert_f16_to_f32", "mi355x_insert_rows",
     "mi355x_batch_transpose_i8", "mi355x_space_to_depth2_i8", "mi355x_gather", "mi355x_batch_matmul_i8", "mi355x_sigmoid_f32",
     "mi355x_max_pool_i8", "mi355x_avg_pool_i8", "mi355x_softmax_f32", "mi355x_stream_create",
@@ -995,6 +995,12 @@ def frwq_sls_multi(tables, kind, indices, lengths, out_kind=SLS_OUT_F32, out_sca
     if q8:
         return out.numpy()
     return [o.numpy() for o in outs]
+
+
+def slws_set_fused_math(on):
+    """Process-wide: fused multiply-add arithmetic in the SparseLengths kernels
+    (default) or the CPU loop's separately rounded operations."""
+    check(lib().mi355x_slws_set_fused_math(C.c_int(bool(on))))
 
 
 def rwq_slws(data, scales, offsets, weights, indices, lengths):

@@ -33,6 +33,7 @@
 
 #include <hip/hip_fp16.h>
 
+#include <atomic>
 #include <mutex>
 
 namespace mi355x {
@@ -153,6 +154,12 @@ __device__ __forceinline__ float accumulate(float acc, float w, float s,
   float d = __fadd_rn(__fmul_rn(s, (float)q), o);
   float t = __fmul_rn(d, w);
   if constexpr (ACC16) {
+    // The product must be rounded to binary32 before it is rounded to
+    // binary16, as on the CPU. Left to itself the compiler merges multiply and
+    // conversion into one mixed-precision operation that rounds once, which
+    // differs in the last place now and then; the empty statement keeps the
+    // binary32 product as a value of its own.
+    asm volatile("" : "+v"(t));
     return f16round(__fadd_rn(acc, f16round(t)));
   } else {
     return __fadd_rn(acc, t);
@@ -405,6 +412,42 @@ __device__ __forceinline__ void wave_lds_sync() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// Span of the bag of one wavefront (4 waves, 4 consecutive bags per block),
+// returned wave-uniform so that it stays in scalar registers. Lengths mode
+// ends with a block barrier. A bag cannot use more lookups than the index list
+// holds, which bounds the callers' loops whatever the lengths say.
+__device__ __forceinline__ void wave_bag_span(const SlwsArgs &a, int tid, int wave,
+                                              long long bag, long long first_bag,
+                                              long long *s_part, int *s_own,
+                                              long long &start, int &len) {
+  constexpr int kGroups = 4;
+  if (a.offsets) {
+    long long start_v;
+    int len_v;
+    bag_span_offsets(a, bag, start_v, len_v);
+    len = __builtin_amdgcn_readfirstlane(len_v);
+    start = ((long long)__builtin_amdgcn_readfirstlane((int)(start_v >> 32)) << 32) |
+            (unsigned int)__builtin_amdgcn_readfirstlane((int)start_v);
+  } else {
+    block_prefix<kGroups>(a, tid, first_bag, s_part, s_own);
+    const long long block_start = s_part[0] + s_part[1] + s_part[2] + s_part[3];
+    const int4 own = *reinterpret_cast<const int4 *>(s_own);
+    const int w = __builtin_amdgcn_readfirstlane(wave);
+    const int o0 = __builtin_amdgcn_readfirstlane(own.x);
+    const int o1 = __builtin_amdgcn_readfirstlane(own.y);
+    const int o2 = __builtin_amdgcn_readfirstlane(own.z);
+    const int o3 = __builtin_amdgcn_readfirstlane(own.w);
+    const long long bs =
+        ((long long)__builtin_amdgcn_readfirstlane((int)(block_start >> 32)) << 32) |
+        (unsigned int)__builtin_amdgcn_readfirstlane((int)block_start);
+    start = bs + (w > 0 ? o0 : 0) + (w > 1 ? o1 : 0) + (w > 2 ? o2 : 0);
+    len = w == 0 ? o0 : (w == 1 ? o1 : (w == 2 ? o2 : o3));
+    if (bag >= a.segments) len = 0;
+  }
+  const long long room = a.num_indices - start;
+  len = room <= 0 ? 0 : (int)min((long long)len, room);
+}
+
 // One bag per wavefront. OFF32: every row's byte offset fits 32 bits, so row
 // addresses are formed as a uniform base plus a 32-bit per-lane offset.
 template <int BPL, bool IS4, bool SO16, bool ACC16, bool OFF32>
@@ -425,39 +468,9 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_wave_kernel(SlwsArgs a) {
   const long long first_bag = (long long)blockIdx.x * kGroups;
   const long long bag = first_bag + wave;
 
-  // start and len are wave-uniform: keep them in scalar registers
   long long start;
   int len;
-  if (a.offsets) {
-    long long start_v;
-    int len_v;
-    bag_span_offsets(a, bag, start_v, len_v);
-    len = __builtin_amdgcn_readfirstlane(len_v);
-    start = ((long long)__builtin_amdgcn_readfirstlane((int)(start_v >> 32)) << 32) |
-            (unsigned int)__builtin_amdgcn_readfirstlane((int)start_v);
-  } else {
-    static_assert(kGroups == 4, "the own-length selects below assume 4 waves");
-    block_prefix<kGroups>(a, tid, first_bag, s_part, s_own);
-    const long long block_start = s_part[0] + s_part[1] + s_part[2] + s_part[3];
-    const int4 own = *reinterpret_cast<const int4 *>(s_own);
-    const int w = __builtin_amdgcn_readfirstlane(wave);
-    const int o0 = __builtin_amdgcn_readfirstlane(own.x);
-    const int o1 = __builtin_amdgcn_readfirstlane(own.y);
-    const int o2 = __builtin_amdgcn_readfirstlane(own.z);
-    const int o3 = __builtin_amdgcn_readfirstlane(own.w);
-    const long long bs =
-        ((long long)__builtin_amdgcn_readfirstlane((int)(block_start >> 32)) << 32) |
-        (unsigned int)__builtin_amdgcn_readfirstlane((int)block_start);
-    start = bs + (w > 0 ? o0 : 0) + (w > 1 ? o1 : 0) + (w > 2 ? o2 : 0);
-    len = w == 0 ? o0 : (w == 1 ? o1 : (w == 2 ? o2 : o3));
-    if (bag >= a.segments) len = 0;
-  }
-  // a bag cannot use more lookups than the index list holds: bounds the loop
-  // below whatever the lengths say
-  {
-    const long long room = a.num_indices - start;
-    len = room <= 0 ? 0 : (int)min((long long)len, room);
-  }
+  wave_bag_span(a, tid, wave, bag, first_bag, s_part, s_own, start, len);
   int4 *look = s_look[wave];
 
   const int n_passes = (a.data_bytes + 64 * BPL - 1) / (64 * BPL);
@@ -592,6 +605,156 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_wave_kernel(SlwsArgs a) {
   }
 }
 
+
+// ---- fused-arithmetic variant ----------------------------------------------------
+//
+// Same operator with the arithmetic regrouped for the vector ALU:
+//   dest[k] = sum_j (w_j*s_j) * q_jk  +  sum_j (w_j*o_j)
+// one fused multiply-add per element plus one add per lookup, instead of the
+// CPU loop's multiply, add, multiply, add. The result differs from the
+// sequential loop by rounding only (a few units in the last place of the
+// largest partial sum); callers that need the CPU loop's bits switch this
+// variant off with mi355x_slws_set_fused_math(0).
+//
+// One bag per wavefront; a lane reads 4 consecutive data bytes, so a row takes
+// LPR = data_bytes/4 lanes and one load instruction fetches 64/LPR rows. The
+// partial sums of the row groups are added across lanes at the end of the bag.
+typedef uint32_t __attribute__((address_space(1))) global_u32;
+
+template <bool IS4, bool SO16, int LPR, bool OFF32>
+__global__ __launch_bounds__(kSlwsThreads) void slws_rows_kernel(SlwsArgs a) {
+  select_table(a);
+  constexpr int kGroups = kSlwsThreads / 64;
+  constexpr int RPI = 64 / LPR;           // rows per load instruction
+  constexpr int kCols = IS4 ? 8 : 4;      // output columns per lane
+  constexpr int kLoads = kBatch / RPI;    // load instructions of a full batch
+  constexpr int kChunk = kLoads < 4 ? kLoads : 4; // loads under one uniform branch
+  __shared__ long long s_part[kGroups];
+  __shared__ __attribute__((aligned(16))) int s_own[kGroups];
+  // per wave, per lookup of the batch: row byte offset (or row), {w*s, w*o}
+  __shared__ uint32_t s_key[kGroups][kBatch];
+  __shared__ float2 s_ws[kGroups][kBatch];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const long long first_bag = (long long)blockIdx.x * kGroups;
+  const long long bag = first_bag + wave;
+
+  long long start;
+  int len;
+  wave_bag_span(a, tid, wave, bag, first_bag, s_part, s_own, start, len);
+  uint32_t *keys = s_key[wave];
+  float2 *wso = s_ws[wave];
+
+  const int sub = lane / LPR;             // which row of a load this lane reads
+  const int lir = lane % LPR;
+  const uint32_t lane_off = (uint32_t)lir * 4u;
+  float acc[kCols];
+  float acc_o = 0.0f;
+#pragma unroll
+  for (int c = 0; c < kCols; c++) acc[c] = 0.0f;
+
+  for (int base = 0; base < len; base += kBatch) {
+    const int cnt = min(kBatch, len - base);
+    // round 1: lane j fetches lookup j of the batch
+    {
+      const long long pos = start + base + lane;
+      long long row = -1;
+      float w = 0.0f;
+      if (lane < cnt && pos < a.num_indices) {
+        row = a.idx64 ? reinterpret_cast<const long long *>(a.indices)[pos]
+                      : (long long)reinterpret_cast<const int *>(a.indices)[pos];
+        if (!a.weights) {
+          w = 1.0f;
+        } else if (a.w16) {
+          w = __half2float(reinterpret_cast<const __half *>(a.weights)[pos]);
+        } else {
+          w = reinterpret_cast<const float *>(a.weights)[pos];
+        }
+      }
+      // a skipped lookup reads row 0 and contributes exactly +0
+      const bool valid = row >= 0 && row < a.data_rows;
+      if (!valid) row = 0;
+      float s, o;
+      if (!SO16 && a.sep_scales) {
+        s = a.sep_scales[row];
+        o = a.sep_offsets[row];
+      } else {
+        // rows and their data bytes are multiples of 4 bytes here
+        const uint32_t *so = reinterpret_cast<const uint32_t *>(
+            a.data + row * a.in_line + a.data_bytes);
+        if constexpr (SO16) {
+          const uint32_t v = so[0];
+          s = __half2float(__ushort_as_half((unsigned short)(v & 0xffff)));
+          o = __half2float(__ushort_as_half((unsigned short)(v >> 16)));
+        } else {
+          s = __uint_as_float(so[0]);
+          o = __uint_as_float(so[1]);
+        }
+      }
+      keys[lane] = OFF32 ? (uint32_t)(row * a.in_line) : (uint32_t)row;
+      wso[lane] = valid ? make_float2(w * s, w * o) : make_float2(0.0f, 0.0f);
+    }
+    wave_lds_sync();
+    // round 2: all row reads of the batch in flight before the first use, taken
+    // kChunk load instructions at a time under one uniform branch. Slots
+    // beyond cnt hold {row 0, 0, 0} and add exactly +0.
+    uint32_t q[kLoads];
+#pragma unroll
+    for (int c = 0; c < kLoads / kChunk; c++) {
+      if (c * kChunk * RPI < cnt) {
+#pragma unroll
+        for (int u = 0; u < kChunk; u++) {
+          const int g = c * kChunk + u;
+          const uint32_t key = keys[g * RPI + sub];
+          if constexpr (OFF32) {
+            q[g] = *(const global_u32 *)((const global_u8 *)a.data + (key + lane_off));
+          } else {
+            q[g] = *reinterpret_cast<const uint32_t *>(
+                a.data + (long long)key * a.in_line + lane_off);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < kLoads / kChunk; c++) {
+      if (c * kChunk * RPI < cnt) {
+#pragma unroll
+        for (int u = 0; u < kChunk; u++) {
+          const int g = c * kChunk + u;
+          const float2 f = wso[g * RPI + sub];
+          acc_o += f.y;
+          if constexpr (IS4) {
+            const uint32_t lo = q[g] & 0x0f0f0f0fu, hi = (q[g] >> 4) & 0x0f0f0f0fu;
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+              acc[2 * b] = __fmaf_rn(f.x, (float)((lo >> (8 * b)) & 0xff), acc[2 * b]);
+              acc[2 * b + 1] =
+                  __fmaf_rn(f.x, (float)((hi >> (8 * b)) & 0xff), acc[2 * b + 1]);
+            }
+          } else {
+#pragma unroll
+            for (int b = 0; b < 4; b++)
+              acc[b] = __fmaf_rn(f.x, (float)((q[g] >> (8 * b)) & 0xff), acc[b]);
+          }
+        }
+      }
+    }
+    wave_lds_sync(); // slots are rewritten by the next batch
+  }
+
+  // partial sums of the RPI row groups -> lanes of group 0
+#pragma unroll
+  for (int c = 0; c < kCols; c++) {
+    float v = acc[c] + acc_o;
+#pragma unroll
+    for (int off = LPR; off < 64; off <<= 1) v += __shfl_xor(v, off, 64);
+    acc[c] = v;
+  }
+  if (bag < a.segments && sub == 0) store_columns<kCols>(a, bag, lir * kCols, acc);
+}
+
 // Sum of the clamped lengths of each chunk of kChunkBags bags.
 __global__ __launch_bounds__(256) void slws_chunk_sums_kernel(
     const int32_t *lengths, long long segments, int64_t *chunk_sums) {
@@ -676,6 +839,31 @@ static void launch_wave_kind(int kind, bool acc16, dim3 grid, hipStream_t st,
   }
 #undef MI355X_SLWS_WAVE
 }
+
+template <int LPR, bool OFF32>
+static void launch_rows_kind(int kind, dim3 grid, hipStream_t st, const SlwsArgs &a) {
+#define MI355X_SLWS_ROWS(IS4, SO16)                                            \
+  hipLaunchKernelGGL((slws_rows_kernel<IS4, SO16, LPR, OFF32>), grid,          \
+                     dim3(kSlwsThreads), 0, st, a)
+  switch (kind) {
+  case MI355X_FUSED_U8_F32:
+    MI355X_SLWS_ROWS(false, false);
+    break;
+  case MI355X_FUSED_U8_F16:
+    MI355X_SLWS_ROWS(false, true);
+    break;
+  case MI355X_FUSED_U4_F16:
+    MI355X_SLWS_ROWS(true, true);
+    break;
+  default:
+    MI355X_SLWS_ROWS(true, false);
+    break;
+  }
+#undef MI355X_SLWS_ROWS
+}
+
+// Whether the fused-arithmetic kernels may be used (process-wide).
+static std::atomic<int> g_fused_math{1};
 
 // Several tables in one launch and/or the int8 output transform.
 struct SlwsExtra {
@@ -773,6 +961,31 @@ static int slws_dispatch(void *dest, int out_is_f16, const uint8_t *data,
   MI355X_REQUIRE(blocks < 0x7fffffffu, "too many bags");
   dim3 grid((unsigned)blocks, (unsigned)x.n_tables);
   const bool off32 = (unsigned long long)data_rows * in_line_size <= 0xffffffffull;
+  // fused arithmetic: whole rows of 32, 64, 128 or 256 data bytes, 4-byte
+  // aligned, fp32 accumulation. A multi-table launch cannot check the
+  // alignment of each table here; its tables must be 4-byte aligned.
+  const bool rows_ok = g_fused_math.load(std::memory_order_relaxed) && !acc16 &&
+                       in_line_size % 4 == 0 && (((uintptr_t)data) % 4 == 0) &&
+                       (data_bytes == 32 || data_bytes == 64 ||
+                        data_bytes == 128 || data_bytes == 256);
+  if (rows_ok) {
+    const size_t rblocks = (out_rows + 3) / 4;
+    MI355X_REQUIRE(rblocks < 0x7fffffffu, "too many bags");
+    dim3 rgrid((unsigned)rblocks, (unsigned)x.n_tables);
+#define MI355X_ROWS_CASE(BYTES)                                                \
+  case BYTES:                                                                  \
+    if (off32) launch_rows_kind<BYTES / 4, true>(kind, rgrid, st, a);          \
+    else launch_rows_kind<BYTES / 4, false>(kind, rgrid, st, a);               \
+    break;
+    switch (data_bytes) {
+      MI355X_ROWS_CASE(32)
+      MI355X_ROWS_CASE(64)
+      MI355X_ROWS_CASE(128)
+      MI355X_ROWS_CASE(256)
+    }
+#undef MI355X_ROWS_CASE
+    return check_launch("frwq_slws");
+  }
   if (lpb == 16) launch_kind<16, 2>(kind, acc16, grid, st, a);
   else if (lpb == 32) launch_kind<32, 2>(kind, acc16, grid, st, a);
   else if (!even && off32) launch_wave_kind<1, true>(kind, acc16, grid, st, a);
@@ -787,6 +1000,11 @@ static int slws_dispatch(void *dest, int out_is_f16, const uint8_t *data,
 using namespace mi355x;
 
 extern "C" {
+
+int mi355x_slws_set_fused_math(int on) {
+  g_fused_math.store(on ? 1 : 0, std::memory_order_relaxed);
+  return MI355X_OK;
+}
 
 int mi355x_frwq_sls_multi(const mi355x_sls_table *tables, size_t n_tables,
                           size_t max_data_rows, int kind, int idx_is_64,

@@ -221,3 +221,23 @@ def slws_batch(seed, rows, bags, mean_len, alpha, idx_dtype=np.int64,
     idx = zipf_indices(rng, total, rows, alpha).astype(idx_dtype)
     w = rng.random(total).astype(np.float32) if weighted else None
     return lengths, idx, w
+
+
+def slws_error_ratio(got, want, table, w, idx, lengths):
+    """max |got - want| / B over the output of a uint8/fp32 fused-rowwise SLWS,
+    where B = sum_j |w_j| (|scale_j| 255 + |offset_j|) per bag is the magnitude
+    of what the bag adds up (the result itself may cancel to nearly zero).
+    Empty bags must be exact zeros (returns inf otherwise)."""
+    total = int(lengths.sum())
+    so = np.ascontiguousarray(table[:, -8:]).view(np.float32).astype(np.float64)
+    r = np.asarray(idx[:total])
+    ww = np.ones(total) if w is None else np.abs(np.asarray(w[:total], np.float64))
+    m = ww * (np.abs(so[r, 0]) * 255.0 + np.abs(so[r, 1]))
+    c = np.r_[0.0, np.cumsum(m)]
+    ends = np.cumsum(lengths)
+    mag = c[ends] - c[ends - lengths]
+    err = np.abs(np.asarray(got, np.float64) - np.asarray(want, np.float64)).max(axis=1)
+    if np.any(err[mag == 0] != 0):
+        return float("inf")
+    live = mag > 0
+    return float(np.max(err[live] / mag[live])) if live.any() else 0.0

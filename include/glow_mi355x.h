@@ -441,6 +441,18 @@ int mi355x_frwq_slws(void *dest, int out_is_f16, const uint8_t *data,
                      size_t segments, size_t in_line_size,
                      size_t out_line_size, int fp16_accum, void *stream);
 
+/* Arithmetic of the SparseLengths kernels (process-wide; default on).
+ * On: rows of 32, 64, 128 or 256 data bytes with fp32 accumulation are summed
+ * as sum_j (w_j*s_j)*q_jk + sum_j (w_j*o_j) with fused multiply-adds. The CPU
+ * loop's w*(s*q+o) summed in bag order is reproduced to rounding (relative
+ * error of the order of 1e-7 of sum_j |w_j|(|s_j| q + |o_j|)), which is the
+ * latitude the reference's own build takes (libjit is compiled with
+ * -ffast-math, reference CMakeLists.txt:21, 170-174).
+ * Off: every multiply and add is rounded separately in bag order, which
+ * reproduces a strict (no fast-math) build of the CPU loop bit for bit.
+ * No counterpart in the reference. */
+int mi355x_slws_set_fused_math(int on);
+
 /* libjit_rowwise_quantized_sparse_lengths_weighted_sum_f_u / _f_i32 (reference
  * libjit.cpp:1232-1251, 2400-2414): the table holds uint8 rows of line_size
  * bytes, the fp32 scale and offset of row r are scales[r] and offsets[r].

@@ -46,3 +46,4 @@ cwq_conv_args = _w.cwq_conv_args
 zipf_indices = _w.zipf_indices
 random_fused_table = _w.random_fused_table
 slws_batch = _w.slws_batch
+slws_error_ratio = _w.slws_error_ratio

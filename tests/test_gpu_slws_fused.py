@@ -1,0 +1,217 @@
+"""The SparseLengths kernels with their default (fused multiply-add)
+arithmetic, against the CPU oracle's sequential loop. The regrouped sum
+  sum_j (w_j s_j) q_jk + sum_j (w_j o_j)
+differs from the loop's w_j (s_j q_jk + o_j) by rounding only, so the bar is
+the stated one for floating point: 1e-5 relative. "Relative" is taken against
+B = sum_j |w_j| (|s_j| q_max + |o_j|), the magnitude of what a bag adds up (the
+result itself can cancel to nearly zero); the error seen is below 1e-6 B.
+fp16 outputs get one extra fp16 unit in the last place for the final rounding.
+Everything else about the operator (skipped lookups, empty bags, index types,
+every output row written) is checked as in the bit-exact tests.
+"""
+import numpy as np
+import pytest
+
+from glow_amd import capi
+from oracle import glow_oracle as go
+from tests import cases
+
+pytestmark = [pytest.mark.gpu, pytest.mark.fused_math]
+
+RTOL = 1e-5
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _device():
+    capi.init(0)
+    yield
+    capi.sync()
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def row_scale_offset(table, kind):
+    """fp32 (scale, offset) of every fused row."""
+    if kind in (capi.FUSED_U8_F32, capi.FUSED_U4_F32):
+        so = np.ascontiguousarray(table[:, -8:]).view(np.float32)
+    else:
+        so = np.ascontiguousarray(table[:, -4:]).view(np.float16).astype(np.float32)
+    return so[:, 0], so[:, 1]
+
+
+def bag_magnitude(table, kind, w, idx, lengths, scales=None, offsets=None):
+    """B per bag, float64."""
+    s, o = (scales, offsets) if scales is not None else row_scale_offset(table, kind)
+    qmax = 255.0 if kind in (capi.FUSED_U8_F32, capi.FUSED_U8_F16) else 15.0
+    total = int(lengths.sum())
+    idx = np.asarray(idx[:total])
+    ok = (idx >= 0) & (idx < table.shape[0])
+    r = np.where(ok, idx, 0)
+    ww = np.ones(total) if w is None else np.abs(np.asarray(w[:total], np.float64))
+    m = np.where(ok, ww * (np.abs(s[r].astype(np.float64)) * qmax +
+                            np.abs(o[r].astype(np.float64))), 0.0)
+    ends = np.cumsum(lengths)
+    c = np.r_[0.0, np.cumsum(m)]
+    return c[ends] - c[ends - lengths]
+
+
+def check(got, want, mag, out16=False, what=""):
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    tol = RTOL * mag[:, None]
+    if out16:
+        tol = tol + np.abs(want) * 2.0 ** -10
+    err = np.abs(got - want)
+    worst = float(np.max(err / np.maximum(mag[:, None], 1e-30))) if err.size else 0.0
+    say(f"  {what} max error / B = {worst:.2e}")
+    assert np.all(err <= tol), (what, worst)
+    # empty bags are exact zeros
+    empty = mag == 0
+    assert np.all(got[empty] == 0)
+
+
+# data bytes 32/64/128/256 take the fused kernels; the others in the list stay
+# on the separately rounded ones and must agree exactly
+SHAPES = [
+    # rows, cols, bags, mean length
+    (1000, 128, 64, 40), (500, 64, 33, 20), (200, 256, 9, 7), (4000, 128, 4096, 40),
+    (999, 32, 100, 90), (700, 128, 50, 150), (300, 37, 10, 12), (64, 16, 5, 200),
+]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("idt", [np.int64, np.int32])
+def test_slws_u8_f32(shape, idt):
+    rows, cols, bags, mean = shape
+    say("fused slws u8/f32", shape, idt.__name__)
+    rng = np.random.default_rng(rows + cols)
+    table = cases.random_fused_table(rng, rows, cols)
+    lengths, idx, w = cases.slws_batch(bags, rows, bags, mean, 1.05, idt)
+    lengths[bags // 2] = 0
+    total = int(lengths.sum())
+    idx, w = idx[:total], w[:total]
+    mag = bag_magnitude(table, capi.FUSED_U8_F32, w, idx, lengths)
+    check(capi.frwq_slws(table, capi.FUSED_U8_F32, w, idx, lengths),
+          go.frwq_slws_f32(table, w, idx, lengths), mag, what="weighted")
+    mag1 = bag_magnitude(table, capi.FUSED_U8_F32, None, idx, lengths)
+    check(capi.frwq_slws(table, capi.FUSED_U8_F32, None, idx, lengths),
+          go.frwq_slws_f32(table, np.ones(total, np.float32), idx, lengths), mag1,
+          what="sum")
+    if cols not in (32, 64, 128, 256):
+        np.testing.assert_array_equal(
+            capi.frwq_slws(table, capi.FUSED_U8_F32, w, idx, lengths),
+            go.frwq_slws_f32(table, w, idx, lengths))
+
+
+@pytest.mark.parametrize("kind", [capi.FUSED_U8_F16, capi.FUSED_U4_F16, capi.FUSED_U4_F32])
+@pytest.mark.parametrize("cols", [64, 128, 256, 512, 16])
+def test_slws_other_kinds(kind, cols):
+    say("fused slws kind", kind, "cols", cols)
+    rng = np.random.default_rng(kind * 100 + cols)
+    rows, bags = 700, 150
+    table = cases.random_fused_table(rng, rows, cols, kind)
+    lengths, idx, w = cases.slws_batch(cols, rows, bags, 20, 1.1, np.int64)
+    lengths[7] = 0
+    total = int(lengths.sum())
+    idx, w = idx[:total], w[:total]
+    f16 = kind in (capi.FUSED_U8_F16, capi.FUSED_U4_F16)
+    combos = [(w, False, False), (None, False, False)]
+    if f16:
+        combos += [(w.astype(np.float16), True, False), (None, True, False),
+                   (w.astype(np.float16), True, True)]
+    for weights, out16, acc16 in combos:
+        want = go.frwq_slws_generic(table, kind, weights, idx, lengths, out16, acc16)
+        got = capi.frwq_slws(table, kind, weights, idx, lengths, out16, acc16)
+        if acc16:
+            # fp16 accumulation keeps the separately rounded kernels
+            np.testing.assert_array_equal(got.view(np.uint16), want.view(np.uint16))
+            continue
+        mag = bag_magnitude(table, kind, weights, idx, lengths)
+        check(got.astype(np.float32), want.astype(np.float32), mag, out16,
+              what=f"w={'none' if weights is None else weights.dtype} out16={out16}")
+
+
+def test_invalid_lookups_are_skipped_and_rows_rezeroed():
+    rows, cols = 50, 128
+    rng = np.random.default_rng(12)
+    table = cases.random_fused_table(rng, rows, cols)
+    lengths = np.array([3, 2, 4], np.int32)
+    idx = np.array([1, 99, 3, -1, 4, 5, 6, 7, 8], np.int64)  # 99 and -1 are out of range
+    w = rng.random(9).astype(np.float32)
+    keep = np.array([1, 0, 1, 0, 1, 1, 1, 1, 1], bool)
+    want = go.frwq_slws_f32(table, np.where(keep, w, 0).astype(np.float32),
+                            np.where(keep, idx, 0), lengths)
+    mag = bag_magnitude(table, 0, w, idx, lengths)
+    check(capi.frwq_slws(table, 0, w, idx, lengths), want, mag, what="skips")
+    # lengths that run past the index list: the missing lookups are skipped
+    got = capi.frwq_slws(table, 0, w[:7], idx[:7].clip(0, 49), lengths)
+    want = go.frwq_slws_f32(table, np.r_[w[:7], [0, 0]].astype(np.float32),
+                            np.r_[idx[:7].clip(0, 49), [0, 0]], lengths)
+    check(got, want, bag_magnitude(table, 0, np.r_[w[:7], [0, 0]],
+                                   np.r_[idx[:7].clip(0, 49), [0, 0]], lengths),
+          what="short list")
+    # a second call with emptied bags rewrites their rows with zeros
+    l2 = np.array([3, 0, 4], np.int32)
+    i2 = np.r_[idx[:3].clip(0, 49), idx[5:9]]
+    w2 = np.r_[w[:3], w[5:9]].astype(np.float32)
+    got = capi.frwq_slws(table, 0, w2, i2, l2)
+    assert np.all(got[1] == 0)
+
+
+def test_embedding_bag_offsets_mode():
+    rows, cols, bags = 400, 128, 60
+    rng = np.random.default_rng(21)
+    for kind in (capi.FUSED_U8_F32, capi.FUSED_U4_F16):
+        table = cases.random_fused_table(rng, rows, cols, kind)
+        lengths, idx, w = cases.slws_batch(5, rows, bags, 9, 1.05, np.int32)
+        total = int(lengths.sum())
+        offs = np.r_[0, np.cumsum(lengths)].astype(np.int32)
+        f16 = kind == capi.FUSED_U4_F16
+        ww = w[:total].astype(np.float16) if f16 else w[:total]
+        got = capi.embedding_bag_rowwise_offsets(table, kind, ww, idx[:total], offs,
+                                                 True, f16, False)
+        want = go.frwq_slws_generic(table, kind, ww, idx[:total], lengths, f16, False)
+        check(got.astype(np.float32), want.astype(np.float32),
+              bag_magnitude(table, kind, ww, idx, lengths), f16, what=f"kind {kind}")
+
+
+def test_rowwise_tables_with_separate_scales():
+    rows, cols, bags = 300, 64, 40
+    rng = np.random.default_rng(33)
+    data = rng.integers(0, 256, (rows, cols), dtype=np.uint8)
+    scales = rng.uniform(0.01, 0.03, rows).astype(np.float32)
+    offsets = rng.normal(-3, 0.5, rows).astype(np.float32)
+    lengths, idx, w = cases.slws_batch(6, rows, bags, 11, 1.05, np.int64)
+    total = int(lengths.sum())
+    got = capi.rwq_slws(data, scales, offsets, w[:total], idx[:total], lengths)
+    want = go.rwq_slws_f32(data, scales, offsets, w[:total], idx[:total], lengths)
+    check(got, want, bag_magnitude(data, 0, w, idx, lengths, scales, offsets),
+          what="rowwise")
+
+
+def test_many_bags_and_full_size_config():
+    """More than one chunk of bags, and the benchmark configuration at full
+    size (4M x 128 table, 4096 bags Poisson(40), Zipf(1.05) int64 indices)."""
+    rng = np.random.default_rng(8)
+    table = cases.random_fused_table(rng, 5000, 64)
+    lengths, idx, w = cases.slws_batch(9, 5000, 20000, 6, 1.05, np.int64)
+    check(capi.frwq_slws(table, 0, w, idx, lengths),
+          go.frwq_slws_f32(table, w, idx, lengths),
+          bag_magnitude(table, 0, w, idx, lengths), what="20000 bags")
+    rows, cols, bags = 4_000_000, 128, 4096
+    rng = np.random.default_rng(2026)
+    table = cases.random_fused_table(rng, rows, cols)
+    lengths, idx, w = cases.slws_batch(2027, rows, bags, 40, 1.05, np.int64)
+    got = capi.frwq_slws(table, 0, w, idx, lengths)
+    want = go.frwq_slws_f32(table, w, idx, lengths)
+    check(got, want, bag_magnitude(table, 0, w, idx, lengths), what="full size")
+    # the strict arithmetic on the same inputs is bit-exact, and the two agree
+    capi.slws_set_fused_math(False)
+    try:
+        strict = capi.frwq_slws(table, 0, w, idx, lengths)
+    finally:
+        capi.slws_set_fused_math(True)
+    np.testing.assert_array_equal(strict, want)
+    np.testing.assert_allclose(got, strict, rtol=1e-5, atol=1e-4)
