@@ -149,6 +149,15 @@ static int conv_common(int8_t *out, const int8_t *in, const int8_t *filter,
                     ((((uintptr_t)in) & 15) == 0);
   const bool al_b = (K % 16 == 0) && ((((uintptr_t)filter) & 15) == 0);
   const bool need_sb = ep.a_off != 0 && !ep.sum_b;
+  // A pointwise convolution over the whole image is a plain matrix product:
+  // row m of A is pixel m of the input, no taps to locate and no padding.
+  if (g->KH == 1 && g->KW == 1 && g->strideH == 1 && g->strideW == 1 &&
+      g->padT == 0 && g->padL == 0 && g->group == 1 && g->OH == g->IH &&
+      g->OW == g->IW) {
+    DenseRows Ad{in, g->IC, (int)M};
+    return gemm_dispatch(Ad, B, ep, (int)M, OCg, (int)K, 1, 0, need_sa, need_sb,
+                         al_a && al_b, as_stream(stream));
+  }
   return gemm_dispatch(A, B, ep, (int)M, OCg, (int)K, g->group,
                        (long long)OCg * K, need_sa, need_sb, al_a && al_b,
                        as_stream(stream));
