@@ -221,6 +221,7 @@ __device__ __forceinline__ void gemm_epilogue_impl(
   if (ep.act == 2) {
     lo = clip_i8(ep.a0);
     hi = clip_i8(ep.a1);
+    if (lo > hi) lo = hi; // min(max(y, lo), hi) is hi then; so is the median
   }
 
 #pragma unroll
@@ -258,8 +259,7 @@ __device__ __forceinline__ void gemm_epilogue_impl(
             y = scale_i32((int32_t)((uint32_t)y - (uint32_t)ep.out_off), ep.a0,
                           ep.a1, ep.a2, ep.out_off);
         }
-        s_out[ml * OUT_STRIDE + wn * WN + j * 32 + l32] =
-            (int8_t)min(max(y, lo), hi);
+        s_out[ml * OUT_STRIDE + wn * WN + j * 32 + l32] = (int8_t)med3_i32(y, lo, hi);
       }
     }
   }

@@ -42,6 +42,14 @@ __device__ __forceinline__ int32_t clip_i8(int32_t v) {
   return min(max(v, -128), 127);
 }
 
+// min(max(v, lo), hi) for lo <= hi as one instruction (the compiler cannot
+// merge the pair itself without knowing lo <= hi).
+__device__ __forceinline__ int32_t med3_i32(int32_t v, int32_t lo, int32_t hi) {
+  int32_t r;
+  asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "v"(lo), "v"(hi));
+  return r;
+}
+
 // libjit_activation_i32; act follows glow::FusedActivation.
 __device__ __forceinline__ int32_t activation_i32(int32_t v, int32_t offset,
                                                   int32_t act, int32_t a0,
