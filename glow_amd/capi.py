@@ -24,7 +24,7 @@ EXPORTS = [
     "mi355x_host_free", "mi355x_memcpy_h2d", "mi355x_memcpy_d2h",
     "mi355x_memcpy_d2d", "mi355x_fill_u8", "mi355x_copy_u8", "mi355x_gemm_tile_override",
     "mi355x_cwq_conv2d_add_i8", "mi355x_frwq_sls_multi",
-    "mi355x_specialize_bias_weights_qparams", "mi355x_rwq_slws", "mi355x_slws_set_fused_math", "mi355x_add_i8", "mi355x_add_relu_i8",
+    "mi355x_specialize_bias_weights_qparams", "mi355x_rwq_slws", "mi355x_slws_set_fused_math", "mi355x_batch_matmul_nt_i8", "mi355x_add_i8", "mi355x_add_relu_i8",
     "mi355x_relu_i8", "mi355x_convert_f16_to_f32", "mi355x_insert_rows",
     "mi355x_batch_transpose_i8", "mi355x_space_to_depth2_i8", "mi355x_gather", "mi355x_batch_matmul_i8", "mi355x_sigmoid_f32",
     "mi355x_max_pool_i8", "mi355x_avg_pool_i8", "mi355x_softmax_f32", "mi355x_stream_create",
@@ -923,6 +923,20 @@ def batch_matmul_i8(lhs, rhs, out_offset, lhs_offset, rhs_offset, outP):
     check(lib().mi355x_batch_matmul_i8(_vp(out), _vp(dl), _vp(dr), _sz(b), _sz(m), _sz(k),
                                        _sz(n), _i32(out_offset), _i32(lhs_offset),
                                        _i32(rhs_offset), *_i32s(outP), _vp(None)))
+    return out.numpy()
+
+
+def batch_matmul_nt_i8(lhs, rhs_nk, out_offset, lhs_offset, rhs_offset, outP):
+    """lhs [B, M, K] x transpose of rhs_nk [B, N, K]."""
+    lhs = np.ascontiguousarray(lhs, np.int8)
+    rhs_nk = np.ascontiguousarray(rhs_nk, np.int8)
+    b, m, k = lhs.shape
+    n = rhs_nk.shape[1]
+    dl, dr = to_device(lhs), to_device(rhs_nk)
+    out = DeviceBuffer.empty((b, m, n), np.int8)
+    check(lib().mi355x_batch_matmul_nt_i8(_vp(out), _vp(dl), _vp(dr), _sz(b), _sz(m), _sz(k),
+                                          _sz(n), _i32(out_offset), _i32(lhs_offset),
+                                          _i32(rhs_offset), *_i32s(outP), _vp(None)))
     return out.numpy()
 
 

@@ -339,6 +339,63 @@ __global__ __launch_bounds__(kGlueThreads) void batch_matmul_i8_kernel(
   }
 }
 
+// out[b] = clip(scale(sum_k (L[m][k]-lo)(R[n][k]-ro); outP) + oo) for a batch of
+// small matrix pairs with BOTH operands K-contiguous (L [M x K], R [N x K]):
+// libjit_matmul_i8 of L and the transpose of R. One wavefront per sample; each
+// 32 x 32 block of the result is K/32 matrix-core instructions on raw bytes,
+// the offsets enter through the row sums as in the large contraction kernel.
+typedef int nt_v4i __attribute__((ext_vector_type(4)));
+typedef int nt_v16i __attribute__((ext_vector_type(16)));
+
+__global__ __launch_bounds__(kGlueThreads) void batch_matmul_nt_i8_kernel(
+    int8_t *__restrict__ out, const int8_t *__restrict__ lhs, const int8_t *__restrict__ rhs,
+    long long batch, int M, int K, int N, int32_t oo, int32_t lo, int32_t ro, int32_t pre,
+    int32_t post, int32_t scale) {
+  const int lane = threadIdx.x & 63;
+  const long long b = (long long)blockIdx.x * (kGlueThreads / 64) + (threadIdx.x >> 6);
+  if (b >= batch) return;
+  const int l32 = lane & 31, lhi = lane >> 5;
+  const int8_t *L = lhs + b * (long long)M * K, *R = rhs + b * (long long)N * K;
+  int8_t *O = out + b * (long long)M * N;
+  const uint32_t kconst = (uint32_t)K * (uint32_t)lo * (uint32_t)ro;
+  for (int tm = 0; tm < M; tm += 32) {
+    for (int tn = 0; tn < N; tn += 32) {
+      nt_v16i acc;
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[r] = 0;
+      int sa = 0, sb = 0;
+      const bool a_ok = tm + l32 < M, b_ok = tn + l32 < N;
+      const int8_t *ap = L + (long long)(a_ok ? tm + l32 : 0) * K + lhi * 16;
+      const int8_t *bp = R + (long long)(b_ok ? tn + l32 : 0) * K + lhi * 16;
+      for (int k0 = 0; k0 < K; k0 += 32) {
+        // the upper half of the last slice is empty when K % 32 == 16
+        const bool k_ok = k0 + lhi * 16 < K;
+        nt_v4i a = {0, 0, 0, 0}, bb = {0, 0, 0, 0};
+        if (a_ok && k_ok) a = *reinterpret_cast<const nt_v4i *>(ap + k0);
+        if (b_ok && k_ok) bb = *reinterpret_cast<const nt_v4i *>(bp + k0);
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          sa = __builtin_amdgcn_sdot4(a[q], 0x01010101, sa, false);
+          sb = __builtin_amdgcn_sdot4(bb[q], 0x01010101, sb, false);
+        }
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bb, acc, 0, 0, 0);
+      }
+      sa += __shfl_xor(sa, 32, 64);
+      sb += __shfl_xor(sb, 32, 64);
+      // lane: column tn + l32; register r: row tm + 8*(r/4) + 4*lhi + r%4
+      const uint32_t colc = kconst - (uint32_t)lo * (uint32_t)sb;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int ml = (r >> 2) * 8 + lhi * 4 + (r & 3);
+        const int row_sum = __shfl(sa, ml, 64);
+        const uint32_t v = (uint32_t)acc[r] + colc - (uint32_t)ro * (uint32_t)row_sum;
+        const int32_t y = clip_i8(scale_i32((int32_t)v, pre, post, scale, oo));
+        if (tm + ml < M && b_ok) O[(long long)(tm + ml) * N + tn + l32] = (int8_t)y;
+      }
+    }
+  }
+}
+
 // dst[n][bh][bw][(dh*2+dw)*C + c] = src[n][2bh+dh-padT][2bw+dw-padL][c]; positions
 // outside the image and channels from 4C up hold `fill`. One thread per
 // destination pixel.
@@ -596,6 +653,25 @@ int mi355x_batch_matmul_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs, si
                      as_stream(stream), out, lhs, rhs, (int)M, (int)K, (int)N, out_offset,
                      lhs_offset, rhs_offset, out_pre, out_post, out_scale);
   return check_launch("batch_matmul_i8");
+}
+
+int mi355x_batch_matmul_nt_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs_nk, size_t batch,
+                              size_t M, size_t K, size_t N, int32_t out_offset,
+                              int32_t lhs_offset, int32_t rhs_offset, int32_t out_pre,
+                              int32_t out_post, int32_t out_scale, void *stream) {
+  if (batch == 0 || M == 0 || N == 0) return MI355X_OK;
+  MI355X_REQUIRE(out && lhs && rhs_nk, "NULL tensor");
+  MI355X_REQUIRE(shift_ok(out_pre) && shift_ok(out_post), "pre/post shift outside [0, 31]");
+  MI355X_REQUIRE(K > 0 && K % 16 == 0 && K < (1u << 20) && M < (1u << 15) && N < (1u << 15),
+                 "needs K %% 16 == 0 and matrices below 32768 rows (K = %zu)", K);
+  MI355X_REQUIRE((((uintptr_t)lhs | (uintptr_t)rhs_nk) & 15) == 0, "operands must be 16-byte aligned");
+  MI355X_REQUIRE(batch < (1ull << 31), "batch too large");
+  const size_t per_block = kGlueThreads / 64;
+  hipLaunchKernelGGL(batch_matmul_nt_i8_kernel, dim3((unsigned)((batch + per_block - 1) / per_block)),
+                     dim3(kGlueThreads), 0, as_stream(stream), out, lhs, rhs_nk, (long long)batch,
+                     (int)M, (int)K, (int)N, out_offset, lhs_offset, rhs_offset, out_pre, out_post,
+                     out_scale);
+  return check_launch("batch_matmul_nt_i8");
 }
 
 int mi355x_space_to_depth2_i8(int8_t *dst, const int8_t *src, size_t N, size_t IH, size_t IW,

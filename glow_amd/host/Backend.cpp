@@ -121,9 +121,25 @@ public:
       case Kind::SoftMax: MI355X_RETURN_IF_ERR(softmax(I, out)); break;
       case Kind::RowwiseQuantizedSparseLengthsWeightedSum:
       case Kind::EmbeddingBagByteRowwiseOffsets: MI355X_RETURN_IF_ERR(otherLookups(I, out)); break;
+      case Kind::Transpose: {
+        // a {0,2,1} shuffle read only by the BatchMatMul right behind it as its
+        // right operand: the product reads the untransposed tensor instead
+        if (opts_.fuseTransposeMatMul && at + 1 < insts_.size() &&
+            insts_[at + 1].kind == Kind::BatchMatMul &&
+            insts_[at + 1].operands[2] == I.operands[0] &&
+            insts_[at + 1].operands[1] != I.operands[0] &&
+            I.iattrs == std::vector<int64_t>{0, 2, 1} &&
+            M_.value(I.operands[0]).category == SymbolCategory::Activation &&
+            readers(I.operands[0]) == 1 && matmulNtOk(I, insts_[at + 1])) {
+          MI355X_RETURN_IF_ERR(matmulNt(I, insts_[at + 1], out));
+          at++;
+        } else {
+          MI355X_RETURN_IF_ERR(movement(I, out));
+        }
+        break;
+      }
       case Kind::ConvertTo:
       case Kind::InsertTensor:
-      case Kind::Transpose:
       case Kind::Gather:
       case Kind::BatchMatMul:
       case Kind::Sigmoid: MI355X_RETURN_IF_ERR(movement(I, out)); break;
@@ -500,6 +516,43 @@ private:
       return Error::success();
     }
     }
+  }
+
+  // Whether Transpose T followed by BatchMatMul B fits the K-contiguous kernel.
+  bool matmulNtOk(const Instruction &T, const Instruction &B) const {
+    const Type &src = M_.value(T.operands[1]).type, &tr = M_.value(T.operands[0]).type;
+    const Type &lhs = M_.value(B.operands[1]).type, &dst = M_.value(B.operands[0]).type;
+    if (src.kind != ElemKind::Int8QTy || tr.kind != ElemKind::Int8QTy ||
+        lhs.kind != ElemKind::Int8QTy || dst.kind != ElemKind::Int8QTy)
+      return false;
+    if (src.dims.size() != 3 || tr.dims.size() != 3 || lhs.dims.size() != 3 || dst.dims.size() != 3)
+      return false;
+    if (src.scale != tr.scale || src.offset != tr.offset) return false;
+    // src [B,N,K] -> tr [B,K,N]; lhs [B,M,K]; dst [B,M,N]
+    const int64_t Bn = src.dims[0], N = src.dims[1], K = src.dims[2], Mm = lhs.dims[1];
+    if (tr.dims[0] != Bn || tr.dims[1] != K || tr.dims[2] != N) return false;
+    if (lhs.dims[0] != Bn || lhs.dims[2] != K) return false;
+    if (dst.dims[0] != Bn || dst.dims[1] != Mm || dst.dims[2] != N) return false;
+    return K % 16 == 0 && Mm < (1 << 15) && N < (1 << 15) &&
+           M_.value(T.operands[1]).offset % 16 == 0 && M_.value(B.operands[1]).offset % 16 == 0;
+  }
+
+  Error matmulNt(const Instruction &T, const Instruction &I, MI355XFunction &out) {
+    Operand d = op(I, 0), s = op(I, 1), r = op(T, 1);
+    const size_t B = (size_t)s.ty().dims[0], M = (size_t)s.ty().dims[1], K = (size_t)s.ty().dims[2],
+                 N = (size_t)r.ty().dims[1];
+    const S32To8 p = s32to8(s.ty().scale * r.ty().scale / d.ty().scale);
+    const int32_t oo = d.ty().offset, lo = s.ty().offset, ro = r.ty().offset;
+    out.launches.push_back({"mi355x_batch_matmul_nt_i8", I.name,
+                            strFormat(" B=%zu M=%zu K=%zu N=%zu", B, M, K, N) + kv("out_offset", oo) +
+                                kv("lhs_offset", lo) + kv("rhs_offset", ro) + kv("out_pre", p.pre) +
+                                kv("out_post", p.post) + kv("out_scale", p.scale),
+                            [=](const DeviceBindings &b) {
+                              return mi355x_batch_matmul_nt_i8((int8_t *)d.ptr(b), (const int8_t *)s.ptr(b),
+                                                               (const int8_t *)r.ptr(b), B, M, K, N, oo, lo,
+                                                               ro, p.pre, p.post, p.scale, b.stream);
+                            }});
+    return Error::success();
   }
 
   Error softmax(const Instruction &I, MI355XFunction &out) {

@@ -148,6 +148,7 @@ struct BackendOptions {
   bool fuseConvAdd = true;             // convolution + ElementAdd (+ Relu) in one kernel
   bool spaceToDepthStem = true;        // stride-2 convolutions over <= 4 channels via space-to-depth
   bool fuseSlsChains = true;           // pooled lookups + ConvertTo/Quantize/InsertTensor, many tables per launch
+  bool fuseTransposeMatMul = true;     // BatchMatMul(L, Transpose(R)) without materialising the transpose
 };
 
 class MI355XBackend {

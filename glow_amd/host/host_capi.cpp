@@ -123,6 +123,7 @@ int mi355x_host_compile(mi355x_host_module *m, int function, int options) {
   o.fuseConvAdd = (options & MI355X_HOST_OPT_FUSE_CONV_ADD) != 0;
   o.spaceToDepthStem = (options & MI355X_HOST_OPT_SPACE_TO_DEPTH_STEM) != 0;
   o.fuseSlsChains = (options & MI355X_HOST_OPT_FUSE_SLS_CHAINS) != 0;
+  o.fuseTransposeMatMul = (options & MI355X_HOST_OPT_FUSE_TRANSPOSE_MATMUL) != 0;
   auto r = MI355XBackend().compile(*f, o);
   if (!r) return fail(r.error());
   m->compiled[function] = std::move(r.get());

@@ -265,6 +265,16 @@ int mi355x_batch_matmul_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs, si
                            size_t M, size_t K, size_t N, int32_t out_offset, int32_t lhs_offset,
                            int32_t rhs_offset, int32_t out_pre, int32_t out_post,
                            int32_t out_scale, void *stream);
+/* The same product with the right operand given K-contiguous, rhs_nk [N x K]
+ * per sample: out = lhs x transpose(rhs_nk), i.e. BatchMatMul(lhs,
+ * Transpose(rhs_nk, {0,2,1})) without materialising the transpose (the feature
+ * interaction of a ranking model multiplies a matrix with its own transpose).
+ * Runs on the matrix cores, one wavefront per sample. K % 16 == 0, operands
+ * 16-byte aligned. Same arithmetic as libjit_matmul_i8 (libjit_matmul.cpp:353-371). */
+int mi355x_batch_matmul_nt_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs_nk, size_t batch,
+                              size_t M, size_t K, size_t N, int32_t out_offset,
+                              int32_t lhs_offset, int32_t rhs_offset, int32_t out_pre,
+                              int32_t out_post, int32_t out_scale, void *stream);
 /* Space-to-depth by 2 of a padded NHWC int8 image, the layout change that turns
  * a stride-2 convolution over few channels into a stride-1 convolution over
  * 4x the channels (SpaceToDepth with block size 2, plus padding):

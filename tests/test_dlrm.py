@@ -24,8 +24,11 @@ def test_builds_and_compiles():
     multi = rows[k.index("mi355x_frwq_sls_multi")]
     assert (multi["tables"], multi["out_kind"], multi["stride"]) == (3, 3, 4 * 16)
     assert k.count("mi355x_convert_f16_to_f32") == 0 and k.count("mi355x_insert_rows") == 3
+    # the interaction's Transpose + BatchMatMul read the features as they lie
+    assert k.count("mi355x_batch_matmul_nt_i8") == 1 and k.count("mi355x_batch_transpose_i8") == 0
+    assert k.count("mi355x_batch_matmul_i8") == 0
     m, f = netlib.to_module(net)
-    m.compile(f, fuse_sls_chains=False)
+    m.compile(f, fuse_sls_chains=False, fuse_transpose_matmul=False)
     k = [r["kernel"] for r in H.parse_listing(m.describe(f)) if r["phase"] == "launch"]
     assert k.count("mi355x_frwq_slws") == 3 and k.count("mi355x_rwq_fc_i8") == 4
     assert k.count("mi355x_convert_f16_to_f32") == 3 and k.count("mi355x_insert_rows") == 6
@@ -50,7 +53,7 @@ def test_device_matches_oracle(fuse):
     cfg = dict(tables=4, rows=5000, dim=64, batch=256, mean_len=8, bottom=(64, 64), top=(128, 1))
     net, max_idx = dlrm.make(seed=3, **cfg)
     m, f = netlib.to_module(net)
-    m.compile(f, fuse_sls_chains=fuse)
+    m.compile(f, fuse_sls_chains=fuse, fuse_transpose_matmul=fuse)
     dm = H.DeviceManager().init()
     try:
         dm.add_network(m)

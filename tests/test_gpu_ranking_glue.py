@@ -118,3 +118,18 @@ def test_rowwise_quantized_slws(cols, idt):
     ones = np.ones(idx.size, np.float32)
     np.testing.assert_array_equal(capi.rwq_slws(data, scales, offsets, None, idx, lengths),
                                   go.rwq_slws_f32(data, scales, offsets, ones, idx, lengths))
+
+
+@pytest.mark.parametrize("shape", [(37, 27, 64, 27), (5, 32, 32, 32), (3, 40, 48, 70), (9, 1, 16, 5),
+                                   (4, 64, 128, 33)])
+def test_batch_matmul_with_k_contiguous_right_operand(shape):
+    """lhs x transpose(rhs_nk) equals BatchMatMul(lhs, transposed copy), bit for bit."""
+    b, m, k, n = shape
+    rng = np.random.default_rng(sum(shape))
+    lhs = rng.integers(-128, 128, (b, m, k)).astype(np.int8)
+    rhs_nk = rng.integers(-128, 128, (b, n, k)).astype(np.int8)
+    for (oo, lo, ro, outP) in ((3, -5, 7, (2, 9, 300)), (-128, 127, -128, (0, 14, 411)),
+                               (0, 0, 0, (0, 0, 1))):
+        want = go.batch_matmul_i8(lhs, np.ascontiguousarray(rhs_nk.transpose(0, 2, 1)), oo, lo, ro, outP)
+        got = capi.batch_matmul_nt_i8(lhs, rhs_nk, oo, lo, ro, outP)
+        np.testing.assert_array_equal(got, want)
