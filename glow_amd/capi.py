@@ -24,7 +24,7 @@ EXPORTS = [
     "mi355x_host_free", "mi355x_memcpy_h2d", "mi355x_memcpy_d2h",
     "mi355x_memcpy_d2d", "mi355x_fill_u8", "mi355x_copy_u8", "mi355x_gemm_tile_override",
     "mi355x_cwq_conv2d_add_i8", "mi355x_frwq_sls_multi",
-    "mi355x_specialize_bias_weights_qparams", "mi355x_rwq_slws", "mi355x_slws_set_fused_math", "mi355x_batch_matmul_nt_i8", "mi355x_add_i8", "mi355x_add_relu_i8",
+    "mi355x_specialize_bias_weights_qparams", "mi355x_rwq_slws", "mi355x_slws_set_fused_math", "mi355x_batch_matmul_nt_i8", "mi355x_rwq_fc_relu_i8", "mi355x_add_i8", "mi355x_add_relu_i8",
     "mi355x_relu_i8", "mi355x_convert_f16_to_f32", "mi355x_insert_rows",
     "mi355x_batch_transpose_i8", "mi355x_space_to_depth2_i8", "mi355x_gather", "mi355x_batch_matmul_i8", "mi355x_sigmoid_f32",
     "mi355x_max_pool_i8", "mi355x_avg_pool_i8", "mi355x_softmax_f32", "mi355x_stream_create",
@@ -597,6 +597,30 @@ def rwq_fc_i8(x, w_nk, bias, w_offsets, bias_pre, bias_post, bias_scale,
     d_sums = _row_sums_dev(d_w, N, K, precomputed_sums)
     launch_rwq_fc_i8(d_out, d_x, d_w, d_b, b8, *vs, M, K, N, out_offset,
                      in_offset, bias_offset, w_offsets_all_zero, d_sums)
+    return d_out.numpy()
+
+
+def rwq_fc_relu_i8(x, w_nk, bias, w_offsets, bias_pre, bias_post, bias_scale,
+                   out_pre, out_post, out_scale, fc_offset, in_offset, bias_offset,
+                   relu_offset, reluP, w_offsets_all_zero=None, precomputed_sums=True):
+    """RowwiseQuantizedFullyConnected + Relu in one kernel; reluP = (pre, post, scale)."""
+    x = np.ascontiguousarray(x, np.int8)
+    w_nk = np.ascontiguousarray(w_nk, np.int8)
+    M, K = x.shape
+    N = w_nk.shape[0]
+    if w_offsets_all_zero is None:
+        w_offsets_all_zero = not np.any(w_offsets)
+    d_x, d_w = to_device(x), to_device(w_nk)
+    d_b, b8 = _bias_dev(bias)
+    vs = [_dev_i32(v) for v in (w_offsets, bias_pre, bias_post, bias_scale,
+                                out_pre, out_post, out_scale)]
+    d_out = DeviceBuffer.empty((M, N), np.int8)
+    d_sums = _row_sums_dev(d_w, N, K, precomputed_sums)
+    check(lib().mi355x_rwq_fc_relu_i8(
+        _vp(d_out), _vp(d_x), _vp(d_w), _vp(d_b), C.c_int(b8), *[_vp(v) for v in vs],
+        _sz(M), _sz(K), _sz(N), _i32(fc_offset), _i32(in_offset), _i32(bias_offset),
+        C.c_int(bool(w_offsets_all_zero)), _vp(d_sums), _i32(relu_offset), *_i32s(reluP),
+        _vp(None)))
     return d_out.numpy()
 
 

@@ -152,6 +152,53 @@ int mi355x_rwq_fc_i8(int8_t *out, const int8_t *in, const int8_t *weights,
                    stream);
 }
 
+int mi355x_rwq_fc_relu_i8(int8_t *out, const int8_t *in, const int8_t *weights,
+                          const void *bias, int bias_is_i8,
+                          const int32_t *weights_offsets, const int32_t *bias_pre,
+                          const int32_t *bias_post, const int32_t *bias_scale,
+                          const int32_t *out_pre, const int32_t *out_post,
+                          const int32_t *out_scale, size_t M, size_t K, size_t N,
+                          int32_t fc_offset, int32_t in_offset, int32_t bias_offset,
+                          int weights_offsets_all_zero, const int32_t *weights_row_sums,
+                          int32_t relu_offset, int32_t relu_pre, int32_t relu_post,
+                          int32_t relu_scale, void *stream) {
+  if (M == 0 || N == 0) return MI355X_OK;
+  MI355X_REQUIRE(out && in && weights && bias, "NULL tensor");
+  MI355X_REQUIRE(weights_offsets && bias_pre && bias_post && bias_scale &&
+                     out_pre && out_post && out_scale,
+                 "NULL per-row parameter vector");
+  MI355X_REQUIRE(shift_ok(relu_pre) && shift_ok(relu_post), "relu pre/post shift outside [0, 31]");
+  MI355X_REQUIRE(fc_offset >= -128 && fc_offset <= 127,
+                 "offset %d of the FullyConnected result outside the int8 range", fc_offset);
+  int rc = check_dims(M, K, N);
+  if (rc != MI355X_OK) return rc;
+  Epilogue ep{};
+  ep.bias = bias;
+  ep.bias_is_i8 = bias_is_i8;
+  ep.b_off = ColParam{nullptr, bias_offset};
+  ep.bias_pre = ColParam{bias_pre, 0};
+  ep.bias_post = ColParam{bias_post, 0};
+  ep.bias_scale = ColParam{bias_scale, 0};
+  ep.w_off = ColParam{weights_offsets, 0};
+  ep.out_pre = ColParam{out_pre, 0};
+  ep.out_post = ColParam{out_post, 0};
+  ep.out_scale = ColParam{out_scale, 0};
+  ep.a_off = in_offset;
+  ep.out_off = fc_offset;
+  ep.act = MI355X_ACT_NONE;
+  ep.sum_b = weights_row_sums;
+  ep.add.res = nullptr;
+  ep.add.relu = 1;
+  ep.add.sum_off = fc_offset;
+  ep.add.dest_off = relu_offset;
+  ep.add.dest_pre = relu_pre;
+  ep.add.dest_post = relu_post;
+  ep.add.dest_scale = relu_scale;
+  ep.add.small = relu_scale > -(1 << 23) && relu_scale < (1 << 23);
+  return fc_common(out, in, weights, ep, M, K, N, !weights_offsets_all_zero,
+                   stream);
+}
+
 int mi355x_fc_i8(int8_t *out, const int8_t *in, const int8_t *weights_kn,
                  int8_t *weights_nk_workspace, int repack, const void *bias,
                  int bias_is_i8, size_t M, size_t K, size_t N,

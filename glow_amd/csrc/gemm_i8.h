@@ -52,6 +52,9 @@ struct ColParam {
 // output tile is written, optionally followed by Relu: what ElementAdd and Relu
 // instructions behind a convolution compute, without the round trip through
 // memory. Same arithmetic as the standalone kernels.
+// With res == NULL and relu != 0 only the Relu stage runs, on this kernel's own
+// result: a Relu instruction (with its own output scale and offset) behind a
+// FullyConnected. sum_off is then the offset of the kernel's result.
 struct FusedAdd {
   const int8_t *res;    // [M x ldc] like the output, or NULL
   int32_t sum_off, own_off, res_off;
@@ -89,6 +92,24 @@ __device__ __forceinline__ uint32_t fused_add_word_t(uint32_t own, uint32_t res,
                                          (int32_t)(int8_t)(res >> (8 * b)), f) & 0xff)
          << (8 * b);
   return o;
+}
+
+// libjit_element_relu_i8-style stage alone: clip(scale(max(v, so) - so) + dest_off)
+template <bool SMALL>
+__device__ __forceinline__ uint32_t fused_relu_word_t(uint32_t own, const FusedAdd &f) {
+  const int32_t so = (int32_t)(int8_t)f.sum_off;
+  uint32_t o = 0;
+#pragma unroll
+  for (int b = 0; b < 4; b++) {
+    const int32_t v = max((int32_t)(int8_t)(own >> (8 * b)), so);
+    o |= (uint32_t)(clip_i8(scale_i32_sel<SMALL>(v - so, f.dest_pre, f.dest_post,
+                                                 f.dest_scale, f.dest_off)) & 0xff)
+         << (8 * b);
+  }
+  return o;
+}
+__device__ __forceinline__ uint32_t fused_relu_word(uint32_t own, const FusedAdd &f) {
+  return f.small ? fused_relu_word_t<true>(own, f) : fused_relu_word_t<false>(own, f);
 }
 
 // int8 operands minus int8-range offsets stay far below 2^23, so the 24-bit
@@ -285,6 +306,11 @@ __device__ __forceinline__ void gemm_epilogue_impl(
         v.y = (int)fused_add_word((uint32_t)v.y, (uint32_t)q.y, ep.add);
         v.z = (int)fused_add_word((uint32_t)v.z, (uint32_t)q.z, ep.add);
         v.w = (int)fused_add_word((uint32_t)v.w, (uint32_t)q.w, ep.add);
+      } else if (ep.add.relu) {
+        v.x = (int)fused_relu_word((uint32_t)v.x, ep.add);
+        v.y = (int)fused_relu_word((uint32_t)v.y, ep.add);
+        v.z = (int)fused_relu_word((uint32_t)v.z, ep.add);
+        v.w = (int)fused_relu_word((uint32_t)v.w, ep.add);
       }
       *reinterpret_cast<int4 *>(obase + (long long)r * ep.ldc + s * 16) = v;
     }
@@ -293,6 +319,7 @@ __device__ __forceinline__ void gemm_epilogue_impl(
       const int r = c / cols_here, s = c - r * cols_here;
       int32_t v = s_out[r * OUT_STRIDE + s];
       if (rbase) v = fused_add_one<false>(v, rbase[(long long)r * ep.ldc + s], ep.add);
+      else if (ep.add.relu) v = (int32_t)(int8_t)fused_relu_word_t<false>((uint32_t)v & 0xff, ep.add);
       obase[(long long)r * ep.ldc + s] = (int8_t)v;
     }
   }

@@ -147,7 +147,20 @@ public:
       case Kind::Dequantize: MI355X_RETURN_IF_ERR(dequantize(I, out)); break;
       case Kind::RescaleQuantized: MI355X_RETURN_IF_ERR(rescale(I, out)); break;
       case Kind::FullyConnected: MI355X_RETURN_IF_ERR(fc(I, out)); break;
-      case Kind::RowwiseQuantizedFullyConnected: MI355X_RETURN_IF_ERR(rwqfc(I, out)); break;
+      case Kind::RowwiseQuantizedFullyConnected: {
+        // a Relu instruction right behind it that is the only reader of its result
+        const Instruction *reluI = nullptr;
+        if (opts_.fuseFcRelu && at + 1 < insts_.size() && insts_[at + 1].kind == Kind::Relu &&
+            insts_[at + 1].operands[1] == I.operands[0] &&
+            M_.value(I.operands[0]).category == SymbolCategory::Activation &&
+            readers(I.operands[0]) == 1 &&
+            M_.value(insts_[at + 1].operands[0]).type.kind == ElemKind::Int8QTy &&
+            M_.value(insts_[at + 1].operands[0]).type.dims == M_.value(I.operands[0]).type.dims)
+          reluI = &insts_[at + 1];
+        MI355X_RETURN_IF_ERR(rwqfc(I, out, reluI));
+        if (reluI) at++;
+        break;
+      }
       case Kind::MatMul: MI355X_RETURN_IF_ERR(matmul(I, out)); break;
       case Kind::Convolution: MI355X_RETURN_IF_ERR(conv(I, out, false)); break;
       case Kind::ChannelwiseQuantizedConvolution: {
@@ -190,7 +203,8 @@ public:
         const std::string &kn = out.launches[l].kernel;
         out.launches[l].tunable = kn == "mi355x_fc_i8" || kn == "mi355x_rwq_fc_i8" ||
                                   kn == "mi355x_matmul_i8" || kn == "mi355x_conv2d_i8" ||
-                                  kn == "mi355x_cwq_conv2d_i8" || kn == "mi355x_cwq_conv2d_add_i8";
+                                  kn == "mi355x_cwq_conv2d_i8" || kn == "mi355x_cwq_conv2d_add_i8" ||
+                                  kn == "mi355x_rwq_fc_relu_i8";
       }
     }
     assignLevels(out);
@@ -719,7 +733,7 @@ private:
     return Error::success();
   }
 
-  Error rwqfc(const Instruction &I, MI355XFunction &out) {
+  Error rwqfc(const Instruction &I, MI355XFunction &out, const Instruction *reluI = nullptr) {
     Operand d = op(I, 0), s = op(I, 1), w = op(I, 2), bi = op(I, 3), sc = op(I, 4), of = op(I, 5);
     CHECK_OP(d.ty().kind == ElemKind::Int8QTy && s.ty().kind == ElemKind::Int8QTy &&
                  w.ty().kind == ElemKind::Int8QTy && biasKindOk(bi.ty().kind),
@@ -760,6 +774,31 @@ private:
                              return mi355x_rowsum_i8((int32_t *)sumPtr(b), (const int8_t *)w.ptr(b), N,
                                                      K, b.stream);
                            }});
+    if (reluI) {
+      // the kernel's result keeps the FullyConnected's scale and offset; the
+      // Relu stage maps it to the Relu's output type
+      Operand rd = op(*reluI, 0);
+      const S32To8 rp = s32to8(d.ty().scale / rd.ty().scale);
+      const int32_t ro = rd.ty().offset;
+      out.launches.push_back(
+          {"mi355x_rwq_fc_relu_i8", I.name,
+           strFormat(" M=%zu K=%zu N=%zu", M, K, N) + kv("fc_offset", oo) + kv("in_offset", io) +
+               kv("bias_offset", bo) + kv("bias_is_i8", bias8) + kv("weights_offsets_all_zero", allZero) +
+               kv("row_sums", sums) + kv("relu_offset", ro) + kv("relu_pre", rp.pre) +
+               kv("relu_post", rp.post) + kv("relu_scale", rp.scale) + vecStr("bias_pre", bpre) +
+               vecStr("bias_post", bpost) + vecStr("bias_scale", bscale) + vecStr("out_pre", opre) +
+               vecStr("out_post", opost) + vecStr("out_scale", oscale),
+           [=](const DeviceBindings &b) {
+             auto g = [&](size_t o) { return (const int32_t *)(b.generated + o); };
+             return mi355x_rwq_fc_relu_i8((int8_t *)rd.ptr(b), (const int8_t *)s.ptr(b),
+                                          (const int8_t *)w.ptr(b), bi.ptr(b), bias8,
+                                          (const int32_t *)of.ptr(b), g(o0), g(o1), g(o2), g(o3), g(o4),
+                                          g(o5), M, K, N, oo, io, bo, allZero ? 1 : 0,
+                                          sums ? (const int32_t *)sumPtr(b) : nullptr, ro, rp.pre,
+                                          rp.post, rp.scale, b.stream);
+           }});
+      return Error::success();
+    }
     out.launches.push_back(
         {"mi355x_rwq_fc_i8", I.name,
          strFormat(" M=%zu K=%zu N=%zu", M, K, N) + kv("out_offset", oo) + kv("in_offset", io) +

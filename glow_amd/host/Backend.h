@@ -149,6 +149,7 @@ struct BackendOptions {
   bool spaceToDepthStem = true;        // stride-2 convolutions over <= 4 channels via space-to-depth
   bool fuseSlsChains = true;           // pooled lookups + ConvertTo/Quantize/InsertTensor, many tables per launch
   bool fuseTransposeMatMul = true;     // BatchMatMul(L, Transpose(R)) without materialising the transpose
+  bool fuseFcRelu = true;              // RowwiseQuantizedFullyConnected + Relu of its result in one kernel
 };
 
 class MI355XBackend {

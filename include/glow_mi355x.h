@@ -317,6 +317,23 @@ int mi355x_rwq_fc_i8(int8_t *out, const int8_t *in, const int8_t *weights,
                      int32_t bias_offset, int weights_offsets_all_zero,
                      const int32_t *weights_row_sums, void *stream);
 
+/* RowwiseQuantizedFullyConnected followed by a Relu instruction of its result
+ * (libjit_element_relu_i8, reference libjit.cpp:1851-1858, parameters from
+ * LLVMIRGen.cpp:1465-1499) in one kernel. The FullyConnected result is
+ * clipped to int8 at `fc_offset` exactly as mi355x_rwq_fc_i8 would store it;
+ * then out = clip(scale(max(v, fc_offset) - fc_offset; reluP) + relu_offset)
+ * with reluP = quantizeScaleOffset32To8(fcScale / reluScale). */
+int mi355x_rwq_fc_relu_i8(int8_t *out, const int8_t *in, const int8_t *weights,
+                          const void *bias, int bias_is_i8,
+                          const int32_t *weights_offsets, const int32_t *bias_pre,
+                          const int32_t *bias_post, const int32_t *bias_scale,
+                          const int32_t *out_pre, const int32_t *out_post,
+                          const int32_t *out_scale, size_t M, size_t K, size_t N,
+                          int32_t fc_offset, int32_t in_offset, int32_t bias_offset,
+                          int weights_offsets_all_zero, const int32_t *weights_row_sums,
+                          int32_t relu_offset, int32_t relu_pre, int32_t relu_post,
+                          int32_t relu_scale, void *stream);
+
 /* libjit_fc_i8_i32 / _i8_i8 (libjit_matmul.cpp:254-280, 395-422).
  * weights_kn is [K x N] as Glow stores FullyConnected weights; the kernel
  * consumes the [N x K] transpose, which is written to `weights_nk_workspace`

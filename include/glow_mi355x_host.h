@@ -118,7 +118,8 @@ enum {
   MI355X_HOST_OPT_SPACE_TO_DEPTH_STEM = 8, /* stride-2 convolutions over <= 4 channels via space-to-depth */
   MI355X_HOST_OPT_FUSE_SLS_CHAINS = 16, /* pooled lookups + ConvertTo/Quantize/InsertTensor, many tables per launch */
   MI355X_HOST_OPT_FUSE_TRANSPOSE_MATMUL = 32, /* BatchMatMul(L, Transpose(R)) reads R as it lies */
-  MI355X_HOST_OPT_DEFAULT = 63
+  MI355X_HOST_OPT_FUSE_FC_RELU = 64, /* RowwiseQuantizedFullyConnected + Relu in one kernel */
+  MI355X_HOST_OPT_DEFAULT = 127
 };
 int mi355x_host_compile(mi355x_host_module *m, int function, int options);
 /* Listing of the compiled function's launches and derived parameters; returns

@@ -27,8 +27,10 @@ def test_builds_and_compiles():
     # the interaction's Transpose + BatchMatMul read the features as they lie
     assert k.count("mi355x_batch_matmul_nt_i8") == 1 and k.count("mi355x_batch_transpose_i8") == 0
     assert k.count("mi355x_batch_matmul_i8") == 0
+    # every hidden layer's Relu runs inside its FullyConnected
+    assert k.count("mi355x_relu_i8") == 0 and k.count("mi355x_rwq_fc_relu_i8") >= 2
     m, f = netlib.to_module(net)
-    m.compile(f, fuse_sls_chains=False, fuse_transpose_matmul=False)
+    m.compile(f, fuse_sls_chains=False, fuse_transpose_matmul=False, fuse_fc_relu=False)
     k = [r["kernel"] for r in H.parse_listing(m.describe(f)) if r["phase"] == "launch"]
     assert k.count("mi355x_frwq_slws") == 3 and k.count("mi355x_rwq_fc_i8") == 4
     assert k.count("mi355x_convert_f16_to_f32") == 3 and k.count("mi355x_insert_rows") == 6
@@ -53,7 +55,7 @@ def test_device_matches_oracle(fuse):
     cfg = dict(tables=4, rows=5000, dim=64, batch=256, mean_len=8, bottom=(64, 64), top=(128, 1))
     net, max_idx = dlrm.make(seed=3, **cfg)
     m, f = netlib.to_module(net)
-    m.compile(f, fuse_sls_chains=fuse, fuse_transpose_matmul=fuse)
+    m.compile(f, fuse_sls_chains=fuse, fuse_transpose_matmul=fuse, fuse_fc_relu=fuse)
     dm = H.DeviceManager().init()
     try:
         dm.add_network(m)

@@ -120,6 +120,23 @@ def test_rwq_fc_vs_oracle(shape):
                                   go.rwq_fc_i8(*cases.rwq_fc_args(c)))
 
 
+@pytest.mark.parametrize("shape", [(128, 1024, 1024), (300, 13, 512), (77, 415, 96), (4096, 512, 256)])
+def test_rwq_fc_with_fused_relu(shape):
+    """RowwiseQuantizedFullyConnected + Relu in one kernel equals the two
+    instructions run one after the other, for both multiplier paths of the
+    Relu rescale."""
+    M, K, N = shape
+    say("rwq_fc+relu", shape)
+    c = cases.rwq_fc_case(M + K, M, K, N, symmetric=(K % 2 == 0))
+    args = cases.rwq_fc_args(c)
+    fc = go.rwq_fc_i8(*args)
+    for relu_offset, reluP in ((-128, (0, 8, 300)), (5, (1, 9, 1 << 24)), (-3, (0, 0, 1))):
+        want = go.relu_i8(fc, c["out_offset"], relu_offset, reluP)
+        got = capi.rwq_fc_relu_i8(*args[:10], c["out_offset"], c["in_offset"], c["bias_offset"],
+                                  relu_offset, reluP)
+        np.testing.assert_array_equal(got, want)
+
+
 def test_rwq_fc_large_tiles_properties():
     """A shape that takes the 256x256 tile. The oracle runs on a row sample;
     all rows are checked through linearity in the batch dimension: identical
