@@ -755,6 +755,141 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_rows_kernel(SlwsArgs a) {
   if (bag < a.segments && sub == 0) store_columns<kCols>(a, bag, lir * kCols, acc);
 }
 
+// The same arithmetic for short rows (32 or 64 data bytes): a row takes only
+// LPR = 8 or 16 lanes, so a wavefront works on 64/LPR bags side by side, one
+// per lane group, and nothing has to be added across lanes at the end. A
+// group's lanes fetch its lookups (index, weight, scale, offset) kGB at a
+// time and hand them to each other through a wave-private LDS table.
+template <bool IS4, bool SO16, int LPR, bool OFF32>
+__global__ __launch_bounds__(kSlwsThreads) void slws_groups_kernel(SlwsArgs a) {
+  select_table(a);
+  constexpr int kGroups = kSlwsThreads / LPR; // bags per block
+  constexpr int kCols = IS4 ? 8 : 4;          // output columns per lane
+  constexpr int kGB = 32;                     // lookups of a bag per round
+  constexpr int kPer = kGB / LPR;             // lookups one lane fetches per round
+  constexpr int kChunk = 8;                   // row reads under one uniform branch
+  __shared__ long long s_part[kSlwsThreads / 64];
+  __shared__ int s_own[kGroups];
+  __shared__ uint32_t s_key[kGroups][kGB];
+  __shared__ float2 s_ws[kGroups][kGB];
+
+  const int tid = threadIdx.x;
+  const int grp = tid / LPR, lir = tid % LPR;
+  const long long first_bag = (long long)blockIdx.x * kGroups;
+  const long long bag = first_bag + grp;
+
+  long long start = 0;
+  int len = 0;
+  bag_span<kGroups>(a, tid, grp, bag, first_bag, s_part, s_own, start, len);
+  {
+    const long long room = a.num_indices - start;
+    len = room <= 0 ? 0 : (int)min((long long)len, room);
+  }
+  // the loops below run as long as the longest bag of the wavefront needs
+  int wave_len = len;
+#pragma unroll
+  for (int off = LPR; off < 64; off <<= 1) wave_len = max(wave_len, __shfl_xor(wave_len, off, 64));
+  wave_len = __builtin_amdgcn_readfirstlane(wave_len);
+
+  uint32_t *keys = s_key[grp];
+  float2 *wso = s_ws[grp];
+  const uint32_t lane_off = (uint32_t)lir * 4u;
+  float acc[kCols];
+  float acc_o = 0.0f;
+#pragma unroll
+  for (int c = 0; c < kCols; c++) acc[c] = 0.0f;
+
+  for (int base = 0; base < wave_len; base += kGB) {
+    const int cnt = min(kGB, len - base);           // this bag's share (may be <= 0)
+    const int wave_cnt = min(kGB, wave_len - base); // uniform
+#pragma unroll
+    for (int k = 0; k < kPer; k++) {
+      const int j = lir + k * LPR;
+      const long long pos = start + base + j;
+      long long row = -1;
+      float w = 0.0f;
+      if (j < cnt && pos < a.num_indices) {
+        row = a.idx64 ? reinterpret_cast<const long long *>(a.indices)[pos]
+                      : (long long)reinterpret_cast<const int *>(a.indices)[pos];
+        if (!a.weights) {
+          w = 1.0f;
+        } else if (a.w16) {
+          w = __half2float(reinterpret_cast<const __half *>(a.weights)[pos]);
+        } else {
+          w = reinterpret_cast<const float *>(a.weights)[pos];
+        }
+      }
+      // a skipped lookup reads row 0 and contributes exactly +0
+      const bool valid = row >= 0 && row < a.data_rows;
+      if (!valid) row = 0;
+      float s, o;
+      if (!SO16 && a.sep_scales) {
+        s = a.sep_scales[row];
+        o = a.sep_offsets[row];
+      } else {
+        const uint32_t *so = reinterpret_cast<const uint32_t *>(
+            a.data + row * a.in_line + a.data_bytes);
+        if constexpr (SO16) {
+          const uint32_t v = so[0];
+          s = __half2float(__ushort_as_half((unsigned short)(v & 0xffff)));
+          o = __half2float(__ushort_as_half((unsigned short)(v >> 16)));
+        } else {
+          s = __uint_as_float(so[0]);
+          o = __uint_as_float(so[1]);
+        }
+      }
+      keys[j] = OFF32 ? (uint32_t)(row * a.in_line) : (uint32_t)row;
+      wso[j] = valid ? make_float2(w * s, w * o) : make_float2(0.0f, 0.0f);
+    }
+    wave_lds_sync();
+    uint32_t q[kGB];
+#pragma unroll
+    for (int c = 0; c < kGB / kChunk; c++) {
+      if (c * kChunk < wave_cnt) {
+#pragma unroll
+        for (int u = 0; u < kChunk; u++) {
+          const int j = c * kChunk + u;
+          const uint32_t key = keys[j];
+          if constexpr (OFF32) {
+            q[j] = *(const global_u32 *)((const global_u8 *)a.data + (key + lane_off));
+          } else {
+            q[j] = *reinterpret_cast<const uint32_t *>(
+                a.data + (long long)key * a.in_line + lane_off);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < kGB / kChunk; c++) {
+      if (c * kChunk < wave_cnt) {
+#pragma unroll
+        for (int u = 0; u < kChunk; u++) {
+          const int j = c * kChunk + u;
+          const float2 f = wso[j];
+          acc_o += f.y;
+          if constexpr (IS4) {
+            const uint32_t lo = q[j] & 0x0f0f0f0fu, hi = (q[j] >> 4) & 0x0f0f0f0fu;
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+              acc[2 * b] = __fmaf_rn(f.x, (float)((lo >> (8 * b)) & 0xff), acc[2 * b]);
+              acc[2 * b + 1] =
+                  __fmaf_rn(f.x, (float)((hi >> (8 * b)) & 0xff), acc[2 * b + 1]);
+            }
+          } else {
+#pragma unroll
+            for (int b = 0; b < 4; b++)
+              acc[b] = __fmaf_rn(f.x, (float)((q[j] >> (8 * b)) & 0xff), acc[b]);
+          }
+        }
+      }
+    }
+    wave_lds_sync(); // slots are rewritten by the next round
+  }
+#pragma unroll
+  for (int c = 0; c < kCols; c++) acc[c] += acc_o;
+  if (bag < a.segments) store_columns<kCols>(a, bag, lir * kCols, acc);
+}
+
 // Sum of the clamped lengths of each chunk of kChunkBags bags.
 __global__ __launch_bounds__(256) void slws_chunk_sums_kernel(
     const int32_t *lengths, long long segments, int64_t *chunk_sums) {
@@ -860,6 +995,28 @@ static void launch_rows_kind(int kind, dim3 grid, hipStream_t st, const SlwsArgs
     break;
   }
 #undef MI355X_SLWS_ROWS
+}
+
+template <int LPR, bool OFF32>
+static void launch_groups_kind(int kind, dim3 grid, hipStream_t st, const SlwsArgs &a) {
+#define MI355X_SLWS_GROUPS(IS4, SO16)                                          \
+  hipLaunchKernelGGL((slws_groups_kernel<IS4, SO16, LPR, OFF32>), grid,        \
+                     dim3(kSlwsThreads), 0, st, a)
+  switch (kind) {
+  case MI355X_FUSED_U8_F32:
+    MI355X_SLWS_GROUPS(false, false);
+    break;
+  case MI355X_FUSED_U8_F16:
+    MI355X_SLWS_GROUPS(false, true);
+    break;
+  case MI355X_FUSED_U4_F16:
+    MI355X_SLWS_GROUPS(true, true);
+    break;
+  default:
+    MI355X_SLWS_GROUPS(true, false);
+    break;
+  }
+#undef MI355X_SLWS_GROUPS
 }
 
 // Whether the fused-arithmetic kernels may be used (process-wide).
@@ -968,6 +1125,21 @@ static int slws_dispatch(void *dest, int out_is_f16, const uint8_t *data,
                        in_line_size % 4 == 0 && (((uintptr_t)data) % 4 == 0) &&
                        (data_bytes == 32 || data_bytes == 64 ||
                         data_bytes == 128 || data_bytes == 256);
+  if (rows_ok && data_bytes <= 64) {
+    // short rows: several bags per wavefront
+    const size_t per_block = kSlwsThreads / (data_bytes / 4);
+    const size_t gblocks = (out_rows + per_block - 1) / per_block;
+    MI355X_REQUIRE(gblocks < 0x7fffffffu, "too many bags");
+    dim3 ggrid((unsigned)gblocks, (unsigned)x.n_tables);
+    if (data_bytes == 32) {
+      if (off32) launch_groups_kind<8, true>(kind, ggrid, st, a);
+      else launch_groups_kind<8, false>(kind, ggrid, st, a);
+    } else {
+      if (off32) launch_groups_kind<16, true>(kind, ggrid, st, a);
+      else launch_groups_kind<16, false>(kind, ggrid, st, a);
+    }
+    return check_launch("frwq_slws");
+  }
   if (rows_ok) {
     const size_t rblocks = (out_rows + 3) / 4;
     MI355X_REQUIRE(rblocks < 0x7fffffffu, "too many bags");
