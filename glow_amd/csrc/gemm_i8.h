@@ -112,6 +112,49 @@ __device__ __forceinline__ uint32_t fused_relu_word(uint32_t own, const FusedAdd
   return f.small ? fused_relu_word_t<true>(own, f) : fused_relu_word_t<false>(own, f);
 }
 
+// The common case of both stages: every scale below 2^23 in magnitude and no
+// pre-shift (rescale factors near one). Then ((x - off) * s + rtn) equals
+// x * s + (rtn - off * s) modulo 2^32, one 24-bit multiply-add per value with
+// a constant formed once, and the result is bit for bit that of scale_i32.
+struct FusedAddConsts {
+  int32_t own_c, res_c, relu_c;
+};
+__device__ __forceinline__ FusedAddConsts fused_add_consts(const FusedAdd &f) {
+  auto rtn = [](int32_t post) { return post > 0 ? (1u << (post - 1)) : 0u; };
+  FusedAddConsts c;
+  c.own_c = (int32_t)(rtn(f.own_post) - (uint32_t)f.own_off * (uint32_t)f.own_scale);
+  c.res_c = (int32_t)(rtn(f.res_post) - (uint32_t)f.res_off * (uint32_t)f.res_scale);
+  c.relu_c = (int32_t)(rtn(f.dest_post) -
+                       (uint32_t)(int32_t)(int8_t)f.sum_off * (uint32_t)f.dest_scale);
+  return c;
+}
+template <bool ADD>
+__device__ __forceinline__ uint32_t fused_word_fast(uint32_t own, uint32_t res,
+                                                    const FusedAdd &f,
+                                                    const FusedAddConsts &c) {
+  const int32_t so = (int32_t)(int8_t)f.sum_off;
+  int32_t r[4];
+#pragma unroll
+  for (int b = 0; b < 4; b++) {
+    int32_t v = (int32_t)(int8_t)(own >> (8 * b));
+    if constexpr (ADD) {
+      const int32_t x = (int32_t)(int8_t)(res >> (8 * b));
+      const int32_t a = (int32_t)((uint32_t)__mul24(v, f.own_scale) + (uint32_t)c.own_c) >> f.own_post;
+      const int32_t bb = (int32_t)((uint32_t)__mul24(x, f.res_scale) + (uint32_t)c.res_c) >> f.res_post;
+      v = med3_i32((int32_t)((uint32_t)a + (uint32_t)bb + (uint32_t)f.sum_off), -128, 127);
+    }
+    if (!ADD || f.relu) {
+      v = max(v, so);
+      v = (int32_t)((uint32_t)__mul24(v, f.dest_scale) + (uint32_t)c.relu_c) >> f.dest_post;
+      v = med3_i32((int32_t)((uint32_t)v + (uint32_t)f.dest_off), -128, 127);
+    }
+    r[b] = v;
+  }
+  return __builtin_amdgcn_perm(
+      __builtin_amdgcn_perm((uint32_t)r[3], (uint32_t)r[2], 0x0c0c0400u),
+      __builtin_amdgcn_perm((uint32_t)r[1], (uint32_t)r[0], 0x0c0c0400u), 0x05040100u);
+}
+
 // int8 operands minus int8-range offsets stay far below 2^23, so the 24-bit
 // multiplier applies whenever the scales do (f.small, set on the host).
 __device__ __forceinline__ uint32_t fused_add_word(uint32_t own, uint32_t res,
@@ -296,10 +339,28 @@ __device__ __forceinline__ void gemm_epilogue_impl(
       ep.add.res ? ep.add.res + (long long)m0 * ep.ldc + n_base + n0 : nullptr;
   if (vec_ok && (!rbase || ((((uintptr_t)rbase) & 15) == 0))) {
     const int segs = cols_here / 16;
+    // every scale small and no pre-shift in the stages that run
+    const bool fast =
+        ep.add.small &&
+        (!rbase || (ep.add.own_pre == 0 && ep.add.res_pre == 0)) &&
+        (!ep.add.relu || ep.add.dest_pre == 0);
+    const FusedAddConsts fc = fused_add_consts(ep.add);
     for (int c = tid; c < rows_here * segs; c += THREADS) {
       const int r = c / segs, s = c - r * segs;
       int4 v = *reinterpret_cast<const int4 *>(s_out + r * OUT_STRIDE + s * 16);
-      if (rbase) {
+      if (rbase && fast) {
+        const int4 q =
+            *reinterpret_cast<const int4 *>(rbase + (long long)r * ep.ldc + s * 16);
+        v.x = (int)fused_word_fast<true>((uint32_t)v.x, (uint32_t)q.x, ep.add, fc);
+        v.y = (int)fused_word_fast<true>((uint32_t)v.y, (uint32_t)q.y, ep.add, fc);
+        v.z = (int)fused_word_fast<true>((uint32_t)v.z, (uint32_t)q.z, ep.add, fc);
+        v.w = (int)fused_word_fast<true>((uint32_t)v.w, (uint32_t)q.w, ep.add, fc);
+      } else if (!rbase && ep.add.relu && fast) {
+        v.x = (int)fused_word_fast<false>((uint32_t)v.x, 0u, ep.add, fc);
+        v.y = (int)fused_word_fast<false>((uint32_t)v.y, 0u, ep.add, fc);
+        v.z = (int)fused_word_fast<false>((uint32_t)v.z, 0u, ep.add, fc);
+        v.w = (int)fused_word_fast<false>((uint32_t)v.w, 0u, ep.add, fc);
+      } else if (rbase) {
         const int4 q =
             *reinterpret_cast<const int4 *>(rbase + (long long)r * ep.ldc + s * 16);
         v.x = (int)fused_add_word((uint32_t)v.x, (uint32_t)q.x, ep.add);

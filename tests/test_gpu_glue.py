@@ -136,6 +136,33 @@ def test_conv_with_fused_residual_add(shape, relu):
     np.testing.assert_array_equal(got, want)
 
 
+@pytest.mark.parametrize("relu", [False, True])
+@pytest.mark.parametrize("params", [
+    # (conv, residual, relu) rescale triples (pre, post, scale)
+    ((0, 9, 300), (0, 8, 411), (0, 9, 333)),         # no pre-shift, small scales: folded constants
+    ((0, 0, 1), (0, 0, 1), (0, 0, 1)),               # identities
+    ((1, 9, 300), (0, 8, 411), (0, 9, 333)),         # a pre-shift in the add
+    ((0, 9, 300), (0, 8, 411), (2, 9, 333)),         # a pre-shift in the relu
+    ((0, 20, 1 << 24), (0, 8, 411), (0, 9, 333)),    # a scale beyond the 24-bit multiplier
+])
+def test_fused_residual_add_parameter_paths(params, relu):
+    """Every arithmetic path of the fused add (+ Relu) stage gives the bits of
+    the separate instructions."""
+    from tests import cases
+    cp, rp, dp = params
+    c = cases.cwq_conv_case(93, 2, 10, 10, 32, 64, kernel=(1, 1), pads=(0,) * 4,
+                            act=cases._w.ACT_NONE, in_offset=3, out_offset=-7)
+    conv = go.cwq_conv2d_i8(*cases.cwq_conv_args(c))
+    res = np.random.default_rng(94).integers(-128, 128, conv.shape).astype(np.int8)
+    for sum_off, res_off, dest_off in ((11, -20, -128), (-128, 127, 127), (0, 0, 0)):
+        want = go.add_i8(conv, res, sum_off, c["out_offset"], res_off, cp, rp)
+        if relu:
+            want = go.relu_i8(want, sum_off, dest_off, dp)
+        add = capi.fused_add(sum_off, res_off, cp, rp, relu, dest_off, dp)
+        got = capi.cwq_conv2d_add_i8(*cases.cwq_conv_args(c), res, add)
+        np.testing.assert_array_equal(got, want)
+
+
 @pytest.mark.parametrize("shape,pads", [((2, 16, 16, 3), (3, 3)), ((1, 9, 7, 4), (0, 1)), ((3, 8, 8, 1), (1, 0))])
 def test_space_to_depth(shape, pads):
     rng = np.random.default_rng(shape[1])
