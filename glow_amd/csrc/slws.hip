@@ -19,6 +19,12 @@
 // keeps the vector ALU for the five operations per element the arithmetic
 // needs (convert, multiply, add, multiply, add).
 //
+// That is the strict form of the arithmetic (slws_kernel, slws_wave_kernel).
+// By default rows of 32, 64, 128 or 256 data bytes with fp32 accumulation run
+// the fused form further down (slws_rows_kernel, slws_groups_kernel): the same
+// sum regrouped into one fused multiply-add per element, equal to the CPU loop
+// to rounding; mi355x_slws_set_fused_math(0) switches back to the strict form.
+//
 // The start of a bag in the index list is the exclusive prefix sum of the
 // lengths. A block sums the lengths in front of it itself (from the start of
 // its chunk of kChunkBags bags, plus one pre-summed value per earlier chunk),
