@@ -44,11 +44,33 @@ struct ConvRows {
   // come from (ICg % 16 == 0, so a chunk never straddles a tap)
   struct Loc {
     int dh, dw, c;
+    int k, fy; // the K position and the tap's column, for advance()
   };
   __device__ __forceinline__ Loc locate(int k) const {
     const int tap = k / ICg, c = k - tap * ICg;
     const int fx = tap / KW, fy = tap - fx * KW;
-    return Loc{fx * dilH, fy * dilW, c};
+    return Loc{fx * dilH, fy * dilW, c, k, fy};
+  }
+  // The location one K step (64 bytes) further on. With at least 64 channels
+  // per group a step crosses at most one tap boundary, which takes a compare
+  // and a few selects instead of the two integer divisions of locate().
+  __device__ __forceinline__ void advance(Loc &l) const {
+    l.k += 64;
+    if (ICg < 64) {
+      l = locate(l.k);
+      return;
+    }
+    l.c += 64;
+    if (l.c >= ICg) {
+      l.c -= ICg;
+      l.fy += 1;
+      l.dw += dilW;
+      if (l.fy == KW) {
+        l.fy = 0;
+        l.dw = 0;
+        l.dh += dilH;
+      }
+    }
   }
   // address of those bytes for an existing row: inside the image, or a chunk
   // of input-offset bytes for a padding tap

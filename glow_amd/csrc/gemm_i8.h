@@ -195,6 +195,8 @@ struct DenseRows {
     int k;
   };
   __device__ __forceinline__ Loc locate(int k) const { return Loc{k}; }
+  // the location one K step (kBK bytes) further on
+  __device__ __forceinline__ void advance(Loc &l) const { l.k += 64; }
   // address of those bytes in a row that exists
   __device__ __forceinline__ const int8_t *chunk_ptr(const Row &r, const Loc &l) const {
     return r.base + l.k;
@@ -630,7 +632,18 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
   constexpr int H0 = LOADS / 2;
   // `loc` is A.locate() of this lane's chunk of tile nk (one locate serves
   // every row of the tile and both halves of its loads)
-  auto locate_tile = [&](int nk) { return A.locate(min(nk, KT - 1) * kBK + kc_lane); };
+  // Tiles are located in order, one K step at a time (nk never decreases and
+  // grows by at most one between calls; past the end the last tile stays).
+  typename ARows::Loc run_loc = A.locate(kc_lane);
+  int run_tile = 0;
+  auto locate_tile = [&](int nk) {
+    const int t = min(nk, KT - 1);
+    if (t != run_tile) {
+      A.advance(run_loc);
+      run_tile = t;
+    }
+    return run_loc;
+  };
   auto issue_load = [&](int nk, int i, const typename ARows::Loc &loc) {
     const uint32_t slot = lds0 + (uint32_t)(nk % STAGES) * STAGE;
     const int k0 = min(nk, KT - 1) * kBK;
