@@ -243,6 +243,12 @@ CONV_CASES = [
     dict(N=2, H=32, W=32, IC=3, OC=64, kernel=(7, 7), stride=(2, 2), pads=(3, 3, 3, 3)),
     dict(N=1, H=6, W=7, IC=4, OC=8, in_offset=7),
     dict(N=3, H=5, W=5, IC=6, OC=10, group=2, kernel=(5, 5), pads=(2, 2, 2, 2), symmetric=False),
+    # 64 or more channels per group, not a multiple of the 64-byte K step: the
+    # tap location advances across tap and filter-row boundaries mid-step
+    dict(N=1, H=9, W=9, IC=80, OC=32, kernel=(3, 3), dilation=(2, 2), pads=(2, 2, 2, 2)),
+    dict(N=2, H=7, W=6, IC=192, OC=64, group=2, kernel=(2, 3), stride=(1, 2), pads=(1, 1, 0, 1),
+         in_offset=11),
+    dict(N=1, H=8, W=8, IC=48, OC=16, kernel=(3, 2), pads=(1, 0, 1, 1)),   # fewer than 64
 ]
 
 
