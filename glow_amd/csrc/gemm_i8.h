@@ -33,6 +33,8 @@
 #include "common.h"
 #include "requant.h"
 
+#include <atomic>
+
 namespace mi355x {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -798,26 +800,35 @@ template <int BM, int BN, int STAGES> constexpr size_t gemm_dma_lds_bytes() {
 
 // LDS a block may use on the current device (cached per process).
 static size_t lds_limit() {
-  static size_t limit = 0;
-  if (!limit) {
+  static std::atomic<size_t> limit{0};
+  size_t v = limit.load(std::memory_order_relaxed);
+  if (!v) {
     int dev = 0;
     hipDeviceProp_t p;
     if (hipGetDevice(&dev) == hipSuccess &&
         hipGetDeviceProperties(&p, dev) == hipSuccess)
-      limit = p.sharedMemPerBlock;
+      v = p.sharedMemPerBlock;
     else
-      limit = 64 * 1024;
+      v = 64 * 1024;
+    limit.store(v, std::memory_order_relaxed);
   }
-  return limit;
+  return v;
 }
 
+// Kernels that want more than 48 KiB of dynamic LDS have to say so once per
+// device; `done` holds one bit per device (any host thread may get here first,
+// setting the attribute twice is harmless).
 template <class Kern>
-static int set_lds_attr(Kern kern, size_t lds, bool &done) {
-  if (lds > 48 * 1024 && !done) {
+static int set_lds_attr(Kern kern, size_t lds, std::atomic<uint64_t> &done) {
+  if (lds <= 48 * 1024) return MI355X_OK;
+  int dev = 0;
+  MI355X_HIP(hipGetDevice(&dev));
+  const uint64_t bit = 1ull << (dev & 63);
+  if (!(done.load(std::memory_order_acquire) & bit)) {
     MI355X_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                    hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)lds));
-    done = true;
+    done.fetch_or(bit, std::memory_order_release);
   }
   return MI355X_OK;
 }
@@ -835,7 +846,7 @@ static int gemm_launch(const ARows &A, const DenseRows &B, const Epilogue &ep,
   constexpr int THREADS = (BM / WM) * (BN / WN) * 64;
   constexpr size_t lds = gemm_lds_bytes<BM, BN>();
   auto kern = gemm_i8_kernel<BM, BN, WM, WN, true, true, AL_A, AL_B, ARows>;
-  static bool attr_set = false; // per instantiation
+  static std::atomic<uint64_t> attr_set{0}; // per instantiation, one bit per device
   int rc = set_lds_attr(kern, lds, attr_set);
   if (rc != MI355X_OK) return rc;
   const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
@@ -856,7 +867,7 @@ static int gemm_dma_launch(const ARows &A, const DenseRows &B,
   constexpr int THREADS = (BM / WM) * (BN / WN) * 64;
   constexpr size_t lds = gemm_dma_lds_bytes<BM, BN, STAGES>();
   auto kern = gemm_i8_dma_kernel<BM, BN, WM, WN, STAGES, SA, SB, ARows>;
-  static bool attr_set = false; // per instantiation
+  static std::atomic<uint64_t> attr_set{0}; // per instantiation, one bit per device
   int rc = set_lds_attr(kern, lds, attr_set);
   if (rc != MI355X_OK) return rc;
   const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
