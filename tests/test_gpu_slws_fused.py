@@ -215,3 +215,53 @@ def test_many_bags_and_full_size_config():
         capi.slws_set_fused_math(True)
     np.testing.assert_array_equal(strict, want)
     np.testing.assert_allclose(got, strict, rtol=1e-5, atol=1e-4)
+
+
+@pytest.mark.parametrize("kind,cols", [(capi.FUSED_U4_F16, 64), (capi.FUSED_U8_F32, 32),
+                                       (capi.FUSED_U8_F16, 64), (capi.FUSED_U4_F32, 128)])
+def test_short_rows_with_uneven_bags(kind, cols):
+    """Rows of 32 or 64 data bytes put 8 or 4 bags side by side in a wavefront:
+    neighbours with very different lengths (empty, one lookup, several rounds
+    of 32) must not disturb each other, for both index types."""
+    rows = 900
+    rng = np.random.default_rng(kind * 7 + cols)
+    table = cases.random_fused_table(rng, rows, cols, kind)
+    lengths = np.array([0, 1, 33, 0, 70, 2, 0, 0, 32, 31, 100, 0, 5, 64, 65, 1, 0, 3] * 3 + [0, 97],
+                       np.int32)
+    total = int(lengths.sum())
+    f16 = kind in (capi.FUSED_U8_F16, capi.FUSED_U4_F16)
+    for idt in (np.int64, np.int32):
+        idx = rng.integers(0, rows, total).astype(idt)
+        w = rng.random(total).astype(np.float16 if f16 else np.float32)
+        for weights in (w, None):
+            want = go.frwq_slws_generic(table, kind, weights, idx, lengths, f16, False)
+            got = capi.frwq_slws(table, kind, weights, idx, lengths, f16, False)
+            check(got.astype(np.float32), want.astype(np.float32),
+                  bag_magnitude(table, kind, weights, idx, lengths), f16,
+                  what=f"{idt.__name__} weights={'yes' if weights is not None else 'no'}")
+
+
+def test_many_tables_in_one_launch_with_int8_store():
+    """The multi-table launch with the fused ConvertTo + Quantize + InsertTensor
+    store: dense outputs within the fp32 bar of the sequential loop, the int8
+    concatenation within one quantization step of it (a value can land on the
+    other side of a rounding boundary), and nearly everywhere equal."""
+    kind, cols, rows, bags, n = capi.FUSED_U4_F16, 64, 3000, 500, 5
+    rng = np.random.default_rng(77)
+    tables = [cases.random_fused_table(rng, rows, cols, kind) for _ in range(n)]
+    batches = [cases.slws_batch(80 + t, rows, bags, 20, 1.1, np.int64, weighted=False)
+               for t in range(n)]
+    lens = [b[0] for b in batches]
+    idx = [b[1][:int(b[0].sum())] for b in batches]
+    outs = capi.frwq_sls_multi(tables, kind, idx, lens, capi.SLS_OUT_F16)
+    q = capi.frwq_sls_multi(tables, kind, idx, lens, capi.SLS_OUT_I8_VIA_F16, 0.05, -3)
+    assert q.shape == (bags, n * cols)
+    off = 0
+    for t in range(n):
+        want = go.frwq_slws_generic(tables[t], kind, None, idx[t], lens[t], True, False)
+        check(outs[t].astype(np.float32), want.astype(np.float32),
+              bag_magnitude(tables[t], kind, None, idx[t], lens[t]), True, what=f"table {t}")
+        wq = go.quantize_i8(want.astype(np.float32), 0.05, -3)
+        d = np.abs(q[:, off:off + cols].astype(np.int32) - wq.astype(np.int32))
+        assert d.max() <= 1 and (d > 0).mean() < 0.01, (t, d.max(), (d > 0).mean())
+        off += cols
