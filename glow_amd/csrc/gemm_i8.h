@@ -574,10 +574,16 @@ __device__ __forceinline__ uint32_t lds_address(const void *p) {
       (const __attribute__((address_space(3))) void *)p);
 }
 
+// SHORT: the K loop has fewer steps than the ring has slots and the launch
+// provides LDS for those KT slots only, so that more workgroups share a CU
+// (what such a layer needs: it is all load latency and epilogue). Re-reads
+// past the end then go to the last tile's own slot (the same bytes again)
+// instead of slots nobody consumes. Only the 128x128 tile without in-kernel
+// row sums has this variant; it is compiled for four waves per SIMD.
 template <int BM, int BN, int WM, int WN, int STAGES, bool NEED_SA,
-          bool NEED_SB, class ARows>
+          bool NEED_SB, class ARows, bool SHORT = false>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
-                             (BM * BN == 256 * 128) ? 2 : 1) void gemm_i8_dma_kernel(
+                             (BM * BN == 256 * 128) ? 2 : SHORT ? 4 : 1) void gemm_i8_dma_kernel(
     ARows A, DenseRows B, Epilogue ep, int M, int N, int K, int tiles_m,
     int tiles_n, long long b_group_stride, int n_per_group) {
   constexpr int WAVES_N = BN / WN;
@@ -647,7 +653,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
     return run_loc;
   };
   auto issue_load = [&](int nk, int i, const typename ARows::Loc &loc) {
-    const uint32_t slot = lds0 + (uint32_t)(nk % STAGES) * STAGE;
+    const int slot_of = SHORT ? min(nk, KT - 1) : nk % STAGES;
+    const uint32_t slot = lds0 + (uint32_t)slot_of * STAGE;
     const int k0 = min(nk, KT - 1) * kBK;
     if (i < A_LOADS)
       dma16(A.chunk_ptr(arow[i], loc), slot + a_dst[i]);
@@ -756,7 +763,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
   for (int f = 0; f < FRAGS; f++) read_frag(lds, 0, 0, f);
   for (int kt = 0; kt < KT; kt++) {
     const int8_t *cur = lds + (kt % STAGES) * STAGE;
-    const int8_t *nxt = lds + ((kt + 1) % STAGES) * STAGE;
+    // (the fragments read past the end are not used)
+    const int8_t *nxt = lds + (SHORT ? min(kt + 1, KT - 1) : (kt + 1) % STAGES) * STAGE;
     // slice 0 runs while the fragments of slice 1 arrive and the second half
     // of tile kt+STAGES-1 is requested (its slot held tile kt-1, which every
     // wave had read before the previous barrier)
@@ -866,13 +874,27 @@ static int gemm_dma_launch(const ARows &A, const DenseRows &B,
                            hipStream_t st) {
   constexpr int THREADS = (BM / WM) * (BN / WN) * 64;
   constexpr size_t lds = gemm_dma_lds_bytes<BM, BN, STAGES>();
+  const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
+  const long long total = (long long)tiles_m * tiles_n;
+  MI355X_REQUIRE(total < 0x7fffffffLL && g.groups < 65536, "problem too large");
+  if constexpr (BM == 128 && BN == 128 && !SA && !SB) {
+    const int KT = g.K / kBK;
+    if (KT < STAGES) {
+      // KT ring slots (or the epilogue's staging area if that is larger): under
+      // 48 KiB, so no attribute is needed
+      const size_t ring = (size_t)KT * (BM + BN) * kBK;
+      const size_t epi = gemm_epilogue_lds_bytes<BM, BN>();
+      hipLaunchKernelGGL((gemm_i8_dma_kernel<BM, BN, WM, WN, STAGES, SA, SB, ARows, true>),
+                         dim3((unsigned)total, (unsigned)g.groups), dim3(THREADS),
+                         ring > epi ? ring : epi, st, A, B, ep, g.M, g.N, g.K, tiles_m,
+                         tiles_n, g.b_group_stride, g.N);
+      return check_launch("gemm_i8_dma");
+    }
+  }
   auto kern = gemm_i8_dma_kernel<BM, BN, WM, WN, STAGES, SA, SB, ARows>;
   static std::atomic<uint64_t> attr_set{0}; // per instantiation, one bit per device
   int rc = set_lds_attr(kern, lds, attr_set);
   if (rc != MI355X_OK) return rc;
-  const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
-  const long long total = (long long)tiles_m * tiles_n;
-  MI355X_REQUIRE(total < 0x7fffffffLL && g.groups < 65536, "problem too large");
   hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)g.groups),
                      dim3(THREADS), lds, st, A, B, ep, g.M, g.N, g.K, tiles_m,
                      tiles_n, g.b_group_stride, g.N);
