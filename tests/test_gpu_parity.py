@@ -515,6 +515,28 @@ def test_rescale_both_multiplier_paths():
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("tile", list(range(6)))
+@pytest.mark.parametrize("K", [64, 128, 192])
+def test_short_k_loops_on_every_tile(tile, K):
+    """K loops of one, two and three steps (shorter than, or as long as, the
+    ring of load stages), symmetric weights with precomputed row sums: the
+    128x128 tile has a variant of its own for these."""
+    c = cases.rwq_fc_case(90 + tile + K, 390, K, 260, symmetric=True)
+    cc = cases.cwq_conv_case(95 + tile + K, 2, 14, 14, K, 160, kernel=(1, 1), pads=(0, 0, 0, 0),
+                             in_offset=-128)
+    want_fc = go.rwq_fc_i8(*cases.rwq_fc_args(c))
+    want_cv = go.cwq_conv2d_i8(*cases.cwq_conv_args(cc))
+    capi.check(capi.lib().mi355x_gemm_tile_override(tile))
+    try:
+        got_fc = capi.rwq_fc_i8(*cases.rwq_fc_args(c))
+        got_cv = capi.cwq_conv2d_i8(*cases.cwq_conv_args(cc))
+    finally:
+        capi.check(capi.lib().mi355x_gemm_tile_override(-1))
+    np.testing.assert_array_equal(got_fc, want_fc)
+    np.testing.assert_array_equal(got_cv, want_cv)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tile", list(range(6)))
 def test_every_gemm_tile_gives_the_same_result(tile):
     """Results do not depend on the workgroup tile."""
     c = cases.rwq_fc_case(60 + tile, 700, 192, 330, symmetric=False)
