@@ -190,7 +190,8 @@ __global__ __launch_bounds__(kGlueThreads) void avg_pool_i8_kernel(
 #pragma unroll
   for (int i = 0; i < VEC; i++) s[i] = 0;
   for (int fh = 0; fh < hl; fh++)
-    for (int fw = 0; fw < wl; fw++) {
+#pragma unroll 8
+    for (int fw = 0; fw < wl; fw++) { // unrolled: several taps' loads in flight
       const int8_t *p = in + (((long long)n * g.IH + (ih_min + h0 + fh)) * g.IW +
                               (iw_min + w0 + fw)) * g.C + c0;
       if constexpr (VEC == 4) {
