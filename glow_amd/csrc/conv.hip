@@ -129,10 +129,8 @@ static int conv_common(int8_t *out, const int8_t *in, const int8_t *filter,
   const int ICg = g->IC / g->group, OCg = g->OC / g->group;
   const long long K = (long long)g->KH * g->KW * ICg;
   MI355X_REQUIRE(M < (1LL << 30) && K < (1LL << 30), "convolution too large");
-  // the last tap of the last output pixel must start inside pad + image
-  MI355X_REQUIRE((long long)(g->OH - 1) * g->strideH - g->padT < g->IH &&
-                     (long long)(g->OW - 1) * g->strideW - g->padL < g->IW,
-                 "output size inconsistent with input size, stride and pads");
+  // (OH, OW carry the bottom and right padding: an output pixel whose window
+  // lies wholly in the padding is legal and sees the input offset everywhere)
   MI355X_REQUIRE(ep.a_off >= -128 && ep.a_off <= 127,
                  "input offset %d outside the int8 range", ep.a_off);
   MI355X_REQUIRE(ep.act == MI355X_ACT_NONE || ep.act == MI355X_ACT_RELU ||
