@@ -265,3 +265,40 @@ def test_many_tables_in_one_launch_with_int8_store():
         d = np.abs(q[:, off:off + cols].astype(np.int32) - wq.astype(np.int32))
         assert d.max() <= 1 and (d > 0).mean() < 0.01, (t, d.max(), (d > 0).mean())
         off += cols
+
+
+import os  # noqa: E402
+
+_MORE = max(1, int(os.environ.get("MI355X_TEST_SEEDS", "1")))
+
+
+@pytest.mark.parametrize("seed", range(40 * _MORE))
+def test_random_tables_and_batches(seed):
+    """Seeded random kinds, row widths (those the fused kernels take and some
+    they do not), table sizes, bag-length distributions, index and weight
+    types, lengths and offsets mode."""
+    rng = np.random.default_rng(9000 + seed)
+    kind = int(rng.integers(0, 4))
+    is4 = kind in (capi.FUSED_U4_F16, capi.FUSED_U4_F32)
+    data_bytes = int(rng.choice([32, 64, 128, 256, 256, 128, 20, 96]))
+    cols = data_bytes * (2 if is4 else 1)
+    rows, bags = int(rng.integers(1, 3000)), int(rng.integers(1, 400))
+    table = cases.random_fused_table(rng, rows, cols, kind)
+    mean = float(rng.choice([0.3, 2, 20, 45, 90]))
+    lengths, idx, w = cases.slws_batch(seed, rows, bags, mean, 1.05,
+                                       rng.choice([np.int64, np.int32]))
+    total = int(lengths.sum())
+    idx, w = idx[:total], w[:total]
+    f16 = kind in (capi.FUSED_U8_F16, capi.FUSED_U4_F16)
+    out16 = f16 and bool(rng.integers(0, 2))
+    weights = None if rng.random() < 0.3 else (w.astype(np.float16) if out16 else w)
+    say("random", kind, cols, rows, bags, total, out16)
+    want = go.frwq_slws_generic(table, kind, weights, idx, lengths, out16, False)
+    mag = bag_magnitude(table, kind, weights, idx, lengths)
+    got = capi.frwq_slws(table, kind, weights, idx, lengths, out16, False)
+    check(got.astype(np.float32), want.astype(np.float32), mag, out16, what="lengths")
+    if idx.dtype == np.int32:
+        offs = np.r_[0, np.cumsum(lengths)].astype(np.int32)
+        ww = weights if weights is not None else np.ones(total, np.float16 if out16 else np.float32)
+        got = capi.embedding_bag_rowwise_offsets(table, kind, ww, idx, offs, True, out16, False)
+        check(got.astype(np.float32), want.astype(np.float32), mag, out16, what="offsets")
