@@ -114,8 +114,31 @@ __device__ __forceinline__ void pool_window(int in_min, int in_size, int k, int 
   len = max(0, hi - lo);
 }
 
+// Walks the valid taps of a pooling window in row-major order without a
+// division per tap and without branches (selects only, so that the loads of a
+// group stay in one basic block). `off` is the tap's element offset from the
+// window's first tap; past the last tap it stays on the last one.
+struct TapWalk {
+  long long off;
+  int fw, wl, left;
+  long long col_step, row_step;
+  __device__ __forceinline__ TapWalk(int hl, int wl_, int iw, int c)
+      : off(0), fw(0), wl(wl_), left(hl * wl_), col_step(c),
+        row_step((long long)(iw - wl_ + 1) * c) {}
+  __device__ __forceinline__ void step() {
+    const bool adv = left > 1;
+    const bool wrap = fw + 1 == wl;
+    off += adv ? (wrap ? row_step : col_step) : 0;
+    fw = adv ? (wrap ? 0 : fw + 1) : fw;
+    --left;
+  }
+};
+
 // One thread per output pixel and group of VEC channels (VEC bytes per load).
-template <int VEC>
+// The taps are read U at a time, all loads of a group issued before the first
+// is used; a group's slots beyond the window re-read its last tap, which a
+// maximum does not see.
+template <int VEC, int U>
 __global__ __launch_bounds__(kGlueThreads) void max_pool_i8_kernel(
     int8_t *__restrict__ out, const int8_t *__restrict__ in, PoolGeom g,
     int32_t out_offset, long long total) {
@@ -132,23 +155,40 @@ __global__ __launch_bounds__(kGlueThreads) void max_pool_i8_kernel(
   const int ih_min = oh * g.SH - g.padT, iw_min = ow * g.SW - g.padL;
   pool_window(ih_min, g.IH, g.KH, h0, hl);
   pool_window(iw_min, g.IW, g.KW, w0, wl);
+  const bool empty = hl == 0 || wl == 0;
   int32_t m[VEC];
 #pragma unroll
   for (int i = 0; i < VEC; i++) m[i] = -128;
-  for (int fh = 0; fh < hl; fh++)
-    for (int fw = 0; fw < wl; fw++) {
-      const int8_t *p = in + (((long long)n * g.IH + (ih_min + h0 + fh)) * g.IW +
-                              (iw_min + w0 + fw)) * g.C + c0;
+  if (!empty) {
+    const int8_t *base =
+        in + (((long long)n * g.IH + (ih_min + h0)) * g.IW + (iw_min + w0)) * g.C + c0;
+    TapWalk tw(hl, wl, g.IW, g.C);
+    while (tw.left > 0) {
       if constexpr (VEC == 16) {
-        const uint4 v = *reinterpret_cast<const uint4 *>(p);
-        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        uint4 v[U];
 #pragma unroll
-        for (int i = 0; i < 16; i++) m[i] = max(m[i], sx8(w[i >> 2], i & 3));
+        for (int u = 0; u < U; u++) {
+          v[u] = *reinterpret_cast<const uint4 *>(base + tw.off);
+          tw.step();
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+          const uint32_t w[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+          for (int i = 0; i < 16; i++) m[i] = max(m[i], sx8(w[i >> 2], i & 3));
+        }
       } else {
-        m[0] = max(m[0], (int32_t)p[0]);
+        int32_t v[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+          v[u] = base[tw.off];
+          tw.step();
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) m[0] = max(m[0], v[u]);
       }
     }
-  const bool empty = hl == 0 || wl == 0;
+  }
   int8_t *q = out + (((long long)n * g.OH + oh) * g.OW + ow) * g.C + c0;
   if constexpr (VEC == 16) {
     uint32_t o[4];
@@ -168,7 +208,9 @@ __device__ __forceinline__ int32_t div_round_i32(int32_t v, int32_t d) {
   return v > 0 ? (v + rnd) / d : (v - rnd) / d;
 }
 
-template <int VEC>
+// Taps are read U at a time like the maximum's; here the slots beyond the
+// window are left out of the sum.
+template <int VEC, int U>
 __global__ __launch_bounds__(kGlueThreads) void avg_pool_i8_kernel(
     int8_t *__restrict__ out, const int8_t *__restrict__ in, PoolGeom g,
     int count_include_pads, int32_t out_offset, int32_t in_offset, int32_t pre,
@@ -189,19 +231,37 @@ __global__ __launch_bounds__(kGlueThreads) void avg_pool_i8_kernel(
   int32_t s[VEC];
 #pragma unroll
   for (int i = 0; i < VEC; i++) s[i] = 0;
-  for (int fh = 0; fh < hl; fh++)
-#pragma unroll 8
-    for (int fw = 0; fw < wl; fw++) { // unrolled: several taps' loads in flight
-      const int8_t *p = in + (((long long)n * g.IH + (ih_min + h0 + fh)) * g.IW +
-                              (iw_min + w0 + fw)) * g.C + c0;
+  if (hl > 0 && wl > 0) {
+    const int8_t *base =
+        in + (((long long)n * g.IH + (ih_min + h0)) * g.IW + (iw_min + w0)) * g.C + c0;
+    TapWalk tw(hl, wl, g.IW, g.C);
+    while (tw.left > 0) {
+      const int live = tw.left;
       if constexpr (VEC == 4) {
-        const uint32_t w = *reinterpret_cast<const uint32_t *>(p);
+        uint32_t v[U];
 #pragma unroll
-        for (int i = 0; i < 4; i++) s[i] += sx8(w, i) - in_offset;
+        for (int u = 0; u < U; u++) {
+          v[u] = *reinterpret_cast<const uint32_t *>(base + tw.off);
+          tw.step();
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+          const bool keep = u < live;
+#pragma unroll
+          for (int i = 0; i < 4; i++) s[i] += keep ? sx8(v[u], i) - in_offset : 0;
+        }
       } else {
-        s[0] += (int32_t)p[0] - in_offset;
+        int32_t v[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+          v[u] = base[tw.off];
+          tw.step();
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) s[0] += u < live ? v[u] - in_offset : 0;
       }
     }
+  }
   const int32_t area = hl * wl;
   int32_t r[VEC];
 #pragma unroll
@@ -419,6 +479,38 @@ __global__ __launch_bounds__(kGlueThreads) void space_to_depth2_i8_kernel(
   for (int c = 4 * C; c < Cout; c++) d[c] = (int8_t)fill;
 }
 
+// The same for 16 output channels (the 3-channel image stem): the 16 bytes of a
+// block are put together in registers and leave in one store.
+template <int C>
+__global__ __launch_bounds__(kGlueThreads) void space_to_depth2_c16_i8_kernel(
+    uint4 *__restrict__ dst, const int8_t *__restrict__ src, int N, int IH, int IW, int padT,
+    int padL, int BH, int BW, int fill, long long total) {
+  const long long t = (long long)blockIdx.x * kGlueThreads + threadIdx.x;
+  if (t >= total) return;
+  const int bw = (int)(t % BW);
+  long long r = t / BW;
+  const int bh = (int)(r % BH);
+  const int n = (int)(r / BH);
+  uint8_t b[16];
+#pragma unroll
+  for (int i = 0; i < 16; i++) b[i] = (uint8_t)fill;
+#pragma unroll
+  for (int q = 0; q < 4; q++) {
+    const int ih = 2 * bh + (q >> 1) - padT, iw = 2 * bw + (q & 1) - padL;
+    if (ih >= 0 && ih < IH && iw >= 0 && iw < IW) {
+      const int8_t *p = src + (((long long)n * IH + ih) * IW + iw) * C;
+#pragma unroll
+      for (int c = 0; c < C; c++) b[q * C + c] = (uint8_t)p[c];
+    }
+  }
+  uint32_t w[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++)
+    w[j] = (uint32_t)b[4 * j] | ((uint32_t)b[4 * j + 1] << 8) | ((uint32_t)b[4 * j + 2] << 16) |
+           ((uint32_t)b[4 * j + 3] << 24);
+  dst[t] = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
 // libjit_sigmoid_kernel_f: 1 / (expf(-x) + 1)
 __global__ __launch_bounds__(kGlueThreads) void sigmoid_f32_kernel(
     float *__restrict__ dst, const float *__restrict__ src, size_t n) {
@@ -544,12 +636,21 @@ int mi355x_max_pool_i8(int8_t *out, const int8_t *in, size_t N, size_t IH, size_
   const bool vec = (C % 16 == 0) && al16(out, in, in);
   const long long total = (long long)N * OH * OW * (vec ? C / 16 : C);
   MI355X_REQUIRE(total / kGlueThreads < 0x7fffffffLL, "tensor too large");
-  if (vec)
-    hipLaunchKernelGGL(max_pool_i8_kernel<16>, dim3(glue_blocks((size_t)total)),
-                       dim3(kGlueThreads), 0, as_stream(stream), out, in, g, out_offset, total);
-  else
-    hipLaunchKernelGGL(max_pool_i8_kernel<1>, dim3(glue_blocks((size_t)total)),
-                       dim3(kGlueThreads), 0, as_stream(stream), out, in, g, out_offset, total);
+  // taps read per group: the whole window when it has at most 9 taps
+  const bool small = kH * kW <= 4, mid = kH * kW <= 9;
+#define MI355X_MAX_POOL(VEC, U)                                                              \
+  hipLaunchKernelGGL((max_pool_i8_kernel<VEC, U>), dim3(glue_blocks((size_t)total)),          \
+                     dim3(kGlueThreads), 0, as_stream(stream), out, in, g, out_offset, total)
+  if (vec) {
+    if (small) MI355X_MAX_POOL(16, 4);
+    else if (mid) MI355X_MAX_POOL(16, 9);
+    else MI355X_MAX_POOL(16, 8);
+  } else {
+    if (small) MI355X_MAX_POOL(1, 4);
+    else if (mid) MI355X_MAX_POOL(1, 9);
+    else MI355X_MAX_POOL(1, 8);
+  }
+#undef MI355X_MAX_POOL
   return check_launch("max_pool_i8");
 }
 
@@ -567,14 +668,21 @@ int mi355x_avg_pool_i8(int8_t *out, const int8_t *in, size_t N, size_t IH, size_
   const bool vec = (C % 4 == 0) && ((((uintptr_t)out | (uintptr_t)in) & 3) == 0);
   const long long total = (long long)N * OH * OW * (vec ? C / 4 : C);
   MI355X_REQUIRE(total / kGlueThreads < 0x7fffffffLL, "tensor too large");
-  if (vec)
-    hipLaunchKernelGGL(avg_pool_i8_kernel<4>, dim3(glue_blocks((size_t)total)),
-                       dim3(kGlueThreads), 0, as_stream(stream), out, in, g, count_include_pads,
-                       out_offset, in_offset, out_pre, out_post, out_scale, total);
-  else
-    hipLaunchKernelGGL(avg_pool_i8_kernel<1>, dim3(glue_blocks((size_t)total)),
-                       dim3(kGlueThreads), 0, as_stream(stream), out, in, g, count_include_pads,
-                       out_offset, in_offset, out_pre, out_post, out_scale, total);
+  const bool small = kH * kW <= 4, mid = kH * kW <= 9;
+#define MI355X_AVG_POOL(VEC, U)                                                              \
+  hipLaunchKernelGGL((avg_pool_i8_kernel<VEC, U>), dim3(glue_blocks((size_t)total)),          \
+                     dim3(kGlueThreads), 0, as_stream(stream), out, in, g, count_include_pads, \
+                     out_offset, in_offset, out_pre, out_post, out_scale, total)
+  if (vec) {
+    if (small) MI355X_AVG_POOL(4, 4);
+    else if (mid) MI355X_AVG_POOL(4, 9);
+    else MI355X_AVG_POOL(4, 16);
+  } else {
+    if (small) MI355X_AVG_POOL(1, 4);
+    else if (mid) MI355X_AVG_POOL(1, 9);
+    else MI355X_AVG_POOL(1, 16);
+  }
+#undef MI355X_AVG_POOL
   return check_launch("avg_pool_i8");
 }
 
@@ -687,6 +795,13 @@ int mi355x_space_to_depth2_i8(int8_t *dst, const int8_t *src, size_t N, size_t I
   MI355X_REQUIRE(fill >= -128 && fill <= 127, "fill outside the int8 range");
   const long long total = (long long)N * BH * BW;
   MI355X_REQUIRE(total / kGlueThreads < 0x7fffffffLL, "tensor too large");
+  if (Cout == 16 && (C == 3 || C == 4) && (((uintptr_t)dst) & 15) == 0) {
+    auto kern = C == 3 ? space_to_depth2_c16_i8_kernel<3> : space_to_depth2_c16_i8_kernel<4>;
+    hipLaunchKernelGGL(kern, dim3(glue_blocks((size_t)total)), dim3(kGlueThreads), 0,
+                       as_stream(stream), (uint4 *)dst, src, (int)N, (int)IH, (int)IW, (int)padT,
+                       (int)padL, (int)BH, (int)BW, fill, total);
+    return check_launch("space_to_depth2_i8");
+  }
   hipLaunchKernelGGL(space_to_depth2_i8_kernel, dim3(glue_blocks((size_t)total)),
                      dim3(kGlueThreads), 0, as_stream(stream), dst, src, (int)N, (int)IH, (int)IW,
                      (int)C, (int)padT, (int)padL, (int)BH, (int)BW, (int)Cout, fill, total);

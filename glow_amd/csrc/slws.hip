@@ -626,6 +626,8 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_wave_kernel(SlwsArgs a) {
 // LPR = data_bytes/4 lanes and one load instruction fetches 64/LPR rows. The
 // partial sums of the row groups are added across lanes at the end of the bag.
 typedef uint32_t __attribute__((address_space(1))) global_u32;
+typedef int32_t __attribute__((address_space(1))) global_i32;
+typedef long long __attribute__((address_space(1))) global_i64;
 
 template <bool IS4, bool SO16, int LPR, bool OFF32>
 __global__ __launch_bounds__(kSlwsThreads) void slws_rows_kernel(SlwsArgs a) {
@@ -664,13 +666,16 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_rows_kernel(SlwsArgs a) {
   for (int base = 0; base < len; base += kBatch) {
     const int cnt = min(kBatch, len - base);
     // round 1: lane j fetches lookup j of the batch
+    uint32_t so_lo = 0, so_hi = 0;
+    float my_w;
+    bool my_valid;
     {
       const long long pos = start + base + lane;
       long long row = -1;
       float w = 0.0f;
       if (lane < cnt && pos < a.num_indices) {
-        row = a.idx64 ? reinterpret_cast<const long long *>(a.indices)[pos]
-                      : (long long)reinterpret_cast<const int *>(a.indices)[pos];
+        row = a.idx64 ? ((const global_i64 *)a.indices)[pos]
+                      : (long long)((const global_i32 *)a.indices)[pos];
         if (!a.weights) {
           w = 1.0f;
         } else if (a.w16) {
@@ -680,27 +685,26 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_rows_kernel(SlwsArgs a) {
         }
       }
       // a skipped lookup reads row 0 and contributes exactly +0
-      const bool valid = row >= 0 && row < a.data_rows;
-      if (!valid) row = 0;
-      float s, o;
+      my_valid = row >= 0 && row < a.data_rows;
+      if (!my_valid) row = 0;
+      my_w = w;
+      // The row's scale and offset are requested here and consumed only after
+      // the row reads below have been issued, so that the two round trips that
+      // depend on the index (scale/offset, row bytes) overlap.
+      // (Loads through global-address pointers: a generic-address load also
+      // counts as an LDS operation, and the wait for the keys below would then
+      // wait for it.)
       if (!SO16 && a.sep_scales) {
-        s = a.sep_scales[row];
-        o = a.sep_offsets[row];
+        so_lo = ((const global_u32 *)a.sep_scales)[row];
+        so_hi = ((const global_u32 *)a.sep_offsets)[row];
       } else {
         // rows and their data bytes are multiples of 4 bytes here
-        const uint32_t *so = reinterpret_cast<const uint32_t *>(
-            a.data + row * a.in_line + a.data_bytes);
-        if constexpr (SO16) {
-          const uint32_t v = so[0];
-          s = __half2float(__ushort_as_half((unsigned short)(v & 0xffff)));
-          o = __half2float(__ushort_as_half((unsigned short)(v >> 16)));
-        } else {
-          s = __uint_as_float(so[0]);
-          o = __uint_as_float(so[1]);
-        }
+        const global_u32 *so = (const global_u32 *)((const global_u8 *)a.data +
+                                                    (row * a.in_line + a.data_bytes));
+        so_lo = so[0];
+        if constexpr (!SO16) so_hi = so[1];
       }
       keys[lane] = OFF32 ? (uint32_t)(row * a.in_line) : (uint32_t)row;
-      wso[lane] = valid ? make_float2(w * s, w * o) : make_float2(0.0f, 0.0f);
     }
     wave_lds_sync();
     // round 2: all row reads of the batch in flight before the first use, taken
@@ -723,6 +727,18 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_rows_kernel(SlwsArgs a) {
         }
       }
     }
+    {
+      float sc, of;
+      if constexpr (SO16) {
+        sc = __half2float(__ushort_as_half((unsigned short)(so_lo & 0xffff)));
+        of = __half2float(__ushort_as_half((unsigned short)(so_lo >> 16)));
+      } else {
+        sc = __uint_as_float(so_lo);
+        of = __uint_as_float(so_hi);
+      }
+      wso[lane] = my_valid ? make_float2(my_w * sc, my_w * of) : make_float2(0.0f, 0.0f);
+    }
+    wave_lds_sync();
 #pragma unroll
     for (int c = 0; c < kLoads / kChunk; c++) {
       if (c * kChunk * RPI < cnt) {
