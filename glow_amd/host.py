@@ -194,6 +194,11 @@ def parse_listing(text):
 
 
 class DeviceManager:
+    """use_launch_graphs: False = kernel by kernel; True = launch graphs with
+    the default number of parallel branches; n > 1 = up to n branches (the first
+    nine requests of a function compare its recordings with all branches, one
+    chain and two branches; the fastest stays); -n = exactly n branches."""
+
     def __init__(self, device=0, memory_bytes=0, use_launch_graphs=True):
         self._h = C.c_void_p(lib().mi355x_host_dm_create(
             device, C.c_uint64(memory_bytes), int(use_launch_graphs)))

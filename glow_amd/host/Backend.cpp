@@ -1442,15 +1442,40 @@ Error MI355XFunction::captureGraph(const DeviceBindings &b, const std::vector<vo
   for (size_t i = 0; i < n; i++)
     for (size_t j = 0; j < i; j++)
       if (launchesConflict(launches[j], launches[i])) preds[i].push_back(j);
+  // Lanes. A launch hands its lane to the successor with the longest chain of
+  // launches still behind it, so the critical path runs down one stream and
+  // only the shorter branches pay for an event wait.
+  std::vector<int> height(n, 1), depth(n, 1);
+  std::vector<long long> heir(n, -1);
+  for (size_t i = n; i-- > 0;)
+    for (size_t p : preds[i])
+      if (height[i] + 1 > height[p]) height[p] = height[i] + 1;
+  for (size_t i = 0; i < n; i++)
+    for (size_t p : preds[i]) {
+      if (depth[p] + 1 > depth[i]) depth[i] = depth[p] + 1;
+      if (heir[p] < 0 || height[i] > height[(size_t)heir[p]]) heir[p] = (long long)i;
+    }
   std::vector<int> lane(n, 0);
   std::vector<long long> last(nLanes, -1);    // last launch put on each lane
   for (size_t i = 0; i < n; i++) {
     int pick = -1;
-    for (auto it = preds[i].rbegin(); it != preds[i].rend() && pick < 0; ++it)
-      if (last[(size_t)lane[*it]] == (long long)*it) pick = lane[*it]; // continue a chain
+    // the heir continues; the heir of several launches follows the deepest
+    long long from = -1;
+    for (size_t p : preds[i])
+      if (heir[p] == (long long)i && (from < 0 || depth[p] >= depth[(size_t)from])) from = (long long)p;
+    if (from >= 0) pick = lane[(size_t)from];
     if (pick < 0)
       for (size_t l = 0; l < nLanes && pick < 0; l++)
         if (last[l] < 0) pick = (int)l;                                  // an unused lane
+    // lanes whose last launch still waits for its heir are kept for it
+    auto kept = [&](size_t l) { return heir[(size_t)last[l]] > (long long)i; };
+    if (pick < 0)
+      for (auto it = preds[i].rbegin(); it != preds[i].rend() && pick < 0; ++it)
+        if (last[(size_t)lane[*it]] == (long long)*it && !kept((size_t)lane[*it]))
+          pick = lane[*it];                                              // behind a predecessor
+    if (pick < 0)
+      for (size_t l = 0; l < nLanes; l++)                                // idle longest
+        if (!kept(l) && (pick < 0 || last[l] < last[(size_t)pick])) pick = (int)l;
     if (pick < 0) pick = preds[i].empty() ? 0 : lane[preds[i].back()];
     lane[i] = pick;
     last[(size_t)pick] = (long long)i;

@@ -201,11 +201,13 @@ Expected<float> MI355XDeviceManager::timeFunction(const std::string &functionNam
     void *e0 = nullptr, *e1 = nullptr;
     Error err;
     float ms = 0.0f;
+    // the comparison of recordings, if still going on, finishes untimed
+    while (!fr.branchesTuned && !err) err = executeTuned(fr, &ctx);
     int rc = mi355x_event_create(&e0);
     if (rc == MI355X_OK) rc = mi355x_event_create(&e1);
     if (rc == MI355X_OK) rc = mi355x_stream_sync(stream_);
     if (rc == MI355X_OK) rc = mi355x_event_record(e0, stream_);
-    if (rc != MI355X_OK) err = fromStatus(rc, "timing set-up");
+    if (rc != MI355X_OK && !err) err = fromStatus(rc, "timing set-up");
     for (int i = 0; i < iterations && !err; i++) err = fr.fn->execute(&ctx);
     if (!err) {
       rc = mi355x_event_record(e1, stream_);
@@ -320,8 +322,75 @@ Error MI355XDeviceManager::makeResident(const Module *module, const std::string 
     }
     Error e = fn->captureGraph(fr.bindings, sideStreams_);
     if (e) return failWith(std::move(e));
+    const int all = (int)sideStreams_.size() + 1;
+    if (config_.autotuneBranches && all > 1) {
+      fr.branchCandidates = {all, 1};
+      if (all > 2) fr.branchCandidates.push_back(2);
+      fr.branchesTuned = false;
+    }
   }
   functions_.emplace(name, fr);
+  return Error::success();
+}
+
+Error MI355XDeviceManager::captureWithBranches(FunctionResident &fr, int branches) {
+  std::vector<void *> side(sideStreams_.begin(),
+                           sideStreams_.begin() + std::min<size_t>(sideStreams_.size(),
+                                                                   (size_t)std::max(0, branches - 1)));
+  return fr.fn->captureGraph(fr.bindings, side);
+}
+
+// Runs one request. While the recordings of a function are still being
+// compared it also re-records and times as the phase says; every request
+// computes the same results whichever recording replays it.
+Error MI355XDeviceManager::executeTuned(FunctionResident &fr, ExecutionContext *ctx) {
+  if (fr.branchesTuned) return fr.fn->execute(ctx);
+  constexpr int kPerCandidate = 3;       // one warm-up and two timed requests
+  const size_t cand = (size_t)(fr.branchPhase / kPerCandidate);
+  const bool timed = fr.branchPhase % kPerCandidate != 0;
+  Error err;
+  if (!timed) {
+    // candidate 0 is the recording made at load time
+    if (cand > 0) err = captureWithBranches(fr, fr.branchCandidates[cand]);
+    if (!err) err = fr.fn->execute(ctx);
+  } else {
+    void *e0 = nullptr, *e1 = nullptr;
+    float ms = 0.0f;
+    int rc = mi355x_event_create(&e0);
+    if (rc == MI355X_OK) rc = mi355x_event_create(&e1);
+    if (rc == MI355X_OK) rc = mi355x_stream_sync(stream_);
+    if (rc == MI355X_OK) rc = mi355x_event_record(e0, stream_);
+    if (rc == MI355X_OK) {
+      err = fr.fn->execute(ctx);
+      if (!err) {
+        rc = mi355x_event_record(e1, stream_);
+        if (rc == MI355X_OK) rc = mi355x_event_sync(e1);
+        if (rc == MI355X_OK) rc = mi355x_event_elapsed_ms(e0, e1, &ms);
+      }
+    }
+    if (e0) mi355x_event_destroy(e0);
+    if (e1) mi355x_event_destroy(e1);
+    if (!err && rc != MI355X_OK) err = fromStatus(rc, "branch timing");
+    if (!err) {
+      if (fr.branchMs.size() <= cand) fr.branchMs.push_back(ms);
+      else fr.branchMs[cand] = std::min(fr.branchMs[cand], ms);
+    }
+  }
+  if (err) {
+    // fall back to the recording with all branches and stop comparing
+    fr.branchesTuned = true;
+    Error again = captureWithBranches(fr, fr.branchCandidates[0]);
+    (void)again;
+    return err;
+  }
+  if (++fr.branchPhase == kPerCandidate * (int)fr.branchCandidates.size()) {
+    size_t best = 0;
+    for (size_t i = 1; i < fr.branchMs.size(); i++)
+      if (fr.branchMs[i] < fr.branchMs[best]) best = i;
+    fr.branchesTuned = true;
+    if (best + 1 != fr.branchCandidates.size())
+      return captureWithBranches(fr, fr.branchCandidates[best]);
+  }
   return Error::success();
 }
 
@@ -458,7 +527,7 @@ void MI355XDeviceManager::runFunctionImpl(RunIdentifierTy id, std::string functi
   }
   if (!err) {
     ctx->setDeviceBindings(std::unique_ptr<DeviceBindings>(new DeviceBindings(fr.bindings)));
-    err = fr.fn->execute(ctx.get());
+    err = executeTuned(fr, ctx.get());
   }
   if (!err) {
     for (const auto &kv : pb->pairs()) {

@@ -34,6 +34,12 @@ struct DeviceConfig {
   bool useLaunchGraphs = true; // record each function once, replay per run
   int graphBranches = 4;       // independent launches recorded side by side (1 = a chain)
   bool autotuneTiles = true;   // time the tile candidates of each matrix-core launch at load
+  // The first requests of a function replay it recorded with all branches, as
+  // one chain and with two branches (a warm-up and two timed requests each); the
+  // fastest recording serves the requests after them. Waiting for another
+  // stream costs microseconds, so short side branches can lose more than they
+  // overlap, and how long a launch runs depends on the request's data.
+  bool autotuneBranches = true;
 };
 
 struct DeviceInfo {
@@ -85,6 +91,11 @@ private:
     mi355x_arena *arena = nullptr; // generated constants + activations
     uint64_t bytes = 0;
     DeviceBindings bindings;
+    // branch tuning: requests 3c, 3c+1, 3c+2 go to candidate c (warm-up, timed, timed)
+    std::vector<int> branchCandidates;
+    std::vector<float> branchMs;
+    int branchPhase = 0;
+    bool branchesTuned = true;
   };
 
   void addNetworkImpl(const Module *module, FunctionMapTy functions, ReadyCBTy readyCB);
@@ -93,6 +104,8 @@ private:
                        std::unique_ptr<ExecutionContext> ctx, ResultCBTy resultCB);
   Error makeResident(const Module *module, const std::string &name, MI355XFunction *fn);
   Error tuneTiles(MI355XFunction *fn, const DeviceBindings &b);
+  Error captureWithBranches(FunctionResident &fr, int branches);
+  Error executeTuned(FunctionResident &fr, ExecutionContext *ctx);
   void release(FunctionResident &fr);
   void enqueue(std::function<void()> work);
   void workerLoop();

@@ -160,6 +160,10 @@ mi355x_host_dm *mi355x_host_dm_create(int device, uint64_t memory_bytes, int gra
   c.deviceMemory = memory_bytes;
   c.useLaunchGraphs = graphs != 0;
   if (graphs > 1) c.graphBranches = graphs; // 1 keeps the default
+  if (graphs < 0) {
+    c.graphBranches = -graphs;
+    c.autotuneBranches = false;
+  }
   return new mi355x_host_dm(c);
 }
 void mi355x_host_dm_destroy(mi355x_host_dm *dm) { delete dm; }

@@ -131,8 +131,10 @@ int mi355x_host_bundle_sizes(mi355x_host_module *m, int function, uint64_t out[4
 /* DeviceManager. memory_bytes 0 = what the device reports free.
  * use_launch_graphs: 0 = launch kernel by kernel; 1 = record each function as a
  * launch graph whose independent launches form parallel branches (default
- * width); n > 1 = the same with up to n branches (n = 2 ... ; a chain needs
- * the C++ DeviceConfig). */
+ * width); n > 1 = the same with up to n branches. For n >= 1 the first nine
+ * requests of a function compare its recordings with all branches, as one
+ * chain and with two branches, and the fastest serves the requests after
+ * them. n < 0 = exactly -n branches (-1 = a chain), nothing compared. */
 mi355x_host_dm *mi355x_host_dm_create(int device, uint64_t memory_bytes, int use_launch_graphs);
 void mi355x_host_dm_destroy(mi355x_host_dm *dm);
 int mi355x_host_dm_init(mi355x_host_dm *dm);

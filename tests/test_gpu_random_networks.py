@@ -74,3 +74,30 @@ def test_random_ranking_net(seed):
         np.testing.assert_allclose(prob, want["prob"], rtol=1e-5, atol=1e-30)
     finally:
         dm.stop()
+
+
+@pytest.mark.parametrize("graphs", [1, 2, -1, -3])
+def test_every_recording_of_a_function_gives_the_same_results(graphs):
+    """The first nine requests of a function go to its three recordings (all
+    branches, one chain, two branches) in turn and later ones to the fastest:
+    each request, with its own inputs, must match the oracle. Negative values
+    fix the number of branches."""
+    tables, dim, batch, rows, dense = 3, 32, 64, 500, 13
+    net, max_idx = dlrm.make(tables=tables, rows=rows, dim=dim, batch=batch, mean_len=6.0,
+                             dense_features=dense, bottom=(64, dim), top=(32, 1), seed=5)
+    m, f = netlib.to_module(net)
+    m.compile(f)
+    dm = H.DeviceManager(use_launch_graphs=graphs).init()
+    try:
+        dm.add_network(m)
+        for request in range(12):
+            inp = dlrm.Inputs(400 + request, tables, rows, batch, 6.0, 1.1, dense)
+            b = dlrm.bindings(net, inp, max_idx)
+            logit = np.zeros((batch, 1), np.int8)
+            prob = np.zeros((batch, 1), np.float32)
+            dm.run("main", dict(b, logit_q=logit, prob=prob))
+            want = oracle_exec.run(net, b)
+            np.testing.assert_array_equal(logit, want["logit_q"], err_msg=f"request {request}")
+            np.testing.assert_allclose(prob, want["prob"], rtol=1e-5, atol=1e-30)
+    finally:
+        dm.stop()
