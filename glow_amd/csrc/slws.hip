@@ -824,6 +824,11 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_groups_kernel(SlwsArgs a) {
   for (int base = 0; base < wave_len; base += kGB) {
     const int cnt = min(kGB, len - base);           // this bag's share (may be <= 0)
     const int wave_cnt = min(kGB, wave_len - base); // uniform
+    // scale and offset are requested with the index in hand and consumed after
+    // the row reads have been issued (global-address loads: see slws_rows_kernel)
+    uint32_t so_lo[kPer], so_hi[kPer];
+    float my_w[kPer];
+    bool my_valid[kPer];
 #pragma unroll
     for (int k = 0; k < kPer; k++) {
       const int j = lir + k * LPR;
@@ -831,8 +836,8 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_groups_kernel(SlwsArgs a) {
       long long row = -1;
       float w = 0.0f;
       if (j < cnt && pos < a.num_indices) {
-        row = a.idx64 ? reinterpret_cast<const long long *>(a.indices)[pos]
-                      : (long long)reinterpret_cast<const int *>(a.indices)[pos];
+        row = a.idx64 ? ((const global_i64 *)a.indices)[pos]
+                      : (long long)((const global_i32 *)a.indices)[pos];
         if (!a.weights) {
           w = 1.0f;
         } else if (a.w16) {
@@ -842,26 +847,20 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_groups_kernel(SlwsArgs a) {
         }
       }
       // a skipped lookup reads row 0 and contributes exactly +0
-      const bool valid = row >= 0 && row < a.data_rows;
-      if (!valid) row = 0;
-      float s, o;
+      my_valid[k] = row >= 0 && row < a.data_rows;
+      if (!my_valid[k]) row = 0;
+      my_w[k] = w;
+      so_hi[k] = 0;
       if (!SO16 && a.sep_scales) {
-        s = a.sep_scales[row];
-        o = a.sep_offsets[row];
+        so_lo[k] = ((const global_u32 *)a.sep_scales)[row];
+        so_hi[k] = ((const global_u32 *)a.sep_offsets)[row];
       } else {
-        const uint32_t *so = reinterpret_cast<const uint32_t *>(
-            a.data + row * a.in_line + a.data_bytes);
-        if constexpr (SO16) {
-          const uint32_t v = so[0];
-          s = __half2float(__ushort_as_half((unsigned short)(v & 0xffff)));
-          o = __half2float(__ushort_as_half((unsigned short)(v >> 16)));
-        } else {
-          s = __uint_as_float(so[0]);
-          o = __uint_as_float(so[1]);
-        }
+        const global_u32 *so = (const global_u32 *)((const global_u8 *)a.data +
+                                                    (row * a.in_line + a.data_bytes));
+        so_lo[k] = so[0];
+        if constexpr (!SO16) so_hi[k] = so[1];
       }
       keys[j] = OFF32 ? (uint32_t)(row * a.in_line) : (uint32_t)row;
-      wso[j] = valid ? make_float2(w * s, w * o) : make_float2(0.0f, 0.0f);
     }
     wave_lds_sync();
     uint32_t q[kGB];
@@ -881,6 +880,20 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_groups_kernel(SlwsArgs a) {
         }
       }
     }
+#pragma unroll
+    for (int k = 0; k < kPer; k++) {
+      float sc, of;
+      if constexpr (SO16) {
+        sc = __half2float(__ushort_as_half((unsigned short)(so_lo[k] & 0xffff)));
+        of = __half2float(__ushort_as_half((unsigned short)(so_lo[k] >> 16)));
+      } else {
+        sc = __uint_as_float(so_lo[k]);
+        of = __uint_as_float(so_hi[k]);
+      }
+      wso[lir + k * LPR] =
+          my_valid[k] ? make_float2(my_w[k] * sc, my_w[k] * of) : make_float2(0.0f, 0.0f);
+    }
+    wave_lds_sync();
 #pragma unroll
     for (int c = 0; c < kGB / kChunk; c++) {
       if (c * kChunk < wave_cnt) {
