@@ -737,12 +737,18 @@ def _fused_cols(in_line, kind):
 
 
 def frwq_slws(data, kind, weights, indices, lengths, out_f16=False,
-              fp16_accum=False, d_data=None):
+              fp16_accum=False, d_data=None, row_pitch=None):
     """weights: None (plain SLS), float32 or float16 array. `d_data` lets a
-    caller reuse a table already resident on the device."""
+    caller reuse a table already resident on the device. `row_pitch` lays the
+    table out with its rows that many bytes apart (the gaps hold junk)."""
     data_shape = data.shape
     in_line = data_shape[1]
     out_line = _fused_cols(in_line, kind)
+    if row_pitch is not None:
+        wide = np.full((data_shape[0], row_pitch), 0xA5, np.uint8)
+        wide[:, :in_line] = data
+        d_data = to_device(wide)
+        in_line = row_pitch
     if d_data is None:
         d_data = to_device(np.ascontiguousarray(data, np.uint8))
     indices = np.ascontiguousarray(indices)

@@ -1084,13 +1084,15 @@ static int slws_dispatch(void *dest, int out_is_f16, const uint8_t *data,
   const bool is4 = kind == MI355X_FUSED_U4_F16 || kind == MI355X_FUSED_U4_F32;
   const bool so16 = kind == MI355X_FUSED_U8_F16 || kind == MI355X_FUSED_U4_F16;
   const size_t so_bytes = x.sep_scales ? 0 : (so16 ? 4 : 8);
-  MI355X_REQUIRE(in_line_size > so_bytes, "in_line_size %zu too small",
-                 in_line_size);
-  const size_t data_bytes = in_line_size - so_bytes;
-  const size_t cols = is4 ? data_bytes * 2 : data_bytes;
-  MI355X_REQUIRE(out_line_size == cols,
-                 "out_line_size %zu does not match %zu columns of the fused row",
-                 out_line_size, cols);
+  // in_line_size is the distance between rows: the fused row's own size, or
+  // more when the table has been laid out with padded rows
+  MI355X_REQUIRE(out_line_size > 0 && (!is4 || out_line_size % 2 == 0),
+                 "out_line_size %zu is not a row of this kind", out_line_size);
+  const size_t cols = out_line_size;
+  const size_t data_bytes = is4 ? cols / 2 : cols;
+  MI355X_REQUIRE(in_line_size >= data_bytes + so_bytes,
+                 "in_line_size %zu does not hold %zu columns of the fused row",
+                 in_line_size, cols);
   MI355X_REQUIRE(in_line_size < (1u << 20) && data_rows < (1ull << 31) &&
                      out_rows < (1ull << 40),
                  "table or batch too large");

@@ -593,6 +593,37 @@ private:
     return [base, rel](const DeviceBindings &b) { return b.generated + *base + rel; };
   }
 
+  // Where a lookup reads a table and how far apart its rows are. A constant
+  // table whose rows take 33..63 bytes is copied once, at load time, to rows 64
+  // bytes apart: memory is fetched in 64-byte pieces, a 36-byte row at a 36-byte
+  // pitch straddles two of them more often than not, and at 64 bytes it never
+  // does. Costs 64/inLine of the table's size in device memory.
+  struct TableView {
+    std::function<const uint8_t *(const DeviceBindings &)> ptr;
+    size_t pitch;
+  };
+  TableView tableView(const Operand &data, size_t rows, size_t inLine, MI355XFunction &out) {
+    if (!opts_.padTableRows || data.v->category != SymbolCategory::Constant || inLine <= 32 ||
+        inLine >= 64 || rows == 0)
+      return {[data](const DeviceBindings &b) { return (const uint8_t *)data.ptr(b); }, inLine};
+    auto it = paddedTables_.find(data.v);
+    if (it == paddedTables_.end()) {
+      constexpr size_t kPitch = 64;
+      auto dst = scratchPtr(gen_.addScratch(rows * kPitch));
+      out.setup.push_back({"mi355x_insert_rows", data.v->name + ".pad_rows",
+                           strFormat(" rows=%zu row_bytes=%zu pitch=%zu", rows, inLine, kPitch),
+                           [=](const DeviceBindings &b) {
+                             return mi355x_insert_rows(dst(b), data.ptr(b), rows, inLine, kPitch, 0,
+                                                       b.stream);
+                           }});
+      it = paddedTables_.emplace(data.v, TableView{[dst](const DeviceBindings &b) {
+                                                     return (const uint8_t *)dst(b);
+                                                   },
+                                                   kPitch}).first;
+    }
+    return it->second;
+  }
+
   Error quantize(const Instruction &I, MI355XFunction &out) {
     Operand d = op(I, 0), s = op(I, 1);
     CHECK_OP(d.ty().kind == ElemKind::Int8QTy && s.ty().kind == ElemKind::FloatTy,
@@ -1225,6 +1256,10 @@ private:
     const SlsChain g = group[0];
     size_t maxRows = 0;
     for (const auto &c : group) maxRows = std::max(maxRows, c.rows);
+    // tables of one group have one row size, so all of them are re-laid or none
+    std::vector<TableView> views;
+    for (const auto &c : group) views.push_back(tableView(c.data, c.rows, c.inLine, out));
+    const size_t pitch = views[0].pitch;
     auto tabPtr = scratchPtr(gen_.addScratch(n * sizeof(mi355x_sls_table)));
     const size_t stride = (size_t)g.dest.ty().dims[1];
     const std::string name = insts_[at].name + (n > 1 ? "..." + insts_[pos - 1].name : "");
@@ -1233,7 +1268,7 @@ private:
                          [=](const DeviceBindings &b) {
                            std::vector<mi355x_sls_table> t(n);
                            for (size_t i = 0; i < n; i++) {
-                             t[i].data = group[i].data.ptr(b);
+                             t[i].data = views[i].ptr(b);
                              t[i].indices = group[i].idx.ptr(b);
                              t[i].lengths = (const int32_t *)group[i].len.ptr(b);
                              t[i].dest = group[i].dest.ptr(b) + group[i].colOffset;
@@ -1249,13 +1284,13 @@ private:
     out.launches.push_back(
         {"mi355x_frwq_sls_multi", name,
          strFormat(" tables=%zu max_rows=%zu in_line=%zu out_line=%zu segments=%zu stride=%zu", n, maxRows,
-                   g.inLine, g.cols, g.segs, stride) +
+                   pitch, g.cols, g.segs, stride) +
              kv("kind", g.kind) + kv("idx_is_64", g.idx64) + kv("out_kind", outKind) +
              strFormat(" out_scale=%.9g", (double)g.qScale) + kv("out_offset", g.qOffset) +
              kv("fp16_accum", g.acc16),
          [=](const DeviceBindings &b) {
            return mi355x_frwq_sls_multi((const mi355x_sls_table *)tabPtr(b), n, maxRows, g.kind, g.idx64,
-                                        g.segs, g.inLine, g.cols, outKind, g.qScale, g.qOffset, stride,
+                                        g.segs, pitch, g.cols, outKind, g.qScale, g.qOffset, stride,
                                         g.acc16, b.stream);
          }});
     return pos - at;
@@ -1302,16 +1337,18 @@ private:
     const size_t nIdx = (size_t)idx.ty().size(), segs = (size_t)len.ty().size();
     const int out16 = dk == ElemKind::Float16Ty, w16 = wk == ElemKind::Float16Ty;
     const int idx64 = idx.ty().kind == ElemKind::Int64ITy;
+    const TableView table = tableView(data, rows, inLine, out);
+    const size_t pitch = table.pitch;
     out.launches.push_back(
         {"mi355x_frwq_slws", I.name,
-         strFormat(" rows=%zu in_line=%zu out_line=%zu segments=%zu num_indices=%zu", rows, inLine,
+         strFormat(" rows=%zu in_line=%zu out_line=%zu segments=%zu num_indices=%zu", rows, pitch,
                    outLine, segs, nIdx) +
              kv("kind", kind) + kv("out_is_f16", out16) + kv("weighted", weighted) +
              kv("weights_are_f16", w16) + kv("idx_is_64", idx64) + kv("fp16_accum", acc16),
          [=](const DeviceBindings &b) {
-           return mi355x_frwq_slws(d.ptr(b), out16, data.ptr(b), rows, kind,
+           return mi355x_frwq_slws(d.ptr(b), out16, table.ptr(b), rows, kind,
                                    weighted ? (const void *)w.ptr(b) : nullptr, w16, idx.ptr(b), idx64,
-                                   nIdx, (const int32_t *)len.ptr(b), segs, inLine, outLine,
+                                   nIdx, (const int32_t *)len.ptr(b), segs, pitch, outLine,
                                    acc16 ? 1 : 0, b.stream);
          }});
     return Error::success();
@@ -1325,6 +1362,7 @@ private:
   size_t scratchBase_ = 0, genTotal_ = 0;
   std::shared_ptr<size_t> scratchBasePtr_ = std::make_shared<size_t>(0);
   std::map<int, std::pair<bool, bool>> io_; // value id -> (read, written)
+  std::map<const Value *, TableView> paddedTables_;
 };
 
 constexpr int Compiler::kArity[];

@@ -150,6 +150,7 @@ struct BackendOptions {
   bool fuseSlsChains = true;           // pooled lookups + ConvertTo/Quantize/InsertTensor, many tables per launch
   bool fuseTransposeMatMul = true;     // BatchMatMul(L, Transpose(R)) without materialising the transpose
   bool fuseFcRelu = true;              // RowwiseQuantizedFullyConnected + Relu of its result in one kernel
+  bool padTableRows = true;            // constant lookup tables with 33..63-byte rows re-laid 64 bytes apart at load
 };
 
 class MI355XBackend {

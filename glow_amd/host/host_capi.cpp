@@ -125,6 +125,7 @@ int mi355x_host_compile(mi355x_host_module *m, int function, int options) {
   o.fuseSlsChains = (options & MI355X_HOST_OPT_FUSE_SLS_CHAINS) != 0;
   o.fuseTransposeMatMul = (options & MI355X_HOST_OPT_FUSE_TRANSPOSE_MATMUL) != 0;
   o.fuseFcRelu = (options & MI355X_HOST_OPT_FUSE_FC_RELU) != 0;
+  o.padTableRows = (options & MI355X_HOST_OPT_PAD_TABLE_ROWS) != 0;
   auto r = MI355XBackend().compile(*f, o);
   if (!r) return fail(r.error());
   m->compiled[function] = std::move(r.get());

@@ -452,7 +452,11 @@ int mi355x_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
  * lib/Backends/Interpreter/InterpreterNodes.cpp:5764-5889) for the other
  * kinds, fp16 weights/output and fp16 accumulation.
  *   dest     [segments x out_line_size] fp32, or fp16 when out_is_f16
- *   data     [data_rows x in_line_size] fused rows
+ *   data     [data_rows x in_line_size] fused rows; in_line_size is the distance
+ *            between rows and may exceed the fused row's own size (quantized
+ *            bytes of out_line_size columns, then scale and offset): a table
+ *            re-laid with padded rows, e.g. 36-byte rows 64 bytes apart so
+ *            that a lookup touches one 64-byte piece of memory instead of 1.5
  *   weights  fp32 (or fp16 when weights_are_f16); NULL = all ones
  *            (FusedRowwiseQuantizedSparseLengthsSum, Lower.cpp:1590-1606)
  *   indices  int64 when idx_is_64 else int32, num_indices entries of which

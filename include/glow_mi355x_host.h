@@ -119,7 +119,9 @@ enum {
   MI355X_HOST_OPT_FUSE_SLS_CHAINS = 16, /* pooled lookups + ConvertTo/Quantize/InsertTensor, many tables per launch */
   MI355X_HOST_OPT_FUSE_TRANSPOSE_MATMUL = 32, /* BatchMatMul(L, Transpose(R)) reads R as it lies */
   MI355X_HOST_OPT_FUSE_FC_RELU = 64, /* RowwiseQuantizedFullyConnected + Relu in one kernel */
-  MI355X_HOST_OPT_DEFAULT = 127
+  MI355X_HOST_OPT_PAD_TABLE_ROWS = 128, /* constant lookup tables with rows of 33..63 bytes are copied
+                                          at load time to rows 64 bytes apart */
+  MI355X_HOST_OPT_DEFAULT = 255
 };
 int mi355x_host_compile(mi355x_host_module *m, int function, int options);
 /* Listing of the compiled function's launches and derived parameters; returns

@@ -40,6 +40,29 @@ def test_builds_and_compiles():
     assert net.tensors["top_in"].shape == (64, 22)
 
 
+def test_small_table_rows_are_relaid_64_bytes_apart():
+    """64 four-bit columns with fp16 scale/offset make 36-byte rows: each
+    constant table gets one set-up copy to a 64-byte pitch and the lookups are
+    told that pitch; switched off, they read the packed rows."""
+    cfg = dict(tables=3, rows=300, dim=64, batch=32, mean_len=4, bottom=(32, 64), top=(32, 1))
+    net, _ = dlrm.make(seed=4, **cfg)
+    for fuse in (True, False):
+        m, f = netlib.to_module(net)
+        m.compile(f, fuse_sls_chains=fuse)
+        rows = H.parse_listing(m.describe(f))
+        pads = [r for r in rows if r["phase"] == "setup" and r["inst"].endswith(".pad_rows")]
+        assert len(pads) == 3 and all((r["kernel"], r["row_bytes"], r["pitch"]) ==
+                                      ("mi355x_insert_rows", 36, 64) for r in pads)
+        look = [r for r in rows if r["phase"] == "launch" and "_sl" in r["kernel"]]
+        assert len(look) == (1 if fuse else 3) and all(r["in_line"] == 64 for r in look)
+        m, f = netlib.to_module(net)
+        m.compile(f, fuse_sls_chains=fuse, pad_table_rows=False)
+        rows = H.parse_listing(m.describe(f))
+        assert not [r for r in rows if r["inst"].endswith(".pad_rows")]
+        assert all(r["in_line"] == 36 for r in rows
+                   if r["phase"] == "launch" and "_sl" in r["kernel"])
+
+
 def test_oracle_executes_the_small_network():
     net, max_idx = dlrm.make(seed=2, **SMALL)
     inp = dlrm.Inputs(7, 3, 2000, 64, 5, 1.1, 13)
@@ -50,12 +73,14 @@ def test_oracle_executes_the_small_network():
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("pad", [True, False])
 @pytest.mark.parametrize("fuse", [True, False])
-def test_device_matches_oracle(fuse):
+def test_device_matches_oracle(fuse, pad):
     cfg = dict(tables=4, rows=5000, dim=64, batch=256, mean_len=8, bottom=(64, 64), top=(128, 1))
     net, max_idx = dlrm.make(seed=3, **cfg)
     m, f = netlib.to_module(net)
-    m.compile(f, fuse_sls_chains=fuse, fuse_transpose_matmul=fuse, fuse_fc_relu=fuse)
+    m.compile(f, fuse_sls_chains=fuse, fuse_transpose_matmul=fuse, fuse_fc_relu=fuse,
+              pad_table_rows=pad)
     dm = H.DeviceManager().init()
     try:
         dm.add_network(m)

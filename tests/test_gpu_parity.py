@@ -400,6 +400,30 @@ def test_slws_other_kinds_bit_exact(kind, cols):
                                       want.view(np.uint16 if out16 else np.uint32))
 
 
+@pytest.mark.parametrize("kind,cols,pitch", [
+    (capi.FUSED_U4_F16, 64, 64), (capi.FUSED_U8_F32, 32, 64), (capi.FUSED_U8_F32, 128, 192),
+    (capi.FUSED_U8_F16, 30, 35), (capi.FUSED_U4_F32, 130, 80),
+])
+def test_slws_padded_rows_bit_exact(kind, cols, pitch):
+    """in_line_size above the fused row's own size: rows that far apart."""
+    say("slws padded rows kind", kind, "cols", cols, "pitch", pitch)
+    rng = np.random.default_rng(kind * 77 + cols)
+    rows, bags = 600, 90
+    table = cases.random_fused_table(rng, rows, cols, kind)
+    lengths, idx, w = cases.slws_batch(cols + 2, rows, bags, 15, 1.1, np.int32)
+    total = int(lengths.sum())
+    idx, w = idx[:total], w[:total]
+    f16 = kind in (capi.FUSED_U8_F16, capi.FUSED_U4_F16)
+    combos = [(w, False, False), (None, False, False)]
+    if f16:
+        combos += [(w.astype(np.float16), True, True)]
+    for weights, out16, acc16 in combos:
+        want = go.frwq_slws_generic(table, kind, weights, idx, lengths, out16, acc16)
+        got = capi.frwq_slws(table, kind, weights, idx, lengths, out16, acc16, row_pitch=pitch)
+        np.testing.assert_array_equal(got.view(np.uint16 if out16 else np.uint32),
+                                      want.view(np.uint16 if out16 else np.uint32))
+
+
 def test_slws_fp16_accumulation_rounds_the_product_twice():
     """fp16 accumulation rounds w*(s*q+o) to binary32 and then to binary16, as
     the CPU does; a single rounding differs in the last place about once in

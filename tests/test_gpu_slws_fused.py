@@ -133,6 +133,39 @@ def test_slws_other_kinds(kind, cols):
               what=f"w={'none' if weights is None else weights.dtype} out16={out16}")
 
 
+@pytest.mark.parametrize("kind,cols,pitch", [
+    (capi.FUSED_U4_F16, 64, 64),     # 36-byte rows, several bags per wavefront
+    (capi.FUSED_U8_F32, 32, 64),     # 40-byte rows
+    (capi.FUSED_U8_F16, 64, 128),    # 68-byte rows
+    (capi.FUSED_U8_F32, 128, 192),   # 136-byte rows, one wavefront per bag
+    (capi.FUSED_U8_F32, 256, 272),
+    (capi.FUSED_U4_F32, 60, 40),     # 38-byte rows on the general kernel
+    (capi.FUSED_U8_F16, 30, 35),     # odd pitch: byte loads
+])
+def test_rows_further_apart_than_their_size(kind, cols, pitch):
+    """A table laid out with padded rows (in_line_size above the fused row's
+    size) gives what the packed table gives: the same bits from the same
+    kernel, and the oracle's values to the stated tolerance."""
+    say("padded table kind", kind, "cols", cols, "pitch", pitch)
+    rng = np.random.default_rng(kind * 1000 + cols)
+    rows, bags = 900, 130
+    table = cases.random_fused_table(rng, rows, cols, kind)
+    assert table.shape[1] <= pitch
+    lengths, idx, w = cases.slws_batch(cols + 1, rows, bags, 18, 1.1, np.int64)
+    lengths[3] = 0
+    total = int(lengths.sum())
+    idx, w = idx[:total], w[:total]
+    f16 = kind in (capi.FUSED_U8_F16, capi.FUSED_U4_F16)
+    for weights in (w, None):
+        want = go.frwq_slws_generic(table, kind, weights, idx, lengths, f16, False)
+        packed = capi.frwq_slws(table, kind, weights, idx, lengths, f16)
+        padded = capi.frwq_slws(table, kind, weights, idx, lengths, f16, row_pitch=pitch)
+        assert np.array_equal(padded.view(np.uint8), packed.view(np.uint8))
+        check(padded.astype(np.float32), want.astype(np.float32),
+              bag_magnitude(table, kind, weights, idx, lengths), f16,
+              what=f"w={'none' if weights is None else 'f32'}")
+
+
 def test_invalid_lookups_are_skipped_and_rows_rezeroed():
     rows, cols = 50, 128
     rng = np.random.default_rng(12)

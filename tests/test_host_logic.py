@@ -50,11 +50,17 @@ def test_argument_validation_needs_no_gpu():
     rc = lib.mi355x_rescale_i8(C.c_void_p(16), C.c_void_p(16), C.c_size_t(4),
                                0, 0, 40, 0, 1, None)
     assert rc == -1 and b"shift" in lib.mi355x_last_error()
-    # out_line_size inconsistent with the fused row
+    # rows too close together for out_line_size columns plus scale and offset
     rc = lib.mi355x_frwq_slws(C.c_void_p(16), 0, C.c_void_p(16), C.c_size_t(10),
                               0, None, 0, C.c_void_p(16), 1, C.c_size_t(4),
                               C.c_void_p(16), C.c_size_t(2), C.c_size_t(136),
-                              C.c_size_t(64), 0, None)
+                              C.c_size_t(130), 0, None)
+    assert rc == -1 and b"in_line_size" in lib.mi355x_last_error()
+    # an odd number of 4-bit columns
+    rc = lib.mi355x_frwq_slws(C.c_void_p(16), 1, C.c_void_p(16), C.c_size_t(10),
+                              2, None, 0, C.c_void_p(16), 1, C.c_size_t(4),
+                              C.c_void_p(16), C.c_size_t(2), C.c_size_t(36),
+                              C.c_size_t(63), 0, None)
     assert rc == -1 and b"out_line_size" in lib.mi355x_last_error()
     # unknown schema
     s, o = C.c_float(), C.c_int32()
