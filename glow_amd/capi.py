@@ -26,7 +26,8 @@ EXPORTS = [
     "mi355x_cwq_conv2d_add_i8", "mi355x_frwq_sls_multi",
     "mi355x_specialize_bias_weights_qparams", "mi355x_rwq_slws", "mi355x_slws_set_fused_math", "mi355x_batch_matmul_nt_i8", "mi355x_rwq_fc_relu_i8", "mi355x_add_i8", "mi355x_add_relu_i8",
     "mi355x_relu_i8", "mi355x_convert_f16_to_f32", "mi355x_insert_rows",
-    "mi355x_batch_transpose_i8", "mi355x_space_to_depth2_i8", "mi355x_gather", "mi355x_batch_matmul_i8", "mi355x_sigmoid_f32",
+    "mi355x_batch_transpose_i8", "mi355x_space_to_depth2_i8", "mi355x_gather", "mi355x_gather_rows", "mi355x_rescale_rows_i8",
+    "mi355x_dequantize_sigmoid", "mi355x_batch_matmul_i8", "mi355x_sigmoid_f32",
     "mi355x_max_pool_i8", "mi355x_avg_pool_i8", "mi355x_softmax_f32", "mi355x_stream_create",
     "mi355x_stream_destroy", "mi355x_stream_sync", "mi355x_device_sync",
     "mi355x_event_create", "mi355x_event_destroy", "mi355x_event_record", "mi355x_stream_wait_event",
@@ -940,6 +941,45 @@ def gather(data, indices, batch_dims=0):
     check(lib().mi355x_gather(_vp(out), _vp(dd), _vp(di), C.c_int(indices.dtype == np.int64),
                               _sz(indices.size), _sz(slice_bytes), _sz(samples),
                               _sz(sample_bytes), _vp(None)))
+    return out.numpy()
+
+
+def gather_rows(data, indices, into, col):
+    """Gather with one batch dimension whose samples land in the 2-D array
+    `into` starting at element column `col`; returns the updated array."""
+    data = np.ascontiguousarray(data)
+    indices = np.ascontiguousarray(indices)
+    into = np.ascontiguousarray(into)
+    assert into.dtype == data.dtype and into.ndim == 2 and into.shape[0] == data.shape[0]
+    es = data.dtype.itemsize
+    slice_bytes = int(np.prod(data.shape[2:], dtype=np.int64)) * es
+    sample_bytes = data.shape[1] * slice_bytes
+    dd, di, out = to_device(data), to_device(indices), to_device(into)
+    check(lib().mi355x_gather_rows(_vp(out.ptr + col * es), _vp(dd), _vp(di),
+                                   C.c_int(indices.dtype == np.int64), _sz(indices.size),
+                                   _sz(slice_bytes), _sz(data.shape[0]), _sz(sample_bytes),
+                                   _sz(into.shape[1] * es), _vp(None)))
+    return out.numpy()
+
+
+def rescale_rows_i8(q, into, col, out_offset, in_offset, pre, post, scale):
+    """Rescale of the 2-D int8 array `q` written into `into` at column `col`."""
+    q = np.ascontiguousarray(q, np.int8)
+    into = np.ascontiguousarray(into, np.int8)
+    d_in, out = to_device(q), to_device(into)
+    check(lib().mi355x_rescale_rows_i8(_vp(out.ptr + col), _vp(d_in), _sz(q.shape[0]),
+                                       _sz(q.shape[1]), _sz(into.shape[1]), _i32(out_offset),
+                                       _i32(in_offset), _i32(pre), _i32(post), _i32(scale),
+                                       _vp(None)))
+    return out.numpy()
+
+
+def dequantize_sigmoid(q, scale, offset):
+    q = np.ascontiguousarray(q, np.int8)
+    d_in = to_device(q)
+    out = DeviceBuffer.empty(q.shape, np.float32)
+    check(lib().mi355x_dequantize_sigmoid(_vp(out), _vp(d_in), _sz(q.size), C.c_float(scale),
+                                          _i32(offset), _vp(None)))
     return out.numpy()
 
 

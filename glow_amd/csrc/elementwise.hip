@@ -117,6 +117,45 @@ __global__ __launch_bounds__(kEwThreads) void rescale_i8_kernel(
                                                   post, scale, out_offset));
 }
 
+// RescaleQuantized of a [rows x cols] tensor written as a slice of a wider one
+// (dst rows dst_row_stride bytes apart): V bytes per lane.
+template <int V>
+__global__ __launch_bounds__(kEwThreads) void rescale_rows_i8_kernel(
+    int8_t *__restrict__ dst, const int8_t *__restrict__ src, long long rows, int cols,
+    long long dst_row_stride, int32_t out_offset, int32_t in_offset, int32_t pre,
+    int32_t post, int32_t scale) {
+  const int per_row = cols / V;
+  const long long total = rows * per_row;
+  const long long stride = (long long)gridDim.x * kEwThreads;
+  for (long long i = (long long)blockIdx.x * kEwThreads + threadIdx.x; i < total; i += stride) {
+    const long long r = i / per_row;
+    const int c = (int)(i - r * per_row) * V;
+    if constexpr (V == 4) {
+      const uint32_t w = *reinterpret_cast<const uint32_t *>(src + r * cols + c);
+      int32_t q[4];
+#pragma unroll
+      for (int b = 0; b < 4; b++)
+        q[b] = clip_i8(scale_i32(sext8(w, b) - in_offset, pre, post, scale, out_offset));
+      *reinterpret_cast<uint32_t *>(dst + r * dst_row_stride + c) = pack4(q[0], q[1], q[2], q[3]);
+    } else {
+      dst[r * dst_row_stride + c] = (int8_t)clip_i8(
+          scale_i32((int32_t)src[r * cols + c] - in_offset, pre, post, scale, out_offset));
+    }
+  }
+}
+
+// Dequantize followed by Sigmoid (libjit_sigmoid_kernel_f on the dequantized
+// value): 1 / (expf(-(scale * (q - offset))) + 1).
+__global__ __launch_bounds__(kEwThreads) void dequantize_sigmoid_kernel(
+    float *__restrict__ dst, const int8_t *__restrict__ src, size_t n, float scale,
+    int32_t offset) {
+  const size_t stride = (size_t)gridDim.x * kEwThreads;
+  for (size_t i = (size_t)blockIdx.x * kEwThreads + threadIdx.x; i < n; i += stride) {
+    const float x = __fmul_rn(scale, (float)((int32_t)src[i] - offset));
+    dst[i] = __fdiv_rn(1.0f, __fadd_rn(expf(-x), 1.0f));
+  }
+}
+
 static bool aligned16(const void *a, const void *b) {
   return (((uintptr_t)a | (uintptr_t)b) & 15) == 0;
 }
@@ -180,6 +219,44 @@ int mi355x_rescale_i8(int8_t *dst, const int8_t *src, size_t n,
                        dim3(kEwThreads), 0, as_stream(stream), dst, src, n,
                        chunks, out_offset, in_offset, pre, post, scale);
   return check_launch("rescale_i8");
+}
+
+int mi355x_rescale_rows_i8(int8_t *dst, const int8_t *src, size_t rows, size_t cols,
+                           size_t dst_row_stride, int32_t out_offset, int32_t in_offset,
+                           int32_t pre, int32_t post, int32_t scale, void *stream) {
+  if (rows == 0 || cols == 0) return MI355X_OK;
+  MI355X_REQUIRE(dst && src, "NULL tensor");
+  MI355X_REQUIRE(shift_ok(pre) && shift_ok(post),
+                 "pre/post shift outside [0, 31]: %d %d", pre, post);
+  MI355X_REQUIRE(dst_row_stride >= cols, "rows of %zu bytes overlap at a stride of %zu", cols,
+                 dst_row_stride);
+  MI355X_REQUIRE(rows < (1ull << 40) && cols < (1u << 30) && dst_row_stride < (1ull << 40),
+                 "tensor too large");
+  const bool vec = cols % 4 == 0 && dst_row_stride % 4 == 0 &&
+                   ((((uintptr_t)dst) | ((uintptr_t)src)) & 3) == 0;
+  const size_t work = rows * (vec ? cols / 4 : cols);
+  size_t blocks = (work + kEwThreads - 1) / kEwThreads;
+  if (blocks > 256 * 64) blocks = 256 * 64;
+  if (vec)
+    hipLaunchKernelGGL(rescale_rows_i8_kernel<4>, dim3((unsigned)blocks), dim3(kEwThreads), 0,
+                       as_stream(stream), dst, src, (long long)rows, (int)cols,
+                       (long long)dst_row_stride, out_offset, in_offset, pre, post, scale);
+  else
+    hipLaunchKernelGGL(rescale_rows_i8_kernel<1>, dim3((unsigned)blocks), dim3(kEwThreads), 0,
+                       as_stream(stream), dst, src, (long long)rows, (int)cols,
+                       (long long)dst_row_stride, out_offset, in_offset, pre, post, scale);
+  return check_launch("rescale_rows_i8");
+}
+
+int mi355x_dequantize_sigmoid(float *dst, const int8_t *src, size_t n, float scale,
+                              int32_t offset, void *stream) {
+  if (n == 0) return MI355X_OK;
+  MI355X_REQUIRE(dst && src, "NULL tensor");
+  size_t blocks = (n + kEwThreads - 1) / kEwThreads;
+  if (blocks > 256 * 64) blocks = 256 * 64;
+  hipLaunchKernelGGL(dequantize_sigmoid_kernel, dim3((unsigned)blocks), dim3(kEwThreads), 0,
+                     as_stream(stream), dst, src, n, scale, offset);
+  return check_launch("dequantize_sigmoid");
 }
 
 } // extern "C"

@@ -364,7 +364,8 @@ __global__ __launch_bounds__(kGlueThreads) void batch_transpose_i8_kernel(
 template <typename IDX>
 __global__ __launch_bounds__(kGlueThreads) void gather_kernel(
     uint8_t *__restrict__ dst, const uint8_t *__restrict__ data, const IDX *__restrict__ idx,
-    long long num_indices, long long slice_bytes, long long samples, long long sample_bytes) {
+    long long num_indices, long long slice_bytes, long long samples, long long sample_bytes,
+    long long dst_sample_stride) {
   const long long total = samples * num_indices * slice_bytes;
   const long long stride = (long long)gridDim.x * kGlueThreads;
   const long long slices = sample_bytes / slice_bytes;
@@ -373,7 +374,8 @@ __global__ __launch_bounds__(kGlueThreads) void gather_kernel(
     const long long t = i / slice_bytes;
     const long long k = t % num_indices, smp = t / num_indices;
     const long long sl = (long long)idx[k];
-    dst[i] = (sl >= 0 && sl < slices) ? data[smp * sample_bytes + sl * slice_bytes + b] : 0;
+    dst[smp * dst_sample_stride + k * slice_bytes + b] =
+        (sl >= 0 && sl < slices) ? data[smp * sample_bytes + sl * slice_bytes + b] : 0;
   }
 }
 
@@ -723,27 +725,40 @@ int mi355x_batch_transpose_i8(int8_t *dst, const int8_t *src, size_t batch, size
   return check_launch("batch_transpose_i8");
 }
 
-int mi355x_gather(void *dst, const void *data, const void *indices, int idx_is_64,
-                  size_t num_indices, size_t slice_bytes, size_t num_samples,
-                  size_t sample_bytes, void *stream) {
+int mi355x_gather_rows(void *dst, const void *data, const void *indices, int idx_is_64,
+                       size_t num_indices, size_t slice_bytes, size_t num_samples,
+                       size_t sample_bytes, size_t dst_sample_stride, void *stream) {
   if (num_indices == 0 || slice_bytes == 0 || num_samples == 0) return MI355X_OK;
   MI355X_REQUIRE(dst && data && indices, "NULL tensor");
   MI355X_REQUIRE(sample_bytes % slice_bytes == 0, "sample is not a whole number of slices");
   MI355X_REQUIRE(num_indices < (1ull << 32) && slice_bytes < (1ull << 32) &&
-                     num_samples < (1ull << 32) && sample_bytes < (1ull << 40),
+                     num_samples < (1ull << 32) && sample_bytes < (1ull << 40) &&
+                     dst_sample_stride < (1ull << 40),
                  "tensor too large");
+  MI355X_REQUIRE(dst_sample_stride >= num_indices * slice_bytes,
+                 "gathered samples of %zu bytes overlap at a stride of %zu",
+                 num_indices * slice_bytes, dst_sample_stride);
   const size_t total = num_samples * num_indices * slice_bytes;
   if (idx_is_64)
     hipLaunchKernelGGL(gather_kernel<long long>, dim3(capped_blocks(total)), dim3(kGlueThreads), 0,
                        as_stream(stream), (uint8_t *)dst, (const uint8_t *)data,
                        (const long long *)indices, (long long)num_indices, (long long)slice_bytes,
-                       (long long)num_samples, (long long)sample_bytes);
+                       (long long)num_samples, (long long)sample_bytes,
+                       (long long)dst_sample_stride);
   else
     hipLaunchKernelGGL(gather_kernel<int>, dim3(capped_blocks(total)), dim3(kGlueThreads), 0,
                        as_stream(stream), (uint8_t *)dst, (const uint8_t *)data,
                        (const int *)indices, (long long)num_indices, (long long)slice_bytes,
-                       (long long)num_samples, (long long)sample_bytes);
+                       (long long)num_samples, (long long)sample_bytes,
+                       (long long)dst_sample_stride);
   return check_launch("gather");
+}
+
+int mi355x_gather(void *dst, const void *data, const void *indices, int idx_is_64,
+                  size_t num_indices, size_t slice_bytes, size_t num_samples,
+                  size_t sample_bytes, void *stream) {
+  return mi355x_gather_rows(dst, data, indices, idx_is_64, num_indices, slice_bytes, num_samples,
+                            sample_bytes, num_indices * slice_bytes, stream);
 }
 
 int mi355x_batch_matmul_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs, size_t batch,

@@ -99,9 +99,12 @@ public:
 
   Error run(MI355XFunction &out) {
     for (const auto &I : insts_) MI355X_RETURN_IF_ERR(checkOperands(I));
+    absorbed_.assign(insts_.size(), 0);
     for (size_t at = 0; at < insts_.size(); at++) {
+      if (absorbed_[at]) continue; // folded into an earlier launch
       const Instruction &I = insts_[at];
       const size_t firstLaunch = out.launches.size(), firstInst = at;
+      std::vector<size_t> folded;   // instructions further down that this launch also covers
       switch (I.kind) {
       case Kind::ElementAdd: {
         // an add whose only reader is the Relu right behind it becomes one pass
@@ -140,12 +143,37 @@ public:
       }
       case Kind::ConvertTo:
       case Kind::InsertTensor:
-      case Kind::Gather:
       case Kind::BatchMatMul:
       case Kind::Sigmoid: MI355X_RETURN_IF_ERR(movement(I, out)); break;
+      case Kind::Gather: {
+        // a result that is only inserted into a wider tensor is gathered there
+        const size_t ins =
+            opts_.fuseInsert && I.iattrs.size() == 1 && I.iattrs[0] == 1 ? soleInsertOf(at) : 0;
+        MI355X_RETURN_IF_ERR(movement(I, out, ins ? &insts_[ins] : nullptr));
+        if (ins) { absorbed_[ins] = 1; folded.push_back(ins); }
+        break;
+      }
       case Kind::Quantize: MI355X_RETURN_IF_ERR(quantize(I, out)); break;
-      case Kind::Dequantize: MI355X_RETURN_IF_ERR(dequantize(I, out)); break;
-      case Kind::RescaleQuantized: MI355X_RETURN_IF_ERR(rescale(I, out)); break;
+      case Kind::Dequantize: {
+        // a Sigmoid right behind it that is the only reader of its result
+        const Instruction *sig = nullptr;
+        if (opts_.fuseDequantizeSigmoid && at + 1 < insts_.size() &&
+            insts_[at + 1].kind == Kind::Sigmoid && insts_[at + 1].operands[1] == I.operands[0] &&
+            M_.value(I.operands[0]).category == SymbolCategory::Activation &&
+            readers(I.operands[0]) == 1 &&
+            M_.value(insts_[at + 1].operands[0]).type.kind == ElemKind::FloatTy &&
+            M_.value(insts_[at + 1].operands[0]).type.size() == M_.value(I.operands[0]).type.size())
+          sig = &insts_[at + 1];
+        MI355X_RETURN_IF_ERR(dequantize(I, out, sig));
+        if (sig) at++;
+        break;
+      }
+      case Kind::RescaleQuantized: {
+        const size_t ins = opts_.fuseInsert ? soleInsertOf(at) : 0;
+        MI355X_RETURN_IF_ERR(rescale(I, out, ins ? &insts_[ins] : nullptr));
+        if (ins) { absorbed_[ins] = 1; folded.push_back(ins); }
+        break;
+      }
       case Kind::FullyConnected: MI355X_RETURN_IF_ERR(fc(I, out)); break;
       case Kind::RowwiseQuantizedFullyConnected: {
         // a Relu instruction right behind it that is the only reader of its result
@@ -200,6 +228,7 @@ public:
       // what the launches of instructions [firstInst, at] read and write
       for (size_t l = firstLaunch; l < out.launches.size(); l++) {
         for (size_t k = firstInst; k <= at; k++) noteAccesses(insts_[k], out.launches[l]);
+        for (size_t k : folded) noteAccesses(insts_[k], out.launches[l]);
         const std::string &kn = out.launches[l].kernel;
         out.launches[l].tunable = kn == "mi355x_fc_i8" || kn == "mi355x_rwq_fc_i8" ||
                                   kn == "mi355x_matmul_i8" || kn == "mi355x_conv2d_i8" ||
@@ -299,6 +328,70 @@ private:
       for (size_t i = 1; i < I.operands.size(); i++)
         n += M_.validId(I.operands[i]) && M_.value(I.operands[i]).root == root;
     return n;
+  }
+
+  int writers(int id) const {
+    const int root = M_.value(id).root;
+    int n = 0;
+    for (const auto &I : insts_)
+      n += M_.validId(I.operands[0]) && M_.value(I.operands[0]).root == root;
+    return n;
+  }
+
+  // The InsertTensor (its position, 0 if none) that is the only reader of the
+  // 2-D result of instruction `at` and can take effect at `at` already: nothing
+  // in between reads the tensor it inserts into, and whatever writes that
+  // tensor in between is an InsertTensor of other columns.
+  size_t soleInsertOf(size_t at) const {
+    const Instruction &P = insts_[at];
+    const int v = P.operands[0];
+    const Value &pv = M_.value(v);
+    if (pv.category != SymbolCategory::Activation || pv.root != v || pv.type.dims.size() != 2 ||
+        readers(v) != 1 || writers(v) != 1)
+      return 0;
+    size_t j = at + 1;
+    for (; j < insts_.size(); j++) {
+      bool reads = false;
+      for (size_t i = 1; i < insts_[j].operands.size(); i++) reads = reads || insts_[j].operands[i] == v;
+      if (reads) break;
+    }
+    if (j >= insts_.size()) return 0;
+    const Instruction &J = insts_[j];
+    if (J.kind != Kind::InsertTensor || J.operands[1] != v || J.iattrs.size() != 1 || J.iattrs[0] < 0)
+      return 0;
+    const Value &D = M_.value(J.operands[0]);
+    if (D.type.dims.size() != 2 || D.type.kind != pv.type.kind || D.type.dims[0] != pv.type.dims[0] ||
+        J.iattrs[0] + pv.type.dims[1] > D.type.dims[1] || D.root == pv.root)
+      return 0;
+    if (isQuantized(D.type.kind) && (D.type.scale != pv.type.scale || D.type.offset != pv.type.offset))
+      return 0;
+    // the producer itself must not read the tensor it would now write
+    for (size_t i = 1; i < P.operands.size(); i++)
+      if (M_.value(P.operands[i]).root == D.root) return 0;
+    const int64_t lo = J.iattrs[0], hi = lo + pv.type.dims[1];
+    for (size_t k = at + 1; k < j; k++) {
+      const Instruction &K = insts_[k];
+      for (size_t i = 1; i < K.operands.size(); i++)
+        if (M_.value(K.operands[i]).root == D.root) return 0;
+      if (M_.value(K.operands[0]).root != D.root) continue;
+      if (K.kind != Kind::InsertTensor || K.operands[0] != J.operands[0] || K.iattrs.size() != 1)
+        return 0;
+      const int64_t klo = K.iattrs[0], khi = klo + M_.value(K.operands[1]).type.dims.back();
+      if (klo < hi && lo < khi) return 0;
+    }
+    return j;
+  }
+
+  // where a producer folded with InsertTensor `ins` writes: the wide tensor,
+  // the byte offset of the slice in a row, and the row pitch in bytes
+  struct SliceDest {
+    Operand wide;
+    size_t offset, pitch;
+  };
+  SliceDest sliceDest(const Instruction &ins) const {
+    Operand wide = op(ins, 0);
+    const size_t es = elemSize(wide.ty().kind);
+    return {wide, (size_t)ins.iattrs[0] * es, (size_t)wide.ty().dims[1] * es};
   }
 
   Error add(const Instruction &I, const Instruction *reluI, MI355XFunction &out) {
@@ -415,7 +508,7 @@ private:
   }
 
   // data movement and the small operators of ranking models
-  Error movement(const Instruction &I, MI355XFunction &out) {
+  Error movement(const Instruction &I, MI355XFunction &out, const Instruction *ins = nullptr) {
     Operand d = op(I, 0), s = op(I, 1);
     switch (I.kind) {
     case Kind::ConvertTo: {
@@ -496,6 +589,18 @@ private:
       const size_t nIdx = (size_t)idx.ty().size();
       CHECK_OP((size_t)d.ty().sizeInBytes() == samples * nIdx * slice, "result size mismatch");
       const int i64 = idx.ty().kind == ElemKind::Int64ITy;
+      if (ins) {
+        const SliceDest sl = sliceDest(*ins);
+        out.launches.push_back(
+            {"mi355x_gather_rows", I.name + "+" + ins->name,
+             strFormat(" num_indices=%zu slice_bytes=%zu samples=%zu sample_bytes=%zu stride=%zu offset=%zu",
+                       nIdx, slice, samples, sample, sl.pitch, sl.offset),
+             [=](const DeviceBindings &b) {
+               return mi355x_gather_rows(sl.wide.ptr(b) + sl.offset, s.ptr(b), idx.ptr(b), i64, nIdx, slice,
+                                         samples, sample, sl.pitch, b.stream);
+             }});
+        return Error::success();
+      }
       out.launches.push_back({"mi355x_gather", I.name,
                               strFormat(" num_indices=%zu slice_bytes=%zu samples=%zu sample_bytes=%zu", nIdx, slice, samples, sample),
                               [=](const DeviceBindings &b) {
@@ -641,7 +746,7 @@ private:
     return Error::success();
   }
 
-  Error dequantize(const Instruction &I, MI355XFunction &out) {
+  Error dequantize(const Instruction &I, MI355XFunction &out, const Instruction *sig = nullptr) {
     Operand d = op(I, 0), s = op(I, 1);
     CHECK_OP(d.ty().kind == ElemKind::FloatTy && s.ty().kind == ElemKind::Int8QTy,
              "needs i8 -> float, has %s -> %s", s.ty().str().c_str(), d.ty().str().c_str());
@@ -649,6 +754,16 @@ private:
     const size_t n = (size_t)d.ty().size();
     const float sc = s.ty().scale;
     const int32_t off = s.ty().offset;
+    if (sig) {
+      Operand y = op(*sig, 0);
+      out.launches.push_back({"mi355x_dequantize_sigmoid", I.name + "+" + sig->name,
+                              strFormat(" n=%zu scale=%.9g offset=%d", n, (double)sc, off),
+                              [=](const DeviceBindings &b) {
+                                return mi355x_dequantize_sigmoid((float *)y.ptr(b), (const int8_t *)s.ptr(b),
+                                                                 n, sc, off, b.stream);
+                              }});
+      return Error::success();
+    }
     out.launches.push_back({"mi355x_dequantize_i8", I.name,
                             strFormat(" n=%zu scale=%.9g offset=%d", n, (double)sc, off),
                             [=](const DeviceBindings &b) {
@@ -658,7 +773,7 @@ private:
     return Error::success();
   }
 
-  Error rescale(const Instruction &I, MI355XFunction &out) {
+  Error rescale(const Instruction &I, MI355XFunction &out, const Instruction *ins = nullptr) {
     Operand d = op(I, 0), s = op(I, 1);
     CHECK_OP(d.ty().kind == ElemKind::Int8QTy && s.ty().kind == ElemKind::Int8QTy,
              "needs i8 -> i8");
@@ -666,6 +781,20 @@ private:
     const size_t n = (size_t)d.ty().size();
     const S32To8 p = s32to8(s.ty().scale / d.ty().scale);
     const int32_t oo = d.ty().offset, io = s.ty().offset;
+    if (ins) {
+      const SliceDest sd = sliceDest(*ins);
+      const size_t rows = (size_t)d.ty().dims[0], cols = (size_t)d.ty().dims[1];
+      out.launches.push_back(
+          {"mi355x_rescale_rows_i8", I.name + "+" + ins->name,
+           strFormat(" rows=%zu cols=%zu stride=%zu offset=%zu", rows, cols, sd.pitch, sd.offset) +
+               kv("out_offset", oo) + kv("in_offset", io) + kv("pre", p.pre) + kv("post", p.post) +
+               kv("scale", p.scale),
+           [=](const DeviceBindings &b) {
+             return mi355x_rescale_rows_i8((int8_t *)sd.wide.ptr(b) + sd.offset, (const int8_t *)s.ptr(b),
+                                           rows, cols, sd.pitch, oo, io, p.pre, p.post, p.scale, b.stream);
+           }});
+      return Error::success();
+    }
     out.launches.push_back(
         {"mi355x_rescale_i8", I.name,
          strFormat(" n=%zu", n) + kv("out_offset", oo) + kv("in_offset", io) +
@@ -1363,6 +1492,7 @@ private:
   std::shared_ptr<size_t> scratchBasePtr_ = std::make_shared<size_t>(0);
   std::map<int, std::pair<bool, bool>> io_; // value id -> (read, written)
   std::map<const Value *, TableView> paddedTables_;
+  std::vector<char> absorbed_; // instructions folded into the launch of an earlier one
 };
 
 constexpr int Compiler::kArity[];

@@ -151,6 +151,8 @@ struct BackendOptions {
   bool fuseTransposeMatMul = true;     // BatchMatMul(L, Transpose(R)) without materialising the transpose
   bool fuseFcRelu = true;              // RowwiseQuantizedFullyConnected + Relu of its result in one kernel
   bool padTableRows = true;            // constant lookup tables with 33..63-byte rows re-laid 64 bytes apart at load
+  bool fuseInsert = true;              // Gather / RescaleQuantized write straight into the tensor their result is inserted into
+  bool fuseDequantizeSigmoid = true;   // Dequantize + Sigmoid of its result in one kernel
 };
 
 class MI355XBackend {

@@ -190,6 +190,19 @@ int mi355x_dequantize_i8(float *dst, const int8_t *src, size_t n, float scale,
 int mi355x_rescale_i8(int8_t *dst, const int8_t *src, size_t n,
                       int32_t out_offset, int32_t in_offset, int32_t pre,
                       int32_t post, int32_t scale, void *stream);
+/* The same rescale of a [rows x cols] tensor, written as a slice of a wider
+ * tensor: row r goes to dst + r*dst_row_stride (the caller adds the slice's
+ * offset to dst). RescaleQuantized followed by the InsertTensor that is the
+ * only reader of its result (libjit.cpp:3031-3038, then libjit_insert_tensor
+ * :156-260) in one pass. */
+int mi355x_rescale_rows_i8(int8_t *dst, const int8_t *src, size_t rows, size_t cols,
+                           size_t dst_row_stride, int32_t out_offset, int32_t in_offset,
+                           int32_t pre, int32_t post, int32_t scale, void *stream);
+/* Dequantize (libjit.cpp:3016-3019) followed by Sigmoid (libjit.cpp:1913-1916)
+ * of its result in one pass; the dequantized value is the same fp32 number,
+ * the sigmoid agrees with the CPU to fp32 rounding of expf (1e-5 relative). */
+int mi355x_dequantize_sigmoid(float *dst, const int8_t *src, size_t n, float scale,
+                              int32_t offset, void *stream);
 
 /* ---- int8 glue operators ------------------------------------------------------ */
 
@@ -258,6 +271,12 @@ int mi355x_batch_transpose_i8(int8_t *dst, const int8_t *src, size_t batch, size
 int mi355x_gather(void *dst, const void *data, const void *indices, int idx_is_64,
                   size_t num_indices, size_t slice_bytes, size_t num_samples,
                   size_t sample_bytes, void *stream);
+/* The same gather with the samples of the result dst_sample_stride bytes apart
+ * (Gather followed by the InsertTensor that is the only reader of its result;
+ * the caller adds the slice's offset to dst). */
+int mi355x_gather_rows(void *dst, const void *data, const void *indices, int idx_is_64,
+                       size_t num_indices, size_t slice_bytes, size_t num_samples,
+                       size_t sample_bytes, size_t dst_sample_stride, void *stream);
 /* BatchMatMul of small int8 matrices, i.e. libjit_matmul_i8
  * (libjit_matmul.cpp:353-371) on every [M x K] x [K x N] pair of the batch (what
  * the node lowers to). (M + N) * K must not exceed 64 KiB. */

@@ -121,7 +121,10 @@ enum {
   MI355X_HOST_OPT_FUSE_FC_RELU = 64, /* RowwiseQuantizedFullyConnected + Relu in one kernel */
   MI355X_HOST_OPT_PAD_TABLE_ROWS = 128, /* constant lookup tables with rows of 33..63 bytes are copied
                                           at load time to rows 64 bytes apart */
-  MI355X_HOST_OPT_DEFAULT = 255
+  MI355X_HOST_OPT_FUSE_INSERT = 256, /* Gather / RescaleQuantized whose result is only inserted into a
+                                        wider tensor write there directly */
+  MI355X_HOST_OPT_FUSE_DEQUANTIZE_SIGMOID = 512, /* Dequantize + Sigmoid of its result in one kernel */
+  MI355X_HOST_OPT_DEFAULT = 1023
 };
 int mi355x_host_compile(mi355x_host_module *m, int function, int options);
 /* Listing of the compiled function's launches and derived parameters; returns

@@ -23,14 +23,20 @@ def test_builds_and_compiles():
     assert k.count("mi355x_frwq_sls_multi") == 1 and "mi355x_frwq_slws" not in k
     multi = rows[k.index("mi355x_frwq_sls_multi")]
     assert (multi["tables"], multi["out_kind"], multi["stride"]) == (3, 3, 4 * 16)
-    assert k.count("mi355x_convert_f16_to_f32") == 0 and k.count("mi355x_insert_rows") == 3
+    assert k.count("mi355x_convert_f16_to_f32") == 0
+    # no InsertTensor is left: the bottom MLP's rescaled output and the upper
+    # triangle of the interaction are written where they are inserted
+    assert k.count("mi355x_insert_rows") == 0 and k.count("mi355x_rescale_rows_i8") == 2
+    assert k.count("mi355x_gather_rows") == 1 and k.count("mi355x_gather") == 0
+    assert k[-1] == "mi355x_dequantize_sigmoid"
     # the interaction's Transpose + BatchMatMul read the features as they lie
     assert k.count("mi355x_batch_matmul_nt_i8") == 1 and k.count("mi355x_batch_transpose_i8") == 0
     assert k.count("mi355x_batch_matmul_i8") == 0
     # every hidden layer's Relu runs inside its FullyConnected
     assert k.count("mi355x_relu_i8") == 0 and k.count("mi355x_rwq_fc_relu_i8") >= 2
     m, f = netlib.to_module(net)
-    m.compile(f, fuse_sls_chains=False, fuse_transpose_matmul=False, fuse_fc_relu=False)
+    m.compile(f, fuse_sls_chains=False, fuse_transpose_matmul=False, fuse_fc_relu=False,
+              fuse_insert=False, fuse_dequantize_sigmoid=False)
     k = [r["kernel"] for r in H.parse_listing(m.describe(f)) if r["phase"] == "launch"]
     assert k.count("mi355x_frwq_slws") == 3 and k.count("mi355x_rwq_fc_i8") == 4
     assert k.count("mi355x_convert_f16_to_f32") == 3 and k.count("mi355x_insert_rows") == 6
@@ -80,7 +86,7 @@ def test_device_matches_oracle(fuse, pad):
     net, max_idx = dlrm.make(seed=3, **cfg)
     m, f = netlib.to_module(net)
     m.compile(f, fuse_sls_chains=fuse, fuse_transpose_matmul=fuse, fuse_fc_relu=fuse,
-              pad_table_rows=pad)
+              pad_table_rows=pad, fuse_insert=fuse, fuse_dequantize_sigmoid=fuse)
     dm = H.DeviceManager().init()
     try:
         dm.add_network(m)

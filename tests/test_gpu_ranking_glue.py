@@ -133,3 +133,44 @@ def test_batch_matmul_with_k_contiguous_right_operand(shape):
         want = go.batch_matmul_i8(lhs, np.ascontiguousarray(rhs_nk.transpose(0, 2, 1)), oo, lo, ro, outP)
         got = capi.batch_matmul_nt_i8(lhs, rhs_nk, oo, lo, ro, outP)
         np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("rows,cols,wide,col", [(33, 64, 200, 64), (7, 13, 29, 5), (1, 4, 4, 0),
+                                                (300, 16, 48, 32)])
+def test_rescale_written_as_a_slice(rows, cols, wide, col):
+    """RescaleQuantized + InsertTensor in one pass: the slice holds the oracle's
+    rescale, every other byte of the wide tensor is untouched."""
+    rng = np.random.default_rng(rows + cols)
+    q = rng.integers(-128, 128, (rows, cols)).astype(np.int8)
+    into = rng.integers(-128, 128, (rows, wide)).astype(np.int8)
+    for ratio, oo, io in [(1.7, 3, -4), (0.013, -128, 100), (300.0, 0, 0)]:
+        pre, post, scale, _ = go.quantize_scale_offset_32to8(ratio, 0)
+        want = into.copy()
+        want[:, col:col + cols] = go.rescale_i8(q, oo, io, pre, post, scale)
+        np.testing.assert_array_equal(capi.rescale_rows_i8(q, into, col, oo, io, pre, post, scale), want)
+
+
+@pytest.mark.parametrize("idt", [np.int32, np.int64])
+def test_gather_written_as_a_slice(idt):
+    rng = np.random.default_rng(8)
+    data = rng.integers(-128, 128, (33, 729)).astype(np.int8)
+    iu = np.triu_indices(27, 1)
+    idx = (iu[0] * 27 + iu[1]).astype(idt)
+    into = rng.integers(-128, 128, (33, 64 + idx.size + 3)).astype(np.int8)
+    want = into.copy()
+    want[:, 64:64 + idx.size] = go.gather(data, idx, 1)
+    np.testing.assert_array_equal(capi.gather_rows(data, idx, into, 64), want)
+    # wider slices (fp32 rows of 4 values)
+    table = rng.normal(0, 1, (20, 6, 4)).astype(np.float32)
+    pick = np.array([5, 0, 5, 2], idt)
+    into = np.zeros((20, 40), np.float32)
+    want = into.copy()
+    want[:, 8:24] = go.gather(table, pick, 1).reshape(20, 16)
+    np.testing.assert_array_equal(capi.gather_rows(table, pick, into, 8), want)
+
+
+def test_dequantize_then_sigmoid_in_one_pass():
+    q = np.arange(-128, 128).astype(np.int8).reshape(16, 16)
+    for scale, offset in [(0.05, 3), (0.7, -128), (1e-3, 127)]:
+        want = go.sigmoid_f32(go.dequantize_i8(q, scale, offset))
+        np.testing.assert_allclose(capi.dequantize_sigmoid(q, scale, offset), want, rtol=1e-5, atol=1e-37)

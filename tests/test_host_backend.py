@@ -243,3 +243,82 @@ def test_pool_parameters_and_checks():
     wrong = m.placeholder("wrong", (2, 4, 4, 16), H.INT8Q, np.int8, 0.06, -9)
     ok, why = m.is_op_supported(H.MAX_POOL, [wrong, x], attrs)
     assert not ok and "computed 5 x 5" in why
+
+
+def _slice_module(between=None, second_reader=False, y_is_placeholder=False):
+    """x --Rescale--> y --InsertTensor(cols 5..20)--> wide, optionally with
+    another instruction between the two."""
+    m = H.Module()
+    x = m.placeholder("x", (8, 16), H.INT8Q, np.int8, 0.30, 2)
+    x2 = m.placeholder("x2", (8, 5), H.INT8Q, np.int8, 0.11, -3)
+    wide = m.placeholder("wide", (8, 40), H.INT8Q, np.int8, 0.11, -3)
+    spare = m.placeholder("spare", (8, 40), H.INT8Q, np.int8, 0.2, 0)
+    spare16 = m.placeholder("spare16", (8, 16), H.INT8Q, np.int8, 0.2, 0)
+    f = m.function("main")
+    y = (m.placeholder("y", (8, 16), H.INT8Q, np.int8, 0.11, -3) if y_is_placeholder
+         else m.activation(f, "y", (8, 16), H.INT8Q, 0.11, -3))
+    m.instruction(f, H.RESCALE_QUANTIZED, "r", [y, x])
+    if between == "reads_wide":
+        m.instruction(f, H.RESCALE_QUANTIZED, "peek", [spare, wide])
+    elif between == "other_columns":
+        m.instruction(f, H.INSERT_TENSOR, "left", [wide, x2], [0])
+    elif between == "same_columns":
+        m.instruction(f, H.INSERT_TENSOR, "clash", [wide, x2], [18])
+    m.instruction(f, H.INSERT_TENSOR, "ins", [wide, y], [5])
+    if second_reader:
+        m.instruction(f, H.RESCALE_QUANTIZED, "again", [spare16, y])
+    return m, f
+
+
+def test_insert_is_folded_into_the_producer_only_when_nothing_can_tell():
+    def kernels(**kw):
+        m, f = _slice_module(**kw)
+        m.compile(f)
+        return [(r["kernel"], r["inst"]) for r in H.parse_listing(m.describe(f)) if r["phase"] == "launch"]
+    assert kernels() == [("mi355x_rescale_rows_i8", "r+ins")]
+    m, f = _slice_module()
+    m.compile(f)
+    r = _launch(m, f, "mi355x_rescale_rows_i8")
+    assert (r["rows"], r["cols"], r["stride"], r["offset"]) == (8, 16, 40, 5)
+    pre, post, scale, _ = go.quantize_scale_offset_32to8(float(np.float32(0.30) / np.float32(0.11)), 0)
+    assert (r["pre"], r["post"], r["scale"], r["in_offset"], r["out_offset"]) == (pre, post, scale, 2, -3)
+    # an insert of other columns in between does not stand in the way
+    assert kernels(between="other_columns") == [("mi355x_rescale_rows_i8", "r+ins"),
+                                                 ("mi355x_insert_rows", "left")]
+    # a reader of the wide tensor, an insert overlapping the slice, a second
+    # reader of the result, or a result the caller can see: two launches
+    for kw in (dict(between="reads_wide"), dict(between="same_columns"), dict(second_reader=True),
+               dict(y_is_placeholder=True)):
+        k = [n for n, _ in kernels(**kw)]
+        assert "mi355x_rescale_rows_i8" not in k and k.count("mi355x_rescale_i8") >= 1, kw
+    m, f = _slice_module()
+    m.compile(f, fuse_insert=False)
+    assert [r["kernel"] for r in H.parse_listing(m.describe(f)) if r["phase"] == "launch"] == \
+        ["mi355x_rescale_i8", "mi355x_insert_rows"]
+
+
+def test_dequantize_and_sigmoid_become_one_launch():
+    def build(extra_reader):
+        m = H.Module()
+        q = m.placeholder("q", (6, 3), H.INT8Q, np.int8, 0.04, 7)
+        p = m.placeholder("p", (6, 3), H.FLOAT, np.float32)
+        p2 = m.placeholder("p2", (6, 3), H.FLOAT, np.float32)
+        f = m.function("main")
+        x = m.activation(f, "x", (6, 3), H.FLOAT)
+        m.instruction(f, H.DEQUANTIZE, "deq", [x, q])
+        m.instruction(f, H.SIGMOID, "sig", [p, x])
+        if extra_reader:
+            m.instruction(f, H.SIGMOID, "sig2", [p2, x])
+        return m, f
+    m, f = build(False)
+    m.compile(f)
+    r = _launch(m, f, "mi355x_dequantize_sigmoid")
+    assert (r["inst"], r["n"], r["offset"]) == ("deq+sig", 18, 7) and abs(r["scale"] - 0.04) < 1e-7
+    m, f = build(True)
+    m.compile(f)
+    assert [r["kernel"] for r in H.parse_listing(m.describe(f))] == \
+        ["mi355x_dequantize_i8", "mi355x_sigmoid_f32", "mi355x_sigmoid_f32"]
+    m, f = build(False)
+    m.compile(f, fuse_dequantize_sigmoid=False)
+    assert [r["kernel"] for r in H.parse_listing(m.describe(f))] == \
+        ["mi355x_dequantize_i8", "mi355x_sigmoid_f32"]
