@@ -217,10 +217,32 @@ struct DenseRows {
         const Chunk c = *reinterpret_cast<const Chunk *>(r.base + k);
         return make_int4(c.x, c.y, c.z, c.w);
       }
+      // The row's last, partial chunk (n = K - k bytes, 1..15), without a
+      // chain of dependent byte loads.
+      const int n = K - k;
+      if (K >= 16) {
+        // the 16 bytes that end with the row, moved down by 16 - n bytes
+        struct __attribute__((packed, aligned(1))) Chunk { uint32_t x, y, z, w; };
+        const Chunk c = *reinterpret_cast<const Chunk *>(r.base + K - 16);
+        const int s = 16 - n, ws = s >> 2, bs = (s & 3) * 8;
+        const uint32_t in[8] = {c.x, c.y, c.z, c.w, 0, 0, 0, 0};
+        uint32_t t[5];
+#pragma unroll
+        for (int j = 0; j < 5; j++)
+          t[j] = ws == 0 ? in[j] : ws == 1 ? in[j + 1] : ws == 2 ? in[j + 2] : in[j + 3];
+        uint32_t o[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) o[j] = __funnelshift_r(t[j], t[j + 1], bs);
+        return make_int4((int)o[0], (int)o[1], (int)o[2], (int)o[3]);
+      }
+      // rows shorter than a chunk: every byte on its own, all loads in flight
+      // (slots beyond the row re-read its last byte and are masked)
       uint32_t w[4] = {0, 0, 0, 0};
-      const int n = min(16, K - k);
-      for (int b = 0; b < n; b++)
-        w[b >> 2] |= (uint32_t)(uint8_t)r.base[k + b] << (8 * (b & 3));
+#pragma unroll
+      for (int b = 0; b < 16; b++) {
+        const uint32_t v = (uint8_t)r.base[k + min(b, n - 1)];
+        w[b >> 2] |= (b < n ? v : 0u) << (8 * (b & 3));
+      }
       return make_int4((int)w[0], (int)w[1], (int)w[2], (int)w[3]);
     }
   }
@@ -469,69 +491,78 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_i8_kernel(
   for (int j = 0; j < TN; j++) sb[j] = 0;
 
   const int KT = (K + kBK - 1) / kBK;
-  int4 ra[A_CH], rb[B_CH];
+  // Tiles are fetched into registers D K-steps ahead of their use (small tiles
+  // have the registers for it): a step of this loop is short, so with one tile
+  // in flight every step would wait out a full memory round trip.
+  constexpr int D = (A_CH + B_CH <= 2) ? 3 : (A_CH + B_CH <= 4) ? 2 : 1;
+  int4 ra[D][A_CH], rb[D][B_CH];
+  auto fetch = [&](int slot, int kt) {
+    const int k0 = kt * kBK;
 #pragma unroll
-  for (int i = 0; i < A_CH; i++) ra[i] = A.template load<AL_A>(arow[i], a_k[i], K);
+    for (int i = 0; i < A_CH; i++) ra[slot][i] = A.template load<AL_A>(arow[i], k0 + a_k[i], K);
 #pragma unroll
-  for (int i = 0; i < B_CH; i++) rb[i] = B.template load<AL_B>(brow[i], b_k[i], K);
+    for (int i = 0; i < B_CH; i++) rb[slot][i] = B.template load<AL_B>(brow[i], k0 + b_k[i], K);
+  };
+  auto park = [&](int slot, int8_t *stage) {
 #pragma unroll
-  for (int i = 0; i < A_CH; i++) *reinterpret_cast<int4 *>(lds + a_lds[i]) = ra[i];
+    for (int i = 0; i < A_CH; i++) *reinterpret_cast<int4 *>(stage + a_lds[i]) = ra[slot][i];
 #pragma unroll
-  for (int i = 0; i < B_CH; i++) *reinterpret_cast<int4 *>(lds + b_lds[i]) = rb[i];
+    for (int i = 0; i < B_CH; i++) *reinterpret_cast<int4 *>(stage + b_lds[i]) = rb[slot][i];
+  };
+  fetch(0, 0);
+  park(0, lds);
+  // tiles 1..D on their way; tile t lives in register slot (t - 1) % D
+#pragma unroll
+  for (int t = 1; t <= D; t++)
+    if (t < KT) fetch((t - 1) % D, t);
   __syncthreads();
 
   const int a_frag = (wm * WM + l32) * kLdsStride + lhi * 16;
   const int b_frag = (BM + wn * WN + l32) * kLdsStride + lhi * 16;
 
-  for (int kt = 0; kt < KT; kt++) {
-    const int8_t *cur = lds + (kt & 1) * STAGE;
-    const bool more = kt + 1 < KT;
-    if (more) {
-      const int k0 = (kt + 1) * kBK;
+  for (int kb = 0; kb < KT; kb += D) {
 #pragma unroll
-      for (int i = 0; i < A_CH; i++)
-        ra[i] = A.template load<AL_A>(arow[i], k0 + a_k[i], K);
+    for (int u = 0; u < D; u++) {
+      const int kt = kb + u;
+      if (kt >= KT) break;
+      const int8_t *cur = lds + (kt & 1) * STAGE;
 #pragma unroll
-      for (int i = 0; i < B_CH; i++)
-        rb[i] = B.template load<AL_B>(brow[i], k0 + b_k[i], K);
-    }
+      for (int ks = 0; ks < kBK / 32; ks++) {
+        v4i af[TM], bf[TN];
 #pragma unroll
-    for (int ks = 0; ks < kBK / 32; ks++) {
-      v4i af[TM], bf[TN];
+        for (int i = 0; i < TM; i++)
+          af[i] = *reinterpret_cast<const v4i *>(cur + a_frag + i * 32 * kLdsStride + ks * 32);
 #pragma unroll
-      for (int i = 0; i < TM; i++)
-        af[i] = *reinterpret_cast<const v4i *>(cur + a_frag + i * 32 * kLdsStride + ks * 32);
+        for (int j = 0; j < TN; j++)
+          bf[j] = *reinterpret_cast<const v4i *>(cur + b_frag + j * 32 * kLdsStride + ks * 32);
+        if constexpr (NEED_SA) {
 #pragma unroll
-      for (int j = 0; j < TN; j++)
-        bf[j] = *reinterpret_cast<const v4i *>(cur + b_frag + j * 32 * kLdsStride + ks * 32);
-      if constexpr (NEED_SA) {
+          for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+              sa[i] = __builtin_amdgcn_sdot4(af[i][q], 0x01010101, sa[i], false);
+        }
+        if constexpr (NEED_SB) {
+#pragma unroll
+          for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+              sb[j] = __builtin_amdgcn_sdot4(bf[j][q], 0x01010101, sb[j], false);
+        }
 #pragma unroll
         for (int i = 0; i < TM; i++)
 #pragma unroll
-          for (int q = 0; q < 4; q++)
-            sa[i] = __builtin_amdgcn_sdot4(af[i][q], 0x01010101, sa[i], false);
+          for (int j = 0; j < TN; j++)
+            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
       }
-      if constexpr (NEED_SB) {
-#pragma unroll
-        for (int j = 0; j < TN; j++)
-#pragma unroll
-          for (int q = 0; q < 4; q++)
-            sb[j] = __builtin_amdgcn_sdot4(bf[j][q], 0x01010101, sb[j], false);
+      if (kt + 1 < KT) {
+        // tile kt+1 sits in slot u (it was fetched D steps ago); the slot then
+        // takes tile kt+1+D
+        park(u, lds + ((kt + 1) & 1) * STAGE);
+        if (kt + 1 + D < KT) fetch(u, kt + 1 + D);
       }
-#pragma unroll
-      for (int i = 0; i < TM; i++)
-#pragma unroll
-        for (int j = 0; j < TN; j++)
-          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
+      __syncthreads();
     }
-    if (more) {
-      int8_t *nxt = lds + ((kt + 1) & 1) * STAGE;
-#pragma unroll
-      for (int i = 0; i < A_CH; i++) *reinterpret_cast<int4 *>(nxt + a_lds[i]) = ra[i];
-#pragma unroll
-      for (int i = 0; i < B_CH; i++) *reinterpret_cast<int4 *>(nxt + b_lds[i]) = rb[i];
-    }
-    __syncthreads();
   }
 
   gemm_epilogue<BM, BN, WM, WN, NEED_SA, NEED_SB>(acc, sa, sb, lds, ep, M, N, K,

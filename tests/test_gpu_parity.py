@@ -120,6 +120,18 @@ def test_rwq_fc_vs_oracle(shape):
                                   go.rwq_fc_i8(*cases.rwq_fc_args(c)))
 
 
+def test_rwq_fc_every_row_length_up_to_three_chunks():
+    """Rows that are not a whole number of 16-byte chunks: every remainder 1..15
+    both for rows shorter than one chunk and for longer ones (the last chunk is
+    read as the 16 bytes that end with the row and shifted down)."""
+    for K in range(1, 50):
+        for M, N in [(9, 5), (70, 66)]:
+            c = cases.rwq_fc_case(1000 + K, M, K, N, symmetric=False)
+            want = go.rwq_fc_i8(*cases.rwq_fc_args(c))
+            got = capi.rwq_fc_i8(*cases.rwq_fc_args(c), precomputed_sums=False)
+            assert np.array_equal(got, want), (M, K, N)
+
+
 @pytest.mark.parametrize("shape", [(128, 1024, 1024), (300, 13, 512), (77, 415, 96), (4096, 512, 256)])
 def test_rwq_fc_with_fused_relu(shape):
     """RowwiseQuantizedFullyConnected + Relu in one kernel equals the two
