@@ -157,6 +157,26 @@ def bench_slws_with_h2d(capi, s, args, d_table):
                 h2d_bytes_per_step=s["mean_lookups"] * 12 + bags * 4)
 
 
+def bench_slws_more_bags(capi, cases, args, d_table, bags):
+    """The headline lookup on the same table with a larger batch: the part of a
+    launch that does not shrink with the batch (dispatch, bag offsets, the
+    index -> row dependent round trips) is spread over more bytes."""
+    rows, cols = args.rows, 128
+    lengths, idx, w = cases.slws_batch(2000 + bags, rows, bags, 40, 1.05, np.int64)
+    total = int(lengths.sum())
+    d_len, d_idx, d_w = capi.to_device(lengths), capi.to_device(idx), capi.to_device(w)
+    d_out = capi.DeviceBuffer.empty((bags, cols), np.float32)
+
+    def step(_, stream):
+        capi.launch_frwq_slws(d_out, False, d_table, rows, capi.FUSED_U8_F32, d_w, False, d_idx,
+                              True, total, d_len, bags, cols + 8, cols, stream=stream)
+
+    sec = timed_launches(capi, step, max(20, args.steps // 4), max(3, args.warmup // 4))
+    nbytes = slws_bytes(total, bags, cols, cols + 8)
+    return dict(workload=f"SLWS, same table, {bags} bags ({total} lookups)", ms=sec * 1e3,
+                gbps=nbytes / sec / 1e9, frac_of_hbm_peak=nbytes / sec / 1e9 / HBM_PEAK_GBPS)
+
+
 def cpu_all_cores_slws(table, batches, budget_s):
     """The oracle on every host core this process may use, one whole batch per
     thread at a time (the reference's CPU backend exposes one device per
@@ -509,6 +529,8 @@ def main():
     if not args.no_extra and not only:
         st, wu = max(20, args.steps // 4), max(3, args.warmup // 4)
         extra["slws_with_h2d"] = bench_slws_with_h2d(capi, s, args, d_table)
+        extra["slws_more_bags"] = [bench_slws_more_bags(capi, cases, args, d_table, n)
+                                   for n in (16384, 65536)]
         if args.cpu_seconds > 0:
             extra["cpu_all_cores"] = cpu_all_cores_slws(table, s["batches"],
                                                         args.cpu_seconds / 2)
