@@ -24,7 +24,7 @@ EXPORTS = [
     "mi355x_host_free", "mi355x_memcpy_h2d", "mi355x_memcpy_d2h",
     "mi355x_memcpy_d2d", "mi355x_fill_u8", "mi355x_copy_u8", "mi355x_gemm_tile_override",
     "mi355x_cwq_conv2d_add_i8", "mi355x_frwq_sls_multi",
-    "mi355x_specialize_bias_weights_qparams", "mi355x_rwq_slws", "mi355x_slws_set_fused_math", "mi355x_batch_matmul_nt_i8", "mi355x_rwq_fc_relu_i8", "mi355x_add_i8", "mi355x_add_relu_i8",
+    "mi355x_specialize_bias_weights_qparams", "mi355x_rwq_slws", "mi355x_slws_set_fused_math", "mi355x_batch_matmul_nt_i8", "mi355x_batch_matmul_nt_select_i8", "mi355x_rwq_fc_relu_i8", "mi355x_add_i8", "mi355x_add_relu_i8",
     "mi355x_relu_i8", "mi355x_convert_f16_to_f32", "mi355x_insert_rows",
     "mi355x_batch_transpose_i8", "mi355x_space_to_depth2_i8", "mi355x_gather", "mi355x_gather_rows", "mi355x_rescale_rows_i8",
     "mi355x_dequantize_sigmoid", "mi355x_batch_matmul_i8", "mi355x_sigmoid_f32",
@@ -1007,6 +1007,24 @@ def batch_matmul_nt_i8(lhs, rhs_nk, out_offset, lhs_offset, rhs_offset, outP):
     check(lib().mi355x_batch_matmul_nt_i8(_vp(out), _vp(dl), _vp(dr), _sz(b), _sz(m), _sz(k),
                                           _sz(n), _i32(out_offset), _i32(lhs_offset),
                                           _i32(rhs_offset), *_i32s(outP), _vp(None)))
+    return out.numpy()
+
+
+def batch_matmul_nt_select_i8(lhs, rhs_nk, out_offset, lhs_offset, rhs_offset, outP, dest_of,
+                              into, col):
+    """The product's elements e with dest_of[e] >= 0 written into the 2-D int8
+    array `into` at column col + dest_of[e]; returns the updated array."""
+    lhs = np.ascontiguousarray(lhs, np.int8)
+    rhs_nk = np.ascontiguousarray(rhs_nk, np.int8)
+    b, m, k = lhs.shape
+    n = rhs_nk.shape[1]
+    dest_of = np.ascontiguousarray(dest_of, np.int32)
+    assert dest_of.size == m * n
+    into = np.ascontiguousarray(into, np.int8)
+    dl, dr, dd, out = to_device(lhs), to_device(rhs_nk), to_device(dest_of), to_device(into)
+    check(lib().mi355x_batch_matmul_nt_select_i8(
+        _vp(out.ptr + col), _vp(dl), _vp(dr), _sz(b), _sz(m), _sz(k), _sz(n), _i32(out_offset),
+        _i32(lhs_offset), _i32(rhs_offset), *_i32s(outP), _vp(dd), _sz(into.shape[1]), _vp(None)))
     return out.numpy()
 
 

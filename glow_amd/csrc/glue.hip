@@ -413,13 +413,15 @@ typedef int nt_v16i __attribute__((ext_vector_type(16)));
 __global__ __launch_bounds__(kGlueThreads) void batch_matmul_nt_i8_kernel(
     int8_t *__restrict__ out, const int8_t *__restrict__ lhs, const int8_t *__restrict__ rhs,
     long long batch, int M, int K, int N, int32_t oo, int32_t lo, int32_t ro, int32_t pre,
-    int32_t post, int32_t scale) {
+    int32_t post, int32_t scale, const int32_t *__restrict__ dest_of, long long out_stride) {
+  // dest_of (optional): where in the sample's output row element (m, n) goes,
+  // negative = nowhere; without it the whole matrix is written
   const int lane = threadIdx.x & 63;
   const long long b = (long long)blockIdx.x * (kGlueThreads / 64) + (threadIdx.x >> 6);
   if (b >= batch) return;
   const int l32 = lane & 31, lhi = lane >> 5;
   const int8_t *L = lhs + b * (long long)M * K, *R = rhs + b * (long long)N * K;
-  int8_t *O = out + b * (long long)M * N;
+  int8_t *O = out + b * out_stride;
   const uint32_t kconst = (uint32_t)K * (uint32_t)lo * (uint32_t)ro;
   for (int tm = 0; tm < M; tm += 32) {
     for (int tn = 0; tn < N; tn += 32) {
@@ -453,7 +455,11 @@ __global__ __launch_bounds__(kGlueThreads) void batch_matmul_nt_i8_kernel(
         const int row_sum = __shfl(sa, ml, 64);
         const uint32_t v = (uint32_t)acc[r] + colc - (uint32_t)ro * (uint32_t)row_sum;
         const int32_t y = clip_i8(scale_i32((int32_t)v, pre, post, scale, oo));
-        if (tm + ml < M && b_ok) O[(long long)(tm + ml) * N + tn + l32] = (int8_t)y;
+        if (tm + ml < M && b_ok) {
+          const int at = (tm + ml) * N + tn + l32;
+          const int to = dest_of ? dest_of[at] : at;
+          if (to >= 0) O[to] = (int8_t)y;
+        }
       }
     }
   }
@@ -783,8 +789,21 @@ int mi355x_batch_matmul_nt_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs_
                               size_t M, size_t K, size_t N, int32_t out_offset,
                               int32_t lhs_offset, int32_t rhs_offset, int32_t out_pre,
                               int32_t out_post, int32_t out_scale, void *stream) {
+  return mi355x_batch_matmul_nt_select_i8(out, lhs, rhs_nk, batch, M, K, N, out_offset, lhs_offset,
+                                          rhs_offset, out_pre, out_post, out_scale, nullptr, M * N,
+                                          stream);
+}
+
+int mi355x_batch_matmul_nt_select_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs_nk,
+                                     size_t batch, size_t M, size_t K, size_t N,
+                                     int32_t out_offset, int32_t lhs_offset, int32_t rhs_offset,
+                                     int32_t out_pre, int32_t out_post, int32_t out_scale,
+                                     const int32_t *dest_of, size_t out_sample_stride,
+                                     void *stream) {
   if (batch == 0 || M == 0 || N == 0) return MI355X_OK;
   MI355X_REQUIRE(out && lhs && rhs_nk, "NULL tensor");
+  MI355X_REQUIRE(out_sample_stride < (1ull << 40), "output stride too large");
+  MI355X_REQUIRE(dest_of || out_sample_stride >= M * N, "output samples overlap");
   MI355X_REQUIRE(shift_ok(out_pre) && shift_ok(out_post), "pre/post shift outside [0, 31]");
   MI355X_REQUIRE(K > 0 && K % 16 == 0 && K < (1u << 20) && M < (1u << 15) && N < (1u << 15),
                  "needs K %% 16 == 0 and matrices below 32768 rows (K = %zu)", K);
@@ -794,7 +813,7 @@ int mi355x_batch_matmul_nt_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs_
   hipLaunchKernelGGL(batch_matmul_nt_i8_kernel, dim3((unsigned)((batch + per_block - 1) / per_block)),
                      dim3(kGlueThreads), 0, as_stream(stream), out, lhs, rhs_nk, (long long)batch,
                      (int)M, (int)K, (int)N, out_offset, lhs_offset, rhs_offset, out_pre, out_post,
-                     out_scale);
+                     out_scale, dest_of, (long long)out_sample_stride);
   return check_launch("batch_matmul_nt_i8");
 }
 

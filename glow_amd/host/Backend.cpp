@@ -134,7 +134,15 @@ public:
             I.iattrs == std::vector<int64_t>{0, 2, 1} &&
             M_.value(I.operands[0]).category == SymbolCategory::Activation &&
             readers(I.operands[0]) == 1 && matmulNtOk(I, insts_[at + 1])) {
-          MI355X_RETURN_IF_ERR(matmulNt(I, insts_[at + 1], out));
+          // ... and a Gather of single elements of the product (then maybe the
+          // InsertTensor of what it gathers) behind it
+          std::vector<int32_t> destOf;
+          const size_t g = opts_.fuseInsert ? soleGatherOf(at + 1, destOf) : 0;
+          const size_t ins = g ? soleInsertOf(at + 1, insts_[g].operands[0], insts_[at + 1]) : 0;
+          MI355X_RETURN_IF_ERR(matmulNt(I, insts_[at + 1], out, g ? &insts_[g] : nullptr, destOf,
+                                        ins ? &insts_[ins] : nullptr));
+          if (g) { absorbed_[g] = 1; folded.push_back(g); }
+          if (ins) { absorbed_[ins] = 1; folded.push_back(ins); }
           at++;
         } else {
           MI355X_RETURN_IF_ERR(movement(I, out));
@@ -342,9 +350,11 @@ private:
   // 2-D result of instruction `at` and can take effect at `at` already: nothing
   // in between reads the tensor it inserts into, and whatever writes that
   // tensor in between is an InsertTensor of other columns.
-  size_t soleInsertOf(size_t at) const {
-    const Instruction &P = insts_[at];
-    const int v = P.operands[0];
+  size_t soleInsertOf(size_t at) const { return soleInsertOf(at, insts_[at].operands[0], insts_[at]); }
+
+  // The same for value `v`, which launch `P` at position `at` is going to write
+  // (P's own result, or that of an instruction folded into P).
+  size_t soleInsertOf(size_t at, int v, const Instruction &P) const {
     const Value &pv = M_.value(v);
     if (pv.category != SymbolCategory::Activation || pv.root != v || pv.type.dims.size() != 2 ||
         readers(v) != 1 || writers(v) != 1)
@@ -656,12 +666,89 @@ private:
            M_.value(T.operands[1]).offset % 16 == 0 && M_.value(B.operands[1]).offset % 16 == 0;
   }
 
-  Error matmulNt(const Instruction &T, const Instruction &I, MI355XFunction &out) {
+  // The Gather (its position, 0 if none) that is the only reader of the result
+  // of the BatchMatMul at `at`, picks single elements of each sample's flattened
+  // matrix by a constant list without repeats, and keeps the quantization
+  // parameters: the product can then write the picked elements directly.
+  // `destOf` receives, per element of a sample's matrix, its place in the
+  // gathered row or -1.
+  size_t soleGatherOf(size_t at, std::vector<int32_t> &destOf) const {
+    const Instruction &P = insts_[at];
+    const int z = P.operands[0];
+    const Value &zv = M_.value(z);
+    if (zv.category != SymbolCategory::Activation || zv.root != z || zv.type.dims.size() != 3 ||
+        readers(z) != 1 || writers(z) != 1)
+      return 0;
+    size_t j = at + 1;
+    for (; j < insts_.size(); j++) {
+      bool touches = false;
+      for (size_t i = 0; i < insts_[j].operands.size(); i++)
+        touches = touches || M_.value(insts_[j].operands[i]).root == z;
+      if (touches) break;
+    }
+    if (j >= insts_.size()) return 0;
+    const Instruction &G = insts_[j];
+    if (G.kind != Kind::Gather || G.iattrs != std::vector<int64_t>{1}) return 0;
+    const Value &src = M_.value(G.operands[1]), &idx = M_.value(G.operands[2]),
+                &dst = M_.value(G.operands[0]);
+    const int64_t per = zv.type.dims[1] * zv.type.dims[2];
+    if (src.root != z || src.offset != zv.offset || src.type.dims.size() != 2 ||
+        src.type.dims[0] != zv.type.dims[0] || src.type.dims[1] != per ||
+        src.type.kind != ElemKind::Int8QTy)
+      return 0;
+    if (idx.category != SymbolCategory::Constant || idx.type.dims.size() != 1 ||
+        (idx.type.kind != ElemKind::Int64ITy && idx.type.kind != ElemKind::Int32ITy))
+      return 0;
+    if (dst.category != SymbolCategory::Activation || dst.root != G.operands[0] ||
+        dst.type.kind != ElemKind::Int8QTy || dst.type.dims.size() != 2 ||
+        dst.type.dims[0] != zv.type.dims[0] || dst.type.dims[1] != idx.type.dims[0] ||
+        dst.type.scale != zv.type.scale || dst.type.offset != zv.type.offset ||
+        writers(G.operands[0]) != 1)
+      return 0;
+    for (size_t k = at + 1; k < j; k++)
+      for (size_t i = 0; i < insts_[k].operands.size(); i++)
+        if (M_.value(insts_[k].operands[i]).root == dst.root) return 0;
+    destOf.assign((size_t)per, -1);
+    const Operand io{&idx};
+    for (int64_t k = 0; k < idx.type.dims[0]; k++) {
+      const int64_t e = idx.type.kind == ElemKind::Int64ITy ? constData<int64_t>(io)[k]
+                                                            : (int64_t)constData<int32_t>(io)[k];
+      if (e < 0 || e >= per || destOf[(size_t)e] >= 0) return 0;
+      destOf[(size_t)e] = (int32_t)k;
+    }
+    return j;
+  }
+
+  // Transpose + BatchMatMul, optionally with the Gather `G` of single elements
+  // (destOf as soleGatherOf fills it) and the InsertTensor `ins` of the gathered
+  // rows folded in.
+  Error matmulNt(const Instruction &T, const Instruction &I, MI355XFunction &out,
+                 const Instruction *G = nullptr, const std::vector<int32_t> &destOf = {},
+                 const Instruction *ins = nullptr) {
     Operand d = op(I, 0), s = op(I, 1), r = op(T, 1);
     const size_t B = (size_t)s.ty().dims[0], M = (size_t)s.ty().dims[1], K = (size_t)s.ty().dims[2],
                  N = (size_t)r.ty().dims[1];
     const S32To8 p = s32to8(s.ty().scale * r.ty().scale / d.ty().scale);
     const int32_t oo = d.ty().offset, lo = s.ty().offset, ro = r.ty().offset;
+    if (G) {
+      Operand picked = op(*G, 0);
+      SliceDest sd{picked, 0, (size_t)picked.ty().dims[1]};
+      if (ins) sd = sliceDest(*ins);
+      const size_t map = gen_.addI32(destOf);
+      out.launches.push_back(
+          {"mi355x_batch_matmul_nt_select_i8", I.name + "+" + G->name + (ins ? "+" + ins->name : ""),
+           strFormat(" B=%zu M=%zu K=%zu N=%zu picked=%zu stride=%zu offset=%zu", B, M, K, N,
+                     (size_t)picked.ty().dims[1], sd.pitch, sd.offset) +
+               kv("out_offset", oo) + kv("lhs_offset", lo) + kv("rhs_offset", ro) + kv("out_pre", p.pre) +
+               kv("out_post", p.post) + kv("out_scale", p.scale),
+           [=](const DeviceBindings &b) {
+             return mi355x_batch_matmul_nt_select_i8(
+                 (int8_t *)sd.wide.ptr(b) + sd.offset, (const int8_t *)s.ptr(b), (const int8_t *)r.ptr(b),
+                 B, M, K, N, oo, lo, ro, p.pre, p.post, p.scale, (const int32_t *)(b.generated + map),
+                 sd.pitch, b.stream);
+           }});
+      return Error::success();
+    }
     out.launches.push_back({"mi355x_batch_matmul_nt_i8", I.name,
                             strFormat(" B=%zu M=%zu K=%zu N=%zu", B, M, K, N) + kv("out_offset", oo) +
                                 kv("lhs_offset", lo) + kv("rhs_offset", ro) + kv("out_pre", p.pre) +

@@ -294,6 +294,20 @@ int mi355x_batch_matmul_nt_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs_
                               size_t M, size_t K, size_t N, int32_t out_offset,
                               int32_t lhs_offset, int32_t rhs_offset, int32_t out_pre,
                               int32_t out_post, int32_t out_scale, void *stream);
+/* The same product of which only chosen elements are kept: element (m, n) of
+ * sample b goes to out[b*out_sample_stride + dest_of[m*N + n]] when that entry
+ * of the DEVICE array dest_of[M*N] is not negative (the caller keeps the
+ * entries below out_sample_stride and free of repeats). BatchMatMul followed by
+ * a Gather of single elements with a constant index list (libjit_gather,
+ * libjit.cpp:418-440) and possibly the InsertTensor of the gathered rows, in
+ * one pass; dest_of NULL writes the whole matrix. No counterpart in the
+ * reference. */
+int mi355x_batch_matmul_nt_select_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs_nk,
+                                     size_t batch, size_t M, size_t K, size_t N,
+                                     int32_t out_offset, int32_t lhs_offset, int32_t rhs_offset,
+                                     int32_t out_pre, int32_t out_post, int32_t out_scale,
+                                     const int32_t *dest_of, size_t out_sample_stride,
+                                     void *stream);
 /* Space-to-depth by 2 of a padded NHWC int8 image, the layout change that turns
  * a stride-2 convolution over few channels into a stride-1 convolution over
  * 4x the channels (SpaceToDepth with block size 2, plus padding):

@@ -27,10 +27,14 @@ def test_builds_and_compiles():
     # no InsertTensor is left: the bottom MLP's rescaled output and the upper
     # triangle of the interaction are written where they are inserted
     assert k.count("mi355x_insert_rows") == 0 and k.count("mi355x_rescale_rows_i8") == 2
-    assert k.count("mi355x_gather_rows") == 1 and k.count("mi355x_gather") == 0
+    # ... the interaction writes the picked pairs itself
+    assert k.count("mi355x_gather_rows") == 0 and k.count("mi355x_gather") == 0
+    sel = rows[k.index("mi355x_batch_matmul_nt_select_i8")]
+    assert (sel["inst"], sel["picked"], sel["stride"], sel["offset"]) == \
+        ("interact+upper_triangle+insert_pairs", 6, 22, 16)
     assert k[-1] == "mi355x_dequantize_sigmoid"
     # the interaction's Transpose + BatchMatMul read the features as they lie
-    assert k.count("mi355x_batch_matmul_nt_i8") == 1 and k.count("mi355x_batch_transpose_i8") == 0
+    assert k.count("mi355x_batch_matmul_nt_select_i8") == 1 and k.count("mi355x_batch_transpose_i8") == 0
     assert k.count("mi355x_batch_matmul_i8") == 0
     # every hidden layer's Relu runs inside its FullyConnected
     assert k.count("mi355x_relu_i8") == 0 and k.count("mi355x_rwq_fc_relu_i8") >= 2

@@ -174,3 +174,24 @@ def test_dequantize_then_sigmoid_in_one_pass():
     for scale, offset in [(0.05, 3), (0.7, -128), (1e-3, 127)]:
         want = go.sigmoid_f32(go.dequantize_i8(q, scale, offset))
         np.testing.assert_allclose(capi.dequantize_sigmoid(q, scale, offset), want, rtol=1e-5, atol=1e-37)
+
+
+@pytest.mark.parametrize("b,m,k,n", [(64, 27, 64, 27), (5, 40, 32, 33), (3, 4, 16, 9)])
+def test_product_of_which_only_picked_elements_are_written(b, m, k, n):
+    """BatchMatMul + Gather of single elements + InsertTensor in one pass: the
+    picked elements of the oracle's product land where the list says, the rest
+    of the wide tensor is untouched."""
+    rng = np.random.default_rng(b * m)
+    lhs = rng.integers(-128, 128, (b, m, k)).astype(np.int8)
+    rhs = rng.integers(-128, 128, (b, n, k)).astype(np.int8)
+    pick = rng.permutation(m * n)[: max(1, (m * n) // 3)].astype(np.int64)
+    dest_of = np.full(m * n, -1, np.int32)
+    dest_of[pick] = np.arange(pick.size, dtype=np.int32)
+    into = rng.integers(-128, 128, (b, pick.size + 11)).astype(np.int8)
+    for oo, lo, ro, ratio in [(3, -4, 5, 0.004), (-128, 0, 0, 0.0007)]:
+        p = go.quantize_scale_offset_32to8(ratio, 0)[:3]
+        z = go.batch_matmul_i8(lhs, np.ascontiguousarray(rhs.transpose(0, 2, 1)), oo, lo, ro, p)
+        want = into.copy()
+        want[:, 7:7 + pick.size] = go.gather(z.reshape(b, m * n), pick, 1)
+        got = capi.batch_matmul_nt_select_i8(lhs, rhs, oo, lo, ro, p, dest_of, into, 7)
+        np.testing.assert_array_equal(got, want)

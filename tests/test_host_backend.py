@@ -322,3 +322,41 @@ def test_dequantize_and_sigmoid_become_one_launch():
     m.compile(f, fuse_dequantize_sigmoid=False)
     assert [r["kernel"] for r in H.parse_listing(m.describe(f))] == \
         ["mi355x_dequantize_i8", "mi355x_sigmoid_f32"]
+
+
+def _interaction_module(idx, peek=False):
+    """x [B,4,16] -> Transpose -> BatchMatMul -> (flat view) Gather(idx) ->
+    InsertTensor into the output at column 3."""
+    m = H.Module()
+    B = 6
+    x = m.placeholder("x", (B, 4, 16), H.INT8Q, np.int8, 0.1, 2)
+    wide = m.placeholder("wide", (B, 3 + len(idx)), H.INT8Q, np.int8, 0.3, -5)
+    spare = m.placeholder("spare", (B, 16), H.INT8Q, np.int8, 0.3, -5)
+    ix = m.constant("idx", np.asarray(idx, np.int64), H.INT64I)
+    f = m.function("main")
+    xt = m.activation(f, "xT", (B, 16, 4), H.INT8Q, 0.1, 2)
+    z = m.activation(f, "z", (B, 4, 4), H.INT8Q, 0.3, -5)
+    zf = m.view("z_flat", z, (B, 16), H.INT8Q, 0.3, -5)
+    pairs = m.activation(f, "pairs", (B, len(idx)), H.INT8Q, 0.3, -5)
+    m.instruction(f, H.TRANSPOSE, "t", [xt, x], [0, 2, 1])
+    m.instruction(f, H.BATCH_MATMUL, "mm", [z, x, xt])
+    if peek:
+        m.instruction(f, H.RESCALE_QUANTIZED, "peek", [spare, zf])
+    m.instruction(f, H.GATHER, "pick", [pairs, zf, ix], [1])
+    m.instruction(f, H.INSERT_TENSOR, "ins", [wide, pairs], [3])
+    m.compile(f)
+    return [(r["kernel"], r["inst"]) for r in H.parse_listing(m.describe(f)) if r["phase"] == "launch"], m, f
+
+
+def test_gather_of_product_elements_is_folded_into_the_product():
+    k, m, f = _interaction_module([1, 2, 3, 6, 7, 11])
+    assert k == [("mi355x_batch_matmul_nt_select_i8", "mm+pick+ins")]
+    r = _launch(m, f, "mi355x_batch_matmul_nt_select_i8")
+    assert (r["picked"], r["stride"], r["offset"], r["M"], r["N"], r["K"]) == (6, 9, 3, 4, 4, 16)
+    # an index picked twice, an index outside the matrix, or a second reader of
+    # the product: the product is written whole and gathered afterwards
+    for idx, peek in (([1, 2, 2], False), ([1, 16], False), ([1, 2, 3], True)):
+        k, _, _ = _interaction_module(idx, peek)
+        names = [n for n, _ in k]
+        assert "mi355x_batch_matmul_nt_select_i8" not in names and "mi355x_batch_matmul_nt_i8" in names
+        assert "mi355x_gather_rows" in names
