@@ -118,29 +118,41 @@ __global__ __launch_bounds__(kEwThreads) void rescale_i8_kernel(
 }
 
 // RescaleQuantized of a [rows x cols] tensor written as a slice of a wider one
-// (dst rows dst_row_stride bytes apart): V bytes per lane.
+// (dst rows dst_row_stride bytes apart): V bytes per lane. The host keeps
+// rows * cols / V below 2^31, so the index arithmetic is 32-bit.
 template <int V>
 __global__ __launch_bounds__(kEwThreads) void rescale_rows_i8_kernel(
-    int8_t *__restrict__ dst, const int8_t *__restrict__ src, long long rows, int cols,
+    int8_t *__restrict__ dst, const int8_t *__restrict__ src, unsigned total, unsigned per_row,
     long long dst_row_stride, int32_t out_offset, int32_t in_offset, int32_t pre,
     int32_t post, int32_t scale) {
-  const int per_row = cols / V;
-  const long long total = rows * per_row;
-  const long long stride = (long long)gridDim.x * kEwThreads;
-  for (long long i = (long long)blockIdx.x * kEwThreads + threadIdx.x; i < total; i += stride) {
-    const long long r = i / per_row;
-    const int c = (int)(i - r * per_row) * V;
-    if constexpr (V == 4) {
-      const uint32_t w = *reinterpret_cast<const uint32_t *>(src + r * cols + c);
+  const unsigned i = blockIdx.x * kEwThreads + threadIdx.x;
+  if (i >= total) return;
+  const unsigned r = i / per_row;
+  const unsigned c = (i - r * per_row) * V;
+  const int8_t *s = src + (size_t)i * V;
+  int8_t *d = dst + (long long)r * dst_row_stride + c;
+  if constexpr (V == 1) {
+    d[0] = (int8_t)clip_i8(scale_i32((int32_t)s[0] - in_offset, pre, post, scale, out_offset));
+  } else {
+    uint32_t w[V / 4];
+    if constexpr (V == 16) {
+      const uint4 q = *reinterpret_cast<const uint4 *>(s);
+      w[0] = q.x; w[1] = q.y; w[2] = q.z; w[3] = q.w;
+    } else {
+      w[0] = *reinterpret_cast<const uint32_t *>(s);
+    }
+#pragma unroll
+    for (int j = 0; j < V / 4; j++) {
       int32_t q[4];
 #pragma unroll
       for (int b = 0; b < 4; b++)
-        q[b] = clip_i8(scale_i32(sext8(w, b) - in_offset, pre, post, scale, out_offset));
-      *reinterpret_cast<uint32_t *>(dst + r * dst_row_stride + c) = pack4(q[0], q[1], q[2], q[3]);
-    } else {
-      dst[r * dst_row_stride + c] = (int8_t)clip_i8(
-          scale_i32((int32_t)src[r * cols + c] - in_offset, pre, post, scale, out_offset));
+        q[b] = clip_i8(scale_i32(sext8(w[j], b) - in_offset, pre, post, scale, out_offset));
+      w[j] = pack4(q[0], q[1], q[2], q[3]);
     }
+    if constexpr (V == 16)
+      *reinterpret_cast<uint4 *>(d) = make_uint4(w[0], w[1], w[2], w[3]);
+    else
+      *reinterpret_cast<uint32_t *>(d) = w[0];
   }
 }
 
@@ -232,19 +244,21 @@ int mi355x_rescale_rows_i8(int8_t *dst, const int8_t *src, size_t rows, size_t c
                  dst_row_stride);
   MI355X_REQUIRE(rows < (1ull << 40) && cols < (1u << 30) && dst_row_stride < (1ull << 40),
                  "tensor too large");
-  const bool vec = cols % 4 == 0 && dst_row_stride % 4 == 0 &&
-                   ((((uintptr_t)dst) | ((uintptr_t)src)) & 3) == 0;
-  const size_t work = rows * (vec ? cols / 4 : cols);
-  size_t blocks = (work + kEwThreads - 1) / kEwThreads;
-  if (blocks > 256 * 64) blocks = 256 * 64;
-  if (vec)
-    hipLaunchKernelGGL(rescale_rows_i8_kernel<4>, dim3((unsigned)blocks), dim3(kEwThreads), 0,
-                       as_stream(stream), dst, src, (long long)rows, (int)cols,
-                       (long long)dst_row_stride, out_offset, in_offset, pre, post, scale);
-  else
-    hipLaunchKernelGGL(rescale_rows_i8_kernel<1>, dim3((unsigned)blocks), dim3(kEwThreads), 0,
-                       as_stream(stream), dst, src, (long long)rows, (int)cols,
-                       (long long)dst_row_stride, out_offset, in_offset, pre, post, scale);
+  const uintptr_t both = (uintptr_t)dst | (uintptr_t)src;
+  const int v = (cols % 16 == 0 && dst_row_stride % 16 == 0 && (both & 15) == 0)  ? 16
+                : (cols % 4 == 0 && dst_row_stride % 4 == 0 && (both & 3) == 0) ? 4
+                                                                                  : 1;
+  const size_t work = rows * (cols / v);
+  MI355X_REQUIRE(work < 0x7fffffffu, "tensor too large");
+  const unsigned blocks = (unsigned)((work + kEwThreads - 1) / kEwThreads);
+#define MI355X_RESCALE_ROWS(V)                                                                  \
+  hipLaunchKernelGGL(rescale_rows_i8_kernel<V>, dim3(blocks), dim3(kEwThreads), 0,              \
+                     as_stream(stream), dst, src, (unsigned)work, (unsigned)(cols / V),         \
+                     (long long)dst_row_stride, out_offset, in_offset, pre, post, scale)
+  if (v == 16) MI355X_RESCALE_ROWS(16);
+  else if (v == 4) MI355X_RESCALE_ROWS(4);
+  else MI355X_RESCALE_ROWS(1);
+#undef MI355X_RESCALE_ROWS
   return check_launch("rescale_rows_i8");
 }
 
