@@ -267,6 +267,38 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
   tn = in_panel / rows_here;
 }
 
+// The per-column parameters one lane's output columns need in the epilogue,
+// as they lie in memory. The direct-to-LDS kernel requests them before its
+// first tile load, so that they have long arrived when the K loop ends and
+// the epilogue starts without a memory round trip of its own.
+struct ColRaw {
+  int32_t woff, opre, opost, oscale, sumb, bias, boff, bpre, bpost, bscale;
+};
+template <int TN, int WN>
+__device__ __forceinline__ void load_col_raw(ColRaw (&c)[TN], const Epilogue &ep, int N, int n0,
+                                             int n_base, int wn, int l32) {
+#pragma unroll
+  for (int j = 0; j < TN; j++) {
+    const int nl = n0 + wn * WN + j * 32 + l32;   // column within the group
+    const int n = n_base + (nl < N ? nl : 0);     // global output column
+    c[j].woff = ep.w_off.at(n);
+    c[j].opre = ep.out_pre.at(n);
+    c[j].opost = ep.out_post.at(n);
+    c[j].oscale = ep.out_scale.at(n);
+    c[j].sumb = ep.sum_b ? ep.sum_b[n] : 0;
+    c[j].bias = 0;
+    c[j].boff = c[j].bpre = c[j].bpost = c[j].bscale = 0;
+    if (ep.bias) {
+      c[j].bias = ep.bias_is_i8 ? (int32_t) reinterpret_cast<const int8_t *>(ep.bias)[n]
+                                : reinterpret_cast<const int32_t *>(ep.bias)[n];
+      c[j].boff = ep.b_off.at(n);
+      c[j].bpre = ep.bias_pre.at(n);
+      c[j].bpost = ep.bias_post.at(n);
+      c[j].bscale = ep.bias_scale.at(n);
+    }
+  }
+}
+
 // Shared epilogue. Accumulator layout of v_mfma_i32_32x32x32_i8: lane l holds
 // column l % 32 and, in register r, row 8*(r/4) + 4*(l/32) + r%4 of the tile.
 // Must be entered after a block barrier (LDS is reused).
@@ -275,7 +307,7 @@ template <int BM, int BN, int WM, int WN, bool NEED_SA, bool NEED_SB,
 __device__ __forceinline__ void gemm_epilogue_impl(
     v16i (&acc)[WM / 32][WN / 32], int (&sa)[WM / 32], int (&sb)[WN / 32],
     int8_t *lds, const Epilogue &ep, int M, int N, int K, int m0, int n0,
-    int n_base) {
+    int n_base, const ColRaw (&col)[WN / 32]) {
   constexpr int WAVES_N = BN / WN;
   constexpr int THREADS = (BM / WM) * (BN / WN) * 64;
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -316,26 +348,18 @@ __device__ __forceinline__ void gemm_epilogue_impl(
 
 #pragma unroll
   for (int j = 0; j < TN; j++) {
-    const int nl = n0 + wn * WN + j * 32 + l32;   // column within the group
-    const bool n_ok = nl < N;
-    const int n = n_base + (n_ok ? nl : 0);       // global output column
-    const int32_t woff = ep.w_off.at(n);
-    const int32_t opre = ep.out_pre.at(n), opost = ep.out_post.at(n);
-    const int32_t oscale = ep.out_scale.at(n);
+    const int32_t woff = col[j].woff;
+    const int32_t opre = col[j].opre, opost = col[j].opost;
+    const int32_t oscale = col[j].oscale;
     uint32_t colc = (uint32_t)K * (uint32_t)ep.a_off * (uint32_t)woff;
     if constexpr (NEED_SB) {
       colc -= (uint32_t)ep.a_off * (uint32_t)sb[j];
     } else if (ep.sum_b) {
-      colc -= (uint32_t)ep.a_off * (uint32_t)ep.sum_b[n];
+      colc -= (uint32_t)ep.a_off * (uint32_t)col[j].sumb;
     }
-    if (ep.bias) {
-      const int32_t b = ep.bias_is_i8
-                            ? (int32_t) reinterpret_cast<const int8_t *>(ep.bias)[n]
-                            : reinterpret_cast<const int32_t *>(ep.bias)[n];
-      colc += (uint32_t)scale_i32((int32_t)((uint32_t)b - (uint32_t)ep.b_off.at(n)),
-                                  ep.bias_pre.at(n), ep.bias_post.at(n),
-                                  ep.bias_scale.at(n), 0);
-    }
+    if (ep.bias)
+      colc += (uint32_t)scale_i32((int32_t)((uint32_t)col[j].bias - (uint32_t)col[j].boff),
+                                  col[j].bpre, col[j].bpost, col[j].bscale, 0);
 #pragma unroll
     for (int i = 0; i < TM; i++) {
 #pragma unroll
@@ -416,13 +440,13 @@ template <int BM, int BN, int WM, int WN, bool NEED_SA, bool NEED_SB>
 __device__ __forceinline__ void gemm_epilogue(
     v16i (&acc)[WM / 32][WN / 32], int (&sa)[WM / 32], int (&sb)[WN / 32],
     int8_t *lds, const Epilogue &ep, int M, int N, int K, int m0, int n0,
-    int n_base) {
+    int n_base, const ColRaw (&col)[WN / 32]) {
   if (ep.act == 5) // LEAKY_RELU: rare, kept out of the common instruction stream
     gemm_epilogue_impl<BM, BN, WM, WN, NEED_SA, NEED_SB, true>(
-        acc, sa, sb, lds, ep, M, N, K, m0, n0, n_base);
+        acc, sa, sb, lds, ep, M, N, K, m0, n0, n_base, col);
   else
     gemm_epilogue_impl<BM, BN, WM, WN, NEED_SA, NEED_SB, false>(
-        acc, sa, sb, lds, ep, M, N, K, m0, n0, n_base);
+        acc, sa, sb, lds, ep, M, N, K, m0, n0, n_base, col);
 }
 
 template <int BM, int BN, int WM, int WN, bool NEED_SA, bool NEED_SB,
@@ -565,8 +589,10 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_i8_kernel(
     }
   }
 
+  ColRaw col[TN];
+  load_col_raw<TN, WN>(col, ep, N, n0, n_base, wn, l32);
   gemm_epilogue<BM, BN, WM, WN, NEED_SA, NEED_SB>(acc, sa, sb, lds, ep, M, N, K,
-                                                  m0, n0, n_base);
+                                                  m0, n0, n_base, col);
 }
 
 // ---- direct-to-LDS main loop ---------------------------------------------------
@@ -692,6 +718,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
     else
       dma16(bptr[i - A_LOADS] + k0, slot + b_dst[i - A_LOADS]);
   };
+  // requested first, consumed in the epilogue
+  ColRaw col[TN];
+  load_col_raw<TN, WN>(col, ep, N, n0, n_base, wn, l32);
   // prologue: tiles 0..STAGES-2 and the first half of tile STAGES-1 in flight
   // (tiles past the end are re-reads of the last one into slots nobody
   // consumes, which keeps the counts uniform)
@@ -818,7 +847,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
   dma_wait<0>(); // drain the re-reads before LDS is reused
   __syncthreads();
   gemm_epilogue<BM, BN, WM, WN, NEED_SA, NEED_SB>(acc, sa, sb, lds, ep, M, N, K,
-                                                  m0, n0, n_base);
+                                                  m0, n0, n_base, col);
 }
 
 template <int BM, int BN> constexpr size_t gemm_epilogue_lds_bytes() {
