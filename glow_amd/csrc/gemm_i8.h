@@ -640,7 +640,10 @@ __device__ __forceinline__ uint32_t lds_address(const void *p) {
 template <int BM, int BN, int WM, int WN, int STAGES, bool NEED_SA,
           bool NEED_SB, class ARows, bool SHORT = false>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
-                             (BM * BN == 256 * 128) ? 2 : SHORT ? 4 : 1) void gemm_i8_dma_kernel(
+                             (BM * BN == 256 * 128)   ? 2
+                             : SHORT                  ? 4
+                             : (BM * BN == 128 * 128) ? 3
+                                                      : 1) void gemm_i8_dma_kernel(
     ARows A, DenseRows B, Epilogue ep, int M, int N, int K, int tiles_m,
     int tiles_n, long long b_group_stride, int n_per_group) {
   constexpr int WAVES_N = BN / WN;
