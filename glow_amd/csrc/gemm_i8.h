@@ -533,6 +533,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_i8_kernel(
 #pragma unroll
     for (int i = 0; i < B_CH; i++) *reinterpret_cast<int4 *>(stage + b_lds[i]) = rb[slot][i];
   };
+  // the epilogue's per-column parameters, requested with the first tile
+  ColRaw col[TN];
+  load_col_raw<TN, WN>(col, ep, N, n0, n_base, wn, l32);
   fetch(0, 0);
   park(0, lds);
   // tiles 1..D on their way; tile t lives in register slot (t - 1) % D
@@ -589,8 +592,6 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_i8_kernel(
     }
   }
 
-  ColRaw col[TN];
-  load_col_raw<TN, WN>(col, ep, N, n0, n_base, wn, l32);
   gemm_epilogue<BM, BN, WM, WN, NEED_SA, NEED_SB>(acc, sa, sb, lds, ep, M, N, K,
                                                   m0, n0, n_base, col);
 }
