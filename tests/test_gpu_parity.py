@@ -120,6 +120,40 @@ def test_rwq_fc_vs_oracle(shape):
                                   go.rwq_fc_i8(*cases.rwq_fc_args(c)))
 
 
+@pytest.mark.parametrize("K", [64, 256, 448, 511, 512])
+def test_rwq_fc_with_accumulators_and_constants_around_2_to_the_23(K):
+    """Operands that give the largest possible sums (every product +16384),
+    column constants that bring accumulator + constant to just below and just
+    above 2^23, scales up to 2^23 - 1 (products that wrap around 32 bits):
+    where a shortcut through a narrower multiplier would first go wrong."""
+    M, N = 96, 128
+    rng = np.random.default_rng(K)
+    lim = (1 << 23) - min(K, 511) * 16384
+    x = np.full((M, K), -128, np.int8)
+    w = np.full((N, K), -128, np.int8)        # every product +16384: the largest sum
+    x[M // 2:] = 127
+    w[1::2, ::3] = 127
+    bias = np.empty(N, np.int32)
+    bias[0::4] = lim - 1
+    bias[1::4] = -lim
+    bias[2::4] = rng.integers(-1000, 1000, N // 4)
+    bias[3::4] = lim - 1
+    for outside in (False, True):
+        b = bias.copy()
+        if outside:
+            b[3::4] = lim + 5                 # one column in four leaves the bound
+        one = np.ones(N, np.int32)
+        zero = np.zeros(N, np.int32)
+        out_scale = rng.integers(256, 512, N).astype(np.int32)
+        out_scale[::5] = (1 << 23) - 1
+        out_pre = rng.integers(0, 9, N).astype(np.int32)
+        out_post = rng.integers(8, 24, N).astype(np.int32)
+        args = (x, w, b, zero, zero, zero, one, out_pre, out_post, out_scale, 3, 0, 0)
+        want = go.rwq_fc_i8(*args)
+        assert len(np.unique(want)) > 3
+        np.testing.assert_array_equal(capi.rwq_fc_i8(*args), want)
+
+
 def test_rwq_fc_every_row_length_up_to_three_chunks():
     """Rows that are not a whole number of 16-byte chunks: every remainder 1..15
     both for rows shorter than one chunk and for longer ones (the last chunk is
