@@ -57,7 +57,7 @@ def parse():
                     help="headline workload only")
     ap.add_argument("--only", default="",
                     help="run a single extra kernel (profiling aid): "
-                         "slws|fc_large|fc_large_zero|fc_c1|conv_c3|quantize|dequantize|"
+                         "slws|fc_large|fc_large_zero|fc_c1|fc_m16384|conv_c3|quantize|dequantize|"
                          "rescale|copy|resnet50|dlrm")
     return ap.parse_args()
 
@@ -498,14 +498,16 @@ def main():
     extra = {}
     only = args.only
 
-    if only in ("fc_large", "fc_large_zero", "fc_c1", "conv_c3", "quantize", "dequantize",
-                "rescale", "copy"):
+    if only in ("fc_large", "fc_large_zero", "fc_c1", "fc_m16384", "conv_c3", "quantize",
+                "dequantize", "rescale", "copy"):
         if only == "fc_large":
             r = bench_fc(capi, cases, 8192, 4096, 4096, args.steps, args.warmup)
         elif only == "fc_large_zero":
             r = bench_fc(capi, cases, 8192, 4096, 4096, args.steps, args.warmup, zero_leg=True)
         elif only == "fc_c1":
             r = bench_fc(capi, cases, 128, 1024, 1024, args.steps, args.warmup)
+        elif only == "fc_m16384":
+            r = bench_fc(capi, cases, 16384, 1024, 1024, args.steps, args.warmup)
         elif only == "conv_c3":
             r = bench_conv(capi, cases, args.steps, args.warmup)
         else:
@@ -539,6 +541,9 @@ def main():
         # enough launches for the clock to settle under the power limit
         extra["rwq_fc_large"] = bench_fc(capi, cases, 8192, 4096, 4096, max(st, 300), max(wu, 30),
                                              zero_leg=True)
+        # the single-FC configuration's own K and N at a large batch
+        extra["rwq_fc_m16384"] = bench_fc(capi, cases, 16384, 1024, 1024, max(st, 300),
+                                          max(wu, 30))
         extra["cwq_conv_c3"] = bench_conv(capi, cases, args.steps, args.warmup)
         for w in ("quantize", "dequantize", "rescale"):
             extra[w] = bench_elementwise(capi, w, st, wu)
