@@ -795,8 +795,9 @@ private:
     size_t pitch;
   };
   TableView tableView(const Operand &data, size_t rows, size_t inLine, MI355XFunction &out) {
+    // (tables whose copy would pass 8 GiB keep their packed rows)
     if (!opts_.padTableRows || data.v->category != SymbolCategory::Constant || inLine <= 32 ||
-        inLine >= 64 || rows == 0)
+        inLine >= 64 || rows == 0 || rows > ((size_t)8 << 30) / 64)
       return {[data](const DeviceBindings &b) { return (const uint8_t *)data.ptr(b); }, inLine};
     auto it = paddedTables_.find(data.v);
     if (it == paddedTables_.end()) {
