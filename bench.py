@@ -57,8 +57,11 @@ def parse():
                     help="headline workload only")
     ap.add_argument("--only", default="",
                     help="run a single extra kernel (profiling aid): "
-                         "slws|fc_large|fc_large_zero|fc_c1|fc_m16384|conv_c3|quantize|dequantize|"
+                         "slws|fc_large|fc_large_zero|fc_c1|fc_m16384|fc_mid|conv_c3|quantize|dequantize|"
                          "rescale|copy|resnet50|dlrm")
+    ap.add_argument("--tile", type=int, default=-1,
+                    help="force a workgroup tile for the matrix-core legs of --only "
+                         "(0..5, see mi355x_gemm_tile_override; default: chosen from the shape)")
     return ap.parse_args()
 
 
@@ -497,8 +500,10 @@ def main():
     info = capi.device_info()
     extra = {}
     only = args.only
+    if args.tile >= 0:
+        capi.check(capi.lib().mi355x_gemm_tile_override(args.tile))
 
-    if only in ("fc_large", "fc_large_zero", "fc_c1", "fc_m16384", "conv_c3", "quantize",
+    if only in ("fc_large", "fc_large_zero", "fc_c1", "fc_m16384", "fc_mid", "conv_c3", "quantize",
                 "dequantize", "rescale", "copy"):
         if only == "fc_large":
             r = bench_fc(capi, cases, 8192, 4096, 4096, args.steps, args.warmup)
@@ -508,6 +513,10 @@ def main():
             r = bench_fc(capi, cases, 128, 1024, 1024, args.steps, args.warmup)
         elif only == "fc_m16384":
             r = bench_fc(capi, cases, 16384, 1024, 1024, args.steps, args.warmup)
+        elif only == "fc_mid":
+            # a 3x3 convolution of ResNet-50's 14x14 stage as a plain product:
+            # 196 workgroups of 128x128, fewer than the part has CUs
+            r = bench_fc(capi, cases, 12544, 2304, 256, args.steps, args.warmup)
         elif only == "conv_c3":
             r = bench_conv(capi, cases, args.steps, args.warmup)
         else:

@@ -713,10 +713,12 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
     }
     return run_loc;
   };
-  auto issue_load = [&](int nk, int i, const typename ARows::Loc &loc) {
-    const int slot_of = SHORT ? min(nk, KT - 1) : nk % STAGES;
+  // `ring` is the ring slot tile nk goes to (nk % STAGES, carried by the caller
+  // instead of divided out for every load) and k0 its K offset, already
+  // clamped to the last tile
+  auto issue_load = [&](int nk, int ring, int k0, int i, const typename ARows::Loc &loc) {
+    const int slot_of = SHORT ? min(nk, KT - 1) : ring;
     const uint32_t slot = lds0 + (uint32_t)slot_of * STAGE;
-    const int k0 = min(nk, KT - 1) * kBK;
     if (i < A_LOADS)
       dma16(A.chunk_ptr(arow[i], loc), slot + a_dst[i]);
     else
@@ -732,12 +734,13 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
   for (int s = 0; s < STAGES - 1; s++) {
     const typename ARows::Loc loc = locate_tile(s);
 #pragma unroll
-    for (int i = 0; i < LOADS; i++) issue_load(s, i, loc);
+    for (int i = 0; i < LOADS; i++) issue_load(s, s, min(s, KT - 1) * kBK, i, loc);
   }
   // the tile whose second half is still to be requested
   typename ARows::Loc half_loc = locate_tile(STAGES - 1);
 #pragma unroll
-  for (int i = 0; i < H0; i++) issue_load(STAGES - 1, i, half_loc);
+  for (int i = 0; i < H0; i++)
+    issue_load(STAGES - 1, STAGES - 1, min(STAGES - 1, KT - 1) * kBK, i, half_loc);
 
   v16i acc[TM][TN];
 #pragma unroll
@@ -812,12 +815,12 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
     for (int f = t * FRAGS / MFMAS; f < (t + 1) * FRAGS / MFMAS; f++)
       read_frag(stage, ks, buf, f);
   };
-  auto loads_in_slot = [&](int t, int nk, int first, int n,
+  auto loads_in_slot = [&](int t, int nk, int ring, int k0, int first, int n,
                            const typename ARows::Loc &loc) {
 #pragma unroll
     for (int x = 0; x < n; x++)
       if (min(MFMAS - 1, (2 * x + 1) * MFMAS / (2 * n)) == t)
-        issue_load(nk, first + x, loc);
+        issue_load(nk, ring, k0, first + x, loc);
   };
 
   // tile 0 has landed once only the newer requests are pending
@@ -825,16 +828,26 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
   __syncthreads();
 #pragma unroll
   for (int f = 0; f < FRAGS; f++) read_frag(lds, 0, 0, f);
+  // Ring positions and K offsets are carried from step to step: the slot of
+  // tile kt, of tile kt-1 (which tile kt+STAGES-1 takes over) and the clamped K
+  // offsets of the two tiles a step requests. One wave per SIMD issues an
+  // instruction every four cycles at best, so every scalar instruction of this
+  // bookkeeping is time the matrix cores idle when workgroups are few.
+  int ring_cur = 0, ring_prev = STAGES - 1;
+  const int k_last = (KT - 1) * kBK;
+  int k_far0 = min(STAGES - 1, KT - 1) * kBK; // tile kt+STAGES-1
+  int k_far1 = min(STAGES, KT - 1) * kBK;     // tile kt+STAGES
   for (int kt = 0; kt < KT; kt++) {
-    const int8_t *cur = lds + (kt % STAGES) * STAGE;
+    const int ring_next = ring_cur + 1 == STAGES ? 0 : ring_cur + 1;
+    const int8_t *cur = lds + (SHORT ? kt : ring_cur) * STAGE;
     // (the fragments read past the end are not used)
-    const int8_t *nxt = lds + (SHORT ? min(kt + 1, KT - 1) : (kt + 1) % STAGES) * STAGE;
+    const int8_t *nxt = lds + (SHORT ? min(kt + 1, KT - 1) : ring_next) * STAGE;
     // slice 0 runs while the fragments of slice 1 arrive and the second half
     // of tile kt+STAGES-1 is requested (its slot held tile kt-1, which every
     // wave had read before the previous barrier)
     multiply(0, [&](int t) {
       frags_in_slot(t, cur, 1, 1);
-      loads_in_slot(t, kt + STAGES - 1, H0, LOADS - H0, half_loc);
+      loads_in_slot(t, kt + STAGES - 1, ring_prev, k_far0, H0, LOADS - H0, half_loc);
     });
     // tile kt+1 has landed once only tiles kt+2..kt+STAGES-1 are pending; past
     // the barrier every wave holds tile kt in registers, so its slot is free
@@ -845,8 +858,12 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
     half_loc = locate_tile(kt + STAGES);
     multiply(1, [&](int t) {
       frags_in_slot(t, nxt, 0, 0);
-      loads_in_slot(t, kt + STAGES, 0, H0, half_loc);
+      loads_in_slot(t, kt + STAGES, ring_cur, k_far1, 0, H0, half_loc);
     });
+    ring_prev = ring_cur;
+    ring_cur = ring_next;
+    k_far0 = min(k_far0 + kBK, k_last);
+    k_far1 = min(k_far1 + kBK, k_last);
   }
   dma_wait<0>(); // drain the re-reads before LDS is reused
   __syncthreads();
