@@ -603,6 +603,16 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_i8_kernel(
 // through inline assembly so that the compiler's own wait-count insertion
 // does not serialise later LDS reads against loads still in flight; the
 // kernel below waits explicitly with dma_wait<N>().
+// The same with the LDS address given as the sum of two wave-uniform parts
+// (a ring slot's offset and the load's place in the slot): the scalar add
+// writes M0 itself.
+__device__ __forceinline__ void dma16(const void *gptr, uint32_t lds_a, uint32_t lds_b) {
+  asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off"
+               :
+               : "s"(lds_a), "s"(lds_b), "v"(gptr)
+               : "memory", "scc");
+}
+
 __device__ __forceinline__ void dma16(const void *gptr, uint32_t lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
                :
@@ -686,13 +696,13 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
   for (int i = 0; i < A_LOADS; i++) {
     const int g = i * WAVES + wave;
     arow[i] = A.row(min(m0 + g * 16 + row_in_grp, M - 1));
-    a_dst[i] = g * 1024;
+    a_dst[i] = lds0 + g * 1024;
   }
 #pragma unroll
   for (int i = 0; i < B_LOADS; i++) {
     const int g = i * WAVES + wave;
     bptr[i] = B.p + (long long)min(n0 + g * 16 + row_in_grp, N - 1) * B.ld + kc_lane;
-    b_dst[i] = BM * kBK + g * 1024;
+    b_dst[i] = lds0 + BM * kBK + g * 1024;
   }
 
   const int KT = K / kBK;
@@ -713,16 +723,15 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
     }
     return run_loc;
   };
-  // `ring` is the ring slot tile nk goes to (nk % STAGES, carried by the caller
-  // instead of divided out for every load) and k0 its K offset, already
-  // clamped to the last tile
-  auto issue_load = [&](int nk, int ring, int k0, int i, const typename ARows::Loc &loc) {
-    const int slot_of = SHORT ? min(nk, KT - 1) : ring;
-    const uint32_t slot = lds0 + (uint32_t)slot_of * STAGE;
+  // `ring` is the byte offset of the ring slot tile nk goes to (slot nk %
+  // STAGES, carried by the caller instead of divided out for every load) and
+  // k0 the tile's K offset, already clamped to the last tile
+  auto issue_load = [&](int nk, uint32_t ring, int k0, int i, const typename ARows::Loc &loc) {
+    const uint32_t slot = SHORT ? (uint32_t)min(nk, KT - 1) * STAGE : ring;
     if (i < A_LOADS)
-      dma16(A.chunk_ptr(arow[i], loc), slot + a_dst[i]);
+      dma16(A.chunk_ptr(arow[i], loc), slot, a_dst[i]);
     else
-      dma16(bptr[i - A_LOADS] + k0, slot + b_dst[i - A_LOADS]);
+      dma16(bptr[i - A_LOADS] + k0, slot, b_dst[i - A_LOADS]);
   };
   // requested first, consumed in the epilogue
   ColRaw col[TN];
@@ -734,13 +743,13 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
   for (int s = 0; s < STAGES - 1; s++) {
     const typename ARows::Loc loc = locate_tile(s);
 #pragma unroll
-    for (int i = 0; i < LOADS; i++) issue_load(s, s, min(s, KT - 1) * kBK, i, loc);
+    for (int i = 0; i < LOADS; i++) issue_load(s, s * STAGE, min(s, KT - 1) * kBK, i, loc);
   }
   // the tile whose second half is still to be requested
   typename ARows::Loc half_loc = locate_tile(STAGES - 1);
 #pragma unroll
   for (int i = 0; i < H0; i++)
-    issue_load(STAGES - 1, STAGES - 1, min(STAGES - 1, KT - 1) * kBK, i, half_loc);
+    issue_load(STAGES - 1, (STAGES - 1) * STAGE, min(STAGES - 1, KT - 1) * kBK, i, half_loc);
 
   v16i acc[TM][TN];
 #pragma unroll
@@ -815,7 +824,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
     for (int f = t * FRAGS / MFMAS; f < (t + 1) * FRAGS / MFMAS; f++)
       read_frag(stage, ks, buf, f);
   };
-  auto loads_in_slot = [&](int t, int nk, int ring, int k0, int first, int n,
+  auto loads_in_slot = [&](int t, int nk, uint32_t ring, int k0, int first, int n,
                            const typename ARows::Loc &loc) {
 #pragma unroll
     for (int x = 0; x < n; x++)
@@ -833,15 +842,15 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
   // offsets of the two tiles a step requests. One wave per SIMD issues an
   // instruction every four cycles at best, so every scalar instruction of this
   // bookkeeping is time the matrix cores idle when workgroups are few.
-  int ring_cur = 0, ring_prev = STAGES - 1;
+  uint32_t ring_cur = 0, ring_prev = (STAGES - 1) * STAGE; // byte offsets
   const int k_last = (KT - 1) * kBK;
   int k_far0 = min(STAGES - 1, KT - 1) * kBK; // tile kt+STAGES-1
   int k_far1 = min(STAGES, KT - 1) * kBK;     // tile kt+STAGES
   for (int kt = 0; kt < KT; kt++) {
-    const int ring_next = ring_cur + 1 == STAGES ? 0 : ring_cur + 1;
-    const int8_t *cur = lds + (SHORT ? kt : ring_cur) * STAGE;
+    const uint32_t ring_next = ring_cur + STAGE == STAGES * STAGE ? 0u : ring_cur + STAGE;
+    const int8_t *cur = lds + (SHORT ? (uint32_t)kt * STAGE : ring_cur);
     // (the fragments read past the end are not used)
-    const int8_t *nxt = lds + (SHORT ? min(kt + 1, KT - 1) : ring_next) * STAGE;
+    const int8_t *nxt = lds + (SHORT ? (uint32_t)min(kt + 1, KT - 1) * STAGE : ring_next);
     // slice 0 runs while the fragments of slice 1 arrive and the second half
     // of tile kt+STAGES-1 is requested (its slot held tile kt-1, which every
     // wave had read before the previous barrier)
