@@ -184,9 +184,10 @@ def test_rwq_fc_with_fused_relu(shape):
 
 
 def test_rwq_fc_large_tiles_properties():
-    """A shape that takes the 256x256 tile. The oracle runs on a row sample;
-    all rows are checked through linearity in the batch dimension: identical
-    input rows must give identical output rows."""
+    """A mid-size product with whatever tile the shape rules pick (the forced
+    tiles on long K loops are in test_gpu_gemm_tiles.py). The oracle runs on a
+    row sample; all rows are checked through independence in the batch
+    dimension: identical input rows must give identical output rows."""
     M, K, N = 4096, 1024, 1024
     say("rwq_fc large", (M, K, N))
     c = cases.rwq_fc_case(77, M, K, N, symmetric=False)
