@@ -44,6 +44,7 @@ EXPORTS = [
     "mi355x_fc_i8", "mi355x_matmul_i8", "mi355x_transpose2d_i8",
     "mi355x_cwq_conv2d_i8", "mi355x_conv2d_i8", "mi355x_frwq_slws",
     "mi355x_embedding_bag_rowwise_offsets",
+    "mi355x_slws_reserve_stream",
 ]
 
 
@@ -738,7 +739,7 @@ def _fused_cols(in_line, kind):
 
 
 def frwq_slws(data, kind, weights, indices, lengths, out_f16=False,
-              fp16_accum=False, d_data=None, row_pitch=None):
+              fp16_accum=False, d_data=None, row_pitch=None, stream=None):
     """weights: None (plain SLS), float32 or float16 array. `d_data` lets a
     caller reuse a table already resident on the device. `row_pitch` lays the
     table out with its rows that many bytes apart (the gaps hold junk)."""
@@ -768,9 +769,13 @@ def frwq_slws(data, kind, weights, indices, lengths, out_f16=False,
     d_out = DeviceBuffer.empty((lengths.size, out_line),
                                np.float16 if out_f16 else np.float32)
     d_out.fill(0xFF)  # poison: every row must be written by the kernel
+    if stream is not None:
+        sync()        # streams of this library do not wait for the default stream
     launch_frwq_slws(d_out, out_f16, d_data, data_shape[0], kind, d_w, w16,
                      d_idx, indices.dtype == np.int64, indices.size, d_len,
-                     lengths.size, in_line, out_line, fp16_accum)
+                     lengths.size, in_line, out_line, fp16_accum, stream=stream)
+    if stream is not None:
+        stream.sync()
     return d_out.numpy()
 
 

@@ -26,6 +26,12 @@ constexpr int kWave = 64;
 
 inline bool shift_ok(int32_t s) { return s >= 0 && s <= 31; }
 
+// SparseLengths scratch (slws.hip). A stream the library knows has a buffer for
+// the bag-offset pre-pass of launches with more than 4096 bags; reserving
+// allocates (once per device and stream), launches never do.
+int slws_reserve_stream(hipStream_t st);
+int slws_release_stream(hipStream_t st);
+
 } // namespace mi355x
 
 #define MI355X_HIP(expr)                                                       \

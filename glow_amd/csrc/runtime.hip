@@ -105,7 +105,8 @@ int mi355x_init(int device) {
                 "device %d is %s; this library only carries gfx950 code",
                 device, p.gcnArchName);
   }
-  return MI355X_OK;
+  // SparseLengths scratch for launches on the default stream
+  return slws_reserve_stream(nullptr);
 }
 
 int mi355x_device_info(mi355x_info *info) {
@@ -206,12 +207,23 @@ int mi355x_stream_create(void **stream) {
   hipStream_t s;
   // default priority only
   MI355X_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  int rc = slws_reserve_stream(s);
+  if (rc != MI355X_OK) {
+    (void)hipStreamDestroy(s);
+    return rc;
+  }
   *stream = s;
   return MI355X_OK;
 }
 
 int mi355x_stream_destroy(void *stream) {
-  if (stream) MI355X_HIP(hipStreamDestroy(as_stream(stream)));
+  if (stream) {
+    // the stream's work is finished before its scratch goes away
+    MI355X_HIP(hipStreamSynchronize(as_stream(stream)));
+    int rc = slws_release_stream(as_stream(stream));
+    if (rc != MI355X_OK) return rc;
+    MI355X_HIP(hipStreamDestroy(as_stream(stream)));
+  }
   return MI355X_OK;
 }
 

@@ -41,6 +41,7 @@
 
 #include <atomic>
 #include <mutex>
+#include <vector>
 
 namespace mi355x {
 
@@ -944,20 +945,66 @@ __global__ __launch_bounds__(256) void slws_chunk_sums_kernel(
     chunk_sums[blockIdx.x] = s_part[0] + s_part[1] + s_part[2] + s_part[3];
 }
 
-// Per-device workspace for the chunk sums, allocated on first use and kept.
+// Scratch for the chunk sums (lengths mode with more than kChunkBags bags):
+// one int64 per chunk, written by slws_chunk_sums_kernel and read by the
+// lookup kernel behind it on the same stream.
+//
+// The ordinary entry points take it from a registry keyed by (device, stream):
+// launches on one stream are ordered, so they may share a buffer; launches on
+// different streams never do. A buffer is allocated when the stream is made
+// known to the library (mi355x_init for the device's default stream,
+// mi355x_stream_create, mi355x_slws_reserve_stream), never inside a launch.
+struct StreamScratch {
+  int dev;
+  hipStream_t stream;
+  int64_t *ws;
+};
 static std::mutex g_ws_mutex;
-static int64_t *g_ws[64] = {nullptr};
+static std::vector<StreamScratch> g_ws;
 
-static int chunk_workspace(int64_t **ws) {
+int slws_reserve_stream(hipStream_t st) {
   int dev = 0;
   MI355X_HIP(hipGetDevice(&dev));
-  MI355X_REQUIRE(dev >= 0 && dev < 64, "device index %d out of range", dev);
   std::lock_guard<std::mutex> lock(g_ws_mutex);
-  if (!g_ws[dev]) {
-    MI355X_HIP(hipMalloc((void **)&g_ws[dev], kMaxChunks * sizeof(int64_t)));
-  }
-  *ws = g_ws[dev];
+  for (const StreamScratch &e : g_ws)
+    if (e.dev == dev && e.stream == st) return MI355X_OK;
+  int64_t *ws = nullptr;
+  MI355X_HIP(hipMalloc((void **)&ws, kMaxChunks * sizeof(int64_t)));
+  g_ws.push_back(StreamScratch{dev, st, ws});
   return MI355X_OK;
+}
+
+int slws_release_stream(hipStream_t st) {
+  int dev = 0;
+  MI355X_HIP(hipGetDevice(&dev));
+  int64_t *ws = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    for (size_t i = 0; i < g_ws.size(); i++)
+      if (g_ws[i].dev == dev && g_ws[i].stream == st) {
+        ws = g_ws[i].ws;
+        g_ws.erase(g_ws.begin() + (long)i);
+        break;
+      }
+  }
+  if (ws) MI355X_HIP(hipFree(ws));
+  return MI355X_OK;
+}
+
+static int stream_scratch(hipStream_t st, int64_t **ws) {
+  int dev = 0;
+  MI355X_HIP(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  for (const StreamScratch &e : g_ws)
+    if (e.dev == dev && e.stream == st) {
+      *ws = e.ws;
+      return MI355X_OK;
+    }
+  return fail(MI355X_ERR_INVALID_ARGUMENT,
+              "more than %d bags on a stream without scratch for the bag offsets: "
+              "use a stream from mi355x_stream_create (or the default stream after "
+              "mi355x_init), or call mi355x_slws_reserve_stream(stream) once before",
+              kChunkBags);
 }
 
 template <int LPB, int BPL>
@@ -1132,10 +1179,10 @@ static int slws_dispatch(void *dest, int out_is_f16, const uint8_t *data,
   if (!offsets) {
     const size_t chunks = (out_rows + kChunkBags - 1) / kChunkBags;
     if (chunks > 1) {
+      int64_t *ws = nullptr;
       MI355X_REQUIRE(chunks <= (size_t)kMaxChunks, "more than %d bags",
                      kMaxChunks * kChunkBags);
-      int64_t *ws = nullptr;
-      int rc = chunk_workspace(&ws);
+      int rc = stream_scratch(st, &ws);
       if (rc != MI355X_OK) return rc;
       hipLaunchKernelGGL(slws_chunk_sums_kernel, dim3((unsigned)chunks),
                          dim3(256), 0, st, lengths, (long long)out_rows, ws);
@@ -1263,6 +1310,10 @@ int mi355x_frwq_slws(void *dest, int out_is_f16, const uint8_t *data,
                        weights_are_f16, indices, idx_is_64, num_indices,
                        lengths, nullptr, 0, segments, in_line_size,
                        out_line_size, fp16_accum, stream);
+}
+
+int mi355x_slws_reserve_stream(void *stream) {
+  return slws_reserve_stream(as_stream(stream));
 }
 
 int mi355x_embedding_bag_rowwise_offsets(

@@ -21,6 +21,8 @@ S32To8 s32to8(float ratio) {
   return {o[0], o[1], o[2]};
 }
 
+bool shiftsOk(const S32To8 &p) { return p.pre >= 0 && p.pre <= 31 && p.post >= 0 && p.post <= 31; }
+
 // quantization::quantize<int32_t> (reference Base.h:323-329)
 int32_t quantizeI32(float x, float scale, int32_t offset) {
   float r = x / scale + (float)offset;
@@ -282,15 +284,9 @@ private:
   Operand op(const Instruction &I, int i) const { return Operand{&M_.value(I.operands[(size_t)i])}; }
 
   void noteAccesses(const Instruction &J, KernelLaunch &L) const {
-    // pooled lookups over more than 4096 bags go through a per-device scratch
-    // buffer inside the kernel library: such launches must not overlap
-    if ((J.kind == Kind::FusedRowwiseQuantizedSparseLengthsWeightedSum ||
-         J.kind == Kind::FusedRowwiseQuantizedSparseLengthsSum) &&
-        M_.value(J.operands.back()).type.size() > 4096) {
-      Access shared;
-      shared.root = -2;
-      L.writes.push_back(shared);
-    }
+    // (Pooled lookups over more than 4096 bags use scratch inside the kernel
+    // library that belongs to the stream they are launched on, so launches on
+    // different branches of the graph need no ordering for its sake.)
     for (size_t i = 0; i < J.operands.size(); i++) {
       const Value &v = M_.value(J.operands[i]);
       Access a;
@@ -1009,6 +1005,12 @@ private:
       bpre[j] = bp.pre; bpost[j] = bp.post; bscale[j] = bp.scale;
       opre[j] = opp.pre; opost[j] = opp.post; oscale[j] = opp.scale;
       allZero = allZero && offsets[j] == 0;
+      // the kernels shift by these amounts: what the scalar parameters are held
+      // to at every entry point holds for each row's too
+      CHECK_OP(shiftsOk(bp) && shiftsOk(opp),
+               "row %zu: scales %g (input) x %g (weights), %g (bias), %g (output) give a "
+               "shift outside [0, 31]", j, (double)s.ty().scale, (double)scales[j],
+               (double)bi.ty().scale, (double)d.ty().scale);
     }
     const size_t o0 = gen_.addI32(bpre), o1 = gen_.addI32(bpost), o2 = gen_.addI32(bscale),
                  o3 = gen_.addI32(opre), o4 = gen_.addI32(opost), o5 = gen_.addI32(oscale);
@@ -1167,6 +1169,10 @@ private:
       bpre[c] = bp.pre; bpost[c] = bp.post; bscale[c] = bp.scale;
       opre[c] = opp.pre; opost[c] = opp.post; oscale[c] = opp.scale;
       allZero = allZero && fof[c] == 0;
+      CHECK_OP(shiftsOk(bp) && shiftsOk(opp),
+               "channel %zu: scales %g (input) x %g (filter), %g (bias), %g (output) give a "
+               "shift outside [0, 31]", c, (double)s.ty().scale, (double)fsc[c], (double)bsc[c],
+               (double)d.ty().scale);
     }
     const size_t o0 = gen_.addI32(bpre), o1 = gen_.addI32(bpost), o2 = gen_.addI32(bscale),
                  o3 = gen_.addI32(opre), o4 = gen_.addI32(opost), o5 = gen_.addI32(oscale);

@@ -102,9 +102,8 @@ int mi355x_event_elapsed_ms(void *start, void *stop, float *ms);
  * launch cost of every kernel; replaces the per-instruction dispatch loop of
  * LLVMCompiledFunction::execute / jitmain (reference
  * lib/LLVMIRCodeGen/LLVMCompiledFunction.cpp:73-150). Capture needs a stream
- * made by mi355x_stream_create (not the default stream). Entry points that
- * allocate on first use (mi355x_frwq_slws with more than 4096 bags) must have
- * run once on the device before they are captured. */
+ * made by mi355x_stream_create (not the default stream). No launch entry
+ * point allocates. */
 typedef struct mi355x_graph mi355x_graph;
 int mi355x_graph_begin_capture(void *stream);
 int mi355x_graph_end_capture(void *stream, mi355x_graph **graph);
@@ -504,6 +503,17 @@ int mi355x_frwq_slws(void *dest, int out_is_f16, const uint8_t *data,
                      size_t num_indices, const int32_t *lengths,
                      size_t segments, size_t in_line_size,
                      size_t out_line_size, int fp16_accum, void *stream);
+
+/* Scratch of the lengths-mode SparseLengths entry points (mi355x_frwq_slws,
+ * mi355x_rwq_slws). With more than 4096 bags a small pre-pass sums the lengths
+ * of each 4096-bag chunk into a 256 KiB buffer that belongs to the (device,
+ * stream) pair of the launch: launches on one stream are ordered and share it,
+ * launches on different streams never do. mi355x_init gives the device's
+ * default stream its buffer, mi355x_stream_create every stream it makes; a
+ * stream made elsewhere is registered here once (this call allocates, launches
+ * do not; a launch with more than 4096 bags on an unregistered stream fails
+ * with MI355X_ERR_INVALID_ARGUMENT). No counterpart in the reference. */
+int mi355x_slws_reserve_stream(void *stream);
 
 /* Arithmetic of the SparseLengths kernels (process-wide; default on).
  * On: rows of 32, 64, 128 or 256 data bytes with fp32 accumulation are summed

@@ -360,3 +360,26 @@ def test_gather_of_product_elements_is_folded_into_the_product():
         names = [n for n, _ in k]
         assert "mi355x_batch_matmul_nt_select_i8" not in names and "mi355x_batch_matmul_nt_i8" in names
         assert "mi355x_gather_rows" in names
+
+
+def test_per_row_and_per_channel_shifts_are_checked_at_compile_time():
+    """A row scale so small that its rescale needs a shift beyond 31 bits is a
+    compile error (the scalar parameters of every entry point are held to
+    [0, 31]; the per-row vectors live in device memory, so the backend checks
+    them where it makes them)."""
+    c = cases.rwq_fc_case(1, 8, 64, 48)
+    c["w_scales"] = c["w_scales"].copy()
+    c["w_scales"][17] = 1e-22
+    m, f = host_cases.rwq_fc_module(c)
+    with pytest.raises(H.HostError) as e:
+        m.compile(f)
+    assert "row 17" in str(e.value) and "[0, 31]" in str(e.value)
+    cc = cases.cwq_conv_case(2, 1, 6, 6, 16, 8)
+    cc["f_scales"] = cc["f_scales"].copy()
+    cc["b_scales"] = cc["b_scales"].copy()
+    cc["f_scales"][5] = 1e-22
+    cc["b_scales"][5] = 1e-22 * 0.05
+    m, f = host_cases.cwq_conv_module(cc)
+    with pytest.raises(H.HostError) as e:
+        m.compile(f)
+    assert "channel 5" in str(e.value)
