@@ -44,7 +44,7 @@ EXPORTS = [
     "mi355x_fc_i8", "mi355x_matmul_i8", "mi355x_transpose2d_i8",
     "mi355x_cwq_conv2d_i8", "mi355x_conv2d_i8", "mi355x_frwq_slws",
     "mi355x_embedding_bag_rowwise_offsets",
-    "mi355x_slws_reserve_stream",
+    "mi355x_slws_reserve_stream", "mi355x_frwq_slws_noalloc",
 ]
 
 
@@ -508,8 +508,11 @@ def launch_cwq_conv2d_add_i8(out, x, filt, bias, bias_is_i8, geom, conv_offset,
 def launch_frwq_slws(dest, out_is_f16, data, data_rows, kind, weights,
                      weights_are_f16, indices, idx_is_64, num_indices, lengths,
                      segments, in_line, out_line, fp16_accum=False,
-                     stream=None):
-    check(lib().mi355x_frwq_slws(
+                     stream=None, noalloc=False):
+    """noalloc: through mi355x_frwq_slws_noalloc (scratch in the library's fixed
+    device array) instead of mi355x_frwq_slws (per-stream scratch)."""
+    fn = lib().mi355x_frwq_slws_noalloc if noalloc else lib().mi355x_frwq_slws
+    check(fn(
         _vp(dest), C.c_int(bool(out_is_f16)), _vp(data), _sz(data_rows),
         C.c_int(kind), _vp(weights), C.c_int(bool(weights_are_f16)),
         _vp(indices), C.c_int(bool(idx_is_64)), _sz(num_indices), _vp(lengths),
@@ -739,7 +742,8 @@ def _fused_cols(in_line, kind):
 
 
 def frwq_slws(data, kind, weights, indices, lengths, out_f16=False,
-              fp16_accum=False, d_data=None, row_pitch=None, stream=None):
+              fp16_accum=False, d_data=None, row_pitch=None, stream=None,
+              noalloc=False):
     """weights: None (plain SLS), float32 or float16 array. `d_data` lets a
     caller reuse a table already resident on the device. `row_pitch` lays the
     table out with its rows that many bytes apart (the gaps hold junk)."""
@@ -773,7 +777,8 @@ def frwq_slws(data, kind, weights, indices, lengths, out_f16=False,
         sync()        # streams of this library do not wait for the default stream
     launch_frwq_slws(d_out, out_f16, d_data, data_shape[0], kind, d_w, w16,
                      d_idx, indices.dtype == np.int64, indices.size, d_len,
-                     lengths.size, in_line, out_line, fp16_accum, stream=stream)
+                     lengths.size, in_line, out_line, fp16_accum, stream=stream,
+                     noalloc=noalloc)
     if stream is not None:
         stream.sync()
     return d_out.numpy()

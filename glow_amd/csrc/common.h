@@ -31,6 +31,9 @@ inline bool shift_ok(int32_t s) { return s >= 0 && s <= 31; }
 // allocates (once per device and stream), launches never do.
 int slws_reserve_stream(hipStream_t st);
 int slws_release_stream(hipStream_t st);
+// Looks up, once per device, the address of the fixed scratch array used by
+// mi355x_frwq_slws_noalloc on the current device.
+int slws_init_device();
 
 } // namespace mi355x
 

@@ -105,7 +105,10 @@ int mi355x_init(int device) {
                 "device %d is %s; this library only carries gfx950 code",
                 device, p.gcnArchName);
   }
-  // SparseLengths scratch for launches on the default stream
+  // per-device set-up of the SparseLengths scratch: the fixed array's address
+  // and a buffer for launches on the default stream
+  rc = slws_init_device();
+  if (rc != MI355X_OK) return rc;
   return slws_reserve_stream(nullptr);
 }
 

@@ -1007,6 +1007,44 @@ static int stream_scratch(hipStream_t st, int64_t **ws) {
               kChunkBags);
 }
 
+// The same scratch for callers that must not allocate: a fixed array in the
+// code object, one copy per device, found once per device with
+// hipGetSymbolAddress. Host code never uses the array's name as an address.
+constexpr int kStaticChunks = 4096;   // 32 KiB; 4096 * 4096 = 16.7M bags
+static __device__ __align__(256) int64_t scratch[kStaticChunks];
+static std::mutex g_static_mutex;
+static int64_t *g_static_ptr[64] = {nullptr};
+
+int slws_init_device() {
+  int dev = 0;
+  MI355X_HIP(hipGetDevice(&dev));
+  MI355X_REQUIRE(dev >= 0 && dev < 64, "device index %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_static_mutex);
+  if (!g_static_ptr[dev]) {
+    int64_t *ptr = nullptr;
+    MI355X_HIP(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
+    MI355X_REQUIRE(ptr, "hipGetSymbolAddress returned a NULL address");
+    g_static_ptr[dev] = ptr;
+  }
+  return MI355X_OK;
+}
+
+static int static_scratch(int64_t **ws) {
+  int dev = 0;
+  MI355X_HIP(hipGetDevice(&dev));
+  MI355X_REQUIRE(dev >= 0 && dev < 64, "device index %d out of range", dev);
+  {
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    *ws = g_static_ptr[dev];
+  }
+  if (*ws) return MI355X_OK;
+  int rc = slws_init_device();   // first call on this device
+  if (rc != MI355X_OK) return rc;
+  std::lock_guard<std::mutex> lock(g_static_mutex);
+  *ws = g_static_ptr[dev];
+  return MI355X_OK;
+}
+
 template <int LPB, int BPL>
 static void launch_kind(int kind, bool acc16, dim3 grid, hipStream_t st,
                         const SlwsArgs &a) {
@@ -1113,6 +1151,7 @@ struct SlwsExtra {
   float q_scale = 1.0f;
   int32_t q_offset = 0;
   size_t q_stride = 0;
+  bool static_scratch = false; // chunk sums in the code object's fixed array
 };
 
 static int slws_dispatch(void *dest, int out_is_f16, const uint8_t *data,
@@ -1180,9 +1219,17 @@ static int slws_dispatch(void *dest, int out_is_f16, const uint8_t *data,
     const size_t chunks = (out_rows + kChunkBags - 1) / kChunkBags;
     if (chunks > 1) {
       int64_t *ws = nullptr;
-      MI355X_REQUIRE(chunks <= (size_t)kMaxChunks, "more than %d bags",
-                     kMaxChunks * kChunkBags);
-      int rc = stream_scratch(st, &ws);
+      int rc;
+      if (x.static_scratch) {
+        MI355X_REQUIRE(chunks <= (size_t)kStaticChunks,
+                       "%zu bags: the entry point that allocates nothing takes at "
+                       "most %d", out_rows, kStaticChunks * kChunkBags);
+        rc = static_scratch(&ws);
+      } else {
+        MI355X_REQUIRE(chunks <= (size_t)kMaxChunks, "more than %d bags",
+                       kMaxChunks * kChunkBags);
+        rc = stream_scratch(st, &ws);
+      }
       if (rc != MI355X_OK) return rc;
       hipLaunchKernelGGL(slws_chunk_sums_kernel, dim3((unsigned)chunks),
                          dim3(256), 0, st, lengths, (long long)out_rows, ws);
@@ -1310,6 +1357,24 @@ int mi355x_frwq_slws(void *dest, int out_is_f16, const uint8_t *data,
                        weights_are_f16, indices, idx_is_64, num_indices,
                        lengths, nullptr, 0, segments, in_line_size,
                        out_line_size, fp16_accum, stream);
+}
+
+int mi355x_frwq_slws_noalloc(void *dest, int out_is_f16, const uint8_t *data,
+                             size_t data_rows, int kind, const void *weights,
+                             int weights_are_f16, const void *indices, int idx_is_64,
+                             size_t num_indices, const int32_t *lengths,
+                             size_t segments, size_t in_line_size,
+                             size_t out_line_size, int fp16_accum, void *stream) {
+  MI355X_REQUIRE(segments == 0 || lengths, "lengths is NULL");
+  MI355X_REQUIRE(segments <= (size_t)kStaticChunks * kChunkBags,
+                 "%zu bags: mi355x_frwq_slws_noalloc takes at most %d", segments,
+                 kStaticChunks * kChunkBags);
+  SlwsExtra x;
+  x.static_scratch = true;
+  return slws_dispatch(dest, out_is_f16, data, data_rows, kind, weights,
+                       weights_are_f16, indices, idx_is_64, num_indices,
+                       lengths, nullptr, 0, segments, in_line_size,
+                       out_line_size, fp16_accum, stream, x);
 }
 
 int mi355x_slws_reserve_stream(void *stream) {

@@ -515,6 +515,25 @@ int mi355x_frwq_slws(void *dest, int out_is_f16, const uint8_t *data,
  * with MI355X_ERR_INVALID_ARGUMENT). No counterpart in the reference. */
 int mi355x_slws_reserve_stream(void *stream);
 
+/* mi355x_frwq_slws for callers that cannot allocate device memory at all (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc): same arguments, same kernels, same results, but the scratch of
+ * the bag-offset pre-pass is a fixed 32 KiB array inside the library's code
+ * object (one copy per GPU, held until the process ends) instead of a
+ * per-stream buffer, so neither this call nor any set-up it needs calls
+ * hipMalloc or hipFree. At most 4096 * 4096 = 16 777 216 bags per call (more
+ * is MI355X_ERR_INVALID_ARGUMENT). All calls on one GPU share the array: calls
+ * that overlap in time on one GPU (different streams) race on it when either
+ * has more than 4096 bags; calls on one stream are ordered and safe. Nothing
+ * in the array has to start at zero: the pre-pass writes every entry the
+ * lookup reads. No counterpart in the reference. */
+int mi355x_frwq_slws_noalloc(void *dest, int out_is_f16, const uint8_t *data,
+                             size_t data_rows, int kind, const void *weights,
+                             int weights_are_f16, const void *indices, int idx_is_64,
+                             size_t num_indices, const int32_t *lengths,
+                             size_t segments, size_t in_line_size,
+                             size_t out_line_size, int fp16_accum, void *stream);
+
 /* Arithmetic of the SparseLengths kernels (process-wide; default on).
  * On: rows of 32, 64, 128 or 256 data bytes with fp32 accumulation are summed
  * as sum_j (w_j*s_j)*q_jk + sum_j (w_j*o_j) with fused multiply-adds. The CPU
