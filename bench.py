@@ -9,11 +9,20 @@ reference's SLS benchmark counts bytes (tests/benchmark/CommonSLSEB.h:120-176:
 every lookup moves its row, scale and offset, index and weight; plus lengths
 and output; no credit for cache hits).
 
+The timed steps cycle through 64 distinct index batches (about 22 MB of table
+rows each, 1.4 GB in all) and the caches are flushed with a 1 GiB copy between
+the untimed and the timed replay, so the rows a step reads come from HBM and
+not from the 256 MB last-level cache; the rows that Zipf makes hot stay hot
+across steps, as they would in service.
+
 Prints ONE JSON line. Besides the headline it reports, under "extra", the
-int8 matrix-core kernels (RowwiseQuantizedFullyConnected at the single-FC
-configuration and at a large shape, ChannelwiseQuantizedConvolution at the
-ResNet-50 3x3x64 layer shape) and the elementwise kernels, each with its own
-roofline fraction, and times the CPU oracle on this host's cores.
+same lookup with a cache-resident working set and with the strict (bit-exact)
+arithmetic, the int8 matrix-core kernels (RowwiseQuantizedFullyConnected at
+the single-FC configuration and at a large shape,
+ChannelwiseQuantizedConvolution at the ResNet-50 3x3x64 layer shape) and the
+elementwise kernels, each with its own roofline fraction and a comparison of
+a sample of its output with the CPU oracle, the two networks, and times the
+CPU oracle on this host's cores.
 
   python bench.py --gpus 1 --steps 200 --warmup 20
 """
@@ -43,13 +52,18 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--batches", type=int, default=8,
+    ap.add_argument("--batches", type=int, default=64,
                     help="distinct index batches cycled through by the steps")
     ap.add_argument("--rows", type=int, default=4_000_000)
     ap.add_argument("--bags", type=int, default=4096,
                     help="bags per step (4096 is the headline configuration)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0,
                     help="wall-clock budget of the CPU baseline leg")
+    ap.add_argument("--cpu-threads", type=int, default=16,
+                    help="threads of the all-cores CPU leg: the CPU share of a one-GPU job "
+                         "on the benchmark host (capped by the cores this process may use)")
+    ap.add_argument("--net-replays", type=int, default=30,
+                    help="timed replays of the two networks (at least 20)")
     ap.add_argument("--resnet-batch", type=int, default=64)
     ap.add_argument("--resnet-profile-images", type=int, default=100)
     ap.add_argument("--dlrm-rows", type=int, default=1_000_000)
@@ -57,21 +71,24 @@ def parse():
                     help="headline workload only")
     ap.add_argument("--only", default="",
                     help="run a single extra kernel (profiling aid): "
-                         "slws|fc_large|fc_large_zero|fc_c1|fc_m16384|fc_mid|conv_c3|quantize|dequantize|"
-                         "rescale|copy|resnet50|dlrm")
+                         "slws|slws_warm|slws_strict|fc_large|fc_large_zero|fc_c1|fc_m16384|fc_mid|"
+                         "conv_c3|quantize|dequantize|rescale|copy|resnet50|dlrm")
     ap.add_argument("--tile", type=int, default=-1,
                     help="force a workgroup tile for the matrix-core legs of --only "
                          "(0..5, see mi355x_gemm_tile_override; default: chosen from the shape)")
     return ap.parse_args()
 
 
-def timed_launches(capi, fn, steps, warmup):
+def timed_launches(capi, fn, steps, warmup, flush=None, during=None):
     """Average seconds per launch. `fn(i, stream)` issues launch i. After
     `warmup` eager launches, the `steps` timed launches are recorded into one
     launch graph and replayed, so the figure is the device-side rate and not
     the host's enqueue rate (a Python -> ctypes -> HIP launch costs 4-6 us,
     more than some of these kernels take). HIP events bracket the replay on
-    the stream it runs on, with the device idle before and after."""
+    the stream it runs on, with the device idle before and after.
+    `flush(stream)` runs between the untimed and the timed replay (cache
+    flush); `during()` is called while the timed replay runs (it may queue work
+    on other streams) and its result is returned beside the time."""
     stream = capi.Stream()
     for i in range(warmup):
         fn(i, stream)
@@ -81,16 +98,70 @@ def timed_launches(capi, fn, steps, warmup):
             fn(warmup + i, stream)
     graph.launch()          # untimed first replay (uploads the graph)
     stream.sync()
+    if flush is not None:
+        flush(stream)
+        stream.sync()
     capi.sync()
     e0, e1 = capi.Event(), capi.Event()
     e0.record(stream)
     graph.launch()
     e1.record(stream)
+    seen = during() if during is not None else None
     e1.sync()
     capi.sync()
     sec = e0.elapsed_ms(e1) * 1e-3 / steps
     graph.destroy()
-    return sec
+    return (sec, seen) if during is not None else sec
+
+
+class CacheFlush:
+    """A 1 GiB device copy: four times the 256 MB last-level cache, so whatever
+    earlier launches left in the caches is gone when it ends."""
+
+    def __init__(self, capi, nbytes=1 << 30):
+        self.capi, self.n = capi, nbytes
+        self.src = capi.DeviceBuffer.empty((nbytes,), np.uint8)
+        self.dst = capi.DeviceBuffer.empty((nbytes,), np.uint8)
+        self.src.fill(1)
+        capi.sync()
+
+    def __call__(self, stream):
+        self.capi.launch_copy_u8(self.dst, self.src, self.n, stream)
+
+
+class ClockProbe:
+    """`probes` clock probes of `micros` us each on a stream of their own:
+    launch() queues them (nothing in it waits for the device, so it can be
+    called while other work runs), result() gives the shader clock each saw."""
+
+    def __init__(self, capi, micros=200, probes=24):
+        import ctypes as C
+        self.capi, self.micros, self.probes = capi, micros, probes
+        self.stream = capi.Stream()
+        self.out = capi.DeviceBuffer.empty((probes, 2), np.uint64)
+        self.out.fill(0)
+        khz = C.c_int(0)
+        capi.check(capi.lib().mi355x_wall_clock_khz(C.byref(khz)))
+        self.khz = khz.value
+        capi.sync()
+
+    def launch(self):
+        import ctypes as C
+        for i in range(self.probes):
+            self.capi.check(self.capi.lib().mi355x_shader_clock_probe(
+                C.c_void_p(self.out.ptr + 16 * i), C.c_uint32(self.micros),
+                C.c_void_p(self.stream.ptr)))
+        return self
+
+    def result(self):
+        self.stream.sync()
+        v = self.out.numpy().astype(np.float64)
+        ok = v[:, 1] > 0
+        if not ok.any():
+            return None
+        mhz = v[ok, 0] / v[ok, 1] * self.khz / 1e3
+        return dict(median=float(np.median(mhz)), min=float(mhz.min()), max=float(mhz.max()),
+                    probes=int(ok.sum()), probe_us=self.micros)
 
 
 def slws_bytes(total_lookups, bags, cols, row_bytes):
@@ -98,16 +169,22 @@ def slws_bytes(total_lookups, bags, cols, row_bytes):
     return total_lookups * (row_bytes + 8 + 4) + bags * 4 + bags * cols * 4
 
 
-def bench_slws(capi, cases, args, table, d_table):
-    rows, cols, bags = args.rows, 128, args.bags
-    row_bytes = cols + 8
+def make_slws_batches(capi, cases, args, count):
     batches = []
-    for b in range(args.batches):
-        lengths, idx, w = cases.slws_batch(1000 + b, rows, bags, 40, 1.05, np.int64)
+    for b in range(count):
+        lengths, idx, w = cases.slws_batch(1000 + b, args.rows, args.bags, 40, 1.05, np.int64)
         batches.append(dict(
             lengths=lengths, idx=idx, w=w, total=int(lengths.sum()),
             d_len=capi.to_device(lengths), d_idx=capi.to_device(idx),
             d_w=capi.to_device(w)))
+    return batches
+
+
+def bench_slws(capi, args, d_table, batches, flush):
+    """Times args.steps launches that cycle through `batches`; `flush` (or None)
+    empties the caches before the timed replay."""
+    rows, cols, bags = args.rows, 128, args.bags
+    row_bytes = cols + 8
     d_out = capi.DeviceBuffer.empty((bags, cols), np.float32)
 
     def step(i, stream):
@@ -116,12 +193,24 @@ def bench_slws(capi, cases, args, table, d_table):
                               b["d_w"], False, b["d_idx"], True, b["total"],
                               b["d_len"], bags, row_bytes, cols, stream=stream)
 
-    sec = timed_launches(capi, step, args.steps, args.warmup)
+    sec = timed_launches(capi, step, args.steps, args.warmup, flush=flush)
     mean_total = float(np.mean([batches[(args.warmup + i) % len(batches)]["total"]
                                 for i in range(args.steps)]))
     nbytes = slws_bytes(mean_total, bags, cols, row_bytes)
+    last = batches[(args.warmup + args.steps - 1) % len(batches)]
     return dict(sec=sec, bytes=nbytes, batches=batches, mean_lookups=mean_total,
-                d_out=d_out)
+                d_out=d_out, last=last)
+
+
+def slws_errors(got, want, table, b):
+    """(max error over the magnitude a bag adds up, max element-wise relative
+    error over the outputs with |want| >= 1, share of outputs above that floor)."""
+    from glow_amd import workloads
+    ratio = workloads.slws_error_ratio(got, want, table, b["w"], b["idx"], b["lengths"])
+    big = np.abs(want) >= 1.0
+    rel = float(np.max(np.abs(got[big].astype(np.float64) - want[big]) / np.abs(want[big]))) \
+        if big.any() else 0.0
+    return ratio, rel, float(big.mean())
 
 
 def bench_slws_with_h2d(capi, s, args, d_table):
@@ -160,34 +249,45 @@ def bench_slws_with_h2d(capi, s, args, d_table):
                 h2d_bytes_per_step=s["mean_lookups"] * 12 + bags * 4)
 
 
-def bench_slws_more_bags(capi, cases, args, d_table, bags):
+def bench_slws_more_bags(capi, cases, args, d_table, bags, flush):
     """The headline lookup on the same table with a larger batch: the part of a
     launch that does not shrink with the batch (dispatch, bag offsets, the
-    index -> row dependent round trips) is spread over more bytes."""
+    index -> row dependent round trips) is spread over more bytes. Enough
+    distinct batches are cycled that their rows exceed the last-level cache
+    twice over, and the caches are flushed before the timed replay."""
     rows, cols = args.rows, 128
-    lengths, idx, w = cases.slws_batch(2000 + bags, rows, bags, 40, 1.05, np.int64)
-    total = int(lengths.sum())
-    d_len, d_idx, d_w = capi.to_device(lengths), capi.to_device(idx), capi.to_device(w)
+    count = max(2, int(np.ceil(600e6 / (bags * 40 * 136.0))))
+    bs = []
+    for k in range(count):
+        lengths, idx, w = cases.slws_batch(2000 + bags + k, rows, bags, 40, 1.05, np.int64)
+        bs.append((int(lengths.sum()), capi.to_device(lengths), capi.to_device(idx),
+                   capi.to_device(w)))
     d_out = capi.DeviceBuffer.empty((bags, cols), np.float32)
 
-    def step(_, stream):
+    def step(i, stream):
+        total, d_len, d_idx, d_w = bs[i % count]
         capi.launch_frwq_slws(d_out, False, d_table, rows, capi.FUSED_U8_F32, d_w, False, d_idx,
                               True, total, d_len, bags, cols + 8, cols, stream=stream)
 
-    sec = timed_launches(capi, step, max(20, args.steps // 4), max(3, args.warmup // 4))
+    steps, warmup = max(20, args.steps // 4), max(3, args.warmup // 4)
+    sec = timed_launches(capi, step, steps, warmup, flush=flush)
+    total = float(np.mean([bs[(warmup + i) % count][0] for i in range(steps)]))
     nbytes = slws_bytes(total, bags, cols, cols + 8)
-    return dict(workload=f"SLWS, same table, {bags} bags ({total} lookups)", ms=sec * 1e3,
-                gbps=nbytes / sec / 1e9, frac_of_hbm_peak=nbytes / sec / 1e9 / HBM_PEAK_GBPS)
+    return dict(workload=f"SLWS, same table, {bags} bags ({total:.0f} lookups), {count} batches cycled",
+                ms=sec * 1e3, gbps=nbytes / sec / 1e9,
+                frac_of_hbm_peak=nbytes / sec / 1e9 / HBM_PEAK_GBPS)
 
 
-def cpu_all_cores_slws(table, batches, budget_s):
-    """The oracle on every host core this process may use, one whole batch per
-    thread at a time (the reference's CPU backend exposes one device per
-    hardware thread, lib/Backends/CPU/CPUBackend.cpp:114-116)."""
+def cpu_all_cores_slws(table, batches, budget_s, threads):
+    """The oracle on the host cores of this job, one whole batch per thread at a
+    time (the reference's CPU backend exposes one device per hardware thread,
+    lib/Backends/CPU/CPUBackend.cpp:114-116). `threads` is the job's CPU share
+    (16 for a one-GPU job on the benchmark host, whatever the machine has),
+    capped by the cores this process may run on."""
     import threading
     from oracle import glow_oracle as go
-    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
-    cores = max(1, min(cores, 16))
+    avail = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
+    cores = max(1, min(avail, threads))
     done = [0.0] * cores
     t0 = time.perf_counter()
 
@@ -198,7 +298,6 @@ def cpu_all_cores_slws(table, batches, budget_s):
             go.frwq_slws_f32(table, b["w"], b["idx"], b["lengths"])
             done[t] += slws_bytes(b["total"], b["lengths"].size, 128, 136)
             n += cores
-
     th = [threading.Thread(target=work, args=(t,)) for t in range(cores)]
     for t in th:
         t.start()
@@ -206,21 +305,14 @@ def cpu_all_cores_slws(table, batches, budget_s):
         t.join()
     el = time.perf_counter() - t0
     return dict(value=sum(done) / el / 1e9, unit="GB/s", cores=cores, kind="port",
+                cores_visible=avail,
                 sample=f"whole batches for {el:.1f} s, one batch per thread at a time")
 
 
-def cpu_baseline_slws(table, batches, budget_s, gpu_out, gpu_batch):
+def cpu_baseline_slws(table, batches, budget_s, native):
     """The CPU leg: the oracle (the restated libjit loop, one thread) over
-    whole batches of the same workload until the time budget is used. As the
-    checker it also confirms the GPU output of the last timed step."""
+    whole batches of the same workload until the time budget is used."""
     from oracle import glow_oracle as go
-    want = go.frwq_slws_f32(table, gpu_batch["w"], gpu_batch["idx"],
-                            gpu_batch["lengths"])
-    # default (fused multiply-add) arithmetic: equal to the sequential CPU loop
-    # to rounding; the bar is 1e-5 of the magnitude a bag adds up
-    from glow_amd import workloads
-    parity = workloads.slws_error_ratio(gpu_out, want, table, gpu_batch["w"],
-                                        gpu_batch["idx"], gpu_batch["lengths"])
     done_bytes, n = 0.0, 0
     t0 = time.perf_counter()
     while True:
@@ -231,12 +323,47 @@ def cpu_baseline_slws(table, batches, budget_s, gpu_out, gpu_batch):
         el = time.perf_counter() - t0
         if el >= budget_s or n >= 4000:
             break
+    build = "-O3 -march=native, built on this host" if native else "-O3, portable build"
     return dict(value=done_bytes / el / 1e9, unit="GB/s", cores=1, kind="port",
                 sample=f"{n} full batches of {batches[0]['lengths'].size} bags (single thread, "
-                       f"{el:.1f} s) of the same table and index batches"), parity
+                       f"{el:.1f} s) of the same table and index batches; oracle compiled {build}")
 
 
-def bench_fc(capi, cases, M, K, N, steps, warmup, seed=5, zero_leg=False):
+def cpu_reference_libjit_slws(table, batches, budget_s):
+    """The reference's own libjit (its sources compiled unmodified, with the
+    reference's default -ffast-math flags, -O2, portable code) on the same
+    batches, one thread; None where that library has not been built."""
+    from oracle import libjit_ref
+    if not libjit_ref.available(fastmath=True):
+        return None
+    done_bytes, n = 0.0, 0
+    t0 = time.perf_counter()
+    while True:
+        b = batches[n % len(batches)]
+        libjit_ref.frwq_slws_f32(table, b["w"], b["idx"], b["lengths"], fastmath=True)
+        done_bytes += slws_bytes(b["total"], b["lengths"].size, 128, 136)
+        n += 1
+        el = time.perf_counter() - t0
+        if el >= budget_s or n >= 4000:
+            break
+    return dict(value=done_bytes / el / 1e9, unit="GB/s", cores=1, kind="reference",
+                sample=f"{n} full batches (single thread, {el:.1f} s); libjit.cpp compiled "
+                       "-O2 -ffast-math -fno-finite-math-only for generic x86-64")
+
+
+def oracle_rows_check(capi, c, d_out, M, rows):
+    """Rows `rows` of the device result against the oracle run on those rows."""
+    from oracle import glow_oracle as go
+    got = d_out.numpy()
+    cs = dict(c, x=np.ascontiguousarray(c["x"][rows]))
+    want = go.rwq_fc_i8(cs["x"], c["w"], c["bias"], c["w_offsets"], c["bias_pre"],
+                        c["bias_post"], c["bias_scale"], c["out_pre"], c["out_post"],
+                        c["out_scale"], c["out_offset"], c["in_offset"], c["bias_offset"])
+    return bool(np.array_equal(got[rows], want)), int(len(rows))
+
+
+def bench_fc(capi, cases, M, K, N, steps, warmup, seed=5, zero_leg=False, check=True,
+             clock=False):
     c = cases.rwq_fc_case(seed, M, K, N) if M * K <= (1 << 24) else None
     rng = np.random.default_rng(seed)
     if c is None:
@@ -260,8 +387,23 @@ def bench_fc(capi, cases, M, K, N, steps, warmup, seed=5, zero_leg=False):
                               c["in_offset"], c["bias_offset"], True,
                               w_row_sums=d_sums, stream=stream)
 
-    sec = timed_launches(capi, step, steps, warmup)
+    clocks = None
+    if clock:
+        # the shader clock the part holds while this kernel runs, sampled from
+        # a second stream during the timed replay, and the clock of the idle part
+        idle = ClockProbe(capi).launch().result()
+        probe = ClockProbe(capi)
+        sec, _ = timed_launches(capi, step, steps, warmup, during=probe.launch)
+        clocks = dict(during_timed_launches_mhz=probe.result(), idle_mhz=idle)
+    else:
+        sec = timed_launches(capi, step, steps, warmup)
     ops = 2.0 * M * N * K
+    parity = None
+    if check:
+        # the oracle on a row sample of what the timed launches left behind
+        step_rows = max(1, M // 24)
+        rows = np.unique(np.r_[0:min(M, 8), np.arange(0, M, step_rows), M - 1])[:40]
+        parity = oracle_rows_check(capi, c, d_out, M, rows)
     zero = None
     if zero_leg:
         # The same launch on all-zero operands: identical instruction stream,
@@ -271,7 +413,12 @@ def bench_fc(capi, cases, M, K, N, steps, warmup, seed=5, zero_leg=False):
         d["x"].fill(0)
         d["w"].fill(0)
         capi.sync()
-        zsec = timed_launches(capi, step, steps, warmup)
+        if clock:
+            probe = ClockProbe(capi)
+            zsec, _ = timed_launches(capi, step, steps, warmup, during=probe.launch)
+            clocks["zero_operands_mhz"] = probe.result()
+        else:
+            zsec = timed_launches(capi, step, steps, warmup)
         zero = dict(ms=zsec * 1e3, tops=ops / zsec / 1e12)
     normal = None
     if zero_leg:
@@ -288,6 +435,9 @@ def bench_fc(capi, cases, M, K, N, steps, warmup, seed=5, zero_leg=False):
         normal = dict(ms=nsec * 1e3, tops=ops / nsec / 1e12)
     return dict(workload=f"rwq_fc M{M} K{K} N{N}", ms=sec * 1e3,
                 tops=ops / sec / 1e12, zero_operands=zero, normal_weights=normal,
+                shader_clock=clocks,
+                parity_with_oracle=(None if parity is None else parity[0]),
+                rows_checked=(None if parity is None else parity[1]),
                 roofline=dict(bound="mfma", achieved=ops / sec / 1e12,
                               peak=INT8_PEAK_TOPS, unit="TOP/s",
                               frac=ops / sec / 1e12 / INT8_PEAK_TOPS,
@@ -296,7 +446,7 @@ def bench_fc(capi, cases, M, K, N, steps, warmup, seed=5, zero_leg=False):
                 gbps=(M * K + N * K + M * N + 8 * 4 * N) / sec / 1e9)
 
 
-def bench_conv(capi, cases, steps, warmup):
+def bench_conv(capi, cases, steps, warmup, check=True):
     c = cases.cwq_conv_case(7, 32, 56, 56, 64, 64, in_offset=-128)
     g = capi._geom(c["geom"])
     d = {k: capi.to_device(np.ascontiguousarray(v)) for k, v in c.items()
@@ -315,10 +465,22 @@ def bench_conv(capi, cases, steps, warmup):
                                   stream=stream)
 
     sec = timed_launches(capi, step, steps, warmup)
+    parity = None
+    if check:
+        # images 0 and 31 of what the timed launches left behind, on the oracle
+        from oracle import glow_oracle as go
+        got = d_out.numpy()
+        pick = [0, g.N - 1]
+        c2 = dict(c, x=np.ascontiguousarray(c["x"][pick]),
+                  geom=go.conv_geom(len(pick), g.IH, g.IW, g.IC, g.OC, (g.KH, g.KW),
+                                    (g.strideH, g.strideW), (g.padT, g.padL, g.padT, g.padL)))
+        want = go.cwq_conv2d_i8(*cases.cwq_conv_args(c2))
+        parity = bool(np.array_equal(got[pick], want))
     ops = 2.0 * g.N * g.OH * g.OW * g.OC * g.KH * g.KW * g.IC
     nbytes = c["x"].size + d_out.nbytes + c["filt"].size + 9 * 4 * g.OC
     return dict(workload="cwq_conv2d 32x56x56x64 3x3x64->64 s1 p1 relu",
                 ms=sec * 1e3, tops=ops / sec / 1e12, gbps=nbytes / sec / 1e9,
+                parity_with_oracle=parity, images_checked=(2 if check else None),
                 roofline=dict(bound="mfma", achieved=ops / sec / 1e12,
                               peak=INT8_PEAK_TOPS, unit="TOP/s",
                               frac=ops / sec / 1e12 / INT8_PEAK_TOPS,
@@ -394,21 +556,25 @@ def cpu_baseline_mfma_kernels(budget_s):
     return out
 
 
-def bench_resnet50(args):
+def bench_resnet50(args, check=True):
     """Int8 ResNet-50 at batch 64, 224x224 through MI355XDeviceManager:
     images/s of the resident network replayed on device-resident input
     (device time), and of whole requests including the fp32 input upload and
-    the result download."""
+    the result download. The first and the last image of the batch are run
+    through the oracle executing the same quantized graph."""
     from glow_amd import host as H
     from glow_amd.harness import net as netlib
     from glow_amd.harness import resnet50
     batch, size = args.resnet_batch, 224
     t0 = time.perf_counter()
-    net = resnet50.make(batch=batch, size=size, profile_images=args.resnet_profile_images)
+    steps = resnet50.build_fp32(0)
+    ranges = resnet50.profile(steps, resnet50.synthetic_images(1, args.resnet_profile_images, size))
+    net = resnet50.build_int8(steps, ranges, batch, size)
     t_build = time.perf_counter() - t0
     m, f = netlib.to_module(net)
     m.compile(f)
     dm = H.DeviceManager().init()
+    reps = max(20, args.net_replays)
     try:
         dm.add_network(m)
         # request buffers in pinned host memory (allocateDeviceIOBuffer)
@@ -417,7 +583,6 @@ def bench_resnet50(args):
         prob = capi.pinned_empty((batch, 1000), np.float32)
         logits = capi.pinned_empty((batch, 1000), np.int8)
         dm.run("main", {"input": x, "prob": prob, "logits_q": logits})
-        reps = max(3, args.steps // 10)
         ms = dm.time_function("main", reps)
         t1 = time.perf_counter()
         for _ in range(3):
@@ -425,22 +590,34 @@ def bench_resnet50(args):
         e2e = (time.perf_counter() - t1) / 3
     finally:
         dm.stop()
+    parity = None
+    if check:
+        from tests import oracle_exec
+        pick = [0, batch - 1]
+        two = resnet50.build_int8(steps, ranges, len(pick), size)
+        want = oracle_exec.run(two, {"input": np.ascontiguousarray(np.asarray(x)[pick])})
+        parity = bool(np.array_equal(np.asarray(logits)[pick], want["logits_q"]) and
+                      np.allclose(np.asarray(prob)[pick], want["prob"], rtol=1e-5, atol=1e-30))
     ops = net.ops_count()
     return dict(workload=f"int8 ResNet-50, batch {batch}, {size}x{size}x3, channelwise-quantized "
                          f"convolutions, rowwise-quantized FC, fp32 softmax; "
                          f"{args.resnet_profile_images} profiling images",
-                images_per_s=batch / (ms * 1e-3), ms_per_batch=ms,
+                images_per_s=batch / (ms * 1e-3), ms_per_batch=ms, timed_replays=reps,
                 images_per_s_with_host_copies=batch / e2e,
                 tops=ops / (ms * 1e-3) / 1e12, gop_per_image=ops / batch / 1e9,
                 launches_per_batch=len([r for r in H.parse_listing(m.describe(f))
                                         if r["phase"] == "launch"]),
+                parity_with_oracle=parity, images_checked=(2 if check else None),
                 prob_row_sum=float(prob[0].sum()), host_build_seconds=t_build)
 
 
-def bench_dlrm(args):
+def bench_dlrm(args, check=True):
     """DLRM-style ranking net, batch 4096: 26 tables of 1M x 64 (4-bit fused,
     fp16 scale/offset), Poisson(20) bags of Zipf(1.1) int64 indices, int8 MLPs
-    13-512-256-64 and 415-512-256-1, dot interaction, sigmoid."""
+    13-512-256-64 and 415-512-256-1, dot interaction, sigmoid. The whole batch
+    is run through the oracle executing the same quantized graph; the lookups
+    run the library's default (fused multiply-add) arithmetic, which may move
+    an int8 logit by one quantization step against the sequential CPU sum."""
     from glow_amd import host as H
     from glow_amd.harness import dlrm
     from glow_amd.harness import net as netlib
@@ -451,30 +628,41 @@ def bench_dlrm(args):
     m, f = netlib.to_module(net)
     m.compile(f)
     dm = H.DeviceManager().init()
+    reps = max(20, args.net_replays)
     try:
         dm.add_network(m)
         inp = dlrm.Inputs(99, tables, args.dlrm_rows, batch, 20, 1.1, 13)
         from glow_amd import capi
-        b = {k: capi.pinned_copy(v) for k, v in dlrm.bindings(net, inp, max_idx).items()}
+        hb = dlrm.bindings(net, inp, max_idx)
+        b = {k: capi.pinned_copy(v) for k, v in hb.items()}
         prob = capi.pinned_empty((batch, 1), np.float32)
-        dm.run("main", dict(b, prob=prob))
-        reps = max(5, args.steps // 4)
+        logit = capi.pinned_empty((batch, 1), np.int8)
+        dm.run("main", dict(b, prob=prob, logit_q=logit))
         ms = dm.time_function("main", reps)
         t1 = time.perf_counter()
         for _ in range(3):
-            dm.run("main", dict(b, prob=prob))
+            dm.run("main", dict(b, prob=prob, logit_q=logit))
         e2e = (time.perf_counter() - t1) / 3
     finally:
         dm.stop()
+    parity, off_by_one = None, None
+    if check:
+        from tests import oracle_exec
+        want = oracle_exec.run(net, hb)
+        d = np.abs(np.asarray(logit).astype(np.int32) - want["logit_q"].astype(np.int32))
+        off_by_one = int((d == 1).sum())
+        parity = bool(d.max() <= 1 and (d > 0).mean() <= 0.05)
     lookups = int(sum(int(l.sum()) for l in inp.lengths))
     sls_bytes = lookups * (36 + 8) + tables * batch * (4 + 64 * 2)
     return dict(workload=f"DLRM-style net, batch {batch}, {tables} tables x {args.dlrm_rows} rows x 64 "
                          "(4-bit fused, fp16 scale/offset), Poisson(20) bags, Zipf(1.1) int64 indices",
-                samples_per_s=batch / (ms * 1e-3), ms_per_batch=ms,
+                samples_per_s=batch / (ms * 1e-3), ms_per_batch=ms, timed_replays=reps,
                 samples_per_s_with_host_copies=batch / e2e,
                 lookups_per_batch=lookups, sls_algorithmic_mb_per_batch=sls_bytes / 1e6,
                 launches_per_batch=len([r for r in H.parse_listing(m.describe(f))
                                         if r["phase"] == "launch"]),
+                parity_with_oracle=parity, logits_one_step_off=off_by_one,
+                samples_checked=(batch if check else None),
                 prob_mean=float(prob.mean()), host_build_seconds=t_build)
 
 
@@ -503,12 +691,18 @@ def main():
     if args.tile >= 0:
         capi.check(capi.lib().mi355x_gemm_tile_override(args.tile))
 
+    if only and only not in ("slws", "slws_warm", "slws_strict", "fc_large", "fc_large_zero",
+                             "fc_c1", "fc_m16384", "fc_mid", "conv_c3", "quantize", "dequantize",
+                             "rescale", "copy"):
+        print(f"unknown --only {only}", file=sys.stderr)
+        sys.exit(2)
     if only in ("fc_large", "fc_large_zero", "fc_c1", "fc_m16384", "fc_mid", "conv_c3", "quantize",
                 "dequantize", "rescale", "copy"):
         if only == "fc_large":
             r = bench_fc(capi, cases, 8192, 4096, 4096, args.steps, args.warmup)
         elif only == "fc_large_zero":
-            r = bench_fc(capi, cases, 8192, 4096, 4096, args.steps, args.warmup, zero_leg=True)
+            r = bench_fc(capi, cases, 8192, 4096, 4096, args.steps, args.warmup, zero_leg=True,
+                         clock=True)
         elif only == "fc_c1":
             r = bench_fc(capi, cases, 128, 1024, 1024, args.steps, args.warmup)
         elif only == "fc_m16384":
@@ -527,35 +721,78 @@ def main():
     rng = np.random.default_rng(42)
     table = cases.random_fused_table(rng, args.rows, 128)
     d_table = capi.to_device(table)
-    s = bench_slws(capi, cases, args, table, d_table)
+    flush = CacheFlush(capi)
+    batches = make_slws_batches(capi, cases, args, args.batches)
+
+    if only == "slws_warm":
+        # the cache-resident variant: 8 batches, no flush
+        s = bench_slws(capi, args, d_table, batches[:8], None)
+    elif only == "slws_strict":
+        capi.slws_set_fused_math(False)
+        s = bench_slws(capi, args, d_table, batches, flush)
+        capi.slws_set_fused_math(True)
+    else:
+        s = bench_slws(capi, args, d_table, batches, flush)
     gbps = s["bytes"] / s["sec"] / 1e9
 
-    # CPU leg: baseline timing, and the check of the last timed step's output
-    last = s["batches"][(args.warmup + args.steps - 1) % len(s["batches"])]
-    cpu, parity = None, None
+    # the check of the last timed step's output (portable build of the oracle),
+    # then the CPU leg on the build for this host
+    cpu, parity, rel, share = None, None, None, None
     if not only and args.cpu_seconds > 0:
-        cpu, parity = cpu_baseline_slws(table, s["batches"], args.cpu_seconds,
-                                        s["d_out"].numpy(), last)
+        from oracle import glow_oracle as go
+        want = go.frwq_slws_f32(table, s["last"]["w"], s["last"]["idx"], s["last"]["lengths"])
+        parity, rel, share = slws_errors(s["d_out"].numpy(), want, table, s["last"])
+        native = go.use_native_build()
+        cpu = cpu_baseline_slws(table, batches, args.cpu_seconds, native)
 
     if not args.no_extra and not only:
         st, wu = max(20, args.steps // 4), max(3, args.warmup // 4)
+        # the same launches with a working set that stays in the last-level
+        # cache: 8 batches (176 MB of rows), no flush
+        w8 = bench_slws(capi, args, d_table, batches[:8], None)
+        extra["slws_warm"] = dict(
+            workload="headline lookup, 8 index batches cycled, caches not flushed "
+                     "(working set inside the 256 MB last-level cache)",
+            ms=w8["sec"] * 1e3, gbps=w8["bytes"] / w8["sec"] / 1e9,
+            frac_of_hbm_peak=w8["bytes"] / w8["sec"] / 1e9 / HBM_PEAK_GBPS)
+        # strict arithmetic: every multiply and add rounded on its own, in bag
+        # order; bit for bit the CPU loop
+        capi.slws_set_fused_math(False)
+        try:
+            ss = bench_slws(capi, args, d_table, batches, flush)
+            bit_exact = None
+            if args.cpu_seconds > 0:
+                from oracle import glow_oracle as go
+                want = go.frwq_slws_f32(table, ss["last"]["w"], ss["last"]["idx"],
+                                        ss["last"]["lengths"])
+                bit_exact = bool(np.array_equal(ss["d_out"].numpy(), want))
+        finally:
+            capi.slws_set_fused_math(True)
+        extra["slws_strict"] = dict(
+            workload="headline lookup with mi355x_slws_set_fused_math(0)",
+            ms=ss["sec"] * 1e3, gbps=ss["bytes"] / ss["sec"] / 1e9,
+            frac_of_hbm_peak=ss["bytes"] / ss["sec"] / 1e9 / HBM_PEAK_GBPS,
+            bit_exact_with_oracle=bit_exact)
         extra["slws_with_h2d"] = bench_slws_with_h2d(capi, s, args, d_table)
-        extra["slws_more_bags"] = [bench_slws_more_bags(capi, cases, args, d_table, n)
+        extra["slws_more_bags"] = [bench_slws_more_bags(capi, cases, args, d_table, n, flush)
                                    for n in (16384, 65536)]
         if args.cpu_seconds > 0:
-            extra["cpu_all_cores"] = cpu_all_cores_slws(table, s["batches"],
-                                                        args.cpu_seconds / 2)
+            extra["cpu_all_cores"] = cpu_all_cores_slws(table, batches, args.cpu_seconds / 2,
+                                                        args.cpu_threads)
+            extra["cpu_reference_libjit"] = cpu_reference_libjit_slws(table, batches,
+                                                                      args.cpu_seconds / 2)
             extra["cpu_mfma_kernels"] = cpu_baseline_mfma_kernels(args.cpu_seconds / 2)
         extra["rwq_fc_c1"] = bench_fc(capi, cases, 128, 1024, 1024, args.steps, args.warmup)
         # enough launches for the clock to settle under the power limit
         extra["rwq_fc_large"] = bench_fc(capi, cases, 8192, 4096, 4096, max(st, 300), max(wu, 30),
-                                             zero_leg=True)
+                                         zero_leg=True, clock=True)
         # the single-FC configuration's own K and N at a large batch
         extra["rwq_fc_m16384"] = bench_fc(capi, cases, 16384, 1024, 1024, max(st, 300),
                                           max(wu, 30))
         extra["cwq_conv_c3"] = bench_conv(capi, cases, args.steps, args.warmup)
         for w in ("quantize", "dequantize", "rescale"):
             extra[w] = bench_elementwise(capi, w, st, wu)
+        del flush
         extra["resnet50_int8"] = bench_resnet50(args)
         extra["dlrm_int8"] = bench_dlrm(args)
 
@@ -585,11 +822,16 @@ def main():
         },
         "parity_with_oracle": (None if parity is None else bool(parity <= 1e-5)),
         "max_error_over_bag_magnitude": parity,
+        "max_rel_error_elementwise": rel,
+        "rel_error_floor": "outputs with |oracle value| >= 1.0",
+        "share_of_outputs_above_floor": share,
+        "cache_state": ("caches flushed before the timed replay; "
+                        f"{args.batches} distinct index batches cycled"),
         "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
                      "traffic": (MEASURED_TRAFFIC["slws"]
                                  if (args.rows, args.bags, args.batches) ==
-                                 (4_000_000, 4096, 8) else None),
+                                 (4_000_000, 4096, 64) and not only else None),
                      "kernel": "slws_rows_kernel<false,false,32,true>"},
         "cpu_baseline": cpu,
         "extra": extra,

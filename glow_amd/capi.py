@@ -45,6 +45,7 @@ EXPORTS = [
     "mi355x_cwq_conv2d_i8", "mi355x_conv2d_i8", "mi355x_frwq_slws",
     "mi355x_embedding_bag_rowwise_offsets",
     "mi355x_slws_reserve_stream", "mi355x_frwq_slws_noalloc",
+    "mi355x_shader_clock_probe", "mi355x_wall_clock_khz",
 ]
 
 

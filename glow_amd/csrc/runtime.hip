@@ -53,6 +53,27 @@ __global__ __launch_bounds__(256) void copy_u8_kernel(uint8_t *__restrict__ dst,
   for (size_t i = done + tid; i < n; i += stride) dst[i] = src[i];
 }
 
+// One wavefront that waits `wall_ticks` ticks of the constant-rate device
+// clock and reports how many shader-clock cycles went by meanwhile:
+// out[0] = shader cycles, out[1] = constant-rate ticks. The wait sleeps between
+// polls and ends after max_polls polls at the latest.
+__global__ __launch_bounds__(64) void clock_probe_kernel(unsigned long long *out,
+                                                         unsigned wall_ticks,
+                                                         unsigned max_polls) {
+  const unsigned long long w0 = wall_clock64();
+  const unsigned long long c0 = clock64();
+  unsigned long long w = w0;
+  for (unsigned i = 0; i < max_polls && w - w0 < wall_ticks; i++) {
+    __builtin_amdgcn_s_sleep(32);
+    w = wall_clock64();
+  }
+  const unsigned long long c1 = clock64();
+  if (threadIdx.x == 0) {
+    out[0] = c1 - c0;
+    out[1] = w - w0;
+  }
+}
+
 } // namespace mi355x
 
 using namespace mi355x;
@@ -203,6 +224,29 @@ int mi355x_copy_u8(void *dst, const void *src, size_t bytes, void *stream) {
                      as_stream(stream), (uint8_t *)dst, (const uint8_t *)src,
                      bytes, vec_ok);
   return check_launch("copy_u8");
+}
+
+int mi355x_shader_clock_probe(uint64_t *out2, uint32_t micros, void *stream) {
+  MI355X_REQUIRE(out2, "out2 is NULL");
+  MI355X_REQUIRE(micros >= 1 && micros <= 100000, "probe time %u us outside [1, 100000]", micros);
+  int dev = 0, khz = 0;
+  MI355X_HIP(hipGetDevice(&dev));
+  MI355X_HIP(hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev));
+  MI355X_REQUIRE(khz > 0, "the device reports no constant-rate clock");
+  const unsigned ticks = (unsigned)((uint64_t)micros * (uint64_t)khz / 1000);
+  // a poll takes well over 100 ns: this many polls outlast the requested time
+  const unsigned max_polls = micros * 16 + 1024;
+  hipLaunchKernelGGL(clock_probe_kernel, dim3(1), dim3(64), 0, as_stream(stream),
+                     (unsigned long long *)out2, ticks, max_polls);
+  return check_launch("clock_probe");
+}
+
+int mi355x_wall_clock_khz(int *khz) {
+  MI355X_REQUIRE(khz, "khz is NULL");
+  int dev = 0;
+  MI355X_HIP(hipGetDevice(&dev));
+  MI355X_HIP(hipDeviceGetAttribute(khz, hipDeviceAttributeWallClockRate, dev));
+  return MI355X_OK;
 }
 
 int mi355x_stream_create(void **stream) {

@@ -82,6 +82,15 @@ int mi355x_fill_u8(void *dst, int value, size_t bytes, void *stream);
  * byte counters are calibrated against. */
 int mi355x_copy_u8(void *dst, const void *src, size_t bytes, void *stream);
 
+/* Measurement aid (no counterpart in the reference): one wavefront waits
+ * `micros` microseconds of the device's constant-rate clock and writes
+ * out2[0] = shader-clock cycles that went by, out2[1] = constant-rate ticks
+ * (mi355x_wall_clock_khz per millisecond), both uint64 in DEVICE memory. Run on
+ * a second stream while a kernel runs on the first, cycles / ticks is the
+ * shader clock the part holds under that kernel's power draw. */
+int mi355x_shader_clock_probe(uint64_t *out2, uint32_t micros, void *stream);
+int mi355x_wall_clock_khz(int *khz);
+
 int mi355x_stream_create(void **stream);
 int mi355x_stream_destroy(void *stream);
 int mi355x_stream_sync(void *stream);

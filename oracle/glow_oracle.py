@@ -48,6 +48,25 @@ def conv_geom(N, IH, IW, IC, OC, kernel, stride, pads, group=1, dilation=(1, 1))
 _lib = None
 
 
+def use_native_build():
+    """Switches this module to a build of the same source for the host it runs
+    on (-O3 -march=native, made here and now by the Makefile's `native`
+    target): what the timed CPU baseline uses. Returns True when that build is
+    in use, False when it could not be made (the portable build stays)."""
+    global _lib, _LIB_PATH
+    native = os.path.join(_HERE, "_native", "libglow_oracle_native.so")
+    try:
+        subprocess.check_call(["make", "-C", _HERE, "native"], stdout=subprocess.DEVNULL,
+                              stderr=subprocess.DEVNULL)
+    except (subprocess.CalledProcessError, OSError):
+        return False
+    if not os.path.exists(native):
+        return False
+    _LIB_PATH = native
+    _lib = None
+    return True
+
+
 def lib():
     global _lib
     if _lib is None:
