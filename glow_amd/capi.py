@@ -46,6 +46,7 @@ EXPORTS = [
     "mi355x_embedding_bag_rowwise_offsets",
     "mi355x_slws_reserve_stream", "mi355x_frwq_slws_noalloc",
     "mi355x_shader_clock_probe", "mi355x_wall_clock_khz",
+    "mi355x_specialize_bias_qparams", "mi355x_channelwise_quantize_conv_host",
 ]
 
 
@@ -395,6 +396,34 @@ def specialize_bias_weights_qparams(bias_scale, bias_offset, input_scale, weight
         C.byref(bs), C.byref(bo), C.c_float(input_scale), C.byref(ws),
         C.c_int(int(bias_is_i32)), C.c_int(int(bias_is_zero))))
     return bs.value, bo.value, ws.value
+
+
+def specialize_bias_qparams(bias_scale, bias_offset, input_scale, weights_scale,
+                            bias_is_i32=True, bias_is_zero=False):
+    """specializeBiasQuantizationParams -> (bias_scale, bias_offset)."""
+    bs, bo = C.c_float(bias_scale), C.c_int32(bias_offset)
+    check(lib().mi355x_specialize_bias_qparams(
+        C.byref(bs), C.byref(bo), C.c_float(input_scale), C.c_float(weights_scale),
+        C.c_int(bool(bias_is_i32)), C.c_int(bool(bias_is_zero))))
+    return bs.value, bo.value
+
+
+def channelwise_quantize_conv_host(filter_f, bias_f, input_scale, schema=SCHEMA_SYMMETRIC):
+    """createChannelwiseQuantizedConv's constants for a float filter [OC, ...] and
+    float bias [OC] -> (filter_q int8, bias_q int32, filter_scales, filter_offsets,
+    bias_scales, bias_offsets)."""
+    f = np.ascontiguousarray(filter_f, np.float32)
+    b = np.ascontiguousarray(bias_f, np.float32)
+    oc = f.shape[0]
+    per = f.size // max(oc, 1)
+    fq = np.empty(f.shape, np.int8)
+    bq = np.empty(oc, np.int32)
+    fs, bs = np.empty(oc, np.float32), np.empty(oc, np.float32)
+    fo, bo = np.empty(oc, np.int32), np.empty(oc, np.int32)
+    check(lib().mi355x_channelwise_quantize_conv_host(
+        _vp(f), _vp(b), _sz(oc), _sz(per), C.c_float(input_scale), C.c_int(schema),
+        _vp(fq), _vp(bq), _vp(fs), _vp(fo), _vp(bs), _vp(bo)))
+    return fq, bq, fs, fo, bs, bo
 
 
 def fused_row_bytes(cols, kind):

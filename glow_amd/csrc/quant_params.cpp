@@ -226,6 +226,53 @@ int mi355x_specialize_bias_weights_qparams(float *bias_scale, int32_t *bias_offs
   return MI355X_OK;
 }
 
+int mi355x_specialize_bias_qparams(float *bias_scale, int32_t *bias_offset, float input_scale,
+                                   float weights_scale, int bias_is_i32, int bias_is_zero) {
+  MI355X_REQUIRE(bias_scale && bias_offset, "NULL argument");
+  if (bias_is_i32) *bias_offset = 0;
+  const float product = input_scale * weights_scale;
+  // the accumulator's scale is taken only when it does not make the bias saturate
+  if (product >= *bias_scale || bias_is_zero) *bias_scale = product;
+  return MI355X_OK;
+}
+
+int mi355x_channelwise_quantize_conv_host(const float *filter, const float *bias,
+                                          size_t channels, size_t per_channel,
+                                          float input_scale, int schema, int8_t *filter_q,
+                                          int32_t *bias_q, float *filter_scales,
+                                          int32_t *filter_offsets, float *bias_scales,
+                                          int32_t *bias_offsets) {
+  if (channels == 0) return MI355X_OK;
+  MI355X_REQUIRE(filter && bias && filter_q && bias_q && filter_scales && filter_offsets &&
+                     bias_scales && bias_offsets && per_channel > 0,
+                 "NULL or empty tensor");
+  for (size_t c = 0; c < channels; c++) {
+    const float *f = filter + c * per_channel;
+    // filter parameters of the channel from its own range
+    float mn, mx;
+    row_min_max(f, per_channel, mn, mx);
+    int rc = mi355x_choose_quantization_params(mn, mx, schema, MI355X_QTY_INT8,
+                                               &filter_scales[c], &filter_offsets[c]);
+    if (rc != MI355X_OK) return rc;
+    // bias parameters from the one value the channel has, as an int32 tensor
+    rc = mi355x_choose_quantization_params(bias[c], bias[c], schema, MI355X_QTY_INT32,
+                                           &bias_scales[c], &bias_offsets[c]);
+    if (rc != MI355X_OK) return rc;
+    // then both are made to agree: bias scale == input scale * filter scale
+    rc = mi355x_specialize_bias_weights_qparams(&bias_scales[c], &bias_offsets[c], input_scale,
+                                                &filter_scales[c], 1, bias[c] == 0.0f);
+    if (rc != MI355X_OK) return rc;
+    for (size_t j = 0; j < per_channel; j++)
+      filter_q[c * per_channel + j] = quantize_to_i8(f[j], filter_scales[c], filter_offsets[c]);
+    const float r = bias[c] / bias_scales[c] + (float)bias_offsets[c];
+    double v = (double)nearbyintf(r);
+    if (v > 2147483647.0) v = 2147483647.0;
+    if (v < -2147483648.0) v = -2147483648.0;
+    bias_q[c] = (int32_t)v;
+  }
+  return MI355X_OK;
+}
+
 int mi355x_rowwise_quantize_i8_host(const float *in, size_t rows, size_t cols,
                                     int schema, int8_t *out, float *scales,
                                     int32_t *offsets) {

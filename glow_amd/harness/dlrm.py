@@ -14,6 +14,7 @@ import numpy as np
 from glow_amd import capi
 from glow_amd import host as H
 from glow_amd import workloads
+from glow_amd.harness import resnet50
 from glow_amd.harness.net import Net
 
 
@@ -108,11 +109,10 @@ def make(tables=26, rows=1_000_000, dim=64, batch=4096, mean_len=20, alpha=1.1,
         for i, (w, b) in enumerate(layers):
             n, k = w.shape
             q, ws, wo = capi.rowwise_quantize_i8_host(w, capi.SCHEMA_SYMMETRIC)
-            bscale = float(np.float32(cur_tq[0]) * np.float32(ws.mean()))
+            bq, bscale, boff = resnet50.quantize_fc_bias(b, w, cur_tq[0])
             name = f"{prefix}{i}"
             net.constant(name + "_w", q, H.INT8Q)
-            net.constant(name + "_b", np.clip(np.rint(b / np.float32(bscale)), -2 ** 31, 2 ** 31 - 1)
-                         .astype(np.int32), H.INT32Q, bscale, 0)
+            net.constant(name + "_b", bq, H.INT32Q, bscale, boff)
             net.constant(name + "_s", ws, H.FLOAT)
             net.constant(name + "_o", wo, H.INT32I)
             relu = last_relu or i + 1 < len(layers)

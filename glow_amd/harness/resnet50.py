@@ -3,9 +3,13 @@ the reference's tests/benchmark/ResNetBench.cpp:138-385 builds it), quantized
 from a profile the way Glow's profile-guided flow does: random He-normal fp32
 weights (BatchNorm folded away), min/max of every activation over synthetic
 N(0.45, 0.25) images, chooseQuantizationParams with the SymmetricWithUInt8
-schema for activations, channelwise symmetric int8 filters with int32 biases
-at scale inScale*filterScale, a RowwiseQuantizedFullyConnected classifier,
-Dequantize and an fp32 SoftMax.
+schema for activations; filters and biases of the convolutions through
+createChannelwiseQuantizedConv's own preparation (per-channel parameters,
+specializeBiasWeightsQuantizationParams, int32 biases at scale
+inScale*filterScale); a RowwiseQuantizedFullyConnected classifier whose bias
+is typed the way the quantizer types a FullyConnected bias; Dequantize and an
+fp32 SoftMax. (The optimizer's rescale folding does not apply: this graph is
+built without the Quantize/Dequantize pairs it removes.)
 
 The fp32 profiling pass runs in numpy on the host; everything that is timed
 runs on the GPU through the host layer."""
@@ -119,14 +123,28 @@ def _tqp(rng_):
                                            capi.QTY_INT8)
 
 
+SCHEMA = capi.SCHEMA_SYMMETRIC_WITH_UNSIGNED
+
+
 def _quantize_rows(w2d):
     q, scales, offsets = capi.rowwise_quantize_i8_host(w2d, capi.SCHEMA_SYMMETRIC)
     return q, scales, offsets
 
 
-def _quantize_bias(b, scales):
-    v = np.rint(b.astype(np.float32) / scales.astype(np.float32))
-    return np.clip(v, -2 ** 31, 2 ** 31 - 1).astype(np.int32)
+def quantize_fc_bias(bias, weights, in_scale):
+    """The int32 bias of a FullyConnected as Glow's quantizer types it before the
+    node becomes rowwise-quantized (reference lib/Quantization/Quantization.cpp:
+    103-113, 142-152): its own range as an Int32QTy tensor, specialised against
+    the input's scale and the scale of the WHOLE weight tensor
+    (specializeBiasQuantizationParams). Returns (int32 values, scale, offset)."""
+    w_scale, _ = capi.choose_quantization_params(float(weights.min()), float(weights.max()),
+                                                 SCHEMA, capi.QTY_INT8)
+    own_scale, own_off = capi.choose_quantization_params(float(bias.min()), float(bias.max()),
+                                                         SCHEMA, capi.QTY_INT32)
+    scale, off = capi.specialize_bias_qparams(own_scale, own_off, in_scale, w_scale,
+                                              bias_is_i32=True, bias_is_zero=not bias.any())
+    q = np.rint(bias.astype(np.float32) / np.float32(scale) + np.float32(off))
+    return np.clip(q, -2 ** 31, 2 ** 31 - 1).astype(np.int32), scale, off
 
 
 def build_int8(steps, ranges, batch, size):
@@ -147,14 +165,16 @@ def build_int8(steps, ranges, batch, size):
             oh = (h + 2 * prm.pad - prm.k) // prm.stride + 1
             ow = (w + 2 * prm.pad - prm.k) // prm.stride + 1
             shapes[out] = (n, oh, ow, oc)
-            q, fs, fo = _quantize_rows(prm.w.reshape(oc, -1))
-            bs = (np.float32(tq[ins[0]][0]) * fs).astype(np.float32)
-            net.constant(out + "_filter", q.reshape(prm.w.shape), H.INT8Q)
-            net.constant(out + "_bias", _quantize_bias(prm.b, bs), H.INT32Q)
+            # what Quantizer::enableChannelwise makes of a Convolution with
+            # constant fp32 filter and bias (createChannelwiseQuantizedConv)
+            q, bq, fs, fo, bs, bo = capi.channelwise_quantize_conv_host(
+                prm.w, prm.b, tq[ins[0]][0], SCHEMA)
+            net.constant(out + "_filter", q, H.INT8Q)
+            net.constant(out + "_bias", bq, H.INT32Q)
             net.constant(out + "_fscales", fs, H.FLOAT)
             net.constant(out + "_foffsets", fo, H.INT32I)
             net.constant(out + "_bscales", bs, H.FLOAT)
-            net.constant(out + "_boffsets", np.zeros(oc, np.int32), H.INT32I)
+            net.constant(out + "_boffsets", bo, H.INT32I)
             net.activation(out, shapes[out], H.INT8Q, *tq[out])
             net.op(H.CHANNELWISE_QUANTIZED_CONV, out,
                    [out, src, out + "_filter", out + "_bias", out + "_fscales", out + "_foffsets",
@@ -188,10 +208,9 @@ def build_int8(steps, ranges, batch, size):
             classes, k = fw.shape
             shapes[out] = (n, classes)
             q, ws, wo = _quantize_rows(fw)
-            bscale = float(np.float32(tq[ins[0]][0]) * np.float32(ws.mean()))
+            bq, bscale, boff = quantize_fc_bias(fb, fw, tq[ins[0]][0])
             net.constant("fc_weights", q, H.INT8Q)
-            net.constant("fc_bias", np.clip(np.rint(fb / np.float32(bscale)), -2 ** 31, 2 ** 31 - 1)
-                         .astype(np.int32), H.INT32Q, bscale, 0)
+            net.constant("fc_bias", bq, H.INT32Q, bscale, boff)
             net.constant("fc_scales", ws, H.FLOAT)
             net.constant("fc_offsets", wo, H.INT32I)
             # the pooled [N,1,1,C] tensor is read as [N,C]: same bytes

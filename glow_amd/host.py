@@ -33,6 +33,7 @@ EXPORTS = [
     "mi355x_host_dm_destroy", "mi355x_host_dm_init", "mi355x_host_dm_stop",
     "mi355x_host_dm_add_network", "mi355x_host_dm_evict_network", "mi355x_host_dm_run",
     "mi355x_host_dm_time_function", "mi355x_host_dm_maximum_memory", "mi355x_host_dm_available_memory",
+    "mi355x_host_dm_add_functions", "mi355x_host_dm_transfer_static_placeholder",
 ]
 
 
@@ -223,9 +224,22 @@ class DeviceManager:
         except Exception:
             pass
 
-    def add_network(self, module):
-        _check(lib().mi355x_host_dm_add_network(self._h, module._h))
+    def add_network(self, module, functions=None):
+        """functions: indices of the compiled functions to load (default: all)."""
+        if functions is None:
+            _check(lib().mi355x_host_dm_add_network(self._h, module._h))
+        else:
+            fs = (C.c_int * len(functions))(*[int(f) for f in functions])
+            _check(lib().mi355x_host_dm_add_functions(self._h, module._h, fs, len(functions)))
         self._modules.append(module)   # the device manager keeps pointers into it
+
+    def transfer_static_placeholder(self, module, name, array):
+        """transferStaticPlaceholderToDevice: host array -> the placeholder's
+        device slot; later requests that do not bind it read this value."""
+        assert array.flags["C_CONTIGUOUS"]
+        _check(lib().mi355x_host_dm_transfer_static_placeholder(
+            self._h, module._h, name.encode(), C.c_void_p(array.ctypes.data),
+            C.c_size_t(array.nbytes)))
 
     def evict_network(self, name):
         _check(lib().mi355x_host_dm_evict_network(self._h, name.encode()))

@@ -177,6 +177,43 @@ RunIdentifierTy MI355XDeviceManager::runFunction(std::string functionName,
   return id;
 }
 
+void MI355XDeviceManager::transferStaticPlaceholderToDevice(
+    const Module *module, std::string placeholderName, Tensor *tensor,
+    std::function<void(Error)> resultCB) {
+  {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (!running_ || stopping_) {
+      resultCB(MI355X_MAKE_ERR(ErrorCode::RUNTIME_REQUEST_REFUSED, "device manager is not running"));
+      return;
+    }
+  }
+  enqueue([this, module, placeholderName, tensor, resultCB] {
+    auto mit = modules_.find(module);
+    if (!module || mit == modules_.end() || !mit->second.arena || !tensor) {
+      resultCB(MI355X_MAKE_ERR(ErrorCode::RUNTIME_ERROR,
+                               "cannot copy placeholder %s: its module has no function on this device",
+                               placeholderName.c_str()));
+      return;
+    }
+    const int id = module->getValueByName(placeholderName);
+    if (id < 0 || module->value(id).category != SymbolCategory::Placeholder) {
+      resultCB(MI355X_MAKE_ERR(ErrorCode::RUNTIME_ERROR, "%s is not a placeholder of the module",
+                               placeholderName.c_str()));
+      return;
+    }
+    const Value &v = module->value(id);
+    if (tensor->sizeInBytes() > v.type.sizeInBytes()) {
+      resultCB(MI355X_MAKE_ERR(ErrorCode::RUNTIME_ERROR, "tensor for %s has %zu bytes, slot %zu",
+                               placeholderName.c_str(), tensor->sizeInBytes(), v.type.sizeInBytes()));
+      return;
+    }
+    int rc = mi355x_arena_upload(mit->second.arena, MI355X_REGION_MUTABLE, v.offset, tensor->data(),
+                                 tensor->sizeInBytes(), stream_);
+    if (rc == MI355X_OK) rc = mi355x_stream_sync(stream_);
+    resultCB(rc == MI355X_OK ? Error::success() : fromStatus(rc, "placeholder copy"));
+  });
+}
+
 Expected<float> MI355XDeviceManager::timeFunction(const std::string &functionName, int iterations) {
   {
     std::lock_guard<std::mutex> lk(mu_);

@@ -65,6 +65,16 @@ public:
   RunIdentifierTy runFunction(std::string functionName, std::unique_ptr<ExecutionContext> ctx,
                               ResultCBTy resultCB);
 
+  // DeviceManager::transferStaticPlaceholderToDevice (reference
+  // include/glow/Backends/DeviceManager.h:166-171): copies `tensor` into the
+  // device slot of the module's placeholder `placeholderName`. Requests that
+  // do not bind that placeholder afterwards run on the transferred value (a
+  // static placeholder: uploaded once, read by many requests). The module must
+  // have a function resident on this device; a tensor larger than the slot, an
+  // unknown name or a value that is no placeholder is a RUNTIME_ERROR.
+  void transferStaticPlaceholderToDevice(const Module *module, std::string placeholderName,
+                                         Tensor *tensor, std::function<void(Error)> resultCB);
+
   // Benchmark aid without a counterpart in the reference: replays a resident
   // function `iterations` times on the data its placeholders already hold (no
   // host copies) and reports the average device time per replay, measured

@@ -193,6 +193,37 @@ int mi355x_host_dm_add_network(mi355x_host_dm *dm, mi355x_host_module *m) {
   return e ? fail(e) : 0;
 }
 
+int mi355x_host_dm_add_functions(mi355x_host_dm *dm, mi355x_host_module *m, const int *functions,
+                                 int n) {
+  if (!dm || !m || n < 0 || (n > 0 && !functions))
+    return failMsg(ErrorCode::RUNTIME_ERROR, "NULL handle");
+  FunctionMapTy fm;
+  for (int i = 0; i < n; i++) {
+    auto it = m->compiled.find(functions[i]);
+    if (it == m->compiled.end())
+      return failMsg(ErrorCode::COMPILE_CONTEXT_MALFORMED, "function is not compiled");
+    fm[it->second->name()] = it->second.get();
+  }
+  std::promise<Error> p;
+  auto fut = p.get_future();
+  dm->dm.addNetwork(&m->module, fm, [&p](const Module *, Error e) { p.set_value(std::move(e)); });
+  Error e = fut.get();
+  return e ? fail(e) : 0;
+}
+
+int mi355x_host_dm_transfer_static_placeholder(mi355x_host_dm *dm, mi355x_host_module *m,
+                                               const char *name, void *buffer, size_t bytes) {
+  if (!dm || !m || !name || (!buffer && bytes))
+    return failMsg(ErrorCode::RUNTIME_ERROR, "NULL argument");
+  Tensor t = Tensor::unowned(Type(ElemKind::Int8QTy, {(int64_t)bytes}), buffer, bytes);
+  std::promise<Error> p;
+  auto fut = p.get_future();
+  dm->dm.transferStaticPlaceholderToDevice(&m->module, name, &t,
+                                           [&p](Error e) { p.set_value(std::move(e)); });
+  Error e = fut.get();
+  return e ? fail(e) : 0;
+}
+
 int mi355x_host_dm_evict_network(mi355x_host_dm *dm, const char *name) {
   if (!dm || !name) return failMsg(ErrorCode::RUNTIME_ERROR, "NULL handle");
   std::promise<Error> p;

@@ -169,6 +169,30 @@ int mi355x_specialize_bias_weights_qparams(float *bias_scale, int32_t *bias_offs
                                            float input_scale, float *weights_scale,
                                            int bias_is_i32, int bias_is_zero);
 
+/* quantization::specializeBiasQuantizationParams (reference
+ * lib/Quantization/Base/Base.cpp:567-592): what the quantizer applies to the
+ * bias of a Convolution or FullyConnected whose weights keep their scale
+ * (lib/Quantization/Quantization.cpp:103-113). In/out: bias_scale, bias_offset. */
+int mi355x_specialize_bias_qparams(float *bias_scale, int32_t *bias_offset, float input_scale,
+                                   float weights_scale, int bias_is_i32, int bias_is_zero);
+
+/* The constant preparation of Function::createChannelwiseQuantizedConv for a
+ * float filter and a float bias without given parameters, int8 filter and
+ * int32 bias (reference lib/Graph/Graph.cpp:3576-3700, what
+ * Quantizer::enableChannelwise triggers, lib/Quantization/Quantization.cpp:762-844):
+ * per output channel, filter parameters from the channel's range
+ * (getTensorQuantizationParams, Base.cpp:632-691), bias parameters from the
+ * channel's bias value as an Int32QTy range, both specialised by
+ * specializeBiasWeightsQuantizationParams (Base.cpp:594-629), then the filter
+ * and the bias quantized with them (quantizeTensor, Base.cpp:707-760).
+ * HOST buffers; filter is [channels x per_channel] row-major. */
+int mi355x_channelwise_quantize_conv_host(const float *filter, const float *bias,
+                                          size_t channels, size_t per_channel,
+                                          float input_scale, int schema, int8_t *filter_q,
+                                          int32_t *bias_q, float *filter_scales,
+                                          int32_t *filter_offsets, float *bias_scales,
+                                          int32_t *bias_offsets);
+
 /* Fused-rowwise element kinds (reference include/glow/Base/Type.h:424-433):
  * row = [data | scale | offset], scale/offset fp32 or fp16; 4-bit rows hold
  * two columns per byte, even column in the low nibble. */

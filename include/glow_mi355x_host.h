@@ -146,6 +146,16 @@ int mi355x_host_dm_init(mi355x_host_dm *dm);
 int mi355x_host_dm_stop(mi355x_host_dm *dm);
 /* addNetwork with every compiled function of the module; waits for the callback. */
 int mi355x_host_dm_add_network(mi355x_host_dm *dm, mi355x_host_module *m);
+/* addNetwork with a subset of the module's compiled functions (by function
+ * index): the reference's FunctionMapTy may hold any part of a module, and the
+ * rest may follow in a later call (DeviceManagerTest.cpp:573 "ReuseModule"). */
+int mi355x_host_dm_add_functions(mi355x_host_dm *dm, mi355x_host_module *m, const int *functions,
+                                 int n);
+/* DeviceManager::transferStaticPlaceholderToDevice (reference
+ * include/glow/Backends/DeviceManager.h:166-171): host bytes -> the device
+ * slot of the module's placeholder `name`; blocks until copied. */
+int mi355x_host_dm_transfer_static_placeholder(mi355x_host_dm *dm, mi355x_host_module *m,
+                                               const char *name, void *buffer, size_t bytes);
 int mi355x_host_dm_evict_network(mi355x_host_dm *dm, const char *function_name);
 /* runFunction; binds n host buffers to placeholders by name (inputs are read,
  * outputs written, `bytes[i]` may be smaller than the placeholder), waits for

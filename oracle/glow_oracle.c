@@ -7,6 +7,7 @@
  */
 #include "glow_oracle.h"
 
+#include <float.h>
 #include <math.h>
 #include <stdlib.h>
 #include <string.h>
@@ -239,6 +240,19 @@ void go_specialize_bias_weights_qparams(float *biasScale, int32_t *biasOffset,
   *weightsScale = ws;
 }
 
+/* Base.cpp:567-592 (specializeBiasQuantizationParams): the weights keep their
+ * scale; the bias takes inputScale * weightsScale unless that is smaller than
+ * the scale its own range asks for (and the bias is not all zero). */
+void go_specialize_bias_qparams(float *biasScale, int32_t *biasOffset, float inputScale,
+                                float weightsScale, int biasIsI32, int biasZero) {
+  int32_t off = *biasOffset;
+  if (biasIsI32) off = 0;
+  float bs = *biasScale;
+  if (inputScale * weightsScale >= bs || biasZero) bs = inputScale * weightsScale;
+  *biasScale = bs;
+  *biasOffset = off;
+}
+
 /* Base.h:323-329: clip<int64, DestTy>((int64)nearbyintf(x/scale + offset)) */
 static int64_t quantize_value_i64(float x, float scale, int32_t offset) {
   float r = x / scale + (float)offset;
@@ -275,6 +289,40 @@ void go_rowwise_quantize_i8(const float *in, size_t rows, size_t cols,
     scales[i] = s;
     offsets[i] = o;
   }
+}
+
+/* Graph.cpp:3576-3700 (createChannelwiseQuantizedConv with a float filter and a
+ * float bias, no parameters given, int8 filter / int32 bias), in the order of
+ * the reference: all filter parameters (getTensorQuantizationParams over
+ * dimension 0, Base.cpp:632-691), all bias parameters (each channel's bias is a
+ * one-element group, so min == max == bias[c]; Int32QTy), the specialisation
+ * loop (Base.cpp:594-629), then quantizeTensor of the filter and of the bias
+ * (Base.cpp:707-760 with quantize<T>, Base.h:323-329). */
+void go_channelwise_quantize_conv(const float *filter, const float *bias, size_t channels,
+                                  size_t perChannel, float inputScale, int schema,
+                                  int8_t *filterQ, int32_t *biasQ, float *filterScales,
+                                  int32_t *filterOffsets, float *biasScales,
+                                  int32_t *biasOffsets) {
+  for (size_t c = 0; c < channels; c++) {
+    float lo = FLT_MAX, hi = -FLT_MAX;
+    for (size_t j = 0; j < perChannel; j++) {
+      const float v = filter[c * perChannel + j];
+      if (v < lo) lo = v;
+      if (v > hi) hi = v;
+    }
+    go_choose_qparams(lo, hi, schema, 8, &filterScales[c], &filterOffsets[c]);
+  }
+  for (size_t c = 0; c < channels; c++)
+    go_choose_qparams(bias[c], bias[c], schema, 32, &biasScales[c], &biasOffsets[c]);
+  for (size_t c = 0; c < channels; c++)
+    go_specialize_bias_weights_qparams(&biasScales[c], &biasOffsets[c], inputScale,
+                                       &filterScales[c], 1, bias[c] == 0.f);
+  for (size_t c = 0; c < channels; c++)
+    for (size_t j = 0; j < perChannel; j++)
+      filterQ[c * perChannel + j] =
+          go_quantize_value_i8(filter[c * perChannel + j], filterScales[c], filterOffsets[c]);
+  for (size_t c = 0; c < channels; c++)
+    biasQ[c] = go_quantize_value_i32(bias[c], biasScales[c], biasOffsets[c]);
 }
 
 size_t go_fused_row_bytes(size_t cols, int kind) {

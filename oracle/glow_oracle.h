@@ -76,6 +76,20 @@ void go_choose_qparams(float min, float max, int schema, int qty,
 void go_specialize_bias_weights_qparams(float *biasScale, int32_t *biasOffset,
                                         float inputScale, float *weightsScale,
                                         int biasIsI32, int biasZero);
+/* Base.cpp:567-592 (specializeBiasQuantizationParams). Updates *biasScale,
+ * *biasOffset. */
+void go_specialize_bias_qparams(float *biasScale, int32_t *biasOffset, float inputScale,
+                                float weightsScale, int biasIsI32, int biasZero);
+/* Graph.cpp:3576-3700: constants of a ChannelwiseQuantizedConvolution from a
+ * float filter [channels x perChannel] and float bias. Pinned by the closed
+ * forms tests/test_oracle_kats.py states (bias scale == input scale * filter
+ * scale bit for bit; the filter scale gives way exactly when the bias would
+ * saturate; round trip within half a step). */
+void go_channelwise_quantize_conv(const float *filter, const float *bias, size_t channels,
+                                  size_t perChannel, float inputScale, int schema,
+                                  int8_t *filterQ, int32_t *biasQ, float *filterScales,
+                                  int32_t *filterOffsets, float *biasScales,
+                                  int32_t *biasOffsets);
 
 /* Base.h:323-329 quantize<int8_t> / quantize<int32_t> on one value. */
 int8_t go_quantize_value_i8(float x, float scale, int32_t offset);

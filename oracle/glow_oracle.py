@@ -153,6 +153,31 @@ def specialize_bias_weights_qparams(bias_scale, bias_offset, input_scale,
     return bs.value, bo.value, ws.value
 
 
+def specialize_bias_qparams(bias_scale, bias_offset, input_scale, weights_scale,
+                            bias_is_i32=True, bias_zero=False):
+    bs = C.c_float(bias_scale)
+    bo = C.c_int32(bias_offset)
+    lib().go_specialize_bias_qparams(C.byref(bs), C.byref(bo), C.c_float(input_scale),
+                                     C.c_float(weights_scale), C.c_int(bias_is_i32),
+                                     C.c_int(bias_zero))
+    return bs.value, bo.value
+
+
+def channelwise_quantize_conv(filter_f, bias_f, input_scale, schema=SYMMETRIC):
+    f = _c(filter_f, np.float32)
+    b = _c(bias_f, np.float32)
+    oc = f.shape[0]
+    per = f.size // max(oc, 1)
+    fq = np.empty(f.shape, np.int8)
+    bq = np.empty(oc, np.int32)
+    fs, bs = np.empty(oc, np.float32), np.empty(oc, np.float32)
+    fo, bo = np.empty(oc, np.int32), np.empty(oc, np.int32)
+    lib().go_channelwise_quantize_conv(_p(f), _p(b), C.c_size_t(oc), C.c_size_t(per),
+                                       C.c_float(input_scale), C.c_int(schema), _p(fq), _p(bq),
+                                       _p(fs), _p(fo), _p(bs), _p(bo))
+    return fq, bq, fs, fo, bs, bo
+
+
 def quantize_value_i8(x, scale, offset):
     return lib().go_quantize_value_i8(x, scale, offset)
 

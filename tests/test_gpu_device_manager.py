@@ -272,3 +272,90 @@ def test_other_lookup_forms(dm):
     np.testing.assert_array_equal(r1, go.rwq_slws_f32(data, scales, offs, w, idx, lengths))
     np.testing.assert_array_equal(
         r2, go.embedding_bag_byte_rowwise_offsets_f32(fused, w, idx, starts, True))
+
+
+def test_multi_module(dm):
+    """Two modules built the same way under different function names, both
+    resident, both run (reference DeviceManagerTest.cpp:488 MultiModule)."""
+    c = cases.rwq_fc_case(31, 8, 64, 32, symmetric=False)
+    m1, f1 = host_cases.rwq_fc_module(c, name="func1")
+    m2, f2 = host_cases.rwq_fc_module(c, name="func2")
+    m1.compile(f1)
+    m2.compile(f2)
+    dm.add_network(m1)
+    dm.add_network(m2)
+    rng = np.random.default_rng(3)
+    x1 = rng.integers(-128, 128, c["x"].shape).astype(np.int8)
+    x2 = rng.integers(-128, 128, c["x"].shape).astype(np.int8)
+    o1, o2 = np.zeros((8, 32), np.int8), np.zeros((8, 32), np.int8)
+    dm.run("func1", {"input": x1, "output": o1})
+    dm.run("func2", {"input": x2, "output": o2})
+    # each module has its own placeholders: the second run did not disturb the first
+    assert np.array_equal(o1, _rwq_expected(c, x1))
+    assert np.array_equal(o2, _rwq_expected(c, x2))
+
+
+def test_reuse_module(dm):
+    """The functions of ONE module added by two addNetwork calls; both see the
+    module's placeholders and constants (reference DeviceManagerTest.cpp:573
+    ReuseModule)."""
+    c = cases.rwq_fc_case(32, 8, 64, 32)
+    m, f = host_cases.rwq_fc_module(c, name="func1")
+    g = m.function("func2")
+    r = m.placeholder("func2_output", (8, 64), H.INT8Q, np.int8, 0.07, 2)
+    m.instruction(g, H.RESCALE_QUANTIZED, "r", [r, 0])      # value 0 is "input"
+    m.compile(f)
+    m.compile(g)
+    before = dm.available_memory
+    dm.add_network(m, functions=[f])
+    after_first = dm.available_memory
+    dm.add_network(m, functions=[g])
+    # the module's constants and placeholders were made resident once
+    assert before - after_first > after_first - dm.available_memory >= 0
+    out = np.zeros((8, 32), np.int8)
+    dm.run("func1", {"input": c["x"], "output": out})
+    assert np.array_equal(out, _rwq_expected(c))
+    res = np.zeros((8, 64), np.int8)
+    dm.run("func2", {"input": c["x"], "func2_output": res})
+    pre, post, scale, _ = go.quantize_scale_offset_32to8(
+        float(np.float32(c["in_scale_f"]) / np.float32(0.07)), 0)
+    assert np.array_equal(res, go.rescale_i8(c["x"], 2, c["in_offset"], pre, post, scale))
+    # the same name cannot be added twice
+    with pytest.raises(H.HostError):
+        dm.add_network(m, functions=[g])
+    dm.evict_network("func1")
+    res[:] = 0
+    dm.run("func2", {"input": c["x"], "func2_output": res})
+    assert np.array_equal(res, go.rescale_i8(c["x"], 2, c["in_offset"], pre, post, scale))
+    dm.evict_network("func2")
+    assert dm.available_memory == before
+
+
+def test_transfer_static_placeholder(dm):
+    """transferStaticPlaceholderToDevice (reference DeviceManagerTest.cpp:239):
+    a placeholder filled once on the device serves later requests that do not
+    bind it."""
+    c = cases.rwq_fc_case(33, 8, 64, 32, symmetric=False)
+    m, f = host_cases.rwq_fc_module(c)
+    m.compile(f)
+    dm.add_network(m)
+    rng = np.random.default_rng(5)
+    static_x = rng.integers(-128, 128, c["x"].shape).astype(np.int8)
+    dm.transfer_static_placeholder(m, "input", static_x)
+    for _ in range(2):
+        out = np.zeros((8, 32), np.int8)
+        dm.run("main", {"output": out})            # "input" is not bound
+        assert np.array_equal(out, _rwq_expected(c, static_x))
+    # a bound tensor still replaces it for that and later requests
+    out = np.zeros((8, 32), np.int8)
+    dm.run("main", {"input": c["x"], "output": out})
+    assert np.array_equal(out, _rwq_expected(c))
+    with pytest.raises(H.HostError):
+        dm.transfer_static_placeholder(m, "weights", static_x)       # a constant
+    with pytest.raises(H.HostError):
+        dm.transfer_static_placeholder(m, "nothing", static_x)
+    with pytest.raises(H.HostError):
+        dm.transfer_static_placeholder(m, "input", np.zeros(10_000, np.int8))   # too large
+    other, f2 = host_cases.rwq_fc_module(c, name="elsewhere")
+    with pytest.raises(H.HostError):
+        dm.transfer_static_placeholder(other, "input", static_x)    # module not resident

@@ -132,3 +132,28 @@ def test_specialize_bias_weights_qparams_equals_oracle():
             for zero in (False, True):
                 assert capi.specialize_bias_weights_qparams(bs, bo, ins, ws, i32, zero) == \
                     go.specialize_bias_weights_qparams(bs, bo, ins, ws, i32, zero)
+
+
+def test_channelwise_conv_constants_equal_the_oracle():
+    """mi355x_channelwise_quantize_conv_host and mi355x_specialize_bias_qparams
+    against the oracle's restatement of Graph.cpp:3576-3700 / Base.cpp:567-592."""
+    from glow_amd import capi
+    rng = np.random.default_rng(21)
+    for trial in range(30):
+        oc, per = int(rng.integers(1, 40)), int(rng.integers(1, 200))
+        filt = (rng.standard_normal((oc, per)) * rng.uniform(1e-3, 5.0, (oc, 1))).astype(np.float32)
+        bias = (rng.standard_normal(oc) * 10.0 ** rng.uniform(-3, 7, oc)).astype(np.float32)
+        bias[rng.random(oc) < 0.2] = 0.0
+        in_scale = float(np.float32(10.0 ** rng.uniform(-3, 0)))
+        for schema in (go.SYMMETRIC, go.ASYMMETRIC, go.SYMMETRIC_WITH_UNSIGNED):
+            got = capi.channelwise_quantize_conv_host(filt, bias, in_scale, schema)
+            want = go.channelwise_quantize_conv(filt, bias, in_scale, schema)
+            for g, w in zip(got, want):
+                np.testing.assert_array_equal(g, w)
+    for _ in range(2000):
+        a = [float(np.float32(10.0 ** rng.uniform(-8, 2))) for _ in range(3)]
+        off = int(rng.integers(-100, 100))
+        for i32 in (True, False):
+            for zero in (True, False):
+                assert capi.specialize_bias_qparams(a[0], off, a[1], a[2], i32, zero) == \
+                    go.specialize_bias_qparams(a[0], off, a[1], a[2], i32, zero)

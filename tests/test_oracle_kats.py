@@ -574,3 +574,61 @@ def test_embedding_bag_offsets_equals_lengths_form():
     np.testing.assert_array_equal(a, b)
     c = go.embedding_bag_byte_rowwise_offsets_f32(f, w, idx, offs[:-1], False)
     np.testing.assert_array_equal(a, c)
+
+
+# ---- bias specialisation and channelwise convolution constants --------------------
+# Base.cpp:567-629, Graph.cpp:3576-3700. The reference's tests hold no exact
+# vectors for these (its operator tests compare against fp32 within a
+# tolerance), so the restatement is pinned by what the algorithm fixes.
+
+def test_specialize_bias_closed_forms():
+    f = np.float32
+    # the accumulator's scale is at least the bias's own: the bias takes it
+    bs, bo = go.specialize_bias_qparams(1e-6, 7, 0.05, 0.01)
+    assert f(bs) == f(0.05) * f(0.01) and bo == 0
+    # the bias's own scale is larger: it is kept, the weights are untouched
+    bs, bo = go.specialize_bias_qparams(1e-2, 7, 0.05, 0.01)
+    assert f(bs) == f(1e-2) and bo == 0
+    # ... unless the bias is all zero
+    bs, bo = go.specialize_bias_qparams(1e-2, 7, 0.05, 0.01, bias_zero=True)
+    assert f(bs) == f(0.05) * f(0.01)
+    # an int8 bias keeps its offset
+    assert go.specialize_bias_qparams(1e-6, 7, 0.05, 0.01, bias_is_i32=False)[1] == 7
+    # bias-and-weights variant: the weights scale gives way, and the product is
+    # re-formed so that it equals the bias scale bit for bit
+    bs, bo, ws = go.specialize_bias_weights_qparams(1e-2, 3, 0.05, 0.01)
+    assert f(ws) == f(1e-2) / f(0.05) and f(bs) == f(0.05) * f(ws) and bo == 0
+    bs, bo, ws = go.specialize_bias_weights_qparams(1e-6, 3, 0.05, 0.01)
+    assert f(ws) == f(0.01) and f(bs) == f(0.05) * f(0.01)
+
+
+def test_channelwise_conv_constants_invariants():
+    rng = np.random.default_rng(12)
+    oc, per = 24, 3 * 3 * 16
+    filt = (rng.standard_normal((oc, per)) * rng.uniform(0.01, 2.0, (oc, 1))).astype(np.float32)
+    bias = (rng.standard_normal(oc) * 0.1).astype(np.float32)
+    bias[3] = 0.0
+    bias[5] = 3.0e6        # so large that inScale * filterScale would saturate int32
+    in_scale = np.float32(0.02)
+    fq, bq, fs, fo, bs, bo = go.channelwise_quantize_conv(filt, bias, in_scale, go.SYMMETRIC)
+    assert not fo.any() and not bo.any()                 # symmetric filter, int32 bias
+    # the defining property (asserted by the reference itself): bit-exact product
+    np.testing.assert_array_equal(bs, in_scale * fs)
+    for c in range(oc):
+        own_scale, own_off = go.choose_qparams(float(filt[c].min()), float(filt[c].max()),
+                                               go.SYMMETRIC, 8)
+        bias_own, _ = go.choose_qparams(float(bias[c]), float(bias[c]), go.SYMMETRIC, 32)
+        if c == 5:
+            # the filter scale gave way to keep the bias inside int32
+            assert fs[c] > np.float32(own_scale) and fs[c] == np.float32(bias_own) / in_scale
+        else:
+            assert fs[c] == np.float32(own_scale)
+        # each value is quantized by x / scale, round-half-even, clipped
+        want = np.clip(np.rint(filt[c] / fs[c] + np.float32(fo[c])), -128, 127)
+        np.testing.assert_array_equal(fq[c], want.astype(np.int8))
+        wb = np.clip(np.rint(np.float64(np.float32(bias[c]) / bs[c])), -2 ** 31, 2 ** 31 - 1)
+        assert bq[c] == int(wb)
+        # round trip: within half a step where nothing was clipped
+        assert np.abs(fq[c].astype(np.float32) * fs[c] - filt[c]).max() <= fs[c] * 0.5001
+    # (the Int32QTy range the parameters are chosen for is 30 bits wide)
+    assert bq[3] == 0 and abs(int(bq[5])) >= 2 ** 29 - 1
