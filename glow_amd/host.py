@@ -15,7 +15,7 @@ _LIB = None
 (QUANTIZE, DEQUANTIZE, RESCALE_QUANTIZED, FULLY_CONNECTED, ROWWISE_QUANTIZED_FC,
  MATMUL, CONVOLUTION, CHANNELWISE_QUANTIZED_CONV, FRWQ_SLWS, FRWQ_SLS, ELEMENT_ADD,
  RELU, MAX_POOL, AVG_POOL, SOFTMAX, CONVERT_TO, INSERT_TENSOR, TRANSPOSE, GATHER,
- BATCH_MATMUL, SIGMOID, RWQ_SLWS, EMBEDDING_BAG_BYTE_ROWWISE_OFFSETS) = range(23)
+ BATCH_MATMUL, SIGMOID, RWQ_SLWS, EMBEDDING_BAG_BYTE_ROWWISE_OFFSETS, COPY) = range(24)
 ACT_NONE, ACT_RELU, ACT_CLIP, ACT_TANH, ACT_SIGMOID, ACT_LEAKY_RELU = range(6)
 
 ERROR_NAMES = ["SUCCESS", "UNKNOWN", "RUNTIME_ERROR", "RUNTIME_OUT_OF_DEVICE_MEMORY",

@@ -154,6 +154,7 @@ public:
       case Kind::ConvertTo:
       case Kind::InsertTensor:
       case Kind::BatchMatMul:
+      case Kind::Copy:
       case Kind::Sigmoid: MI355X_RETURN_IF_ERR(movement(I, out)); break;
       case Kind::Gather: {
         // a result that is only inserted into a wider tensor is gathered there
@@ -260,7 +261,7 @@ public:
 
 private:
   static constexpr int kArity[(int)Kind::NumKinds] = {2, 2, 2, 4, 6, 3, 4, 8, 5, 4, 3, 2, 2, 2, 2,
-                                                       2, 2, 2, 3, 3, 2, 7, 5};
+                                                       2, 2, 2, 3, 3, 2, 7, 5, 2};
 
   Error checkOperands(const Instruction &I) {
     CHECK_OP((int)I.kind >= 0 && (int)I.kind < (int)Kind::NumKinds, "unknown kind");
@@ -525,6 +526,19 @@ private:
       out.launches.push_back({"mi355x_convert_f16_to_f32", I.name, strFormat(" n=%zu", n),
                               [=](const DeviceBindings &b) {
                                 return mi355x_convert_f16_to_f32((float *)d.ptr(b), s.ptr(b), n, b.stream);
+                              }});
+      return Error::success();
+    }
+    case Kind::Copy: {
+      // libjit_copy_buffer / CopyInst: the bytes of Src into Dest
+      CHECK_OP(d.ty().kind == s.ty().kind && d.ty().sizeInBytes() == s.ty().sizeInBytes(),
+               "needs two tensors of one element kind and size");
+      CHECK_OP(!isQuantized(d.ty().kind) || (d.ty().scale == s.ty().scale && d.ty().offset == s.ty().offset),
+               "source and destination must share scale and offset");
+      const size_t n = d.ty().sizeInBytes();
+      out.launches.push_back({"mi355x_copy_u8", I.name, strFormat(" bytes=%zu", n),
+                              [=](const DeviceBindings &b) {
+                                return mi355x_copy_u8(d.ptr(b), s.ptr(b), n, b.stream);
                               }});
       return Error::success();
     }

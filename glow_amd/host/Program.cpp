@@ -100,6 +100,7 @@ const char *kindName(Kind k) {
   case Kind::Sigmoid: return "Sigmoid";
   case Kind::RowwiseQuantizedSparseLengthsWeightedSum: return "RowwiseQuantizedSparseLengthsWeightedSum";
   case Kind::EmbeddingBagByteRowwiseOffsets: return "EmbeddingBagByteRowwiseOffsets";
+  case Kind::Copy: return "Copy";
   default: return "?";
   }
 }

@@ -59,6 +59,7 @@ enum class Kind : int32_t {
   Sigmoid,                      // (Dest, Src) float
   RowwiseQuantizedSparseLengthsWeightedSum, // (Dest, Data u8 [rows,cols], Scales, Offsets, Weights, Indices, Lengths)
   EmbeddingBagByteRowwiseOffsets, // (Dest, Data, Weights, Indices, Offsets); iattrs {hasEndOffset}
+  Copy,                         // (Dest, Src): same bytes (what Save and Reshape lower to)
   NumKinds
 };
 const char *kindName(Kind k);

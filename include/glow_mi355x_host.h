@@ -75,7 +75,8 @@ enum {
   MI355X_HOST_BATCH_MATMUL = 19,       /* Dest [B,M,N], LHS [B,M,K], RHS [B,K,N] int8 */
   MI355X_HOST_SIGMOID = 20,            /* Dest, Src float */
   MI355X_HOST_RWQ_SLWS = 21,           /* Dest, Data u8, Scales, Offsets, Weights, Indices, Lengths */
-  MI355X_HOST_EMBEDDING_BAG_BYTE_ROWWISE_OFFSETS = 22 /* Dest, Data, Weights, Indices, Offsets; iattrs {hasEndOffset} */
+  MI355X_HOST_EMBEDDING_BAG_BYTE_ROWWISE_OFFSETS = 22, /* Dest, Data, Weights, Indices, Offsets; iattrs {hasEndOffset} */
+  MI355X_HOST_COPY = 23                /* Dest, Src: same bytes (CopyInst) */
 };
 /* Convolution iattrs: kernelH, kernelW, strideH, strideW, padT, padL, padB,
  * padR, group, dilationH, dilationW, fusedActivation (glow::FusedActivation);

@@ -117,6 +117,8 @@ def run(net, inputs):
                                      fp16_accum=bool(o.iattrs and o.iattrs[0]))
         elif o.kind == H.CONVERT_TO:
             r = a[1].astype(np.float32)
+        elif o.kind == H.COPY:
+            r = np.ascontiguousarray(a[1]).reshape(d.shape)
         elif o.kind == H.SIGMOID:
             r = go.sigmoid_f32(a[1])
         elif o.kind == H.INSERT_TENSOR:

@@ -359,3 +359,25 @@ def test_transfer_static_placeholder(dm):
     other, f2 = host_cases.rwq_fc_module(c, name="elsewhere")
     with pytest.raises(H.HostError):
         dm.transfer_static_placeholder(other, "input", static_x)    # module not resident
+
+
+def test_copy_into_an_output_placeholder(dm):
+    """RWQ-FC into an activation, then a Copy into the output placeholder (the
+    shape a Save node takes when the optimizer cannot write in place)."""
+    c = cases.rwq_fc_case(34, 8, 64, 32)
+    m = H.Module("copied")
+    x = m.placeholder("input", (8, 64), H.INT8Q, np.int8, c["in_scale_f"], c["in_offset"])
+    out = m.placeholder("output", (256,), H.INT8Q, np.int8, c["out_scale_f"], c["out_offset"])
+    w = m.constant("weights", c["w"], H.INT8Q)
+    b = m.constant("bias", c["bias"], H.INT32Q, c["bias_scale_f"], c["bias_offset"])
+    sc = m.constant("scales", c["w_scales"].astype(np.float32))
+    of = m.constant("offsets", c["w_offsets"].astype(np.int32), H.INT32I)
+    f = m.function("main")
+    y = m.activation(f, "y", (8, 32), H.INT8Q, c["out_scale_f"], c["out_offset"])
+    m.instruction(f, H.ROWWISE_QUANTIZED_FC, "fc", [y, x, w, b, sc, of])
+    m.instruction(f, H.COPY, "save", [out, y])
+    m.compile(f)
+    dm.add_network(m)
+    got = np.zeros(256, np.int8)
+    dm.run("main", {"input": c["x"], "output": got})
+    assert np.array_equal(got.reshape(8, 32), _rwq_expected(c))

@@ -383,3 +383,21 @@ def test_per_row_and_per_channel_shifts_are_checked_at_compile_time():
     with pytest.raises(H.HostError) as e:
         m.compile(f)
     assert "channel 5" in str(e.value)
+
+
+def test_copy_instruction():
+    """CopyInst (what Save and Reshape lower to): one device copy of the bytes;
+    element kinds, sizes and quantization parameters must agree."""
+    m = H.Module("copy")
+    a = m.placeholder("a", (4, 48), H.INT8Q, np.int8, 0.1, 3)
+    b = m.placeholder("b", (192,), H.INT8Q, np.int8, 0.1, 3)
+    c = m.placeholder("c", (192,), H.INT8Q, np.int8, 0.2, 3)
+    f = m.function("main")
+    m.instruction(f, H.COPY, "save", [b, a])
+    m.compile(f)
+    r = _launch(m, f, "mi355x_copy_u8")
+    assert r["bytes"] == 192 and r["inst"] == "save"
+    g = m.function("bad")
+    m.instruction(g, H.COPY, "rescaling_copy", [c, a])
+    with pytest.raises(H.HostError):
+        m.compile(g)
