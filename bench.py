@@ -72,7 +72,9 @@ def parse():
     ap.add_argument("--only", default="",
                     help="run a single extra kernel (profiling aid): "
                          "slws|slws_warm|slws_strict|fc_large|fc_large_zero|fc_c1|fc_m16384|fc_mid|"
-                         "conv_c3|quantize|dequantize|rescale|copy|resnet50|dlrm")
+                         "fc|conv_c3|quantize|dequantize|rescale|copy|resnet50|dlrm")
+    ap.add_argument("--shape", default="",
+                    help="MxKxN of --only fc (a RowwiseQuantizedFullyConnected of that shape)")
     ap.add_argument("--tile", type=int, default=-1,
                     help="force a workgroup tile for the matrix-core legs of --only "
                          "(0..5, see mi355x_gemm_tile_override; default: chosen from the shape)")
@@ -691,14 +693,17 @@ def main():
     if args.tile >= 0:
         capi.check(capi.lib().mi355x_gemm_tile_override(args.tile))
 
-    if only and only not in ("slws", "slws_warm", "slws_strict", "fc_large", "fc_large_zero",
+    if only and only not in ("slws", "slws_warm", "slws_strict", "fc", "fc_large", "fc_large_zero",
                              "fc_c1", "fc_m16384", "fc_mid", "conv_c3", "quantize", "dequantize",
                              "rescale", "copy"):
         print(f"unknown --only {only}", file=sys.stderr)
         sys.exit(2)
-    if only in ("fc_large", "fc_large_zero", "fc_c1", "fc_m16384", "fc_mid", "conv_c3", "quantize",
+    if only in ("fc", "fc_large", "fc_large_zero", "fc_c1", "fc_m16384", "fc_mid", "conv_c3", "quantize",
                 "dequantize", "rescale", "copy"):
-        if only == "fc_large":
+        if only == "fc":
+            M, K, N = (int(v) for v in args.shape.split("x"))
+            r = bench_fc(capi, cases, M, K, N, args.steps, args.warmup)
+        elif only == "fc_large":
             r = bench_fc(capi, cases, 8192, 4096, 4096, args.steps, args.warmup)
         elif only == "fc_large_zero":
             r = bench_fc(capi, cases, 8192, 4096, 4096, args.steps, args.warmup, zero_leg=True,

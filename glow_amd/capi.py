@@ -47,6 +47,7 @@ EXPORTS = [
     "mi355x_slws_reserve_stream", "mi355x_frwq_slws_noalloc",
     "mi355x_shader_clock_probe", "mi355x_wall_clock_khz",
     "mi355x_specialize_bias_qparams", "mi355x_channelwise_quantize_conv_host",
+    "mi355x_gemm_requant_hint", "mi355x_gemm_requant_hint_host",
 ]
 
 
@@ -424,6 +425,43 @@ def channelwise_quantize_conv_host(filter_f, bias_f, input_scale, schema=SCHEMA_
         _vp(f), _vp(b), _sz(oc), _sz(per), C.c_float(input_scale), C.c_int(schema),
         _vp(fq), _vp(bq), _vp(fs), _vp(fo), _vp(bs), _vp(bo)))
     return fq, bq, fs, fo, bs, bo
+
+
+def gemm_requant_hint_host(K, in_offset, out_offset, w_offsets, bias, bias_offset, bias_pre,
+                           bias_post, bias_scale, out_pre, out_post, out_scale,
+                           bias_offsets=None):
+    """Requantisation hint flags for a launch with these (host) parameter
+    vectors; `bias_offset` scalar or `bias_offsets` per column."""
+    N = len(out_pre)
+    i32 = lambda v: None if v is None else np.ascontiguousarray(v, np.int32)
+    vs = [i32(v) for v in (w_offsets, bias_offsets, bias_pre, bias_post, bias_scale,
+                           out_pre, out_post, out_scale)]
+    b8 = 0
+    if bias is not None:
+        bias = np.ascontiguousarray(bias)
+        b8 = int(bias.dtype == np.int8)
+        if not b8:
+            bias = bias.astype(np.int32)
+    flags = C.c_int(0)
+    check(lib().mi355x_gemm_requant_hint_host(
+        _sz(K), _sz(N), _i32(in_offset), _i32(out_offset), _vp(vs[0]), _vp(bias), C.c_int(b8),
+        _vp(vs[1]), _i32(bias_offset), _vp(vs[2]), _vp(vs[3]), _vp(vs[4]), _vp(vs[5]),
+        _vp(vs[6]), _vp(vs[7]), C.byref(flags)))
+    return flags.value
+
+
+class requant_hint:
+    """with requant_hint(flags): ... applies the hint to the launches inside."""
+
+    def __init__(self, flags):
+        self.flags = int(flags)
+
+    def __enter__(self):
+        check(lib().mi355x_gemm_requant_hint(self.flags))
+
+    def __exit__(self, *exc):
+        check(lib().mi355x_gemm_requant_hint(0))
+        return False
 
 
 def fused_row_bytes(cols, kind):

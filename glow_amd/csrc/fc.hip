@@ -9,6 +9,7 @@
 namespace mi355x {
 
 thread_local int g_tile_override = -1;
+thread_local int g_requant_hint = 0;
 
 // dst [cols x rows] = src [rows x cols]^T through a 64x64 LDS tile.
 __global__ __launch_bounds__(256) void transpose2d_i8_kernel(
@@ -89,6 +90,13 @@ extern "C" {
 int mi355x_gemm_tile_override(int tile) {
   MI355X_REQUIRE(tile >= -1 && tile <= 5, "tile %d outside [-1, 5]", tile);
   g_tile_override = tile;
+  return MI355X_OK;
+}
+
+int mi355x_gemm_requant_hint(int flags) {
+  MI355X_REQUIRE(flags >= 0 && flags <= 3 && flags != 2,
+                 "hint %d: bit 1 (no pre-shifts) needs bit 0 (24-bit operands)", flags);
+  g_requant_hint = flags;
   return MI355X_OK;
 }
 

@@ -177,6 +177,12 @@ struct Epilogue {
   int32_t out_off;
   int32_t act, a0, a1, a2;
   FusedAdd add;         // add.res == NULL: none
+  // Requantisation hints from the caller (mi355x_gemm_requant_hint):
+  // bit 0: every value this launch can form in front of the output multiply
+  //        fits 24 bits after its column's pre-shift, every output scale fits
+  //        24 bits, and product + rounding term + (out_off << post) stays
+  //        inside 32 bits; bit 1: every output pre-shift is zero.
+  int32_t fast;
 };
 
 // Row-major [rows x K] operand (activations, or weights with K contiguous).
@@ -303,7 +309,7 @@ __device__ __forceinline__ void load_col_raw(ColRaw (&c)[TN], const Epilogue &ep
 // column l % 32 and, in register r, row 8*(r/4) + 4*(l/32) + r%4 of the tile.
 // Must be entered after a block barrier (LDS is reused).
 template <int BM, int BN, int WM, int WN, bool NEED_SA, bool NEED_SB,
-          bool LEAKY>
+          bool LEAKY, int FAST = 0>
 __device__ __forceinline__ void gemm_epilogue_impl(
     v16i (&acc)[WM / 32][WN / 32], int (&sa)[WM / 32], int (&sb)[WN / 32],
     int8_t *lds, const Epilogue &ep, int M, int N, int K, int m0, int n0,
@@ -360,14 +366,37 @@ __device__ __forceinline__ void gemm_epilogue_impl(
     if (ep.bias)
       colc += (uint32_t)scale_i32((int32_t)((uint32_t)col[j].bias - (uint32_t)col[j].boff),
                                   col[j].bpre, col[j].bpost, col[j].bscale, 0);
+    // FAST: the caller vouches for 24-bit operands and for room for the
+    // output offset below the post-shift, so that
+    //   ((x * s + rtn) >> post) + off == (x * s + (rtn + (off << post))) >> post
+    // with a 24-bit multiply-add; with no pre-shift anywhere the column
+    // constant goes through the multiply once per column as well. Same bits as
+    // scale_i32 in half (a third) of the instruction slots: the 32-bit multiply
+    // alone takes four.
+    uint32_t fold = 0;
+    if constexpr (FAST != 0) {
+      fold = (opost > 0 ? (1u << (opost - 1)) : 0u) + ((uint32_t)ep.out_off << opost);
+      if constexpr (FAST == 2) fold += colc * (uint32_t)oscale;
+    }
 #pragma unroll
     for (int i = 0; i < TM; i++) {
 #pragma unroll
       for (int r = 0; r < 16; r++) {
         const int ml = wm * WM + i * 32 + (r >> 2) * 8 + lhi * 4 + (r & 3);
-        uint32_t v = (uint32_t)acc[i][j][r] + colc;
-        if constexpr (NEED_SA) v -= (uint32_t)woff * (uint32_t)s_sumA[ml];
-        int32_t y = scale_i32((int32_t)v, opre, opost, oscale, ep.out_off);
+        int32_t y;
+        if constexpr (FAST == 2) {
+          uint32_t x = (uint32_t)acc[i][j][r];
+          if constexpr (NEED_SA) x -= (uint32_t)woff * (uint32_t)s_sumA[ml];
+          y = (int32_t)((uint32_t)__mul24((int32_t)x, oscale) + fold) >> opost;
+        } else if constexpr (FAST == 1) {
+          uint32_t x = (uint32_t)acc[i][j][r] + colc;
+          if constexpr (NEED_SA) x -= (uint32_t)woff * (uint32_t)s_sumA[ml];
+          y = (int32_t)((uint32_t)__mul24((int32_t)x >> opre, oscale) + fold) >> opost;
+        } else {
+          uint32_t v = (uint32_t)acc[i][j][r] + colc;
+          if constexpr (NEED_SA) v -= (uint32_t)woff * (uint32_t)s_sumA[ml];
+          y = scale_i32((int32_t)v, opre, opost, oscale, ep.out_off);
+        }
         if constexpr (LEAKY) {
           if (y < ep.out_off)
             y = scale_i32((int32_t)((uint32_t)y - (uint32_t)ep.out_off), ep.a0,
@@ -443,6 +472,12 @@ __device__ __forceinline__ void gemm_epilogue(
     int n_base, const ColRaw (&col)[WN / 32]) {
   if (ep.act == 5) // LEAKY_RELU: rare, kept out of the common instruction stream
     gemm_epilogue_impl<BM, BN, WM, WN, NEED_SA, NEED_SB, true>(
+        acc, sa, sb, lds, ep, M, N, K, m0, n0, n_base, col);
+  else if ((ep.fast & 3) == 3)
+    gemm_epilogue_impl<BM, BN, WM, WN, NEED_SA, NEED_SB, false, 2>(
+        acc, sa, sb, lds, ep, M, N, K, m0, n0, n_base, col);
+  else if (ep.fast & 1)
+    gemm_epilogue_impl<BM, BN, WM, WN, NEED_SA, NEED_SB, false, 1>(
         acc, sa, sb, lds, ep, M, N, K, m0, n0, n_base, col);
   else
     gemm_epilogue_impl<BM, BN, WM, WN, NEED_SA, NEED_SB, false>(
@@ -998,6 +1033,8 @@ enum class Tile { T256, T128, T128x64, T64, T256x128, T128x256 };
 // Tuning aid: a value in [0, 5] forces that tile for the following launches of
 // the calling thread.
 extern thread_local int g_tile_override;
+// Requantisation hints for the following launches of the calling thread.
+extern thread_local int g_requant_hint;
 static Tile pick_tile(const GemmShape &g, size_t lds_256) {
   auto tiles = [&](int bm, int bn) {
     return (long long)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * g.groups;
@@ -1066,11 +1103,13 @@ static int gemm_staged_tiles(const ARows &A, const DenseRows &B,
 // ep.sum_b). aligned: both operands allow 16-byte chunk
 // loads (16-byte aligned rows; for convolutions also IC/group % 16 == 0).
 template <class ARows>
-static int gemm_dispatch(const ARows &A, const DenseRows &B, const Epilogue &ep,
+static int gemm_dispatch(const ARows &A, const DenseRows &B, const Epilogue &ep_in,
                          int M, int N, int K, int groups,
                          long long b_group_stride, bool need_sa, bool need_sb,
                          bool aligned, hipStream_t st) {
   const GemmShape g{M, N, K, groups, b_group_stride};
+  Epilogue ep = ep_in;
+  ep.fast = g_requant_hint & 3;
   if (aligned && K >= kBK && K % kBK == 0) {
     if (need_sa && need_sb) return gemm_dma_tiles<true, true>(A, B, ep, g, st);
     if (need_sa) return gemm_dma_tiles<true, false>(A, B, ep, g, st);

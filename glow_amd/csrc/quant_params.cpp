@@ -273,6 +273,56 @@ int mi355x_channelwise_quantize_conv_host(const float *filter, const float *bias
   return MI355X_OK;
 }
 
+int mi355x_gemm_requant_hint_host(size_t K, size_t N, int32_t in_offset, int32_t out_offset,
+                                  const int32_t *w_offsets, const void *bias, int bias_is_i8,
+                                  const int32_t *bias_offsets, int32_t bias_offset,
+                                  const int32_t *bias_pre, const int32_t *bias_post,
+                                  const int32_t *bias_scale, const int32_t *out_pre,
+                                  const int32_t *out_post, const int32_t *out_scale,
+                                  int *flags) {
+  MI355X_REQUIRE(flags, "flags is NULL");
+  *flags = 0;
+  MI355X_REQUIRE(out_pre && out_post && out_scale, "NULL output parameter vector");
+  MI355X_REQUIRE(!bias || (bias_pre && bias_post && bias_scale), "NULL bias parameter vector");
+  if (N == 0) return MI355X_OK;
+  const int64_t k = (int64_t)K;
+  const int64_t aoff = in_offset < 0 ? -(int64_t)in_offset : in_offset;
+  const int64_t ooff = out_offset < 0 ? -(int64_t)out_offset : out_offset;
+  bool ok = true, no_pre = true;
+  for (size_t n = 0; n < N && ok; n++) {
+    const int32_t pre = out_pre[n], post = out_post[n];
+    if (pre < 0 || pre > 31 || post < 0 || post > 31) return MI355X_OK; // no hint for such a launch
+    int64_t woff = w_offsets ? w_offsets[n] : 0;
+    if (woff < 0) woff = -woff;
+    int64_t scaled_bias = 0;
+    if (bias) {
+      const int32_t b = bias_is_i8 ? (int32_t) reinterpret_cast<const int8_t *>(bias)[n]
+                                   : reinterpret_cast<const int32_t *>(bias)[n];
+      const int32_t bo = bias_offsets ? bias_offsets[n] : bias_offset;
+      const int32_t bp = bias_pre[n], bq = bias_post[n];
+      if (bp < 0 || bp > 31 || bq < 0 || bq > 31) return MI355X_OK;
+      // libjit_scale with 32-bit wrap-around, as the kernel computes it
+      const uint32_t in = (uint32_t)b - (uint32_t)bo;
+      const uint32_t rtn = bq > 0 ? (1u << (bq - 1)) : 0u;
+      const uint32_t m = (uint32_t)((int32_t)in >> bp) * (uint32_t)bias_scale[n] + rtn;
+      scaled_bias = (int64_t)((int32_t)m >> bq);
+      if (scaled_bias < 0) scaled_bias = -scaled_bias;
+    }
+    // the largest magnitude the kernel can meet in front of the output multiply:
+    // sum A*B over raw bytes, the two row-sum corrections, the column constant
+    const int64_t bound = k * 128 * 128 + woff * k * 128 + k * aoff * woff + aoff * k * 128 +
+                          scaled_bias;
+    const int64_t x = (bound >> pre) + 1;
+    int64_t sc = out_scale[n];
+    if (sc < 0) sc = -sc;
+    ok = ok && x < (1 << 23) && sc < (1 << 23) &&
+         x * sc + ((int64_t)1 << post) * (ooff + 2) < ((int64_t)1 << 31);
+    no_pre = no_pre && pre == 0;
+  }
+  if (ok) *flags = MI355X_REQUANT_ACC24 | (no_pre ? MI355X_REQUANT_NO_PRE_SHIFT : 0);
+  return MI355X_OK;
+}
+
 int mi355x_rowwise_quantize_i8_host(const float *in, size_t rows, size_t cols,
                                     int schema, int8_t *out, float *scales,
                                     int32_t *offsets) {

@@ -21,6 +21,21 @@ S32To8 s32to8(float ratio) {
   return {o[0], o[1], o[2]};
 }
 
+// Requantisation hint of a launch whose per-column parameters are these host
+// vectors (bias values from the constant's payload; boffs NULL = boff for all).
+int requantHintFor(size_t K, int32_t inOff, int32_t outOff, const int32_t *wOffs, const void *bias,
+                   int bias8, const int32_t *boffs, int32_t boff, const std::vector<int32_t> &bpre,
+                   const std::vector<int32_t> &bpost, const std::vector<int32_t> &bscale,
+                   const std::vector<int32_t> &opre, const std::vector<int32_t> &opost,
+                   const std::vector<int32_t> &oscale) {
+  int flags = 0;
+  if (mi355x_gemm_requant_hint_host(K, opre.size(), inOff, outOff, wOffs, bias, bias8, boffs, boff,
+                                    bpre.data(), bpost.data(), bscale.data(), opre.data(),
+                                    opost.data(), oscale.data(), &flags) != MI355X_OK)
+    return 0;
+  return flags;
+}
+
 bool shiftsOk(const S32To8 &p) { return p.pre >= 0 && p.pre <= 31 && p.post >= 0 && p.post <= 31; }
 
 // quantization::quantize<int32_t> (reference Base.h:323-329)
@@ -1030,6 +1045,10 @@ private:
                  o3 = gen_.addI32(opre), o4 = gen_.addI32(opost), o5 = gen_.addI32(oscale);
     const int bias8 = bi.ty().kind == ElemKind::Int8QTy;
     const int32_t oo = d.ty().offset, io = s.ty().offset, bo = bi.ty().offset;
+    const int hint = bi.v->category == SymbolCategory::Constant
+                         ? requantHintFor(K, io, oo, offsets, constData<uint8_t>(bi), bias8, nullptr, bo,
+                                          bpre, bpost, bscale, opre, opost, oscale)
+                         : 0;
     const bool sums = opts_.precomputeWeightRowSums && io != 0;
     auto sumPtr = scratchPtr(sums ? gen_.addScratch(N * 4) : 0);
     if (sums)
@@ -1061,6 +1080,7 @@ private:
                                           sums ? (const int32_t *)sumPtr(b) : nullptr, ro, rp.pre,
                                           rp.post, rp.scale, b.stream);
            }});
+      out.launches.back().requantHint = hint;
       return Error::success();
     }
     out.launches.push_back(
@@ -1077,6 +1097,7 @@ private:
                                    g(o3), g(o4), g(o5), M, K, N, oo, io, bo, allZero ? 1 : 0,
                                    sums ? (const int32_t *)sumPtr(b) : nullptr, b.stream);
          }});
+    out.launches.back().requantHint = hint;
     return Error::success();
   }
 
@@ -1190,6 +1211,14 @@ private:
     }
     const size_t o0 = gen_.addI32(bpre), o1 = gen_.addI32(bpost), o2 = gen_.addI32(bscale),
                  o3 = gen_.addI32(opre), o4 = gen_.addI32(opost), o5 = gen_.addI32(oscale);
+    // (K: the longest contraction any form of this convolution runs: the
+    // space-to-depth form pads the taps up to an even count per direction)
+    auto convHint = [&](size_t k) {
+      return bi.v->category == SymbolCategory::Constant
+                 ? requantHintFor(k, io, oo, fof, constData<uint8_t>(bi), bias8,
+                                  constData<int32_t>(bo), 0, bpre, bpost, bscale, opre, opost, oscale)
+                 : 0;
+    };
     // A stride-2 convolution over at most 4 channels (the first layer of an
     // image network) cannot feed the matrix cores 16 bytes at a time. Space-to-
     // depth by 2 turns it into a stride-1 convolution over 16 channels on a
@@ -1258,6 +1287,7 @@ private:
                                          allZero ? 1 : 0, sums ? (const int32_t *)sum2(b) : nullptr,
                                          b.stream);
            }});
+      out.launches.back().requantHint = convHint(K2);
       out.launches.back().reads.push_back(priv);
       return Error::success();
     }
@@ -1314,6 +1344,7 @@ private:
                  sums ? (const int32_t *)sumPtr(b) : nullptr, (const int8_t *)res.ptr(b), &fa,
                  b.stream);
            }});
+      out.launches.back().requantHint = convHint(Kf);
       return Error::success();
     }
     out.launches.push_back(
@@ -1332,6 +1363,7 @@ private:
                                        allZero ? 1 : 0, sums ? (const int32_t *)sumPtr(b) : nullptr,
                                        b.stream);
          }});
+    out.launches.back().requantHint = convHint(Kf);
     return Error::success();
   }
 
@@ -1673,9 +1705,11 @@ unsigned MI355XBackend::numDevices() {
 }
 
 int KernelLaunch::launch(const DeviceBindings &b) const {
-  if (!tunable || tile < 0) return run(b);
+  if (!tunable || (tile < 0 && requantHint == 0)) return run(b);
   mi355x_gemm_tile_override(tile);
+  mi355x_gemm_requant_hint(requantHint);
   const int rc = run(b);
+  mi355x_gemm_requant_hint(0);
   mi355x_gemm_tile_override(-1);
   return rc;
 }
@@ -1849,7 +1883,7 @@ std::string MI355XFunction::describe() const {
      << " activations=" << bundle_.activationsMemSize << "\n";
   for (const auto &l : setup) os << "setup " << l.kernel << " inst=" << l.inst << l.params << "\n";
   for (const auto &l : launches)
-    os << "launch " << l.kernel << " inst=" << l.inst << " level=" << l.level << " tile=" << l.tile
+    os << "launch " << l.kernel << " inst=" << l.inst << " level=" << l.level << " tile=" << l.tile << " requant_hint=" << l.requantHint
        << l.params << "\n";
   return os.str();
 }

@@ -430,6 +430,34 @@ int mi355x_matmul_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs_kn,
  * loaded. */
 int mi355x_gemm_tile_override(int tile);
 
+/* Requantisation hints (no counterpart in the reference) for the following
+ * matrix-core launches of the calling thread (FullyConnected, MatMul and
+ * convolution entry points); 0 = none (the default).
+ *   MI355X_REQUANT_ACC24: the caller guarantees, for every output column n,
+ *     that whatever the operand bytes are, the value in front of the output
+ *     multiply of libjit_scale (accumulator + offset corrections + rescaled
+ *     bias, shifted right by out_pre[n]) is below 2^23 in magnitude, that
+ *     |out_scale[n]| < 2^23, and that product + rounding term +
+ *     (out_offset << out_post[n]) stays inside 32 bits. The epilogue then
+ *     requantises with one 24-bit multiply-add and one shift: the same bits in
+ *     half the instruction slots.
+ *   MI355X_REQUANT_NO_PRE_SHIFT (only with ACC24): every out_pre[n] is zero; the
+ *     column constant is folded through the multiply as well.
+ * A wrong guarantee gives wrong results, not a fault.
+ * mi355x_gemm_requant_hint_host derives the flags from HOST copies of a
+ * launch's parameter vectors with worst-case operand bytes (vectors of N
+ * entries; w_offsets NULL = all zero; bias NULL = no bias; bias_offsets NULL =
+ * bias_offset for every column). */
+enum { MI355X_REQUANT_ACC24 = 1, MI355X_REQUANT_NO_PRE_SHIFT = 2 };
+int mi355x_gemm_requant_hint(int flags);
+int mi355x_gemm_requant_hint_host(size_t K, size_t N, int32_t in_offset, int32_t out_offset,
+                                  const int32_t *w_offsets, const void *bias, int bias_is_i8,
+                                  const int32_t *bias_offsets, int32_t bias_offset,
+                                  const int32_t *bias_pre, const int32_t *bias_post,
+                                  const int32_t *bias_scale, const int32_t *out_pre,
+                                  const int32_t *out_post, const int32_t *out_scale,
+                                  int *flags);
+
 /* libjit_transpose_i8 for a 2-D tensor: dst [cols x rows] = src [rows x cols]^T */
 int mi355x_transpose2d_i8(int8_t *dst, const int8_t *src, size_t rows,
                           size_t cols, void *stream);

@@ -174,3 +174,73 @@ def test_rwq_fc_m4096_k1024_n1024_all_tiles_agree():
             np.testing.assert_array_equal(got[2048:], got[:2048])
         else:
             np.testing.assert_array_equal(got, ref)
+
+
+# ---- requantisation hints ---------------------------------------------------------
+
+def _hint_for_fc(c, K):
+    return capi.gemm_requant_hint_host(K, c["in_offset"], c["out_offset"], c["w_offsets"], c["bias"],
+                                       c["bias_offset"], c["bias_pre"], c["bias_post"],
+                                       c["bias_scale"], c["out_pre"], c["out_post"], c["out_scale"])
+
+
+@pytest.mark.parametrize("tile", list(TILES))
+def test_requant_hint_gives_the_same_bytes_on_every_tile(tile):
+    """With the hint the host derives from a launch's parameters the epilogue
+    runs its 24-bit multiply-add forms; the results are those of libjit_scale."""
+    seen = set()
+    for K, wr, sym in ((64, (0.0002, 0.002), True), (64, (0.02, 0.1), True),
+                       (256, (0.0002, 0.002), False), (576, (0.0002, 0.001), True)):
+        c = cases.rwq_fc_case(300 + K, 300, K, 200, w_scale_range=wr, symmetric=sym)
+        hint = _hint_for_fc(c, K)
+        seen.add(hint)
+        want = go.rwq_fc_i8(*cases.rwq_fc_args(c))
+        say("hint", hint, "tile", TILES[tile], "K", K, "pre", int(c["out_pre"].min()),
+            int(c["out_pre"].max()))
+        with forced_tile(tile), capi.requant_hint(hint):
+            got = capi.rwq_fc_i8(*cases.rwq_fc_args(c))
+            got2 = capi.rwq_fc_i8(*cases.rwq_fc_args(c), precomputed_sums=False)
+        np.testing.assert_array_equal(got, want)
+        np.testing.assert_array_equal(got2, want)
+    assert {1, 3} <= seen          # both fast forms were exercised
+
+
+def test_requant_hint_holds_for_the_largest_accumulators():
+    """The hint is derived for worst-case operand bytes: operands that give the
+    largest possible sums of either sign still requantise exactly."""
+    K, M, N = 64, 96, 160
+    c = cases.rwq_fc_case(7, M, K, N, w_scale_range=(0.02, 0.1), symmetric=False, in_offset=-128)
+    c["x"][:] = 127
+    c["x"][M // 2:] = -128
+    c["w"][:] = -128
+    c["w"][::2] = 127
+    c["w_offsets"][:] = 20
+    c["w_offsets"][::3] = -20
+    c["bias"][:] = 1000
+    c["bias"][::2] = -1000
+    hint = _hint_for_fc(c, K)
+    assert hint & 1, "this launch fits 24 bits by construction"
+    want = go.rwq_fc_i8(*cases.rwq_fc_args(c))
+    with capi.requant_hint(hint):
+        np.testing.assert_array_equal(capi.rwq_fc_i8(*cases.rwq_fc_args(c)), want)
+        np.testing.assert_array_equal(
+            capi.rwq_fc_i8(*cases.rwq_fc_args(c), precomputed_sums=False), want)
+    assert len(np.unique(want)) > 2
+
+
+def test_requant_hint_with_convolutions_and_the_fused_add():
+    for kw in (dict(N=2, H=20, W=20, IC=64, OC=96), dict(N=1, H=14, W=14, IC=128, OC=64, kernel=(1, 1),
+                                                          pads=(0, 0, 0, 0)),
+               dict(N=2, H=9, W=9, IC=32, OC=48, symmetric=False, act=go.ACT_CLIP)):
+        c = cases.cwq_conv_case(55, in_offset=-128, **kw)
+        g = c["geom"]
+        K = g.KH * g.KW * g.IC // g.group
+        hint = capi.gemm_requant_hint_host(K, c["in_offset"], c["out_offset"], c["f_offsets"],
+                                           c["bias"], 0, c["bias_pre"], c["bias_post"],
+                                           c["bias_scale"], c["out_pre"], c["out_post"],
+                                           c["out_scale"], bias_offsets=c["b_offsets"])
+        say("conv hint", hint, kw)
+        assert hint & 1
+        want = go.cwq_conv2d_i8(*cases.cwq_conv_args(c))
+        with capi.requant_hint(hint):
+            np.testing.assert_array_equal(capi.cwq_conv2d_i8(*cases.cwq_conv_args(c)), want)

@@ -157,3 +157,27 @@ def test_channelwise_conv_constants_equal_the_oracle():
             for zero in (True, False):
                 assert capi.specialize_bias_qparams(a[0], off, a[1], a[2], i32, zero) == \
                     go.specialize_bias_qparams(a[0], off, a[1], a[2], i32, zero)
+
+
+def test_requant_hint_is_refused_when_24_bits_cannot_be_guaranteed():
+    """Worst-case accumulators of a long contraction without a pre-shift do not
+    fit 24 bits: no hint. With enough pre-shift they do."""
+    N = 8
+    one, zero = np.ones(N, np.int32), np.zeros(N, np.int32)
+    sc = np.full(N, 300, np.int32)
+    post = np.full(N, 15, np.int32)
+    args = lambda K, pre: (K, -128, 0, None, None, 0, None, None, None, np.full(N, pre, np.int32), post, sc)
+    assert capi.gemm_requant_hint_host(*args(64, 0)) == 3
+    assert capi.gemm_requant_hint_host(*args(4096, 0)) == 0
+    assert capi.gemm_requant_hint_host(*args(4096, 5)) == 1
+    # a scale of 24 bits or more, or an offset that does not fit below the post-shift
+    big = sc.copy()
+    big[3] = 1 << 23
+    assert capi.gemm_requant_hint_host(64, 0, 0, None, None, 0, None, None, None, zero, post, big) == 0
+    assert capi.gemm_requant_hint_host(64, 0, 100, None, None, 0, None, None, None, zero,
+                                       np.full(N, 25, np.int32), sc) == 0
+    # a huge bias moves the bound too
+    bias = np.full(N, 2 ** 30, np.int32)
+    assert capi.gemm_requant_hint_host(64, 0, 0, None, bias, 0, zero, zero, one, zero, post, sc) == 0
+    with pytest.raises(capi.MI355XError):
+        capi.check(capi.lib().mi355x_gemm_requant_hint(2))
