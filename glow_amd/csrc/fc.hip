@@ -5,6 +5,7 @@
 // per-row weight offsets and requantisation vectors for the rowwise form,
 // scalars for the other two.
 #include "gemm_i8.h"
+#include "gemm_skinny.h"
 
 namespace mi355x {
 
@@ -77,6 +78,16 @@ static int fc_common(int8_t *out, const int8_t *in, const int8_t *w_nk,
   ep.ldc = (long long)N;
   const bool aligned = aligned_rows(in, K) && aligned_rows(w_nk, K);
   const bool need_sb = ep.a_off != 0 && !ep.sum_b;
+  // few output tiles: 32x32 tiles with the K loop split over the waves (tile 6
+  // forces it wherever the kernel can run at all, for tuning)
+  const GemmShape g{(int)M, (int)N, (int)K, 1, 0};
+  const bool can_skinny = aligned && !need_sa && !need_sb && !ep.add.res && K >= 32 &&
+                          K % 32 == 0 && (long long)((M + 31) / 32) * ((N + 31) / 32) < (1 << 22);
+  if ((g_tile_override == 6 && can_skinny) ||
+      (g_tile_override < 0 && skinny_applies(g, ep, need_sa, need_sb, aligned))) {
+    ep.fast = g_requant_hint & 3;
+    return gemm_skinny_launch(A, B, ep, g, as_stream(stream));
+  }
   return gemm_dispatch(A, B, ep, (int)M, (int)N, (int)K, 1, 0, need_sa, need_sb,
                        aligned, as_stream(stream));
 }
@@ -88,7 +99,7 @@ using namespace mi355x;
 extern "C" {
 
 int mi355x_gemm_tile_override(int tile) {
-  MI355X_REQUIRE(tile >= -1 && tile <= 5, "tile %d outside [-1, 5]", tile);
+  MI355X_REQUIRE(tile >= -1 && tile <= 6, "tile %d outside [-1, 6]", tile);
   g_tile_override = tile;
   return MI355X_OK;
 }

@@ -424,8 +424,11 @@ int mi355x_matmul_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs_kn,
 
 /* Tuning aid (no counterpart in the reference): forces the workgroup tile of
  * the following matrix-core launches of the calling thread: 0 = 256x256,
- * 1 = 128x128, 2 = 128x64, 3 = 64x64, 4 = 256x128, 5 = 128x256; -1 = chosen from
- * the problem shape (the default). Results do not depend on the tile. A device
+ * 1 = 128x128, 2 = 128x64, 3 = 64x64, 4 = 256x128, 5 = 128x256, 6 = 32x32 with
+ * the K loop split over the workgroup's waves (FullyConnected forms with
+ * symmetric weights, precomputed row sums and K % 32 == 0 only; launches it
+ * cannot serve ignore it); -1 = chosen from the problem shape (the default).
+ * Results do not depend on the tile. A device
  * manager uses it to time the candidates of each layer once, when a network is
  * loaded. */
 int mi355x_gemm_tile_override(int tile);

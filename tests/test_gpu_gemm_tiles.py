@@ -22,7 +22,8 @@ from tests import cases
 
 pytestmark = pytest.mark.gpu
 
-TILES = {0: "256x256", 1: "128x128", 2: "128x64", 3: "64x64", 4: "256x128", 5: "128x256"}
+TILES = {0: "256x256", 1: "128x128", 2: "128x64", 3: "64x64", 4: "256x128", 5: "128x256",
+         6: "32x32 split-K"}
 
 
 @pytest.fixture(scope="module", autouse=True)
@@ -244,3 +245,56 @@ def test_requant_hint_with_convolutions_and_the_fused_add():
         want = go.cwq_conv2d_i8(*cases.cwq_conv_args(c))
         with capi.requant_hint(hint):
             np.testing.assert_array_equal(capi.cwq_conv2d_i8(*cases.cwq_conv_args(c)), want)
+
+
+# ---- 32x32 tiles with the K loop split over the waves ------------------------------
+
+SKINNY_SHAPES = [(128, 1024, 1024), (1, 128, 1), (7, 160, 33), (33, 96, 70), (64, 4096, 256),
+                 (130, 32, 90), (16, 2048 + 32, 1000), (256, 512, 128)]
+
+
+@pytest.mark.parametrize("shape", SKINNY_SHAPES)
+def test_split_k_small_tiles_vs_oracle(shape):
+    """Symmetric weights with precomputed row sums (what the kernel serves), both
+    by the shape rule and forced; int32 and int8 bias, zero and non-zero input
+    offset, with and without the requantisation hint, and the fused Relu."""
+    M, K, N = shape
+    for seed, b8, in_off in ((1, False, None), (2, True, None), (3, False, 0)):
+        c = cases.rwq_fc_case(seed + M + K, M, K, N, symmetric=True, bias_i8=b8,
+                              bias_scale=(0.01 if b8 else 5e-5), bias_offset=(3 if b8 else 0),
+                              in_offset=in_off)
+        args = cases.rwq_fc_args(c)
+        want = go.rwq_fc_i8(*args)
+        hint = _hint_for_fc(c, K)
+        say("split-K", shape, "bias8" if b8 else "bias32", "in_offset", c["in_offset"], "hint", hint)
+        for forced in (6, None):
+            for h in sorted({0, hint}):
+                with capi.requant_hint(h):
+                    if forced is None:
+                        got = capi.rwq_fc_i8(*args)
+                    else:
+                        with forced_tile(forced):
+                            got = capi.rwq_fc_i8(*args)
+                np.testing.assert_array_equal(got, want)
+        fc = want
+        for relu_offset, reluP in ((-128, (0, 8, 300)), (5, (1, 9, 1 << 24))):
+            want_relu = go.relu_i8(fc, c["out_offset"], relu_offset, reluP)
+            with forced_tile(6):
+                got = capi.rwq_fc_relu_i8(*args[:10], c["out_offset"], c["in_offset"],
+                                          c["bias_offset"], relu_offset, reluP)
+            np.testing.assert_array_equal(got, want_relu)
+
+
+def test_split_k_tile_is_ignored_where_it_cannot_run():
+    """Weight offsets, missing row sums or a K that is no multiple of 32: tile 6
+    falls back to the tiled kernels, same results."""
+    for kw, sums in ((dict(symmetric=False), True), (dict(symmetric=True), False)):
+        c = cases.rwq_fc_case(9, 40, 256, 72, **kw)
+        want = go.rwq_fc_i8(*cases.rwq_fc_args(c))
+        with forced_tile(6):
+            got = capi.rwq_fc_i8(*cases.rwq_fc_args(c), precomputed_sums=sums)
+        np.testing.assert_array_equal(got, want)
+    c = cases.rwq_fc_case(10, 40, 272, 72)           # K % 32 == 16
+    with forced_tile(6):
+        np.testing.assert_array_equal(capi.rwq_fc_i8(*cases.rwq_fc_args(c)),
+                                      go.rwq_fc_i8(*cases.rwq_fc_args(c)))
