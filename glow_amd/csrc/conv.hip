@@ -10,6 +10,7 @@
 // (in - inOffset) = 0 just the same, so out-of-image taps are filled with the
 // input offset and the dense contraction of gemm_i8.h applies unchanged.
 #include "gemm_i8.h"
+#include "conv_halo.h"
 
 namespace mi355x {
 
@@ -169,6 +170,16 @@ static int conv_common(int8_t *out, const int8_t *in, const int8_t *filter,
                     ((((uintptr_t)in) & 15) == 0);
   const bool al_b = (K % 16 == 0) && ((((uintptr_t)filter) & 15) == 0);
   const bool need_sb = ep.a_off != 0 && !ep.sum_b;
+  // 3x3, stride 1, 64 input channels, symmetric filters: operands resident in
+  // LDS (conv_halo.h). Tile 7 forces it, tiles 0..6 keep the implicit GEMM.
+  if ((g_tile_override < 0 || g_tile_override == 7) && !need_sa && !need_sb && al_a && al_b) {
+    int halo_rows = 0;
+    const size_t lds = conv_halo_lds_bytes(g, halo_rows);
+    if (lds != 0 && lds <= lds_limit()) {
+      ep.fast = g_requant_hint & 3;
+      return conv_halo_launch(in, filter, g, ep, lds, halo_rows, as_stream(stream));
+    }
+  }
   // A pointwise convolution over the whole image is a plain matrix product:
   // row m of A is pixel m of the input, no taps to locate and no padding.
   if (g->KH == 1 && g->KW == 1 && g->strideH == 1 && g->strideW == 1 &&

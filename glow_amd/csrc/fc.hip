@@ -99,7 +99,7 @@ using namespace mi355x;
 extern "C" {
 
 int mi355x_gemm_tile_override(int tile) {
-  MI355X_REQUIRE(tile >= -1 && tile <= 6, "tile %d outside [-1, 6]", tile);
+  MI355X_REQUIRE(tile >= -1 && tile <= 7, "tile %d outside [-1, 7]", tile);
   g_tile_override = tile;
   return MI355X_OK;
 }

@@ -427,8 +427,10 @@ int mi355x_matmul_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs_kn,
  * 1 = 128x128, 2 = 128x64, 3 = 64x64, 4 = 256x128, 5 = 128x256, 6 = 32x32 with
  * the K loop split over the workgroup's waves (FullyConnected forms with
  * symmetric weights, precomputed row sums and K % 32 == 0 only; launches it
- * cannot serve ignore it); -1 = chosen from the problem shape (the default).
- * Results do not depend on the tile. A device
+ * cannot serve ignore it), 7 = the 3x3 stride-1 convolution over 64 input
+ * channels with filter and input rows resident in LDS (other launches ignore
+ * it; tiles 0..6 keep such a convolution on the tiled kernels); -1 = chosen
+ * from the problem shape (the default). Results do not depend on the tile. A device
  * manager uses it to time the candidates of each layer once, when a network is
  * loaded. */
 int mi355x_gemm_tile_override(int tile);
