@@ -172,12 +172,14 @@ static int conv_common(int8_t *out, const int8_t *in, const int8_t *filter,
   const bool need_sb = ep.a_off != 0 && !ep.sum_b;
   // 3x3, stride 1, 64 input channels, symmetric filters: operands resident in
   // LDS (conv_halo.h). Tile 7 forces it, tiles 0..6 keep the implicit GEMM.
-  if ((g_tile_override < 0 || g_tile_override == 7) && !need_sa && !need_sb && al_a && al_b) {
-    int halo_rows = 0;
-    const size_t lds = conv_halo_lds_bytes(g, halo_rows);
-    if (lds != 0 && lds <= lds_limit()) {
+  const bool al_out = ((((uintptr_t)out) | ((uintptr_t)ep.add.res)) & 15) == 0;
+  if ((g_tile_override < 0 || g_tile_override == 7) && !need_sa && !need_sb && al_a && al_b &&
+      al_out) {
+    size_t lds = 0;
+    const int rows = conv_halo_rows(g, device_cus(), lds);
+    if (rows != 0 && lds <= lds_limit()) {
       ep.fast = g_requant_hint & 3;
-      return conv_halo_launch(in, filter, g, ep, lds, halo_rows, as_stream(stream));
+      return conv_halo_launch(in, filter, g, ep, lds, rows, as_stream(stream));
     }
   }
   // A pointwise convolution over the whole image is a plain matrix product:

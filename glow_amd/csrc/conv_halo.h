@@ -3,23 +3,29 @@
 // with the operands held in LDS the way the matrix cores want them, instead
 // of the implicit-GEMM gather of gemm_i8.h:
 //
-//   * the filter slice of a workgroup (64 output channels x 576 bytes, 37 KB)
-//     is loaded once and stays in LDS while the workgroup walks over output
-//     tiles (persistent workgroups, tiles taken round-robin);
-//   * per tile of 128 consecutive output pixels of one image, the input rows
-//     those pixels need (at most six rows of 58 pixels for a 56x56 image,
-//     padding columns and rows materialised as input-offset bytes) are staged
-//     once: every input byte is read from memory once per tile instead of once
-//     per tap;
+//   * a workgroup computes a tile of whole output rows of one image (as many
+//     rows as give at most 256 pixels: four rows of a 56-wide image) for 64
+//     output channels, one wave per 32 consecutive pixels, so the block size
+//     follows the image (seven waves for 4 x 56 pixels);
+//   * the filter slice (64 output channels x 576 bytes, 37 KB) and the input
+//     rows the tile needs (its rows plus one above and below, one pixel left
+//     and right; padding materialised as input-offset bytes) are staged in LDS
+//     once, all loads of a thread in flight together: every input byte is read
+//     from memory once per tile instead of once per tap;
 //   * the nine taps are then LDS address arithmetic: a lane's fragment of tap
 //     (fx, fy) sits a constant distance from its pixel's base address, so the
-//     K loop is ds_read_b128 + v_mfma with nothing else in it.
+//     K loop is ds_read_b128 + v_mfma with nothing else in it;
+//   * the filter is the first matrix-core operand and its rows are placed in LDS
+//     in such an order that a lane's sixteen accumulators of a channel tile are
+//     sixteen consecutive channels of one pixel: they are requantised, packed
+//     and written with one 16-byte store each, straight from registers. There is
+//     no barrier after the one that ends the staging: every wave finishes its
+//     32 pixels on its own.
 //
 // Pixels and filter rows are 16 bytes apart from a power-of-two stride in LDS
 // (80 and 592 bytes), which spreads the 16-byte fragment reads of consecutive
-// rows over all banks. A wave owns 32 pixels x 64 channels (two 32x32x32
-// accumulator tiles), four waves a tile. The epilogue is the shared one of
-// gemm_i8.h (requantisation, activation, optional fused residual add).
+// rows over all banks. The arithmetic is that of the shared epilogue of
+// gemm_i8.h (requantisation, activation, the optional fused residual add).
 //
 // Padded taps hold the input offset, so (in - inOffset) contributes zero for
 // them exactly as the CPU loop's skipped taps do; the results are bit for bit
@@ -34,183 +40,316 @@ namespace mi355x {
 struct HaloConv {
   const int8_t *in;      // NHWC, 64 channels
   const int8_t *filter;  // [OC][3][3][64]
-  int N, IH, IW, OH, OW, OC;
+  int IH, IW, OH, OW, OC;
   int padT, padL;
-  int tiles_per_image, total_tiles;
-  int halo_rows;         // LDS rows reserved: rows a tile can span + 2
+  int rows;              // output rows per tile
+  int tiles_per_image;
   uint32_t fill;         // input offset replicated into four bytes
 };
 
-constexpr int kHaloBM = 128, kHaloBN = 64, kHaloIC = 64, kHaloK = 9 * kHaloIC;
+constexpr int kHaloMaxPix = 256, kHaloBN = 64, kHaloIC = 64, kHaloK = 9 * kHaloIC;
 constexpr int kHaloPix = kHaloIC + 16;        // bytes between pixels in LDS
 constexpr int kHaloFRow = kHaloK + 16;        // bytes between filter rows in LDS
 constexpr int kHaloFilterBytes = kHaloBN * kHaloFRow;
+// (rows + 2) x (OW + 2) pixels with rows * OW <= 256 is largest for one row of 256
+constexpr size_t kHaloMaxLds =
+    kHaloFilterBytes + 5 * kHaloBN * 4 + (size_t)3 * (kHaloMaxPix + 2) * kHaloPix;
+constexpr int kHaloFilterChunks = kHaloBN * (kHaloK / 16);   // 16-byte chunks
 
-__global__ __launch_bounds__(256, 2) void conv3x3_halo_kernel(HaloConv cv, Epilogue ep) {
+// Per-channel requantisation constants of a workgroup's 64 output channels, in
+// LDS as five arrays of 64 ints: in the accumulator layout used here a lane
+// holds 32 different channels, so it reads them (four consecutive channels per
+// ds_read_b128, the same address across half a wave) instead of keeping them.
+enum { kParColc = 0, kParPre = 1, kParScale = 2, kParPost = 3, kParFold = 4, kParArrays = 5 };
+constexpr int kHaloParBytes = kParArrays * kHaloBN * 4;
+
+// Filter row (output channel) c of a workgroup's 64 sits in LDS slot
+// halo_filter_slot(c): matrix-core row 8 q + 4 h + i of channel tile j holds
+// channel 32 h + 16 j + 4 q + i, so that lane (pixel, h) ends up with channels
+// 32 h + 16 j + [0, 16) of its pixel in the sixteen accumulators of tile j, in
+// order: sixteen consecutive output bytes.
+__device__ __forceinline__ int halo_filter_slot(int c) {
+  return 32 * ((c >> 4) & 1) + 8 * ((c >> 2) & 3) + 4 * (c >> 5) + (c & 3);
+}
+
+// Requantises a lane's 2 x 16 accumulators (pixel l % 32, channels
+// 32 (l / 32) + 16 j + r for register r of tile j) and writes them as two
+// 16-byte stores straight from registers; `out` points at the pixel's 64
+// channels (NULL: the lane's pixel lies past the tile), `res` at the residual's.
+// MODE 0: scale_i32; 1: 24-bit multiply with pre-shift; 3: 24-bit multiply,
+// no pre-shift, column constant folded (the caller's requantisation hints).
+template <int MODE, bool LEAKY>
+__device__ __forceinline__ void halo_requant_store(const v16i (&acc)[2], const int32_t *s_par,
+                                                   const Epilogue &ep, int lhi, int8_t *out,
+                                                   const int8_t *res) {
+  int32_t lo = -128, hi = 127;
+  if (ep.act == 1) lo = clip_i8(ep.out_off);
+  if (ep.act == 2) {
+    lo = clip_i8(ep.a0);
+    hi = clip_i8(ep.a1);
+    if (lo > hi) lo = hi;
+  }
+  const bool fast = fused_out_is_fast(ep);
+  const FusedAddConsts fc = fused_add_consts(ep.add);
+#pragma unroll
+  for (int j = 0; j < 2; j++) {
+    const int cbase = 32 * lhi + 16 * j;
+    uint32_t w[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      const int ch = cbase + 4 * q;
+      const v4i scale = *reinterpret_cast<const v4i *>(s_par + kParScale * kHaloBN + ch);
+      const v4i post = *reinterpret_cast<const v4i *>(s_par + kParPost * kHaloBN + ch);
+      v4i colc, pre, fold;
+      if constexpr (MODE != 3) {
+        colc = *reinterpret_cast<const v4i *>(s_par + kParColc * kHaloBN + ch);
+        pre = *reinterpret_cast<const v4i *>(s_par + kParPre * kHaloBN + ch);
+      }
+      if constexpr (MODE != 0) fold = *reinterpret_cast<const v4i *>(s_par + kParFold * kHaloBN + ch);
+      uint32_t b[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const uint32_t x = (uint32_t)acc[j][4 * q + i];
+        int32_t y;
+        if constexpr (MODE == 3) {
+          y = (int32_t)((uint32_t)__mul24((int32_t)x, scale[i]) + (uint32_t)fold[i]) >> post[i];
+        } else if constexpr (MODE == 1) {
+          y = (int32_t)((uint32_t)__mul24((int32_t)(x + (uint32_t)colc[i]) >> pre[i], scale[i]) +
+                        (uint32_t)fold[i]) >> post[i];
+        } else {
+          y = scale_i32((int32_t)(x + (uint32_t)colc[i]), pre[i], post[i], scale[i], ep.out_off);
+        }
+        if constexpr (LEAKY) {
+          if (y < ep.out_off)
+            y = scale_i32((int32_t)((uint32_t)y - (uint32_t)ep.out_off), ep.a0, ep.a1, ep.a2,
+                          ep.out_off);
+        }
+        b[i] = (uint32_t)med3_i32(y, lo, hi);
+      }
+      // low bytes of four registers -> one word
+      const uint32_t w01 = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);
+      const uint32_t w23 = __builtin_amdgcn_perm(b[3], b[2], 0x0c0c0400u);
+      w[q] = __builtin_amdgcn_perm(w23, w01, 0x05040100u);
+    }
+    if (out) {
+      int4 v = make_int4((int)w[0], (int)w[1], (int)w[2], (int)w[3]);
+      v = fused_out_words(v, res ? res + cbase : nullptr, ep, fc, fast);
+      *reinterpret_cast<int4 *>(out + cbase) = v;
+    }
+  }
+}
+
+// SKIP leaves phases out so that the others can be timed (1: staging, 2: the
+// matrix-core loop, 4: requantisation and copy-out); the library uses 0.
+template <int SKIP = 0>
+__global__ __launch_bounds__(512, 2) void conv3x3_halo_kernel(HaloConv cv, Epilogue ep) {
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   int8_t *s_filter = lds;
-  int8_t *s_halo = lds + kHaloFilterBytes;    // also the epilogue's staging area
+  int32_t *s_par = reinterpret_cast<int32_t *>(lds + kHaloFilterBytes);
+  int8_t *s_halo = lds + kHaloFilterBytes + kHaloParBytes;
 
   const int tid = threadIdx.x;
+  const int nthreads = blockDim.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, lhi = lane >> 5;
   const int n0 = blockIdx.y * kHaloBN;        // first output channel of the slice
 
-  // the epilogue's per-column parameters, requested first
-  ColRaw col[2];
-  load_col_raw<2, 64>(col, ep, cv.OC, n0, 0, 0, l32);
+  const int n = blockIdx.x / cv.tiles_per_image;
+  const int oh_first = (blockIdx.x - n * cv.tiles_per_image) * cv.rows;
+  const int rows = min(cv.rows, cv.OH - oh_first);
+  const int npix = rows * cv.OW;
+  const int hw = cv.OW + 2;                   // halo pixels per row
+  const int mode = ep.act == 5 ? 0 : ep.fast & 3;
 
-  // filter slice -> LDS, once
-  {
-    constexpr int kChunks = kHaloBN * (kHaloK / 16);   // 16-byte chunks
+  // the channels' raw parameters, requested first (by the last wave: the first
+  // ones carry the staging loop's remainders)
+  const bool par_wave = wave == (int)(nthreads >> 6) - 1;
+  ColRaw col[1];
+  if (par_wave) load_col_raw<1, 64>(col, ep, cv.OC, n0, 0, 0, lane);
+
+  // ---- stage the tile's input rows and the filter slice -------------------------
+  if constexpr (!(SKIP & 1)) {
+    const int4 fill4 = make_int4((int)cv.fill, (int)cv.fill, (int)cv.fill, (int)cv.fill);
+    const int8_t *img = cv.in + (long long)n * cv.IH * cv.IW * kHaloIC;
     const int8_t *f = cv.filter + (long long)n0 * kHaloK;
-#pragma unroll
-    for (int i = 0; i < (kChunks + 255) / 256; i++) {
-      const int c = tid + i * 256;
-      if (c < kChunks) {
-        const int row = c / (kHaloK / 16), kc = c - row * (kHaloK / 16);
-        *reinterpret_cast<int4 *>(s_filter + row * kHaloFRow + kc * 16) =
-            *reinterpret_cast<const int4 *>(f + (long long)row * kHaloK + kc * 16);
+    const int halo_chunks = (rows + 2) * hw * (kHaloIC / 16);
+    constexpr int HU = 4, FU = 6;
+    // chunk c of the halo: pixel c / 4 of the (rows + 2) x hw patch, bytes
+    // 16 * (c % 4) of its channels
+    auto halo_load = [&](int c) -> int4 {
+      int4 v = fill4;
+      if (c < halo_chunks) {
+        const int px = c >> 2, kc = c & 3;
+        const int hr = px / hw, hc = px - hr * hw;
+        const int ih = oh_first - cv.padT + hr, iw = hc - cv.padL;
+        if (ih >= 0 && ih < cv.IH && iw >= 0 && iw < cv.IW)
+          v = *reinterpret_cast<const int4 *>(img + ((long long)ih * cv.IW + iw) * kHaloIC +
+                                              kc * 16);
       }
+      return v;
+    };
+    auto halo_store = [&](int c, const int4 &v) {
+      if (c < halo_chunks)
+        *reinterpret_cast<int4 *>(s_halo + (c >> 2) * kHaloPix + (c & 3) * 16) = v;
+    };
+    auto filter_load = [&](int c) -> int4 {
+      int4 v = fill4;
+      if (c < kHaloFilterChunks) {
+        const int row = c / (kHaloK / 16), kc = c - row * (kHaloK / 16);
+        v = *reinterpret_cast<const int4 *>(f + (long long)row * kHaloK + kc * 16);
+      }
+      return v;
+    };
+    auto filter_store = [&](int c, const int4 &v) {
+      if (c < kHaloFilterChunks) {
+        const int row = c / (kHaloK / 16), kc = c - row * (kHaloK / 16);
+        *reinterpret_cast<int4 *>(s_filter + halo_filter_slot(row) * kHaloFRow + kc * 16) = v;
+      }
+    };
+    // first batch of both in flight together
+    int4 hv[HU], fv[FU];
+#pragma unroll
+    for (int u = 0; u < HU; u++) hv[u] = halo_load(tid + u * nthreads);
+#pragma unroll
+    for (int u = 0; u < FU; u++) fv[u] = filter_load(tid + u * nthreads);
+#pragma unroll
+    for (int u = 0; u < HU; u++) halo_store(tid + u * nthreads, hv[u]);
+#pragma unroll
+    for (int u = 0; u < FU; u++) filter_store(tid + u * nthreads, fv[u]);
+    for (int base = HU * nthreads; base < halo_chunks; base += HU * nthreads) {
+#pragma unroll
+      for (int u = 0; u < HU; u++) hv[u] = halo_load(base + tid + u * nthreads);
+#pragma unroll
+      for (int u = 0; u < HU; u++) halo_store(base + tid + u * nthreads, hv[u]);
+    }
+    for (int base = FU * nthreads; base < kHaloFilterChunks; base += FU * nthreads) {
+#pragma unroll
+      for (int u = 0; u < FU; u++) fv[u] = filter_load(base + tid + u * nthreads);
+#pragma unroll
+      for (int u = 0; u < FU; u++) filter_store(base + tid + u * nthreads, fv[u]);
     }
   }
 
-  const int hw = cv.OW + 2;                    // halo pixels per row
-  const int pix_per_image = cv.OH * cv.OW;
-  const int4 fill4 = make_int4((int)cv.fill, (int)cv.fill, (int)cv.fill, (int)cv.fill);
-  // where this lane's B fragments start: filter row l32 (+32 for the second
-  // column tile), k-bytes lhi*16..
-  const int b_base = l32 * kHaloFRow + lhi * 16;
+  // ---- the channels' requantisation constants -> LDS --------------------------------
+  if (par_wave) {
+    const ColRaw &c = col[0];
+    uint32_t colc = (uint32_t)kHaloK * (uint32_t)ep.a_off * (uint32_t)c.woff;
+    if (ep.sum_b) colc -= (uint32_t)ep.a_off * (uint32_t)c.sumb;
+    if (ep.bias)
+      colc += (uint32_t)scale_i32((int32_t)((uint32_t)c.bias - (uint32_t)c.boff), c.bpre,
+                                  c.bpost, c.bscale, 0);
+    uint32_t fold = (c.opost > 0 ? (1u << (c.opost - 1)) : 0u) + ((uint32_t)ep.out_off << c.opost);
+    if (mode == 3) fold += colc * (uint32_t)c.oscale;
+    s_par[kParColc * kHaloBN + lane] = (int32_t)colc;
+    s_par[kParPre * kHaloBN + lane] = c.opre;
+    s_par[kParScale * kHaloBN + lane] = c.oscale;
+    s_par[kParPost * kHaloBN + lane] = c.opost;
+    s_par[kParFold * kHaloBN + lane] = (int32_t)fold;
+  }
+  __syncthreads();
 
-  for (int t = blockIdx.x; t < cv.total_tiles; t += gridDim.x) {
-    const int n = t / cv.tiles_per_image;
-    const int p0 = (t - n * cv.tiles_per_image) * kHaloBM;
-    const int npix = min(kHaloBM, pix_per_image - p0);
-    const int oh_first = p0 / cv.OW;
-    const int oh_last = (p0 + npix - 1) / cv.OW;
-    const int hrows = oh_last - oh_first + 3;
-
-    __syncthreads();   // the previous tile's copy-out has left the staging area
-    // ---- stage the input rows of this tile ------------------------------------
-    {
-      const int total = hrows * hw * (kHaloIC / 16);
-      const int8_t *img = cv.in + (long long)n * cv.IH * cv.IW * kHaloIC;
-      for (int base = 0; base < total; base += 256 * 8) {
-        int4 v[8];
+  // ---- nine taps x two 32-byte k slices -------------------------------------------
+  v16i acc[2];
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
-          const int c = base + tid + u * 256;
-          v[u] = fill4;
-          if (c < total) {
-            const int px = c >> 2, kc = c & 3;
-            const int hr = px / hw, hc = px - hr * hw;
-            const int ih = oh_first - cv.padT + hr, iw = hc - cv.padL;
-            if (ih >= 0 && ih < cv.IH && iw >= 0 && iw < cv.IW)
-              v[u] = *reinterpret_cast<const int4 *>(
-                  img + ((long long)ih * cv.IW + iw) * kHaloIC + kc * 16);
-          }
-        }
+  for (int j = 0; j < 2; j++)
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
-          const int c = base + tid + u * 256;
-          if (c < total) {
-            const int px = c >> 2, kc = c & 3;
-            *reinterpret_cast<int4 *>(s_halo + px * kHaloPix + kc * 16) = v[u];
-          }
-        }
-      }
-    }
-    __syncthreads();
-
-    // ---- nine taps x two 32-byte k slices ---------------------------------------
-    v16i acc[1][2];
+    for (int r = 0; r < 16; r++) acc[j][r] = (SKIP & 2) ? tid + r : 0;
+  if constexpr (!(SKIP & 2)) {
+    // this lane's pixel (lanes past the tile's end recompute its last pixel;
+    // the copy-out does not store them)
+    const int p = min(wave * 32 + l32, npix - 1);
+    const int orow = p / cv.OW, ow = p - orow * cv.OW;
+    const int8_t *a_base = s_halo + (orow * hw + ow) * kHaloPix + lhi * 16;
+    // this lane's filter slot l32 (+32 for the second channel tile), k-bytes lhi*16..
+    const int8_t *b_base = s_filter + l32 * kHaloFRow + lhi * 16;
+    const int row_step = hw * kHaloPix;
 #pragma unroll
-    for (int j = 0; j < 2; j++)
+    for (int fx = 0; fx < 3; fx++) {
 #pragma unroll
-      for (int r = 0; r < 16; r++) acc[0][j][r] = 0;
-    {
-      // this lane's pixel (lanes past the tile's end recompute its last pixel;
-      // the epilogue does not store them)
-      const int p = p0 + min(wave * 32 + l32, npix - 1);
-      const int oh = p / cv.OW, ow = p - oh * cv.OW;
-      const int8_t *a_base = s_halo + ((oh - oh_first) * hw + ow) * kHaloPix + lhi * 16;
-      const int row_step = hw * kHaloPix;
+      for (int fy = 0; fy < 3; fy++) {
 #pragma unroll
-      for (int fx = 0; fx < 3; fx++) {
-#pragma unroll
-        for (int fy = 0; fy < 3; fy++) {
-#pragma unroll
-          for (int ks = 0; ks < kHaloIC / 32; ks++) {
-            const v4i af = *reinterpret_cast<const v4i *>(a_base + fx * row_step +
-                                                          fy * kHaloPix + ks * 32);
-            const int kb = (fx * 3 + fy) * kHaloIC + ks * 32;
-            const v4i b0 = *reinterpret_cast<const v4i *>(s_filter + b_base + kb);
-            const v4i b1 =
-                *reinterpret_cast<const v4i *>(s_filter + b_base + 32 * kHaloFRow + kb);
-            acc[0][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, b0, acc[0][0], 0, 0, 0);
-            acc[0][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, b1, acc[0][1], 0, 0, 0);
-          }
+        for (int ks = 0; ks < kHaloIC / 32; ks++) {
+          const v4i af = *reinterpret_cast<const v4i *>(a_base + fx * row_step +
+                                                        fy * kHaloPix + ks * 32);
+          const int kb = (fx * 3 + fy) * kHaloIC + ks * 32;
+          const v4i b0 = *reinterpret_cast<const v4i *>(b_base + kb);
+          const v4i b1 = *reinterpret_cast<const v4i *>(b_base + 32 * kHaloFRow + kb);
+          // filter rows first: the result's rows are channels, its columns pixels
+          acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b0, af, acc[0], 0, 0, 0);
+          acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b1, af, acc[1], 0, 0, 0);
         }
       }
     }
-    __syncthreads();   // every wave has read its halo: the area becomes staging
-
-    int sa[1] = {0}, sb[2] = {0, 0};
-    const int m0 = n * pix_per_image + p0;
-    // rows past the tile's end belong to the next tile (or image): M bounds them
-    gemm_epilogue<kHaloBM, kHaloBN, 32, 64, false, false>(acc, sa, sb, s_halo, ep, m0 + npix,
-                                                          cv.OC, kHaloK, m0, n0, 0, col);
+  }
+  // no barrier: the waves finish on their own, nothing in LDS is reused
+  if constexpr (!(SKIP & 4)) {
+    const int p = wave * 32 + l32;
+    const long long m = (long long)(n * cv.OH + oh_first) * cv.OW + p;
+    int8_t *out = p < npix ? ep.out + m * ep.ldc + n0 : nullptr;
+    const int8_t *res = ep.add.res ? ep.add.res + m * ep.ldc + n0 : nullptr;
+    if (ep.act == 5) halo_requant_store<0, true>(acc, s_par, ep, lhi, out, res);
+    else if (mode == 3) halo_requant_store<3, false>(acc, s_par, ep, lhi, out, res);
+    else if (mode & 1) halo_requant_store<1, false>(acc, s_par, ep, lhi, out, res);
+    else halo_requant_store<0, false>(acc, s_par, ep, lhi, out, res);
+  } else {
+    int x = 0;
+#pragma unroll
+    for (int r = 0; r < 16; r++) x += acc[0][r] ^ acc[1][r];
+    if (x == 0x12345678) ep.out[tid] = (int8_t)x;
   }
 }
 
-// LDS the kernel needs for this geometry, or 0 when the shape is not its own.
-static size_t conv_halo_lds_bytes(const mi355x_conv_geom *g, int &halo_rows) {
+// Output rows per tile for this geometry, or 0 when the shape is not the
+// kernel's own; lds receives the dynamic LDS a block needs.
+static int conv_halo_rows(const mi355x_conv_geom *g, int cus, size_t &lds) {
   if (g->KH != 3 || g->KW != 3 || g->strideH != 1 || g->strideW != 1 || g->dilH != 1 ||
       g->dilW != 1 || g->group != 1 || g->IC != kHaloIC || g->OC % kHaloBN != 0)
     return 0;
-  if (g->OH <= 0 || g->OW <= 0) return 0;
-  // rows that 128 consecutive pixels of one image can touch
-  int rows = (kHaloBM + g->OW - 2) / g->OW + 1;
+  if (g->OH <= 0 || g->OW <= 0 || g->OW > kHaloMaxPix) return 0;
+  int rows = kHaloMaxPix / g->OW;
   if (rows > g->OH) rows = g->OH;
-  halo_rows = rows + 2;
-  const size_t halo = (size_t)halo_rows * (g->OW + 2) * kHaloPix;
-  const size_t epi = gemm_epilogue_lds_bytes<kHaloBM, kHaloBN>();
-  return kHaloFilterBytes + (halo > epi ? halo : epi);
+  // fewer rows per tile while that gives the chip more tiles than CUs and a
+  // tile keeps at least a wave's worth of pixels
+  const long long slices = g->OC / kHaloBN;
+  while (rows > 1 && (long long)g->N * ((g->OH + rows - 1) / rows) * slices < cus &&
+         (rows - 1) * g->OW >= 32)
+    rows--;
+  const int waves = (rows * g->OW + 31) / 32;
+  const size_t halo = (size_t)(rows + 2) * (g->OW + 2) * kHaloPix;
+  lds = kHaloFilterBytes + kHaloParBytes + halo;
+  return rows;
 }
 
 static int conv_halo_launch(const int8_t *in, const int8_t *filter, const mi355x_conv_geom *g,
-                            const Epilogue &ep, size_t lds, int halo_rows, hipStream_t st) {
+                            const Epilogue &ep, size_t lds, int rows, hipStream_t st) {
   HaloConv cv;
   cv.in = in;
   cv.filter = filter;
-  cv.N = g->N; cv.IH = g->IH; cv.IW = g->IW; cv.OH = g->OH; cv.OW = g->OW; cv.OC = g->OC;
+  cv.IH = g->IH; cv.IW = g->IW; cv.OH = g->OH; cv.OW = g->OW; cv.OC = g->OC;
   cv.padT = g->padT; cv.padL = g->padL;
-  cv.tiles_per_image = (g->OH * g->OW + kHaloBM - 1) / kHaloBM;
+  cv.rows = rows;
+  cv.tiles_per_image = (g->OH + rows - 1) / rows;
   const long long total = (long long)g->N * cv.tiles_per_image;
-  MI355X_REQUIRE(total < 0x7fffffffLL, "problem too large");
-  cv.total_tiles = (int)total;
-  cv.halo_rows = halo_rows;
+  MI355X_REQUIRE(total < 0x7fffffffLL && (long long)g->N * g->OH * g->OW < 0x7fffffffLL,
+                 "problem too large");
   cv.fill = 0x01010101u * (uint32_t)(uint8_t)(int8_t)ep.a_off;
   static std::atomic<uint64_t> attr_set{0};
-  int rc = set_lds_attr(conv3x3_halo_kernel, lds, attr_set);
+  // the attribute is set once per device: to the most any geometry can ask for
+  int rc = set_lds_attr(conv3x3_halo_kernel<0>, kHaloMaxLds, attr_set);
   if (rc != MI355X_OK) return rc;
-  // persistent workgroups: as many as stay resident (two per CU while the LDS
-  // allows), fewer when there are fewer tiles
-  int dev = 0, cus = 256;
-  if (hipGetDevice(&dev) == hipSuccess) {
-    int v = 0;
-    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
-      cus = v;
-  }
-  const int slices = g->OC / kHaloBN;
-  const int per_cu = lds * 2 <= 160 * 1024 ? 2 : 1;
-  long long gx = (long long)cus * per_cu / slices;
-  if (gx < 1) gx = 1;
-  if (gx > total) gx = total;
-  hipLaunchKernelGGL(conv3x3_halo_kernel, dim3((unsigned)gx, (unsigned)slices), dim3(256), lds, st,
-                     cv, ep);
+  const int waves = (rows * g->OW + 31) / 32;
+  hipLaunchKernelGGL(conv3x3_halo_kernel<0>, dim3((unsigned)total, (unsigned)(g->OC / kHaloBN)),
+                     dim3(64 * waves), lds, st, cv, ep);
   return check_launch("conv3x3_halo");
+}
+
+static int device_cus() {
+  int dev = 0, v = 0;
+  if (hipGetDevice(&dev) == hipSuccess &&
+      hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+    return v;
+  return 256;
 }
 
 } // namespace mi355x

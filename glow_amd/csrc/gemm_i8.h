@@ -305,11 +305,92 @@ __device__ __forceinline__ void load_col_raw(ColRaw (&c)[TN], const Epilogue &ep
   }
 }
 
+// The fused residual add / Relu on 16 staged output bytes; res16 points at the
+// 16 residual bytes of the same place (NULL: no residual). `fast`: every scale
+// small and no pre-shift in the stages that run.
+__device__ __forceinline__ bool fused_out_is_fast(const Epilogue &ep) {
+  return ep.add.small &&
+         (!ep.add.res || (ep.add.own_pre == 0 && ep.add.res_pre == 0)) &&
+         (!ep.add.relu || ep.add.dest_pre == 0);
+}
+__device__ __forceinline__ int4 fused_out_words(int4 v, const int8_t *res16, const Epilogue &ep,
+                                                const FusedAddConsts &fc, bool fast) {
+  if (res16 && fast) {
+    const int4 q = *reinterpret_cast<const int4 *>(res16);
+    v.x = (int)fused_word_fast<true>((uint32_t)v.x, (uint32_t)q.x, ep.add, fc);
+    v.y = (int)fused_word_fast<true>((uint32_t)v.y, (uint32_t)q.y, ep.add, fc);
+    v.z = (int)fused_word_fast<true>((uint32_t)v.z, (uint32_t)q.z, ep.add, fc);
+    v.w = (int)fused_word_fast<true>((uint32_t)v.w, (uint32_t)q.w, ep.add, fc);
+  } else if (!res16 && ep.add.relu && fast) {
+    v.x = (int)fused_word_fast<false>((uint32_t)v.x, 0u, ep.add, fc);
+    v.y = (int)fused_word_fast<false>((uint32_t)v.y, 0u, ep.add, fc);
+    v.z = (int)fused_word_fast<false>((uint32_t)v.z, 0u, ep.add, fc);
+    v.w = (int)fused_word_fast<false>((uint32_t)v.w, 0u, ep.add, fc);
+  } else if (res16) {
+    const int4 q = *reinterpret_cast<const int4 *>(res16);
+    v.x = (int)fused_add_word((uint32_t)v.x, (uint32_t)q.x, ep.add);
+    v.y = (int)fused_add_word((uint32_t)v.y, (uint32_t)q.y, ep.add);
+    v.z = (int)fused_add_word((uint32_t)v.z, (uint32_t)q.z, ep.add);
+    v.w = (int)fused_add_word((uint32_t)v.w, (uint32_t)q.w, ep.add);
+  } else if (ep.add.relu) {
+    v.x = (int)fused_relu_word((uint32_t)v.x, ep.add);
+    v.y = (int)fused_relu_word((uint32_t)v.y, ep.add);
+    v.z = (int)fused_relu_word((uint32_t)v.z, ep.add);
+    v.w = (int)fused_relu_word((uint32_t)v.w, ep.add);
+  }
+  return v;
+}
+
+// Copy-out of a staged int8 output tile (rows OUT_STRIDE = BN + 16 bytes apart
+// in LDS), with the fused residual add / Relu applied on the way: 16-byte row
+// segments where the output allows it. WAVE_ROWS: a wave copies out rows
+// [wm * WM, wm * WM + WM) of the tile, the ones its own lanes staged; otherwise
+// the block's THREADS threads share all rows.
+template <int BM, int BN, int WM, int THREADS, bool WAVE_ROWS>
+__device__ __forceinline__ void epilogue_copy_out(const int8_t *s_out, const Epilogue &ep, int M,
+                                                  int N, int m0, int n0, int n_base, int wm) {
+  constexpr int OUT_STRIDE = BN + 16;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int cols_here = min(BN, N - n0);
+  const int rows_here = min(BM, M - m0);
+  int8_t *obase = ep.out + (long long)m0 * ep.ldc + n_base + n0;
+  const bool vec_ok = (cols_here % 16 == 0) && (ep.ldc % 16 == 0) &&
+                      ((((uintptr_t)obase) & 15) == 0);
+  const int8_t *rbase =
+      ep.add.res ? ep.add.res + (long long)m0 * ep.ldc + n_base + n0 : nullptr;
+  // WAVE_ROWS: a wave copies out the rows it staged itself (first, step, end)
+  const int first = WAVE_ROWS ? lane : tid;
+  constexpr int STEP = WAVE_ROWS ? 64 : THREADS;
+  const int row_lo = WAVE_ROWS ? wm * WM : 0;
+  const int row_n = WAVE_ROWS ? max(0, min(WM, rows_here - row_lo)) : rows_here;
+  if (vec_ok && (!rbase || ((((uintptr_t)rbase) & 15) == 0))) {
+    const int segs = cols_here / 16;
+    // every scale small and no pre-shift in the stages that run
+    const bool fast = fused_out_is_fast(ep);
+    const FusedAddConsts fc = fused_add_consts(ep.add);
+    for (int c = first; c < row_n * segs; c += STEP) {
+      const int r = row_lo + c / segs, s = c % segs;
+      int4 v = *reinterpret_cast<const int4 *>(s_out + r * OUT_STRIDE + s * 16);
+      v = fused_out_words(v, rbase ? rbase + (long long)r * ep.ldc + s * 16 : nullptr, ep, fc, fast);
+      *reinterpret_cast<int4 *>(obase + (long long)r * ep.ldc + s * 16) = v;
+    }
+  } else {
+    for (int c = first; c < row_n * cols_here; c += STEP) {
+      const int r = row_lo + c / cols_here, s = c % cols_here;
+      int32_t v = s_out[r * OUT_STRIDE + s];
+      if (rbase) v = fused_add_one<false>(v, rbase[(long long)r * ep.ldc + s], ep.add);
+      else if (ep.add.relu) v = (int32_t)(int8_t)fused_relu_word_t<false>((uint32_t)v & 0xff, ep.add);
+      obase[(long long)r * ep.ldc + s] = (int8_t)v;
+    }
+  }
+}
+
 // Shared epilogue. Accumulator layout of v_mfma_i32_32x32x32_i8: lane l holds
 // column l % 32 and, in register r, row 8*(r/4) + 4*(l/32) + r%4 of the tile.
 // Must be entered after a block barrier (LDS is reused).
 template <int BM, int BN, int WM, int WN, bool NEED_SA, bool NEED_SB,
-          bool LEAKY, int FAST = 0>
+          bool LEAKY, int FAST = 0, bool WAVE_ROWS = false>
 __device__ __forceinline__ void gemm_epilogue_impl(
     v16i (&acc)[WM / 32][WN / 32], int (&sa)[WM / 32], int (&sb)[WN / 32],
     int8_t *lds, const Epilogue &ep, int M, int N, int K, int m0, int n0,
@@ -406,81 +487,36 @@ __device__ __forceinline__ void gemm_epilogue_impl(
       }
     }
   }
-  __syncthreads();
-
-  // coalesced copy-out: 16-byte row segments where the output allows it
-  const int cols_here = min(BN, N - n0);
-  const int rows_here = min(BM, M - m0);
-  int8_t *obase = ep.out + (long long)m0 * ep.ldc + n_base + n0;
-  const bool vec_ok = (cols_here % 16 == 0) && (ep.ldc % 16 == 0) &&
-                      ((((uintptr_t)obase) & 15) == 0);
-  const int8_t *rbase =
-      ep.add.res ? ep.add.res + (long long)m0 * ep.ldc + n_base + n0 : nullptr;
-  if (vec_ok && (!rbase || ((((uintptr_t)rbase) & 15) == 0))) {
-    const int segs = cols_here / 16;
-    // every scale small and no pre-shift in the stages that run
-    const bool fast =
-        ep.add.small &&
-        (!rbase || (ep.add.own_pre == 0 && ep.add.res_pre == 0)) &&
-        (!ep.add.relu || ep.add.dest_pre == 0);
-    const FusedAddConsts fc = fused_add_consts(ep.add);
-    for (int c = tid; c < rows_here * segs; c += THREADS) {
-      const int r = c / segs, s = c - r * segs;
-      int4 v = *reinterpret_cast<const int4 *>(s_out + r * OUT_STRIDE + s * 16);
-      if (rbase && fast) {
-        const int4 q =
-            *reinterpret_cast<const int4 *>(rbase + (long long)r * ep.ldc + s * 16);
-        v.x = (int)fused_word_fast<true>((uint32_t)v.x, (uint32_t)q.x, ep.add, fc);
-        v.y = (int)fused_word_fast<true>((uint32_t)v.y, (uint32_t)q.y, ep.add, fc);
-        v.z = (int)fused_word_fast<true>((uint32_t)v.z, (uint32_t)q.z, ep.add, fc);
-        v.w = (int)fused_word_fast<true>((uint32_t)v.w, (uint32_t)q.w, ep.add, fc);
-      } else if (!rbase && ep.add.relu && fast) {
-        v.x = (int)fused_word_fast<false>((uint32_t)v.x, 0u, ep.add, fc);
-        v.y = (int)fused_word_fast<false>((uint32_t)v.y, 0u, ep.add, fc);
-        v.z = (int)fused_word_fast<false>((uint32_t)v.z, 0u, ep.add, fc);
-        v.w = (int)fused_word_fast<false>((uint32_t)v.w, 0u, ep.add, fc);
-      } else if (rbase) {
-        const int4 q =
-            *reinterpret_cast<const int4 *>(rbase + (long long)r * ep.ldc + s * 16);
-        v.x = (int)fused_add_word((uint32_t)v.x, (uint32_t)q.x, ep.add);
-        v.y = (int)fused_add_word((uint32_t)v.y, (uint32_t)q.y, ep.add);
-        v.z = (int)fused_add_word((uint32_t)v.z, (uint32_t)q.z, ep.add);
-        v.w = (int)fused_add_word((uint32_t)v.w, (uint32_t)q.w, ep.add);
-      } else if (ep.add.relu) {
-        v.x = (int)fused_relu_word((uint32_t)v.x, ep.add);
-        v.y = (int)fused_relu_word((uint32_t)v.y, ep.add);
-        v.z = (int)fused_relu_word((uint32_t)v.z, ep.add);
-        v.w = (int)fused_relu_word((uint32_t)v.w, ep.add);
-      }
-      *reinterpret_cast<int4 *>(obase + (long long)r * ep.ldc + s * 16) = v;
-    }
+  if constexpr (WAVE_ROWS) {
+    // a wave reads back only what its own lanes wrote: LDS serves one wave's
+    // accesses in order, so the compiler is all that has to be held back
+    static_assert(BN == WN && !NEED_SA, "a wave must own whole rows of the tile");
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   } else {
-    for (int c = tid; c < rows_here * cols_here; c += THREADS) {
-      const int r = c / cols_here, s = c - r * cols_here;
-      int32_t v = s_out[r * OUT_STRIDE + s];
-      if (rbase) v = fused_add_one<false>(v, rbase[(long long)r * ep.ldc + s], ep.add);
-      else if (ep.add.relu) v = (int32_t)(int8_t)fused_relu_word_t<false>((uint32_t)v & 0xff, ep.add);
-      obase[(long long)r * ep.ldc + s] = (int8_t)v;
-    }
+    __syncthreads();
   }
+
+  epilogue_copy_out<BM, BN, WM, THREADS, WAVE_ROWS>(s_out, ep, M, N, m0, n0, n_base, wm);
 }
 
-template <int BM, int BN, int WM, int WN, bool NEED_SA, bool NEED_SB>
+template <int BM, int BN, int WM, int WN, bool NEED_SA, bool NEED_SB, bool WAVE_ROWS = false>
 __device__ __forceinline__ void gemm_epilogue(
     v16i (&acc)[WM / 32][WN / 32], int (&sa)[WM / 32], int (&sb)[WN / 32],
     int8_t *lds, const Epilogue &ep, int M, int N, int K, int m0, int n0,
     int n_base, const ColRaw (&col)[WN / 32]) {
   if (ep.act == 5) // LEAKY_RELU: rare, kept out of the common instruction stream
-    gemm_epilogue_impl<BM, BN, WM, WN, NEED_SA, NEED_SB, true>(
+    gemm_epilogue_impl<BM, BN, WM, WN, NEED_SA, NEED_SB, true, 0, WAVE_ROWS>(
         acc, sa, sb, lds, ep, M, N, K, m0, n0, n_base, col);
   else if ((ep.fast & 3) == 3)
-    gemm_epilogue_impl<BM, BN, WM, WN, NEED_SA, NEED_SB, false, 2>(
+    gemm_epilogue_impl<BM, BN, WM, WN, NEED_SA, NEED_SB, false, 2, WAVE_ROWS>(
         acc, sa, sb, lds, ep, M, N, K, m0, n0, n_base, col);
   else if (ep.fast & 1)
-    gemm_epilogue_impl<BM, BN, WM, WN, NEED_SA, NEED_SB, false, 1>(
+    gemm_epilogue_impl<BM, BN, WM, WN, NEED_SA, NEED_SB, false, 1, WAVE_ROWS>(
         acc, sa, sb, lds, ep, M, N, K, m0, n0, n_base, col);
   else
-    gemm_epilogue_impl<BM, BN, WM, WN, NEED_SA, NEED_SB, false>(
+    gemm_epilogue_impl<BM, BN, WM, WN, NEED_SA, NEED_SB, false, 0, WAVE_ROWS>(
         acc, sa, sb, lds, ep, M, N, K, m0, n0, n_base, col);
 }
 

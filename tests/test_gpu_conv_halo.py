@@ -41,10 +41,14 @@ class forced_tile:
 HALO_CASES = [
     dict(N=2, H=56, W=56, OC=64),                               # the ResNet layer shape
     dict(N=3, H=13, W=9, OC=64),                                # tiles that end inside an image
-    dict(N=1, H=5, W=130, OC=128, pads=(1, 1, 1, 1)),           # a row longer than a tile
+    dict(N=1, H=5, W=130, OC=128, pads=(1, 1, 1, 1)),           # one row per tile, five waves
     dict(N=2, H=20, W=20, OC=192, pads=(0, 0, 0, 0)),           # no padding: output 18x18
     dict(N=2, H=11, W=12, OC=64, pads=(2, 0, 1, 3)),            # uneven padding
     dict(N=1, H=3, W=3, OC=64, pads=(1, 1, 1, 1)),              # a single small tile
+    dict(N=1, H=4, W=256, OC=64),                               # the widest row the kernel takes
+    dict(N=1, H=3, W=257, OC=64),                               # wider: the implicit GEMM serves it
+    dict(N=2, H=300, W=1, OC=64),                               # tall and thin: 256 rows per tile
+    dict(N=300, H=9, W=9, OC=64),                               # more tiles than resident workgroups
     dict(N=5, H=7, W=7, OC=128, in_offset=0, act=go.ACT_NONE),  # no input offset, no row sums used
     dict(N=1, H=28, W=28, OC=64, in_offset=7, out_offset=5, act=go.ACT_CLIP),
     dict(N=1, H=16, W=16, OC=64, act=go.ACT_LEAKY_RELU, out_offset=10, bias_i8=True),
