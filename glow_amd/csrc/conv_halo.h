@@ -56,88 +56,14 @@ constexpr size_t kHaloMaxLds =
     kHaloFilterBytes + 5 * kHaloBN * 4 + (size_t)3 * (kHaloMaxPix + 2) * kHaloPix;
 constexpr int kHaloFilterChunks = kHaloBN * (kHaloK / 16);   // 16-byte chunks
 
-// Per-channel requantisation constants of a workgroup's 64 output channels, in
-// LDS as five arrays of 64 ints: in the accumulator layout used here a lane
-// holds 32 different channels, so it reads them (four consecutive channels per
-// ds_read_b128, the same address across half a wave) instead of keeping them.
-enum { kParColc = 0, kParPre = 1, kParScale = 2, kParPost = 3, kParFold = 4, kParArrays = 5 };
-constexpr int kHaloParBytes = kParArrays * kHaloBN * 4;
-
 // Filter row (output channel) c of a workgroup's 64 sits in LDS slot
-// halo_filter_slot(c): matrix-core row 8 q + 4 h + i of channel tile j holds
-// channel 32 h + 16 j + 4 q + i, so that lane (pixel, h) ends up with channels
-// 32 h + 16 j + [0, 16) of its pixel in the sixteen accumulators of tile j, in
-// order: sixteen consecutive output bytes.
+// halo_filter_slot(c), the inverse of perm_row16 within each 32-channel tile:
+// lane (pixel, h) then holds channels 32 j + 16 h + [0, 16) of its pixel in
+// the sixteen accumulators of tile j, in order (see gemm_i8.h).
 __device__ __forceinline__ int halo_filter_slot(int c) {
-  return 32 * ((c >> 4) & 1) + 8 * ((c >> 2) & 3) + 4 * (c >> 5) + (c & 3);
+  return (c & 32) + 8 * ((c >> 2) & 3) + 4 * ((c >> 4) & 1) + (c & 3);
 }
-
-// Requantises a lane's 2 x 16 accumulators (pixel l % 32, channels
-// 32 (l / 32) + 16 j + r for register r of tile j) and writes them as two
-// 16-byte stores straight from registers; `out` points at the pixel's 64
-// channels (NULL: the lane's pixel lies past the tile), `res` at the residual's.
-// MODE 0: scale_i32; 1: 24-bit multiply with pre-shift; 3: 24-bit multiply,
-// no pre-shift, column constant folded (the caller's requantisation hints).
-template <int MODE, bool LEAKY>
-__device__ __forceinline__ void halo_requant_store(const v16i (&acc)[2], const int32_t *s_par,
-                                                   const Epilogue &ep, int lhi, int8_t *out,
-                                                   const int8_t *res) {
-  int32_t lo = -128, hi = 127;
-  if (ep.act == 1) lo = clip_i8(ep.out_off);
-  if (ep.act == 2) {
-    lo = clip_i8(ep.a0);
-    hi = clip_i8(ep.a1);
-    if (lo > hi) lo = hi;
-  }
-  const bool fast = fused_out_is_fast(ep);
-  const FusedAddConsts fc = fused_add_consts(ep.add);
-#pragma unroll
-  for (int j = 0; j < 2; j++) {
-    const int cbase = 32 * lhi + 16 * j;
-    uint32_t w[4];
-#pragma unroll
-    for (int q = 0; q < 4; q++) {
-      const int ch = cbase + 4 * q;
-      const v4i scale = *reinterpret_cast<const v4i *>(s_par + kParScale * kHaloBN + ch);
-      const v4i post = *reinterpret_cast<const v4i *>(s_par + kParPost * kHaloBN + ch);
-      v4i colc, pre, fold;
-      if constexpr (MODE != 3) {
-        colc = *reinterpret_cast<const v4i *>(s_par + kParColc * kHaloBN + ch);
-        pre = *reinterpret_cast<const v4i *>(s_par + kParPre * kHaloBN + ch);
-      }
-      if constexpr (MODE != 0) fold = *reinterpret_cast<const v4i *>(s_par + kParFold * kHaloBN + ch);
-      uint32_t b[4];
-#pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const uint32_t x = (uint32_t)acc[j][4 * q + i];
-        int32_t y;
-        if constexpr (MODE == 3) {
-          y = (int32_t)((uint32_t)__mul24((int32_t)x, scale[i]) + (uint32_t)fold[i]) >> post[i];
-        } else if constexpr (MODE == 1) {
-          y = (int32_t)((uint32_t)__mul24((int32_t)(x + (uint32_t)colc[i]) >> pre[i], scale[i]) +
-                        (uint32_t)fold[i]) >> post[i];
-        } else {
-          y = scale_i32((int32_t)(x + (uint32_t)colc[i]), pre[i], post[i], scale[i], ep.out_off);
-        }
-        if constexpr (LEAKY) {
-          if (y < ep.out_off)
-            y = scale_i32((int32_t)((uint32_t)y - (uint32_t)ep.out_off), ep.a0, ep.a1, ep.a2,
-                          ep.out_off);
-        }
-        b[i] = (uint32_t)med3_i32(y, lo, hi);
-      }
-      // low bytes of four registers -> one word
-      const uint32_t w01 = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);
-      const uint32_t w23 = __builtin_amdgcn_perm(b[3], b[2], 0x0c0c0400u);
-      w[q] = __builtin_amdgcn_perm(w23, w01, 0x05040100u);
-    }
-    if (out) {
-      int4 v = make_int4((int)w[0], (int)w[1], (int)w[2], (int)w[3]);
-      v = fused_out_words(v, res ? res + cbase : nullptr, ep, fc, fast);
-      *reinterpret_cast<int4 *>(out + cbase) = v;
-    }
-  }
-}
+constexpr int kHaloParBytes = kParArrays * kHaloBN * 4;
 
 // SKIP leaves phases out so that the others can be timed (1: staging, 2: the
 // matrix-core loop, 4: requantisation and copy-out); the library uses 0.
@@ -160,7 +86,7 @@ __global__ __launch_bounds__(512, 2) void conv3x3_halo_kernel(HaloConv cv, Epilo
   const int rows = min(cv.rows, cv.OH - oh_first);
   const int npix = rows * cv.OW;
   const int hw = cv.OW + 2;                   // halo pixels per row
-  const int mode = ep.act == 5 ? 0 : ep.fast & 3;
+  const int mode = requant_mode(ep);
 
   // the channels' raw parameters, requested first (by the last wave: the first
   // ones carry the staging loop's remainders)
@@ -232,29 +158,15 @@ __global__ __launch_bounds__(512, 2) void conv3x3_halo_kernel(HaloConv cv, Epilo
   }
 
   // ---- the channels' requantisation constants -> LDS --------------------------------
-  if (par_wave) {
-    const ColRaw &c = col[0];
-    uint32_t colc = (uint32_t)kHaloK * (uint32_t)ep.a_off * (uint32_t)c.woff;
-    if (ep.sum_b) colc -= (uint32_t)ep.a_off * (uint32_t)c.sumb;
-    if (ep.bias)
-      colc += (uint32_t)scale_i32((int32_t)((uint32_t)c.bias - (uint32_t)c.boff), c.bpre,
-                                  c.bpost, c.bscale, 0);
-    uint32_t fold = (c.opost > 0 ? (1u << (c.opost - 1)) : 0u) + ((uint32_t)ep.out_off << c.opost);
-    if (mode == 3) fold += colc * (uint32_t)c.oscale;
-    s_par[kParColc * kHaloBN + lane] = (int32_t)colc;
-    s_par[kParPre * kHaloBN + lane] = c.opre;
-    s_par[kParScale * kHaloBN + lane] = c.oscale;
-    s_par[kParPost * kHaloBN + lane] = c.opost;
-    s_par[kParFold * kHaloBN + lane] = (int32_t)fold;
-  }
+  if (par_wave) par_table_store<kHaloBN>(s_par, lane, col[0], ep, kHaloK, mode);
   __syncthreads();
 
   // ---- nine taps x two 32-byte k slices -------------------------------------------
-  v16i acc[2];
+  v16i acc[1][2];
 #pragma unroll
   for (int j = 0; j < 2; j++)
 #pragma unroll
-    for (int r = 0; r < 16; r++) acc[j][r] = (SKIP & 2) ? tid + r : 0;
+    for (int r = 0; r < 16; r++) acc[0][j][r] = (SKIP & 2) ? tid + r : 0;
   if constexpr (!(SKIP & 2)) {
     // this lane's pixel (lanes past the tile's end recompute its last pixel;
     // the copy-out does not store them)
@@ -276,26 +188,22 @@ __global__ __launch_bounds__(512, 2) void conv3x3_halo_kernel(HaloConv cv, Epilo
           const v4i b0 = *reinterpret_cast<const v4i *>(b_base + kb);
           const v4i b1 = *reinterpret_cast<const v4i *>(b_base + 32 * kHaloFRow + kb);
           // filter rows first: the result's rows are channels, its columns pixels
-          acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b0, af, acc[0], 0, 0, 0);
-          acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b1, af, acc[1], 0, 0, 0);
+          acc[0][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b0, af, acc[0][0], 0, 0, 0);
+          acc[0][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b1, af, acc[0][1], 0, 0, 0);
         }
       }
     }
   }
   // no barrier: the waves finish on their own, nothing in LDS is reused
   if constexpr (!(SKIP & 4)) {
-    const int p = wave * 32 + l32;
-    const long long m = (long long)(n * cv.OH + oh_first) * cv.OW + p;
-    int8_t *out = p < npix ? ep.out + m * ep.ldc + n0 : nullptr;
-    const int8_t *res = ep.add.res ? ep.add.res + m * ep.ldc + n0 : nullptr;
-    if (ep.act == 5) halo_requant_store<0, true>(acc, s_par, ep, lhi, out, res);
-    else if (mode == 3) halo_requant_store<3, false>(acc, s_par, ep, lhi, out, res);
-    else if (mode & 1) halo_requant_store<1, false>(acc, s_par, ep, lhi, out, res);
-    else halo_requant_store<0, false>(acc, s_par, ep, lhi, out, res);
+    // rows past the tile's end belong to the next tile (or image): M bounds them
+    const int m0 = (n * cv.OH + oh_first) * cv.OW;
+    gemm_epilogue_direct<kHaloBN, 32, 64>(acc, s_par, ep, m0 + npix, cv.OC, m0, n0, 0, wave, 0,
+                                          l32, lhi);
   } else {
     int x = 0;
 #pragma unroll
-    for (int r = 0; r < 16; r++) x += acc[0][r] ^ acc[1][r];
+    for (int r = 0; r < 16; r++) x += acc[0][0][r] ^ acc[0][1][r];
     if (x == 0x12345678) ep.out[tid] = (int8_t)x;
   }
 }

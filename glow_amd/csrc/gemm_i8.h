@@ -34,6 +34,7 @@
 #include "requant.h"
 
 #include <atomic>
+#include <type_traits>
 
 namespace mi355x {
 
@@ -384,6 +385,189 @@ __device__ __forceinline__ void epilogue_copy_out(const int8_t *s_out, const Epi
       obase[(long long)r * ep.ldc + s] = (int8_t)v;
     }
   }
+}
+
+// f(std::integral_constant<int, I>) for I in [I0, N): a loop whose index is a
+// compile-time constant in the body whatever the unroller decides.
+template <int I, int N, class F> __device__ __forceinline__ void static_for(F &&f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
+
+// ---- requantisation from transposed accumulators ---------------------------------
+// With the weights as the first matrix-core operand, lane l of a 32x32 result
+// holds output row (pixel) l % 32 and, in register r, weight row
+// 8 (r / 4) + 4 (l / 32) + r % 4 of the 32-row sub-tile. When the weight row that
+// feeds matrix-core row rho is perm_row16(rho), register r of lane half h is
+// output column 16 h + r: the sixteen accumulators of a lane are sixteen
+// consecutive output bytes, requantised, packed and written with one 16-byte
+// store straight from registers (no staging in LDS, no barrier).
+__device__ __forceinline__ int perm_row16(int rho) {
+  return 16 * ((rho >> 2) & 1) + 4 * (rho >> 3) + (rho & 3);
+}
+
+// A lane then needs the constants of 16 columns per sub-tile instead of one
+// column's: they are kept in LDS as kParArrays arrays of BN ints (four
+// consecutive columns per ds_read_b128, one address per half wave).
+enum { kParColc = 0, kParPre = 1, kParScale = 2, kParPost = 3, kParFold = 4, kParArrays = 5 };
+
+// Requantisation variants: 0 scale_i32; 1 the 24-bit multiply with pre-shift;
+// 3 the 24-bit multiply without pre-shift and with the column constant folded
+// (the caller's requantisation hints); LEAKY_RELU always takes 0.
+__device__ __forceinline__ int requant_mode(const Epilogue &ep) {
+  return ep.act == 5 ? 0 : ((ep.fast & 3) == 3 ? 3 : (ep.fast & 1));
+}
+
+// Column c's constants from its raw parameters (the arithmetic of the shared
+// epilogue below).
+template <int BN>
+__device__ __forceinline__ void par_table_store(int32_t *s_par, int c, const ColRaw &r,
+                                                const Epilogue &ep, int K, int mode) {
+  uint32_t colc = (uint32_t)K * (uint32_t)ep.a_off * (uint32_t)r.woff;
+  if (ep.sum_b) colc -= (uint32_t)ep.a_off * (uint32_t)r.sumb;
+  if (ep.bias)
+    colc += (uint32_t)scale_i32((int32_t)((uint32_t)r.bias - (uint32_t)r.boff), r.bpre, r.bpost,
+                                r.bscale, 0);
+  uint32_t fold = (r.opost > 0 ? (1u << (r.opost - 1)) : 0u) + ((uint32_t)ep.out_off << r.opost);
+  if (mode == 3) fold += colc * (uint32_t)r.oscale;
+  s_par[kParColc * BN + c] = (int32_t)colc;
+  s_par[kParPre * BN + c] = r.opre;
+  s_par[kParScale * BN + c] = r.oscale;
+  s_par[kParPost * BN + c] = r.opost;
+  s_par[kParFold * BN + c] = (int32_t)fold;
+}
+
+// Sixteen accumulators -> sixteen output bytes (before the fused add); par
+// points at the first of the sixteen columns in the table.
+template <int MODE, bool LEAKY, int BN>
+__device__ __forceinline__ int4 requant_pack16(const v16i &acc, const int32_t *par,
+                                               const Epilogue &ep, int32_t lo, int32_t hi) {
+  uint32_t w[4];
+#pragma unroll
+  for (int q = 0; q < 4; q++) {
+    const v4i scale = *reinterpret_cast<const v4i *>(par + kParScale * BN + 4 * q);
+    const v4i post = *reinterpret_cast<const v4i *>(par + kParPost * BN + 4 * q);
+    v4i colc, pre, fold;
+    if constexpr (MODE != 3) {
+      colc = *reinterpret_cast<const v4i *>(par + kParColc * BN + 4 * q);
+      pre = *reinterpret_cast<const v4i *>(par + kParPre * BN + 4 * q);
+    }
+    if constexpr (MODE != 0) fold = *reinterpret_cast<const v4i *>(par + kParFold * BN + 4 * q);
+    uint32_t b[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const uint32_t x = (uint32_t)acc[4 * q + i];
+      int32_t y;
+      if constexpr (MODE == 3) {
+        y = (int32_t)((uint32_t)__mul24((int32_t)x, scale[i]) + (uint32_t)fold[i]) >> post[i];
+      } else if constexpr (MODE == 1) {
+        y = (int32_t)((uint32_t)__mul24((int32_t)(x + (uint32_t)colc[i]) >> pre[i], scale[i]) +
+                      (uint32_t)fold[i]) >> post[i];
+      } else {
+        y = scale_i32((int32_t)(x + (uint32_t)colc[i]), pre[i], post[i], scale[i], ep.out_off);
+      }
+      if constexpr (LEAKY) {
+        if (y < ep.out_off)
+          y = scale_i32((int32_t)((uint32_t)y - (uint32_t)ep.out_off), ep.a0, ep.a1, ep.a2,
+                        ep.out_off);
+      }
+      b[i] = (uint32_t)med3_i32(y, lo, hi);
+    }
+    // low bytes of four registers -> one word
+    const uint32_t w01 = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);
+    const uint32_t w23 = __builtin_amdgcn_perm(b[3], b[2], 0x0c0c0400u);
+    w[q] = __builtin_amdgcn_perm(w23, w01, 0x05040100u);
+  }
+  return make_int4((int)w[0], (int)w[1], (int)w[2], (int)w[3]);
+}
+
+// Activation and the final int8 clip as one clamp to [lo, hi]:
+// clip(min(max(y, a0), a1)) == min(max(y, clip(a0)), clip(a1)), RELU being
+// the clamp [out_off, +inf) and NONE the clamp (-inf, +inf).
+__device__ __forceinline__ void activation_clamp(const Epilogue &ep, int32_t &lo, int32_t &hi) {
+  lo = -128;
+  hi = 127;
+  if (ep.act == 1) lo = clip_i8(ep.out_off);
+  if (ep.act == 2) {
+    lo = clip_i8(ep.a0);
+    hi = clip_i8(ep.a1);
+    if (lo > hi) lo = hi; // min(max(y, lo), hi) is hi then; so is the median
+  }
+}
+
+// Writes sixteen requantised bytes of output row `out_row` (and residual row
+// res_row, or NULL) at column n of N: one 16-byte store where the addresses
+// allow it (vec) and the columns all exist, bytes otherwise.
+__device__ __forceinline__ void store16(int4 v, int8_t *out_row, const int8_t *res_row, int n,
+                                        int N, bool vec, const Epilogue &ep,
+                                        const FusedAddConsts &fc, bool fast) {
+  if (vec && n + 16 <= N) {
+    v = fused_out_words(v, res_row ? res_row + n : nullptr, ep, fc, fast);
+    *reinterpret_cast<int4 *>(out_row + n) = v;
+    return;
+  }
+  // (rare: kept as a rolled loop so that it stays small next to the fast path)
+#pragma unroll 1
+  for (int b = 0; b < 16; b++) {
+    if (n + b < N) {
+      const uint32_t word = (uint32_t)(b < 4 ? v.x : b < 8 ? v.y : b < 12 ? v.z : v.w);
+      int32_t x = (int32_t)(int8_t)(word >> (8 * (b & 3)));
+      if (res_row) x = fused_add_one<false>(x, res_row[n + b], ep.add);
+      else if (ep.add.relu) x = (int32_t)(int8_t)fused_relu_word_t<false>((uint32_t)x & 0xff, ep.add);
+      out_row[n + b] = (int8_t)x;
+    }
+  }
+}
+
+template <int BN, int WM, int WN, int MODE, bool LEAKY>
+__device__ __forceinline__ void gemm_epilogue_direct_impl(
+    v16i (&acc)[WM / 32][WN / 32], const int32_t *s_par, const Epilogue &ep, int M, int N,
+    int m0, int n0, int n_base, int wm, int wn, int l32, int lhi) {
+  constexpr int TM = WM / 32, TN = WN / 32;
+  int32_t lo, hi;
+  activation_clamp(ep, lo, hi);
+  const bool fast = fused_out_is_fast(ep);
+  const FusedAddConsts fc = fused_add_consts(ep.add);
+  const bool vec = (ep.ldc % 16 == 0) && ((n_base + n0) % 16 == 0) &&
+                   (((((uintptr_t)ep.out) | ((uintptr_t)ep.add.res)) & 15) == 0);
+  // (compile-time indices: the accumulators must stay in registers however
+  // large the unrolled body gets)
+  static_for<0, TM>([&](auto ic) {
+    constexpr int i = decltype(ic)::value;
+    const int m = m0 + wm * WM + i * 32 + l32;
+    int8_t *out_row = ep.out + (long long)m * ep.ldc + n_base;
+    const int8_t *res_row = ep.add.res ? ep.add.res + (long long)m * ep.ldc + n_base : nullptr;
+    static_for<0, TN>([&](auto jc) {
+      constexpr int j = decltype(jc)::value;
+      const int cl = wn * WN + j * 32 + 16 * lhi;   // column within the tile
+      const int4 v = requant_pack16<MODE, LEAKY, BN>(acc[i][j], s_par + cl, ep, lo, hi);
+      if (m < M) store16(v, out_row, res_row, n0 + cl, N, vec, ep, fc, fast);
+      // one sub-tile at a time: hoisting the next ones' table reads over this
+      // one's arithmetic costs more registers than the kernels have
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  });
+}
+
+template <int BN, int WM, int WN>
+__device__ __forceinline__ void gemm_epilogue_direct(
+    v16i (&acc)[WM / 32][WN / 32], const int32_t *s_par, const Epilogue &ep, int M, int N,
+    int m0, int n0, int n_base, int wm, int wn, int l32, int lhi) {
+  const int mode = requant_mode(ep);
+  if (ep.act == 5)
+    gemm_epilogue_direct_impl<BN, WM, WN, 0, true>(acc, s_par, ep, M, N, m0, n0, n_base, wm, wn,
+                                                   l32, lhi);
+  else if (mode == 3)
+    gemm_epilogue_direct_impl<BN, WM, WN, 3, false>(acc, s_par, ep, M, N, m0, n0, n_base, wm, wn,
+                                                    l32, lhi);
+  else if (mode == 1)
+    gemm_epilogue_direct_impl<BN, WM, WN, 1, false>(acc, s_par, ep, M, N, m0, n0, n_base, wm, wn,
+                                                    l32, lhi);
+  else
+    gemm_epilogue_direct_impl<BN, WM, WN, 0, false>(acc, s_par, ep, M, N, m0, n0, n_base, wm, wn,
+                                                    l32, lhi);
 }
 
 // Shared epilogue. Accumulator layout of v_mfma_i32_32x32x32_i8: lane l holds
