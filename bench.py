@@ -178,19 +178,27 @@ def make_slws_batches(capi, cases, args, count):
         batches.append(dict(
             lengths=lengths, idx=idx, w=w, total=int(lengths.sum()),
             d_len=capi.to_device(lengths), d_idx=capi.to_device(idx),
-            d_w=capi.to_device(w)))
+            d_w=capi.to_device(w),
+            d_off=capi.to_device(capi.slws_bag_offsets_host(lengths))))
     return batches
 
 
-def bench_slws(capi, args, d_table, batches, flush):
+def bench_slws(capi, args, d_table, batches, flush, bag_offsets=False):
     """Times args.steps launches that cycle through `batches`; `flush` (or None)
-    empties the caches before the timed replay."""
+    empties the caches before the timed replay. bag_offsets: the bags as the
+    positions a device manager derives from the lengths on the host
+    (mi355x_frwq_slws_offsets) instead of the lengths themselves."""
     rows, cols, bags = args.rows, 128, args.bags
     row_bytes = cols + 8
     d_out = capi.DeviceBuffer.empty((bags, cols), np.float32)
 
     def step(i, stream):
         b = batches[i % len(batches)]
+        if bag_offsets:
+            capi.launch_frwq_slws_offsets(d_out, False, d_table, rows, capi.FUSED_U8_F32,
+                                          b["d_w"], False, b["d_idx"], True, b["total"],
+                                          b["d_off"], bags, row_bytes, cols, stream=stream)
+            return
         capi.launch_frwq_slws(d_out, False, d_table, rows, capi.FUSED_U8_F32,
                               b["d_w"], False, b["d_idx"], True, b["total"],
                               b["d_len"], bags, row_bytes, cols, stream=stream)
@@ -788,6 +796,25 @@ def main():
             ms=ss["sec"] * 1e3, gbps=ss["bytes"] / ss["sec"] / 1e9,
             frac_of_hbm_peak=ss["bytes"] / ss["sec"] / 1e9 / HBM_PEAK_GBPS,
             bit_exact_with_oracle=bit_exact)
+        # the bags as positions (what the device manager hands over for lengths it
+        # uploads itself): no prefix sum in front of a bag's first index load
+        so = bench_slws(capi, args, d_table, batches, flush, bag_offsets=True)
+        same = None
+        if args.cpu_seconds > 0:
+            # against the lengths entry point on the same (last) batch, bit for bit
+            ref = capi.DeviceBuffer.empty((args.bags, 128), np.float32)
+            b = so["last"]
+            capi.launch_frwq_slws(ref, False, d_table, args.rows, capi.FUSED_U8_F32, b["d_w"],
+                                  False, b["d_idx"], True, b["total"], b["d_len"], args.bags,
+                                  136, 128)
+            capi.sync()
+            same = bool(np.array_equal(so["d_out"].numpy(), ref.numpy()))
+        extra["slws_bag_offsets"] = dict(
+            workload="headline lookup through mi355x_frwq_slws_offsets (bag positions "
+                     "precomputed on the host from the lengths), same batches, caches flushed",
+            ms=so["sec"] * 1e3, gbps=so["bytes"] / so["sec"] / 1e9,
+            frac_of_hbm_peak=so["bytes"] / so["sec"] / 1e9 / HBM_PEAK_GBPS,
+            ms_lengths_entry_point=s["sec"] * 1e3, equal_to_lengths_entry_point=same)
         extra["slws_with_h2d"] = bench_slws_with_h2d(capi, s, args, d_table)
         extra["slws_more_bags"] = [bench_slws_more_bags(capi, cases, args, d_table, n, flush)
                                    for n in (16384, 65536)]

@@ -45,6 +45,7 @@ EXPORTS = [
     "mi355x_cwq_conv2d_i8", "mi355x_conv2d_i8", "mi355x_frwq_slws",
     "mi355x_embedding_bag_rowwise_offsets",
     "mi355x_slws_reserve_stream", "mi355x_frwq_slws_noalloc",
+    "mi355x_frwq_slws_offsets", "mi355x_slws_bag_offsets_host",
     "mi355x_shader_clock_probe", "mi355x_wall_clock_khz",
     "mi355x_specialize_bias_qparams", "mi355x_channelwise_quantize_conv_host",
     "mi355x_gemm_requant_hint", "mi355x_gemm_requant_hint_host",
@@ -588,6 +589,28 @@ def launch_frwq_slws(dest, out_is_f16, data, data_rows, kind, weights,
         _vp(stream)))
 
 
+def launch_frwq_slws_offsets(dest, out_is_f16, data, data_rows, kind, weights,
+                             weights_are_f16, indices, idx_is_64, num_indices,
+                             bag_offsets, segments, in_line, out_line, fp16_accum=False,
+                             stream=None):
+    """mi355x_frwq_slws_offsets: bags by their segments + 1 positions."""
+    check(lib().mi355x_frwq_slws_offsets(
+        _vp(dest), C.c_int(bool(out_is_f16)), _vp(data), _sz(data_rows),
+        C.c_int(kind), _vp(weights), C.c_int(bool(weights_are_f16)),
+        _vp(indices), C.c_int(bool(idx_is_64)), _sz(num_indices), _vp(bag_offsets),
+        _sz(segments), _sz(in_line), _sz(out_line), C.c_int(bool(fp16_accum)),
+        _vp(stream)))
+
+
+def slws_bag_offsets_host(lengths):
+    """Exclusive prefix sums (segments + 1 int32) of the clamped lengths, made
+    by the library on the host."""
+    lengths = np.ascontiguousarray(lengths, np.int32)
+    out = np.empty(lengths.size + 1, np.int32)
+    check(lib().mi355x_slws_bag_offsets_host(_vp(lengths), _sz(lengths.size), _vp(out)))
+    return out
+
+
 # ---- numpy in / numpy out conveniences (tests, smoke) --------------------------
 
 def _geom(g):
@@ -811,10 +834,12 @@ def _fused_cols(in_line, kind):
 
 def frwq_slws(data, kind, weights, indices, lengths, out_f16=False,
               fp16_accum=False, d_data=None, row_pitch=None, stream=None,
-              noalloc=False):
+              noalloc=False, bag_offsets=False):
     """weights: None (plain SLS), float32 or float16 array. `d_data` lets a
     caller reuse a table already resident on the device. `row_pitch` lays the
-    table out with its rows that many bytes apart (the gaps hold junk)."""
+    table out with its rows that many bytes apart (the gaps hold junk).
+    `bag_offsets`: through mi355x_frwq_slws_offsets, with the positions that
+    mi355x_slws_bag_offsets_host makes of the lengths (or the array given)."""
     data_shape = data.shape
     in_line = data_shape[1]
     out_line = _fused_cols(in_line, kind)
@@ -843,10 +868,19 @@ def frwq_slws(data, kind, weights, indices, lengths, out_f16=False,
     d_out.fill(0xFF)  # poison: every row must be written by the kernel
     if stream is not None:
         sync()        # streams of this library do not wait for the default stream
-    launch_frwq_slws(d_out, out_f16, d_data, data_shape[0], kind, d_w, w16,
-                     d_idx, indices.dtype == np.int64, indices.size, d_len,
-                     lengths.size, in_line, out_line, fp16_accum, stream=stream,
-                     noalloc=noalloc)
+    if bag_offsets is not False:
+        offs = slws_bag_offsets_host(lengths) if bag_offsets is True else \
+            np.ascontiguousarray(bag_offsets, np.int32)
+        assert offs.size == lengths.size + 1
+        launch_frwq_slws_offsets(d_out, out_f16, d_data, data_shape[0], kind, d_w, w16,
+                                 d_idx, indices.dtype == np.int64, indices.size,
+                                 to_device(offs), lengths.size, in_line, out_line,
+                                 fp16_accum, stream=stream)
+    else:
+        launch_frwq_slws(d_out, out_f16, d_data, data_shape[0], kind, d_w, w16,
+                         d_idx, indices.dtype == np.int64, indices.size, d_len,
+                         lengths.size, in_line, out_line, fp16_accum, stream=stream,
+                         noalloc=noalloc)
     if stream is not None:
         stream.sync()
     return d_out.numpy()

@@ -1377,6 +1377,35 @@ int mi355x_frwq_slws_noalloc(void *dest, int out_is_f16, const uint8_t *data,
                        out_line_size, fp16_accum, stream, x);
 }
 
+int mi355x_frwq_slws_offsets(void *dest, int out_is_f16, const uint8_t *data,
+                             size_t data_rows, int kind, const void *weights,
+                             int weights_are_f16, const void *indices, int idx_is_64,
+                             size_t num_indices, const int32_t *bag_offsets,
+                             size_t segments, size_t in_line_size,
+                             size_t out_line_size, int fp16_accum, void *stream) {
+  MI355X_REQUIRE(segments == 0 || bag_offsets, "bag_offsets is NULL");
+  // segments + 1 offsets: every bag reads its two ends, no prefix sum, no
+  // scratch and no second launch whatever the number of bags
+  return slws_dispatch(dest, out_is_f16, data, data_rows, kind, weights,
+                       weights_are_f16, indices, idx_is_64, num_indices, nullptr,
+                       bag_offsets, 1, segments, in_line_size, out_line_size,
+                       fp16_accum, stream);
+}
+
+int mi355x_slws_bag_offsets_host(const int32_t *lengths, size_t segments,
+                                 int32_t *bag_offsets) {
+  MI355X_REQUIRE(bag_offsets && (segments == 0 || lengths), "NULL vector");
+  uint64_t sum = 0;
+  bag_offsets[0] = 0;
+  for (size_t i = 0; i < segments; i++) {
+    sum += lengths[i] > 0 ? (uint64_t)lengths[i] : 0u;   // as the kernels clamp
+    MI355X_REQUIRE(sum <= 0x7fffffffull,
+                   "the lengths sum past 2^31 - 1 at bag %zu: use the lengths entry point", i);
+    bag_offsets[i + 1] = (int32_t)sum;
+  }
+  return MI355X_OK;
+}
+
 int mi355x_slws_reserve_stream(void *stream) {
   return slws_reserve_stream(as_stream(stream));
 }

@@ -570,6 +570,31 @@ int mi355x_frwq_slws(void *dest, int out_is_f16, const uint8_t *data,
                      size_t segments, size_t in_line_size,
                      size_t out_line_size, int fp16_accum, void *stream);
 
+/* mi355x_frwq_slws with the bags given as positions instead of lengths: the
+ * same operator (libjit.cpp:1253-1276; InterpreterNodes.cpp:5764-5889) for a
+ * caller that holds the lengths on the host anyway (a device manager about to
+ * upload them) and hands their exclusive prefix sums along. bag_offsets has
+ * segments + 1 entries, bag i covering index positions
+ * [bag_offsets[i], bag_offsets[i + 1]); with the vector that
+ * mi355x_slws_bag_offsets_host makes of `lengths` the result is bit for bit
+ * that of mi355x_frwq_slws(lengths). A bag then reads its two ends instead of
+ * summing the lengths in front of it: no scratch, one launch for any number
+ * of bags. Ends outside [0, num_indices] or decreasing give short or empty
+ * bags, never a read outside the index list. */
+int mi355x_frwq_slws_offsets(void *dest, int out_is_f16, const uint8_t *data,
+                             size_t data_rows, int kind, const void *weights,
+                             int weights_are_f16, const void *indices, int idx_is_64,
+                             size_t num_indices, const int32_t *bag_offsets,
+                             size_t segments, size_t in_line_size,
+                             size_t out_line_size, int fp16_accum, void *stream);
+
+/* Host side, no GPU call: bag_offsets[0] = 0, bag_offsets[i + 1] =
+ * bag_offsets[i] + max(lengths[i], 0) (negative lengths count as empty bags,
+ * as in the kernels). Fails with MI355X_ERR_INVALID_ARGUMENT when the sum does
+ * not fit int32; such batches go through mi355x_frwq_slws. */
+int mi355x_slws_bag_offsets_host(const int32_t *lengths, size_t segments,
+                                 int32_t *bag_offsets);
+
 /* Scratch of the lengths-mode SparseLengths entry points (mi355x_frwq_slws,
  * mi355x_rwq_slws). With more than 4096 bags a small pre-pass sums the lengths
  * of each 4096-bag chunk into a 256 KiB buffer that belongs to the (device,

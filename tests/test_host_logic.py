@@ -181,3 +181,18 @@ def test_requant_hint_is_refused_when_24_bits_cannot_be_guaranteed():
     assert capi.gemm_requant_hint_host(64, 0, 0, None, bias, 0, zero, zero, one, zero, post, sc) == 0
     with pytest.raises(capi.MI355XError):
         capi.check(capi.lib().mi355x_gemm_requant_hint(2))
+
+
+def test_slws_bag_offsets_host():
+    """Exclusive prefix sums of the clamped lengths; sums past int32 are refused."""
+    rng = np.random.default_rng(3)
+    lengths = rng.integers(-3, 50, 5000).astype(np.int32)
+    offs = capi.slws_bag_offsets_host(lengths)
+    want = np.r_[0, np.cumsum(np.maximum(lengths, 0))]
+    np.testing.assert_array_equal(offs, want)
+    assert offs.dtype == np.int32 and offs.size == lengths.size + 1
+    np.testing.assert_array_equal(capi.slws_bag_offsets_host(np.zeros(0, np.int32)), [0])
+    big = np.full(3, 2**30, np.int32)
+    with pytest.raises(capi.MI355XError):
+        capi.slws_bag_offsets_host(big)
+    np.testing.assert_array_equal(capi.slws_bag_offsets_host(big[:1]), [0, 2**30])
