@@ -1162,14 +1162,15 @@ def space_to_depth2_i8(x, pad_t, pad_l, bh, bw, cout, fill):
 class SlsTable(C.Structure):
     """mi355x_sls_table: one table of a multi-table pooled lookup."""
     _fields_ = [("data", C.c_void_p), ("indices", C.c_void_p), ("lengths", C.c_void_p),
-                ("dest", C.c_void_p), ("data_rows", C.c_uint64), ("num_indices", C.c_uint64)]
+                ("dest", C.c_void_p), ("data_rows", C.c_uint64), ("num_indices", C.c_uint64),
+                ("bag_offsets", C.c_void_p)]
 
 
 SLS_OUT_F32, SLS_OUT_F16, SLS_OUT_I8, SLS_OUT_I8_VIA_F16 = range(4)
 
 
 def frwq_sls_multi(tables, kind, indices, lengths, out_kind=SLS_OUT_F32, out_scale=1.0,
-                   out_offset=0, fp16_accum=False):
+                   out_offset=0, fp16_accum=False, bag_offsets=False):
     """tables, indices, lengths: equally long lists (one entry per table; tables
     of one shape, indices of one dtype). Dense output kinds return a list of
     [bags x cols] arrays; the int8 kinds return the concatenation
@@ -1194,10 +1195,12 @@ def frwq_sls_multi(tables, kind, indices, lengths, out_kind=SLS_OUT_F32, out_sca
         outs = [DeviceBuffer.empty((bags, cols), dt) for _ in range(n)]
         dests = [o.ptr for o in outs]
         stride = 0
+    # bag_offsets: every table's bags as host-made positions instead of lengths
+    d_o = [to_device(slws_bag_offsets_host(l)) for l in lengths] if bag_offsets else None
     arr = (SlsTable * n)()
     for t in range(n):
         arr[t] = SlsTable(d_t[t].ptr, d_i[t].ptr, d_l[t].ptr, dests[t], tabs[t].shape[0],
-                          idx[t].size)
+                          idx[t].size, d_o[t].ptr if bag_offsets else None)
     d_arr = DeviceBuffer(C.sizeof(arr))
     check(lib().mi355x_memcpy_h2d(_vp(d_arr), C.byref(arr), _sz(C.sizeof(arr)), _vp(None)))
     sync()

@@ -87,6 +87,8 @@ __device__ __forceinline__ void select_table(SlwsArgs &a) {
     a.data = t.data;
     a.indices = t.indices;
     a.lengths = t.lengths;
+    a.offsets = t.bag_offsets;
+    a.offsets_have_end = 1;
     a.dest = t.dest;
     a.data_rows = (int64_t)t.data_rows;
     a.num_indices = (int64_t)t.num_indices;

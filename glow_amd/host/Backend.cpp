@@ -1530,6 +1530,12 @@ private:
     for (const auto &c : group) views.push_back(tableView(c.data, c.rows, c.inLine, out));
     const size_t pitch = views[0].pitch;
     auto tabPtr = scratchPtr(gen_.addScratch(n * sizeof(mi355x_sls_table)));
+    std::vector<std::function<uint8_t *(const DeviceBindings &)>> offs;
+    size_t nDerived = 0;
+    for (const auto &c : group) {
+      offs.push_back(derivedOffsets(c.len, out));
+      nDerived += offs.back() ? 1 : 0;
+    }
     const size_t stride = (size_t)g.dest.ty().dims[1];
     const std::string name = insts_[at].name + (n > 1 ? "..." + insts_[pos - 1].name : "");
     // the table array holds device addresses: written once the buffers are bound
@@ -1543,6 +1549,7 @@ private:
                              t[i].dest = group[i].dest.ptr(b) + group[i].colOffset;
                              t[i].data_rows = group[i].rows;
                              t[i].num_indices = group[i].nIdx;
+                             t[i].bag_offsets = offs[i] ? (const int32_t *)offs[i](b) : nullptr;
                            }
                            int rc = mi355x_memcpy_h2d(tabPtr(b), t.data(), n * sizeof(mi355x_sls_table),
                                                       b.stream);
@@ -1556,13 +1563,35 @@ private:
                    pitch, g.cols, g.segs, stride) +
              kv("kind", g.kind) + kv("idx_is_64", g.idx64) + kv("out_kind", outKind) +
              strFormat(" out_scale=%.9g", (double)g.qScale) + kv("out_offset", g.qOffset) +
-             kv("fp16_accum", g.acc16),
+             kv("fp16_accum", g.acc16) + kv("bag_offsets_from_host", (long long)nDerived),
          [=](const DeviceBindings &b) {
            return mi355x_frwq_sls_multi((const mi355x_sls_table *)tabPtr(b), n, maxRows, g.kind, g.idx64,
                                         g.segs, pitch, g.cols, outKind, g.qScale, g.qOffset, stride,
                                         g.acc16, b.stream);
          }});
     return pos - at;
+  }
+
+  // The bag positions of a lookup whose lengths are an input of the function
+  // (a placeholder no instruction writes): a scratch vector the device manager
+  // fills when it uploads the lengths. Empty function: read the lengths.
+  std::function<uint8_t *(const DeviceBindings &)> derivedOffsets(const Operand &len,
+                                                                 MI355XFunction &out) {
+    if (!opts_.deriveBagOffsets || len.v->category != SymbolCategory::Placeholder ||
+        len.v->id != len.v->root)
+      return nullptr;
+    auto w = io_.find(len.v->id);
+    if (w != io_.end() && w->second.second) return nullptr; // written on the device
+    auto it = derived_.find(len.v->id);
+    if (it != derived_.end()) return out.derivedBagOffsets[it->second].ptr;
+    const size_t segs = (size_t)len.ty().size();
+    MI355XFunction::DerivedBagOffsets d;
+    d.lengths = len.v->name;
+    d.segments = segs;
+    d.ptr = scratchPtr(gen_.addScratch((segs + 1) * sizeof(int32_t)));
+    derived_[len.v->id] = out.derivedBagOffsets.size();
+    out.derivedBagOffsets.push_back(d);
+    return d.ptr;
   }
 
   Error slws(const Instruction &I, MI355XFunction &out, bool weighted) {
@@ -1608,6 +1637,22 @@ private:
     const int idx64 = idx.ty().kind == ElemKind::Int64ITy;
     const TableView table = tableView(data, rows, inLine, out);
     const size_t pitch = table.pitch;
+    if (auto offs = derivedOffsets(len, out)) {
+      out.launches.push_back(
+          {"mi355x_frwq_slws_offsets", I.name,
+           strFormat(" rows=%zu in_line=%zu out_line=%zu segments=%zu num_indices=%zu", rows, pitch,
+                     outLine, segs, nIdx) +
+               kv("kind", kind) + kv("out_is_f16", out16) + kv("weighted", weighted) +
+               kv("weights_are_f16", w16) + kv("idx_is_64", idx64) + kv("fp16_accum", acc16) +
+               " bag_offsets=host(" + len.v->name + ")",
+           [=](const DeviceBindings &b) {
+             return mi355x_frwq_slws_offsets(d.ptr(b), out16, table.ptr(b), rows, kind,
+                                             weighted ? (const void *)w.ptr(b) : nullptr, w16,
+                                             idx.ptr(b), idx64, nIdx, (const int32_t *)offs(b), segs,
+                                             pitch, outLine, acc16 ? 1 : 0, b.stream);
+           }});
+      return Error::success();
+    }
     out.launches.push_back(
         {"mi355x_frwq_slws", I.name,
          strFormat(" rows=%zu in_line=%zu out_line=%zu segments=%zu num_indices=%zu", rows, pitch,
@@ -1632,6 +1677,7 @@ private:
   std::shared_ptr<size_t> scratchBasePtr_ = std::make_shared<size_t>(0);
   std::map<int, std::pair<bool, bool>> io_; // value id -> (read, written)
   std::map<const Value *, TableView> paddedTables_;
+  std::map<int, size_t> derived_; // lengths value id -> index in derivedBagOffsets
   std::vector<char> absorbed_; // instructions folded into the launch of an earlier one
 };
 
@@ -1873,6 +1919,16 @@ Error MI355XFunction::execute(ExecutionContext *ctx) {
                              "%s (%s): %s", l.kernel.c_str(), l.inst.c_str(), mi355x_last_error());
   }
   return Error::success();
+}
+
+std::vector<int32_t> MI355XFunction::bagOffsets(const int32_t *lengths, size_t n, size_t segments) {
+  std::vector<int32_t> o(segments + 1, 0);
+  int64_t sum = 0;
+  for (size_t i = 0; i < segments; i++) {
+    if (i < n && lengths[i] > 0) sum = std::min<int64_t>(sum + lengths[i], 0x7fffffff);
+    o[i + 1] = (int32_t)sum;
+  }
+  return o;
 }
 
 std::string MI355XFunction::describe() const {

@@ -130,6 +130,20 @@ public:
   std::vector<KernelLaunch> setup, launches;
   // Host image of the generated constants (uploaded by the device manager).
   std::vector<uint8_t> generated;
+  // Lookups whose lengths are an input placeholder read their bags as
+  // positions: whoever uploads `lengths` also writes segments + 1 int32
+  // exclusive prefix sums of the (clamped) lengths to ptr(bindings).
+  struct DerivedBagOffsets {
+    std::string lengths; // placeholder name
+    size_t segments = 0;
+    std::function<uint8_t *(const DeviceBindings &)> ptr;
+  };
+  std::vector<DerivedBagOffsets> derivedBagOffsets;
+  // Host side of that contract: the positions for `lengths` (n of the
+  // placeholder's `segments` entries given; the missing ones count as empty
+  // bags). Sums saturate at INT32_MAX, which lies at or past the end of any
+  // index list, where the kernels clamp positions anyway.
+  static std::vector<int32_t> bagOffsets(const int32_t *lengths, size_t n, size_t segments);
   // Text listing of the launches with their parameters.
   std::string describe() const;
 
@@ -157,6 +171,7 @@ struct BackendOptions {
   bool padTableRows = true;            // constant lookup tables with 33..63-byte rows re-laid 64 bytes apart at load
   bool fuseInsert = true;              // Gather / RescaleQuantized write straight into the tensor their result is inserted into
   bool fuseDequantizeSigmoid = true;   // Dequantize + Sigmoid of its result in one kernel
+  bool deriveBagOffsets = true;        // lookups whose lengths are an input: bag positions summed on the host at upload
 };
 
 class MI355XBackend {

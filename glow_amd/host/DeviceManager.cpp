@@ -7,6 +7,26 @@
 namespace glow_mi355x {
 
 namespace {
+// The other half of MI355XFunction::derivedBagOffsets: `lengths` (n int32) has
+// just been copied into placeholder `name`; the positions its lookups read go
+// to the function's scratch. `staged` keeps the host vectors alive until the
+// caller has synchronised the stream.
+int uploadBagOffsets(const MI355XFunction &fn, const DeviceBindings &b, const std::string &name,
+                     const void *lengths, size_t bytes, void *stream,
+                     std::vector<std::vector<int32_t>> &staged) {
+  for (const auto &d : fn.derivedBagOffsets) {
+    if (d.lengths != name) continue;
+    staged.push_back(MI355XFunction::bagOffsets(static_cast<const int32_t *>(lengths),
+                                                bytes / sizeof(int32_t), d.segments));
+    const int rc = mi355x_memcpy_h2d(d.ptr(b), staged.back().data(),
+                                     staged.back().size() * sizeof(int32_t), stream);
+    if (rc != MI355X_OK) return rc;
+  }
+  return MI355X_OK;
+}
+} // namespace
+
+namespace {
 Error fromStatus(int rc, const char *what) {
   if (rc == MI355X_OK) return Error::success();
   ErrorCode c = ErrorCode::RUNTIME_ERROR;
@@ -209,6 +229,12 @@ void MI355XDeviceManager::transferStaticPlaceholderToDevice(
     }
     int rc = mi355x_arena_upload(mit->second.arena, MI355X_REGION_MUTABLE, v.offset, tensor->data(),
                                  tensor->sizeInBytes(), stream_);
+    // lookups of the module's functions that take their bags from this placeholder
+    std::vector<std::vector<int32_t>> staged;
+    for (auto &f : functions_)
+      if (rc == MI355X_OK && f.second.module == module)
+        rc = uploadBagOffsets(*f.second.fn, f.second.bindings, placeholderName, tensor->data(),
+                              tensor->sizeInBytes(), stream_, staged);
     if (rc == MI355X_OK) rc = mi355x_stream_sync(stream_);
     resultCB(rc == MI355X_OK ? Error::success() : fromStatus(rc, "placeholder copy"));
   });
@@ -337,6 +363,22 @@ Error MI355XDeviceManager::makeResident(const Module *module, const std::string 
     rc = mi355x_arena_upload(fr.arena, MI355X_REGION_CONSTANTS, 0, fn->generated.data(),
                              fn->generated.size(), stream_);
     if (rc != MI355X_OK) return failWith(fromStatus(rc, "generated constants upload"));
+  }
+  // bag positions of lookups that take them from the host: from what the
+  // lengths placeholders hold right now (zeros on a new module)
+  for (const auto &d : fn->derivedBagOffsets) {
+    auto st = rb.symbolTable.find(d.lengths);
+    if (st == rb.symbolTable.end()) continue;
+    std::vector<int32_t> cur(d.segments, 0);
+    rc = mi355x_memcpy_d2h(cur.data(), fr.bindings.mutableMem + st->second.offset,
+                           d.segments * sizeof(int32_t), stream_);
+    if (rc == MI355X_OK) rc = mi355x_stream_sync(stream_);
+    std::vector<std::vector<int32_t>> staged;
+    if (rc == MI355X_OK)
+      rc = uploadBagOffsets(*fn, fr.bindings, d.lengths, cur.data(), cur.size() * sizeof(int32_t),
+                            stream_, staged);
+    if (rc == MI355X_OK) rc = mi355x_stream_sync(stream_);
+    if (rc != MI355X_OK) return failWith(fromStatus(rc, "bag offsets"));
   }
   for (const auto &l : fn->setup) {
     rc = l.run(fr.bindings);
@@ -554,6 +596,7 @@ void MI355XDeviceManager::runFunctionImpl(RunIdentifierTy id, std::string functi
   const RuntimeBundle &rb = fr.fn->getRuntimeBundle();
   PlaceholderBindings *pb = ctx->getPlaceholderBindings();
   Error err;
+  std::vector<std::vector<int32_t>> staged; // bag positions on their way to the device
   // inputs: host tensor -> placeholder slot (a tensor smaller than the slot
   // fills its front, like the reference's partial tensors)
   for (const auto &kv : pb->pairs()) {
@@ -568,6 +611,9 @@ void MI355XDeviceManager::runFunctionImpl(RunIdentifierTy id, std::string functi
     }
     int rc = mi355x_memcpy_h2d(fr.bindings.mutableMem + st->second.offset, kv.second->data(),
                                kv.second->sizeInBytes(), stream_);
+    if (rc == MI355X_OK)
+      rc = uploadBagOffsets(*fr.fn, fr.bindings, kv.first, kv.second->data(),
+                            kv.second->sizeInBytes(), stream_, staged);
     if (rc != MI355X_OK) {
       err = fromStatus(rc, "input copy");
       break;

@@ -663,7 +663,9 @@ int mi355x_rwq_slws(float *dest, const uint8_t *data, size_t data_rows,
  *             converted back (_I8_VIA_F16: lookup with a Float16 result, ConvertTo
  *             Float, Quantize), int8 rows dest_row_stride bytes apart starting at
  *             tables[t].dest (InsertTensor into a wider tensor).
- * Indices are int64 (idx_is_64) or int32 for all tables; no weights. */
+ * Indices are int64 (idx_is_64) or int32 for all tables; no weights.
+ * A table whose bag_offsets is not NULL gives its bags as segments + 1 positions
+ * (see mi355x_frwq_slws_offsets) and its lengths are not read. */
 typedef struct {
   const uint8_t *data;
   const void *indices;
@@ -671,6 +673,7 @@ typedef struct {
   void *dest;
   uint64_t data_rows;
   uint64_t num_indices;
+  const int32_t *bag_offsets;
 } mi355x_sls_table;
 enum { MI355X_SLS_OUT_F32 = 0, MI355X_SLS_OUT_F16 = 1, MI355X_SLS_OUT_I8 = 2,
        MI355X_SLS_OUT_I8_VIA_F16 = 3 };

@@ -125,7 +125,10 @@ enum {
   MI355X_HOST_OPT_FUSE_INSERT = 256, /* Gather / RescaleQuantized whose result is only inserted into a
                                         wider tensor write there directly */
   MI355X_HOST_OPT_FUSE_DEQUANTIZE_SIGMOID = 512, /* Dequantize + Sigmoid of its result in one kernel */
-  MI355X_HOST_OPT_DEFAULT = 1023
+  MI355X_HOST_OPT_DERIVE_BAG_OFFSETS = 1024, /* lookups whose lengths are an input placeholder read
+                                              * their bags as positions that the device manager sums
+                                              * on the host when it uploads the lengths */
+  MI355X_HOST_OPT_DEFAULT = 2047
 };
 int mi355x_host_compile(mi355x_host_module *m, int function, int options);
 /* Listing of the compiled function's launches and derived parameters; returns

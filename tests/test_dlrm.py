@@ -23,6 +23,8 @@ def test_builds_and_compiles():
     assert k.count("mi355x_frwq_sls_multi") == 1 and "mi355x_frwq_slws" not in k
     multi = rows[k.index("mi355x_frwq_sls_multi")]
     assert (multi["tables"], multi["out_kind"], multi["stride"]) == (3, 3, 4 * 16)
+    # the lengths are inputs: every table's bags come as positions summed on the host
+    assert multi["bag_offsets_from_host"] == 3
     assert k.count("mi355x_convert_f16_to_f32") == 0
     # no InsertTensor is left: the bottom MLP's rescaled output and the upper
     # triangle of the interaction are written where they are inserted
@@ -42,7 +44,7 @@ def test_builds_and_compiles():
     m.compile(f, fuse_sls_chains=False, fuse_transpose_matmul=False, fuse_fc_relu=False,
               fuse_insert=False, fuse_dequantize_sigmoid=False)
     k = [r["kernel"] for r in H.parse_listing(m.describe(f)) if r["phase"] == "launch"]
-    assert k.count("mi355x_frwq_slws") == 3 and k.count("mi355x_rwq_fc_i8") == 4
+    assert k.count("mi355x_frwq_slws_offsets") == 3 and k.count("mi355x_rwq_fc_i8") == 4
     assert k.count("mi355x_convert_f16_to_f32") == 3 and k.count("mi355x_insert_rows") == 6
     assert k.count("mi355x_batch_matmul_i8") == 1 and k.count("mi355x_gather") == 1
     assert k[-1] == "mi355x_sigmoid_f32"

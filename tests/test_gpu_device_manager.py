@@ -214,6 +214,45 @@ def test_slws_network(dm):
     assert np.array_equal(res, go.frwq_slws_f32(table, w, idx, lengths))
 
 
+def test_slws_network_bag_positions_follow_every_upload(dm):
+    """The lookup reads bag positions that the device manager derives from the
+    lengths it uploads: per request, for a partial lengths tensor (the missing
+    bags are empty), and after transferStaticPlaceholderToDevice."""
+    rng = np.random.default_rng(28)
+    rows, cols, bags = 3000, 64, 200
+    table = cases.random_fused_table(rng, rows, cols)
+    m = H.Module("slws_positions")
+    data = m.constant("data", table, H.UINT8_FUSED)
+    n = 4000
+    wv = m.placeholder("weights", (n,), H.FLOAT, np.float32)
+    iv = m.placeholder("indices", (n,), H.INT64I, np.int64)
+    lv = m.placeholder("lengths", (bags,), H.INT32I, np.int32)
+    out = m.placeholder("output", (bags, cols), H.FLOAT, np.float32)
+    f = m.function("main")
+    m.instruction(f, H.FRWQ_SLWS, "slws", [out, data, wv, iv, lv], [0])
+    m.compile(f)
+    assert "mi355x_frwq_slws_offsets" in m.describe(f)
+    dm.add_network(m)
+    res = np.zeros((bags, cols), np.float32)
+    for seed, mean in ((1, 12), (2, 3), (3, 15)):
+        lengths, idx, w = cases.slws_batch(seed, rows, bags, mean, 1.05, np.int64)
+        lengths[seed] = -4     # a negative length is an empty bag
+        dm.run("main", {"weights": w, "indices": idx, "lengths": lengths, "output": res})
+        want = go.frwq_slws_f32(table, w, idx, np.maximum(lengths, 0))
+        np.testing.assert_array_equal(res, want)
+    # half the lengths: the other bags are empty
+    lengths, idx, w = cases.slws_batch(4, rows, bags, 10, 1.05, np.int64)
+    half = lengths[:bags // 2].copy()
+    dm.run("main", {"weights": w, "indices": idx, "lengths": half, "output": res})
+    padded = np.r_[half, np.zeros(bags - half.size, np.int32)].astype(np.int32)
+    np.testing.assert_array_equal(res, go.frwq_slws_f32(table, w, idx, padded))
+    # lengths sent on their own, then a request that does not bind them
+    lengths, idx, w = cases.slws_batch(5, rows, bags, 8, 1.05, np.int64)
+    dm.transfer_static_placeholder(m, "lengths", lengths)
+    dm.run("main", {"weights": w, "indices": idx, "output": res})
+    np.testing.assert_array_equal(res, go.frwq_slws_f32(table, w, idx, lengths))
+
+
 def test_fc_and_conv_networks(dm):
     c = cases.fc_case(20, 24, 96, 80)
     m, f = host_cases.fc_module(c)

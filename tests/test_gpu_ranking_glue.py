@@ -99,6 +99,15 @@ def test_multi_table_sls(kind, cols, idt):
     gq = capi.frwq_sls_multi(tables, kind, idx, lens,
                              capi.SLS_OUT_I8_VIA_F16 if f16 else capi.SLS_OUT_I8, scale, off)
     np.testing.assert_array_equal(gq, wq)
+    # the bags of every table as positions instead of lengths: the same bytes
+    got = capi.frwq_sls_multi(tables, kind, idx, lens,
+                              capi.SLS_OUT_F16 if f16 else capi.SLS_OUT_F32, bag_offsets=True)
+    for t in range(n):
+        np.testing.assert_array_equal(got[t], want[t], err_msg=f"table {t}, bag offsets")
+    gq = capi.frwq_sls_multi(tables, kind, idx, lens,
+                             capi.SLS_OUT_I8_VIA_F16 if f16 else capi.SLS_OUT_I8, scale, off,
+                             bag_offsets=True)
+    np.testing.assert_array_equal(gq, wq)
 
 
 @pytest.mark.parametrize("cols,idt", [(128, np.int64), (37, np.int32), (64, np.int64), (16, np.int32)])

@@ -401,3 +401,29 @@ def test_copy_instruction():
     m.instruction(g, H.COPY, "rescaling_copy", [c, a])
     with pytest.raises(H.HostError):
         m.compile(g)
+
+
+def test_lookups_with_input_lengths_read_host_made_bag_positions():
+    """Lengths that are an input placeholder: the launch goes through
+    mi355x_frwq_slws_offsets with positions the device manager sums on the host;
+    lengths an instruction writes on the device, or the option off: through the
+    lengths entry point."""
+    m, ops = _slws_module(H.UINT8_FUSED, H.FLOAT, H.FLOAT)
+    f = m.function("main")
+    m.instruction(f, H.FRWQ_SLWS, "slws", ops, [0])
+    m.compile(f)
+    rows = [r for r in H.parse_listing(m.describe(f)) if r["phase"] == "launch"]
+    assert [r["kernel"] for r in rows] == ["mi355x_frwq_slws_offsets"]
+    assert rows[0]["bag_offsets"] == "host(len)" and rows[0]["segments"] == 3
+    m.compile(f, derive_bag_offsets=False)
+    rows = [r for r in H.parse_listing(m.describe(f)) if r["phase"] == "launch"]
+    assert [r["kernel"] for r in rows] == ["mi355x_frwq_slws"]
+    # lengths copied on the device from another placeholder
+    m, ops = _slws_module(H.UINT8_FUSED, H.FLOAT, H.FLOAT)
+    src = m.placeholder("len_src", (3,), H.INT32I, np.int32)
+    f = m.function("main")
+    m.instruction(f, H.COPY, "copy_len", [ops[4], src])
+    m.instruction(f, H.FRWQ_SLWS, "slws", ops, [0])
+    m.compile(f)
+    rows = [r for r in H.parse_listing(m.describe(f)) if r["phase"] == "launch"]
+    assert [r["kernel"] for r in rows] == ["mi355x_copy_u8", "mi355x_frwq_slws"]
