@@ -30,7 +30,11 @@
  *   go_frwq_slws_generic (Interpreter formula, 4-bit and fp16 scale)
  *       -> near-exact KAT OperatorTest.cpp:16152-16295, KATs :17401-17407,
  *          :17531-17547, brute force in numpy on tiny tables, and equality
- *          with go_frwq_slws_f32 on the 8-bit/fp32 form.
+ *          with go_frwq_slws_f32 on the 8-bit/fp32 form; the float16
+ *          accumulator branch (InterpreterNodes.cpp:5799-5836 with AccumT =
+ *          float16_t) by a numpy-float16 brute force on inputs that are not
+ *          representable in half, on which dropping either rounding (of the
+ *          product, of the partial sum) changes bits.
  */
 #ifndef GLOW_ORACLE_H
 #define GLOW_ORACLE_H

@@ -542,6 +542,53 @@ def test_slws_generic_brute_force_numpy():
             np.testing.assert_array_equal(got, want)
 
 
+def test_slws_fp16_accumulation_brute_force_numpy():
+    """The float16-accumulator branch (reference InterpreterNodes.cpp:5799-5836
+    with AccumT = float16_t, Float16.h operator+=): every product is rounded to
+    half on its own, and so is every partial sum. numpy's float16 is an
+    independent implementation of the roundings; the inputs are not
+    representable in half, so dropping either rounding changes bits."""
+    rng = np.random.default_rng(2024)
+    rows, cols = 40, 16
+    x = rng.normal(0, 3, (rows, cols)).astype(np.float32)
+    lens = np.array([7, 0, 12, 1, 30], np.int32)
+    idx = rng.integers(0, rows, lens.sum()).astype(np.int64)
+    w = rng.uniform(-2, 2, lens.sum()).astype(np.float16)
+    differs_from_f32_accum = differs_from_unrounded_product = 0
+    for kind in (go.U8_F16, go.U4_F16):
+        f = go.fused_rowwise_quantize(x, kind)
+        sc = f[:, -4:-2].copy().view(np.float16).astype(np.float32).ravel()
+        of = f[:, -2:].copy().view(np.float16).astype(np.float32).ravel()
+        if kind == go.U4_F16:
+            b = f[:, :cols // 2]
+            q = np.empty((rows, cols), np.float32)
+            q[:, 0::2] = b & 15
+            q[:, 1::2] = b >> 4
+        else:
+            q = f[:, :cols].astype(np.float32)
+        deq = (q * sc[:, None]).astype(np.float32) + of[:, None]   # fp32, separately rounded
+        want = np.zeros((lens.size, cols), np.float16)
+        loose = np.zeros((lens.size, cols), np.float16)            # product left in fp32
+        cur = 0
+        for i, L in enumerate(lens):
+            acc = np.zeros(cols, np.float16)
+            acc2 = np.zeros(cols, np.float16)
+            for _ in range(L):
+                prod = deq[idx[cur]] * np.float32(w[cur])           # fp32
+                term = prod.astype(np.float16)                      # rounded to half
+                acc = (acc.astype(np.float32) + term.astype(np.float32)).astype(np.float16)
+                acc2 = (acc2.astype(np.float32) + prod).astype(np.float16)
+                cur += 1
+            want[i], loose[i] = acc, acc2
+        got = go.frwq_slws_generic(f, kind, w, idx, lens, out_f16=True, fp16_accum=True)
+        np.testing.assert_array_equal(got.view(np.uint16), want.view(np.uint16))
+        f32acc = go.frwq_slws_generic(f, kind, w, idx, lens, out_f16=True, fp16_accum=False)
+        differs_from_f32_accum += int((f32acc.view(np.uint16) != want.view(np.uint16)).sum())
+        differs_from_unrounded_product += int((loose.view(np.uint16) != want.view(np.uint16)).sum())
+    # the check discriminates: both simplifications change bits on these inputs
+    assert differs_from_f32_accum > 0 and differs_from_unrounded_product > 0
+
+
 def test_slws_invariants():
     rng = np.random.default_rng(10)
     x = rng.normal(0, 1, (50, 16)).astype(np.float32)
