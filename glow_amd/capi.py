@@ -46,6 +46,9 @@ EXPORTS = [
     "mi355x_embedding_bag_rowwise_offsets",
     "mi355x_slws_reserve_stream", "mi355x_frwq_slws_noalloc",
     "mi355x_frwq_slws_offsets", "mi355x_slws_bag_offsets_host",
+    "mi355x_quantize_i16", "mi355x_quantize_i32", "mi355x_dequantize_i16",
+    "mi355x_dequantize_i32", "mi355x_rescale_i16", "mi355x_rescale_i32",
+    "mi355x_transpose_nd", "mi355x_cwq_conv3d_i8",
     "mi355x_shader_clock_probe", "mi355x_wall_clock_khz",
     "mi355x_specialize_bias_qparams", "mi355x_channelwise_quantize_conv_host",
     "mi355x_gemm_requant_hint", "mi355x_gemm_requant_hint_host",
@@ -69,6 +72,23 @@ class ConvGeom(C.Structure):
     _fields_ = [(n, C.c_int32) for n in (
         "N", "IH", "IW", "IC", "OH", "OW", "OC", "KH", "KW", "strideH",
         "strideW", "padT", "padL", "dilH", "dilW", "group")]
+
+
+class Conv3dGeom(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in (
+        "N", "IT", "IH", "IW", "IC", "OT", "OH", "OW", "OC", "KT", "KH", "KW",
+        "strideT", "strideH", "strideW", "padN", "padT", "padL", "group")]
+
+
+def conv3d_geom(N, IT, IH, IW, IC, OC, kernel, stride, pads, group=1):
+    """pads = (near, far, top, bottom, left, right); output extents as Glow
+    computes them (include/glow/Graph/Nodes.h, calculate3DConvPoolOutputDims)."""
+    KT, KH, KW = kernel
+    st, sh, sw = stride
+    pn, pf, pt, pb, pl, pr = pads
+    return Conv3dGeom(N, IT, IH, IW, IC, (IT + pn + pf - KT) // st + 1,
+                      (IH + pt + pb - KH) // sh + 1, (IW + pl + pr - KW) // sw + 1, OC,
+                      KT, KH, KW, st, sh, sw, pn, pt, pl, group)
 
 
 _lib = None
@@ -912,6 +932,72 @@ def embedding_bag_rowwise_offsets(data, kind, weights, indices, offsets,
         C.c_int(kind), _vp(d_w), C.c_int(w16), _vp(d_idx), _sz(indices.size),
         _vp(d_off), _sz(offsets.size), C.c_int(bool(has_end_offset)),
         _sz(in_line), _sz(out_line), C.c_int(bool(fp16_accum)), _vp(None)))
+    return d_out.numpy()
+
+
+# ---- 16/32-bit elementwise forms, N-D transpose, 3-D convolution ---------------
+
+_WIDE = {16: np.int16, 32: np.int32}
+
+
+def quantize_wide(x, scale, offset, bits):
+    x = np.ascontiguousarray(x, np.float32)
+    d_in, d_out = to_device(x), DeviceBuffer.empty(x.shape, _WIDE[bits])
+    check(getattr(lib(), f"mi355x_quantize_i{bits}")(
+        _vp(d_out), _vp(d_in), _sz(x.size), C.c_float(scale), _i32(offset), _vp(None)))
+    return d_out.numpy()
+
+
+def dequantize_wide(q, scale, offset):
+    q = np.ascontiguousarray(q)
+    d_in, d_out = to_device(q), DeviceBuffer.empty(q.shape, np.float32)
+    check(getattr(lib(), f"mi355x_dequantize_i{q.itemsize * 8}")(
+        _vp(d_out), _vp(d_in), _sz(q.size), C.c_float(scale), _i32(offset), _vp(None)))
+    return d_out.numpy()
+
+
+def rescale_wide(q, out_offset, in_offset, pre, post, scale):
+    q = np.ascontiguousarray(q)
+    d_in, d_out = to_device(q), DeviceBuffer.empty(q.shape, q.dtype)
+    check(getattr(lib(), f"mi355x_rescale_i{q.itemsize * 8}")(
+        _vp(d_out), _vp(d_in), _sz(q.size), _i32(out_offset), _i32(in_offset), _i32(pre),
+        _i32(post), _i32(scale), _vp(None)))
+    return d_out.numpy()
+
+
+def transpose_nd(x, shuffle):
+    """Output dimension d is input dimension shuffle[d] (numpy's transpose)."""
+    x = np.ascontiguousarray(x)
+    nd = x.ndim
+    dims = (C.c_size_t * nd)(*x.shape)
+    sh = (C.c_size_t * nd)(*shuffle)
+    out_shape = [x.shape[d] for d in shuffle] if sorted(shuffle) == list(range(nd)) else x.shape
+    d_in, d_out = to_device(x), DeviceBuffer.empty(out_shape, x.dtype)
+    check(lib().mi355x_transpose_nd(_vp(d_out), _vp(d_in), dims, sh, _sz(nd), _sz(x.itemsize),
+                                    _vp(None)))
+    return d_out.numpy()
+
+
+def cwq_conv3d_i8(x, filt, bias, geom, out_offset, in_offset, filter_offsets,
+                  bias_offsets, bias_pre, bias_post, bias_scale, out_pre, out_post,
+                  out_scale, act=0, act_args=()):
+    g = geom if isinstance(geom, Conv3dGeom) else \
+        Conv3dGeom(*[getattr(geom, n) for n, _ in Conv3dGeom._fields_])
+    bias = np.ascontiguousarray(bias)
+    b8 = int(bias.dtype == np.int8)
+    if not b8:
+        bias = bias.astype(np.int32)
+    d = [to_device(np.ascontiguousarray(v, np.int8)) for v in (x, filt)]
+    vs = [to_device(np.ascontiguousarray(v, np.int32)) for v in (
+        filter_offsets, bias_offsets, bias_pre, bias_post, bias_scale, out_pre, out_post,
+        out_scale)]
+    d_bias = to_device(bias)
+    d_out = DeviceBuffer.empty((g.N, g.OT, g.OH, g.OW, g.OC), np.int8)
+    d_out.fill(0x55)
+    aa = (C.c_int32 * 3)(*(list(act_args) + [0, 0, 0])[:3])
+    check(lib().mi355x_cwq_conv3d_i8(
+        _vp(d_out), _vp(d[0]), _vp(d[1]), _vp(d_bias), C.c_int(b8), C.byref(g),
+        _i32(out_offset), _i32(in_offset), *[_vp(v) for v in vs], _i32(act), aa, _vp(None)))
     return d_out.numpy()
 
 

@@ -223,7 +223,6 @@ static int conv_halo_rows(const mi355x_conv_geom *g, int cus, size_t &lds) {
   while (rows > 1 && (long long)g->N * ((g->OH + rows - 1) / rows) * slices < cus &&
          (rows - 1) * g->OW >= 32)
     rows--;
-  const int waves = (rows * g->OW + 31) / 32;
   const size_t halo = (size_t)(rows + 2) * (g->OW + 2) * kHaloPix;
   lds = kHaloFilterBytes + kHaloParBytes + halo;
   return rows;

@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB = None
 
 (FLOAT, FLOAT16, INT8Q, INT32Q, INT32I, INT64I, UINT8_FUSED, UINT8_FUSED_FP16,
- UINT4_FUSED_FP16, UINT4_FUSED, BOOL) = range(11)
+ UINT4_FUSED_FP16, UINT4_FUSED, BOOL, INT16Q) = range(12)
 (QUANTIZE, DEQUANTIZE, RESCALE_QUANTIZED, FULLY_CONNECTED, ROWWISE_QUANTIZED_FC,
  MATMUL, CONVOLUTION, CHANNELWISE_QUANTIZED_CONV, FRWQ_SLWS, FRWQ_SLS, ELEMENT_ADD,
  RELU, MAX_POOL, AVG_POOL, SOFTMAX, CONVERT_TO, INSERT_TENSOR, TRANSPOSE, GATHER,

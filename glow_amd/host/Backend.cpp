@@ -218,6 +218,10 @@ public:
       case Kind::MatMul: MI355X_RETURN_IF_ERR(matmul(I, out)); break;
       case Kind::Convolution: MI355X_RETURN_IF_ERR(conv(I, out, false)); break;
       case Kind::ChannelwiseQuantizedConvolution: {
+        if (M_.value(I.operands[1]).type.dims.size() == 5) {   // NTHWC: the 3-D form
+          MI355X_RETURN_IF_ERR(conv3d(I, out));
+          break;
+        }
         // conv -> ElementAdd(conv, residual) [-> Relu] with no other reader of
         // the intermediate tensors: one kernel
         const Instruction *addI = nullptr, *reluI = nullptr;
@@ -585,20 +589,44 @@ private:
       return Error::success();
     }
     case Kind::Transpose: {
-      CHECK_OP(d.ty().kind == ElemKind::Int8QTy && s.ty().kind == ElemKind::Int8QTy, "needs i8 tensors");
-      CHECK_OP(d.ty().scale == s.ty().scale && d.ty().offset == s.ty().offset,
+      CHECK_OP(d.ty().kind == s.ty().kind && !isFused(s.ty().kind), "needs tensors of one plain element kind");
+      CHECK_OP(!isQuantized(s.ty().kind) || (d.ty().scale == s.ty().scale && d.ty().offset == s.ty().offset),
                "input and output must share scale and offset");
       const auto &sd = s.ty().dims;
       const auto &dd = d.ty().dims;
       size_t batch = 1, rows = 0, cols = 0;
-      if (I.iattrs == std::vector<int64_t>{1, 0} && sd.size() == 2) {
+      const bool i8 = s.ty().kind == ElemKind::Int8QTy;
+      if (i8 && I.iattrs == std::vector<int64_t>{1, 0} && sd.size() == 2) {
         rows = (size_t)sd[0]; cols = (size_t)sd[1];
         CHECK_OP(dd.size() == 2 && dd[0] == sd[1] && dd[1] == sd[0], "shape mismatch");
-      } else if (I.iattrs == std::vector<int64_t>{0, 2, 1} && sd.size() == 3) {
+      } else if (i8 && I.iattrs == std::vector<int64_t>{0, 2, 1} && sd.size() == 3) {
         batch = (size_t)sd[0]; rows = (size_t)sd[1]; cols = (size_t)sd[2];
         CHECK_OP(dd.size() == 3 && dd[0] == sd[0] && dd[1] == sd[2] && dd[2] == sd[1], "shape mismatch");
       } else {
-        CHECK_OP(false, "only the shuffles {1,0} and {0,2,1} are supported");
+        // any other shuffle of up to six dimensions, any element size
+        const size_t nd = sd.size();
+        CHECK_OP(nd >= 1 && nd <= 6 && I.iattrs.size() == nd && dd.size() == nd,
+                 "needs a shuffle of 1 to 6 dimensions");
+        std::vector<size_t> dims(nd), shuf(nd);
+        unsigned seen = 0;
+        for (size_t i = 0; i < nd; i++) {
+          CHECK_OP(I.iattrs[i] >= 0 && (size_t)I.iattrs[i] < nd && !(seen & (1u << I.iattrs[i])),
+                   "the shuffle is not a permutation");
+          seen |= 1u << I.iattrs[i];
+          dims[i] = (size_t)sd[i];
+          shuf[i] = (size_t)I.iattrs[i];
+        }
+        for (size_t i = 0; i < nd; i++) CHECK_OP(dd[i] == sd[shuf[i]], "shape mismatch");
+        const size_t es = elemSize(s.ty().kind);
+        std::string sh;
+        for (size_t i = 0; i < nd; i++) sh += (i ? "," : "") + std::to_string(shuf[i]);
+        out.launches.push_back({"mi355x_transpose_nd", I.name,
+                                strFormat(" dims=%zu elem_size=%zu shuffle=[%s]", nd, es, sh.c_str()),
+                                [=](const DeviceBindings &b) {
+                                  return mi355x_transpose_nd(d.ptr(b), s.ptr(b), dims.data(), shuf.data(),
+                                                             nd, es, b.stream);
+                                }});
+        return Error::success();
       }
       out.launches.push_back({"mi355x_batch_transpose_i8", I.name,
                               strFormat(" batch=%zu rows=%zu cols=%zu", batch, rows, cols),
@@ -842,14 +870,30 @@ private:
     return it->second;
   }
 
+  static bool wideKind(ElemKind k) { return k == ElemKind::Int16QTy || k == ElemKind::Int32QTy; }
+
   Error quantize(const Instruction &I, MI355XFunction &out) {
     Operand d = op(I, 0), s = op(I, 1);
-    CHECK_OP(d.ty().kind == ElemKind::Int8QTy && s.ty().kind == ElemKind::FloatTy,
-             "needs float -> i8, has %s -> %s", s.ty().str().c_str(), d.ty().str().c_str());
+    CHECK_OP((d.ty().kind == ElemKind::Int8QTy || wideKind(d.ty().kind)) &&
+                 s.ty().kind == ElemKind::FloatTy,
+             "needs float -> i8, i16 or i32, has %s -> %s", s.ty().str().c_str(),
+             d.ty().str().c_str());
     CHECK_OP(d.ty().size() == s.ty().size(), "size mismatch");
     const size_t n = (size_t)d.ty().size();
     const float sc = d.ty().scale;
     const int32_t off = d.ty().offset;
+    if (wideKind(d.ty().kind)) {
+      const bool w16 = d.ty().kind == ElemKind::Int16QTy;
+      out.launches.push_back({w16 ? "mi355x_quantize_i16" : "mi355x_quantize_i32", I.name,
+                              strFormat(" n=%zu scale=%.9g offset=%d", n, (double)sc, off),
+                              [=](const DeviceBindings &b) {
+                                return w16 ? mi355x_quantize_i16((int16_t *)d.ptr(b), (const float *)s.ptr(b),
+                                                                 n, sc, off, b.stream)
+                                           : mi355x_quantize_i32((int32_t *)d.ptr(b), (const float *)s.ptr(b),
+                                                                 n, sc, off, b.stream);
+                              }});
+      return Error::success();
+    }
     out.launches.push_back({"mi355x_quantize_i8", I.name,
                             strFormat(" n=%zu scale=%.9g offset=%d", n, (double)sc, off),
                             [=](const DeviceBindings &b) {
@@ -861,12 +905,26 @@ private:
 
   Error dequantize(const Instruction &I, MI355XFunction &out, const Instruction *sig = nullptr) {
     Operand d = op(I, 0), s = op(I, 1);
-    CHECK_OP(d.ty().kind == ElemKind::FloatTy && s.ty().kind == ElemKind::Int8QTy,
-             "needs i8 -> float, has %s -> %s", s.ty().str().c_str(), d.ty().str().c_str());
+    CHECK_OP(d.ty().kind == ElemKind::FloatTy &&
+                 (s.ty().kind == ElemKind::Int8QTy || (wideKind(s.ty().kind) && !sig)),
+             "needs i8, i16 or i32 -> float, has %s -> %s", s.ty().str().c_str(),
+             d.ty().str().c_str());
     CHECK_OP(d.ty().size() == s.ty().size(), "size mismatch");
     const size_t n = (size_t)d.ty().size();
     const float sc = s.ty().scale;
     const int32_t off = s.ty().offset;
+    if (wideKind(s.ty().kind)) {
+      const bool w16 = s.ty().kind == ElemKind::Int16QTy;
+      out.launches.push_back({w16 ? "mi355x_dequantize_i16" : "mi355x_dequantize_i32", I.name,
+                              strFormat(" n=%zu scale=%.9g offset=%d", n, (double)sc, off),
+                              [=](const DeviceBindings &b) {
+                                return w16 ? mi355x_dequantize_i16((float *)d.ptr(b), (const int16_t *)s.ptr(b),
+                                                                   n, sc, off, b.stream)
+                                           : mi355x_dequantize_i32((float *)d.ptr(b), (const int32_t *)s.ptr(b),
+                                                                   n, sc, off, b.stream);
+                              }});
+      return Error::success();
+    }
     if (sig) {
       Operand y = op(*sig, 0);
       out.launches.push_back({"mi355x_dequantize_sigmoid", I.name + "+" + sig->name,
@@ -888,12 +946,29 @@ private:
 
   Error rescale(const Instruction &I, MI355XFunction &out, const Instruction *ins = nullptr) {
     Operand d = op(I, 0), s = op(I, 1);
-    CHECK_OP(d.ty().kind == ElemKind::Int8QTy && s.ty().kind == ElemKind::Int8QTy,
-             "needs i8 -> i8");
+    CHECK_OP(d.ty().kind == s.ty().kind &&
+                 (d.ty().kind == ElemKind::Int8QTy || (wideKind(d.ty().kind) && !ins)),
+             "needs i8 -> i8, i16 -> i16 or i32 -> i32");
     CHECK_OP(d.ty().size() == s.ty().size(), "size mismatch");
     const size_t n = (size_t)d.ty().size();
     const S32To8 p = s32to8(s.ty().scale / d.ty().scale);
     const int32_t oo = d.ty().offset, io = s.ty().offset;
+    if (wideKind(d.ty().kind)) {
+      CHECK_OP(shiftsOk(p), "scales %g -> %g give a shift outside [0, 31]", (double)s.ty().scale,
+               (double)d.ty().scale);
+      const bool w16 = d.ty().kind == ElemKind::Int16QTy;
+      out.launches.push_back(
+          {w16 ? "mi355x_rescale_i16" : "mi355x_rescale_i32", I.name,
+           strFormat(" n=%zu", n) + kv("out_offset", oo) + kv("in_offset", io) + kv("pre", p.pre) +
+               kv("post", p.post) + kv("scale", p.scale),
+           [=](const DeviceBindings &b) {
+             return w16 ? mi355x_rescale_i16((int16_t *)d.ptr(b), (const int16_t *)s.ptr(b), n, oo, io,
+                                             p.pre, p.post, p.scale, b.stream)
+                        : mi355x_rescale_i32((int32_t *)d.ptr(b), (const int32_t *)s.ptr(b), n, oo, io,
+                                             p.pre, p.post, p.scale, b.stream);
+           }});
+      return Error::success();
+    }
     if (ins) {
       const SliceDest sd = sliceDest(*ins);
       const size_t rows = (size_t)d.ty().dims[0], cols = (size_t)d.ty().dims[1];
@@ -1098,6 +1173,99 @@ private:
                                    sums ? (const int32_t *)sumPtr(b) : nullptr, b.stream);
          }});
     out.launches.back().requantHint = hint;
+    return Error::success();
+  }
+
+  // ChannelwiseQuantizedConvolution over NTHWC tensors. Integer attributes:
+  // {KT, KH, KW, strideT, strideH, strideW, padNear, padFar, padTop, padBottom,
+  // padLeft, padRight, group, activation}.
+  Error conv3d(const Instruction &I, MI355XFunction &out) {
+    Operand d = op(I, 0), s = op(I, 1), f = op(I, 2), bi = op(I, 3);
+    Operand fs = op(I, 4), fo = op(I, 5), bs = op(I, 6), bo = op(I, 7);
+    CHECK_OP(I.iattrs.size() == 14, "the 3-D form expects 14 integer attributes");
+    CHECK_OP(d.ty().kind == ElemKind::Int8QTy && s.ty().kind == ElemKind::Int8QTy &&
+                 f.ty().kind == ElemKind::Int8QTy && biasKindOk(bi.ty().kind),
+             "needs i8 input, filter and output and an i32 or i8 bias");
+    CHECK_OP(s.ty().dims.size() == 5 && f.ty().dims.size() == 5 && d.ty().dims.size() == 5,
+             "needs NTHWC input and output and an [OC,KT,KH,KW,IC/group] filter");
+    const auto &a = I.iattrs;
+    for (int i = 0; i < 13; i++) CHECK_OP(a[i] >= 0 && a[i] < (1 << 20), "attribute %d out of range", i);
+    mi355x_conv3d_geom g;
+    g.N = (int32_t)s.ty().dims[0]; g.IT = (int32_t)s.ty().dims[1]; g.IH = (int32_t)s.ty().dims[2];
+    g.IW = (int32_t)s.ty().dims[3]; g.IC = (int32_t)s.ty().dims[4];
+    g.OT = (int32_t)d.ty().dims[1]; g.OH = (int32_t)d.ty().dims[2]; g.OW = (int32_t)d.ty().dims[3];
+    g.OC = (int32_t)d.ty().dims[4];
+    g.KT = (int32_t)a[0]; g.KH = (int32_t)a[1]; g.KW = (int32_t)a[2];
+    g.strideT = (int32_t)a[3]; g.strideH = (int32_t)a[4]; g.strideW = (int32_t)a[5];
+    g.padN = (int32_t)a[6]; g.padT = (int32_t)a[8]; g.padL = (int32_t)a[10];
+    g.group = (int32_t)a[12];
+    const int32_t act = (int32_t)a[13];
+    CHECK_OP(g.KT > 0 && g.KH > 0 && g.KW > 0 && g.strideT > 0 && g.strideH > 0 && g.strideW > 0 &&
+                 g.group > 0, "invalid kernel, stride or group");
+    CHECK_OP(g.IC % g.group == 0 && g.OC % g.group == 0, "channels not divisible by group");
+    CHECK_OP(f.ty().dims[0] == g.OC && f.ty().dims[1] == g.KT && f.ty().dims[2] == g.KH &&
+                 f.ty().dims[3] == g.KW && f.ty().dims[4] == g.IC / g.group,
+             "filter %s does not match", f.ty().str().c_str());
+    CHECK_OP(d.ty().dims[0] == g.N && bi.ty().size() == g.OC, "batch or bias size mismatch");
+    // calculate3DConvPoolOutputDims (reference include/glow/Graph/Nodes.h)
+    const int64_t ot = (g.IT + a[6] + a[7] - g.KT) / g.strideT + 1;
+    const int64_t oh = (g.IH + a[8] + a[9] - g.KH) / g.strideH + 1;
+    const int64_t ow = (g.IW + a[10] + a[11] - g.KW) / g.strideW + 1;
+    CHECK_OP(ot == g.OT && oh == g.OH && ow == g.OW,
+             "output %s does not match the computed %lld x %lld x %lld", d.ty().str().c_str(),
+             (long long)ot, (long long)oh, (long long)ow);
+    CHECK_OP(act == NONE || act == RELU || act == CLIP || act == LEAKY_RELU,
+             "fused activation %d is not supported for quantized types", act);
+    std::vector<int32_t> actArgs(3, 0);
+    if (act == CLIP) {
+      CHECK_OP(I.fattrs.size() == 2, "fused Clip needs {min, max}");
+      actArgs[0] = quantizeI32(I.fattrs[0], d.ty().scale, d.ty().offset);
+      actArgs[1] = quantizeI32(I.fattrs[1], d.ty().scale, d.ty().offset);
+    } else if (act == LEAKY_RELU) {
+      CHECK_OP(I.fattrs.size() == 1, "fused LeakyRelu needs {alpha}");
+      const S32To8 p = s32to8(I.fattrs[0]);
+      actArgs = {p.pre, p.post, p.scale};
+    } else {
+      CHECK_OP(I.fattrs.empty(), "activation takes no arguments");
+    }
+    CHECK_OP(fs.ty().kind == ElemKind::FloatTy && bs.ty().kind == ElemKind::FloatTy &&
+                 fo.ty().kind == ElemKind::Int32ITy && bo.ty().kind == ElemKind::Int32ITy,
+             "needs float scales and int32 offsets");
+    CHECK_OP(fs.v->category == SymbolCategory::Constant && fo.v->category == SymbolCategory::Constant &&
+                 bs.v->category == SymbolCategory::Constant && bo.v->category == SymbolCategory::Constant,
+             "filter/bias scales and offsets must be constants");
+    const size_t OC = (size_t)g.OC;
+    CHECK_OP((size_t)fs.ty().size() == OC && (size_t)fo.ty().size() == OC &&
+                 (size_t)bs.ty().size() == OC && (size_t)bo.ty().size() == OC,
+             "per-channel vectors must have one entry per output channel");
+    const float *fsc = constData<float>(fs), *bsc = constData<float>(bs);
+    std::vector<int32_t> bpre(OC), bpost(OC), bscale(OC), opre(OC), opost(OC), oscale(OC);
+    for (size_t c = 0; c < OC; c++) {
+      const float mm = s.ty().scale * fsc[c];
+      const S32To8 bp = s32to8(bsc[c] / mm), opp = s32to8(mm / d.ty().scale);
+      bpre[c] = bp.pre; bpost[c] = bp.post; bscale[c] = bp.scale;
+      opre[c] = opp.pre; opost[c] = opp.post; oscale[c] = opp.scale;
+      CHECK_OP(shiftsOk(bp) && shiftsOk(opp), "channel %zu: the scales give a shift outside [0, 31]", c);
+    }
+    const size_t o0 = gen_.addI32(bpre), o1 = gen_.addI32(bpost), o2 = gen_.addI32(bscale),
+                 o3 = gen_.addI32(opre), o4 = gen_.addI32(opost), o5 = gen_.addI32(oscale);
+    const int bias8 = bi.ty().kind == ElemKind::Int8QTy;
+    const int32_t oo = d.ty().offset, io = s.ty().offset;
+    out.launches.push_back(
+        {"mi355x_cwq_conv3d_i8", I.name,
+         strFormat(" N=%d IT=%d IH=%d IW=%d IC=%d OT=%d OH=%d OW=%d OC=%d KT=%d KH=%d KW=%d sT=%d sH=%d "
+                   "sW=%d padN=%d padT=%d padL=%d group=%d", g.N, g.IT, g.IH, g.IW, g.IC, g.OT, g.OH,
+                   g.OW, g.OC, g.KT, g.KH, g.KW, g.strideT, g.strideH, g.strideW, g.padN, g.padT,
+                   g.padL, g.group) +
+             kv("out_offset", oo) + kv("in_offset", io) + kv("act", act) + vecStr("act_args", actArgs) +
+             kv("bias_is_i8", bias8),
+         [=](const DeviceBindings &b) {
+           auto gp = [&](size_t o) { return (const int32_t *)(b.generated + o); };
+           return mi355x_cwq_conv3d_i8((int8_t *)d.ptr(b), (const int8_t *)s.ptr(b), (const int8_t *)f.ptr(b),
+                                       bi.ptr(b), bias8, &g, oo, io, (const int32_t *)fo.ptr(b),
+                                       (const int32_t *)bo.ptr(b), gp(o0), gp(o1), gp(o2), gp(o3), gp(o4),
+                                       gp(o5), act, actArgs.data(), b.stream);
+         }});
     return Error::success();
   }
 

@@ -51,6 +51,7 @@ const char *elemKindName(ElemKind k) {
   case ElemKind::UInt4FusedFP16QTy: return "ui4fusedfp16";
   case ElemKind::UInt4FusedQTy: return "ui4fused";
   case ElemKind::BoolTy: return "bool";
+  case ElemKind::Int16QTy: return "i16";
   }
   return "?";
 }
@@ -58,7 +59,7 @@ const char *elemKindName(ElemKind k) {
 size_t elemSize(ElemKind k) {
   switch (k) {
   case ElemKind::FloatTy: case ElemKind::Int32QTy: case ElemKind::Int32ITy: return 4;
-  case ElemKind::Float16Ty: return 2;
+  case ElemKind::Float16Ty: case ElemKind::Int16QTy: return 2;
   case ElemKind::Int64ITy: return 8;
   default: return 1;
   }

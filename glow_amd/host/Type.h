@@ -25,12 +25,13 @@ enum class ElemKind : int32_t {
   UInt4FusedFP16QTy,  // u4 data, fp16 scale+offset
   UInt4FusedQTy,      // u4 data, fp32 scale+offset
   BoolTy,
+  Int16QTy,
 };
 
 const char *elemKindName(ElemKind k);
 size_t elemSize(ElemKind k);
 inline bool isQuantized(ElemKind k) {
-  return k == ElemKind::Int8QTy || k == ElemKind::Int32QTy;
+  return k == ElemKind::Int8QTy || k == ElemKind::Int32QTy || k == ElemKind::Int16QTy;
 }
 inline bool isFused(ElemKind k) {
   return k == ElemKind::UInt8FusedQTy || k == ElemKind::UInt8FusedFP16QTy ||

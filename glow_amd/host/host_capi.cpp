@@ -33,7 +33,7 @@ int failMsg(ErrorCode c, const std::string &m) {
 Type makeType(int kind, const int64_t *dims, int nd, float scale, int32_t offset) {
   return Type((ElemKind)kind, std::vector<int64_t>(dims, dims + (nd > 0 ? nd : 0)), scale, offset);
 }
-bool kindOk(int k) { return k >= 0 && k <= (int)ElemKind::BoolTy; }
+bool kindOk(int k) { return k >= 0 && k <= (int)ElemKind::Int16QTy; }
 Function *fn(mi355x_host_module *m, int f) {
   if (!m || f < 0 || (size_t)f >= m->module.functions().size()) return nullptr;
   return m->module.functions()[(size_t)f].get();

@@ -32,6 +32,9 @@ class Host:
         return capi.ConvGeom(N, IH, IW, IC, OH, OW, OC, KH, KW, sh, sw, pt, pl,
                              dh, dw, group)
 
+    def conv3d_geom(self, *a, **kw):
+        return capi.conv3d_geom(*a, **kw)
+
     def fused_row_bytes(self, cols, kind):
         return (cols // 2 if kind in (U4_F16, U4_F32) else cols) + \
             (8 if kind in (U8_F32, U4_F32) else 4)
@@ -176,6 +179,49 @@ def cwq_conv_args(c):
             c["in_offset"], c["f_offsets"], c["b_offsets"], c["bias_pre"],
             c["bias_post"], c["bias_scale"], c["out_pre"], c["out_post"],
             c["out_scale"], c["act"], c["act_args"])
+
+
+def cwq_conv3d_case(seed, N, T, H, W, IC, OC, kernel=(3, 3, 3), stride=(1, 1, 1),
+                    pads=(1, 1, 1, 1, 1, 1), group=1, act=ACT_RELU, in_scale=0.05,
+                    in_offset=0, out_offset=-128, symmetric=True, bias_i8=False, host=None):
+    """Operands and per-channel parameters of the channelwise quantized 3-D
+    convolution (NTHWC), derived like cwq_conv_case."""
+    host = host or default_host()
+    rng = np.random.default_rng(seed)
+    x = rng.integers(-128, 128, (N, T, H, W, IC)).astype(np.int8)
+    filt = rng.integers(-127, 128, (OC, *kernel, IC // group)).astype(np.int8)
+    f_scales = rng.uniform(0.002, 0.02, OC).astype(np.float32)
+    f_offsets = (np.zeros(OC, np.int32) if symmetric
+                 else rng.integers(-10, 11, OC).astype(np.int32))
+    mm = np.float32(in_scale) * f_scales
+    if bias_i8:
+        bias = rng.integers(-128, 128, OC).astype(np.int8)
+        b_scales = mm * np.float32(37.0)
+        b_offsets = rng.integers(-5, 6, OC).astype(np.int32)
+    else:
+        bias = rng.integers(-20000, 20001, OC).astype(np.int32)
+        b_scales = mm
+        b_offsets = np.zeros(OC, np.int32)
+    k = kernel[0] * kernel[1] * kernel[2] * (IC // group)
+    out_scale = float(np.sqrt(k) * 74 * 74 * in_scale * f_scales.mean() / 40)
+    bpre, bpost, bscale = s32to8_vec(b_scales / mm, host)
+    opre, opost, oscale = s32to8_vec(mm / np.float32(out_scale), host)
+    g = host.conv3d_geom(N, T, H, W, IC, OC, kernel, stride, pads, group)
+    act_args, act_fargs = (), ()
+    if act == ACT_CLIP:
+        act_fargs = (0.0, float(np.float32(6.0 * out_scale * 20)))
+        act_args = (host.quantize_value_i32(act_fargs[0], out_scale, out_offset),
+                    host.quantize_value_i32(act_fargs[1], out_scale, out_offset))
+    elif act == ACT_LEAKY_RELU:
+        act_fargs = (0.1,)
+        act_args = host.s32to8(0.1, 0)[:3]
+    return dict(x=x, filt=filt, bias=bias, geom=g, out_offset=int(out_offset),
+                in_offset=int(in_offset), f_offsets=f_offsets, b_offsets=b_offsets,
+                bias_pre=bpre, bias_post=bpost, bias_scale=bscale, out_pre=opre,
+                out_post=opost, out_scale=oscale, act=act, act_args=act_args,
+                act_fargs=act_fargs, f_scales=f_scales,
+                b_scales=np.asarray(b_scales, np.float32), in_scale_f=float(in_scale),
+                out_scale_f=float(out_scale))
 
 
 def zipf_indices(rng, n, rows, alpha):

@@ -222,6 +222,25 @@ int mi355x_dequantize_i8(float *dst, const int8_t *src, size_t n, float scale,
 int mi355x_rescale_i8(int8_t *dst, const int8_t *src, size_t n,
                       int32_t out_offset, int32_t in_offset, int32_t pre,
                       int32_t post, int32_t scale, void *stream);
+/* The 16- and 32-bit forms: libjit_element_quantize_kernel_i16 / _i32
+ * (libjit.cpp:3004-3014; the 32-bit one does not clip),
+ * libjit_element_dequantize_kernel_i16 / _i32 (libjit.cpp:3021-3029) and
+ * libjit_element_rescale_kernel_i16 / _i32 (libjit.cpp:3040-3056, which run
+ * libjit_scale<int64_t>: 64-bit products, result truncated to 32 bits). */
+int mi355x_quantize_i16(int16_t *dst, const float *src, size_t n, float scale,
+                        int32_t offset, void *stream);
+int mi355x_quantize_i32(int32_t *dst, const float *src, size_t n, float scale,
+                        int32_t offset, void *stream);
+int mi355x_dequantize_i16(float *dst, const int16_t *src, size_t n, float scale,
+                          int32_t offset, void *stream);
+int mi355x_dequantize_i32(float *dst, const int32_t *src, size_t n, float scale,
+                          int32_t offset, void *stream);
+int mi355x_rescale_i16(int16_t *dst, const int16_t *src, size_t n,
+                       int32_t out_offset, int32_t in_offset, int32_t pre,
+                       int32_t post, int32_t scale, void *stream);
+int mi355x_rescale_i32(int32_t *dst, const int32_t *src, size_t n,
+                       int32_t out_offset, int32_t in_offset, int32_t pre,
+                       int32_t post, int32_t scale, void *stream);
 /* The same rescale of a [rows x cols] tensor, written as a slice of a wider
  * tensor: row r goes to dst + r*dst_row_stride (the caller adds the slice's
  * offset to dst). RescaleQuantized followed by the InsertTensor that is the
@@ -467,6 +486,13 @@ int mi355x_gemm_requant_hint_host(size_t K, size_t N, int32_t in_offset, int32_t
 int mi355x_transpose2d_i8(int8_t *dst, const int8_t *src, size_t rows,
                           size_t cols, void *stream);
 
+/* libjit_transpose_i8 / _f / _u / _b (libjit.cpp:565-653, 3162-3184) for 1 to 6
+ * dimensions and elements of 1, 2, 4 or 8 bytes: output dimension d is input
+ * dimension shuffle[d] (in_dims and shuffle are HOST arrays of num_dims). */
+int mi355x_transpose_nd(void *dst, const void *src, const size_t *in_dims,
+                        const size_t *shuffle, size_t num_dims, size_t elem_size,
+                        void *stream);
+
 /* ---- Convolution -------------------------------------------------------------- */
 
 /* NHWC input [N,IH,IW,IC], filter [OC,KH,KW,IC/group], output [N,OH,OW,OC];
@@ -503,6 +529,32 @@ int mi355x_cwq_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
                          const int32_t *act_args,
                          int filter_offsets_all_zero,
                          const int32_t *filter_row_sums, void *stream);
+
+/* NTHWC input [N,IT,IH,IW,IC], filter [OC,KT,KH,KW,IC/group], output
+ * [N,OT,OH,OW,OC]; pads are {near, top, left}; the output size carries
+ * far/bottom/right. */
+typedef struct {
+  int32_t N, IT, IH, IW, IC;
+  int32_t OT, OH, OW, OC;
+  int32_t KT, KH, KW;
+  int32_t strideT, strideH, strideW;
+  int32_t padN, padT, padL;
+  int32_t group;
+} mi355x_conv3d_geom;
+
+/* libjit_channelwise_quantized_conv3d_i8_i32 / _i8_i8 (reference
+ * lib/LLVMIRCodeGen/libjit/libjit_conv.cpp:244-349, 564-596; no dilation, as
+ * there). Parameters as mi355x_cwq_conv2d_i8; the per-channel shifts must lie
+ * in [0, 31]. */
+int mi355x_cwq_conv3d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
+                         const void *bias, int bias_is_i8,
+                         const mi355x_conv3d_geom *geom, int32_t out_offset,
+                         int32_t in_offset, const int32_t *filter_offsets,
+                         const int32_t *bias_offsets, const int32_t *bias_pre,
+                         const int32_t *bias_post, const int32_t *bias_scale,
+                         const int32_t *out_pre, const int32_t *out_post,
+                         const int32_t *out_scale, int32_t act_type,
+                         const int32_t *act_args, void *stream);
 
 /* ChannelwiseQuantizedConvolution whose result feeds an ElementAdd with a
  * residual tensor of the output's shape, optionally followed by Relu: the

@@ -47,7 +47,7 @@ enum {
   MI355X_HOST_INT32Q = 3, MI355X_HOST_INT32I = 4, MI355X_HOST_INT64I = 5,
   MI355X_HOST_UINT8_FUSED = 6, MI355X_HOST_UINT8_FUSED_FP16 = 7,
   MI355X_HOST_UINT4_FUSED_FP16 = 8, MI355X_HOST_UINT4_FUSED = 9,
-  MI355X_HOST_BOOL = 10
+  MI355X_HOST_BOOL = 10, MI355X_HOST_INT16Q = 11
 };
 
 /* Instruction kinds: Glow's IR instruction names (operand order of

@@ -420,6 +420,94 @@ void go_rescale_i8(int8_t *dst, const int8_t *src, size_t n, int32_t outOffset,
   }
 }
 
+/* libjit_defs.h:151-153 */
+static inline int16_t clip_i16(int32_t v) {
+  return (int16_t)(v < -32768 ? -32768 : (v > 32767 ? 32767 : v));
+}
+
+/* libjit_defs.h:158-173 instantiated as libjit_scale<int64_t> (DestTy stays
+ * int32_t): the arithmetic runs in 64 bits and the result is truncated. */
+static inline int32_t scale_i64(int64_t input, int32_t pre, int32_t post, int32_t scale,
+                                int32_t offset) {
+  const int64_t rtn = (post > 0) ? (int64_t)(1 << (post - 1)) : 0;
+  const int64_t v = ((((input >> pre) * (int64_t)scale) + rtn) >> post) + (int64_t)offset;
+  return (int32_t)(uint32_t)(uint64_t)v;
+}
+
+static inline int32_t round_to_i32(float r) {
+  /* saturating where the reference's conversion is undefined (see go_quantize_i8) */
+  if (r >= 2147483648.0f) return INT32_MAX;
+  if (r <= -2147483648.0f) return INT32_MIN;
+  return (int32_t)r;
+}
+
+/* libjit.cpp:3004-3008 */
+void go_quantize_i16(int16_t *dst, const float *src, size_t n, float scale, int32_t offset) {
+  for (size_t i = 0; i < n; i++)
+    dst[i] = clip_i16(round_to_i32(nearbyintf(src[i] / scale + (float)offset)));
+}
+
+/* libjit.cpp:3010-3014 (no clip) */
+void go_quantize_i32(int32_t *dst, const float *src, size_t n, float scale, int32_t offset) {
+  for (size_t i = 0; i < n; i++)
+    dst[i] = round_to_i32(nearbyintf(src[i] / scale + (float)offset));
+}
+
+/* libjit.cpp:3021-3024 */
+void go_dequantize_i16(float *dst, const int16_t *src, size_t n, float scale, int32_t offset) {
+  for (size_t i = 0; i < n; i++) dst[i] = scale * (float)((int32_t)src[i] - offset);
+}
+
+/* libjit.cpp:3026-3029: the subtraction is 32-bit (wraps) */
+void go_dequantize_i32(float *dst, const int32_t *src, size_t n, float scale, int32_t offset) {
+  for (size_t i = 0; i < n; i++)
+    dst[i] = scale * (float)(int32_t)((uint32_t)src[i] - (uint32_t)offset);
+}
+
+/* libjit.cpp:3040-3047 */
+void go_rescale_i16(int16_t *dst, const int16_t *src, size_t n, int32_t outOffset,
+                    int32_t inOffset, int32_t pre, int32_t post, int32_t scale) {
+  for (size_t i = 0; i < n; i++)
+    dst[i] = clip_i16(scale_i64((int64_t)((int32_t)src[i] - inOffset), pre, post, scale,
+                                outOffset));
+}
+
+/* libjit.cpp:3049-3056: in - inOffset is 32-bit (wraps), then widened */
+void go_rescale_i32(int32_t *dst, const int32_t *src, size_t n, int32_t outOffset,
+                    int32_t inOffset, int32_t pre, int32_t post, int32_t scale) {
+  for (size_t i = 0; i < n; i++)
+    dst[i] = scale_i64((int64_t)(int32_t)((uint32_t)src[i] - (uint32_t)inOffset), pre, post,
+                       scale, outOffset);
+}
+
+/* libjit.cpp:565-653 (libjit_transpose_generic; the tiling there only orders
+ * the copies): out[x0..] = in[source coordinate], where source dimension
+ * shuffle[d] runs with output dimension d. elemSize bytes per element
+ * (libjit_transpose_i8 / _f / _u / _b: 1, 4, 8, 1). */
+void go_transpose(void *out, const void *in, const size_t *idim, const size_t *shuffle,
+                  size_t numDims, size_t elemSize) {
+  size_t odim[6], istride[6], oc[6] = {0, 0, 0, 0, 0, 0};
+  size_t total = 1;
+  for (size_t d = 0; d < numDims; d++) {
+    odim[d] = idim[shuffle[d]];
+    total *= idim[d];
+  }
+  size_t st = 1;
+  for (size_t d = numDims; d-- > 0;) {
+    istride[d] = st;
+    st *= idim[d];
+  }
+  for (size_t o = 0; o < total; o++) {
+    size_t src = 0;
+    for (size_t d = 0; d < numDims; d++) src += oc[d] * istride[shuffle[d]];
+    memcpy((char *)out + o * elemSize, (const char *)in + src * elemSize, elemSize);
+    for (size_t d = numDims; d-- > 0;) {
+      if (++oc[d] < odim[d]) break;
+      oc[d] = 0;
+    }
+  }
+}
+
 /* ------------------------------------------------------------------------ */
 /* FullyConnected / MatMul                                                  */
 /* ------------------------------------------------------------------------ */
@@ -592,6 +680,48 @@ void go_cwq_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
 
 /* ------------------------------------------------------------------------ */
 /* FusedRowwiseQuantizedSparseLengthsWeightedSum                            */
+/* libjit_conv.cpp:244-349 (channelwise quantized 3-D convolution, NTHWC;
+ * pads are {near, far, top, bottom, left, right}, of which the near, top and
+ * left ones are read; the dilation is ignored there as here). */
+void go_cwq_conv3d_i8(int8_t *out, const int8_t *in, const int8_t *filter, const void *bias,
+                      int biasIsI8, const go_conv3d_geom *g, int32_t outOffset,
+                      int32_t inOffset, const int32_t *filterOffsets,
+                      const int32_t *biasOffsets, const int32_t *biasPre,
+                      const int32_t *biasPost, const int32_t *biasScale, const int32_t *outPre,
+                      const int32_t *outPost, const int32_t *outScale, int32_t actType,
+                      const int32_t *actArgs) {
+  const size_t icg = (size_t)(g->IC / g->group), ocg = (size_t)(g->OC / g->group);
+  for (size_t n = 0; n < (size_t)g->N; n++)
+    for (size_t grp = 0; grp < (size_t)g->group; grp++)
+      for (size_t d = grp * ocg; d < (grp + 1) * ocg; d++)
+        for (size_t at = 0; at < (size_t)g->OT; at++)
+          for (size_t ax = 0; ax < (size_t)g->OH; ax++)
+            for (size_t ay = 0; ay < (size_t)g->OW; ay++) {
+              int32_t sum = go_scale_i32(bias_at(bias, biasIsI8, d) - biasOffsets[d], biasPre[d],
+                                         biasPost[d], biasScale[d], 0);
+              for (size_t ft = 0; ft < (size_t)g->KT; ft++)
+                for (size_t fx = 0; fx < (size_t)g->KH; fx++)
+                  for (size_t fy = 0; fy < (size_t)g->KW; fy++) {
+                    const long ot = (long)(at * g->strideT + ft) - g->padN;
+                    const long ox = (long)(ax * g->strideH + fx) - g->padT;
+                    const long oy = (long)(ay * g->strideW + fy) - g->padL;
+                    if (ot < 0 || ox < 0 || oy < 0 || ot >= g->IT || ox >= g->IH || oy >= g->IW)
+                      continue;
+                    const int8_t *ip =
+                        in + ((((n * g->IT + (size_t)ot) * g->IH + (size_t)ox) * g->IW +
+                               (size_t)oy) * g->IC + grp * icg);
+                    const int8_t *fp =
+                        filter + ((((d * g->KT + ft) * g->KH + fx) * g->KW + fy) * icg);
+                    for (size_t fd = 0; fd < icg; fd++)
+                      sum = mac32(sum, (int32_t)fp[fd] - filterOffsets[d],
+                                  (int32_t)ip[fd] - inOffset);
+                  }
+              int32_t v = go_scale_i32(sum, outPre[d], outPost[d], outScale[d], outOffset);
+              v = go_activation_i32(v, outOffset, actType, actArgs);
+              out[(((n * g->OT + at) * g->OH + ax) * g->OW + ay) * g->OC + d] = go_clip_i8(v);
+            }
+}
+
 /* ------------------------------------------------------------------------ */
 
 static inline int64_t index_at(const void *idx, int is64, size_t i) {

@@ -14,7 +14,9 @@
  * How each function is pinned (none is "parity unpinned"):
  *   go_scale_i32 / go_clip_i8 / go_quantize_i8 / go_dequantize_i8 /
  *   go_rescale_i8 / go_fc_i8 / go_rwq_fc_i8 / go_matmul_i8 / go_conv2d_i8 /
- *   go_cwq_conv2d_i8 / go_frwq_slws_f32 / glue ops
+ *   go_cwq_conv2d_i8 / go_cwq_conv3d_i8 / go_frwq_slws_f32 / glue ops /
+ *   go_quantize_i16, _i32 / go_dequantize_i16, _i32 / go_rescale_i16, _i32 /
+ *   go_transpose
  *       -> compared against the reference's own libjit sources compiled into
  *          oracle/_ref (tests/test_oracle_vs_ref.py), committed golden vectors
  *          produced by that build (tests/golden), the exact known-answer
@@ -126,6 +128,22 @@ void go_dequantize_i8(float *dst, const int8_t *src, size_t n, float scale,
 void go_rescale_i8(int8_t *dst, const int8_t *src, size_t n, int32_t outOffset,
                    int32_t inOffset, int32_t pre, int32_t post, int32_t scale);
 
+/* libjit.cpp:3004-3014, 3021-3029, 3040-3056: the 16- and 32-bit forms (the
+ * rescales run libjit_scale<int64_t>; the 32-bit quantize does not clip). */
+void go_quantize_i16(int16_t *dst, const float *src, size_t n, float scale, int32_t offset);
+void go_quantize_i32(int32_t *dst, const float *src, size_t n, float scale, int32_t offset);
+void go_dequantize_i16(float *dst, const int16_t *src, size_t n, float scale, int32_t offset);
+void go_dequantize_i32(float *dst, const int32_t *src, size_t n, float scale, int32_t offset);
+void go_rescale_i16(int16_t *dst, const int16_t *src, size_t n, int32_t outOffset,
+                    int32_t inOffset, int32_t pre, int32_t post, int32_t scale);
+void go_rescale_i32(int32_t *dst, const int32_t *src, size_t n, int32_t outOffset,
+                    int32_t inOffset, int32_t pre, int32_t post, int32_t scale);
+
+/* libjit.cpp:565-653, 3162-3184: transpose of up to 6 dimensions; output
+ * dimension d is input dimension shuffle[d]. */
+void go_transpose(void *out, const void *in, const size_t *idim, const size_t *shuffle,
+                  size_t numDims, size_t elemSize);
+
 /* ---- FullyConnected / MatMul ------------------------------------------ */
 
 /* libjit_matmul.cpp:254-280. in [M x K], weights [K x N], bias int32 or int8
@@ -184,6 +202,24 @@ void go_cwq_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
                       const int32_t *biasScale, const int32_t *outPre,
                       const int32_t *outPost, const int32_t *outScale,
                       int32_t actType, const int32_t *actArgs);
+
+typedef struct {
+  int32_t N, IT, IH, IW, IC;
+  int32_t OT, OH, OW, OC;
+  int32_t KT, KH, KW;
+  int32_t strideT, strideH, strideW;
+  int32_t padN, padT, padL; /* near, top, left */
+  int32_t group;
+} go_conv3d_geom;
+
+/* libjit_conv.cpp:244-349, 564-596 */
+void go_cwq_conv3d_i8(int8_t *out, const int8_t *in, const int8_t *filter, const void *bias,
+                      int biasIsI8, const go_conv3d_geom *g, int32_t outOffset,
+                      int32_t inOffset, const int32_t *filterOffsets,
+                      const int32_t *biasOffsets, const int32_t *biasPre,
+                      const int32_t *biasPost, const int32_t *biasScale, const int32_t *outPre,
+                      const int32_t *outPost, const int32_t *outScale, int32_t actType,
+                      const int32_t *actArgs);
 
 /* ---- FusedRowwiseQuantizedSparseLengthsWeightedSum -------------------- */
 

@@ -228,6 +228,50 @@ def dequantize_i8(q, scale, offset):
     return out
 
 
+_WIDE = {16: np.int16, 32: np.int32}
+
+
+def quantize_wide(x, scale, offset, bits):
+    """Quantize to int16 (clipped) or int32 (not clipped)."""
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, _WIDE[bits])
+    getattr(lib(), f"go_quantize_i{bits}")(_p(out), _p(x), C.c_size_t(x.size), C.c_float(scale),
+                                          C.c_int32(offset))
+    return out
+
+
+def dequantize_wide(q, scale, offset):
+    q = np.ascontiguousarray(q)
+    bits = {np.dtype(np.int16): 16, np.dtype(np.int32): 32}[q.dtype]
+    out = np.empty(q.shape, np.float32)
+    getattr(lib(), f"go_dequantize_i{bits}")(_p(out), _p(q), C.c_size_t(q.size), C.c_float(scale),
+                                            C.c_int32(offset))
+    return out
+
+
+def rescale_wide(q, out_offset, in_offset, pre, post, scale):
+    q = np.ascontiguousarray(q)
+    bits = {np.dtype(np.int16): 16, np.dtype(np.int32): 32}[q.dtype]
+    out = np.empty(q.shape, q.dtype)
+    getattr(lib(), f"go_rescale_i{bits}")(_p(out), _p(q), C.c_size_t(q.size),
+                                         C.c_int32(out_offset), C.c_int32(in_offset),
+                                         C.c_int32(pre), C.c_int32(post), C.c_int32(scale))
+    return out
+
+
+def transpose(x, shuffle):
+    """Transpose of up to six dimensions: output dimension d is input dimension
+    shuffle[d] (numpy's x.transpose(shuffle))."""
+    x = np.ascontiguousarray(x)
+    nd = x.ndim
+    assert nd <= 6 and sorted(shuffle) == list(range(nd))
+    idim = (C.c_size_t * nd)(*x.shape)
+    sh = (C.c_size_t * nd)(*shuffle)
+    out = np.empty([x.shape[d] for d in shuffle], x.dtype)
+    lib().go_transpose(_p(out), _p(x), idim, sh, C.c_size_t(nd), C.c_size_t(x.itemsize))
+    return out
+
+
 def rescale_i8(q, out_offset, in_offset, pre, post, scale):
     q = _c(q, np.int8)
     out = np.empty(q.shape, np.int8)
@@ -328,6 +372,42 @@ def cwq_conv2d_i8(x, filt, bias, geom, out_offset, in_offset, filter_offsets,
     out = np.empty((geom.N, geom.OH, geom.OW, geom.OC), np.int8)
     aa = _act_args(act_args)
     lib().go_cwq_conv2d_i8(_p(out), _p(x), _p(filt), _p(bias), C.c_int(b8),
+                           C.byref(geom), C.c_int32(out_offset),
+                           C.c_int32(in_offset), *[_p(v) for v in vs],
+                           C.c_int32(act), _p(aa))
+    return out
+
+
+class Conv3dGeom(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in (
+        "N", "IT", "IH", "IW", "IC", "OT", "OH", "OW", "OC", "KT", "KH", "KW",
+        "strideT", "strideH", "strideW", "padN", "padT", "padL", "group")]
+
+
+def conv3d_geom(N, IT, IH, IW, IC, OC, kernel, stride, pads, group=1):
+    """pads = (near, far, top, bottom, left, right). Output size as Glow computes
+    it (calculate3DConvPoolOutputDims, include/glow/Graph/Nodes.h)."""
+    KT, KH, KW = kernel
+    st, sh, sw = stride
+    pn, pf, pt, pb, pl, pr = pads
+    OT = (IT + pn + pf - KT) // st + 1
+    OH = (IH + pt + pb - KH) // sh + 1
+    OW = (IW + pl + pr - KW) // sw + 1
+    return Conv3dGeom(N, IT, IH, IW, IC, OT, OH, OW, OC, KT, KH, KW, st, sh, sw, pn, pt, pl,
+                      group)
+
+
+def cwq_conv3d_i8(x, filt, bias, geom, out_offset, in_offset, filter_offsets,
+                  bias_offsets, bias_pre, bias_post, bias_scale, out_pre,
+                  out_post, out_scale, act=ACT_NONE, act_args=()):
+    x = _c(x, np.int8)
+    filt = _c(filt, np.int8)
+    bias, b8 = _bias(bias)
+    vs = [_i32v(v) for v in (filter_offsets, bias_offsets, bias_pre, bias_post,
+                             bias_scale, out_pre, out_post, out_scale)]
+    out = np.empty((geom.N, geom.OT, geom.OH, geom.OW, geom.OC), np.int8)
+    aa = _act_args(act_args)
+    lib().go_cwq_conv3d_i8(_p(out), _p(x), _p(filt), _p(bias), C.c_int(b8),
                            C.byref(geom), C.c_int32(out_offset),
                            C.c_int32(in_offset), *[_p(v) for v in vs],
                            C.c_int32(act), _p(aa))

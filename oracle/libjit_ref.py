@@ -39,6 +39,13 @@ def lib(fastmath=False):
         l.libjit_element_rescale_kernel_i8.restype = C.c_int8
         l.libjit_element_rescale_kernel_i8.argtypes = [
             C.c_uint64, C.c_void_p] + [C.c_int32] * 5
+        for bits, ct in ((16, C.c_int16), (32, C.c_int32)):
+            q = getattr(l, f"libjit_element_quantize_kernel_i{bits}")
+            q.restype, q.argtypes = ct, [C.c_uint64, C.c_void_p, C.c_float, C.c_int32]
+            d = getattr(l, f"libjit_element_dequantize_kernel_i{bits}")
+            d.restype, d.argtypes = C.c_float, [C.c_uint64, C.c_void_p, C.c_float, C.c_int32]
+            r = getattr(l, f"libjit_element_rescale_kernel_i{bits}")
+            r.restype, r.argtypes = ct, [C.c_uint64, C.c_void_p] + [C.c_int32] * 5
         _libs[fastmath] = l
     return _libs[fastmath]
 
@@ -79,6 +86,67 @@ def rescale_i8(q, out_offset, in_offset, pre, post, scale, fastmath=False):
     pq = q.ctypes.data
     return np.array([f(i, pq, out_offset, in_offset, pre, post, scale)
                      for i in range(q.size)], np.int8)
+
+
+_WIDE = {16: np.int16, 32: np.int32}
+
+
+def quantize_wide(x, scale, offset, bits, fastmath=False):
+    x = _c(x, np.float32).ravel()
+    f = getattr(lib(fastmath), f"libjit_element_quantize_kernel_i{bits}")
+    px = x.ctypes.data
+    return np.array([f(i, px, scale, offset) for i in range(x.size)], _WIDE[bits])
+
+
+def dequantize_wide(q, scale, offset, fastmath=False):
+    q = np.ascontiguousarray(q).ravel()
+    f = getattr(lib(fastmath), f"libjit_element_dequantize_kernel_i{q.itemsize * 8}")
+    pq = q.ctypes.data
+    return np.array([f(i, pq, scale, offset) for i in range(q.size)], np.float32)
+
+
+def rescale_wide(q, out_offset, in_offset, pre, post, scale, fastmath=False):
+    q = np.ascontiguousarray(q).ravel()
+    f = getattr(lib(fastmath), f"libjit_element_rescale_kernel_i{q.itemsize * 8}")
+    pq = q.ctypes.data
+    return np.array([f(i, pq, out_offset, in_offset, pre, post, scale)
+                     for i in range(q.size)], q.dtype)
+
+
+def transpose_i8(x, shuffle, fastmath=False):
+    x = _c(x, np.int8)
+    out = np.empty([x.shape[d] for d in shuffle], np.int8)
+    lib(fastmath).libjit_transpose_i8(_p(x), _p(out), _p(_dims(*x.shape)), _p(_dims(*out.shape)),
+                                      _p(_dims(*shuffle)), C.c_uint64(x.ndim))
+    return out
+
+
+def cwq_conv3d_i8(x, filt, bias, g, out_offset, in_offset, filter_offsets,
+                  bias_offsets, bias_pre, bias_post, bias_scale, out_pre,
+                  out_post, out_scale, act=0, act_args=(), fastmath=False):
+    """g: the oracle's Conv3dGeom."""
+    x = _c(x, np.int8)
+    filt = _c(filt, np.int8)
+    bias = np.ascontiguousarray(bias)
+    out = np.empty((g.N, g.OT, g.OH, g.OW, g.OC), np.int8)
+    od = _dims(g.N, g.OT, g.OH, g.OW, g.OC)
+    idm = _dims(g.N, g.IT, g.IH, g.IW, g.IC)
+    fd, bd = _dims(*filt.shape), _dims(g.OC)
+    ks, st = _dims(g.KT, g.KH, g.KW), _dims(g.strideT, g.strideH, g.strideW)
+    # the far / bottom / right pads are not read; the output dims carry them
+    pd = _dims(g.padN, g.padN, g.padT, g.padT, g.padL, g.padL)
+    dl = _dims(1, 1, 1)
+    vs = [_i32v(v) for v in (filter_offsets, bias_offsets, bias_pre, bias_post,
+                             bias_scale, out_pre, out_post, out_scale)]
+    aa = _i32v(list(act_args) + [0, 0, 0])
+    fn = (lib(fastmath).libjit_channelwise_quantized_conv3d_i8_i8
+          if bias.dtype == np.int8
+          else lib(fastmath).libjit_channelwise_quantized_conv3d_i8_i32)
+    fn(_p(out), _p(x), _p(filt), _p(bias), _p(od), _p(idm), _p(fd), _p(bd),
+       _p(ks), _p(st), _p(pd), C.c_uint64(g.group), _p(dl),
+       C.c_int32(out_offset), C.c_int32(in_offset), *[_p(v) for v in vs],
+       C.c_int32(act), _p(aa))
+    return out
 
 
 def fc_i8(x, w_kn, bias, out_offset, in_offset, w_offset, bias_offset, biasP,

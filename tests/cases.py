@@ -17,6 +17,9 @@ class _OracleHost(_w.Host):
     def conv_geom(self, *a, **kw):
         return go.conv_geom(*a, **kw)
 
+    def conv3d_geom(self, *a, **kw):
+        return go.conv3d_geom(*a, **kw)
+
     def fused_row_bytes(self, cols, kind):
         return go.fused_row_bytes(cols, kind)
 
@@ -38,6 +41,10 @@ def fc_case(*a, **kw):
 
 def cwq_conv_case(*a, **kw):
     return _w.cwq_conv_case(*a, host=_HOST, **kw)
+
+
+def cwq_conv3d_case(*a, **kw):
+    return _w.cwq_conv3d_case(*a, host=_HOST, **kw)
 
 
 rwq_fc_args = _w.rwq_fc_args

@@ -71,10 +71,67 @@ def glue():
     save("glue", **gl)
 
 
+WIDE_CONV3D = [
+    ("relu3", dict(N=2, T=4, H=5, W=6, IC=8, OC=8)),
+    ("stride_group", dict(N=1, T=5, H=7, W=6, IC=8, OC=12, kernel=(2, 3, 1), stride=(2, 1, 2),
+                          pads=(1, 0, 0, 2, 1, 1), group=2, act=go.ACT_NONE, symmetric=False,
+                          in_offset=-9, out_offset=5)),
+    ("clip_b8", dict(N=1, T=3, H=3, W=3, IC=3, OC=5, kernel=(3, 3, 3), act=go.ACT_CLIP,
+                     bias_i8=True)),
+    ("leaky", dict(N=1, T=2, H=4, W=4, IC=4, OC=4, kernel=(1, 2, 2), pads=(0, 0, 1, 0, 0, 1),
+                   act=go.ACT_LEAKY_RELU, out_offset=10)),
+]
+WIDE_TRANSPOSES = [((5, 7), (1, 0)), ((3, 4, 5), (2, 0, 1)), ((2, 3, 4, 5), (0, 3, 1, 2)),
+                   ((2, 3, 4, 5), (3, 2, 1, 0)), ((2, 3, 2, 3, 4), (4, 0, 3, 1, 2)),
+                   ((2, 2, 3, 2, 3, 2), (5, 3, 1, 4, 2, 0))]
+
+
+def wide():
+    """The 16/32-bit elementwise forms, N-D transposes and the 3-D channelwise
+    convolution, as the reference's compiled libjit computes them."""
+    rng = np.random.default_rng(700)
+    wd = {}
+    x = np.concatenate([rng.normal(0, 300, 1500), rng.normal(0, 3e5, 500),
+                        (np.arange(-100, 100) + 0.5) * 0.25]).astype(np.float32)
+    wd["x"] = x
+    for bits in (16, 32):
+        dt = np.int16 if bits == 16 else np.int32
+        lim = 2 ** (bits - 1)
+        q = np.concatenate([rng.integers(-lim, lim, 1500), [-lim, lim - 1, 0, 1, -1]]).astype(dt)
+        wd[f"q{bits}"] = q
+        for i, (s, o) in enumerate([(0.25, 4), (0.05, -7), (17.3, 33)]):
+            wd[f"quant{bits}_{i}_params"] = np.array([s, o], np.float64)
+            wd[f"quant{bits}_{i}_out"] = ref.quantize_wide(x, s, o, bits)
+            wd[f"dequant{bits}_{i}_out"] = ref.dequantize_wide(q, s, o)
+        # rescale ratios whose 64-bit products stay well inside int64
+        for i, (r, io, oo) in enumerate([(0.0123, -5, 7), (0.5, 0, -128), (1.7, 20, -3),
+                                         (2.0, 1, 1)]):
+            pre, post, sc, _ = go.quantize_scale_offset_32to8(r, 0)
+            wd[f"rescale{bits}_{i}_params"] = np.array([oo, io, pre, post, sc], np.int32)
+            wd[f"rescale{bits}_{i}_out"] = ref.rescale_wide(q, oo, io, pre, post, sc)
+    for i, (shape, shuffle) in enumerate(WIDE_TRANSPOSES):
+        t = rng.integers(-128, 128, shape).astype(np.int8)
+        wd[f"transpose{i}_in"] = t
+        wd[f"transpose{i}_shuffle"] = np.array(shuffle, np.int32)
+        wd[f"transpose{i}_out"] = ref.transpose_i8(t, shuffle)
+    for tag, kw in WIDE_CONV3D:
+        c = cases.cwq_conv3d_case(800, **kw)
+        for k, v in c.items():
+            if k == "geom":
+                wd[f"conv3d_{tag}_geom"] = geom_vec(v)
+            elif k not in ("act_fargs", "f_scales", "b_scales", "in_scale_f", "out_scale_f"):
+                wd[f"conv3d_{tag}_{k}"] = np.asarray(v, dtype=np.int32 if k == "act_args" else None)
+        wd[f"conv3d_{tag}_out"] = ref.cwq_conv3d_i8(*cases.cwq_conv_args(c))
+    save("wide", **wd)
+
+
 def main():
     assert ref.available(), "build oracle/_ref first (make -C oracle)"
     if sys.argv[1:] == ["glue"]:
         glue()
+        return
+    if sys.argv[1:] == ["wide"]:
+        wide()
         return
 
     # elementwise
@@ -157,6 +214,7 @@ def main():
         sl[f"{tag}_out"] = ref.frwq_slws_f32(table, w, idx, lengths)
     save("frwq_slws", **sl)
     glue()
+    wide()
 
 
 if __name__ == "__main__":

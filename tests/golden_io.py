@@ -91,3 +91,23 @@ def glue():
                                                                        p[2], p[3:6]),
                         d[f"avgpool{i}_{cip}_out"]))
     return out, d["logits"], d["softmax_out"]
+
+
+def wide():
+    """The 16/32-bit elementwise vectors, transposes and 3-D convolutions."""
+    return _load("wide")
+
+
+def conv3d_cases():
+    d = _load("wide")
+    tags = sorted({k[len("conv3d_"):-len("_out")] for k in d
+                   if k.startswith("conv3d_") and k.endswith("_out")})
+    for t in tags:
+        g = lambda k: d[f"conv3d_{t}_{k}"]
+        geom = go.Conv3dGeom(*[int(v) for v in g("geom")])
+        args = (g("x"), g("filt"), g("bias"), geom, int(g("out_offset")),
+                int(g("in_offset")), g("f_offsets"), g("b_offsets"),
+                g("bias_pre"), g("bias_post"), g("bias_scale"), g("out_pre"),
+                g("out_post"), g("out_scale"), int(g("act")),
+                tuple(int(v) for v in g("act_args")))
+        yield t, args, g("out")

@@ -55,3 +55,23 @@ def cwq_conv_module(c, kernel=(3, 3), stride=(1, 1), pads=(1, 1, 1, 1), group=1,
                   H.conv_attrs(kernel, stride, pads, group, dilation, c["act"]),
                   c["act_fargs"])
     return m, f
+
+
+def cwq_conv3d_module(c, kernel, stride, pads, group=1, bias_i8=False, name="main"):
+    """ChannelwiseQuantizedConvolution over NTHWC tensors; pads are
+    (near, far, top, bottom, left, right)."""
+    g = c["geom"]
+    m = H.Module("conv3d")
+    x = m.placeholder("input", c["x"].shape, H.INT8Q, np.int8, c["in_scale_f"], c["in_offset"])
+    out = m.placeholder("output", (g.N, g.OT, g.OH, g.OW, g.OC), H.INT8Q, np.int8,
+                        c["out_scale_f"], c["out_offset"])
+    filt = m.constant("filter", c["filt"], H.INT8Q)
+    b = m.constant("bias", c["bias"], H.INT8Q if bias_i8 else H.INT32Q)
+    fs = m.constant("filterScales", c["f_scales"])
+    fo = m.constant("filterOffsets", c["f_offsets"], H.INT32I)
+    bs = m.constant("biasScales", c["b_scales"])
+    bo = m.constant("biasOffsets", c["b_offsets"], H.INT32I)
+    f = m.function(name)
+    m.instruction(f, H.CHANNELWISE_QUANTIZED_CONV, "conv3d", [out, x, filt, b, fs, fo, bs, bo],
+                  [*kernel, *stride, *pads, group, c["act"]], c["act_fargs"])
+    return m, f

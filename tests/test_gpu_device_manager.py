@@ -274,6 +274,60 @@ def test_fc_and_conv_networks(dm):
         dm.evict_network("main")
 
 
+def test_wide_kinds_transposes_and_3d_convolution_networks(dm):
+    """Quantize -> RescaleQuantized -> Dequantize through int16 and int32
+    tensors, transposes beyond the two tiled shuffles, and the NTHWC
+    convolution, each as a function on the device manager."""
+    rng = np.random.default_rng(41)
+    x = rng.normal(0, 40, (32, 50)).astype(np.float32)
+    m = H.Module("wide")
+    px = m.placeholder("x", x.shape, H.FLOAT, np.float32)
+    f = m.function("main")
+    outs = {}
+    for kind, tag, bits in ((H.INT16Q, "i16", 16), (H.INT32Q, "i32", 32)):
+        q = m.activation(f, f"q_{tag}", x.shape, kind, 0.01, 3)
+        r = m.activation(f, f"r_{tag}", x.shape, kind, 0.02, -5)
+        y = m.placeholder(f"y_{tag}", x.shape, H.FLOAT, np.float32)
+        m.instruction(f, H.QUANTIZE, f"quant_{tag}", [q, px])
+        m.instruction(f, H.RESCALE_QUANTIZED, f"rescale_{tag}", [r, q])
+        m.instruction(f, H.DEQUANTIZE, f"dequant_{tag}", [y, r])
+        pre, post, sc, _ = go.quantize_scale_offset_32to8(float(np.float32(0.01) / np.float32(0.02)), 0)
+        want = go.dequantize_wide(
+            go.rescale_wide(go.quantize_wide(x, 0.01, 3, bits), -5, 3, pre, post, sc), 0.02, -5)
+        outs[f"y_{tag}"] = (np.zeros(x.shape, np.float32), want)
+    t = rng.integers(-128, 128, (3, 16, 9, 11)).astype(np.int8)
+    pt = m.placeholder("t_in", t.shape, H.INT8Q, np.int8, 0.1, 1)
+    po = m.placeholder("t_out", (3, 9, 11, 16), H.INT8Q, np.int8, 0.1, 1)
+    m.instruction(f, H.TRANSPOSE, "nchw2nhwc", [po, pt], [0, 2, 3, 1])
+    ft = rng.normal(0, 1, (7, 5, 3)).astype(np.float32)
+    pf = m.placeholder("f_in", ft.shape, H.FLOAT, np.float32)
+    pfo = m.placeholder("f_out", (3, 7, 5), H.FLOAT, np.float32)
+    m.instruction(f, H.TRANSPOSE, "float_t", [pfo, pf], [2, 0, 1])
+    m.compile(f)
+    dm.add_network(m)
+    t_out, f_out = np.zeros((3, 9, 11, 16), np.int8), np.zeros((3, 7, 5), np.float32)
+    bind = {"x": x, "t_in": t, "f_in": ft, "t_out": t_out, "f_out": f_out}
+    bind.update({k: v[0] for k, v in outs.items()})
+    dm.run("main", bind)
+    for k, (got, want) in outs.items():
+        np.testing.assert_array_equal(got, want, err_msg=k)
+    np.testing.assert_array_equal(t_out, t.transpose(0, 2, 3, 1))
+    np.testing.assert_array_equal(f_out, ft.transpose(2, 0, 1))
+    dm.evict_network("main")
+
+    kernel, stride, pads = (2, 3, 3), (1, 2, 1), (1, 0, 1, 1, 0, 2)
+    c = cases.cwq_conv3d_case(43, N=2, T=4, H=9, W=8, IC=8, OC=12, kernel=kernel, stride=stride,
+                              pads=pads, act=cases._w.ACT_CLIP, in_offset=6, symmetric=False)
+    mc, fc = host_cases.cwq_conv3d_module(c, kernel, stride, pads)
+    mc.compile(fc)
+    dm.add_network(mc)
+    g = c["geom"]
+    o = np.zeros((g.N, g.OT, g.OH, g.OW, g.OC), np.int8)
+    dm.run("main", {"input": c["x"], "output": o})
+    np.testing.assert_array_equal(o, go.cwq_conv3d_i8(*cases.cwq_conv_args(c)))
+    dm.evict_network("main")
+
+
 def test_other_lookup_forms(dm):
     """RowwiseQuantizedSparseLengthsWeightedSum and EmbeddingBagByteRowwiseOffsets
     as instructions of one function."""

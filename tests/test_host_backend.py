@@ -427,3 +427,48 @@ def test_lookups_with_input_lengths_read_host_made_bag_positions():
     m.compile(f)
     rows = [r for r in H.parse_listing(m.describe(f)) if r["phase"] == "launch"]
     assert [r["kernel"] for r in rows] == ["mi355x_copy_u8", "mi355x_frwq_slws"]
+
+
+def test_wide_kinds_transposes_and_3d_convolutions_compile():
+    """int16 / int32 Quantize, RescaleQuantized, Dequantize; shuffles other than
+    the two tiled ones; the NTHWC form of ChannelwiseQuantizedConvolution."""
+    m = H.Module("wide")
+    x = m.placeholder("x", (4, 6), H.FLOAT, np.float32)
+    y = m.placeholder("y", (4, 6), H.FLOAT, np.float32)
+    f = m.function("main")
+    for kind, tag in ((H.INT16Q, "i16"), (H.INT32Q, "i32")):
+        q = m.activation(f, f"q_{tag}", (4, 6), kind, 0.01, 3)
+        r = m.activation(f, f"r_{tag}", (4, 6), kind, 0.02, -5)
+        m.instruction(f, H.QUANTIZE, f"quant_{tag}", [q, x])
+        m.instruction(f, H.RESCALE_QUANTIZED, f"rescale_{tag}", [r, q])
+        m.instruction(f, H.DEQUANTIZE, f"dequant_{tag}", [y, r])
+    t_in = m.placeholder("t_in", (2, 3, 4, 5), H.INT8Q, np.int8, 0.1, 1)
+    t_out = m.placeholder("t_out", (2, 4, 5, 3), H.INT8Q, np.int8, 0.1, 1)
+    m.instruction(f, H.TRANSPOSE, "nchw2nhwc", [t_out, t_in], [0, 2, 3, 1])
+    f_in = m.placeholder("f_in", (3, 5), H.FLOAT, np.float32)
+    f_out = m.placeholder("f_out", (5, 3), H.FLOAT, np.float32)
+    m.instruction(f, H.TRANSPOSE, "float_t", [f_out, f_in], [1, 0])
+    m.compile(f)
+    k = [r["kernel"] for r in H.parse_listing(m.describe(f)) if r["phase"] == "launch"]
+    assert k == ["mi355x_quantize_i16", "mi355x_rescale_i16", "mi355x_dequantize_i16",
+                 "mi355x_quantize_i32", "mi355x_rescale_i32", "mi355x_dequantize_i32",
+                 "mi355x_transpose_nd", "mi355x_transpose_nd"]
+    # mismatched kinds and a shuffle that is no permutation are refused
+    q16 = m.activation(f, "q16b", (4, 6), H.INT16Q, 0.01, 0)
+    q32 = m.activation(f, "q32b", (4, 6), H.INT32Q, 0.01, 0)
+    assert not m.is_op_supported(H.RESCALE_QUANTIZED, [q32, q16])[0]
+    assert not m.is_op_supported(H.TRANSPOSE, [t_out, t_in], [0, 2, 2, 1])[0]
+    assert not m.is_op_supported(H.TRANSPOSE, [t_out, t_in], [0, 3, 2, 1])[0]   # shape mismatch
+
+    c = cases.cwq_conv3d_case(5, N=1, T=4, H=5, W=5, IC=4, OC=6, kernel=(2, 3, 3),
+                              stride=(1, 2, 1), pads=(1, 0, 1, 1, 0, 2))
+    mc, fc = host_cases.cwq_conv3d_module(c, (2, 3, 3), (1, 2, 1), (1, 0, 1, 1, 0, 2))
+    mc.compile(fc)
+    rows = [r for r in H.parse_listing(mc.describe(fc)) if r["phase"] == "launch"]
+    assert [r["kernel"] for r in rows] == ["mi355x_cwq_conv3d_i8"]
+    g = c["geom"]
+    assert (rows[0]["OT"], rows[0]["OH"], rows[0]["OW"]) == (g.OT, g.OH, g.OW)
+    # an output shape that the attributes do not give is refused
+    bad, fb = host_cases.cwq_conv3d_module(c, (2, 3, 3), (1, 1, 1), (1, 0, 1, 1, 0, 2))
+    with pytest.raises(H.HostError):
+        bad.compile(fb)

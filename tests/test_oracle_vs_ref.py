@@ -205,3 +205,54 @@ def test_rwq_slws_vs_ref(idt):
     w = rng.random(idx.size).astype(np.float32)
     np.testing.assert_array_equal(go.rwq_slws_f32(data, scales, offsets, w, idx, lengths),
                                   ref.rwq_slws_f32(data, scales, offsets, w, idx, lengths))
+
+
+@pytest.mark.parametrize("fastmath", FM)
+@pytest.mark.parametrize("bits", [16, 32])
+def test_wide_elementwise_vs_ref(bits, fastmath):
+    rng = np.random.default_rng(bits)
+    dt = np.int16 if bits == 16 else np.int32
+    lim = 2 ** (bits - 1)
+    q = np.concatenate([rng.integers(-lim, lim, 800), [-lim, lim - 1, 0]]).astype(dt)
+    x = np.concatenate([rng.normal(0, 1000, 800), rng.normal(0, 1e6, 200),
+                        (np.arange(-40, 40) + 0.5)]).astype(np.float32)
+    for scale, off in [(0.5, 3), (0.013, -77), (40.0, 1000)]:
+        if not fastmath:    # fast-math may replace the division (see the int8 test)
+            np.testing.assert_array_equal(go.quantize_wide(x, scale, off, bits),
+                                          ref.quantize_wide(x, scale, off, bits))
+        np.testing.assert_array_equal(go.dequantize_wide(q, scale, off),
+                                      ref.dequantize_wide(q, scale, off, fastmath))
+    for r in (0.0003, 0.05, 0.5, 1.0, 1.7, 8.0):
+        pre, post, sc, _ = go.quantize_scale_offset_32to8(r, 0)
+        io, oo = int(rng.integers(-128, 128)), int(rng.integers(-128, 128))
+        np.testing.assert_array_equal(go.rescale_wide(q, oo, io, pre, post, sc),
+                                      ref.rescale_wide(q, oo, io, pre, post, sc, fastmath))
+
+
+def test_transpose_vs_ref():
+    rng = np.random.default_rng(5)
+    for nd in range(2, 7):     # the reference's loop nests cover 2 to 6 dimensions
+        for _ in range(4):
+            shape = tuple(int(v) for v in rng.integers(1, 6, nd))
+            sh = [int(v) for v in rng.permutation(nd)]
+            x = rng.integers(-128, 128, shape).astype(np.int8)
+            np.testing.assert_array_equal(go.transpose(x, sh), ref.transpose_i8(x, sh))
+
+
+@pytest.mark.parametrize("fastmath", FM)
+def test_cwq_conv3d_vs_ref(fastmath):
+    rng = np.random.default_rng(6)
+    for i in range(8):
+        kt, kh, kw = (int(v) for v in rng.integers(1, 4, 3))
+        grp = int(rng.choice([1, 1, 2]))
+        kw_ = dict(N=int(rng.integers(1, 3)), T=int(rng.integers(kt, kt + 4)),
+                   H=int(rng.integers(kh, kh + 5)), W=int(rng.integers(kw, kw + 5)),
+                   IC=grp * int(rng.integers(1, 6)), OC=grp * int(rng.integers(1, 6)),
+                   kernel=(kt, kh, kw), stride=tuple(int(v) for v in rng.integers(1, 3, 3)),
+                   pads=tuple(int(v) for v in rng.integers(0, 2, 6)), group=grp,
+                   act=int(rng.choice([go.ACT_NONE, go.ACT_RELU, go.ACT_CLIP, go.ACT_LEAKY_RELU])),
+                   symmetric=bool(i % 2), in_offset=int(rng.integers(-128, 128)),
+                   out_offset=int(rng.integers(-128, 100)), bias_i8=bool(i % 3 == 0))
+        c = cases.cwq_conv3d_case(900 + i, **kw_)
+        np.testing.assert_array_equal(go.cwq_conv3d_i8(*cases.cwq_conv_args(c)),
+                                      ref.cwq_conv3d_i8(*cases.cwq_conv_args(c), fastmath=fastmath))
