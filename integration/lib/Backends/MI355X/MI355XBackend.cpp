@@ -111,21 +111,28 @@ static bool fusedLookupTypesOk(ElemKind data, bool hasWeights, ElemKind weights,
   }
 }
 
+static bool isQuantizedIntKind(ElemKind k) {
+  return k == ElemKind::Int8QTy || k == ElemKind::Int16QTy || k == ElemKind::Int32QTy;
+}
+
 bool MI355XBackend::isOpSupported(const NodeInfo &NI) const {
   // "X ==> Y" below: Node X is IRGen'd into Instruction Y.
   switch (NI.getKind()) {
 
   // ---- the quantization boundary -----------------------------------------
+  // (int8 is the hot path; the 16- and 32-bit forms of
+  // libjit.cpp:3004-3056 run as plain elementwise kernels)
   case Kinded::Kind::QuantizeNodeKind:
     return NI.getInElemTy(QuantizeNode::InputIdx) == ElemKind::FloatTy &&
-           NI.getOutElemTy(QuantizeNode::ResultIdx) == ElemKind::Int8QTy;
+           isQuantizedIntKind(NI.getOutElemTy(QuantizeNode::ResultIdx));
 
   case Kinded::Kind::DequantizeNodeKind:
-    return NI.getInElemTy(DequantizeNode::InputIdx) == ElemKind::Int8QTy &&
+    return isQuantizedIntKind(NI.getInElemTy(DequantizeNode::InputIdx)) &&
            NI.getOutElemTy(DequantizeNode::ResultIdx) == ElemKind::FloatTy;
 
   case Kinded::Kind::RescaleQuantizedNodeKind:
-    return NI.allInputsAndOutputsHaveSameElemKind({ElemKind::Int8QTy});
+    return NI.allInputsAndOutputsHaveSameElemKind(
+        {ElemKind::Int8QTy, ElemKind::Int16QTy, ElemKind::Int32QTy});
 
   // ---- matrix-core operators ---------------------------------------------
   case Kinded::Kind::FullyConnectedNodeKind:
@@ -270,8 +277,14 @@ bool MI355XBackend::isOpSupported(const NodeInfo &NI) const {
            NI.getOutElemTy(ConvertToNode::ResultIdx) == ElemKind::FloatTy;
 
   case Kinded::Kind::InsertTensorNodeKind:
-  case Kinded::Kind::TransposeNodeKind:
     return NI.allInputsAndOutputsHaveSameElemKind({ElemKind::Int8QTy});
+
+  // any shuffle of up to six dimensions, any plain element kind
+  // (libjit_transpose_i8 / _f / _u / _b, libjit.cpp:3162-3184)
+  case Kinded::Kind::TransposeNodeKind:
+    return NI.allInputsAndOutputsHaveSameElemKind(
+        {ElemKind::Int8QTy, ElemKind::Int16QTy, ElemKind::Int32QTy, ElemKind::FloatTy,
+         ElemKind::Float16Ty, ElemKind::Int32ITy, ElemKind::Int64ITy, ElemKind::BoolTy});
 
   case Kinded::Kind::GatherNodeKind:
     return NI.allInputsAndOutputsHaveSameElemKind({ElemKind::Int8QTy},

@@ -78,6 +78,9 @@ static bool toHostType(const Type &t, hm::Type &out) {
   case ElemKind::Int32QTy:
     k = hm::ElemKind::Int32QTy;
     break;
+  case ElemKind::Int16QTy:
+    k = hm::ElemKind::Int16QTy;
+    break;
   case ElemKind::Int32ITy:
     k = hm::ElemKind::Int32ITy;
     break;
@@ -292,8 +295,30 @@ private:
     }
     case Kinded::Kind::ChannelwiseQuantizedConvolutionInstKind: {
       const auto *C = cast<ChannelwiseQuantizedConvolutionInst>(&I);
+      if (C->getSrc()->dims().size() == 5) {
+        // NTHWC: kernels {T,H,W}, strides {T,H,W}, pads {near, far, top, bottom,
+        // left, right} (PaddingNFTBLR), group, fused activation, in the order
+        // the host layer's 3-D form takes its integer attributes
+        std::vector<int64_t> ia;
+        for (auto v : C->getKernels()) ia.push_back((int64_t)v);
+        for (auto v : C->getStrides()) ia.push_back((int64_t)v);
+        for (auto v : C->getPads()) ia.push_back((int64_t)v);
+        if (ia.size() != 12) {
+          return unsupported(I, "a 3-D convolution needs 3 kernels, 3 strides and 6 pads");
+        }
+        for (auto d : C->getDilation()) {
+          if (d != 1) return unsupported(I, "dilated 3-D convolutions are not supported");
+        }
+        ia.push_back((int64_t)C->getGroup());
+        ia.push_back((int64_t)C->getFusedActivation());
+        std::vector<int> ops;
+        ASSIGN_VALUE_OR_RETURN_ERR(ops, operandIds(I));
+        fn_->addInstruction(hm::Kind::ChannelwiseQuantizedConvolution, I.getName().str(), ops,
+                            std::move(ia), C->getFusedActivationArgs());
+        return Error::success();
+      }
       if (C->getSrc()->dims().size() != 4) {
-        return unsupported(I, "3-D channelwise convolutions are not supported");
+        return unsupported(I, "needs an NHWC or NTHWC input");
       }
       const hm::ConvAttrs a = convAttrs(C);
       std::vector<int> ops;

@@ -43,6 +43,8 @@ ALLOW = {
         "ChannelwiseQuantizedConv2D", "ChannelwiseQuantizedConv2D_Int32Bias_SmallFilterData",
         "ChannelwiseQuantizedConv2D_Int32Bias_ZeroBiasData",
         "ChannelwiseQuantizedConv2D_NonZero_QuantizedBias",
+        # ... and its NTHWC form (libjit_conv.cpp:244-349)
+        "ChannelwiseQuantizedConv3D",
         # fused-rowwise pooled lookups (libjit.cpp:1253-1276, 2416-2481;
         # InterpreterNodes.cpp:5764-5889)
         "FusedRowwiseQuantizedSparseLengthsWeightedSum_Float",
@@ -62,7 +64,11 @@ ALLOW = {
         # int8 glue
         "Int8AvgPool", "Int8AvgPoolCountExcludePads", "Int8MaxPool", "Relu_Int8",
         "GatherDataInt8IdxInt32", "GatherDataInt8IdxInt64", "QuantizeSimpleInt8",
+        "QuantizeSimpleInt16", "QuantizeSimpleInt32",
         "TestQuantizedRescaleSequence",
+        # Transpose of 2 to 6 dimensions, any plain element kind (libjit.cpp:565-653)
+        "Transpose2Dims", "FP16Transpose2Dims", "BoolTranspose2Dims", "Transpose6Dims",
+        "Transpose3Dims_Float", "Transpose3Dims_Float16", "Transpose3Dims_Int8",
         # RowwiseQuantizedFullyConnected / FullyConnected
         "rowwiseQuantizedFCTest_Int8_BiasInt8", "rowwiseQuantizedFCTest_Int8_BiasInt32",
         "rowwiseQuantizedFCTestSymmetric",
