@@ -75,6 +75,9 @@ def parse():
                          "fc|conv_c3|quantize|dequantize|rescale|copy|resnet50|dlrm")
     ap.add_argument("--shape", default="",
                     help="MxKxN of --only fc (a RowwiseQuantizedFullyConnected of that shape)")
+    ap.add_argument("--hint", action="store_true",
+                    help="--only fc: run with the requantisation hint the backend derives "
+                         "from the launch's constants")
     ap.add_argument("--tile", type=int, default=-1,
                     help="force a workgroup tile for the matrix-core legs of --only "
                          "(0..5, see mi355x_gemm_tile_override; default: chosen from the shape)")
@@ -373,7 +376,7 @@ def oracle_rows_check(capi, c, d_out, M, rows):
 
 
 def bench_fc(capi, cases, M, K, N, steps, warmup, seed=5, zero_leg=False, check=True,
-             clock=False):
+             clock=False, use_hint=False):
     c = cases.rwq_fc_case(seed, M, K, N) if M * K <= (1 << 24) else None
     rng = np.random.default_rng(seed)
     if c is None:
@@ -397,6 +400,15 @@ def bench_fc(capi, cases, M, K, N, steps, warmup, seed=5, zero_leg=False, check=
                               c["in_offset"], c["bias_offset"], True,
                               w_row_sums=d_sums, stream=stream)
 
+    hint = 0
+    if use_hint:
+        # as the backend compiles it: the requantisation hints derived from the
+        # launch's constants (host-verified bounds)
+        hint = capi.gemm_requant_hint_host(K, c["in_offset"], c["out_offset"], c["w_offsets"],
+                                           c["bias"], c["bias_offset"], c["bias_pre"],
+                                           c["bias_post"], c["bias_scale"], c["out_pre"],
+                                           c["out_post"], c["out_scale"])
+        capi.check(capi.lib().mi355x_gemm_requant_hint(hint))
     clocks = None
     if clock:
         # the shader clock the part holds while this kernel runs, sampled from
@@ -443,7 +455,9 @@ def bench_fc(capi, cases, M, K, N, steps, warmup, seed=5, zero_leg=False, check=
         capi.sync()
         nsec = timed_launches(capi, step, steps, warmup)
         normal = dict(ms=nsec * 1e3, tops=ops / nsec / 1e12)
-    return dict(workload=f"rwq_fc M{M} K{K} N{N}", ms=sec * 1e3,
+    if use_hint:
+        capi.check(capi.lib().mi355x_gemm_requant_hint(0))
+    return dict(workload=f"rwq_fc M{M} K{K} N{N}", requant_hint=hint, ms=sec * 1e3,
                 tops=ops / sec / 1e12, zero_operands=zero, normal_weights=normal,
                 shader_clock=clocks,
                 parity_with_oracle=(None if parity is None else parity[0]),
@@ -720,7 +734,7 @@ def main():
                 "dequantize", "rescale", "copy"):
         if only == "fc":
             M, K, N = (int(v) for v in args.shape.split("x"))
-            r = bench_fc(capi, cases, M, K, N, args.steps, args.warmup)
+            r = bench_fc(capi, cases, M, K, N, args.steps, args.warmup, use_hint=args.hint)
         elif only == "fc_large":
             r = bench_fc(capi, cases, 8192, 4096, 4096, args.steps, args.warmup)
         elif only == "fc_large_zero":

@@ -11,6 +11,7 @@
 // input offset and the dense contraction of gemm_i8.h applies unchanged.
 #include "gemm_i8.h"
 #include "conv_halo.h"
+#include "gemm_stream.h"
 
 namespace mi355x {
 
@@ -181,6 +182,21 @@ static int conv_common(int8_t *out, const int8_t *in, const int8_t *filter,
       ep.fast = g_requant_hint & 3;
       return conv_halo_launch(in, filter, g, ep, lds, rows, as_stream(stream));
     }
+  }
+  // Pointwise convolutions (any stride) over 64, 128 or 256 channels: the
+  // streaming kernel (gemm_stream.h), by its shape rule or when tile 8 is
+  // asked for.
+  if (g->KH == 1 && g->KW == 1 && g->padT == 0 && g->padL == 0 && g->group == 1 &&
+      (long long)(g->OH - 1) * g->strideH < g->IH && (long long)(g->OW - 1) * g->strideW < g->IW &&
+      (g_tile_override == 8 || (g_tile_override < 0 && stream_applies((int)M, OCg))) &&
+      stream_can_run((int)M, OCg, (int)K, need_sa, need_sb, al_a && al_b, ep)) {
+    StreamRows R;
+    R.in = in; R.ld = g->IC;
+    R.dense = g->strideH == 1 && g->strideW == 1 && g->OH == g->IH && g->OW == g->IW;
+    R.OW = g->OW; R.OHW = g->OH * g->OW; R.IH = g->IH; R.IW = g->IW; R.IC = g->IC;
+    R.sH = g->strideH; R.sW = g->strideW;
+    ep.fast = g_requant_hint & 3;
+    return gemm_stream_launch(R, filter, ep, (int)M, OCg, (int)K, as_stream(stream));
   }
   // A pointwise convolution over the whole image is a plain matrix product:
   // row m of A is pixel m of the input, no taps to locate and no padding.

@@ -57,12 +57,8 @@ constexpr size_t kHaloMaxLds =
 constexpr int kHaloFilterChunks = kHaloBN * (kHaloK / 16);   // 16-byte chunks
 
 // Filter row (output channel) c of a workgroup's 64 sits in LDS slot
-// halo_filter_slot(c), the inverse of perm_row16 within each 32-channel tile:
-// lane (pixel, h) then holds channels 32 j + 16 h + [0, 16) of its pixel in
-// the sixteen accumulators of tile j, in order (see gemm_i8.h).
-__device__ __forceinline__ int halo_filter_slot(int c) {
-  return (c & 32) + 8 * ((c >> 2) & 3) + 4 * ((c >> 4) & 1) + (c & 3);
-}
+// perm_slot16(c): lane (pixel, h) then holds channels 32 j + 16 h + [0, 16) of
+// its pixel in the sixteen accumulators of tile j, in order (see gemm_i8.h).
 constexpr int kHaloParBytes = kParArrays * kHaloBN * 4;
 
 // SKIP leaves phases out so that the others can be timed (1: staging, 2: the
@@ -130,7 +126,7 @@ __global__ __launch_bounds__(512, 2) void conv3x3_halo_kernel(HaloConv cv, Epilo
     auto filter_store = [&](int c, const int4 &v) {
       if (c < kHaloFilterChunks) {
         const int row = c / (kHaloK / 16), kc = c - row * (kHaloK / 16);
-        *reinterpret_cast<int4 *>(s_filter + halo_filter_slot(row) * kHaloFRow + kc * 16) = v;
+        *reinterpret_cast<int4 *>(s_filter + perm_slot16(row) * kHaloFRow + kc * 16) = v;
       }
     };
     // first batch of both in flight together

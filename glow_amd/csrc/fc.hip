@@ -6,6 +6,7 @@
 // scalars for the other two.
 #include "gemm_i8.h"
 #include "gemm_skinny.h"
+#include "gemm_stream.h"
 
 namespace mi355x {
 
@@ -88,6 +89,15 @@ static int fc_common(int8_t *out, const int8_t *in, const int8_t *w_nk,
     ep.fast = g_requant_hint & 3;
     return gemm_skinny_launch(A, B, ep, g, as_stream(stream));
   }
+  // many rows over 64, 128 or 256 inputs: the streaming kernel (by its shape
+  // rule, or tile 8)
+  if ((g_tile_override == 8 || (g_tile_override < 0 && stream_applies((int)M, (int)N))) &&
+      stream_can_run((int)M, (int)N, (int)K, need_sa, need_sb, aligned, ep)) {
+    StreamRows R{};
+    R.in = in; R.ld = (long long)K; R.dense = 1;
+    ep.fast = g_requant_hint & 3;
+    return gemm_stream_launch(R, w_nk, ep, (int)M, (int)N, (int)K, as_stream(stream));
+  }
   return gemm_dispatch(A, B, ep, (int)M, (int)N, (int)K, 1, 0, need_sa, need_sb,
                        aligned, as_stream(stream));
 }
@@ -99,7 +109,7 @@ using namespace mi355x;
 extern "C" {
 
 int mi355x_gemm_tile_override(int tile) {
-  MI355X_REQUIRE(tile >= -1 && tile <= 7, "tile %d outside [-1, 7]", tile);
+  MI355X_REQUIRE(tile >= -1 && tile <= 8, "tile %d outside [-1, 8]", tile);
   g_tile_override = tile;
   return MI355X_OK;
 }

@@ -408,6 +408,12 @@ __device__ __forceinline__ int perm_row16(int rho) {
   return 16 * ((rho >> 2) & 1) + 4 * (rho >> 3) + (rho & 3);
 }
 
+// The slot (row position in LDS) of weight row c when slots are read in
+// order: the inverse of perm_row16 within each group of 32 rows.
+__device__ __forceinline__ int perm_slot16(int c) {
+  return (c & ~31) + 8 * ((c >> 2) & 3) + 4 * ((c >> 4) & 1) + (c & 3);
+}
+
 // A lane then needs the constants of 16 columns per sub-tile instead of one
 // column's: they are kept in LDS as kParArrays arrays of BN ints (four
 // consecutive columns per ds_read_b128, one address per half wave).
@@ -430,7 +436,10 @@ __device__ __forceinline__ void par_table_store(int32_t *s_par, int c, const Col
   if (ep.bias)
     colc += (uint32_t)scale_i32((int32_t)((uint32_t)r.bias - (uint32_t)r.boff), r.bpre, r.bpost,
                                 r.bscale, 0);
-  uint32_t fold = (r.opost > 0 ? (1u << (r.opost - 1)) : 0u) + ((uint32_t)ep.out_off << r.opost);
+  // the rounding term of the post-shift, with what the variant may fold into
+  // it: the output offset (modes 1 and 3) and the column constant (mode 3)
+  uint32_t fold = r.opost > 0 ? (1u << (r.opost - 1)) : 0u;
+  if (mode != 0) fold += (uint32_t)ep.out_off << r.opost;
   if (mode == 3) fold += colc * (uint32_t)r.oscale;
   s_par[kParColc * BN + c] = (int32_t)colc;
   s_par[kParPre * BN + c] = r.opre;
@@ -449,12 +458,12 @@ __device__ __forceinline__ int4 requant_pack16(const v16i &acc, const int32_t *p
   for (int q = 0; q < 4; q++) {
     const v4i scale = *reinterpret_cast<const v4i *>(par + kParScale * BN + 4 * q);
     const v4i post = *reinterpret_cast<const v4i *>(par + kParPost * BN + 4 * q);
-    v4i colc, pre, fold;
+    v4i colc, pre;
     if constexpr (MODE != 3) {
       colc = *reinterpret_cast<const v4i *>(par + kParColc * BN + 4 * q);
       pre = *reinterpret_cast<const v4i *>(par + kParPre * BN + 4 * q);
     }
-    if constexpr (MODE != 0) fold = *reinterpret_cast<const v4i *>(par + kParFold * BN + 4 * q);
+    const v4i fold = *reinterpret_cast<const v4i *>(par + kParFold * BN + 4 * q);
     uint32_t b[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
@@ -466,7 +475,11 @@ __device__ __forceinline__ int4 requant_pack16(const v16i &acc, const int32_t *p
         y = (int32_t)((uint32_t)__mul24((int32_t)(x + (uint32_t)colc[i]) >> pre[i], scale[i]) +
                       (uint32_t)fold[i]) >> post[i];
       } else {
-        y = scale_i32((int32_t)(x + (uint32_t)colc[i]), pre[i], post[i], scale[i], ep.out_off);
+        // scale_i32 with the rounding term from the table: in this layout every
+        // accumulator has its own column, so nothing per column is amortised
+        const uint32_t m = (uint32_t)((int32_t)(x + (uint32_t)colc[i]) >> pre[i]) *
+                               (uint32_t)scale[i] + (uint32_t)fold[i];
+        y = (int32_t)((uint32_t)((int32_t)m >> post[i]) + (uint32_t)ep.out_off);
       }
       if constexpr (LEAKY) {
         if (y < ep.out_off)

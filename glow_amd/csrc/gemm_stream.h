@@ -1,0 +1,200 @@
+// The int8 contraction for short K and many rows: pointwise convolutions of an
+// image network's early stages and FullyConnected layers over 64, 128 or 256
+// inputs, where a launch is all memory traffic and requantisation and the
+// tiled kernels of gemm_i8.h spend their time in load latency, barriers and
+// output staging.
+//
+//   * the weights of a workgroup's column slice (at most 256 columns, 37 KB)
+//     and the columns' requantisation constants are put in LDS once; from then
+//     on the workgroup's waves never meet again;
+//   * a wave walks over tiles of 32 rows: a lane loads its row's K bytes
+//     straight from global memory into registers in the matrix-core layout
+//     (every byte of A is read by exactly one lane), multiplies them with the
+//     weight fragments read from LDS, 32 columns at a time, and requantises,
+//     packs and stores sixteen output bytes per lane from registers
+//     (the transposed-accumulator epilogue of gemm_i8.h), with the fused
+//     residual add read the same way;
+//   * latency is hidden by occupancy (four waves per SIMD) instead of by a
+//     pipeline: while one wave waits for its rows, the others multiply and
+//     requantise.
+//
+// Results are bit for bit those of the tiled kernels (same integer sums, same
+// requantisation).
+#ifndef GLOW_MI355X_GEMM_STREAM_H
+#define GLOW_MI355X_GEMM_STREAM_H
+
+#include "gemm_i8.h"
+
+namespace mi355x {
+
+constexpr int kStreamMaxBN = 256;   // columns per workgroup slice (and the table's stride)
+constexpr int kStreamParBytes = kParArrays * kStreamMaxBN * 4;
+
+// Rows of A: dense (row m at in + m * ld), or the pixels a strided pointwise
+// convolution reads (output pixel m of an [N, OH, OW] grid -> input pixel
+// (n, oh * sH, ow * sW) of an [N, IH, IW, IC] tensor).
+struct StreamRows {
+  const int8_t *in;
+  long long ld;
+  int dense;
+  int OW, OHW, IH, IW, IC, sH, sW;
+  __device__ __forceinline__ const int8_t *row(int m) const {
+    if (dense) return in + (long long)m * ld;
+    const int n = m / OHW, r = m - n * OHW;
+    const int oh = r / OW, ow = r - oh * OW;
+    return in + (((long long)n * IH + (long long)oh * sH) * IW + (long long)ow * sW) * IC;
+  }
+};
+
+template <int KS, int MODE, bool LEAKY>
+__device__ __forceinline__ void stream_tiles(const StreamRows &A, const int8_t *s_w,
+                                             const int32_t *s_par, const Epilogue &ep, int M,
+                                             int N, int n0, int bn, int tiles32, int first,
+                                             int step, int l32, int lhi) {
+  constexpr int WSTRIDE = KS * 32 + 16;
+  int32_t lo, hi;
+  activation_clamp(ep, lo, hi);
+  const bool fast = fused_out_is_fast(ep);
+  const FusedAddConsts fc = fused_add_consts(ep.add);
+  const bool vec = (ep.ldc % 16 == 0) && (n0 % 16 == 0) &&
+                   (((((uintptr_t)ep.out) | ((uintptr_t)ep.add.res)) & 15) == 0);
+  const int8_t *w_lane = s_w + l32 * WSTRIDE + lhi * 16;
+  for (int t = first; t < tiles32; t += step) {
+    const int m = t * 32 + l32;
+    // rows past the end re-read the last row; their results are not stored
+    const int8_t *ar = A.row(min(m, M - 1)) + lhi * 16;
+    v4i af[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) af[ks] = *reinterpret_cast<const v4i *>(ar + ks * 32);
+    int8_t *out_row = ep.out + (long long)m * ep.ldc;
+    const int8_t *res_row = ep.add.res ? ep.add.res + (long long)m * ep.ldc : nullptr;
+    for (int j = 0; j < bn / 32; j++) {
+      v16i acc;
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[r] = 0;
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) {
+        const v4i b = *reinterpret_cast<const v4i *>(w_lane + j * 32 * WSTRIDE + ks * 32);
+        // weights first: the result's rows are columns of the output
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(b, af[ks], acc, 0, 0, 0);
+      }
+      const int cl = j * 32 + 16 * lhi;
+      const int4 v = requant_pack16<MODE, LEAKY, kStreamMaxBN>(acc, s_par + cl, ep, lo, hi);
+      if (m < M) store16(v, out_row, res_row, n0 + cl, N, vec, ep, fc, fast);
+    }
+  }
+}
+
+// KS: K / 32 (2, 4 or 8). blockIdx.y: column slice of bn columns.
+template <int KS>
+__global__ __launch_bounds__(256, 4) void gemm_i8_stream_kernel(StreamRows A, const int8_t *W,
+                                                                Epilogue ep, int M, int N, int bn,
+                                                                int tiles32) {
+  constexpr int K = KS * 32, WSTRIDE = K + 16;
+  extern __shared__ __attribute__((aligned(16))) int8_t lds[];
+  int32_t *s_par = reinterpret_cast<int32_t *>(lds);
+  int8_t *s_w = lds + kStreamParBytes;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, lhi = lane >> 5;
+  const int n0 = blockIdx.y * bn;
+  const int cols = min(bn, N - n0);          // a multiple of 32
+  const int mode = requant_mode(ep);
+
+  // the slice's constants and weights -> LDS, once
+  if (tid < cols) {
+    ColRaw col[1];
+    load_col_raw<1, kStreamMaxBN>(col, ep, N, n0, 0, 0, tid);
+    par_table_store<kStreamMaxBN>(s_par, tid, col[0], ep, K, mode);
+  }
+  {
+    constexpr int CH = K / 16;               // 16-byte chunks per weight row
+    const int chunks = cols * CH;
+    const int8_t *w0 = W + (long long)n0 * K;
+    for (int base = 0; base < chunks; base += 256 * 4) {
+      int4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int c = min(base + tid + u * 256, chunks - 1);
+        v[u] = *reinterpret_cast<const int4 *>(w0 + (long long)c * 16);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int c = base + tid + u * 256;
+        if (c < chunks) {
+          const int row = c / CH, kc = c - row * CH;
+          *reinterpret_cast<int4 *>(s_w + perm_slot16(row) * WSTRIDE + kc * 16) = v[u];
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  // from here on every wave is on its own
+  const int first = blockIdx.x * 4 + wave, step = gridDim.x * 4;
+  if (ep.act == 5)
+    stream_tiles<KS, 0, true>(A, s_w, s_par, ep, M, N, n0, cols, tiles32, first, step, l32, lhi);
+  else if (mode == 3)
+    stream_tiles<KS, 3, false>(A, s_w, s_par, ep, M, N, n0, cols, tiles32, first, step, l32, lhi);
+  else if (mode == 1)
+    stream_tiles<KS, 1, false>(A, s_w, s_par, ep, M, N, n0, cols, tiles32, first, step, l32, lhi);
+  else
+    stream_tiles<KS, 0, false>(A, s_w, s_par, ep, M, N, n0, cols, tiles32, first, step, l32, lhi);
+}
+
+// Whether the streaming kernel can run this product at all: K of 64, 128 or
+// 256, 16-byte aligned operands and output, whole 32-column tiles, weight
+// offsets all zero with their row sums precomputed (no in-kernel row sums).
+static bool stream_can_run(int M, int N, int K, bool need_sa, bool need_sb, bool aligned,
+                           const Epilogue &ep) {
+  if (need_sa || need_sb || !aligned) return false;
+  if (K != 64 && K != 128 && K != 256) return false;
+  if (N % 32 != 0 || M < 1) return false;
+  if (ep.ldc % 16 != 0 || (((((uintptr_t)ep.out) | ((uintptr_t)ep.add.res)) & 15) != 0))
+    return false;
+  return true;
+}
+
+// Whether it is the default for such a product. Measured against the best
+// tiled kernel (us, M200704): K64 N64 9.0 vs 12.2, K64 N256 27.0 vs 28.2, K256
+// N64 15.9 vs 18.5, K256 N128 24.2 vs 25.5; with more columns the weight
+// slices multiply the reads of A and the tiled kernels are level or ahead
+// (M50176 K128 N512 19.9 vs 18.6, M12544 K256 N1024 15.2 vs 14.3).
+static bool stream_applies(int M, int N) { return M >= 4096 && N <= kStreamMaxBN; }
+
+static int gemm_stream_launch(const StreamRows &A, const int8_t *W, const Epilogue &ep, int M,
+                              int N, int K, hipStream_t st) {
+  // columns per slice: the weights of a slice stay under ~37 KB of LDS
+  const int bn = K == 256 ? 128 : kStreamMaxBN;
+  const int slices = (N + bn - 1) / bn;
+  const size_t lds = (size_t)kStreamParBytes + (size_t)std::min(bn, N) * (K + 16);
+  const int tiles32 = (M + 31) / 32;
+  int dev = 0, cus = 256;
+  if (hipGetDevice(&dev) == hipSuccess) {
+    int v = 0;
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+      cus = v;
+  }
+  const int per_cu = (int)std::min<size_t>(4, (160 * 1024) / lds);
+  long long gx = std::max(1LL, (long long)cus * per_cu / slices);
+  gx = std::min<long long>(gx, (tiles32 + 3) / 4);
+  MI355X_REQUIRE(slices < 65536, "problem too large");
+  const dim3 grid((unsigned)gx, (unsigned)slices), block(256);
+  switch (K) {
+  case 64:
+    hipLaunchKernelGGL(gemm_i8_stream_kernel<2>, grid, block, lds, st, A, W, ep, M, N, bn, tiles32);
+    break;
+  case 128:
+    hipLaunchKernelGGL(gemm_i8_stream_kernel<4>, grid, block, lds, st, A, W, ep, M, N, bn, tiles32);
+    break;
+  default:
+    hipLaunchKernelGGL(gemm_i8_stream_kernel<8>, grid, block, lds, st, A, W, ep, M, N, bn, tiles32);
+    break;
+  }
+  return check_launch("gemm_i8_stream");
+}
+
+} // namespace mi355x
+#endif

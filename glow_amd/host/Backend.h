@@ -109,7 +109,7 @@ struct KernelLaunch {
   // Issues the launch (with its tile, if it has one).
   int launch(const DeviceBindings &b) const;
 };
-constexpr int kNumTiles = 8;
+constexpr int kNumTiles = 9;
 
 class MI355XFunction {
 public:

@@ -448,7 +448,11 @@ int mi355x_matmul_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs_kn,
  * symmetric weights, precomputed row sums and K % 32 == 0 only; launches it
  * cannot serve ignore it), 7 = the 3x3 stride-1 convolution over 64 input
  * channels with filter and input rows resident in LDS (other launches ignore
- * it; tiles 0..6 keep such a convolution on the tiled kernels); -1 = chosen
+ * it; tiles 0..6 keep such a convolution on the tiled kernels), 8 = the
+ * streaming kernel for K of 64, 128 or 256 (FullyConnected and pointwise
+ * convolutions with symmetric weights and precomputed row sums: weights and
+ * constants resident in LDS, rows straight from memory into registers; other
+ * launches ignore it); -1 = chosen
  * from the problem shape (the default). Results do not depend on the tile. A device
  * manager uses it to time the candidates of each layer once, when a network is
  * loaded. */
