@@ -17,10 +17,11 @@
 //     K loop is ds_read_b128 + v_mfma with nothing else in it;
 //   * the filter is the first matrix-core operand and its rows are placed in LDS
 //     in such an order that a lane's sixteen accumulators of a channel tile are
-//     sixteen consecutive channels of one pixel: they are requantised, packed
-//     and written with one 16-byte store each, straight from registers. There is
-//     no barrier after the one that ends the staging: every wave finishes its
-//     32 pixels on its own.
+//     sixteen consecutive channels of one pixel: they are requantised and
+//     packed in registers, and leave through a wave-private transpose in the
+//     (by then free) halo area, so that whole 64-byte pixels are stored (stores
+//     of 16-byte pieces straight from registers wrote 1.5 x the bytes at the
+//     memory side).
 //
 // Pixels and filter rows are 16 bytes apart from a power-of-two stride in LDS
 // (80 and 592 bytes), which spreads the 16-byte fragment reads of consecutive
@@ -53,13 +54,35 @@ constexpr int kHaloFRow = kHaloK + 16;        // bytes between filter rows in LD
 constexpr int kHaloFilterBytes = kHaloBN * kHaloFRow;
 // (rows + 2) x (OW + 2) pixels with rows * OW <= 256 is largest for one row of 256
 constexpr size_t kHaloMaxLds =
-    kHaloFilterBytes + 5 * kHaloBN * 4 + (size_t)3 * (kHaloMaxPix + 2) * kHaloPix;
+    kHaloFilterBytes + 5 * kHaloBN * 4 + (size_t)3 * (kHaloMaxPix + 2) * kHaloPix;   // > 8 staging tiles
 constexpr int kHaloFilterChunks = kHaloBN * (kHaloK / 16);   // 16-byte chunks
 
 // Filter row (output channel) c of a workgroup's 64 sits in LDS slot
 // perm_slot16(c): lane (pixel, h) then holds channels 32 j + 16 h + [0, 16) of
 // its pixel in the sixteen accumulators of tile j, in order (see gemm_i8.h).
 constexpr int kHaloParBytes = kParArrays * kHaloBN * 4;
+
+// Requantises a wave's 32 pixels x 64 channels and writes them as whole rows
+// through its staging tile (gemm_i8.h: requant_pack16, wave_rows_copy_out).
+constexpr int kHaloStageStride = kHaloBN + 16;
+template <int MODE, bool LEAKY>
+__device__ __forceinline__ void halo_finish(const v16i (&acc)[2], const int32_t *s_par,
+                                            int8_t *stage, const Epilogue &ep, int lane, int m0,
+                                            int M, int n0) {
+  const int l32 = lane & 31, lhi = lane >> 5;
+  int32_t lo, hi;
+  activation_clamp(ep, lo, hi);
+  const bool fast = fused_out_is_fast(ep);
+  const FusedAddConsts fc = fused_add_consts(ep.add);
+#pragma unroll
+  for (int j = 0; j < 2; j++) {
+    const int cl = 32 * j + 16 * lhi;
+    const int4 v = requant_pack16<MODE, LEAKY, kHaloBN>(acc[j], s_par + cl, ep, lo, hi);
+    *reinterpret_cast<int4 *>(stage + l32 * kHaloStageStride + cl) = v;
+  }
+  wave_fence();
+  wave_rows_copy_out(stage, kHaloStageStride, kHaloBN, lane, m0, M, n0, ep, fc, fast);
+}
 
 // SKIP leaves phases out so that the others can be timed (1: staging, 2: the
 // matrix-core loop, 4: requantisation and copy-out); the library uses 0.
@@ -190,12 +213,17 @@ __global__ __launch_bounds__(512, 2) void conv3x3_halo_kernel(HaloConv cv, Epilo
       }
     }
   }
-  // no barrier: the waves finish on their own, nothing in LDS is reused
+  __syncthreads();   // every wave has read its halo: the area becomes output staging
+
+  // from here on each wave works on its own 32 pixels
   if constexpr (!(SKIP & 4)) {
     // rows past the tile's end belong to the next tile (or image): M bounds them
     const int m0 = (n * cv.OH + oh_first) * cv.OW;
-    gemm_epilogue_direct<kHaloBN, 32, 64>(acc, s_par, ep, m0 + npix, cv.OC, m0, n0, 0, wave, 0,
-                                          l32, lhi);
+    int8_t *stage = s_halo + wave * (32 * kHaloStageStride);
+    if (ep.act == 5) halo_finish<0, true>(acc[0], s_par, stage, ep, lane, m0 + wave * 32, m0 + npix, n0);
+    else if (mode == 3) halo_finish<3, false>(acc[0], s_par, stage, ep, lane, m0 + wave * 32, m0 + npix, n0);
+    else if (mode == 1) halo_finish<1, false>(acc[0], s_par, stage, ep, lane, m0 + wave * 32, m0 + npix, n0);
+    else halo_finish<0, false>(acc[0], s_par, stage, ep, lane, m0 + wave * 32, m0 + npix, n0);
   } else {
     int x = 0;
 #pragma unroll
@@ -220,7 +248,8 @@ static int conv_halo_rows(const mi355x_conv_geom *g, int cus, size_t &lds) {
          (rows - 1) * g->OW >= 32)
     rows--;
   const size_t halo = (size_t)(rows + 2) * (g->OW + 2) * kHaloPix;
-  lds = kHaloFilterBytes + kHaloParBytes + halo;
+  const size_t stage = (size_t)((rows * g->OW + 31) / 32) * 32 * kHaloStageStride;
+  lds = kHaloFilterBytes + kHaloParBytes + (halo > stage ? halo : stage);
   return rows;
 }
 

@@ -534,6 +534,41 @@ __device__ __forceinline__ void store16(int4 v, int8_t *out_row, const int8_t *r
   }
 }
 
+// A wave holds the requantised results of 32 output rows as 16-byte pieces, one
+// row per lane pair, staged in a wave-private LDS tile (rows `stride` bytes
+// apart, `group` bytes per row: 32 to 128). Stores straight from registers
+// would reach memory as 16-byte pieces of many lines (measured: 1.5 to 1.85 x
+// the output bytes written at the memory side); here the tile is read back with
+// group / 16 lanes per row, so that a store instruction writes whole rows of
+// the group (whole 128-byte lines for a 128-byte group), with the fused residual
+// add / Relu applied to words read the same way. `lane` is the lane index in
+// the wave; output row r of the tile is row m0 + r of the output (rows at and
+// past M are not written), its first byte of the group is column col0.
+__device__ __forceinline__ void wave_fence() {
+  // a wave reads back only what its own lanes wrote: LDS serves one wave's
+  // accesses in order, so the compiler is all that has to be held back
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+__device__ __forceinline__ void wave_rows_copy_out(const int8_t *s_stage, int stride, int group,
+                                                   int lane, int m0, int M, int col0,
+                                                   const Epilogue &ep, const FusedAddConsts &fc,
+                                                   bool fast) {
+  const int lpr = group / 16;                  // lanes per row
+  const int rpp = 64 / lpr;                    // rows per pass
+  const int rb_row = lane / lpr, rb_seg = lane - rb_row * lpr;
+  for (int r0 = 0; r0 < 32; r0 += rpp) {
+    const int row = r0 + rb_row, m = m0 + row;
+    if (row < 32 && m < M) {
+      int4 v = *reinterpret_cast<const int4 *>(s_stage + row * stride + rb_seg * 16);
+      const long long at = (long long)m * ep.ldc + col0 + rb_seg * 16;
+      v = fused_out_words(v, ep.add.res ? ep.add.res + at : nullptr, ep, fc, fast);
+      *reinterpret_cast<int4 *>(ep.out + at) = v;
+    }
+  }
+}
+
 template <int BN, int WM, int WN, int MODE, bool LEAKY>
 __device__ __forceinline__ void gemm_epilogue_direct_impl(
     v16i (&acc)[WM / 32][WN / 32], const int32_t *s_par, const Epilogue &ep, int M, int N,

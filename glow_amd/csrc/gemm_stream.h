@@ -10,10 +10,11 @@
 //   * a wave walks over tiles of 32 rows: a lane loads its row's K bytes
 //     straight from global memory into registers in the matrix-core layout
 //     (every byte of A is read by exactly one lane), multiplies them with the
-//     weight fragments read from LDS, 32 columns at a time, and requantises,
-//     packs and stores sixteen output bytes per lane from registers
-//     (the transposed-accumulator epilogue of gemm_i8.h), with the fused
-//     residual add read the same way;
+//     weight fragments read from LDS, 32 columns at a time, and requantises and
+//     packs sixteen output bytes per lane (the transposed-accumulator epilogue
+//     of gemm_i8.h); groups of up to 128 columns go through a wave-private
+//     transpose in LDS so that they are written as whole 128-byte lines, with
+//     the fused residual add read the same way;
 //   * latency is hidden by occupancy (four waves per SIMD) instead of by a
 //     pipeline: while one wave waits for its rows, the others multiply and
 //     requantise.
@@ -46,41 +47,55 @@ struct StreamRows {
   }
 };
 
+// Bytes between the rows of a wave's staging tile: a group of up to 128 output
+// columns plus 16 (consecutive rows start 36 banks apart).
+constexpr int kStreamGroup = 128;
+constexpr int kStreamStageStride = kStreamGroup + 16;
+constexpr int kStreamStageBytes = 32 * kStreamStageStride;   // per wave
+
+// The results leave through a wave-private transpose in LDS
+// (wave_rows_copy_out): groups of up to 128 columns are staged, then read back
+// with eight lanes per row, so that a store instruction writes whole 128-byte
+// lines and the residual is read the same way.
 template <int KS, int MODE, bool LEAKY>
 __device__ __forceinline__ void stream_tiles(const StreamRows &A, const int8_t *s_w,
-                                             const int32_t *s_par, const Epilogue &ep, int M,
-                                             int N, int n0, int bn, int tiles32, int first,
-                                             int step, int l32, int lhi) {
+                                             const int32_t *s_par, int8_t *s_stage,
+                                             const Epilogue &ep, int M, int N, int n0, int bn,
+                                             int tiles32, int first, int step, int lane) {
   constexpr int WSTRIDE = KS * 32 + 16;
+  const int l32 = lane & 31, lhi = lane >> 5;
   int32_t lo, hi;
   activation_clamp(ep, lo, hi);
   const bool fast = fused_out_is_fast(ep);
   const FusedAddConsts fc = fused_add_consts(ep.add);
-  const bool vec = (ep.ldc % 16 == 0) && (n0 % 16 == 0) &&
-                   (((((uintptr_t)ep.out) | ((uintptr_t)ep.add.res)) & 15) == 0);
   const int8_t *w_lane = s_w + l32 * WSTRIDE + lhi * 16;
+  // column groups of this slice: 128 columns, or all of a narrower slice
+  const int group = min(bn, kStreamGroup);         // bytes per row and group
   for (int t = first; t < tiles32; t += step) {
-    const int m = t * 32 + l32;
+    const int m0 = t * 32;
     // rows past the end re-read the last row; their results are not stored
-    const int8_t *ar = A.row(min(m, M - 1)) + lhi * 16;
+    const int8_t *ar = A.row(min(m0 + l32, M - 1)) + lhi * 16;
     v4i af[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) af[ks] = *reinterpret_cast<const v4i *>(ar + ks * 32);
-    int8_t *out_row = ep.out + (long long)m * ep.ldc;
-    const int8_t *res_row = ep.add.res ? ep.add.res + (long long)m * ep.ldc : nullptr;
-    for (int j = 0; j < bn / 32; j++) {
-      v16i acc;
+    for (int c0 = 0; c0 < bn; c0 += group) {
+      for (int j = c0 / 32; j < (c0 + group) / 32; j++) {
+        v16i acc;
 #pragma unroll
-      for (int r = 0; r < 16; r++) acc[r] = 0;
+        for (int r = 0; r < 16; r++) acc[r] = 0;
 #pragma unroll
-      for (int ks = 0; ks < KS; ks++) {
-        const v4i b = *reinterpret_cast<const v4i *>(w_lane + j * 32 * WSTRIDE + ks * 32);
-        // weights first: the result's rows are columns of the output
-        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(b, af[ks], acc, 0, 0, 0);
+        for (int ks = 0; ks < KS; ks++) {
+          const v4i b = *reinterpret_cast<const v4i *>(w_lane + j * 32 * WSTRIDE + ks * 32);
+          // weights first: the result's rows are columns of the output
+          acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(b, af[ks], acc, 0, 0, 0);
+        }
+        const int cl = j * 32 + 16 * lhi;
+        const int4 v = requant_pack16<MODE, LEAKY, kStreamMaxBN>(acc, s_par + cl, ep, lo, hi);
+        *reinterpret_cast<int4 *>(s_stage + l32 * kStreamStageStride + (cl - c0)) = v;
       }
-      const int cl = j * 32 + 16 * lhi;
-      const int4 v = requant_pack16<MODE, LEAKY, kStreamMaxBN>(acc, s_par + cl, ep, lo, hi);
-      if (m < M) store16(v, out_row, res_row, n0 + cl, N, vec, ep, fc, fast);
+      wave_fence();
+      wave_rows_copy_out(s_stage, kStreamStageStride, group, lane, m0, M, n0 + c0, ep, fc, fast);
+      wave_fence();
     }
   }
 }
@@ -93,12 +108,12 @@ __global__ __launch_bounds__(256, 4) void gemm_i8_stream_kernel(StreamRows A, co
   constexpr int K = KS * 32, WSTRIDE = K + 16;
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   int32_t *s_par = reinterpret_cast<int32_t *>(lds);
-  int8_t *s_w = lds + kStreamParBytes;
+  int8_t *s_stage = lds + kStreamParBytes;               // one tile per wave
+  int8_t *s_w = s_stage + 4 * kStreamStageBytes;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int l32 = lane & 31, lhi = lane >> 5;
   const int n0 = blockIdx.y * bn;
   const int cols = min(bn, N - n0);          // a multiple of 32
   const int mode = requant_mode(ep);
@@ -135,13 +150,17 @@ __global__ __launch_bounds__(256, 4) void gemm_i8_stream_kernel(StreamRows A, co
   // from here on every wave is on its own
   const int first = blockIdx.x * 4 + wave, step = gridDim.x * 4;
   if (ep.act == 5)
-    stream_tiles<KS, 0, true>(A, s_w, s_par, ep, M, N, n0, cols, tiles32, first, step, l32, lhi);
+    stream_tiles<KS, 0, true>(A, s_w, s_par, s_stage + wave * kStreamStageBytes, ep, M, N, n0,
+                              cols, tiles32, first, step, lane);
   else if (mode == 3)
-    stream_tiles<KS, 3, false>(A, s_w, s_par, ep, M, N, n0, cols, tiles32, first, step, l32, lhi);
+    stream_tiles<KS, 3, false>(A, s_w, s_par, s_stage + wave * kStreamStageBytes, ep, M, N, n0,
+                              cols, tiles32, first, step, lane);
   else if (mode == 1)
-    stream_tiles<KS, 1, false>(A, s_w, s_par, ep, M, N, n0, cols, tiles32, first, step, l32, lhi);
+    stream_tiles<KS, 1, false>(A, s_w, s_par, s_stage + wave * kStreamStageBytes, ep, M, N, n0,
+                              cols, tiles32, first, step, lane);
   else
-    stream_tiles<KS, 0, false>(A, s_w, s_par, ep, M, N, n0, cols, tiles32, first, step, l32, lhi);
+    stream_tiles<KS, 0, false>(A, s_w, s_par, s_stage + wave * kStreamStageBytes, ep, M, N, n0,
+                              cols, tiles32, first, step, lane);
 }
 
 // Whether the streaming kernel can run this product at all: K of 64, 128 or
@@ -151,25 +170,28 @@ static bool stream_can_run(int M, int N, int K, bool need_sa, bool need_sb, bool
                            const Epilogue &ep) {
   if (need_sa || need_sb || !aligned) return false;
   if (K != 64 && K != 128 && K != 256) return false;
-  if (N % 32 != 0 || M < 1) return false;
+  // whole 32-column tiles, and whole 128-column groups once there are more than 128
+  if (N % 32 != 0 || (N > kStreamGroup && N % kStreamGroup != 0) || M < 1) return false;
   if (ep.ldc % 16 != 0 || (((((uintptr_t)ep.out) | ((uintptr_t)ep.add.res)) & 15) != 0))
     return false;
   return true;
 }
 
-// Whether it is the default for such a product. Measured against the best
-// tiled kernel (us, M200704): K64 N64 9.0 vs 12.2, K64 N256 27.0 vs 28.2, K256
-// N64 15.9 vs 18.5, K256 N128 24.2 vs 25.5; with more columns the weight
-// slices multiply the reads of A and the tiled kernels are level or ahead
-// (M50176 K128 N512 19.9 vs 18.6, M12544 K256 N1024 15.2 vs 14.3).
-static bool stream_applies(int M, int N) { return M >= 4096 && N <= kStreamMaxBN; }
+// Whether it is the default for such a product. Measured with the backend's
+// requantisation hint against the best tiled kernel (us): M200704 K64 N64 8.8
+// vs 12.2, K64 N256 23.8 vs 28.0, K256 N64 15.3 vs 18.5, K256 N128 23.6 vs 25.0;
+// M50176 K128 N512 17.5 vs 18.6, K256 N512 24.1 vs 23.9; M12544 K256 N1024 14.5
+// vs 14.3: level once the weight slices multiply the reads of A.
+static bool stream_applies(int M, int N) { return M >= 4096 && N <= 512; }
 
 static int gemm_stream_launch(const StreamRows &A, const int8_t *W, const Epilogue &ep, int M,
                               int N, int K, hipStream_t st) {
-  // columns per slice: the weights of a slice stay under ~37 KB of LDS
-  const int bn = K == 256 ? 128 : kStreamMaxBN;
+  // columns per slice: 256 for K = 64, 128 beyond (the weights of a slice stay
+  // under 35 KB, beside 18 KB of staging tiles and the 5 KB constants table)
+  const int bn = K == 64 ? kStreamMaxBN : 128;
   const int slices = (N + bn - 1) / bn;
-  const size_t lds = (size_t)kStreamParBytes + (size_t)std::min(bn, N) * (K + 16);
+  const size_t lds = (size_t)kStreamParBytes + 4 * (size_t)kStreamStageBytes +
+                     (size_t)std::min(bn, N) * (K + 16);
   const int tiles32 = (M + 31) / 32;
   int dev = 0, cus = 256;
   if (hipGetDevice(&dev) == hipSuccess) {
@@ -189,9 +211,14 @@ static int gemm_stream_launch(const StreamRows &A, const int8_t *W, const Epilog
   case 128:
     hipLaunchKernelGGL(gemm_i8_stream_kernel<4>, grid, block, lds, st, A, W, ep, M, N, bn, tiles32);
     break;
-  default:
+  default: {
+    // 128 columns x 272 bytes of weights: past the 48 KiB a launch gets unasked
+    static std::atomic<uint64_t> attr_set{0};
+    const int rc = set_lds_attr(gemm_i8_stream_kernel<8>, 64 * 1024, attr_set);
+    if (rc != MI355X_OK) return rc;
     hipLaunchKernelGGL(gemm_i8_stream_kernel<8>, grid, block, lds, st, A, W, ep, M, N, bn, tiles32);
     break;
+  }
   }
   return check_launch("gemm_i8_stream");
 }
