@@ -75,12 +75,15 @@ public:
 
 struct Operand {
   const Value *v;
+  // an activation's place in its region, in the compiled function's table
+  // (filled when every launch of the function is known)
+  const size_t *actOffset = nullptr;
   // region + offset -> device pointer at launch time
   uint8_t *ptr(const DeviceBindings &b) const {
     switch (v->category) {
     case SymbolCategory::Constant: return b.constants + v->offset;
     case SymbolCategory::Placeholder: return b.mutableMem + v->offset;
-    default: return b.activations + v->offset;
+    default: return b.activations + (actOffset ? *actOffset : v->offset);
     }
   }
   const Type &ty() const { return v->type; }
@@ -112,7 +115,10 @@ public:
   // a negative one accepts any activation (single-instruction probes).
   Compiler(const Module &M, const std::vector<Instruction> &insts, int function,
            const BackendOptions &o)
-      : M_(M), insts_(insts), function_(function), opts_(o) {}
+      : M_(M), insts_(insts), function_(function), opts_(o),
+        actOff_(std::make_shared<std::vector<size_t>>((size_t)M.numValues(), 0)) {
+    for (int id = 0; id < M.numValues(); id++) (*actOff_)[(size_t)id] = M.value(id).offset;
+  }
 
   Error run(MI355XFunction &out) {
     for (const auto &I : insts_) MI355X_RETURN_IF_ERR(checkOperands(I));
@@ -266,6 +272,7 @@ public:
                                   kn == "mi355x_rwq_fc_relu_i8";
       }
     }
+    planActivations(out);
     assignLevels(out);
     // scratch buffers follow the initialised image
     scratchBase_ = alignUp(gen_.image_.size(), 256);
@@ -301,7 +308,8 @@ private:
     return Error::success();
   }
 
-  Operand op(const Instruction &I, int i) const { return Operand{&M_.value(I.operands[(size_t)i])}; }
+  Operand op(const Instruction &I, int i) const { return opOf(M_.value(I.operands[(size_t)i])); }
+  Operand opOf(const Value &v) const { return Operand{&v, &(*actOff_)[(size_t)v.id]}; }
 
   void noteAccesses(const Instruction &J, KernelLaunch &L) const {
     // (Pooled lookups over more than 4096 bags use scratch inside the kernel
@@ -321,6 +329,143 @@ private:
       }
       (i == 0 ? L.writes : L.reads).push_back(a);
     }
+  }
+
+  // Places the function's activations (AllocationsInfo::allocateActivations,
+  // AllocationsInfo.cpp:128-156, over MemoryAllocator::allocate,
+  // MemoryAllocator.cpp:58-91: first fit by address). Launches, not
+  // instructions, are the unit of a value's life, because a fused launch reads
+  // and writes all of its instructions' operands at once; and a life ends not
+  // at a position in the launch list but in the dependence graph (see deadFor),
+  // because the launches of independent chains run side by side. Values no
+  // launch touches get no memory. The byte ranges are recorded in the accesses,
+  // so that `conflict` sees launches whose values share bytes.
+  void planActivations(MI355XFunction &out) {
+    auto &L = out.launches;
+    const size_t nv = (size_t)M_.numValues();
+    std::vector<long long> first(nv, -1), last(nv, -1);
+    auto isAct = [&](int root) {
+      return root >= 0 && M_.value(root).category == SymbolCategory::Activation;
+    };
+    for (size_t i = 0; i < L.size(); i++)
+      for (const auto *set : {&L[i].reads, &L[i].writes})
+        for (const Access &a : *set)
+          if (isAct(a.root)) {
+            if (first[(size_t)a.root] < 0) first[(size_t)a.root] = (long long)i;
+            last[(size_t)a.root] = (long long)i;
+          }
+    constexpr size_t kAlign = 256;
+    std::vector<size_t> rootOff(nv, 0), rootSize(nv, 0);
+    size_t total = 0;
+    auto bytesOf = [&](size_t r) {
+      return alignUp(std::max<size_t>(1, M_.value((int)r).type.sizeInBytes()), kAlign);
+    };
+    // A value that a single launch both writes and reads, and no other launch
+    // touches, is a result handed from one instruction to the next inside a
+    // fused launch: the kernel keeps it in registers. It gets no memory of its
+    // own (it is put at the start of the region, which is at least its size).
+    std::vector<char> inner(nv, 0);
+    if (opts_.reuseActivations)
+      for (size_t r = 0; r < nv; r++) {
+        if (first[r] < 0 || first[r] != last[r]) continue;
+        const KernelLaunch &l = L[(size_t)first[r]];
+        bool rd = false, wr = false;
+        for (const Access &a : l.reads) rd = rd || a.root == (int)r;
+        for (const Access &a : l.writes) wr = wr || a.root == (int)r;
+        if (rd && wr) {
+          inner[r] = 1;
+          rootSize[r] = bytesOf(r);
+          total = std::max(total, rootSize[r]);
+          first[r] = last[r] = -1;
+        }
+      }
+    if (opts_.reuseActivations) {
+      // anc[i]: the launches that run before launch i in every order the
+      // dependences allow (its ancestors in the graph of conflicts by value)
+      const size_t n = L.size(), words = (n + 63) / 64;
+      std::vector<std::vector<uint64_t>> anc(n, std::vector<uint64_t>(words, 0));
+      for (size_t i = 0; i < n; i++)
+        for (size_t j = i; j-- > 0;) {
+          if ((anc[i][j / 64] >> (j % 64)) & 1) continue;
+          if (!conflict(L[j], L[i])) continue;
+          anc[i][j / 64] |= 1ull << (j % 64);
+          for (size_t w = 0; w < words; w++) anc[i][w] |= anc[j][w];
+        }
+      std::vector<std::vector<size_t>> touchers(nv);
+      for (size_t i = 0; i < n; i++)
+        for (const auto *set : {&L[i].reads, &L[i].writes})
+          for (const Access &a : *set)
+            if (isAct(a.root) && first[(size_t)a.root] >= 0 &&
+                (touchers[(size_t)a.root].empty() || touchers[(size_t)a.root].back() != i))
+              touchers[(size_t)a.root].push_back(i);
+      // The bytes of value q may pass to value r when every launch that touches
+      // q is an ancestor of every launch that touches r (r may have several
+      // independent writers, e.g. slices inserted by parallel chains): the
+      // hand-over then adds no ordering that the data flow does not already
+      // impose, so independent chains stay independent.
+      auto deadFor = [&](int q, size_t r) {
+        for (size_t tr : touchers[r])
+          for (size_t tq : touchers[(size_t)q])
+            if (!((anc[tr][tq / 64] >> (tq % 64)) & 1)) return false;
+        return true;
+      };
+      struct Seg { size_t lo, hi; int root; };
+      std::vector<Seg> segs;                    // disjoint, sorted by address
+      for (size_t i = 0; i < n; i++)
+        for (size_t r = 0; r < nv; r++) {
+          if (first[r] != (long long)i) continue;
+          const size_t need = bytesOf(r);
+          // first fit: the lowest address whose bytes are free or dead for r
+          size_t at = 0;
+          for (bool moved = true; moved;) {
+            moved = false;
+            for (const Seg &g : segs)
+              if (g.lo < at + need && at < g.hi && !deadFor(g.root, r)) {
+                at = g.hi;
+                moved = true;
+              }
+          }
+          // what r covers of the dead values' segments is taken from them
+          std::vector<Seg> next;
+          for (const Seg &g : segs) {
+            if (g.hi <= at || g.lo >= at + need) { next.push_back(g); continue; }
+            if (g.lo < at) next.push_back(Seg{g.lo, at, g.root});
+            if (g.hi > at + need) next.push_back(Seg{at + need, g.hi, g.root});
+          }
+          next.push_back(Seg{at, at + need, (int)r});
+          std::sort(next.begin(), next.end(), [](const Seg &x, const Seg &y) { return x.lo < y.lo; });
+          segs.swap(next);
+          rootOff[r] = at;
+          rootSize[r] = need;
+          total = std::max(total, at + need);
+        }
+    } else {
+      for (size_t r = 0; r < nv; r++) {
+        if (first[r] < 0) continue;
+        rootSize[r] = bytesOf(r);
+        rootOff[r] = total;
+        total += rootSize[r];
+      }
+    }
+    // views lie where their root lies
+    for (size_t id = 0; id < nv; id++) {
+      const Value &v = M_.value((int)id);
+      if (v.category != SymbolCategory::Activation) continue;
+      if (function_ >= 0 && v.function != function_) continue;
+      (*actOff_)[id] = isAct(v.root) ? rootOff[(size_t)v.root] : 0;
+    }
+    for (auto &l : L)
+      for (auto *set : {&l.reads, &l.writes})
+        for (Access &a : *set)
+          if (isAct(a.root) && !inner[(size_t)a.root]) {
+            a.actLo = (long long)rootOff[(size_t)a.root];
+            a.actHi = a.actLo + (long long)rootSize[(size_t)a.root];
+          }
+    for (size_t r = 0; r < nv; r++)
+      if (first[r] >= 0)
+        out.activationPlan.push_back({M_.value((int)r).name, (int)r, rootOff[r], rootSize[r]});
+    out.activationOffsets = actOff_;
+    out.activationsBytes = total;
   }
 
   static bool conflict(const KernelLaunch &early, const KernelLaunch &late) {
@@ -1661,10 +1806,10 @@ private:
     c.acc16 = !S.iattrs.empty() && S.iattrs[0] != 0 && fp16Scale;
     c.qScale = qv.type.scale;
     c.qOffset = qv.type.offset;
-    c.data = Operand{&data};
-    c.idx = Operand{&idx};
-    c.len = Operand{&len};
-    c.dest = Operand{&dv};
+    c.data = opOf(data);
+    c.idx = opOf(idx);
+    c.len = opOf(len);
+    c.dest = opOf(dv);
     c.length = p + 2 - at;
     return true;
   }
@@ -1764,7 +1909,7 @@ private:
 
   Error slws(const Instruction &I, MI355XFunction &out, bool weighted) {
     Operand d = op(I, 0), data = op(I, 1);
-    Operand w = weighted ? op(I, 2) : Operand{nullptr};
+    Operand w = weighted ? op(I, 2) : Operand{nullptr, nullptr};
     Operand idx = op(I, weighted ? 3 : 2), len = op(I, weighted ? 4 : 3);
     CHECK_OP(isFused(data.ty().kind) && data.ty().dims.size() == 2,
              "data must be a 2-D fused-rowwise tensor, has %s", data.ty().str().c_str());
@@ -1843,6 +1988,7 @@ private:
   Generated gen_;
   size_t scratchBase_ = 0, genTotal_ = 0;
   std::shared_ptr<size_t> scratchBasePtr_ = std::make_shared<size_t>(0);
+  std::shared_ptr<std::vector<size_t>> actOff_;   // value id -> place in the activations region
   std::map<int, std::pair<bool, bool>> io_; // value id -> (read, written)
   std::map<const Value *, TableView> paddedTables_;
   std::map<int, size_t> derived_; // lengths value id -> index in derivedBagOffsets
@@ -1863,14 +2009,15 @@ Expected<std::unique_ptr<MI355XFunction>> MI355XBackend::compile(const Function 
   RuntimeBundle rb;
   rb.constantWeightVarsMemSize = M.constantsSize();
   rb.mutableWeightVarsMemSize = M.mutableSize();
-  rb.activationsMemSize = F.activationsSize();
+  rb.activationsMemSize = fn->activationsBytes;
   rb.generatedConstantsMemSize = C.generatedTotal();
   for (int id = 0; id < M.numValues(); id++) {
     const Value &v = M.value(id);
     if (v.category == SymbolCategory::Activation && v.function != F.index()) continue;
     RuntimeSymbolInfo si;
     si.size = v.type.sizeInBytes();
-    si.offset = v.offset;
+    si.offset = v.category == SymbolCategory::Activation ? (*fn->activationOffsets)[(size_t)id]
+                                                         : v.offset;
     si.type = v.type;
     si.symbolCategory = v.category;
     auto it = C.io().find(id);
@@ -1962,10 +2109,25 @@ Error MI355XFunction::captureGraph(const DeviceBindings &b, const std::vector<vo
   if (!b.stream)
     return MI355X_MAKE_ERR(ErrorCode::RUNTIME_ERROR, "graph capture needs a created stream");
   const size_t n = launches.size(), nLanes = sideStreams.size() + 1;
+  // Direct predecessors only: a conflicting launch that is already an ancestor
+  // of a later predecessor is ordered through it (memory shared by values whose
+  // lives do not meet makes a launch conflict with every earlier owner of its
+  // bytes; recorded as edges, those made graphs the runtime could not walk).
   std::vector<std::vector<size_t>> preds(n);
-  for (size_t i = 0; i < n; i++)
-    for (size_t j = 0; j < i; j++)
-      if (launchesConflict(launches[j], launches[i])) preds[i].push_back(j);
+  {
+    const size_t words = (n + 63) / 64;
+    std::vector<std::vector<uint64_t>> anc(n, std::vector<uint64_t>(words, 0));
+    for (size_t i = 0; i < n; i++) {
+      for (size_t j = i; j-- > 0;) {
+        if ((anc[i][j / 64] >> (j % 64)) & 1) continue;
+        if (!launchesConflict(launches[j], launches[i])) continue;
+        preds[i].push_back(j);
+        anc[i][j / 64] |= 1ull << (j % 64);
+        for (size_t w = 0; w < words; w++) anc[i][w] |= anc[j][w];
+      }
+      std::reverse(preds[i].begin(), preds[i].end());   // ascending, as the lane choice expects
+    }
+  }
   // Lanes. A launch hands its lane to the successor with the longest chain of
   // launches still behind it, so the critical path runs down one stream and
   // only the shorter branches pay for an event wait.
@@ -2106,9 +2268,26 @@ std::string MI355XFunction::describe() const {
      << " mutable=" << bundle_.mutableWeightVarsMemSize
      << " activations=" << bundle_.activationsMemSize << "\n";
   for (const auto &l : setup) os << "setup " << l.kernel << " inst=" << l.inst << l.params << "\n";
-  for (const auto &l : launches)
+  auto accesses = [&](const char *k, const std::vector<Access> &v) {
+    // value ids (views by their root) and the byte range inside a row, -1 = all
+    for (const char *part : {"", "_lo", "_hi"}) {
+      os << " " << k << part << "=[";
+      for (size_t i = 0; i < v.size(); i++)
+        os << (i ? "," : "") << (*part == 0 ? (long long)v[i].root : part[1] == 'l' ? v[i].lo : v[i].hi);
+      os << "]";
+    }
+  };
+  for (const auto &l : launches) {
     os << "launch " << l.kernel << " inst=" << l.inst << " level=" << l.level << " tile=" << l.tile << " requant_hint=" << l.requantHint
-       << l.params << "\n";
+       << l.params;
+    accesses("reads", l.reads);
+    accesses("writes", l.writes);
+    os << "\n";
+  }
+  // where the activations with memory of their own lie
+  for (const auto &a : activationPlan)
+    os << "activation name=" << a.name << " id=" << a.id << " offset=" << a.offset
+       << " bytes=" << a.bytes << "\n";
   return os.str();
 }
 

@@ -78,8 +78,11 @@ struct RuntimeBundle {
 struct Access {
   int root = -1;
   long long lo = 0, hi = -1; // hi < 0: the whole value
+  // activations only: the bytes [actLo, actHi) of the activations region the
+  // root occupies (different values share memory when their lives do not meet)
+  long long actLo = 0, actHi = 0;
   bool overlaps(const Access &o) const {
-    if (root != o.root) return false;
+    if (root != o.root) return actLo < o.actHi && o.actLo < actHi;
     if (hi < 0 || o.hi < 0) return true;
     return lo < o.hi && o.lo < hi;
   }
@@ -130,6 +133,17 @@ public:
   std::vector<KernelLaunch> setup, launches;
   // Host image of the generated constants (uploaded by the device manager).
   std::vector<uint8_t> generated;
+  // Where each value of the module lies in this function's activations region
+  // (by value id; meaningful for the function's activations only). The launches
+  // read it when they run.
+  std::shared_ptr<std::vector<size_t>> activationOffsets;
+  size_t activationsBytes = 0;   // size of the region so planned
+  struct ActivationPlace {
+    std::string name;
+    int id;
+    size_t offset, bytes;
+  };
+  std::vector<ActivationPlace> activationPlan;   // the values with memory of their own
   // Lookups whose lengths are an input placeholder read their bags as
   // positions: whoever uploads `lengths` also writes segments + 1 int32
   // exclusive prefix sums of the (clamped) lengths to ptr(bindings).
@@ -172,6 +186,7 @@ struct BackendOptions {
   bool fuseInsert = true;              // Gather / RescaleQuantized write straight into the tensor their result is inserted into
   bool fuseDequantizeSigmoid = true;   // Dequantize + Sigmoid of its result in one kernel
   bool deriveBagOffsets = true;        // lookups whose lengths are an input: bag positions summed on the host at upload
+  bool reuseActivations = true;        // activations whose lives do not meet share memory (first fit over the launch order)
 };
 
 class MI355XBackend {

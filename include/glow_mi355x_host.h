@@ -128,7 +128,10 @@ enum {
   MI355X_HOST_OPT_DERIVE_BAG_OFFSETS = 1024, /* lookups whose lengths are an input placeholder read
                                               * their bags as positions that the device manager sums
                                               * on the host when it uploads the lengths */
-  MI355X_HOST_OPT_DEFAULT = 2047
+  MI355X_HOST_OPT_REUSE_ACTIVATIONS = 2048, /* activations whose lives do not meet in the dependence
+                                             * graph share memory (AllocationsInfo.cpp:128-156); off:
+                                             * every value has bytes of its own */
+  MI355X_HOST_OPT_DEFAULT = 4095
 };
 int mi355x_host_compile(mi355x_host_module *m, int function, int options);
 /* Listing of the compiled function's launches and derived parameters; returns
