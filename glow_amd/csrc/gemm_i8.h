@@ -119,23 +119,39 @@ __device__ __forceinline__ uint32_t fused_relu_word(uint32_t own, const FusedAdd
 // pre-shift (rescale factors near one). Then ((x - off) * s + rtn) equals
 // x * s + (rtn - off * s) modulo 2^32, one 24-bit multiply-add per value with
 // a constant formed once, and the result is bit for bit that of scale_i32.
+// The Relu stage folds further (fused_out_is_fast checks the bounds that keep
+// every sum inside 32 bits): clip to int8 followed by max(., so) is one clamp
+// to [max(-128, so), 127], and the offset added behind the post-shift goes
+// into the constant in front of it ((X >> p) + d == (X + (d << p)) >> p).
 struct FusedAddConsts {
-  int32_t own_c, res_c, relu_c;
+  int32_t own_c, res_c, relu_c, sum_lo;
+  int32_t relu_scale, relu_post;   // 1 and 0 (with relu_c 0) when no Relu follows the add
 };
 __device__ __forceinline__ FusedAddConsts fused_add_consts(const FusedAdd &f) {
   auto rtn = [](int32_t post) { return post > 0 ? (1u << (post - 1)) : 0u; };
+  const int32_t so = (int32_t)(int8_t)f.sum_off;
   FusedAddConsts c;
   c.own_c = (int32_t)(rtn(f.own_post) - (uint32_t)f.own_off * (uint32_t)f.own_scale);
   c.res_c = (int32_t)(rtn(f.res_post) - (uint32_t)f.res_off * (uint32_t)f.res_scale);
-  c.relu_c = (int32_t)(rtn(f.dest_post) -
-                       (uint32_t)(int32_t)(int8_t)f.sum_off * (uint32_t)f.dest_scale);
+  c.relu_c = (int32_t)(rtn(f.dest_post) - (uint32_t)so * (uint32_t)f.dest_scale +
+                       ((uint32_t)f.dest_off << (f.dest_post & 31)));
+  c.sum_lo = max(-128, so);
+  c.relu_scale = f.dest_scale;
+  c.relu_post = f.dest_post;
+  if (!f.relu) {
+    // the same instructions leave the clipped sum as it is: v * 1 + 0 >> 0
+    c.relu_c = 0;
+    c.sum_lo = -128;
+    c.relu_scale = 1;
+    c.relu_post = 0;
+  }
+  asm volatile("" : "+v"(c.own_c), "+v"(c.res_c), "+v"(c.relu_c), "+v"(c.sum_lo));
   return c;
 }
 template <bool ADD>
 __device__ __forceinline__ uint32_t fused_word_fast(uint32_t own, uint32_t res,
                                                     const FusedAdd &f,
                                                     const FusedAddConsts &c) {
-  const int32_t so = (int32_t)(int8_t)f.sum_off;
   int32_t r[4];
 #pragma unroll
   for (int b = 0; b < 4; b++) {
@@ -144,13 +160,13 @@ __device__ __forceinline__ uint32_t fused_word_fast(uint32_t own, uint32_t res,
       const int32_t x = (int32_t)(int8_t)(res >> (8 * b));
       const int32_t a = (int32_t)((uint32_t)__mul24(v, f.own_scale) + (uint32_t)c.own_c) >> f.own_post;
       const int32_t bb = (int32_t)((uint32_t)__mul24(x, f.res_scale) + (uint32_t)c.res_c) >> f.res_post;
-      v = med3_i32((int32_t)((uint32_t)a + (uint32_t)bb + (uint32_t)f.sum_off), -128, 127);
+      // the int8 clip of the sum and the Relu's lower bound in one clamp
+      v = med3_i32((int32_t)((uint32_t)a + (uint32_t)bb + (uint32_t)f.sum_off), c.sum_lo, 127);
+    } else {
+      v = max(v, c.sum_lo);
     }
-    if (!ADD || f.relu) {
-      v = max(v, so);
-      v = (int32_t)((uint32_t)__mul24(v, f.dest_scale) + (uint32_t)c.relu_c) >> f.dest_post;
-      v = med3_i32((int32_t)((uint32_t)v + (uint32_t)f.dest_off), -128, 127);
-    }
+    v = (int32_t)((uint32_t)__mul24(v, c.relu_scale) + (uint32_t)c.relu_c) >> c.relu_post;
+    v = med3_i32(v, -128, 127);
     r[b] = v;
   }
   return __builtin_amdgcn_perm(
@@ -310,17 +326,27 @@ __device__ __forceinline__ void load_col_raw(ColRaw (&c)[TN], const Epilogue &ep
 // 16 residual bytes of the same place (NULL: no residual). `fast`: every scale
 // small and no pre-shift in the stages that run.
 __device__ __forceinline__ bool fused_out_is_fast(const Epilogue &ep) {
+  // Relu stage: (v - so) * scale is below 2^8 * 2^22, the folded offset
+  // |dest_off| << post at most 2^7 * 2^22, the rounding term 2^21
+  const bool relu_ok = ep.add.dest_pre == 0 && ep.add.dest_post <= 22 &&
+                       ep.add.dest_scale > -(1 << 22) && ep.add.dest_scale < (1 << 22) &&
+                       ep.add.dest_off >= -128 && ep.add.dest_off <= 127;
   return ep.add.small &&
          (!ep.add.res || (ep.add.own_pre == 0 && ep.add.res_pre == 0)) &&
-         (!ep.add.relu || ep.add.dest_pre == 0);
+         (!ep.add.relu || relu_ok);
 }
 __device__ __forceinline__ int4 fused_out_words(int4 v, const int8_t *res16, const Epilogue &ep,
                                                 const FusedAddConsts &fc, bool fast) {
   if (res16 && fast) {
     const int4 q = *reinterpret_cast<const int4 *>(res16);
+    // (a word at a time: sixteen values in flight at once cost the tiled kernels
+    // twenty registers)
     v.x = (int)fused_word_fast<true>((uint32_t)v.x, (uint32_t)q.x, ep.add, fc);
+    __builtin_amdgcn_sched_barrier(0);
     v.y = (int)fused_word_fast<true>((uint32_t)v.y, (uint32_t)q.y, ep.add, fc);
+    __builtin_amdgcn_sched_barrier(0);
     v.z = (int)fused_word_fast<true>((uint32_t)v.z, (uint32_t)q.z, ep.add, fc);
+    __builtin_amdgcn_sched_barrier(0);
     v.w = (int)fused_word_fast<true>((uint32_t)v.w, (uint32_t)q.w, ep.add, fc);
   } else if (!res16 && ep.add.relu && fast) {
     v.x = (int)fused_word_fast<false>((uint32_t)v.x, 0u, ep.add, fc);
