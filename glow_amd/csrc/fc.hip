@@ -109,7 +109,7 @@ using namespace mi355x;
 extern "C" {
 
 int mi355x_gemm_tile_override(int tile) {
-  MI355X_REQUIRE(tile >= -1 && tile <= 8, "tile %d outside [-1, 8]", tile);
+  MI355X_REQUIRE(tile >= -1 && tile <= 11, "tile %d outside [-1, 11]", tile);
   g_tile_override = tile;
   return MI355X_OK;
 }

@@ -980,7 +980,9 @@ __device__ __forceinline__ uint32_t lds_address(const void *p) {
 template <int BM, int BN, int WM, int WN, int STAGES, bool NEED_SA,
           bool NEED_SB, class ARows, bool SHORT = false>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
-                             (BM * BN == 256 * 128)   ? 2
+                             ((BM / WM) * (BN / WN) == 8 && BM * BN <= 256 * 128)
+                                 ? (BM * BN == 256 * 128 ? 1 : 2)
+                             : (BM * BN == 256 * 128) ? 2
                              : SHORT                  ? 4
                              : (BM * BN == 128 * 128) ? 3
                                                       : 1) void gemm_i8_dma_kernel(
@@ -1323,9 +1325,9 @@ static int gemm_dma_launch(const ARows &A, const DenseRows &B,
 // Tile choice from the problem size: 256x256 for large problems (a wave owns
 // 128x128, which halves LDS traffic per MFMA), smaller tiles when the grid
 // would otherwise not fill 256 CUs.
-enum class Tile { T256, T128, T128x64, T64, T256x128, T128x256 };
-// Tuning aid: a value in [0, 5] forces that tile for the following launches of
-// the calling thread.
+enum class Tile { T256, T128, T128x64, T64, T256x128, T128x256, T128w8 = 9, T256x128w8 = 10, T256w8 = 11 };
+// Tuning aid: a value in [0, 5] or [9, 11] forces that tile for the following
+// launches of the calling thread (w8: eight waves per workgroup instead of four).
 extern thread_local int g_tile_override;
 // Requantisation hints for the following launches of the calling thread.
 extern thread_local int g_requant_hint;
@@ -1333,22 +1335,23 @@ static Tile pick_tile(const GemmShape &g, size_t lds_256) {
   auto tiles = [&](int bm, int bn) {
     return (long long)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * g.groups;
   };
-  if (g_tile_override >= 0 && g_tile_override <= 5 &&
-      (g_tile_override != 0 || lds_256 <= lds_limit()))
+  if (((g_tile_override >= 0 && g_tile_override <= 5) ||
+       (g_tile_override >= 9 && g_tile_override <= 11)) &&
+      ((g_tile_override != 0 && g_tile_override != 11) || lds_256 <= lds_limit()))
     return (Tile)g_tile_override;
-  // Measured on the convolution shapes of ResNet-50 and on large FCs: the
-  // 256x256 tile (one wave per SIMD) only pays off when the K loop is long
-  // enough to amortise its prologue and epilogue; short K loops want many
-  // small resident workgroups; few-row problems want 64x64 to fill the chip.
-  // (M16384 K1024 N1024: 256x128 28.7 us, 256x256 29.5; M32768: 51.3 vs 56.2;
-  // M16384 K2048 N2048: 80.9 vs 82.7; M8192 K4096 N4096: 150 vs 137)
-  if (tiles(256, 256) >= 256 && g.N >= 256 && g.K > 2048 &&
-      lds_256 <= lds_limit())
-    return Tile::T256;
-  // shorter K loops with wide outputs: 256x128 tiles, two workgroups per CU, so
-  // one workgroup's epilogue overlaps the other's loads
-  if (tiles(256, 128) >= 256 && g.N >= 256 && g.K <= 2048) return Tile::T256x128;
-  if (tiles(128, 128) >= 256 && g.N >= 128 && g.K >= 512) return Tile::T128;
+  // Measured on the convolution shapes of ResNet-50 and on large FCs. The big
+  // tiles run with eight waves (two per SIMD: one wave's fragment reads and
+  // bookkeeping hide behind the other's matrix-core work), which beat their
+  // four-wave forms on every large shape tried (us, four waves / eight):
+  // M8192 K4096 N4096 137.8 / 130.4, M16384 K2048 N4096 161.2 / 144.3,
+  // M16384 K1024 N1024 30.4 / 25.9, M32768 K2048 N1024 83.7 / 74.9. 256x256
+  // needs a grid that fills the chip; below that 256x128, then 128x128, then
+  // many small resident workgroups; few-row problems want 64x64.
+  if (tiles(256, 256) >= 256 && g.N >= 256 && g.K >= 1024 && lds_256 <= lds_limit())
+    return Tile::T256w8;
+  // two workgroups per CU, so one workgroup's epilogue overlaps the other's loads
+  if (tiles(256, 128) >= 256 && g.N >= 256) return Tile::T256x128;
+  if (tiles(128, 128) >= 256 && g.N >= 128 && g.K >= 512) return Tile::T128w8;
   if (tiles(128, 64) >= 256) return Tile::T128x64;
   if (tiles(64, 64) >= 256 || g.M < 1024) return Tile::T64;
   return Tile::T128x64;
@@ -1368,6 +1371,12 @@ static int gemm_dma_tiles(const ARows &A, const DenseRows &B, const Epilogue &ep
     return gemm_dma_launch<256, 128, 128, 64, 3, SA, SB>(A, B, ep, g, st);
   case Tile::T128x256:
     return gemm_dma_launch<128, 256, 64, 128, 3, SA, SB>(A, B, ep, g, st);
+  case Tile::T128w8:
+    return gemm_dma_launch<128, 128, 64, 32, 3, SA, SB>(A, B, ep, g, st);
+  case Tile::T256x128w8:
+    return gemm_dma_launch<256, 128, 64, 64, 3, SA, SB>(A, B, ep, g, st);
+  case Tile::T256w8:
+    return gemm_dma_launch<256, 256, 128, 64, 4, SA, SB>(A, B, ep, g, st);
   default:
     return gemm_dma_launch<64, 64, 32, 32, 4, SA, SB>(A, B, ep, g, st);
   }
@@ -1386,6 +1395,9 @@ static int gemm_staged_tiles(const ARows &A, const DenseRows &B,
     return gemm_launch<128, 64, 32, 64, AL_A, AL_B>(A, B, ep, g, st);
   case Tile::T256x128:
   case Tile::T128x256:
+  case Tile::T128w8:
+  case Tile::T256x128w8:
+  case Tile::T256w8:
     return gemm_launch<128, 128, 64, 64, AL_A, AL_B>(A, B, ep, g, st);
   default:
     return gemm_launch<64, 64, 32, 32, AL_A, AL_B>(A, B, ep, g, st);

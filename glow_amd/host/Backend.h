@@ -112,7 +112,7 @@ struct KernelLaunch {
   // Issues the launch (with its tile, if it has one).
   int launch(const DeviceBindings &b) const;
 };
-constexpr int kNumTiles = 9;
+constexpr int kNumTiles = 12;
 
 class MI355XFunction {
 public:

@@ -452,7 +452,8 @@ int mi355x_matmul_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs_kn,
  * streaming kernel for K of 64, 128 or 256 (FullyConnected and pointwise
  * convolutions with symmetric weights and precomputed row sums: weights and
  * constants resident in LDS, rows straight from memory into registers; other
- * launches ignore it); -1 = chosen
+ * launches ignore it), 9 = 128x128, 10 = 256x128 and 11 = 256x256 with
+ * eight waves per workgroup instead of four; -1 = chosen
  * from the problem shape (the default). Results do not depend on the tile. A device
  * manager uses it to time the candidates of each layer once, when a network is
  * loaded. */

@@ -23,7 +23,8 @@ from tests import cases
 pytestmark = pytest.mark.gpu
 
 TILES = {0: "256x256", 1: "128x128", 2: "128x64", 3: "64x64", 4: "256x128", 5: "128x256",
-         6: "32x32 split-K"}
+         6: "32x32 split-K", 9: "128x128, 8 waves", 10: "256x128, 8 waves",
+         11: "256x256, 8 waves"}
 
 
 @pytest.fixture(scope="module", autouse=True)
@@ -137,7 +138,8 @@ def _check_large(M, K, N, seed, symmetric, distinct, sample, tile=None):
 
 
 def test_rwq_fc_m8192_k4096_n4096():
-    """The benchmark's large FullyConnected (256x256 tiles by the shape rule)."""
+    """The benchmark's large FullyConnected (256x256 tiles with eight waves by the
+    shape rule)."""
     say("rwq_fc M8192 K4096 N4096")
     rows = np.r_[0:24, 250:262, 500:512]
     _check_large(8192, 4096, 4096, 81, True, 512, rows)
@@ -149,17 +151,17 @@ def test_rwq_fc_m8192_k4096_n4096_asymmetric_weights():
     _check_large(8192, 4096, 4096, 82, False, 512, rows)
 
 
-@pytest.mark.parametrize("tile", [None, 0, 4, 5])
+@pytest.mark.parametrize("tile", [None, 0, 4, 5, 10])
 def test_rwq_fc_m16384_k1024_n1024(tile):
-    """The benchmark's M = 16384 variant of the single-FC shape (256x128 tiles by
-    the shape rule; the other large tiles forced)."""
+    """The benchmark's M = 16384 variant of the single-FC shape (256x256 tiles
+    with eight waves by the shape rule; the other large tiles forced)."""
     say("rwq_fc M16384 K1024 N1024 tile", TILES.get(tile, "by shape"))
     rows = np.r_[0:40, 1000:1040, 2040:2048]
-    _check_large(16384, 1024, 1024, 83 + (tile or 0), tile in (None, 4), 2048, rows, tile)
+    _check_large(16384, 1024, 1024, 83 + (tile or 0), tile in (None, 4, 10), 2048, rows, tile)
 
 
 def test_rwq_fc_m4096_k1024_n1024_all_tiles_agree():
-    """One mid-size product on all six tiles: identical bytes."""
+    """One mid-size product on every tile: identical bytes."""
     c = cases.rwq_fc_case(77, 4096, 1024, 1024, symmetric=False)
     c["x"][2048:] = c["x"][:2048]
     ref = None
