@@ -183,18 +183,28 @@ static int conv_common(int8_t *out, const int8_t *in, const int8_t *filter,
       return conv_halo_launch(in, filter, g, ep, lds, rows, as_stream(stream));
     }
   }
-  // Pointwise convolutions (any stride) over 64, 128 or 256 channels: the
+  // Pointwise convolutions (any stride) over 64, 128 or 256 channels, and
+  // windows without padding or dilation whose rows are whole 32-byte chunks
+  // (KW * IC of 32, 64 or 128 bytes; the stem of an image network after
+  // space-to-depth: 4x4 over 16 channels) with K of 64, 128 or 256: the
   // streaming kernel (gemm_stream.h), by its shape rule or when tile 8 is
   // asked for.
-  if (g->KH == 1 && g->KW == 1 && g->padT == 0 && g->padL == 0 && g->group == 1 &&
-      (long long)(g->OH - 1) * g->strideH < g->IH && (long long)(g->OW - 1) * g->strideW < g->IW &&
+  const long long seg = (long long)g->KW * g->IC;        // bytes per window row
+  const bool seg_ok = g->KH == 1 ? g->KW == 1
+                                 : (seg == 32 || seg == 64 || seg == 128) && g->dilH == 1 &&
+                                       g->dilW == 1 && g->IC % 16 == 0;
+  if (seg_ok && g->padT == 0 && g->padL == 0 && g->group == 1 &&
+      (long long)(g->OH - 1) * g->strideH + g->KH <= g->IH &&
+      (long long)(g->OW - 1) * g->strideW + g->KW <= g->IW &&
       (g_tile_override == 8 || (g_tile_override < 0 && stream_applies((int)M, OCg))) &&
       stream_can_run((int)M, OCg, (int)K, need_sa, need_sb, al_a && al_b, ep)) {
     StreamRows R;
     R.in = in; R.ld = g->IC;
-    R.dense = g->strideH == 1 && g->strideW == 1 && g->OH == g->IH && g->OW == g->IW;
+    R.dense = g->KH == 1 && g->strideH == 1 && g->strideW == 1 && g->OH == g->IH && g->OW == g->IW;
     R.OW = g->OW; R.OHW = g->OH * g->OW; R.IH = g->IH; R.IW = g->IW; R.IC = g->IC;
     R.sH = g->strideH; R.sW = g->strideW;
+    R.seg_chunks = g->KH > 1 ? (int)(seg / 32) : (int)(K / 32);
+    R.seg_stride = (long long)g->IW * g->IC;
     ep.fast = g_requant_hint & 3;
     return gemm_stream_launch(R, filter, ep, (int)M, OCg, (int)K, as_stream(stream));
   }

@@ -94,7 +94,7 @@ static int fc_common(int8_t *out, const int8_t *in, const int8_t *w_nk,
   if ((g_tile_override == 8 || (g_tile_override < 0 && stream_applies((int)M, (int)N))) &&
       stream_can_run((int)M, (int)N, (int)K, need_sa, need_sb, aligned, ep)) {
     StreamRows R{};
-    R.in = in; R.ld = (long long)K; R.dense = 1;
+    R.in = in; R.ld = (long long)K; R.dense = 1; R.seg_chunks = (int)(K / 32);
     ep.fast = g_requant_hint & 3;
     return gemm_stream_launch(R, w_nk, ep, (int)M, (int)N, (int)K, as_stream(stream));
   }

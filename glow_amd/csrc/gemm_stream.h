@@ -31,19 +31,27 @@ namespace mi355x {
 constexpr int kStreamMaxBN = 256;   // columns per workgroup slice (and the table's stride)
 constexpr int kStreamParBytes = kParArrays * kStreamMaxBN * 4;
 
-// Rows of A: dense (row m at in + m * ld), or the pixels a strided pointwise
-// convolution reads (output pixel m of an [N, OH, OW] grid -> input pixel
-// (n, oh * sH, ow * sW) of an [N, IH, IW, IC] tensor).
+// Rows of A: dense (row m at in + m * ld), or the window a convolution without
+// padding and dilation reads for output pixel m of an [N, OH, OW] grid: it
+// starts at input pixel (n, oh * sH, ow * sW) of an [N, IH, IW, IC] tensor and
+// has KH segments of KW * IC contiguous bytes, one input row apart (a pointwise
+// convolution: one segment of IC bytes).
 struct StreamRows {
   const int8_t *in;
   long long ld;
   int dense;
   int OW, OHW, IH, IW, IC, sH, sW;
+  int seg_chunks;        // 32-byte chunks per segment (a power of two; K / 32: one segment)
+  long long seg_stride;  // bytes between segments
   __device__ __forceinline__ const int8_t *row(int m) const {
     if (dense) return in + (long long)m * ld;
     const int n = m / OHW, r = m - n * OHW;
     const int oh = r / OW, ow = r - oh * OW;
     return in + (((long long)n * IH + (long long)oh * sH) * IW + (long long)ow * sW) * IC;
+  }
+  // byte offset of chunk ks of a row from the row's start
+  __device__ __forceinline__ long long chunk(int ks) const {
+    return (long long)(ks / seg_chunks) * seg_stride + (ks % seg_chunks) * 32;
   }
 };
 
@@ -76,8 +84,13 @@ __device__ __forceinline__ void stream_tiles(const StreamRows &A, const int8_t *
     // rows past the end re-read the last row; their results are not stored
     const int8_t *ar = A.row(min(m0 + l32, M - 1)) + lhi * 16;
     v4i af[KS];
+    if (A.seg_chunks >= KS) {
 #pragma unroll
-    for (int ks = 0; ks < KS; ks++) af[ks] = *reinterpret_cast<const v4i *>(ar + ks * 32);
+      for (int ks = 0; ks < KS; ks++) af[ks] = *reinterpret_cast<const v4i *>(ar + ks * 32);
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) af[ks] = *reinterpret_cast<const v4i *>(ar + A.chunk(ks));
+    }
     for (int c0 = 0; c0 < bn; c0 += group) {
       for (int j = c0 / 32; j < (c0 + group) / 32; j++) {
         v16i acc;

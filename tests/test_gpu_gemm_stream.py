@@ -117,6 +117,35 @@ def test_stream_pointwise_conv_vs_oracle(kw):
     assert want.std() > 1
 
 
+WINDOW_CASES = [
+    # the stem of an image network after space-to-depth: 4x4 over 16 channels
+    dict(N=2, H=115, W=115, IC=16, OC=64, kernel=(4, 4)),
+    dict(N=1, H=9, W=11, IC=16, OC=32, kernel=(2, 2), act=go.ACT_CLIP),             # K 64
+    dict(N=3, H=8, W=8, IC=32, OC=96, kernel=(2, 2), stride=(2, 2), in_offset=4),   # K 128
+    dict(N=1, H=10, W=7, IC=64, OC=64, kernel=(2, 2), stride=(1, 2)),               # K 256
+    dict(N=2, H=6, W=12, IC=16, OC=256, kernel=(2, 8), act=go.ACT_LEAKY_RELU),      # rows of 128 bytes
+    dict(N=1, H=7, W=7, IC=32, OC=64, kernel=(4, 1), bias_i8=True),                 # rows of 32 bytes
+]
+
+
+@pytest.mark.parametrize("kw", WINDOW_CASES)
+def test_stream_window_conv_vs_oracle(kw):
+    """Windows without padding whose rows are whole 32-byte chunks run on the
+    streaming kernel as rows of several segments."""
+    kw = dict(kw)
+    kw.setdefault("in_offset", -128)
+    c = cases.cwq_conv_case(63, pads=(0, 0, 0, 0), **kw)
+    g = c["geom"]
+    say("stream window conv", kw, "output", g.OH, "x", g.OW)
+    want = go.cwq_conv2d_i8(*cases.cwq_conv_args(c))
+    with forced_tile(8):
+        got = capi.cwq_conv2d_i8(*cases.cwq_conv_args(c))
+    np.testing.assert_array_equal(got, want)
+    with forced_tile(2):
+        np.testing.assert_array_equal(capi.cwq_conv2d_i8(*cases.cwq_conv_args(c)), want)
+    assert want.std() > 1
+
+
 @pytest.mark.parametrize("relu", [False, True])
 @pytest.mark.parametrize("IC,OC", [(64, 256), (128, 512), (256, 1024)])
 def test_stream_conv_with_fused_residual_add(IC, OC, relu):
