@@ -2108,7 +2108,8 @@ Error MI355XFunction::captureGraph(const DeviceBindings &b, const std::vector<vo
   if (launches.empty()) return Error::success();
   if (!b.stream)
     return MI355X_MAKE_ERR(ErrorCode::RUNTIME_ERROR, "graph capture needs a created stream");
-  const size_t n = launches.size(), nLanes = sideStreams.size() + 1;
+  const size_t n = launches.size();
+  size_t nLanes = sideStreams.size() + 1;
   // Direct predecessors only: a conflicting launch that is already an ancestor
   // of a later predecessor is ordered through it (memory shared by values whose
   // lives do not meet makes a launch conflict with every earlier owner of its
@@ -2141,30 +2142,53 @@ Error MI355XFunction::captureGraph(const DeviceBindings &b, const std::vector<vo
       if (depth[p] + 1 > depth[i]) depth[i] = depth[p] + 1;
       if (heir[p] < 0 || height[i] > height[(size_t)heir[p]]) heir[p] = (long long)i;
     }
+  // The waits between side streams must not run in a circle (stream 1 waits
+  // for 2, 2 for 3, 3 for 1, each at a different point of the recording): the
+  // runtime's end-of-capture walk over the streams that joined a capture does
+  // not come back from such a ring. The capturing stream is exempt (every side
+  // stream forks from it and joins it). When the assignment below produces a
+  // ring it is redone with one lane fewer; with a single side stream there is
+  // none.
   std::vector<int> lane(n, 0);
-  std::vector<long long> last(nLanes, -1);    // last launch put on each lane
-  for (size_t i = 0; i < n; i++) {
-    int pick = -1;
-    // the heir continues; the heir of several launches follows the deepest
-    long long from = -1;
-    for (size_t p : preds[i])
-      if (heir[p] == (long long)i && (from < 0 || depth[p] >= depth[(size_t)from])) from = (long long)p;
-    if (from >= 0) pick = lane[(size_t)from];
-    if (pick < 0)
-      for (size_t l = 0; l < nLanes && pick < 0; l++)
-        if (last[l] < 0) pick = (int)l;                                  // an unused lane
-    // lanes whose last launch still waits for its heir are kept for it
-    auto kept = [&](size_t l) { return heir[(size_t)last[l]] > (long long)i; };
-    if (pick < 0)
-      for (auto it = preds[i].rbegin(); it != preds[i].rend() && pick < 0; ++it)
-        if (last[(size_t)lane[*it]] == (long long)*it && !kept((size_t)lane[*it]))
-          pick = lane[*it];                                              // behind a predecessor
-    if (pick < 0)
-      for (size_t l = 0; l < nLanes; l++)                                // idle longest
-        if (!kept(l) && (pick < 0 || last[l] < last[(size_t)pick])) pick = (int)l;
-    if (pick < 0) pick = preds[i].empty() ? 0 : lane[preds[i].back()];
-    lane[i] = pick;
-    last[(size_t)pick] = (long long)i;
+  std::vector<long long> last;
+  for (;; nLanes--) {
+    std::fill(lane.begin(), lane.end(), 0);
+    last.assign(nLanes, -1);                  // last launch put on each lane
+    for (size_t i = 0; i < n; i++) {
+      int pick = -1;
+      // the heir continues; the heir of several launches follows the deepest
+      long long from = -1;
+      for (size_t p : preds[i])
+        if (heir[p] == (long long)i && (from < 0 || depth[p] >= depth[(size_t)from])) from = (long long)p;
+      if (from >= 0) pick = lane[(size_t)from];
+      if (pick < 0)
+        for (size_t l = 0; l < nLanes && pick < 0; l++)
+          if (last[l] < 0) pick = (int)l;                                  // an unused lane
+      // lanes whose last launch still waits for its heir are kept for it
+      auto kept = [&](size_t l) { return heir[(size_t)last[l]] > (long long)i; };
+      if (pick < 0)
+        for (auto it = preds[i].rbegin(); it != preds[i].rend() && pick < 0; ++it)
+          if (last[(size_t)lane[*it]] == (long long)*it && !kept((size_t)lane[*it]))
+            pick = lane[*it];                                              // behind a predecessor
+      if (pick < 0)
+        for (size_t l = 0; l < nLanes; l++)                                // idle longest
+          if (!kept(l) && (pick < 0 || last[l] < last[(size_t)pick])) pick = (int)l;
+      if (pick < 0) pick = preds[i].empty() ? 0 : lane[preds[i].back()];
+      lane[i] = pick;
+      last[(size_t)pick] = (long long)i;
+    }
+    if (nLanes <= 2) break;
+    std::vector<std::vector<char>> waits(nLanes, std::vector<char>(nLanes, 0));
+    for (size_t i = 0; i < n; i++)
+      for (size_t p : preds[i])
+        if (lane[p] != lane[i] && lane[p] != 0 && lane[i] != 0) waits[(size_t)lane[p]][(size_t)lane[i]] = 1;
+    for (size_t k = 1; k < nLanes; k++)       // transitive closure over the side lanes
+      for (size_t a = 1; a < nLanes; a++)
+        for (size_t c = 1; c < nLanes; c++)
+          if (waits[a][k] && waits[k][c]) waits[a][c] = 1;
+    bool ring = false;
+    for (size_t a = 1; a < nLanes; a++) ring = ring || waits[a][a];
+    if (!ring) break;
   }
   // which launches need an event recorded behind them
   std::vector<char> needsEvent(n, 0);

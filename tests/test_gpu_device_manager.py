@@ -474,3 +474,55 @@ def test_copy_into_an_output_placeholder(dm):
     got = np.zeros(256, np.int8)
     dm.run("main", {"input": c["x"], "output": got})
     assert np.array_equal(got.reshape(8, 32), _rwq_expected(c))
+
+
+def test_chains_that_wait_for_each_other_in_a_ring():
+    """Three chains of adds where the second waits for the first, the third for
+    the second and the first, further on, for the third: recorded on one side
+    stream per chain, the waits between the streams would run in a circle. The
+    recording must come out (with fewer streams) and compute the same sums."""
+    n, shape = 4, (64, 256)
+    m = H.Module()
+    ty = (H.INT8Q, np.int8, 0.1, 0)
+    ins = [m.placeholder(f"in{i}", shape, *ty) for i in range(n)]
+    outs = [m.placeholder(f"out{i}", shape, *ty) for i in range(n)]
+    f = m.function("main")
+    act = lambda name: m.activation(f, name, shape, H.INT8Q, 0.1, 0)
+    ops = []                       # (dest, lhs, rhs) by name, for the restatement below
+
+    def add(dest, lhs, rhs, names):
+        m.instruction(f, H.ELEMENT_ADD, names[0], [dest, lhs, rhs])
+        ops.append(names)
+
+    v = {}
+    for i in range(n):             # every chain starts on its own
+        v[f"c{i}_0"] = act(f"c{i}_0")
+        add(v[f"c{i}_0"], ins[i], ins[i], (f"c{i}_0", f"in{i}", f"in{i}"))
+    # chain 0 is long (it keeps the capturing stream); 1 -> 2 -> 3 -> 1 cross over
+    for k in range(1, 5):
+        v[f"c0_{k}"] = act(f"c0_{k}")
+        add(v[f"c0_{k}"], v[f"c0_{k-1}"], ins[0], (f"c0_{k}", f"c0_{k-1}", "in0"))
+    v["c2_1"] = act("c2_1"); add(v["c2_1"], v["c2_0"], v["c1_0"], ("c2_1", "c2_0", "c1_0"))
+    v["c3_1"] = act("c3_1"); add(v["c3_1"], v["c3_0"], v["c2_1"], ("c3_1", "c3_0", "c2_1"))
+    v["c1_1"] = act("c1_1"); add(v["c1_1"], v["c1_0"], v["c3_1"], ("c1_1", "c1_0", "c3_1"))
+    v["c2_2"] = act("c2_2"); add(v["c2_2"], v["c2_1"], v["c1_1"], ("c2_2", "c2_1", "c1_1"))
+    for i, last in enumerate(["c0_4", "c1_1", "c2_2", "c3_1"]):
+        add(outs[i], v[last], ins[i], (f"out{i}", last, f"in{i}"))
+    m.compile(f)
+    rng = np.random.default_rng(5)
+    x = {f"in{i}": rng.integers(-20, 21, shape).astype(np.int8) for i in range(n)}
+    one = go.quantize_scale_offset_32to8(1.0, 0)[:3]
+    want = dict(x)
+    for dest, lhs, rhs in ops:
+        want[dest] = go.add_i8(want[lhs], want[rhs], 0, 0, 0, one, one)
+    for graphs in (-4, True, False):
+        dm = H.DeviceManager(use_launch_graphs=graphs).init()
+        try:
+            dm.add_network(m)
+            for _ in range(2):
+                got = {f"out{i}": np.zeros(shape, np.int8) for i in range(n)}
+                dm.run("main", dict(x, **got))
+                for i in range(n):
+                    np.testing.assert_array_equal(got[f"out{i}"], want[f"out{i}"])
+        finally:
+            dm.stop()
