@@ -26,7 +26,7 @@ EXPORTS = [
     "mi355x_cwq_conv2d_add_i8", "mi355x_frwq_sls_multi",
     "mi355x_specialize_bias_weights_qparams", "mi355x_rwq_slws", "mi355x_slws_set_fused_math", "mi355x_batch_matmul_nt_i8", "mi355x_batch_matmul_nt_select_i8", "mi355x_rwq_fc_relu_i8", "mi355x_add_i8", "mi355x_add_relu_i8",
     "mi355x_relu_i8", "mi355x_convert_f16_to_f32", "mi355x_insert_rows",
-    "mi355x_batch_transpose_i8", "mi355x_space_to_depth2_i8", "mi355x_gather", "mi355x_gather_rows", "mi355x_rescale_rows_i8",
+    "mi355x_batch_transpose_i8", "mi355x_space_to_depth2_i8", "mi355x_quantize_space_to_depth2_i8", "mi355x_gather", "mi355x_gather_rows", "mi355x_rescale_rows_i8",
     "mi355x_dequantize_sigmoid", "mi355x_batch_matmul_i8", "mi355x_sigmoid_f32",
     "mi355x_max_pool_i8", "mi355x_avg_pool_i8", "mi355x_softmax_f32", "mi355x_stream_create",
     "mi355x_stream_destroy", "mi355x_stream_sync", "mi355x_device_sync",
@@ -1242,6 +1242,17 @@ def space_to_depth2_i8(x, pad_t, pad_l, bh, bw, cout, fill):
     check(lib().mi355x_space_to_depth2_i8(_vp(out), _vp(dx), _sz(n), _sz(ih), _sz(iw), _sz(c),
                                           _sz(pad_t), _sz(pad_l), _sz(bh), _sz(bw), _sz(cout),
                                           _i32(fill), _vp(None)))
+    return out.numpy()
+
+
+def quantize_space_to_depth2_i8(x, pad_t, pad_l, bh, bw, cout, fill, scale, offset):
+    x = np.ascontiguousarray(x, np.float32)
+    n, ih, iw, c = x.shape
+    dx = to_device(x)
+    out = DeviceBuffer.empty((n, bh, bw, cout), np.int8)
+    check(lib().mi355x_quantize_space_to_depth2_i8(
+        _vp(out), _vp(dx), _sz(n), _sz(ih), _sz(iw), _sz(c), _sz(pad_t), _sz(pad_l), _sz(bh),
+        _sz(bw), _sz(cout), _i32(fill), C.c_float(scale), _i32(offset), _vp(None)))
     return out.numpy()
 
 

@@ -519,6 +519,43 @@ __global__ __launch_bounds__(kGlueThreads) void space_to_depth2_c16_i8_kernel(
   dst[t] = make_uint4(w[0], w[1], w[2], w[3]);
 }
 
+// Quantize (libjit_quantize_kernel: clip(nearbyintf(x / scale + offset)), every
+// operation rounded on its own) and space-to-depth in one pass: the float
+// image is read once and the int8 image in between is never written. The
+// values are those of mi355x_quantize_i8 followed by mi355x_space_to_depth2_i8.
+template <int C>
+__global__ __launch_bounds__(kGlueThreads) void quantize_space_to_depth2_c16_kernel(
+    uint4 *__restrict__ dst, const float *__restrict__ src, int N, int IH, int IW, int padT,
+    int padL, int BH, int BW, int fill, float scale, float offset, long long total) {
+  const long long t = (long long)blockIdx.x * kGlueThreads + threadIdx.x;
+  if (t >= total) return;
+  const int bw = (int)(t % BW);
+  long long r = t / BW;
+  const int bh = (int)(r % BH);
+  const int n = (int)(r / BH);
+  uint8_t b[16];
+#pragma unroll
+  for (int i = 0; i < 16; i++) b[i] = (uint8_t)fill;
+#pragma unroll
+  for (int q = 0; q < 4; q++) {
+    const int ih = 2 * bh + (q >> 1) - padT, iw = 2 * bw + (q & 1) - padL;
+    if (ih >= 0 && ih < IH && iw >= 0 && iw < IW) {
+      const float *p = src + (((long long)n * IH + ih) * IW + iw) * C;
+#pragma unroll
+      for (int c = 0; c < C; c++) {
+        const float v = rintf(__fadd_rn(__fdiv_rn(p[c], scale), offset));
+        b[q * C + c] = (uint8_t)clip_i8((int32_t)v);
+      }
+    }
+  }
+  uint32_t w[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++)
+    w[j] = (uint32_t)b[4 * j] | ((uint32_t)b[4 * j + 1] << 8) | ((uint32_t)b[4 * j + 2] << 16) |
+           ((uint32_t)b[4 * j + 3] << 24);
+  dst[t] = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
 // libjit_sigmoid_kernel_f: 1 / (expf(-x) + 1)
 __global__ __launch_bounds__(kGlueThreads) void sigmoid_f32_kernel(
     float *__restrict__ dst, const float *__restrict__ src, size_t n) {
@@ -840,6 +877,27 @@ int mi355x_space_to_depth2_i8(int8_t *dst, const int8_t *src, size_t N, size_t I
                      dim3(kGlueThreads), 0, as_stream(stream), dst, src, (int)N, (int)IH, (int)IW,
                      (int)C, (int)padT, (int)padL, (int)BH, (int)BW, (int)Cout, fill, total);
   return check_launch("space_to_depth2_i8");
+}
+
+int mi355x_quantize_space_to_depth2_i8(int8_t *dst, const float *src, size_t N, size_t IH,
+                                       size_t IW, size_t C, size_t padT, size_t padL, size_t BH,
+                                       size_t BW, size_t Cout, int32_t fill, float scale,
+                                       int32_t offset, void *stream) {
+  if (N == 0 || BH == 0 || BW == 0) return MI355X_OK;
+  MI355X_REQUIRE(dst && src, "NULL tensor");
+  MI355X_REQUIRE((C == 3 || C == 4) && Cout == 16, "3 or 4 channels into 16 only");
+  MI355X_REQUIRE((((uintptr_t)dst) & 15) == 0 && (((uintptr_t)src) & 3) == 0, "unaligned tensor");
+  const size_t lim = 1u << 30;
+  MI355X_REQUIRE(N < lim && IH < lim && IW < lim && BH < lim && BW < lim && padT < lim && padL < lim,
+                 "dimensions too large");
+  MI355X_REQUIRE(fill >= -128 && fill <= 127, "fill outside the int8 range");
+  const long long total = (long long)N * BH * BW;
+  MI355X_REQUIRE(total / kGlueThreads < 0x7fffffffLL, "tensor too large");
+  auto kern = C == 3 ? quantize_space_to_depth2_c16_kernel<3> : quantize_space_to_depth2_c16_kernel<4>;
+  hipLaunchKernelGGL(kern, dim3(glue_blocks((size_t)total)), dim3(kGlueThreads), 0,
+                     as_stream(stream), (uint4 *)dst, src, (int)N, (int)IH, (int)IW, (int)padT,
+                     (int)padL, (int)BH, (int)BW, fill, scale, (float)offset, total);
+  return check_launch("quantize_space_to_depth2_i8");
 }
 
 int mi355x_sigmoid_f32(float *dst, const float *src, size_t n, void *stream) {

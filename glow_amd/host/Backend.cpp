@@ -185,7 +185,27 @@ public:
         if (ins) { absorbed_[ins] = 1; folded.push_back(ins); }
         break;
       }
-      case Kind::Quantize: MI355X_RETURN_IF_ERR(quantize(I, out)); break;
+      case Kind::Quantize: {
+        // a Quantize read only by the convolution right behind it: when that
+        // convolution goes through space-to-depth (the stem of an image
+        // network), the layout change quantizes on the way
+        const Instruction *cv = at + 1 < insts_.size() ? &insts_[at + 1] : nullptr;
+        const bool convKind = cv && (cv->kind == Kind::Convolution ||
+                                     cv->kind == Kind::ChannelwiseQuantizedConvolution);
+        if (opts_.fuseQuantizeStem && convKind && cv->operands[1] == I.operands[0] &&
+            M_.value(I.operands[0]).category == SymbolCategory::Activation &&
+            M_.value(I.operands[0]).type.kind == ElemKind::Int8QTy &&
+            M_.value(I.operands[0]).type.dims.size() == 4 && readers(I.operands[0]) == 1 &&
+            writers(I.operands[0]) == 1 &&
+            !(at + 2 < insts_.size() && insts_[at + 2].kind == Kind::ElementAdd)) {
+          MI355X_RETURN_IF_ERR(conv(*cv, out, cv->kind == Kind::ChannelwiseQuantizedConvolution,
+                                    nullptr, nullptr, &I));
+          at++;
+        } else {
+          MI355X_RETURN_IF_ERR(quantize(I, out));
+        }
+        break;
+      }
       case Kind::Dequantize: {
         // a Sigmoid right behind it that is the only reader of its result
         const Instruction *sig = nullptr;
@@ -1414,8 +1434,12 @@ private:
     return Error::success();
   }
 
+  // quantI: the Quantize whose result this convolution alone reads (it is
+  // emitted here: folded into the space-to-depth pass, or as its own launch
+  // in front of everything else)
   Error conv(const Instruction &I, MI355XFunction &out, bool channelwise,
-             const Instruction *addI = nullptr, const Instruction *reluI = nullptr) {
+             const Instruction *addI = nullptr, const Instruction *reluI = nullptr,
+             const Instruction *quantI = nullptr) {
     Operand d = op(I, 0), s = op(I, 1), f = op(I, 2), bi = op(I, 3);
     CHECK_OP((int)I.iattrs.size() == ConvAttrs::kCount, "expects %d integer attributes",
              ConvAttrs::kCount);
@@ -1478,6 +1502,7 @@ private:
                                     "padT=%d padL=%d dH=%d dW=%d group=%d",
                                     g.N, g.IH, g.IW, g.IC, g.OH, g.OW, g.OC, g.KH, g.KW, g.strideH,
                                     g.strideW, g.padT, g.padL, g.dilH, g.dilW, g.group);
+    if (quantI && !channelwise) MI355X_RETURN_IF_ERR(quantize(*quantI, out));
     if (!channelwise) {
       const float mm = s.ty().scale * f.ty().scale;
       const S32To8 bp = s32to8(bi.ty().scale / mm), opp = s32to8(mm / d.ty().scale);
@@ -1573,14 +1598,31 @@ private:
       priv.root = -100 - (int)out.launches.size();
       const size_t N = (size_t)g.N, IH = (size_t)g.IH, IW = (size_t)g.IW, IC = (size_t)g.IC,
                    pT = (size_t)g.padT, pL = (size_t)g.padL;
-      out.launches.push_back(
-          {"mi355x_space_to_depth2_i8", I.name + ".s2d",
-           strFormat(" N=%zu IH=%zu IW=%zu C=%zu padT=%zu padL=%zu BH=%zu BW=%zu Cout=%d", N, IH, IW, IC,
-                     pT, pL, BH, BW, C2) + kv("fill", io),
-           [=](const DeviceBindings &b) {
-             return mi355x_space_to_depth2_i8((int8_t *)sPtr(b), (const int8_t *)s.ptr(b), N, IH, IW, IC,
-                                              pT, pL, BH, BW, (size_t)C2, io, b.stream);
-           }});
+      if (quantI && (IC == 3 || IC == 4) && op(*quantI, 1).ty().kind == ElemKind::FloatTy &&
+          op(*quantI, 1).ty().size() == s.ty().size()) {
+        // the float image is quantized while it is re-laid
+        Operand qs = op(*quantI, 1);
+        const float qscale = s.ty().scale;
+        out.launches.push_back(
+            {"mi355x_quantize_space_to_depth2_i8", quantI->name + "+" + I.name + ".s2d",
+             strFormat(" N=%zu IH=%zu IW=%zu C=%zu padT=%zu padL=%zu BH=%zu BW=%zu Cout=%d scale=%.9g", N,
+                       IH, IW, IC, pT, pL, BH, BW, C2, (double)qscale) + kv("offset", io) + kv("fill", io),
+             [=](const DeviceBindings &b) {
+               return mi355x_quantize_space_to_depth2_i8((int8_t *)sPtr(b), (const float *)qs.ptr(b), N,
+                                                         IH, IW, IC, pT, pL, BH, BW, (size_t)C2, io,
+                                                         qscale, io, b.stream);
+             }});
+      } else {
+        if (quantI) MI355X_RETURN_IF_ERR(quantize(*quantI, out));
+        out.launches.push_back(
+            {"mi355x_space_to_depth2_i8", I.name + ".s2d",
+             strFormat(" N=%zu IH=%zu IW=%zu C=%zu padT=%zu padL=%zu BH=%zu BW=%zu Cout=%d", N, IH, IW, IC,
+                       pT, pL, BH, BW, C2) + kv("fill", io),
+             [=](const DeviceBindings &b) {
+               return mi355x_space_to_depth2_i8((int8_t *)sPtr(b), (const int8_t *)s.ptr(b), N, IH, IW, IC,
+                                                pT, pL, BH, BW, (size_t)C2, io, b.stream);
+             }});
+      }
       out.launches.back().writes.push_back(priv);
       out.launches.push_back(
           {"mi355x_cwq_conv2d_i8", I.name,
@@ -1604,6 +1646,7 @@ private:
       out.launches.back().reads.push_back(priv);
       return Error::success();
     }
+    if (quantI) MI355X_RETURN_IF_ERR(quantize(*quantI, out));
     if (addI) {
       const Instruction &A = *addI;
       const bool convIsLhs = A.operands[1] == I.operands[0];

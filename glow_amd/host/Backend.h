@@ -186,6 +186,7 @@ struct BackendOptions {
   bool fuseInsert = true;              // Gather / RescaleQuantized write straight into the tensor their result is inserted into
   bool fuseDequantizeSigmoid = true;   // Dequantize + Sigmoid of its result in one kernel
   bool deriveBagOffsets = true;        // lookups whose lengths are an input: bag positions summed on the host at upload
+  bool fuseQuantizeStem = true;        // Quantize read only by a space-to-depth convolution: quantized while re-laid
   bool reuseActivations = true;        // activations whose lives do not meet share memory (first fit over the launch order)
 };
 

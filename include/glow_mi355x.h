@@ -367,6 +367,14 @@ int mi355x_batch_matmul_nt_select_i8(int8_t *out, const int8_t *lhs, const int8_
 int mi355x_space_to_depth2_i8(int8_t *dst, const int8_t *src, size_t N, size_t IH, size_t IW,
                               size_t C, size_t padT, size_t padL, size_t BH, size_t BW,
                               size_t Cout, int32_t fill, void *stream);
+/* mi355x_quantize_i8 (libjit_quantize_kernel, libjit.cpp:1683-1698 over
+ * libjit_defs.h:118-124) followed by mi355x_space_to_depth2_i8 in one pass over
+ * the float image [N, IH, IW, C], C of 3 or 4 into Cout = 16: the same bytes,
+ * without the int8 image in between. No counterpart in the reference. */
+int mi355x_quantize_space_to_depth2_i8(int8_t *dst, const float *src, size_t N, size_t IH,
+                                       size_t IW, size_t C, size_t padT, size_t padL, size_t BH,
+                                       size_t BW, size_t Cout, int32_t fill, float scale,
+                                       int32_t offset, void *stream);
 /* libjit_sigmoid_kernel_f (libjit.cpp:1913-1916): 1 / (expf(-x) + 1); agrees
  * with the CPU to fp32 rounding of expf (1e-5 relative). */
 int mi355x_sigmoid_f32(float *dst, const float *src, size_t n, void *stream);

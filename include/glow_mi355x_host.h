@@ -131,7 +131,9 @@ enum {
   MI355X_HOST_OPT_REUSE_ACTIVATIONS = 2048, /* activations whose lives do not meet in the dependence
                                              * graph share memory (AllocationsInfo.cpp:128-156); off:
                                              * every value has bytes of its own */
-  MI355X_HOST_OPT_DEFAULT = 4095
+  MI355X_HOST_OPT_FUSE_QUANTIZE_STEM = 4096, /* a Quantize read only by a convolution that goes
+                                              * through space-to-depth is applied by that pass */
+  MI355X_HOST_OPT_DEFAULT = 8191
 };
 int mi355x_host_compile(mi355x_host_module *m, int function, int options);
 /* Listing of the compiled function's launches and derived parameters; returns

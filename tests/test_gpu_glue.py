@@ -180,6 +180,23 @@ def test_space_to_depth(shape, pads):
     np.testing.assert_array_equal(capi.space_to_depth2_i8(x, pads[0], pads[1], bh, bw, cout, fill), want)
 
 
+@pytest.mark.parametrize("shape,pads", [((2, 16, 16, 3), (3, 3)), ((1, 9, 7, 4), (0, 1)), ((2, 224, 224, 3), (3, 3))])
+def test_quantize_and_space_to_depth_in_one_pass(shape, pads):
+    """The fused pass writes what Quantize (against the oracle) followed by the
+    layout change writes."""
+    rng = np.random.default_rng(shape[1] + 1)
+    x = rng.normal(0.45, 0.25, shape).astype(np.float32)
+    x.reshape(-1)[:8] = [0.0, -0.0, 1e9, -1e9, 0.0125, -0.0125, 0.0375, 3.175]   # ties and clips
+    scale, offset = 0.025, -128
+    q = go.quantize_i8(x, scale, offset)
+    n, ih, iw, c = shape
+    bh, bw, cout, fill = (ih + pads[0] + 4) // 2, (iw + pads[1] + 4) // 2, 16, offset
+    want = capi.space_to_depth2_i8(q, pads[0], pads[1], bh, bw, cout, fill)
+    got = capi.quantize_space_to_depth2_i8(x, pads[0], pads[1], bh, bw, cout, fill, scale, offset)
+    np.testing.assert_array_equal(got, want)
+    assert len(np.unique(got)) > 20
+
+
 def test_add_with_scales_beyond_24_bits():
     """Parameters outside the 24-bit fast path take the 32-bit multiplier."""
     rng = np.random.default_rng(31)

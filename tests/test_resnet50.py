@@ -41,10 +41,16 @@ def test_small_network_compiles_and_fuses():
     m2.compile(f2, fuse_conv_add=False, space_to_depth_stem=False)
     k2 = [r["kernel"] for r in H.parse_listing(m2.describe(f2)) if r["phase"] == "launch"]
     assert k2.count("mi355x_add_relu_i8") == 3 and k2.count("mi355x_cwq_conv2d_i8") == 11
-    assert kernels[-1] == "mi355x_softmax_f32" and kernels[0] == "mi355x_quantize_i8"
     # the 7x7 stride-2 stem over 3 channels runs as a 4x4 stride-1 convolution
-    # over a space-to-depth image of 16 channels
-    assert kernels[1] == "mi355x_space_to_depth2_i8"
+    # over a space-to-depth image of 16 channels, which is quantized from the
+    # float input while it is re-laid
+    assert kernels[-1] == "mi355x_softmax_f32"
+    assert kernels[0] == "mi355x_quantize_space_to_depth2_i8" and "mi355x_quantize_i8" not in kernels
+    m3, f3 = netlib.to_module(net)
+    m3.compile(f3, fuse_quantize_stem=False)
+    k3 = [r["kernel"] for r in H.parse_listing(m3.describe(f3)) if r["phase"] == "launch"]
+    assert k3[:2] == ["mi355x_quantize_i8", "mi355x_space_to_depth2_i8"] and k3[2:] == kernels[1:]
+    assert k2[0] == "mi355x_quantize_i8" and "mi355x_space_to_depth2_i8" not in k2
     stem = [r for r in rows if r.get("space_to_depth") == 1][0]
     assert (stem["KH"], stem["KW"], stem["IC"], stem["IH"]) == (4, 4, 16, 16 + 3)
     # post-ReLU tensors use the unsigned range: offset -128
@@ -62,12 +68,14 @@ def test_oracle_executes_the_small_network():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("fuse", [(True, True, True), (True, False, False), (False, False, True)])
+@pytest.mark.parametrize("fuse", [(True, True, True), (True, False, False), (False, False, True),
+                                  (True, True, True, False)])
 def test_device_matches_oracle(fuse):
     net = resnet50.make(batch=2, size=64, profile_images=4, seed=5,
                         layers=((64, 2, 1), (128, 2, 2), (256, 1, 2)), classes=100)
     m, f = netlib.to_module(net)
-    m.compile(f, fuse_conv_add=fuse[0], fuse_add_relu=fuse[1], space_to_depth_stem=fuse[2])
+    m.compile(f, fuse_conv_add=fuse[0], fuse_add_relu=fuse[1], space_to_depth_stem=fuse[2],
+              fuse_quantize_stem=len(fuse) < 4)
     dm = H.DeviceManager().init()
     try:
         dm.add_network(m)
