@@ -104,7 +104,7 @@ def make(tables=26, rows=1_000_000, dim=64, batch=4096, mean_len=20, alpha=1.1,
     net.activation("dense_q", (batch, dense_features), H.INT8Q, *tq["dense"])
     net.op(H.QUANTIZE, "quantize_dense", ["dense_q", "dense"])
 
-    def fc_stack(layers, src, src_tq, prefix, last_relu):
+    def fc_stack(layers, src, src_tq, prefix, last_relu, out_placeholder=None):
         cur, cur_tq = src, src_tq
         for i, (w, b) in enumerate(layers):
             n, k = w.shape
@@ -125,6 +125,12 @@ def make(tables=26, rows=1_000_000, dim=64, batch=4096, mean_len=20, alpha=1.1,
                                                       name + "_s", name + "_o"])
                 net.activation(name, (batch, n), H.INT8Q, *out_tq)
                 net.op(H.RELU, name + "_relu", [name, name + "_pre"])
+            elif out_placeholder and i + 1 == len(layers):
+                # an output of the network: the last FC writes it where it is saved
+                net.placeholder(out_placeholder, (batch, n), H.INT8Q, *out_tq)
+                net.op(H.ROWWISE_QUANTIZED_FC, name, [out_placeholder, cur, name + "_w", name + "_b",
+                                                      name + "_s", name + "_o"])
+                name = out_placeholder
             else:
                 net.activation(name, (batch, n), H.INT8Q, *out_tq)
                 net.op(H.ROWWISE_QUANTIZED_FC, name, [name, cur, name + "_w", name + "_b",
@@ -163,9 +169,7 @@ def make(tables=26, rows=1_000_000, dim=64, batch=4096, mean_len=20, alpha=1.1,
     net.op(H.RESCALE_QUANTIZED, "bot_to_top", ["bot_z", bot_out])
     net.op(H.INSERT_TENSOR, "insert_dense", ["top_in", "bot_z"], [0])
     net.op(H.INSERT_TENSOR, "insert_pairs", ["top_in", "pairs"], [dim])
-    top_out, _ = fc_stack(topl, "top_in", tq["z"], "top", False)
-    net.placeholder("logit_q", (batch, top[-1]), H.INT8Q, *tq[f"top{len(topl) - 1}"])
-    net.op(H.RESCALE_QUANTIZED, "save_logit", ["logit_q", top_out])
+    top_out, _ = fc_stack(topl, "top_in", tq["z"], "top", False, "logit_q")
     net.activation("logit_f", (batch, top[-1]), H.FLOAT)
     net.op(H.DEQUANTIZE, "dequantize", ["logit_f", top_out])
     net.placeholder("prob", (batch, top[-1]), H.FLOAT)

@@ -213,18 +213,20 @@ def build_int8(steps, ranges, batch, size):
             net.constant("fc_bias", bq, H.INT32Q, bscale, boff)
             net.constant("fc_scales", ws, H.FLOAT)
             net.constant("fc_offsets", wo, H.INT32I)
-            # the pooled [N,1,1,C] tensor is read as [N,C]: same bytes
-            net.activation("gap_2d", (n, k), H.INT8Q, *tq[ins[0]])
-            net.op(H.RESCALE_QUANTIZED, "flatten", ["gap_2d", src])
-            net.activation(out, shapes[out], H.INT8Q, *tq[out])
-            net.op(H.ROWWISE_QUANTIZED_FC, "fc", [out, "gap_2d", "fc_weights", "fc_bias",
+            # the pooled [N,1,1,C] tensor is read as [N,C]: the same bytes (a
+            # Reshape is a TensorView in Glow's IR, no instruction)
+            net.view("gap_2d", src, (n, k))
+            # the int8 logits are an output of the network: the FC writes them
+            # where they are saved
+            net.placeholder("logits_q", shapes[out], H.INT8Q, *tq[out])
+            net.op(H.ROWWISE_QUANTIZED_FC, "fc", ["logits_q", "gap_2d", "fc_weights", "fc_bias",
                                                   "fc_scales", "fc_offsets"])
+            name_of[out] = "logits_q"
+            continue
         name_of[out] = out
     n, classes = shapes["logits"]
-    net.placeholder("logits_q", (n, classes), H.INT8Q, *tq["logits"])
-    net.op(H.RESCALE_QUANTIZED, "save_logits", ["logits_q", "logits"])
     net.activation("logits_f", (n, classes), H.FLOAT)
-    net.op(H.DEQUANTIZE, "dequantize", ["logits_f", "logits"])
+    net.op(H.DEQUANTIZE, "dequantize", ["logits_f", "logits_q"])
     net.placeholder("prob", (n, classes), H.FLOAT)
     net.op(H.SOFTMAX, "softmax", ["prob", "logits_f"])
     return net
