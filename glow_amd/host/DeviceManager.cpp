@@ -488,28 +488,42 @@ Error MI355XDeviceManager::tuneTiles(MI355XFunction *fn, const DeviceBindings &b
   for (int pass = 0; pass < 3 && rc == MI355X_OK; pass++)
     for (auto &l : fn->launches)
       if (rc == MI355X_OK) rc = l.launch(b);
+  // seconds of kRuns launches of launch l with tile t (the faster of kSeries
+  // series); negative when the tile cannot serve the launch
+  auto timeTile = [&](KernelLaunch &l, int t) -> float {
+    l.tile = t;
+    if (l.launch(b) != MI355X_OK) return -1.0f;   // warm-up, also rejects tiles the shape cannot use
+    float ms = 0.0f;
+    for (int s = 0; s < kSeries && rc == MI355X_OK; s++) {
+      rc = mi355x_event_record(e0, stream_);
+      for (int i = 0; i < kRuns && rc == MI355X_OK; i++) rc = l.launch(b);
+      if (rc == MI355X_OK) rc = mi355x_event_record(e1, stream_);
+      if (rc == MI355X_OK) rc = mi355x_event_sync(e1);
+      float one = 0.0f;
+      if (rc == MI355X_OK) rc = mi355x_event_elapsed_ms(e0, e1, &one);
+      if (s == 0 || one < ms) ms = one;
+    }
+    return ms;
+  };
   for (auto &l : fn->launches) {
     if (!l.tunable || rc != MI355X_OK) continue;
     float best = 0.0f;
     int bestTile = -1;
     for (int t = -1; t < kNumTiles && rc == MI355X_OK; t++) {
-      l.tile = t;
-      rc = l.launch(b); // warm-up, also rejects tiles the shape cannot use
-      if (rc != MI355X_OK) { rc = MI355X_OK; continue; }
-      float ms = 0.0f;
-      for (int s = 0; s < kSeries && rc == MI355X_OK; s++) {
-        rc = mi355x_event_record(e0, stream_);
-        for (int i = 0; i < kRuns && rc == MI355X_OK; i++) rc = l.launch(b);
-        if (rc == MI355X_OK) rc = mi355x_event_record(e1, stream_);
-        if (rc == MI355X_OK) rc = mi355x_event_sync(e1);
-        float one = 0.0f;
-        if (rc == MI355X_OK) rc = mi355x_event_elapsed_ms(e0, e1, &one);
-        if (s == 0 || one < ms) ms = one;
-      }
-      if (rc == MI355X_OK && (bestTile == -1 && t == -1 ? true : ms < best)) {
+      const float ms = timeTile(l, t);
+      if (ms < 0.0f) continue;
+      if (rc == MI355X_OK && (t == -1 || ms < best)) {
         best = ms;
         bestTile = t;
       }
+    }
+    // A dozen candidates a few per cent apart: the fastest of one pass is often
+    // a lucky measurement (several tile numbers run the very kernel the shape
+    // rule picks). The winner has to beat the library's own choice again, by
+    // two per cent, in a second pass, or that choice stays.
+    if (bestTile != -1 && rc == MI355X_OK) {
+      const float again = timeTile(l, bestTile), base = timeTile(l, -1);
+      if (!(again >= 0.0f && base >= 0.0f && again < 0.98f * base)) bestTile = -1;
     }
     l.tile = bestTile;
   }
