@@ -11,6 +11,7 @@
 // input offset and the dense contraction of gemm_i8.h applies unchanged.
 #include "gemm_i8.h"
 #include "conv_halo.h"
+#include "conv_halo_wide.h"
 #include "gemm_stream.h"
 
 namespace mi355x {
@@ -181,6 +182,19 @@ static int conv_common(int8_t *out, const int8_t *in, const int8_t *filter,
     if (rows != 0 && lds <= lds_limit()) {
       ep.fast = g_requant_hint & 3;
       return conv_halo_launch(in, filter, g, ep, lds, rows, as_stream(stream));
+    }
+  }
+  // The same over 128, 256 or 512 input channels: the input patch resident in
+  // LDS, the filter slice streamed through it tap by tap (conv_halo_wide.h).
+  if ((g_tile_override < 0 || g_tile_override == 7) && !need_sa && !need_sb && al_a && al_b &&
+      al_out) {
+    HaloWide cv{};
+    size_t lds = 0;
+    const size_t lds_max = lds_limit();
+    const int waves = conv_halo_wide_plan(g, lds_max, cv, lds);
+    if (waves != 0) {
+      ep.fast = g_requant_hint & 3;
+      return conv_halo_wide_launch(in, filter, g, ep, cv, lds, lds_max, waves, as_stream(stream));
     }
   }
   // Pointwise convolutions (any stride) over 64, 128 or 256 channels, and
