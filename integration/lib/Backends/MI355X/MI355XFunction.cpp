@@ -433,6 +433,9 @@ Error MI355XFunction::build(const IRFunction &IR, const Module &mod,
   if (off("fuseInsert")) ho.fuseInsert = false;
   if (off("fuseDequantizeSigmoid")) ho.fuseDequantizeSigmoid = false;
   if (off("precomputeWeightRowSums")) ho.precomputeWeightRowSums = false;
+  if (off("deriveBagOffsets")) ho.deriveBagOffsets = false;
+  if (off("reuseActivations")) ho.reuseActivations = false;
+  if (off("fuseQuantizeStem")) ho.fuseQuantizeStem = false;
 
   hm::MI355XBackend hostBackend;
   auto compiled = hostBackend.compile(*fn, ho);
