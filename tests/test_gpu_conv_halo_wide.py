@@ -114,3 +114,27 @@ def test_wide_halo_conv_full_batch(IC, H):
     np.testing.assert_array_equal(got[:2], want)
     for i in range(2, 64):
         np.testing.assert_array_equal(got[i], want[i % 2])
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_wide_halo_conv_random_geometry(seed):
+    """Seeded shapes around the tiling's corners: rows per tile, images per
+    tile, the last tile of an image or of the batch, every padding."""
+    rng = np.random.default_rng(500 + seed)
+    IC = int(rng.choice([128, 256, 512]))
+    H, W = int(rng.integers(3, 31)), int(rng.integers(3, 41))
+    if IC == 512:
+        H, W = min(H, 16), min(W, 16)
+    N = int(rng.integers(1, 7))
+    pads = tuple(int(v) for v in rng.integers(0, 3, 4))
+    kw = dict(IC=IC, N=N, H=H, W=W, OC=64 * int(rng.integers(1, 3)), pads=pads,
+              in_offset=int(rng.integers(-128, 128)), out_offset=int(rng.integers(-128, 128)),
+              act=[go.ACT_NONE, go.ACT_RELU, go.ACT_CLIP][seed % 3])
+    c = cases.cwq_conv_case(600 + seed, **kw)
+    g = c["geom"]
+    if g.OH <= 0 or g.OW <= 0:
+        pytest.skip("empty output")
+    say("wide halo conv", kw, "output", g.OH, "x", g.OW)
+    want = go.cwq_conv2d_i8(*cases.cwq_conv_args(c))
+    with forced_tile(7):
+        np.testing.assert_array_equal(capi.cwq_conv2d_i8(*cases.cwq_conv_args(c)), want)
