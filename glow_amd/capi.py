@@ -28,7 +28,7 @@ EXPORTS = [
     "mi355x_relu_i8", "mi355x_convert_f16_to_f32", "mi355x_insert_rows",
     "mi355x_batch_transpose_i8", "mi355x_space_to_depth2_i8", "mi355x_quantize_space_to_depth2_i8", "mi355x_gather", "mi355x_gather_rows", "mi355x_rescale_rows_i8",
     "mi355x_dequantize_sigmoid", "mi355x_batch_matmul_i8", "mi355x_sigmoid_f32",
-    "mi355x_max_pool_i8", "mi355x_avg_pool_i8", "mi355x_softmax_f32", "mi355x_stream_create",
+    "mi355x_max_pool_i8", "mi355x_avg_pool_i8", "mi355x_softmax_f32", "mi355x_dequantize_softmax", "mi355x_stream_create",
     "mi355x_stream_destroy", "mi355x_stream_sync", "mi355x_device_sync",
     "mi355x_event_create", "mi355x_event_destroy", "mi355x_event_record", "mi355x_stream_wait_event",
     "mi355x_event_sync", "mi355x_event_elapsed_ms", "mi355x_arena_create",
@@ -1085,6 +1085,15 @@ def softmax_f32(x):
     out = DeviceBuffer.empty(x.shape, np.float32)
     check(lib().mi355x_softmax_f32(_vp(out), _vp(dx), _sz(x.shape[0]), _sz(x.shape[1]),
                                    _vp(None)))
+    return out.numpy()
+
+
+def dequantize_softmax(q, scale, offset):
+    q = np.ascontiguousarray(q, np.int8)
+    dq = to_device(q)
+    out = DeviceBuffer.empty(q.shape, np.float32)
+    check(lib().mi355x_dequantize_softmax(_vp(out), _vp(dq), _sz(q.shape[0]), _sz(q.shape[1]),
+                                          C.c_float(scale), _i32(offset), _vp(None)))
     return out.numpy()
 
 

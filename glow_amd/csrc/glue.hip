@@ -300,17 +300,26 @@ __device__ __forceinline__ float block_reduce(float v, float *s, bool is_max) {
 // One block per row: max, exp and sum, divide (libjit_softmax_f). The sum is
 // formed in a different order than the CPU's sequential loop, so results agree
 // to fp32 rounding, not bit for bit.
+// DEQ: the row is int8 and dequantized on the way in (scale * (q - offset),
+// the very float Dequantize writes), which saves the float tensor in between.
+template <bool DEQ>
 __global__ __launch_bounds__(kGlueThreads) void softmax_f32_kernel(
-    float *__restrict__ out, const float *__restrict__ in, int cols) {
+    float *__restrict__ out, const void *__restrict__ in, int cols, float scale, int32_t offset) {
   __shared__ float s[kGlueThreads / 64];
-  const float *x = in + (long long)blockIdx.x * cols;
-  float *y = out + (long long)blockIdx.x * cols;
+  const long long row0 = (long long)blockIdx.x * cols;
+  auto x = [&](int i) -> float {
+    if constexpr (DEQ)
+      return __fmul_rn(scale, (float)((int32_t)reinterpret_cast<const int8_t *>(in)[row0 + i] - offset));
+    else
+      return reinterpret_cast<const float *>(in)[row0 + i];
+  };
+  float *y = out + row0;
   float m = -INFINITY;
-  for (int i = threadIdx.x; i < cols; i += kGlueThreads) m = fmaxf(m, x[i]);
+  for (int i = threadIdx.x; i < cols; i += kGlueThreads) m = fmaxf(m, x(i));
   m = block_reduce(m, s, true);
   float sum = 0.0f;
   for (int i = threadIdx.x; i < cols; i += kGlueThreads) {
-    const float e = expf(__fsub_rn(x[i], m));
+    const float e = expf(__fsub_rn(x(i), m));
     y[i] = e;
     sum = __fadd_rn(sum, e);
   }
@@ -912,9 +921,19 @@ int mi355x_softmax_f32(float *out, const float *in, size_t rows, size_t cols, vo
   if (rows == 0 || cols == 0) return MI355X_OK;
   MI355X_REQUIRE(out && in, "NULL tensor");
   MI355X_REQUIRE(rows < 0x7fffffffu && cols < 0x7fffffffu, "tensor too large");
-  hipLaunchKernelGGL(softmax_f32_kernel, dim3((unsigned)rows), dim3(kGlueThreads), 0,
-                     as_stream(stream), out, in, (int)cols);
+  hipLaunchKernelGGL(softmax_f32_kernel<false>, dim3((unsigned)rows), dim3(kGlueThreads), 0,
+                     as_stream(stream), out, (const void *)in, (int)cols, 1.0f, 0);
   return check_launch("softmax_f32");
+}
+
+int mi355x_dequantize_softmax(float *out, const int8_t *in, size_t rows, size_t cols, float scale,
+                              int32_t offset, void *stream) {
+  if (rows == 0 || cols == 0) return MI355X_OK;
+  MI355X_REQUIRE(out && in, "NULL tensor");
+  MI355X_REQUIRE(rows < 0x7fffffffu && cols < 0x7fffffffu, "tensor too large");
+  hipLaunchKernelGGL(softmax_f32_kernel<true>, dim3((unsigned)rows), dim3(kGlueThreads), 0,
+                     as_stream(stream), out, (const void *)in, (int)cols, scale, offset);
+  return check_launch("dequantize_softmax");
 }
 
 } // extern "C"

@@ -216,8 +216,20 @@ public:
             M_.value(insts_[at + 1].operands[0]).type.kind == ElemKind::FloatTy &&
             M_.value(insts_[at + 1].operands[0]).type.size() == M_.value(I.operands[0]).type.size())
           sig = &insts_[at + 1];
-        MI355X_RETURN_IF_ERR(dequantize(I, out, sig));
-        if (sig) at++;
+        // ... or a SoftMax over its rows
+        const Instruction *smax = nullptr;
+        if (!sig && opts_.fuseDequantizeSigmoid && at + 1 < insts_.size() &&
+            insts_[at + 1].kind == Kind::SoftMax && insts_[at + 1].operands[1] == I.operands[0] &&
+            M_.value(I.operands[0]).category == SymbolCategory::Activation &&
+            readers(I.operands[0]) == 1 && writers(I.operands[0]) == 1 &&
+            M_.value(I.operands[1]).type.kind == ElemKind::Int8QTy &&
+            M_.value(I.operands[0]).type.dims.size() == 2 &&
+            M_.value(insts_[at + 1].operands[0]).type.kind == ElemKind::FloatTy &&
+            M_.value(insts_[at + 1].operands[0]).type.dims == M_.value(I.operands[0]).type.dims &&
+            M_.value(I.operands[1]).type.size() == M_.value(I.operands[0]).type.size())
+          smax = &insts_[at + 1];
+        MI355X_RETURN_IF_ERR(dequantize(I, out, sig, smax));
+        if (sig || smax) at++;
         break;
       }
       case Kind::RescaleQuantized: {
@@ -1068,7 +1080,8 @@ private:
     return Error::success();
   }
 
-  Error dequantize(const Instruction &I, MI355XFunction &out, const Instruction *sig = nullptr) {
+  Error dequantize(const Instruction &I, MI355XFunction &out, const Instruction *sig = nullptr,
+                   const Instruction *smax = nullptr) {
     Operand d = op(I, 0), s = op(I, 1);
     CHECK_OP(d.ty().kind == ElemKind::FloatTy &&
                  (s.ty().kind == ElemKind::Int8QTy || (wideKind(s.ty().kind) && !sig)),
@@ -1097,6 +1110,17 @@ private:
                               [=](const DeviceBindings &b) {
                                 return mi355x_dequantize_sigmoid((float *)y.ptr(b), (const int8_t *)s.ptr(b),
                                                                  n, sc, off, b.stream);
+                              }});
+      return Error::success();
+    }
+    if (smax) {
+      Operand y = op(*smax, 0);
+      const size_t rows = (size_t)d.ty().dims[0], cols = (size_t)d.ty().dims[1];
+      out.launches.push_back({"mi355x_dequantize_softmax", I.name + "+" + smax->name,
+                              strFormat(" rows=%zu cols=%zu scale=%.9g offset=%d", rows, cols, (double)sc, off),
+                              [=](const DeviceBindings &b) {
+                                return mi355x_dequantize_softmax((float *)y.ptr(b), (const int8_t *)s.ptr(b),
+                                                                 rows, cols, sc, off, b.stream);
                               }});
       return Error::success();
     }

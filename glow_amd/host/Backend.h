@@ -184,7 +184,7 @@ struct BackendOptions {
   bool fuseFcRelu = true;              // RowwiseQuantizedFullyConnected + Relu of its result in one kernel
   bool padTableRows = true;            // constant lookup tables with 33..63-byte rows re-laid 64 bytes apart at load
   bool fuseInsert = true;              // Gather / RescaleQuantized write straight into the tensor their result is inserted into
-  bool fuseDequantizeSigmoid = true;   // Dequantize + Sigmoid of its result in one kernel
+  bool fuseDequantizeSigmoid = true;   // Dequantize + the Sigmoid or SoftMax of its result in one kernel
   bool deriveBagOffsets = true;        // lookups whose lengths are an input: bag positions summed on the host at upload
   bool fuseQuantizeStem = true;        // Quantize read only by a space-to-depth convolution: quantized while re-laid
   bool reuseActivations = true;        // activations whose lives do not meet share memory (first fit over the launch order)

@@ -254,6 +254,11 @@ int mi355x_rescale_rows_i8(int8_t *dst, const int8_t *src, size_t rows, size_t c
  * the sigmoid agrees with the CPU to fp32 rounding of expf (1e-5 relative). */
 int mi355x_dequantize_sigmoid(float *dst, const int8_t *src, size_t n, float scale,
                               int32_t offset, void *stream);
+/* Dequantize (libjit.cpp:3016-3019) followed by SoftMax over the rows of its
+ * result (libjit_softmax_f, libjit.cpp:3058-3082) in one pass: the dequantized
+ * values are the same fp32 numbers, the rest is mi355x_softmax_f32. */
+int mi355x_dequantize_softmax(float *out, const int8_t *in, size_t rows, size_t cols, float scale,
+                              int32_t offset, void *stream);
 
 /* ---- int8 glue operators ------------------------------------------------------ */
 

@@ -124,7 +124,7 @@ enum {
                                           at load time to rows 64 bytes apart */
   MI355X_HOST_OPT_FUSE_INSERT = 256, /* Gather / RescaleQuantized whose result is only inserted into a
                                         wider tensor write there directly */
-  MI355X_HOST_OPT_FUSE_DEQUANTIZE_SIGMOID = 512, /* Dequantize + Sigmoid of its result in one kernel */
+  MI355X_HOST_OPT_FUSE_DEQUANTIZE_SIGMOID = 512, /* Dequantize + the Sigmoid or SoftMax of its result in one kernel */
   MI355X_HOST_OPT_DERIVE_BAG_OFFSETS = 1024, /* lookups whose lengths are an input placeholder read
                                               * their bags as positions that the device manager sums
                                               * on the host when it uploads the lengths */

@@ -102,6 +102,19 @@ def test_softmax(rows, cols):
     np.testing.assert_allclose(got.sum(axis=1), 1.0, rtol=1e-5)
 
 
+@pytest.mark.parametrize("rows,cols", [(1, 1), (3, 7), (64, 1000), (5, 5000)])
+def test_dequantize_and_softmax_in_one_pass(rows, cols):
+    rng = np.random.default_rng(rows * 31 + cols)
+    q = rng.integers(-128, 128, (rows, cols)).astype(np.int8)
+    scale, offset = np.float32(0.0731), -17
+    want = go.softmax_f32(go.dequantize_i8(q, scale, offset))
+    got = capi.dequantize_softmax(q, scale, offset)
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-30)
+    # the two-launch path gives the same numbers
+    np.testing.assert_allclose(got, capi.softmax_f32(capi.dequantize_i8(q, scale, offset)),
+                               rtol=1e-6, atol=1e-30)
+
+
 def test_argument_errors():
     with pytest.raises(capi.MI355XError):
         capi.add_i8(np.zeros(4, np.int8), np.zeros(4, np.int8), 0, 0, 0, (0, 40, 1), (0, 0, 1))

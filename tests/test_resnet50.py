@@ -44,7 +44,12 @@ def test_small_network_compiles_and_fuses():
     # the 7x7 stride-2 stem over 3 channels runs as a 4x4 stride-1 convolution
     # over a space-to-depth image of 16 channels, which is quantized from the
     # float input while it is re-laid
-    assert kernels[-1] == "mi355x_softmax_f32"
+    # the int8 logits become probabilities in one launch
+    assert kernels[-1] == "mi355x_dequantize_softmax" and "mi355x_dequantize_i8" not in kernels
+    m4, f4 = netlib.to_module(net)
+    m4.compile(f4, fuse_dequantize_sigmoid=False)
+    k4 = [r["kernel"] for r in H.parse_listing(m4.describe(f4)) if r["phase"] == "launch"]
+    assert k4[-2:] == ["mi355x_dequantize_i8", "mi355x_softmax_f32"] and k4[:-2] == kernels[:-1]
     assert kernels[0] == "mi355x_quantize_space_to_depth2_i8" and "mi355x_quantize_i8" not in kernels
     m3, f3 = netlib.to_module(net)
     m3.compile(f3, fuse_quantize_stem=False)
