@@ -368,6 +368,38 @@ __device__ __forceinline__ int4 fused_out_words(int4 v, const int8_t *res16, con
   return v;
 }
 
+// The same on a residual that is already in registers (loaded ahead of the
+// arithmetic that produced v, so that its latency is not waited for here).
+__device__ __forceinline__ int4 fused_out_words_loaded(int4 v, int4 q, bool has_res,
+                                                       const Epilogue &ep,
+                                                       const FusedAddConsts &fc, bool fast) {
+  if (has_res && fast) {
+    v.x = (int)fused_word_fast<true>((uint32_t)v.x, (uint32_t)q.x, ep.add, fc);
+    __builtin_amdgcn_sched_barrier(0);
+    v.y = (int)fused_word_fast<true>((uint32_t)v.y, (uint32_t)q.y, ep.add, fc);
+    __builtin_amdgcn_sched_barrier(0);
+    v.z = (int)fused_word_fast<true>((uint32_t)v.z, (uint32_t)q.z, ep.add, fc);
+    __builtin_amdgcn_sched_barrier(0);
+    v.w = (int)fused_word_fast<true>((uint32_t)v.w, (uint32_t)q.w, ep.add, fc);
+  } else if (!has_res && ep.add.relu && fast) {
+    v.x = (int)fused_word_fast<false>((uint32_t)v.x, 0u, ep.add, fc);
+    v.y = (int)fused_word_fast<false>((uint32_t)v.y, 0u, ep.add, fc);
+    v.z = (int)fused_word_fast<false>((uint32_t)v.z, 0u, ep.add, fc);
+    v.w = (int)fused_word_fast<false>((uint32_t)v.w, 0u, ep.add, fc);
+  } else if (has_res) {
+    v.x = (int)fused_add_word((uint32_t)v.x, (uint32_t)q.x, ep.add);
+    v.y = (int)fused_add_word((uint32_t)v.y, (uint32_t)q.y, ep.add);
+    v.z = (int)fused_add_word((uint32_t)v.z, (uint32_t)q.z, ep.add);
+    v.w = (int)fused_add_word((uint32_t)v.w, (uint32_t)q.w, ep.add);
+  } else if (ep.add.relu) {
+    v.x = (int)fused_relu_word((uint32_t)v.x, ep.add);
+    v.y = (int)fused_relu_word((uint32_t)v.y, ep.add);
+    v.z = (int)fused_relu_word((uint32_t)v.z, ep.add);
+    v.w = (int)fused_relu_word((uint32_t)v.w, ep.add);
+  }
+  return v;
+}
+
 // Copy-out of a staged int8 output tile (rows OUT_STRIDE = BN + 16 bytes apart
 // in LDS), with the fused residual add / Relu applied on the way: 16-byte row
 // segments where the output allows it. WAVE_ROWS: a wave copies out rows
@@ -396,6 +428,9 @@ __device__ __forceinline__ void epilogue_copy_out(const int8_t *s_out, const Epi
     // every scale small and no pre-shift in the stages that run
     const bool fast = fused_out_is_fast(ep);
     const FusedAddConsts fc = fused_add_consts(ep.add);
+    // (the residual is read where it is used, a piece at a time: asking for
+    // four pieces ahead costs the tiled kernels twenty registers and a wave per
+    // SIMD)
     for (int c = first; c < row_n * segs; c += STEP) {
       const int r = row_lo + c / segs, s = c % segs;
       int4 v = *reinterpret_cast<const int4 *>(s_out + r * OUT_STRIDE + s * 16);

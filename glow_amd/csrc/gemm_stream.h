@@ -15,9 +15,10 @@
 //     of gemm_i8.h); groups of up to 128 columns go through a wave-private
 //     transpose in LDS so that they are written as whole 128-byte lines, with
 //     the fused residual add read the same way;
-//   * latency is hidden by occupancy (four waves per SIMD) instead of by a
-//     pipeline: while one wave waits for its rows, the others multiply and
-//     requantise.
+//   * a wave asks for its next tile's rows before it works on the current one
+//     and for a column group's residual bytes before that group's multiplies,
+//     so that neither is waited for; three workgroups per CU (the LDS allows no
+//     more with 256 columns of weights) cover what is left.
 //
 // Results are bit for bit those of the tiled kernels (same integer sums, same
 // requantisation).
@@ -61,12 +62,112 @@ constexpr int kStreamGroup = 128;
 constexpr int kStreamStageStride = kStreamGroup + 16;
 constexpr int kStreamStageBytes = 32 * kStreamStageStride;   // per wave
 
-// The results leave through a wave-private transpose in LDS
-// (wave_rows_copy_out): groups of up to 128 columns are staged, then read back
-// with eight lanes per row, so that a store instruction writes whole 128-byte
-// lines and the residual is read the same way.
+// The results leave through a wave-private transpose in LDS: groups of up to
+// 128 columns are staged, then read back with group / 16 lanes per row, so that
+// a store instruction writes whole lines and the residual is read the same way.
+// NP: passes of the copy-out (four for groups of 96 and 128 columns, two for
+// narrower ones); RES: a residual is added. Both are template parameters so
+// that every load has exactly one place that uses it, on every path: the
+// compiler then waits for a load where it is used and nowhere else.
+// A lane's share of the rows of tile t: KS pieces of 16 bytes in the
+// matrix-core layout (rows past the end re-read the last row; their results are
+// not stored).
+template <int KS>
+__device__ __forceinline__ void stream_load_rows(const StreamRows &A, v4i (&dst)[KS], int t, int M,
+                                                 int lane) {
+  const int8_t *ar = A.row(min(t * 32 + (lane & 31), M - 1)) + (lane >> 5) * 16;
+  if (A.seg_chunks >= KS) {
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) dst[ks] = *reinterpret_cast<const v4i *>(ar + ks * 32);
+  } else {
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) dst[ks] = *reinterpret_cast<const v4i *>(ar + A.chunk(ks));
+  }
+}
+
+// af: the rows of the wave's first tile, asked for by the caller.
+template <int KS, int NP, bool RES, int MODE, bool LEAKY>
+__device__ __forceinline__ void stream_tiles(const StreamRows &A, v4i (&af)[KS], const int8_t *s_w,
+                                             const int32_t *s_par, int8_t *s_stage,
+                                             const Epilogue &ep, int M, int N, int n0,
+                                             int bn, int tiles32, int first, int step, int lane) {
+  constexpr int WSTRIDE = KS * 32 + 16;
+  const int l32 = lane & 31, lhi = lane >> 5;
+  int32_t lo, hi;
+  activation_clamp(ep, lo, hi);
+  const bool fast = fused_out_is_fast(ep);
+  const FusedAddConsts fc = fused_add_consts(ep.add);
+  const int8_t *w_lane = s_w + l32 * WSTRIDE + lhi * 16;
+  // column groups of this slice: 128 columns, or all of a narrower slice
+  const int group = min(bn, kStreamGroup);         // bytes per row and group
+  // copy-out: lpr lanes per row, rpp rows per pass
+  const int lpr = group / 16, rpp = 64 / lpr;
+  const int rb_row = lane / lpr, rb_seg = lane - rb_row * lpr;
+  v4i an[KS];
+  // (waited for here, once: inside the loop af is known to have arrived, and no
+  // multiply waits behind the stores of the tile before)
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++) asm volatile("" : "+v"(af[ks]));
+  for (int t = first; t < tiles32; t += step) {
+    const int m0 = t * 32;
+    const int last_row = min(31, M - 1 - m0);      // of this tile
+    // the next tile's rows are on their way while this one is worked on
+    stream_load_rows<KS>(A, an, min(t + step, tiles32 - 1), M, lane);
+    for (int c0 = 0; c0 < bn; c0 += group) {
+      // the group's residual bytes, in the layout of the copy-out, asked for
+      // before the arithmetic they are added to. A lane whose row is past the
+      // tile or the end works on the tile's last row instead and stores the
+      // same bytes to the same place as that row's own lane: with every load
+      // and store issued by every lane the waits can be counted exactly.
+      int4 rq[NP];
+      if constexpr (RES) {
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+          const int m = m0 + min(p * rpp + rb_row, last_row);
+          rq[p] = *reinterpret_cast<const int4 *>(ep.add.res + (long long)m * ep.ldc + n0 + c0 +
+                                                  rb_seg * 16);
+        }
+      }
+      for (int j = c0 / 32; j < (c0 + group) / 32; j++) {
+        v16i acc;
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[r] = 0;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+          const v4i b = *reinterpret_cast<const v4i *>(w_lane + j * 32 * WSTRIDE + ks * 32);
+          // weights first: the result's rows are columns of the output
+          acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(b, af[ks], acc, 0, 0, 0);
+        }
+        const int cl = j * 32 + 16 * lhi;
+        const int4 v = requant_pack16<MODE, LEAKY, kStreamMaxBN>(acc, s_par + cl, ep, lo, hi);
+        *reinterpret_cast<int4 *>(s_stage + l32 * kStreamStageStride + (cl - c0)) = v;
+      }
+      wave_fence();
+#pragma unroll
+      for (int p = 0; p < NP; p++) {
+        const int row = min(p * rpp + rb_row, last_row), m = m0 + row;
+        int4 v = *reinterpret_cast<const int4 *>(s_stage + row * kStreamStageStride + rb_seg * 16);
+        if constexpr (RES)
+          v = fused_out_words_loaded(v, rq[p], true, ep, fc, fast);
+        else
+          v = fused_out_words_loaded(v, v, false, ep, fc, fast);
+        *reinterpret_cast<int4 *>(ep.out + (long long)m * ep.ldc + n0 + c0 + rb_seg * 16) = v;
+      }
+      wave_fence();
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) af[ks] = an[ks];
+  }
+}
+
+// K = 256: the plain form of the loop. A lane's rows alone are 32 registers
+// there; with the next tile's rows and a group's residual bytes asked for ahead
+// the loop needs more registers than three waves per SIMD leave (spills, whose
+// reloads wait behind the stores), and at two waves per SIMD it is slower than
+// this: rows asked for at the top of the tile, the residual where it is added,
+// four waves per SIMD if the LDS allows.
 template <int KS, int MODE, bool LEAKY>
-__device__ __forceinline__ void stream_tiles(const StreamRows &A, const int8_t *s_w,
+__device__ __forceinline__ void stream_tiles_simple(const StreamRows &A, const int8_t *s_w,
                                              const int32_t *s_par, int8_t *s_stage,
                                              const Epilogue &ep, int M, int N, int n0, int bn,
                                              int tiles32, int first, int step, int lane) {
@@ -113,9 +214,31 @@ __device__ __forceinline__ void stream_tiles(const StreamRows &A, const int8_t *
   }
 }
 
+// The requantisation variant is a template parameter as well (each variant
+// keeps its own constants in registers; all four in one loop spill).
+template <int KS, int NP, bool RES>
+__device__ __forceinline__ void stream_tiles_mode(const StreamRows &A, v4i (&af)[KS],
+                                                  const int8_t *s_w, const int32_t *s_par,
+                                                  int8_t *s_stage, const Epilogue &ep, int mode,
+                                                  int M, int N, int n0, int bn, int tiles32,
+                                                  int first, int step, int lane) {
+  if (ep.act == 5)
+    stream_tiles<KS, NP, RES, 0, true>(A, af, s_w, s_par, s_stage, ep, M, N, n0, bn, tiles32, first,
+                                       step, lane);
+  else if (mode == 3)
+    stream_tiles<KS, NP, RES, 3, false>(A, af, s_w, s_par, s_stage, ep, M, N, n0, bn, tiles32,
+                                        first, step, lane);
+  else if (mode == 1)
+    stream_tiles<KS, NP, RES, 1, false>(A, af, s_w, s_par, s_stage, ep, M, N, n0, bn, tiles32,
+                                        first, step, lane);
+  else
+    stream_tiles<KS, NP, RES, 0, false>(A, af, s_w, s_par, s_stage, ep, M, N, n0, bn, tiles32,
+                                        first, step, lane);
+}
+
 // KS: K / 32 (2, 4 or 8). blockIdx.y: column slice of bn columns.
 template <int KS>
-__global__ __launch_bounds__(256, 4) void gemm_i8_stream_kernel(StreamRows A, const int8_t *W,
+__global__ __launch_bounds__(256, KS == 8 ? 4 : 3) void gemm_i8_stream_kernel(StreamRows A, const int8_t *W,
                                                                 Epilogue ep, int M, int N, int bn,
                                                                 int tiles32) {
   constexpr int K = KS * 32, WSTRIDE = K + 16;
@@ -130,6 +253,12 @@ __global__ __launch_bounds__(256, 4) void gemm_i8_stream_kernel(StreamRows A, co
   const int n0 = blockIdx.y * bn;
   const int cols = min(bn, N - n0);          // a multiple of 32
   const int mode = requant_mode(ep);
+
+  // the wave's first rows are asked for before anything else, so that they
+  // arrive while the slice is being put in LDS
+  const int first = blockIdx.x * 4 + wave, step = gridDim.x * 4;
+  v4i af[KS];
+  if constexpr (KS < 8) stream_load_rows<KS>(A, af, min(first, tiles32 - 1), M, lane);
 
   // the slice's constants and weights -> LDS, once
   if (tid < cols) {
@@ -161,19 +290,38 @@ __global__ __launch_bounds__(256, 4) void gemm_i8_stream_kernel(StreamRows A, co
   __syncthreads();
 
   // from here on every wave is on its own
-  const int first = blockIdx.x * 4 + wave, step = gridDim.x * 4;
-  if (ep.act == 5)
-    stream_tiles<KS, 0, true>(A, s_w, s_par, s_stage + wave * kStreamStageBytes, ep, M, N, n0,
-                              cols, tiles32, first, step, lane);
-  else if (mode == 3)
-    stream_tiles<KS, 3, false>(A, s_w, s_par, s_stage + wave * kStreamStageBytes, ep, M, N, n0,
-                              cols, tiles32, first, step, lane);
-  else if (mode == 1)
-    stream_tiles<KS, 1, false>(A, s_w, s_par, s_stage + wave * kStreamStageBytes, ep, M, N, n0,
-                              cols, tiles32, first, step, lane);
-  else
-    stream_tiles<KS, 0, false>(A, s_w, s_par, s_stage + wave * kStreamStageBytes, ep, M, N, n0,
-                              cols, tiles32, first, step, lane);
+  int8_t *stage = s_stage + wave * kStreamStageBytes;
+  if constexpr (KS == 8) {
+    if (ep.act == 5)
+      stream_tiles_simple<KS, 0, true>(A, s_w, s_par, stage, ep, M, N, n0, cols, tiles32, first,
+                                       step, lane);
+    else if (mode == 3)
+      stream_tiles_simple<KS, 3, false>(A, s_w, s_par, stage, ep, M, N, n0, cols, tiles32, first,
+                                        step, lane);
+    else if (mode == 1)
+      stream_tiles_simple<KS, 1, false>(A, s_w, s_par, stage, ep, M, N, n0, cols, tiles32, first,
+                                        step, lane);
+    else
+      stream_tiles_simple<KS, 0, false>(A, s_w, s_par, stage, ep, M, N, n0, cols, tiles32, first,
+                                        step, lane);
+  } else {
+  const bool narrow = cols <= 64;            // two passes of the copy-out, not four
+  if (ep.add.res) {
+    if (narrow)
+      stream_tiles_mode<KS, 2, true>(A, af, s_w, s_par, stage, ep, mode, M, N, n0, cols, tiles32, first,
+                                step, lane);
+    else
+      stream_tiles_mode<KS, 4, true>(A, af, s_w, s_par, stage, ep, mode, M, N, n0, cols, tiles32, first,
+                                step, lane);
+  } else {
+    if (narrow)
+      stream_tiles_mode<KS, 2, false>(A, af, s_w, s_par, stage, ep, mode, M, N, n0, cols, tiles32, first,
+                                 step, lane);
+    else
+      stream_tiles_mode<KS, 4, false>(A, af, s_w, s_par, stage, ep, mode, M, N, n0, cols, tiles32, first,
+                                 step, lane);
+  }
+  }
 }
 
 // Whether the streaming kernel can run this product at all: K of 64, 128 or
@@ -212,7 +360,7 @@ static int gemm_stream_launch(const StreamRows &A, const int8_t *W, const Epilog
     if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
       cus = v;
   }
-  const int per_cu = (int)std::min<size_t>(4, (160 * 1024) / lds);
+  const int per_cu = (int)std::min<size_t>(K == 256 ? 4 : 3, (160 * 1024) / lds);
   long long gx = std::max(1LL, (long long)cus * per_cu / slices);
   gx = std::min<long long>(gx, (tiles32 + 3) / 4);
   MI355X_REQUIRE(slices < 65536, "problem too large");
