@@ -4,7 +4,7 @@
 // tiled kernels of gemm_i8.h spend their time in load latency, barriers and
 // output staging.
 //
-//   * the weights of a workgroup's column slice (at most 256 columns, 37 KB)
+//   * the weights of a workgroup's column slice (128 columns, at most 35 KB)
 //     and the columns' requantisation constants are put in LDS once; from then
 //     on the workgroup's waves never meet again;
 //   * a wave walks over tiles of 32 rows: a lane loads its row's K bytes
@@ -17,8 +17,9 @@
 //     the fused residual add read the same way;
 //   * a wave asks for its next tile's rows before it works on the current one
 //     and for a column group's residual bytes before that group's multiplies,
-//     so that neither is waited for; three workgroups per CU (the LDS allows no
-//     more with 256 columns of weights) cover what is left.
+//     so that neither is waited for (K = 64 and 128; at K = 256 the rows alone
+//     are 32 registers a lane and the loop stays plain); three workgroups per
+//     CU, the registers allow no more, cover what is left.
 //
 // Results are bit for bit those of the tiled kernels (same integer sums, same
 // requantisation).
@@ -347,9 +348,13 @@ static bool stream_applies(int M, int N) { return M >= 4096 && N <= 512; }
 
 static int gemm_stream_launch(const StreamRows &A, const int8_t *W, const Epilogue &ep, int M,
                               int N, int K, hipStream_t st) {
-  // columns per slice: 256 for K = 64, 128 beyond (the weights of a slice stay
-  // under 35 KB, beside 18 KB of staging tiles and the 5 KB constants table)
-  const int bn = K == 64 ? kStreamMaxBN : 128;
+  // 128 columns per slice: a slice's weights stay under 35 KB beside 18 KB of
+  // staging tiles and the 5 KB constants table, and a unit of work (32 rows of
+  // one slice) is small enough that the last round of tiles, which only some of
+  // the waves take part in, costs little (K = 64, 256 output columns, 200704
+  // rows: 37.7 us in slices of 128 against 38.6 us in one of 256, though the
+  // rows are then read twice)
+  const int bn = 128;
   const int slices = (N + bn - 1) / bn;
   const size_t lds = (size_t)kStreamParBytes + 4 * (size_t)kStreamStageBytes +
                      (size_t)std::min(bn, N) * (K + 16);
