@@ -180,3 +180,57 @@ def test_stream_conv_full_batch():
     np.testing.assert_array_equal(got[:2], want)
     for i in range(2, 64):
         np.testing.assert_array_equal(got[i], want[i % 2])
+
+
+@pytest.mark.parametrize("IC,OC,slow", [(64, 64, False), (128, 96, False), (64, 32, True),
+                                        (128, 256, True), (64, 128, False)])
+def test_stream_add_narrow_slices_and_general_scales(IC, OC, slow):
+    """Slices of 32, 64 and 96 columns (two and four passes of the copy-out,
+    lanes past the tile's rows) with the residual, and add parameters outside
+    the short form (a pre-shift, a scale beyond 23 bits)."""
+    c = cases.cwq_conv_case(75 + IC + OC, 3, 11, 13, IC, OC, kernel=(1, 1), pads=(0, 0, 0, 0),
+                            act=go.ACT_NONE, in_offset=-128, out_offset=-3)
+    conv = go.cwq_conv2d_i8(*cases.cwq_conv_args(c))
+    rng = np.random.default_rng(76)
+    res = rng.integers(-128, 128, conv.shape).astype(np.int8)
+    p = lambda r: go.quantize_scale_offset_32to8(float(np.float32(r)), 0)[:3]
+    cp, rp, dp = p(0.8), p(0.61), p(0.7)
+    if slow:
+        cp = (1, cp[1], cp[2] * 2)                 # the same ratio through a pre-shift
+        rp = (0, 24, int(round(0.61 * (1 << 24))))
+    want = go.relu_i8(go.add_i8(conv, res, 7, c["out_offset"], -9, cp, rp), 7, -128, dp)
+    add = capi.fused_add(7, -9, cp, rp, True, -128, dp)
+    say("stream add", IC, OC, "slow" if slow else "short form", cp, rp)
+    with forced_tile(8):
+        got = capi.cwq_conv2d_add_i8(*cases.cwq_conv_args(c), res, add)
+    np.testing.assert_array_equal(got, want)
+    with forced_tile(2):
+        np.testing.assert_array_equal(capi.cwq_conv2d_add_i8(*cases.cwq_conv_args(c), res, add), want)
+    assert len(np.unique(want)) > 20
+
+
+def test_stream_add_several_tiles_per_wave():
+    """More 32-row tiles than the launch has waves, with the residual: a wave's
+    next rows and residual bytes are asked for while it works on a tile. Two
+    images and two residual images on the oracle, the rest through batch
+    independence."""
+    n = 44                                           # 137984 rows = 4312 tiles
+    c = cases.cwq_conv_case(93, n, 56, 56, 64, 64, kernel=(1, 1), pads=(0, 0, 0, 0),
+                            act=go.ACT_NONE, in_offset=-128)
+    c["x"][2::2] = c["x"][0]
+    c["x"][3::2] = c["x"][1]
+    rng = np.random.default_rng(94)
+    res = np.empty((n, 56, 56, 64), np.int8)
+    res[0::2] = rng.integers(-128, 128, (56, 56, 64)).astype(np.int8)
+    res[1::2] = rng.integers(-128, 128, (56, 56, 64)).astype(np.int8)
+    p = lambda r: go.quantize_scale_offset_32to8(float(np.float32(r)), 0)[:3]
+    cp, rp, dp = p(0.9), p(0.5), p(0.66)
+    add = capi.fused_add(2, 5, cp, rp, True, -128, dp)
+    with forced_tile(8):
+        got = capi.cwq_conv2d_add_i8(*cases.cwq_conv_args(c), res, add)
+    c2 = dict(c, x=c["x"][:2], geom=go.conv_geom(2, 56, 56, 64, 64, (1, 1), (1, 1), (0, 0, 0, 0)))
+    conv = go.cwq_conv2d_i8(*cases.cwq_conv_args(c2))
+    want = go.relu_i8(go.add_i8(conv, res[:2], 2, c["out_offset"], 5, cp, rp), 2, -128, dp)
+    for i in range(n):
+        np.testing.assert_array_equal(got[i], want[i % 2])
+    assert len(np.unique(want)) > 20
