@@ -30,7 +30,8 @@
 
 namespace mi355x {
 
-constexpr int kStreamMaxBN = 256;   // columns per workgroup slice (and the table's stride)
+constexpr int kStreamMaxBN = 256;   // most columns a slice may have (the constants table's stride);
+                                    // launches use slices of 128
 constexpr int kStreamParBytes = kParArrays * kStreamMaxBN * 4;
 
 // Rows of A: dense (row m at in + m * ld), or the window a convolution without
