@@ -1323,7 +1323,7 @@ def frwq_sls_multi(tables, kind, indices, lengths, out_kind=SLS_OUT_F32, out_sca
 def slws_set_fused_math(on):
     """Process-wide: fused multiply-add arithmetic in the SparseLengths kernels
     (default) or the CPU loop's separately rounded operations."""
-    check(lib().mi355x_slws_set_fused_math(C.c_int(bool(on))))
+    check(lib().mi355x_slws_set_fused_math(C.c_int(int(on))))
 
 
 def rwq_slws(data, scales, offsets, weights, indices, lengths):

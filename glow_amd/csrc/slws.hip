@@ -40,6 +40,7 @@
 #include <hip/hip_fp16.h>
 
 #include <atomic>
+#include <utility>
 #include <mutex>
 #include <vector>
 
@@ -49,6 +50,10 @@ constexpr int kSlwsThreads = 256;
 constexpr int kBatch = 64;         // lookups fetched per round
 constexpr int kChunkBags = 4096;   // bags per pre-summed chunk
 constexpr int kMaxChunks = 32768;  // workspace entries (int64 each)
+#ifndef MI355X_SLWS_ROWS_WAVES
+#define MI355X_SLWS_ROWS_WAVES 8
+#endif
+constexpr int kRowsWaves = MI355X_SLWS_ROWS_WAVES; // bags per block of slws_rows_kernel
 
 struct SlwsArgs {
   void *dest;
@@ -222,7 +227,7 @@ __device__ __forceinline__ void bag_span_offsets(const SlwsArgs &a,
 // Lengths mode, first half: every wave leaves the sum of the clamped lengths
 // it has seen in front of the block in s_part[wave], and the block's own
 // clamped lengths go to s_own[]. Ends with a block barrier.
-template <int kGroups>
+template <int kGroups, int kThreads = kSlwsThreads>
 __device__ __forceinline__ void block_prefix(const SlwsArgs &a, int tid,
                                              long long first_bag,
                                              long long *s_part, int *s_own) {
@@ -232,7 +237,7 @@ __device__ __forceinline__ void block_prefix(const SlwsArgs &a, int tid,
   const int n_before = (int)(first_bag - lo); // < kChunkBags, multiple of 4
   uint32_t part = 0;
   if ((((uintptr_t)lbase) & 15) == 0) {
-    constexpr int kVecTrips = kChunkBags / 4 / kSlwsThreads;
+    constexpr int kVecTrips = (kChunkBags / 4 + kThreads - 1) / kThreads;
     const int4 *l4 = reinterpret_cast<const int4 *>(lbase);
     const int nvec = n_before / 4;
     if (nvec > 0) {
@@ -241,20 +246,20 @@ __device__ __forceinline__ void block_prefix(const SlwsArgs &a, int tid,
       int4 x[kVecTrips];
 #pragma unroll
       for (int u = 0; u < kVecTrips; u++)
-        x[u] = l4[min(tid + u * kSlwsThreads, nvec - 1)];
+        x[u] = l4[min(tid + u * kThreads, nvec - 1)];
 #pragma unroll
       for (int u = 0; u < kVecTrips; u++) {
         const uint32_t t = clamp_len(x[u].x) + clamp_len(x[u].y) +
                            clamp_len(x[u].z) + clamp_len(x[u].w);
-        part += (tid + u * kSlwsThreads < nvec) ? t : 0u;
+        part += (tid + u * kThreads < nvec) ? t : 0u;
       }
     }
   } else {
-    for (int i = tid; i < n_before; i += kSlwsThreads) part += clamp_len(lbase[i]);
+    for (int i = tid; i < n_before; i += kThreads) part += clamp_len(lbase[i]);
   }
   long long below = 0;
   if (a.chunk_sums) {
-    for (long long c = tid; c < chunk; c += kSlwsThreads) below += a.chunk_sums[c];
+    for (long long c = tid; c < chunk; c += kThreads) below += a.chunk_sums[c];
     below = (long long)wave_sum_u32((uint32_t)below) +
             ((long long)wave_sum_u32((uint32_t)(below >> 32)) << 32);
   }
@@ -615,48 +620,170 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_wave_kernel(SlwsArgs a) {
 }
 
 
-// ---- fused-arithmetic variant ----------------------------------------------------
+// ---- fused-arithmetic variants ---------------------------------------------------
 //
-// Same operator with the arithmetic regrouped for the vector ALU:
+// Same operator with fused multiply-adds, for rows of 32, 64, 128 or 256 data
+// bytes with fp32 accumulation.
+//
+// kMathElement (the default):
+//   v = fma(s_j, q_jk, o_j);  dest[k] = fma(w_j, v, dest[k])
+// the CPU loop's own expression w*(s*q+o) per element, with the two roundings
+// of its products left out: three vector instructions per element (convert,
+// fma, fma) instead of five. Each term differs from the CPU loop's by at most
+// half a unit in the last place of s*q and of w*v, and nothing is regrouped,
+// so a sum that cancels cancels here exactly where it does on the CPU.
+//
+// kMathRegrouped (on request only):
 //   dest[k] = sum_j (w_j*s_j) * q_jk  +  sum_j (w_j*o_j)
-// one fused multiply-add per element plus one add per lookup, instead of the
-// CPU loop's multiply, add, multiply, add. The result differs from the
-// sequential loop by rounding only (a few units in the last place of the
-// largest partial sum); callers that need the CPU loop's bits switch this
-// variant off with mi355x_slws_set_fused_math(0).
+// two instructions per element, but the two partial sums are large and of
+// opposite sign for tables with a negative offset, so the error is relative to
+// the magnitude a bag adds up and not to the result.
 //
 // One bag per wavefront; a lane reads 4 consecutive data bytes, so a row takes
 // LPR = data_bytes/4 lanes and one load instruction fetches 64/LPR rows. The
 // partial sums of the row groups are added across lanes at the end of the bag.
+constexpr int kMathStrict = 0, kMathElement = 1, kMathRegrouped = 2;
+
+// Cut points of the measurement entry point mi355x_frwq_slws_probe: the kernel
+// stops after the named stage and stores a value that depends on what it read.
+constexpr int kProbeOff = 0, kProbeSpan = 1, kProbeIndex = 2, kProbeScaleOffset = 3,
+              kProbeRows = 4;
+
+template <int MATH>
+__device__ __forceinline__ float fused_term(const float4 &f, float q, float acc) {
+  if constexpr (MATH == kMathElement) {
+    return __fmaf_rn(f.x, __fmaf_rn(f.y, q, f.z), acc);   // f = {w, s, o}
+  } else {
+    return __fmaf_rn(f.x, q, acc);                        // f = {w*s, w*o}
+  }
+}
+
 typedef uint32_t __attribute__((address_space(1))) global_u32;
 typedef int32_t __attribute__((address_space(1))) global_i32;
 typedef long long __attribute__((address_space(1))) global_i64;
 
-template <bool IS4, bool SO16, int LPR, bool OFF32>
-__global__ __launch_bounds__(kSlwsThreads) void slws_rows_kernel(SlwsArgs a) {
+// Sum of v over each row of 16 lanes, left in all 16 lanes of the row.
+__device__ __forceinline__ uint32_t row16_sum_u32(uint32_t v) {
+  int x = (int)v;
+  x += __builtin_amdgcn_update_dpp(0, x, 0xB1, 0xf, 0xf, true);  // quad_perm [1,0,3,2]
+  x += __builtin_amdgcn_update_dpp(0, x, 0x4E, 0xf, 0xf, true);  // quad_perm [2,3,0,1]
+  x += __builtin_amdgcn_update_dpp(0, x, 0x141, 0xf, 0xf, true); // row_half_mirror
+  x += __builtin_amdgcn_update_dpp(0, x, 0x140, 0xf, 0xf, true); // row_mirror
+  return (uint32_t)x;
+}
+
+typedef int __attribute__((ext_vector_type(4))) i32x4;
+typedef i32x4 __attribute__((address_space(1))) global_i32x4;
+
+// Span of the bag of wavefront `wave` of a block of WAVES wavefronts (WAVES
+// consecutive bags per block), wave-uniform. Lengths mode: the block sums the
+// clamped lengths in front of it (from the start of its chunk of kChunkBags
+// bags, one 16-byte load per thread and trip, trips beyond the block's position
+// skipped), one barrier, then lane g of every wave takes wave g's partial sum
+// and bag g's length and a 16-lane sum gives the wave its start. The whole of
+// it is about fifty vector instructions: with four waves on a SIMD every
+// instruction a wave issues costs the launch sixteen cycles.
+template <int WAVES>
+__device__ __forceinline__ void rows_bag_span(const SlwsArgs &a, int tid, int lane, int wave,
+                                              long long first_bag, uint32_t *s_part,
+                                              long long *s_below, int *s_own,
+                                              long long &start, int &len) {
+  static_assert(WAVES % 4 == 0 && WAVES <= 16, "4, 8, 12 or 16 waves per block");
+  constexpr int T = WAVES * 64;
+  const long long bag = first_bag + wave;
+  if (a.offsets) {
+    long long start_v;
+    int len_v;
+    bag_span_offsets(a, bag, start_v, len_v);
+    len = __builtin_amdgcn_readfirstlane(len_v);
+    start = ((long long)__builtin_amdgcn_readfirstlane((int)(start_v >> 32)) << 32) |
+            (unsigned int)__builtin_amdgcn_readfirstlane((int)start_v);
+  } else {
+    const long long chunk = first_bag / kChunkBags;
+    const long long lo = chunk * kChunkBags;
+    const int32_t *lbase = a.lengths + lo;
+    const int n_before = (int)(first_bag - lo);   // < kChunkBags, a multiple of WAVES
+    uint32_t part = 0;
+    if ((((uintptr_t)lbase) & 15) == 0) {
+      constexpr int kTrips = (kChunkBags / 4 + T - 1) / T;
+      const global_i32x4 *l4 = (const global_i32x4 *)lbase;
+      const int nvec = n_before >> 2;
+      i32x4 x[kTrips];
+#pragma unroll
+      for (int u = 0; u < kTrips; u++)
+        if (u * T < nvec) x[u] = l4[min(tid + u * T, nvec - 1)];
+#pragma unroll
+      for (int u = 0; u < kTrips; u++) {
+        if (u * T < nvec) {
+          const uint32_t t = clamp_len(x[u].x) + clamp_len(x[u].y) + clamp_len(x[u].z) +
+                             clamp_len(x[u].w);
+          part += (tid + u * T < nvec) ? t : 0u;
+        }
+      }
+    } else {
+      for (int i = tid; i < n_before; i += T) part += clamp_len(lbase[i]);
+    }
+    if (tid < WAVES) {
+      const long long b = first_bag + tid;
+      s_own[tid] = (int)min(clamp_len(b < a.segments ? a.lengths[b] : 0), 0x7fffffffu);
+    }
+    if (a.chunk_sums) {
+      long long below = 0;
+      for (long long c = tid; c < chunk; c += T) below += a.chunk_sums[c];
+      below = (long long)wave_sum_u32((uint32_t)below) +
+              ((long long)wave_sum_u32((uint32_t)(below >> 32)) << 32);
+      if (lane == 0) s_below[wave] = below;
+    }
+    part = wave_sum_u32(part);
+    if (lane == 0) s_part[wave] = part;
+    __syncthreads();
+    const uint32_t p = lane < WAVES ? s_part[lane] : 0u;
+    const int own = lane < WAVES ? s_own[lane] : 0;
+    const uint32_t before = row16_sum_u32(p + (lane < wave ? (uint32_t)own : 0u));
+    start = (long long)(uint32_t)__builtin_amdgcn_readlane((int)before, 0);
+    if (a.chunk_sums) {
+      long long below = 0;
+#pragma unroll
+      for (int g = 0; g < WAVES; g++) below += s_below[g];
+      start += ((long long)__builtin_amdgcn_readfirstlane((int)(below >> 32)) << 32) |
+               (unsigned int)__builtin_amdgcn_readfirstlane((int)below);
+    }
+    len = bag < a.segments ? __builtin_amdgcn_readlane(own, wave) : 0;
+  }
+  const long long room = a.num_indices - start;
+  len = room <= 0 ? 0 : (int)min((long long)len, room);
+}
+
+// One bag per wavefront, WAVES bags per block; whole rows of LPR * 4 data bytes.
+// The caller guarantees a 4-byte aligned table and row pitch.
+template <bool IS4, bool SO16, int LPR, bool OFF32, int MATH, int WAVES,
+          int PROBE = kProbeOff>
+__global__ __launch_bounds__(WAVES * 64) void slws_rows_kernel(SlwsArgs a) {
   select_table(a);
-  constexpr int kGroups = kSlwsThreads / 64;
   constexpr int RPI = 64 / LPR;           // rows per load instruction
   constexpr int kCols = IS4 ? 8 : 4;      // output columns per lane
   constexpr int kLoads = kBatch / RPI;    // load instructions of a full batch
   constexpr int kChunk = kLoads < 4 ? kLoads : 4; // loads under one uniform branch
-  __shared__ long long s_part[kGroups];
-  __shared__ __attribute__((aligned(16))) int s_own[kGroups];
-  // per wave, per lookup of the batch: row byte offset (or row), {w*s, w*o}
-  __shared__ uint32_t s_key[kGroups][kBatch];
-  __shared__ float2 s_ws[kGroups][kBatch];
+  constexpr int kDataBytes = LPR * 4;
+  __shared__ uint32_t s_part[WAVES];
+  __shared__ long long s_below[WAVES];
+  __shared__ int s_own[WAVES];
+  // per wave, per lookup of the batch: row byte offset (or row) and
+  // {w, s, o} (kMathElement) or {w*s, w*o} (kMathRegrouped)
+  __shared__ uint32_t s_key[WAVES][kBatch];
+  __shared__ float4 s_ws[WAVES][kBatch];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const long long first_bag = (long long)blockIdx.x * kGroups;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const long long first_bag = (long long)blockIdx.x * WAVES;
   const long long bag = first_bag + wave;
 
   long long start;
   int len;
-  wave_bag_span(a, tid, wave, bag, first_bag, s_part, s_own, start, len);
+  rows_bag_span<WAVES>(a, tid, lane, wave, first_bag, s_part, s_below, s_own, start, len);
   uint32_t *keys = s_key[wave];
-  float2 *wso = s_ws[wave];
+  float4 *wso = s_ws[wave];
 
   const int sub = lane / LPR;             // which row of a load this lane reads
   const int lir = lane % LPR;
@@ -665,54 +792,81 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_rows_kernel(SlwsArgs a) {
   float acc_o = 0.0f;
 #pragma unroll
   for (int c = 0; c < kCols; c++) acc[c] = 0.0f;
+  if constexpr (PROBE == kProbeSpan) {
+    // measurement only: the launch up to the bags' positions
+    if (bag < a.segments && lane == 0)
+      reinterpret_cast<float *>(a.dest)[bag * a.out_cols] = (float)(start + len);
+    return;
+  }
+  const bool sep = !SO16 && a.sep_scales != nullptr;   // uniform
 
   for (int base = 0; base < len; base += kBatch) {
     const int cnt = min(kBatch, len - base);
-    // round 1: lane j fetches lookup j of the batch
+    // round 1: lane j fetches lookup j of the batch. len never reaches past
+    // the index list (see rows_bag_span), so lane < cnt is the only check.
     uint32_t so_lo = 0, so_hi = 0;
-    float my_w;
-    bool my_valid;
+    float my_w = 0.0f;
+    bool my_valid = false;
     {
-      const long long pos = start + base + lane;
-      long long row = -1;
-      float w = 0.0f;
-      if (lane < cnt && pos < a.num_indices) {
-        row = a.idx64 ? ((const global_i64 *)a.indices)[pos]
-                      : (long long)((const global_i32 *)a.indices)[pos];
-        if (!a.weights) {
-          w = 1.0f;
-        } else if (a.w16) {
-          w = __half2float(reinterpret_cast<const __half *>(a.weights)[pos]);
+      const long long at = start + base;   // uniform: scalar base + lane offset
+      uint32_t row = 0;
+      if (lane < cnt) {
+        if (a.idx64) {
+          const long long r = ((const global_i64 *)a.indices + at)[lane];
+          my_valid = (unsigned long long)r < (unsigned long long)a.data_rows;
+          row = (uint32_t)r;
         } else {
-          w = reinterpret_cast<const float *>(a.weights)[pos];
+          row = (uint32_t)((const global_i32 *)a.indices + at)[lane];
+          my_valid = row < (uint32_t)a.data_rows;
+        }
+        if (!a.weights) {
+          my_w = 1.0f;
+        } else if (a.w16) {
+          my_w = __half2float(
+              __ushort_as_half(((const global_u16 *)a.weights + at)[lane]));
+        } else {
+          my_w = __uint_as_float(((const global_u32 *)a.weights + at)[lane]);
         }
       }
       // a skipped lookup reads row 0 and contributes exactly +0
-      my_valid = row >= 0 && row < a.data_rows;
       if (!my_valid) row = 0;
-      my_w = w;
       // The row's scale and offset are requested here and consumed only after
       // the row reads below have been issued, so that the two round trips that
       // depend on the index (scale/offset, row bytes) overlap.
       // (Loads through global-address pointers: a generic-address load also
       // counts as an LDS operation, and the wait for the keys below would then
       // wait for it.)
-      if (!SO16 && a.sep_scales) {
+      if (sep) {
         so_lo = ((const global_u32 *)a.sep_scales)[row];
         so_hi = ((const global_u32 *)a.sep_offsets)[row];
+      } else if constexpr (OFF32) {
+        const uint32_t key = row * (uint32_t)a.in_line;
+        const global_u32 *so =
+            (const global_u32 *)((const global_u8 *)a.data + kDataBytes) ;
+        so_lo = *(const global_u32 *)((const global_u8 *)so + key);
+        if constexpr (!SO16) so_hi = *(const global_u32 *)((const global_u8 *)so + key + 4u);
       } else {
-        // rows and their data bytes are multiples of 4 bytes here
         const global_u32 *so = (const global_u32 *)((const global_u8 *)a.data +
-                                                    (row * a.in_line + a.data_bytes));
+                                                    ((long long)row * a.in_line + kDataBytes));
         so_lo = so[0];
         if constexpr (!SO16) so_hi = so[1];
       }
-      keys[lane] = OFF32 ? (uint32_t)(row * a.in_line) : (uint32_t)row;
+      keys[lane] = OFF32 ? row * (uint32_t)a.in_line : row;
+      if constexpr (PROBE == kProbeIndex) {
+        // measurement only: up to the index and weight of every lookup
+        acc_o += my_w + (float)row;
+        continue;
+      }
+    }
+    if constexpr (PROBE == kProbeScaleOffset) {
+      // measurement only: up to the scale and offset of every lookup
+      acc_o += my_valid ? my_w * __uint_as_float(so_lo) + __uint_as_float(so_hi) : 0.0f;
+      continue;
     }
     wave_lds_sync();
     // round 2: all row reads of the batch in flight before the first use, taken
     // kChunk load instructions at a time under one uniform branch. Slots
-    // beyond cnt hold {row 0, 0, 0} and add exactly +0.
+    // beyond cnt hold {row 0, 0, 0, 0} and add exactly +0.
     uint32_t q[kLoads];
 #pragma unroll
     for (int c = 0; c < kLoads / kChunk; c++) {
@@ -739,7 +893,12 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_rows_kernel(SlwsArgs a) {
         sc = __uint_as_float(so_lo);
         of = __uint_as_float(so_hi);
       }
-      wso[lane] = my_valid ? make_float2(my_w * sc, my_w * of) : make_float2(0.0f, 0.0f);
+      if constexpr (MATH == kMathElement)
+        wso[lane] = my_valid ? make_float4(my_w, sc, of, 0.0f)
+                             : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      else
+        wso[lane] = my_valid ? make_float4(my_w * sc, my_w * of, 0.0f, 0.0f)
+                             : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     }
     wave_lds_sync();
 #pragma unroll
@@ -748,36 +907,52 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_rows_kernel(SlwsArgs a) {
 #pragma unroll
         for (int u = 0; u < kChunk; u++) {
           const int g = c * kChunk + u;
-          const float2 f = wso[g * RPI + sub];
-          acc_o += f.y;
+          if constexpr (PROBE == kProbeRows) {
+            // measurement only: every row read, no arithmetic
+            acc_o = __uint_as_float(__float_as_uint(acc_o) ^ q[g]);
+            continue;
+          }
+          const float4 f = wso[g * RPI + sub];
+          if constexpr (MATH == kMathRegrouped) acc_o += f.y;
           if constexpr (IS4) {
             const uint32_t lo = q[g] & 0x0f0f0f0fu, hi = (q[g] >> 4) & 0x0f0f0f0fu;
 #pragma unroll
             for (int b = 0; b < 4; b++) {
-              acc[2 * b] = __fmaf_rn(f.x, (float)((lo >> (8 * b)) & 0xff), acc[2 * b]);
+              acc[2 * b] = fused_term<MATH>(f, (float)((lo >> (8 * b)) & 0xff), acc[2 * b]);
               acc[2 * b + 1] =
-                  __fmaf_rn(f.x, (float)((hi >> (8 * b)) & 0xff), acc[2 * b + 1]);
+                  fused_term<MATH>(f, (float)((hi >> (8 * b)) & 0xff), acc[2 * b + 1]);
             }
           } else {
 #pragma unroll
             for (int b = 0; b < 4; b++)
-              acc[b] = __fmaf_rn(f.x, (float)((q[g] >> (8 * b)) & 0xff), acc[b]);
+              acc[b] = fused_term<MATH>(f, (float)((q[g] >> (8 * b)) & 0xff), acc[b]);
           }
         }
       }
     }
     wave_lds_sync(); // slots are rewritten by the next batch
   }
+  if constexpr (PROBE == kProbeRows) acc_o = (float)(__float_as_uint(acc_o) & 0xffu);
 
   // partial sums of the RPI row groups -> lanes of group 0
 #pragma unroll
   for (int c = 0; c < kCols; c++) {
-    float v = acc[c] + acc_o;
+    float v = MATH == kMathRegrouped || PROBE != kProbeOff ? acc[c] + acc_o : acc[c];
 #pragma unroll
     for (int off = LPR; off < 64; off <<= 1) v += __shfl_xor(v, off, 64);
     acc[c] = v;
   }
-  if (bag < a.segments && sub == 0) store_columns<kCols>(a, bag, lir * kCols, acc);
+  if (bag < a.segments && sub == 0) {
+    float *d = reinterpret_cast<float *>(a.dest) + (bag * (long long)(LPR * kCols) + lir * kCols);
+    if (!a.out_q8 && !a.out16 && ((((uintptr_t)a.dest) & 15) == 0)) {
+      // dense fp32 rows of exactly LPR * kCols columns: 16-byte stores
+#pragma unroll
+      for (int c = 0; c < kCols; c += 4)
+        *reinterpret_cast<float4 *>(d + c) = make_float4(acc[c], acc[c + 1], acc[c + 2], acc[c + 3]);
+    } else {
+      store_columns<kCols>(a, bag, lir * kCols, acc);
+    }
+  }
 }
 
 // The same arithmetic for short rows (32 or 64 data bytes): a row takes only
@@ -785,7 +960,7 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_rows_kernel(SlwsArgs a) {
 // per lane group, and nothing has to be added across lanes at the end. A
 // group's lanes fetch its lookups (index, weight, scale, offset) kGB at a
 // time and hand them to each other through a wave-private LDS table.
-template <bool IS4, bool SO16, int LPR, bool OFF32>
+template <bool IS4, bool SO16, int LPR, bool OFF32, int MATH>
 __global__ __launch_bounds__(kSlwsThreads) void slws_groups_kernel(SlwsArgs a) {
   select_table(a);
   constexpr int kGroups = kSlwsThreads / LPR; // bags per block
@@ -796,7 +971,7 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_groups_kernel(SlwsArgs a) {
   __shared__ long long s_part[kSlwsThreads / 64];
   __shared__ int s_own[kGroups];
   __shared__ uint32_t s_key[kGroups][kGB];
-  __shared__ float2 s_ws[kGroups][kGB];
+  __shared__ float4 s_ws[kGroups][kGB];
 
   const int tid = threadIdx.x;
   const int grp = tid / LPR, lir = tid % LPR;
@@ -817,7 +992,7 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_groups_kernel(SlwsArgs a) {
   wave_len = __builtin_amdgcn_readfirstlane(wave_len);
 
   uint32_t *keys = s_key[grp];
-  float2 *wso = s_ws[grp];
+  float4 *wso = s_ws[grp];
   const uint32_t lane_off = (uint32_t)lir * 4u;
   float acc[kCols];
   float acc_o = 0.0f;
@@ -893,8 +1068,12 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_groups_kernel(SlwsArgs a) {
         sc = __uint_as_float(so_lo[k]);
         of = __uint_as_float(so_hi[k]);
       }
-      wso[lir + k * LPR] =
-          my_valid[k] ? make_float2(my_w[k] * sc, my_w[k] * of) : make_float2(0.0f, 0.0f);
+      if constexpr (MATH == kMathElement)
+        wso[lir + k * LPR] = my_valid[k] ? make_float4(my_w[k], sc, of, 0.0f)
+                                         : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      else
+        wso[lir + k * LPR] = my_valid[k] ? make_float4(my_w[k] * sc, my_w[k] * of, 0.0f, 0.0f)
+                                         : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     }
     wave_lds_sync();
 #pragma unroll
@@ -903,20 +1082,20 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_groups_kernel(SlwsArgs a) {
 #pragma unroll
         for (int u = 0; u < kChunk; u++) {
           const int j = c * kChunk + u;
-          const float2 f = wso[j];
-          acc_o += f.y;
+          const float4 f = wso[j];
+          if constexpr (MATH == kMathRegrouped) acc_o += f.y;
           if constexpr (IS4) {
             const uint32_t lo = q[j] & 0x0f0f0f0fu, hi = (q[j] >> 4) & 0x0f0f0f0fu;
 #pragma unroll
             for (int b = 0; b < 4; b++) {
-              acc[2 * b] = __fmaf_rn(f.x, (float)((lo >> (8 * b)) & 0xff), acc[2 * b]);
+              acc[2 * b] = fused_term<MATH>(f, (float)((lo >> (8 * b)) & 0xff), acc[2 * b]);
               acc[2 * b + 1] =
-                  __fmaf_rn(f.x, (float)((hi >> (8 * b)) & 0xff), acc[2 * b + 1]);
+                  fused_term<MATH>(f, (float)((hi >> (8 * b)) & 0xff), acc[2 * b + 1]);
             }
           } else {
 #pragma unroll
             for (int b = 0; b < 4; b++)
-              acc[b] = __fmaf_rn(f.x, (float)((q[j] >> (8 * b)) & 0xff), acc[b]);
+              acc[b] = fused_term<MATH>(f, (float)((q[j] >> (8 * b)) & 0xff), acc[b]);
           }
         }
       }
@@ -926,6 +1105,11 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_groups_kernel(SlwsArgs a) {
 #pragma unroll
   for (int c = 0; c < kCols; c++) acc[c] += acc_o;
   if (bag < a.segments) store_columns<kCols>(a, bag, lir * kCols, acc);
+}
+
+// A launch that does nothing (measurement: what any launch of this shape costs).
+__global__ __launch_bounds__(kRowsWaves * 64) void slws_empty_kernel(float *dest) {
+  if (dest == nullptr && threadIdx.x == 12345) dest[0] = 0.0f; // never taken
 }
 
 // Sum of the clamped lengths of each chunk of kChunkBags bags.
@@ -1097,11 +1281,11 @@ static void launch_wave_kind(int kind, bool acc16, dim3 grid, hipStream_t st,
 #undef MI355X_SLWS_WAVE
 }
 
-template <int LPR, bool OFF32>
+template <int LPR, bool OFF32, int MATH>
 static void launch_rows_kind(int kind, dim3 grid, hipStream_t st, const SlwsArgs &a) {
 #define MI355X_SLWS_ROWS(IS4, SO16)                                            \
-  hipLaunchKernelGGL((slws_rows_kernel<IS4, SO16, LPR, OFF32>), grid,          \
-                     dim3(kSlwsThreads), 0, st, a)
+  hipLaunchKernelGGL((slws_rows_kernel<IS4, SO16, LPR, OFF32, MATH, kRowsWaves>), grid, \
+                     dim3(kRowsWaves * 64), 0, st, a)
   switch (kind) {
   case MI355X_FUSED_U8_F32:
     MI355X_SLWS_ROWS(false, false);
@@ -1119,10 +1303,10 @@ static void launch_rows_kind(int kind, dim3 grid, hipStream_t st, const SlwsArgs
 #undef MI355X_SLWS_ROWS
 }
 
-template <int LPR, bool OFF32>
+template <int LPR, bool OFF32, int MATH>
 static void launch_groups_kind(int kind, dim3 grid, hipStream_t st, const SlwsArgs &a) {
 #define MI355X_SLWS_GROUPS(IS4, SO16)                                          \
-  hipLaunchKernelGGL((slws_groups_kernel<IS4, SO16, LPR, OFF32>), grid,        \
+  hipLaunchKernelGGL((slws_groups_kernel<IS4, SO16, LPR, OFF32, MATH>), grid,  \
                      dim3(kSlwsThreads), 0, st, a)
   switch (kind) {
   case MI355X_FUSED_U8_F32:
@@ -1141,8 +1325,8 @@ static void launch_groups_kind(int kind, dim3 grid, hipStream_t st, const SlwsAr
 #undef MI355X_SLWS_GROUPS
 }
 
-// Whether the fused-arithmetic kernels may be used (process-wide).
-static std::atomic<int> g_fused_math{1};
+// Arithmetic of the launches that do not name one (process-wide default).
+static std::atomic<int> g_fused_math{kMathElement};
 
 // Several tables in one launch and/or the int8 output transform.
 struct SlwsExtra {
@@ -1154,6 +1338,8 @@ struct SlwsExtra {
   int32_t q_offset = 0;
   size_t q_stride = 0;
   bool static_scratch = false; // chunk sums in the code object's fixed array
+  int math = -1;               // kMath*; -1 = the process-wide default
+  int probe = kProbeOff;       // measurement cut point (mi355x_frwq_slws_probe)
 };
 
 static int slws_dispatch(void *dest, int out_is_f16, const uint8_t *data,
@@ -1254,33 +1440,72 @@ static int slws_dispatch(void *dest, int out_is_f16, const uint8_t *data,
   // fused arithmetic: whole rows of 32, 64, 128 or 256 data bytes, 4-byte
   // aligned, fp32 accumulation. A multi-table launch cannot check the
   // alignment of each table here; its tables must be 4-byte aligned.
-  const bool rows_ok = g_fused_math.load(std::memory_order_relaxed) && !acc16 &&
+  const int math = x.math >= 0 ? x.math : g_fused_math.load(std::memory_order_relaxed);
+  MI355X_REQUIRE(math >= kMathStrict && math <= kMathRegrouped,
+                 "unknown SparseLengths arithmetic %d", math);
+  const bool rows_ok = math != kMathStrict && !acc16 &&
                        in_line_size % 4 == 0 && (((uintptr_t)data) % 4 == 0) &&
                        (data_bytes == 32 || data_bytes == 64 ||
                         data_bytes == 128 || data_bytes == 256);
+  if (x.probe != kProbeOff) {
+    MI355X_REQUIRE(rows_ok && kind == MI355X_FUSED_U8_F32 && data_bytes == 128 && off32 &&
+                       !x.tables && !x.out_q8 && math == kMathElement,
+                   "the probe covers uint8 rows of 128 columns with fp32 scale and offset");
+    const size_t rblocks = (out_rows + kRowsWaves - 1) / kRowsWaves;
+    MI355X_REQUIRE(rblocks < 0x7fffffffu, "too many bags");
+    dim3 rgrid((unsigned)rblocks);
+#define MI355X_PROBE_CASE(P)                                                   \
+  case P:                                                                      \
+    hipLaunchKernelGGL(                                                        \
+        (slws_rows_kernel<false, false, 32, true, kMathElement, kRowsWaves, P>), rgrid,     \
+        dim3(kRowsWaves * 64), 0, st, a);                                      \
+    break;
+    switch (x.probe) {
+      MI355X_PROBE_CASE(kProbeSpan)
+      MI355X_PROBE_CASE(kProbeIndex)
+      MI355X_PROBE_CASE(kProbeScaleOffset)
+      MI355X_PROBE_CASE(kProbeRows)
+    default:
+      return fail(MI355X_ERR_INVALID_ARGUMENT, "unknown probe stage %d", x.probe);
+    }
+#undef MI355X_PROBE_CASE
+    return check_launch("frwq_slws_probe");
+  }
   if (rows_ok && data_bytes <= 64) {
     // short rows: several bags per wavefront
     const size_t per_block = kSlwsThreads / (data_bytes / 4);
     const size_t gblocks = (out_rows + per_block - 1) / per_block;
     MI355X_REQUIRE(gblocks < 0x7fffffffu, "too many bags");
     dim3 ggrid((unsigned)gblocks, (unsigned)x.n_tables);
+#define MI355X_GROUPS_CASE(LPR)                                                \
+  if (math == kMathElement) {                                                  \
+    if (off32) launch_groups_kind<LPR, true, kMathElement>(kind, ggrid, st, a);  \
+    else launch_groups_kind<LPR, false, kMathElement>(kind, ggrid, st, a);     \
+  } else {                                                                     \
+    if (off32) launch_groups_kind<LPR, true, kMathRegrouped>(kind, ggrid, st, a); \
+    else launch_groups_kind<LPR, false, kMathRegrouped>(kind, ggrid, st, a);   \
+  }
     if (data_bytes == 32) {
-      if (off32) launch_groups_kind<8, true>(kind, ggrid, st, a);
-      else launch_groups_kind<8, false>(kind, ggrid, st, a);
+      MI355X_GROUPS_CASE(8)
     } else {
-      if (off32) launch_groups_kind<16, true>(kind, ggrid, st, a);
-      else launch_groups_kind<16, false>(kind, ggrid, st, a);
+      MI355X_GROUPS_CASE(16)
     }
+#undef MI355X_GROUPS_CASE
     return check_launch("frwq_slws");
   }
   if (rows_ok) {
-    const size_t rblocks = (out_rows + 3) / 4;
+    const size_t rblocks = (out_rows + kRowsWaves - 1) / kRowsWaves;
     MI355X_REQUIRE(rblocks < 0x7fffffffu, "too many bags");
     dim3 rgrid((unsigned)rblocks, (unsigned)x.n_tables);
 #define MI355X_ROWS_CASE(BYTES)                                                \
   case BYTES:                                                                  \
-    if (off32) launch_rows_kind<BYTES / 4, true>(kind, rgrid, st, a);          \
-    else launch_rows_kind<BYTES / 4, false>(kind, rgrid, st, a);               \
+    if (math == kMathElement) {                                                \
+      if (off32) launch_rows_kind<BYTES / 4, true, kMathElement>(kind, rgrid, st, a); \
+      else launch_rows_kind<BYTES / 4, false, kMathElement>(kind, rgrid, st, a); \
+    } else {                                                                   \
+      if (off32) launch_rows_kind<BYTES / 4, true, kMathRegrouped>(kind, rgrid, st, a); \
+      else launch_rows_kind<BYTES / 4, false, kMathRegrouped>(kind, rgrid, st, a); \
+    }                                                                          \
     break;
     switch (data_bytes) {
       MI355X_ROWS_CASE(32)
@@ -1307,8 +1532,31 @@ using namespace mi355x;
 extern "C" {
 
 int mi355x_slws_set_fused_math(int on) {
-  g_fused_math.store(on ? 1 : 0, std::memory_order_relaxed);
+  MI355X_REQUIRE(on >= kMathStrict && on <= kMathRegrouped,
+                 "unknown SparseLengths arithmetic %d", on);
+  g_fused_math.store(on, std::memory_order_relaxed);
   return MI355X_OK;
+}
+
+int mi355x_frwq_slws_probe(int stage, float *dest, const uint8_t *data, size_t data_rows,
+                           const float *weights, const int64_t *indices,
+                           size_t num_indices, const int32_t *lengths, size_t segments,
+                           size_t in_line_size, void *stream) {
+  MI355X_REQUIRE(segments == 0 || lengths, "lengths is NULL");
+  if (stage == 0) {
+    // a launch of the same shape that does nothing
+    if (segments == 0) return MI355X_OK;
+    hipLaunchKernelGGL(slws_empty_kernel,
+                       dim3((unsigned)((segments + kRowsWaves - 1) / kRowsWaves)),
+                       dim3(kRowsWaves * 64), 0, as_stream(stream), dest);
+    return check_launch("slws_empty");
+  }
+  SlwsExtra x;
+  x.math = kMathElement;
+  x.probe = stage;
+  return slws_dispatch(dest, 0, data, data_rows, MI355X_FUSED_U8_F32, weights, 0, indices, 1,
+                       num_indices, lengths, nullptr, 0, segments, in_line_size, 128, 0,
+                       stream, x);
 }
 
 int mi355x_frwq_sls_multi(const mi355x_sls_table *tables, size_t n_tables,
