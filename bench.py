@@ -769,9 +769,9 @@ def main():
         # the cache-resident variant: 8 batches, no flush
         s = bench_slws(capi, args, d_table, batches[:8], None)
     elif only == "slws_strict":
-        capi.slws_set_fused_math(False)
+        capi.slws_set_fused_math(capi.SLWS_MATH_STRICT)
         s = bench_slws(capi, args, d_table, batches, flush)
-        capi.slws_set_fused_math(True)
+        capi.slws_set_fused_math(capi.SLWS_MATH_ELEMENT)
     else:
         s = bench_slws(capi, args, d_table, batches, flush)
     gbps = s["bytes"] / s["sec"] / 1e9
@@ -798,7 +798,7 @@ def main():
             frac_of_hbm_peak=w8["bytes"] / w8["sec"] / 1e9 / HBM_PEAK_GBPS)
         # strict arithmetic: every multiply and add rounded on its own, in bag
         # order; bit for bit the CPU loop
-        capi.slws_set_fused_math(False)
+        capi.slws_set_fused_math(capi.SLWS_MATH_STRICT)
         try:
             ss = bench_slws(capi, args, d_table, batches, flush)
             bit_exact = None
@@ -808,9 +808,9 @@ def main():
                                         ss["last"]["lengths"])
                 bit_exact = bool(np.array_equal(ss["d_out"].numpy(), want))
         finally:
-            capi.slws_set_fused_math(True)
+            capi.slws_set_fused_math(capi.SLWS_MATH_ELEMENT)
         extra["slws_strict"] = dict(
-            workload="headline lookup with mi355x_slws_set_fused_math(0)",
+            workload="headline lookup with MI355X_SLWS_MATH_STRICT",
             ms=ss["sec"] * 1e3, gbps=ss["bytes"] / ss["sec"] / 1e9,
             frac_of_hbm_peak=ss["bytes"] / ss["sec"] / 1e9 / HBM_PEAK_GBPS,
             bit_exact_with_oracle=bit_exact)
@@ -880,11 +880,17 @@ def main():
             "device": info.name.decode() or "MI355X", "arch": info.arch.decode(),
             "compute_units": info.compute_units,
         },
-        "parity_with_oracle": (None if parity is None else bool(parity <= 1e-5)),
-        "max_error_over_bag_magnitude": parity,
+        # the stated bar, element by element: |got - oracle| <= 1e-5 |oracle| for
+        # every output at or above the floor, and the outputs below it (sums that
+        # have cancelled) within 1e-5 of the magnitude their bag adds up
+        "parity_with_oracle": (None if parity is None
+                               else bool(rel <= 1e-5 and parity <= 1e-5)),
         "max_rel_error_elementwise": rel,
         "rel_error_floor": "outputs with |oracle value| >= 1.0",
         "share_of_outputs_above_floor": share,
+        "max_error_over_bag_magnitude": parity,
+        "arithmetic": "v = fma(s, q, o); acc = fma(w, v, acc) per element in bag order "
+                      "(MI355X_SLWS_MATH_ELEMENT, the library's default)",
         "cache_state": ("caches flushed before the timed replay; "
                         f"{args.batches} distinct index batches cycled"),
         "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS,
@@ -892,12 +898,15 @@ def main():
                      "traffic": (MEASURED_TRAFFIC["slws"]
                                  if (args.rows, args.bags, args.batches) ==
                                  (4_000_000, 4096, 64) and not only else None),
-                     "kernel": "slws_rows_kernel<false,false,32,true>"},
+                     "traffic_source": "profiles/slws_rows_kernel__slws_u8_4Mx128_4096bags.md "
+                                       "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not "
+                                       "measured in this run)",
+                     "kernel": "slws_rows_kernel<false,false,32,true,1,8>"},
         "cpu_baseline": cpu,
         "extra": extra,
     }
     print(json.dumps(out))
-    if parity is not None and not parity <= 1e-5:
+    if parity is not None and not (rel <= 1e-5 and parity <= 1e-5):
         sys.exit(1)
 
 

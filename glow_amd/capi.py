@@ -19,13 +19,13 @@ REGION_CONSTANTS, REGION_MUTABLE, REGION_ACTIVATIONS = 0, 1, 2
 
 # Every symbol include/glow_mi355x.h declares (checked by the CPU test suite).
 EXPORTS = [
-    "mi355x_last_error", "mi355x_num_devices", "mi355x_init",
+    "mi355x_last_error", "mi355x_num_devices", "mi355x_init", "mi355x_rwq_fc_i8_opts", "mi355x_rwq_fc_relu_i8_opts", "mi355x_fc_i8_opts", "mi355x_matmul_i8_opts", "mi355x_cwq_conv2d_i8_opts", "mi355x_cwq_conv2d_add_i8_opts", "mi355x_conv2d_i8_opts", "mi355x_frwq_slws_opts", "mi355x_frwq_slws_offsets_opts", "mi355x_frwq_slws_noalloc_opts", "mi355x_frwq_sls_multi_opts", "mi355x_rwq_slws_opts", "mi355x_embedding_bag_rowwise_offsets_opts", "mi355x_frwq_slws_probe",
     "mi355x_device_info", "mi355x_malloc", "mi355x_free", "mi355x_host_alloc",
     "mi355x_host_free", "mi355x_memcpy_h2d", "mi355x_memcpy_d2h",
     "mi355x_memcpy_d2d", "mi355x_fill_u8", "mi355x_copy_u8", "mi355x_gemm_tile_override",
     "mi355x_cwq_conv2d_add_i8", "mi355x_frwq_sls_multi",
     "mi355x_specialize_bias_weights_qparams", "mi355x_rwq_slws", "mi355x_slws_set_fused_math", "mi355x_batch_matmul_nt_i8", "mi355x_batch_matmul_nt_select_i8", "mi355x_rwq_fc_relu_i8", "mi355x_add_i8", "mi355x_add_relu_i8",
-    "mi355x_relu_i8", "mi355x_convert_f16_to_f32", "mi355x_insert_rows",
+    "mi355x_relu_i8", "mi355x_clip_i8", "mi355x_leaky_relu_i8", "mi355x_max_splat_i8", "mi355x_batched_add_i8", "mi355x_convert_f16_to_f32", "mi355x_insert_rows",
     "mi355x_batch_transpose_i8", "mi355x_space_to_depth2_i8", "mi355x_quantize_space_to_depth2_i8", "mi355x_gather", "mi355x_gather_rows", "mi355x_rescale_rows_i8",
     "mi355x_dequantize_sigmoid", "mi355x_batch_matmul_i8", "mi355x_sigmoid_f32",
     "mi355x_max_pool_i8", "mi355x_avg_pool_i8", "mi355x_softmax_f32", "mi355x_dequantize_softmax", "mi355x_stream_create",
@@ -538,30 +538,54 @@ def launch_rowsum_i8(sums, rows, n_rows, K, stream=None):
                                  _vp(stream)))
 
 
+SLWS_MATH_STRICT, SLWS_MATH_ELEMENT, SLWS_MATH_REGROUPED = 0, 1, 2
+
+
+class LaunchOpts(C.Structure):
+    """mi355x_launch_opts: options that hold for one call of an <entry>_opts
+    entry point (workgroup tile, requantisation hint, SparseLengths
+    arithmetic)."""
+    _fields_ = [("struct_size", C.c_uint32), ("gemm_tile", C.c_int32),
+                ("requant_hint", C.c_int32), ("slws_math", C.c_int32)]
+
+    def __init__(self, gemm_tile=-1, requant_hint=0, slws_math=-1):
+        super().__init__(C.sizeof(LaunchOpts), gemm_tile, requant_hint, slws_math)
+
+
+def _entry(name, opts):
+    """(function, trailing arguments) of entry point `name`: its _opts twin when
+    options are given."""
+    if opts is None:
+        return getattr(lib(), name), ()
+    return getattr(lib(), name + "_opts"), (C.byref(opts),)
+
+
 def launch_rwq_fc_i8(out, x, w, bias, bias_is_i8, w_offsets, bias_pre,
                      bias_post, bias_scale, out_pre, out_post, out_scale, M, K,
                      N, out_offset, in_offset, bias_offset,
-                     w_offsets_all_zero=False, w_row_sums=None, stream=None):
-    check(lib().mi355x_rwq_fc_i8(
+                     w_offsets_all_zero=False, w_row_sums=None, stream=None, opts=None):
+    fn, tail = _entry("mi355x_rwq_fc_i8", opts)
+    check(fn(
         _vp(out), _vp(x), _vp(w), _vp(bias), C.c_int(bias_is_i8),
         _vp(w_offsets), _vp(bias_pre), _vp(bias_post), _vp(bias_scale),
         _vp(out_pre), _vp(out_post), _vp(out_scale), _sz(M), _sz(K), _sz(N),
         _i32(out_offset), _i32(in_offset), _i32(bias_offset),
-        C.c_int(bool(w_offsets_all_zero)), _vp(w_row_sums), _vp(stream)))
+        C.c_int(bool(w_offsets_all_zero)), _vp(w_row_sums), _vp(stream), *tail))
 
 
 def launch_cwq_conv2d_i8(out, x, filt, bias, bias_is_i8, geom, out_offset,
                          in_offset, f_offsets, b_offsets, bias_pre, bias_post,
                          bias_scale, out_pre, out_post, out_scale, act,
                          act_args, f_offsets_all_zero=False, f_row_sums=None,
-                         stream=None):
+                         stream=None, opts=None):
     aa = (C.c_int32 * 3)(*(list(act_args) + [0, 0, 0])[:3])
-    check(lib().mi355x_cwq_conv2d_i8(
+    fn, tail = _entry("mi355x_cwq_conv2d_i8", opts)
+    check(fn(
         _vp(out), _vp(x), _vp(filt), _vp(bias), C.c_int(bias_is_i8),
         C.byref(geom), _i32(out_offset), _i32(in_offset), _vp(f_offsets),
         _vp(b_offsets), _vp(bias_pre), _vp(bias_post), _vp(bias_scale),
         _vp(out_pre), _vp(out_post), _vp(out_scale), _i32(act), aa,
-        C.c_int(bool(f_offsets_all_zero)), _vp(f_row_sums), _vp(stream)))
+        C.c_int(bool(f_offsets_all_zero)), _vp(f_row_sums), _vp(stream), *tail))
 
 
 class FusedAdd(C.Structure):
@@ -597,29 +621,30 @@ def launch_cwq_conv2d_add_i8(out, x, filt, bias, bias_is_i8, geom, conv_offset,
 def launch_frwq_slws(dest, out_is_f16, data, data_rows, kind, weights,
                      weights_are_f16, indices, idx_is_64, num_indices, lengths,
                      segments, in_line, out_line, fp16_accum=False,
-                     stream=None, noalloc=False):
+                     stream=None, noalloc=False, opts=None):
     """noalloc: through mi355x_frwq_slws_noalloc (scratch in the library's fixed
     device array) instead of mi355x_frwq_slws (per-stream scratch)."""
-    fn = lib().mi355x_frwq_slws_noalloc if noalloc else lib().mi355x_frwq_slws
+    fn, tail = _entry("mi355x_frwq_slws_noalloc" if noalloc else "mi355x_frwq_slws", opts)
     check(fn(
         _vp(dest), C.c_int(bool(out_is_f16)), _vp(data), _sz(data_rows),
         C.c_int(kind), _vp(weights), C.c_int(bool(weights_are_f16)),
         _vp(indices), C.c_int(bool(idx_is_64)), _sz(num_indices), _vp(lengths),
         _sz(segments), _sz(in_line), _sz(out_line), C.c_int(bool(fp16_accum)),
-        _vp(stream)))
+        _vp(stream), *tail))
 
 
 def launch_frwq_slws_offsets(dest, out_is_f16, data, data_rows, kind, weights,
                              weights_are_f16, indices, idx_is_64, num_indices,
                              bag_offsets, segments, in_line, out_line, fp16_accum=False,
-                             stream=None):
+                             stream=None, opts=None):
     """mi355x_frwq_slws_offsets: bags by their segments + 1 positions."""
-    check(lib().mi355x_frwq_slws_offsets(
+    fn, tail = _entry("mi355x_frwq_slws_offsets", opts)
+    check(fn(
         _vp(dest), C.c_int(bool(out_is_f16)), _vp(data), _sz(data_rows),
         C.c_int(kind), _vp(weights), C.c_int(bool(weights_are_f16)),
         _vp(indices), C.c_int(bool(idx_is_64)), _sz(num_indices), _vp(bag_offsets),
         _sz(segments), _sz(in_line), _sz(out_line), C.c_int(bool(fp16_accum)),
-        _vp(stream)))
+        _vp(stream), *tail))
 
 
 def slws_bag_offsets_host(lengths):
@@ -854,7 +879,7 @@ def _fused_cols(in_line, kind):
 
 def frwq_slws(data, kind, weights, indices, lengths, out_f16=False,
               fp16_accum=False, d_data=None, row_pitch=None, stream=None,
-              noalloc=False, bag_offsets=False):
+              noalloc=False, bag_offsets=False, opts=None):
     """weights: None (plain SLS), float32 or float16 array. `d_data` lets a
     caller reuse a table already resident on the device. `row_pitch` lays the
     table out with its rows that many bytes apart (the gaps hold junk).
@@ -895,12 +920,12 @@ def frwq_slws(data, kind, weights, indices, lengths, out_f16=False,
         launch_frwq_slws_offsets(d_out, out_f16, d_data, data_shape[0], kind, d_w, w16,
                                  d_idx, indices.dtype == np.int64, indices.size,
                                  to_device(offs), lengths.size, in_line, out_line,
-                                 fp16_accum, stream=stream)
+                                 fp16_accum, stream=stream, opts=opts)
     else:
         launch_frwq_slws(d_out, out_f16, d_data, data_shape[0], kind, d_w, w16,
                          d_idx, indices.dtype == np.int64, indices.size, d_len,
                          lengths.size, in_line, out_line, fp16_accum, stream=stream,
-                         noalloc=noalloc)
+                         noalloc=noalloc, opts=opts)
     if stream is not None:
         stream.sync()
     return d_out.numpy()
@@ -1057,6 +1082,50 @@ def _pool_sizes(x, kernel, stride, pads):
     sz = [_sz(int(v)) for v in (N, IH, IW, Cn, OH, OW, kernel[0], kernel[1], stride[0],
                                 stride[1], pads[0], pads[1])]
     return (N, OH, OW, Cn), sz
+
+
+def clip_elem_i8(src, clip_min, clip_max, src_offset, dest_offset, destP):
+    src = np.ascontiguousarray(src, np.int8)
+    ds = to_device(src)
+    out = DeviceBuffer.empty(src.shape, np.int8)
+    check(lib().mi355x_clip_i8(_vp(out), _vp(ds), _sz(src.size), _i32(clip_min), _i32(clip_max),
+                               _i32(src_offset), _i32(dest_offset),
+                               *[_i32(int(v)) for v in destP], _vp(None)))
+    return out.numpy()
+
+
+def leaky_relu_i8(src, src_offset, dest_offset, posP, negP):
+    src = np.ascontiguousarray(src, np.int8)
+    ds = to_device(src)
+    out = DeviceBuffer.empty(src.shape, np.int8)
+    check(lib().mi355x_leaky_relu_i8(_vp(out), _vp(ds), _sz(src.size), _i32(src_offset),
+                                     _i32(dest_offset), *[_i32(int(v)) for v in posP],
+                                     *[_i32(int(v)) for v in negP], _vp(None)))
+    return out.numpy()
+
+
+def max_splat_i8(src, value):
+    src = np.ascontiguousarray(src, np.int8)
+    ds = to_device(src)
+    out = DeviceBuffer.empty(src.shape, np.int8)
+    check(lib().mi355x_max_splat_i8(_vp(out), _vp(ds), _sz(src.size), _i32(value), _vp(None)))
+    return out.numpy()
+
+
+def batched_add_i8(batch, slice_, dest_offset, batch_offset, slice_offset, batchP, sliceP):
+    batch = np.ascontiguousarray(batch, np.int8)
+    slice_ = np.ascontiguousarray(slice_)
+    i32 = slice_.dtype == np.int32
+    if not i32:
+        slice_ = slice_.astype(np.int8)
+    db, dsl = to_device(batch), to_device(slice_)
+    out = DeviceBuffer.empty(batch.shape, np.int8)
+    check(lib().mi355x_batched_add_i8(_vp(out), _vp(db), _vp(dsl), C.c_int(int(i32)),
+                                      _sz(batch.shape[0]), _sz(slice_.size), _i32(dest_offset),
+                                      _i32(batch_offset), _i32(slice_offset),
+                                      *[_i32(int(v)) for v in batchP],
+                                      *[_i32(int(v)) for v in sliceP], _vp(None)))
+    return out.numpy()
 
 
 def max_pool_i8(x, kernel, stride, pads, out_offset):

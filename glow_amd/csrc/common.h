@@ -35,6 +35,47 @@ int slws_release_stream(hipStream_t st);
 // mi355x_frwq_slws_noalloc on the current device.
 int slws_init_device();
 
+// Options of the launch being issued on this thread. The entry points with an
+// options argument set them for the duration of the call (OptsScope); the ones
+// without leave the thread's defaults in place (the legacy setters
+// mi355x_gemm_tile_override, mi355x_gemm_requant_hint; the process-wide
+// mi355x_slws_set_fused_math). Nothing outlives a call that names its options.
+extern thread_local int g_tile_override;   // -1: chosen from the shape
+extern thread_local int g_requant_hint;    // MI355X_REQUANT_* flags
+extern thread_local int g_slws_math;       // -1: the process default
+
+struct OptsScope {
+  int rc = MI355X_OK;
+  int tile, hint, math;
+  explicit OptsScope(const mi355x_launch_opts *o)
+      : tile(g_tile_override), hint(g_requant_hint), math(g_slws_math) {
+    if (!o) return;
+    if (o->struct_size != sizeof(mi355x_launch_opts)) {
+      rc = fail(MI355X_ERR_INVALID_ARGUMENT, "mi355x_launch_opts: struct_size %u, expected %zu",
+                o->struct_size, sizeof(mi355x_launch_opts));
+    } else if (o->gemm_tile < -1 || o->gemm_tile > 11) {
+      rc = fail(MI355X_ERR_INVALID_ARGUMENT, "gemm_tile %d outside [-1, 11]", o->gemm_tile);
+    } else if (o->requant_hint < 0 || o->requant_hint > 3 || o->requant_hint == 2) {
+      rc = fail(MI355X_ERR_INVALID_ARGUMENT,
+                "requant_hint %d: bit 1 (no pre-shifts) needs bit 0 (24-bit operands)",
+                o->requant_hint);
+    } else if (o->slws_math < -1 || o->slws_math > MI355X_SLWS_MATH_REGROUPED) {
+      rc = fail(MI355X_ERR_INVALID_ARGUMENT, "slws_math %d outside [-1, 2]", o->slws_math);
+    } else {
+      g_tile_override = o->gemm_tile;
+      g_requant_hint = o->requant_hint;
+      g_slws_math = o->slws_math;
+    }
+  }
+  ~OptsScope() {
+    g_tile_override = tile;
+    g_requant_hint = hint;
+    g_slws_math = math;
+  }
+  OptsScope(const OptsScope &) = delete;
+  OptsScope &operator=(const OptsScope &) = delete;
+};
+
 } // namespace mi355x
 
 #define MI355X_HIP(expr)                                                       \

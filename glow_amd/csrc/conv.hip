@@ -222,6 +222,12 @@ static int conv_common(int8_t *out, const int8_t *in, const int8_t *filter,
     ep.fast = g_requant_hint & 3;
     return gemm_stream_launch(R, filter, ep, (int)M, OCg, (int)K, as_stream(stream));
   }
+  // Tiles 6..8 name one special kernel each; a launch that kernel cannot serve
+  // says so instead of running another kernel under the asked-for number.
+  if (g_tile_override >= 6 && g_tile_override <= 8)
+    return fail(MI355X_ERR_NOT_SUPPORTED,
+                "tile %d does not apply to this convolution (shape, alignment or offsets)",
+                g_tile_override);
   // A pointwise convolution over the whole image is a plain matrix product:
   // row m of A is pixel m of the input, no taps to locate and no padding.
   if (g->KH == 1 && g->KW == 1 && g->strideH == 1 && g->strideW == 1 &&
@@ -257,7 +263,7 @@ using namespace mi355x;
 
 extern "C" {
 
-int mi355x_cwq_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
+static int mi355x_cwq_conv2d_i8_impl(int8_t *out, const int8_t *in, const int8_t *filter,
                          const void *bias, int bias_is_i8,
                          const mi355x_conv_geom *geom, int32_t out_offset,
                          int32_t in_offset, const int32_t *filter_offsets,
@@ -292,7 +298,36 @@ int mi355x_cwq_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
                      stream);
 }
 
-int mi355x_cwq_conv2d_add_i8(
+int mi355x_cwq_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
+                         const void *bias, int bias_is_i8,
+                         const mi355x_conv_geom *geom, int32_t out_offset,
+                         int32_t in_offset, const int32_t *filter_offsets,
+                         const int32_t *bias_offsets, const int32_t *bias_pre,
+                         const int32_t *bias_post, const int32_t *bias_scale,
+                         const int32_t *out_pre, const int32_t *out_post,
+                         const int32_t *out_scale, int32_t act_type,
+                         const int32_t *act_args, int filter_offsets_all_zero,
+                         const int32_t *filter_row_sums, void *stream) {
+  return mi355x_cwq_conv2d_i8_impl(out, in, filter, bias, bias_is_i8, geom, out_offset, in_offset, filter_offsets, bias_offsets, bias_pre, bias_post, bias_scale, out_pre, out_post, out_scale, act_type, act_args, filter_offsets_all_zero, filter_row_sums, stream);
+}
+
+int mi355x_cwq_conv2d_i8_opts(int8_t *out, const int8_t *in, const int8_t *filter,
+                         const void *bias, int bias_is_i8,
+                         const mi355x_conv_geom *geom, int32_t out_offset,
+                         int32_t in_offset, const int32_t *filter_offsets,
+                         const int32_t *bias_offsets, const int32_t *bias_pre,
+                         const int32_t *bias_post, const int32_t *bias_scale,
+                         const int32_t *out_pre, const int32_t *out_post,
+                         const int32_t *out_scale, int32_t act_type,
+                         const int32_t *act_args, int filter_offsets_all_zero,
+                         const int32_t *filter_row_sums, void *stream,
+    const mi355x_launch_opts *opts) {
+  OptsScope scope(opts);
+  if (scope.rc != MI355X_OK) return scope.rc;
+  return mi355x_cwq_conv2d_i8_impl(out, in, filter, bias, bias_is_i8, geom, out_offset, in_offset, filter_offsets, bias_offsets, bias_pre, bias_post, bias_scale, out_pre, out_post, out_scale, act_type, act_args, filter_offsets_all_zero, filter_row_sums, stream);
+}
+
+static int mi355x_cwq_conv2d_add_i8_impl(
     int8_t *out, const int8_t *in, const int8_t *filter, const void *bias,
     int bias_is_i8, const mi355x_conv_geom *geom, int32_t conv_offset,
     int32_t in_offset, const int32_t *filter_offsets,
@@ -348,7 +383,36 @@ int mi355x_cwq_conv2d_add_i8(
                      stream);
 }
 
-int mi355x_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
+int mi355x_cwq_conv2d_add_i8(
+    int8_t *out, const int8_t *in, const int8_t *filter, const void *bias,
+    int bias_is_i8, const mi355x_conv_geom *geom, int32_t conv_offset,
+    int32_t in_offset, const int32_t *filter_offsets,
+    const int32_t *bias_offsets, const int32_t *bias_pre,
+    const int32_t *bias_post, const int32_t *bias_scale, const int32_t *out_pre,
+    const int32_t *out_post, const int32_t *out_scale, int32_t act_type,
+    const int32_t *act_args, int filter_offsets_all_zero,
+    const int32_t *filter_row_sums, const int8_t *residual,
+    const mi355x_fused_add *add, void *stream) {
+  return mi355x_cwq_conv2d_add_i8_impl(out, in, filter, bias, bias_is_i8, geom, conv_offset, in_offset, filter_offsets, bias_offsets, bias_pre, bias_post, bias_scale, out_pre, out_post, out_scale, act_type, act_args, filter_offsets_all_zero, filter_row_sums, residual, add, stream);
+}
+
+int mi355x_cwq_conv2d_add_i8_opts(
+    int8_t *out, const int8_t *in, const int8_t *filter, const void *bias,
+    int bias_is_i8, const mi355x_conv_geom *geom, int32_t conv_offset,
+    int32_t in_offset, const int32_t *filter_offsets,
+    const int32_t *bias_offsets, const int32_t *bias_pre,
+    const int32_t *bias_post, const int32_t *bias_scale, const int32_t *out_pre,
+    const int32_t *out_post, const int32_t *out_scale, int32_t act_type,
+    const int32_t *act_args, int filter_offsets_all_zero,
+    const int32_t *filter_row_sums, const int8_t *residual,
+    const mi355x_fused_add *add, void *stream,
+    const mi355x_launch_opts *opts) {
+  OptsScope scope(opts);
+  if (scope.rc != MI355X_OK) return scope.rc;
+  return mi355x_cwq_conv2d_add_i8_impl(out, in, filter, bias, bias_is_i8, geom, conv_offset, in_offset, filter_offsets, bias_offsets, bias_pre, bias_post, bias_scale, out_pre, out_post, out_scale, act_type, act_args, filter_offsets_all_zero, filter_row_sums, residual, add, stream);
+}
+
+static int mi355x_conv2d_i8_impl(int8_t *out, const int8_t *in, const int8_t *filter,
                      const void *bias, int bias_is_i8,
                      const mi355x_conv_geom *geom, int32_t out_offset,
                      int32_t in_offset, int32_t filter_offset,
@@ -380,6 +444,33 @@ int mi355x_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
   set_act(ep, act_type, act_args);
   ep.sum_b = filter_row_sums;
   return conv_common(out, in, filter, geom, ep, filter_offset != 0, stream);
+}
+
+int mi355x_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
+                     const void *bias, int bias_is_i8,
+                     const mi355x_conv_geom *geom, int32_t out_offset,
+                     int32_t in_offset, int32_t filter_offset,
+                     int32_t bias_offset, int32_t bias_pre, int32_t bias_post,
+                     int32_t bias_scale, int32_t out_pre, int32_t out_post,
+                     int32_t out_scale, int32_t act_type,
+                     const int32_t *act_args, const int32_t *filter_row_sums,
+                     void *stream) {
+  return mi355x_conv2d_i8_impl(out, in, filter, bias, bias_is_i8, geom, out_offset, in_offset, filter_offset, bias_offset, bias_pre, bias_post, bias_scale, out_pre, out_post, out_scale, act_type, act_args, filter_row_sums, stream);
+}
+
+int mi355x_conv2d_i8_opts(int8_t *out, const int8_t *in, const int8_t *filter,
+                     const void *bias, int bias_is_i8,
+                     const mi355x_conv_geom *geom, int32_t out_offset,
+                     int32_t in_offset, int32_t filter_offset,
+                     int32_t bias_offset, int32_t bias_pre, int32_t bias_post,
+                     int32_t bias_scale, int32_t out_pre, int32_t out_post,
+                     int32_t out_scale, int32_t act_type,
+                     const int32_t *act_args, const int32_t *filter_row_sums,
+                     void *stream,
+    const mi355x_launch_opts *opts) {
+  OptsScope scope(opts);
+  if (scope.rc != MI355X_OK) return scope.rc;
+  return mi355x_conv2d_i8_impl(out, in, filter, bias, bias_is_i8, geom, out_offset, in_offset, filter_offset, bias_offset, bias_pre, bias_post, bias_scale, out_pre, out_post, out_scale, act_type, act_args, filter_row_sums, stream);
 }
 
 } // extern "C"

@@ -98,6 +98,12 @@ static int fc_common(int8_t *out, const int8_t *in, const int8_t *w_nk,
     ep.fast = g_requant_hint & 3;
     return gemm_stream_launch(R, w_nk, ep, (int)M, (int)N, (int)K, as_stream(stream));
   }
+  // Tiles 6..8 name one special kernel each; a launch that kernel cannot serve
+  // says so instead of running another kernel under the asked-for number.
+  if (g_tile_override >= 6 && g_tile_override <= 8)
+    return fail(MI355X_ERR_NOT_SUPPORTED,
+                "tile %d does not apply to this product (shape, alignment or offsets)",
+                g_tile_override);
   return gemm_dispatch(A, B, ep, (int)M, (int)N, (int)K, 1, 0, need_sa, need_sb,
                        aligned, as_stream(stream));
 }
@@ -146,7 +152,7 @@ int mi355x_rowsum_i8(int32_t *sums, const int8_t *rows, size_t n_rows, size_t K,
   return check_launch("rowsum_i8");
 }
 
-int mi355x_rwq_fc_i8(int8_t *out, const int8_t *in, const int8_t *weights,
+static int mi355x_rwq_fc_i8_impl(int8_t *out, const int8_t *in, const int8_t *weights,
                      const void *bias, int bias_is_i8,
                      const int32_t *weights_offsets, const int32_t *bias_pre,
                      const int32_t *bias_post, const int32_t *bias_scale,
@@ -181,7 +187,34 @@ int mi355x_rwq_fc_i8(int8_t *out, const int8_t *in, const int8_t *weights,
                    stream);
 }
 
-int mi355x_rwq_fc_relu_i8(int8_t *out, const int8_t *in, const int8_t *weights,
+int mi355x_rwq_fc_i8(int8_t *out, const int8_t *in, const int8_t *weights,
+                     const void *bias, int bias_is_i8,
+                     const int32_t *weights_offsets, const int32_t *bias_pre,
+                     const int32_t *bias_post, const int32_t *bias_scale,
+                     const int32_t *out_pre, const int32_t *out_post,
+                     const int32_t *out_scale, size_t M, size_t K, size_t N,
+                     int32_t out_offset, int32_t in_offset,
+                     int32_t bias_offset, int weights_offsets_all_zero,
+                     const int32_t *weights_row_sums, void *stream) {
+  return mi355x_rwq_fc_i8_impl(out, in, weights, bias, bias_is_i8, weights_offsets, bias_pre, bias_post, bias_scale, out_pre, out_post, out_scale, M, K, N, out_offset, in_offset, bias_offset, weights_offsets_all_zero, weights_row_sums, stream);
+}
+
+int mi355x_rwq_fc_i8_opts(int8_t *out, const int8_t *in, const int8_t *weights,
+                     const void *bias, int bias_is_i8,
+                     const int32_t *weights_offsets, const int32_t *bias_pre,
+                     const int32_t *bias_post, const int32_t *bias_scale,
+                     const int32_t *out_pre, const int32_t *out_post,
+                     const int32_t *out_scale, size_t M, size_t K, size_t N,
+                     int32_t out_offset, int32_t in_offset,
+                     int32_t bias_offset, int weights_offsets_all_zero,
+                     const int32_t *weights_row_sums, void *stream,
+    const mi355x_launch_opts *opts) {
+  OptsScope scope(opts);
+  if (scope.rc != MI355X_OK) return scope.rc;
+  return mi355x_rwq_fc_i8_impl(out, in, weights, bias, bias_is_i8, weights_offsets, bias_pre, bias_post, bias_scale, out_pre, out_post, out_scale, M, K, N, out_offset, in_offset, bias_offset, weights_offsets_all_zero, weights_row_sums, stream);
+}
+
+static int mi355x_rwq_fc_relu_i8_impl(int8_t *out, const int8_t *in, const int8_t *weights,
                           const void *bias, int bias_is_i8,
                           const int32_t *weights_offsets, const int32_t *bias_pre,
                           const int32_t *bias_post, const int32_t *bias_scale,
@@ -228,7 +261,36 @@ int mi355x_rwq_fc_relu_i8(int8_t *out, const int8_t *in, const int8_t *weights,
                    stream);
 }
 
-int mi355x_fc_i8(int8_t *out, const int8_t *in, const int8_t *weights_kn,
+int mi355x_rwq_fc_relu_i8(int8_t *out, const int8_t *in, const int8_t *weights,
+                          const void *bias, int bias_is_i8,
+                          const int32_t *weights_offsets, const int32_t *bias_pre,
+                          const int32_t *bias_post, const int32_t *bias_scale,
+                          const int32_t *out_pre, const int32_t *out_post,
+                          const int32_t *out_scale, size_t M, size_t K, size_t N,
+                          int32_t fc_offset, int32_t in_offset, int32_t bias_offset,
+                          int weights_offsets_all_zero, const int32_t *weights_row_sums,
+                          int32_t relu_offset, int32_t relu_pre, int32_t relu_post,
+                          int32_t relu_scale, void *stream) {
+  return mi355x_rwq_fc_relu_i8_impl(out, in, weights, bias, bias_is_i8, weights_offsets, bias_pre, bias_post, bias_scale, out_pre, out_post, out_scale, M, K, N, fc_offset, in_offset, bias_offset, weights_offsets_all_zero, weights_row_sums, relu_offset, relu_pre, relu_post, relu_scale, stream);
+}
+
+int mi355x_rwq_fc_relu_i8_opts(int8_t *out, const int8_t *in, const int8_t *weights,
+                          const void *bias, int bias_is_i8,
+                          const int32_t *weights_offsets, const int32_t *bias_pre,
+                          const int32_t *bias_post, const int32_t *bias_scale,
+                          const int32_t *out_pre, const int32_t *out_post,
+                          const int32_t *out_scale, size_t M, size_t K, size_t N,
+                          int32_t fc_offset, int32_t in_offset, int32_t bias_offset,
+                          int weights_offsets_all_zero, const int32_t *weights_row_sums,
+                          int32_t relu_offset, int32_t relu_pre, int32_t relu_post,
+                          int32_t relu_scale, void *stream,
+    const mi355x_launch_opts *opts) {
+  OptsScope scope(opts);
+  if (scope.rc != MI355X_OK) return scope.rc;
+  return mi355x_rwq_fc_relu_i8_impl(out, in, weights, bias, bias_is_i8, weights_offsets, bias_pre, bias_post, bias_scale, out_pre, out_post, out_scale, M, K, N, fc_offset, in_offset, bias_offset, weights_offsets_all_zero, weights_row_sums, relu_offset, relu_pre, relu_post, relu_scale, stream);
+}
+
+static int mi355x_fc_i8_impl(int8_t *out, const int8_t *in, const int8_t *weights_kn,
                  int8_t *weights_nk_workspace, int repack, const void *bias,
                  int bias_is_i8, size_t M, size_t K, size_t N,
                  int32_t out_offset, int32_t in_offset, int32_t weights_offset,
@@ -267,7 +329,32 @@ int mi355x_fc_i8(int8_t *out, const int8_t *in, const int8_t *weights_kn,
                    weights_offset != 0, stream);
 }
 
-int mi355x_matmul_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs_kn,
+int mi355x_fc_i8(int8_t *out, const int8_t *in, const int8_t *weights_kn,
+                 int8_t *weights_nk_workspace, int repack, const void *bias,
+                 int bias_is_i8, size_t M, size_t K, size_t N,
+                 int32_t out_offset, int32_t in_offset, int32_t weights_offset,
+                 int32_t bias_offset, int32_t bias_pre, int32_t bias_post,
+                 int32_t bias_scale, int32_t out_pre, int32_t out_post,
+                 int32_t out_scale, const int32_t *weights_row_sums,
+                 void *stream) {
+  return mi355x_fc_i8_impl(out, in, weights_kn, weights_nk_workspace, repack, bias, bias_is_i8, M, K, N, out_offset, in_offset, weights_offset, bias_offset, bias_pre, bias_post, bias_scale, out_pre, out_post, out_scale, weights_row_sums, stream);
+}
+
+int mi355x_fc_i8_opts(int8_t *out, const int8_t *in, const int8_t *weights_kn,
+                 int8_t *weights_nk_workspace, int repack, const void *bias,
+                 int bias_is_i8, size_t M, size_t K, size_t N,
+                 int32_t out_offset, int32_t in_offset, int32_t weights_offset,
+                 int32_t bias_offset, int32_t bias_pre, int32_t bias_post,
+                 int32_t bias_scale, int32_t out_pre, int32_t out_post,
+                 int32_t out_scale, const int32_t *weights_row_sums,
+                 void *stream,
+    const mi355x_launch_opts *opts) {
+  OptsScope scope(opts);
+  if (scope.rc != MI355X_OK) return scope.rc;
+  return mi355x_fc_i8_impl(out, in, weights_kn, weights_nk_workspace, repack, bias, bias_is_i8, M, K, N, out_offset, in_offset, weights_offset, bias_offset, bias_pre, bias_post, bias_scale, out_pre, out_post, out_scale, weights_row_sums, stream);
+}
+
+static int mi355x_matmul_i8_impl(int8_t *out, const int8_t *lhs, const int8_t *rhs_kn,
                      int8_t *rhs_nk_workspace, int repack, size_t M, size_t K,
                      size_t N, int32_t out_offset, int32_t lhs_offset,
                      int32_t rhs_offset, int32_t out_pre, int32_t out_post,
@@ -294,6 +381,25 @@ int mi355x_matmul_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs_kn,
   ep.act = MI355X_ACT_NONE;
   return fc_common(out, lhs, rhs_nk_workspace, ep, M, K, N, rhs_offset != 0,
                    stream);
+}
+
+int mi355x_matmul_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs_kn,
+                     int8_t *rhs_nk_workspace, int repack, size_t M, size_t K,
+                     size_t N, int32_t out_offset, int32_t lhs_offset,
+                     int32_t rhs_offset, int32_t out_pre, int32_t out_post,
+                     int32_t out_scale, void *stream) {
+  return mi355x_matmul_i8_impl(out, lhs, rhs_kn, rhs_nk_workspace, repack, M, K, N, out_offset, lhs_offset, rhs_offset, out_pre, out_post, out_scale, stream);
+}
+
+int mi355x_matmul_i8_opts(int8_t *out, const int8_t *lhs, const int8_t *rhs_kn,
+                     int8_t *rhs_nk_workspace, int repack, size_t M, size_t K,
+                     size_t N, int32_t out_offset, int32_t lhs_offset,
+                     int32_t rhs_offset, int32_t out_pre, int32_t out_post,
+                     int32_t out_scale, void *stream,
+    const mi355x_launch_opts *opts) {
+  OptsScope scope(opts);
+  if (scope.rc != MI355X_OK) return scope.rc;
+  return mi355x_matmul_i8_impl(out, lhs, rhs_kn, rhs_nk_workspace, repack, M, K, N, out_offset, lhs_offset, rhs_offset, out_pre, out_post, out_scale, stream);
 }
 
 } // extern "C"

@@ -1361,11 +1361,8 @@ static int gemm_dma_launch(const ARows &A, const DenseRows &B,
 // 128x128, which halves LDS traffic per MFMA), smaller tiles when the grid
 // would otherwise not fill 256 CUs.
 enum class Tile { T256, T128, T128x64, T64, T256x128, T128x256, T128w8 = 9, T256x128w8 = 10, T256w8 = 11 };
-// Tuning aid: a value in [0, 5] or [9, 11] forces that tile for the following
-// launches of the calling thread (w8: eight waves per workgroup instead of four).
-extern thread_local int g_tile_override;
-// Requantisation hints for the following launches of the calling thread.
-extern thread_local int g_requant_hint;
+// g_tile_override (common.h) in [0, 5] or [9, 11] forces that tile for the launch
+// being issued (w8: eight waves per workgroup instead of four).
 static Tile pick_tile(const GemmShape &g, size_t lds_256) {
   auto tiles = [&](int bm, int bn) {
     return (long long)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * g.groups;

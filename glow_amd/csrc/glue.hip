@@ -103,6 +103,82 @@ __global__ __launch_bounds__(kGlueThreads) void relu_i8_kernel(
     dst[i] = (int8_t)relu_one(src[i], so, doff, pre, post, scale);
 }
 
+// One int8 value -> one int8 value, 16 values per lane; F(v) is the operation.
+template <class F>
+__device__ __forceinline__ void map_i8(int8_t *__restrict__ dst, const int8_t *__restrict__ src,
+                                       size_t n, size_t vec_chunks, F f) {
+  const size_t t = (size_t)blockIdx.x * kGlueThreads + threadIdx.x;
+  if (t < vec_chunks) {
+    const uint4 a = reinterpret_cast<const uint4 *>(src)[t];
+    const uint32_t wa[4] = {a.x, a.y, a.z, a.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      o[j] = pack4b(f(sx8(wa[j], 0)), f(sx8(wa[j], 1)), f(sx8(wa[j], 2)), f(sx8(wa[j], 3)));
+    reinterpret_cast<uint4 *>(dst)[t] = make_uint4(o[0], o[1], o[2], o[3]);
+  }
+  const size_t stride = (size_t)gridDim.x * kGlueThreads;
+  for (size_t i = vec_chunks * 16 + t; i < n; i += stride) dst[i] = (int8_t)f((int32_t)src[i]);
+}
+
+// libjit_element_clip_i8: clip(scale(min(max(v, lo), hi) - so) + doff)
+__global__ __launch_bounds__(kGlueThreads) void clip_i8_kernel(
+    int8_t *__restrict__ dst, const int8_t *__restrict__ src, size_t n, size_t vec_chunks,
+    int32_t lo, int32_t hi, int32_t so, int32_t doff, int32_t pre, int32_t post, int32_t scale) {
+  map_i8(dst, src, n, vec_chunks, [=](int32_t v) {
+    v = min(max(v, lo), hi);
+    return clip_i8(scale_i32(v - so, pre, post, scale, doff));
+  });
+}
+
+// libjit_element_leaky_relu_i8: one rescale for values at or above the input
+// offset, another (alpha folded in) below it
+__global__ __launch_bounds__(kGlueThreads) void leaky_relu_i8_kernel(
+    int8_t *__restrict__ dst, const int8_t *__restrict__ src, size_t n, size_t vec_chunks,
+    int32_t so, int32_t doff, int32_t ppre, int32_t ppost, int32_t pscale, int32_t npre,
+    int32_t npost, int32_t nscale) {
+  map_i8(dst, src, n, vec_chunks, [=](int32_t v) {
+    const bool pos = v >= so;
+    return clip_i8(scale_i32(v - so, pos ? ppre : npre, pos ? ppost : npost,
+                             pos ? pscale : nscale, doff));
+  });
+}
+
+// libjit_element_maxsplat_kernel_i8: max(v, value)
+__global__ __launch_bounds__(kGlueThreads) void max_splat_i8_kernel(
+    int8_t *__restrict__ dst, const int8_t *__restrict__ src, size_t n, size_t vec_chunks,
+    int32_t value) {
+  map_i8(dst, src, n, vec_chunks, [=](int32_t v) { return max(v, value); });
+}
+
+// libjit_batchedadd_i8 / _i32_i8: dest[n][i] = clip(scale(batch[n][i] - bo) +
+// scale(slice[i] - so) + doff). One lane per 4 consecutive elements of a slice
+// position (slice_size % 4 == 0) or per element.
+template <class ST>
+__global__ __launch_bounds__(kGlueThreads) void batched_add_i8_kernel(
+    int8_t *__restrict__ dst, const int8_t *__restrict__ batch, const ST *__restrict__ slice,
+    size_t total, size_t slice_size, int vec4, int32_t doff, int32_t bo, int32_t so,
+    int32_t bpre, int32_t bpost, int32_t bscale, int32_t spre, int32_t spost, int32_t sscale) {
+  const size_t stride = (size_t)gridDim.x * kGlueThreads;
+  auto one = [=](int32_t b, int32_t s) {
+    const int32_t x = scale_i32((int32_t)((uint32_t)b - (uint32_t)bo), bpre, bpost, bscale, 0);
+    const int32_t y = scale_i32((int32_t)((uint32_t)s - (uint32_t)so), spre, spost, sscale, 0);
+    return clip_i8((int32_t)((uint32_t)x + (uint32_t)y + (uint32_t)doff));
+  };
+  if (vec4) {
+    for (size_t q = (size_t)blockIdx.x * kGlueThreads + threadIdx.x; q < total / 4; q += stride) {
+      const size_t i = (q * 4) % slice_size;
+      const uint32_t w = reinterpret_cast<const uint32_t *>(batch)[q];
+      reinterpret_cast<uint32_t *>(dst)[q] =
+          pack4b(one(sx8(w, 0), (int32_t)slice[i]), one(sx8(w, 1), (int32_t)slice[i + 1]),
+                 one(sx8(w, 2), (int32_t)slice[i + 2]), one(sx8(w, 3), (int32_t)slice[i + 3]));
+    }
+  } else {
+    for (size_t e = (size_t)blockIdx.x * kGlueThreads + threadIdx.x; e < total; e += stride)
+      dst[e] = (int8_t)one((int32_t)batch[e], (int32_t)slice[e % slice_size]);
+  }
+}
+
 struct PoolGeom {
   int N, IH, IW, C, OH, OW, KH, KW, SH, SW, padT, padL;
 };
@@ -677,6 +753,82 @@ int mi355x_relu_i8(int8_t *dst, const int8_t *src, size_t n, int32_t src_offset,
                      as_stream(stream), dst, src, n, chunks, src_offset, dest_offset, dest_pre,
                      dest_post, dest_scale);
   return check_launch("relu_i8");
+}
+
+int mi355x_clip_i8(int8_t *dst, const int8_t *src, size_t n, int32_t clip_min, int32_t clip_max,
+                   int32_t src_offset, int32_t dest_offset, int32_t dest_pre, int32_t dest_post,
+                   int32_t dest_scale, void *stream) {
+  if (n == 0) return MI355X_OK;
+  MI355X_REQUIRE(dst && src, "NULL tensor");
+  MI355X_REQUIRE(shifts_ok(dest_pre, dest_post), "pre/post shift outside [0, 31]");
+  MI355X_REQUIRE(src_offset >= -128 && src_offset <= 127 && dest_offset >= -128 &&
+                     dest_offset <= 127 && clip_min >= -128 && clip_min <= 127 &&
+                     clip_max >= -128 && clip_max <= 127,
+                 "offsets or clip bounds outside the int8 range");
+  MI355X_REQUIRE(n / 16 / kGlueThreads < 0x7fffffffu, "tensor too large");
+  const size_t chunks = al16(dst, src, src) ? n / 16 : 0;
+  hipLaunchKernelGGL(clip_i8_kernel, dim3(glue_blocks(chunks)), dim3(kGlueThreads), 0,
+                     as_stream(stream), dst, src, n, chunks, clip_min, clip_max, src_offset,
+                     dest_offset, dest_pre, dest_post, dest_scale);
+  return check_launch("clip_i8");
+}
+
+int mi355x_leaky_relu_i8(int8_t *dst, const int8_t *src, size_t n, int32_t src_offset,
+                         int32_t dest_offset, int32_t pos_pre, int32_t pos_post,
+                         int32_t pos_scale, int32_t neg_pre, int32_t neg_post, int32_t neg_scale,
+                         void *stream) {
+  if (n == 0) return MI355X_OK;
+  MI355X_REQUIRE(dst && src, "NULL tensor");
+  MI355X_REQUIRE(shifts_ok(pos_pre, pos_post) && shifts_ok(neg_pre, neg_post),
+                 "pre/post shift outside [0, 31]");
+  MI355X_REQUIRE(src_offset >= -128 && src_offset <= 127 && dest_offset >= -128 &&
+                     dest_offset <= 127,
+                 "offsets outside the int8 range");
+  MI355X_REQUIRE(n / 16 / kGlueThreads < 0x7fffffffu, "tensor too large");
+  const size_t chunks = al16(dst, src, src) ? n / 16 : 0;
+  hipLaunchKernelGGL(leaky_relu_i8_kernel, dim3(glue_blocks(chunks)), dim3(kGlueThreads), 0,
+                     as_stream(stream), dst, src, n, chunks, src_offset, dest_offset, pos_pre,
+                     pos_post, pos_scale, neg_pre, neg_post, neg_scale);
+  return check_launch("leaky_relu_i8");
+}
+
+int mi355x_max_splat_i8(int8_t *dst, const int8_t *src, size_t n, int32_t value, void *stream) {
+  if (n == 0) return MI355X_OK;
+  MI355X_REQUIRE(dst && src, "NULL tensor");
+  MI355X_REQUIRE(value >= -128 && value <= 127, "splat value outside the int8 range");
+  MI355X_REQUIRE(n / 16 / kGlueThreads < 0x7fffffffu, "tensor too large");
+  const size_t chunks = al16(dst, src, src) ? n / 16 : 0;
+  hipLaunchKernelGGL(max_splat_i8_kernel, dim3(glue_blocks(chunks)), dim3(kGlueThreads), 0,
+                     as_stream(stream), dst, src, n, chunks, value);
+  return check_launch("max_splat_i8");
+}
+
+int mi355x_batched_add_i8(int8_t *dst, const int8_t *batch, const void *slice, int slice_is_i32,
+                          size_t num_slices, size_t slice_size, int32_t dest_offset,
+                          int32_t batch_offset, int32_t slice_offset, int32_t batch_pre,
+                          int32_t batch_post, int32_t batch_scale, int32_t slice_pre,
+                          int32_t slice_post, int32_t slice_scale, void *stream) {
+  if (num_slices == 0 || slice_size == 0) return MI355X_OK;
+  MI355X_REQUIRE(dst && batch && slice, "NULL tensor");
+  MI355X_REQUIRE(shifts_ok(batch_pre, batch_post) && shifts_ok(slice_pre, slice_post),
+                 "pre/post shift outside [0, 31]");
+  MI355X_REQUIRE(num_slices < (1ull << 40) / slice_size, "tensor too large");
+  const size_t total = num_slices * slice_size;
+  const int vec4 = slice_size % 4 == 0 && ((((uintptr_t)dst) | ((uintptr_t)batch)) & 3) == 0;
+  const size_t work = vec4 ? total / 4 : total;
+  const size_t blocks = (work + kGlueThreads - 1) / kGlueThreads;
+  const dim3 grid((unsigned)(blocks < 65536 * 4 ? (blocks ? blocks : 1) : 65536 * 4));
+  if (slice_is_i32)
+    hipLaunchKernelGGL((batched_add_i8_kernel<int32_t>), grid, dim3(kGlueThreads), 0,
+                       as_stream(stream), dst, batch, (const int32_t *)slice, total, slice_size,
+                       vec4, dest_offset, batch_offset, slice_offset, batch_pre, batch_post,
+                       batch_scale, slice_pre, slice_post, slice_scale);
+  else
+    hipLaunchKernelGGL((batched_add_i8_kernel<int8_t>), grid, dim3(kGlueThreads), 0,
+                       as_stream(stream), dst, batch, (const int8_t *)slice, total, slice_size,
+                       vec4, dest_offset, batch_offset, slice_offset, batch_pre, batch_post,
+                       batch_scale, slice_pre, slice_post, slice_scale);
+  return check_launch("batched_add_i8");
 }
 
 int mi355x_max_pool_i8(int8_t *out, const int8_t *in, size_t N, size_t IH, size_t IW, size_t C,

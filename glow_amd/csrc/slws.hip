@@ -40,7 +40,6 @@
 #include <hip/hip_fp16.h>
 
 #include <atomic>
-#include <utility>
 #include <mutex>
 #include <vector>
 
@@ -642,7 +641,8 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_wave_kernel(SlwsArgs a) {
 // One bag per wavefront; a lane reads 4 consecutive data bytes, so a row takes
 // LPR = data_bytes/4 lanes and one load instruction fetches 64/LPR rows. The
 // partial sums of the row groups are added across lanes at the end of the bag.
-constexpr int kMathStrict = 0, kMathElement = 1, kMathRegrouped = 2;
+constexpr int kMathStrict = MI355X_SLWS_MATH_STRICT, kMathElement = MI355X_SLWS_MATH_ELEMENT,
+              kMathRegrouped = MI355X_SLWS_MATH_REGROUPED;
 
 // Cut points of the measurement entry point mi355x_frwq_slws_probe: the kernel
 // stops after the named stage and stores a value that depends on what it read.
@@ -1327,6 +1327,8 @@ static void launch_groups_kind(int kind, dim3 grid, hipStream_t st, const SlwsAr
 
 // Arithmetic of the launches that do not name one (process-wide default).
 static std::atomic<int> g_fused_math{kMathElement};
+// Arithmetic named by the call being issued on this thread (OptsScope); -1: none.
+thread_local int g_slws_math = -1;
 
 // Several tables in one launch and/or the int8 output transform.
 struct SlwsExtra {
@@ -1440,7 +1442,9 @@ static int slws_dispatch(void *dest, int out_is_f16, const uint8_t *data,
   // fused arithmetic: whole rows of 32, 64, 128 or 256 data bytes, 4-byte
   // aligned, fp32 accumulation. A multi-table launch cannot check the
   // alignment of each table here; its tables must be 4-byte aligned.
-  const int math = x.math >= 0 ? x.math : g_fused_math.load(std::memory_order_relaxed);
+  const int math = x.math >= 0     ? x.math
+                   : g_slws_math >= 0 ? g_slws_math
+                                      : g_fused_math.load(std::memory_order_relaxed);
   MI355X_REQUIRE(math >= kMathStrict && math <= kMathRegrouped,
                  "unknown SparseLengths arithmetic %d", math);
   const bool rows_ok = math != kMathStrict && !acc16 &&
@@ -1531,7 +1535,7 @@ using namespace mi355x;
 
 extern "C" {
 
-int mi355x_slws_set_fused_math(int on) {
+int mi355x_slws_set_fused_math(int on) {  // on: MI355X_SLWS_MATH_*
   MI355X_REQUIRE(on >= kMathStrict && on <= kMathRegrouped,
                  "unknown SparseLengths arithmetic %d", on);
   g_fused_math.store(on, std::memory_order_relaxed);
@@ -1559,7 +1563,7 @@ int mi355x_frwq_slws_probe(int stage, float *dest, const uint8_t *data, size_t d
                        stream, x);
 }
 
-int mi355x_frwq_sls_multi(const mi355x_sls_table *tables, size_t n_tables,
+static int mi355x_frwq_sls_multi_impl(const mi355x_sls_table *tables, size_t n_tables,
                           size_t max_data_rows, int kind, int idx_is_64,
                           size_t segments, size_t in_line_size,
                           size_t out_line_size, int out_kind, float out_scale,
@@ -1581,7 +1585,28 @@ int mi355x_frwq_sls_multi(const mi355x_sls_table *tables, size_t n_tables,
                        out_line_size, fp16_accum, stream, x);
 }
 
-int mi355x_rwq_slws(float *dest, const uint8_t *data, size_t data_rows,
+int mi355x_frwq_sls_multi(const mi355x_sls_table *tables, size_t n_tables,
+                          size_t max_data_rows, int kind, int idx_is_64,
+                          size_t segments, size_t in_line_size,
+                          size_t out_line_size, int out_kind, float out_scale,
+                          int32_t out_offset, size_t dest_row_stride,
+                          int fp16_accum, void *stream) {
+  return mi355x_frwq_sls_multi_impl(tables, n_tables, max_data_rows, kind, idx_is_64, segments, in_line_size, out_line_size, out_kind, out_scale, out_offset, dest_row_stride, fp16_accum, stream);
+}
+
+int mi355x_frwq_sls_multi_opts(const mi355x_sls_table *tables, size_t n_tables,
+                          size_t max_data_rows, int kind, int idx_is_64,
+                          size_t segments, size_t in_line_size,
+                          size_t out_line_size, int out_kind, float out_scale,
+                          int32_t out_offset, size_t dest_row_stride,
+                          int fp16_accum, void *stream,
+    const mi355x_launch_opts *opts) {
+  OptsScope scope(opts);
+  if (scope.rc != MI355X_OK) return scope.rc;
+  return mi355x_frwq_sls_multi_impl(tables, n_tables, max_data_rows, kind, idx_is_64, segments, in_line_size, out_line_size, out_kind, out_scale, out_offset, dest_row_stride, fp16_accum, stream);
+}
+
+static int mi355x_rwq_slws_impl(float *dest, const uint8_t *data, size_t data_rows,
                     const float *scales, const float *offsets, const float *weights,
                     const void *indices, int idx_is_64, size_t num_indices,
                     const int32_t *lengths, size_t segments, size_t line_size,
@@ -1596,7 +1621,26 @@ int mi355x_rwq_slws(float *dest, const uint8_t *data, size_t data_rows,
                        line_size, 0, stream, x);
 }
 
-int mi355x_frwq_slws(void *dest, int out_is_f16, const uint8_t *data,
+int mi355x_rwq_slws(float *dest, const uint8_t *data, size_t data_rows,
+                    const float *scales, const float *offsets, const float *weights,
+                    const void *indices, int idx_is_64, size_t num_indices,
+                    const int32_t *lengths, size_t segments, size_t line_size,
+                    void *stream) {
+  return mi355x_rwq_slws_impl(dest, data, data_rows, scales, offsets, weights, indices, idx_is_64, num_indices, lengths, segments, line_size, stream);
+}
+
+int mi355x_rwq_slws_opts(float *dest, const uint8_t *data, size_t data_rows,
+                    const float *scales, const float *offsets, const float *weights,
+                    const void *indices, int idx_is_64, size_t num_indices,
+                    const int32_t *lengths, size_t segments, size_t line_size,
+                    void *stream,
+    const mi355x_launch_opts *opts) {
+  OptsScope scope(opts);
+  if (scope.rc != MI355X_OK) return scope.rc;
+  return mi355x_rwq_slws_impl(dest, data, data_rows, scales, offsets, weights, indices, idx_is_64, num_indices, lengths, segments, line_size, stream);
+}
+
+static int mi355x_frwq_slws_impl(void *dest, int out_is_f16, const uint8_t *data,
                      size_t data_rows, int kind, const void *weights,
                      int weights_are_f16, const void *indices, int idx_is_64,
                      size_t num_indices, const int32_t *lengths,
@@ -1609,7 +1653,28 @@ int mi355x_frwq_slws(void *dest, int out_is_f16, const uint8_t *data,
                        out_line_size, fp16_accum, stream);
 }
 
-int mi355x_frwq_slws_noalloc(void *dest, int out_is_f16, const uint8_t *data,
+int mi355x_frwq_slws(void *dest, int out_is_f16, const uint8_t *data,
+                     size_t data_rows, int kind, const void *weights,
+                     int weights_are_f16, const void *indices, int idx_is_64,
+                     size_t num_indices, const int32_t *lengths,
+                     size_t segments, size_t in_line_size,
+                     size_t out_line_size, int fp16_accum, void *stream) {
+  return mi355x_frwq_slws_impl(dest, out_is_f16, data, data_rows, kind, weights, weights_are_f16, indices, idx_is_64, num_indices, lengths, segments, in_line_size, out_line_size, fp16_accum, stream);
+}
+
+int mi355x_frwq_slws_opts(void *dest, int out_is_f16, const uint8_t *data,
+                     size_t data_rows, int kind, const void *weights,
+                     int weights_are_f16, const void *indices, int idx_is_64,
+                     size_t num_indices, const int32_t *lengths,
+                     size_t segments, size_t in_line_size,
+                     size_t out_line_size, int fp16_accum, void *stream,
+    const mi355x_launch_opts *opts) {
+  OptsScope scope(opts);
+  if (scope.rc != MI355X_OK) return scope.rc;
+  return mi355x_frwq_slws_impl(dest, out_is_f16, data, data_rows, kind, weights, weights_are_f16, indices, idx_is_64, num_indices, lengths, segments, in_line_size, out_line_size, fp16_accum, stream);
+}
+
+static int mi355x_frwq_slws_noalloc_impl(void *dest, int out_is_f16, const uint8_t *data,
                              size_t data_rows, int kind, const void *weights,
                              int weights_are_f16, const void *indices, int idx_is_64,
                              size_t num_indices, const int32_t *lengths,
@@ -1627,7 +1692,28 @@ int mi355x_frwq_slws_noalloc(void *dest, int out_is_f16, const uint8_t *data,
                        out_line_size, fp16_accum, stream, x);
 }
 
-int mi355x_frwq_slws_offsets(void *dest, int out_is_f16, const uint8_t *data,
+int mi355x_frwq_slws_noalloc(void *dest, int out_is_f16, const uint8_t *data,
+                             size_t data_rows, int kind, const void *weights,
+                             int weights_are_f16, const void *indices, int idx_is_64,
+                             size_t num_indices, const int32_t *lengths,
+                             size_t segments, size_t in_line_size,
+                             size_t out_line_size, int fp16_accum, void *stream) {
+  return mi355x_frwq_slws_noalloc_impl(dest, out_is_f16, data, data_rows, kind, weights, weights_are_f16, indices, idx_is_64, num_indices, lengths, segments, in_line_size, out_line_size, fp16_accum, stream);
+}
+
+int mi355x_frwq_slws_noalloc_opts(void *dest, int out_is_f16, const uint8_t *data,
+                             size_t data_rows, int kind, const void *weights,
+                             int weights_are_f16, const void *indices, int idx_is_64,
+                             size_t num_indices, const int32_t *lengths,
+                             size_t segments, size_t in_line_size,
+                             size_t out_line_size, int fp16_accum, void *stream,
+    const mi355x_launch_opts *opts) {
+  OptsScope scope(opts);
+  if (scope.rc != MI355X_OK) return scope.rc;
+  return mi355x_frwq_slws_noalloc_impl(dest, out_is_f16, data, data_rows, kind, weights, weights_are_f16, indices, idx_is_64, num_indices, lengths, segments, in_line_size, out_line_size, fp16_accum, stream);
+}
+
+static int mi355x_frwq_slws_offsets_impl(void *dest, int out_is_f16, const uint8_t *data,
                              size_t data_rows, int kind, const void *weights,
                              int weights_are_f16, const void *indices, int idx_is_64,
                              size_t num_indices, const int32_t *bag_offsets,
@@ -1640,6 +1726,27 @@ int mi355x_frwq_slws_offsets(void *dest, int out_is_f16, const uint8_t *data,
                        weights_are_f16, indices, idx_is_64, num_indices, nullptr,
                        bag_offsets, 1, segments, in_line_size, out_line_size,
                        fp16_accum, stream);
+}
+
+int mi355x_frwq_slws_offsets(void *dest, int out_is_f16, const uint8_t *data,
+                             size_t data_rows, int kind, const void *weights,
+                             int weights_are_f16, const void *indices, int idx_is_64,
+                             size_t num_indices, const int32_t *bag_offsets,
+                             size_t segments, size_t in_line_size,
+                             size_t out_line_size, int fp16_accum, void *stream) {
+  return mi355x_frwq_slws_offsets_impl(dest, out_is_f16, data, data_rows, kind, weights, weights_are_f16, indices, idx_is_64, num_indices, bag_offsets, segments, in_line_size, out_line_size, fp16_accum, stream);
+}
+
+int mi355x_frwq_slws_offsets_opts(void *dest, int out_is_f16, const uint8_t *data,
+                             size_t data_rows, int kind, const void *weights,
+                             int weights_are_f16, const void *indices, int idx_is_64,
+                             size_t num_indices, const int32_t *bag_offsets,
+                             size_t segments, size_t in_line_size,
+                             size_t out_line_size, int fp16_accum, void *stream,
+    const mi355x_launch_opts *opts) {
+  OptsScope scope(opts);
+  if (scope.rc != MI355X_OK) return scope.rc;
+  return mi355x_frwq_slws_offsets_impl(dest, out_is_f16, data, data_rows, kind, weights, weights_are_f16, indices, idx_is_64, num_indices, bag_offsets, segments, in_line_size, out_line_size, fp16_accum, stream);
 }
 
 int mi355x_slws_bag_offsets_host(const int32_t *lengths, size_t segments,
@@ -1660,7 +1767,7 @@ int mi355x_slws_reserve_stream(void *stream) {
   return slws_reserve_stream(as_stream(stream));
 }
 
-int mi355x_embedding_bag_rowwise_offsets(
+static int mi355x_embedding_bag_rowwise_offsets_impl(
     void *dest, int out_is_f16, const uint8_t *data, size_t data_rows,
     int kind, const void *weights, int weights_are_f16, const int32_t *indices,
     size_t num_indices, const int32_t *offsets, size_t segments,
@@ -1675,6 +1782,27 @@ int mi355x_embedding_bag_rowwise_offsets(
                        weights_are_f16, indices, 0, num_indices, nullptr,
                        offsets, has_end_offset, segments, in_line_size,
                        out_line_size, fp16_accum, stream);
+}
+
+int mi355x_embedding_bag_rowwise_offsets(
+    void *dest, int out_is_f16, const uint8_t *data, size_t data_rows,
+    int kind, const void *weights, int weights_are_f16, const int32_t *indices,
+    size_t num_indices, const int32_t *offsets, size_t segments,
+    int has_end_offset, size_t in_line_size, size_t out_line_size,
+    int fp16_accum, void *stream) {
+  return mi355x_embedding_bag_rowwise_offsets_impl(dest, out_is_f16, data, data_rows, kind, weights, weights_are_f16, indices, num_indices, offsets, segments, has_end_offset, in_line_size, out_line_size, fp16_accum, stream);
+}
+
+int mi355x_embedding_bag_rowwise_offsets_opts(
+    void *dest, int out_is_f16, const uint8_t *data, size_t data_rows,
+    int kind, const void *weights, int weights_are_f16, const int32_t *indices,
+    size_t num_indices, const int32_t *offsets, size_t segments,
+    int has_end_offset, size_t in_line_size, size_t out_line_size,
+    int fp16_accum, void *stream,
+    const mi355x_launch_opts *opts) {
+  OptsScope scope(opts);
+  if (scope.rc != MI355X_OK) return scope.rc;
+  return mi355x_embedding_bag_rowwise_offsets_impl(dest, out_is_f16, data, data_rows, kind, weights, weights_are_f16, indices, num_indices, offsets, segments, has_end_offset, in_line_size, out_line_size, fp16_accum, stream);
 }
 
 } // extern "C"

@@ -15,7 +15,8 @@ _LIB = None
 (QUANTIZE, DEQUANTIZE, RESCALE_QUANTIZED, FULLY_CONNECTED, ROWWISE_QUANTIZED_FC,
  MATMUL, CONVOLUTION, CHANNELWISE_QUANTIZED_CONV, FRWQ_SLWS, FRWQ_SLS, ELEMENT_ADD,
  RELU, MAX_POOL, AVG_POOL, SOFTMAX, CONVERT_TO, INSERT_TENSOR, TRANSPOSE, GATHER,
- BATCH_MATMUL, SIGMOID, RWQ_SLWS, EMBEDDING_BAG_BYTE_ROWWISE_OFFSETS, COPY) = range(24)
+ BATCH_MATMUL, SIGMOID, RWQ_SLWS, EMBEDDING_BAG_BYTE_ROWWISE_OFFSETS, COPY, CLIP, LEAKY_RELU,
+ CPU_MAX_SPLAT, BATCHED_ADD) = range(28)
 ACT_NONE, ACT_RELU, ACT_CLIP, ACT_TANH, ACT_SIGMOID, ACT_LEAKY_RELU = range(6)
 
 ERROR_NAMES = ["SUCCESS", "UNKNOWN", "RUNTIME_ERROR", "RUNTIME_OUT_OF_DEVICE_MEMORY",
@@ -29,7 +30,7 @@ EXPORTS = [
     "mi355x_host_module_destroy", "mi355x_host_add_constant", "mi355x_host_add_placeholder",
     "mi355x_host_create_function", "mi355x_host_add_activation", "mi355x_host_add_view",
     "mi355x_host_add_instruction", "mi355x_host_is_op_supported", "mi355x_host_compile",
-    "mi355x_host_describe", "mi355x_host_bundle_sizes", "mi355x_host_dm_create",
+    "mi355x_host_describe", "mi355x_host_bundle_sizes", "mi355x_host_dm_create", "mi355x_host_dm_create_opts",
     "mi355x_host_dm_destroy", "mi355x_host_dm_init", "mi355x_host_dm_stop",
     "mi355x_host_dm_add_network", "mi355x_host_dm_evict_network", "mi355x_host_dm_run",
     "mi355x_host_dm_time_function", "mi355x_host_dm_maximum_memory", "mi355x_host_dm_available_memory",
@@ -58,6 +59,7 @@ def lib():
         L.mi355x_host_error_name.restype = C.c_char_p
         L.mi355x_host_module_create.restype = C.c_void_p
         L.mi355x_host_dm_create.restype = C.c_void_p
+        L.mi355x_host_dm_create_opts.restype = C.c_void_p
         L.mi355x_host_dm_maximum_memory.restype = C.c_uint64
         L.mi355x_host_dm_available_memory.restype = C.c_uint64
         _LIB = L
@@ -220,9 +222,11 @@ class DeviceManager:
     nine requests of a function compare its recordings with all branches, one
     chain and two branches; the fastest stays); -n = exactly n branches."""
 
-    def __init__(self, device=0, memory_bytes=0, use_launch_graphs=True):
-        self._h = C.c_void_p(lib().mi355x_host_dm_create(
-            device, C.c_uint64(memory_bytes), int(use_launch_graphs)))
+    def __init__(self, device=0, memory_bytes=0, use_launch_graphs=True, slws_math=-1):
+        """slws_math: arithmetic of this device manager's SparseLengths launches
+        (capi.SLWS_MATH_*; -1 = the library's default), passed with every call."""
+        self._h = C.c_void_p(lib().mi355x_host_dm_create_opts(
+            device, C.c_uint64(memory_bytes), int(use_launch_graphs), int(slws_math)))
         self._modules = []
 
     def init(self):

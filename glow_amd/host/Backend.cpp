@@ -142,6 +142,10 @@ public:
         break;
       }
       case Kind::Relu: MI355X_RETURN_IF_ERR(relu(I, out)); break;
+      case Kind::Clip:
+      case Kind::LeakyRelu:
+      case Kind::CPUMaxSplat: MI355X_RETURN_IF_ERR(elementUnary(I, out)); break;
+      case Kind::BatchedAdd: MI355X_RETURN_IF_ERR(batchedAdd(I, out)); break;
       case Kind::MaxPool: MI355X_RETURN_IF_ERR(pool(I, out, false)); break;
       case Kind::AvgPool: MI355X_RETURN_IF_ERR(pool(I, out, true)); break;
       case Kind::SoftMax: MI355X_RETURN_IF_ERR(softmax(I, out)); break;
@@ -319,7 +323,7 @@ public:
 
 private:
   static constexpr int kArity[(int)Kind::NumKinds] = {2, 2, 2, 4, 6, 3, 4, 8, 5, 4, 3, 2, 2, 2, 2,
-                                                       2, 2, 2, 3, 3, 2, 7, 5, 2};
+                                                       2, 2, 2, 3, 3, 2, 7, 5, 2, 2, 2, 2, 3};
 
   Error checkOperands(const Instruction &I) {
     CHECK_OP((int)I.kind >= 0 && (int)I.kind < (int)Kind::NumKinds, "unknown kind");
@@ -655,6 +659,94 @@ private:
          [=](const DeviceBindings &b) {
            return mi355x_relu_i8((int8_t *)d.ptr(b), (const int8_t *)s.ptr(b), n, so, doff, p.pre,
                                  p.post, p.scale, b.stream);
+         }});
+    return Error::success();
+  }
+
+  // ClipInst, LeakyReluInst and CPUMaxSplatInst on int8 (reference
+  // LLVMIRGen.cpp:1501-1590, CPULLVMIRGen.cpp:135-167).
+  Error elementUnary(const Instruction &I, MI355XFunction &out) {
+    Operand d = op(I, 0), s = op(I, 1);
+    CHECK_OP(d.ty().kind == ElemKind::Int8QTy && s.ty().kind == ElemKind::Int8QTy, "needs i8 -> i8");
+    CHECK_OP(d.ty().size() == s.ty().size(), "size mismatch");
+    const size_t n = (size_t)d.ty().size();
+    const int32_t so = s.ty().offset, doff = d.ty().offset;
+    auto q8 = [&](float x) {
+      // quantization::quantize<int8_t> with the source tensor's parameters
+      const int32_t v = quantizeI32(x, s.ty().scale, so);
+      return v < -128 ? -128 : (v > 127 ? 127 : v);
+    };
+    if (I.kind == Kind::Clip) {
+      CHECK_OP(I.fattrs.size() == 2, "Clip needs {min, max}");
+      const int32_t lo = q8(I.fattrs[0]), hi = q8(I.fattrs[1]);
+      const S32To8 p = s32to8(s.ty().scale / d.ty().scale);
+      out.launches.push_back(
+          {"mi355x_clip_i8", I.name,
+           strFormat(" n=%zu", n) + kv("clip_min", lo) + kv("clip_max", hi) + kv("src_offset", so) +
+               kv("dest_offset", doff) + kv("pre", p.pre) + kv("post", p.post) + kv("scale", p.scale),
+           [=](const DeviceBindings &b) {
+             return mi355x_clip_i8((int8_t *)d.ptr(b), (const int8_t *)s.ptr(b), n, lo, hi, so, doff,
+                                   p.pre, p.post, p.scale, b.stream);
+           }});
+      return Error::success();
+    }
+    if (I.kind == Kind::LeakyRelu) {
+      CHECK_OP(I.fattrs.size() == 1, "LeakyRelu needs {alpha}");
+      const S32To8 pp = s32to8(s.ty().scale / d.ty().scale);
+      const S32To8 np = s32to8(s.ty().scale * I.fattrs[0] / d.ty().scale);
+      out.launches.push_back(
+          {"mi355x_leaky_relu_i8", I.name,
+           strFormat(" n=%zu", n) + kv("src_offset", so) + kv("dest_offset", doff) +
+               kv("pos_pre", pp.pre) + kv("pos_post", pp.post) + kv("pos_scale", pp.scale) +
+               kv("neg_pre", np.pre) + kv("neg_post", np.post) + kv("neg_scale", np.scale),
+           [=](const DeviceBindings &b) {
+             return mi355x_leaky_relu_i8((int8_t *)d.ptr(b), (const int8_t *)s.ptr(b), n, so, doff,
+                                         pp.pre, pp.post, pp.scale, np.pre, np.post, np.scale,
+                                         b.stream);
+           }});
+      return Error::success();
+    }
+    // Max(x, Splat(v)) keeps its operand's type (the node the CPU backend makes
+    // of it has one)
+    CHECK_OP(I.fattrs.size() == 1, "CPUMaxSplat needs {splatValue}");
+    CHECK_OP(d.ty().scale == s.ty().scale && doff == so,
+             "source and destination must share scale and offset");
+    const int32_t v = q8(I.fattrs[0]);
+    out.launches.push_back({"mi355x_max_splat_i8", I.name, strFormat(" n=%zu", n) + kv("value", v),
+                            [=](const DeviceBindings &b) {
+                              return mi355x_max_splat_i8((int8_t *)d.ptr(b), (const int8_t *)s.ptr(b),
+                                                         n, v, b.stream);
+                            }});
+    return Error::success();
+  }
+
+  // BatchedAddInst on an int8 batch with an int8 or int32 slice (reference
+  // LLVMIRGen.cpp:2322-2375).
+  Error batchedAdd(const Instruction &I, MI355XFunction &out) {
+    Operand d = op(I, 0), bt = op(I, 1), sl = op(I, 2);
+    CHECK_OP(d.ty().kind == ElemKind::Int8QTy && bt.ty().kind == ElemKind::Int8QTy,
+             "needs an i8 batch and result");
+    CHECK_OP(sl.ty().kind == ElemKind::Int8QTy || sl.ty().kind == ElemKind::Int32QTy,
+             "needs an i8 or i32 slice");
+    CHECK_OP(d.ty().dims == bt.ty().dims, "batch and result differ in shape");
+    CHECK_OP(!bt.ty().dims.empty() && bt.ty().dims[0] > 0 &&
+                 sl.ty().size() * bt.ty().dims[0] == bt.ty().size(),
+             "slice %s is not one slice of batch %s", sl.ty().str().c_str(), bt.ty().str().c_str());
+    const size_t numSlice = (size_t)bt.ty().dims[0], sliceSize = (size_t)sl.ty().size();
+    const int i32 = sl.ty().kind == ElemKind::Int32QTy;
+    const S32To8 bp = s32to8(bt.ty().scale / d.ty().scale);
+    const S32To8 sp = s32to8(sl.ty().scale / d.ty().scale);
+    const int32_t doff = d.ty().offset, bo = bt.ty().offset, so = sl.ty().offset;
+    out.launches.push_back(
+        {"mi355x_batched_add_i8", I.name,
+         strFormat(" slices=%zu slice_size=%zu", numSlice, sliceSize) + kv("slice_is_i32", i32) +
+             kv("dest_offset", doff) + kv("batch_offset", bo) + kv("slice_offset", so) +
+             kv("batch_pre", bp.pre) + kv("batch_post", bp.post) + kv("batch_scale", bp.scale) +
+             kv("slice_pre", sp.pre) + kv("slice_post", sp.post) + kv("slice_scale", sp.scale),
+         [=](const DeviceBindings &b) {
+           return mi355x_batched_add_i8((int8_t *)d.ptr(b), (const int8_t *)bt.ptr(b), sl.ptr(b), i32,
+                                        numSlice, sliceSize, doff, bo, so, bp.pre, bp.post, bp.scale,
+                                        sp.pre, sp.post, sp.scale, b.stream);
          }});
     return Error::success();
   }
@@ -1228,10 +1320,10 @@ private:
              kv("out_post", opp.post) + kv("out_scale", opp.scale) + kv("bias_is_i8", bias8) +
              kv("repack", repack) + kv("row_sums", sums),
          [=](const DeviceBindings &b) {
-           return mi355x_fc_i8((int8_t *)d.ptr(b), (const int8_t *)s.ptr(b), (const int8_t *)w.ptr(b),
+           return mi355x_fc_i8_opts((int8_t *)d.ptr(b), (const int8_t *)s.ptr(b), (const int8_t *)w.ptr(b),
                                (int8_t *)work(b), repack, bi.ptr(b), bias8, M, K, N, oo, io, wo, bo,
                                bp.pre, bp.post, bp.scale, opp.pre, opp.post, opp.scale,
-                               sums ? (const int32_t *)sumPtr(b) : nullptr, b.stream);
+                               sums ? (const int32_t *)sumPtr(b) : nullptr, b.stream, &b.opts);
          }});
     return Error::success();
   }
@@ -1263,9 +1355,9 @@ private:
              kv("rhs_offset", ro) + kv("out_pre", p.pre) + kv("out_post", p.post) +
              kv("out_scale", p.scale) + kv("repack", repack),
          [=](const DeviceBindings &b) {
-           return mi355x_matmul_i8((int8_t *)d.ptr(b), (const int8_t *)l.ptr(b), (const int8_t *)r.ptr(b),
+           return mi355x_matmul_i8_opts((int8_t *)d.ptr(b), (const int8_t *)l.ptr(b), (const int8_t *)r.ptr(b),
                                    (int8_t *)work(b), repack, M, K, N, oo, lo, ro, p.pre, p.post,
-                                   p.scale, b.stream);
+                                   p.scale, b.stream, &b.opts);
          }});
     return Error::success();
   }
@@ -1337,12 +1429,12 @@ private:
                vecStr("out_post", opost) + vecStr("out_scale", oscale),
            [=](const DeviceBindings &b) {
              auto g = [&](size_t o) { return (const int32_t *)(b.generated + o); };
-             return mi355x_rwq_fc_relu_i8((int8_t *)rd.ptr(b), (const int8_t *)s.ptr(b),
+             return mi355x_rwq_fc_relu_i8_opts((int8_t *)rd.ptr(b), (const int8_t *)s.ptr(b),
                                           (const int8_t *)w.ptr(b), bi.ptr(b), bias8,
                                           (const int32_t *)of.ptr(b), g(o0), g(o1), g(o2), g(o3), g(o4),
                                           g(o5), M, K, N, oo, io, bo, allZero ? 1 : 0,
                                           sums ? (const int32_t *)sumPtr(b) : nullptr, ro, rp.pre,
-                                          rp.post, rp.scale, b.stream);
+                                          rp.post, rp.scale, b.stream, &b.opts);
            }});
       out.launches.back().requantHint = hint;
       return Error::success();
@@ -1356,10 +1448,10 @@ private:
              vecStr("out_scale", oscale),
          [=](const DeviceBindings &b) {
            auto g = [&](size_t o) { return (const int32_t *)(b.generated + o); };
-           return mi355x_rwq_fc_i8((int8_t *)d.ptr(b), (const int8_t *)s.ptr(b), (const int8_t *)w.ptr(b),
+           return mi355x_rwq_fc_i8_opts((int8_t *)d.ptr(b), (const int8_t *)s.ptr(b), (const int8_t *)w.ptr(b),
                                    bi.ptr(b), bias8, (const int32_t *)of.ptr(b), g(o0), g(o1), g(o2),
                                    g(o3), g(o4), g(o5), M, K, N, oo, io, bo, allZero ? 1 : 0,
-                                   sums ? (const int32_t *)sumPtr(b) : nullptr, b.stream);
+                                   sums ? (const int32_t *)sumPtr(b) : nullptr, b.stream, &b.opts);
          }});
     out.launches.back().requantHint = hint;
     return Error::success();
@@ -1539,10 +1631,10 @@ private:
                kv("out_scale", opp.scale) + kv("act", act) + vecStr("act_args", actArgs) +
                kv("bias_is_i8", bias8) + kv("row_sums", sums),
            [=](const DeviceBindings &b) {
-             return mi355x_conv2d_i8((int8_t *)d.ptr(b), (const int8_t *)s.ptr(b), (const int8_t *)f.ptr(b),
+             return mi355x_conv2d_i8_opts((int8_t *)d.ptr(b), (const int8_t *)s.ptr(b), (const int8_t *)f.ptr(b),
                                      bi.ptr(b), bias8, &g, oo, io, fo, bo, bp.pre, bp.post, bp.scale,
                                      opp.pre, opp.post, opp.scale, act, actArgs.data(),
-                                     sums ? (const int32_t *)sumPtr(b) : nullptr, b.stream);
+                                     sums ? (const int32_t *)sumPtr(b) : nullptr, b.stream, &b.opts);
            }});
       return Error::success();
     }
@@ -1659,12 +1751,12 @@ private:
                vecStr("out_pre", opre) + vecStr("out_post", opost) + vecStr("out_scale", oscale),
            [=](const DeviceBindings &b) {
              auto gp = [&](size_t o) { return (const int32_t *)(b.generated + o); };
-             return mi355x_cwq_conv2d_i8((int8_t *)d.ptr(b), (const int8_t *)sPtr(b),
+             return mi355x_cwq_conv2d_i8_opts((int8_t *)d.ptr(b), (const int8_t *)sPtr(b),
                                          (const int8_t *)(b.generated + f2), bi.ptr(b), bias8, &g2, oo, io,
                                          (const int32_t *)fo.ptr(b), (const int32_t *)bo.ptr(b), gp(o0),
                                          gp(o1), gp(o2), gp(o3), gp(o4), gp(o5), act, actArgs.data(),
                                          allZero ? 1 : 0, sums ? (const int32_t *)sum2(b) : nullptr,
-                                         b.stream);
+                                         b.stream, &b.opts);
            }});
       out.launches.back().requantHint = convHint(K2);
       out.launches.back().reads.push_back(priv);
@@ -1717,12 +1809,12 @@ private:
                kv("relu_scale", fa.dest_scale),
            [=](const DeviceBindings &b) {
              auto gp = [&](size_t o) { return (const int32_t *)(b.generated + o); };
-             return mi355x_cwq_conv2d_add_i8(
+             return mi355x_cwq_conv2d_add_i8_opts(
                  (int8_t *)fin.ptr(b), (const int8_t *)s.ptr(b), (const int8_t *)f.ptr(b), bi.ptr(b),
                  bias8, &g, oo, io, (const int32_t *)fo.ptr(b), (const int32_t *)bo.ptr(b), gp(o0),
                  gp(o1), gp(o2), gp(o3), gp(o4), gp(o5), act, actArgs.data(), allZero ? 1 : 0,
                  sums ? (const int32_t *)sumPtr(b) : nullptr, (const int8_t *)res.ptr(b), &fa,
-                 b.stream);
+                 b.stream, &b.opts);
            }});
       out.launches.back().requantHint = convHint(Kf);
       return Error::success();
@@ -1736,12 +1828,12 @@ private:
              vecStr("out_post", opost) + vecStr("out_scale", oscale),
          [=](const DeviceBindings &b) {
            auto gp = [&](size_t o) { return (const int32_t *)(b.generated + o); };
-           return mi355x_cwq_conv2d_i8((int8_t *)d.ptr(b), (const int8_t *)s.ptr(b),
+           return mi355x_cwq_conv2d_i8_opts((int8_t *)d.ptr(b), (const int8_t *)s.ptr(b),
                                        (const int8_t *)f.ptr(b), bi.ptr(b), bias8, &g, oo, io,
                                        (const int32_t *)fo.ptr(b), (const int32_t *)bo.ptr(b), gp(o0),
                                        gp(o1), gp(o2), gp(o3), gp(o4), gp(o5), act, actArgs.data(),
                                        allZero ? 1 : 0, sums ? (const int32_t *)sumPtr(b) : nullptr,
-                                       b.stream);
+                                       b.stream, &b.opts);
          }});
     out.launches.back().requantHint = convHint(Kf);
     return Error::success();
@@ -1772,9 +1864,9 @@ private:
                               strFormat(" rows=%zu line=%zu segments=%zu num_indices=%zu", rows, line, segs, nIdx) +
                                   kv("idx_is_64", i64),
                               [=](const DeviceBindings &b) {
-                                return mi355x_rwq_slws((float *)d.ptr(b), data.ptr(b), rows, (const float *)sc.ptr(b),
+                                return mi355x_rwq_slws_opts((float *)d.ptr(b), data.ptr(b), rows, (const float *)sc.ptr(b),
                                                        (const float *)of.ptr(b), (const float *)w.ptr(b), idx.ptr(b),
-                                                       i64, nIdx, (const int32_t *)len.ptr(b), segs, line, b.stream);
+                                                       i64, nIdx, (const int32_t *)len.ptr(b), segs, line, b.stream, &b.opts);
                               }});
       return Error::success();
     }
@@ -1793,10 +1885,10 @@ private:
                             strFormat(" rows=%zu in_line=%zu segments=%zu num_indices=%zu", rows, line, segs, nIdx) +
                                 kv("has_end_offset", hasEnd),
                             [=](const DeviceBindings &b) {
-                              return mi355x_embedding_bag_rowwise_offsets(
+                              return mi355x_embedding_bag_rowwise_offsets_opts(
                                   d.ptr(b), 0, data.ptr(b), rows, MI355X_FUSED_U8_F32, w.ptr(b), 0,
                                   (const int32_t *)idx.ptr(b), nIdx, (const int32_t *)offs.ptr(b), segs, hasEnd,
-                                  line, line - 8, 0, b.stream);
+                                  line, line - 8, 0, b.stream, &b.opts);
                             }});
     return Error::success();
   }
@@ -1945,9 +2037,9 @@ private:
              strFormat(" out_scale=%.9g", (double)g.qScale) + kv("out_offset", g.qOffset) +
              kv("fp16_accum", g.acc16) + kv("bag_offsets_from_host", (long long)nDerived),
          [=](const DeviceBindings &b) {
-           return mi355x_frwq_sls_multi((const mi355x_sls_table *)tabPtr(b), n, maxRows, g.kind, g.idx64,
+           return mi355x_frwq_sls_multi_opts((const mi355x_sls_table *)tabPtr(b), n, maxRows, g.kind, g.idx64,
                                         g.segs, pitch, g.cols, outKind, g.qScale, g.qOffset, stride,
-                                        g.acc16, b.stream);
+                                        g.acc16, b.stream, &b.opts);
          }});
     return pos - at;
   }
@@ -2026,10 +2118,10 @@ private:
                kv("weights_are_f16", w16) + kv("idx_is_64", idx64) + kv("fp16_accum", acc16) +
                " bag_offsets=host(" + len.v->name + ")",
            [=](const DeviceBindings &b) {
-             return mi355x_frwq_slws_offsets(d.ptr(b), out16, table.ptr(b), rows, kind,
+             return mi355x_frwq_slws_offsets_opts(d.ptr(b), out16, table.ptr(b), rows, kind,
                                              weighted ? (const void *)w.ptr(b) : nullptr, w16,
                                              idx.ptr(b), idx64, nIdx, (const int32_t *)offs(b), segs,
-                                             pitch, outLine, acc16 ? 1 : 0, b.stream);
+                                             pitch, outLine, acc16 ? 1 : 0, b.stream, &b.opts);
            }});
       return Error::success();
     }
@@ -2040,10 +2132,10 @@ private:
              kv("kind", kind) + kv("out_is_f16", out16) + kv("weighted", weighted) +
              kv("weights_are_f16", w16) + kv("idx_is_64", idx64) + kv("fp16_accum", acc16),
          [=](const DeviceBindings &b) {
-           return mi355x_frwq_slws(d.ptr(b), out16, table.ptr(b), rows, kind,
+           return mi355x_frwq_slws_opts(d.ptr(b), out16, table.ptr(b), rows, kind,
                                    weighted ? (const void *)w.ptr(b) : nullptr, w16, idx.ptr(b), idx64,
                                    nIdx, (const int32_t *)len.ptr(b), segs, pitch, outLine,
-                                   acc16 ? 1 : 0, b.stream);
+                                   acc16 ? 1 : 0, b.stream, &b.opts);
          }});
     return Error::success();
   }
@@ -2114,6 +2206,8 @@ bool MI355XBackend::shouldLower(Kind k) const {
   case Kind::RowwiseQuantizedFullyConnected:
   case Kind::ChannelwiseQuantizedConvolution:
   case Kind::Relu:
+  case Kind::Clip:
+  case Kind::LeakyRelu:
   case Kind::SoftMax:
     return false;
   default:
@@ -2134,12 +2228,11 @@ unsigned MI355XBackend::numDevices() {
 
 int KernelLaunch::launch(const DeviceBindings &b) const {
   if (!tunable || (tile < 0 && requantHint == 0)) return run(b);
-  mi355x_gemm_tile_override(tile);
-  mi355x_gemm_requant_hint(requantHint);
-  const int rc = run(b);
-  mi355x_gemm_requant_hint(0);
-  mi355x_gemm_tile_override(-1);
-  return rc;
+  // the launch's own tile and hint travel with the call, nothing is left set
+  DeviceBindings mine = b;
+  mine.opts.gemm_tile = tile;
+  mine.opts.requant_hint = requantHint;
+  return run(mine);
 }
 
 MI355XFunction::~MI355XFunction() { dropGraph(); }

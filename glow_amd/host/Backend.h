@@ -7,6 +7,7 @@
 #define GLOW_MI355X_HOST_BACKEND_H
 
 #include "Program.h"
+#include "glow_mi355x.h"
 
 #include <functional>
 #include <map>
@@ -26,6 +27,10 @@ struct DeviceBindings {
   uint8_t *mutableMem = nullptr;  // placeholders
   uint8_t *activations = nullptr; // one function's activations
   void *stream = nullptr;
+  // Options every launch passes to the kernel library with the call itself
+  // (the <entry>_opts forms): the device manager's SparseLengths arithmetic;
+  // KernelLaunch::launch adds the launch's own tile and requantisation hint.
+  mi355x_launch_opts opts = MI355X_LAUNCH_OPTS_INIT;
 };
 
 // PlaceholderBindings: placeholder name -> host tensor (not owned).

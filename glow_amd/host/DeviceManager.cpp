@@ -359,6 +359,7 @@ Error MI355XDeviceManager::makeResident(const Module *module, const std::string 
   mi355x_arena_ptr(fr.arena, MI355X_REGION_ACTIVATIONS, 0, &p);
   fr.bindings.activations = (uint8_t *)p;
   fr.bindings.stream = stream_;
+  fr.bindings.opts.slws_math = config_.slwsMath;
   if (!fn->generated.empty()) {
     rc = mi355x_arena_upload(fr.arena, MI355X_REGION_CONSTANTS, 0, fn->generated.data(),
                              fn->generated.size(), stream_);

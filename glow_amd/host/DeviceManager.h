@@ -40,6 +40,10 @@ struct DeviceConfig {
   // stream costs microseconds, so short side branches can lose more than they
   // overlap, and how long a launch runs depends on the request's data.
   bool autotuneBranches = true;
+  // Arithmetic of this device manager's SparseLengths launches, passed with
+  // every such call (mi355x_launch_opts::slws_math): MI355X_SLWS_MATH_*, or -1
+  // for the library's default.
+  int slwsMath = -1;
 };
 
 struct DeviceInfo {

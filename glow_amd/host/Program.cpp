@@ -102,6 +102,10 @@ const char *kindName(Kind k) {
   case Kind::RowwiseQuantizedSparseLengthsWeightedSum: return "RowwiseQuantizedSparseLengthsWeightedSum";
   case Kind::EmbeddingBagByteRowwiseOffsets: return "EmbeddingBagByteRowwiseOffsets";
   case Kind::Copy: return "Copy";
+  case Kind::Clip: return "Clip";
+  case Kind::LeakyRelu: return "LeakyRelu";
+  case Kind::CPUMaxSplat: return "CPUMaxSplat";
+  case Kind::BatchedAdd: return "BatchedAdd";
   default: return "?";
   }
 }

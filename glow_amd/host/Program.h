@@ -60,6 +60,10 @@ enum class Kind : int32_t {
   RowwiseQuantizedSparseLengthsWeightedSum, // (Dest, Data u8 [rows,cols], Scales, Offsets, Weights, Indices, Lengths)
   EmbeddingBagByteRowwiseOffsets, // (Dest, Data, Weights, Indices, Offsets); iattrs {hasEndOffset}
   Copy,                         // (Dest, Src): same bytes (what Save and Reshape lower to)
+  Clip,                         // (Dest, Src) int8; fattrs {min, max}
+  LeakyRelu,                    // (Dest, Src) int8; fattrs {alpha}
+  CPUMaxSplat,                  // (Dest, Src) int8 of one type; fattrs {splatValue}: max(x, splat)
+  BatchedAdd,                   // (Dest, Batch, Slice) int8 batch; slice int8 or int32
   NumKinds
 };
 const char *kindName(Kind k);

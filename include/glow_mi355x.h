@@ -104,6 +104,49 @@ int mi355x_stream_wait_event(void *stream, void *event);
 int mi355x_event_sync(void *event);
 int mi355x_event_elapsed_ms(void *start, void *stop, float *ms);
 
+/* ---- per-launch options ------------------------------------------------------ */
+/* Every entry point whose result bits or kernel choice can be steered has a
+ * twin <name>_opts with one more argument, `const mi355x_launch_opts *opts`,
+ * declared directly behind it; the options hold for that one call and nothing
+ * of them outlives it, so callers on one thread or on many (two device
+ * managers in a process) cannot change each other's launches. opts == NULL
+ * means the calling thread's defaults, which is also what the plain entry
+ * point uses. No counterpart in the reference, whose kernels have one form.
+ *   struct_size   sizeof(mi355x_launch_opts) (MI355X_LAUNCH_OPTS_INIT sets it)
+ *   gemm_tile     matrix-core launches (FullyConnected, MatMul, convolution):
+ *                 the workgroup tile, -1 = chosen from the problem shape. Values
+ *                 as listed at mi355x_gemm_tile_override. Results do not depend
+ *                 on it. A tile in 6..8 names one special kernel; a launch that
+ *                 kernel cannot serve fails with MI355X_ERR_NOT_SUPPORTED (a
+ *                 tuner skips the candidate) instead of running another one.
+ *   requant_hint  MI355X_REQUANT_* guarantees about the launch's constants, as
+ *                 mi355x_gemm_requant_hint_host derives them; 0 = none. A wrong
+ *                 guarantee gives wrong results, so only pass what that
+ *                 function returned for this launch's own vectors.
+ *   slws_math     arithmetic of the SparseLengths entry points, -1 = the
+ *                 default (MI355X_SLWS_MATH_ELEMENT unless
+ *                 mi355x_slws_set_fused_math changed it):
+ *                 MI355X_SLWS_MATH_STRICT    acc = acc + (s*q + o)*w with every
+ *                   operation rounded on its own, in bag order: the bits of a
+ *                   plain (no fast-math) build of libjit.cpp:1253-1276;
+ *                 MI355X_SLWS_MATH_ELEMENT   v = fma(s, q, o); acc = fma(w, v,
+ *                   acc): the same expression per element without the two
+ *                   intermediate roundings (three vector instructions per
+ *                   element instead of five); rows of 32, 64, 128 or 256 data
+ *                   bytes with fp32 accumulation, anything else runs strict;
+ *                 MI355X_SLWS_MATH_REGROUPED sum_j (w_j s_j) q_jk + sum_j w_j o_j
+ *                   (two instructions per element); its error is relative to
+ *                   the magnitude a bag adds up, not to the result, and
+ *                   exceeds 1e-5 of results that cancel: on request only. */
+enum { MI355X_SLWS_MATH_STRICT = 0, MI355X_SLWS_MATH_ELEMENT = 1, MI355X_SLWS_MATH_REGROUPED = 2 };
+typedef struct {
+  uint32_t struct_size;
+  int32_t gemm_tile;
+  int32_t requant_hint;
+  int32_t slws_math;
+} mi355x_launch_opts;
+#define MI355X_LAUNCH_OPTS_INIT { (uint32_t)sizeof(mi355x_launch_opts), -1, 0, -1 }
+
 /* ---- launch graphs ---------------------------------------------------------- */
 /* A compiled function is a fixed sequence of kernel launches on fixed
  * addresses (Glow plans all memory statically), so the sequence can be
@@ -287,6 +330,42 @@ int mi355x_add_relu_i8(int8_t *dst, const int8_t *lhs, const int8_t *rhs,
 int mi355x_relu_i8(int8_t *dst, const int8_t *src, size_t n, int32_t src_offset,
                    int32_t dest_offset, int32_t dest_pre, int32_t dest_post,
                    int32_t dest_scale, void *stream);
+/* libjit_element_clip_i8 (libjit.cpp:1865-1873), the un-lowered ClipInst on
+ * int8: clip(scale(min(max(src, clip_min), clip_max) - src_offset; destP,
+ * dest_offset)). clip_min / clip_max are the float bounds quantized with the
+ * SOURCE tensor's parameters and destP = quantizeScaleOffset32To8(srcScale /
+ * destScale) (LLVMIRGen.cpp:1501-1546). */
+int mi355x_clip_i8(int8_t *dst, const int8_t *src, size_t n, int32_t clip_min,
+                   int32_t clip_max, int32_t src_offset, int32_t dest_offset,
+                   int32_t dest_pre, int32_t dest_post, int32_t dest_scale, void *stream);
+/* libjit_element_leaky_relu_i8 (libjit.cpp:1880-1892), the un-lowered
+ * LeakyReluInst on int8: values at or above src_offset are rescaled with posP =
+ * quantizeScaleOffset32To8(srcScale / destScale), the others with negP =
+ * quantizeScaleOffset32To8(srcScale * alpha / destScale) (LLVMIRGen.cpp:1549-1590);
+ * clip(scale(src - src_offset; P, dest_offset)). */
+int mi355x_leaky_relu_i8(int8_t *dst, const int8_t *src, size_t n, int32_t src_offset,
+                         int32_t dest_offset, int32_t pos_pre, int32_t pos_post,
+                         int32_t pos_scale, int32_t neg_pre, int32_t neg_post,
+                         int32_t neg_scale, void *stream);
+/* libjit_element_maxsplat_kernel_i8 (lib/Backends/CPU/libjit_cpu/libjit_cpu.cpp:45-46),
+ * the CPU backend's CPUMaxSplatInst (Max(x, Splat(v)): a Relu that keeps its
+ * input's type): max(src, value), value = v quantized with the source
+ * tensor's parameters (CPULLVMIRGen.cpp:135-167). */
+int mi355x_max_splat_i8(int8_t *dst, const int8_t *src, size_t n, int32_t value,
+                        void *stream);
+/* libjit_batchedadd_i8 / libjit_batchedadd_i32_i8 (libjit.cpp:997-1015,
+ * 1945-1969), BatchedAddInst (what a FullyConnected lowers to behind its
+ * MatMul): dest[n][i] = clip(scale(batch[n][i] - batch_offset; batchP, 0) +
+ * scale(slice[i] - slice_offset; sliceP, 0) + dest_offset) for num_slices
+ * slices of slice_size elements; slice is int8, or int32 when slice_is_i32.
+ * batchP / sliceP = quantizeScaleOffset32To8(scale / destScale)
+ * (LLVMIRGen.cpp:2322-2375). */
+int mi355x_batched_add_i8(int8_t *dst, const int8_t *batch, const void *slice,
+                          int slice_is_i32, size_t num_slices, size_t slice_size,
+                          int32_t dest_offset, int32_t batch_offset, int32_t slice_offset,
+                          int32_t batch_pre, int32_t batch_post, int32_t batch_scale,
+                          int32_t slice_pre, int32_t slice_post, int32_t slice_scale,
+                          void *stream);
 /* libjit_max_pool_i8 (libjit.cpp:812-884, 2592-2597): NHWC int8, pads {top,
  * left}; a window with no valid tap yields out_offset. */
 int mi355x_max_pool_i8(int8_t *out, const int8_t *in, size_t N, size_t IH,
@@ -413,6 +492,16 @@ int mi355x_rwq_fc_i8(int8_t *out, const int8_t *in, const int8_t *weights,
                      int32_t out_offset, int32_t in_offset,
                      int32_t bias_offset, int weights_offsets_all_zero,
                      const int32_t *weights_row_sums, void *stream);
+int mi355x_rwq_fc_i8_opts(int8_t *out, const int8_t *in, const int8_t *weights,
+                     const void *bias, int bias_is_i8,
+                     const int32_t *weights_offsets, const int32_t *bias_pre,
+                     const int32_t *bias_post, const int32_t *bias_scale,
+                     const int32_t *out_pre, const int32_t *out_post,
+                     const int32_t *out_scale, size_t M, size_t K, size_t N,
+                     int32_t out_offset, int32_t in_offset,
+                     int32_t bias_offset, int weights_offsets_all_zero,
+                     const int32_t *weights_row_sums, void *stream,
+    const mi355x_launch_opts *opts);
 
 /* RowwiseQuantizedFullyConnected followed by a Relu instruction of its result
  * (libjit_element_relu_i8, reference libjit.cpp:1851-1858, parameters from
@@ -430,6 +519,17 @@ int mi355x_rwq_fc_relu_i8(int8_t *out, const int8_t *in, const int8_t *weights,
                           int weights_offsets_all_zero, const int32_t *weights_row_sums,
                           int32_t relu_offset, int32_t relu_pre, int32_t relu_post,
                           int32_t relu_scale, void *stream);
+int mi355x_rwq_fc_relu_i8_opts(int8_t *out, const int8_t *in, const int8_t *weights,
+                          const void *bias, int bias_is_i8,
+                          const int32_t *weights_offsets, const int32_t *bias_pre,
+                          const int32_t *bias_post, const int32_t *bias_scale,
+                          const int32_t *out_pre, const int32_t *out_post,
+                          const int32_t *out_scale, size_t M, size_t K, size_t N,
+                          int32_t fc_offset, int32_t in_offset, int32_t bias_offset,
+                          int weights_offsets_all_zero, const int32_t *weights_row_sums,
+                          int32_t relu_offset, int32_t relu_pre, int32_t relu_post,
+                          int32_t relu_scale, void *stream,
+    const mi355x_launch_opts *opts);
 
 /* libjit_fc_i8_i32 / _i8_i8 (libjit_matmul.cpp:254-280, 395-422).
  * weights_kn is [K x N] as Glow stores FullyConnected weights; the kernel
@@ -445,6 +545,15 @@ int mi355x_fc_i8(int8_t *out, const int8_t *in, const int8_t *weights_kn,
                  int32_t bias_scale, int32_t out_pre, int32_t out_post,
                  int32_t out_scale, const int32_t *weights_row_sums,
                  void *stream);
+int mi355x_fc_i8_opts(int8_t *out, const int8_t *in, const int8_t *weights_kn,
+                 int8_t *weights_nk_workspace, int repack, const void *bias,
+                 int bias_is_i8, size_t M, size_t K, size_t N,
+                 int32_t out_offset, int32_t in_offset, int32_t weights_offset,
+                 int32_t bias_offset, int32_t bias_pre, int32_t bias_post,
+                 int32_t bias_scale, int32_t out_pre, int32_t out_post,
+                 int32_t out_scale, const int32_t *weights_row_sums,
+                 void *stream,
+    const mi355x_launch_opts *opts);
 
 /* libjit_matmul_i8 (libjit_matmul.cpp:353-371). lhs [M x K], rhs_kn [K x N];
  * workspace and repack as for mi355x_fc_i8. */
@@ -453,6 +562,12 @@ int mi355x_matmul_i8(int8_t *out, const int8_t *lhs, const int8_t *rhs_kn,
                      size_t N, int32_t out_offset, int32_t lhs_offset,
                      int32_t rhs_offset, int32_t out_pre, int32_t out_post,
                      int32_t out_scale, void *stream);
+int mi355x_matmul_i8_opts(int8_t *out, const int8_t *lhs, const int8_t *rhs_kn,
+                     int8_t *rhs_nk_workspace, int repack, size_t M, size_t K,
+                     size_t N, int32_t out_offset, int32_t lhs_offset,
+                     int32_t rhs_offset, int32_t out_pre, int32_t out_post,
+                     int32_t out_scale, void *stream,
+    const mi355x_launch_opts *opts);
 
 /* Tuning aid (no counterpart in the reference): forces the workgroup tile of
  * the following matrix-core launches of the calling thread: 0 = 256x256,
@@ -547,6 +662,18 @@ int mi355x_cwq_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
                          const int32_t *act_args,
                          int filter_offsets_all_zero,
                          const int32_t *filter_row_sums, void *stream);
+int mi355x_cwq_conv2d_i8_opts(int8_t *out, const int8_t *in, const int8_t *filter,
+                         const void *bias, int bias_is_i8,
+                         const mi355x_conv_geom *geom, int32_t out_offset,
+                         int32_t in_offset, const int32_t *filter_offsets,
+                         const int32_t *bias_offsets, const int32_t *bias_pre,
+                         const int32_t *bias_post, const int32_t *bias_scale,
+                         const int32_t *out_pre, const int32_t *out_post,
+                         const int32_t *out_scale, int32_t act_type,
+                         const int32_t *act_args,
+                         int filter_offsets_all_zero,
+                         const int32_t *filter_row_sums, void *stream,
+    const mi355x_launch_opts *opts);
 
 /* NTHWC input [N,IT,IH,IW,IC], filter [OC,KT,KH,KW,IC/group], output
  * [N,OT,OH,OW,OC]; pads are {near, top, left}; the output size carries
@@ -599,6 +726,17 @@ int mi355x_cwq_conv2d_add_i8(
     const int32_t *act_args, int filter_offsets_all_zero,
     const int32_t *filter_row_sums, const int8_t *residual,
     const mi355x_fused_add *add, void *stream);
+int mi355x_cwq_conv2d_add_i8_opts(
+    int8_t *out, const int8_t *in, const int8_t *filter, const void *bias,
+    int bias_is_i8, const mi355x_conv_geom *geom, int32_t conv_offset,
+    int32_t in_offset, const int32_t *filter_offsets,
+    const int32_t *bias_offsets, const int32_t *bias_pre,
+    const int32_t *bias_post, const int32_t *bias_scale, const int32_t *out_pre,
+    const int32_t *out_post, const int32_t *out_scale, int32_t act_type,
+    const int32_t *act_args, int filter_offsets_all_zero,
+    const int32_t *filter_row_sums, const int8_t *residual,
+    const mi355x_fused_add *add, void *stream,
+    const mi355x_launch_opts *opts);
 
 /* libjit_conv2d_i8_i32 / _i8_i8 (libjit_conv.cpp:49-147, 496-528). */
 int mi355x_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
@@ -610,6 +748,16 @@ int mi355x_conv2d_i8(int8_t *out, const int8_t *in, const int8_t *filter,
                      int32_t out_scale, int32_t act_type,
                      const int32_t *act_args, const int32_t *filter_row_sums,
                      void *stream);
+int mi355x_conv2d_i8_opts(int8_t *out, const int8_t *in, const int8_t *filter,
+                     const void *bias, int bias_is_i8,
+                     const mi355x_conv_geom *geom, int32_t out_offset,
+                     int32_t in_offset, int32_t filter_offset,
+                     int32_t bias_offset, int32_t bias_pre, int32_t bias_post,
+                     int32_t bias_scale, int32_t out_pre, int32_t out_post,
+                     int32_t out_scale, int32_t act_type,
+                     const int32_t *act_args, const int32_t *filter_row_sums,
+                     void *stream,
+    const mi355x_launch_opts *opts);
 
 /* ---- fused-rowwise SparseLengths(Weighted)Sum ----------------------------------- */
 
@@ -639,6 +787,13 @@ int mi355x_frwq_slws(void *dest, int out_is_f16, const uint8_t *data,
                      size_t num_indices, const int32_t *lengths,
                      size_t segments, size_t in_line_size,
                      size_t out_line_size, int fp16_accum, void *stream);
+int mi355x_frwq_slws_opts(void *dest, int out_is_f16, const uint8_t *data,
+                     size_t data_rows, int kind, const void *weights,
+                     int weights_are_f16, const void *indices, int idx_is_64,
+                     size_t num_indices, const int32_t *lengths,
+                     size_t segments, size_t in_line_size,
+                     size_t out_line_size, int fp16_accum, void *stream,
+    const mi355x_launch_opts *opts);
 
 /* mi355x_frwq_slws with the bags given as positions instead of lengths: the
  * same operator (libjit.cpp:1253-1276; InterpreterNodes.cpp:5764-5889) for a
@@ -657,6 +812,13 @@ int mi355x_frwq_slws_offsets(void *dest, int out_is_f16, const uint8_t *data,
                              size_t num_indices, const int32_t *bag_offsets,
                              size_t segments, size_t in_line_size,
                              size_t out_line_size, int fp16_accum, void *stream);
+int mi355x_frwq_slws_offsets_opts(void *dest, int out_is_f16, const uint8_t *data,
+                             size_t data_rows, int kind, const void *weights,
+                             int weights_are_f16, const void *indices, int idx_is_64,
+                             size_t num_indices, const int32_t *bag_offsets,
+                             size_t segments, size_t in_line_size,
+                             size_t out_line_size, int fp16_accum, void *stream,
+    const mi355x_launch_opts *opts);
 
 /* Host side, no GPU call: bag_offsets[0] = 0, bag_offsets[i + 1] =
  * bag_offsets[i] + max(lengths[i], 0) (negative lengths count as empty bags,
@@ -694,18 +856,34 @@ int mi355x_frwq_slws_noalloc(void *dest, int out_is_f16, const uint8_t *data,
                              size_t num_indices, const int32_t *lengths,
                              size_t segments, size_t in_line_size,
                              size_t out_line_size, int fp16_accum, void *stream);
+int mi355x_frwq_slws_noalloc_opts(void *dest, int out_is_f16, const uint8_t *data,
+                             size_t data_rows, int kind, const void *weights,
+                             int weights_are_f16, const void *indices, int idx_is_64,
+                             size_t num_indices, const int32_t *lengths,
+                             size_t segments, size_t in_line_size,
+                             size_t out_line_size, int fp16_accum, void *stream,
+    const mi355x_launch_opts *opts);
 
-/* Arithmetic of the SparseLengths kernels (process-wide; default on).
- * On: rows of 32, 64, 128 or 256 data bytes with fp32 accumulation are summed
- * as sum_j (w_j*s_j)*q_jk + sum_j (w_j*o_j) with fused multiply-adds. The CPU
- * loop's w*(s*q+o) summed in bag order is reproduced to rounding (relative
- * error of the order of 1e-7 of sum_j |w_j|(|s_j| q + |o_j|)), which is the
- * latitude the reference's own build takes (libjit is compiled with
- * -ffast-math, reference CMakeLists.txt:21, 170-174).
- * Off: every multiply and add is rounded separately in bag order, which
- * reproduces a strict (no fast-math) build of the CPU loop bit for bit.
- * No counterpart in the reference. */
-int mi355x_slws_set_fused_math(int on);
+/* Process-wide default of mi355x_launch_opts::slws_math for the calls that do
+ * not name an arithmetic themselves (the plain entry points, and _opts calls
+ * with slws_math = -1): MI355X_SLWS_MATH_STRICT, _ELEMENT (what the library
+ * starts with) or _REGROUPED. Kept for tools that time or test one arithmetic
+ * across many calls; a caller that shares the process passes slws_math with
+ * its calls instead. No counterpart in the reference. */
+int mi355x_slws_set_fused_math(int math);
+
+/* Measurement aid (no counterpart in the reference): the uint8 / fp32
+ * SparseLengthsWeightedSum over rows of 128 columns (int64 indices, fp32
+ * weights, lengths), cut off behind one of its dependent stages, to time what
+ * a launch costs up to there. stage 0: a launch of the same shape that does
+ * nothing; 1: the bags' positions (the prefix over the lengths); 2: index and
+ * weight of every lookup; 3: scale and offset of every row; 4: every row read,
+ * no arithmetic. The output holds values that depend on what was read and
+ * nothing else of use. */
+int mi355x_frwq_slws_probe(int stage, float *dest, const uint8_t *data, size_t data_rows,
+                           const float *weights, const int64_t *indices,
+                           size_t num_indices, const int32_t *lengths, size_t segments,
+                           size_t in_line_size, void *stream);
 
 /* libjit_rowwise_quantized_sparse_lengths_weighted_sum_f_u / _f_i32 (reference
  * libjit.cpp:1232-1251, 2400-2414): the table holds uint8 rows of line_size
@@ -716,6 +894,12 @@ int mi355x_rwq_slws(float *dest, const uint8_t *data, size_t data_rows,
                     const void *indices, int idx_is_64, size_t num_indices,
                     const int32_t *lengths, size_t segments, size_t line_size,
                     void *stream);
+int mi355x_rwq_slws_opts(float *dest, const uint8_t *data, size_t data_rows,
+                    const float *scales, const float *offsets, const float *weights,
+                    const void *indices, int idx_is_64, size_t num_indices,
+                    const int32_t *lengths, size_t segments, size_t line_size,
+                    void *stream,
+    const mi355x_launch_opts *opts);
 
 /* FusedRowwiseQuantizedSparseLengthsSum over several tables of one shape in ONE
  * launch (a ranking model pools dozens of tables per request, each too small
@@ -753,6 +937,13 @@ int mi355x_frwq_sls_multi(const mi355x_sls_table *tables, size_t n_tables,
                           size_t out_line_size, int out_kind, float out_scale,
                           int32_t out_offset, size_t dest_row_stride,
                           int fp16_accum, void *stream);
+int mi355x_frwq_sls_multi_opts(const mi355x_sls_table *tables, size_t n_tables,
+                          size_t max_data_rows, int kind, int idx_is_64,
+                          size_t segments, size_t in_line_size,
+                          size_t out_line_size, int out_kind, float out_scale,
+                          int32_t out_offset, size_t dest_row_stride,
+                          int fp16_accum, void *stream,
+    const mi355x_launch_opts *opts);
 
 /* libjit_embedding_bag_byte_rowwise_offsets_f (libjit.cpp:2454-2481) and the
  * Interpreter's 4-bit / fp16 twin: bags are given by int32 start offsets
@@ -764,6 +955,13 @@ int mi355x_embedding_bag_rowwise_offsets(
     size_t num_indices, const int32_t *offsets, size_t segments,
     int has_end_offset, size_t in_line_size, size_t out_line_size,
     int fp16_accum, void *stream);
+int mi355x_embedding_bag_rowwise_offsets_opts(
+    void *dest, int out_is_f16, const uint8_t *data, size_t data_rows,
+    int kind, const void *weights, int weights_are_f16, const int32_t *indices,
+    size_t num_indices, const int32_t *offsets, size_t segments,
+    int has_end_offset, size_t in_line_size, size_t out_line_size,
+    int fp16_accum, void *stream,
+    const mi355x_launch_opts *opts);
 
 #ifdef __cplusplus
 }

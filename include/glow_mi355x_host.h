@@ -150,6 +150,12 @@ int mi355x_host_bundle_sizes(mi355x_host_module *m, int function, uint64_t out[4
  * chain and with two branches, and the fastest serves the requests after
  * them. n < 0 = exactly -n branches (-1 = a chain), nothing compared. */
 mi355x_host_dm *mi355x_host_dm_create(int device, uint64_t memory_bytes, int use_launch_graphs);
+/* The same with DeviceConfig::slwsMath: the arithmetic this device manager's
+ * SparseLengths launches ask for with every call (MI355X_SLWS_MATH_*; -1 = the
+ * library's default). Each device manager passes its own setting explicitly, so
+ * several of them in one process do not influence one another. */
+mi355x_host_dm *mi355x_host_dm_create_opts(int device, uint64_t memory_bytes,
+                                           int use_launch_graphs, int slws_math);
 void mi355x_host_dm_destroy(mi355x_host_dm *dm);
 int mi355x_host_dm_init(mi355x_host_dm *dm);
 int mi355x_host_dm_stop(mi355x_host_dm *dm);

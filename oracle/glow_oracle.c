@@ -873,6 +873,54 @@ void go_relu_i8(int8_t *dest, const int8_t *src, size_t n, int8_t srcOffset,
   }
 }
 
+/* libjit.cpp:1865-1873 */
+void go_clip_elem_i8(int8_t *dest, const int8_t *src, size_t n, int8_t clipMin, int8_t clipMax,
+                     int8_t srcOffset, int8_t destOffset, int32_t destPre, int32_t destPost,
+                     int32_t destScale) {
+  for (size_t i = 0; i < n; i++) {
+    int32_t v = src[i] > clipMin ? src[i] : clipMin;
+    v = v < clipMax ? v : clipMax;
+    dest[i] = go_clip_i8(go_scale_i32(v - srcOffset, destPre, destPost, destScale, destOffset));
+  }
+}
+
+/* libjit.cpp:1880-1892 */
+void go_leaky_relu_i8(int8_t *dest, const int8_t *src, size_t n, int8_t srcOffset,
+                      int8_t destOffset, int32_t posPre, int32_t posPost, int32_t posScale,
+                      int32_t negPre, int32_t negPost, int32_t negScale) {
+  for (size_t i = 0; i < n; i++) {
+    const int32_t v = src[i];
+    dest[i] = go_clip_i8(v >= srcOffset
+                             ? go_scale_i32(v - srcOffset, posPre, posPost, posScale, destOffset)
+                             : go_scale_i32(v - srcOffset, negPre, negPost, negScale, destOffset));
+  }
+}
+
+/* lib/Backends/CPU/libjit_cpu/libjit_cpu.cpp:45-46 */
+void go_max_splat_i8(int8_t *dest, const int8_t *src, size_t n, int8_t value) {
+  for (size_t i = 0; i < n; i++) dest[i] = src[i] > value ? src[i] : value;
+}
+
+/* libjit.cpp:997-1015 (libjit_batchedadd_i8 and _i32_i8, :1945-1969); the
+ * subtraction and the sum wrap in 32 bits like the compiled reference */
+void go_batched_add_i8(int8_t *dest, const int8_t *batch, const void *slice, int sliceIsI32,
+                       size_t numSlice, size_t sliceSize, int32_t destOffset,
+                       int32_t batchOffset, int32_t sliceOffset, int32_t batchPre,
+                       int32_t batchPost, int32_t batchScale, int32_t slicePre,
+                       int32_t slicePost, int32_t sliceScale) {
+  for (size_t n = 0; n < numSlice; n++) {
+    const size_t base = n * sliceSize;
+    for (size_t i = 0; i < sliceSize; i++) {
+      const int32_t sv = sliceIsI32 ? ((const int32_t *)slice)[i] : ((const int8_t *)slice)[i];
+      const int32_t b = (int32_t)((uint32_t)batch[base + i] - (uint32_t)batchOffset);
+      const int32_t s = (int32_t)((uint32_t)sv - (uint32_t)sliceOffset);
+      const int32_t x = go_scale_i32(b, batchPre, batchPost, batchScale, 0);
+      const int32_t y = go_scale_i32(s, slicePre, slicePost, sliceScale, 0);
+      dest[base + i] = go_clip_i8((int32_t)((uint32_t)x + (uint32_t)y + (uint32_t)destOffset));
+    }
+  }
+}
+
 /* window limits of libjit_defs.h:257-275 */
 static void window(ptrdiff_t inMin, size_t inSize, size_t k, ptrdiff_t *lo, ptrdiff_t *len) {
   const ptrdiff_t fmin = inMin < 0 ? -inMin : 0;

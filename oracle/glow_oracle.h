@@ -264,6 +264,22 @@ void go_add_i8(int8_t *dest, const int8_t *lhs, const int8_t *rhs, size_t n,
                int32_t destOffset, int32_t lhsOffset, int32_t rhsOffset,
                int32_t lhsPre, int32_t lhsPost, int32_t lhsScale,
                int32_t rhsPre, int32_t rhsPost, int32_t rhsScale);
+/* libjit_element_clip_i8 (libjit.cpp:1865-1873) over n. */
+void go_clip_elem_i8(int8_t *dest, const int8_t *src, size_t n, int8_t clipMin, int8_t clipMax,
+                     int8_t srcOffset, int8_t destOffset, int32_t destPre, int32_t destPost,
+                     int32_t destScale);
+/* libjit_element_leaky_relu_i8 (libjit.cpp:1880-1892) over n. */
+void go_leaky_relu_i8(int8_t *dest, const int8_t *src, size_t n, int8_t srcOffset,
+                      int8_t destOffset, int32_t posPre, int32_t posPost, int32_t posScale,
+                      int32_t negPre, int32_t negPost, int32_t negScale);
+/* libjit_element_maxsplat_kernel_i8 (libjit_cpu.cpp:45-46) over n. */
+void go_max_splat_i8(int8_t *dest, const int8_t *src, size_t n, int8_t value);
+/* libjit_batchedadd_i8 / _i32_i8 (libjit.cpp:997-1015, 1945-1969). */
+void go_batched_add_i8(int8_t *dest, const int8_t *batch, const void *slice, int sliceIsI32,
+                       size_t numSlice, size_t sliceSize, int32_t destOffset,
+                       int32_t batchOffset, int32_t sliceOffset, int32_t batchPre,
+                       int32_t batchPost, int32_t batchScale, int32_t slicePre,
+                       int32_t slicePost, int32_t sliceScale);
 /* libjit_element_relu_i8 (libjit.cpp:1851-1858) over n. */
 void go_relu_i8(int8_t *dest, const int8_t *src, size_t n, int8_t srcOffset,
                 int8_t destOffset, int32_t destPre, int32_t destPost,

@@ -501,6 +501,51 @@ def relu_i8(src, src_offset, dest_offset, destP):
     return out
 
 
+def clip_elem_i8(src, clip_min, clip_max, src_offset, dest_offset, destP):
+    """libjit_element_clip_i8 over a tensor."""
+    src = _c(src, np.int8)
+    out = np.empty(src.shape, np.int8)
+    lib().go_clip_elem_i8(_p(out), _p(src), C.c_size_t(src.size), C.c_int8(clip_min),
+                          C.c_int8(clip_max), C.c_int8(src_offset), C.c_int8(dest_offset),
+                          *[C.c_int32(int(v)) for v in destP])
+    return out
+
+
+def leaky_relu_i8(src, src_offset, dest_offset, posP, negP):
+    """libjit_element_leaky_relu_i8 over a tensor."""
+    src = _c(src, np.int8)
+    out = np.empty(src.shape, np.int8)
+    lib().go_leaky_relu_i8(_p(out), _p(src), C.c_size_t(src.size), C.c_int8(src_offset),
+                           C.c_int8(dest_offset), *[C.c_int32(int(v)) for v in posP],
+                           *[C.c_int32(int(v)) for v in negP])
+    return out
+
+
+def max_splat_i8(src, value):
+    """libjit_element_maxsplat_kernel_i8 over a tensor."""
+    src = _c(src, np.int8)
+    out = np.empty(src.shape, np.int8)
+    lib().go_max_splat_i8(_p(out), _p(src), C.c_size_t(src.size), C.c_int8(value))
+    return out
+
+
+def batched_add_i8(batch, slice_, dest_offset, batch_offset, slice_offset, batchP, sliceP):
+    """libjit_batchedadd_i8 (int8 slice) / libjit_batchedadd_i32_i8 (int32 slice):
+    batch [numSlice x ...], slice [...]."""
+    batch = _c(batch, np.int8)
+    slice_ = np.ascontiguousarray(slice_)
+    i32 = slice_.dtype == np.int32
+    if not i32:
+        slice_ = _c(slice_, np.int8)
+    out = np.empty(batch.shape, np.int8)
+    lib().go_batched_add_i8(_p(out), _p(batch), _p(slice_), C.c_int(int(i32)),
+                            C.c_size_t(batch.shape[0]), C.c_size_t(slice_.size),
+                            C.c_int32(dest_offset), C.c_int32(batch_offset),
+                            C.c_int32(slice_offset), *[C.c_int32(int(v)) for v in batchP],
+                            *[C.c_int32(int(v)) for v in sliceP])
+    return out
+
+
 def pool_out_dims(IH, IW, kernel, stride, pads):
     """pads = (top, left, bottom, right)."""
     OH = (IH + pads[0] + pads[2] - kernel[0]) // stride[0] + 1

@@ -16,7 +16,10 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 
 
 def path(fastmath=False):
-    name = "libjit_ref_fastmath.so" if fastmath else "libjit_ref.so"
+    """fastmath: False = plain build, True = the reference's default fast-math
+    flags, "fma" = those flags on a host with fused multiply-add (-mfma)."""
+    name = {False: "libjit_ref.so", True: "libjit_ref_fastmath.so",
+            "fma": "libjit_ref_fma.so"}[fastmath]
     return os.path.join(_HERE, "_ref", name)
 
 
@@ -316,6 +319,54 @@ def relu_i8(src, src_offset, dest_offset, destP, fastmath=False):
     ps = src.ctypes.data
     return np.array([f(i, ps, src_offset, dest_offset, *[int(v) for v in destP])
                      for i in range(src.size)], np.int8)
+
+
+def clip_elem_i8(src, clip_min, clip_max, src_offset, dest_offset, destP, fastmath=False):
+    src = _c(src, np.int8).ravel()
+    f = lib(fastmath).libjit_element_clip_i8
+    f.restype = C.c_int8
+    f.argtypes = [C.c_uint64, C.c_void_p] + [C.c_int8] * 4 + [C.c_int32] * 3
+    ps = src.ctypes.data
+    return np.array([f(i, ps, clip_min, clip_max, src_offset, dest_offset,
+                       *[int(v) for v in destP]) for i in range(src.size)], np.int8)
+
+
+def leaky_relu_i8(src, src_offset, dest_offset, posP, negP, fastmath=False):
+    src = _c(src, np.int8).ravel()
+    f = lib(fastmath).libjit_element_leaky_relu_i8
+    f.restype = C.c_int8
+    f.argtypes = [C.c_uint64, C.c_void_p, C.c_int8, C.c_int8] + [C.c_int32] * 6
+    ps = src.ctypes.data
+    return np.array([f(i, ps, src_offset, dest_offset, *[int(v) for v in posP],
+                       *[int(v) for v in negP]) for i in range(src.size)], np.int8)
+
+
+def max_splat_i8(src, value, fastmath=False):
+    """libjit_element_maxsplat_kernel_i8 of the CPU backend's own kernel file
+    (lib/Backends/CPU/libjit_cpu/libjit_cpu.cpp)."""
+    src = _c(src, np.int8).ravel()
+    f = lib(fastmath).libjit_element_maxsplat_kernel_i8
+    f.restype = C.c_int8
+    f.argtypes = [C.c_uint64, C.c_int8, C.c_void_p, C.c_void_p]
+    ps = src.ctypes.data
+    return np.array([f(i, value, ps, None) for i in range(src.size)], np.int8)
+
+
+def batched_add_i8(batch, slice_, dest_offset, batch_offset, slice_offset, batchP, sliceP,
+                   fastmath=False):
+    batch = _c(batch, np.int8)
+    slice_ = np.ascontiguousarray(slice_)
+    if slice_.dtype == np.int32:
+        f = lib(fastmath).libjit_batchedadd_i32_i8
+    else:
+        slice_ = _c(slice_, np.int8)
+        f = lib(fastmath).libjit_batchedadd_i8
+    f.restype = None
+    f.argtypes = [C.c_void_p] * 3 + [C.c_uint64] * 2 + [C.c_int32] * 9
+    out = np.empty(batch.shape, np.int8)
+    f(_p(out), _p(batch), _p(slice_), batch.shape[0], slice_.size, dest_offset, batch_offset,
+      slice_offset, *[int(v) for v in batchP], *[int(v) for v in sliceP])
+    return out
 
 
 def _pool_dims(x, kernel, stride, pads):

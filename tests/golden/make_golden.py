@@ -71,6 +71,20 @@ def glue():
     save("glue", **gl)
 
 
+def element_ops():
+    """Clip, LeakyRelu, Max(x, Splat) and BatchedAdd on int8: inputs, integer
+    parameters and what the compiled reference returns for them."""
+    el = {}
+    names = []
+    for name, fn, args in cases.element_op_cases():
+        names.append(f"{name}:{fn}")
+        for k, v in enumerate(args):
+            el[f"{name}_arg{k}"] = np.asarray(v)
+        el[f"{name}_out"] = np.asarray(getattr(ref, fn)(*args)).reshape(np.asarray(args[0]).shape)
+    el["names"] = np.array(names)
+    save("element_ops", **el)
+
+
 WIDE_CONV3D = [
     ("relu3", dict(N=2, T=4, H=5, W=6, IC=8, OC=8)),
     ("stride_group", dict(N=1, T=5, H=7, W=6, IC=8, OC=12, kernel=(2, 3, 1), stride=(2, 1, 2),
@@ -218,4 +232,9 @@ def main():
 
 
 if __name__ == "__main__":
-    main()
+    if len(sys.argv) > 1:      # only the named files: python make_golden.py element_ops
+        for what in sys.argv[1:]:
+            globals()[what]()
+    else:
+        main()
+        element_ops()

@@ -93,6 +93,22 @@ def glue():
     return out, d["logits"], d["softmax_out"]
 
 
+def element_ops():
+    """Golden Clip / LeakyRelu / Max(x, Splat) / BatchedAdd cases. Yields
+    (name, function name in the oracle wrappers' naming, args, want)."""
+    d = _load("element_ops")
+    for entry in d["names"]:
+        name, fn = str(entry).split(":")
+        args = []
+        k = 0
+        while f"{name}_arg{k}" in d:
+            v = d[f"{name}_arg{k}"]
+            args.append(v if v.ndim and v.size > 3 else
+                        (tuple(int(x) for x in v) if v.ndim else int(v)))
+            k += 1
+        yield name, fn, tuple(args), d[f"{name}_out"]
+
+
 def wide():
     """The 16/32-bit elementwise vectors, transposes and 3-D convolutions."""
     return _load("wide")

@@ -72,6 +72,23 @@ def run(net, inputs):
                           _s(_f(t[1].scale) / _f(d.scale)), _s(_f(t[2].scale) / _f(d.scale)))
         elif o.kind == H.RELU:
             r = go.relu_i8(a[1], t[1].offset, d.offset, _s(_f(t[1].scale) / _f(d.scale)))
+        elif o.kind == H.CLIP:
+            # bounds quantized with the source tensor's parameters (LLVMIRGen.cpp:1515-1518)
+            lo, hi = (int(np.clip(go.quantize_value_i32(x, t[1].scale, t[1].offset), -128, 127))
+                      for x in o.fattrs)
+            r = go.clip_elem_i8(a[1], lo, hi, t[1].offset, d.offset,
+                                _s(_f(t[1].scale) / _f(d.scale)))
+        elif o.kind == H.LEAKY_RELU:
+            r = go.leaky_relu_i8(a[1], t[1].offset, d.offset, _s(_f(t[1].scale) / _f(d.scale)),
+                                 _s(_f(t[1].scale) * _f(o.fattrs[0]) / _f(d.scale)))
+        elif o.kind == H.CPU_MAX_SPLAT:
+            val = int(np.clip(go.quantize_value_i32(o.fattrs[0], t[1].scale, t[1].offset),
+                              -128, 127))
+            r = go.max_splat_i8(a[1], val)
+        elif o.kind == H.BATCHED_ADD:
+            r = go.batched_add_i8(a[1], a[2], d.offset, t[1].offset, t[2].offset,
+                                  _s(_f(t[1].scale) / _f(d.scale)),
+                                  _s(_f(t[2].scale) / _f(d.scale)))
         elif o.kind == H.MAX_POOL:
             k = o.iattrs
             r = go.max_pool_i8(a[1], k[0:2], k[2:4], k[4:8], d.offset)

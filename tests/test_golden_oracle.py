@@ -108,3 +108,13 @@ def test_cwq_conv3d_golden():
         np.testing.assert_array_equal(go.cwq_conv3d_i8(*args), want)
         n += 1
     assert n == 4
+
+
+def test_element_ops_golden():
+    """Clip, LeakyRelu, Max(x, Splat) and BatchedAdd against what the compiled
+    reference produced (tests/golden/element_ops.npz)."""
+    n = 0
+    for name, fn, args, want in gio.element_ops():
+        np.testing.assert_array_equal(getattr(go, fn)(*args), want, err_msg=name)
+        n += 1
+    assert n >= 19

@@ -10,7 +10,7 @@ import pytest
 
 from glow_amd import capi
 from oracle import glow_oracle as go
-from tests import cases
+from tests import cases, tiles
 
 pytestmark = pytest.mark.gpu
 
@@ -46,7 +46,7 @@ HALO_CASES = [
     dict(N=2, H=11, W=12, OC=64, pads=(2, 0, 1, 3)),            # uneven padding
     dict(N=1, H=3, W=3, OC=64, pads=(1, 1, 1, 1)),              # a single small tile
     dict(N=1, H=4, W=256, OC=64),                               # the widest row the kernel takes
-    dict(N=1, H=3, W=257, OC=64),                               # wider: the implicit GEMM serves it
+    dict(N=1, H=3, W=257, OC=64, served=False),                 # wider: refused, the implicit GEMM serves it
     dict(N=2, H=300, W=1, OC=64),                               # tall and thin: 256 rows per tile
     dict(N=300, H=9, W=9, OC=64),                               # more tiles than resident workgroups
     dict(N=5, H=7, W=7, OC=128, in_offset=0, act=go.ACT_NONE),  # no input offset, no row sums used
@@ -59,10 +59,16 @@ HALO_CASES = [
 def test_halo_conv_vs_oracle(kw):
     kw = dict(kw)
     kw.setdefault("in_offset", -128)
+    served = kw.pop("served", True)
     c = cases.cwq_conv_case(17, IC=64, **kw)
     g = c["geom"]
     say("halo conv", kw, "output", g.OH, "x", g.OW)
     want = go.cwq_conv2d_i8(*cases.cwq_conv_args(c))
+    if not served:
+        # the kernel refuses the shape; the shape rule runs the implicit GEMM
+        assert tiles.refused(7, lambda: capi.cwq_conv2d_i8(*cases.cwq_conv_args(c)))
+        np.testing.assert_array_equal(capi.cwq_conv2d_i8(*cases.cwq_conv_args(c)), want)
+        return
     with forced_tile(7):
         got = capi.cwq_conv2d_i8(*cases.cwq_conv_args(c))
     np.testing.assert_array_equal(got, want)
@@ -89,17 +95,19 @@ def test_halo_conv_vs_oracle(kw):
                                       go.conv2d_i8(*args))
 
 
-def test_halo_conv_is_not_used_where_it_cannot_run():
+def test_halo_conv_refuses_what_it_cannot_run():
     """Filter offsets (the kernel would need input row sums), missing filter row
-    sums, other channel counts, strides or dilations: tile 7 is ignored."""
+    sums, other channel counts, strides or dilations: asked for by number (tile
+    7) the kernel refuses the launch, and the shape rule runs another one."""
     for kw, sums in ((dict(IC=64, symmetric=False), True), (dict(IC=64), False),
                      (dict(IC=32), True), (dict(IC=64, stride=(2, 2)), True),
                      (dict(IC=64, dilation=(2, 2), pads=(2, 2, 2, 2)), True),
                      (dict(IC=128, group=2), True)):
         c = cases.cwq_conv_case(19, 2, 12, 12, OC=64, in_offset=-9, **kw)
         want = go.cwq_conv2d_i8(*cases.cwq_conv_args(c))
-        with forced_tile(7):
-            got = capi.cwq_conv2d_i8(*cases.cwq_conv_args(c), precomputed_sums=sums)
+        assert tiles.refused(7, lambda: capi.cwq_conv2d_i8(*cases.cwq_conv_args(c),
+                                                           precomputed_sums=sums))
+        got = capi.cwq_conv2d_i8(*cases.cwq_conv_args(c), precomputed_sums=sums)
         np.testing.assert_array_equal(got, want)
 
 

@@ -12,7 +12,7 @@ import pytest
 
 from glow_amd import capi
 from oracle import glow_oracle as go
-from tests import cases
+from tests import cases, tiles
 
 pytestmark = pytest.mark.gpu
 
@@ -50,7 +50,7 @@ WIDE_CASES = [
     dict(IC=512, N=1, H=14, W=14, OC=64),                        # LDS allows nine rows: two tiles of seven
     dict(IC=128, N=1, H=4, W=256, OC=64),                        # the widest row the kernel takes
     dict(IC=256, N=1, H=3, W=40, OC=64),                         # 120 pixels: four waves, the fewest
-    dict(IC=128, N=1, H=5, W=5, OC=64),                          # too few pixels: the implicit GEMM serves it
+    dict(IC=128, N=1, H=5, W=5, OC=64, served=False),            # too few pixels: refused, the implicit GEMM serves it
     dict(IC=256, N=2, H=14, W=14, OC=64, in_offset=0, act=go.ACT_NONE),
     dict(IC=128, N=1, H=28, W=28, OC=64, in_offset=7, out_offset=5, act=go.ACT_CLIP),
     dict(IC=256, N=1, H=14, W=14, OC=64, act=go.ACT_LEAKY_RELU, out_offset=10, bias_i8=True),
@@ -61,10 +61,15 @@ WIDE_CASES = [
 def test_wide_halo_conv_vs_oracle(kw):
     kw = dict(kw)
     kw.setdefault("in_offset", -128)
+    served = kw.pop("served", True)
     c = cases.cwq_conv_case(23, **kw)
     g = c["geom"]
     say("wide halo conv", kw, "output", g.OH, "x", g.OW)
     want = go.cwq_conv2d_i8(*cases.cwq_conv_args(c))
+    if not served:
+        assert tiles.refused(7, lambda: capi.cwq_conv2d_i8(*cases.cwq_conv_args(c)))
+        np.testing.assert_array_equal(capi.cwq_conv2d_i8(*cases.cwq_conv_args(c)), want)
+        return
     with forced_tile(7):
         got = capi.cwq_conv2d_i8(*cases.cwq_conv_args(c))
     np.testing.assert_array_equal(got, want)
@@ -136,5 +141,10 @@ def test_wide_halo_conv_random_geometry(seed):
         pytest.skip("empty output")
     say("wide halo conv", kw, "output", g.OH, "x", g.OW)
     want = go.cwq_conv2d_i8(*cases.cwq_conv_args(c))
-    with forced_tile(7):
-        np.testing.assert_array_equal(capi.cwq_conv2d_i8(*cases.cwq_conv_args(c)), want)
+    got = tiles.forced_or_refused(7, lambda: capi.cwq_conv2d_i8(*cases.cwq_conv_args(c)))
+    if got is None:
+        # the kernel refuses the shape (too few pixels for four waves, a patch
+        # that does not fit LDS): what the shape rule picks must serve it
+        say("  refused by the kernel; served by the shape rule's choice")
+        got = capi.cwq_conv2d_i8(*cases.cwq_conv_args(c))
+    np.testing.assert_array_equal(got, want)

@@ -10,7 +10,7 @@ import pytest
 
 from glow_amd import capi
 from oracle import glow_oracle as go
-from tests import cases
+from tests import cases, tiles
 
 pytestmark = pytest.mark.gpu
 
@@ -71,17 +71,20 @@ def test_stream_fc_vs_oracle(shape):
                                       go.rwq_fc_i8(*cases.rwq_fc_args(c2)))
 
 
-def test_stream_is_ignored_where_it_cannot_run():
+def test_stream_refuses_what_it_cannot_run():
     """Weight offsets (row sums of A would be needed), other K, sums not
-    precomputed: tile 8 falls through to the tiled kernels."""
-    for K, kw, sums in ((64, dict(symmetric=False), True), (192, dict(), True), (64, dict(), False),
+    precomputed: asked for by number (tile 8) the kernel refuses the launch,
+    and the shape rule runs the tiled kernels."""
+    for K, kw, sums in ((64, dict(symmetric=False), True), (192, dict(), True),
+                        (64, dict(in_offset=5), False),   # an input offset needs the row sums
                         (320, dict(), True)):
         c = cases.rwq_fc_case(850 + K, 100, K, 64, **kw)
         if kw.get("symmetric", True):
             c["w_offsets"][:] = 0
         want = go.rwq_fc_i8(*cases.rwq_fc_args(c))
-        with forced_tile(8):
-            got = capi.rwq_fc_i8(*cases.rwq_fc_args(c), precomputed_sums=sums)
+        assert tiles.refused(8, lambda: capi.rwq_fc_i8(*cases.rwq_fc_args(c),
+                                                       precomputed_sums=sums))
+        got = capi.rwq_fc_i8(*cases.rwq_fc_args(c), precomputed_sums=sums)
         np.testing.assert_array_equal(got, want)
 
 

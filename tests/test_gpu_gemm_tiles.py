@@ -18,7 +18,7 @@ import pytest
 
 from glow_amd import capi
 from oracle import glow_oracle as go
-from tests import cases
+from tests import cases, tiles
 
 pytestmark = pytest.mark.gpu
 
@@ -77,11 +77,19 @@ def test_rwq_fc_long_k_on_every_tile(tile, K):
     for variant in ("symmetric", "asymmetric", "asymmetric_bias8", "no_offsets"):
         c, want = _fc_case(K, variant)
         say("rwq_fc tile", TILES[tile], "K", K, variant, c["x"].shape, c["w"].shape)
-        with forced_tile(tile):
-            got = capi.rwq_fc_i8(*cases.rwq_fc_args(c))
-            got_own_sums = capi.rwq_fc_i8(*cases.rwq_fc_args(c), precomputed_sums=False)
-        np.testing.assert_array_equal(got, want)
-        np.testing.assert_array_equal(got_own_sums, want)
+        # the split-K kernel (tile 6) refuses weight offsets and missing row sums
+        got = tiles.forced_or_refused(tile, lambda: capi.rwq_fc_i8(*cases.rwq_fc_args(c)))
+        got_own_sums = tiles.forced_or_refused(
+            tile, lambda: capi.rwq_fc_i8(*cases.rwq_fc_args(c), precomputed_sums=False))
+        assert tile == 6 or (got is not None and got_own_sums is not None)
+        if tile == 6:
+            assert (got is not None) == (variant in ("symmetric", "no_offsets"))
+            # without precomputed row sums it runs only where none are needed
+            assert (got_own_sums is not None) == (variant == "no_offsets")
+        if got is not None:
+            np.testing.assert_array_equal(got, want)
+        if got_own_sums is not None:
+            np.testing.assert_array_equal(got_own_sums, want)
         assert want.std() > 5
 
 
@@ -111,6 +119,10 @@ def test_cwq_conv_long_k_on_every_tile(tile, IC):
         g = c["geom"]
         say("cwq_conv tile", TILES[tile], "IC", IC, variant,
             "K", g.KH * g.KW * IC // g.group)
+        if tile == 6:
+            # the split-K kernel serves FullyConnected forms only
+            assert tiles.refused(6, lambda: capi.cwq_conv2d_i8(*cases.cwq_conv_args(c)))
+            continue
         with forced_tile(tile):
             got = capi.cwq_conv2d_i8(*cases.cwq_conv_args(c))
             got_own_sums = capi.cwq_conv2d_i8(*cases.cwq_conv_args(c), precomputed_sums=False)
@@ -167,6 +179,9 @@ def test_rwq_fc_m4096_k1024_n1024_all_tiles_agree():
     ref = None
     for tile in TILES:
         say("rwq_fc M4096 K1024 N1024 tile", TILES[tile])
+        if tile == 6:   # weight offsets: refused by the split-K kernel
+            assert tiles.refused(6, lambda: capi.rwq_fc_i8(*cases.rwq_fc_args(c)))
+            continue
         with forced_tile(tile):
             got = capi.rwq_fc_i8(*cases.rwq_fc_args(c))
         if ref is None:
@@ -200,11 +215,17 @@ def test_requant_hint_gives_the_same_bytes_on_every_tile(tile):
         want = go.rwq_fc_i8(*cases.rwq_fc_args(c))
         say("hint", hint, "tile", TILES[tile], "K", K, "pre", int(c["out_pre"].min()),
             int(c["out_pre"].max()))
-        with forced_tile(tile), capi.requant_hint(hint):
-            got = capi.rwq_fc_i8(*cases.rwq_fc_args(c))
-            got2 = capi.rwq_fc_i8(*cases.rwq_fc_args(c), precomputed_sums=False)
-        np.testing.assert_array_equal(got, want)
-        np.testing.assert_array_equal(got2, want)
+        with capi.requant_hint(hint):
+            got = tiles.forced_or_refused(tile, lambda: capi.rwq_fc_i8(*cases.rwq_fc_args(c)))
+            got2 = tiles.forced_or_refused(
+                tile, lambda: capi.rwq_fc_i8(*cases.rwq_fc_args(c), precomputed_sums=False))
+        assert tile == 6 or (got is not None and got2 is not None)
+        if tile == 6:   # split-K: symmetric weights with precomputed sums only
+            assert (got is not None) == sym and (got2 is None or c["in_offset"] == 0)
+        if got is not None:
+            np.testing.assert_array_equal(got, want)
+        if got2 is not None:
+            np.testing.assert_array_equal(got2, want)
     assert {1, 3} <= seen          # both fast forms were exercised
 
 
@@ -287,16 +308,18 @@ def test_split_k_small_tiles_vs_oracle(shape):
             np.testing.assert_array_equal(got, want_relu)
 
 
-def test_split_k_tile_is_ignored_where_it_cannot_run():
-    """Weight offsets, missing row sums or a K that is no multiple of 32: tile 6
-    falls back to the tiled kernels, same results."""
+def test_split_k_tile_refuses_what_it_cannot_run():
+    """Weight offsets, missing row sums or a K that is no multiple of 32: asked
+    for by number (tile 6) the kernel refuses the launch; the shape rule runs
+    the tiled kernels, same results."""
     for kw, sums in ((dict(symmetric=False), True), (dict(symmetric=True), False)):
         c = cases.rwq_fc_case(9, 40, 256, 72, **kw)
         want = go.rwq_fc_i8(*cases.rwq_fc_args(c))
-        with forced_tile(6):
-            got = capi.rwq_fc_i8(*cases.rwq_fc_args(c), precomputed_sums=sums)
+        assert tiles.refused(6, lambda: capi.rwq_fc_i8(*cases.rwq_fc_args(c),
+                                                       precomputed_sums=sums))
+        got = capi.rwq_fc_i8(*cases.rwq_fc_args(c), precomputed_sums=sums)
         np.testing.assert_array_equal(got, want)
     c = cases.rwq_fc_case(10, 40, 272, 72)           # K % 32 == 16
-    with forced_tile(6):
-        np.testing.assert_array_equal(capi.rwq_fc_i8(*cases.rwq_fc_args(c)),
-                                      go.rwq_fc_i8(*cases.rwq_fc_args(c)))
+    assert tiles.refused(6, lambda: capi.rwq_fc_i8(*cases.rwq_fc_args(c)))
+    np.testing.assert_array_equal(capi.rwq_fc_i8(*cases.rwq_fc_args(c)),
+                                  go.rwq_fc_i8(*cases.rwq_fc_args(c)))

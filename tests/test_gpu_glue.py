@@ -223,3 +223,28 @@ def test_add_with_scales_beyond_24_bits():
         dp = (0, 22, (1 << 23) + 77)
         np.testing.assert_array_equal(capi.add_relu_i8(a, b, 5, lo, ro, lp, rp, -3, dp),
                                       go.relu_i8(want, 5, -3, dp))
+
+
+def test_unlowered_element_ops_golden_and_oracle():
+    """Clip, LeakyRelu, Max(x, Splat) and BatchedAdd (what the CPU backend keeps
+    un-lowered besides Relu; libjit.cpp:1865-1892, 997-1015, libjit_cpu.cpp:45-46):
+    the golden vectors of the compiled reference, then larger and unaligned
+    tensors against the oracle."""
+    for name, fn, args, want in gio.element_ops():
+        np.testing.assert_array_equal(getattr(capi, fn)(*args), want, err_msg=name)
+    rng = np.random.default_rng(77)
+    p = lambda r: go.quantize_scale_offset_32to8(float(np.float32(r)), 0)[:3]
+    for n in (1, 15, 16, 17, 4099, 1 << 20):
+        a = rng.integers(-128, 128, n).astype(np.int8)
+        np.testing.assert_array_equal(capi.clip_elem_i8(a, -30, 90, -5, 7, p(0.37)),
+                                      go.clip_elem_i8(a, -30, 90, -5, 7, p(0.37)))
+        np.testing.assert_array_equal(capi.leaky_relu_i8(a, 4, -9, p(1.9), p(0.19)),
+                                      go.leaky_relu_i8(a, 4, -9, p(1.9), p(0.19)))
+        np.testing.assert_array_equal(capi.max_splat_i8(a, -3), np.maximum(a, np.int8(-3)))
+    for ns, ss in ((1, 1), (7, 5), (64, 1000), (300, 1024), (4096, 512)):
+        b = rng.integers(-128, 128, (ns, ss)).astype(np.int8)
+        for sl in (rng.integers(-128, 128, ss).astype(np.int8),
+                   rng.integers(-100000, 100000, ss).astype(np.int32)):
+            sp = p(0.9) if sl.dtype == np.int8 else p(0.0007)
+            np.testing.assert_array_equal(capi.batched_add_i8(b, sl, -2, 3, -1, p(1.3), sp),
+                                          go.batched_add_i8(b, sl, -2, 3, -1, p(1.3), sp))

@@ -1,10 +1,18 @@
 """The SparseLengths kernels with their default (fused multiply-add)
-arithmetic, against the CPU oracle's sequential loop. The regrouped sum
-  sum_j (w_j s_j) q_jk + sum_j (w_j o_j)
-differs from the loop's w_j (s_j q_jk + o_j) by rounding only, so the bar is
-the stated one for floating point: 1e-5 relative. "Relative" is taken against
-B = sum_j |w_j| (|s_j| q_max + |o_j|), the magnitude of what a bag adds up (the
-result itself can cancel to nearly zero); the error seen is below 1e-6 B.
+arithmetic, against the CPU oracle's sequential loop. The default form
+  v = fma(s_j, q_jk, o_j);  acc_k = fma(w_j, v, acc_k)
+is the loop's own expression w_j (s_j q_jk + o_j) per element without the two
+intermediate roundings (what the reference's libjit becomes on a host with
+fused multiply-add), with the lookups of a bag summed in two interleaved
+partial sums. The bar is the stated one for floating point, element by
+element: |got - want| <= 1e-5 |want| for every output with
+|want| >= max(1, B / 128), where B = sum_j |w_j| (|s_j| q_max + |o_j|) is the
+magnitude of what the bag adds up. A result that has cancelled further than
+that is held to 1e-5 max(1, B / 128) instead: a sum of L terms taken in another
+order moves by about sqrt(L) units in the last place of its partial sums, which
+no relative bar on a cancelled result can absorb (the reference's own builds
+differ among themselves in the same way:
+tests/test_oracle_vs_ref.py::test_slws_reference_builds_differ_by_rounding).
 fp16 outputs get one extra fp16 unit in the last place for the final rounding.
 Everything else about the operator (skipped lookups, empty bags, index types,
 every output row written) is checked as in the bit-exact tests.
@@ -19,6 +27,7 @@ from tests import cases
 pytestmark = [pytest.mark.gpu, pytest.mark.fused_math]
 
 RTOL = 1e-5
+FLOOR = 1.0   # element-wise bar applies to outputs at least this large
 
 
 @pytest.fixture(scope="module", autouse=True)
@@ -65,8 +74,14 @@ def check(got, want, mag, out16=False, what=""):
         tol = tol + np.abs(want) * 2.0 ** -10
     err = np.abs(got - want)
     worst = float(np.max(err / np.maximum(mag[:, None], 1e-30))) if err.size else 0.0
-    say(f"  {what} max error / B = {worst:.2e}")
+    floor = np.maximum(FLOOR, mag[:, None] / 128.0) * np.ones_like(want)
+    big = np.abs(want) >= floor
+    etol = RTOL * np.maximum(np.abs(want), floor) + (np.abs(want) * 2.0 ** -10 if out16 else 0.0)
+    worst_rel = float(np.max(err[big] / np.abs(want[big]))) if big.any() else 0.0
+    say(f"  {what} max error / B = {worst:.2e}; max |got - want| / |want| over the "
+        f"{big.mean():.0%} of outputs with |want| >= max({FLOOR:g}, B/128): {worst_rel:.2e}")
     assert np.all(err <= tol), (what, worst)
+    assert np.all(err <= etol), (what, worst_rel)
     # empty bags are exact zeros
     empty = mag == 0
     assert np.all(got[empty] == 0)

@@ -141,6 +141,50 @@ def test_slws_vs_ref(idt):
             a, go.frwq_slws_generic(table, go.U8_F32, w, idx, lengths))
 
 
+def test_slws_reference_builds_differ_by_rounding():
+    """How far the reference's own builds of libjit.cpp:1253-1276 lie apart on
+    the headline lookup's bags (4096 bags, Poisson(40) lengths, Zipf(1.05)
+    indices, 128 columns; the table is a tenth of the benchmark's 4M rows, which
+    changes no arithmetic): its default fast-math flags change nothing on a host
+    without fused multiply-add, and with -mfma the loop contracts to
+    v = fma(s, q, o); acc = fma(w, v, acc), which moves the outputs at or above
+    1 in magnitude by a few 1e-6 relative. That is the latitude the reference
+    takes itself, and the expression the kernels' default arithmetic evaluates."""
+    if not ref.available("fma"):
+        pytest.skip("oracle/_ref/libjit_ref_fma.so is not built")
+    rng = np.random.default_rng(42)
+    rows, bags = 400_000, 4096
+    table = cases.random_fused_table(rng, rows, 128)
+    lengths, idx, w = cases.slws_batch(1000, rows, bags, 40, 1.05, np.int64)
+    plain = ref.frwq_slws_f32(table, w, idx, lengths)
+    fast = ref.frwq_slws_f32(table, w, idx, lengths, fastmath=True)
+    fma = ref.frwq_slws_f32(table, w, idx, lengths, fastmath="fma")
+    np.testing.assert_array_equal(plain, go.frwq_slws_f32(table, w, idx, lengths))
+    np.testing.assert_array_equal(fast, plain)
+    big = np.abs(plain) >= 1.0
+    rel = np.abs(fma[big].astype(np.float64) - plain[big]) / np.abs(plain[big])
+    print(f"reference with -mfma against its plain build: {np.mean(fma != plain):.0%} of the "
+          f"outputs differ, max relative difference {rel.max():.2e} over the {big.mean():.0%} "
+          "with |value| >= 1", flush=True)
+    assert 0 < rel.max() <= 1e-5
+    # the contracted loop is the kernels' default expression, evaluated in bag
+    # order: v = fma(s, q, o); acc = fma(w, v, acc), through float64 (products of
+    # two floats are exact there, so each step rounds once)
+    so = np.ascontiguousarray(table[:, 128:136]).view(np.float32)
+    f64 = np.float64
+    pos, worst = 0, 0
+    for b in range(64):
+        acc = np.zeros(128, np.float32)
+        for j in range(lengths[b]):
+            r = idx[pos + j]
+            v = (f64(so[r, 0]) * table[r, :128].astype(f64) + f64(so[r, 1])).astype(np.float32)
+            acc = (f64(w[pos + j]) * v.astype(f64) + acc.astype(f64)).astype(np.float32)
+        pos += lengths[b]
+        worst = max(worst, int(np.abs(acc.view(np.int32).astype(np.int64) -
+                                      fma[b].view(np.int32).astype(np.int64)).max()))
+    assert worst == 0, f"the -mfma build is not the contracted loop ({worst} units apart)"
+
+
 def test_embedding_bag_vs_ref():
     rng = np.random.default_rng(4)
     table = cases.random_fused_table(rng, 200, 16)
@@ -256,3 +300,17 @@ def test_cwq_conv3d_vs_ref(fastmath):
         c = cases.cwq_conv3d_case(900 + i, **kw_)
         np.testing.assert_array_equal(go.cwq_conv3d_i8(*cases.cwq_conv_args(c)),
                                       ref.cwq_conv3d_i8(*cases.cwq_conv_args(c), fastmath=fastmath))
+
+
+@pytest.mark.parametrize("fastmath", FM)
+def test_unlowered_element_ops_vs_ref(fastmath):
+    """Clip, LeakyRelu, Max(x, Splat) and BatchedAdd on int8 against the
+    compiled reference (libjit.cpp:1865-1892, 997-1015; libjit_cpu.cpp:45-46),
+    every int8 input value included."""
+    for name, fn, args in cases.element_op_cases():
+        got = getattr(go, fn)(*args)
+        want = getattr(ref, fn)(*args, fastmath=fastmath)
+        np.testing.assert_array_equal(got.ravel(), np.asarray(want).ravel(), err_msg=name)
+    # Max(x, Splat) is numpy's maximum
+    a = cases.element_op_cases()[0][2][0]
+    np.testing.assert_array_equal(go.max_splat_i8(a, -7), np.maximum(a, np.int8(-7)))
