@@ -2044,6 +2044,21 @@ private:
     return pos - at;
   }
 
+  // Whether an instruction of any function of the module writes `root` or a view of it.
+  bool writtenInModule(int root) const {
+    auto writes = [&](const std::vector<Instruction> &insts) {
+      for (const auto &I : insts)
+        if (!I.operands.empty() && M_.validId(I.operands[0]) &&
+            M_.value(I.operands[0]).root == root)
+          return true;
+      return false;
+    };
+    if (writes(insts_)) return true;
+    for (const auto &f : M_.functions())
+      if (f && writes(f->instructions())) return true;
+    return false;
+  }
+
   // The bag positions of a lookup whose lengths are an input of the function
   // (a placeholder no instruction writes): a scratch vector the device manager
   // fills when it uploads the lengths. Empty function: read the lengths.
@@ -2052,8 +2067,9 @@ private:
     if (!opts_.deriveBagOffsets || len.v->category != SymbolCategory::Placeholder ||
         len.v->id != len.v->root)
       return nullptr;
-    auto w = io_.find(len.v->id);
-    if (w != io_.end() && w->second.second) return nullptr; // written on the device
+    // written on the device, directly or through a view, by this function or by
+    // another one the module holds so far: the host's copy would be stale
+    if (writtenInModule(len.v->id)) return nullptr;
     auto it = derived_.find(len.v->id);
     if (it != derived_.end()) return out.derivedBagOffsets[it->second].ptr;
     const size_t segs = (size_t)len.ty().size();
@@ -2165,6 +2181,14 @@ Expected<std::unique_ptr<MI355XFunction>> MI355XBackend::compile(const Function 
   auto fn = std::unique_ptr<MI355XFunction>(new MI355XFunction(RuntimeBundle(), F.name()));
   Error e = C.run(*fn);
   if (e) return e;
+  for (const auto &I : F.instructions()) {
+    if (I.operands.empty() || !M.validId(I.operands[0])) continue;
+    const Value &root = M.value(M.value(I.operands[0]).root);
+    if (root.category == SymbolCategory::Placeholder &&
+        std::find(fn->writtenPlaceholders.begin(), fn->writtenPlaceholders.end(), root.name) ==
+            fn->writtenPlaceholders.end())
+      fn->writtenPlaceholders.push_back(root.name);
+  }
   RuntimeBundle rb;
   rb.constantWeightVarsMemSize = M.constantsSize();
   rb.mutableWeightVarsMemSize = M.mutableSize();

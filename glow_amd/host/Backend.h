@@ -158,6 +158,11 @@ public:
     std::function<uint8_t *(const DeviceBindings &)> ptr;
   };
   std::vector<DerivedBagOffsets> derivedBagOffsets;
+  // Placeholders (by name; a view counts for the value it views) that some
+  // instruction of this function writes. Nobody may derive bag positions on
+  // the host from such a placeholder: the device manager refuses to load two
+  // functions of a module of which one writes what the other derives from.
+  std::vector<std::string> writtenPlaceholders;
   // Host side of that contract: the positions for `lengths` (n of the
   // placeholder's `segments` entries given; the missing ones count as empty
   // bags). Sums saturate at INT32_MAX, which lies at or past the end of any

@@ -24,6 +24,12 @@ int uploadBagOffsets(const MI355XFunction &fn, const DeviceBindings &b, const st
   }
   return MI355X_OK;
 }
+// Whether any lookup of `fn` takes its bag positions from placeholder `name`.
+bool derivesFrom(const MI355XFunction &fn, const std::string &name) {
+  for (const auto &d : fn.derivedBagOffsets)
+    if (d.lengths == name) return true;
+  return false;
+}
 } // namespace
 
 namespace {
@@ -231,10 +237,12 @@ void MI355XDeviceManager::transferStaticPlaceholderToDevice(
                                  tensor->sizeInBytes(), stream_);
     // lookups of the module's functions that take their bags from this placeholder
     std::vector<std::vector<int32_t>> staged;
-    for (auto &f : functions_)
-      if (rc == MI355X_OK && f.second.module == module)
-        rc = uploadBagOffsets(*f.second.fn, f.second.bindings, placeholderName, tensor->data(),
-                              tensor->sizeInBytes(), stream_, staged);
+    if (rc == MI355X_OK) {
+      void *slot = nullptr;
+      mi355x_arena_ptr(mit->second.arena, MI355X_REGION_MUTABLE, v.offset, &slot);
+      rc = lengthsUploaded(module, placeholderName, (uint8_t *)slot, v.type.sizeInBytes(),
+                           tensor->data(), tensor->sizeInBytes(), staged);
+    }
     if (rc == MI355X_OK) rc = mi355x_stream_sync(stream_);
     resultCB(rc == MI355X_OK ? Error::success() : fromStatus(rc, "placeholder copy"));
   });
@@ -301,9 +309,51 @@ void MI355XDeviceManager::release(FunctionResident &fr) {
   }
 }
 
+// `bytes` of placeholder `name` of `module` have just been copied into its slot
+// (slotBytes long). If lookups of any resident function of the module take
+// their bag positions from it, the rest of the slot is cleared (a partial
+// tensor: the missing bags are empty for the kernels that read the lengths and
+// for the positions alike) and every such function's positions are refreshed:
+// the slot belongs to the module, so a function that is not the one being run
+// must not keep positions of the lengths it held before.
+int MI355XDeviceManager::lengthsUploaded(const Module *module, const std::string &name,
+                                         uint8_t *slot, size_t slotBytes, const void *data,
+                                         size_t bytes,
+                                         std::vector<std::vector<int32_t>> &staged) {
+  bool derived = false;
+  for (auto &f : functions_)
+    if (f.second.module == module && derivesFrom(*f.second.fn, name)) derived = true;
+  if (!derived) return MI355X_OK;
+  int rc = MI355X_OK;
+  if (bytes < slotBytes) rc = mi355x_fill_u8(slot + bytes, 0, slotBytes - bytes, stream_);
+  for (auto &f : functions_)
+    if (rc == MI355X_OK && f.second.module == module)
+      rc = uploadBagOffsets(*f.second.fn, f.second.bindings, name, data, bytes, stream_, staged);
+  return rc;
+}
+
 Error MI355XDeviceManager::makeResident(const Module *module, const std::string &name,
                                         MI355XFunction *fn) {
   const RuntimeBundle &rb = fn->getRuntimeBundle();
+  // A function that writes a placeholder on the device and one that derives bag
+  // positions from the host's copy of the same placeholder cannot share a module.
+  for (const auto &f : functions_) {
+    if (f.second.module != module) continue;
+    for (const auto &w : fn->writtenPlaceholders)
+      if (derivesFrom(*f.second.fn, w))
+        return MI355X_MAKE_ERR(ErrorCode::DEVICE_FEATURE_NOT_SUPPORTED,
+                               "function %s writes placeholder %s, from which resident function "
+                               "%s takes bag positions made on the host: compile that one with "
+                               "deriveBagOffsets off",
+                               name.c_str(), w.c_str(), f.first.c_str());
+    for (const auto &w : f.second.fn->writtenPlaceholders)
+      if (derivesFrom(*fn, w))
+        return MI355X_MAKE_ERR(ErrorCode::DEVICE_FEATURE_NOT_SUPPORTED,
+                               "function %s takes bag positions made on the host from placeholder "
+                               "%s, which resident function %s writes: compile it with "
+                               "deriveBagOffsets off",
+                               name.c_str(), w.c_str(), f.first.c_str());
+  }
   ModuleResident &mr = modules_[module];
   if (!mr.arena && mr.users == 0) {
     int rc = mi355x_arena_create(module->constantsSize(), module->mutableSize(), 0, &mr.arena);
@@ -627,8 +677,8 @@ void MI355XDeviceManager::runFunctionImpl(RunIdentifierTy id, std::string functi
     int rc = mi355x_memcpy_h2d(fr.bindings.mutableMem + st->second.offset, kv.second->data(),
                                kv.second->sizeInBytes(), stream_);
     if (rc == MI355X_OK)
-      rc = uploadBagOffsets(*fr.fn, fr.bindings, kv.first, kv.second->data(),
-                            kv.second->sizeInBytes(), stream_, staged);
+      rc = lengthsUploaded(fr.module, kv.first, fr.bindings.mutableMem + st->second.offset,
+                           st->second.size, kv.second->data(), kv.second->sizeInBytes(), staged);
     if (rc != MI355X_OK) {
       err = fromStatus(rc, "input copy");
       break;

@@ -122,6 +122,9 @@ private:
   Error executeTuned(FunctionResident &fr, ExecutionContext *ctx);
   void release(FunctionResident &fr);
   void enqueue(std::function<void()> work);
+  int lengthsUploaded(const Module *module, const std::string &name, uint8_t *slot,
+                      size_t slotBytes, const void *data, size_t bytes,
+                      std::vector<std::vector<int32_t>> &staged);
   void workerLoop();
 
   DeviceConfig config_;

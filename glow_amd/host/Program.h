@@ -51,7 +51,7 @@ enum class Kind : int32_t {
   MaxPool,                      // (Dest, Src); iattrs {kernelH, kernelW, strideH, strideW, padT, padL, padB, padR}
   AvgPool,                      // (Dest, Src); MaxPool's iattrs + {countIncludePads}
   SoftMax,                      // (Dest, Src), float [rows x cols]
-  ConvertTo,                    // (Dest float, Src float16)
+  ConvertTo,                    // (Result float, Input float16)
   InsertTensor,                 // (Dest [R,W], Src [R,w]); iattrs {offset in the inner dimension}
   Transpose,                    // (Dest, Src) int8; iattrs = shuffle, {1,0} or {0,2,1}
   Gather,                       // (Dest, Data, Indices); iattrs {batchDims (0 or 1)}

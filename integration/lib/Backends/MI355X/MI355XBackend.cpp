@@ -253,10 +253,27 @@ bool MI355XBackend::isOpSupported(const NodeInfo &NI) const {
                ElemKind::FloatTy;
 
   // ---- int8 glue of a quantized image network --------------------------------
-  case Kinded::Kind::AddNodeKind:  // ==> ElementAdd
-  case Kinded::Kind::ReluNodeKind: // stays un-lowered, ==> Relu
+  case Kinded::Kind::AddNodeKind:       // ==> ElementAdd
+  case Kinded::Kind::ReluNodeKind:      // stays un-lowered, ==> Relu
+  case Kinded::Kind::ClipNodeKind:      // stays un-lowered, ==> Clip
+  case Kinded::Kind::LeakyReluNodeKind: // stays un-lowered, ==> LeakyRelu
   case Kinded::Kind::AvgPoolNodeKind:
     return NI.allInputsAndOutputsHaveSameElemKind({ElemKind::Int8QTy});
+
+  // what a FullyConnected that some other pass lowered leaves behind its
+  // MatMul (lib/Optimizer/Lower/Lower.cpp): int8 batch, int8 or int32 slice
+  case Kinded::Kind::BatchedAddNodeKind:
+    return NI.getInElemTy(BatchedAddNode::BatchIdx) == ElemKind::Int8QTy &&
+           NI.getOutElemTy(BatchedAddNode::ResultIdx) == ElemKind::Int8QTy &&
+           (NI.getInElemTy(BatchedAddNode::SliceIdx) == ElemKind::Int8QTy ||
+            NI.getInElemTy(BatchedAddNode::SliceIdx) == ElemKind::Int32QTy);
+
+#ifdef GLOW_WITH_CPU
+  // Max(x, Splat(v)) as the CPU backend's node (the class exists when that
+  // backend is built; transformPostLowering below makes it)
+  case Kinded::Kind::CPUMaxSplatNodeKind:
+    return NI.allInputsAndOutputsHaveSameElemKind({ElemKind::Int8QTy});
+#endif
 
   case Kinded::Kind::MaxPoolNodeKind:
     // the Argmax result is not produced: accepted only when it is unused,
@@ -302,6 +319,41 @@ bool MI355XBackend::isOpSupported(const NodeInfo &NI) const {
   default:
     return false;
   }
+}
+
+Expected<bool> MI355XBackend::transformPostLowering(
+    Function *F, CompilationContext &cctx,
+    const glow::runtime::DeviceInfo *devInfo) const {
+  (void)cctx;
+  (void)devInfo;
+  bool changed = false;
+#ifdef GLOW_WITH_CPU
+  // Max(x, Splat(v)) on int8 of one type (a Relu that keeps its input's
+  // parameters) becomes the CPU backend's CPUMaxSplatNode, as in
+  // lib/Backends/CPU/Transforms.cpp: one elementwise pass instead of a Splat
+  // tensor and a two-operand Max, for which this backend has no kernel.
+  for (auto &node : F->getNodes()) {
+    auto *MN = llvm::dyn_cast<MaxNode>(&node);
+    if (!MN || MN->getResult().getElementType() != ElemKind::Int8QTy) {
+      continue;
+    }
+    SplatNode *splat = llvm::dyn_cast<SplatNode>(MN->getLHS().getNode());
+    NodeValue input = MN->getRHS();
+    if (!splat) {
+      splat = llvm::dyn_cast<SplatNode>(MN->getRHS().getNode());
+      input = MN->getLHS();
+    }
+    if (!splat || input.getType() != MN->getResult().getType()) {
+      continue;
+    }
+    auto *MS = F->addNode(new CPUMaxSplatNode(MN->getName(), input, splat->getValue()));
+    MN->getResult().replaceAllUsesOfWith(MS->getResult());
+    changed = true;
+  }
+#else
+  (void)F;
+#endif
+  return changed;
 }
 
 bool MI355XBackend::shouldLower(const Node *N) const {

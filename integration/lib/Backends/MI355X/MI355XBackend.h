@@ -56,12 +56,7 @@ public:
   /// the final buffers and their single readers.
   Expected<bool> transformPostLowering(
       Function *F, CompilationContext &cctx,
-      const glow::runtime::DeviceInfo *devInfo = nullptr) const override {
-    (void)F;
-    (void)cctx;
-    (void)devInfo;
-    return false;
-  }
+      const glow::runtime::DeviceInfo *devInfo = nullptr) const override;
 
   /// int64 -> int32 index demotion everywhere except the SparseLengths family
   /// (the kernels take either; the reference keeps them int64 on the CPU,

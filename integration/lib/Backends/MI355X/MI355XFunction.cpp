@@ -353,6 +353,22 @@ private:
       return add(I, hm::Kind::ElementAdd);
     case Kinded::Kind::ReluInstKind:
       return add(I, hm::Kind::Relu);
+    case Kinded::Kind::ClipInstKind: {
+      const auto *C = cast<ClipInst>(&I);
+      return add(I, hm::Kind::Clip, {}, {C->getMin(), C->getMax()});
+    }
+    case Kinded::Kind::LeakyReluInstKind: {
+      const auto *L = cast<LeakyReluInst>(&I);
+      return add(I, hm::Kind::LeakyRelu, {}, {L->getAlpha()});
+    }
+    case Kinded::Kind::BatchedAddInstKind:
+      return add(I, hm::Kind::BatchedAdd);
+#ifdef GLOW_WITH_CPU
+    case Kinded::Kind::CPUMaxSplatInstKind: {
+      const auto *S = cast<CPUMaxSplatInst>(&I);
+      return add(I, hm::Kind::CPUMaxSplat, {}, {S->getSplatValue()});
+    }
+#endif
     case Kinded::Kind::MaxPoolInstKind: {
       const auto *P = cast<MaxPoolInst>(&I);
       if (P->getLayout() != NHWC) {

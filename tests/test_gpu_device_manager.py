@@ -253,6 +253,80 @@ def test_slws_network_bag_positions_follow_every_upload(dm):
     np.testing.assert_array_equal(res, go.frwq_slws_f32(table, w, idx, lengths))
 
 
+def _two_lookup_functions(table, bags, cols, n, writer=False, derive_second=True):
+    """One module, one lengths placeholder, two functions that each pool the
+    same table over it (into outputs of their own); `writer` adds a third
+    function that copies another placeholder into the lengths on the device."""
+    m = H.Module("shared_lengths")
+    data = m.constant("data", table, H.UINT8_FUSED)
+    wv = m.placeholder("weights", (n,), H.FLOAT, np.float32)
+    iv = m.placeholder("indices", (n,), H.INT64I, np.int64)
+    lv = m.placeholder("lengths", (bags,), H.INT32I, np.int32)
+    out_a = m.placeholder("out_a", (bags, cols), H.FLOAT, np.float32)
+    out_b = m.placeholder("out_b", (bags, cols), H.FLOAT, np.float32)
+    fw = None
+    if writer:
+        src = m.placeholder("new_lengths", (bags,), H.INT32I, np.int32)
+        fw = m.function("set_lengths")
+        m.instruction(fw, H.COPY, "store", [lv, src])
+    fa = m.function("a")
+    m.instruction(fa, H.FRWQ_SLWS, "slws_a", [out_a, data, wv, iv, lv], [0])
+    fb = m.function("b")
+    m.instruction(fb, H.FRWQ_SLS, "sls_b", [out_b, data, iv, lv], [0])
+    return m, fa, fb, fw
+
+
+def test_bag_positions_of_every_function_of_a_module_follow_an_upload(dm):
+    """The lengths placeholder belongs to the module: a request to one function
+    that binds new lengths must also refresh the bag positions of the module's
+    other functions, which read the same slot without binding it."""
+    rng = np.random.default_rng(41)
+    rows, cols, bags, n = 2000, 64, 150, 3000
+    table = cases.random_fused_table(rng, rows, cols)
+    m, fa, fb, _ = _two_lookup_functions(table, bags, cols, n)
+    m.compile(fa)
+    m.compile(fb)
+    assert "mi355x_frwq_slws_offsets" in m.describe(fa) and "_offsets" in m.describe(fb)
+    dm.add_network(m)
+    ra, rb = np.zeros((bags, cols), np.float32), np.zeros((bags, cols), np.float32)
+    ones = np.ones(n, np.float32)
+    for seed, mean in ((1, 12), (2, 4)):
+        lengths, idx, w = cases.slws_batch(seed, rows, bags, mean, 1.05, np.int64)
+        dm.run("a", {"weights": w, "indices": idx, "lengths": lengths, "out_a": ra})
+        np.testing.assert_array_equal(ra, go.frwq_slws_f32(table, w, idx, lengths))
+        # b reads the lengths a's request left in the module's slot
+        dm.run("b", {"indices": idx, "out_b": rb})
+        np.testing.assert_array_equal(rb, go.frwq_slws_f32(table, ones[:idx.size], idx, lengths))
+    # a partial lengths tensor after longer ones: the rest of the slot is cleared,
+    # so both functions see empty bags there
+    lengths, idx, w = cases.slws_batch(3, rows, bags, 9, 1.05, np.int64)
+    half = lengths[:bags // 3].copy()
+    padded = np.r_[half, np.zeros(bags - half.size, np.int32)].astype(np.int32)
+    dm.run("b", {"indices": idx, "lengths": half, "out_b": rb})
+    np.testing.assert_array_equal(rb, go.frwq_slws_f32(table, ones[:idx.size], idx, padded))
+    dm.run("a", {"weights": w, "indices": idx, "out_a": ra})
+    np.testing.assert_array_equal(ra, go.frwq_slws_f32(table, w, idx, padded))
+
+
+def test_lengths_written_on_the_device_are_not_summed_on_the_host(dm):
+    """A function of the module that writes the lengths placeholder: the lookups
+    compiled after it read the lengths themselves; one compiled before it (with
+    positions from the host) cannot share a device with it."""
+    rng = np.random.default_rng(42)
+    rows, cols, bags, n = 1500, 64, 90, 2000
+    table = cases.random_fused_table(rng, rows, cols)
+    m, fa, fb, fw = _two_lookup_functions(table, bags, cols, n, writer=True)
+    for f in (fw, fa, fb):
+        m.compile(f)
+    assert "_offsets" not in m.describe(fa) and "_offsets" not in m.describe(fb)
+    dm.add_network(m)
+    ra = np.zeros((bags, cols), np.float32)
+    lengths, idx, w = cases.slws_batch(7, rows, bags, 10, 1.05, np.int64)
+    dm.run("set_lengths", {"new_lengths": lengths})
+    dm.run("a", {"weights": w, "indices": idx, "out_a": ra})
+    np.testing.assert_array_equal(ra, go.frwq_slws_f32(table, w, idx, lengths))
+
+
 def test_fc_and_conv_networks(dm):
     c = cases.fc_case(20, 24, 96, 80)
     m, f = host_cases.fc_module(c)

@@ -472,3 +472,34 @@ def test_wide_kinds_transposes_and_3d_convolutions_compile():
     bad, fb = host_cases.cwq_conv3d_module(c, (2, 3, 3), (1, 1, 1), (1, 0, 1, 1, 0, 2))
     with pytest.raises(H.HostError):
         bad.compile(fb)
+
+
+def test_bag_positions_are_not_derived_from_lengths_some_function_writes():
+    """Bag positions summed on the host need lengths only the host writes: a
+    write through a view, or by another function of the module, switches the
+    lookup back to reading the lengths on the device."""
+    rng = np.random.default_rng(5)
+    table = rng.integers(0, 256, (50, 72)).astype(np.uint8)
+
+    def build(view_write, other_function):
+        m = H.Module("w")
+        data = m.constant("data", table, H.UINT8_FUSED)
+        iv = m.placeholder("indices", (400,), H.INT64I, np.int64)
+        lv = m.placeholder("lengths", (32,), H.INT32I, np.int32)
+        src = m.placeholder("src", (32,), H.INT32I, np.int32)
+        out = m.placeholder("out", (32, 64), H.FLOAT, np.float32)
+        f = m.function("main")
+        if other_function:
+            g = m.function("writer")
+            m.instruction(g, H.COPY, "store", [lv, src])
+        if view_write:
+            half = m.view("first_half", lv, (16,), H.INT32I)
+            src_half = m.view("src_half", src, (16,), H.INT32I)
+            m.instruction(f, H.COPY, "store_half", [half, src_half])
+        m.instruction(f, H.FRWQ_SLS, "sls", [out, data, iv, lv], [0])
+        m.compile(f)
+        return m.describe(f)
+
+    assert "mi355x_frwq_slws_offsets" in build(False, False)
+    assert "mi355x_frwq_slws_offsets" not in build(True, False)
+    assert "mi355x_frwq_slws_offsets" not in build(False, True)
