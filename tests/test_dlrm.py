@@ -132,6 +132,6 @@ def test_device_with_fused_lookup_arithmetic_stays_within_one_step():
         want = oracle_exec.run(net, b)
         d = np.abs(logit.astype(np.int32) - want["logit_q"].astype(np.int32))
         print("logits off by one step:", int((d == 1).sum()), "of", d.size, flush=True)
-        assert d.max() <= 1 and (d > 0).mean() <= 0.05
+        assert d.max() <= 1 and (d > 0).sum() <= 1
     finally:
         dm.stop()
