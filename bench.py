@@ -41,7 +41,7 @@ if ROOT not in sys.path:
 # HBM bytes per launch of the default workloads (FETCH_SIZE + WRITE_SIZE of two
 # counter runs, scaled by what the counters read for a plain copy of known
 # size). They hold for the default sizes only; other sizes report null.
-MEASURED_TRAFFIC = {"slws": 23.98e6, "fc_large": 236.0e6, "conv_c3": 19.63e6}
+MEASURED_TRAFFIC = {"slws": 23.87e6, "fc_large": 236.0e6, "conv_c3": 19.63e6}
 
 HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E, published
 INT8_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA, published (5.0 POP/s)
@@ -71,7 +71,7 @@ def parse():
                     help="headline workload only")
     ap.add_argument("--only", default="",
                     help="run a single extra kernel (profiling aid): "
-                         "slws|slws_warm|slws_strict|fc_large|fc_large_zero|fc_c1|fc_m16384|fc_mid|"
+                         "slws|slws_warm|slws_strict|slws_probe|fc_large|fc_large_zero|fc_c1|fc_m16384|fc_mid|"
                          "fc|conv_c3|quantize|dequantize|rescale|copy|resnet50|dlrm")
     ap.add_argument("--shape", default="",
                     help="MxKxN of --only fc (a RowwiseQuantizedFullyConnected of that shape)")
@@ -84,7 +84,7 @@ def parse():
     return ap.parse_args()
 
 
-def timed_launches(capi, fn, steps, warmup, flush=None, during=None):
+def timed_launches(capi, fn, steps, warmup, flush=None, during=None, lanes=1):
     """Average seconds per launch. `fn(i, stream)` issues launch i. After
     `warmup` eager launches, the `steps` timed launches are recorded into one
     launch graph and replayed, so the figure is the device-side rate and not
@@ -94,14 +94,31 @@ def timed_launches(capi, fn, steps, warmup, flush=None, during=None):
     `flush(stream)` runs between the untimed and the timed replay (cache
     flush, queued directly in front of the timed region); `during()` is called
     while the timed replay runs (it may queue work
-    on other streams) and its result is returned beside the time."""
+    on other streams) and its result is returned beside the time.
+    lanes > 1: the recorded launches are dealt round-robin onto that many
+    streams that fork from and join the recording stream, so launch i need
+    not wait for launch i - 1 (independent requests in flight together, what
+    the reference's benchmarks call asyncLaunchSize); fn then gets the lane as
+    a third argument and must keep the lanes' outputs apart."""
     stream = capi.Stream()
     for i in range(warmup):
-        fn(i, stream)
+        fn(i, stream) if lanes == 1 else fn(i, stream, 0)
     stream.sync()
+    side = [capi.Stream() for _ in range(lanes - 1)]
     with capi.Graph(stream) as graph:
-        for i in range(steps):
-            fn(warmup + i, stream)
+        if lanes == 1:
+            for i in range(steps):
+                fn(warmup + i, stream)
+        else:
+            events = [capi.Event() for _ in range(lanes)]   # alive until the capture ends
+            events[0].record(stream)
+            for s in side:
+                s.wait_event(events[0])
+            for i in range(steps):
+                fn(warmup + i, ([stream] + side)[i % lanes], i % lanes)
+            for s, done in zip(side, events[1:]):
+                done.record(s)
+                stream.wait_event(done)
     graph.launch()          # untimed first replay (uploads the graph)
     stream.sync()
     capi.sync()
@@ -190,17 +207,27 @@ def make_slws_batches(capi, cases, args, count):
     return batches
 
 
-def bench_slws(capi, args, d_table, batches, flush, bag_offsets=False):
+def bench_slws(capi, args, d_table, batches, flush, bag_offsets=False, probe_stage=None, lanes=1):
     """Times args.steps launches that cycle through `batches`; `flush` (or None)
     empties the caches before the timed replay. bag_offsets: the bags as the
     positions a device manager derives from the lengths on the host
-    (mi355x_frwq_slws_offsets) instead of the lengths themselves."""
+    (mi355x_frwq_slws_offsets) instead of the lengths themselves. probe_stage:
+    the launch cut off behind that stage (mi355x_frwq_slws_probe)."""
+    import ctypes as C
     rows, cols, bags = args.rows, 128, args.bags
     row_bytes = cols + 8
-    d_out = capi.DeviceBuffer.empty((bags, cols), np.float32)
+    d_outs = [capi.DeviceBuffer.empty((bags, cols), np.float32) for _ in range(lanes)]
 
-    def step(i, stream):
+    def step(i, stream, lane=0):
         b = batches[i % len(batches)]
+        d_out = d_outs[lane]
+        if probe_stage is not None:
+            capi.check(capi.lib().mi355x_frwq_slws_probe(
+                C.c_int(probe_stage), C.c_void_p(d_out.ptr), C.c_void_p(d_table.ptr),
+                C.c_size_t(rows), C.c_void_p(b["d_w"].ptr), C.c_void_p(b["d_idx"].ptr),
+                C.c_size_t(b["total"]), C.c_void_p(b["d_len"].ptr), C.c_size_t(bags),
+                C.c_size_t(row_bytes), C.c_void_p(stream.ptr)))
+            return
         if bag_offsets:
             capi.launch_frwq_slws_offsets(d_out, False, d_table, rows, capi.FUSED_U8_F32,
                                           b["d_w"], False, b["d_idx"], True, b["total"],
@@ -210,7 +237,8 @@ def bench_slws(capi, args, d_table, batches, flush, bag_offsets=False):
                               b["d_w"], False, b["d_idx"], True, b["total"],
                               b["d_len"], bags, row_bytes, cols, stream=stream)
 
-    sec = timed_launches(capi, step, args.steps, args.warmup, flush=flush)
+    sec = timed_launches(capi, step, args.steps, args.warmup, flush=flush, lanes=lanes)
+    d_out = d_outs[(args.steps - 1) % lanes]    # the last timed step's output
     mean_total = float(np.mean([batches[(args.warmup + i) % len(batches)]["total"]
                                 for i in range(args.steps)]))
     nbytes = slws_bytes(mean_total, bags, cols, row_bytes)
@@ -228,6 +256,24 @@ def slws_errors(got, want, table, b):
     rel = float(np.max(np.abs(got[big].astype(np.float64) - want[big]) / np.abs(want[big]))) \
         if big.any() else 0.0
     return ratio, rel, float(big.mean())
+
+
+def slws_stage_probe(capi, args, d_table, batches, flush, s):
+    """The headline launch cut off behind each of its dependent stages, same
+    grid, same batches, same flush: what the decomposition costs before any
+    arithmetic. `s` is the headline's own bench_slws result."""
+    stages = ("empty launch", "bag positions (prefix over the lengths)",
+              "index and weight of every lookup", "scale and offset of every row",
+              "every row read, no arithmetic")
+    probe = [bench_slws(capi, args, d_table, batches, flush, probe_stage=k)["sec"] * 1e6
+             for k in range(len(stages))]
+    return dict(
+        workload="headline launch cut off behind a stage (mi355x_frwq_slws_probe), "
+                 "cumulative microseconds per launch",
+        stages={name: round(us, 3) for name, us in zip(stages, probe)},
+        floor_us=probe[-1],
+        floor_frac_of_hbm_peak=s["bytes"] / (probe[-1] * 1e-6) / 1e9 / HBM_PEAK_GBPS,
+        headline_us=s["sec"] * 1e6)
 
 
 def bench_slws_with_h2d(capi, s, args, d_table):
@@ -729,7 +775,7 @@ def main():
     if args.tile >= 0:
         capi.check(capi.lib().mi355x_gemm_tile_override(args.tile))
 
-    if only and only not in ("slws", "slws_warm", "slws_strict", "fc", "fc_large", "fc_large_zero",
+    if only and only not in ("slws", "slws_warm", "slws_strict", "slws_probe", "fc", "fc_large", "fc_large_zero",
                              "fc_c1", "fc_m16384", "fc_mid", "conv_c3", "quantize", "dequantize",
                              "rescale", "copy"):
         print(f"unknown --only {only}", file=sys.stderr)
@@ -774,6 +820,8 @@ def main():
         capi.slws_set_fused_math(capi.SLWS_MATH_ELEMENT)
     else:
         s = bench_slws(capi, args, d_table, batches, flush)
+    if only == "slws_probe":
+        extra["slws_stage_probe"] = slws_stage_probe(capi, args, d_table, batches, flush, s)
     gbps = s["bytes"] / s["sec"] / 1e9
 
     # the check of the last timed step's output (portable build of the oracle),
@@ -814,6 +862,26 @@ def main():
             ms=ss["sec"] * 1e3, gbps=ss["bytes"] / ss["sec"] / 1e9,
             frac_of_hbm_peak=ss["bytes"] / ss["sec"] / 1e9 / HBM_PEAK_GBPS,
             bit_exact_with_oracle=bit_exact)
+        extra["slws_stage_probe"] = slws_stage_probe(capi, args, d_table, batches, flush, s)
+        # Independent requests in flight together: the same launches dealt onto 2
+        # and 4 streams (each with an output of its own), so one launch's
+        # dependent trips run while another's rows stream. Throughput of the
+        # job, not the duration of a launch.
+        extra["slws_requests_in_flight"] = []
+        for lanes in (2, 4):
+            sl = bench_slws(capi, args, d_table, batches, flush, lanes=lanes)
+            same = None
+            if args.cpu_seconds > 0:
+                want = go.frwq_slws_f32(table, sl["last"]["w"], sl["last"]["idx"],
+                                        sl["last"]["lengths"])
+                _, rel_l, _ = slws_errors(sl["d_out"].numpy(), want, table, sl["last"])
+                same = bool(rel_l <= 1e-5)
+            extra["slws_requests_in_flight"].append(dict(
+                workload=f"headline launches on {lanes} streams that fork from and join the "
+                         "timed stream (independent batches, one output each), caches flushed",
+                streams=lanes, us_per_step=sl["sec"] * 1e6, gbps=sl["bytes"] / sl["sec"] / 1e9,
+                frac_of_hbm_peak=sl["bytes"] / sl["sec"] / 1e9 / HBM_PEAK_GBPS,
+                parity_with_oracle=same))
         # the bags as positions (what the device manager hands over for lengths it
         # uploads itself): no prefix sum in front of a bag's first index load
         so = bench_slws(capi, args, d_table, batches, flush, bag_offsets=True)

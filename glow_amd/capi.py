@@ -277,6 +277,10 @@ class Stream:
     def sync(self):
         check(lib().mi355x_stream_sync(_vp(self.ptr)))
 
+    def wait_event(self, event):
+        """Work queued on this stream from here on starts after `event`."""
+        check(lib().mi355x_stream_wait_event(_vp(self.ptr), _vp(event.ptr)))
+
     def __del__(self):
         try:
             if self.ptr:

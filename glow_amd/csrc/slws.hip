@@ -19,11 +19,14 @@
 // keeps the vector ALU for the five operations per element the arithmetic
 // needs (convert, multiply, add, multiply, add).
 //
-// That is the strict form of the arithmetic (slws_kernel, slws_wave_kernel).
-// By default rows of 32, 64, 128 or 256 data bytes with fp32 accumulation run
-// the fused form further down (slws_rows_kernel, slws_groups_kernel): the same
-// sum regrouped into one fused multiply-add per element, equal to the CPU loop
-// to rounding; mi355x_slws_set_fused_math(0) switches back to the strict form.
+// That is the strict form of the arithmetic (slws_kernel, slws_wave_kernel;
+// MI355X_SLWS_MATH_STRICT). By default rows of 32, 64, 128 or 256 data bytes
+// with fp32 accumulation run the fused kernels further down (slws_rows_kernel,
+// slws_groups_kernel): the CPU loop's own expression per element in bag order,
+// with two fused multiply-adds (MI355X_SLWS_MATH_ELEMENT), or on request the
+// sum regrouped into one fused multiply-add per element (_REGROUPED). A call
+// names its arithmetic in mi355x_launch_opts; mi355x_slws_set_fused_math sets
+// what the calls that name none get.
 //
 // The start of a bag in the index list is the exclusive prefix sum of the
 // lengths. A block sums the lengths in front of it itself (from the start of
