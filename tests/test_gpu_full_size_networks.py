@@ -34,7 +34,8 @@ def say(*a):
 def test_resnet50_batch_64_at_224():
     batch, size = 64, 224
     steps = resnet50.build_fp32(0)
-    ranges = resnet50.profile(steps, resnet50.synthetic_images(1, 4, size))
+    # the configuration's own profile: 100 synthetic images
+    ranges = resnet50.profile(steps, resnet50.synthetic_images(1, 100, size))
     net = resnet50.build_int8(steps, ranges, batch, size)
     two = resnet50.build_int8(steps, ranges, 2, size)     # same constants and scales
     x2 = resnet50.synthetic_images(21, 2, size)
