@@ -66,6 +66,9 @@ def parse():
                     help="timed replays of the two networks (at least 20)")
     ap.add_argument("--resnet-batch", type=int, default=64)
     ap.add_argument("--resnet-profile-images", type=int, default=100)
+    ap.add_argument("--resnet-chains", type=int, default=1,
+                    help="compute the ResNet-50 batch as this many independent instruction "
+                         "chains over equal slices of it (constants shared)")
     ap.add_argument("--dlrm-rows", type=int, default=1_000_000)
     ap.add_argument("--no-extra", action="store_true",
                     help="headline workload only")
@@ -653,7 +656,7 @@ def bench_resnet50(args, check=True):
     t0 = time.perf_counter()
     steps = resnet50.build_fp32(0)
     ranges = resnet50.profile(steps, resnet50.synthetic_images(1, args.resnet_profile_images, size))
-    net = resnet50.build_int8(steps, ranges, batch, size)
+    net = resnet50.build_int8(steps, ranges, batch, size, chains=args.resnet_chains)
     t_build = time.perf_counter() - t0
     m, f = netlib.to_module(net)
     m.compile(f)

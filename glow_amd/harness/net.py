@@ -48,12 +48,20 @@ class Net:
     def activation(self, name, shape, kind, scale=1.0, offset=0):
         return self._add(Tensor(name, kind, shape, "activation", scale, offset))
 
-    def view(self, name, source, shape):
-        """The bytes of `source` under another shape (same kind and parameters)."""
+    def view(self, name, source, shape, first=0):
+        """The bytes of `source` under another shape (same kind and parameters),
+        from element `first` of the source on (a slice of a placeholder's or
+        constant's outermost dimension when not 0)."""
         s = self.tensors[source]
         t = Tensor(name, s.kind, shape, "view", s.scale, s.offset)
-        t.source = source
+        t.source, t.first = source, int(first)
+        assert t.first + int(np.prod(t.shape, dtype=np.int64)) <= int(np.prod(s.shape, dtype=np.int64))
         return self._add(t)
+
+    def first_element(self, name):
+        """Where `name` starts inside its root, in elements."""
+        t = self.tensors[name]
+        return t.first + self.first_element(t.source) if t.role == "view" else 0
 
     def root(self, name):
         t = self.tensors[name]
@@ -96,7 +104,8 @@ def to_module(net, function="main"):
         elif t.role == "view":      # sources precede their views in insertion order
             if t.source not in ids:
                 raise ValueError(f"view {t.name} precedes its source {t.source}")
-            ids[t.name] = m.view(t.name, ids[t.source], t.shape, t.kind, t.scale, t.offset)
+            ids[t.name] = m.view(t.name, ids[t.source], t.shape, t.kind, t.scale, t.offset,
+                                 byte_offset=t.first * t.dtype.itemsize)
     for o in net.ops:
         m.instruction(f, o.kind, o.name, [ids[n] for n in o.operands], o.iattrs, o.fattrs)
     return m, f

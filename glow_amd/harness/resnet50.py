@@ -147,88 +147,121 @@ def quantize_fc_bias(bias, weights, in_scale):
     return np.clip(q, -2 ** 31, 2 ** 31 - 1).astype(np.int32), scale, off
 
 
-def build_int8(steps, ranges, batch, size):
-    """The quantized network as lowered instructions."""
+def build_int8(steps, ranges, batch, size, chains=1):
+    """The quantized network as lowered instructions. chains > 1: the batch is
+    computed as that many independent instruction chains over equal slices of
+    the input and output placeholders, sharing every constant (the data-parallel
+    split of Glow's parallelizeOps, reference
+    include/glow/Optimizer/GraphOptimizer/GraphOptimizer.h:199-211): nothing
+    orders one chain's launches against another's, so a device manager may run
+    them side by side."""
+    assert batch % chains == 0
     net = Net("resnet50_int8")
-    shapes = {"input": (batch, size, size, 3)}
     tq = {k: _tqp(v) for k, v in ranges.items()}
-    net.placeholder("input", shapes["input"], H.FLOAT)
-    net.activation("input_q", shapes["input"], H.INT8Q, *tq["input"])
-    net.op(H.QUANTIZE, "quantize", ["input_q", "input"])
-    name_of = {"input": "input_q"}
-    for op, out, ins, prm in steps:
-        src = name_of[ins[0]]
-        ishape = shapes[ins[0]]
-        if op == "conv":
-            n, h, w, ic = ishape
-            oc = prm.w.shape[0]
-            oh = (h + 2 * prm.pad - prm.k) // prm.stride + 1
-            ow = (w + 2 * prm.pad - prm.k) // prm.stride + 1
-            shapes[out] = (n, oh, ow, oc)
-            # what Quantizer::enableChannelwise makes of a Convolution with
-            # constant fp32 filter and bias (createChannelwiseQuantizedConv)
-            q, bq, fs, fo, bs, bo = capi.channelwise_quantize_conv_host(
-                prm.w, prm.b, tq[ins[0]][0], SCHEMA)
-            net.constant(out + "_filter", q, H.INT8Q)
-            net.constant(out + "_bias", bq, H.INT32Q)
-            net.constant(out + "_fscales", fs, H.FLOAT)
-            net.constant(out + "_foffsets", fo, H.INT32I)
-            net.constant(out + "_bscales", bs, H.FLOAT)
-            net.constant(out + "_boffsets", bo, H.INT32I)
-            net.activation(out, shapes[out], H.INT8Q, *tq[out])
-            net.op(H.CHANNELWISE_QUANTIZED_CONV, out,
-                   [out, src, out + "_filter", out + "_bias", out + "_fscales", out + "_foffsets",
-                    out + "_bscales", out + "_boffsets"],
-                   H.conv_attrs((prm.k, prm.k), (prm.stride, prm.stride), (prm.pad,) * 4,
-                                act=H.ACT_RELU if prm.relu else H.ACT_NONE))
-        elif op == "maxpool":
-            k, s, p = prm
-            n, h, w, c = ishape
-            shapes[out] = (n, (h + 2 * p - k) // s + 1, (w + 2 * p - k) // s + 1, c)
-            # max pool passes values through: it keeps its input's parameters
-            tq[out] = tq[ins[0]]
-            net.activation(out, shapes[out], H.INT8Q, *tq[out])
-            net.op(H.MAX_POOL, out, [out, src], [k, k, s, s, p, p, p, p])
-        elif op == "add":
-            shapes[out] = ishape
-            net.activation(out, ishape, H.INT8Q, *tq[out])
-            net.op(H.ELEMENT_ADD, out, [out, src, name_of[ins[1]]])
-        elif op == "relu":
-            shapes[out] = ishape
-            net.activation(out, ishape, H.INT8Q, *tq[out])
-            net.op(H.RELU, out, [out, src])
-        elif op == "avgpool":
-            n, h, w, c = ishape
-            shapes[out] = (n, 1, 1, c)
-            net.activation(out, shapes[out], H.INT8Q, *tq[out])
-            net.op(H.AVG_POOL, out, [out, src], [h, w, 1, 1, 0, 0, 0, 0, 1])
+    per = batch // chains
+    net.placeholder("input", (batch, size, size, 3), H.FLOAT)
+    classes = [prm[0].shape[0] for op, _, _, prm in steps if op == "fc"][0]
+    out_q = None
+    for c in range(chains):
+        sfx = "" if chains == 1 else f"@{c}"
+        first = c == 0
+        shapes = {"input": (per, size, size, 3)}
+        if chains == 1:
+            x = "input"
         else:
-            fw, fb = prm
-            n = ishape[0]
-            classes, k = fw.shape
-            shapes[out] = (n, classes)
-            q, ws, wo = _quantize_rows(fw)
-            bq, bscale, boff = quantize_fc_bias(fb, fw, tq[ins[0]][0])
-            net.constant("fc_weights", q, H.INT8Q)
-            net.constant("fc_bias", bq, H.INT32Q, bscale, boff)
-            net.constant("fc_scales", ws, H.FLOAT)
-            net.constant("fc_offsets", wo, H.INT32I)
-            # the pooled [N,1,1,C] tensor is read as [N,C]: the same bytes (a
-            # Reshape is a TensorView in Glow's IR, no instruction)
-            net.view("gap_2d", src, (n, k))
-            # the int8 logits are an output of the network: the FC writes them
-            # where they are saved
-            net.placeholder("logits_q", shapes[out], H.INT8Q, *tq[out])
-            net.op(H.ROWWISE_QUANTIZED_FC, "fc", ["logits_q", "gap_2d", "fc_weights", "fc_bias",
-                                                  "fc_scales", "fc_offsets"])
-            name_of[out] = "logits_q"
-            continue
-        name_of[out] = out
-    n, classes = shapes["logits"]
-    net.activation("logits_f", (n, classes), H.FLOAT)
-    net.op(H.DEQUANTIZE, "dequantize", ["logits_f", "logits_q"])
-    net.placeholder("prob", (n, classes), H.FLOAT)
-    net.op(H.SOFTMAX, "softmax", ["prob", "logits_f"])
+            x = net.view("input" + sfx, "input", shapes["input"], first=c * per * size * size * 3)
+        net.activation("input_q" + sfx, shapes["input"], H.INT8Q, *tq["input"])
+        net.op(H.QUANTIZE, "quantize" + sfx, ["input_q" + sfx, x])
+        name_of = {"input": "input_q" + sfx}
+        for op, out, ins, prm in steps:
+            src = name_of[ins[0]]
+            ishape = shapes[ins[0]]
+            o = out + sfx
+            if op == "conv":
+                n, h, w, ic = ishape
+                oc = prm.w.shape[0]
+                oh = (h + 2 * prm.pad - prm.k) // prm.stride + 1
+                ow = (w + 2 * prm.pad - prm.k) // prm.stride + 1
+                shapes[out] = (n, oh, ow, oc)
+                if first:
+                    # what Quantizer::enableChannelwise makes of a Convolution with
+                    # constant fp32 filter and bias (createChannelwiseQuantizedConv)
+                    q, bq, fs, fo, bs, bo = capi.channelwise_quantize_conv_host(
+                        prm.w, prm.b, tq[ins[0]][0], SCHEMA)
+                    net.constant(out + "_filter", q, H.INT8Q)
+                    net.constant(out + "_bias", bq, H.INT32Q)
+                    net.constant(out + "_fscales", fs, H.FLOAT)
+                    net.constant(out + "_foffsets", fo, H.INT32I)
+                    net.constant(out + "_bscales", bs, H.FLOAT)
+                    net.constant(out + "_boffsets", bo, H.INT32I)
+                net.activation(o, shapes[out], H.INT8Q, *tq[out])
+                net.op(H.CHANNELWISE_QUANTIZED_CONV, o,
+                       [o, src, out + "_filter", out + "_bias", out + "_fscales",
+                        out + "_foffsets", out + "_bscales", out + "_boffsets"],
+                       H.conv_attrs((prm.k, prm.k), (prm.stride, prm.stride), (prm.pad,) * 4,
+                                    act=H.ACT_RELU if prm.relu else H.ACT_NONE))
+            elif op == "maxpool":
+                k, s, p = prm
+                n, h, w, ch = ishape
+                shapes[out] = (n, (h + 2 * p - k) // s + 1, (w + 2 * p - k) // s + 1, ch)
+                # max pool passes values through: it keeps its input's parameters
+                tq[out] = tq[ins[0]]
+                net.activation(o, shapes[out], H.INT8Q, *tq[out])
+                net.op(H.MAX_POOL, o, [o, src], [k, k, s, s, p, p, p, p])
+            elif op == "add":
+                shapes[out] = ishape
+                net.activation(o, ishape, H.INT8Q, *tq[out])
+                net.op(H.ELEMENT_ADD, o, [o, src, name_of[ins[1]]])
+            elif op == "relu":
+                shapes[out] = ishape
+                net.activation(o, ishape, H.INT8Q, *tq[out])
+                net.op(H.RELU, o, [o, src])
+            elif op == "avgpool":
+                n, h, w, ch = ishape
+                shapes[out] = (n, 1, 1, ch)
+                net.activation(o, shapes[out], H.INT8Q, *tq[out])
+                net.op(H.AVG_POOL, o, [o, src], [h, w, 1, 1, 0, 0, 0, 0, 1])
+            else:
+                fw, fb = prm
+                n = ishape[0]
+                _, k = fw.shape
+                shapes[out] = (n, classes)
+                if first:
+                    q, ws, wo = _quantize_rows(fw)
+                    bq, bscale, boff = quantize_fc_bias(fb, fw, tq[ins[0]][0])
+                    net.constant("fc_weights", q, H.INT8Q)
+                    net.constant("fc_bias", bq, H.INT32Q, bscale, boff)
+                    net.constant("fc_scales", ws, H.FLOAT)
+                    net.constant("fc_offsets", wo, H.INT32I)
+                    # the int8 logits are an output of the network: the FC writes
+                    # them where they are saved
+                    net.placeholder("logits_q", (batch, classes), H.INT8Q, *tq[out])
+                # the pooled [N,1,1,C] tensor is read as [N,C]: the same bytes (a
+                # Reshape is a TensorView in Glow's IR, no instruction)
+                net.view("gap_2d" + sfx, src, (n, k))
+                out_q = "logits_q"
+                if chains > 1:
+                    out_q = net.view("logits_q" + sfx, "logits_q", (n, classes),
+                                     first=c * per * classes)
+                net.op(H.ROWWISE_QUANTIZED_FC, "fc" + sfx,
+                       [out_q, "gap_2d" + sfx, "fc_weights", "fc_bias", "fc_scales", "fc_offsets"])
+                name_of[out] = out_q
+                continue
+            name_of[out] = o
+        net.activation("logits_f" + sfx, (per, classes), H.FLOAT)
+        net.op(H.DEQUANTIZE, "dequantize" + sfx, ["logits_f" + sfx, out_q])
+        if first:
+            net.placeholder("prob", (batch, classes), H.FLOAT)
+        prob = "prob"
+        if chains > 1:
+            prob = net.view("prob" + sfx, "prob", (per, classes), first=c * per * classes)
+        net.op(H.SOFTMAX, "softmax" + sfx, [prob, "logits_f" + sfx])
+    if chains > 1:
+        # step k of every chain before step k + 1 of any: a device manager that
+        # records the list stream by stream then finds each chain's launches
+        # behind one another on a stream of their own, not behind another chain's
+        per_chain = len(net.ops) // chains
+        net.ops = [net.ops[c * per_chain + k] for k in range(per_chain) for c in range(chains)]
     return net
 
 
@@ -237,7 +270,7 @@ def synthetic_images(seed, n, size):
     return rng.normal(0.45, 0.25, (n, size, size, 3)).astype(np.float32)
 
 
-def make(batch=64, size=224, profile_images=100, seed=0, layers=LAYERS, classes=1000):
+def make(batch=64, size=224, profile_images=100, seed=0, layers=LAYERS, classes=1000, chains=1):
     steps = build_fp32(seed, layers, classes)
     ranges = profile(steps, synthetic_images(seed + 1, profile_images, size))
-    return build_int8(steps, ranges, batch, size)
+    return build_int8(steps, ranges, batch, size, chains)

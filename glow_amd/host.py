@@ -28,7 +28,7 @@ ERROR_NAMES = ["SUCCESS", "UNKNOWN", "RUNTIME_ERROR", "RUNTIME_OUT_OF_DEVICE_MEM
 EXPORTS = [
     "mi355x_host_last_error", "mi355x_host_error_name", "mi355x_host_module_create",
     "mi355x_host_module_destroy", "mi355x_host_add_constant", "mi355x_host_add_placeholder",
-    "mi355x_host_create_function", "mi355x_host_add_activation", "mi355x_host_add_view",
+    "mi355x_host_create_function", "mi355x_host_add_activation", "mi355x_host_add_view", "mi355x_host_add_view_at",
     "mi355x_host_add_instruction", "mi355x_host_is_op_supported", "mi355x_host_compile",
     "mi355x_host_describe", "mi355x_host_bundle_sizes", "mi355x_host_dm_create", "mi355x_host_dm_create_opts",
     "mi355x_host_dm_destroy", "mi355x_host_dm_init", "mi355x_host_dm_stop",
@@ -124,8 +124,12 @@ class Module:
         return _check(lib().mi355x_host_add_activation(
             self._h, fn, name.encode(), kind, d, nd, C.c_float(scale), C.c_int32(offset)))
 
-    def view(self, name, source, shape, kind, scale=1.0, offset=0):
+    def view(self, name, source, shape, kind, scale=1.0, offset=0, byte_offset=0):
         d, nd = _dims(shape)
+        if byte_offset:
+            return _check(lib().mi355x_host_add_view_at(
+                self._h, name.encode(), source, kind, d, nd, C.c_float(scale), C.c_int32(offset),
+                C.c_size_t(byte_offset)))
         return _check(lib().mi355x_host_add_view(
             self._h, name.encode(), source, kind, d, nd, C.c_float(scale), C.c_int32(offset)))
 

@@ -338,8 +338,11 @@ private:
                "operand %zu is an activation of another function", i);
       CHECK_OP(!(i == 0 && v.category == SymbolCategory::Constant),
                "destination is a constant");
-      auto &f = io_[id];
-      if (i == 0) f.second = true; else f.first = true;
+      // (a placeholder read or written through a view is an input or output itself)
+      for (int who : {id, v.root}) {
+        auto &f = io_[who];
+        if (i == 0) f.second = true; else f.first = true;
+      }
     }
     return Error::success();
   }

@@ -110,15 +110,17 @@ const char *kindName(Kind k) {
   }
 }
 
-int Module::createView(const std::string &name, int src, const Type &t) {
+int Module::createView(const std::string &name, int src, const Type &t, size_t byteOffset) {
   if (!validId(src)) return -1;
   const Value &s = values_[(size_t)src];
-  if (t.sizeInBytes() > s.type.sizeInBytes()) return -1;
+  if (byteOffset > s.type.sizeInBytes() || t.sizeInBytes() > s.type.sizeInBytes() - byteOffset)
+    return -1;
+  if (byteOffset != 0 && s.category == SymbolCategory::Activation) return -1;
   Value v;
   v.name = name;
   v.type = t;
   v.category = s.category;
-  v.offset = s.offset;
+  v.offset = s.offset + byteOffset;
   v.function = s.function;
   v.root = s.root;
   return addValue(std::move(v));

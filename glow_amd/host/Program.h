@@ -169,9 +169,12 @@ public:
   // Module::createPlaceholder
   int createPlaceholder(const std::string &name, const Type &t);
   Function *createFunction(const std::string &name);
-  // TensorViewInst: another type over the bytes of `src` (a reshape); the view
-  // must not be larger than its source. Returns -1 when it is.
-  int createView(const std::string &name, int src, const Type &t);
+  // TensorViewInst: another type over the bytes of `src` from `byteOffset` on (a
+  // reshape, or a slice of the outermost dimension); the view must lie inside
+  // its source. Returns -1 when it does not, or when a view that does not
+  // start at its source's first byte is asked of an activation (activations are
+  // placed by the backend; placeholders and constants have fixed offsets).
+  int createView(const std::string &name, int src, const Type &t, size_t byteOffset = 0);
 
   const Value &value(int id) const { return values_.at((size_t)id); }
   bool validId(int id) const { return id >= 0 && (size_t)id < values_.size(); }

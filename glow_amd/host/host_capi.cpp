@@ -86,6 +86,20 @@ int mi355x_host_add_view(mi355x_host_module *m, const char *name, int source, in
   return id;
 }
 
+int mi355x_host_add_view_at(mi355x_host_module *m, const char *name, int source, int kind,
+                            const int64_t *dims, int nd, float scale, int32_t offset,
+                            size_t byte_offset) {
+  if (!m || !name || !kindOk(kind) || (nd > 0 && !dims))
+    return failMsg(ErrorCode::COMPILE_CONTEXT_MALFORMED, "invalid view description");
+  const int id =
+      m->module.createView(name, source, makeType(kind, dims, nd, scale, offset), byte_offset);
+  if (id < 0)
+    return failMsg(ErrorCode::COMPILE_CONTEXT_MALFORMED,
+                   "view " + std::string(name) +
+                       " does not fit its source (or slices an activation)");
+  return id;
+}
+
 int mi355x_host_add_instruction(mi355x_host_module *m, int function, int kind, const char *name,
                                 const int *operands, int n_operands, const int64_t *iattrs,
                                 int n_iattrs, const float *fattrs, int n_fattrs) {

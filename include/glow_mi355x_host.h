@@ -102,6 +102,12 @@ int mi355x_host_add_activation(mi355x_host_module *m, int function, const char *
 /* TensorViewInst: a value of another type over the bytes of `source` (reshape). */
 int mi355x_host_add_view(mi355x_host_module *m, const char *name, int source, int elem_kind,
                          const int64_t *dims, int ndims, float scale, int32_t offset);
+/* The same with the view starting `byte_offset` bytes into a placeholder or
+ * constant (a slice of its outermost dimension, as TensorViewInst's offsets
+ * give; reference lib/Backends/BackendUtils.cpp:600-636). */
+int mi355x_host_add_view_at(mi355x_host_module *m, const char *name, int source, int elem_kind,
+                            const int64_t *dims, int ndims, float scale, int32_t offset,
+                            size_t byte_offset);
 int mi355x_host_add_instruction(mi355x_host_module *m, int function, int kind, const char *name,
                                 const int *operands, int n_operands, const int64_t *iattrs,
                                 int n_iattrs, const float *fattrs, int n_fattrs);

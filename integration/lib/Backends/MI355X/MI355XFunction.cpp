@@ -242,11 +242,20 @@ private:
       return Error::success();
     case Kinded::Kind::TensorViewInstKind: {
       const auto *TV = cast<TensorViewInst>(&I);
-      // a reshape of the whole buffer; slices by offset are not a view here
-      for (dim_t o : TV->getOffsets()) {
-        if (o != 0) {
-          return unsupported(I, "tensor views with offsets are not supported");
+      // a reshape of the buffer, or a slice of the outermost dimension of a
+      // placeholder or constant (the bytes stay contiguous): the flat offset of
+      // Tensor::getUnowned(ty, offsets) for offsets = {o, 0, 0, ...}
+      size_t byteOffset = 0;
+      const auto offs = TV->getOffsets();
+      for (size_t k = 1; k < offs.size(); k++) {
+        if (offs[k] != 0) {
+          return unsupported(I, "tensor views with inner offsets are not supported");
         }
+      }
+      if (!offs.empty() && offs[0] != 0) {
+        const TypeRef srcTy = TV->getSrc()->getType();
+        byteOffset = (size_t)offs[0] * (srcTy->size() / srcTy->dims()[0]) *
+                     srcTy->getElementSize();
       }
       hm::Type ty;
       if (!toHostType(*TV->getTy(), ty)) {
@@ -254,9 +263,9 @@ private:
       }
       int src;
       ASSIGN_VALUE_OR_RETURN_ERR(src, idOf(I, TV->getSrc()));
-      const int id = out_.createView(I.getName().str(), src, ty);
+      const int id = out_.createView(I.getName().str(), src, ty, byteOffset);
       if (id < 0) {
-        return unsupported(I, "view larger than its source");
+        return unsupported(I, "view outside its source, or a slice of an activation");
       }
       ids_[&I] = id;
       return Error::success();

@@ -35,13 +35,15 @@ class _Values:
     def get(self, name):
         t = self.net.tensors[name]
         n = int(np.prod(t.shape, dtype=np.int64))
-        return self._storage(name)[:n].reshape(t.shape)
+        at = self.net.first_element(name)
+        return self._storage(name)[at:at + n].reshape(t.shape)
 
     def set(self, name, value):
         t = self.net.tensors[name]
         value = np.asarray(value)
         flat = self._storage(name)
-        flat[:value.size] = value.astype(t.dtype, copy=False).ravel()
+        at = self.net.first_element(name)
+        flat[at:at + value.size] = value.astype(t.dtype, copy=False).ravel()
 
     def __getitem__(self, name):
         return self.get(name)

@@ -98,3 +98,64 @@ def test_device_matches_oracle(fuse):
         assert dm.time_function("main", 3) > 0
     finally:
         dm.stop()
+
+
+def test_batch_as_independent_chains_is_the_same_network_on_the_oracle():
+    """The batch computed as chains over slices of the input and output
+    placeholders (views that start inside their source, constants shared)
+    gives the single chain's outputs; in the launch list no chain's launch
+    depends on another chain's before the outputs."""
+    steps = resnet50.build_fp32(3, SMALL, 10)
+    ranges = resnet50.profile(steps, resnet50.synthetic_images(4, 4, 32))
+    one = resnet50.build_int8(steps, ranges, 4, 32)
+    two = resnet50.build_int8(steps, ranges, 4, 32, chains=2)
+    assert len(two.ops) == 2 * len(one.ops)
+    assert sum(t.role == "constant" for t in two.tensors.values()) == \
+        sum(t.role == "constant" for t in one.tensors.values())
+    x = resnet50.synthetic_images(9, 4, 32)
+    a, b = oracle_exec.run(one, {"input": x}), oracle_exec.run(two, {"input": x})
+    np.testing.assert_array_equal(a["logits_q"], b["logits_q"])
+    np.testing.assert_array_equal(a["prob"], b["prob"])
+    m, f = netlib.to_module(two)
+    m.compile(f)
+    rows = [r for r in H.parse_listing(m.describe(f)) if r["phase"] == "launch"]
+    levels = {c: [r["level"] for r in rows if r["inst"].split("+")[0].endswith(f"@{c}")]
+              for c in (0, 1)}
+    # (the launches that write the shared output placeholders are ordered)
+    assert levels[0][:-3] == levels[1][:-3] and levels[0][0] == 0
+
+
+def test_views_that_start_inside_their_source():
+    m = H.Module("views")
+    p = m.placeholder("p", (4, 8), H.INT8Q, np.int8, 0.1, 0)
+    f = m.function("main")
+    act = m.activation(f, "a", (4, 8), H.INT8Q, 0.1, 0)
+    assert m.view("rows23", p, (2, 8), H.INT8Q, 0.1, 0, byte_offset=16) >= 0
+    with pytest.raises(H.HostError):
+        m.view("past_the_end", p, (2, 8), H.INT8Q, 0.1, 0, byte_offset=24)
+    with pytest.raises(H.HostError):        # activations are placed by the backend
+        m.view("of_activation", act, (2, 8), H.INT8Q, 0.1, 0, byte_offset=16)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("chains", [2, 4])
+def test_device_runs_the_batch_as_independent_chains(chains):
+    steps = resnet50.build_fp32(5, ((64, 2, 1), (128, 1, 2)), 100)
+    ranges = resnet50.profile(steps, resnet50.synthetic_images(6, 4, 64))
+    net = resnet50.build_int8(steps, ranges, 4, 64, chains=chains)
+    m, f = netlib.to_module(net)
+    m.compile(f)
+    dm = H.DeviceManager().init()
+    try:
+        dm.add_network(m)
+        # more requests than the device manager spends on choosing a recording
+        for seed in range(12):
+            x = resnet50.synthetic_images(20 + seed, 4, 64)
+            logits = np.zeros((4, 100), np.int8)
+            prob = np.zeros((4, 100), np.float32)
+            dm.run("main", {"input": x, "logits_q": logits, "prob": prob})
+            want = oracle_exec.run(net, {"input": x})
+            np.testing.assert_array_equal(logits, want["logits_q"])
+            np.testing.assert_allclose(prob, want["prob"], rtol=1e-5, atol=1e-30)
+    finally:
+        dm.stop()
