@@ -501,7 +501,7 @@ int mi355x_rwq_fc_i8_opts(int8_t *out, const int8_t *in, const int8_t *weights,
                      int32_t out_offset, int32_t in_offset,
                      int32_t bias_offset, int weights_offsets_all_zero,
                      const int32_t *weights_row_sums, void *stream,
-    const mi355x_launch_opts *opts);
+                     const mi355x_launch_opts *opts);
 
 /* RowwiseQuantizedFullyConnected followed by a Relu instruction of its result
  * (libjit_element_relu_i8, reference libjit.cpp:1851-1858, parameters from
@@ -529,7 +529,7 @@ int mi355x_rwq_fc_relu_i8_opts(int8_t *out, const int8_t *in, const int8_t *weig
                           int weights_offsets_all_zero, const int32_t *weights_row_sums,
                           int32_t relu_offset, int32_t relu_pre, int32_t relu_post,
                           int32_t relu_scale, void *stream,
-    const mi355x_launch_opts *opts);
+                          const mi355x_launch_opts *opts);
 
 /* libjit_fc_i8_i32 / _i8_i8 (libjit_matmul.cpp:254-280, 395-422).
  * weights_kn is [K x N] as Glow stores FullyConnected weights; the kernel
@@ -553,7 +553,7 @@ int mi355x_fc_i8_opts(int8_t *out, const int8_t *in, const int8_t *weights_kn,
                  int32_t bias_scale, int32_t out_pre, int32_t out_post,
                  int32_t out_scale, const int32_t *weights_row_sums,
                  void *stream,
-    const mi355x_launch_opts *opts);
+                 const mi355x_launch_opts *opts);
 
 /* libjit_matmul_i8 (libjit_matmul.cpp:353-371). lhs [M x K], rhs_kn [K x N];
  * workspace and repack as for mi355x_fc_i8. */
@@ -567,7 +567,7 @@ int mi355x_matmul_i8_opts(int8_t *out, const int8_t *lhs, const int8_t *rhs_kn,
                      size_t N, int32_t out_offset, int32_t lhs_offset,
                      int32_t rhs_offset, int32_t out_pre, int32_t out_post,
                      int32_t out_scale, void *stream,
-    const mi355x_launch_opts *opts);
+                     const mi355x_launch_opts *opts);
 
 /* Tuning aid (no counterpart in the reference): forces the workgroup tile of
  * the following matrix-core launches of the calling thread: 0 = 256x256,
@@ -673,7 +673,7 @@ int mi355x_cwq_conv2d_i8_opts(int8_t *out, const int8_t *in, const int8_t *filte
                          const int32_t *act_args,
                          int filter_offsets_all_zero,
                          const int32_t *filter_row_sums, void *stream,
-    const mi355x_launch_opts *opts);
+                         const mi355x_launch_opts *opts);
 
 /* NTHWC input [N,IT,IH,IW,IC], filter [OC,KT,KH,KW,IC/group], output
  * [N,OT,OH,OW,OC]; pads are {near, top, left}; the output size carries
@@ -757,7 +757,7 @@ int mi355x_conv2d_i8_opts(int8_t *out, const int8_t *in, const int8_t *filter,
                      int32_t out_scale, int32_t act_type,
                      const int32_t *act_args, const int32_t *filter_row_sums,
                      void *stream,
-    const mi355x_launch_opts *opts);
+                     const mi355x_launch_opts *opts);
 
 /* ---- fused-rowwise SparseLengths(Weighted)Sum ----------------------------------- */
 
@@ -793,7 +793,7 @@ int mi355x_frwq_slws_opts(void *dest, int out_is_f16, const uint8_t *data,
                      size_t num_indices, const int32_t *lengths,
                      size_t segments, size_t in_line_size,
                      size_t out_line_size, int fp16_accum, void *stream,
-    const mi355x_launch_opts *opts);
+                     const mi355x_launch_opts *opts);
 
 /* mi355x_frwq_slws with the bags given as positions instead of lengths: the
  * same operator (libjit.cpp:1253-1276; InterpreterNodes.cpp:5764-5889) for a
@@ -818,7 +818,7 @@ int mi355x_frwq_slws_offsets_opts(void *dest, int out_is_f16, const uint8_t *dat
                              size_t num_indices, const int32_t *bag_offsets,
                              size_t segments, size_t in_line_size,
                              size_t out_line_size, int fp16_accum, void *stream,
-    const mi355x_launch_opts *opts);
+                             const mi355x_launch_opts *opts);
 
 /* Host side, no GPU call: bag_offsets[0] = 0, bag_offsets[i + 1] =
  * bag_offsets[i] + max(lengths[i], 0) (negative lengths count as empty bags,
@@ -862,7 +862,7 @@ int mi355x_frwq_slws_noalloc_opts(void *dest, int out_is_f16, const uint8_t *dat
                              size_t num_indices, const int32_t *lengths,
                              size_t segments, size_t in_line_size,
                              size_t out_line_size, int fp16_accum, void *stream,
-    const mi355x_launch_opts *opts);
+                             const mi355x_launch_opts *opts);
 
 /* Process-wide default of mi355x_launch_opts::slws_math for the calls that do
  * not name an arithmetic themselves (the plain entry points, and _opts calls
@@ -899,7 +899,7 @@ int mi355x_rwq_slws_opts(float *dest, const uint8_t *data, size_t data_rows,
                     const void *indices, int idx_is_64, size_t num_indices,
                     const int32_t *lengths, size_t segments, size_t line_size,
                     void *stream,
-    const mi355x_launch_opts *opts);
+                    const mi355x_launch_opts *opts);
 
 /* FusedRowwiseQuantizedSparseLengthsSum over several tables of one shape in ONE
  * launch (a ranking model pools dozens of tables per request, each too small
@@ -943,7 +943,7 @@ int mi355x_frwq_sls_multi_opts(const mi355x_sls_table *tables, size_t n_tables,
                           size_t out_line_size, int out_kind, float out_scale,
                           int32_t out_offset, size_t dest_row_stride,
                           int fp16_accum, void *stream,
-    const mi355x_launch_opts *opts);
+                          const mi355x_launch_opts *opts);
 
 /* libjit_embedding_bag_byte_rowwise_offsets_f (libjit.cpp:2454-2481) and the
  * Interpreter's 4-bit / fp16 twin: bags are given by int32 start offsets
