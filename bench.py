@@ -429,7 +429,7 @@ def oracle_rows_check(capi, c, d_out, M, rows):
 
 
 def bench_fc(capi, cases, M, K, N, steps, warmup, seed=5, zero_leg=False, check=True,
-             clock=False, use_hint=False):
+             clock=False, use_hint=False, split_k=False):
     c = cases.rwq_fc_case(seed, M, K, N) if M * K <= (1 << 24) else None
     rng = np.random.default_rng(seed)
     if c is None:
@@ -445,13 +445,21 @@ def bench_fc(capi, cases, M, K, N, steps, warmup, seed=5, zero_leg=False, check=
     d_sums = capi.DeviceBuffer.empty((N,), np.int32)
     capi.launch_rowsum_i8(d_sums, d["w"], N, K)
 
+    opts = None
+    if split_k:
+        # a zero-filled workspace with the call: the library may split the K loop
+        # over workgroups (it does when the grid would leave half the CUs idle)
+        ws = capi.DeviceBuffer(max(256, capi.gemm_splitk_workspace_bytes(M, N, K)))
+        ws.fill(0)
+        opts = capi.LaunchOpts(workspace=ws)
+
     def step(_, stream):
         capi.launch_rwq_fc_i8(d_out, d["x"], d["w"], d["bias"], False,
                               d["w_offsets"], d["bias_pre"], d["bias_post"],
                               d["bias_scale"], d["out_pre"], d["out_post"],
                               d["out_scale"], M, K, N, c["out_offset"],
                               c["in_offset"], c["bias_offset"], True,
-                              w_row_sums=d_sums, stream=stream)
+                              w_row_sums=d_sums, stream=stream, opts=opts)
 
     hint = 0
     if use_hint:
@@ -920,6 +928,16 @@ def main():
         # the single-FC configuration's own K and N at a large batch
         extra["rwq_fc_m16384"] = bench_fc(capi, cases, 16384, 1024, 1024, max(st, 300),
                                           max(wu, 30))
+        # few output tiles and a long K (the product of ResNet-50's 7x7 stage
+        # 3x3 convolutions): as it runs by itself, and with a workspace in the
+        # call's options, which lets the library split K over workgroups
+        plain = bench_fc(capi, cases, 3136, 4608, 512, max(st, 100), max(wu, 10))
+        split = bench_fc(capi, cases, 3136, 4608, 512, max(st, 100), max(wu, 10), split_k=True)
+        extra["rwq_fc_split_k"] = dict(
+            workload="rwq_fc M3136 K4608 N512 (100 tiles of 128x128)",
+            ms=plain["ms"], ms_with_workspace=split["ms"],
+            workspace_bytes=capi.gemm_splitk_workspace_bytes(3136, 512, 4608),
+            parity_with_oracle=bool(plain["parity_with_oracle"] and split["parity_with_oracle"]))
         extra["cwq_conv_c3"] = bench_conv(capi, cases, args.steps, args.warmup)
         for w in ("quantize", "dequantize", "rescale"):
             extra[w] = bench_elementwise(capi, w, st, wu)

@@ -22,7 +22,7 @@ EXPORTS = [
     "mi355x_last_error", "mi355x_num_devices", "mi355x_init", "mi355x_rwq_fc_i8_opts", "mi355x_rwq_fc_relu_i8_opts", "mi355x_fc_i8_opts", "mi355x_matmul_i8_opts", "mi355x_cwq_conv2d_i8_opts", "mi355x_cwq_conv2d_add_i8_opts", "mi355x_conv2d_i8_opts", "mi355x_frwq_slws_opts", "mi355x_frwq_slws_offsets_opts", "mi355x_frwq_slws_noalloc_opts", "mi355x_frwq_sls_multi_opts", "mi355x_rwq_slws_opts", "mi355x_embedding_bag_rowwise_offsets_opts", "mi355x_frwq_slws_probe",
     "mi355x_device_info", "mi355x_malloc", "mi355x_free", "mi355x_host_alloc",
     "mi355x_host_free", "mi355x_memcpy_h2d", "mi355x_memcpy_d2h",
-    "mi355x_memcpy_d2d", "mi355x_fill_u8", "mi355x_copy_u8", "mi355x_gemm_tile_override",
+    "mi355x_memcpy_d2d", "mi355x_fill_u8", "mi355x_copy_u8", "mi355x_gemm_tile_override", "mi355x_gemm_splitk_workspace_bytes",
     "mi355x_cwq_conv2d_add_i8", "mi355x_frwq_sls_multi",
     "mi355x_specialize_bias_weights_qparams", "mi355x_rwq_slws", "mi355x_slws_set_fused_math", "mi355x_batch_matmul_nt_i8", "mi355x_batch_matmul_nt_select_i8", "mi355x_rwq_fc_relu_i8", "mi355x_add_i8", "mi355x_add_relu_i8",
     "mi355x_relu_i8", "mi355x_clip_i8", "mi355x_leaky_relu_i8", "mi355x_max_splat_i8", "mi355x_batched_add_i8", "mi355x_convert_f16_to_f32", "mi355x_insert_rows",
@@ -550,10 +550,27 @@ class LaunchOpts(C.Structure):
     entry point (workgroup tile, requantisation hint, SparseLengths
     arithmetic)."""
     _fields_ = [("struct_size", C.c_uint32), ("gemm_tile", C.c_int32),
-                ("requant_hint", C.c_int32), ("slws_math", C.c_int32)]
+                ("requant_hint", C.c_int32), ("slws_math", C.c_int32),
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64)]
 
-    def __init__(self, gemm_tile=-1, requant_hint=0, slws_math=-1):
-        super().__init__(C.sizeof(LaunchOpts), gemm_tile, requant_hint, slws_math)
+    def __init__(self, gemm_tile=-1, requant_hint=0, slws_math=-1, workspace=None):
+        """workspace: a zero-filled DeviceBuffer for launches that split K over
+        workgroups (gemm_splitk_workspace_bytes), or None."""
+        super().__init__(C.sizeof(LaunchOpts), gemm_tile, requant_hint, slws_math,
+                         workspace.ptr if workspace is not None else None,
+                         workspace.nbytes if workspace is not None else 0)
+        self._keep = workspace
+
+
+TILE_SPLIT_K = 12
+
+
+def gemm_splitk_workspace_bytes(M, N, K, groups=1, named=False):
+    """Bytes of workspace a K-split launch of this product uses (0: none)."""
+    n = C.c_size_t(0)
+    check(lib().mi355x_gemm_splitk_workspace_bytes(_sz(M), _sz(N), _sz(K), _sz(groups),
+                                                   C.c_int(int(named)), C.byref(n)))
+    return n.value
 
 
 def _entry(name, opts):
@@ -727,7 +744,7 @@ def _row_sums_dev(d_rows, n, K, wanted):
 
 def rwq_fc_i8(x, w_nk, bias, w_offsets, bias_pre, bias_post, bias_scale,
               out_pre, out_post, out_scale, out_offset, in_offset, bias_offset,
-              w_offsets_all_zero=None, precomputed_sums=True):
+              w_offsets_all_zero=None, precomputed_sums=True, opts=None):
     x = np.ascontiguousarray(x, np.int8)
     w_nk = np.ascontiguousarray(w_nk, np.int8)
     M, K = x.shape
@@ -741,7 +758,7 @@ def rwq_fc_i8(x, w_nk, bias, w_offsets, bias_pre, bias_post, bias_scale,
     d_out = DeviceBuffer.empty((M, N), np.int8)
     d_sums = _row_sums_dev(d_w, N, K, precomputed_sums)
     launch_rwq_fc_i8(d_out, d_x, d_w, d_b, b8, *vs, M, K, N, out_offset,
-                     in_offset, bias_offset, w_offsets_all_zero, d_sums)
+                     in_offset, bias_offset, w_offsets_all_zero, d_sums, opts=opts)
     return d_out.numpy()
 
 
@@ -820,7 +837,7 @@ def transpose2d_i8(a):
 def cwq_conv2d_i8(x, filt, bias, geom, out_offset, in_offset, f_offsets,
                   b_offsets, bias_pre, bias_post, bias_scale, out_pre, out_post,
                   out_scale, act=ACT_NONE, act_args=(), f_offsets_all_zero=None,
-                  precomputed_sums=True):
+                  precomputed_sums=True, opts=None):
     g = _geom(geom)
     x = np.ascontiguousarray(x, np.int8)
     filt = np.ascontiguousarray(filt, np.int8)
@@ -833,7 +850,7 @@ def cwq_conv2d_i8(x, filt, bias, geom, out_offset, in_offset, f_offsets,
     d_out = DeviceBuffer.empty((g.N, g.OH, g.OW, g.OC), np.int8)
     d_sums = _row_sums_dev(d_f, g.OC, filt.size // g.OC, precomputed_sums)
     launch_cwq_conv2d_i8(d_out, d_x, d_f, d_b, b8, g, out_offset, in_offset,
-                         *vs, act, act_args, f_offsets_all_zero, d_sums)
+                         *vs, act, act_args, f_offsets_all_zero, d_sums, opts=opts)
     return d_out.numpy()
 
 

@@ -43,18 +43,26 @@ int slws_init_device();
 extern thread_local int g_tile_override;   // -1: chosen from the shape
 extern thread_local int g_requant_hint;    // MI355X_REQUANT_* flags
 extern thread_local int g_slws_math;       // -1: the process default
+extern thread_local void *g_workspace;     // device memory a matrix-core launch may use
+extern thread_local size_t g_workspace_bytes;
 
 struct OptsScope {
   int rc = MI355X_OK;
   int tile, hint, math;
+  void *ws;
+  size_t ws_bytes;
+  // the struct may end behind slws_math (callers built before the workspace
+  // fields existed) or hold all of it
+  static constexpr size_t kSizeWithoutWorkspace = offsetof(mi355x_launch_opts, workspace);
   explicit OptsScope(const mi355x_launch_opts *o)
-      : tile(g_tile_override), hint(g_requant_hint), math(g_slws_math) {
+      : tile(g_tile_override), hint(g_requant_hint), math(g_slws_math), ws(g_workspace),
+        ws_bytes(g_workspace_bytes) {
     if (!o) return;
-    if (o->struct_size != sizeof(mi355x_launch_opts)) {
+    if (o->struct_size != sizeof(mi355x_launch_opts) && o->struct_size != kSizeWithoutWorkspace) {
       rc = fail(MI355X_ERR_INVALID_ARGUMENT, "mi355x_launch_opts: struct_size %u, expected %zu",
                 o->struct_size, sizeof(mi355x_launch_opts));
-    } else if (o->gemm_tile < -1 || o->gemm_tile > 11) {
-      rc = fail(MI355X_ERR_INVALID_ARGUMENT, "gemm_tile %d outside [-1, 11]", o->gemm_tile);
+    } else if (o->gemm_tile < -1 || o->gemm_tile > 12) {
+      rc = fail(MI355X_ERR_INVALID_ARGUMENT, "gemm_tile %d outside [-1, 12]", o->gemm_tile);
     } else if (o->requant_hint < 0 || o->requant_hint > 3 || o->requant_hint == 2) {
       rc = fail(MI355X_ERR_INVALID_ARGUMENT,
                 "requant_hint %d: bit 1 (no pre-shifts) needs bit 0 (24-bit operands)",
@@ -65,12 +73,17 @@ struct OptsScope {
       g_tile_override = o->gemm_tile;
       g_requant_hint = o->requant_hint;
       g_slws_math = o->slws_math;
+      const bool has_ws = o->struct_size == sizeof(mi355x_launch_opts);
+      g_workspace = has_ws ? o->workspace : nullptr;
+      g_workspace_bytes = has_ws && o->workspace ? (size_t)o->workspace_bytes : 0;
     }
   }
   ~OptsScope() {
     g_tile_override = tile;
     g_requant_hint = hint;
     g_slws_math = math;
+    g_workspace = ws;
+    g_workspace_bytes = ws_bytes;
   }
   OptsScope(const OptsScope &) = delete;
   OptsScope &operator=(const OptsScope &) = delete;

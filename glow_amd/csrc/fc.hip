@@ -11,6 +11,8 @@
 namespace mi355x {
 
 thread_local int g_tile_override = -1;
+thread_local void *g_workspace = nullptr;
+thread_local size_t g_workspace_bytes = 0;
 thread_local int g_requant_hint = 0;
 
 // dst [cols x rows] = src [rows x cols]^T through a 64x64 LDS tile.
@@ -115,8 +117,21 @@ using namespace mi355x;
 extern "C" {
 
 int mi355x_gemm_tile_override(int tile) {
-  MI355X_REQUIRE(tile >= -1 && tile <= 11, "tile %d outside [-1, 11]", tile);
+  MI355X_REQUIRE(tile >= -1 && tile <= 12, "tile %d outside [-1, 12]", tile);
   g_tile_override = tile;
+  return MI355X_OK;
+}
+
+int mi355x_gemm_splitk_workspace_bytes(size_t M, size_t N, size_t K, size_t groups, int named,
+                                       size_t *bytes) {
+  MI355X_REQUIRE(bytes, "NULL result");
+  *bytes = 0;
+  if (M == 0 || N == 0 || K < 2 * (size_t)kBK || K % kBK != 0 || groups == 0) return MI355X_OK;
+  MI355X_REQUIRE(M < (1ull << 31) && N < (1ull << 31) && K < (1ull << 31) && groups < 65536,
+                 "problem too large");
+  const GemmShape g{(int)M, (int)N, (int)K, (int)groups, 0};
+  const int splits = splitk_choice(g, gemm_cus(), named != 0);
+  if (splits >= 2) *bytes = splitk_workspace_bytes(g, splits);
   return MI355X_OK;
 }
 

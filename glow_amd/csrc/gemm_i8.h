@@ -1012,8 +1012,21 @@ __device__ __forceinline__ uint32_t lds_address(const void *p) {
 // past the end then go to the last tile's own slot (the same bytes again)
 // instead of slots nobody consumes. Only the 128x128 tile without in-kernel
 // row sums has this variant; it is compiled for four waves per SIMD.
+// K split over workgroups (blockIdx.z = the split): every workgroup of an
+// output tile multiplies its share of the K steps and leaves its int32
+// accumulators in the caller's workspace; the one that arrives last at the
+// tile's counter adds the others' to its own (int32 sums wrap, so the order
+// does not matter: the reference's sum, libjit_matmul.cpp:284-316) and runs the
+// epilogue. Nobody waits for anybody. Counters are zero before a launch and
+// are left zero by it.
+struct SplitK {
+  int32_t *partials = nullptr;   // [group][tile][split][BM * BN], in the accumulators' own order
+  uint32_t *counters = nullptr;  // [group][tile]
+  int splits = 1;
+};
+
 template <int BM, int BN, int WM, int WN, int STAGES, bool NEED_SA,
-          bool NEED_SB, class ARows, bool SHORT = false>
+          bool NEED_SB, class ARows, bool SHORT = false, bool SPLITK = false>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
                              ((BM / WM) * (BN / WN) == 8 && BM * BN <= 256 * 128)
                                  ? (BM * BN == 256 * 128 ? 1 : 2)
@@ -1022,7 +1035,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
                              : (BM * BN == 128 * 128) ? 3
                                                       : 1) void gemm_i8_dma_kernel(
     ARows A, DenseRows B, Epilogue ep, int M, int N, int K, int tiles_m,
-    int tiles_n, long long b_group_stride, int n_per_group) {
+    int tiles_n, long long b_group_stride, int n_per_group, SplitK sk) {
+  static_assert(!SPLITK || (!NEED_SA && !NEED_SB && !SHORT), "split K: no in-kernel row sums");
   constexpr int WAVES_N = BN / WN;
   constexpr int WAVES = (BM / WM) * (BN / WN);
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -1071,7 +1085,16 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
     b_dst[i] = lds0 + BM * kBK + g * 1024;
   }
 
-  const int KT = K / kBK;
+  // this workgroup's K steps: all of them, or its share (every split has at
+  // least one: the launch sees to that)
+  int KT = K / kBK, k_begin = 0;
+  if constexpr (SPLITK) {
+    const int per = (KT + sk.splits - 1) / sk.splits;
+    k_begin = (int)blockIdx.z * per * kBK;
+    KT = min(per, KT - (int)blockIdx.z * per);
+#pragma unroll
+    for (int i = 0; i < B_LOADS; i++) bptr[i] += k_begin;
+  }
   // A tile's loads are issued in two halves, H0 then H1, so that the memory
   // pipeline sees a steady trickle instead of one burst per K step.
   constexpr int H0 = LOADS / 2;
@@ -1079,7 +1102,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
   // every row of the tile and both halves of its loads)
   // Tiles are located in order, one K step at a time (nk never decreases and
   // grows by at most one between calls; past the end the last tile stays).
-  typename ARows::Loc run_loc = A.locate(kc_lane);
+  typename ARows::Loc run_loc = A.locate(kc_lane + k_begin);
   int run_tile = 0;
   auto locate_tile = [&](int nk) {
     const int t = min(nk, KT - 1);
@@ -1242,6 +1265,53 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
   }
   dma_wait<0>(); // drain the re-reads before LDS is reused
   __syncthreads();
+  if constexpr (SPLITK) {
+    constexpr int THREADS = WAVES * 64;
+    const size_t tile_id = (size_t)grp * ((size_t)tiles_m * tiles_n) + blockIdx.x;
+    int32_t *mine = sk.partials + (tile_id * sk.splits + blockIdx.z) * (size_t)(BM * BN);
+    // Accumulators as they lie in the registers: value v of a lane at
+    // [v][thread]. The sums pass between workgroups that may sit on different
+    // dies, each with an L2 of its own: they are stored and loaded as
+    // device-scope accesses (written through to, and read from, the memory
+    // side), which costs nothing beyond the access itself. A device-scope
+    // fence would write back and invalidate the whole L2 once per workgroup
+    // (measured: 65 us on top of a 20 us launch).
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+          __hip_atomic_store(mine + ((i * TN + j) * 16 + r) * THREADS + tid, acc[i][j][r],
+                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // every store of this workgroup has been acknowledged before its arrival
+    // is counted
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    uint32_t *s_arrived = reinterpret_cast<uint32_t *>(lds);
+    if (tid == 0)
+      *s_arrived = __hip_atomic_fetch_add(sk.counters + tile_id, 1u, __ATOMIC_RELAXED,
+                                          __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    const uint32_t arrived = *s_arrived;
+    __syncthreads();                  // LDS is the epilogue's from here on
+    if (arrived != (uint32_t)sk.splits - 1) return;   // the whole workgroup leaves
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    for (int s = 0; s < sk.splits; s++) {
+      if (s == (int)blockIdx.z) continue;
+      const int32_t *theirs = sk.partials + (tile_id * sk.splits + s) * (size_t)(BM * BN);
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+          for (int r = 0; r < 16; r++)
+            acc[i][j][r] += __hip_atomic_load(theirs + ((i * TN + j) * 16 + r) * THREADS + tid,
+                                              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (tid == 0)                     // as the next launch expects it
+      __hip_atomic_store(sk.counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
   gemm_epilogue<BM, BN, WM, WN, NEED_SA, NEED_SB>(acc, sa, sb, lds, ep, M, N, K,
                                                   m0, n0, n_base, col);
 }
@@ -1343,7 +1413,7 @@ static int gemm_dma_launch(const ARows &A, const DenseRows &B,
       hipLaunchKernelGGL((gemm_i8_dma_kernel<BM, BN, WM, WN, STAGES, SA, SB, ARows, true>),
                          dim3((unsigned)total, (unsigned)g.groups), dim3(THREADS),
                          ring > epi ? ring : epi, st, A, B, ep, g.M, g.N, g.K, tiles_m,
-                         tiles_n, g.b_group_stride, g.N);
+                         tiles_n, g.b_group_stride, g.N, SplitK{});
       return check_launch("gemm_i8_dma");
     }
   }
@@ -1353,8 +1423,83 @@ static int gemm_dma_launch(const ARows &A, const DenseRows &B,
   if (rc != MI355X_OK) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)g.groups),
                      dim3(THREADS), lds, st, A, B, ep, g.M, g.N, g.K, tiles_m,
-                     tiles_n, g.b_group_stride, g.N);
+                     tiles_n, g.b_group_stride, g.N, SplitK{});
   return check_launch("gemm_i8_dma");
+}
+
+// The 128x128 tile of eight waves with K split over `splits` workgroups per
+// output tile (see SplitK). The workspace holds the tiles' counters (zero
+// before the launch, zero after it), then the partial sums.
+constexpr size_t kSplitTile = 128;
+static size_t splitk_counter_bytes(const GemmShape &g) {
+  const size_t tiles = ((g.M + kSplitTile - 1) / kSplitTile) * ((g.N + kSplitTile - 1) / kSplitTile);
+  return (tiles * (size_t)g.groups * sizeof(uint32_t) + 255) & ~(size_t)255;
+}
+static size_t splitk_workspace_bytes(const GemmShape &g, int splits) {
+  const size_t tiles = ((g.M + kSplitTile - 1) / kSplitTile) * ((g.N + kSplitTile - 1) / kSplitTile);
+  return splitk_counter_bytes(g) +
+         tiles * (size_t)g.groups * (size_t)splits * kSplitTile * kSplitTile * sizeof(int32_t);
+}
+// How many workgroups share an output tile's K loop: enough to give every CU
+// one, at most four, each with at least 32 K steps (handing the sums over costs
+// about what 24 steps take: measured, K of 4608 over 100 tiles 22.5 -> 19.8 us,
+// K of 2048 9.9 -> 13.3 us); 1 = not split (the grid already fills half the
+// chip, or K is short).
+// forced (the caller named the tile): at least two whenever K has two steps.
+static int splitk_choice(const GemmShape &g, int cus, bool forced) {
+  const long long tiles = (long long)((g.M + kSplitTile - 1) / kSplitTile) *
+                          ((g.N + kSplitTile - 1) / kSplitTile) * g.groups;
+  const int KT = g.K / kBK;
+  int s = 1;
+  if (tiles > 0 && tiles * 2 <= cus) {
+    s = (int)std::min<long long>(4, cus / tiles);
+    while (s > 1 && KT / s < 32) s--;
+  }
+  if (forced && s < 2 && KT >= 2) s = 2;
+  return s;
+}
+
+static int gemm_cus() {
+  static std::atomic<int> cached{0};
+  int v = cached.load(std::memory_order_relaxed);
+  if (v > 0) return v;
+  int dev = 0;
+  v = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
+    v = 256;
+  cached.store(v, std::memory_order_relaxed);
+  return v;
+}
+
+template <class ARows>
+static int gemm_dma_launch_splitk(const ARows &A, const DenseRows &B, const Epilogue &ep,
+                                  const GemmShape &g, int splits, void *workspace,
+                                  hipStream_t st) {
+  constexpr int BM = 128, BN = 128, WM = 64, WN = 32, STAGES = 3;
+  constexpr int THREADS = (BM / WM) * (BN / WN) * 64;
+  constexpr size_t lds = gemm_dma_lds_bytes<BM, BN, STAGES>();
+  const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
+  const long long total = (long long)tiles_m * tiles_n;
+  MI355X_REQUIRE(total < 0x7fffffffLL && g.groups < 65536 && splits >= 2 && splits <= 64,
+                 "problem too large");
+  // every split has at least one K step (the kernel counts on it)
+  const int KT = g.K / kBK, per = (KT + splits - 1) / splits;
+  MI355X_REQUIRE(g.K % kBK == 0 && (splits - 1) * per < KT, "K of %d cannot be split %d ways",
+                 g.K, splits);
+  auto kern = gemm_i8_dma_kernel<BM, BN, WM, WN, STAGES, false, false, ARows, false, true>;
+  static std::atomic<uint64_t> attr_set{0}; // per instantiation, one bit per device
+  int rc = set_lds_attr(kern, lds, attr_set);
+  if (rc != MI355X_OK) return rc;
+  SplitK sk;
+  sk.counters = reinterpret_cast<uint32_t *>(workspace);
+  sk.partials = reinterpret_cast<int32_t *>(reinterpret_cast<uint8_t *>(workspace) +
+                                            splitk_counter_bytes(g));
+  sk.splits = splits;
+  hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)g.groups, (unsigned)splits),
+                     dim3(THREADS), lds, st, A, B, ep, g.M, g.N, g.K, tiles_m, tiles_n,
+                     g.b_group_stride, g.N, sk);
+  return check_launch("gemm_i8_dma_splitk");
 }
 
 // Tile choice from the problem size: 256x256 for large problems (a wave owns
@@ -1389,9 +1534,31 @@ static Tile pick_tile(const GemmShape &g, size_t lds_256) {
   return Tile::T128x64;
 }
 
+constexpr int kTileSplitK = 12;   // tile number of the K-split launch
+
 template <bool SA, bool SB, class ARows>
 static int gemm_dma_tiles(const ARows &A, const DenseRows &B, const Epilogue &ep,
                           const GemmShape &g, hipStream_t st) {
+  // K split over workgroups: when the call brings a workspace and the grid
+  // would leave half the chip idle, or when the call names the tile
+  const bool named = g_tile_override == kTileSplitK;
+  if (named || (g_tile_override < 0 && g_workspace)) {
+    if constexpr (!SA && !SB) {
+      const int splits = splitk_choice(g, gemm_cus(), named);
+      if (splits >= 2 && g_workspace && (((uintptr_t)g_workspace) & 255) == 0 &&
+          g_workspace_bytes >= splitk_workspace_bytes(g, splits))
+        return gemm_dma_launch_splitk(A, B, ep, g, splits, g_workspace, st);
+      if (named)
+        return fail(MI355X_ERR_NOT_SUPPORTED,
+                    "tile %d (K split over workgroups) needs two K steps and a 256-byte "
+                    "aligned workspace of %zu bytes in the launch's options",
+                    kTileSplitK, splitk_workspace_bytes(g, splits < 2 ? 2 : splits));
+    } else if (named) {
+      return fail(MI355X_ERR_NOT_SUPPORTED,
+                  "tile %d (K split over workgroups) needs precomputed weight row sums and "
+                  "zero weight offsets", kTileSplitK);
+    }
+  }
   switch (pick_tile(g, gemm_dma_lds_bytes<256, 256, 4>())) {
   case Tile::T256:
     return gemm_dma_launch<256, 256, 128, 128, 4, SA, SB>(A, B, ep, g, st);
@@ -1454,6 +1621,10 @@ static int gemm_dispatch(const ARows &A, const DenseRows &B, const Epilogue &ep_
     if (need_sb) return gemm_dma_tiles<false, true>(A, B, ep, g, st);
     return gemm_dma_tiles<false, false>(A, B, ep, g, st);
   }
+  if (g_tile_override == kTileSplitK)
+    return fail(MI355X_ERR_NOT_SUPPORTED,
+                "tile %d (K split over workgroups) needs K a multiple of 64 and 16-byte "
+                "aligned operands", kTileSplitK);
   // K tails and unaligned operands: register-staged loop, both row sums kept
   if (aligned) return gemm_staged_tiles<true, true>(A, B, ep, g, st);
   return gemm_staged_tiles<false, false>(A, B, ep, g, st);

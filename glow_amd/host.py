@@ -154,7 +154,7 @@ class Module:
                 fuse_transpose_matmul=True, fuse_fc_relu=True,
                 pad_table_rows=True, fuse_insert=True, fuse_dequantize_sigmoid=True,
                 derive_bag_offsets=True, reuse_activations=True,
-                fuse_quantize_stem=True):
+                fuse_quantize_stem=True, split_k=True):
         opts = ((1 if precompute_weight_row_sums else 0) | (2 if fuse_add_relu else 0) |
                 (4 if fuse_conv_add else 0) | (8 if space_to_depth_stem else 0) |
                 (16 if fuse_sls_chains else 0) | (32 if fuse_transpose_matmul else 0) |
@@ -162,7 +162,7 @@ class Module:
                 (128 if pad_table_rows else 0) | (256 if fuse_insert else 0) |
                 (512 if fuse_dequantize_sigmoid else 0) |
                 (1024 if derive_bag_offsets else 0) | (2048 if reuse_activations else 0) |
-                (4096 if fuse_quantize_stem else 0))
+                (4096 if fuse_quantize_stem else 0) | (8192 if split_k else 0))
         _check(lib().mi355x_host_compile(self._h, fn, opts))
 
     def describe(self, fn):

@@ -1110,6 +1110,25 @@ private:
     return [base, rel](const DeviceBindings &b) { return b.generated + *base + rel; };
   }
 
+  // The matrix-core launch just emitted multiplies [M x K] by [K x N] (per
+  // group): when the library would split its K loop over workgroups given a
+  // workspace, it gets one of its own (launches of one function may run side by
+  // side), zero-filled once when the function is loaded.
+  void planSplitK(MI355XFunction &out, size_t M, size_t N, size_t K, size_t groups) {
+    if (!opts_.splitK) return;
+    size_t bytes = 0;
+    if (mi355x_gemm_splitk_workspace_bytes(M, N, K, groups, 0, &bytes) != MI355X_OK || bytes == 0)
+      return;
+    KernelLaunch &l = out.launches.back();
+    l.workspaceRel = gen_.addScratch(bytes);
+    l.workspaceBytes = bytes;
+    l.scratchBase = scratchBasePtr_;
+    l.params += strFormat(" splitk_workspace=%zu", bytes);
+    auto p = scratchPtr(l.workspaceRel);
+    out.setup.push_back({"mi355x_fill_u8", l.inst + ".splitk_workspace", strFormat(" bytes=%zu", bytes),
+                         [=](const DeviceBindings &b) { return mi355x_fill_u8(p(b), 0, bytes, b.stream); }});
+  }
+
   // Where a lookup reads a table and how far apart its rows are. A constant
   // table whose rows take 33..63 bytes is copied once, at load time, to rows 64
   // bytes apart: memory is fetched in 64-byte pieces, a 36-byte row at a 36-byte
@@ -1440,6 +1459,7 @@ private:
                                           rp.post, rp.scale, b.stream, &b.opts);
            }});
       out.launches.back().requantHint = hint;
+      planSplitK(out, M, N, K, 1);
       return Error::success();
     }
     out.launches.push_back(
@@ -1457,6 +1477,7 @@ private:
                                    sums ? (const int32_t *)sumPtr(b) : nullptr, b.stream, &b.opts);
          }});
     out.launches.back().requantHint = hint;
+    planSplitK(out, M, N, K, 1);
     return Error::success();
   }
 
@@ -1762,6 +1783,7 @@ private:
                                          b.stream, &b.opts);
            }});
       out.launches.back().requantHint = convHint(K2);
+      planSplitK(out, (size_t)g2.N * g2.OH * g2.OW, (size_t)g2.OC, (size_t)K2, 1);
       out.launches.back().reads.push_back(priv);
       return Error::success();
     }
@@ -1820,6 +1842,7 @@ private:
                  b.stream, &b.opts);
            }});
       out.launches.back().requantHint = convHint(Kf);
+      planSplitK(out, (size_t)g.N * g.OH * g.OW, (size_t)g.OC / g.group, (size_t)Kf, (size_t)g.group);
       return Error::success();
     }
     out.launches.push_back(
@@ -1839,6 +1862,7 @@ private:
                                        b.stream, &b.opts);
          }});
     out.launches.back().requantHint = convHint(Kf);
+    planSplitK(out, (size_t)g.N * g.OH * g.OW, (size_t)g.OC / g.group, (size_t)Kf, (size_t)g.group);
     return Error::success();
   }
 
@@ -2254,11 +2278,15 @@ unsigned MI355XBackend::numDevices() {
 }
 
 int KernelLaunch::launch(const DeviceBindings &b) const {
-  if (!tunable || (tile < 0 && requantHint == 0)) return run(b);
-  // the launch's own tile and hint travel with the call, nothing is left set
+  if (!tunable || (tile < 0 && requantHint == 0 && workspaceBytes == 0)) return run(b);
+  // the launch's own tile, hint and workspace travel with the call, nothing is left set
   DeviceBindings mine = b;
   mine.opts.gemm_tile = tile;
   mine.opts.requant_hint = requantHint;
+  if (workspaceBytes && scratchBase) {
+    mine.opts.workspace = b.generated + *scratchBase + workspaceRel;
+    mine.opts.workspace_bytes = workspaceBytes;
+  }
   return run(mine);
 }
 

@@ -114,7 +114,13 @@ struct KernelLaunch {
   // derived at compile time from the launch's constants with worst-case
   // operand bytes; 0 = none.
   int requantHint = 0;
-  // Issues the launch (with its tile, if it has one).
+  // Workspace of a matrix-core launch whose K loop the library may split over
+  // workgroups (mi355x_gemm_splitk_workspace_bytes): workspaceBytes at
+  // generated + *scratchBase + workspaceRel, its counters zeroed by a set-up
+  // launch when the function is loaded; 0 bytes = none.
+  size_t workspaceRel = 0, workspaceBytes = 0;
+  std::shared_ptr<size_t> scratchBase;
+  // Issues the launch (with its tile, hint and workspace, if it has them).
   int launch(const DeviceBindings &b) const;
 };
 constexpr int kNumTiles = 12;
@@ -198,6 +204,7 @@ struct BackendOptions {
   bool deriveBagOffsets = true;        // lookups whose lengths are an input: bag positions summed on the host at upload
   bool fuseQuantizeStem = true;        // Quantize read only by a space-to-depth convolution: quantized while re-laid
   bool reuseActivations = true;        // activations whose lives do not meet share memory (first fit over the launch order)
+  bool splitK = true;                  // matrix-core launches with few output tiles and a long K get a workspace, so the library may split K over workgroups
 };
 
 class MI355XBackend {

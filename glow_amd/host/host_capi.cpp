@@ -145,6 +145,7 @@ int mi355x_host_compile(mi355x_host_module *m, int function, int options) {
   o.deriveBagOffsets = (options & MI355X_HOST_OPT_DERIVE_BAG_OFFSETS) != 0;
   o.reuseActivations = (options & MI355X_HOST_OPT_REUSE_ACTIVATIONS) != 0;
   o.fuseQuantizeStem = (options & MI355X_HOST_OPT_FUSE_QUANTIZE_STEM) != 0;
+  o.splitK = (options & MI355X_HOST_OPT_SPLIT_K) != 0;
   auto r = MI355XBackend().compile(*f, o);
   if (!r) return fail(r.error());
   m->compiled[function] = std::move(r.get());

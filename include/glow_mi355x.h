@@ -116,8 +116,8 @@ int mi355x_event_elapsed_ms(void *start, void *stop, float *ms);
  *   gemm_tile     matrix-core launches (FullyConnected, MatMul, convolution):
  *                 the workgroup tile, -1 = chosen from the problem shape. Values
  *                 as listed at mi355x_gemm_tile_override. Results do not depend
- *                 on it. A tile in 6..8 names one special kernel; a launch that
- *                 kernel cannot serve fails with MI355X_ERR_NOT_SUPPORTED (a
+ *                 on it. A tile in 6..8 or 12 names one special kernel; a launch
+ *                 that kernel cannot serve fails with MI355X_ERR_NOT_SUPPORTED (a
  *                 tuner skips the candidate) instead of running another one.
  *   requant_hint  MI355X_REQUANT_* guarantees about the launch's constants, as
  *                 mi355x_gemm_requant_hint_host derives them; 0 = none. A wrong
@@ -137,15 +137,23 @@ int mi355x_event_elapsed_ms(void *start, void *stop, float *ms);
  *                 MI355X_SLWS_MATH_REGROUPED sum_j (w_j s_j) q_jk + sum_j w_j o_j
  *                   (two instructions per element); its error is relative to
  *                   the magnitude a bag adds up, not to the result, and
- *                   exceeds 1e-5 of results that cancel: on request only. */
+ *                   exceeds 1e-5 of results that cancel: on request only.
+ *   workspace, workspace_bytes   device memory the launch may use for sums that
+ *                 several workgroups share (matrix-core launches whose K loop is
+ *                 split over workgroups, see mi355x_gemm_splitk_workspace_bytes
+ *                 for the size and the zero-fill rule); NULL = none. A caller
+ *                 built before these two fields existed passes the smaller
+ *                 struct_size and gets none. */
 enum { MI355X_SLWS_MATH_STRICT = 0, MI355X_SLWS_MATH_ELEMENT = 1, MI355X_SLWS_MATH_REGROUPED = 2 };
 typedef struct {
   uint32_t struct_size;
   int32_t gemm_tile;
   int32_t requant_hint;
   int32_t slws_math;
+  void *workspace;
+  uint64_t workspace_bytes;
 } mi355x_launch_opts;
-#define MI355X_LAUNCH_OPTS_INIT { (uint32_t)sizeof(mi355x_launch_opts), -1, 0, -1 }
+#define MI355X_LAUNCH_OPTS_INIT { (uint32_t)sizeof(mi355x_launch_opts), -1, 0, -1, 0, 0 }
 
 /* ---- launch graphs ---------------------------------------------------------- */
 /* A compiled function is a fixed sequence of kernel launches on fixed
@@ -573,19 +581,36 @@ int mi355x_matmul_i8_opts(int8_t *out, const int8_t *lhs, const int8_t *rhs_kn,
  * the following matrix-core launches of the calling thread: 0 = 256x256,
  * 1 = 128x128, 2 = 128x64, 3 = 64x64, 4 = 256x128, 5 = 128x256, 6 = 32x32 with
  * the K loop split over the workgroup's waves (FullyConnected forms with
- * symmetric weights, precomputed row sums and K % 32 == 0 only; launches it
- * cannot serve ignore it), 7 = the 3x3 stride-1 convolution over 64 input
- * channels with filter and input rows resident in LDS (other launches ignore
- * it; tiles 0..6 keep such a convolution on the tiled kernels), 8 = the
- * streaming kernel for K of 64, 128 or 256 (FullyConnected and pointwise
- * convolutions with symmetric weights and precomputed row sums: weights and
- * constants resident in LDS, rows straight from memory into registers; other
- * launches ignore it), 9 = 128x128, 10 = 256x128 and 11 = 256x256 with
- * eight waves per workgroup instead of four; -1 = chosen
- * from the problem shape (the default). Results do not depend on the tile. A device
- * manager uses it to time the candidates of each layer once, when a network is
- * loaded. */
+ * symmetric weights, precomputed row sums and K % 32 == 0 only), 7 = the 3x3
+ * stride-1 convolution over 64, 128, 256 or 512 input channels with the input
+ * rows resident in LDS (tiles 0..6 keep such a convolution on the tiled
+ * kernels), 8 = the streaming kernel for K of 64, 128 or 256 (FullyConnected
+ * and pointwise convolutions with symmetric weights and precomputed row sums:
+ * weights and constants resident in LDS, rows straight from memory into
+ * registers), 9 = 128x128, 10 = 256x128 and 11 = 256x256 with eight waves per
+ * workgroup instead of four, 12 = 128x128 with eight waves and the K loop
+ * split over two to four workgroups per output tile, which leave their int32
+ * sums in the workspace of the launch's options (what the library also picks
+ * by itself when the options bring a workspace and the 128x128 grid would
+ * leave half of the CUs idle; int32 sums wrap, so the order in which they are
+ * added does not matter: the reference's sum, libjit_matmul.cpp:284-316);
+ * -1 = chosen from the problem shape (the default). Results do not depend on
+ * the tile. A tile in 6..8 or 12 names one kernel: a launch that kernel cannot
+ * serve fails with MI355X_ERR_NOT_SUPPORTED. A device manager uses the tiles
+ * to time the candidates of each layer once, when a network is loaded. */
 int mi355x_gemm_tile_override(int tile);
+
+/* Bytes of workspace a K-split launch of the product [M x K] x [K x N] (times
+ * `groups` for a grouped convolution, M = output pixels, K = taps x channels
+ * of a group, N = channels of a group) uses: with named = 0 what the library
+ * would split by itself (0: it would not), with named != 0 what tile 12 needs
+ * (0: K has fewer than two steps of 64). The workspace is device memory,
+ * 256-byte aligned, zero-filled once before its first use (its first bytes are
+ * per-tile counters, which every launch leaves zero again); launches that may
+ * run at the same time need workspaces of their own. No counterpart in the
+ * reference. */
+int mi355x_gemm_splitk_workspace_bytes(size_t M, size_t N, size_t K, size_t groups, int named,
+                                       size_t *bytes);
 
 /* Requantisation hints (no counterpart in the reference) for the following
  * matrix-core launches of the calling thread (FullyConnected, MatMul and

@@ -139,7 +139,10 @@ enum {
                                              * every value has bytes of its own */
   MI355X_HOST_OPT_FUSE_QUANTIZE_STEM = 4096, /* a Quantize read only by a convolution that goes
                                               * through space-to-depth is applied by that pass */
-  MI355X_HOST_OPT_DEFAULT = 8191
+  MI355X_HOST_OPT_SPLIT_K = 8192, /* matrix-core launches with few output tiles and a long K get
+                                   * a workspace in the generated region, so the kernel library
+                                   * may split their K loop over workgroups */
+  MI355X_HOST_OPT_DEFAULT = 16383
 };
 int mi355x_host_compile(mi355x_host_module *m, int function, int options);
 /* Listing of the compiled function's launches and derived parameters; returns

@@ -37,6 +37,30 @@ def test_basic(dm):
 
 
 @pytest.mark.parametrize("graphs", [True, False])
+def test_product_with_its_k_loop_split_over_workgroups(graphs):
+    """Few output tiles and a long K: the compiled launch carries a workspace and
+    the library splits its K loop; request after request gives the oracle's
+    bytes (the workspace's counters are left zero by every launch), also while
+    the device manager times the launch's candidate tiles."""
+    d = H.DeviceManager(use_launch_graphs=graphs).init()
+    try:
+        c = cases.rwq_fc_case(31, 300, 4608, 256, symmetric=True)
+        m, f = host_cases.rwq_fc_module(c)
+        m.compile(f)
+        assert "splitk_workspace" in [r for r in H.parse_listing(m.describe(f))
+                                      if r["kernel"] == "mi355x_rwq_fc_i8"][0]
+        d.add_network(m)
+        rng = np.random.default_rng(1)
+        for _ in range(12):
+            x = rng.integers(-128, 128, c["x"].shape).astype(np.int8)
+            out = np.zeros((300, 256), np.int8)
+            d.run("main", {"input": x, "output": out})
+            assert np.array_equal(out, _rwq_expected(c, x))
+    finally:
+        d.stop()
+
+
+@pytest.mark.parametrize("graphs", [True, False])
 def test_multi_run(graphs):
     d = H.DeviceManager(use_launch_graphs=graphs).init()
     try:

@@ -9,6 +9,7 @@ import re
 import numpy as np
 import pytest
 
+from glow_amd import capi
 from glow_amd import host as H
 from tests import cases, host_cases
 from oracle import glow_oracle as go
@@ -503,3 +504,27 @@ def test_bag_positions_are_not_derived_from_lengths_some_function_writes():
     assert "mi355x_frwq_slws_offsets" in build(False, False)
     assert "mi355x_frwq_slws_offsets" not in build(True, False)
     assert "mi355x_frwq_slws_offsets" not in build(False, True)
+
+
+def test_long_k_products_with_few_tiles_get_a_workspace():
+    """A matrix-core launch whose 128x128 grid would leave half the chip idle and
+    whose K loop is long gets a workspace in the generated region (zero-filled
+    by a set-up launch), so that the kernel library may split K over workgroups;
+    other launches get none, and the option switches it off."""
+    c = cases.rwq_fc_case(21, 300, 4608, 256, symmetric=True)
+    m, f = host_cases.rwq_fc_module(c)
+    m.compile(f)
+    r = _launch(m, f, "mi355x_rwq_fc_i8")
+    want = capi.gemm_splitk_workspace_bytes(300, 256, 4608)
+    assert want > 0 and r["splitk_workspace"] == want
+    fills = [x for x in H.parse_listing(m.describe(f))
+             if x["phase"] == "setup" and x["kernel"] == "mi355x_fill_u8"]
+    assert len(fills) == 1 and fills[0]["bytes"] == want
+    assert m.bundle_sizes(f)["generated"] >= want
+    m2, f2 = host_cases.rwq_fc_module(c)
+    m2.compile(f2, split_k=False)
+    assert "splitk_workspace" not in _launch(m2, f2, "mi355x_rwq_fc_i8")
+    small = cases.rwq_fc_case(22, 300, 512, 256, symmetric=True)     # K too short to share
+    m3, f3 = host_cases.rwq_fc_module(small)
+    m3.compile(f3)
+    assert "splitk_workspace" not in _launch(m3, f3, "mi355x_rwq_fc_i8")

@@ -27,7 +27,11 @@ def test_options_are_validated_on_the_host():
     bad = capi.LaunchOpts()
     bad.struct_size = 8
     assert _slws_opts_call(bad) == -1 and b"struct_size" in capi.lib().mi355x_last_error()
-    for field, value in (("gemm_tile", 12), ("gemm_tile", -2), ("requant_hint", 2),
+    # a caller built before the workspace fields existed passes the shorter struct
+    short = capi.LaunchOpts()
+    short.struct_size = 16
+    assert _slws_opts_call(short) == 0
+    for field, value in (("gemm_tile", 13), ("gemm_tile", -2), ("requant_hint", 2),
                          ("requant_hint", 4), ("slws_math", 3), ("slws_math", -2)):
         o = capi.LaunchOpts()
         setattr(o, field, value)
