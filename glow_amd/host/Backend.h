@@ -123,7 +123,7 @@ struct KernelLaunch {
   // Issues the launch (with its tile, hint and workspace, if it has them).
   int launch(const DeviceBindings &b) const;
 };
-constexpr int kNumTiles = 12;
+constexpr int kNumTiles = 13;   // candidates -1 .. 12 of the tile tuner
 
 class MI355XFunction {
 public:
