@@ -225,3 +225,49 @@ def test_other_lookup_forms(seed):
     np.testing.assert_array_equal(capi.gather(d, gi, 1), go.gather(d, gi, 1))
     g0 = rng.integers(0, d.shape[0], 17).astype(np.int64)
     np.testing.assert_array_equal(capi.gather(d, g0, 0), go.gather(d, g0, 0))
+
+
+@pytest.mark.parametrize("seed", range(30 * _MORE))
+def test_unlowered_element_operators(seed):
+    """Clip, LeakyRelu, Max(x, Splat) and BatchedAdd over random sizes
+    (aligned and not, below and above one 16-byte piece) and parameters."""
+    rng = np.random.default_rng(9000 + seed)
+    n = int(rng.choice([1, 5, 15, 16, 17, 63, 1000, 4099, 65537]))
+    q = rng.integers(-128, 128, n).astype(np.int8)
+    so, do = int(rng.integers(-128, 128)), int(rng.integers(-128, 128))
+    lo, hi = sorted(int(v) for v in rng.integers(-128, 128, 2))
+    P, Q = _params(rng), _params(rng)
+    print("element operators", n, so, do, lo, hi, P, Q, flush=True)
+    np.testing.assert_array_equal(capi.clip_elem_i8(q, lo, hi, so, do, P),
+                                  go.clip_elem_i8(q, lo, hi, so, do, P))
+    np.testing.assert_array_equal(capi.leaky_relu_i8(q, so, do, P, Q),
+                                  go.leaky_relu_i8(q, so, do, P, Q))
+    v = int(rng.integers(-128, 128))
+    np.testing.assert_array_equal(capi.max_splat_i8(q, v), go.max_splat_i8(q, v))
+    slices, size = int(rng.integers(1, 40)), int(rng.choice([1, 3, 4, 12, 64, 250, 1000]))
+    batch = rng.integers(-128, 128, (slices, size)).astype(np.int8)
+    sl = (rng.integers(-30000, 30000, size).astype(np.int32) if rng.integers(0, 2)
+          else rng.integers(-128, 128, size).astype(np.int8))
+    bo, slo = int(rng.integers(-128, 128)), int(rng.integers(-128, 128))
+    np.testing.assert_array_equal(capi.batched_add_i8(batch, sl, do, bo, slo, P, Q),
+                                  go.batched_add_i8(batch, sl, do, bo, slo, P, Q))
+
+
+@pytest.mark.parametrize("seed", range(20 * _MORE))
+def test_k_loop_split_over_workgroups(seed):
+    """The named K-split tile on random products (K a multiple of 64 with at
+    least two steps, symmetric weights): the oracle's bytes, and the workspace
+    ready for the next launch."""
+    rng = np.random.default_rng(9500 + seed)
+    M, N = _dim(rng, 500), _dim(rng, 400)
+    K = 64 * int(rng.integers(2, 40))
+    c = cases.rwq_fc_case(seed, M, K, N, symmetric=True, bias_i8=bool(rng.integers(0, 2)),
+                          out_offset=int(rng.integers(-128, 128)))
+    print("rwq_fc, K split", M, K, N, flush=True)
+    need = capi.gemm_splitk_workspace_bytes(M, N, K, named=True)
+    ws = capi.DeviceBuffer(need)
+    ws.fill(0)
+    opts = capi.LaunchOpts(gemm_tile=capi.TILE_SPLIT_K, workspace=ws)
+    want = go.rwq_fc_i8(*cases.rwq_fc_args(c))
+    for _ in range(2):
+        np.testing.assert_array_equal(capi.rwq_fc_i8(*cases.rwq_fc_args(c), opts=opts), want)
