@@ -605,7 +605,10 @@ def bench_elementwise(capi, which, steps, warmup):
     else:
         src = capi.to_device(rng.integers(-128, 128, n).astype(np.int8))
         dst = capi.DeviceBuffer.empty((n,), np.int8)
-        fn = lambda _, st: capi.launch_rescale_i8(dst, src, n, 3, -5, 2, 15, 300, st)
+        # the parameters of a rescale between scales 0.05 and 0.07
+        # (quantizeScaleOffset32To8(0.714) = {pre 0, post 9, scale 366}; a
+        # pre-shift only appears for ratios below 2^-7)
+        fn = lambda _, st: capi.launch_rescale_i8(dst, src, n, 3, -5, 0, 9, 366, st)
         nbytes = n * 2
     sec = timed_launches(capi, fn, steps, warmup)
     return dict(workload=f"{which}_u8 n={n}" if which == "copy" else f"{which}_i8 n={n}", ms=sec * 1e3,

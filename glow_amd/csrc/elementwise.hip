@@ -90,6 +90,34 @@ __global__ __launch_bounds__(kEwThreads) void dequantize_i8_kernel(
     dst[i] = __fmul_rn(scale, (float)((int32_t)src[i] - offset));
 }
 
+// RescaleQuantized with no pre-shift, a scale below 2^23 and room below the
+// post-shift for the offsets: ((q - in_off) * s + rtn) >> post) + out_off
+// == (q * s + folded) >> post with folded = rtn - in_off * s + (out_off << post),
+// exact in 32 bits under the bound the caller checks (no intermediate leaves
+// int32, so (A >> p) + d == (A + (d << p)) >> p). One 24-bit multiply-add, one
+// shift and one clamp per value instead of nine instructions: the kernel is
+// bound by its instruction stream, not by memory.
+__global__ __launch_bounds__(kEwThreads) void rescale_folded_i8_kernel(
+    int8_t *__restrict__ dst, const int8_t *__restrict__ src, size_t n, size_t vec_chunks,
+    int32_t folded, int32_t post, int32_t scale) {
+  auto one = [=](int32_t q) {
+    return med3_i32((int32_t)((uint32_t)__mul24(q, scale) + (uint32_t)folded) >> post, -128, 127);
+  };
+  const size_t t = (size_t)blockIdx.x * kEwThreads + threadIdx.x;
+  if (t < vec_chunks) {
+    uint4 q = reinterpret_cast<const uint4 *>(src)[t];
+    uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      w[j] = pack4(one(sext8(w[j], 0)), one(sext8(w[j], 1)), one(sext8(w[j], 2)),
+                   one(sext8(w[j], 3)));
+    reinterpret_cast<uint4 *>(dst)[t] = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+  const size_t tail0 = vec_chunks * kEwPerLane;
+  const size_t stride = (size_t)gridDim.x * kEwThreads;
+  for (size_t i = tail0 + t; i < n; i += stride) dst[i] = (int8_t)one((int32_t)src[i]);
+}
+
 template <bool SMALL>
 __global__ __launch_bounds__(kEwThreads) void rescale_i8_kernel(
     int8_t *__restrict__ dst, const int8_t *__restrict__ src, size_t n,
@@ -222,6 +250,19 @@ int mi355x_rescale_i8(int8_t *dst, const int8_t *src, size_t n,
   // with a scale below 2^23 too, the 24-bit multiplier is exact
   const bool small = scale > -(1 << 23) && scale < (1 << 23) &&
                      in_offset > -(1 << 22) && in_offset < (1 << 22);
+  // everything folded into one constant: |(q - in_off) * s| + rtn + |out_off << post|
+  // stays below 2^31 (q int8, so |q - in_off| < 2^8 + |in_off|)
+  const long long mag = (256ll + std::llabs((long long)in_offset)) * std::llabs((long long)scale) +
+                        (post > 0 ? (1ll << (post - 1)) : 0) +
+                        (std::llabs((long long)out_offset) << post);
+  if (small && pre == 0 && mag < (1ll << 31)) {
+    const int32_t folded = (int32_t)((post > 0 ? (1ll << (post - 1)) : 0) -
+                                     (long long)in_offset * scale +
+                                     ((long long)out_offset << post));
+    hipLaunchKernelGGL(rescale_folded_i8_kernel, dim3(ew_blocks(chunks)), dim3(kEwThreads), 0,
+                       as_stream(stream), dst, src, n, chunks, folded, post, scale);
+    return check_launch("rescale_i8");
+  }
   if (small)
     hipLaunchKernelGGL(rescale_i8_kernel<true>, dim3(ew_blocks(chunks)),
                        dim3(kEwThreads), 0, as_stream(stream), dst, src, n,
