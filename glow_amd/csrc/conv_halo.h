@@ -65,6 +65,28 @@ constexpr int kHaloParBytes = kParArrays * kHaloBN * 4;
 // Requantises a wave's 32 pixels x 64 channels and writes them as whole rows
 // through its staging tile (gemm_i8.h: requant_pack16, wave_rows_copy_out).
 constexpr int kHaloStageStride = kHaloBN + 16;
+// Copy-out of one staged block of 32 pixels x 64 channels: eight consecutive
+// lanes read the same 16-byte piece of eight consecutive pixels (eight
+// different bank groups at the 80-byte stride; four lanes per pixel put every
+// second pixel's piece on the banks of the one before), and a wave's store
+// instruction still covers sixteen whole pixels of 64 bytes.
+__device__ __forceinline__ void halo_rows_copy_out(const int8_t *s_stage, int lane, int m0, int M,
+                                                   int col0, const Epilogue &ep,
+                                                   const FusedAddConsts &fc, bool fast) {
+  const int seg = (lane >> 3) & 3;
+  const int row_in_pass = (lane & 7) + 8 * (lane >> 5);
+#pragma unroll
+  for (int r0 = 0; r0 < 32; r0 += 16) {
+    const int row = r0 + row_in_pass, m = m0 + row;
+    if (m < M) {
+      int4 v = *reinterpret_cast<const int4 *>(s_stage + row * kHaloStageStride + seg * 16);
+      const long long at = (long long)m * ep.ldc + col0 + seg * 16;
+      v = fused_out_words(v, ep.add.res ? ep.add.res + at : nullptr, ep, fc, fast);
+      *reinterpret_cast<int4 *>(ep.out + at) = v;
+    }
+  }
+}
+
 template <int MODE, bool LEAKY>
 __device__ __forceinline__ void halo_finish(const v16i (&acc)[2], const int32_t *s_par,
                                             int8_t *stage, const Epilogue &ep, int lane, int m0,
@@ -81,7 +103,7 @@ __device__ __forceinline__ void halo_finish(const v16i (&acc)[2], const int32_t 
     *reinterpret_cast<int4 *>(stage + l32 * kHaloStageStride + cl) = v;
   }
   wave_fence();
-  wave_rows_copy_out(stage, kHaloStageStride, kHaloBN, lane, m0, M, n0, ep, fc, fast);
+  halo_rows_copy_out(stage, lane, m0, M, n0, ep, fc, fast);
 }
 
 // SKIP leaves phases out so that the others can be timed (1: staging, 2: the
@@ -118,14 +140,19 @@ __global__ __launch_bounds__(512, 2) void conv3x3_halo_kernel(HaloConv cv, Epilo
     const int4 fill4 = make_int4((int)cv.fill, (int)cv.fill, (int)cv.fill, (int)cv.fill);
     const int8_t *img = cv.in + (long long)n * cv.IH * cv.IW * kHaloIC;
     const int8_t *f = cv.filter + (long long)n0 * kHaloK;
-    const int halo_chunks = (rows + 2) * hw * (kHaloIC / 16);
+    const int halo_pixels = (rows + 2) * hw;
+    // work items of the halo: 32 per group of eight pixels
+    const int halo_chunks = ((halo_pixels + 7) >> 3) * 32;
     constexpr int HU = 4, FU = 6;
-    // chunk c of the halo: pixel c / 4 of the (rows + 2) x hw patch, bytes
-    // 16 * (c % 4) of its channels
+    // item c of the halo: pixel 8 (c / 32) + c % 8 of the (rows + 2) x hw patch,
+    // bytes 16 * ((c / 8) % 4) of its channels. Eight consecutive lanes then
+    // store the same 16-byte piece of eight consecutive pixels, 80 bytes apart:
+    // eight different bank groups (four lanes per pixel, the plain order, put
+    // the piece of every second pixel on the banks of the one before).
     auto halo_load = [&](int c) -> int4 {
       int4 v = fill4;
-      if (c < halo_chunks) {
-        const int px = c >> 2, kc = c & 3;
+      const int px = ((c >> 5) << 3) + (c & 7), kc = (c >> 3) & 3;
+      if (px < halo_pixels) {
         const int hr = px / hw, hc = px - hr * hw;
         const int ih = oh_first - cv.padT + hr, iw = hc - cv.padL;
         if (ih >= 0 && ih < cv.IH && iw >= 0 && iw < cv.IW)
@@ -135,8 +162,8 @@ __global__ __launch_bounds__(512, 2) void conv3x3_halo_kernel(HaloConv cv, Epilo
       return v;
     };
     auto halo_store = [&](int c, const int4 &v) {
-      if (c < halo_chunks)
-        *reinterpret_cast<int4 *>(s_halo + (c >> 2) * kHaloPix + (c & 3) * 16) = v;
+      const int px = ((c >> 5) << 3) + (c & 7), kc = (c >> 3) & 3;
+      if (px < halo_pixels) *reinterpret_cast<int4 *>(s_halo + px * kHaloPix + kc * 16) = v;
     };
     auto filter_load = [&](int c) -> int4 {
       int4 v = fill4;
