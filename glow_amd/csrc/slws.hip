@@ -333,7 +333,7 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_kernel(SlwsArgs a) {
 
     for (int base = 0; base < len; base += kBatch) {
       const int cnt = min(kBatch, len - base);
-      // round 1: lookup `sub + k*LPB` of the batch is fetched by lane `sub`
+      // first pass: lookup `sub + k*LPB` of the batch is fetched by lane `sub`
       constexpr int kPerLane = kBatch / LPB;
       int row_lo[kPerLane];
       float wgt[kPerLane], scl[kPerLane], ofs[kPerLane];
@@ -377,7 +377,7 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_kernel(SlwsArgs a) {
         scl[k] = s;
         ofs[k] = o;
       }
-      // round 2: all row reads of the batch in flight before the first use
+      // second pass: all row reads of the batch in flight before the first use
       uint32_t q[kBatch];
 #pragma unroll
       for (int j = 0; j < kBatch; j++) {
@@ -501,7 +501,7 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_wave_kernel(SlwsArgs a) {
 
     for (int base = 0; base < len; base += kBatch) {
       const int cnt = min(kBatch, len - base);
-      // round 1: lane j fetches lookup j of the batch
+      // first pass: lane j fetches lookup j of the batch
       int my_key;
       uint32_t so_lo = 0, so_hi = 0;
       float my_w;
@@ -542,7 +542,7 @@ __global__ __launch_bounds__(kSlwsThreads) void slws_wave_kernel(SlwsArgs a) {
           if constexpr (!SO16) so_hi = load_u32_any(so + 4);
         }
       }
-      // round 2: all row reads of the batch in flight before the first use.
+      // second pass: all row reads of the batch in flight before the first use.
       // Lookups are taken four at a time under one uniform branch; slots
       // beyond cnt hold {row 0, w 0, scale 0, offset 0} and add exactly +0.
       uint32_t q[kBatch];
@@ -805,7 +805,7 @@ __global__ __launch_bounds__(WAVES * 64) void slws_rows_kernel(SlwsArgs a) {
 
   for (int base = 0; base < len; base += kBatch) {
     const int cnt = min(kBatch, len - base);
-    // round 1: lane j fetches lookup j of the batch. len never reaches past
+    // first pass: lane j fetches lookup j of the batch. len never reaches past
     // the index list (see rows_bag_span), so lane < cnt is the only check.
     uint32_t so_lo = 0, so_hi = 0;
     float my_w = 0.0f;
@@ -867,7 +867,7 @@ __global__ __launch_bounds__(WAVES * 64) void slws_rows_kernel(SlwsArgs a) {
       continue;
     }
     wave_lds_sync();
-    // round 2: all row reads of the batch in flight before the first use, taken
+    // second pass: all row reads of the batch in flight before the first use, taken
     // kChunk load instructions at a time under one uniform branch. Slots
     // beyond cnt hold {row 0, 0, 0, 0} and add exactly +0.
     uint32_t q[kLoads];
