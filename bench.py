@@ -75,6 +75,7 @@ def parse():
     ap.add_argument("--only", default="",
                     help="run a single extra kernel (profiling aid): "
                          "slws|slws_warm|slws_strict|slws_probe|fc_large|fc_large_zero|fc_c1|fc_m16384|fc_mid|"
+                         "fc_split_k|"
                          "fc|conv_c3|quantize|dequantize|rescale|copy|resnet50|dlrm")
     ap.add_argument("--shape", default="",
                     help="MxKxN of --only fc (a RowwiseQuantizedFullyConnected of that shape)")
@@ -790,12 +791,12 @@ def main():
         capi.check(capi.lib().mi355x_gemm_tile_override(args.tile))
 
     if only and only not in ("slws", "slws_warm", "slws_strict", "slws_probe", "fc", "fc_large", "fc_large_zero",
-                             "fc_c1", "fc_m16384", "fc_mid", "conv_c3", "quantize", "dequantize",
-                             "rescale", "copy"):
+                             "fc_c1", "fc_m16384", "fc_mid", "fc_split_k", "conv_c3", "quantize",
+                             "dequantize", "rescale", "copy"):
         print(f"unknown --only {only}", file=sys.stderr)
         sys.exit(2)
-    if only in ("fc", "fc_large", "fc_large_zero", "fc_c1", "fc_m16384", "fc_mid", "conv_c3", "quantize",
-                "dequantize", "rescale", "copy"):
+    if only in ("fc", "fc_large", "fc_large_zero", "fc_c1", "fc_m16384", "fc_mid", "fc_split_k", "conv_c3",
+                "quantize", "dequantize", "rescale", "copy"):
         if only == "fc":
             M, K, N = (int(v) for v in args.shape.split("x"))
             r = bench_fc(capi, cases, M, K, N, args.steps, args.warmup, use_hint=args.hint)
@@ -812,6 +813,10 @@ def main():
             # a 3x3 convolution of ResNet-50's 14x14 stage as a plain product:
             # 196 workgroups of 128x128, fewer than the part has CUs
             r = bench_fc(capi, cases, 12544, 2304, 256, args.steps, args.warmup)
+        elif only == "fc_split_k":
+            # few output tiles and a long K: the K loop split over workgroups
+            # through a caller's workspace
+            r = bench_fc(capi, cases, 3136, 4608, 512, args.steps, args.warmup, split_k=True)
         elif only == "conv_c3":
             r = bench_conv(capi, cases, args.steps, args.warmup)
         else:

@@ -1284,8 +1284,11 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
         for (int r = 0; r < 16; r++)
           __hip_atomic_store(mine + ((i * TN + j) * 16 + r) * THREADS + tid, acc[i][j][r],
                              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    // every store of this workgroup has been acknowledged before its arrival
-    // is counted
+    // Every store of this workgroup has been acknowledged before its arrival
+    // is counted: each wave waits for its own stores (a workgroup-scope
+    // release fence does not: it orders the waves of a CU through their
+    // shared cache, which these stores pass by), then the waves meet.
+    dma_wait<0>();
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
     uint32_t *s_arrived = reinterpret_cast<uint32_t *>(lds);
