@@ -88,10 +88,14 @@ def parse():
     return ap.parse_args()
 
 
+DIRECT_MAX_STEPS = 64   # launches the host surely queues while a cache flush runs
+
+
 def timed_launches(capi, fn, steps, warmup, flush=None, during=None, lanes=1):
     """Average seconds per launch. `fn(i, stream)` issues launch i. After
     `warmup` eager launches, the `steps` timed launches are recorded into one
-    launch graph and replayed, so the figure is the device-side rate and not
+    launch graph and replayed (or, behind a cache flush and up to
+    DIRECT_MAX_STEPS of them, queued directly while the flush runs), so the figure is the device-side rate and not
     the host's enqueue rate (a Python -> ctypes -> HIP launch costs 4-6 us,
     more than some of these kernels take). HIP events bracket the replay on
     the stream it runs on, with the device idle before and after.
@@ -108,6 +112,22 @@ def timed_launches(capi, fn, steps, warmup, flush=None, during=None, lanes=1):
     for i in range(warmup):
         fn(i, stream) if lanes == 1 else fn(i, stream, 0)
     stream.sync()
+    if flush is not None and lanes == 1 and during is None and steps <= DIRECT_MAX_STEPS:
+        # Behind a flush a short run needs no graph: the flush runs for several
+        # hundred microseconds, the host queues the K launches behind it
+        # meanwhile (5 us each), and the device then finds them back to back.
+        # A replay has a start-up of ~11 us of its own whatever it holds, which
+        # at K = 20 would be 0.5 us on every step.
+        capi.sync()
+        e0, e1 = capi.Event(), capi.Event()
+        flush(stream)
+        e0.record(stream)
+        for i in range(steps):
+            fn(warmup + i, stream)
+        e1.record(stream)
+        e1.sync()
+        capi.sync()
+        return e0.elapsed_ms(e1) * 1e-3 / steps
     side = [capi.Stream() for _ in range(lanes - 1)]
     with capi.Graph(stream) as graph:
         if lanes == 1:
@@ -998,7 +1018,8 @@ def main():
                      "traffic_source": "profiles/slws_rows_kernel__slws_u8_4Mx128_4096bags.md "
                                        "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not "
                                        "measured in this run)",
-                     "kernel": "slws_rows_kernel<false,false,32,true,1,8>"},
+                     "kernel": "slws_rows_kernel<false,false,32,true,1,%d>"
+                               % (16 if args.bags < 16384 else 8)},
         "cpu_baseline": cpu,
         "extra": extra,
     }
