@@ -95,9 +95,9 @@ def timed_launches(capi, fn, steps, warmup, flush=None, during=None, lanes=1):
     """Average seconds per launch. `fn(i, stream)` issues launch i. After
     `warmup` eager launches, the `steps` timed launches are recorded into one
     launch graph and replayed (or, behind a cache flush and up to
-    DIRECT_MAX_STEPS of them, queued directly while the flush runs), so the figure is the device-side rate and not
-    the host's enqueue rate (a Python -> ctypes -> HIP launch costs 4-6 us,
-    more than some of these kernels take). HIP events bracket the replay on
+    DIRECT_MAX_STEPS of them, queued directly while the flush runs), so the
+    figure is the device-side rate and not the host's enqueue rate (a Python ->
+    ctypes -> HIP launch costs 4-6 us, more than some of these kernels take). HIP events bracket the replay on
     the stream it runs on, with the device idle before and after.
     `flush(stream)` runs between the untimed and the timed replay (cache
     flush, queued directly in front of the timed region); `during()` is called
@@ -113,11 +113,13 @@ def timed_launches(capi, fn, steps, warmup, flush=None, during=None, lanes=1):
         fn(i, stream) if lanes == 1 else fn(i, stream, 0)
     stream.sync()
     if flush is not None and lanes == 1 and during is None and steps <= DIRECT_MAX_STEPS:
-        # Behind a flush a short run needs no graph: the flush runs for several
-        # hundred microseconds, the host queues the K launches behind it
-        # meanwhile (5 us each), and the device then finds them back to back.
-        # A replay has a start-up of ~11 us of its own whatever it holds, which
-        # at K = 20 would be 0.5 us on every step.
+        # Behind a flush a short run needs no graph: the flush keeps the stream
+        # busy for several hundred microseconds, the host queues the K launches
+        # behind it meanwhile (5 us each), and the device then finds them back
+        # to back. A replay has a start-up of ~11 us of its own whatever it
+        # holds, which at K = 20 would be 0.5 us on every step. (Without a
+        # flush the replay stays: launches of a few microseconds queued one by
+        # one leave wider gaps than the nodes of a graph, measured.)
         capi.sync()
         e0, e1 = capi.Event(), capi.Event()
         flush(stream)
