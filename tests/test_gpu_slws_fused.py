@@ -350,3 +350,31 @@ def test_random_tables_and_batches(seed):
         ww = weights if weights is not None else np.ones(total, np.float16 if out16 else np.float32)
         got = capi.embedding_bag_rowwise_offsets(table, kind, ww, idx, offs, True, out16, False)
         check(got.astype(np.float32), want.astype(np.float32), mag, out16, what="offsets")
+
+
+@pytest.mark.parametrize("cols", [128, 256])
+def test_bags_per_workgroup_do_not_change_a_bit(cols):
+    """Whole rows of 128 and 256 bytes run sixteen bags per workgroup below
+    16 384 bags per launch and eight from there on. The same bags must come
+    out bit for bit the same whichever launch they are part of, on both sides
+    of the boundary, through the lengths and through host-made positions, and
+    within the element-wise bar of the oracle."""
+    rows = 3000
+    rng = np.random.default_rng(100 + cols)
+    table = cases.random_fused_table(rng, rows, cols)
+    lengths, idx, w = cases.slws_batch(41, rows, 20001, 5, 1.05, np.int64)
+    outs = {}
+    for bags in (4095, 16383, 16384, 20001):
+        L = np.ascontiguousarray(lengths[:bags])
+        total = int(L.sum())
+        say(f"cols {cols} bags {bags} lookups {total}")
+        got = capi.frwq_slws(table, 0, w[:total], idx[:total], L)
+        outs[bags] = got
+        off = capi.frwq_slws(table, 0, w[:total], idx[:total], L, bag_offsets=True)
+        assert np.array_equal(got.view(np.uint32), off.view(np.uint32)), f"offsets, {bags} bags"
+    for small in (4095, 16383, 16384):
+        assert np.array_equal(outs[small].view(np.uint32),
+                              outs[20001][:small].view(np.uint32)), f"{small} of 20001 bags"
+    total = int(lengths.sum())
+    check(outs[20001], go.frwq_slws_f32(table, w[:total], idx[:total], lengths),
+          bag_magnitude(table, 0, w, idx, lengths), what=f"20001 bags of {cols} columns")
