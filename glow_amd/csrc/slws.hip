@@ -43,6 +43,7 @@
 #include <hip/hip_fp16.h>
 
 #include <atomic>
+#include <type_traits>
 #include <mutex>
 #include <vector>
 
@@ -872,72 +873,83 @@ __global__ __launch_bounds__(WAVES * 64) void slws_rows_kernel(SlwsArgs a) {
       continue;
     }
     wave_lds_sync();
-    // second pass: all row reads of the batch in flight before the first use, taken
-    // kChunk load instructions at a time under one uniform branch. Slots
+    // second pass: all row reads of the batch in flight before the first use,
+    // kChunk load instructions per chunk, as many chunks as the batch has
+    // lookups for. The chunk count is wave-uniform and picks one straight-line
+    // body (loads of N chunks, the park of {w, s, o}, arithmetic of N chunks):
+    // with the chunks under separate branches the loaded words become values
+    // carried around the loop and cost a register copy each per batch. Slots
     // beyond cnt hold {row 0, 0, 0, 0} and add exactly +0.
-    uint32_t q[kLoads];
+    auto second_pass = [&](auto nc) {
+      constexpr int N = decltype(nc)::value;   // chunks
+      uint32_t q[N * kChunk];
 #pragma unroll
-    for (int c = 0; c < kLoads / kChunk; c++) {
-      if (c * kChunk * RPI < cnt) {
-#pragma unroll
-        for (int u = 0; u < kChunk; u++) {
-          const int g = c * kChunk + u;
-          const uint32_t key = keys[g * RPI + sub];
-          if constexpr (OFF32) {
-            q[g] = *(const global_u32 *)((const global_u8 *)a.data + (key + lane_off));
-          } else {
-            q[g] = *reinterpret_cast<const uint32_t *>(
-                a.data + (long long)key * a.in_line + lane_off);
-          }
+      for (int g = 0; g < N * kChunk; g++) {
+        const uint32_t key = keys[g * RPI + sub];
+        if constexpr (OFF32) {
+          q[g] = *(const global_u32 *)((const global_u8 *)a.data + (key + lane_off));
+        } else {
+          q[g] = *reinterpret_cast<const uint32_t *>(
+              a.data + (long long)key * a.in_line + lane_off);
         }
       }
-    }
-    {
-      float sc, of;
-      if constexpr (SO16) {
-        sc = __half2float(__ushort_as_half((unsigned short)(so_lo & 0xffff)));
-        of = __half2float(__ushort_as_half((unsigned short)(so_lo >> 16)));
-      } else {
-        sc = __uint_as_float(so_lo);
-        of = __uint_as_float(so_hi);
+      {
+        float sc, of;
+        if constexpr (SO16) {
+          sc = __half2float(__ushort_as_half((unsigned short)(so_lo & 0xffff)));
+          of = __half2float(__ushort_as_half((unsigned short)(so_lo >> 16)));
+        } else {
+          sc = __uint_as_float(so_lo);
+          of = __uint_as_float(so_hi);
+        }
+        if constexpr (MATH == kMathElement)
+          wso[lane] = my_valid ? make_float4(my_w, sc, of, 0.0f)
+                               : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        else
+          wso[lane] = my_valid ? make_float4(my_w * sc, my_w * of, 0.0f, 0.0f)
+                               : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
       }
-      if constexpr (MATH == kMathElement)
-        wso[lane] = my_valid ? make_float4(my_w, sc, of, 0.0f)
-                             : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-      else
-        wso[lane] = my_valid ? make_float4(my_w * sc, my_w * of, 0.0f, 0.0f)
-                             : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-    }
-    wave_lds_sync();
+      wave_lds_sync();
 #pragma unroll
-    for (int c = 0; c < kLoads / kChunk; c++) {
-      if (c * kChunk * RPI < cnt) {
+      for (int g = 0; g < N * kChunk; g++) {
+        if constexpr (PROBE == kProbeRows) {
+          // measurement only: every row read, no arithmetic
+          acc_o = __uint_as_float(__float_as_uint(acc_o) ^ q[g]);
+          continue;
+        }
+        const float4 f = wso[g * RPI + sub];
+        if constexpr (MATH == kMathRegrouped) acc_o += f.y;
+        if constexpr (IS4) {
+          const uint32_t lo = q[g] & 0x0f0f0f0fu, hi = (q[g] >> 4) & 0x0f0f0f0fu;
 #pragma unroll
-        for (int u = 0; u < kChunk; u++) {
-          const int g = c * kChunk + u;
-          if constexpr (PROBE == kProbeRows) {
-            // measurement only: every row read, no arithmetic
-            acc_o = __uint_as_float(__float_as_uint(acc_o) ^ q[g]);
-            continue;
+          for (int b = 0; b < 4; b++) {
+            acc[2 * b] = fused_term<MATH>(f, (float)((lo >> (8 * b)) & 0xff), acc[2 * b]);
+            acc[2 * b + 1] =
+                fused_term<MATH>(f, (float)((hi >> (8 * b)) & 0xff), acc[2 * b + 1]);
           }
-          const float4 f = wso[g * RPI + sub];
-          if constexpr (MATH == kMathRegrouped) acc_o += f.y;
-          if constexpr (IS4) {
-            const uint32_t lo = q[g] & 0x0f0f0f0fu, hi = (q[g] >> 4) & 0x0f0f0f0fu;
+        } else {
 #pragma unroll
-            for (int b = 0; b < 4; b++) {
-              acc[2 * b] = fused_term<MATH>(f, (float)((lo >> (8 * b)) & 0xff), acc[2 * b]);
-              acc[2 * b + 1] =
-                  fused_term<MATH>(f, (float)((hi >> (8 * b)) & 0xff), acc[2 * b + 1]);
-            }
-          } else {
-#pragma unroll
-            for (int b = 0; b < 4; b++)
-              acc[b] = fused_term<MATH>(f, (float)((q[g] >> (8 * b)) & 0xff), acc[b]);
-          }
+          for (int b = 0; b < 4; b++)
+            acc[b] = fused_term<MATH>(f, (float)((q[g] >> (8 * b)) & 0xff), acc[b]);
         }
       }
+    };
+    constexpr int kChunks = kLoads / kChunk;
+    static_assert(kChunks <= 16, "one case per chunk count");
+    const int chunks = (cnt + kChunk * RPI - 1) / (kChunk * RPI);   // 1..kChunks, uniform
+#define MI355X_SECOND_PASS(n)                                                  \
+  case n:                                                                      \
+    if constexpr (n <= kChunks) second_pass(std::integral_constant<int, (n <= kChunks ? n : 1)>()); \
+    break;
+    switch (chunks) {
+      MI355X_SECOND_PASS(1) MI355X_SECOND_PASS(2) MI355X_SECOND_PASS(3) MI355X_SECOND_PASS(4)
+      MI355X_SECOND_PASS(5) MI355X_SECOND_PASS(6) MI355X_SECOND_PASS(7) MI355X_SECOND_PASS(8)
+      MI355X_SECOND_PASS(9) MI355X_SECOND_PASS(10) MI355X_SECOND_PASS(11) MI355X_SECOND_PASS(12)
+      MI355X_SECOND_PASS(13) MI355X_SECOND_PASS(14) MI355X_SECOND_PASS(15) MI355X_SECOND_PASS(16)
+    default:
+      break;
     }
+#undef MI355X_SECOND_PASS
     wave_lds_sync(); // slots are rewritten by the next batch
   }
   if constexpr (PROBE == kProbeRows) acc_o = (float)(__float_as_uint(acc_o) & 0xffu);
