@@ -41,7 +41,7 @@ if ROOT not in sys.path:
 # HBM bytes per launch of the default workloads (FETCH_SIZE + WRITE_SIZE of two
 # counter runs, scaled by what the counters read for a plain copy of known
 # size). They hold for the default sizes only; other sizes report null.
-MEASURED_TRAFFIC = {"slws": 23.80e6, "fc_large": 236.0e6, "conv_c3": 19.63e6}
+MEASURED_TRAFFIC = {"slws": 24.00e6, "fc_large": 236.0e6, "conv_c3": 19.63e6}
 
 HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E, published
 INT8_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA, published (5.0 POP/s)
