@@ -50,10 +50,6 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_skinny_kernel(DenseRows A, Den
   const int tm = blockIdx.x / tiles_n, tn = blockIdx.x - tm * tiles_n;
   const int m0 = tm * 32, n0 = tn * 32;
 
-  // the epilogue's per-column parameters of this lane's column, requested first
-  ColRaw col[1];
-  load_col_raw<1, 32>(col, ep, N, n0, 0, 0, l32);
-
   // rows past the end re-read the last row; their results are not stored
   const int8_t *arow = A.p + (long long)min(m0 + l32, M - 1) * A.ld + lhi * 16;
   const int8_t *brow = B.p + (long long)min(n0 + l32, N - 1) * B.ld + lhi * 16;
@@ -63,9 +59,10 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_skinny_kernel(DenseRows A, Den
   for (int r = 0; r < 16; r++) acc[r] = 0;
 
   const int steps = K / 32;                       // 32-byte K steps in all
-  // wave w takes steps w, w + 4, w + 8, ...
-  for (int base = wave; base < steps; base += 4 * kSkinnyChunk) {
-    v4i af[kSkinnyChunk], bf[kSkinnyChunk];
+  // wave w takes steps w, w + 4, w + 8, ..., kSkinnyChunk of them in flight at
+  // a time
+  v4i af[kSkinnyChunk], bf[kSkinnyChunk];
+  auto request = [&](int base) {
 #pragma unroll
     for (int u = 0; u < kSkinnyChunk; u++) {
       // steps past the end re-read the last step of this wave and are not used
@@ -73,10 +70,26 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_skinny_kernel(DenseRows A, Den
       af[u] = *reinterpret_cast<const v4i *>(arow + s * 32);
       bf[u] = *reinterpret_cast<const v4i *>(brow + s * 32);
     }
+  };
+  int base = wave;
+  request(base);
+  // The epilogue's per-column parameters of this lane's column are asked for
+  // behind the first operands: their ten optional arrays are some two hundred
+  // instructions of address arithmetic and null checks, which in front of the
+  // operand loads is time the whole launch waits (it is a few microseconds
+  // long), and behind them runs while the operands are on their way.
+  __builtin_amdgcn_sched_barrier(0);
+  ColRaw col[1];
+  load_col_raw<1, 32>(col, ep, N, n0, 0, 0, l32);
+  __builtin_amdgcn_sched_barrier(0);
+  while (true) {
 #pragma unroll
     for (int u = 0; u < kSkinnyChunk; u++)
       if (base + 4 * u < steps)
         acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[u], bf[u], acc, 0, 0, 0);
+    base += 4 * kSkinnyChunk;
+    if (base >= steps) break;
+    request(base);
   }
 
   // the four partial tiles meet in LDS
