@@ -897,10 +897,14 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_i8_kernel(
 #pragma unroll
     for (int i = 0; i < B_CH; i++) *reinterpret_cast<int4 *>(stage + b_lds[i]) = rb[slot][i];
   };
-  // the epilogue's per-column parameters, requested with the first tile
+  // the first tile is requested ahead of the epilogue's per-column parameters
+  // (two hundred instructions of address arithmetic and null checks over ten
+  // optional arrays, which then run while the tile is on its way)
+  fetch(0, 0);
+  __builtin_amdgcn_sched_barrier(0);
   ColRaw col[TN];
   load_col_raw<TN, WN>(col, ep, N, n0, n_base, wn, l32);
-  fetch(0, 0);
+  __builtin_amdgcn_sched_barrier(0);
   park(0, lds);
   // tiles 1..D on their way; tile t lives in register slot (t - 1) % D
 #pragma unroll
@@ -1122,17 +1126,23 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64,
     else
       dma16(bptr[i - A_LOADS] + k0, slot, b_dst[i - A_LOADS]);
   };
-  // requested first, consumed in the epilogue
-  ColRaw col[TN];
-  load_col_raw<TN, WN>(col, ep, N, n0, n_base, wn, l32);
   // prologue: tiles 0..STAGES-2 and the first half of tile STAGES-1 in flight
   // (tiles past the end are re-reads of the last one into slots nobody
-  // consumes, which keeps the counts uniform)
+  // consumes, which keeps the counts uniform). The columns' constants, which
+  // the epilogue consumes, are requested behind tile 0: the first multiply
+  // waits for that tile, and the constants' address arithmetic (ten optional
+  // arrays) then runs while it is on its way.
+  ColRaw col[TN];
 #pragma unroll
   for (int s = 0; s < STAGES - 1; s++) {
     const typename ARows::Loc loc = locate_tile(s);
 #pragma unroll
     for (int i = 0; i < LOADS; i++) issue_load(s, s * STAGE, min(s, KT - 1) * kBK, i, loc);
+    if (s == 0) {
+      __builtin_amdgcn_sched_barrier(0);
+      load_col_raw<TN, WN>(col, ep, N, n0, n_base, wn, l32);
+      __builtin_amdgcn_sched_barrier(0);
+    }
   }
   // the tile whose second half is still to be requested
   typename ARows::Loc half_loc = locate_tile(STAGES - 1);
