@@ -129,11 +129,12 @@ __global__ __launch_bounds__(512, 2) void conv3x3_halo_kernel(HaloConv cv, Epilo
   const int hw = cv.OW + 2;                   // halo pixels per row
   const int mode = requant_mode(ep);
 
-  // the channels' raw parameters, requested first (by the last wave: the first
-  // ones carry the staging loop's remainders)
+  // the channels' raw parameters are requested by the last wave (the first
+  // ones carry the staging loop's remainders), behind its share of the staging
+  // loads: in front of them their address arithmetic (ten optional arrays)
+  // would hold back loads the whole workgroup waits for at the barrier
   const bool par_wave = wave == (int)(nthreads >> 6) - 1;
   ColRaw col[1];
-  if (par_wave) load_col_raw<1, 64>(col, ep, cv.OC, n0, 0, 0, lane);
 
   // ---- stage the tile's input rows and the filter slice -------------------------
   if constexpr (!(SKIP & 1)) {
@@ -188,6 +189,11 @@ __global__ __launch_bounds__(512, 2) void conv3x3_halo_kernel(HaloConv cv, Epilo
     for (int u = 0; u < HU; u++) hv[u] = halo_load(tid + u * nthreads);
 #pragma unroll
     for (int u = 0; u < FU; u++) fv[u] = filter_load(tid + u * nthreads);
+    if constexpr (SKIP == 0) {
+      __builtin_amdgcn_sched_barrier(0);
+      if (par_wave) load_col_raw<1, 64>(col, ep, cv.OC, n0, 0, 0, lane);
+      __builtin_amdgcn_sched_barrier(0);
+    }
 #pragma unroll
     for (int u = 0; u < HU; u++) halo_store(tid + u * nthreads, hv[u]);
 #pragma unroll
@@ -206,6 +212,9 @@ __global__ __launch_bounds__(512, 2) void conv3x3_halo_kernel(HaloConv cv, Epilo
     }
   }
 
+  if constexpr (SKIP != 0) {
+    if (par_wave) load_col_raw<1, 64>(col, ep, cv.OC, n0, 0, 0, lane);
+  }
   // ---- the channels' requantisation constants -> LDS --------------------------------
   if (par_wave) par_table_store<kHaloBN>(s_par, lane, col[0], ep, kHaloK, mode);
   __syncthreads();
