@@ -1010,7 +1010,7 @@ def main():
         "max_error_over_bag_magnitude": parity,
         "arithmetic": "v = fma(s, q, o); acc = fma(w, v, acc) per element in bag order "
                       "(MI355X_SLWS_MATH_ELEMENT, the library's default)",
-        "cache_state": ("caches flushed before the timed replay; "
+        "cache_state": ("caches flushed before the timed launches; "
                         f"{args.batches} distinct index batches cycled"),
         "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
